@@ -1,0 +1,470 @@
+"""Host-side mirror of Honeycrisp's `Backend` op interface and its MI355X implementation.
+
+`Backend` restates the open class of Sources/Honeycrisp/Backend.swift:28-890 (same method
+names, argument meaning and error behaviour: every op of the bare base class raises
+`BackendError.notImplemented`, `normalize` and `repeated` have the base-class compositions).
+`HIPBackend` is the drop-in for the ops on the hot path: each method enqueues one call of
+the C ABI (include/hchip.h) on the context's in-order stream and returns a device buffer
+(`HIPData`, the `Tensor.Data` of this backend) immediately.
+
+There is no CPU fallback here: an op or dtype the kernels do not cover raises
+`BackendError.notImplemented`, and a missing libhchip.so is an ImportError.
+"""
+import ctypes
+import threading
+from ctypes import byref, c_float, c_int64, c_size_t, c_void_p
+from typing import List, Optional, Sequence, Union
+
+import numpy as np
+
+from . import _lib
+from .descriptors import (BackendError, BroadcastData, BroadcastStrides, ComparisonOp, DType,
+                          ElemwiseOp, NumericBinaryOp, ReduceDims, ReduceOp, RepeatDims,
+                          ScatterGatherIndices, product)
+
+
+class Backend:
+    """Abstract op set (Backend.swift:170-815)."""
+
+    _default: Optional["Backend"] = None
+    _tls = threading.local()
+
+    # -- Backend.defaultBackend / current / use (Backend.swift:44-88)
+    @classmethod
+    def setDefault(cls, backend: "Backend"):
+        Backend._default = backend
+
+    @classmethod
+    def current(cls) -> "Backend":
+        stack = getattr(Backend._tls, "stack", None)
+        if stack:
+            return stack[-1]
+        if Backend._default is None:
+            raise RuntimeError("no default backend installed (Backend.setDefault)")
+        return Backend._default
+
+    class _Use:
+        def __init__(self, backend):
+            self.backend = backend
+
+        def __enter__(self):
+            if not hasattr(Backend._tls, "stack"):
+                Backend._tls.stack = []
+            Backend._tls.stack.append(self.backend)
+            return self.backend
+
+        def __exit__(self, *exc):
+            Backend._tls.stack.pop()
+            return False
+
+    def use(self):
+        return Backend._Use(self)
+
+    def _ni(self, name):
+        raise BackendError.notImplemented(name)
+
+    def allocate(self, byteCount):
+        self._ni("allocate")
+
+    def broadcast(self, a, dtype):
+        self._ni("broadcast")
+
+    def binaryOp(self, a, b, op, dtype, count=None):
+        self._ni("binaryOp")
+
+    def mulAdd(self, input, coeff, bias, dtype):
+        self._ni("mulAdd")
+
+    def addMul(self, input, bias, coeff, dtype):
+        self._ni("addMul")
+
+    def compare(self, a, b, op, dtype, count=None):
+        self._ni("compare")
+
+    def cast(self, a, count, inType, outType):
+        self._ni("cast")
+
+    def pow(self, a, b, scale, scales, count, dtype):
+        self._ni("pow")
+
+    def reduce(self, a, op, dims, dtype):
+        self._ni("reduce")
+
+    def logSoftmax(self, a, dims, dtype):
+        self._ni("logSoftmax")
+
+    def gather(self, a, s, dtype):
+        self._ni("gather")
+
+    def when(self, mask, a, b, dtype):
+        self._ni("when")
+
+    def matmul(self, a, transA, b, transB, transOut, rows, inner, cols, dtype):
+        self._ni("matmul")
+
+    def batchedMatmul(self, matrixCount, a, transA, b, transB, transOut, rows, inner, cols, dtype):
+        self._ni("batchedMatmul")
+
+    def triangular(self, a, batch, rows, cols, upper, offset, dtype):
+        self._ni("triangular")
+
+    def elemwise(self, a, op, scales, count, dtype):
+        self._ni("elemwise")
+
+    def concat(self, inputs, outerCount, innerCounts, dtype):
+        self._ni("concat")
+
+    def constant(self, value, count, dtype):
+        self._ni("constant")
+
+    def collection(self, collection, reverse, dtype):
+        self._ni("collection")
+
+    def axisPermutation(self, permutation, shape):
+        self._ni("axisPermutation")
+
+    # -- base-class compositions
+
+    def repeated(self, a, dims: RepeatDims, dtype):
+        """Backend.swift:590-606."""
+        return self.broadcast(
+            BroadcastData(
+                BroadcastStrides([dims.outerCount, dims.repeatCount, dims.innerCount],
+                                 [dims.innerCount, 0, 1]), a), dtype)
+
+    def normalize(self, input, dims: ReduceDims, eps, dtype):
+        """Backend.swift:265-327: two-pass mean / biased variance, op by op."""
+        full = BroadcastStrides.contiguousForShape([dims.outerCount, dims.reduceCount, dims.innerCount])
+        reduced = BroadcastStrides(full.shape, [dims.innerCount, 0, 1])
+        inv_n = np.float32(1.0) / np.float32(dims.reduceCount)
+        mean = self.binaryOp(self.reduce(input, ReduceOp.sum, dims, dtype), inv_n, NumericBinaryOp.mul,
+                             dtype, count=reduced.dataCount)
+        centered = self.binaryOp(BroadcastData(full, input), BroadcastData(reduced, mean),
+                                 NumericBinaryOp.sub, dtype)
+        variance = self.binaryOp(
+            self.reduce(self.pow(centered, 2.0, 1.0, None, full.dataCount, dtype), ReduceOp.sum, dims, dtype),
+            inv_n, NumericBinaryOp.mul, dtype, count=reduced.dataCount)
+        normalizer = self.pow(
+            self.binaryOp(variance, eps, NumericBinaryOp.add, dtype, count=reduced.dataCount),
+            -0.5, 1.0, None, reduced.dataCount, dtype)
+        return self.binaryOp(BroadcastData(full, centered), BroadcastData(reduced, normalizer),
+                             NumericBinaryOp.mul, dtype)
+
+
+class HIPData:
+    """Device buffer backing a tensor: this backend's `Tensor.Data` (Tensor.swift:69-85)."""
+
+    def __init__(self, backend: "HIPBackend", ptr: int, byteCount: int):
+        self.backend = backend
+        self.ptr = ptr
+        self.byteCount = byteCount
+
+    def wait(self):
+        self.backend.sync()
+
+    def onCPU(self) -> np.ndarray:
+        """Host copy of the bytes (blocking, ordered after all enqueued work)."""
+        host = np.empty(self.byteCount, dtype=np.uint8)
+        if self.byteCount:
+            self.backend._check(self.backend._lib.hc_memcpy_d2h(
+                self.backend._ctx, host.ctypes.data_as(c_void_p), c_void_p(self.ptr), self.byteCount))
+        return host
+
+    def __del__(self):
+        backend, ptr = self.backend, self.ptr
+        self.ptr = None
+        if ptr and backend is not None and backend._ctx:
+            backend._lib.hc_free(backend._ctx, c_void_p(ptr))
+
+
+Scalar = Union[int, float, np.floating, np.integer]
+
+
+class HIPBackend(Backend):
+    """MI355X backend: one device, one in-order stream, kernels from libhchip.so."""
+
+    def __init__(self, device: int = 0):
+        self._ctx = None
+        self._lib = _lib.load()
+        ctx = c_void_p()
+        status = self._lib.hc_init(device, byref(ctx))
+        if status != _lib.HC_OK:
+            self._raise(status)
+        self._ctx = ctx
+
+    def close(self):
+        if self._ctx:
+            self._lib.hc_shutdown(self._ctx)
+            self._ctx = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    # -- errors (mapping of Backend.swift:6-16)
+
+    def _raise(self, status):
+        msg = self._lib.hc_last_error_string().decode("utf-8", "replace")
+        if status == _lib.HC_ERR_ALLOC:
+            raise BackendError.allocationFailed(msg)
+        if status in (_lib.HC_ERR_LOAD, _lib.HC_ERR_NO_DEVICE):
+            raise BackendError.failedToLoadKernels(msg)
+        if status == _lib.HC_ERR_UNSUPPORTED:
+            raise BackendError.notImplemented(msg)
+        raise BackendError.kernelFailed(msg)
+
+    def _check(self, status):
+        if status != _lib.HC_OK:
+            self._raise(status)
+
+    # -- device / stream
+
+    def deviceInfo(self) -> dict:
+        info = _lib.hc_device_info()
+        self._check(self._lib.hc_get_device_info(self._ctx, byref(info)))
+        return {
+            "name": info.name.decode(), "arch": info.arch.decode(), "compute_units": info.compute_units,
+            "clock_mhz": info.clock_mhz, "wavefront_size": info.wavefront_size,
+            "lds_bytes_per_block": info.lds_bytes_per_block, "total_mem": info.total_mem,
+        }
+
+    def sync(self):
+        self._check(self._lib.hc_sync(self._ctx))
+
+    # -- storage (DataAllocator, Backend.swift:894-896)
+
+    def allocate(self, byteCount: int) -> HIPData:
+        ptr = c_void_p()
+        self._check(self._lib.hc_malloc(self._ctx, c_size_t(max(int(byteCount), 0)), byref(ptr)))
+        return HIPData(self, ptr.value, int(byteCount))
+
+    def upload(self, host: np.ndarray) -> HIPData:
+        host = np.ascontiguousarray(host)
+        data = self.allocate(host.nbytes)
+        if host.nbytes:
+            self._check(self._lib.hc_memcpy_h2d(self._ctx, c_void_p(data.ptr),
+                                                host.ctypes.data_as(c_void_p), host.nbytes))
+        return data
+
+    def _dev(self, data) -> HIPData:
+        """Device buffer for `data`; foreign data is uploaded (cf. BackendMPS.swift:585-620)."""
+        if isinstance(data, HIPData) and data.backend is self:
+            return data
+        if isinstance(data, np.ndarray):
+            return self.upload(data)
+        if hasattr(data, "onCPU"):
+            return self.upload(data.onCPU())
+        raise TypeError("cannot use %r as tensor data" % type(data))
+
+    @staticmethod
+    def _s(strides: BroadcastStrides):
+        return _lib.make_strides(strides.shape, strides.strides)
+
+    @staticmethod
+    def _scalar(value, dtype: DType):
+        """(float32 value, int64 value) the way T.toFloat() / T.toInt64() would give them."""
+        if dtype == DType.int64:
+            return c_float(0.0), c_int64(int(value))
+        return c_float(float(np.float32(value))), c_int64(0)
+
+    # -- ops
+
+    def collection(self, collection, reverse: bool, dtype: DType) -> HIPData:
+        """Backend.swift:794-800: host values -> buffer of `dtype` (arrayToPointer conversion)."""
+        arr = np.asarray(list(collection) if not isinstance(collection, np.ndarray) else collection)
+        if reverse:
+            arr = arr[::-1]
+        return self.upload(convert_host_array(arr.reshape(-1), dtype))
+
+    def constant(self, value, count: int, dtype: DType) -> HIPData:
+        out = self.allocate(count * dtype.byteSize)
+        vf, vi = self._scalar(value, dtype)
+        if dtype != DType.int64:
+            vf = c_float(float(np.float32(value)))
+        self._check(self._lib.hc_fill(self._ctx, int(dtype), vf, vi, c_void_p(out.ptr), count))
+        return out
+
+    def broadcast(self, a: BroadcastData, dtype: DType) -> HIPData:
+        out = self.allocate(product(a.strides.shape) * dtype.byteSize)
+        ad = self._dev(a.data)
+        s = self._s(a.strides)
+        self._check(self._lib.hc_broadcast(self._ctx, int(dtype), c_void_p(ad.ptr), byref(s), c_void_p(out.ptr)))
+        return out
+
+    def binaryOp(self, a, b, op: NumericBinaryOp, dtype: DType, count: Optional[int] = None) -> HIPData:
+        if isinstance(a, BroadcastData) and isinstance(b, BroadcastData):
+            out = self.allocate(product(a.strides.shape) * dtype.byteSize)
+            ad, bd = self._dev(a.data), self._dev(b.data)
+            sa, sb = self._s(a.strides), self._s(b.strides)
+            self._check(self._lib.hc_binary_op(self._ctx, int(op), int(dtype), c_void_p(ad.ptr), byref(sa),
+                                               c_void_p(bd.ptr), byref(sb), c_void_p(out.ptr)))
+            return out
+        if count is None:
+            raise TypeError("binaryOp with a scalar needs count")
+        scalar_first = isinstance(a, (int, float, np.floating, np.integer))
+        tensor, scalar = (b, a) if scalar_first else (a, b)
+        out = self.allocate(count * dtype.byteSize)
+        td = self._dev(tensor)
+        sf, si = self._scalar(scalar, dtype)
+        self._check(self._lib.hc_binary_op_scalar(self._ctx, int(op), int(dtype), c_void_p(td.ptr), sf, si,
+                                                  int(scalar_first), c_void_p(out.ptr), count))
+        return out
+
+    def _fused(self, fn, x, y, z, dtype):
+        out = self.allocate(product(x.strides.shape) * dtype.byteSize)
+        xd, yd, zd = self._dev(x.data), self._dev(y.data), self._dev(z.data)
+        sx, sy, sz = self._s(x.strides), self._s(y.strides), self._s(z.strides)
+        self._check(fn(self._ctx, int(dtype), c_void_p(xd.ptr), byref(sx), c_void_p(yd.ptr), byref(sy),
+                       c_void_p(zd.ptr), byref(sz), c_void_p(out.ptr)))
+        return out
+
+    def mulAdd(self, input: BroadcastData, coeff: BroadcastData, bias: BroadcastData, dtype: DType):
+        return self._fused(self._lib.hc_mul_add, input, coeff, bias, dtype)
+
+    def addMul(self, input: BroadcastData, bias: BroadcastData, coeff: BroadcastData, dtype: DType):
+        return self._fused(self._lib.hc_add_mul, input, bias, coeff, dtype)
+
+    def when(self, mask: BroadcastData, a, b, dtype: DType):
+        """a / b: BroadcastData, or ("scalar", value, shape) like Backend.TensorOrScalar
+        (Backend.swift:30-42); scalars become 1-element constants with all-zero strides
+        (BackendCPU.swift:1860-1868)."""
+        def branch(x):
+            if isinstance(x, BroadcastData):
+                return x
+            _, value, shape = x
+            return BroadcastData(BroadcastStrides(shape, [0] * len(shape)), self.constant(value, 1, dtype))
+        return self._fused(self._lib.hc_when, mask, branch(a), branch(b), dtype)
+
+    def compare(self, a, b, op: ComparisonOp, dtype: DType, count: Optional[int] = None) -> HIPData:
+        if isinstance(a, BroadcastData) and isinstance(b, BroadcastData):
+            out = self.allocate(product(a.strides.shape))
+            ad, bd = self._dev(a.data), self._dev(b.data)
+            sa, sb = self._s(a.strides), self._s(b.strides)
+            self._check(self._lib.hc_compare(self._ctx, int(op), int(dtype), c_void_p(ad.ptr), byref(sa),
+                                             c_void_p(bd.ptr), byref(sb), c_void_p(out.ptr)))
+            return out
+        if count is None:
+            raise TypeError("compare with a scalar needs count")
+        scalar_first = isinstance(a, (int, float, bool, np.floating, np.integer, np.bool_))
+        tensor, scalar = (b, a) if scalar_first else (a, b)
+        out = self.allocate(count)
+        td = self._dev(tensor)
+        sf, si = self._scalar(scalar, dtype)
+        self._check(self._lib.hc_compare_scalar(self._ctx, int(op), int(dtype), c_void_p(td.ptr), sf, si,
+                                                int(scalar_first), c_void_p(out.ptr), count))
+        return out
+
+    def cast(self, a, count: int, inType: DType, outType: DType) -> HIPData:
+        out = self.allocate(count * outType.byteSize)
+        ad = self._dev(a)
+        self._check(self._lib.hc_cast(self._ctx, c_void_p(ad.ptr), int(inType), c_void_p(out.ptr),
+                                      int(outType), count))
+        return out
+
+    def pow(self, a, b: Scalar, scale: Scalar, scales, count: int, dtype: DType) -> HIPData:
+        out = self.allocate(count * dtype.byteSize)
+        ad = self._dev(a)
+        sd = self._dev(scales) if scales is not None else None
+        bf, bi = self._scalar(b, dtype)
+        scf, sci = self._scalar(scale, dtype)
+        self._check(self._lib.hc_pow(self._ctx, int(dtype), c_void_p(ad.ptr), bf, scf, bi, sci,
+                                     c_void_p(sd.ptr) if sd else None, c_void_p(out.ptr), count))
+        return out
+
+    def elemwise(self, a, op: ElemwiseOp, scales, count: int, dtype: DType) -> HIPData:
+        out = self.allocate(count * dtype.byteSize)
+        ad = self._dev(a)
+        sd = self._dev(scales) if scales is not None else None
+        self._check(self._lib.hc_elemwise(self._ctx, int(op), int(dtype), c_void_p(ad.ptr),
+                                          c_void_p(sd.ptr) if sd else None, c_void_p(out.ptr), count))
+        return out
+
+    def reduce(self, a, op: ReduceOp, dims: ReduceDims, dtype: DType) -> HIPData:
+        outType = DType.int64 if op.isIntOut else dtype
+        out = self.allocate(dims.outCount * outType.byteSize)
+        ad = self._dev(a)
+        self._check(self._lib.hc_reduce(self._ctx, int(op), int(dtype), c_void_p(ad.ptr), c_void_p(out.ptr),
+                                        dims.outerCount, dims.reduceCount, dims.innerCount))
+        return out
+
+    def logSoftmax(self, a, dims: ReduceDims, dtype: DType) -> HIPData:
+        out = self.allocate(dims.inCount * dtype.byteSize)
+        ad = self._dev(a)
+        self._check(self._lib.hc_log_softmax(self._ctx, int(dtype), c_void_p(ad.ptr), c_void_p(out.ptr),
+                                             dims.outerCount, dims.reduceCount, dims.innerCount))
+        return out
+
+    def normalize(self, input, dims: ReduceDims, eps: Scalar, dtype: DType) -> HIPData:
+        """Fused override of the base-class composition (same arithmetic, one kernel for
+        innerCount == 1)."""
+        out = self.allocate(dims.inCount * dtype.byteSize)
+        ad = self._dev(input)
+        self._check(self._lib.hc_normalize(self._ctx, int(dtype), c_void_p(ad.ptr), c_void_p(out.ptr),
+                                           dims.outerCount, dims.reduceCount, dims.innerCount,
+                                           c_float(float(np.float32(eps)))))
+        return out
+
+    def gather(self, a, s: ScatterGatherIndices, dtype: DType) -> HIPData:
+        out = self.allocate(s.gatherOutCount * dtype.byteSize)
+        ad, idx = self._dev(a), self._dev(s.indices.data)
+        st = self._s(s.indices.strides)
+        self._check(self._lib.hc_gather(self._ctx, int(dtype), c_void_p(ad.ptr), c_void_p(idx.ptr), byref(st),
+                                        c_void_p(out.ptr), s.outerCount, s.middleCount, s.outCount,
+                                        s.innerCount))
+        return out
+
+    def matmul(self, a, transA: bool, b, transB: bool, transOut: bool, rows: int, inner: int, cols: int,
+               dtype: DType) -> HIPData:
+        return self.batchedMatmul(1, a, transA, b, transB, transOut, rows, inner, cols, dtype)
+
+    def batchedMatmul(self, matrixCount: int, a, transA: bool, b, transB: bool, transOut: bool, rows: int,
+                      inner: int, cols: int, dtype: DType) -> HIPData:
+        out = self.allocate(matrixCount * rows * cols * dtype.byteSize)
+        ad, bd = self._dev(a), self._dev(b)
+        self._check(self._lib.hc_matmul(self._ctx, int(dtype), matrixCount, c_void_p(ad.ptr), int(transA),
+                                        c_void_p(bd.ptr), int(transB), int(transOut), rows, inner, cols,
+                                        c_void_p(out.ptr)))
+        return out
+
+    def triangular(self, a, batch: int, rows: int, cols: int, upper: bool, offset: int, dtype: DType):
+        out = self.allocate(batch * rows * cols * dtype.byteSize)
+        ad = self._dev(a)
+        self._check(self._lib.hc_triangular(self._ctx, int(dtype), c_void_p(ad.ptr), c_void_p(out.ptr), batch,
+                                            rows, cols, int(upper), offset))
+        return out
+
+    def concat(self, inputs: Sequence, outerCount: int, innerCounts: Sequence[int], dtype: DType):
+        assert len(inputs) == len(innerCounts)
+        devs = [self._dev(x) for x in inputs]
+        out = self.allocate(outerCount * sum(innerCounts) * dtype.byteSize)
+        n = len(devs)
+        ptrs = (c_void_p * max(n, 1))(*[d.ptr for d in devs])
+        counts = (c_int64 * max(n, 1))(*innerCounts)
+        self._check(self._lib.hc_concat(self._ctx, int(dtype), ptrs, counts, n, outerCount, c_void_p(out.ptr)))
+        return out
+
+    def axisPermutation(self, permutation: List[int], shape: List[int]) -> HIPData:
+        n = len(shape)
+        out = self.allocate(product(shape) * 8)
+        perm = (c_int64 * max(n, 1))(*permutation)
+        shp = (c_int64 * max(n, 1))(*shape)
+        self._check(self._lib.hc_axis_permutation(self._ctx, perm, shp, n, c_void_p(out.ptr)))
+        return out
+
+
+def convert_host_array(arr: np.ndarray, dtype: DType) -> np.ndarray:
+    """Host array -> bytes of `dtype` with the conversions of arrayToPointer
+    (TensorElement.swift:225-260): float sources truncate toward zero into int64, anything
+    becomes bool by `!= 0`, floats round to nearest even into float16."""
+    arr = np.asarray(arr)
+    if dtype == DType.bool:
+        return np.ascontiguousarray(arr != 0)
+    if dtype == DType.int64:
+        if arr.dtype.kind == "f":
+            return np.trunc(arr).astype(np.int64)
+        return arr.astype(np.int64)
+    if dtype == DType.float32:
+        return arr.astype(np.float32)
+    return arr.astype(np.float32).astype(np.float16)

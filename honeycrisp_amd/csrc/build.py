@@ -1,0 +1,68 @@
+"""Build libhchip.so: gfx950 code objects via `hipcc --genco`, embedded into the host library.
+
+Usage: python -m honeycrisp_amd.csrc.build   (or build_all() from Python)
+Outputs, all in this directory: build/*.hsaco (intermediate) and libhchip.so.
+"""
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+KERNEL_DIR = os.path.join(HERE, "kernels")
+BUILD_DIR = os.path.join(HERE, "build")
+LIB_PATH = os.path.join(HERE, "libhchip.so")
+ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
+HIPCC = os.path.join(ROCM, "bin", "hipcc")
+
+# (code object, source, extra flags). -ffp-contract=off: the reference never fuses a*b+c.
+# The packed-fp32 feature is switched off for every HIP compile.
+KERNELS = [
+    ("elementwise", "elementwise.hip", ["-ffp-contract=off"]),
+    ("reduce", "reduce.hip", ["-ffp-contract=off"]),
+    ("gather", "gather.hip", []),
+    ("gemm", "gemm.hip", []),
+]
+DEVICE_FLAGS = [
+    "--offload-arch=gfx950", "--genco", "-O3", "-std=c++17",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+
+def _run(cmd):
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), proc.stdout))
+    return proc.stdout
+
+
+def build_kernel(name, src, extra):
+    out = os.path.join(BUILD_DIR, name + ".hsaco")
+    _run([HIPCC] + DEVICE_FLAGS + extra + ["-o", out, os.path.join(KERNEL_DIR, src)])
+    return out
+
+
+def build_all(verbose=True):
+    os.makedirs(BUILD_DIR, exist_ok=True)
+    with ThreadPoolExecutor(max_workers=4) as pool:
+        futures = [pool.submit(build_kernel, *k) for k in KERNELS]
+        for f in futures:
+            path = f.result()
+            if verbose:
+                print("built", os.path.relpath(path, HERE), os.path.getsize(path), "bytes")
+    host_flags = ["-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-I" + os.path.join(ROCM, "include")]
+    _run(["g++"] + host_flags + [
+        "-Wa,-I," + BUILD_DIR,
+        os.path.join(HERE, "hchip.cpp"), os.path.join(HERE, "embed.S"),
+        "-o", LIB_PATH,
+        "-L" + os.path.join(ROCM, "lib"), "-lamdhip64", "-Wl,-rpath," + os.path.join(ROCM, "lib"),
+        "-lpthread",
+    ])
+    if verbose:
+        print("built", os.path.relpath(LIB_PATH, HERE), os.path.getsize(LIB_PATH), "bytes")
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    build_all()
+    sys.exit(0)

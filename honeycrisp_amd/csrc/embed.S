@@ -1,0 +1,21 @@
+/* Embeds the gfx950 code objects (built by `hipcc --genco`, see build.py) into libhchip.so
+ * as read-only data; hchip.cpp hands them to hipModuleLoadData. The assembler's include
+ * path (-Wa,-I) points at the directory holding the .hsaco files. */
+    .section .rodata
+    .macro EMBED sym, file
+    .balign 4096
+    .global \sym
+    .type \sym, @object
+\sym:
+    .incbin "\file"
+    .global \sym\()_end
+\sym\()_end:
+    .byte 0
+    .endm
+
+    EMBED hc_image_elementwise, "elementwise.hsaco"
+    EMBED hc_image_reduce, "reduce.hsaco"
+    EMBED hc_image_gather, "gather.hsaco"
+    EMBED hc_image_gemm, "gemm.hsaco"
+
+    .section .note.GNU-stack,"",@progbits

@@ -1,0 +1,1256 @@
+// Host side of the hchip C ABI (include/hchip.h): context, caching allocator, code-object
+// loading and the per-operation launchers. Talks to the HIP runtime only through
+// hipMalloc / hipMemcpyAsync / hipModuleLoadData / hipModuleLaunchKernel and friends; the
+// kernels are gfx950 code objects built with `hipcc --genco` and embedded in this library
+// (embed.S), so this file compiles with any host C++ compiler.
+#ifndef __HIP_PLATFORM_AMD__
+#define __HIP_PLATFORM_AMD__ 1
+#endif
+#include <hip/hip_runtime_api.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "../../include/hchip.h"
+#include "kargs.h"
+
+extern "C" {
+extern const unsigned char hc_image_elementwise[], hc_image_elementwise_end[];
+extern const unsigned char hc_image_reduce[], hc_image_reduce_end[];
+extern const unsigned char hc_image_gather[], hc_image_gather_end[];
+extern const unsigned char hc_image_gemm[], hc_image_gemm_end[];
+}
+
+struct hc_module {
+  hipModule_t mod;
+};
+struct hc_function {
+  hipFunction_t fn;
+};
+struct hc_event {
+  hipEvent_t ev;
+};
+
+struct hc_ctx {
+  int device = 0;
+  hipStream_t stream = nullptr;
+  std::mutex mu;
+  std::vector<hipModule_t> modules;
+  std::unordered_map<std::string, hipFunction_t> functions;
+  std::unordered_map<size_t, std::vector<void*>> free_blocks;
+  std::unordered_map<void*, size_t> live;
+  size_t bytes_in_use = 0, bytes_cached = 0;
+  hipDeviceProp_t props;
+};
+
+static thread_local std::string g_last_error;
+
+static int fail(int code, const char* fmt, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  g_last_error = buf;
+  return code;
+}
+
+static int hip_fail(hipError_t e, const char* what) {
+  return fail(HC_ERR_HIP_BASE + (int)e, "%s: %s (%s)", what, hipGetErrorString(e), hipGetErrorName(e));
+}
+
+#define HIP_TRY(expr)                              \
+  do {                                             \
+    hipError_t _e = (expr);                        \
+    if (_e != hipSuccess) return hip_fail(_e, #expr); \
+  } while (0)
+
+#define HC_TRY(expr)          \
+  do {                        \
+    int _s = (expr);          \
+    if (_s != HC_OK) return _s; \
+  } while (0)
+
+#define REQUIRE(cond, ...)                                   \
+  do {                                                       \
+    if (!(cond)) return fail(HC_ERR_INVALID, __VA_ARGS__);   \
+  } while (0)
+
+extern "C" const char* hc_last_error_string(void) { return g_last_error.c_str(); }
+
+// ------------------------------------------------------------------ context
+
+static int load_image(hc_ctx* ctx, const unsigned char* begin, const unsigned char* end, const char* name) {
+  if (end <= begin) return fail(HC_ERR_LOAD, "embedded code object '%s' is empty", name);
+  hipModule_t mod;
+  hipError_t e = hipModuleLoadData(&mod, begin);
+  if (e != hipSuccess)
+    return fail(HC_ERR_LOAD, "hipModuleLoadData(%s): %s", name, hipGetErrorString(e));
+  ctx->modules.push_back(mod);
+  return HC_OK;
+}
+
+extern "C" int hc_init(int device, hc_ctx** out) {
+  REQUIRE(out != nullptr, "hc_init: out is null");
+  *out = nullptr;
+  int count = 0;
+  hipError_t e = hipGetDeviceCount(&count);
+  if (e != hipSuccess || count <= 0)
+    return fail(HC_ERR_NO_DEVICE, "no HIP device available (%s)", hipGetErrorString(e));
+  REQUIRE(device >= 0 && device < count, "hc_init: device %d out of range (have %d)", device, count);
+  HIP_TRY(hipSetDevice(device));
+  hc_ctx* ctx = new hc_ctx();
+  ctx->device = device;
+  e = hipGetDeviceProperties(&ctx->props, device);
+  if (e != hipSuccess) {
+    delete ctx;
+    return hip_fail(e, "hipGetDeviceProperties");
+  }
+  if (strncmp(ctx->props.gcnArchName, "gfx950", 6) != 0) {
+    int s = fail(HC_ERR_LOAD, "device %d is %s; the embedded kernels are built for gfx950 only", device,
+                 ctx->props.gcnArchName);
+    delete ctx;
+    return s;
+  }
+  e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
+  if (e != hipSuccess) {
+    delete ctx;
+    return hip_fail(e, "hipStreamCreateWithFlags");
+  }
+  int s = load_image(ctx, hc_image_elementwise, hc_image_elementwise_end, "elementwise");
+  if (s == HC_OK) s = load_image(ctx, hc_image_reduce, hc_image_reduce_end, "reduce");
+  if (s == HC_OK) s = load_image(ctx, hc_image_gather, hc_image_gather_end, "gather");
+  if (s == HC_OK) s = load_image(ctx, hc_image_gemm, hc_image_gemm_end, "gemm");
+  if (s != HC_OK) {
+    hc_shutdown(ctx);
+    return s;
+  }
+  *out = ctx;
+  return HC_OK;
+}
+
+extern "C" void hc_shutdown(hc_ctx* ctx) {
+  if (!ctx) return;
+  (void)hipSetDevice(ctx->device);
+  if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+  for (auto& kv : ctx->free_blocks)
+    for (void* p : kv.second) (void)hipFree(p);
+  for (auto& kv : ctx->live) (void)hipFree(kv.first);
+  for (hipModule_t m : ctx->modules) (void)hipModuleUnload(m);
+  if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
+  delete ctx;
+}
+
+extern "C" int hc_get_device_info(hc_ctx* ctx, hc_device_info* out) {
+  REQUIRE(ctx && out, "hc_get_device_info: null argument");
+  memset(out, 0, sizeof(*out));
+  snprintf(out->name, sizeof(out->name), "%s", ctx->props.name);
+  snprintf(out->arch, sizeof(out->arch), "%s", ctx->props.gcnArchName);
+  out->compute_units = ctx->props.multiProcessorCount;
+  out->clock_mhz = ctx->props.clockRate / 1000;
+  out->wavefront_size = ctx->props.warpSize;
+  out->lds_bytes_per_block = (int)ctx->props.sharedMemPerBlock;
+  out->total_mem = ctx->props.totalGlobalMem;
+  return HC_OK;
+}
+
+// ------------------------------------------------------------------ memory
+
+// Bucket sizes: powers of two up to 1 MiB, multiples of 2 MiB above. A freed block goes
+// back to its bucket and is handed out again by a later hc_malloc; both happen in host
+// program order and all work runs on one in-order stream, so a kernel enqueued before the
+// free always finishes before a kernel enqueued after the re-allocation touches the block.
+static size_t bucket_size(size_t bytes) {
+  if (bytes < 256) return 256;
+  if (bytes <= ((size_t)1 << 20)) {
+    size_t b = 256;
+    while (b < bytes) b <<= 1;
+    return b;
+  }
+  const size_t g = (size_t)2 << 20;
+  return (bytes + g - 1) / g * g;
+}
+
+static void release_cache_locked(hc_ctx* ctx) {
+  for (auto& kv : ctx->free_blocks)
+    for (void* p : kv.second) (void)hipFree(p);
+  ctx->free_blocks.clear();
+  ctx->bytes_cached = 0;
+}
+
+extern "C" int hc_malloc(hc_ctx* ctx, size_t bytes, void** out) {
+  REQUIRE(ctx && out, "hc_malloc: null argument");
+  *out = nullptr;
+  const size_t b = bucket_size(bytes);
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  auto it = ctx->free_blocks.find(b);
+  void* p = nullptr;
+  if (it != ctx->free_blocks.end() && !it->second.empty()) {
+    p = it->second.back();
+    it->second.pop_back();
+    ctx->bytes_cached -= b;
+  } else {
+    (void)hipSetDevice(ctx->device);
+    hipError_t e = hipMalloc(&p, b);
+    if (e != hipSuccess) {
+      // Give cached blocks back to the driver and retry once.
+      (void)hipGetLastError();
+      (void)hipStreamSynchronize(ctx->stream);
+      release_cache_locked(ctx);
+      e = hipMalloc(&p, b);
+    }
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      return fail(HC_ERR_ALLOC, "hipMalloc(%zu bytes) failed: %s", b, hipGetErrorString(e));
+    }
+  }
+  ctx->live[p] = b;
+  ctx->bytes_in_use += b;
+  *out = p;
+  return HC_OK;
+}
+
+extern "C" int hc_free(hc_ctx* ctx, void* ptr) {
+  REQUIRE(ctx, "hc_free: null context");
+  if (!ptr) return HC_OK;
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  auto it = ctx->live.find(ptr);
+  REQUIRE(it != ctx->live.end(), "hc_free: %p was not allocated by this context (or freed twice)", ptr);
+  const size_t b = it->second;
+  ctx->live.erase(it);
+  ctx->bytes_in_use -= b;
+  ctx->free_blocks[b].push_back(ptr);
+  ctx->bytes_cached += b;
+  return HC_OK;
+}
+
+extern "C" int hc_trim(hc_ctx* ctx) {
+  REQUIRE(ctx, "hc_trim: null context");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  HIP_TRY(hipStreamSynchronize(ctx->stream));
+  release_cache_locked(ctx);
+  return HC_OK;
+}
+
+extern "C" int hc_mem_stats(hc_ctx* ctx, size_t* in_use, size_t* cached) {
+  REQUIRE(ctx, "hc_mem_stats: null context");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  if (in_use) *in_use = ctx->bytes_in_use;
+  if (cached) *cached = ctx->bytes_cached;
+  return HC_OK;
+}
+
+extern "C" int hc_host_alloc(hc_ctx* ctx, size_t bytes, void** out) {
+  REQUIRE(ctx && out, "hc_host_alloc: null argument");
+  *out = nullptr;
+  hipError_t e = hipHostMalloc(out, bytes ? bytes : 1, hipHostMallocDefault);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    return fail(HC_ERR_ALLOC, "hipHostMalloc(%zu bytes) failed: %s", bytes, hipGetErrorString(e));
+  }
+  return HC_OK;
+}
+
+extern "C" int hc_host_free(hc_ctx* ctx, void* ptr) {
+  REQUIRE(ctx, "hc_host_free: null context");
+  if (ptr) HIP_TRY(hipHostFree(ptr));
+  return HC_OK;
+}
+
+static int copy(hc_ctx* ctx, void* dst, const void* src, size_t bytes, hipMemcpyKind kind, bool wait) {
+  REQUIRE(ctx, "memcpy: null context");
+  if (bytes == 0) return HC_OK;
+  REQUIRE(dst && src, "memcpy: null pointer");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  HIP_TRY(hipMemcpyAsync(dst, src, bytes, kind, ctx->stream));
+  if (wait) HIP_TRY(hipStreamSynchronize(ctx->stream));
+  return HC_OK;
+}
+
+extern "C" int hc_memcpy_h2d(hc_ctx* ctx, void* dst, const void* src, size_t bytes) {
+  return copy(ctx, dst, src, bytes, hipMemcpyHostToDevice, true);
+}
+extern "C" int hc_memcpy_d2h(hc_ctx* ctx, void* dst, const void* src, size_t bytes) {
+  return copy(ctx, dst, src, bytes, hipMemcpyDeviceToHost, true);
+}
+extern "C" int hc_memcpy_d2d(hc_ctx* ctx, void* dst, const void* src, size_t bytes) {
+  return copy(ctx, dst, src, bytes, hipMemcpyDeviceToDevice, false);
+}
+extern "C" int hc_memcpy_h2d_async(hc_ctx* ctx, void* dst, const void* src, size_t bytes) {
+  return copy(ctx, dst, src, bytes, hipMemcpyHostToDevice, false);
+}
+extern "C" int hc_memcpy_d2h_async(hc_ctx* ctx, void* dst, const void* src, size_t bytes) {
+  return copy(ctx, dst, src, bytes, hipMemcpyDeviceToHost, false);
+}
+
+// ------------------------------------------------------------------ stream / events
+
+extern "C" int hc_sync(hc_ctx* ctx) {
+  REQUIRE(ctx, "hc_sync: null context");
+  HIP_TRY(hipStreamSynchronize(ctx->stream));
+  return HC_OK;
+}
+
+extern "C" int hc_event_create(hc_ctx* ctx, hc_event** out) {
+  REQUIRE(ctx && out, "hc_event_create: null argument");
+  hc_event* ev = new hc_event();
+  hipError_t e = hipEventCreate(&ev->ev);
+  if (e != hipSuccess) {
+    delete ev;
+    return hip_fail(e, "hipEventCreate");
+  }
+  *out = ev;
+  return HC_OK;
+}
+
+extern "C" int hc_event_record(hc_ctx* ctx, hc_event* ev) {
+  REQUIRE(ctx && ev, "hc_event_record: null argument");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  HIP_TRY(hipEventRecord(ev->ev, ctx->stream));
+  return HC_OK;
+}
+
+extern "C" int hc_event_sync(hc_event* ev) {
+  REQUIRE(ev, "hc_event_sync: null event");
+  HIP_TRY(hipEventSynchronize(ev->ev));
+  return HC_OK;
+}
+
+extern "C" int hc_event_query(hc_event* ev) {
+  REQUIRE(ev, "hc_event_query: null event");
+  hipError_t e = hipEventQuery(ev->ev);
+  if (e == hipSuccess) return 0;
+  if (e == hipErrorNotReady) {
+    (void)hipGetLastError();
+    return 1;
+  }
+  return hip_fail(e, "hipEventQuery");
+}
+
+extern "C" int hc_event_elapsed_ms(hc_event* start, hc_event* stop, float* ms) {
+  REQUIRE(start && stop && ms, "hc_event_elapsed_ms: null argument");
+  HIP_TRY(hipEventElapsedTime(ms, start->ev, stop->ev));
+  return HC_OK;
+}
+
+extern "C" int hc_event_destroy(hc_event* ev) {
+  if (!ev) return HC_OK;
+  hipError_t e = hipEventDestroy(ev->ev);
+  delete ev;
+  if (e != hipSuccess) return hip_fail(e, "hipEventDestroy");
+  return HC_OK;
+}
+
+extern "C" int hc_launch_host_func(hc_ctx* ctx, void (*fn)(void*), void* user) {
+  REQUIRE(ctx && fn, "hc_launch_host_func: null argument");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  HIP_TRY(hipLaunchHostFunc(ctx->stream, fn, user));
+  return HC_OK;
+}
+
+// ------------------------------------------------------------------ raw module API
+
+extern "C" int hc_module_load(hc_ctx* ctx, const void* image, size_t bytes, hc_module** out) {
+  REQUIRE(ctx && image && out && bytes > 0, "hc_module_load: bad argument");
+  hipModule_t mod;
+  hipError_t e = hipModuleLoadData(&mod, image);
+  if (e != hipSuccess) return fail(HC_ERR_LOAD, "hipModuleLoadData: %s", hipGetErrorString(e));
+  *out = new hc_module{mod};
+  return HC_OK;
+}
+
+extern "C" int hc_module_unload(hc_ctx* ctx, hc_module* mod) {
+  REQUIRE(ctx && mod, "hc_module_unload: null argument");
+  hipError_t e = hipModuleUnload(mod->mod);
+  delete mod;
+  if (e != hipSuccess) return hip_fail(e, "hipModuleUnload");
+  return HC_OK;
+}
+
+extern "C" int hc_module_get_function(hc_module* mod, const char* name, hc_function** out) {
+  REQUIRE(mod && name && out, "hc_module_get_function: null argument");
+  hipFunction_t fn;
+  hipError_t e = hipModuleGetFunction(&fn, mod->mod, name);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    return fail(HC_ERR_LOAD, "kernel '%s' not found: %s", name, hipGetErrorString(e));
+  }
+  *out = new hc_function{fn};  // lives as long as the module; a few bytes, never freed
+  return HC_OK;
+}
+
+static int launch_fn(hc_ctx* ctx, hipFunction_t fn, uint32_t gx, uint32_t gy, uint32_t gz, uint32_t bx,
+                     uint32_t shared, const void* kernarg, size_t kernarg_bytes) {
+  void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, const_cast<void*>(kernarg),
+                    HIP_LAUNCH_PARAM_BUFFER_SIZE, &kernarg_bytes, HIP_LAUNCH_PARAM_END};
+  HIP_TRY(hipModuleLaunchKernel(fn, gx, gy, gz, bx, 1, 1, shared, ctx->stream, nullptr, config));
+  return HC_OK;
+}
+
+extern "C" int hc_launch(hc_ctx* ctx, hc_function* fn, const uint32_t grid[3], const uint32_t block[3],
+                         uint32_t shared_bytes, const void* kernarg, size_t kernarg_bytes) {
+  REQUIRE(ctx && fn && grid && block, "hc_launch: null argument");
+  void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, const_cast<void*>(kernarg),
+                    HIP_LAUNCH_PARAM_BUFFER_SIZE, &kernarg_bytes, HIP_LAUNCH_PARAM_END};
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  HIP_TRY(hipModuleLaunchKernel(fn->fn, grid[0], grid[1], grid[2], block[0], block[1], block[2],
+                                shared_bytes, ctx->stream, nullptr, config));
+  return HC_OK;
+}
+
+// Look a kernel up by name in the embedded code objects (cached) and launch it with a
+// 256-lane block.
+static int launch(hc_ctx* ctx, const std::string& name, uint64_t blocks_x, uint32_t blocks_y,
+                  const void* args, size_t bytes) {
+  if (blocks_x == 0 || blocks_y == 0) return HC_OK;
+  if (blocks_x > 0x7fffffffull)
+    return fail(HC_ERR_TOO_LARGE, "%s: grid of %llu blocks exceeds the launch limit", name.c_str(),
+                (unsigned long long)blocks_x);
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  hipFunction_t fn = nullptr;
+  auto it = ctx->functions.find(name);
+  if (it != ctx->functions.end()) {
+    fn = it->second;
+  } else {
+    for (hipModule_t m : ctx->modules) {
+      if (hipModuleGetFunction(&fn, m, name.c_str()) == hipSuccess) break;
+      (void)hipGetLastError();
+      fn = nullptr;
+    }
+    if (!fn) return fail(HC_ERR_LOAD, "kernel '%s' is not in the embedded code objects", name.c_str());
+    ctx->functions[name] = fn;
+  }
+  return launch_fn(ctx, fn, (uint32_t)blocks_x, blocks_y, 1, HCK_BLOCK, 0, args, bytes);
+}
+
+static inline uint64_t ceil_div(uint64_t a, uint64_t b) { return (a + b - 1) / b; }
+
+// ------------------------------------------------------------------ descriptors
+
+static const char* dtype_name(int dtype) {
+  switch (dtype) {
+    case HC_I64: return "i64";
+    case HC_BOOL: return "b8";
+    case HC_F16: return "f16";
+    case HC_F32: return "f32";
+    default: return nullptr;
+  }
+}
+
+static size_t dtype_size(int dtype) {
+  switch (dtype) {
+    case HC_I64: return 8;
+    case HC_BOOL: return 1;
+    case HC_F16: return 2;
+    default: return 4;
+  }
+}
+
+static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
+// Build the joint broadcast descriptor for `nops` operands over one virtual shape:
+// drop size-1 axes, merge axes that are jointly mergeable (stride[d] == stride[d+1] *
+// shape[d+1] for every operand, which also merges runs of broadcast axes), split the
+// innermost axis off and pick the vector width. `vec_max` is the widest vector allowed
+// (elements); `ptrs` are checked for 16-byte alignment. *total receives the element count.
+static int make_bcast(int nops, const hc_strides* const* ops, const void* const* ptrs, const void* out,
+                      int vec_max, hck_bcast* d, int* vec, uint64_t* total) {
+  const hc_strides* s0 = ops[0];
+  REQUIRE(s0->ndim <= HC_MAX_DIMS, "strides: ndim %u exceeds %d", s0->ndim, HC_MAX_DIMS);
+  for (int o = 1; o < nops; o++) {
+    REQUIRE(ops[o]->ndim == s0->ndim, "strides: operand ranks differ (%u vs %u)", ops[o]->ndim, s0->ndim);
+    for (uint32_t k = 0; k < s0->ndim; k++)
+      REQUIRE(ops[o]->shape[k] == s0->shape[k], "strides: operand shapes differ on axis %u", k);
+  }
+  int64_t shape[HC_MAX_DIMS];
+  int64_t stride[3][HC_MAX_DIMS];
+  int n = 0;
+  uint64_t count = 1;
+  for (uint32_t k = 0; k < s0->ndim; k++) {
+    REQUIRE(s0->shape[k] >= 0, "strides: negative extent on axis %u", k);
+    count *= (uint64_t)s0->shape[k];
+  }
+  *total = count;
+  memset(d, 0, sizeof(*d));
+  *vec = 1;
+  if (count == 0) return HC_OK;
+  if (count > 0xffffffffull)
+    return fail(HC_ERR_TOO_LARGE, "broadcast op over %llu elements exceeds the 32-bit index range",
+                (unsigned long long)count);
+  for (uint32_t k = 0; k < s0->ndim; k++) {
+    if (s0->shape[k] == 1) continue;
+    shape[n] = s0->shape[k];
+    for (int o = 0; o < nops; o++) {
+      REQUIRE(ops[o]->strides[k] >= 0 && ops[o]->strides[k] <= 0xffffffffll,
+              "strides: stride %lld on axis %u is out of range", (long long)ops[o]->strides[k], k);
+      stride[o][n] = ops[o]->strides[k];
+    }
+    n++;
+  }
+  // merge from the inside out
+  int m = 0;
+  int64_t mshape[HC_MAX_DIMS];
+  int64_t mstride[3][HC_MAX_DIMS];
+  for (int k = n - 1; k >= 0; k--) {
+    bool merge = m > 0;
+    if (merge)
+      for (int o = 0; o < nops; o++)
+        if (stride[o][k] != mstride[o][m - 1] * mshape[m - 1]) merge = false;
+    if (merge) {
+      mshape[m - 1] *= shape[k];  // strides of the inner axis stay
+    } else {
+      mshape[m] = shape[k];
+      for (int o = 0; o < nops; o++) mstride[o][m] = stride[o][k];
+      m++;
+    }
+  }
+  // mshape[0] is now the innermost axis; it must have stride 0 or 1 for every operand to
+  // be the vector axis, otherwise a unit inner axis is prepended.
+  bool inner_ok = m > 0;
+  if (inner_ok)
+    for (int o = 0; o < nops; o++)
+      if (mstride[o][0] != 0 && mstride[o][0] != 1) inner_ok = false;
+  int first_outer = 0;
+  if (inner_ok) {
+    d->inner = (uint32_t)mshape[0];
+    for (int o = 0; o < nops; o++) d->inner_stride[o] = (uint32_t)mstride[o][0];
+    first_outer = 1;
+  } else {
+    d->inner = 1;
+    for (int o = 0; o < nops; o++) d->inner_stride[o] = 0;
+  }
+  d->n_outer = (uint32_t)(m - first_outer);
+  if (d->n_outer > HCK_MAX_DIMS - 1)
+    return fail(HC_ERR_UNSUPPORTED, "strides: %d non-mergeable axes with a strided innermost axis", m);
+  // outer axes are stored outermost-first (the kernel peels them from the back)
+  for (int k = first_outer; k < m; k++) {
+    const int dst = m - 1 - k;
+    d->outer_shape[dst] = (uint32_t)mshape[k];
+    for (int o = 0; o < nops; o++) d->outer_stride[o][dst] = (uint32_t)mstride[o][k];
+  }
+  int v = vec_max;
+  if (d->inner % (uint32_t)v != 0 || !aligned16(out)) v = 1;
+  for (int o = 0; o < nops && v > 1; o++) {
+    if (!aligned16(ptrs[o])) v = 1;
+    if (d->inner_stride[o] == 1)
+      for (uint32_t k = 0; k < d->n_outer; k++)
+        if (d->outer_stride[o][k] % (uint32_t)v != 0) v = 1;
+  }
+  *vec = v;
+  d->inner_vecs = d->inner / (uint32_t)v;
+  d->total_vecs = (uint32_t)(count / (uint64_t)v);
+  return HC_OK;
+}
+
+static int vec_for_size(size_t el) { return (int)(16 / el); }
+
+// ------------------------------------------------------------------ element-wise ops
+
+static const char* const kBinaryNames[] = {"add", "mul", "sub", "div", "mod"};
+static const char* const kCompareNames[] = {"eq", "ne", "lt", "le", "gt", "ge"};
+
+extern "C" int hc_broadcast(hc_ctx* ctx, int dtype, const void* a, const hc_strides* as, void* out) {
+  REQUIRE(ctx && a && as && out, "hc_broadcast: null argument");
+  REQUIRE(dtype_name(dtype), "hc_broadcast: bad dtype %d", dtype);
+  const size_t el = dtype_size(dtype);
+  hck_binary_args k;
+  memset(&k, 0, sizeof(k));
+  int vec;
+  uint64_t total;
+  const hc_strides* ops[] = {as};
+  const void* ptrs[] = {a};
+  HC_TRY(make_bcast(1, ops, ptrs, out, vec_for_size(el), &k.d, &vec, &total));
+  if (total == 0) return HC_OK;
+  k.a = a;
+  k.out = out;
+  char name[64];
+  snprintf(name, sizeof(name), "hc_broadcast_b%zu_v%d", el, vec);
+  return launch(ctx, name, ceil_div(k.d.total_vecs, HCK_BLOCK), 1, &k, sizeof(k));
+}
+
+extern "C" int hc_binary_op(hc_ctx* ctx, int op, int dtype, const void* a, const hc_strides* as,
+                            const void* b, const hc_strides* bs, void* out) {
+  REQUIRE(ctx && a && as && b && bs && out, "hc_binary_op: null argument");
+  REQUIRE(op >= HC_ADD && op <= HC_MOD, "hc_binary_op: bad op %d", op);
+  if (dtype != HC_F32 && dtype != HC_F16 && dtype != HC_I64)
+    return fail(HC_ERR_UNSUPPORTED, "hc_binary_op: dtype %d is not numeric", dtype);
+  hck_binary_args k;
+  memset(&k, 0, sizeof(k));
+  int vec;
+  uint64_t total;
+  const hc_strides* ops[] = {as, bs};
+  const void* ptrs[] = {a, b};
+  HC_TRY(make_bcast(2, ops, ptrs, out, vec_for_size(dtype_size(dtype)), &k.d, &vec, &total));
+  if (total == 0) return HC_OK;
+  k.a = a;
+  k.b = b;
+  k.out = out;
+  char name[64];
+  snprintf(name, sizeof(name), "hc_binary_%s_%s_v%d", kBinaryNames[op], dtype_name(dtype), vec);
+  return launch(ctx, name, ceil_div(k.d.total_vecs, HCK_BLOCK), 1, &k, sizeof(k));
+}
+
+extern "C" int hc_compare(hc_ctx* ctx, int op, int dtype, const void* a, const hc_strides* as,
+                          const void* b, const hc_strides* bs, void* out) {
+  REQUIRE(ctx && a && as && b && bs && out, "hc_compare: null argument");
+  REQUIRE(op >= HC_EQ && op <= HC_GE, "hc_compare: bad op %d", op);
+  REQUIRE(dtype_name(dtype), "hc_compare: bad dtype %d", dtype);
+  hck_binary_args k;
+  memset(&k, 0, sizeof(k));
+  int vec;
+  uint64_t total;
+  const hc_strides* ops[] = {as, bs};
+  const void* ptrs[] = {a, b};
+  HC_TRY(make_bcast(2, ops, ptrs, out, vec_for_size(dtype_size(dtype)), &k.d, &vec, &total));
+  if (total == 0) return HC_OK;
+  k.a = a;
+  k.b = b;
+  k.out = out;
+  char name[64];
+  snprintf(name, sizeof(name), "hc_compare_%s_%s_v%d", kCompareNames[op], dtype_name(dtype), vec);
+  return launch(ctx, name, ceil_div(k.d.total_vecs, HCK_BLOCK), 1, &k, sizeof(k));
+}
+
+static int fused3(hc_ctx* ctx, const char* kernel, int dtype, const void* x, const hc_strides* xs,
+                  const void* y, const hc_strides* ys, const void* z, const hc_strides* zs, void* out,
+                  size_t el, const char* tname) {
+  hck_ternary_args k;
+  memset(&k, 0, sizeof(k));
+  int vec;
+  uint64_t total;
+  const hc_strides* ops[] = {xs, ys, zs};
+  const void* ptrs[] = {x, y, z};
+  (void)dtype;
+  HC_TRY(make_bcast(3, ops, ptrs, out, vec_for_size(el), &k.d, &vec, &total));
+  if (total == 0) return HC_OK;
+  k.x = x;
+  k.y = y;
+  k.z = z;
+  k.out = out;
+  char name[64];
+  snprintf(name, sizeof(name), "%s_%s_v%d", kernel, tname, vec);
+  return launch(ctx, name, ceil_div(k.d.total_vecs, HCK_BLOCK), 1, &k, sizeof(k));
+}
+
+extern "C" int hc_mul_add(hc_ctx* ctx, int dtype, const void* input, const hc_strides* is,
+                          const void* coeff, const hc_strides* cs, const void* bias,
+                          const hc_strides* bs, void* out) {
+  REQUIRE(ctx && input && is && coeff && cs && bias && bs && out, "hc_mul_add: null argument");
+  if (dtype != HC_F32 && dtype != HC_F16 && dtype != HC_I64)
+    return fail(HC_ERR_UNSUPPORTED, "hc_mul_add: dtype %d is not numeric", dtype);
+  return fused3(ctx, "hc_mul_add", dtype, input, is, coeff, cs, bias, bs, out, dtype_size(dtype),
+                dtype_name(dtype));
+}
+
+extern "C" int hc_add_mul(hc_ctx* ctx, int dtype, const void* input, const hc_strides* is,
+                          const void* bias, const hc_strides* bs, const void* coeff,
+                          const hc_strides* cs, void* out) {
+  REQUIRE(ctx && input && is && coeff && cs && bias && bs && out, "hc_add_mul: null argument");
+  if (dtype != HC_F32 && dtype != HC_F16 && dtype != HC_I64)
+    return fail(HC_ERR_UNSUPPORTED, "hc_add_mul: dtype %d is not numeric", dtype);
+  return fused3(ctx, "hc_add_mul", dtype, input, is, coeff, cs, bias, bs, out, dtype_size(dtype),
+                dtype_name(dtype));
+}
+
+extern "C" int hc_when(hc_ctx* ctx, int dtype, const void* mask, const hc_strides* ms, const void* a,
+                       const hc_strides* as, const void* b, const hc_strides* bs, void* out) {
+  REQUIRE(ctx && mask && ms && a && as && b && bs && out, "hc_when: null argument");
+  REQUIRE(dtype_name(dtype), "hc_when: bad dtype %d", dtype);
+  const size_t el = dtype_size(dtype);
+  char tname[8];
+  snprintf(tname, sizeof(tname), "b%zu", el);
+  return fused3(ctx, "hc_when", dtype, mask, ms, a, as, b, bs, out, el, tname);
+}
+
+static int launch_contiguous(hc_ctx* ctx, const char* name, size_t count, int vec, const void* args,
+                             size_t bytes) {
+  if (count == 0) return HC_OK;
+  // one vector per lane; the ragged tail (< vec elements) rides on block 0
+  const uint64_t lanes = count / (uint64_t)vec ? count / (uint64_t)vec : 1;
+  return launch(ctx, name, ceil_div(lanes, HCK_BLOCK), 1, args, bytes);
+}
+
+extern "C" int hc_binary_op_scalar(hc_ctx* ctx, int op, int dtype, const void* a, float sf,
+                                   int64_t si, int scalar_first, void* out, size_t count) {
+  REQUIRE(ctx, "hc_binary_op_scalar: null context");
+  REQUIRE(op >= HC_ADD && op <= HC_MOD, "hc_binary_op_scalar: bad op %d", op);
+  if (dtype != HC_F32 && dtype != HC_F16 && dtype != HC_I64)
+    return fail(HC_ERR_UNSUPPORTED, "hc_binary_op_scalar: dtype %d is not numeric", dtype);
+  if (count == 0) return HC_OK;
+  REQUIRE(a && out, "hc_binary_op_scalar: null pointer");
+  REQUIRE(aligned16(a) && aligned16(out), "hc_binary_op_scalar: buffers must be 16-byte aligned");
+  hck_scalar_args k;
+  memset(&k, 0, sizeof(k));
+  k.in = a;
+  k.out = out;
+  k.count = count;
+  k.sf = sf;
+  k.si = si;
+  const char* kop = kBinaryNames[op];
+  if (dtype == HC_F32) {
+    // The CPU's vDSP forms (BackendCPU.swift:325-342, 366-389).
+    if (!scalar_first) {
+      if (op == HC_DIV) {
+        k.sf = 1.0f / sf;
+        kop = "mul";
+      } else if (op == HC_SUB) {
+        k.sf = -sf;
+        kop = "add";
+      }
+    } else {
+      if (op == HC_DIV) kop = "rdiv";
+      else if (op == HC_SUB) kop = "rsubf";
+      else if (op == HC_MOD) kop = "rmod";
+    }
+  } else if (scalar_first) {
+    if (op == HC_DIV) kop = "rdiv";
+    else if (op == HC_SUB) kop = "rsub";
+    else if (op == HC_MOD) kop = "rmod";
+  }
+  char name[64];
+  snprintf(name, sizeof(name), "hc_scalar_%s_%s", kop, dtype_name(dtype));
+  return launch_contiguous(ctx, name, count, vec_for_size(dtype_size(dtype)), &k, sizeof(k));
+}
+
+extern "C" int hc_compare_scalar(hc_ctx* ctx, int op, int dtype, const void* a, float sf, int64_t si,
+                                 int scalar_first, void* out, size_t count) {
+  REQUIRE(ctx, "hc_compare_scalar: null context");
+  REQUIRE(op >= HC_EQ && op <= HC_GE, "hc_compare_scalar: bad op %d", op);
+  REQUIRE(dtype_name(dtype), "hc_compare_scalar: bad dtype %d", dtype);
+  if (count == 0) return HC_OK;
+  REQUIRE(a && out, "hc_compare_scalar: null pointer");
+  REQUIRE(aligned16(a) && aligned16(out), "hc_compare_scalar: buffers must be 16-byte aligned");
+  hck_scalar_args k;
+  memset(&k, 0, sizeof(k));
+  k.in = a;
+  k.out = out;
+  k.count = count;
+  k.sf = sf;
+  k.si = si;
+  char name[64];
+  snprintf(name, sizeof(name), "hc_cmps_%s%s_%s", scalar_first ? "r" : "", kCompareNames[op],
+           dtype_name(dtype));
+  const int vec = vec_for_size(dtype_size(dtype));
+  return launch_contiguous(ctx, name, count, vec > 16 ? 16 : vec, &k, sizeof(k));
+}
+
+extern "C" int hc_cast(hc_ctx* ctx, const void* in, int in_type, void* out, int out_type, size_t count) {
+  REQUIRE(ctx, "hc_cast: null context");
+  REQUIRE(dtype_name(in_type) && dtype_name(out_type), "hc_cast: bad dtype %d -> %d", in_type, out_type);
+  if (count == 0) return HC_OK;
+  REQUIRE(in && out, "hc_cast: null pointer");
+  if (in_type == out_type) return hc_memcpy_d2d(ctx, out, in, count * dtype_size(in_type));
+  REQUIRE(aligned16(in) && aligned16(out), "hc_cast: buffers must be 16-byte aligned");
+  hck_map_args k;
+  memset(&k, 0, sizeof(k));
+  k.in = in;
+  k.out = out;
+  k.count = count;
+  char name[64];
+  snprintf(name, sizeof(name), "hc_cast_%s_%s", dtype_name(in_type), dtype_name(out_type));
+  const int vi = vec_for_size(dtype_size(in_type)), vo = vec_for_size(dtype_size(out_type));
+  return launch_contiguous(ctx, name, count, vi < vo ? vi : vo, &k, sizeof(k));
+}
+
+extern "C" int hc_pow(hc_ctx* ctx, int dtype, const void* in, float bf, float scalef, int64_t bi,
+                      int64_t scalei, const void* scales, void* out, size_t count) {
+  REQUIRE(ctx, "hc_pow: null context");
+  if (dtype != HC_F32 && dtype != HC_F16 && dtype != HC_I64)
+    return fail(HC_ERR_UNSUPPORTED, "hc_pow: dtype %d is not numeric", dtype);
+  if (count == 0) return HC_OK;
+  REQUIRE(in && out, "hc_pow: null pointer");
+  REQUIRE(aligned16(in) && aligned16(out), "hc_pow: buffers must be 16-byte aligned");
+  hck_map_args k;
+  memset(&k, 0, sizeof(k));
+  k.in = in;
+  k.scales = scales;
+  k.out = out;
+  k.count = count;
+  k.p0 = bf;
+  k.p1 = scalef;
+  k.i0 = bi;
+  k.i1 = scalei;
+  const char* mode = "generic";
+  if (dtype == HC_F32) {
+    if (bf == 2.0f) mode = "square";
+    else if (bf == -1.0f) mode = "recip";
+    else if (bf == 1.0f) mode = "linear";
+  }
+  char name[64];
+  snprintf(name, sizeof(name), "hc_pow_%s_%s", mode, dtype_name(dtype));
+  return launch_contiguous(ctx, name, count, vec_for_size(dtype_size(dtype)), &k, sizeof(k));
+}
+
+static const char* const kElemwiseNames[HC_ELEMWISE_COUNT] = {
+    "sin", "cos", "minus_sin", "tan", "tan_grad", "atan", "atan_grad", "acos", "acos_grad", "asin",
+    "asin_grad", "exp", "log", "recip", "sigmoid", "sigmoid_grad", "relu", "relu_grad", "abs",
+    "abs_grad", "gelu_approx", "gelu_approx_grad", "gelu_exact", "gelu_exact_grad", "erf", "erf_grad",
+    "floor", "ceil", "round"};
+
+extern "C" int hc_elemwise(hc_ctx* ctx, int op, int dtype, const void* in, const void* scales,
+                           void* out, size_t count) {
+  REQUIRE(ctx, "hc_elemwise: null context");
+  REQUIRE(op >= 0 && op < HC_ELEMWISE_COUNT, "hc_elemwise: bad op %d", op);
+  if (dtype != HC_F32 && dtype != HC_F16)
+    return fail(HC_ERR_UNSUPPORTED, "hc_elemwise: dtype %d is not a float type", dtype);
+  if (count == 0) return HC_OK;
+  REQUIRE(in && out, "hc_elemwise: null pointer");
+  REQUIRE(aligned16(in) && aligned16(out), "hc_elemwise: buffers must be 16-byte aligned");
+  hck_map_args k;
+  memset(&k, 0, sizeof(k));
+  k.in = in;
+  k.scales = scales;
+  k.out = out;
+  k.count = count;
+  char name[64];
+  snprintf(name, sizeof(name), "hc_elemwise_%s_%s", kElemwiseNames[op], dtype_name(dtype));
+  return launch_contiguous(ctx, name, count, vec_for_size(dtype_size(dtype)), &k, sizeof(k));
+}
+
+static uint16_t f32_to_f16_bits(float f) {
+  // IEEE binary32 -> binary16, round-to-nearest-even, overflow to inf (host-side, for fill).
+  uint32_t x;
+  memcpy(&x, &f, 4);
+  const uint32_t sign = (x >> 16) & 0x8000u, absx = x & 0x7fffffffu;
+  if (absx >= 0x7f800000u) return (uint16_t)(sign | (absx > 0x7f800000u ? 0x7e00u : 0x7c00u));
+  if (absx >= 0x477ff000u) return (uint16_t)(sign | 0x7c00u);
+  if (absx < 0x38800000u) {
+    if (absx < 0x33000000u) return (uint16_t)sign;
+    const int shift = 126 - (int)(absx >> 23);
+    const uint32_t mant = (absx & 0x7fffffu) | 0x800000u;
+    uint32_t res = mant >> shift;
+    const uint32_t rem = mant & ((1u << shift) - 1u), half = 1u << (shift - 1);
+    if (rem > half || (rem == half && (res & 1u))) res++;
+    return (uint16_t)(sign | res);
+  }
+  uint32_t res = (((absx >> 23) - 112u) << 10) | ((absx & 0x7fffffu) >> 13);
+  const uint32_t rem = absx & 0x1fffu;
+  if (rem > 0x1000u || (rem == 0x1000u && (res & 1u))) res++;
+  return (uint16_t)(sign | res);
+}
+
+extern "C" int hc_fill(hc_ctx* ctx, int dtype, float vf, int64_t vi, void* out, size_t count) {
+  REQUIRE(ctx, "hc_fill: null context");
+  REQUIRE(dtype_name(dtype), "hc_fill: bad dtype %d", dtype);
+  if (count == 0) return HC_OK;
+  REQUIRE(out, "hc_fill: null pointer");
+  REQUIRE(aligned16(out), "hc_fill: buffer must be 16-byte aligned");
+  hck_map_args k;
+  memset(&k, 0, sizeof(k));
+  k.out = out;
+  k.count = count;
+  switch (dtype) {
+    case HC_I64: k.i0 = vi; break;
+    case HC_BOOL: k.i0 = vf == 0 ? 0 : 1; break;
+    case HC_F16: k.i0 = f32_to_f16_bits(vf); break;
+    default: {
+      uint32_t bits;
+      memcpy(&bits, &vf, 4);
+      k.i0 = bits;
+    }
+  }
+  const size_t el = dtype_size(dtype);
+  char name[64];
+  snprintf(name, sizeof(name), "hc_fill_b%zu", el);
+  return launch_contiguous(ctx, name, count, vec_for_size(el), &k, sizeof(k));
+}
+
+// ------------------------------------------------------------------ reductions
+
+static const char* const kReduceNames[] = {"sum", "prod", "argmax", "argmin"};
+
+static int check_dims(const char* who, int64_t outer, int64_t reduce, int64_t inner) {
+  REQUIRE(outer >= 0 && reduce >= 0 && inner >= 0, "%s: negative dimension", who);
+  if ((uint64_t)outer > 0xffffffffull || (uint64_t)reduce > 0xffffffffull || (uint64_t)inner > 0xffffffffull ||
+      (double)outer * (double)reduce * (double)inner > 4294967295.0)
+    return fail(HC_ERR_TOO_LARGE, "%s: [%lld, %lld, %lld] exceeds the 32-bit index range", who,
+                (long long)outer, (long long)reduce, (long long)inner);
+  return HC_OK;
+}
+
+extern "C" int hc_reduce(hc_ctx* ctx, int op, int dtype, const void* in, void* out, int64_t outer,
+                         int64_t reduce, int64_t inner) {
+  REQUIRE(ctx, "hc_reduce: null context");
+  REQUIRE(op >= HC_SUM && op <= HC_ARGMIN, "hc_reduce: bad op %d", op);
+  if (dtype != HC_F32 && dtype != HC_F16 && dtype != HC_I64)
+    return fail(HC_ERR_UNSUPPORTED, "hc_reduce: dtype %d is not numeric", dtype);
+  HC_TRY(check_dims("hc_reduce", outer, reduce, inner));
+  if (outer * inner == 0) return HC_OK;
+  REQUIRE(out, "hc_reduce: null output");
+  REQUIRE(reduce > 0 || op == HC_SUM || op == HC_PROD, "hc_reduce: arg-reduction over an empty axis");
+  REQUIRE(in || reduce == 0, "hc_reduce: null input");
+  hck_reduce_args k;
+  memset(&k, 0, sizeof(k));
+  k.in = in;
+  k.out = out;
+  k.outer = (uint32_t)outer;
+  k.reduce = (uint32_t)reduce;
+  k.inner = (uint32_t)inner;
+  char name[64];
+  if (inner == 1) {
+    const bool vec_ok = aligned16(in);
+    REQUIRE(vec_ok, "hc_reduce: input must be 16-byte aligned");
+    if (reduce <= 1024) {
+      snprintf(name, sizeof(name), "hc_reduce_rows64_%s_%s", kReduceNames[op], dtype_name(dtype));
+      return launch(ctx, name, ceil_div((uint64_t)outer, HCK_BLOCK / 64), 1, &k, sizeof(k));
+    }
+    snprintf(name, sizeof(name), "hc_reduce_rows256_%s_%s", kReduceNames[op], dtype_name(dtype));
+    return launch(ctx, name, (uint64_t)outer, 1, &k, sizeof(k));
+  }
+  snprintf(name, sizeof(name), "hc_reduce_cols_%s_%s", kReduceNames[op], dtype_name(dtype));
+  return launch(ctx, name, ceil_div((uint64_t)inner, 64) * (uint64_t)outer, 1, &k, sizeof(k));
+}
+
+extern "C" int hc_log_softmax(hc_ctx* ctx, int dtype, const void* in, void* out, int64_t outer,
+                              int64_t reduce, int64_t inner) {
+  REQUIRE(ctx, "hc_log_softmax: null context");
+  if (dtype != HC_F32 && dtype != HC_F16)
+    return fail(HC_ERR_UNSUPPORTED, "hc_log_softmax: dtype %d is not a float type", dtype);
+  HC_TRY(check_dims("hc_log_softmax", outer, reduce, inner));
+  if (outer * reduce * inner == 0) return HC_OK;
+  REQUIRE(in && out, "hc_log_softmax: null pointer");
+  hck_reduce_args k;
+  memset(&k, 0, sizeof(k));
+  k.in = in;
+  k.out = out;
+  k.outer = (uint32_t)outer;
+  k.reduce = (uint32_t)reduce;
+  k.inner = (uint32_t)inner;
+  char name[64];
+  if (inner == 1) {
+    snprintf(name, sizeof(name), "hc_log_softmax_rows_%s", dtype_name(dtype));
+    return launch(ctx, name, ceil_div((uint64_t)outer, HCK_BLOCK / 64), 1, &k, sizeof(k));
+  }
+  snprintf(name, sizeof(name), "hc_log_softmax_cols_%s", dtype_name(dtype));
+  return launch(ctx, name, ceil_div((uint64_t)inner, HCK_BLOCK) * (uint64_t)outer, 1, &k, sizeof(k));
+}
+
+struct Scratch {
+  hc_ctx* ctx;
+  std::vector<void*> ptrs;
+  explicit Scratch(hc_ctx* c) : ctx(c) {}
+  ~Scratch() {
+    for (void* p : ptrs) (void)hc_free(ctx, p);
+  }
+  int get(size_t bytes, void** out) {
+    int s = hc_malloc(ctx, bytes, out);
+    if (s == HC_OK) ptrs.push_back(*out);
+    return s;
+  }
+};
+
+extern "C" int hc_normalize(hc_ctx* ctx, int dtype, const void* in, void* out, int64_t outer,
+                            int64_t reduce, int64_t inner, float eps) {
+  REQUIRE(ctx, "hc_normalize: null context");
+  if (dtype != HC_F32 && dtype != HC_F16)
+    return fail(HC_ERR_UNSUPPORTED, "hc_normalize: dtype %d is not a float type", dtype);
+  HC_TRY(check_dims("hc_normalize", outer, reduce, inner));
+  if (outer * reduce * inner == 0) return HC_OK;
+  REQUIRE(in && out, "hc_normalize: null pointer");
+  if (inner == 1) {
+    hck_reduce_args k;
+    memset(&k, 0, sizeof(k));
+    k.in = in;
+    k.out = out;
+    k.outer = (uint32_t)outer;
+    k.reduce = (uint32_t)reduce;
+    k.inner = 1;
+    k.eps = eps;
+    char name[64];
+    snprintf(name, sizeof(name), "hc_normalize_rows_%s", dtype_name(dtype));
+    return launch(ctx, name, ceil_div((uint64_t)outer, HCK_BLOCK / 64), 1, &k, sizeof(k));
+  }
+  // inner > 1: the same composition the base class runs (Backend.swift:265-327), on device.
+  const size_t el = dtype_size(dtype);
+  const size_t full = (size_t)(outer * reduce * inner), red = (size_t)(outer * inner);
+  hc_strides fs = {3, 0, {outer, reduce, inner}, {reduce * inner, inner, 1}};
+  hc_strides rs = {3, 0, {outer, reduce, inner}, {inner, 0, 1}};
+  Scratch scratch(ctx);
+  void *t_red, *mean, *centered, *sq, *var, *norm;
+  HC_TRY(scratch.get(red * el, &t_red));
+  HC_TRY(scratch.get(red * el, &mean));
+  HC_TRY(scratch.get(full * el, &centered));
+  HC_TRY(scratch.get(full * el, &sq));
+  HC_TRY(scratch.get(red * el, &var));
+  HC_TRY(scratch.get(red * el, &norm));
+  const float inv_n = 1.0f / (float)reduce;
+  HC_TRY(hc_reduce(ctx, HC_SUM, dtype, in, t_red, outer, reduce, inner));
+  HC_TRY(hc_binary_op_scalar(ctx, HC_MUL, dtype, t_red, inv_n, 0, 0, mean, red));
+  HC_TRY(hc_binary_op(ctx, HC_SUB, dtype, in, &fs, mean, &rs, centered));
+  HC_TRY(hc_pow(ctx, dtype, centered, 2.0f, 1.0f, 2, 1, nullptr, sq, full));
+  HC_TRY(hc_reduce(ctx, HC_SUM, dtype, sq, t_red, outer, reduce, inner));
+  HC_TRY(hc_binary_op_scalar(ctx, HC_MUL, dtype, t_red, inv_n, 0, 0, var, red));
+  HC_TRY(hc_binary_op_scalar(ctx, HC_ADD, dtype, var, eps, 0, 0, t_red, red));
+  HC_TRY(hc_pow(ctx, dtype, t_red, -0.5f, 1.0f, 0, 1, nullptr, norm, red));
+  HC_TRY(hc_binary_op(ctx, HC_MUL, dtype, centered, &fs, norm, &rs, out));
+  return HC_OK;
+}
+
+// ------------------------------------------------------------------ gather & friends
+
+extern "C" int hc_gather(hc_ctx* ctx, int dtype, const void* in, const void* indices,
+                         const hc_strides* idx_strides, void* out, int64_t outer, int64_t middle,
+                         int64_t out_count, int64_t inner) {
+  REQUIRE(ctx && idx_strides, "hc_gather: null argument");
+  REQUIRE(dtype_name(dtype), "hc_gather: bad dtype %d", dtype);
+  REQUIRE(outer >= 0 && middle >= 0 && out_count >= 0 && inner >= 0, "hc_gather: negative dimension");
+  const double out_total = (double)outer * (double)out_count * (double)inner;
+  const double in_total = (double)outer * (double)middle * (double)inner;
+  if (out_total == 0) return HC_OK;
+  if (out_total > 4294967295.0 || in_total > 4294967295.0)
+    return fail(HC_ERR_TOO_LARGE, "hc_gather: more than 2^32-1 elements");
+  REQUIRE(in && indices && out, "hc_gather: null pointer");
+  const uint64_t total = (uint64_t)outer * (uint64_t)out_count * (uint64_t)inner;
+  {
+    uint64_t n = 1;
+    REQUIRE(idx_strides->ndim <= HC_MAX_DIMS, "hc_gather: ndim %u exceeds %d", idx_strides->ndim, HC_MAX_DIMS);
+    for (uint32_t k = 0; k < idx_strides->ndim; k++) n *= (uint64_t)idx_strides->shape[k];
+    REQUIRE(n == total, "hc_gather: index shape has %llu elements, expected %llu", (unsigned long long)n,
+            (unsigned long long)total);
+  }
+  const size_t el = dtype_size(dtype);
+
+  // Row form: trailing axes of the index map that cover exactly `inner` elements all have
+  // stride 0, so the index depends on the row only.
+  bool row_form = false;
+  hc_strides row_strides;
+  memset(&row_strides, 0, sizeof(row_strides));
+  if (inner > 1) {
+    uint64_t tail = 1;
+    int k = (int)idx_strides->ndim;
+    bool zero = true;
+    while (k > 0 && tail < (uint64_t)inner) {
+      k--;
+      tail *= (uint64_t)idx_strides->shape[k];
+      if (idx_strides->strides[k] != 0 && idx_strides->shape[k] != 1) zero = false;
+    }
+    if (zero && tail == (uint64_t)inner) {
+      row_form = true;
+      row_strides.ndim = (uint32_t)k;
+      for (int d = 0; d < k; d++) {
+        row_strides.shape[d] = idx_strides->shape[d];
+        row_strides.strides[d] = idx_strides->strides[d];
+      }
+    }
+  }
+  if (row_form) {
+    const size_t row_bytes = (size_t)inner * el;
+    size_t vb = 16;
+    while (vb > 1 && (row_bytes % vb != 0 || ((uintptr_t)in % vb) != 0 || ((uintptr_t)out % vb) != 0)) vb >>= 1;
+    if (vb < el) vb = el;
+    hck_gather_rows_args k;
+    memset(&k, 0, sizeof(k));
+    k.in = in;
+    k.indices = (const int64_t*)indices;
+    k.out = out;
+    k.out_count = (uint32_t)out_count;
+    k.middle = (uint32_t)middle;
+    k.row_vecs = (uint32_t)(row_bytes / vb);
+    k.total_rows = (uint32_t)(outer * out_count);
+    int vec;
+    uint64_t rows;
+    const hc_strides* ops[] = {&row_strides};
+    const void* ptrs[] = {indices};
+    HC_TRY(make_bcast(1, ops, ptrs, out, 1, &k.idx, &vec, &rows));
+    char name[64];
+    snprintf(name, sizeof(name), "hc_gather_rows_b%zu", vb);
+    return launch(ctx, name, ceil_div((uint64_t)k.total_rows * k.row_vecs, HCK_BLOCK), 1, &k, sizeof(k));
+  }
+  hck_gather_elems_args k;
+  memset(&k, 0, sizeof(k));
+  k.in = in;
+  k.indices = (const int64_t*)indices;
+  k.out = out;
+  k.out_count = (uint32_t)out_count;
+  k.middle = (uint32_t)middle;
+  k.inner = (uint32_t)inner;
+  k.total = (uint32_t)total;
+  int vec;
+  uint64_t n;
+  const hc_strides* ops[] = {idx_strides};
+  const void* ptrs[] = {indices};
+  HC_TRY(make_bcast(1, ops, ptrs, out, 1, &k.idx, &vec, &n));
+  char name[64];
+  snprintf(name, sizeof(name), "hc_gather_elems_b%zu", el);
+  return launch(ctx, name, ceil_div(total, HCK_BLOCK), 1, &k, sizeof(k));
+}
+
+extern "C" int hc_axis_permutation(hc_ctx* ctx, const int64_t* perm, const int64_t* shape, int ndim,
+                                   void* out) {
+  REQUIRE(ctx, "hc_axis_permutation: null context");
+  REQUIRE(ndim >= 0 && ndim <= HC_MAX_DIMS, "hc_axis_permutation: ndim %d out of range", ndim);
+  REQUIRE(ndim == 0 || (perm && shape), "hc_axis_permutation: null argument");
+  hck_axis_perm_args k;
+  memset(&k, 0, sizeof(k));
+  uint64_t total = 1;
+  int64_t old_strides[HC_MAX_DIMS];
+  bool seen[HC_MAX_DIMS] = {false};
+  for (int d = ndim - 1; d >= 0; d--) {
+    REQUIRE(shape[d] >= 0, "hc_axis_permutation: negative extent");
+    old_strides[d] = (int64_t)total;
+    total *= (uint64_t)shape[d];
+    if (total > 0xffffffffull) return fail(HC_ERR_TOO_LARGE, "hc_axis_permutation: more than 2^32-1 elements");
+  }
+  for (int d = 0; d < ndim; d++) {
+    REQUIRE(perm[d] >= 0 && perm[d] < ndim && !seen[perm[d]], "hc_axis_permutation: invalid permutation");
+    seen[perm[d]] = true;
+  }
+  if (total == 0) return HC_OK;
+  REQUIRE(out, "hc_axis_permutation: null output");
+  uint64_t acc = 1;
+  for (int d = ndim - 1; d >= 0; d--) {
+    k.new_shape[d] = (uint32_t)shape[perm[d]];
+    k.permuted_strides[d] = (uint32_t)old_strides[perm[d]];
+    k.new_strides[d] = (uint32_t)acc;
+    acc *= (uint64_t)shape[perm[d]];
+  }
+  k.out = (int64_t*)out;
+  k.total = (uint32_t)total;
+  k.ndim = (uint32_t)ndim;
+  return launch(ctx, "hc_axis_permutation", ceil_div(total, HCK_BLOCK), 1, &k, sizeof(k));
+}
+
+extern "C" int hc_triangular(hc_ctx* ctx, int dtype, const void* in, void* out, int64_t batch,
+                             int64_t rows, int64_t cols, int upper, int64_t offset) {
+  REQUIRE(ctx, "hc_triangular: null context");
+  REQUIRE(dtype_name(dtype), "hc_triangular: bad dtype %d", dtype);
+  REQUIRE(batch >= 0 && rows >= 0 && cols >= 0, "hc_triangular: negative dimension");
+  const double total = (double)batch * (double)rows * (double)cols;
+  if (total == 0) return HC_OK;
+  if (total > 4294967295.0) return fail(HC_ERR_TOO_LARGE, "hc_triangular: more than 2^32-1 elements");
+  REQUIRE(in && out, "hc_triangular: null pointer");
+  hck_triangular_args k;
+  memset(&k, 0, sizeof(k));
+  k.in = in;
+  k.out = out;
+  k.total = (uint32_t)(batch * rows * cols);
+  k.rows = (uint32_t)rows;
+  k.cols = (uint32_t)cols;
+  k.upper = upper ? 1 : 0;
+  k.offset = offset;
+  char name[64];
+  snprintf(name, sizeof(name), "hc_triangular_b%zu", dtype_size(dtype));
+  return launch(ctx, name, ceil_div(k.total, HCK_BLOCK), 1, &k, sizeof(k));
+}
+
+extern "C" int hc_concat(hc_ctx* ctx, int dtype, const void* const* inputs, const int64_t* inner_counts,
+                         int n_inputs, int64_t outer, void* out) {
+  REQUIRE(ctx, "hc_concat: null context");
+  REQUIRE(dtype_name(dtype), "hc_concat: bad dtype %d", dtype);
+  REQUIRE(n_inputs >= 0 && outer >= 0, "hc_concat: negative count");
+  REQUIRE(n_inputs == 0 || (inputs && inner_counts), "hc_concat: null argument");
+  const size_t el = dtype_size(dtype);
+  uint64_t total_inner = 0;
+  for (int t = 0; t < n_inputs; t++) {
+    REQUIRE(inner_counts[t] >= 0, "hc_concat: negative inner count");
+    total_inner += (uint64_t)inner_counts[t] * el;
+  }
+  if (total_inner > 0xffffffffull || (uint64_t)outer > 0xffffffffull)
+    return fail(HC_ERR_TOO_LARGE, "hc_concat: slice larger than 2^32-1 bytes");
+  uint64_t off = 0;
+  for (int t = 0; t < n_inputs; t++) {
+    const uint64_t bytes = (uint64_t)inner_counts[t] * el;
+    if (bytes != 0 && outer != 0) {
+      REQUIRE(inputs[t] && out, "hc_concat: null pointer");
+      hck_concat_args k;
+      memset(&k, 0, sizeof(k));
+      k.in = inputs[t];
+      k.out = out;
+      k.outer = (uint32_t)outer;
+      k.inner = (uint32_t)bytes;
+      k.total_inner = (uint32_t)total_inner;
+      k.out_off = (uint32_t)off;
+      HC_TRY(launch(ctx, "hc_concat_bytes", ceil_div((uint64_t)outer * bytes, HCK_BLOCK), 1, &k, sizeof(k)));
+    }
+    off += bytes;
+  }
+  return HC_OK;
+}
+
+// ------------------------------------------------------------------ matmul
+
+extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, int trans_a,
+                         const void* b, int trans_b, int trans_out, int64_t rows, int64_t inner,
+                         int64_t cols, void* out) {
+  REQUIRE(ctx, "hc_matmul: null context");
+  if (dtype != HC_F32 && dtype != HC_F16)
+    return fail(HC_ERR_UNSUPPORTED, "hc_matmul: dtype %d has no MFMA path (int64 stays on the CPU)", dtype);
+  REQUIRE(batch >= 0 && rows >= 0 && inner >= 0 && cols >= 0, "hc_matmul: negative dimension");
+  if (batch * rows * cols == 0) return HC_OK;
+  REQUIRE(out && (inner == 0 || (a && b)), "hc_matmul: null pointer");
+  if (rows > 0x7fffffffll || cols > 0x7fffffffll || inner > 0x7fffffffll ||
+      (double)rows * (double)inner > 4294967295.0 || (double)inner * (double)cols > 4294967295.0 ||
+      (double)rows * (double)cols > 4294967295.0)
+    return fail(HC_ERR_TOO_LARGE, "hc_matmul: a matrix has more than 2^32-1 elements");
+  const size_t el = dtype_size(dtype);
+  const uint32_t P = (uint32_t)(16 / el);
+  hck_gemm_args k;
+  memset(&k, 0, sizeof(k));
+  uint32_t M = (uint32_t)rows, N = (uint32_t)cols, K = (uint32_t)inner;
+  uint32_t a_rs = trans_a ? 1 : K, a_cs = trans_a ? M : 1;
+  uint32_t b_rs = trans_b ? 1 : N, b_cs = trans_b ? K : 1;
+  k.a = a;
+  k.b = b;
+  k.a_bs = (uint64_t)M * K;
+  k.b_bs = (uint64_t)K * N;
+  k.c_bs = (uint64_t)M * N;
+  if (trans_out) {
+    // C^T = B^T * A^T: swap the operands so that the stored output is row-major again.
+    k.a = b;
+    k.b = a;
+    const uint32_t na_rs = b_cs, na_cs = b_rs, nb_rs = a_cs, nb_cs = a_rs;
+    a_rs = na_rs;
+    a_cs = na_cs;
+    b_rs = nb_rs;
+    b_cs = nb_cs;
+    std::swap(k.a_bs, k.b_bs);
+    std::swap(M, N);
+  }
+  k.c = out;
+  k.M = M;
+  k.N = N;
+  k.K = K;
+  k.a_rs = a_rs;
+  k.a_cs = a_cs;
+  k.b_rs = b_rs;
+  k.b_cs = b_cs;
+  k.c_rs = N;
+  k.c_cs = 1;
+  k.tiles_m = (uint32_t)ceil_div(M, 128);
+  k.tiles_n = (uint32_t)ceil_div(N, 128);
+
+  // Per-operand global->LDS path: 'k' contiguous along K, 'm'/'n' contiguous along M/N
+  // (both need 16-byte aligned rows), 'x' anything else.
+  auto mode = [&](const void* ptr, uint32_t row_stride, uint32_t k_stride, uint64_t batch_stride) -> char {
+    const bool base_ok = aligned16(ptr) && (batch <= 1 || batch_stride % P == 0);
+    if (base_ok && k_stride == 1 && row_stride % P == 0) return 'k';
+    if (base_ok && row_stride == 1 && k_stride % P == 0) return 'r';
+    return 'x';
+  };
+  char ma = mode(k.a, a_rs, a_cs, k.a_bs);
+  char mb = mode(k.b, b_cs, b_rs, k.b_bs);
+  char name[64];
+  if (ma == 'x' || mb == 'x')
+    snprintf(name, sizeof(name), "hc_gemm_%s_xx", dtype_name(dtype));
+  else
+    snprintf(name, sizeof(name), "hc_gemm_%s_%c%c", dtype_name(dtype), ma == 'k' ? 'k' : 'm',
+             mb == 'k' ? 'k' : 'n');
+  const uint64_t tiles = (uint64_t)k.tiles_m * k.tiles_n;
+  // grid.y carries the batch (at most 65535 per launch)
+  for (int64_t b0 = 0; b0 < batch; b0 += 65535) {
+    const uint32_t nb = (uint32_t)(batch - b0 < 65535 ? batch - b0 : 65535);
+    hck_gemm_args kk = k;
+    kk.a = (const char*)k.a + (uint64_t)b0 * k.a_bs * el;
+    kk.b = (const char*)k.b + (uint64_t)b0 * k.b_bs * el;
+    kk.c = (char*)k.c + (uint64_t)b0 * k.c_bs * el;
+    kk.batch = nb;
+    HC_TRY(launch(ctx, name, tiles, nb, &kk, sizeof(kk)));
+  }
+  return HC_OK;
+}

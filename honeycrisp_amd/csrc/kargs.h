@@ -1,0 +1,148 @@
+/*
+ * Kernel argument blocks shared by the host launcher (hchip.cpp) and the gfx950
+ * kernels. Every kernel takes exactly one of these structs by value, so the
+ * host hands the struct itself to hipModuleLaunchKernel as the kernarg buffer.
+ * Plain C layout, natural alignment, no pointers-to-host.
+ */
+#ifndef HC_KARGS_H
+#define HC_KARGS_H
+
+#include <stdint.h>
+
+#define HCK_MAX_DIMS 8
+#define HCK_BLOCK 256
+
+/* Joint broadcast descriptor for up to three operands after the host has dropped
+ * size-1 axes and merged axes that are mergeable for every operand. The innermost
+ * axis is split off: a thread handles `vec` consecutive inner elements, the rest of
+ * the flat index ("row") is unravelled over outer_shape. Strides are in elements;
+ * inner strides are 0 or 1. */
+typedef struct {
+  uint32_t n_outer;
+  uint32_t inner;
+  uint32_t inner_vecs; /* inner / vec */
+  uint32_t total_vecs; /* rows * inner_vecs */
+  uint32_t outer_shape[HCK_MAX_DIMS - 1];
+  uint32_t outer_stride[3][HCK_MAX_DIMS - 1];
+  uint32_t inner_stride[3];
+  uint32_t pad;
+} hck_bcast;
+
+/* out = a (op) b, broadcast; also compare (bool out) and broadcast copy (a only). */
+typedef struct {
+  const void* a;
+  const void* b;
+  void* out;
+  hck_bcast d;
+} hck_binary_args;
+
+/* out = f(in, coeff, bias) for mulAdd / addMul; out = mask ? a : b for when. */
+typedef struct {
+  const void* x;
+  const void* y;
+  const void* z;
+  void* out;
+  hck_bcast d;
+} hck_ternary_args;
+
+/* Contiguous tensor (op) scalar. */
+typedef struct {
+  const void* in;
+  void* out;
+  uint64_t count;
+  float sf;
+  int32_t pad;
+  int64_t si;
+} hck_scalar_args;
+
+/* Contiguous unary map with optional per-element scales: elemwise, pow, cast, fill. */
+typedef struct {
+  const void* in;
+  const void* scales;
+  void* out;
+  uint64_t count;
+  float p0; /* pow: exponent / fill: value */
+  float p1; /* pow: scale */
+  int64_t i0;
+  int64_t i1;
+} hck_map_args;
+
+/* Input viewed as [outer, reduce, inner]. */
+typedef struct {
+  const void* in;
+  void* out;
+  uint32_t outer;
+  uint32_t reduce;
+  uint32_t inner;
+  float eps;
+} hck_reduce_args;
+
+/* Row gather: every output row of row_vecs 16-byte (or narrower) vectors comes from
+ * one source row chosen by an index that only depends on the row. */
+typedef struct {
+  const void* in;
+  const int64_t* indices;
+  void* out;
+  uint32_t out_count; /* rows per outer slice (indices.shape[axis]) */
+  uint32_t middle;    /* source rows per outer slice */
+  uint32_t row_vecs;  /* vectors per row */
+  uint32_t total_rows;
+  hck_bcast idx; /* operand 0 = index offset for a flat row number, vec = 1 */
+} hck_gather_rows_args;
+
+/* Element gather: general index map over the flat output index. */
+typedef struct {
+  const void* in;
+  const int64_t* indices;
+  void* out;
+  uint32_t out_count;
+  uint32_t middle;
+  uint32_t inner;
+  uint32_t total;
+  hck_bcast idx; /* operand 0 = index offset for a flat output element, vec = 1 */
+} hck_gather_elems_args;
+
+typedef struct {
+  int64_t* out;
+  uint32_t total;
+  uint32_t ndim;
+  uint32_t new_shape[HCK_MAX_DIMS];
+  uint32_t new_strides[HCK_MAX_DIMS];
+  uint32_t permuted_strides[HCK_MAX_DIMS];
+} hck_axis_perm_args;
+
+typedef struct {
+  const void* in;
+  void* out;
+  uint32_t total; /* batch * rows * cols */
+  uint32_t rows;
+  uint32_t cols;
+  int32_t upper;
+  int64_t offset;
+} hck_triangular_args;
+
+/* One input of a concat: out[o, out_off + c] = in[o, c], c < inner. */
+typedef struct {
+  const void* in;
+  void* out;
+  uint32_t outer;
+  uint32_t inner;       /* bytes per outer slice of this input */
+  uint32_t total_inner; /* bytes per outer slice of the output */
+  uint32_t out_off;     /* byte offset inside the output slice */
+} hck_concat_args;
+
+/* C[M,N] = op(A) * op(B) per batch element; logical element (i,k) of A is at
+ * a[i*a_rs + k*a_cs], (k,j) of B at b[k*b_rs + j*b_cs], (i,j) of C at c[i*c_rs + j*c_cs]
+ * (strides in elements), batch element m at offsets m*a_bs, m*b_bs, m*c_bs. */
+typedef struct {
+  const void* a;
+  const void* b;
+  void* c;
+  uint32_t M, N, K;
+  uint32_t batch;
+  uint32_t a_rs, a_cs, b_rs, b_cs, c_rs, c_cs;
+  uint64_t a_bs, b_bs, c_bs;
+  uint32_t tiles_m, tiles_n;
+} hck_gemm_args;
+
+#endif

@@ -1,0 +1,114 @@
+// Device-side helpers shared by the gfx950 kernels: element traits, 16-byte vector
+// access, the broadcast index map, and wave64 / block reductions.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../kargs.h"
+
+typedef _Float16 half_t;
+
+#define HC_KERNEL extern "C" __global__ __launch_bounds__(HCK_BLOCK)
+
+// Storage type T -> arithmetic type. The CPU backend stages half through Float and
+// rounds once on store (BackendCPU.swift:2018-2058), int64 stays int64.
+template <typename T> struct Arith { typedef float type; };
+template <> struct Arith<int64_t> { typedef int64_t type; };
+template <> struct Arith<uint8_t> { typedef float type; };
+
+template <typename T> __device__ __forceinline__ typename Arith<T>::type to_arith(T v) {
+  return (typename Arith<T>::type)v;
+}
+template <> __device__ __forceinline__ float to_arith<uint8_t>(uint8_t v) {
+  return v ? 1.0f : 0.0f;
+}
+
+template <typename T> __device__ __forceinline__ T from_arith(typename Arith<T>::type v) {
+  return (T)v;  // float -> half is v_cvt_f16_f32: round-to-nearest-even, overflow to inf
+}
+
+// Round an fp32 intermediate to what the tensor dtype can hold (identity for float).
+template <typename T> __device__ __forceinline__ float round_through(float v) {
+  return (float)(T)v;
+}
+template <> __device__ __forceinline__ float round_through<float>(float v) { return v; }
+
+template <typename T, int N> struct alignas(sizeof(T) * N) Vec {
+  T v[N];
+};
+
+// Elements per 16-byte access.
+template <typename T> struct VecWidth { static constexpr int value = 16 / sizeof(T); };
+
+template <typename T, int N>
+__device__ __forceinline__ void load_vec(const T* base, uint32_t off, uint32_t stride, T (&dst)[N]) {
+  if (N > 1 && stride == 1) {
+    Vec<T, N> t = *reinterpret_cast<const Vec<T, N>*>(base + off);
+#pragma unroll
+    for (int i = 0; i < N; i++) dst[i] = t.v[i];
+  } else {
+#pragma unroll
+    for (int i = 0; i < N; i++) dst[i] = base[off + i * stride];
+  }
+}
+
+template <typename T, int N>
+__device__ __forceinline__ void store_vec(T* base, size_t off, const T (&src)[N]) {
+  Vec<T, N> t;
+#pragma unroll
+  for (int i = 0; i < N; i++) t.v[i] = src[i];
+  *reinterpret_cast<Vec<T, N>*>(base + off) = t;
+}
+
+// Broadcast index map (Broadcast.swift:72-90) for NOPS operands at once: vector number
+// v -> element offsets of the first of VEC inner elements, and the flat output offset.
+template <int NOPS, int VEC>
+__device__ __forceinline__ void bcast_offsets(const hck_bcast& d, uint32_t v, uint32_t (&off)[NOPS],
+                                              size_t& out_off) {
+  uint32_t row = v / d.inner_vecs;
+  uint32_t col = (v - row * d.inner_vecs) * VEC;
+  out_off = (size_t)row * d.inner + col;
+#pragma unroll
+  for (int o = 0; o < NOPS; o++) off[o] = col * d.inner_stride[o];
+  for (int k = (int)d.n_outer - 1; k >= 0; k--) {
+    uint32_t s = d.outer_shape[k];
+    uint32_t q = row / s;
+    uint32_t r = row - q * s;
+#pragma unroll
+    for (int o = 0; o < NOPS; o++) off[o] += r * d.outer_stride[o][k];
+    row = q;
+  }
+}
+
+// ---- wave64 / block reductions ----
+
+template <typename V, typename Op> __device__ __forceinline__ V wave_reduce(V v, Op op) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = op(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+struct SumOp {
+  template <typename V> __device__ __forceinline__ V operator()(V a, V b) const { return a + b; }
+};
+struct ProdOp {
+  template <typename V> __device__ __forceinline__ V operator()(V a, V b) const { return a * b; }
+};
+struct MaxOp {
+  __device__ __forceinline__ float operator()(float a, float b) const { return a > b ? a : b; }
+};
+
+// Reduce across the HCK_BLOCK threads of a block; every thread gets the result.
+template <typename V, typename Op>
+__device__ __forceinline__ V block_reduce(V v, Op op, V* lds /* >= 4 entries */) {
+  v = wave_reduce(v, op);
+  const int wave = threadIdx.x >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) lds[wave] = v;
+  __syncthreads();
+  V r = lds[0];
+#pragma unroll
+  for (int w = 1; w < HCK_BLOCK / 64; w++) r = op(r, lds[w]);
+  return r;
+}

@@ -1,0 +1,93 @@
+// Data-movement kernels for gfx950: int64-indexed gather, axisPermutation, triangular,
+// concat. All bit-exact copies keyed by element size, not dtype.
+//
+// gather (BackendCPU.swift:1108-1147):
+//   out[(i*out_count + j)*inner + k] = in[(i*middle + idx)*inner + k],
+//   idx = indices[index_strides(flat out index)]
+// Row form: when the index does not depend on k and a row is a whole number of vectors,
+// one lane moves one 16-byte vector and reads the (cached) row index once; consecutive
+// lanes cover consecutive vectors of a row, so both the scattered source rows and the
+// dense destination are accessed in full 64-byte-or-larger segments.
+#include "common.hip.h"
+
+template <typename V> __device__ __forceinline__ void gather_rows_impl(const hck_gather_rows_args& p) {
+  const uint64_t v = (uint64_t)blockIdx.x * HCK_BLOCK + threadIdx.x;
+  const uint32_t row = (uint32_t)(v / p.row_vecs);
+  if (row >= p.total_rows) return;
+  const uint32_t c = (uint32_t)(v - (uint64_t)row * p.row_vecs);
+  uint32_t off[1];
+  size_t unused;
+  bcast_offsets<1, 1>(p.idx, row, off, unused);
+  const int64_t idx = p.indices[off[0]];
+  const uint32_t i = row / p.out_count;
+  const int64_t src_row = (int64_t)i * p.middle + idx;
+  ((V*)p.out)[v] = ((const V*)p.in)[src_row * (int64_t)p.row_vecs + c];
+}
+
+struct alignas(16) V16 { uint32_t x[4]; };
+
+HC_KERNEL void hc_gather_rows_b16(hck_gather_rows_args p) { gather_rows_impl<V16>(p); }
+HC_KERNEL void hc_gather_rows_b8(hck_gather_rows_args p) { gather_rows_impl<uint64_t>(p); }
+HC_KERNEL void hc_gather_rows_b4(hck_gather_rows_args p) { gather_rows_impl<uint32_t>(p); }
+HC_KERNEL void hc_gather_rows_b2(hck_gather_rows_args p) { gather_rows_impl<uint16_t>(p); }
+HC_KERNEL void hc_gather_rows_b1(hck_gather_rows_args p) { gather_rows_impl<uint8_t>(p); }
+
+// General form: one lane per output element, full index map.
+template <typename V> __device__ __forceinline__ void gather_elems_impl(const hck_gather_elems_args& p) {
+  const uint32_t o = blockIdx.x * HCK_BLOCK + threadIdx.x;
+  if (o >= p.total) return;
+  uint32_t off[1];
+  size_t unused;
+  bcast_offsets<1, 1>(p.idx, o, off, unused);
+  const int64_t idx = p.indices[off[0]];
+  const uint32_t ij = o / p.inner;
+  const uint32_t k = o - ij * p.inner;
+  const uint32_t i = ij / p.out_count;
+  ((V*)p.out)[o] = ((const V*)p.in)[((int64_t)i * p.middle + idx) * (int64_t)p.inner + k];
+}
+HC_KERNEL void hc_gather_elems_b8(hck_gather_elems_args p) { gather_elems_impl<uint64_t>(p); }
+HC_KERNEL void hc_gather_elems_b4(hck_gather_elems_args p) { gather_elems_impl<uint32_t>(p); }
+HC_KERNEL void hc_gather_elems_b2(hck_gather_elems_args p) { gather_elems_impl<uint16_t>(p); }
+HC_KERNEL void hc_gather_elems_b1(hck_gather_elems_args p) { gather_elems_impl<uint8_t>(p); }
+
+// axisPermutation (BackendCPU.swift:1831-1849): flat source index of every element of the
+// permuted view.
+HC_KERNEL void hc_axis_permutation(hck_axis_perm_args p) {
+  const uint32_t i = blockIdx.x * HCK_BLOCK + threadIdx.x;
+  if (i >= p.total) return;
+  uint32_t flat = 0;
+  for (uint32_t d = 0; d < p.ndim; d++)
+    flat += p.permuted_strides[d] * ((i / p.new_strides[d]) % p.new_shape[d]);
+  p.out[i] = (int64_t)flat;
+}
+
+// triangular (BackendCPU.swift:1315-1348): keep the lower (upper) triangle shifted by
+// `offset`, zero elsewhere. Row j keeps columns [0, j+1+offset) or [j+offset, cols).
+template <typename V> __device__ __forceinline__ void triangular_impl(const hck_triangular_args& p) {
+  const uint32_t o = blockIdx.x * HCK_BLOCK + threadIdx.x;
+  if (o >= p.total) return;
+  const uint32_t col = o % p.cols;
+  const uint32_t row = (o / p.cols) % p.rows;
+  bool keep;
+  if (p.upper) {
+    keep = (int64_t)col >= (int64_t)row + p.offset;
+  } else {
+    keep = (int64_t)col < (int64_t)row + 1 + p.offset;
+  }
+  ((V*)p.out)[o] = keep ? ((const V*)p.in)[o] : (V)0;
+}
+HC_KERNEL void hc_triangular_b8(hck_triangular_args p) { triangular_impl<uint64_t>(p); }
+HC_KERNEL void hc_triangular_b4(hck_triangular_args p) { triangular_impl<uint32_t>(p); }
+HC_KERNEL void hc_triangular_b2(hck_triangular_args p) { triangular_impl<uint16_t>(p); }
+HC_KERNEL void hc_triangular_b1(hck_triangular_args p) { triangular_impl<uint8_t>(p); }
+
+// concat (BackendCPU.swift:1768-1794), one launch per input: byte copy of an
+// [outer, inner] block into a column range of the [outer, total_inner] output.
+HC_KERNEL void hc_concat_bytes(hck_concat_args p) {
+  const uint64_t t = (uint64_t)blockIdx.x * HCK_BLOCK + threadIdx.x;
+  const uint64_t total = (uint64_t)p.outer * p.inner;
+  if (t >= total) return;
+  const uint32_t o = (uint32_t)(t / p.inner);
+  const uint32_t c = (uint32_t)(t - (uint64_t)o * p.inner);
+  ((uint8_t*)p.out)[(uint64_t)o * p.total_inner + p.out_off + c] = ((const uint8_t*)p.in)[t];
+}

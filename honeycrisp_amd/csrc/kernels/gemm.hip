@@ -1,0 +1,232 @@
+// General MFMA GEMM for gfx950: C[M,N] = A[M,K] * B[K,N] per batch element, fp16 inputs
+// with fp32 accumulation (v_mfma_f32_32x32x16_f16) and fp32 (v_mfma_f32_32x32x2_f32).
+// Handles every transpose combination and ragged M, N, K; the tuned kernels in
+// gemm_f16_fast.hip take over for large aligned fp16 problems.
+//
+// Tile: 128 x 128 outputs per 256-lane block, four waves in a 2 x 2 grid, each wave a
+// 64 x 64 sub-tile = 2 x 2 MFMA 32x32 accumulators (64 fp32 VGPRs). K advances in steps
+// of 128 bytes per row (64 halfs / 32 floats). Both operands live in LDS K-contiguous
+// ([row][k], 144-byte pitch) so one ds_read_b128 per lane yields an MFMA operand:
+//   lane l reads row (l % 32), 16-byte chunk (2*s + l / 32) at sub-step s.
+// Any consistent k -> (lane group, slot) assignment is valid because A and B use the same.
+//
+// Global -> LDS, chosen per operand by the host:
+//   LOAD_K   operand contiguous along k: 16-byte loads, 8 lanes per 128-byte row segment.
+//   LOAD_MN  operand contiguous along m (or n): each lane loads 4 k-rows x 16 bytes,
+//            transposes the 4 x P block in registers and writes P chunks of 4 k-values.
+//   LOAD_ANY arbitrary strides / unaligned / ragged: predicated scalar loads.
+// The next K-step is fetched into registers before the MFMAs of the current one.
+#include "common.hip.h"
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+enum { LOAD_K = 0, LOAD_MN = 1, LOAD_ANY = 2 };
+
+#define G_BM 128
+#define G_BN 128
+#define G_ROW_BYTES 128
+#define G_PITCH 144 /* bytes: 128 + 16 pad keeps ds_read_b128 of 32 rows off the same banks */
+
+template <typename T> struct GemmTraits;
+template <> struct GemmTraits<half_t> {
+  static constexpr int P = 8;   // elements per 16 bytes
+  static constexpr int BK = 64; // elements per K-step
+};
+template <> struct GemmTraits<float> {
+  static constexpr int P = 4;
+  static constexpr int BK = 32;
+};
+
+struct alignas(16) Chunk16 {
+  uint32_t w[4];
+};
+
+__device__ __forceinline__ void mma_chunk(floatx16& acc, const Chunk16& a, const Chunk16& b, half_t) {
+  acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const half8*>(&a),
+                                               *reinterpret_cast<const half8*>(&b), acc, 0, 0, 0);
+}
+__device__ __forceinline__ void mma_chunk(floatx16& acc, const Chunk16& a, const Chunk16& b, float) {
+  const float* af = reinterpret_cast<const float*>(&a);
+  const float* bf = reinterpret_cast<const float*>(&b);
+#pragma unroll
+  for (int i = 0; i < 4; i++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i], bf[i], acc, 0, 0, 0);
+}
+
+// Registers holding one operand's share of a K-step (128 rows x 128 bytes / 256 lanes = 64 B).
+template <typename T> struct Staged {
+  Chunk16 v[4];
+};
+
+// Fetch this lane's part of the tile rows [r0, r0+128) x k [k0, k0+BK) of an operand whose
+// logical element (r, k) sits at base[r*rs + k*cs]. Out-of-range elements read as zero.
+template <typename T, int MODE>
+__device__ __forceinline__ void fetch(Staged<T>& st, const T* base, uint32_t rs, uint32_t cs,
+                                      uint32_t r0, uint32_t k0, uint32_t R, uint32_t K) {
+  constexpr int P = GemmTraits<T>::P;
+  constexpr int BK = GemmTraits<T>::BK;
+  const uint32_t t = threadIdx.x;
+  if (MODE == LOAD_K) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const uint32_t id = t + 256 * i;
+      const uint32_t r = r0 + id / 8, k = k0 + (id % 8) * P;
+      Chunk16 z = {{0, 0, 0, 0}};
+      if (r < R && k < K) z = *reinterpret_cast<const Chunk16*>(base + (size_t)r * rs + k);
+      st.v[i] = z;
+    }
+  } else if (MODE == LOAD_MN) {
+    constexpr int MB = G_BM / P;  // 16-byte blocks along the contiguous m/n axis
+    const uint32_t r = r0 + (t % MB) * P, kb = k0 + (t / MB) * 4;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      Chunk16 z = {{0, 0, 0, 0}};
+      if (r < R && kb + i < K) z = *reinterpret_cast<const Chunk16*>(base + (size_t)(kb + i) * cs + r);
+      st.v[i] = z;
+    }
+  } else {
+    T* e = reinterpret_cast<T*>(&st);
+    constexpr int PER = G_BM * BK / 256;
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+      const uint32_t id = t + 256 * i;
+      uint32_t r, k;
+      if (cs <= rs) {  // k is the faster-varying axis in memory
+        r = id / BK;
+        k = id % BK;
+      } else {
+        k = id / G_BM;
+        r = id % G_BM;
+      }
+      T val = (T)0;
+      if (r0 + r < R && k0 + k < K) val = base[(size_t)(r0 + r) * rs + (size_t)(k0 + k) * cs];
+      e[i] = val;
+    }
+  }
+}
+
+// Write the staged registers into the K-contiguous LDS tile.
+template <typename T, int MODE>
+__device__ __forceinline__ void stash(const Staged<T>& st, char* lds, uint32_t rs, uint32_t cs) {
+  constexpr int P = GemmTraits<T>::P;
+  constexpr int BK = GemmTraits<T>::BK;
+  const uint32_t t = threadIdx.x;
+  if (MODE == LOAD_K) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const uint32_t id = t + 256 * i;
+      *reinterpret_cast<Chunk16*>(lds + (id / 8) * G_PITCH + (id % 8) * 16) = st.v[i];
+    }
+  } else if (MODE == LOAD_MN) {
+    constexpr int MB = G_BM / P;
+    const uint32_t r = (t % MB) * P, kb = (t / MB) * 4;
+    const T* e = reinterpret_cast<const T*>(&st);  // e[i*P + p] = element (k = kb+i, row r+p)
+#pragma unroll
+    for (int p = 0; p < P; p++) {
+      T col[4];
+#pragma unroll
+      for (int i = 0; i < 4; i++) col[i] = e[i * P + p];
+      *reinterpret_cast<Vec<T, 4>*>(lds + (r + p) * G_PITCH + kb * sizeof(T)) =
+          *reinterpret_cast<Vec<T, 4>*>(col);
+    }
+  } else {
+    const T* e = reinterpret_cast<const T*>(&st);
+    constexpr int PER = G_BM * BK / 256;
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+      const uint32_t id = t + 256 * i;
+      uint32_t r, k;
+      if (cs <= rs) {
+        r = id / BK;
+        k = id % BK;
+      } else {
+        k = id / G_BM;
+        r = id % G_BM;
+      }
+      *reinterpret_cast<T*>(lds + r * G_PITCH + k * sizeof(T)) = e[i];
+    }
+  }
+}
+
+template <typename T, int MODE_A, int MODE_B>
+__device__ __forceinline__ void gemm_impl(const hck_gemm_args& p) {
+  constexpr int BK = GemmTraits<T>::BK;
+  __shared__ __attribute__((aligned(16))) char lds_a[G_BM * G_PITCH];
+  __shared__ __attribute__((aligned(16))) char lds_b[G_BN * G_PITCH];
+
+  const uint32_t tile = blockIdx.x;
+  const uint32_t tm = tile / p.tiles_n, tn = tile % p.tiles_n;
+  const uint32_t batch = blockIdx.y;
+  const T* A = (const T*)p.a + batch * p.a_bs;
+  const T* B = (const T*)p.b + batch * p.b_bs;
+  T* C = (T*)p.c + batch * p.c_bs;
+  const uint32_t m0 = tm * G_BM, n0 = tn * G_BN;
+
+  const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const uint32_t wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+  const uint32_t lrow = lane & 31, lgrp = lane >> 5;
+
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+
+  Staged<T> sa, sb;
+  // B is addressed as rows = n, so its "row stride" is b_cs and its k stride is b_rs.
+  fetch<T, MODE_A>(sa, A, p.a_rs, p.a_cs, m0, 0, p.M, p.K);
+  fetch<T, MODE_B>(sb, B, p.b_cs, p.b_rs, n0, 0, p.N, p.K);
+
+  for (uint32_t k0 = 0; k0 < p.K; k0 += BK) {
+    __syncthreads();  // previous step's LDS reads are done
+    stash<T, MODE_A>(sa, lds_a, p.a_rs, p.a_cs);
+    stash<T, MODE_B>(sb, lds_b, p.b_cs, p.b_rs);
+    __syncthreads();
+    if (k0 + BK < p.K) {
+      fetch<T, MODE_A>(sa, A, p.a_rs, p.a_cs, m0, k0 + BK, p.M, p.K);
+      fetch<T, MODE_B>(sb, B, p.b_cs, p.b_rs, n0, k0 + BK, p.N, p.K);
+    }
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+      Chunk16 fa[2], fb[2];
+#pragma unroll
+      for (int i = 0; i < 2; i++) {
+        fa[i] = *reinterpret_cast<const Chunk16*>(lds_a + (wm + i * 32 + lrow) * G_PITCH + (2 * s + lgrp) * 16);
+        fb[i] = *reinterpret_cast<const Chunk16*>(lds_b + (wn + i * 32 + lrow) * G_PITCH + (2 * s + lgrp) * 16);
+      }
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) mma_chunk(acc[i][j], fa[i], fb[j], T());
+    }
+  }
+
+  // 32x32 accumulator layout: lane l, register v holds row 8*(v/4) + 4*(l/32) + v%4,
+  // column l%32 of the MFMA tile.
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      const uint32_t col = n0 + wn + j * 32 + lrow;
+#pragma unroll
+      for (int v = 0; v < 16; v++) {
+        const uint32_t row = m0 + wm + i * 32 + 8 * (v / 4) + 4 * lgrp + (v % 4);
+        if (row < p.M && col < p.N) C[(size_t)row * p.c_rs + (size_t)col * p.c_cs] = (T)acc[i][j][v];
+      }
+    }
+}
+
+#define DEF_GEMM(TN, T, AN, AM, BN_, BM_)                                                            \
+  HC_KERNEL void hc_gemm_##TN##_##AN##BN_(hck_gemm_args p) { gemm_impl<T, AM, BM_>(p); }
+#define DEF_GEMM_T(TN, T)                                                                            \
+  DEF_GEMM(TN, T, k, LOAD_K, k, LOAD_K)                                                              \
+  DEF_GEMM(TN, T, k, LOAD_K, n, LOAD_MN)                                                             \
+  DEF_GEMM(TN, T, m, LOAD_MN, k, LOAD_K)                                                             \
+  DEF_GEMM(TN, T, m, LOAD_MN, n, LOAD_MN)                                                            \
+  DEF_GEMM(TN, T, x, LOAD_ANY, x, LOAD_ANY)
+DEF_GEMM_T(f16, half_t)
+DEF_GEMM_T(f32, float)

@@ -1,0 +1,293 @@
+// Axis reductions for gfx950: sum / prod / argmax / argmin over the middle axis of an
+// [outer, reduce, inner] view, logSoftmax and the fused two-pass normalize.
+//
+// inner == 1 ("row" kernels): the reduced axis is contiguous. A wave (short rows) or a
+// 256-lane block (long rows) owns one row, streams it with 16-byte loads, reduces in
+// registers, then across lanes with wave64 shuffles and across waves through LDS.
+// inner > 1 ("col" kernels): lanes run along the contiguous inner axis so every step of
+// the reduction loop is one coalesced access; 4 waves split the reduce axis and meet
+// in LDS.
+//
+// argmax/argmin return the first extremum exactly as the CPU's strict-compare scan from
+// k = 0 does (BackendCPU.swift:848-877): ties go to the smaller index, a NaN at k > 0
+// never replaces the running extremum, and a NaN at k = 0 is never replaced.
+#include "common.hip.h"
+
+#include <math.h>
+
+enum { R_SUM = 0, R_PROD = 1, R_ARGMAX = 2, R_ARGMIN = 3 };
+
+template <typename C> struct ArgPair {
+  C v;
+  uint32_t i;
+};
+
+// Ordering key for one element of an arg-reduction: makes the parallel "better value,
+// or equal value and smaller index" combine reproduce the sequential scan. For floats a
+// NaN at k = 0 becomes the unbeatable extreme and a NaN elsewhere the worst value (it
+// can then only tie with element 0 or later ones of larger index, never win).
+template <int OP> __device__ __forceinline__ float arg_key(float x, uint32_t k) {
+  if (x != x) {
+    const float best = OP == R_ARGMAX ? INFINITY : -INFINITY;
+    return k == 0 ? best : -best;
+  }
+  return x;
+}
+template <int OP> __device__ __forceinline__ int64_t arg_key(int64_t x, uint32_t) { return x; }
+
+template <int OP, typename C>
+__device__ __forceinline__ ArgPair<C> arg_better(ArgPair<C> a, ArgPair<C> b) {
+  bool take_b = OP == R_ARGMAX ? (b.v > a.v) : (b.v < a.v);
+  take_b = take_b || (b.v == a.v && b.i < a.i);
+  return take_b ? b : a;
+}
+
+template <int OP, typename C> __device__ __forceinline__ ArgPair<C> wave_arg_reduce(ArgPair<C> p) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    ArgPair<C> q;
+    q.v = __shfl_xor(p.v, o, 64);
+    q.i = __shfl_xor(p.i, o, 64);
+    p = arg_better<OP>(p, q);
+  }
+  return p;
+}
+
+// Worst possible value, paired with the largest index, so that any real element wins.
+template <int OP> __device__ __forceinline__ void arg_init(ArgPair<float>& p) {
+  p.v = OP == R_ARGMAX ? -INFINITY : INFINITY;
+  p.i = 0xffffffffu;
+}
+template <int OP> __device__ __forceinline__ void arg_init(ArgPair<int64_t>& p) {
+  p.v = OP == R_ARGMAX ? INT64_MIN : INT64_MAX;
+  p.i = 0xffffffffu;
+}
+
+template <int OP, typename C> __device__ __forceinline__ C reduce_identity() {
+  return OP == R_SUM ? (C)0 : (C)1;
+}
+template <int OP, typename C> __device__ __forceinline__ C reduce_combine(C a, C b) {
+  return OP == R_SUM ? a + b : a * b;
+}
+
+// ---------------------------------------------------------------- rows (inner == 1)
+
+// LANES = 64: one wave per row, 4 rows per block. LANES = 256: one block per row.
+template <typename T, int OP, int LANES>
+__device__ __forceinline__ void reduce_rows_impl(const hck_reduce_args& p) {
+  typedef typename Arith<T>::type C;
+  constexpr int VEC = VecWidth<T>::value;
+  constexpr int ROWS_PER_BLOCK = HCK_BLOCK / LANES;
+  const uint32_t lane = threadIdx.x % LANES;
+  const uint32_t row = blockIdx.x * ROWS_PER_BLOCK + threadIdx.x / LANES;
+  const bool active = row < p.outer;
+  const uint32_t n = p.reduce;
+  const T* in = (const T*)p.in + (size_t)(active ? row : 0) * n;
+  // Rows start 16-byte aligned only when the row length is a multiple of VEC.
+  const bool vec_ok = (n % VEC) == 0;
+  __shared__ char lds_raw[sizeof(ArgPair<C>) * (HCK_BLOCK / 64)];
+
+  if (OP == R_SUM || OP == R_PROD) {
+    C acc = reduce_identity<OP, C>();
+    if (active) {
+      if (vec_ok) {
+        for (uint32_t k = lane * VEC; k < n; k += LANES * VEC) {
+          T a[VEC];
+          load_vec<T, VEC>(in, k, 1, a);
+#pragma unroll
+          for (int i = 0; i < VEC; i++) acc = reduce_combine<OP, C>(acc, to_arith(a[i]));
+        }
+      } else {
+        for (uint32_t k = lane; k < n; k += LANES) acc = reduce_combine<OP, C>(acc, to_arith(in[k]));
+      }
+    }
+    if (LANES == 64) {
+      acc = OP == R_SUM ? wave_reduce(acc, SumOp()) : wave_reduce(acc, ProdOp());
+    } else {
+      acc = OP == R_SUM ? block_reduce(acc, SumOp(), (C*)lds_raw)
+                        : block_reduce(acc, ProdOp(), (C*)lds_raw);
+    }
+    if (active && lane == 0) ((T*)p.out)[row] = from_arith<T>(acc);
+  } else {
+    ArgPair<C> best;
+    arg_init<OP>(best);
+    if (active) {
+      if (vec_ok) {
+        for (uint32_t k = lane * VEC; k < n; k += LANES * VEC) {
+          T a[VEC];
+          load_vec<T, VEC>(in, k, 1, a);
+#pragma unroll
+          for (int i = 0; i < VEC; i++) {
+            ArgPair<C> c;
+            c.v = arg_key<OP>(to_arith(a[i]), k + i);
+            c.i = k + i;
+            best = arg_better<OP>(best, c);
+          }
+        }
+      } else {
+        for (uint32_t k = lane; k < n; k += LANES) {
+          ArgPair<C> c;
+          c.v = arg_key<OP>(to_arith(in[k]), k);
+          c.i = k;
+          best = arg_better<OP>(best, c);
+        }
+      }
+    }
+    best = wave_arg_reduce<OP>(best);
+    if (LANES > 64) {
+      ArgPair<C>* lds = (ArgPair<C>*)lds_raw;
+      if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = best;
+      __syncthreads();
+      best = lds[0];
+#pragma unroll
+      for (int w = 1; w < HCK_BLOCK / 64; w++) best = arg_better<OP>(best, lds[w]);
+    }
+    if (active && lane == 0) ((int64_t*)p.out)[row] = (int64_t)best.i;
+  }
+}
+
+// ---------------------------------------------------------------- columns (inner > 1)
+
+// Block = 64 lanes along inner x 4 waves along reduce. grid.x covers inner, grid.y outer.
+template <typename T, int OP> __device__ __forceinline__ void reduce_cols_impl(const hck_reduce_args& p) {
+  typedef typename Arith<T>::type C;
+  const uint32_t j = blockIdx.x * 64 + (threadIdx.x & 63);
+  const uint32_t kw = threadIdx.x >> 6;
+  const uint32_t i = blockIdx.y;
+  const bool active = j < p.inner;
+  const T* in = (const T*)p.in + (size_t)i * p.reduce * p.inner + (active ? j : 0);
+  __shared__ char lds_raw[sizeof(ArgPair<C>) * HCK_BLOCK];
+
+  if (OP == R_SUM || OP == R_PROD) {
+    C acc = reduce_identity<OP, C>();
+    if (active)
+      for (uint32_t k = kw; k < p.reduce; k += 4)
+        acc = reduce_combine<OP, C>(acc, to_arith(in[(size_t)k * p.inner]));
+    C* lds = (C*)lds_raw;
+    lds[threadIdx.x] = acc;
+    __syncthreads();
+    if (kw == 0 && active) {
+      for (int w = 1; w < 4; w++) acc = reduce_combine<OP, C>(acc, lds[threadIdx.x + 64 * w]);
+      ((T*)p.out)[(size_t)i * p.inner + j] = from_arith<T>(acc);
+    }
+  } else {
+    ArgPair<C> best;
+    arg_init<OP>(best);
+    if (active)
+      for (uint32_t k = kw; k < p.reduce; k += 4) {
+        ArgPair<C> c;
+        c.v = arg_key<OP>(to_arith(in[(size_t)k * p.inner]), k);
+        c.i = k;
+        best = arg_better<OP>(best, c);
+      }
+    ArgPair<C>* lds = (ArgPair<C>*)lds_raw;
+    lds[threadIdx.x] = best;
+    __syncthreads();
+    if (kw == 0 && active) {
+      for (int w = 1; w < 4; w++) best = arg_better<OP>(best, lds[threadIdx.x + 64 * w]);
+      ((int64_t*)p.out)[(size_t)i * p.inner + j] = (int64_t)best.i;
+    }
+  }
+}
+
+#define DEF_REDUCE(NAME, OP, TN, T)                                                                   \
+  HC_KERNEL void hc_reduce_rows64_##NAME##_##TN(hck_reduce_args p) { reduce_rows_impl<T, OP, 64>(p); } \
+  HC_KERNEL void hc_reduce_rows256_##NAME##_##TN(hck_reduce_args p) { reduce_rows_impl<T, OP, 256>(p); } \
+  HC_KERNEL void hc_reduce_cols_##NAME##_##TN(hck_reduce_args p) { reduce_cols_impl<T, OP>(p); }
+#define DEF_REDUCE_T(TN, T)                                                                          \
+  DEF_REDUCE(sum, R_SUM, TN, T)                                                                      \
+  DEF_REDUCE(prod, R_PROD, TN, T)                                                                    \
+  DEF_REDUCE(argmax, R_ARGMAX, TN, T)                                                                \
+  DEF_REDUCE(argmin, R_ARGMIN, TN, T)
+DEF_REDUCE_T(f32, float)
+DEF_REDUCE_T(f16, half_t)
+DEF_REDUCE_T(i64, int64_t)
+
+// ---------------------------------------------------------------- logSoftmax
+
+// logSoftmax (BackendCPU.swift:1000-1038): max, sum of expf(x - max), x - (logf(sum) + max),
+// all in Float. Rows: one wave per row; the row is re-read from L1/L2 for passes 2 and 3.
+template <typename T> __device__ __forceinline__ void log_softmax_rows_impl(const hck_reduce_args& p) {
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t row = blockIdx.x * (HCK_BLOCK / 64) + (threadIdx.x >> 6);
+  if (row >= p.outer) return;
+  const uint32_t n = p.reduce;
+  const T* in = (const T*)p.in + (size_t)row * n;
+  T* out = (T*)p.out + (size_t)row * n;
+  // NaNs are skipped by the strict compare here and on the CPU alike; any NaN in the row
+  // then turns the exp-sum, and with it the whole row, into NaN on both.
+  float m = -INFINITY;
+  for (uint32_t k = lane; k < n; k += 64) {
+    float x = (float)in[k];
+    if (x > m) m = x;
+  }
+  m = wave_reduce(m, MaxOp());
+  float s = 0.0f;
+  for (uint32_t k = lane; k < n; k += 64) s += expf((float)in[k] - m);
+  s = wave_reduce(s, SumOp());
+  const float log_sum = logf(s) + m;
+  for (uint32_t k = lane; k < n; k += 64) out[k] = (T)((float)in[k] - log_sum);
+}
+
+// Columns: one lane per (outer, inner) pair, lanes along inner.
+template <typename T> __device__ __forceinline__ void log_softmax_cols_impl(const hck_reduce_args& p) {
+  const uint32_t j = blockIdx.x * HCK_BLOCK + threadIdx.x;
+  const uint32_t i = blockIdx.y;
+  if (j >= p.inner) return;
+  const size_t base = (size_t)i * p.reduce * p.inner + j;
+  const T* in = (const T*)p.in + base;
+  T* out = (T*)p.out + base;
+  float m = 0.0f;
+  for (uint32_t k = 0; k < p.reduce; k++) {
+    float x = (float)in[(size_t)k * p.inner];
+    if (k == 0 || x > m) m = x;
+  }
+  float s = 0.0f;
+  for (uint32_t k = 0; k < p.reduce; k++) s += expf((float)in[(size_t)k * p.inner] - m);
+  const float log_sum = logf(s) + m;
+  for (uint32_t k = 0; k < p.reduce; k++)
+    out[(size_t)k * p.inner] = (T)((float)in[(size_t)k * p.inner] - log_sum);
+}
+
+HC_KERNEL void hc_log_softmax_rows_f32(hck_reduce_args p) { log_softmax_rows_impl<float>(p); }
+HC_KERNEL void hc_log_softmax_rows_f16(hck_reduce_args p) { log_softmax_rows_impl<half_t>(p); }
+HC_KERNEL void hc_log_softmax_cols_f32(hck_reduce_args p) { log_softmax_cols_impl<float>(p); }
+HC_KERNEL void hc_log_softmax_cols_f16(hck_reduce_args p) { log_softmax_cols_impl<half_t>(p); }
+
+// ---------------------------------------------------------------- normalize
+
+// normalize for inner == 1, fused: the base-class composition (Backend.swift:265-327)
+//   mean = sum(x) * (1/n); c = x - mean; var = sum(c^2) * (1/n);
+//   out = c * (var + eps)^-0.5
+// with every intermediate rounded to the tensor dtype where the composed backend calls
+// would have stored it. One wave per row; c^2 is x*x for fp32 (pow special case) and
+// powf(x, 2) for fp16 (generic path), as on the CPU.
+template <typename T> __device__ __forceinline__ void normalize_rows_impl(const hck_reduce_args& p) {
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t row = blockIdx.x * (HCK_BLOCK / 64) + (threadIdx.x >> 6);
+  if (row >= p.outer) return;
+  const uint32_t n = p.reduce;
+  const T* in = (const T*)p.in + (size_t)row * n;
+  T* out = (T*)p.out + (size_t)row * n;
+  const float inv_n = 1.0f / (float)n;
+  float s = 0.0f;
+  for (uint32_t k = lane; k < n; k += 64) s += (float)in[k];
+  s = round_through<T>(wave_reduce(s, SumOp()));
+  const float mean = round_through<T>(s * inv_n);
+  float sq = 0.0f;
+  for (uint32_t k = lane; k < n; k += 64) {
+    float c = round_through<T>((float)in[k] - mean);
+    float c2 = sizeof(T) == 4 ? c * c : 1.0f * 1.0f * powf(c, 2.0f);
+    sq += round_through<T>(c2);
+  }
+  sq = round_through<T>(wave_reduce(sq, SumOp()));
+  const float var = round_through<T>(sq * inv_n);
+  const float shifted = round_through<T>(var + p.eps);
+  const float normer = round_through<T>(1.0f * 1.0f * powf(shifted, -0.5f));
+  for (uint32_t k = lane; k < n; k += 64) {
+    float c = round_through<T>((float)in[k] - mean);
+    out[k] = (T)(c * normer);
+  }
+}
+HC_KERNEL void hc_normalize_rows_f32(hck_reduce_args p) { normalize_rows_impl<float>(p); }
+HC_KERNEL void hc_normalize_rows_f16(hck_reduce_args p) { normalize_rows_impl<half_t>(p); }

@@ -1,0 +1,250 @@
+/*
+ * hchip - C ABI of the MI355X (gfx950) compute backend for Honeycrisp.
+ *
+ * This is the whole boundary a `HIPBackend: Backend` subclass binds: a context
+ * that owns one device, one in-order HIP stream, a caching device allocator
+ * and the embedded gfx950 code objects, plus one entry point per backend
+ * operation. Plain pointers and sizes only; every function returns 0 on
+ * success or a non-zero hc_status / hipError_t-derived code and never throws
+ * or aborts. hc_last_error_string() gives the message for the calling thread.
+ *
+ * Ordering: all work is enqueued on the context's single stream, so an
+ * operation that consumes the output of an earlier call sees its result, and
+ * hc_free() may be called as soon as the last consumer has been enqueued.
+ * Entry points are thread-safe (one mutex around allocator + launch).
+ *
+ * Layout conventions follow the reference backend interface
+ * (Sources/Honeycrisp/Backend.swift:170-815): dense row-major buffers,
+ * dtype codes in Tensor.DType order (Tensor.swift:24-28), strides in elements.
+ */
+#ifndef HCHIP_H
+#define HCHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct hc_ctx hc_ctx;
+typedef struct hc_event hc_event;
+typedef struct hc_module hc_module;
+typedef struct hc_function hc_function;
+
+/* Tensor.DType (Tensor.swift:24-28); byte sizes 8/1/2/4 (:42-53). */
+typedef enum { HC_I64 = 0, HC_BOOL = 1, HC_F16 = 2, HC_F32 = 3 } hc_dtype;
+/* NumericBinaryOp (BinaryOps.swift:2-8). */
+typedef enum { HC_ADD = 0, HC_MUL = 1, HC_SUB = 2, HC_DIV = 3, HC_MOD = 4 } hc_binary;
+/* ReduceOp (ReduceRepeat.swift:53-58). */
+typedef enum { HC_SUM = 0, HC_PROD = 1, HC_ARGMAX = 2, HC_ARGMIN = 3 } hc_reduce_op;
+/* ComparisonOp (Comparison.swift:4-10). */
+typedef enum { HC_EQ = 0, HC_NE = 1, HC_LT = 2, HC_LE = 3, HC_GT = 4, HC_GE = 5 } hc_compare_op;
+/* ElemwiseOp (Elemwise.swift:13-43), same order. */
+typedef enum {
+  HC_SIN = 0, HC_COS, HC_MINUS_SIN, HC_TAN, HC_TAN_GRAD, HC_ATAN, HC_ATAN_GRAD, HC_ACOS,
+  HC_ACOS_GRAD, HC_ASIN, HC_ASIN_GRAD, HC_EXP, HC_LOG, HC_RECIP, HC_SIGMOID, HC_SIGMOID_GRAD,
+  HC_RELU, HC_RELU_GRAD, HC_ABS, HC_ABS_GRAD, HC_GELU_APPROX, HC_GELU_APPROX_GRAD,
+  HC_GELU_EXACT, HC_GELU_EXACT_GRAD, HC_ERF, HC_ERF_GRAD, HC_FLOOR, HC_CEIL, HC_ROUND,
+  HC_ELEMWISE_COUNT
+} hc_elemwise_op;
+
+/* Status codes. Codes >= HC_ERR_HIP_BASE are HC_ERR_HIP_BASE + hipError_t. They map
+ * onto BackendError (Backend.swift:6-16): ALLOC -> .allocationFailed, LOAD ->
+ * .failedToLoadKernels, UNSUPPORTED -> .notImplemented, everything else ->
+ * .kernelFailed(hc_last_error_string()). */
+typedef enum {
+  HC_OK = 0,
+  HC_ERR_INVALID = 1,     /* bad argument (null pointer, negative count, ndim > 8 ...) */
+  HC_ERR_ALLOC = 2,       /* device or pinned-host allocation failed */
+  HC_ERR_LOAD = 3,        /* code object missing / not loadable / kernel symbol missing */
+  HC_ERR_UNSUPPORTED = 4, /* dtype/op combination this backend leaves to the CPU fallback */
+  HC_ERR_TOO_LARGE = 5,   /* element count beyond the kernel's 32-bit index range */
+  HC_ERR_NO_DEVICE = 6,
+  HC_ERR_HIP_BASE = 1000
+} hc_status;
+
+#define HC_MAX_DIMS 8
+
+/* BroadcastStrides (Broadcast.swift:9-30): virtual shape and, per axis, the stride
+ * into the data buffer in elements (0 on broadcast axes). Element i of the virtual
+ * array maps to data index sum_d strides[d] * ((i / prod(shape[d+1:])) % shape[d])
+ * (Broadcast.swift:72-90). */
+typedef struct {
+  uint32_t ndim;
+  uint32_t reserved;
+  int64_t shape[HC_MAX_DIMS];
+  int64_t strides[HC_MAX_DIMS];
+} hc_strides;
+
+typedef struct {
+  char name[256];
+  char arch[64];
+  int compute_units;
+  int clock_mhz;
+  int wavefront_size;
+  int lds_bytes_per_block;
+  size_t total_mem;
+} hc_device_info;
+
+/* ---- context, errors ---- */
+
+/* Create a context on `device` (HIP ordinal): stream, allocator, code objects.
+ * Replaces MPSBackend.init (BackendMPS.swift:373-466) for this backend. */
+int hc_init(int device, hc_ctx** out);
+void hc_shutdown(hc_ctx* ctx);
+const char* hc_last_error_string(void);
+int hc_get_device_info(hc_ctx* ctx, hc_device_info* out);
+
+/* ---- memory: backs Tensor.Data (Tensor.swift:69-85) and DataAllocator
+ * (Backend.swift:894-896; precedent BackendMPS.swift:468-556) ---- */
+
+/* Size-bucketed caching allocator; bytes == 0 yields a valid 1-byte buffer. */
+int hc_malloc(hc_ctx* ctx, size_t bytes, void** out);
+/* Stream-ordered: the block becomes reusable by later hc_malloc calls on the
+ * same stream, so freeing right after the last consumer was enqueued is safe. */
+int hc_free(hc_ctx* ctx, void* ptr);
+/* Return cached blocks to the driver (waits for the stream first). */
+int hc_trim(hc_ctx* ctx);
+/* Bytes currently handed out / held in the cache. */
+int hc_mem_stats(hc_ctx* ctx, size_t* in_use, size_t* cached);
+/* Pinned host staging memory (hipHostMalloc). */
+int hc_host_alloc(hc_ctx* ctx, size_t bytes, void** out);
+int hc_host_free(hc_ctx* ctx, void* ptr);
+/* Blocking copies ordered after everything already enqueued: what Tensor.Data.onCPU /
+ * mutateOnCPU need (Tensor.swift:74-84). */
+int hc_memcpy_h2d(hc_ctx* ctx, void* dst, const void* src, size_t bytes);
+int hc_memcpy_d2h(hc_ctx* ctx, void* dst, const void* src, size_t bytes);
+int hc_memcpy_d2d(hc_ctx* ctx, void* dst, const void* src, size_t bytes);
+/* Enqueue-only copies; the host pointer must be pinned and stay valid until a sync. */
+int hc_memcpy_h2d_async(hc_ctx* ctx, void* dst, const void* src, size_t bytes);
+int hc_memcpy_d2h_async(hc_ctx* ctx, void* dst, const void* src, size_t bytes);
+
+/* ---- stream, events: Tensor.Data.wait() (Tensor.swift:72) and timing ---- */
+
+int hc_sync(hc_ctx* ctx);
+int hc_event_create(hc_ctx* ctx, hc_event** out);
+int hc_event_record(hc_ctx* ctx, hc_event* ev);
+int hc_event_sync(hc_event* ev);
+/* 0 = complete, 1 = still pending, other = error. */
+int hc_event_query(hc_event* ev);
+int hc_event_elapsed_ms(hc_event* start, hc_event* stop, float* ms);
+int hc_event_destroy(hc_event* ev);
+/* Run fn(user) on a runtime thread once prior work completes: the hook a Swift
+ * continuation resumes from (precedent BackendMPS.swift:2663-2720). */
+int hc_launch_host_func(hc_ctx* ctx, void (*fn)(void*), void* user);
+
+/* ---- raw module API (thin wrappers over hipModuleLoadData / hipModuleGetFunction /
+ * hipModuleLaunchKernel) for callers that bring their own gfx950 code objects ---- */
+
+int hc_module_load(hc_ctx* ctx, const void* image, size_t bytes, hc_module** out);
+int hc_module_unload(hc_ctx* ctx, hc_module* mod);
+int hc_module_get_function(hc_module* mod, const char* name, hc_function** out);
+int hc_launch(hc_ctx* ctx, hc_function* fn, const uint32_t grid[3], const uint32_t block[3],
+              uint32_t shared_bytes, const void* kernarg, size_t kernarg_bytes);
+
+/* ---- operations ----
+ * Every pointer below is a device pointer from hc_malloc unless stated otherwise;
+ * outputs are caller-allocated, dense, and never alias inputs. */
+
+/* Backend.broadcast (Backend.swift:170-172; CPU BackendCPU.swift:255-265). */
+int hc_broadcast(hc_ctx* ctx, int dtype, const void* a, const hc_strides* as, void* out);
+
+/* Backend.binaryOp(BroadcastData, BroadcastData) (Backend.swift:178-185; CPU
+ * BackendCPU.swift:267-314). Float dtypes compute in fp32 and round once; mod is
+ * Python-style (TensorElement.swift:124-132, 214-222). */
+int hc_binary_op(hc_ctx* ctx, int op, int dtype, const void* a, const hc_strides* as,
+                 const void* b, const hc_strides* bs, void* out);
+
+/* Backend.binaryOp(Tensor.Data, T) and (T, Tensor.Data) (Backend.swift:190-209; CPU
+ * BackendCPU.swift:316-405). `sf` is used for float dtypes, `si` for int64. fp32
+ * follows the CPU's vDSP forms: x / s == x * (1 / s), x - s == x + (-s),
+ * s - x == x * -1 + s. */
+int hc_binary_op_scalar(hc_ctx* ctx, int op, int dtype, const void* a, float sf, int64_t si,
+                        int scalar_first, void* out, size_t count);
+
+/* Backend.mulAdd / addMul (Backend.swift:240-257; CPU BackendCPU.swift:445-539). */
+int hc_mul_add(hc_ctx* ctx, int dtype, const void* input, const hc_strides* is,
+               const void* coeff, const hc_strides* cs, const void* bias, const hc_strides* bs,
+               void* out);
+int hc_add_mul(hc_ctx* ctx, int dtype, const void* input, const hc_strides* is, const void* bias,
+               const hc_strides* bs, const void* coeff, const hc_strides* cs, void* out);
+
+/* Backend.compare (Backend.swift:457-486; CPU BackendCPU.swift:541-624): bool (1 byte) out. */
+int hc_compare(hc_ctx* ctx, int op, int dtype, const void* a, const hc_strides* as,
+               const void* b, const hc_strides* bs, void* out);
+int hc_compare_scalar(hc_ctx* ctx, int op, int dtype, const void* a, float sf, int64_t si,
+                      int scalar_first, void* out, size_t count);
+
+/* Backend.cast (Backend.swift:489-494; CPU BackendCPU.swift:626-646): f32->f16 is RNE
+ * with overflow to inf; float->int64 truncates; anything->bool is (x != 0). */
+int hc_cast(hc_ctx* ctx, const void* in, int in_type, void* out, int out_type, size_t count);
+
+/* Backend.pow (Backend.swift:500-507; CPU BackendCPU.swift:648-702):
+ * out = scale * scales[i] * x^b with the fp32 special cases b in {2, -1, 1}.
+ * (bf, scalef) apply to float dtypes, (bi, scalei) to int64; scales may be NULL. */
+int hc_pow(hc_ctx* ctx, int dtype, const void* in, float bf, float scalef, int64_t bi,
+           int64_t scalei, const void* scales, void* out, size_t count);
+
+/* Backend.elemwise (Backend.swift:770-774; CPU BackendCPU.swift:1748-1766; formulas
+ * Elemwise.swift:44-183): out = f(x) * scales[i], float dtypes only; scales may be NULL. */
+int hc_elemwise(hc_ctx* ctx, int op, int dtype, const void* in, const void* scales, void* out,
+                size_t count);
+
+/* Backend.reduce (Backend.swift:524-531; CPU BackendCPU.swift:784-886): input viewed as
+ * [outer, reduce, inner]; sum/prod keep the dtype, argmax/argmin write int64 and return
+ * the first extremum (strict compare from k = 0; a NaN at k > 0 never wins, a NaN at
+ * k = 0 yields 0). */
+int hc_reduce(hc_ctx* ctx, int op, int dtype, const void* in, void* out, int64_t outer,
+              int64_t reduce, int64_t inner);
+
+/* Backend.logSoftmax (Backend.swift:571-575; CPU BackendCPU.swift:1000-1038). */
+int hc_log_softmax(hc_ctx* ctx, int dtype, const void* in, void* out, int64_t outer,
+                   int64_t reduce, int64_t inner);
+
+/* Backend.normalize (Backend.swift:265-327: two-pass mean / biased variance,
+ * (var + eps)^-0.5, every intermediate rounded to `dtype`). */
+int hc_normalize(hc_ctx* ctx, int dtype, const void* in, void* out, int64_t outer,
+                 int64_t reduce, int64_t inner, float eps);
+
+/* Backend.gather (Backend.swift:609-616; CPU BackendCPU.swift:1108-1147) with
+ * ScatterGatherIndices flattened (ScatterGather.swift:21-45):
+ * out[(i*out_count + j)*inner + k] = in[(i*middle + idx)*inner + k],
+ * idx = indices[idx_strides(flat out index)] (int64, no bounds check, no wrap). */
+int hc_gather(hc_ctx* ctx, int dtype, const void* in, const void* indices,
+              const hc_strides* idx_strides, void* out, int64_t outer, int64_t middle,
+              int64_t out_count, int64_t inner);
+
+/* Backend.when (Backend.swift:633-641; CPU BackendCPU.swift:1190-1220); a scalar branch is
+ * a 1-element buffer with all-zero strides, as CPUBackend.tensorOrScalarData makes it. */
+int hc_when(hc_ctx* ctx, int dtype, const void* mask, const hc_strides* ms, const void* a,
+            const hc_strides* as, const void* b, const hc_strides* bs, void* out);
+
+/* Backend.matmul / batchedMatmul (Backend.swift:650-669; CPU BackendCPU.swift:1222-1313).
+ * rows/inner/cols are M/K/N after the transposes; A is [M,K] ([K,M] if trans_a), B is
+ * [K,N] ([N,K] if trans_b), C is [M,N] ([N,M] if trans_out); matrix m of the batch is at
+ * element offsets m*M*K, m*K*N, m*M*N. fp16 accumulates in fp32 and rounds once. */
+int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, int trans_a, const void* b,
+              int trans_b, int trans_out, int64_t rows, int64_t inner, int64_t cols, void* out);
+
+/* Backend.triangular (Backend.swift:674-680; CPU BackendCPU.swift:1315-1348). */
+int hc_triangular(hc_ctx* ctx, int dtype, const void* in, void* out, int64_t batch,
+                  int64_t rows, int64_t cols, int upper, int64_t offset);
+
+/* Backend.constant (Backend.swift:787-791; CPU BackendCPU.swift:1796-1815). */
+int hc_fill(hc_ctx* ctx, int dtype, float vf, int64_t vi, void* out, size_t count);
+
+/* Backend.axisPermutation (Backend.swift:803-805; CPU BackendCPU.swift:1831-1849):
+ * `perm` and `shape` are host arrays of ndim entries; out is int64[prod(shape)]. */
+int hc_axis_permutation(hc_ctx* ctx, const int64_t* perm, const int64_t* shape, int ndim,
+                        void* out);
+
+/* Backend.concat (Backend.swift:777-784; CPU BackendCPU.swift:1768-1794): `inputs` and
+ * `inner_counts` are host arrays of n_inputs entries (device pointers / element counts). */
+int hc_concat(hc_ctx* ctx, int dtype, const void* const* inputs, const int64_t* inner_counts,
+              int n_inputs, int64_t outer, void* out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HCHIP_H */

@@ -1,0 +1,32 @@
+import os
+import sys
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+
+
+@pytest.fixture
+def rng():
+    return np.random.default_rng(1234)
+
+
+@pytest.fixture(scope="session")
+def oracle_backend():
+    from oracle.oracle_backend import OracleBackend
+    return OracleBackend()
+
+
+@pytest.fixture(scope="session")
+def hip_backend():
+    from honeycrisp_amd.backend import HIPBackend
+    backend = HIPBackend()
+    yield backend
+    backend.sync()

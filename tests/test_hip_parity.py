@@ -1,0 +1,424 @@
+"""Parity proper: the HIP path (through the C ABI) against the CPU oracle on the same seeded
+inputs. Bit-exact for integer / index / data-movement work and for element-wise fp32
+arithmetic that involves no libm call; otherwise the reference's own criterion
+(|a-b| <= tol or |a/b-1| <= tol, Assertions.swift:16) with tol 1e-4 for fp32 and 1e-2 for
+fp16, plus a norm-wise bound for GEMMs."""
+import numpy as np
+import pytest
+
+from honeycrisp_amd.descriptors import DType, ElemwiseOp, ReduceDims, ReduceOp
+from honeycrisp_amd.tensor import Tensor
+from backend_cases import assert_close_arrays
+
+pytestmark = pytest.mark.gpu
+
+F32, F16, I64, BOOL = DType.float32, DType.float16, DType.int64, DType.bool
+TOL = {F32: 1e-4, F16: 1e-2}
+
+
+def both(hip, oracle, fn):
+    """Run fn() under each backend; returns (hip result, oracle result) as numpy arrays."""
+    with hip.use():
+        got = fn().numpy()
+    with oracle.use():
+        want = fn().numpy()
+    return got, want
+
+
+def check_exact(hip, oracle, fn):
+    got, want = both(hip, oracle, fn)
+    assert got.dtype == want.dtype and got.shape == want.shape
+    if got.dtype.kind == "f":
+        # same bits, except that any NaN matches any NaN
+        nan = np.isnan(want)
+        assert np.array_equal(np.isnan(got), nan)
+        assert np.array_equal(got[~nan].view(np.uint8), want[~nan].view(np.uint8))
+    else:
+        assert np.array_equal(got, want)
+
+
+def check_close(hip, oracle, fn, tol):
+    got, want = both(hip, oracle, fn)
+    assert got.dtype == want.dtype and got.shape == want.shape
+    assert_close_arrays(got, want, tol, tol)
+    return got, want
+
+
+def rand(rng, shape, dtype, scale=1.0):
+    if dtype == I64:
+        return rng.integers(-50, 50, size=shape)
+    return (rng.standard_normal(shape) * scale).astype(dtype.numpy)
+
+
+# ---------------------------------------------------------------- matmul
+
+GEMM_SHAPES = [(128, 128, 128), (256, 64, 384), (127, 1000, 65), (1, 33, 1), (5, 4097, 3), (200, 8, 136),
+               (64, 0, 16), (129, 257, 131)]
+
+
+@pytest.mark.parametrize("dtype", [F32, F16], ids=["f32", "f16"])
+@pytest.mark.parametrize("shape", GEMM_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_matmul_all_flag_combinations(hip_backend, oracle_backend, dtype, shape):
+    M, K, N = shape
+    rng = np.random.default_rng(100 + M + K + N)
+    a = rand(rng, (M, K), dtype, 1.0 / max(K, 1) ** 0.5)
+    b = rand(rng, (K, N), dtype)
+    for transA in (False, True):
+        for transB in (False, True):
+            for transOut in (False, True):
+                print("matmul", dtype.name, shape, transA, transB, transOut, flush=True)
+                sa = np.ascontiguousarray(a.T) if transA else a
+                sb = np.ascontiguousarray(b.T) if transB else b
+                fn = lambda: Tensor.matmul(Tensor(data=sa), transA, Tensor(data=sb), transB, transOut)
+                got, want = check_close(hip_backend, oracle_backend, fn, TOL[dtype])
+                scale = float(np.max(np.abs(want.astype(np.float64)))) if want.size else 0.0
+                if scale > 0:
+                    err = float(np.max(np.abs(got.astype(np.float64) - want.astype(np.float64))))
+                    assert err / scale <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [F32, F16], ids=["f32", "f16"])
+def test_batched_matmul_attention_shapes(hip_backend, oracle_backend, dtype):
+    """Config 3: batch 32, Q[512,64] x K^T -> [512,512], scale 1/8, then scores x V[512,64]."""
+    rng = np.random.default_rng(4)
+    q = rand(rng, (32, 512, 64), dtype)
+    k = rand(rng, (32, 512, 64), dtype)
+    v = rand(rng, (32, 512, 64), dtype)
+
+    def fn():
+        scores = Tensor.batchedMatmul(Tensor(data=q), False, Tensor(data=k), True, False) * 0.125
+        return Tensor.batchedMatmul(scores.softmax(), False, Tensor(data=v), False, False)
+
+    def scores_fn():
+        return Tensor.batchedMatmul(Tensor(data=q), False, Tensor(data=k), True, False) * 0.125
+
+    check_close(hip_backend, oracle_backend, scores_fn, TOL[dtype])
+    check_close(hip_backend, oracle_backend, fn, TOL[dtype])
+
+
+def test_batched_matmul_all_flags_small(hip_backend, oracle_backend):
+    rng = np.random.default_rng(5)
+    for dtype in (F32, F16):
+        a = rand(rng, (7, 24, 40), dtype)
+        b = rand(rng, (7, 40, 56), dtype)
+        for transA in (False, True):
+            for transB in (False, True):
+                for transOut in (False, True):
+                    sa = np.ascontiguousarray(a.transpose(0, 2, 1)) if transA else a
+                    sb = np.ascontiguousarray(b.transpose(0, 2, 1)) if transB else b
+                    fn = lambda: Tensor.batchedMatmul(Tensor(data=sa), transA, Tensor(data=sb), transB, transOut)
+                    check_close(hip_backend, oracle_backend, fn, TOL[dtype])
+
+
+def test_matmul_fp16_4096_against_oracle_slab_and_identity(hip_backend, oracle_backend):
+    """Config 2 at full size: every layout; a 96-row slab of each product is checked against
+    the oracle, and A x I == A exactly."""
+    rng = np.random.default_rng(2)
+    n = 4096
+    a = (rng.standard_normal((n, n)) / np.sqrt(n)).astype(np.float16)
+    b = rng.standard_normal((n, n)).astype(np.float16)
+    rows = np.r_[0:32, 2000:2032, n - 32:n]
+    with oracle_backend.use():
+        want = Tensor.matmul(Tensor(data=a[rows]), False, Tensor(data=b), False, False).numpy()
+    with hip_backend.use():
+        ta, tb = Tensor(data=a), Tensor(data=b)
+        tat, tbt = Tensor(data=np.ascontiguousarray(a.T)), Tensor(data=np.ascontiguousarray(b.T))
+        for transA, transB in [(False, False), (False, True), (True, False), (True, True)]:
+            print("4096^3 layout", transA, transB, flush=True)
+            out = Tensor.matmul(tat if transA else ta, transA, tbt if transB else tb, transB, False).numpy()
+            assert_close_arrays(out[rows], want, 1e-2, 1e-2)
+        eye = Tensor(data=np.eye(n, dtype=np.float16))
+        assert np.array_equal(Tensor.matmul(ta, False, eye, False, False).numpy(), a)
+        assert np.array_equal(Tensor.matmul(eye, False, tb, False, False).numpy(), b)
+
+
+def test_matmul_fp32_1024(hip_backend, oracle_backend):
+    """Config 1: fp32 [1024,1024] x [1024,1024], N(0,1) entries, no transposes."""
+    rng = np.random.default_rng(1)
+    a = rng.standard_normal((1024, 1024)).astype(np.float32)
+    b = rng.standard_normal((1024, 1024)).astype(np.float32)
+    got, want = check_close(hip_backend, oracle_backend,
+                            lambda: Tensor.matmul(Tensor(data=a), False, Tensor(data=b), False, False), 1e-4)
+    assert np.max(np.abs(got - want)) / np.max(np.abs(want)) <= 1e-4
+
+
+# ---------------------------------------------------------------- element-wise
+
+BCAST_PAIRS = [([512, 1024], [1, 1024]), ([512, 1024], [512, 1]), ([33, 1025], [33, 1025]), ([6], [3, 6]),
+               ([3, 1, 6], [1, 2, 6]), ([1, 3, 1, 3, 1], [3, 1, 3, 1, 3]), ([3, 1, 3, 1, 3, 1], [1, 3, 1, 3, 1, 3]),
+               ([8, 8, 64, 64], [64, 64]), ([2, 3, 4, 5, 6, 7, 8], [1, 3, 1, 5, 1, 7, 1]), ([], [4, 4]), ([0, 5], [5])]
+
+
+@pytest.mark.parametrize("dtype", [F32, F16, I64], ids=["f32", "f16", "i64"])
+def test_binary_broadcast_ops(hip_backend, oracle_backend, dtype):
+    rng = np.random.default_rng(11)
+    for sa, sb in BCAST_PAIRS:
+        a = rand(rng, sa, dtype, 3.0)
+        b = rand(rng, sb, dtype, 3.0)
+        if dtype == I64:
+            b = np.where(b == 0, 7, b)
+        print("binary", dtype.name, sa, sb, flush=True)
+        for op in (lambda x, y: x + y, lambda x, y: x - y, lambda x, y: x * y, lambda x, y: x / y,
+                   lambda x, y: x % y):
+            check_exact(hip_backend, oracle_backend,
+                        lambda: op(Tensor(data=a, shape=sa, dtype=dtype), Tensor(data=b, shape=sb, dtype=dtype)))
+        for op in (lambda x, y: x.mul(y, thenAdd=x), lambda x, y: x.add(y, thenMul=y)):
+            check_exact(hip_backend, oracle_backend,
+                        lambda: op(Tensor(data=a, shape=sa, dtype=dtype), Tensor(data=b, shape=sb, dtype=dtype)))
+        for op in (lambda x, y: x < y, lambda x, y: x == y, lambda x, y: x >= y, lambda x, y: x != y):
+            check_exact(hip_backend, oracle_backend,
+                        lambda: op(Tensor(data=a, shape=sa, dtype=dtype), Tensor(data=b, shape=sb, dtype=dtype)))
+
+
+@pytest.mark.parametrize("dtype", [F32, F16, I64], ids=["f32", "f16", "i64"])
+def test_scalar_ops(hip_backend, oracle_backend, dtype):
+    rng = np.random.default_rng(12)
+    for n in (1, 7, 4096, 100003):
+        x = rand(rng, (n,), dtype, 4.0)
+        if dtype == I64:
+            x = np.where(x == 0, 3, x)
+        for s in ([3, -7] if dtype == I64 else [3, 0.125, -2.5]):
+            for op in (lambda t: t + s, lambda t: t - s, lambda t: t * s, lambda t: t / s, lambda t: t % s,
+                       lambda t: s + t, lambda t: s - t, lambda t: s * t, lambda t: s / t, lambda t: s % t,
+                       lambda t: t < s, lambda t: s >= t, lambda t: t == s):
+                check_exact(hip_backend, oracle_backend, lambda: op(Tensor(data=x, dtype=dtype)))
+
+
+@pytest.mark.parametrize("dtype", [F32, F16], ids=["f32", "f16"])
+def test_elemwise_all_ops(hip_backend, oracle_backend, dtype):
+    rng = np.random.default_rng(13)
+    x = np.concatenate([rng.standard_normal(20000) * 2.5, np.linspace(-6, 6, 1203), [0.0, -0.0, 25.0, -25.0]])
+    x = x.astype(dtype.numpy)
+    unit = np.clip(x.astype(np.float32) / 7.0, -0.98, 0.98).astype(dtype.numpy)
+    scales = rng.standard_normal(x.size).astype(dtype.numpy)
+    # fp16 keeps the reference's x100 widening (BackendTests.swift:1065)
+    tol = 1e-4 if dtype == F32 else 1e-2
+    for op in ElemwiseOp:
+        src = unit if op in (ElemwiseOp.acos, ElemwiseOp.asin, ElemwiseOp.acosGrad, ElemwiseOp.asinGrad) else x
+        if op == ElemwiseOp.log:
+            src = np.abs(x) + dtype.numpy(0.01)
+        print("elemwise", op.name, dtype.name, flush=True)
+        for sc in (None, scales):
+            def fn():
+                from honeycrisp_amd.backend import Backend
+                be = Backend.current()
+                t = Tensor(data=src)
+                s = Tensor(data=sc).data if sc is not None else None
+                return Tensor(dataHandle=be.elemwise(t.data, op, s, src.size, dtype), shape=[src.size], dtype=dtype)
+            if op in (ElemwiseOp.relu, ElemwiseOp.reluGrad, ElemwiseOp.abs, ElemwiseOp.absGrad, ElemwiseOp.floor,
+                      ElemwiseOp.ceil, ElemwiseOp.round, ElemwiseOp.recip):
+                check_exact(hip_backend, oracle_backend, fn)
+            else:
+                check_close(hip_backend, oracle_backend, fn, tol)
+
+
+def test_gelu_tail_is_judged_abs_or_rel(hip_backend, oracle_backend):
+    """For x << 0 the (1 + tanh) term of the approximate GELU cancels to about one bit, so a
+    1-ulp expf difference doubles the value at magnitude 1e-7: abs <= 1e-4 is what holds."""
+    x = np.linspace(-12, -3, 4001).astype(np.float32)
+    got, want = check_close(hip_backend, oracle_backend, lambda: Tensor(data=x).gelu(), 1e-4)
+    assert np.max(np.abs(got - want)) < 1e-6
+
+
+@pytest.mark.parametrize("dtype", [F32, F16, I64], ids=["f32", "f16", "i64"])
+def test_pow(hip_backend, oracle_backend, dtype):
+    rng = np.random.default_rng(14)
+    x = np.abs(rand(rng, (5003,), dtype, 2.0)) + (1 if dtype == I64 else dtype.numpy(0.05))
+    sc = rand(rng, (5003,), dtype)
+    from honeycrisp_amd.backend import Backend
+    for b, scale in ([(2, 1), (3, 2)] if dtype == I64 else [(2.0, 1.0), (2.0, 3.0), (-1.0, 0.5), (1.0, 4.0), (0.5, 1.0),
+                                                          (-0.5, 1.0), (3.0, 2.0), (-1.5, 0.25)]):
+        for scales in (None, sc):
+            def fn():
+                be = Backend.current()
+                s = Tensor(data=scales, dtype=dtype).data if scales is not None else None
+                data = be.pow(Tensor(data=x, dtype=dtype).data, b, scale, s, x.size, dtype)
+                return Tensor(dataHandle=data, shape=[x.size], dtype=dtype)
+            if dtype == F32 and b in (2.0, -1.0, 1.0) or dtype == I64:
+                check_exact(hip_backend, oracle_backend, fn)
+            else:
+                check_close(hip_backend, oracle_backend, fn, 1e-4 if dtype == F32 else 1e-2)
+
+
+def test_cast_all_pairs(hip_backend, oracle_backend):
+    rng = np.random.default_rng(15)
+    f = np.concatenate([rng.standard_normal(3001) * 100, [0.0, -0.0, 0.4, -0.6, 65519.0, 65520.0, 1e9, -1e9, 5e-8]])
+    srcs = {F32: f.astype(np.float32), F16: rng.standard_normal(3001).astype(np.float16) * np.float16(50),
+            I64: rng.integers(-2**40, 2**40, size=3001), BOOL: rng.integers(0, 2, size=3001).astype(np.bool_)}
+    for it, src in srcs.items():
+        for ot in DType:
+            if it == F32 and ot == I64:
+                src_ = src[np.abs(src) < 1e6]
+            else:
+                src_ = src
+            check_exact(hip_backend, oracle_backend, lambda: Tensor(data=src_, dtype=it).cast(ot))
+
+
+def test_when_fill_triangular_concat_broadcast(hip_backend, oracle_backend):
+    rng = np.random.default_rng(16)
+    mask = rng.integers(0, 2, size=(6, 1, 40)).astype(np.bool_)
+    for dtype in (F32, F16, I64, BOOL):
+        a = rand(rng, (5, 40), dtype) if dtype != BOOL else rng.integers(0, 2, size=(5, 40)).astype(np.bool_)
+        b = rand(rng, (40,), dtype) if dtype != BOOL else rng.integers(0, 2, size=(40,)).astype(np.bool_)
+        check_exact(hip_backend, oracle_backend,
+                    lambda: Tensor(data=mask).when(Tensor(data=a, dtype=dtype), Tensor(data=b, dtype=dtype)))
+        if dtype != BOOL:
+            check_exact(hip_backend, oracle_backend, lambda: Tensor(data=mask).when(Tensor(data=a, dtype=dtype), 2))
+            check_exact(hip_backend, oracle_backend, lambda: Tensor(data=mask).when(0, -1e4 if dtype != I64 else -7, dtype=dtype))
+        m = rand(rng, (3, 17, 23), dtype) if dtype != BOOL else rng.integers(0, 2, size=(3, 17, 23)).astype(np.bool_)
+        for off in (-20, -3, 0, 2, 30):
+            check_exact(hip_backend, oracle_backend, lambda: Tensor(data=m, dtype=dtype).tril(off))
+            check_exact(hip_backend, oracle_backend, lambda: Tensor(data=m, dtype=dtype).triu(off))
+        check_exact(hip_backend, oracle_backend,
+                    lambda: Tensor.concat([Tensor(data=m, dtype=dtype), Tensor(data=m[:, :5], dtype=dtype)], axis=1))
+        check_exact(hip_backend, oracle_backend,
+                    lambda: Tensor.concat([Tensor(data=m, dtype=dtype), Tensor(data=m[:, :, :9], dtype=dtype)], axis=2))
+        check_exact(hip_backend, oracle_backend, lambda: Tensor(data=b, dtype=dtype).expand([7, 3, 40]))
+        check_exact(hip_backend, oracle_backend, lambda: Tensor(data=a, dtype=dtype).reshape([5, 1, 40]).expand([5, 6, 40]))
+        check_exact(hip_backend, oracle_backend, lambda: Tensor(data=a, dtype=dtype).repeating(1, 3))
+        check_exact(hip_backend, oracle_backend, lambda: Tensor.constant(1 if dtype == BOOL else 3, [1001], dtype))
+
+
+# ---------------------------------------------------------------- reductions
+
+REDUCE_SHAPES = [(8, 4096, 1), (37, 513, 1), (5, 1, 1), (3, 7, 1), (1, 100000, 1), (64, 1024, 1), (4, 33, 65),
+                 (1, 300, 4096), (17, 2, 3), (9, 8192, 2)]
+
+
+@pytest.mark.parametrize("dtype", [F32, F16, I64], ids=["f32", "f16", "i64"])
+def test_reduce_all_ops(hip_backend, oracle_backend, dtype):
+    from honeycrisp_amd.backend import Backend
+    rng = np.random.default_rng(17)
+    for outer, red, inner in REDUCE_SHAPES:
+        x = rand(rng, (outer, red, inner), dtype)
+        if dtype != I64:
+            # plant ties so that first-occurrence matters
+            x = np.round(x * 4) / dtype.numpy(4)
+        dims = ReduceDims(outer, red, inner)
+        print("reduce", dtype.name, (outer, red, inner), flush=True)
+        for op in ReduceOp:
+            if op == ReduceOp.prod:
+                src = (x % 3 + 1) if dtype == I64 else (np.sign(x) + (x == 0)) * (1 + np.abs(x) / dtype.numpy(64))
+                src = src[:, :min(red, 60)].astype(dtype.numpy)
+                d = ReduceDims(outer, src.shape[1], inner)
+            else:
+                src, d = x, dims
+            def fn():
+                be = Backend.current()
+                data = be.reduce(Tensor(data=src, dtype=dtype).data, op, d, dtype)
+                return Tensor(dataHandle=data, shape=[d.outCount], dtype=I64 if op.isIntOut else dtype)
+            if op.isIntOut or dtype == I64:
+                check_exact(hip_backend, oracle_backend, fn)
+            else:
+                # summation order differs from the sequential CPU loop; fp16 sums of up to 1e5
+                # unit-scale terms are judged relative to the magnitude a sequential fp32 sum has
+                got, want = both(hip_backend, oracle_backend, fn)
+                atol = TOL[dtype] * max(1.0, float(np.sqrt(d.reduceCount)))
+                assert_close_arrays(got, want, atol, TOL[dtype])
+
+
+def test_argmax_nan_and_tie_rules(hip_backend, oracle_backend):
+    """Bit-exact first-extremum semantics, including NaN placement (BackendCPU.swift:848-877)."""
+    rng = np.random.default_rng(18)
+    nan, inf = np.nan, np.inf
+    base = np.array([[1, nan, 3, 3], [nan, 5, 9, 1], [-inf, nan, -inf, -inf], [2, 2, nan, 2], [inf, nan, inf, 0],
+                     [nan, nan, nan, nan], [nan, inf, -inf, 0]], dtype=np.float32)
+    for dtype in (F32, F16):
+        for op in (ReduceOp.argmax, ReduceOp.argmin):
+            check_exact(hip_backend, oracle_backend, lambda: Tensor(data=base, dtype=dtype).reduce(op, axis=1))
+            check_exact(hip_backend, oracle_backend, lambda: Tensor(data=base, dtype=dtype).reduce(op, axis=0))
+    # long rows with few distinct values and NaNs sprinkled in, rows and columns
+    x = rng.integers(-2, 3, size=(64, 5000)).astype(np.float32)
+    x[rng.random(x.shape) < 0.01] = nan
+    x[::7, 0] = nan
+    for op in (ReduceOp.argmax, ReduceOp.argmin):
+        check_exact(hip_backend, oracle_backend, lambda: Tensor(data=x).reduce(op, axis=1))
+        check_exact(hip_backend, oracle_backend, lambda: Tensor(data=x).reduce(op, axis=0))
+        check_exact(hip_backend, oracle_backend, lambda: Tensor(data=x[:, :777]).reduce(op, axis=1))
+    # max / min = arg-reduction + gather
+    y = rng.standard_normal((33, 4096)).astype(np.float32)
+    check_exact(hip_backend, oracle_backend, lambda: Tensor(data=y).max(axis=1))
+    check_exact(hip_backend, oracle_backend, lambda: Tensor(data=y).min(axis=0))
+    check_exact(hip_backend, oracle_backend, lambda: Tensor(data=y).max())
+
+
+@pytest.mark.parametrize("dtype", [F32, F16], ids=["f32", "f16"])
+def test_log_softmax_and_normalize(hip_backend, oracle_backend, dtype):
+    rng = np.random.default_rng(19)
+    for shape, axis in [((64, 256), 1), ((16, 8, 32, 32), 3), ((5, 1000), 1), ((7, 33, 9), 1), ((300, 4), 0),
+                        ((2, 1), 1), ((3, 10000), 1)]:
+        x = rand(rng, shape, dtype, 3.0)
+        print("logsoftmax/normalize", dtype.name, shape, axis, flush=True)
+        check_close(hip_backend, oracle_backend, lambda: Tensor(data=x).logSoftmax(axis=axis), TOL[dtype])
+        tol = 1e-4 if dtype == F32 else 2e-2   # the reference's own normalize tolerance (BackendTests.swift:196-197)
+        check_close(hip_backend, oracle_backend, lambda: Tensor(data=x).normalize(axis=axis, eps=1e-5), tol)
+        check_close(hip_backend, oracle_backend, lambda: Tensor(data=x).normalize(axis=axis, eps=0.3), tol)
+    neg = np.full((4, 50), -np.inf, dtype=dtype.numpy)
+    neg[1, 3] = 0
+    neg[2, 7] = np.nan
+    check_close(hip_backend, oracle_backend, lambda: Tensor(data=neg).logSoftmax(), TOL[dtype])
+
+
+# ---------------------------------------------------------------- gather / permute
+
+def test_gather_forms(hip_backend, oracle_backend):
+    rng = np.random.default_rng(20)
+    for dtype in (F32, F16, I64, BOOL):
+        table = rand(rng, (1000, 64), dtype) if dtype != BOOL else rng.integers(0, 2, size=(1000, 64)).astype(np.bool_)
+        ids = rng.integers(0, 1000, size=(4099,))
+        print("gather", dtype.name, flush=True)
+        check_exact(hip_backend, oracle_backend, lambda: Tensor(data=table, dtype=dtype).gather(0, Tensor(data=ids)))
+        x = table.reshape(10, 100, 64)
+        idx3 = rng.integers(0, 100, size=(10, 7, 64))
+        check_exact(hip_backend, oracle_backend, lambda: Tensor(data=x, dtype=dtype).gather(1, Tensor(data=idx3)))
+        idx_last = rng.integers(0, 64, size=(10, 100, 5))
+        check_exact(hip_backend, oracle_backend, lambda: Tensor(data=x, dtype=dtype).gather(2, Tensor(data=idx_last)))
+        idx_b = rng.integers(0, 100, size=(1, 9, 1))
+        check_exact(hip_backend, oracle_backend, lambda: Tensor(data=x, dtype=dtype).gather(1, Tensor(data=idx_b)))
+        odd = table[:, :37]
+        check_exact(hip_backend, oracle_backend, lambda: Tensor(data=odd, dtype=dtype).gather(0, Tensor(data=ids[:300])))
+        check_exact(hip_backend, oracle_backend, lambda: Tensor(data=x, dtype=dtype).t())
+        check_exact(hip_backend, oracle_backend, lambda: Tensor(data=x, dtype=dtype).swap(0, 1))
+        check_exact(hip_backend, oracle_backend, lambda: Tensor(data=x, dtype=dtype).move(2, 0))
+        check_exact(hip_backend, oracle_backend, lambda: Tensor(data=x, dtype=dtype)[2:9, ..., 5])
+
+
+def test_axis_permutation(hip_backend, oracle_backend):
+    from honeycrisp_amd.backend import Backend
+    for perm, shape in [([1, 0], [256, 8]), ([2, 0, 1], [3, 4, 5]), ([0], [7]), ([3, 1, 0, 2], [2, 3, 4, 5]),
+                        ([1, 0], [1, 1]), ([4, 3, 2, 1, 0], [2, 3, 4, 5, 6])]:
+        def fn():
+            data = Backend.current().axisPermutation(perm, shape)
+            return Tensor(dataHandle=data, shape=[int(np.prod(shape))], dtype=I64)
+        check_exact(hip_backend, oracle_backend, fn)
+
+
+# ---------------------------------------------------------------- config 4 at full size
+
+def test_bandwidth_ops_full_size(hip_backend, oracle_backend):
+    """Config 4: X[8192,4096] + bias[1,4096], GELU, sum / max / argmax over axis 1, and an
+    int64 gather of 65536 ids from a [32000,1024] table, all at the benchmark's sizes."""
+    rng = np.random.default_rng(7)
+    x = rng.standard_normal((8192, 4096)).astype(np.float32)
+    bias = np.random.default_rng(8).standard_normal((1, 4096)).astype(np.float32)
+    with hip_backend.use():
+        tx = Tensor(data=x)
+        h = tx + Tensor(data=bias)
+        g = h.gelu()
+        s = h.sum(axis=1)
+        am = h.argmax(axis=1)
+        mx = h.max(axis=1)
+        h_np, g_np, s_np, am_np, mx_np = h.numpy(), g.numpy(), s.numpy(), am.numpy(), mx.numpy()
+    want_h = x + bias
+    assert np.array_equal(h_np, want_h)                        # IEEE add: bit-exact
+    assert np.array_equal(am_np, want_h.argmax(axis=1))        # first maximum
+    assert np.array_equal(mx_np, want_h.max(axis=1))
+    assert_close_arrays(s_np, want_h.astype(np.float64).sum(axis=1), 1e-2, 1e-4)
+    with oracle_backend.use():
+        g_want = Tensor(data=want_h).gelu().numpy()
+    assert_close_arrays(g_np, g_want, 1e-4, 1e-4)
+    table = np.random.default_rng(10).standard_normal((32000, 1024)).astype(np.float32)
+    ids = np.random.default_rng(9).integers(0, 32000, size=(65536,))
+    with hip_backend.use():
+        out = Tensor(data=table).gather(0, Tensor(data=ids)).numpy()
+    assert np.array_equal(out, table[ids])

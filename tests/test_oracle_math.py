@@ -1,0 +1,333 @@
+"""Pins the CPU oracle against what the mathematics fixes, independently of the oracle's own
+formulas: numpy / scipy library routines, brute force on small inputs, closed forms and
+hand-derived special cases (ties, NaNs, rounding boundaries). No GPU needed."""
+import ctypes
+import math
+
+import numpy as np
+import pytest
+import scipy.special
+
+from honeycrisp_amd.descriptors import (BroadcastData, BroadcastStrides, ComparisonOp, DType, ElemwiseOp,
+                                        NumericBinaryOp, ReduceDims, ReduceOp, ScatterGatherIndices)
+from honeycrisp_amd.tensor import Tensor
+from backend_cases import assert_close_arrays
+
+F32, F16, I64, BOOL = DType.float32, DType.float16, DType.int64, DType.bool
+
+
+def arr(backend, data, dtype, count=None):
+    raw = data.onCPU()
+    out = np.frombuffer(raw.tobytes(), dtype=dtype.numpy)
+    return out if count is None else out[:count]
+
+
+def test_half_to_float_all_patterns(oracle_backend):
+    bits = np.arange(65536, dtype=np.uint16)
+    out = np.empty(65536, dtype=np.float32)
+    oracle_backend.lib.ref_f16_to_f32_n(bits.ctypes.data, out.ctypes.data, 65536)
+    want = bits.view(np.float16).astype(np.float32)
+    assert np.array_equal(out.view(np.uint32), want.view(np.uint32))
+
+
+def test_float_to_half_matches_ieee_rne(oracle_backend):
+    rng = np.random.default_rng(0)
+    # random bit patterns cover normals, subnormals, overflow, inf and NaN; add exact
+    # halfway cases between adjacent halfs and the overflow boundary 65520
+    x = rng.integers(0, 2**32, size=400000, dtype=np.uint64).astype(np.uint32).view(np.float32)
+    halves = np.arange(0, 0x7c00, dtype=np.uint16)
+    lo = halves.view(np.float16).astype(np.float64)
+    hi = (halves + 1).astype(np.uint16).view(np.float16).astype(np.float64)
+    with np.errstate(invalid="ignore", over="ignore"):
+        mid = ((lo + hi) / 2).astype(np.float32)
+    special = np.array([65504.0, 65519.996, 65520.0, 65536.0, 5.9604645e-08, 2.9802322e-08, 2.98023224e-08 * 1.0000001,
+                        -0.0, 1e9, -1e9, np.inf, -np.inf], dtype=np.float32)
+    x = np.concatenate([x, mid, -mid, special])
+    out = np.empty(x.size, dtype=np.uint16)
+    oracle_backend.lib.ref_f32_to_f16_n(x.ctypes.data, out.ctypes.data, x.size)
+    with np.errstate(over="ignore", invalid="ignore"):
+        want = x.astype(np.float16)
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(out.view(np.float16)), nan)
+    assert np.array_equal(out[~nan], want.view(np.uint16)[~nan])
+
+
+def test_stride_map_brute_force(oracle_backend):
+    rng = np.random.default_rng(1)
+    for _ in range(40):
+        nd = int(rng.integers(1, 6))
+        shape = [int(rng.integers(1, 5)) for _ in range(nd)]
+        bcast = [bool(rng.integers(0, 2)) for _ in range(nd)]
+        data_shape = [1 if b else s for s, b in zip(shape, bcast)]
+        data = np.arange(int(np.prod(data_shape))).reshape(data_shape)
+        t = Tensor(dataHandle=object(), shape=data_shape, dtype=I64)  # shape bookkeeping only
+        strides = t.expandStrides(shape)
+        want = np.broadcast_to(data, shape).reshape(-1)
+        from honeycrisp_amd._lib import make_strides
+        s = make_strides(strides.shape, strides.strides)
+        got = [oracle_backend.lib.ref_strides_index(s, i) for i in range(want.size)]
+        assert got == [int(v) for v in want]
+        assert got == [strides(i) for i in range(want.size)]  # the Python mirror agrees
+
+
+@pytest.mark.parametrize("dtype", [F32, F16])
+def test_matmul_all_layouts_vs_numpy(oracle_backend, dtype):
+    rng = np.random.default_rng(2)
+    M, K, N, B = 37, 53, 29, 3
+    tol = 1e-4 if dtype == F32 else 1e-2
+    with oracle_backend.use():
+        for transA in (False, True):
+            for transB in (False, True):
+                for transOut in (False, True):
+                    a = rng.standard_normal((B, M, K)).astype(dtype.numpy)
+                    b = rng.standard_normal((B, K, N)).astype(dtype.numpy)
+                    want = np.matmul(a.astype(np.float64), b.astype(np.float64))
+                    sa = np.ascontiguousarray(a.transpose(0, 2, 1)) if transA else a
+                    sb = np.ascontiguousarray(b.transpose(0, 2, 1)) if transB else b
+                    out = oracle_backend.batchedMatmul(B, sa, transA, sb, transB, transOut, M, K, N, dtype)
+                    got = arr(oracle_backend, out, dtype).astype(np.float64)
+                    got = got.reshape(B, N, M).transpose(0, 2, 1) if transOut else got.reshape(B, M, N)
+                    assert_close_arrays(got, want, tol, tol)
+
+
+@pytest.mark.parametrize("dtype", [F32, F16])
+def test_matmul_blocked_loop_is_bit_identical_to_literal_loop(oracle_backend, dtype):
+    """ref_matmul iterates i,k,j for speed; ref_matmul_rows is the reference's literal i,j,k
+    loop. Per output the k order is the same, so the fp32 accumulators agree bit for bit."""
+    rng = np.random.default_rng(3)
+    M, K, N = 19, 301, 23
+    for transA in (False, True):
+        for transB in (False, True):
+            a = rng.standard_normal((M, K)).astype(dtype.numpy)
+            b = rng.standard_normal((K, N)).astype(dtype.numpy)
+            sa = np.ascontiguousarray(a.T) if transA else a
+            sb = np.ascontiguousarray(b.T) if transB else b
+            out = oracle_backend.matmul(sa, transA, sb, transB, False, M, K, N, dtype)
+            got = arr(oracle_backend, out, dtype)
+            acc = np.empty((M, N), dtype=np.float32)
+            oracle_backend.lib.ref_matmul_rows(int(dtype), sa.ctypes.data, int(transA), sb.ctypes.data, int(transB),
+                                               M, K, N, 0, M, acc.ctypes.data)
+            with np.errstate(over="ignore"):
+                want = acc.astype(dtype.numpy).reshape(-1)
+            assert np.array_equal(got.view(np.uint8), want.view(np.uint8))
+            # and the literal loop is the textbook one: sequential fp32 accumulation
+            af, bf = a.astype(np.float32), b.astype(np.float32)
+            ref = np.zeros((M, N), dtype=np.float32)
+            for k in range(K):
+                ref = ref + np.outer(af[:, k], bf[k, :]).astype(np.float32)
+            assert np.array_equal(acc, ref)
+
+
+def test_binary_ops_vs_numpy(oracle_backend):
+    rng = np.random.default_rng(4)
+    with oracle_backend.use():
+        a = rng.standard_normal((5, 1, 7)).astype(np.float32) * 3
+        b = rng.standard_normal((4, 7)).astype(np.float32) + 2.5
+        ta, tb = Tensor(data=a), Tensor(data=b)
+        assert np.array_equal((ta + tb).numpy(), a + b)
+        assert np.array_equal((ta - tb).numpy(), a - b)
+        assert np.array_equal((ta * tb).numpy(), a * b)
+        assert np.array_equal((ta / tb).numpy(), a / b)
+        # Python-style modulus == numpy's mod (sign follows the divisor)
+        nb = -b
+        assert_close_arrays((ta % tb).numpy(), np.mod(a, b), 1e-5, 1e-5)
+        assert_close_arrays((ta % Tensor(data=nb)).numpy(), np.mod(a, nb), 1e-5, 1e-5)
+        ia = rng.integers(-50, 50, size=(6, 5))
+        ib = rng.integers(1, 9, size=(5,)) * rng.choice([-1, 1], size=(5,))
+        tia, tib = Tensor(data=ia), Tensor(data=ib)
+        assert np.array_equal((tia % tib).numpy(), np.mod(ia, ib))
+        assert np.array_equal((tia + tib).numpy(), ia + ib)
+        assert np.array_equal((tia * tib).numpy(), ia * ib)
+        # int64 division truncates toward zero (Swift `/`), unlike numpy's floor division
+        assert np.array_equal((tia / tib).numpy(), np.trunc(ia / ib).astype(np.int64))
+        # fp16: computed in fp32, rounded once == correctly rounded half arithmetic
+        ha, hb = a.astype(np.float16), b.astype(np.float16)
+        got = (Tensor(data=ha) * Tensor(data=hb)).numpy()
+        assert np.array_equal(got, (ha.astype(np.float32) * hb.astype(np.float32)).astype(np.float16))
+
+
+def test_fp32_scalar_forms_follow_vdsp(oracle_backend):
+    """x / s is x * (1/s) and x - s is x + (-s) in fp32 (BackendCPU.swift:325-342); fp16 uses
+    true division. Inputs chosen so that the two forms differ in the last bit."""
+    x = np.array([1.0, 5.0, 7.0, 10.0, 13.0, 25.0, 0.1, 123.456], dtype=np.float32)
+    s = np.float32(3.0)
+    with oracle_backend.use():
+        got = (Tensor(data=x) / 3.0).numpy()
+        recip = x * (np.float32(1.0) / s)
+        assert np.array_equal(got, recip)
+        assert not np.array_equal(recip, x / s)  # the distinction is real for this input
+        assert np.array_equal((3.0 / Tensor(data=x)).numpy(), s / x)
+        assert np.array_equal((3.0 - Tensor(data=x)).numpy(), x * np.float32(-1) + s)
+        h = x.astype(np.float16)
+        assert np.array_equal((Tensor(data=h) / 3.0).numpy(), (h.astype(np.float32) / s).astype(np.float16))
+
+
+def test_elemwise_vs_library(oracle_backend):
+    rng = np.random.default_rng(5)
+    x = np.concatenate([rng.standard_normal(2000) * 3, np.linspace(-8, 8, 401)]).astype(np.float32)
+    x64 = x.astype(np.float64)
+    unit = np.clip(x64 / 9.0, -0.99, 0.99)
+    with oracle_backend.use():
+        t = Tensor(data=x)
+        u = Tensor(data=unit.astype(np.float32))
+        u64 = unit.astype(np.float32).astype(np.float64)
+        checks = [
+            (t.sin(), np.sin(x64)), (t.cos(), np.cos(x64)), (t.atan(), np.arctan(x64)),
+            (u.acos(), np.arccos(u64)), (u.asin(), np.arcsin(u64)),
+            (t.exp(), np.exp(x64)), (t.abs().log(), np.log(np.abs(x64))),
+            (t.sigmoid(), 1 / (1 + np.exp(-x64))), (t.erf(), scipy.special.erf(x64)),
+            (t.relu(), np.maximum(x64, 0)), (t.abs(), np.abs(x64)),
+            (t.gelu("exact"), x64 * 0.5 * (1 + scipy.special.erf(x64 / math.sqrt(2)))),
+            (t.gelu("approx"), 0.5 * x64 * (1 + np.tanh(math.sqrt(2 / math.pi) * (x64 + 0.044715 * x64**3)))),
+            (t.elemwise(ElemwiseOp.sigmoidGrad), (1 / (1 + np.exp(-x64))) * (1 - 1 / (1 + np.exp(-x64)))),
+            (t.elemwise(ElemwiseOp.tanGrad), 1 / np.cos(x64)**2),
+            (t.elemwise(ElemwiseOp.atanGrad), 1 / (1 + x64**2)),
+            (t.elemwise(ElemwiseOp.erfGrad), 2 / math.sqrt(math.pi) * np.exp(-x64**2)),
+            (t.elemwise(ElemwiseOp.minusSin), -np.sin(x64)),
+            (t.elemwise(ElemwiseOp.recip), 1 / x64),
+            (t.floor(), np.floor(x64)), (t.ceil(), np.ceil(x64)),
+            (t.pow(3.0), x64**3), (t.pow(2), x64**2), (t.abs().sqrt(), np.sqrt(np.abs(x64))),
+            (t.tanh(), np.tanh(x64)),
+        ]
+        for got, want in checks:
+            # abs-or-rel, as the reference's assertClose; 2e-6 abs covers the fp32 cancellation
+            # in the (1 + tanh) tail of GELU
+            assert_close_arrays(got.numpy(), want, 2e-6, 2e-5)
+        # derivative formulas against central differences of the forward formulas
+        for fwd, grad in [(ElemwiseOp.geluApprox, ElemwiseOp.geluApproxGrad),
+                          (ElemwiseOp.geluExact, ElemwiseOp.geluExactGrad)]:
+            xs = np.linspace(-4, 4, 161)
+            h = 1e-3
+            f = lambda v: Tensor(data=v.astype(np.float32)).elemwise(fwd).numpy().astype(np.float64)
+            num = (f(xs + h) - f(xs - h)) / (2 * h)
+            got = Tensor(data=xs.astype(np.float32)).elemwise(grad).numpy()
+            assert_close_arrays(got, num, 2e-3, 2e-3)
+        # round half away from zero
+        r = Tensor(data=np.array([-2.5, -1.5, -0.5, 0.5, 1.5, 2.5, 2.4999, -2.4999], dtype=np.float32)).round()
+        assert r.floats() == [-3.0, -2.0, -1.0, 1.0, 2.0, 3.0, 2.0, -2.0]
+        # relu keeps -0.0 and NaN (x < 0 ? 0 : x)
+        z = Tensor(data=np.array([-0.0, np.nan, -1.0], dtype=np.float32)).relu().numpy()
+        assert np.signbit(z[0]) and np.isnan(z[1]) and z[2] == 0
+
+
+def test_pow_special_cases(oracle_backend):
+    x = np.array([0.5, 3.0, -7.0, 11.0], dtype=np.float32)
+    s = np.array([2.0, 0.5, 3.0, -1.0], dtype=np.float32)
+    ob = oracle_backend
+    f = lambda b, scale, scales: arr(ob, ob.pow(x, b, scale, scales, 4, F32), F32)
+    assert np.array_equal(f(2.0, 1.0, None), x * x)
+    assert np.array_equal(f(2.0, 3.0, None), x * x * np.float32(3))
+    assert np.array_equal(f(-1.0, 3.0, None), np.float32(3) / x)
+    assert np.array_equal(f(1.0, 3.0, s), x * np.float32(3) * s)
+    assert_close_arrays(f(0.5, 2.0, s), 2.0 * s * np.sqrt(np.abs(x.astype(np.float64))) * np.where(x < 0, np.nan, 1), 1e-6, 1e-6)
+    ix = np.array([2, -3, 5], dtype=np.int64)
+    assert list(arr(ob, ob.pow(ix, 3, 2, None, 3, I64), I64)) == [16, -54, 250]
+
+
+def test_reduce_vs_numpy_and_tie_rules(oracle_backend):
+    rng = np.random.default_rng(6)
+    ob = oracle_backend
+    x = rng.standard_normal((7, 33, 5)).astype(np.float32)
+    dims = ReduceDims(7, 33, 5)
+    assert_close_arrays(arr(ob, ob.reduce(x, ReduceOp.sum, dims, F32), F32), x.sum(axis=1), 1e-5, 1e-5)
+    assert_close_arrays(arr(ob, ob.reduce(x, ReduceOp.prod, dims, F32), F32), x.astype(np.float64).prod(axis=1), 1e-5, 1e-4)
+    assert np.array_equal(arr(ob, ob.reduce(x, ReduceOp.argmax, dims, F32), I64).reshape(7, 5), x.argmax(axis=1))
+    assert np.array_equal(arr(ob, ob.reduce(x, ReduceOp.argmin, dims, F32), I64).reshape(7, 5), x.argmin(axis=1))
+    ix = rng.integers(-4, 4, size=(3, 50, 2))
+    idims = ReduceDims(3, 50, 2)
+    assert np.array_equal(arr(ob, ob.reduce(ix, ReduceOp.sum, idims, I64), I64).reshape(3, 2), ix.sum(axis=1))
+    # ties: first occurrence (numpy's argmax has the same rule)
+    assert np.array_equal(arr(ob, ob.reduce(ix, ReduceOp.argmax, idims, I64), I64).reshape(3, 2), ix.argmax(axis=1))
+    assert np.array_equal(arr(ob, ob.reduce(ix, ReduceOp.argmin, idims, I64), I64).reshape(3, 2), ix.argmin(axis=1))
+    # NaN rules derived from the strict-compare scan (BackendCPU.swift:848-877): a NaN at
+    # k > 0 never wins; a NaN at k = 0 is never replaced.
+    nan = np.nan
+    rows = np.array([[1, nan, 3, 3], [nan, 5, 9, 1], [-np.inf, nan, -np.inf, -np.inf], [2, 2, nan, 2]], dtype=np.float32)
+    d = ReduceDims(4, 4, 1)
+    assert list(arr(ob, ob.reduce(rows, ReduceOp.argmax, d, F32), I64)) == [2, 0, 0, 0]
+    assert list(arr(ob, ob.reduce(rows, ReduceOp.argmin, d, F32), I64)) == [0, 0, 0, 0]
+
+
+def test_gather_and_permutation_vs_numpy(oracle_backend):
+    rng = np.random.default_rng(7)
+    with oracle_backend.use():
+        x = rng.standard_normal((4, 6, 5)).astype(np.float32)
+        idx = rng.integers(0, 6, size=(4, 3, 5))
+        got = Tensor(data=x).gather(1, Tensor(data=idx)).numpy()
+        assert np.array_equal(got, np.take_along_axis(x, idx, axis=1))
+        rows = rng.integers(0, 4, size=(9,))
+        assert np.array_equal(Tensor(data=x).gather(0, Tensor(data=rows)).numpy(), x[rows])
+        for perm in [(1, 0), (2, 0, 1), (0, 2, 1), (2, 1, 0)]:
+            shape = [3, 4, 5][:len(perm)]
+            want = np.arange(int(np.prod(shape))).reshape(shape).transpose(perm).reshape(-1)
+            data = oracle_backend.axisPermutation(list(perm), shape)
+            assert np.array_equal(arr(oracle_backend, data, I64), want)
+        t = Tensor(data=x)
+        assert np.array_equal(t.t().numpy(), x.transpose(0, 2, 1))
+        assert np.array_equal(t.swap(0, 2).numpy(), x.transpose(2, 1, 0))
+        assert np.array_equal(t.move(0, 2).numpy(), np.moveaxis(x, 0, 2))
+        assert np.array_equal(t[1:3, ..., 2].numpy(), x[1:3, :, 2])
+
+
+def test_log_softmax_vs_scipy(oracle_backend):
+    rng = np.random.default_rng(8)
+    x = (rng.standard_normal((5, 17, 3)) * 4).astype(np.float32)
+    with oracle_backend.use():
+        for axis in (0, 1, 2):
+            got = Tensor(data=x).logSoftmax(axis=axis).numpy()
+            assert_close_arrays(got, scipy.special.log_softmax(x.astype(np.float64), axis=axis), 1e-5, 1e-5)
+        sm = Tensor(data=x).softmax().numpy()
+        assert_close_arrays(sm.sum(axis=-1), np.ones((5, 17)), 1e-5, 1e-5)
+
+
+def test_cast_rules(oracle_backend):
+    with oracle_backend.use():
+        f = Tensor(data=np.array([-2.9, -0.5, 0.0, 0.99, 7.5, 65519.0, 65520.0], dtype=np.float32))
+        assert f.cast(I64).int64s() == [-2, 0, 0, 0, 7, 65519, 65520]   # truncation toward zero
+        assert f.cast(BOOL).int64s() == [1, 1, 0, 1, 1, 1, 1]
+        h = f.cast(F16).numpy()
+        assert h[5] == np.float16(65504.0) and np.isinf(h[6])
+        i = Tensor(data=np.array([0, -3, 2**40 + 1], dtype=np.int64))
+        assert i.cast(F32).floats() == [0.0, -3.0, float(np.float32(2**40 + 1))]
+        assert i.cast(BOOL).int64s() == [0, 1, 1]
+
+
+@pytest.mark.parametrize("dtype", [F32, F16])
+def test_normalize_composition_and_formula(oracle_backend, dtype):
+    rng = np.random.default_rng(9)
+    ob = oracle_backend
+    for outer, red, inner in [(6, 37, 1), (3, 8, 5), (1, 1025, 1)]:
+        x = rng.standard_normal((outer, red, inner)).astype(dtype.numpy)
+        dims = ReduceDims(outer, red, inner)
+        composed = arr(ob, ob.normalize(x, dims, 0.3, dtype), dtype)  # Python mirror of the base class
+        out = np.empty(x.size, dtype=dtype.numpy)
+        ob.lib.ref_normalize(int(dtype), x.ctypes.data, out.ctypes.data, outer, red, inner, ctypes.c_float(0.3))
+        assert np.array_equal(out.view(np.uint8), composed.view(np.uint8))
+        x64 = x.astype(np.float64)
+        mean = x64.mean(axis=1, keepdims=True)
+        var = ((x64 - mean)**2).mean(axis=1, keepdims=True)
+        want = (x64 - mean) / np.sqrt(var + 0.3)
+        tol = 1e-4 if dtype == F32 else 2e-2
+        assert_close_arrays(out, want, tol, tol)
+
+
+def test_compare_when_triangular_fill_concat(oracle_backend):
+    rng = np.random.default_rng(10)
+    with oracle_backend.use():
+        a = rng.integers(-3, 3, size=(4, 5)).astype(np.float32)
+        b = rng.integers(-3, 3, size=(5,)).astype(np.float32)
+        ta, tb = Tensor(data=a), Tensor(data=b)
+        for op, fn in [(lambda x, y: x == y, np.equal), (lambda x, y: x != y, np.not_equal),
+                       (lambda x, y: x < y, np.less), (lambda x, y: x <= y, np.less_equal),
+                       (lambda x, y: x > y, np.greater), (lambda x, y: x >= y, np.greater_equal)]:
+            assert np.array_equal(op(ta, tb).numpy(), fn(a, b))
+            assert np.array_equal(op(ta, 1.0).numpy(), fn(a, 1.0))
+        m = rng.standard_normal((2, 5, 7)).astype(np.float32)
+        for off in (-6, -2, 0, 1, 3, 8):
+            assert np.array_equal(Tensor(data=m).tril(off).numpy(), np.tril(m, off))
+            assert np.array_equal(Tensor(data=m).triu(off).numpy(), np.triu(m, off))
+        assert Tensor.constant(2.5, [3], F16).floats() == [2.5] * 3
+        assert Tensor.constant(7, [2], I64).int64s() == [7, 7]
+        assert Tensor.constant(0.5, [2], BOOL).int64s() == [1, 1]
+        c = Tensor.concat([Tensor(data=a), Tensor(data=a[:, :2])], axis=1).numpy()
+        assert np.array_equal(c, np.concatenate([a, a[:, :2]], axis=1))
