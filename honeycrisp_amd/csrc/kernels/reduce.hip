@@ -148,12 +148,14 @@ __device__ __forceinline__ void reduce_rows_impl(const hck_reduce_args& p) {
 
 // ---------------------------------------------------------------- columns (inner > 1)
 
-// Block = 64 lanes along inner x 4 waves along reduce. grid.x covers inner, grid.y outer.
+// Block = 64 lanes along inner x 4 waves along reduce.
 template <typename T, int OP> __device__ __forceinline__ void reduce_cols_impl(const hck_reduce_args& p) {
   typedef typename Arith<T>::type C;
-  const uint32_t j = blockIdx.x * 64 + (threadIdx.x & 63);
+  // grid.x = outer * ceil(inner / 64): no 65535 limit on outer
+  const uint32_t jblocks = (p.inner + 63) / 64;
+  const uint32_t i = blockIdx.x / jblocks;
+  const uint32_t j = (blockIdx.x - i * jblocks) * 64 + (threadIdx.x & 63);
   const uint32_t kw = threadIdx.x >> 6;
-  const uint32_t i = blockIdx.y;
   const bool active = j < p.inner;
   const T* in = (const T*)p.in + (size_t)i * p.reduce * p.inner + (active ? j : 0);
   __shared__ char lds_raw[sizeof(ArgPair<C>) * HCK_BLOCK];
@@ -231,8 +233,9 @@ template <typename T> __device__ __forceinline__ void log_softmax_rows_impl(cons
 
 // Columns: one lane per (outer, inner) pair, lanes along inner.
 template <typename T> __device__ __forceinline__ void log_softmax_cols_impl(const hck_reduce_args& p) {
-  const uint32_t j = blockIdx.x * HCK_BLOCK + threadIdx.x;
-  const uint32_t i = blockIdx.y;
+  const uint32_t jblocks = (p.inner + HCK_BLOCK - 1) / HCK_BLOCK;
+  const uint32_t i = blockIdx.x / jblocks;
+  const uint32_t j = (blockIdx.x - i * jblocks) * HCK_BLOCK + threadIdx.x;
   if (j >= p.inner) return;
   const size_t base = (size_t)i * p.reduce * p.inner + j;
   const T* in = (const T*)p.in + base;
