@@ -24,13 +24,23 @@ template <> __device__ __forceinline__ float to_arith<uint8_t>(uint8_t v) {
   return v ? 1.0f : 0.0f;
 }
 
-template <typename T> __device__ __forceinline__ T from_arith(typename Arith<T>::type v) {
-  return (T)v;  // float -> half is v_cvt_f16_f32: round-to-nearest-even, overflow to inf
+// fp32 -> storage type. For half this is one v_cvt_f16_f32 (round-to-nearest-even, overflow
+// to inf) of a value that is first pinned in a VGPR: without the pin the compiler folds a
+// preceding multiply into v_fma_mixlo_f16 (a * b + 0), which turns a -0 product into +0.
+template <typename T> __device__ __forceinline__ T narrow(float v) { return (T)v; }
+template <> __device__ __forceinline__ half_t narrow<half_t>(float v) {
+  asm("" : "+v"(v));
+  return (half_t)v;
 }
+
+template <typename T> __device__ __forceinline__ T from_arith(typename Arith<T>::type v) {
+  return (T)v;
+}
+template <> __device__ __forceinline__ half_t from_arith<half_t>(float v) { return narrow<half_t>(v); }
 
 // Round an fp32 intermediate to what the tensor dtype can hold (identity for float).
 template <typename T> __device__ __forceinline__ float round_through(float v) {
-  return (float)(T)v;
+  return (float)narrow<T>(v);
 }
 template <> __device__ __forceinline__ float round_through<float>(float v) { return v; }
 

@@ -358,11 +358,11 @@ template <typename T, int OP> __device__ __forceinline__ void elemwise_impl(cons
   const T* scales = (const T*)p.scales;
   if (scales) {
     map_contiguous((const T*)p.in, (T*)p.out, p.count, [scales](T xv, uint64_t i) {
-      return (T)(elemwise_apply<OP>((float)xv) * (float)scales[i]);
+      return narrow<T>(elemwise_apply<OP>((float)xv) * (float)scales[i]);
     });
   } else {
     map_contiguous((const T*)p.in, (T*)p.out, p.count,
-                   [](T xv, uint64_t) { return (T)(elemwise_apply<OP>((float)xv) * 1.0f); });
+                   [](T xv, uint64_t) { return narrow<T>(elemwise_apply<OP>((float)xv) * 1.0f); });
   }
 }
 
@@ -423,7 +423,7 @@ template <typename T, int MODE> __device__ __forceinline__ void pow_impl(const h
       }
       if (scales) r = r * (float)scales[i];
     }
-    return (T)r;
+    return narrow<T>(r);
   });
 }
 HC_KERNEL void hc_pow_generic_f32(hck_map_args p) { pow_impl<float, 0>(p); }
@@ -432,13 +432,24 @@ HC_KERNEL void hc_pow_square_f32(hck_map_args p) { pow_impl<float, 1>(p); }
 HC_KERNEL void hc_pow_recip_f32(hck_map_args p) { pow_impl<float, 2>(p); }
 HC_KERNEL void hc_pow_linear_f32(hck_map_args p) { pow_impl<float, 3>(p); }
 
-// Int64.pow (TensorElement.swift:205-207): Int64(pow(Double(x), Double(Float(b)))).
+// Int64.pow (TensorElement.swift:205-207): Int64(pow(Double(x), Double(Float(b)))). The
+// exponent is integral here, so the power is formed by squaring in double: exact, hence
+// equal to a correctly rounded pow(), whenever |x^b| < 2^53.
 HC_KERNEL void hc_pow_generic_i64(hck_map_args p) {
   const int64_t* scales = (const int64_t*)p.scales;
   const double b = (double)(float)p.i0;
   const int64_t scale = p.i1;
   map_contiguous((const int64_t*)p.in, (int64_t*)p.out, p.count, [=](int64_t x, uint64_t i) {
-    int64_t pw = (int64_t)pow((double)x, b);
+    double base = (double)x, acc = 1.0;
+    double e = b < 0 ? -b : b;
+    while (e >= 1.0) {
+      const double half_e = floor(e * 0.5);
+      if (e - 2.0 * half_e != 0.0) acc *= base;
+      base *= base;
+      e = half_e;
+    }
+    if (b < 0) acc = 1.0 / acc;
+    int64_t pw = (int64_t)acc;
     return scale * (scales ? scales[i] : (int64_t)1) * pw;
   });
 }
@@ -447,11 +458,11 @@ HC_KERNEL void hc_pow_generic_i64(hck_map_args p) {
 
 // cast (BackendCPU.swift:626-646 + TensorElement.swift:225-323): int64 sources convert
 // directly; every other source is staged through Float.
-template <typename TO> __device__ __forceinline__ TO cast_from_float(float v) { return (TO)v; }
+template <typename TO> __device__ __forceinline__ TO cast_from_float(float v) { return narrow<TO>(v); }
 template <> __device__ __forceinline__ uint8_t cast_from_float<uint8_t>(float v) { return v == 0 ? 0 : 1; }
 template <typename TO> __device__ __forceinline__ TO cast_from_i64(int64_t v) { return (TO)v; }
 template <> __device__ __forceinline__ uint8_t cast_from_i64<uint8_t>(int64_t v) { return v == 0 ? 0 : 1; }
-template <> __device__ __forceinline__ half_t cast_from_i64<half_t>(int64_t v) { return (half_t)(float)v; }
+template <> __device__ __forceinline__ half_t cast_from_i64<half_t>(int64_t v) { return narrow<half_t>((float)v); }
 
 #define DEF_CAST_F(IN, TI, ON, TO)                                                                   \
   HC_KERNEL void hc_cast_##IN##_##ON(hck_map_args p) {                                               \

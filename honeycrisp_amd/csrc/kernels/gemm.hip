@@ -215,7 +215,7 @@ __device__ __forceinline__ void gemm_impl(const hck_gemm_args& p) {
 #pragma unroll
       for (int v = 0; v < 16; v++) {
         const uint32_t row = m0 + wm + i * 32 + 8 * (v / 4) + 4 * lgrp + (v % 4);
-        if (row < p.M && col < p.N) C[(size_t)row * p.c_rs + (size_t)col * p.c_cs] = (T)acc[i][j][v];
+        if (row < p.M && col < p.N) C[(size_t)row * p.c_rs + (size_t)col * p.c_cs] = narrow<T>(acc[i][j][v]);
       }
     }
 }

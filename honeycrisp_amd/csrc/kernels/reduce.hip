@@ -228,7 +228,7 @@ template <typename T> __device__ __forceinline__ void log_softmax_rows_impl(cons
   for (uint32_t k = lane; k < n; k += 64) s += expf((float)in[k] - m);
   s = wave_reduce(s, SumOp());
   const float log_sum = logf(s) + m;
-  for (uint32_t k = lane; k < n; k += 64) out[k] = (T)((float)in[k] - log_sum);
+  for (uint32_t k = lane; k < n; k += 64) out[k] = narrow<T>((float)in[k] - log_sum);
 }
 
 // Columns: one lane per (outer, inner) pair, lanes along inner.
@@ -249,7 +249,7 @@ template <typename T> __device__ __forceinline__ void log_softmax_cols_impl(cons
   for (uint32_t k = 0; k < p.reduce; k++) s += expf((float)in[(size_t)k * p.inner] - m);
   const float log_sum = logf(s) + m;
   for (uint32_t k = 0; k < p.reduce; k++)
-    out[(size_t)k * p.inner] = (T)((float)in[(size_t)k * p.inner] - log_sum);
+    out[(size_t)k * p.inner] = narrow<T>((float)in[(size_t)k * p.inner] - log_sum);
 }
 
 HC_KERNEL void hc_log_softmax_rows_f32(hck_reduce_args p) { log_softmax_rows_impl<float>(p); }
@@ -289,7 +289,7 @@ template <typename T> __device__ __forceinline__ void normalize_rows_impl(const 
   const float normer = round_through<T>(1.0f * 1.0f * powf(shifted, -0.5f));
   for (uint32_t k = lane; k < n; k += 64) {
     float c = round_through<T>((float)in[k] - mean);
-    out[k] = (T)(c * normer);
+    out[k] = narrow<T>(c * normer);
   }
 }
 HC_KERNEL void hc_normalize_rows_f32(hck_reduce_args p) { normalize_rows_impl<float>(p); }
