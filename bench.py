@@ -1,0 +1,277 @@
+#!/usr/bin/env python3
+"""Benchmark of the HIPBackend hot path on one MI355X.
+
+Headline (the one JSON line's `value`): fp16 GEMM, M = N = K = 4096, fp32 accumulate, all four
+transA/transB layouts (NN, NT, TN, TT) per step, inputs N(0,1)/sqrt(K) from fixed seeds and
+resident in HBM before the timed region. FLOPs = 2*M*N*K per GEMM, the formula of the
+reference's HCMatrixBench (Sources/HCMatrixBench/Entrypoint.swift:25).
+
+Also reported in the same line:
+  roofline      the slowest layout's GEMM kernel: algorithmic FLOPs / average launch duration
+                from HIP events recorded on the backend's own stream inside the timed region
+  cpu_baseline  the reference CPUBackend algorithm (oracle/cpu_ref.c restatement, the literal
+                single-thread triple loop) timed on this box's host cores on a bounded row slab
+  extra         the other BASELINE configs: fp32 1024^3, attention-shaped batched GEMMs, the
+                bandwidth-bound ops at [8192,4096] with GB/s against the 8 TB/s HBM peak
+
+Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extra]
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_F16_TFLOPS = 2516.6  # MI355X dense fp16 MFMA
+PEAK_F32_TFLOPS = 157.3   # MI355X fp32 MFMA
+PEAK_HBM_GBS = 8000.0     # MI355X HBM3E
+
+
+class Events:
+    """HIP events on the backend's stream (hc_event_*), for per-launch durations."""
+
+    def __init__(self, backend):
+        self.b = backend
+        self.lib = backend._lib
+
+    def new(self):
+        ev = ctypes.c_void_p()
+        self.b._check(self.lib.hc_event_create(self.b._ctx, ctypes.byref(ev)))
+        return ev
+
+    def record(self, ev):
+        self.b._check(self.lib.hc_event_record(self.b._ctx, ev))
+
+    def elapsed_ms(self, a, b):
+        ms = ctypes.c_float()
+        self.b._check(self.lib.hc_event_elapsed_ms(a, b, ctypes.byref(ms)))
+        return ms.value
+
+    def free(self, ev):
+        self.lib.hc_event_destroy(ev)
+
+
+def timed_launches(backend, events, fn, iters, warmup):
+    """Average duration (ms) of fn() launches, each bracketed by events on the stream."""
+    for _ in range(warmup):
+        fn()
+    pairs = []
+    for _ in range(iters):
+        a, b = events.new(), events.new()
+        events.record(a)
+        fn()
+        events.record(b)
+        pairs.append((a, b))
+    backend.sync()
+    ms = [events.elapsed_ms(a, b) for a, b in pairs]
+    for a, b in pairs:
+        events.free(a)
+        events.free(b)
+    return float(np.mean(ms)), float(np.median(ms))
+
+
+def headline(backend, steps, warmup):
+    from honeycrisp_amd.descriptors import DType
+    n = 4096
+    a = (np.random.default_rng(2).standard_normal((n, n)) / np.sqrt(n)).astype(np.float16)
+    b = (np.random.default_rng(3).standard_normal((n, n)) / np.sqrt(n)).astype(np.float16)
+    # operands stored pre-transposed so that all four layouts compute the same product
+    dev = {
+        ("a", False): backend.upload(a), ("a", True): backend.upload(np.ascontiguousarray(a.T)),
+        ("b", False): backend.upload(b), ("b", True): backend.upload(np.ascontiguousarray(b.T)),
+    }
+    layouts = [("NN", False, False), ("NT", False, True), ("TN", True, False), ("TT", True, True)]
+    events = Events(backend)
+
+    def gemm(ta, tb):
+        return backend.matmul(dev[("a", ta)], ta, dev[("b", tb)], tb, False, n, n, n, DType.float16)
+
+    for _ in range(warmup):
+        for _, ta, tb in layouts:
+            gemm(ta, tb)
+    backend.sync()
+    per_layout = {name: [] for name, _, _ in layouts}
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        for name, ta, tb in layouts:
+            e0, e1 = events.new(), events.new()
+            events.record(e0)
+            gemm(ta, tb)
+            events.record(e1)
+            per_layout[name].append((e0, e1))
+    backend.sync()
+    t1 = time.perf_counter()
+    flops = 2.0 * n * n * n
+    layout_ms = {}
+    for name, pairs in per_layout.items():
+        layout_ms[name] = float(np.mean([events.elapsed_ms(x, y) for x, y in pairs]))
+        for x, y in pairs:
+            events.free(x)
+            events.free(y)
+    ms_per_step = (t1 - t0) * 1e3 / steps
+    value = 4 * flops / (ms_per_step * 1e-3) / 1e12
+    worst = max(layout_ms, key=layout_ms.get)
+    achieved = flops / (layout_ms[worst] * 1e-3) / 1e12
+    roofline = {
+        "bound": "mfma", "kernel": "fp16 GEMM 4096^3 layout %s" % worst, "achieved": round(achieved, 2),
+        "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s", "frac": round(achieved / PEAK_F16_TFLOPS, 4),
+        "traffic": None,
+        "per_layout_tflops": {k: round(flops / (v * 1e-3) / 1e12, 2) for k, v in layout_ms.items()},
+        "per_layout_ms": {k: round(v, 4) for k, v in layout_ms.items()},
+    }
+    return value, ms_per_step, roofline, (a, b)
+
+
+def cpu_baseline(a, b, budget_s=20.0):
+    """The reference algorithm (single worker thread, scalar i/j/k loop with fp32 accumulate,
+    whole-buffer fp16 -> fp32 staging) on a row slab of the same four 4096^3 products."""
+    from oracle.oracle_backend import load
+    lib = load()
+    n = a.shape[0]
+    srcs = {False: (a, b), True: (np.ascontiguousarray(a.T), np.ascontiguousarray(b.T))}
+    out = np.empty((64, n), dtype=np.float32)
+
+    def run(ta, tb, rows):
+        sa, sb = srcs[ta][0], srcs[tb][1]
+        t0 = time.perf_counter()
+        lib.ref_matmul_rows(2, sa.ctypes.data, int(ta), sb.ctypes.data, int(tb), n, n, n, 0, rows, out.ctypes.data)
+        return time.perf_counter() - t0
+
+    probe = run(False, False, 2)            # includes the whole-buffer conversions
+    probe8 = run(False, False, 10)
+    per_row = max((probe8 - probe) / 8.0, 1e-4)
+    rows = int(max(2, min(64, (budget_s / 4.0 - probe) / per_row)))
+    total_t, total_flops = 0.0, 0.0
+    for ta in (False, True):
+        for tb in (False, True):
+            total_t += run(ta, tb, rows)
+            total_flops += 2.0 * rows * n * n
+    return {
+        "value": round(total_flops / total_t / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": "port",
+        "sample": "rows 0..%d of each of the four 4096^3 fp16 products (%.1f s of CPU work), literal "
+                  "CPUBackend loop incl. whole-buffer fp16->fp32 staging" % (rows, total_t),
+    }
+
+
+def extra_workloads(backend):
+    """Configs 1, 3 and 4 of BASELINE.json: per-op launch durations from HIP events."""
+    from honeycrisp_amd.descriptors import (BroadcastData, BroadcastStrides, DType, ElemwiseOp, NumericBinaryOp,
+                                            ReduceDims, ReduceOp, ScatterGatherIndices)
+    ev = Events(backend)
+    out = {}
+    F32, F16, I64 = DType.float32, DType.float16, DType.int64
+
+    def report(name, ms, flops=None, nbytes=None):
+        r = {"ms": round(ms, 4)}
+        if flops is not None:
+            r["tflops"] = round(flops / (ms * 1e-3) / 1e12, 3)
+        if nbytes is not None:
+            r["gbs"] = round(nbytes / (ms * 1e-3) / 1e9, 1)
+            r["hbm_frac"] = round(r["gbs"] / PEAK_HBM_GBS, 4)
+        out[name] = r
+
+    # config 1: fp32 1024^3 (two input sets alternate so the operands are not L2-resident twice in a row)
+    rng = np.random.default_rng(1)
+    sets = [(backend.upload(rng.standard_normal((1024, 1024)).astype(np.float32)),
+             backend.upload(rng.standard_normal((1024, 1024)).astype(np.float32))) for _ in range(2)]
+    it = [0]
+
+    def gemm32():
+        x, y = sets[it[0] & 1]
+        it[0] += 1
+        return backend.matmul(x, False, y, False, False, 1024, 1024, 1024, F32)
+    ms, _ = timed_launches(backend, ev, gemm32, 50, 10)
+    report("cfg1_f32_gemm_1024", ms, flops=2.0 * 1024**3)
+    out["cfg1_f32_gemm_1024"]["mfma_frac"] = round(out["cfg1_f32_gemm_1024"]["tflops"] / PEAK_F32_TFLOPS, 4)
+
+    # config 3: attention-shaped batched GEMMs, fp16, batch 32
+    q, k, v = [backend.upload(np.random.default_rng(s).standard_normal((32, 512, 64)).astype(np.float16))
+               for s in (4, 5, 6)]
+    scores = backend.batchedMatmul(32, q, False, k, True, False, 512, 64, 512, F16)
+    ms, _ = timed_launches(backend, ev, lambda: backend.batchedMatmul(32, q, False, k, True, False, 512, 64, 512, F16), 50, 10)
+    report("cfg3_qk_t", ms, flops=32 * 2.0 * 512 * 64 * 512, nbytes=32 * (2 * 512 * 64 + 512 * 512) * 2)
+    ms, _ = timed_launches(backend, ev, lambda: backend.binaryOp(scores, 0.125, NumericBinaryOp.mul, F16, count=32 * 512 * 512), 50, 10)
+    report("cfg3_scale", ms, nbytes=2 * 32 * 512 * 512 * 2)
+    ms, _ = timed_launches(backend, ev, lambda: backend.batchedMatmul(32, scores, False, v, False, False, 512, 512, 64, F16), 50, 10)
+    report("cfg3_pv", ms, flops=32 * 2.0 * 512 * 512 * 64, nbytes=32 * (2 * 512 * 64 + 512 * 512) * 2)
+
+    # config 4: bandwidth-bound ops at [8192, 4096] fp32
+    R, C = 8192, 4096
+    x = backend.upload(np.random.default_rng(7).standard_normal((R, C)).astype(np.float32))
+    bias = backend.upload(np.random.default_rng(8).standard_normal((1, C)).astype(np.float32))
+    xs = BroadcastStrides([R, C], [C, 1])
+    bs = BroadcastStrides([R, C], [0, 1])
+    nb = R * C * 4
+    ms, _ = timed_launches(backend, ev, lambda: backend.binaryOp(BroadcastData(xs, x), BroadcastData(bs, bias), NumericBinaryOp.add, F32), 50, 10)
+    report("cfg4_bias_add", ms, nbytes=2 * nb + C * 4)
+    ms, _ = timed_launches(backend, ev, lambda: backend.elemwise(x, ElemwiseOp.geluApprox, None, R * C, F32), 50, 10)
+    report("cfg4_gelu", ms, nbytes=2 * nb)
+    dims = ReduceDims(R, C, 1)
+    ms, _ = timed_launches(backend, ev, lambda: backend.reduce(x, ReduceOp.sum, dims, F32), 50, 10)
+    report("cfg4_sum_axis1", ms, nbytes=nb + R * 4)
+    ms, _ = timed_launches(backend, ev, lambda: backend.reduce(x, ReduceOp.argmax, dims, F32), 50, 10)
+    report("cfg4_argmax_axis1", ms, nbytes=nb + R * 8)
+    idx = backend.reduce(x, ReduceOp.argmax, dims, F32)
+    max_gather = ScatterGatherIndices([R, C], 1, BroadcastData(BroadcastStrides([R, 1], [1, 0]), idx))
+
+    def max_axis1():  # Tensor.max(axis:) = argmax + gather (ReduceRepeat.swift:201-209)
+        i = backend.reduce(x, ReduceOp.argmax, dims, F32)
+        return backend.gather(x, ScatterGatherIndices([R, C], 1, BroadcastData(BroadcastStrides([R, 1], [1, 0]), i)), F32)
+    ms, _ = timed_launches(backend, ev, max_axis1, 50, 10)
+    report("cfg4_max_axis1", ms, nbytes=nb + R * 8 + R * 8 + R * 4 + R * 4)
+    table = backend.upload(np.random.default_rng(10).standard_normal((32000, 1024)).astype(np.float32))
+    ids = backend.upload(np.random.default_rng(9).integers(0, 32000, size=(65536,)))
+    emb = ScatterGatherIndices([32000, 1024], 0, BroadcastData(BroadcastStrides([65536, 1024], [1, 0]), ids))
+    ms, _ = timed_launches(backend, ev, lambda: backend.gather(table, emb, F32), 50, 10)
+    report("cfg4_embedding_gather", ms, nbytes=65536 * 8 + 2 * 65536 * 1024 * 4)
+    del max_gather
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="skip the other BASELINE configs")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs the hot path on ONE GPU only (no collectives, no sharding); "
+              "--gpus %d is not supported" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    from honeycrisp_amd.backend import HIPBackend
+    backend = HIPBackend(0)
+    info = backend.deviceInfo()
+    value, ms_per_step, roofline, (a, b) = headline(backend, args.steps, args.warmup)
+    result = {
+        "metric": "matmul TFLOP/s (fp16 in, fp32 accumulate, 4096^3, mean over NN/NT/TN/TT)",
+        "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "configs[1]: fp16 GEMM M=N=K=4096, four transA/transB layouts per step, "
+                               "entries N(0,1)/sqrt(K), seeds 2/3",
+                   "device": info["name"], "arch": info["arch"], "compute_units": info["compute_units"],
+                   "clock_mhz": info["clock_mhz"]},
+        "frac_of_peak": round(value / PEAK_F16_TFLOPS, 4),
+        "roofline": roofline,
+    }
+    if not args.no_extra:
+        result["extra"] = extra_workloads(backend)
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(a, b)
+    else:
+        result["cpu_baseline"] = None
+    backend.sync()
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

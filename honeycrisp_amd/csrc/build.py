@@ -22,6 +22,7 @@ KERNELS = [
     ("reduce", "reduce.hip", ["-ffp-contract=off"]),
     ("gather", "gather.hip", []),
     ("gemm", "gemm.hip", []),
+    ("gemm_f16_fast", "gemm_f16_fast.hip", []),
 ]
 DEVICE_FLAGS = [
     "--offload-arch=gfx950", "--genco", "-O3", "-std=c++17",

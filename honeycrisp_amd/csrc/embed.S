@@ -17,5 +17,6 @@
     EMBED hc_image_reduce, "reduce.hsaco"
     EMBED hc_image_gather, "gather.hsaco"
     EMBED hc_image_gemm, "gemm.hsaco"
+    EMBED hc_image_gemm_f16_fast, "gemm_f16_fast.hsaco"
 
     .section .note.GNU-stack,"",@progbits

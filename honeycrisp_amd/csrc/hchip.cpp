@@ -25,6 +25,7 @@ extern const unsigned char hc_image_elementwise[], hc_image_elementwise_end[];
 extern const unsigned char hc_image_reduce[], hc_image_reduce_end[];
 extern const unsigned char hc_image_gather[], hc_image_gather_end[];
 extern const unsigned char hc_image_gemm[], hc_image_gemm_end[];
+extern const unsigned char hc_image_gemm_f16_fast[], hc_image_gemm_f16_fast_end[];
 }
 
 struct hc_module {
@@ -127,6 +128,7 @@ extern "C" int hc_init(int device, hc_ctx** out) {
   if (s == HC_OK) s = load_image(ctx, hc_image_reduce, hc_image_reduce_end, "reduce");
   if (s == HC_OK) s = load_image(ctx, hc_image_gather, hc_image_gather_end, "gather");
   if (s == HC_OK) s = load_image(ctx, hc_image_gemm, hc_image_gemm_end, "gemm");
+  if (s == HC_OK) s = load_image(ctx, hc_image_gemm_f16_fast, hc_image_gemm_f16_fast_end, "gemm_f16_fast");
   if (s != HC_OK) {
     hc_shutdown(ctx);
     return s;
@@ -1236,7 +1238,38 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
   char ma = mode(k.a, a_rs, a_cs, k.a_bs);
   char mb = mode(k.b, b_cs, b_rs, k.b_bs);
   char name[64];
-  if (ma == 'x' || mb == 'x')
+  // Tuned fp16 kernels: whole tiles only. HCHIP_GEMM_TILE=general|256x256|256x128|128x128
+  // overrides the choice (for measurements).
+  uint32_t bm = 0, bn = 0;
+  if (dtype == HC_F16 && ma != 'x' && mb != 'x' && K > 0 && K % 64 == 0 && aligned16(out)) {
+    const char* force = getenv("HCHIP_GEMM_TILE");
+    auto fits = [&](uint32_t tm, uint32_t tn) { return M % tm == 0 && N % tn == 0; };
+    if (force && *force) {
+      unsigned fm = 0, fn = 0;
+      if (sscanf(force, "%ux%u", &fm, &fn) == 2 && fits(fm, fn)) {
+        bm = fm;
+        bn = fn;
+      }
+    } else {
+      const uint64_t cus = (uint64_t)ctx->props.multiProcessorCount;
+      if (fits(256, 256) && (uint64_t)(M / 256) * (N / 256) * (uint64_t)batch >= cus) {
+        bm = 256;
+        bn = 256;
+      } else if (fits(256, 128) && (uint64_t)(M / 256) * (N / 128) * (uint64_t)batch >= cus) {
+        bm = 256;
+        bn = 128;
+      } else if (fits(128, 128)) {
+        bm = 128;
+        bn = 128;
+      }
+    }
+  }
+  if (bm != 0) {
+    k.tiles_m = M / bm;
+    k.tiles_n = N / bn;
+    snprintf(name, sizeof(name), "hc_gemm_f16_fast_%ux%u_%c%c", bm, bn, ma == 'k' ? 'k' : 'm',
+             mb == 'k' ? 'k' : 'n');
+  } else if (ma == 'x' || mb == 'x')
     snprintf(name, sizeof(name), "hc_gemm_%s_xx", dtype_name(dtype));
   else
     snprintf(name, sizeof(name), "hc_gemm_%s_%c%c", dtype_name(dtype), ma == 'k' ? 'k' : 'm',
