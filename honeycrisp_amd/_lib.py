@@ -8,7 +8,8 @@ from ctypes import (POINTER, Structure, c_char, c_char_p, c_float, c_int, c_int6
                     c_uint32, c_void_p)
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "csrc", "libhchip.so")
+# HCHIP_LIB points at an alternative build of the library (kernel experiments).
+LIB_PATH = os.environ.get("HCHIP_LIB", os.path.join(HERE, "csrc", "libhchip.so"))
 
 HC_MAX_DIMS = 8
 

@@ -11,7 +11,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 KERNEL_DIR = os.path.join(HERE, "kernels")
 BUILD_DIR = os.path.join(HERE, "build")
-LIB_PATH = os.path.join(HERE, "libhchip.so")
+LIB_PATH = os.environ.get("HCHIP_LIB_OUT", os.path.join(HERE, "libhchip.so"))
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 HIPCC = os.path.join(ROCM, "bin", "hipcc")
 
@@ -39,7 +39,9 @@ def _run(cmd):
 
 def build_kernel(name, src, extra):
     out = os.path.join(BUILD_DIR, name + ".hsaco")
-    _run([HIPCC] + DEVICE_FLAGS + extra + ["-o", out, os.path.join(KERNEL_DIR, src)])
+    # HCHIP_EXTRA_FLAGS: additional device-compile flags (kernel experiments, e.g. -DNAME=1)
+    more = os.environ.get("HCHIP_EXTRA_FLAGS", "").split()
+    _run([HIPCC] + DEVICE_FLAGS + extra + more + ["-o", out, os.path.join(KERNEL_DIR, src)])
     return out
 
 
