@@ -210,6 +210,9 @@ def extra_workloads(backend):
     nb = R * C * 4
     ms, _ = timed_launches(backend, ev, lambda: backend.binaryOp(BroadcastData(xs, x), BroadcastData(bs, bias), NumericBinaryOp.add, F32), 50, 10)
     report("cfg4_bias_add", ms, nbytes=2 * nb + C * 4)
+    # plain copy of known size (identity broadcast): the calibration kernel for HBM byte counters
+    ms, _ = timed_launches(backend, ev, lambda: backend.broadcast(BroadcastData(xs, x), F32), 50, 10)
+    report("copy_134MB_calibration", ms, nbytes=2 * nb)
     ms, _ = timed_launches(backend, ev, lambda: backend.elemwise(x, ElemwiseOp.geluApprox, None, R * C, F32), 50, 10)
     report("cfg4_gelu", ms, nbytes=2 * nb)
     dims = ReduceDims(R, C, 1)
@@ -231,6 +234,24 @@ def extra_workloads(backend):
     ms, _ = timed_launches(backend, ev, lambda: backend.gather(table, emb, F32), 50, 10)
     report("cfg4_embedding_gather", ms, nbytes=65536 * 8 + 2 * 65536 * 1024 * 4)
     del max_gather
+
+    # config 5: decoder-only transformer forward, 8 x 256 tokens; tokens/s = 2048 / wall time of
+    # a forward pass ending in wait() on the logits (host-side op dispatch included)
+    from honeycrisp_amd.nn import Transformer
+    from honeycrisp_amd.tensor import Tensor
+    ids = np.random.default_rng(11).integers(0, 8192, size=(8, 256))
+    with backend.use():
+        for name, dtype in (("cfg5_transformer_fwd_f32", F32), ("cfg5_transformer_fwd_f16", F16)):
+            model = Transformer(dtype=dtype)
+            tokens = Tensor(data=ids)
+            for _ in range(2):
+                model(tokens).wait()
+            t0 = time.perf_counter()
+            for _ in range(5):
+                model(tokens).wait()
+            dt = (time.perf_counter() - t0) / 5
+            out[name] = {"ms": round(dt * 1e3, 3), "tokens_per_s": round(2048 / dt, 1),
+                         "tflops": round(100.9e9 / dt / 1e12, 2)}
     return out
 
 

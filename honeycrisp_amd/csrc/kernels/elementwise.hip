@@ -301,6 +301,14 @@ __device__ __forceinline__ float simple_erf_grad(float f) {
   return fabsf(f) > 20.0f ? 0.0f : 1.1283791670955126f * expf(-f * f);
 }
 
+// powf(f, 3.0f) of the reference formula: the cube formed in double and rounded once is the
+// correctly rounded result, which is what a libm powf returns for this exponent, at a
+// fraction of the cost of a general powf.
+__device__ __forceinline__ float cube(float f) {
+  const double d = (double)f;
+  return (float)(d * d * d);
+}
+
 enum {
   E_SIN = 0, E_COS, E_MINUS_SIN, E_TAN, E_TAN_GRAD, E_ATAN, E_ATAN_GRAD, E_ACOS, E_ACOS_GRAD,
   E_ASIN, E_ASIN_GRAD, E_EXP, E_LOG, E_RECIP, E_SIGMOID, E_SIGMOID_GRAD, E_RELU, E_RELU_GRAD,
@@ -331,7 +339,7 @@ template <int OP> __device__ __forceinline__ float elemwise_apply(float f) {
     case E_ABS: return f < 0.0f ? -f : f;
     case E_ABS_GRAD: return f < 0.0f ? -1.0f : 1.0f;
     case E_GELU_APPROX:
-      return 0.5f * f * (1.0f + safe_tanh(0.797884561f * (f + 0.044715f * powf(f, 3.0f))));
+      return 0.5f * f * (1.0f + safe_tanh(0.797884561f * (f + 0.044715f * cube(f))));
     case E_GELU_APPROX_GRAD: {
       float tanh_term = tanhf(0.035677408145115f * powf(f, 3.0f) + 0.797884561f * f);
       return 0.5f * f * (1.0f - powf(tanh_term, 2.0f)) *
