@@ -1,0 +1,262 @@
+// C++ mirror of Honeycrisp's `Backend` op interface for the MI355X backend: same method names
+// and argument meaning as the open class in Sources/Honeycrisp/Backend.swift:170-815, errors
+// mapped onto the BackendError cases of Backend.swift:6-16. Header-only, on top of the C ABI
+// (include/hchip.h); every method enqueues on the context's in-order stream and returns a
+// device buffer (`Data`, the counterpart of Tensor.Data, Tensor.swift:69-85) immediately.
+#pragma once
+
+#include <cstdint>
+#include <cstring>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "../../include/hchip.h"
+
+namespace hc {
+
+enum class DType : int { int64 = HC_I64, boolean = HC_BOOL, float16 = HC_F16, float32 = HC_F32 };
+inline size_t byteSize(DType t) {
+  switch (t) {
+    case DType::int64: return 8;
+    case DType::boolean: return 1;
+    case DType::float16: return 2;
+    default: return 4;
+  }
+}
+
+struct BackendError : std::runtime_error {
+  enum Kind { notImplemented, allocationFailed, kernelFailed, failedToLoadKernels } kind;
+  BackendError(Kind k, const std::string& msg) : std::runtime_error(msg), kind(k) {}
+};
+
+// BroadcastStrides (Broadcast.swift:9-30).
+struct BroadcastStrides {
+  std::vector<int64_t> shape, strides;
+  static BroadcastStrides contiguous(const std::vector<int64_t>& shape) {
+    BroadcastStrides s{shape, std::vector<int64_t>(shape.size())};
+    int64_t acc = 1;
+    for (size_t i = shape.size(); i-- > 0;) {
+      s.strides[i] = acc;
+      acc *= shape[i];
+    }
+    return s;
+  }
+  int64_t count() const {
+    int64_t n = 1;
+    for (int64_t d : shape) n *= d;
+    return n;
+  }
+  hc_strides c() const {
+    if (shape.size() > HC_MAX_DIMS) throw BackendError(BackendError::kernelFailed, "more than 8 axes");
+    hc_strides s;
+    std::memset(&s, 0, sizeof(s));
+    s.ndim = (uint32_t)shape.size();
+    for (size_t i = 0; i < shape.size(); i++) {
+      s.shape[i] = shape[i];
+      s.strides[i] = strides[i];
+    }
+    return s;
+  }
+};
+
+struct ReduceDims {
+  int64_t outerCount, reduceCount, innerCount;
+  int64_t inCount() const { return outerCount * reduceCount * innerCount; }
+  int64_t outCount() const { return outerCount * innerCount; }
+};
+
+class HIPBackend;
+
+// Device buffer; freed (stream-ordered) when the last reference goes away.
+class Buffer {
+ public:
+  Buffer(hc_ctx* ctx, void* ptr, size_t bytes) : ctx_(ctx), ptr_(ptr), bytes_(bytes) {}
+  ~Buffer() { hc_free(ctx_, ptr_); }
+  Buffer(const Buffer&) = delete;
+  Buffer& operator=(const Buffer&) = delete;
+  void* ptr() const { return ptr_; }
+  size_t byteCount() const { return bytes_; }
+
+ private:
+  hc_ctx* ctx_;
+  void* ptr_;
+  size_t bytes_;
+};
+typedef std::shared_ptr<Buffer> Data;
+
+struct BroadcastData {
+  BroadcastStrides strides;
+  Data data;
+};
+
+// ScatterGatherIndices (ScatterGather.swift:4-46).
+struct ScatterGatherIndices {
+  std::vector<int64_t> valueShape;
+  int axis;
+  BroadcastData indices;
+  int64_t outer() const { return prod(0, axis); }
+  int64_t middle() const { return valueShape[axis]; }
+  int64_t inner() const { return prod(axis + 1, (int)valueShape.size()); }
+  int64_t outCount() const { return indices.strides.shape[axis]; }
+  int64_t prod(int a, int b) const {
+    int64_t n = 1;
+    for (int i = a; i < b; i++) n *= valueShape[i];
+    return n;
+  }
+};
+
+class HIPBackend {
+ public:
+  explicit HIPBackend(int device = 0) { check(hc_init(device, &ctx_)); }
+  ~HIPBackend() { hc_shutdown(ctx_); }
+  HIPBackend(const HIPBackend&) = delete;
+  HIPBackend& operator=(const HIPBackend&) = delete;
+  hc_ctx* context() const { return ctx_; }
+
+  // ---- storage
+  Data allocate(size_t byteCount) {
+    void* p = nullptr;
+    check(hc_malloc(ctx_, byteCount, &p));
+    return std::make_shared<Buffer>(ctx_, p, byteCount);
+  }
+  Data upload(const void* host, size_t bytes) {
+    Data d = allocate(bytes);
+    check(hc_memcpy_h2d(ctx_, d->ptr(), host, bytes));
+    return d;
+  }
+  void download(const Data& d, void* host, size_t bytes) { check(hc_memcpy_d2h(ctx_, host, d->ptr(), bytes)); }
+  void wait() { check(hc_sync(ctx_)); }
+
+  // ---- ops (Backend.swift line of each declaration in the comment)
+  Data broadcast(const BroadcastData& a, DType dtype) {  // :170
+    Data out = allocate(a.strides.count() * byteSize(dtype));
+    hc_strides s = a.strides.c();
+    check(hc_broadcast(ctx_, (int)dtype, a.data->ptr(), &s, out->ptr()));
+    return out;
+  }
+  Data binaryOp(const BroadcastData& a, const BroadcastData& b, hc_binary op, DType dtype) {  // :178
+    Data out = allocate(a.strides.count() * byteSize(dtype));
+    hc_strides sa = a.strides.c(), sb = b.strides.c();
+    check(hc_binary_op(ctx_, op, (int)dtype, a.data->ptr(), &sa, b.data->ptr(), &sb, out->ptr()));
+    return out;
+  }
+  template <typename T> Data binaryOp(const Data& a, T b, hc_binary op, size_t count, DType dtype) {  // :190
+    Data out = allocate(count * byteSize(dtype));
+    check(hc_binary_op_scalar(ctx_, op, (int)dtype, a->ptr(), (float)b, (int64_t)b, 0, out->ptr(), count));
+    return out;
+  }
+  template <typename T> Data binaryOp(T a, const Data& b, hc_binary op, size_t count, DType dtype) {  // :202
+    Data out = allocate(count * byteSize(dtype));
+    check(hc_binary_op_scalar(ctx_, op, (int)dtype, b->ptr(), (float)a, (int64_t)a, 1, out->ptr(), count));
+    return out;
+  }
+  Data mulAdd(const BroadcastData& input, const BroadcastData& coeff, const BroadcastData& bias, DType dtype) {  // :240
+    Data out = allocate(input.strides.count() * byteSize(dtype));
+    hc_strides si = input.strides.c(), sc = coeff.strides.c(), sb = bias.strides.c();
+    check(hc_mul_add(ctx_, (int)dtype, input.data->ptr(), &si, coeff.data->ptr(), &sc, bias.data->ptr(), &sb, out->ptr()));
+    return out;
+  }
+  Data addMul(const BroadcastData& input, const BroadcastData& bias, const BroadcastData& coeff, DType dtype) {  // :250
+    Data out = allocate(input.strides.count() * byteSize(dtype));
+    hc_strides si = input.strides.c(), sc = coeff.strides.c(), sb = bias.strides.c();
+    check(hc_add_mul(ctx_, (int)dtype, input.data->ptr(), &si, bias.data->ptr(), &sb, coeff.data->ptr(), &sc, out->ptr()));
+    return out;
+  }
+  Data normalize(const Data& input, ReduceDims dims, float eps, DType dtype) {  // :265
+    Data out = allocate(dims.inCount() * byteSize(dtype));
+    check(hc_normalize(ctx_, (int)dtype, input->ptr(), out->ptr(), dims.outerCount, dims.reduceCount, dims.innerCount, eps));
+    return out;
+  }
+  Data compare(const BroadcastData& a, const BroadcastData& b, hc_compare_op op, DType dtype) {  // :457
+    Data out = allocate(a.strides.count());
+    hc_strides sa = a.strides.c(), sb = b.strides.c();
+    check(hc_compare(ctx_, op, (int)dtype, a.data->ptr(), &sa, b.data->ptr(), &sb, out->ptr()));
+    return out;
+  }
+  Data cast(const Data& a, size_t count, DType inType, DType outType) {  // :489
+    Data out = allocate(count * byteSize(outType));
+    check(hc_cast(ctx_, a->ptr(), (int)inType, out->ptr(), (int)outType, count));
+    return out;
+  }
+  template <typename T> Data pow(const Data& a, T b, T scale, const Data& scales, size_t count, DType dtype) {  // :500
+    Data out = allocate(count * byteSize(dtype));
+    check(hc_pow(ctx_, (int)dtype, a->ptr(), (float)b, (float)scale, (int64_t)b, (int64_t)scale,
+                 scales ? scales->ptr() : nullptr, out->ptr(), count));
+    return out;
+  }
+  Data reduce(const Data& a, hc_reduce_op op, ReduceDims dims, DType dtype) {  // :524
+    const DType outType = (op == HC_ARGMAX || op == HC_ARGMIN) ? DType::int64 : dtype;
+    Data out = allocate(dims.outCount() * byteSize(outType));
+    check(hc_reduce(ctx_, op, (int)dtype, a->ptr(), out->ptr(), dims.outerCount, dims.reduceCount, dims.innerCount));
+    return out;
+  }
+  Data logSoftmax(const Data& a, ReduceDims dims, DType dtype) {  // :571
+    Data out = allocate(dims.inCount() * byteSize(dtype));
+    check(hc_log_softmax(ctx_, (int)dtype, a->ptr(), out->ptr(), dims.outerCount, dims.reduceCount, dims.innerCount));
+    return out;
+  }
+  Data gather(const Data& a, const ScatterGatherIndices& s, DType dtype) {  // :609
+    Data out = allocate(s.indices.strides.count() * byteSize(dtype));
+    hc_strides st = s.indices.strides.c();
+    check(hc_gather(ctx_, (int)dtype, a->ptr(), s.indices.data->ptr(), &st, out->ptr(), s.outer(), s.middle(),
+                    s.outCount(), s.inner()));
+    return out;
+  }
+  Data when(const BroadcastData& mask, const BroadcastData& a, const BroadcastData& b, DType dtype) {  // :633
+    Data out = allocate(mask.strides.count() * byteSize(dtype));
+    hc_strides sm = mask.strides.c(), sa = a.strides.c(), sb = b.strides.c();
+    check(hc_when(ctx_, (int)dtype, mask.data->ptr(), &sm, a.data->ptr(), &sa, b.data->ptr(), &sb, out->ptr()));
+    return out;
+  }
+  Data matmul(const Data& a, bool transA, const Data& b, bool transB, bool transOut, int64_t rows, int64_t inner,
+              int64_t cols, DType dtype) {  // :650
+    return batchedMatmul(1, a, transA, b, transB, transOut, rows, inner, cols, dtype);
+  }
+  Data batchedMatmul(int64_t matrixCount, const Data& a, bool transA, const Data& b, bool transB, bool transOut,
+                     int64_t rows, int64_t inner, int64_t cols, DType dtype) {  // :661
+    Data out = allocate((size_t)(matrixCount * rows * cols) * byteSize(dtype));
+    check(hc_matmul(ctx_, (int)dtype, matrixCount, a->ptr(), transA, b->ptr(), transB, transOut, rows, inner, cols, out->ptr()));
+    return out;
+  }
+  Data triangular(const Data& a, int64_t batch, int64_t rows, int64_t cols, bool upper, int64_t offset, DType dtype) {  // :674
+    Data out = allocate((size_t)(batch * rows * cols) * byteSize(dtype));
+    check(hc_triangular(ctx_, (int)dtype, a->ptr(), out->ptr(), batch, rows, cols, upper, offset));
+    return out;
+  }
+  Data elemwise(const Data& a, hc_elemwise_op op, const Data& scales, size_t count, DType dtype) {  // :770
+    Data out = allocate(count * byteSize(dtype));
+    check(hc_elemwise(ctx_, op, (int)dtype, a->ptr(), scales ? scales->ptr() : nullptr, out->ptr(), count));
+    return out;
+  }
+  template <typename T> Data constant(T value, size_t count, DType dtype) {  // :787
+    Data out = allocate(count * byteSize(dtype));
+    check(hc_fill(ctx_, (int)dtype, (float)value, (int64_t)value, out->ptr(), count));
+    return out;
+  }
+  Data axisPermutation(const std::vector<int64_t>& permutation, const std::vector<int64_t>& shape) {  // :803
+    int64_t n = 1;
+    for (int64_t d : shape) n *= d;
+    Data out = allocate((size_t)n * 8);
+    check(hc_axis_permutation(ctx_, permutation.data(), shape.data(), (int)shape.size(), out->ptr()));
+    return out;
+  }
+
+  void check(int status) {
+    if (status == HC_OK) return;
+    const std::string msg = hc_last_error_string();
+    switch (status) {
+      case HC_ERR_ALLOC: throw BackendError(BackendError::allocationFailed, msg);
+      case HC_ERR_LOAD:
+      case HC_ERR_NO_DEVICE: throw BackendError(BackendError::failedToLoadKernels, msg);
+      case HC_ERR_UNSUPPORTED: throw BackendError(BackendError::notImplemented, msg);
+      default: throw BackendError(BackendError::kernelFailed, msg);
+    }
+  }
+
+ private:
+  hc_ctx* ctx_ = nullptr;
+};
+
+}  // namespace hc

@@ -1,0 +1,39 @@
+// swift-tools-version: 5.10
+// SwiftPM package of the MI355X backend for Honeycrisp. NOT built in the authoring environment
+// (no Swift toolchain there); it is the binding a maintainer adds next to Honeycrisp.
+//
+// CHCHIP is the thin C target: it only re-exports include/hchip.h and links libhchip.so,
+// which wraps hipMalloc / hipMemcpyAsync / hipModuleLaunchKernel over the embedded gfx950
+// code objects. Build libhchip.so first: `python -m honeycrisp_amd.csrc.build`.
+import PackageDescription
+
+let package = Package(
+  name: "HoneycrispHIP",
+  platforms: [.macOS(.v13)],
+  products: [
+    .library(name: "HoneycrispHIP", targets: ["HoneycrispHIP"]),
+    .executable(name: "HCMatrixBench", targets: ["HCMatrixBench"]),
+  ],
+  dependencies: [
+    // A Linux-buildable checkout of Honeycrisp (Accelerate / Metal shim modules in place).
+    .package(path: "../../honeycrisp")
+  ],
+  targets: [
+    .systemLibrary(name: "CHCHIP", path: "Sources/CHCHIP"),
+    .target(
+      name: "HoneycrispHIP",
+      dependencies: ["CHCHIP", .product(name: "Honeycrisp", package: "honeycrisp")],
+      linkerSettings: [
+        .unsafeFlags(["-L../honeycrisp_amd/csrc", "-Xlinker", "-rpath", "-Xlinker", "../honeycrisp_amd/csrc"])
+      ]),
+    .executableTarget(
+      name: "HCMatrixBench",
+      dependencies: ["HoneycrispHIP", .product(name: "Honeycrisp", package: "honeycrisp")]),
+    .testTarget(
+      name: "HoneycrispHIPTests",
+      dependencies: [
+        "HoneycrispHIP", .product(name: "Honeycrisp", package: "honeycrisp"),
+        .product(name: "HCTestUtils", package: "honeycrisp"),
+      ]),
+  ]
+)
