@@ -63,6 +63,15 @@ def build_all(verbose=True):
     ])
     if verbose:
         print("built", os.path.relpath(LIB_PATH, HERE), os.path.getsize(LIB_PATH), "bytes")
+    if LIB_PATH == os.path.join(HERE, "libhchip.so"):
+        # C++ host mirror + HCMatrixBench (links the library just built)
+        cpp = os.path.join(os.path.dirname(HERE), "cpp")
+        bench = os.path.join(cpp, "HCMatrixBench")
+        _run(["g++", "-O2", "-std=c++17", os.path.join(cpp, "HCMatrixBench.cpp"), "-o", bench,
+              "-L" + HERE, "-lhchip", "-Wl,-rpath,$ORIGIN/../csrc",
+              "-L" + os.path.join(ROCM, "lib"), "-Wl,-rpath-link," + os.path.join(ROCM, "lib")])
+        if verbose:
+            print("built", os.path.relpath(bench, HERE))
     return LIB_PATH
 
 
