@@ -31,6 +31,10 @@ sys.path.insert(0, ROOT)
 PEAK_F16_TFLOPS = 2516.6  # MI355X dense fp16 MFMA
 PEAK_F32_TFLOPS = 157.3   # MI355X fp32 MFMA
 PEAK_HBM_GBS = 8000.0     # MI355X HBM3E
+# HBM bytes per 4096^3 fp16 GEMM launch, from rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs of
+# this benchmark scaled by a plain copy kernel (not measurable live; the run that produced it is
+# summarised in profiles/bench_hbm_traffic_fetch_write_size.md): 295062 KiB read + 32768 KiB written.
+GEMM_TRAFFIC_BYTES = (295062 + 32768) * 1024
 
 
 class Events:
@@ -121,7 +125,7 @@ def headline(backend, steps, warmup):
     roofline = {
         "bound": "mfma", "kernel": "fp16 GEMM 4096^3 layout %s" % worst, "achieved": round(achieved, 2),
         "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s", "frac": round(achieved / PEAK_F16_TFLOPS, 4),
-        "traffic": None,
+        "traffic": GEMM_TRAFFIC_BYTES,
         "per_layout_tflops": {k: round(flops / (v * 1e-3) / 1e12, 2) for k, v in layout_ms.items()},
         "per_layout_ms": {k: round(v, 4) for k, v in layout_ms.items()},
     }
