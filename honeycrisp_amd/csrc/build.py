@@ -23,6 +23,7 @@ KERNELS = [
     ("gather", "gather.hip", []),
     ("gemm", "gemm.hip", []),
     ("gemm_f16_fast", "gemm_f16_fast.hip", []),
+    ("gemm_f16_dma", "gemm_f16_dma.hip", []),
 ]
 DEVICE_FLAGS = [
     "--offload-arch=gfx950", "--genco", "-O3", "-std=c++17",
@@ -47,7 +48,7 @@ def build_kernel(name, src, extra):
 
 def build_all(verbose=True):
     os.makedirs(BUILD_DIR, exist_ok=True)
-    with ThreadPoolExecutor(max_workers=4) as pool:
+    with ThreadPoolExecutor(max_workers=6) as pool:
         futures = [pool.submit(build_kernel, *k) for k in KERNELS]
         for f in futures:
             path = f.result()

@@ -26,6 +26,7 @@ extern const unsigned char hc_image_reduce[], hc_image_reduce_end[];
 extern const unsigned char hc_image_gather[], hc_image_gather_end[];
 extern const unsigned char hc_image_gemm[], hc_image_gemm_end[];
 extern const unsigned char hc_image_gemm_f16_fast[], hc_image_gemm_f16_fast_end[];
+extern const unsigned char hc_image_gemm_f16_dma[], hc_image_gemm_f16_dma_end[];
 }
 
 struct hc_module {
@@ -129,6 +130,7 @@ extern "C" int hc_init(int device, hc_ctx** out) {
   if (s == HC_OK) s = load_image(ctx, hc_image_gather, hc_image_gather_end, "gather");
   if (s == HC_OK) s = load_image(ctx, hc_image_gemm, hc_image_gemm_end, "gemm");
   if (s == HC_OK) s = load_image(ctx, hc_image_gemm_f16_fast, hc_image_gemm_f16_fast_end, "gemm_f16_fast");
+  if (s == HC_OK) s = load_image(ctx, hc_image_gemm_f16_dma, hc_image_gemm_f16_dma_end, "gemm_f16_dma");
   if (s != HC_OK) {
     hc_shutdown(ctx);
     return s;
@@ -1267,8 +1269,13 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
   if (bm != 0) {
     k.tiles_m = M / bm;
     k.tiles_n = N / bn;
-    snprintf(name, sizeof(name), "hc_gemm_f16_fast_%ux%u_%c%c", bm, bn, ma == 'k' ? 'k' : 'm',
-             mb == 'k' ? 'k' : 'n');
+    // HCHIP_GEMM_KERNEL=staged selects the register-staged pipeline (for measurements); the
+    // direct-to-LDS pipeline addresses operands with 32-bit byte offsets.
+    const char* which = getenv("HCHIP_GEMM_KERNEL");
+    const bool small = k.a_bs <= 0x7fffffffull && k.b_bs <= 0x7fffffffull;
+    const bool dma = small && !(which && strcmp(which, "staged") == 0);
+    snprintf(name, sizeof(name), "hc_gemm_f16_%s_%ux%u_%c%c", dma ? "dma" : "fast", bm, bn,
+             ma == 'k' ? 'k' : 'm', mb == 'k' ? 'k' : 'n');
   } else if (ma == 'x' || mb == 'x')
     snprintf(name, sizeof(name), "hc_gemm_%s_xx", dtype_name(dtype));
   else

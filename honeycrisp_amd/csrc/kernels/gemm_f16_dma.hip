@@ -1,0 +1,321 @@
+// fp16 GEMM for gfx950 with direct global->LDS loads (global_load_lds_dwordx4) and, for
+// operands that are contiguous along M/N, transposing LDS reads (ds_read_b64_tr_b16).
+// Same tiling as gemm_f16_fast.hip (block BM x BN x 64, 4 waves 2 x 2, fp32 accumulate with
+// v_mfma_f32_32x32x16_f16, whole tiles only), but no operand ever passes through VGPRs on
+// its way to LDS: that removes the register->LDS stores, which cost about 20 % of the MFMA
+// rate when issued from the same waves.
+//
+// LDS: two stages, each [A region: BM*128 bytes][B region: BN*128 bytes].
+//   K-contiguous operand (A of NN/NT, B of NT/TT): rows of 64 halfs = eight 16-byte slots,
+//     chunk c of row r in slot c ^ ((r ^ r>>3) & 7); MFMA operand = one ds_read_b128.
+//   M/N-contiguous operand (A of TN/TT, B of NN/TN): natural [k][m] layout, 64 k-rows of
+//     ROWS halfs, 16-byte slot x of k-row k stored at slot x ^ g(k),
+//     g(k) = ((k&7) ^ ((k>>3&1)<<2)) << 1. MFMA operand = two ds_read_b64_tr_b16: in a group
+//     of 16 lanes, lane r points at k-row k0 + r/4, columns 4*(r%4)..+3 (8 bytes); the
+//     instruction returns to lane i the four k-values of column i. Two reads (k0, k0+4) give
+//     a lane its 8 consecutive k for one m, in the same order as the K-contiguous operand.
+// A wave-level DMA instruction fills 1 KiB of LDS in lane order (lane l -> byte 16*l), so
+// any permutation of 16-byte pieces inside a 1 KiB block is free: the lane simply fetches
+// the global piece that belongs in its slot. Both swizzles stay inside such blocks.
+//
+// Pipeline per K-step (four 16-wide sub-steps): operands of sub-step s+1 are read under the
+// MFMAs of sub-step s. In sub-step 3, after half of the MFMAs: wait for this wave's DMA into
+// the other stage (issued one K-step ago), one LDS barrier, then issue the DMA of K-step k+2
+// into the stage just vacated and read the first operands of K-step k+1, all under the
+// remaining MFMAs. The two stages are distinct __shared__ arrays and the loop is unrolled by
+// two so that every LDS access names its stage statically.
+#include "common.hip.h"
+
+// Measurement switches (never set in the shipped build): bit0 no DMA in the K loop, bit1 no
+// wait/barrier, bit2 no LDS reads in the K loop. Results are wrong with any bit set.
+#ifndef HC_EXP
+#define HC_EXP 0
+#endif
+#ifndef HC_READS_PER_SLOT
+#define HC_READS_PER_SLOT 0
+#endif
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef uint32_t Chunk __attribute__((ext_vector_type(4)));  // 16 bytes = 8 halfs
+
+enum { DMA_K = 0, DMA_MN = 1 };
+
+#define LDS_AS __attribute__((address_space(3)))
+#define GLOBAL_AS __attribute__((address_space(1)))
+
+__device__ __forceinline__ uint32_t swz_k(uint32_t row) { return (row ^ (row >> 3)) & 7u; }
+__device__ __forceinline__ uint32_t swz_mn(uint32_t k) { return (((k & 7u) ^ (((k >> 3) & 1u) << 2)) << 1); }
+
+// LDS-only workgroup barrier.
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+// s_waitcnt vmcnt(0) with the other counters untouched (gfx9 encoding: vmcnt in bits 3:0 and
+// 15:14, expcnt 6:4, lgkmcnt 11:8).
+__device__ __forceinline__ void wait_dma() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
+// One operand of the block tile: where its DMA lanes fetch from and where a wave's MFMA
+// operand reads land.
+template <int ROWS, int MODE> struct DmaOperand {
+  static constexpr int NI = ROWS / 32;                        // DMA instructions per wave and K-step
+  static constexpr int TILES = ROWS / 64;                     // MFMA tiles per wave along this operand
+  static constexpr int READS = MODE == DMA_K ? TILES : 2 * TILES;  // LDS reads per sub-step
+  static constexpr int NADDR = MODE == DMA_K ? TILES * 4 : TILES * 2;
+  static constexpr int ROWB = ROWS * 2;                       // bytes per k-row (DMA_MN layout)
+
+  uint32_t goff[NI];     // byte offset of this lane's 16-byte piece for DMA instruction i (k = 0)
+  uint32_t kstride;      // bytes per unit of k
+  uint32_t raddr[NADDR]; // byte offsets (inside the operand's LDS region) of the MFMA operand reads
+
+  __device__ __forceinline__ void init(uint32_t rs, uint32_t cs, uint32_t r0, uint32_t woff) {
+    const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    if (MODE == DMA_K) {
+      kstride = 2;
+#pragma unroll
+      for (int i = 0; i < NI; i++) {
+        const uint32_t row = (wave * NI + i) * 8 + lane / 8;
+        const uint32_t c = (lane % 8) ^ swz_k(row);
+        goff[i] = ((r0 + row) * rs + c * 8) * 2;
+      }
+      const uint32_t lrow = lane & 31, lgrp = lane >> 5;
+#pragma unroll
+      for (int q = 0; q < TILES; q++) {
+        const uint32_t r = woff + q * 32 + lrow;
+#pragma unroll
+        for (int s = 0; s < 4; s++) raddr[q * 4 + s] = r * 128 + (((2 * s + lgrp) ^ swz_k(r)) * 16);
+      }
+    } else {
+      constexpr int KPI = 512 / ROWS;       // k-rows per DMA instruction
+      constexpr int SLOTS_PER_ROW = ROWS / 8;
+      kstride = cs * 2;
+#pragma unroll
+      for (int i = 0; i < NI; i++) {
+        const uint32_t krow = (wave * NI + i) * KPI + lane / SLOTS_PER_ROW;
+        const uint32_t slot = (lane % SLOTS_PER_ROW) ^ swz_mn(krow);
+        goff[i] = (krow * cs + r0 + slot * 8) * 2;
+      }
+      const uint32_t j = lane >> 4, r16 = lane & 15;
+#pragma unroll
+      for (int q = 0; q < TILES; q++) {
+        const uint32_t m = woff + q * 32 + 16 * (j & 1) + 4 * (r16 & 3);
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+          const uint32_t k = 8 * (j >> 1) + 4 * h + (r16 >> 2);  // + 16 * s as an immediate offset
+          raddr[q * 2 + h] = k * ROWB + (((m >> 3) ^ swz_mn(k)) * 16) + (m & 7) * 2;
+        }
+      }
+    }
+  }
+
+  // DMA instruction i of this wave for the K-slice starting at k0: 1 KiB into `region`.
+  __device__ __forceinline__ void dma(int i, const half_t* base, uint32_t k0, char* region) const {
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const char* src = (const char*)base + (size_t)k0 * kstride + goff[i];
+    __builtin_amdgcn_global_load_lds((const GLOBAL_AS void*)src, (LDS_AS void*)(region + (wave * NI + i) * 1024), 16, 0, 0);
+  }
+
+  // Read number u of sub-step s into the operand registers of tile u (DMA_K) or half u%2 of
+  // tile u/2 (DMA_MN).
+  __device__ __forceinline__ void read(int u, int s, const char* region, Chunk* frag) const {
+    if (MODE == DMA_K) {
+      frag[u] = *reinterpret_cast<const Chunk*>(region + raddr[u * 4 + s]);
+    } else {
+      const int q = u / 2, h = u % 2;
+      typedef short short4v __attribute__((ext_vector_type(4)));
+      const short4v v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (LDS_AS short4v*)(region + raddr[q * 2 + h] + s * 16 * ROWB));
+      typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+      const u32x2 w = __builtin_bit_cast(u32x2, v);
+      frag[q][2 * h] = w[0];
+      frag[q][2 * h + 1] = w[1];
+    }
+  }
+};
+
+template <int BM, int BN, int MODE_A, int MODE_B>
+__device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0, char* lds1) {
+  constexpr int MT = BM / 64, NT = BN / 64;
+  constexpr int SLOTS = MT * NT;
+  typedef DmaOperand<BM, MODE_A> OpA;
+  typedef DmaOperand<BN, MODE_B> OpB;
+  constexpr int READS = OpA::READS + OpB::READS;
+  constexpr int NDMA = OpA::NI + OpB::NI;
+  constexpr int A_BYTES = BM * 128;
+  static_assert(READS <= SLOTS || SLOTS >= 4, "tile too small");
+
+  // XCD-aware tile order: ids equal mod 8 land on one XCD; give that XCD a contiguous band.
+  const uint32_t total = p.tiles_m * p.tiles_n;
+  uint32_t tile = blockIdx.x;
+  if ((total & 7u) == 0) tile = (blockIdx.x & 7u) * (total >> 3) + (blockIdx.x >> 3);
+  const uint32_t tm = tile / p.tiles_n, tn = tile - tm * p.tiles_n;
+  const uint32_t m0 = tm * BM, n0 = tn * BN;
+  const uint32_t batch = blockIdx.y;
+  const half_t* A = (const half_t*)p.a + batch * p.a_bs;
+  const half_t* B = (const half_t*)p.b + batch * p.b_bs;
+  half_t* C = (half_t*)p.c + batch * p.c_bs;
+
+  const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const uint32_t wm = (wave >> 1) * (BM / 2), wn = (wave & 1) * (BN / 2);
+  const uint32_t lrow = lane & 31, lgrp = lane >> 5;
+
+  floatx16 acc[MT][NT];
+#pragma unroll
+  for (int i = 0; i < MT; i++)
+#pragma unroll
+    for (int j = 0; j < NT; j++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+
+  OpA oa;
+  OpB ob;
+  oa.init(p.a_rs, p.a_cs, m0, wm);
+  ob.init(p.b_cs, p.b_rs, n0, wn);
+
+  struct Frags {
+    Chunk a[MT];
+    Chunk b[NT];
+  };
+  // unit u of the operand reads of a sub-step: B's reads first, then A's
+  auto read_unit = [&](Frags& f, const char* stage, int s, int u) {
+    if (HC_EXP & 4) return;
+    if (u < OpB::READS) ob.read(u, s, stage + A_BYTES, f.b);
+    else if (u < READS) oa.read(u - OpB::READS, s, stage, f.a);
+  };
+  auto dma_unit = [&](int u, uint32_t k0, char* stage, bool in_loop = false) {
+    if ((HC_EXP & 1) && in_loop) return;
+    if (u < OpA::NI) oa.dma(u, A, k0, stage);
+    else if (u < NDMA) ob.dma(u - OpA::NI, B, k0, stage + A_BYTES);
+  };
+  // MFMA t of a sub-step; operands swapped (B first) so that a lane holds four consecutive
+  // n for one m (see the epilogue).
+  auto mma_one = [&](const Frags& f, int t) {
+    const int i = t / NT, j = t % NT;
+    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, f.b[j]),
+                                                       __builtin_bit_cast(half8, f.a[i]), acc[i][j], 0, 0, 0);
+  };
+  // reads per MFMA slot, full sub-step
+  constexpr int RPS = HC_READS_PER_SLOT ? HC_READS_PER_SLOT : (READS + SLOTS - 1) / SLOTS;
+  constexpr int RPS_TAIL = (READS + SLOTS / 2 - 1) / (SLOTS / 2);  // ... in half a sub-step
+  constexpr int DPS_TAIL = (NDMA + SLOTS / 2 - 1) / (SLOTS / 2);
+
+  const uint32_t nk = p.K / 64;
+  Frags f0, f1;
+
+  // One K-step computing out of `cur`; `nxt` holds (or is receiving) the next K-step.
+  auto step = [&](char* cur, char* nxt, uint32_t ks) {
+    const uint32_t k2 = (ks + 2 < nk ? ks + 2 : nk - 1) * 64;
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int t = 0; t < SLOTS; t++) {  // sub-step 0
+#pragma unroll
+      for (int e = 0; e < RPS; e++) read_unit(f1, cur, 1, t * RPS + e);
+      mma_one(f0, t);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int t = 0; t < SLOTS; t++) {  // sub-step 1
+#pragma unroll
+      for (int e = 0; e < RPS; e++) read_unit(f0, cur, 2, t * RPS + e);
+      mma_one(f1, t);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int t = 0; t < SLOTS; t++) {  // sub-step 2
+#pragma unroll
+      for (int e = 0; e < RPS; e++) read_unit(f1, cur, 3, t * RPS + e);
+      mma_one(f0, t);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // sub-step 3, first half
+#pragma unroll
+    for (int t = 0; t < SLOTS / 2; t++) mma_one(f1, t);
+    __builtin_amdgcn_sched_barrier(0);
+    if (!(HC_EXP & 2)) {
+      wait_dma();     // this wave's loads into nxt (issued one K-step ago) have landed
+      lds_barrier();  // ... and everybody's; nobody reads cur any more
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int t = SLOTS / 2; t < SLOTS; t++) {  // second half: refill cur, first operands of nxt
+      const int h = t - SLOTS / 2;
+#pragma unroll
+      for (int e = 0; e < DPS_TAIL; e++) dma_unit(h * DPS_TAIL + e, k2, cur, true);
+#pragma unroll
+      for (int e = 0; e < RPS_TAIL; e++) read_unit(f0, nxt, 0, h * RPS_TAIL + e);
+      mma_one(f1, t);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  // prologue: K-steps 0 and 1 into the two stages
+#pragma unroll
+  for (int u = 0; u < NDMA; u++) dma_unit(u, 0, lds0);
+#pragma unroll
+  for (int u = 0; u < NDMA; u++) dma_unit(u, nk > 1 ? 64 : 0, lds1);
+  wait_dma();
+  lds_barrier();
+#pragma unroll
+  for (int u = 0; u < READS; u++) read_unit(f0, lds0, 0, u);
+
+#ifdef HC_PROBE_CLOCKS
+  const uint64_t probe_c0 = __builtin_readcyclecounter(), probe_r0 = __builtin_amdgcn_s_memrealtime();
+#endif
+  uint32_t ks = 0;
+  for (; ks + 1 < nk; ks += 2) {
+    step(lds0, lds1, ks);
+    step(lds1, lds0, ks + 1);
+  }
+  if (ks < nk) step(lds0, lds1, ks);
+  wait_dma();  // no LDS write of this workgroup may be in flight when it ends
+#ifdef HC_PROBE_CLOCKS
+  // measurement build: the first 16 bytes of the block's C tile receive the K-loop duration
+  // in shader cycles and in 100 MHz ticks instead of results
+  const uint64_t probe_c1 = __builtin_readcyclecounter(), probe_r1 = __builtin_amdgcn_s_memrealtime();
+#endif
+
+  // Epilogue. With the operands swapped, the MFMA tile is C^T: lane l holds m = l % 32 and,
+  // in registers 4g..4g+3, the four consecutive columns n = 8g + 4*(l/32) + (0..3).
+#pragma unroll
+  for (int i = 0; i < MT; i++) {
+    const uint32_t row = m0 + wm + i * 32 + lrow;
+#pragma unroll
+    for (int j = 0; j < NT; j++) {
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        half4v h;
+#pragma unroll
+        for (int e = 0; e < 4; e++) h[e] = narrow<half_t>(acc[i][j][4 * g + e]);
+        const uint32_t col = n0 + wn + j * 32 + 8 * g + 4 * lgrp;
+        *reinterpret_cast<half4v*>(C + (size_t)row * p.c_rs + col) = h;
+      }
+    }
+  }
+#ifdef HC_PROBE_CLOCKS
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    uint64_t* dst = reinterpret_cast<uint64_t*>(C + (size_t)m0 * p.c_rs + n0);
+    dst[0] = probe_c1 - probe_c0;
+    dst[1] = probe_r1 - probe_r0;
+  }
+#endif
+}
+
+#define DEF_DMA(BM, BN, AN, AM, BNAME, BMODE)                                                         \
+  extern "C" __global__ __launch_bounds__(256) void hc_gemm_f16_dma_##BM##x##BN##_##AN##BNAME(        \
+      hck_gemm_args p) {                                                                              \
+    __shared__ __attribute__((aligned(1024))) char lds0[(BM + BN) * 128];                             \
+    __shared__ __attribute__((aligned(1024))) char lds1[(BM + BN) * 128];                             \
+    gemm_dma_impl<BM, BN, AM, BMODE>(p, lds0, lds1);                                                  \
+  }
+#define DEF_DMA_TILE(BM, BN)                                                                          \
+  DEF_DMA(BM, BN, k, DMA_K, k, DMA_K)                                                                 \
+  DEF_DMA(BM, BN, k, DMA_K, n, DMA_MN)                                                                \
+  DEF_DMA(BM, BN, m, DMA_MN, k, DMA_K)                                                                \
+  DEF_DMA(BM, BN, m, DMA_MN, n, DMA_MN)
+DEF_DMA_TILE(256, 256)
+DEF_DMA_TILE(256, 128)
+DEF_DMA_TILE(128, 128)
