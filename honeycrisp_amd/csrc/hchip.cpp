@@ -1274,6 +1274,17 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
     const char* which = getenv("HCHIP_GEMM_KERNEL");
     const bool small = k.a_bs <= 0x7fffffffull && k.b_bs <= 0x7fffffffull;
     const bool dma = small && !(which && strcmp(which, "staged") == 0);
+    if (dma && !getenv("HCHIP_GEMM_BAND")) {
+      // largest XCD rectangle whose super-block (4 x 2 XCDs) divides the tile grid
+      static const uint32_t shapes[][2] = {{4, 8}, {2, 4}, {1, 2}};
+      for (auto& sh : shapes)
+        if (k.tiles_m % (4 * sh[0]) == 0 && k.tiles_n % (2 * sh[1]) == 0) {
+          k.xcd_gn = 2;
+          k.xcd_sm = sh[0];
+          k.xcd_sn = sh[1];
+          break;
+        }
+    }
     snprintf(name, sizeof(name), "hc_gemm_f16_%s_%ux%u_%c%c", dma ? "dma" : "fast", bm, bn,
              ma == 'k' ? 'k' : 'm', mb == 'k' ? 'k' : 'n');
   } else if (ma == 'x' || mb == 'x')

@@ -143,6 +143,11 @@ typedef struct {
   uint32_t a_rs, a_cs, b_rs, b_cs, c_rs, c_cs;
   uint64_t a_bs, b_bs, c_bs;
   uint32_t tiles_m, tiles_n;
+  /* Tile order of the direct-to-LDS kernels. xcd_gn == 0: block ids equal mod 8 (one XCD)
+   * get a contiguous band of tiles. Otherwise the tile grid is cut into super-blocks of
+   * (8/xcd_gn * xcd_sm) x (xcd_gn * xcd_sn) tiles, visited one after the other; inside one,
+   * the 8 XCDs form an (8/xcd_gn) x xcd_gn grid and each owns xcd_sm x xcd_sn tiles. */
+  uint32_t xcd_gn, xcd_sm, xcd_sn;
 } hck_gemm_args;
 
 #endif

@@ -1,14 +1,16 @@
 // fp16 GEMM for gfx950 with direct global->LDS loads (global_load_lds_dwordx4) and, for
 // operands that are contiguous along M/N, transposing LDS reads (ds_read_b64_tr_b16).
-// Same tiling as gemm_f16_fast.hip (block BM x BN x 64, 4 waves 2 x 2, fp32 accumulate with
-// v_mfma_f32_32x32x16_f16, whole tiles only), but no operand ever passes through VGPRs on
-// its way to LDS: that removes the register->LDS stores, which cost about 20 % of the MFMA
-// rate when issued from the same waves.
+// Block tile BM x BN, 4 waves 2 x 2, fp32 accumulate with v_mfma_f32_32x32x16_f16, whole
+// tiles only. No operand passes through VGPRs on its way to LDS: that removes the
+// register->LDS stores, which cost about 20 % of the MFMA rate when issued from the same
+// waves.
 //
-// LDS: two stages, each [A region: BM*128 bytes][B region: BN*128 bytes].
-//   K-contiguous operand (A of NN/NT, B of NT/TT): rows of 64 halfs = eight 16-byte slots,
-//     chunk c of row r in slot c ^ ((r ^ r>>3) & 7); MFMA operand = one ds_read_b128.
-//   M/N-contiguous operand (A of TN/TT, B of NN/TN): natural [k][m] layout, 64 k-rows of
+// LDS: a ring of four stages, each one K-slice of 32: [A region: BM*64 bytes][B region:
+// BN*64 bytes].
+//   K-contiguous operand (A of NN/NT, B of NT/TT): rows of 32 halfs = four 16-byte slots,
+//     chunk c of row r in slot c ^ f(r), f(r) = ((r>>1)&3) ^ ((r>>3)&1); MFMA operand = one
+//     ds_read_b128.
+//   M/N-contiguous operand (A of TN/TT, B of NN/TN): natural [k][m] layout, 32 k-rows of
 //     ROWS halfs, 16-byte slot x of k-row k stored at slot x ^ g(k),
 //     g(k) = ((k&7) ^ ((k>>3&1)<<2)) << 1. MFMA operand = two ds_read_b64_tr_b16: in a group
 //     of 16 lanes, lane r points at k-row k0 + r/4, columns 4*(r%4)..+3 (8 bytes); the
@@ -18,12 +20,20 @@
 // any permutation of 16-byte pieces inside a 1 KiB block is free: the lane simply fetches
 // the global piece that belongs in its slot. Both swizzles stay inside such blocks.
 //
-// Pipeline per K-step (four 16-wide sub-steps): operands of sub-step s+1 are read under the
-// MFMAs of sub-step s. In sub-step 3, after half of the MFMAs: wait for this wave's DMA into
-// the other stage (issued one K-step ago), one LDS barrier, then issue the DMA of K-step k+2
-// into the stage just vacated and read the first operands of K-step k+1, all under the
-// remaining MFMAs. The two stages are distinct __shared__ arrays and the loop is unrolled by
-// two so that every LDS access names its stage statically.
+// Pipeline. The texture-address path of a CU accepts one 1 KiB DMA instruction per 16
+// cycles, i.e. a K-slice of 32 for a 256 x 256 tile keeps it busy for 512 of the 1024 cycles
+// its MFMAs take: DMA instructions issued in a burst stall the issuing waves (and their
+// MFMAs) behind that queue, so they are spread evenly, one every few MFMAs. That needs a
+// target stage that is free during the whole K-step, hence four stages: K-step j computes
+// out of stage j%4 in two 16-wide sub-steps,
+//   sub-step 0: MFMAs on operands read earlier; read the operands of sub-step 1; issue the
+//               second half of the DMA of K-step j+3 into stage (j-1)%4
+//   wait until this wave's DMA of K-step j+1 has landed (vmcnt = DMA instructions issued
+//               since), one LDS barrier: stage j%4 is now free, stage (j+1)%4 visible
+//   sub-step 1: MFMAs; read the first operands of K-step j+1; issue the first half of the
+//               DMA of K-step j+4 into stage j%4.
+// The stages are distinct __shared__ arrays and the loop is unrolled by four so that every
+// LDS access names its stage statically.
 #include "common.hip.h"
 
 // Measurement switches (never set in the shipped build): bit0 no DMA in the K loop, bit1 no
@@ -45,27 +55,33 @@ enum { DMA_K = 0, DMA_MN = 1 };
 #define LDS_AS __attribute__((address_space(3)))
 #define GLOBAL_AS __attribute__((address_space(1)))
 
-__device__ __forceinline__ uint32_t swz_k(uint32_t row) { return (row ^ (row >> 3)) & 7u; }
+__device__ __forceinline__ uint32_t swz_k(uint32_t row) { return ((row >> 1) & 3u) ^ ((row >> 3) & 1u); }
 __device__ __forceinline__ uint32_t swz_mn(uint32_t k) { return (((k & 7u) ^ (((k >> 3) & 1u) << 2)) << 1); }
 
-// LDS-only workgroup barrier.
+// Workgroup barrier for LDS traffic only: this wave's LDS reads have returned (lgkmcnt), its
+// DMA is waited for separately (wait_dma), and nothing is said about global memory. A fence
+// builtin would do the same but also waits for every DMA instruction in flight, including
+// those that fill stages nobody is about to read. The "memory" clobber keeps the compiler
+// from moving LDS accesses across it.
 __device__ __forceinline__ void lds_barrier() {
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-  __builtin_amdgcn_s_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
-// s_waitcnt vmcnt(0) with the other counters untouched (gfx9 encoding: vmcnt in bits 3:0 and
-// 15:14, expcnt 6:4, lgkmcnt 11:8).
-__device__ __forceinline__ void wait_dma() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+// s_waitcnt vmcnt(N) with the other counters untouched (gfx9 encoding: vmcnt in bits 3:0 and
+// 15:14, expcnt 6:4, lgkmcnt 11:8): at most N of this wave's DMA instructions still in flight.
+template <int N> __device__ __forceinline__ void wait_dma() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
+}
 
 // One operand of the block tile: where its DMA lanes fetch from and where a wave's MFMA
 // operand reads land.
 template <int ROWS, int MODE> struct DmaOperand {
-  static constexpr int NI = ROWS / 32;                        // DMA instructions per wave and K-step
+  static constexpr int NI = ROWS / 64;                        // DMA instructions per wave and K-step
   static constexpr int TILES = ROWS / 64;                     // MFMA tiles per wave along this operand
   static constexpr int READS = MODE == DMA_K ? TILES : 2 * TILES;  // LDS reads per sub-step
-  static constexpr int NADDR = MODE == DMA_K ? TILES * 4 : TILES * 2;
+  static constexpr int NADDR = TILES * 2;
   static constexpr int ROWB = ROWS * 2;                       // bytes per k-row (DMA_MN layout)
+  static constexpr int BYTES = ROWS * 64;                     // per stage
 
   uint32_t goff[NI];     // byte offset of this lane's 16-byte piece for DMA instruction i (k = 0)
   uint32_t kstride;      // bytes per unit of k
@@ -77,8 +93,8 @@ template <int ROWS, int MODE> struct DmaOperand {
       kstride = 2;
 #pragma unroll
       for (int i = 0; i < NI; i++) {
-        const uint32_t row = (wave * NI + i) * 8 + lane / 8;
-        const uint32_t c = (lane % 8) ^ swz_k(row);
+        const uint32_t row = (wave * NI + i) * 16 + lane / 4;
+        const uint32_t c = (lane % 4) ^ swz_k(row);
         goff[i] = ((r0 + row) * rs + c * 8) * 2;
       }
       const uint32_t lrow = lane & 31, lgrp = lane >> 5;
@@ -86,7 +102,7 @@ template <int ROWS, int MODE> struct DmaOperand {
       for (int q = 0; q < TILES; q++) {
         const uint32_t r = woff + q * 32 + lrow;
 #pragma unroll
-        for (int s = 0; s < 4; s++) raddr[q * 4 + s] = r * 128 + (((2 * s + lgrp) ^ swz_k(r)) * 16);
+        for (int s = 0; s < 2; s++) raddr[q * 2 + s] = r * 64 + (((2 * s + lgrp) ^ swz_k(r)) * 16);
       }
     } else {
       constexpr int KPI = 512 / ROWS;       // k-rows per DMA instruction
@@ -122,7 +138,7 @@ template <int ROWS, int MODE> struct DmaOperand {
   // tile u/2 (DMA_MN).
   __device__ __forceinline__ void read(int u, int s, const char* region, Chunk* frag) const {
     if (MODE == DMA_K) {
-      frag[u] = *reinterpret_cast<const Chunk*>(region + raddr[u * 4 + s]);
+      frag[u] = *reinterpret_cast<const Chunk*>(region + raddr[u * 2 + s]);
     } else {
       const int q = u / 2, h = u % 2;
       typedef short short4v __attribute__((ext_vector_type(4)));
@@ -137,20 +153,32 @@ template <int ROWS, int MODE> struct DmaOperand {
 };
 
 template <int BM, int BN, int MODE_A, int MODE_B>
-__device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0, char* lds1) {
+__device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0, char* lds1, char* lds2, char* lds3) {
   constexpr int MT = BM / 64, NT = BN / 64;
   constexpr int SLOTS = MT * NT;
   typedef DmaOperand<BM, MODE_A> OpA;
   typedef DmaOperand<BN, MODE_B> OpB;
   constexpr int READS = OpA::READS + OpB::READS;
-  constexpr int NDMA = OpA::NI + OpB::NI;
-  constexpr int A_BYTES = BM * 128;
-  static_assert(READS <= SLOTS || SLOTS >= 4, "tile too small");
+  constexpr int NDMA = OpA::NI + OpB::NI;  // per wave and K-step
+  constexpr int HALF = NDMA / 2;
+  constexpr int A_BYTES = OpA::BYTES;
 
-  // XCD-aware tile order: ids equal mod 8 land on one XCD; give that XCD a contiguous band.
+  // XCD-aware tile order. Block ids equal mod 8 run on one XCD and share its L2: give each
+  // XCD a compact rectangle of tiles (few distinct A and B panels), or a contiguous band.
   const uint32_t total = p.tiles_m * p.tiles_n;
   uint32_t tile = blockIdx.x;
-  if ((total & 7u) == 0) tile = (blockIdx.x & 7u) * (total >> 3) + (blockIdx.x >> 3);
+  if (p.xcd_gn != 0) {
+    const uint32_t per = 8 * p.xcd_sm * p.xcd_sn, gm = 8 / p.xcd_gn;
+    const uint32_t group = blockIdx.x / per, w = blockIdx.x - group * per;
+    const uint32_t x = w & 7u, t = w >> 3;
+    const uint32_t sbn = p.tiles_n / (p.xcd_gn * p.xcd_sn);
+    const uint32_t sb_row = group / sbn, sb_col = group - sb_row * sbn;
+    const uint32_t xm = x / p.xcd_gn, xn = x - xm * p.xcd_gn;
+    const uint32_t lm = t / p.xcd_sn, ln = t - lm * p.xcd_sn;
+    tile = (sb_row * gm * p.xcd_sm + xm * p.xcd_sm + lm) * p.tiles_n + sb_col * p.xcd_gn * p.xcd_sn + xn * p.xcd_sn + ln;
+  } else if ((total & 7u) == 0) {
+    tile = (blockIdx.x & 7u) * (total >> 3) + (blockIdx.x >> 3);
+  }
   const uint32_t tm = tile / p.tiles_n, tn = tile - tm * p.tiles_n;
   const uint32_t m0 = tm * BM, n0 = tn * BN;
   const uint32_t batch = blockIdx.y;
@@ -185,6 +213,7 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
     if (u < OpB::READS) ob.read(u, s, stage + A_BYTES, f.b);
     else if (u < READS) oa.read(u - OpB::READS, s, stage, f.a);
   };
+  // unit u of the DMA of the K-slice starting at k0
   auto dma_unit = [&](int u, uint32_t k0, char* stage, bool in_loop = false) {
     if ((HC_EXP & 1) && in_loop) return;
     if (u < OpA::NI) oa.dma(u, A, k0, stage);
@@ -197,66 +226,54 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, f.b[j]),
                                                        __builtin_bit_cast(half8, f.a[i]), acc[i][j], 0, 0, 0);
   };
-  // reads per MFMA slot, full sub-step
+  // reads per MFMA slot
   constexpr int RPS = HC_READS_PER_SLOT ? HC_READS_PER_SLOT : (READS + SLOTS - 1) / SLOTS;
-  constexpr int RPS_TAIL = (READS + SLOTS / 2 - 1) / (SLOTS / 2);  // ... in half a sub-step
-  constexpr int DPS_TAIL = (NDMA + SLOTS / 2 - 1) / (SLOTS / 2);
+  // one DMA instruction every DSTRIDE MFMAs
+  constexpr int DSTRIDE = SLOTS / (NDMA - HALF) > 0 ? SLOTS / (NDMA - HALF) : 1;
+  static_assert(DSTRIDE * (NDMA - HALF) <= SLOTS, "more DMA instructions than MFMA slots");
 
-  const uint32_t nk = p.K / 64;
+  const uint32_t nk = p.K / 32;
   Frags f0, f1;
 
-  // One K-step computing out of `cur`; `nxt` holds (or is receiving) the next K-step.
-  auto step = [&](char* cur, char* nxt, uint32_t ks) {
-    const uint32_t k2 = (ks + 2 < nk ? ks + 2 : nk - 1) * 64;
+  // K-step j out of `cur`; `nxt` holds K-step j+1, `prev` held K-step j-1.
+  auto step = [&](char* cur, char* nxt, char* prev, uint32_t j) {
+    const uint32_t k3 = (j + 3 < nk ? j + 3 : nk - 1) * 32, k4 = (j + 4 < nk ? j + 4 : nk - 1) * 32;
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int t = 0; t < SLOTS; t++) {  // sub-step 0
+      if (t % DSTRIDE == 0 && HALF + t / DSTRIDE < NDMA) dma_unit(HALF + t / DSTRIDE, k3, prev, true);
 #pragma unroll
       for (int e = 0; e < RPS; e++) read_unit(f1, cur, 1, t * RPS + e);
       mma_one(f0, t);
       __builtin_amdgcn_sched_barrier(0);
     }
+    if (!(HC_EXP & 2)) {
+      wait_dma<2 * NDMA>();  // K-step j+1 of this wave has landed ...
+      lds_barrier();         // ... and everybody's; nobody reads cur any more
+    }
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int t = 0; t < SLOTS; t++) {  // sub-step 1
+      if (t % DSTRIDE == 0 && t / DSTRIDE < HALF) dma_unit(t / DSTRIDE, k4, cur, true);
 #pragma unroll
-      for (int e = 0; e < RPS; e++) read_unit(f0, cur, 2, t * RPS + e);
-      mma_one(f1, t);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-#pragma unroll
-    for (int t = 0; t < SLOTS; t++) {  // sub-step 2
-#pragma unroll
-      for (int e = 0; e < RPS; e++) read_unit(f1, cur, 3, t * RPS + e);
-      mma_one(f0, t);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    // sub-step 3, first half
-#pragma unroll
-    for (int t = 0; t < SLOTS / 2; t++) mma_one(f1, t);
-    __builtin_amdgcn_sched_barrier(0);
-    if (!(HC_EXP & 2)) {
-      wait_dma();     // this wave's loads into nxt (issued one K-step ago) have landed
-      lds_barrier();  // ... and everybody's; nobody reads cur any more
-    }
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int t = SLOTS / 2; t < SLOTS; t++) {  // second half: refill cur, first operands of nxt
-      const int h = t - SLOTS / 2;
-#pragma unroll
-      for (int e = 0; e < DPS_TAIL; e++) dma_unit(h * DPS_TAIL + e, k2, cur, true);
-#pragma unroll
-      for (int e = 0; e < RPS_TAIL; e++) read_unit(f0, nxt, 0, h * RPS_TAIL + e);
+      for (int e = 0; e < RPS; e++) read_unit(f0, nxt, 0, t * RPS + e);
       mma_one(f1, t);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
 
-  // prologue: K-steps 0 and 1 into the two stages
+  // prologue: K-steps 0..2 and the first half of K-step 3 (slices past the end repeat the
+  // last one; nobody reads them)
+  auto kclamp = [&](uint32_t j) { return (j < nk ? j : nk - 1) * 32; };
 #pragma unroll
   for (int u = 0; u < NDMA; u++) dma_unit(u, 0, lds0);
 #pragma unroll
-  for (int u = 0; u < NDMA; u++) dma_unit(u, nk > 1 ? 64 : 0, lds1);
-  wait_dma();
+  for (int u = 0; u < NDMA; u++) dma_unit(u, kclamp(1), lds1);
+#pragma unroll
+  for (int u = 0; u < NDMA; u++) dma_unit(u, kclamp(2), lds2);
+#pragma unroll
+  for (int u = 0; u < HALF; u++) dma_unit(u, kclamp(3), lds3);
+  wait_dma<2 * NDMA + HALF>();
   lds_barrier();
 #pragma unroll
   for (int u = 0; u < READS; u++) read_unit(f0, lds0, 0, u);
@@ -264,13 +281,18 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
 #ifdef HC_PROBE_CLOCKS
   const uint64_t probe_c0 = __builtin_readcyclecounter(), probe_r0 = __builtin_amdgcn_s_memrealtime();
 #endif
-  uint32_t ks = 0;
-  for (; ks + 1 < nk; ks += 2) {
-    step(lds0, lds1, ks);
-    step(lds1, lds0, ks + 1);
+  uint32_t j = 0;
+  for (; j + 3 < nk; j += 4) {
+    step(lds0, lds1, lds3, j);
+    step(lds1, lds2, lds0, j + 1);
+    step(lds2, lds3, lds1, j + 2);
+    step(lds3, lds0, lds2, j + 3);
   }
-  if (ks < nk) step(lds0, lds1, ks);
-  wait_dma();  // no LDS write of this workgroup may be in flight when it ends
+  if (j < nk) {  // K is a multiple of 64: two K-steps left
+    step(lds0, lds1, lds3, j);
+    step(lds1, lds2, lds0, j + 1);
+  }
+  wait_dma<0>();  // no LDS write of this workgroup may be in flight when it ends
 #ifdef HC_PROBE_CLOCKS
   // measurement build: the first 16 bytes of the block's C tile receive the K-loop duration
   // in shader cycles and in 100 MHz ticks instead of results
@@ -307,9 +329,11 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
 #define DEF_DMA(BM, BN, AN, AM, BNAME, BMODE)                                                         \
   extern "C" __global__ __launch_bounds__(256) void hc_gemm_f16_dma_##BM##x##BN##_##AN##BNAME(        \
       hck_gemm_args p) {                                                                              \
-    __shared__ __attribute__((aligned(1024))) char lds0[(BM + BN) * 128];                             \
-    __shared__ __attribute__((aligned(1024))) char lds1[(BM + BN) * 128];                             \
-    gemm_dma_impl<BM, BN, AM, BMODE>(p, lds0, lds1);                                                  \
+    __shared__ __attribute__((aligned(1024))) char lds0[(BM + BN) * 64];                              \
+    __shared__ __attribute__((aligned(1024))) char lds1[(BM + BN) * 64];                              \
+    __shared__ __attribute__((aligned(1024))) char lds2[(BM + BN) * 64];                              \
+    __shared__ __attribute__((aligned(1024))) char lds3[(BM + BN) * 64];                              \
+    gemm_dma_impl<BM, BN, AM, BMODE>(p, lds0, lds1, lds2, lds3);                                      \
   }
 #define DEF_DMA_TILE(BM, BN)                                                                          \
   DEF_DMA(BM, BN, k, DMA_K, k, DMA_K)                                                                 \
