@@ -23,7 +23,7 @@ KERNELS = [
     ("gather", "gather.hip", []),
     ("gemm", "gemm.hip", []),
     ("gemm_f16_fast", "gemm_f16_fast.hip", []),
-    ("gemm_f16_dma", "gemm_f16_dma.hip", []),
+    ("gemm_dma", "gemm_dma.hip", []),
 ]
 DEVICE_FLAGS = [
     "--offload-arch=gfx950", "--genco", "-O3", "-std=c++17",

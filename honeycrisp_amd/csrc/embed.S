@@ -18,6 +18,6 @@
     EMBED hc_image_gather, "gather.hsaco"
     EMBED hc_image_gemm, "gemm.hsaco"
     EMBED hc_image_gemm_f16_fast, "gemm_f16_fast.hsaco"
-    EMBED hc_image_gemm_f16_dma, "gemm_f16_dma.hsaco"
+    EMBED hc_image_gemm_dma, "gemm_dma.hsaco"
 
     .section .note.GNU-stack,"",@progbits

@@ -26,7 +26,7 @@ extern const unsigned char hc_image_reduce[], hc_image_reduce_end[];
 extern const unsigned char hc_image_gather[], hc_image_gather_end[];
 extern const unsigned char hc_image_gemm[], hc_image_gemm_end[];
 extern const unsigned char hc_image_gemm_f16_fast[], hc_image_gemm_f16_fast_end[];
-extern const unsigned char hc_image_gemm_f16_dma[], hc_image_gemm_f16_dma_end[];
+extern const unsigned char hc_image_gemm_dma[], hc_image_gemm_dma_end[];
 }
 
 struct hc_module {
@@ -130,7 +130,7 @@ extern "C" int hc_init(int device, hc_ctx** out) {
   if (s == HC_OK) s = load_image(ctx, hc_image_gather, hc_image_gather_end, "gather");
   if (s == HC_OK) s = load_image(ctx, hc_image_gemm, hc_image_gemm_end, "gemm");
   if (s == HC_OK) s = load_image(ctx, hc_image_gemm_f16_fast, hc_image_gemm_f16_fast_end, "gemm_f16_fast");
-  if (s == HC_OK) s = load_image(ctx, hc_image_gemm_f16_dma, hc_image_gemm_f16_dma_end, "gemm_f16_dma");
+  if (s == HC_OK) s = load_image(ctx, hc_image_gemm_dma, hc_image_gemm_dma_end, "gemm_dma");
   if (s != HC_OK) {
     hc_shutdown(ctx);
     return s;
@@ -1240,12 +1240,20 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
   char ma = mode(k.a, a_rs, a_cs, k.a_bs);
   char mb = mode(k.b, b_cs, b_rs, k.b_bs);
   char name[64];
-  // Tuned fp16 kernels: whole tiles only. HCHIP_GEMM_TILE=general|256x256|256x128|128x128
-  // overrides the choice (for measurements).
+  // Tuned kernels: whole tiles only, K in whole 64-byte slices. HCHIP_GEMM_TILE=general|<BM>x<BN>
+  // overrides the choice and HCHIP_GEMM_KERNEL=staged selects the register-staged fp16
+  // pipeline (measurements). The direct-to-LDS kernels address operands with 32-bit byte
+  // offsets.
   uint32_t bm = 0, bn = 0;
-  if (dtype == HC_F16 && ma != 'x' && mb != 'x' && K > 0 && K % 64 == 0 && aligned16(out)) {
+  const char* which = getenv("HCHIP_GEMM_KERNEL");
+  const uint64_t max_elems = 0xffffffffull / el;
+  const bool dma = k.a_bs <= max_elems && k.b_bs <= max_elems && !(which && strcmp(which, "staged") == 0);
+  if ((dtype == HC_F16 || dma) && ma != 'x' && mb != 'x' && K > 0 && K % (64 / el) == 0 && aligned16(out)) {
     const char* force = getenv("HCHIP_GEMM_TILE");
     auto fits = [&](uint32_t tm, uint32_t tn) { return M % tm == 0 && N % tn == 0; };
+    // largest tile first; the direct-to-LDS kernels also come in narrow shapes
+    static const uint32_t tiles[][2] = {{256, 256}, {256, 128}, {128, 128}, {256, 64}, {128, 64}, {64, 64}};
+    const uint64_t cus = (uint64_t)ctx->props.multiProcessorCount;
     if (force && *force) {
       unsigned fm = 0, fn = 0;
       if (sscanf(force, "%ux%u", &fm, &fn) == 2 && fits(fm, fn)) {
@@ -1253,27 +1261,28 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
         bn = fn;
       }
     } else {
-      const uint64_t cus = (uint64_t)ctx->props.multiProcessorCount;
-      if (fits(256, 256) && (uint64_t)(M / 256) * (N / 256) * (uint64_t)batch >= cus) {
-        bm = 256;
-        bn = 256;
-      } else if (fits(256, 128) && (uint64_t)(M / 256) * (N / 128) * (uint64_t)batch >= cus) {
-        bm = 256;
-        bn = 128;
-      } else if (fits(128, 128)) {
-        bm = 128;
-        bn = 128;
+      // the largest tile that still gives every CU a block, else the one with most blocks
+      uint64_t best_blocks = 0;
+      for (auto& t : tiles) {
+        if (!fits(t[0], t[1]) || (!dma && t[1] < 128)) continue;
+        const uint64_t blocks = (uint64_t)(M / t[0]) * (N / t[1]) * (uint64_t)batch;
+        if (blocks >= cus) {
+          bm = t[0];
+          bn = t[1];
+          break;
+        }
+        if (blocks > best_blocks) {
+          best_blocks = blocks;
+          bm = t[0];
+          bn = t[1];
+        }
       }
     }
+    if (!dma && (K % 64 != 0 || bn < 128)) bm = bn = 0;  // the staged kernels step K by 64
   }
   if (bm != 0) {
     k.tiles_m = M / bm;
     k.tiles_n = N / bn;
-    // HCHIP_GEMM_KERNEL=staged selects the register-staged pipeline (for measurements); the
-    // direct-to-LDS pipeline addresses operands with 32-bit byte offsets.
-    const char* which = getenv("HCHIP_GEMM_KERNEL");
-    const bool small = k.a_bs <= 0x7fffffffull && k.b_bs <= 0x7fffffffull;
-    const bool dma = small && !(which && strcmp(which, "staged") == 0);
     if (dma && !getenv("HCHIP_GEMM_BAND")) {
       // largest XCD rectangle whose super-block (4 x 2 XCDs) divides the tile grid
       static const uint32_t shapes[][2] = {{4, 8}, {2, 4}, {1, 2}};
@@ -1285,7 +1294,7 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
           break;
         }
     }
-    snprintf(name, sizeof(name), "hc_gemm_f16_%s_%ux%u_%c%c", dma ? "dma" : "fast", bm, bn,
+    snprintf(name, sizeof(name), "hc_gemm_%s_%s_%ux%u_%c%c", dtype_name(dtype), dma ? "dma" : "fast", bm, bn,
              ma == 'k' ? 'k' : 'm', mb == 'k' ? 'k' : 'n');
   } else if (ma == 'x' || mb == 'x')
     snprintf(name, sizeof(name), "hc_gemm_%s_xx", dtype_name(dtype));

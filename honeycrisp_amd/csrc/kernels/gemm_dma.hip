@@ -1,21 +1,25 @@
-// fp16 GEMM for gfx950 with direct global->LDS loads (global_load_lds_dwordx4) and, for
-// operands that are contiguous along M/N, transposing LDS reads (ds_read_b64_tr_b16).
-// Block tile BM x BN, 4 waves 2 x 2, fp32 accumulate with v_mfma_f32_32x32x16_f16, whole
-// tiles only. No operand passes through VGPRs on its way to LDS: that removes the
-// register->LDS stores, which cost about 20 % of the MFMA rate when issued from the same
-// waves.
+// fp16 and fp32 GEMM for gfx950 with direct global->LDS loads (global_load_lds_dwordx4) and,
+// for fp16 operands that are contiguous along M/N, transposing LDS reads
+// (ds_read_b64_tr_b16). Block tile BM x BN, 4 waves 2 x 2, fp32 accumulate with
+// v_mfma_f32_32x32x16_f16 / v_mfma_f32_32x32x2_f32, whole tiles only. No operand passes
+// through VGPRs on its way to LDS: that removes the register->LDS stores, which cost about
+// 20 % of the MFMA rate when issued from the same waves.
 //
-// LDS: a ring of four stages, each one K-slice of 32: [A region: BM*64 bytes][B region:
-// BN*64 bytes].
-//   K-contiguous operand (A of NN/NT, B of NT/TT): rows of 32 halfs = four 16-byte slots,
+// LDS: a ring of four stages, each one K-slice of 64 bytes (32 halfs, 16 floats):
+// [A region: BM*64 bytes][B region: BN*64 bytes].
+//   K-contiguous operand (A of NN/NT, B of NT/TT): rows of 64 bytes = four 16-byte slots,
 //     chunk c of row r in slot c ^ f(r), f(r) = ((r>>1)&3) ^ ((r>>3)&1); MFMA operand = one
-//     ds_read_b128.
-//   M/N-contiguous operand (A of TN/TT, B of NN/TN): natural [k][m] layout, 32 k-rows of
+//     ds_read_b128. For fp32 the four floats of a chunk feed four consecutive MFMAs; lanes
+//     0..31 take chunk 2s and lanes 32..63 chunk 2s+1 in sub-step s, a permutation of k that
+//     both operands share.
+//   M/N-contiguous fp16 operand (A of TN/TT, B of NN/TN): natural [k][m] layout, 32 k-rows of
 //     ROWS halfs, 16-byte slot x of k-row k stored at slot x ^ g(k),
 //     g(k) = ((k&7) ^ ((k>>3&1)<<2)) << 1. MFMA operand = two ds_read_b64_tr_b16: in a group
 //     of 16 lanes, lane r points at k-row k0 + r/4, columns 4*(r%4)..+3 (8 bytes); the
 //     instruction returns to lane i the four k-values of column i. Two reads (k0, k0+4) give
 //     a lane its 8 consecutive k for one m, in the same order as the K-contiguous operand.
+//   M/N-contiguous fp32 operand: [16 k][ROWS floats], MFMA operands are single ds_read_b32
+//     (32 consecutive floats of k-row k for lanes 0..31, of k-row k+4 for lanes 32..63).
 // A wave-level DMA instruction fills 1 KiB of LDS in lane order (lane l -> byte 16*l), so
 // any permutation of 16-byte pieces inside a 1 KiB block is free: the lane simply fetches
 // the global piece that belongs in its slot. Both swizzles stay inside such blocks.
@@ -25,7 +29,7 @@
 // its MFMAs take: DMA instructions issued in a burst stall the issuing waves (and their
 // MFMAs) behind that queue, so they are spread evenly, one every few MFMAs. That needs a
 // target stage that is free during the whole K-step, hence four stages: K-step j computes
-// out of stage j%4 in two 16-wide sub-steps,
+// out of stage j%4 in two sub-steps (half a stage each),
 //   sub-step 0: MFMAs on operands read earlier; read the operands of sub-step 1; issue the
 //               second half of the DMA of K-step j+3 into stage (j-1)%4
 //   wait until this wave's DMA of K-step j+1 has landed (vmcnt = DMA instructions issued
@@ -48,6 +52,7 @@
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half4v __attribute__((ext_vector_type(4)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef uint32_t Chunk __attribute__((ext_vector_type(4)));  // 16 bytes = 8 halfs
 
 enum { DMA_K = 0, DMA_MN = 1 };
@@ -75,12 +80,15 @@ template <int N> __device__ __forceinline__ void wait_dma() {
 
 // One operand of the block tile: where its DMA lanes fetch from and where a wave's MFMA
 // operand reads land.
-template <int ROWS, int MODE> struct DmaOperand {
+template <typename T, int ROWS, int MODE> struct DmaOperand {
+  static constexpr int ES = sizeof(T);
+  static constexpr bool F32 = ES == 4;
   static constexpr int NI = ROWS / 64;                        // DMA instructions per wave and K-step
   static constexpr int TILES = ROWS / 64;                     // MFMA tiles per wave along this operand
-  static constexpr int READS = MODE == DMA_K ? TILES : 2 * TILES;  // LDS reads per sub-step
+  // LDS reads per sub-step
+  static constexpr int READS = MODE == DMA_K ? TILES : (F32 ? 4 * TILES : 2 * TILES);
   static constexpr int NADDR = TILES * 2;
-  static constexpr int ROWB = ROWS * 2;                       // bytes per k-row (DMA_MN layout)
+  static constexpr int ROWB = ROWS * ES;                      // bytes per k-row (DMA_MN layout)
   static constexpr int BYTES = ROWS * 64;                     // per stage
 
   uint32_t goff[NI];     // byte offset of this lane's 16-byte piece for DMA instruction i (k = 0)
@@ -90,12 +98,12 @@ template <int ROWS, int MODE> struct DmaOperand {
   __device__ __forceinline__ void init(uint32_t rs, uint32_t cs, uint32_t r0, uint32_t woff) {
     const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     if (MODE == DMA_K) {
-      kstride = 2;
+      kstride = ES;
 #pragma unroll
       for (int i = 0; i < NI; i++) {
         const uint32_t row = (wave * NI + i) * 16 + lane / 4;
         const uint32_t c = (lane % 4) ^ swz_k(row);
-        goff[i] = ((r0 + row) * rs + c * 8) * 2;
+        goff[i] = (r0 + row) * rs * ES + c * 16;
       }
       const uint32_t lrow = lane & 31, lgrp = lane >> 5;
 #pragma unroll
@@ -104,14 +112,32 @@ template <int ROWS, int MODE> struct DmaOperand {
 #pragma unroll
         for (int s = 0; s < 2; s++) raddr[q * 2 + s] = r * 64 + (((2 * s + lgrp) ^ swz_k(r)) * 16);
       }
+    } else if (F32) {
+      // [16 k][ROWS floats]; the 128-byte halves of every 256 bytes swap places in k-rows
+      // with bit 2 set: an MFMA operand read touches rows k and k + 4, 32 floats of each
+      constexpr uint32_t KPI = 1024 / ROWB;   // k-rows per DMA instruction
+      constexpr uint32_t PIECES = ROWB / 16;  // 16-byte pieces per k-row
+      kstride = cs * ES;
+#pragma unroll
+      for (int i = 0; i < NI; i++) {
+        const uint32_t krow = (wave * NI + i) * KPI + lane / PIECES;
+        const uint32_t piece = (lane % PIECES) ^ (((krow >> 2) & 1u) << 3);
+        goff[i] = (krow * cs + r0) * ES + piece * 16;
+      }
+      const uint32_t lrow = lane & 31, lgrp = lane >> 5;
+#pragma unroll
+      for (int q = 0; q < TILES; q++) {
+        const uint32_t n = woff + q * 32 + lrow;  // k = 4 * lgrp + e + 8 * s, e and s as immediates
+        raddr[q] = 4 * lgrp * ROWB + ((n ^ (lgrp << 5)) * 4);
+      }
     } else {
       constexpr int KPI = 512 / ROWS;       // k-rows per DMA instruction
-      constexpr int SLOTS_PER_ROW = ROWS / 8;
+      constexpr uint32_t SLOTS_PER_ROW = ROWS / 8;
       kstride = cs * 2;
 #pragma unroll
       for (int i = 0; i < NI; i++) {
         const uint32_t krow = (wave * NI + i) * KPI + lane / SLOTS_PER_ROW;
-        const uint32_t slot = (lane % SLOTS_PER_ROW) ^ swz_mn(krow);
+        const uint32_t slot = (lane % SLOTS_PER_ROW) ^ (swz_mn(krow) & (SLOTS_PER_ROW - 1));
         goff[i] = (krow * cs + r0 + slot * 8) * 2;
       }
       const uint32_t j = lane >> 4, r16 = lane & 15;
@@ -121,24 +147,27 @@ template <int ROWS, int MODE> struct DmaOperand {
 #pragma unroll
         for (int h = 0; h < 2; h++) {
           const uint32_t k = 8 * (j >> 1) + 4 * h + (r16 >> 2);  // + 16 * s as an immediate offset
-          raddr[q * 2 + h] = k * ROWB + (((m >> 3) ^ swz_mn(k)) * 16) + (m & 7) * 2;
+          raddr[q * 2 + h] = k * ROWB + (((m >> 3) ^ (swz_mn(k) & (ROWS / 8 - 1))) * 16) + (m & 7) * 2;
         }
       }
     }
   }
 
   // DMA instruction i of this wave for the K-slice starting at k0: 1 KiB into `region`.
-  __device__ __forceinline__ void dma(int i, const half_t* base, uint32_t k0, char* region) const {
+  __device__ __forceinline__ void dma(int i, const T* base, uint32_t k0, char* region) const {
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const char* src = (const char*)base + (size_t)k0 * kstride + goff[i];
     __builtin_amdgcn_global_load_lds((const GLOBAL_AS void*)src, (LDS_AS void*)(region + (wave * NI + i) * 1024), 16, 0, 0);
   }
 
-  // Read number u of sub-step s into the operand registers of tile u (DMA_K) or half u%2 of
-  // tile u/2 (DMA_MN).
+  // Read number u of sub-step s into the operand registers of tile u (DMA_K), half u%2 of
+  // tile u/2 (DMA_MN, fp16) or element u%4 of tile u/4 (DMA_MN, fp32).
   __device__ __forceinline__ void read(int u, int s, const char* region, Chunk* frag) const {
     if (MODE == DMA_K) {
       frag[u] = *reinterpret_cast<const Chunk*>(region + raddr[u * 2 + s]);
+    } else if (F32) {
+      const int q = u / 4, e = u % 4;
+      frag[q][e] = *reinterpret_cast<const uint32_t*>(region + raddr[q] + (8 * s + e) * ROWB);
     } else {
       const int q = u / 2, h = u % 2;
       typedef short short4v __attribute__((ext_vector_type(4)));
@@ -152,12 +181,14 @@ template <int ROWS, int MODE> struct DmaOperand {
   }
 };
 
-template <int BM, int BN, int MODE_A, int MODE_B>
+template <typename T, int BM, int BN, int MODE_A, int MODE_B>
 __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0, char* lds1, char* lds2, char* lds3) {
   constexpr int MT = BM / 64, NT = BN / 64;
   constexpr int SLOTS = MT * NT;
-  typedef DmaOperand<BM, MODE_A> OpA;
-  typedef DmaOperand<BN, MODE_B> OpB;
+  typedef DmaOperand<T, BM, MODE_A> OpA;
+  typedef DmaOperand<T, BN, MODE_B> OpB;
+  constexpr bool F32 = sizeof(T) == 4;
+  constexpr uint32_t BK = 64 / sizeof(T);  // K-slice of one stage
   constexpr int READS = OpA::READS + OpB::READS;
   constexpr int NDMA = OpA::NI + OpB::NI;  // per wave and K-step
   constexpr int HALF = NDMA / 2;
@@ -182,9 +213,9 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
   const uint32_t tm = tile / p.tiles_n, tn = tile - tm * p.tiles_n;
   const uint32_t m0 = tm * BM, n0 = tn * BN;
   const uint32_t batch = blockIdx.y;
-  const half_t* A = (const half_t*)p.a + batch * p.a_bs;
-  const half_t* B = (const half_t*)p.b + batch * p.b_bs;
-  half_t* C = (half_t*)p.c + batch * p.c_bs;
+  const T* A = (const T*)p.a + batch * p.a_bs;
+  const T* B = (const T*)p.b + batch * p.b_bs;
+  T* C = (T*)p.c + batch * p.c_bs;
 
   const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const uint32_t wm = (wave >> 1) * (BM / 2), wn = (wave & 1) * (BN / 2);
@@ -223,8 +254,18 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
   // n for one m (see the epilogue).
   auto mma_one = [&](const Frags& f, int t) {
     const int i = t / NT, j = t % NT;
-    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, f.b[j]),
-                                                       __builtin_bit_cast(half8, f.a[i]), acc[i][j], 0, 0, 0);
+    if constexpr (F32) {
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        // (copies first: a bit_cast applied directly to a vector element reads element 0)
+        const uint32_t wb = f.b[j][e], wa = f.a[i][e];
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(__builtin_bit_cast(float, wb),
+                                                         __builtin_bit_cast(float, wa), acc[i][j], 0, 0, 0);
+      }
+    } else {
+      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, f.b[j]),
+                                                         __builtin_bit_cast(half8, f.a[i]), acc[i][j], 0, 0, 0);
+    }
   };
   // reads per MFMA slot
   constexpr int RPS = HC_READS_PER_SLOT ? HC_READS_PER_SLOT : (READS + SLOTS - 1) / SLOTS;
@@ -232,12 +273,12 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
   constexpr int DSTRIDE = SLOTS / (NDMA - HALF) > 0 ? SLOTS / (NDMA - HALF) : 1;
   static_assert(DSTRIDE * (NDMA - HALF) <= SLOTS, "more DMA instructions than MFMA slots");
 
-  const uint32_t nk = p.K / 32;
+  const uint32_t nk = p.K / BK;
   Frags f0, f1;
 
   // K-step j out of `cur`; `nxt` holds K-step j+1, `prev` held K-step j-1.
   auto step = [&](char* cur, char* nxt, char* prev, uint32_t j) {
-    const uint32_t k3 = (j + 3 < nk ? j + 3 : nk - 1) * 32, k4 = (j + 4 < nk ? j + 4 : nk - 1) * 32;
+    const uint32_t k3 = (j + 3 < nk ? j + 3 : nk - 1) * BK, k4 = (j + 4 < nk ? j + 4 : nk - 1) * BK;
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int t = 0; t < SLOTS; t++) {  // sub-step 0
@@ -264,7 +305,7 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
 
   // prologue: K-steps 0..2 and the first half of K-step 3 (slices past the end repeat the
   // last one; nobody reads them)
-  auto kclamp = [&](uint32_t j) { return (j < nk ? j : nk - 1) * 32; };
+  auto kclamp = [&](uint32_t j) { return (j < nk ? j : nk - 1) * BK; };
 #pragma unroll
   for (int u = 0; u < NDMA; u++) dma_unit(u, 0, lds0);
 #pragma unroll
@@ -288,10 +329,9 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
     step(lds2, lds3, lds1, j + 2);
     step(lds3, lds0, lds2, j + 3);
   }
-  if (j < nk) {  // K is a multiple of 64: two K-steps left
-    step(lds0, lds1, lds3, j);
-    step(lds1, lds2, lds0, j + 1);
-  }
+  if (j < nk) step(lds0, lds1, lds3, j);
+  if (j + 1 < nk) step(lds1, lds2, lds0, j + 1);
+  if (j + 2 < nk) step(lds2, lds3, lds1, j + 2);
   wait_dma<0>();  // no LDS write of this workgroup may be in flight when it ends
 #ifdef HC_PROBE_CLOCKS
   // measurement build: the first 16 bytes of the block's C tile receive the K-loop duration
@@ -300,21 +340,46 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
 #endif
 
   // Epilogue. With the operands swapped, the MFMA tile is C^T: lane l holds m = l % 32 and,
-  // in registers 4g..4g+3, the four consecutive columns n = 8g + 4*(l/32) + (0..3).
+  // in registers 4g..4g+3, the four consecutive columns n = 8g + 4*(l/32) + (0..3). Stored
+  // directly that would be short pieces of 32 different rows per instruction, so the wave's
+  // part of C goes through LDS in slabs of 32 rows (every stage is free now; wave w uses
+  // stage w) and leaves as 16-byte pieces, whole rows of the slab contiguous. 16-byte unit u
+  // of row r sits at unit u ^ s(r) to spread the column-wise writes over the banks. A wave's
+  // LDS instructions execute in order, so a slab may be overwritten right after its reads.
+  lds_barrier();
+  char* mine = wave == 0 ? lds0 : wave == 1 ? lds1 : wave == 2 ? lds2 : lds3;
+  constexpr uint32_t ES = sizeof(T), WN = BN / 2, RB = WN * ES, UNITS = RB / 16, RPI = 64 / UNITS;
+  constexpr uint32_t SLAB = 32 * RB, NSLAB = (BM + BN) * 64 / SLAB;
+  static_assert(NSLAB >= 1 && UNITS <= 64, "a slab must fit one stage");
+  auto unit_swz = [&](uint32_t r) { return (RB >= 256 ? r : r * RB / 256) & (UNITS - 1); };
 #pragma unroll
   for (int i = 0; i < MT; i++) {
-    const uint32_t row = m0 + wm + i * 32 + lrow;
+    char* slab = mine + (i % NSLAB) * SLAB;
 #pragma unroll
     for (int j = 0; j < NT; j++) {
 #pragma unroll
       for (int g = 0; g < 4; g++) {
-        half4v h;
+        if constexpr (F32) {
+          floatx4 h;
 #pragma unroll
-        for (int e = 0; e < 4; e++) h[e] = narrow<half_t>(acc[i][j][4 * g + e]);
-        const uint32_t col = n0 + wn + j * 32 + 8 * g + 4 * lgrp;
-        *reinterpret_cast<half4v*>(C + (size_t)row * p.c_rs + col) = h;
+          for (int e = 0; e < 4; e++) h[e] = acc[i][j][4 * g + e];
+          *reinterpret_cast<floatx4*>(slab + lrow * RB + (((j * 8 + 2 * g + lgrp) ^ unit_swz(lrow)) * 16)) = h;
+        } else {
+          half4v h;
+#pragma unroll
+          for (int e = 0; e < 4; e++) h[e] = narrow<half_t>(acc[i][j][4 * g + e]);
+          *reinterpret_cast<half4v*>(slab + lrow * RB + (((j * 4 + g) ^ unit_swz(lrow)) * 16) + lgrp * 8) = h;
+        }
       }
     }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // wave-private region: no barrier needed
+#pragma unroll
+    for (uint32_t it = 0; it < 32 / RPI; it++) {
+      const uint32_t r = it * RPI + lane / UNITS, u = lane % UNITS;
+      const Chunk v = *reinterpret_cast<const Chunk*>(slab + r * RB + ((u ^ unit_swz(r)) * 16));
+      *reinterpret_cast<Chunk*>(C + (size_t)(m0 + wm + i * 32 + r) * p.c_rs + n0 + wn + u * (16 / ES)) = v;
+    }
+    asm volatile("" ::: "memory");
   }
 #ifdef HC_PROBE_CLOCKS
   __syncthreads();
@@ -326,20 +391,26 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
 #endif
 }
 
-#define DEF_DMA(BM, BN, AN, AM, BNAME, BMODE)                                                         \
-  extern "C" __global__ __launch_bounds__(256) void hc_gemm_f16_dma_##BM##x##BN##_##AN##BNAME(        \
+#define DEF_DMA(T, TN, BM, BN, AN, AM, BNAME, BMODE)                                                  \
+  extern "C" __global__ __launch_bounds__(256) void hc_gemm_##TN##_dma_##BM##x##BN##_##AN##BNAME(     \
       hck_gemm_args p) {                                                                              \
     __shared__ __attribute__((aligned(1024))) char lds0[(BM + BN) * 64];                              \
     __shared__ __attribute__((aligned(1024))) char lds1[(BM + BN) * 64];                              \
     __shared__ __attribute__((aligned(1024))) char lds2[(BM + BN) * 64];                              \
     __shared__ __attribute__((aligned(1024))) char lds3[(BM + BN) * 64];                              \
-    gemm_dma_impl<BM, BN, AM, BMODE>(p, lds0, lds1, lds2, lds3);                                      \
+    gemm_dma_impl<T, BM, BN, AM, BMODE>(p, lds0, lds1, lds2, lds3);                                   \
   }
-#define DEF_DMA_TILE(BM, BN)                                                                          \
-  DEF_DMA(BM, BN, k, DMA_K, k, DMA_K)                                                                 \
-  DEF_DMA(BM, BN, k, DMA_K, n, DMA_MN)                                                                \
-  DEF_DMA(BM, BN, m, DMA_MN, k, DMA_K)                                                                \
-  DEF_DMA(BM, BN, m, DMA_MN, n, DMA_MN)
-DEF_DMA_TILE(256, 256)
-DEF_DMA_TILE(256, 128)
-DEF_DMA_TILE(128, 128)
+#define DEF_DMA_TILE(T, TN, BM, BN)                                                                   \
+  DEF_DMA(T, TN, BM, BN, k, DMA_K, k, DMA_K)                                                          \
+  DEF_DMA(T, TN, BM, BN, k, DMA_K, n, DMA_MN)                                                         \
+  DEF_DMA(T, TN, BM, BN, m, DMA_MN, k, DMA_K)                                                         \
+  DEF_DMA(T, TN, BM, BN, m, DMA_MN, n, DMA_MN)
+#define DEF_DMA_TYPE(T, TN)                                                                           \
+  DEF_DMA_TILE(T, TN, 256, 256)                                                                       \
+  DEF_DMA_TILE(T, TN, 256, 128)                                                                       \
+  DEF_DMA_TILE(T, TN, 128, 128)                                                                       \
+  DEF_DMA_TILE(T, TN, 256, 64)                                                                        \
+  DEF_DMA_TILE(T, TN, 128, 64)                                                                        \
+  DEF_DMA_TILE(T, TN, 64, 64)
+DEF_DMA_TYPE(half_t, f16)
+DEF_DMA_TYPE(float, f32)
