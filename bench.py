@@ -256,6 +256,20 @@ def extra_workloads(backend):
             dt = (time.perf_counter() - t0) / 5
             out[name] = {"ms": round(dt * 1e3, 3), "tokens_per_s": round(2048 / dt, 1),
                          "tflops": round(100.9e9 / dt / 1e12, 2)}
+            # the same forward pass recorded once and replayed as one graph launch
+            with backend.capture() as cap:
+                logits = model(tokens)
+            for _ in range(3):
+                cap.graph.launch()
+            logits.wait()
+            t0 = time.perf_counter()
+            for _ in range(20):
+                cap.graph.launch()
+                logits.wait()
+            dt = (time.perf_counter() - t0) / 20
+            out[name + "_graph"] = {"ms": round(dt * 1e3, 3), "tokens_per_s": round(2048 / dt, 1),
+                                    "tflops": round(100.9e9 / dt / 1e12, 2)}
+            cap.graph.destroy()
     return out
 
 

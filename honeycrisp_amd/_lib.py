@@ -74,6 +74,11 @@ PROTOTYPES = {
     "hc_event_elapsed_ms": (c_int, [_P, _P, POINTER(c_float)]),
     "hc_event_destroy": (c_int, [_P]),
     "hc_launch_host_func": (c_int, [_P, HOST_FN, _P]),
+    "hc_capture_begin": (c_int, [_P]),
+    "hc_capture_end": (c_int, [_P, POINTER(c_void_p)]),
+    "hc_capture_abort": (c_int, [_P]),
+    "hc_graph_launch": (c_int, [_P, _P]),
+    "hc_graph_destroy": (c_int, [_P, _P]),
     "hc_module_load": (c_int, [_P, _P, c_size_t, POINTER(c_void_p)]),
     "hc_module_unload": (c_int, [_P, _P]),
     "hc_module_get_function": (c_int, [_P, c_char_p, POINTER(c_void_p)]),

@@ -170,6 +170,15 @@ class HIPData:
                 self.backend._ctx, host.ctypes.data_as(c_void_p), c_void_p(self.ptr), self.byteCount))
         return host
 
+    def mutateOnCPU(self, fn):
+        """`fn(host_bytes)` edits a host copy in place; the result is written back
+        (Tensor.Data.mutateOnCPU, Tensor.swift:69-85). Blocking."""
+        host = self.onCPU()
+        fn(host)
+        if self.byteCount:
+            self.backend._check(self.backend._lib.hc_memcpy_h2d(
+                self.backend._ctx, c_void_p(self.ptr), host.ctypes.data_as(c_void_p), self.byteCount))
+
     def __del__(self):
         backend, ptr = self.backend, self.ptr
         self.ptr = None
@@ -178,6 +187,45 @@ class HIPData:
 
 
 Scalar = Union[int, float, np.floating, np.integer]
+
+
+class Graph:
+    """A recorded sequence of backend ops (see HIPBackend.capture)."""
+
+    def __init__(self, backend: "HIPBackend", handle: int):
+        self.backend, self._handle = backend, handle
+
+    def launch(self):
+        self.backend._check(self.backend._lib.hc_graph_launch(self.backend._ctx, c_void_p(self._handle)))
+
+    def destroy(self):
+        if self._handle and self.backend._ctx:
+            self.backend._check(self.backend._lib.hc_graph_destroy(self.backend._ctx, c_void_p(self._handle)))
+        self._handle = None
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:
+            pass
+
+
+class Capture:
+    def __init__(self, backend: "HIPBackend"):
+        self.backend, self.graph = backend, None
+
+    def __enter__(self):
+        self.backend._check(self.backend._lib.hc_capture_begin(self.backend._ctx))
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        if exc_type is not None:
+            self.backend._lib.hc_capture_abort(self.backend._ctx)
+            return False
+        handle = c_void_p()
+        self.backend._check(self.backend._lib.hc_capture_end(self.backend._ctx, byref(handle)))
+        self.graph = Graph(self.backend, handle.value)
+        return False
 
 
 class HIPBackend(Backend):
@@ -232,6 +280,14 @@ class HIPBackend(Backend):
 
     def sync(self):
         self._check(self._lib.hc_sync(self._ctx))
+
+    def capture(self) -> "Capture":
+        """`with backend.capture() as cap: out = model(x)` records every op issued inside the
+        block instead of running it; `cap.graph.launch()` then replays the whole recording with
+        one call and `out` holds the results of the latest replay. Inputs must be on the device
+        before the block (no host transfers inside) and must stay alive while the graph is used.
+        Honeycrisp has no counterpart: it pays one backend call per op (Tensor.swift:634-657)."""
+        return Capture(self)
 
     # -- storage (DataAllocator, Backend.swift:894-896)
 

@@ -39,6 +39,14 @@ struct hc_event {
   hipEvent_t ev;
 };
 
+// A captured recording plus the buffers it owns: `parked` holds, by bucket size, blocks that
+// were freed but must stay out of the general pool while the graph exists.
+struct hc_graph {
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t exec = nullptr;
+  std::unordered_map<size_t, std::vector<void*>> parked;
+};
+
 struct hc_ctx {
   int device = 0;
   hipStream_t stream = nullptr;
@@ -49,6 +57,9 @@ struct hc_ctx {
   std::unordered_map<void*, size_t> live;
   size_t bytes_in_use = 0, bytes_cached = 0;
   hipDeviceProp_t props;
+  hc_graph* capturing = nullptr;                      // the recording in progress, if any
+  std::unordered_map<void*, hc_graph*> block_owner;   // blocks reserved for a graph
+  std::vector<hc_graph*> graphs;
 };
 
 static thread_local std::string g_last_error;
@@ -142,7 +153,20 @@ extern "C" int hc_init(int device, hc_ctx** out) {
 extern "C" void hc_shutdown(hc_ctx* ctx) {
   if (!ctx) return;
   (void)hipSetDevice(ctx->device);
+  if (ctx->capturing) {
+    hipGraph_t dropped = nullptr;
+    (void)hipStreamEndCapture(ctx->stream, &dropped);
+    if (dropped) (void)hipGraphDestroy(dropped);
+    (void)hipGetLastError();
+  }
   if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+  for (hc_graph* g : ctx->graphs) {
+    if (g->exec) (void)hipGraphExecDestroy(g->exec);
+    if (g->graph) (void)hipGraphDestroy(g->graph);
+    for (auto& kv : g->parked)
+      for (void* p : kv.second) (void)hipFree(p);
+    delete g;
+  }
   for (auto& kv : ctx->free_blocks)
     for (void* p : kv.second) (void)hipFree(p);
   for (auto& kv : ctx->live) (void)hipFree(kv.first);
@@ -195,6 +219,18 @@ extern "C" int hc_malloc(hc_ctx* ctx, size_t bytes, void** out) {
   std::lock_guard<std::mutex> lock(ctx->mu);
   auto it = ctx->free_blocks.find(b);
   void* p = nullptr;
+  if (ctx->capturing) {
+    // blocks this recording already owns come first; anything else it takes becomes its own
+    auto& parked = ctx->capturing->parked[b];
+    if (!parked.empty()) {
+      p = parked.back();
+      parked.pop_back();
+      ctx->live[p] = b;
+      ctx->bytes_in_use += b;
+      *out = p;
+      return HC_OK;
+    }
+  }
   if (it != ctx->free_blocks.end() && !it->second.empty()) {
     p = it->second.back();
     it->second.pop_back();
@@ -202,7 +238,7 @@ extern "C" int hc_malloc(hc_ctx* ctx, size_t bytes, void** out) {
   } else {
     (void)hipSetDevice(ctx->device);
     hipError_t e = hipMalloc(&p, b);
-    if (e != hipSuccess) {
+    if (e != hipSuccess && !ctx->capturing) {
       // Give cached blocks back to the driver and retry once.
       (void)hipGetLastError();
       (void)hipStreamSynchronize(ctx->stream);
@@ -216,6 +252,7 @@ extern "C" int hc_malloc(hc_ctx* ctx, size_t bytes, void** out) {
   }
   ctx->live[p] = b;
   ctx->bytes_in_use += b;
+  if (ctx->capturing) ctx->block_owner[p] = ctx->capturing;
   *out = p;
   return HC_OK;
 }
@@ -229,14 +266,25 @@ extern "C" int hc_free(hc_ctx* ctx, void* ptr) {
   const size_t b = it->second;
   ctx->live.erase(it);
   ctx->bytes_in_use -= b;
-  ctx->free_blocks[b].push_back(ptr);
-  ctx->bytes_cached += b;
+  auto owner = ctx->block_owner.find(ptr);
+  if (owner != ctx->block_owner.end()) {
+    // recorded kernels keep using this block on every replay
+    owner->second->parked[b].push_back(ptr);
+  } else if (ctx->capturing) {
+    // allocated before the capture, released inside it: the recording read (or wrote) it
+    ctx->block_owner[ptr] = ctx->capturing;
+    ctx->capturing->parked[b].push_back(ptr);
+  } else {
+    ctx->free_blocks[b].push_back(ptr);
+    ctx->bytes_cached += b;
+  }
   return HC_OK;
 }
 
 extern "C" int hc_trim(hc_ctx* ctx) {
   REQUIRE(ctx, "hc_trim: null context");
   std::lock_guard<std::mutex> lock(ctx->mu);
+  REQUIRE(!ctx->capturing, "hc_trim: not allowed while capturing");
   HIP_TRY(hipStreamSynchronize(ctx->stream));
   release_cache_locked(ctx);
   return HC_OK;
@@ -272,6 +320,8 @@ static int copy(hc_ctx* ctx, void* dst, const void* src, size_t bytes, hipMemcpy
   if (bytes == 0) return HC_OK;
   REQUIRE(dst && src, "memcpy: null pointer");
   std::lock_guard<std::mutex> lock(ctx->mu);
+  REQUIRE(!ctx->capturing || kind == hipMemcpyDeviceToDevice,
+          "memcpy: host transfers are not allowed while capturing (upload inputs before hc_capture_begin)");
   HIP_TRY(hipMemcpyAsync(dst, src, bytes, kind, ctx->stream));
   if (wait) HIP_TRY(hipStreamSynchronize(ctx->stream));
   return HC_OK;
@@ -297,6 +347,7 @@ extern "C" int hc_memcpy_d2h_async(hc_ctx* ctx, void* dst, const void* src, size
 
 extern "C" int hc_sync(hc_ctx* ctx) {
   REQUIRE(ctx, "hc_sync: null context");
+  REQUIRE(!ctx->capturing, "hc_sync: not allowed while capturing");
   HIP_TRY(hipStreamSynchronize(ctx->stream));
   return HC_OK;
 }
@@ -316,6 +367,7 @@ extern "C" int hc_event_create(hc_ctx* ctx, hc_event** out) {
 extern "C" int hc_event_record(hc_ctx* ctx, hc_event* ev) {
   REQUIRE(ctx && ev, "hc_event_record: null argument");
   std::lock_guard<std::mutex> lock(ctx->mu);
+  REQUIRE(!ctx->capturing, "hc_event_record: not allowed while capturing");
   HIP_TRY(hipEventRecord(ev->ev, ctx->stream));
   return HC_OK;
 }
@@ -354,7 +406,92 @@ extern "C" int hc_event_destroy(hc_event* ev) {
 extern "C" int hc_launch_host_func(hc_ctx* ctx, void (*fn)(void*), void* user) {
   REQUIRE(ctx && fn, "hc_launch_host_func: null argument");
   std::lock_guard<std::mutex> lock(ctx->mu);
+  REQUIRE(!ctx->capturing, "hc_launch_host_func: not allowed while capturing");
   HIP_TRY(hipLaunchHostFunc(ctx->stream, fn, user));
+  return HC_OK;
+}
+
+// ------------------------------------------------------------------ capture / graphs
+
+extern "C" int hc_capture_begin(hc_ctx* ctx) {
+  REQUIRE(ctx, "hc_capture_begin: null context");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  REQUIRE(!ctx->capturing, "hc_capture_begin: a capture is already in progress");
+  // relaxed mode: the allocator may still call hipMalloc for sizes its pool does not hold
+  HIP_TRY(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed));
+  ctx->capturing = new hc_graph();
+  ctx->graphs.push_back(ctx->capturing);
+  return HC_OK;
+}
+
+// Gives a graph's parked blocks back to the general pool and forgets its ownership of
+// blocks that are still live. Caller holds the lock.
+static void release_graph_blocks_locked(hc_ctx* ctx, hc_graph* g) {
+  for (auto& kv : g->parked)
+    for (void* p : kv.second) {
+      ctx->free_blocks[kv.first].push_back(p);
+      ctx->bytes_cached += kv.first;
+    }
+  g->parked.clear();
+  for (auto it = ctx->block_owner.begin(); it != ctx->block_owner.end();)
+    it = it->second == g ? ctx->block_owner.erase(it) : std::next(it);
+  for (size_t i = 0; i < ctx->graphs.size(); i++)
+    if (ctx->graphs[i] == g) {
+      ctx->graphs.erase(ctx->graphs.begin() + i);
+      break;
+    }
+}
+
+static int end_capture(hc_ctx* ctx, hc_graph** out) {
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  REQUIRE(ctx->capturing, "hc_capture_end: no capture in progress");
+  hc_graph* g = ctx->capturing;
+  ctx->capturing = nullptr;
+  hipError_t e = hipStreamEndCapture(ctx->stream, &g->graph);
+  if (e == hipSuccess && out) e = hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0);
+  if (e != hipSuccess || !out) {
+    (void)hipGetLastError();
+    if (g->graph) (void)hipGraphDestroy(g->graph);
+    // the recorded kernels never ran and never will: its blocks are ordinary again
+    release_graph_blocks_locked(ctx, g);
+    delete g;
+    if (e != hipSuccess) return hip_fail(e, "hipStreamEndCapture / hipGraphInstantiate");
+    return HC_OK;
+  }
+  *out = g;
+  return HC_OK;
+}
+
+extern "C" int hc_capture_end(hc_ctx* ctx, hc_graph** out) {
+  REQUIRE(ctx && out, "hc_capture_end: null argument");
+  *out = nullptr;
+  return end_capture(ctx, out);
+}
+
+extern "C" int hc_capture_abort(hc_ctx* ctx) {
+  REQUIRE(ctx, "hc_capture_abort: null context");
+  return end_capture(ctx, nullptr);
+}
+
+extern "C" int hc_graph_launch(hc_ctx* ctx, hc_graph* graph) {
+  REQUIRE(ctx && graph && graph->exec, "hc_graph_launch: null argument");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  REQUIRE(!ctx->capturing, "hc_graph_launch: not allowed while capturing");
+  HIP_TRY(hipGraphLaunch(graph->exec, ctx->stream));
+  return HC_OK;
+}
+
+extern "C" int hc_graph_destroy(hc_ctx* ctx, hc_graph* graph) {
+  REQUIRE(ctx, "hc_graph_destroy: null context");
+  if (!graph) return HC_OK;
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  REQUIRE(graph != ctx->capturing, "hc_graph_destroy: this recording is still in progress");
+  // replays already enqueued still use the parked blocks: let them finish first
+  HIP_TRY(hipStreamSynchronize(ctx->stream));
+  if (graph->exec) (void)hipGraphExecDestroy(graph->exec);
+  if (graph->graph) (void)hipGraphDestroy(graph->graph);
+  release_graph_blocks_locked(ctx, graph);
+  delete graph;
   return HC_OK;
 }
 
@@ -391,9 +528,11 @@ extern "C" int hc_module_get_function(hc_module* mod, const char* name, hc_funct
 
 static int launch_fn(hc_ctx* ctx, hipFunction_t fn, uint32_t gx, uint32_t gy, uint32_t gz, uint32_t bx,
                      uint32_t shared, const void* kernarg, size_t kernarg_bytes) {
-  void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, const_cast<void*>(kernarg),
-                    HIP_LAUNCH_PARAM_BUFFER_SIZE, &kernarg_bytes, HIP_LAUNCH_PARAM_END};
-  HIP_TRY(hipModuleLaunchKernel(fn, gx, gy, gz, bx, 1, 1, shared, ctx->stream, nullptr, config));
+  // every built-in kernel takes one struct by value: pass it as the single kernel parameter,
+  // which the runtime copies at enqueue (and into a graph node while capturing)
+  (void)kernarg_bytes;
+  void* params[] = {const_cast<void*>(kernarg)};
+  HIP_TRY(hipModuleLaunchKernel(fn, gx, gy, gz, bx, 1, 1, shared, ctx->stream, params, nullptr));
   return HC_OK;
 }
 

@@ -98,6 +98,7 @@ class Transformer:
                  dtype=DType.float32):
         rng = np.random.default_rng(seed)
         self.dtype, self.seq, self.d_model = dtype, seq, d_model
+        self._masks = {}
         self.table = Tensor(data=(rng.standard_normal((vocab, d_model)) * 0.02).astype(np.float32), dtype=dtype)
         self.pos = Tensor(data=(rng.standard_normal((seq, d_model)) * 0.02).astype(np.float32), dtype=dtype)
         self.blocks = [Block(d_model, heads, mlp, rng, dtype) for _ in range(layers)]
@@ -106,9 +107,12 @@ class Transformer:
         self.unembed = Linear(d_model, vocab, rng, dtype=dtype, castParams=cp)
 
     def causal_mask(self, T: int) -> Tensor:
-        pos = Tensor(data=range(T))
-        # finite in fp16; (pos[:, None] >= pos) is true on and below the diagonal
-        return (pos[..., NewAxis()] >= pos).when(0, -1e4, dtype=self.dtype)
+        # depends on T only: built once per length (also keeps host uploads out of the forward pass)
+        if T not in self._masks:
+            pos = Tensor(data=range(T))
+            # finite in fp16; (pos[:, None] >= pos) is true on and below the diagonal
+            self._masks[T] = (pos[..., NewAxis()] >= pos).when(0, -1e4, dtype=self.dtype)
+        return self._masks[T]
 
     def __call__(self, ids: Tensor) -> Tensor:
         B, T = ids.shape

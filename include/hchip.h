@@ -134,6 +134,27 @@ int hc_event_destroy(hc_event* ev);
  * continuation resumes from (precedent BackendMPS.swift:2663-2720). */
 int hc_launch_host_func(hc_ctx* ctx, void (*fn)(void*), void* user);
 
+/* ---- stream capture and graph replay ----
+ * No counterpart in the reference, which issues one backend call per op (one Task per op,
+ * Tensor.swift:634-657): a model whose forward pass is a few hundred small ops is bound by
+ * that per-op host cost. Between hc_capture_begin and hc_capture_end every op entry point
+ * records its kernels into a graph instead of running them; hc_graph_launch replays the
+ * whole recording with one call, in stream order with everything else.
+ *  - Buffers obtained from hc_malloc during the capture stay reserved for the graph (also
+ *    after hc_free) until hc_graph_destroy, so a replay never writes into memory that was
+ *    handed to somebody else. Buffers allocated before the capture and read by it must be
+ *    kept alive by the caller for as long as the graph is replayed; results are read from
+ *    the buffers the captured ops returned.
+ *  - Host transfers, hc_sync, event and host-function calls are refused while capturing
+ *    (HC_ERR_INVALID). One capture at a time per context. */
+typedef struct hc_graph hc_graph;
+int hc_capture_begin(hc_ctx* ctx);
+int hc_capture_end(hc_ctx* ctx, hc_graph** out);
+/* Ends a capture and throws the recording away (error paths). */
+int hc_capture_abort(hc_ctx* ctx);
+int hc_graph_launch(hc_ctx* ctx, hc_graph* graph);
+int hc_graph_destroy(hc_ctx* ctx, hc_graph* graph);
+
 /* ---- raw module API (thin wrappers over hipModuleLoadData / hipModuleGetFunction /
  * hipModuleLaunchKernel) for callers that bring their own gfx950 code objects ---- */
 
