@@ -97,6 +97,11 @@ PROTOTYPES = {
     "hc_log_softmax": (c_int, [_P, c_int, _P, _P, c_int64, c_int64, c_int64]),
     "hc_normalize": (c_int, [_P, c_int, _P, _P, c_int64, c_int64, c_int64, c_float]),
     "hc_gather": (c_int, [_P, c_int, _P, _P, _S, _P, c_int64, c_int64, c_int64, c_int64]),
+    "hc_scatter": (c_int, [_P, c_int, _P, _P, _S, _P, c_int64, c_int64, c_int64, c_int64, c_int]),
+    "hc_log_softmax_grad": (c_int, [_P, c_int, _P, _P, _P, c_int64, c_int64, c_int64]),
+    "hc_clamp": (c_int, [_P, c_int, _P, _S, _P, _S, _P, _S, _P]),
+    "hc_adamw": (c_int, [_P, c_int, _P, _P, _P, _P, c_float, c_float, c_float, c_float, c_float, c_float,
+                         c_size_t, _P, _P, _P]),
     "hc_when": (c_int, [_P, c_int, _P, _S, _P, _S, _P, _S, _P]),
     "hc_matmul": (c_int, [_P, c_int, c_int64, _P, c_int, _P, c_int, c_int, c_int64, c_int64, c_int64, _P]),
     "hc_triangular": (c_int, [_P, c_int, _P, _P, c_int64, c_int64, c_int64, c_int, c_int64]),

@@ -96,6 +96,15 @@ class Backend:
     def gather(self, a, s, dtype):
         self._ni("gather")
 
+    def scatter(self, a, s, dtype):
+        self._ni("scatter")
+
+    def logSoftmaxGrad(self, a, outGrad, dims, dtype):
+        self._ni("logSoftmaxGrad")
+
+    def clamp(self, a, min, max, dtype):
+        self._ni("clamp")
+
     def when(self, mask, a, b, dtype):
         self._ni("when")
 
@@ -149,6 +158,64 @@ class Backend:
             -0.5, 1.0, None, reduced.dataCount, dtype)
         return self.binaryOp(BroadcastData(full, centered), BroadcastData(reduced, normalizer),
                              NumericBinaryOp.mul, dtype)
+
+
+    def normalizeGrad(self, input, outGrad, dims: ReduceDims, eps, dtype):
+        """Backend.swift:332-455, op by op."""
+        f32 = np.float32
+        full = BroadcastStrides.contiguousForShape([dims.outerCount, dims.reduceCount, dims.innerCount])
+        reduced = BroadcastStrides(full.shape, [dims.innerCount, 0, 1])
+        inv_n = f32(1.0) / f32(dims.reduceCount)
+        n_red = reduced.dataCount
+        bd_full = lambda d: BroadcastData(full, d)
+        bd_red = lambda d: BroadcastData(reduced, d)
+        mean = self.binaryOp(self.reduce(input, ReduceOp.sum, dims, dtype), inv_n, NumericBinaryOp.mul,
+                             dtype, count=n_red)
+        centered = self.binaryOp(bd_full(input), bd_red(mean), NumericBinaryOp.sub, dtype)
+        variance = self.binaryOp(
+            self.reduce(self.pow(centered, 2.0, 1.0, None, full.dataCount, dtype), ReduceOp.sum, dims, dtype),
+            inv_n, NumericBinaryOp.mul, dtype, count=n_red)
+        stable = self.binaryOp(variance, eps, NumericBinaryOp.add, dtype, count=n_red)
+        normalizer1 = self.pow(stable, -0.5, 1.0, None, n_red, dtype)
+        normalizer2 = self.pow(stable, -1.5, f32(1) / f32(dims.reduceCount), None, n_red, dtype)
+        meanGrad = self.binaryOp(self.reduce(outGrad, ReduceOp.sum, dims, dtype), f32(1) / f32(dims.reduceCount),
+                                 NumericBinaryOp.mul, dtype, count=n_red)
+        centeredGrad = self.binaryOp(bd_full(outGrad), bd_red(meanGrad), NumericBinaryOp.sub, dtype)
+        covTerm = self.reduce(self.binaryOp(bd_full(centered), bd_full(outGrad), NumericBinaryOp.mul, dtype),
+                              ReduceOp.sum, dims, dtype)
+        term1 = self.binaryOp(bd_full(centeredGrad), bd_red(normalizer1), NumericBinaryOp.mul, dtype)
+        covTimesCentered = self.binaryOp(bd_full(centered), bd_red(covTerm), NumericBinaryOp.mul, dtype)
+        term2 = self.binaryOp(bd_full(covTimesCentered), bd_red(normalizer2), NumericBinaryOp.mul, dtype)
+        return self.binaryOp(bd_full(term1), bd_full(term2), NumericBinaryOp.sub, dtype)
+
+    def adamW(self, param, grad, moment1, moment2, beta1, beta2, eps, weightDecay, lr, step, count, dtype):
+        """Backend.swift:818-892, op by op; returns (param, moment1, moment2). All scalar
+        arithmetic is in Float as there."""
+        f32 = np.float32
+        beta1, beta2, eps, weightDecay, lr, step = (f32(v) for v in (beta1, beta2, eps, weightDecay, lr, step))
+        bd = lambda d: BroadcastData(BroadcastStrides.contiguousForShape([count]), d)
+        mul, add, sub, div = NumericBinaryOp.mul, NumericBinaryOp.add, NumericBinaryOp.sub, NumericBinaryOp.div
+        newMt = self.binaryOp(bd(self.binaryOp(beta1, moment1, mul, dtype, count=count)),
+                              bd(self.binaryOp(f32(1) - beta1, grad, mul, dtype, count=count)), add, dtype)
+        gradSq = self.pow(grad, 2.0, f32(1) - beta2, None, count, dtype)
+        newVt = self.binaryOp(bd(self.binaryOp(beta2, moment2, mul, dtype, count=count)), bd(gradSq), add, dtype)
+        scaledMt = self.binaryOp(newMt, f32(1.0) / (f32(1) - powf(beta1, step)), mul, dtype, count=count)
+        scaledVt = self.binaryOp(newVt, f32(1.0) / (f32(1) - powf(beta2, step)), mul, dtype, count=count)
+        denom = self.binaryOp(self.pow(scaledVt, 0.5, 1.0, None, count, dtype), eps, add, dtype, count=count)
+        stepDir = self.binaryOp(self.binaryOp(bd(scaledMt), bd(denom), div, dtype), lr, mul, dtype, count=count)
+        decayed = self.binaryOp(param, f32(1) - lr * weightDecay, mul, dtype, count=count)
+        newParam = self.binaryOp(bd(decayed), bd(stepDir), sub, dtype)
+        return newParam, newMt, newVt
+
+
+_libm = ctypes.CDLL("libm.so.6")
+_libm.powf.restype = ctypes.c_float
+_libm.powf.argtypes = [ctypes.c_float, ctypes.c_float]
+
+
+def powf(x, y) -> np.float32:
+    """C powf (Foundation.pow on Float)."""
+    return np.float32(_libm.powf(float(x), float(y)))
 
 
 class HIPData:
@@ -470,6 +537,53 @@ class HIPBackend(Backend):
                                         c_void_p(out.ptr), s.outerCount, s.middleCount, s.outCount,
                                         s.innerCount))
         return out
+
+    def scatter(self, a, s: ScatterGatherIndices, dtype: DType) -> HIPData:
+        out = self.allocate(s.gatherInCount * dtype.byteSize)
+        ad, idx = self._dev(a), self._dev(s.indices.data)
+        st = self._s(s.indices.strides)
+        self._check(self._lib.hc_scatter(self._ctx, int(dtype), c_void_p(ad.ptr), c_void_p(idx.ptr), byref(st),
+                                         c_void_p(out.ptr), s.outerCount, s.middleCount, s.outCount,
+                                         s.innerCount, int(bool(s.indicesAreUnique))))
+        return out
+
+    def logSoftmaxGrad(self, a, outGrad, dims: ReduceDims, dtype: DType) -> HIPData:
+        out = self.allocate(dims.inCount * dtype.byteSize)
+        ad, gd = self._dev(a), self._dev(outGrad)
+        self._check(self._lib.hc_log_softmax_grad(self._ctx, int(dtype), c_void_p(ad.ptr), c_void_p(gd.ptr),
+                                                  c_void_p(out.ptr), dims.outerCount, dims.reduceCount,
+                                                  dims.innerCount))
+        return out
+
+    def clamp(self, a: BroadcastData, min, max, dtype: DType) -> HIPData:
+        """min / max: None, BroadcastData, or ("scalar", value, shape) (Backend.TensorOrScalar)."""
+        if min is None and max is None:
+            raise ValueError("cannot use clamp() without bounds")
+        def bound(x):
+            if x is None or isinstance(x, BroadcastData):
+                return x
+            _, value, shape = x
+            return BroadcastData(BroadcastStrides(shape, [0] * len(shape)), self.constant(value, 1, dtype))
+        lo, hi = bound(min), bound(max)
+        out = self.allocate(product(a.strides.shape) * dtype.byteSize)
+        ad, sa = self._dev(a.data), self._s(a.strides)
+        lod, hid = (self._dev(lo.data) if lo else None), (self._dev(hi.data) if hi else None)
+        sl, sh = (self._s(lo.strides) if lo else None), (self._s(hi.strides) if hi else None)
+        self._check(self._lib.hc_clamp(
+            self._ctx, int(dtype), c_void_p(ad.ptr), byref(sa),
+            c_void_p(lod.ptr) if lo else None, byref(sl) if lo else None,
+            c_void_p(hid.ptr) if hi else None, byref(sh) if hi else None, c_void_p(out.ptr)))
+        return out
+
+    def adamW(self, param, grad, moment1, moment2, beta1, beta2, eps, weightDecay, lr, step, count,
+              dtype: DType):
+        """One fused kernel, bit-identical to the base-class composition (Backend.adamW)."""
+        outs = [self.allocate(count * dtype.byteSize) for _ in range(3)]
+        ins = [self._dev(x) for x in (param, grad, moment1, moment2)]
+        self._check(self._lib.hc_adamw(
+            self._ctx, int(dtype), *[c_void_p(x.ptr) for x in ins], c_float(beta1), c_float(beta2), c_float(eps),
+            c_float(weightDecay), c_float(lr), c_float(step), c_size_t(count), *[c_void_p(o.ptr) for o in outs]))
+        return tuple(outs)
 
     def matmul(self, a, transA: bool, b, transB: bool, transOut: bool, rows: int, inner: int, cols: int,
                dtype: DType) -> HIPData:

@@ -12,6 +12,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <cmath>
 #include <mutex>
 #include <string>
 #include <unordered_map>
@@ -811,6 +812,18 @@ extern "C" int hc_when(hc_ctx* ctx, int dtype, const void* mask, const hc_stride
   return fused3(ctx, "hc_when", dtype, mask, ms, a, as, b, bs, out, el, tname);
 }
 
+extern "C" int hc_clamp(hc_ctx* ctx, int dtype, const void* a, const hc_strides* as, const void* lo,
+                        const hc_strides* ls, const void* hi, const hc_strides* hs, void* out) {
+  REQUIRE(ctx && a && as && out, "hc_clamp: null argument");
+  REQUIRE((lo && ls) || (hi && hs), "hc_clamp: cannot clamp without bounds");
+  if (dtype != HC_F32 && dtype != HC_F16 && dtype != HC_I64)
+    return fail(HC_ERR_UNSUPPORTED, "hc_clamp: dtype %d is not numeric", dtype);
+  const char* kernel = lo && hi ? "hc_clamp_both" : lo ? "hc_clamp_min" : "hc_clamp_max";
+  // an absent bound aliases the input (the kernel does not look at it)
+  return fused3(ctx, kernel, dtype, a, as, lo ? lo : a, lo ? ls : as, hi ? hi : a, hi ? hs : as, out,
+                dtype_size(dtype), dtype_name(dtype));
+}
+
 static int launch_contiguous(hc_ctx* ctx, const char* name, size_t count, int vec, const void* args,
                              size_t bytes) {
   if (count == 0) return HC_OK;
@@ -1074,6 +1087,31 @@ extern "C" int hc_log_softmax(hc_ctx* ctx, int dtype, const void* in, void* out,
   return launch(ctx, name, ceil_div((uint64_t)inner, HCK_BLOCK) * (uint64_t)outer, 1, &k, sizeof(k));
 }
 
+extern "C" int hc_log_softmax_grad(hc_ctx* ctx, int dtype, const void* in, const void* out_grad, void* out,
+                                   int64_t outer, int64_t reduce, int64_t inner) {
+  REQUIRE(ctx, "hc_log_softmax_grad: null context");
+  if (dtype != HC_F32 && dtype != HC_F16)
+    return fail(HC_ERR_UNSUPPORTED, "hc_log_softmax_grad: dtype %d is not a float type", dtype);
+  HC_TRY(check_dims("hc_log_softmax_grad", outer, reduce, inner));
+  if (outer * reduce * inner == 0) return HC_OK;
+  REQUIRE(in && out_grad && out, "hc_log_softmax_grad: null pointer");
+  hck_reduce_args k;
+  memset(&k, 0, sizeof(k));
+  k.in = in;
+  k.in2 = out_grad;
+  k.out = out;
+  k.outer = (uint32_t)outer;
+  k.reduce = (uint32_t)reduce;
+  k.inner = (uint32_t)inner;
+  char name[64];
+  if (inner == 1) {
+    snprintf(name, sizeof(name), "hc_log_softmax_grad_rows_%s", dtype_name(dtype));
+    return launch(ctx, name, ceil_div((uint64_t)outer, HCK_BLOCK / 64), 1, &k, sizeof(k));
+  }
+  snprintf(name, sizeof(name), "hc_log_softmax_grad_cols_%s", dtype_name(dtype));
+  return launch(ctx, name, ceil_div((uint64_t)inner, HCK_BLOCK) * (uint64_t)outer, 1, &k, sizeof(k));
+}
+
 struct Scratch {
   hc_ctx* ctx;
   std::vector<void*> ptrs;
@@ -1222,6 +1260,96 @@ extern "C" int hc_gather(hc_ctx* ctx, int dtype, const void* in, const void* ind
   char name[64];
   snprintf(name, sizeof(name), "hc_gather_elems_b%zu", el);
   return launch(ctx, name, ceil_div(total, HCK_BLOCK), 1, &k, sizeof(k));
+}
+
+extern "C" int hc_scatter(hc_ctx* ctx, int dtype, const void* in, const void* indices,
+                          const hc_strides* idx_strides, void* out, int64_t outer, int64_t middle,
+                          int64_t out_count, int64_t inner, int indices_are_unique) {
+  REQUIRE(ctx && idx_strides, "hc_scatter: null argument");
+  if (dtype != HC_F32 && dtype != HC_F16 && dtype != HC_I64)
+    return fail(HC_ERR_UNSUPPORTED, "hc_scatter: dtype %d is not numeric", dtype);
+  REQUIRE(outer >= 0 && middle >= 0 && out_count >= 0 && inner >= 0, "hc_scatter: negative dimension");
+  const double in_total = (double)outer * (double)out_count * (double)inner;
+  const double out_total = (double)outer * (double)middle * (double)inner;
+  if (out_total == 0) return HC_OK;
+  if (out_total > 4294967295.0 || in_total > 4294967295.0)
+    return fail(HC_ERR_TOO_LARGE, "hc_scatter: more than 2^32-1 elements");
+  REQUIRE(out, "hc_scatter: null pointer");
+  const size_t n_out = (size_t)outer * (size_t)middle * (size_t)inner;
+  const uint64_t total = (uint64_t)outer * (uint64_t)out_count * (uint64_t)inner;
+  // half values with repeated indices add up in a float buffer that is rounded once at the end
+  const bool staged = dtype == HC_F16 && !indices_are_unique;
+  Scratch scratch(ctx);
+  void* acc = out;
+  if (staged) HC_TRY(scratch.get(n_out * 4, &acc));
+  HC_TRY(hc_fill(ctx, staged ? HC_F32 : dtype, 0.0f, 0, acc, n_out));
+  if (total != 0) {
+    REQUIRE(in && indices, "hc_scatter: null pointer");
+    uint64_t n = 1;
+    REQUIRE(idx_strides->ndim <= HC_MAX_DIMS, "hc_scatter: ndim %u exceeds %d", idx_strides->ndim, HC_MAX_DIMS);
+    for (uint32_t k = 0; k < idx_strides->ndim; k++) n *= (uint64_t)idx_strides->shape[k];
+    REQUIRE(n == total, "hc_scatter: index shape has %llu elements, expected %llu", (unsigned long long)n,
+            (unsigned long long)total);
+    hck_gather_elems_args k;
+    memset(&k, 0, sizeof(k));
+    k.in = in;
+    k.indices = (const int64_t*)indices;
+    k.out = acc;
+    k.out_count = (uint32_t)out_count;
+    k.middle = (uint32_t)middle;
+    k.inner = (uint32_t)inner;
+    k.total = (uint32_t)total;
+    int vec;
+    const hc_strides* ops[] = {idx_strides};
+    const void* ptrs[] = {indices};
+    HC_TRY(make_bcast(1, ops, ptrs, acc, 1, &k.idx, &vec, &n));
+    char name[64];
+    if (indices_are_unique) snprintf(name, sizeof(name), "hc_scatter_set_b%zu", dtype_size(dtype));
+    else snprintf(name, sizeof(name), "hc_scatter_add_%s", dtype_name(dtype));
+    HC_TRY(launch(ctx, name, ceil_div(total, HCK_BLOCK), 1, &k, sizeof(k)));
+  }
+  if (staged) HC_TRY(hc_cast(ctx, acc, HC_F32, out, HC_F16, n_out));
+  return HC_OK;
+}
+
+extern "C" int hc_adamw(hc_ctx* ctx, int dtype, const void* param, const void* grad, const void* moment1,
+                        const void* moment2, float beta1, float beta2, float eps, float weight_decay,
+                        float lr, float step, size_t count, void* out_param, void* out_moment1,
+                        void* out_moment2) {
+  REQUIRE(ctx, "hc_adamw: null context");
+  if (dtype != HC_F32 && dtype != HC_F16)
+    return fail(HC_ERR_UNSUPPORTED, "hc_adamw: dtype %d is not a float type", dtype);
+  if (count == 0) return HC_OK;
+  REQUIRE(param && grad && moment1 && moment2 && out_param && out_moment1 && out_moment2,
+          "hc_adamw: null pointer");
+  hck_adamw_args k;
+  memset(&k, 0, sizeof(k));
+  k.param = param;
+  k.grad = grad;
+  k.m1 = moment1;
+  k.m2 = moment2;
+  k.out_param = out_param;
+  k.out_m1 = out_moment1;
+  k.out_m2 = out_moment2;
+  k.count = count;
+  // the scalars of Backend.swift:818-892, all formed in Float
+  k.beta1 = beta1;
+  k.one_minus_beta1 = 1.0f - beta1;
+  k.beta2 = beta2;
+  k.one_minus_beta2 = 1.0f - beta2;
+  k.bias1 = 1.0f / (1.0f - powf(beta1, step));
+  k.bias2 = 1.0f / (1.0f - powf(beta2, step));
+  k.eps = eps;
+  k.lr = lr;
+  k.decay = 1.0f - lr * weight_decay;
+  k.exp_square = 2.0f;
+  k.exp_root = 0.5f;
+  char name[64];
+  snprintf(name, sizeof(name), "hc_adamw_%s", dtype_name(dtype));
+  uint64_t blocks = ceil_div(count, HCK_BLOCK);
+  const uint64_t cap = (uint64_t)ctx->props.multiProcessorCount * 32;
+  if (blocks > cap) blocks = cap;
+  return launch(ctx, name, blocks, 1, &k, sizeof(k));
 }
 
 extern "C" int hc_axis_permutation(hc_ctx* ctx, const int64_t* perm, const int64_t* shape, int ndim,

@@ -75,7 +75,26 @@ typedef struct {
   uint32_t reduce;
   uint32_t inner;
   float eps;
+  const void* in2; /* logSoftmaxGrad: the output gradient */
 } hck_reduce_args;
+
+/* Fused AdamW step over `count` contiguous elements; the scalars are the ones the op-by-op
+ * composition would pass to its tensor-scalar ops. */
+typedef struct {
+  const void* param;
+  const void* grad;
+  const void* m1;
+  const void* m2;
+  void* out_param;
+  void* out_m1;
+  void* out_m2;
+  uint64_t count;
+  float beta1, one_minus_beta1, beta2, one_minus_beta2;
+  float bias1, bias2; /* 1 / (1 - beta^step) */
+  float eps, lr, decay; /* decay = 1 - lr * weightDecay */
+  float exp_square, exp_root; /* 2 and 0.5, passed at run time so that powf is called exactly
+                                 as in the pow kernels (no folding into x*x or sqrt) */
+} hck_adamw_args;
 
 /* Row gather: every output row of row_vecs 16-byte (or narrower) vectors comes from
  * one source row chosen by an index that only depends on the row. */

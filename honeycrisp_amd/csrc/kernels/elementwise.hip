@@ -131,6 +131,36 @@ template <typename T, int VEC> __device__ __forceinline__ void when_impl(const h
   store_vec<T, VEC>((T*)p.out, o, r);
 }
 
+// clamp (BackendCPU.swift:704-782): Swift.min(hi, Swift.max(lo, x)) on Float / Int64, where
+// max(a, b) = b >= a ? b : a and min(a, b) = b < a ? b : a. MODE 0 both bounds, 1 lower
+// only, 2 upper only (the unused operand aliases x).
+template <typename T, int MODE, int VEC> __device__ __forceinline__ void clamp_impl(const hck_ternary_args& p) {
+  typedef typename Arith<T>::type C;
+  uint32_t v = blockIdx.x * HCK_BLOCK + threadIdx.x;
+  if (v >= p.d.total_vecs) return;
+  uint32_t off[3];
+  size_t o;
+  bcast_offsets<3, VEC>(p.d, v, off, o);
+  T x[VEC], lo[VEC], hi[VEC], r[VEC];
+  load_vec<T, VEC>((const T*)p.x, off[0], p.d.inner_stride[0], x);
+  load_vec<T, VEC>((const T*)p.y, off[1], p.d.inner_stride[1], lo);
+  load_vec<T, VEC>((const T*)p.z, off[2], p.d.inner_stride[2], hi);
+#pragma unroll
+  for (int i = 0; i < VEC; i++) {
+    C val = to_arith(x[i]);
+    if (MODE != 2) {
+      const C l = to_arith(lo[i]);
+      val = val >= l ? val : l;
+    }
+    if (MODE != 1) {
+      const C h = to_arith(hi[i]);
+      val = val < h ? val : h;
+    }
+    r[i] = from_arith<T>(val);
+  }
+  store_vec<T, VEC>((T*)p.out, o, r);
+}
+
 #define DEF_BINARY_OPS(TN, T, V)                                                                      \
   HC_KERNEL void hc_binary_add_##TN##_v##V(hck_binary_args p) { binary_impl<T, OP_ADD, V>(p); }      \
   HC_KERNEL void hc_binary_mul_##TN##_v##V(hck_binary_args p) { binary_impl<T, OP_MUL, V>(p); }      \
@@ -144,7 +174,10 @@ template <typename T, int VEC> __device__ __forceinline__ void when_impl(const h
   HC_KERNEL void hc_compare_gt_##TN##_v##V(hck_binary_args p) { compare_impl<T, CMP_GT, V>(p); }     \
   HC_KERNEL void hc_compare_ge_##TN##_v##V(hck_binary_args p) { compare_impl<T, CMP_GE, V>(p); }     \
   HC_KERNEL void hc_mul_add_##TN##_v##V(hck_ternary_args p) { fused3_impl<T, 1, V>(p); }             \
-  HC_KERNEL void hc_add_mul_##TN##_v##V(hck_ternary_args p) { fused3_impl<T, 0, V>(p); }
+  HC_KERNEL void hc_add_mul_##TN##_v##V(hck_ternary_args p) { fused3_impl<T, 0, V>(p); }             \
+  HC_KERNEL void hc_clamp_both_##TN##_v##V(hck_ternary_args p) { clamp_impl<T, 0, V>(p); }           \
+  HC_KERNEL void hc_clamp_min_##TN##_v##V(hck_ternary_args p) { clamp_impl<T, 1, V>(p); }            \
+  HC_KERNEL void hc_clamp_max_##TN##_v##V(hck_ternary_args p) { clamp_impl<T, 2, V>(p); }
 
 DEF_BINARY_OPS(f32, float, 1)
 DEF_BINARY_OPS(f32, float, 4)
@@ -461,6 +494,45 @@ HC_KERNEL void hc_pow_generic_i64(hck_map_args p) {
     return scale * (scales ? scales[i] : (int64_t)1) * pw;
   });
 }
+
+// ---------------------------------------------------------------- adamW
+
+// One AdamW step (Backend.swift:818-892), the base class's op-by-op composition in one pass:
+// every intermediate is rounded to the tensor dtype where the composition would have stored
+// a tensor, squares and roots take the same paths as the pow kernels above (fp32: x*x then
+// *scale unless scale == 1; fp16 and every root: scale * 1 * powf), and the file is built
+// without FMA contraction, so the results equal the composed ones bit for bit.
+template <typename T> __device__ __forceinline__ void adamw_impl(const hck_adamw_args& p) {
+  const uint64_t stride = (uint64_t)gridDim.x * HCK_BLOCK;
+  for (uint64_t i = (uint64_t)blockIdx.x * HCK_BLOCK + threadIdx.x; i < p.count; i += stride) {
+    const float param = (float)((const T*)p.param)[i], g = (float)((const T*)p.grad)[i];
+    const float m = (float)((const T*)p.m1)[i], v = (float)((const T*)p.m2)[i];
+    const float m_scaled = round_through<T>(p.beta1 * m);
+    const float g_scaled = round_through<T>(p.one_minus_beta1 * g);
+    const float new_m = round_through<T>(m_scaled + g_scaled);
+    float g_sq;
+    if (sizeof(T) == 4) {
+      g_sq = g * g;
+      if (p.one_minus_beta2 != 1.0f) g_sq = g_sq * p.one_minus_beta2;
+    } else {
+      g_sq = round_through<T>(p.one_minus_beta2 * 1.0f * powf(g, p.exp_square));
+    }
+    const float v_scaled = round_through<T>(p.beta2 * v);
+    const float new_v = round_through<T>(v_scaled + g_sq);
+    const float m_hat = round_through<T>(new_m * p.bias1);
+    const float v_hat = round_through<T>(new_v * p.bias2);
+    const float root = round_through<T>(1.0f * 1.0f * powf(v_hat, p.exp_root));
+    const float denom = round_through<T>(root + p.eps);
+    const float ratio = round_through<T>(m_hat / denom);
+    const float step_dir = round_through<T>(ratio * p.lr);
+    const float decayed = round_through<T>(param * p.decay);
+    ((T*)p.out_param)[i] = narrow<T>(decayed - step_dir);
+    ((T*)p.out_m1)[i] = narrow<T>(new_m);
+    ((T*)p.out_m2)[i] = narrow<T>(new_v);
+  }
+}
+HC_KERNEL void hc_adamw_f32(hck_adamw_args p) { adamw_impl<float>(p); }
+HC_KERNEL void hc_adamw_f16(hck_adamw_args p) { adamw_impl<half_t>(p); }
 
 // ---------------------------------------------------------------- cast / fill
 

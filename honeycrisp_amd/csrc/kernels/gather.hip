@@ -50,6 +50,47 @@ HC_KERNEL void hc_gather_elems_b4(hck_gather_elems_args p) { gather_elems_impl<u
 HC_KERNEL void hc_gather_elems_b2(hck_gather_elems_args p) { gather_elems_impl<uint16_t>(p); }
 HC_KERNEL void hc_gather_elems_b1(hck_gather_elems_args p) { gather_elems_impl<uint8_t>(p); }
 
+// scatter (BackendCPU.swift:1149-1188): one lane per input element; values that share an
+// index add up. The output is zeroed by the caller. Float sums are formed with hardware
+// atomics, i.e. in no fixed order (the CPU adds in (i, j, k) order); half inputs accumulate
+// into a float buffer that the caller rounds once afterwards, as the CPU does.
+template <typename TI, typename TO> __device__ __forceinline__ void scatter_add_impl(const hck_gather_elems_args& p) {
+  const uint32_t o = blockIdx.x * HCK_BLOCK + threadIdx.x;
+  if (o >= p.total) return;
+  uint32_t off[1];
+  size_t unused;
+  bcast_offsets<1, 1>(p.idx, o, off, unused);
+  const int64_t idx = p.indices[off[0]];
+  const uint32_t ij = o / p.inner;
+  const uint32_t k = o - ij * p.inner;
+  const uint32_t i = ij / p.out_count;
+  TO* dst = (TO*)p.out + ((int64_t)i * p.middle + idx) * (int64_t)p.inner + k;
+  const TO v = (TO)((const TI*)p.in)[o];
+  __hip_atomic_fetch_add(dst, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+HC_KERNEL void hc_scatter_add_f32(hck_gather_elems_args p) { scatter_add_impl<float, float>(p); }
+HC_KERNEL void hc_scatter_add_f16(hck_gather_elems_args p) { scatter_add_impl<half_t, float>(p); }
+HC_KERNEL void hc_scatter_add_i64(hck_gather_elems_args p) {
+  scatter_add_impl<unsigned long long, unsigned long long>(p);
+}
+
+// scatter with indices the caller declares unique: plain stores, any element size.
+template <typename V> __device__ __forceinline__ void scatter_set_impl(const hck_gather_elems_args& p) {
+  const uint32_t o = blockIdx.x * HCK_BLOCK + threadIdx.x;
+  if (o >= p.total) return;
+  uint32_t off[1];
+  size_t unused;
+  bcast_offsets<1, 1>(p.idx, o, off, unused);
+  const int64_t idx = p.indices[off[0]];
+  const uint32_t ij = o / p.inner;
+  const uint32_t k = o - ij * p.inner;
+  const uint32_t i = ij / p.out_count;
+  ((V*)p.out)[((int64_t)i * p.middle + idx) * (int64_t)p.inner + k] = ((const V*)p.in)[o];
+}
+HC_KERNEL void hc_scatter_set_b8(hck_gather_elems_args p) { scatter_set_impl<uint64_t>(p); }
+HC_KERNEL void hc_scatter_set_b4(hck_gather_elems_args p) { scatter_set_impl<uint32_t>(p); }
+HC_KERNEL void hc_scatter_set_b2(hck_gather_elems_args p) { scatter_set_impl<uint16_t>(p); }
+
 // axisPermutation (BackendCPU.swift:1831-1849): flat source index of every element of the
 // permuted view.
 HC_KERNEL void hc_axis_permutation(hck_axis_perm_args p) {

@@ -257,6 +257,58 @@ HC_KERNEL void hc_log_softmax_rows_f16(hck_reduce_args p) { log_softmax_rows_imp
 HC_KERNEL void hc_log_softmax_cols_f32(hck_reduce_args p) { log_softmax_cols_impl<float>(p); }
 HC_KERNEL void hc_log_softmax_cols_f16(hck_reduce_args p) { log_softmax_cols_impl<half_t>(p); }
 
+// logSoftmaxGrad (BackendCPU.swift:1040-1085): g - sum(g) * expf(x - (logf(sum exp(x - max)) + max)).
+template <typename T> __device__ __forceinline__ void log_softmax_grad_rows_impl(const hck_reduce_args& p) {
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t row = blockIdx.x * (HCK_BLOCK / 64) + (threadIdx.x >> 6);
+  if (row >= p.outer) return;
+  const uint32_t n = p.reduce;
+  const T* in = (const T*)p.in + (size_t)row * n;
+  const T* grad = (const T*)p.in2 + (size_t)row * n;
+  T* out = (T*)p.out + (size_t)row * n;
+  float m = -INFINITY, gs = 0.0f;
+  for (uint32_t k = lane; k < n; k += 64) {
+    float x = (float)in[k];
+    if (x > m) m = x;
+    gs += (float)grad[k];
+  }
+  m = wave_reduce(m, MaxOp());
+  gs = wave_reduce(gs, SumOp());
+  float s = 0.0f;
+  for (uint32_t k = lane; k < n; k += 64) s += expf((float)in[k] - m);
+  s = wave_reduce(s, SumOp());
+  const float log_sum = logf(s) + m;
+  for (uint32_t k = lane; k < n; k += 64)
+    out[k] = narrow<T>((float)grad[k] - gs * expf((float)in[k] - log_sum));
+}
+
+template <typename T> __device__ __forceinline__ void log_softmax_grad_cols_impl(const hck_reduce_args& p) {
+  const uint32_t jblocks = (p.inner + HCK_BLOCK - 1) / HCK_BLOCK;
+  const uint32_t i = blockIdx.x / jblocks;
+  const uint32_t j = (blockIdx.x - i * jblocks) * HCK_BLOCK + threadIdx.x;
+  if (j >= p.inner) return;
+  const size_t base = (size_t)i * p.reduce * p.inner + j;
+  const T* in = (const T*)p.in + base;
+  const T* grad = (const T*)p.in2 + base;
+  T* out = (T*)p.out + base;
+  float m = 0.0f, gs = 0.0f;
+  for (uint32_t k = 0; k < p.reduce; k++) {
+    float x = (float)in[(size_t)k * p.inner];
+    gs += (float)grad[(size_t)k * p.inner];
+    if (k == 0 || x > m) m = x;
+  }
+  float s = 0.0f;
+  for (uint32_t k = 0; k < p.reduce; k++) s += expf((float)in[(size_t)k * p.inner] - m);
+  const float log_sum = logf(s) + m;
+  for (uint32_t k = 0; k < p.reduce; k++)
+    out[(size_t)k * p.inner] =
+        narrow<T>((float)grad[(size_t)k * p.inner] - gs * expf((float)in[(size_t)k * p.inner] - log_sum));
+}
+HC_KERNEL void hc_log_softmax_grad_rows_f32(hck_reduce_args p) { log_softmax_grad_rows_impl<float>(p); }
+HC_KERNEL void hc_log_softmax_grad_rows_f16(hck_reduce_args p) { log_softmax_grad_rows_impl<half_t>(p); }
+HC_KERNEL void hc_log_softmax_grad_cols_f32(hck_reduce_args p) { log_softmax_grad_cols_impl<float>(p); }
+HC_KERNEL void hc_log_softmax_grad_cols_f16(hck_reduce_args p) { log_softmax_grad_cols_impl<half_t>(p); }
+
 // ---------------------------------------------------------------- normalize
 
 // normalize for inner == 1, fused: the base-class composition (Backend.swift:265-327)

@@ -590,6 +590,41 @@ class Tensor:
                                  indicesAreUnique), self.dtype)
         return self._new(data, shape=indicesStrides.shape)
 
+    def scatter(self, axis: int, count: int, indices: "Tensor", indicesAreUnique=False) -> "Tensor":
+        """ScatterGather.swift:113-154: the adjoint of gather (values with equal index add up)."""
+        assert len(self.shape) > 0, "cannot scatter() on a zero-dimensional tensor"
+        assert indices.dtype == DType.int64, "can only scatter with indices of dtype int64"
+        axis = self.positiveAxis(axis)
+        indices, indicesStrides = self.expandIndices(axis, indices)
+        assert indices.shape[axis] == self.shape[axis], \
+            "shape %s is not compatible with indices shape %s for scatter along axis %d" % (
+                self.shape, indices.shape, axis)
+        newShape = list(self.shape)
+        newShape[axis] = count
+        data = Backend.current().scatter(
+            self.data,
+            ScatterGatherIndices(newShape, axis, BroadcastData(indicesStrides, indices.data), indicesAreUnique),
+            self.dtype)
+        return self._new(data, shape=newShape)
+
+    def clamp(self, min=None, max=None) -> "Tensor":
+        """Clamp.swift: element-wise min(max, max(min, x)); bounds are tensors or scalars."""
+        assert min is not None or max is not None, "cannot use clamp() without bounds"
+        tensors = [self] + [x for x in (min, max) if isinstance(x, Tensor)]
+        shape, strides = Tensor.lazyBroadcast(tensors)
+        it = iter(strides[1:])
+        bounds = []
+        for x in (min, max):
+            if x is None:
+                bounds.append(None)
+            elif isinstance(x, Tensor):
+                assert x.dtype == self.dtype, "clamp bounds must have the tensor's dtype"
+                bounds.append(BroadcastData(next(it), x.data))
+            else:
+                bounds.append(("scalar", x, shape))
+        data = Backend.current().clamp(BroadcastData(strides[0], self.data), bounds[0], bounds[1], self.dtype)
+        return Tensor(dataHandle=data, shape=shape, dtype=self.dtype)
+
     def __getitem__(self, index) -> "Tensor":
         if not isinstance(index, tuple):
             index = (index,)

@@ -236,6 +236,34 @@ int hc_gather(hc_ctx* ctx, int dtype, const void* in, const void* indices,
               const hc_strides* idx_strides, void* out, int64_t outer, int64_t middle,
               int64_t out_count, int64_t inner);
 
+/* Backend.scatter (Backend.swift:621-626; CPU BackendCPU.swift:1149-1188), the adjoint of
+ * gather: out[(i*middle + idx)*inner + k] += in[(i*out_count + j)*inner + k] over a zeroed
+ * output of outer*middle*inner elements; numeric dtypes. Values sharing an index are added
+ * with atomics (float sums in no fixed order; half values accumulate in float and are
+ * rounded once). indices_are_unique != 0 (ScatterGatherIndices.indicesAreUnique,
+ * ScatterGather.swift:4-19) lets the kernel store instead of add. */
+int hc_scatter(hc_ctx* ctx, int dtype, const void* in, const void* indices,
+               const hc_strides* idx_strides, void* out, int64_t outer, int64_t middle,
+               int64_t out_count, int64_t inner, int indices_are_unique);
+
+/* Backend.logSoftmaxGrad (Backend.swift:578-587; CPU BackendCPU.swift:1040-1085):
+ * out = g - sum_k(g) * exp(logSoftmax(x)) over the reduce axis. */
+int hc_log_softmax_grad(hc_ctx* ctx, int dtype, const void* in, const void* out_grad, void* out,
+                        int64_t outer, int64_t reduce, int64_t inner);
+
+/* Backend.clamp (Backend.swift:512-520; CPU BackendCPU.swift:704-782): min(hi, max(lo, a))
+ * over the broadcast shape of `as`; lo or hi (with its strides) may be NULL, not both. A
+ * scalar bound is a 1-element buffer with all-zero strides. */
+int hc_clamp(hc_ctx* ctx, int dtype, const void* a, const hc_strides* as, const void* lo,
+             const hc_strides* ls, const void* hi, const hc_strides* hs, void* out);
+
+/* Backend.adamW (Backend.swift:818-892), one fused pass that reproduces the base class's
+ * op-by-op composition bit for bit (every intermediate rounded to `dtype`); writes the new
+ * parameter and both new moments. step is the 1-based update count as a Float. */
+int hc_adamw(hc_ctx* ctx, int dtype, const void* param, const void* grad, const void* moment1,
+             const void* moment2, float beta1, float beta2, float eps, float weight_decay, float lr,
+             float step, size_t count, void* out_param, void* out_moment1, void* out_moment2);
+
 /* Backend.when (Backend.swift:633-641; CPU BackendCPU.swift:1190-1220); a scalar branch is
  * a 1-element buffer with all-zero strides, as CPUBackend.tensorOrScalarData makes it. */
 int hc_when(hc_ctx* ctx, int dtype, const void* mask, const hc_strides* ms, const void* a,

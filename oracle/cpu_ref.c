@@ -709,6 +709,115 @@ void ref_gather(int dtype, const void* in, const int64_t* idx, const ref_strides
   }
 }
 
+/* ---- scatter (BackendCPU.swift:1149-1188): sequential accumulation in Float / Int64 ---- */
+
+void ref_scatter(int dtype, const void* in, const int64_t* idx, const ref_strides* idx_strides,
+                 void* out, int64_t outer, int64_t middle, int64_t out_count, int64_t inner) {
+  size_t n_in = (size_t)(outer * out_count * inner), n_out = (size_t)(outer * middle * inner);
+  if (dtype == REF_I64) {
+    const int64_t* x = (const int64_t*)in;
+    int64_t* z = (int64_t*)out;
+    for (size_t t = 0; t < n_out; t++) z[t] = 0;
+    for (int64_t i = 0; i < outer; i++)
+      for (int64_t j = 0; j < out_count; j++)
+        for (int64_t k = 0; k < inner; k++) {
+          int64_t in_idx = (i * out_count + j) * inner + k;
+          int64_t j_out = idx[ref_strides_index(idx_strides, in_idx)];
+          int64_t out_idx = (i * middle + j_out) * inner + k;
+          z[out_idx] = z[out_idx] + x[in_idx];
+        }
+    return;
+  }
+  float *xo, *zo;
+  const float* x = load_f(dtype, in, n_in, &xo);
+  float* z = out_f(dtype, out, n_out, &zo);
+  for (size_t t = 0; t < n_out; t++) z[t] = 0.0f;
+  for (int64_t i = 0; i < outer; i++)
+    for (int64_t j = 0; j < out_count; j++)
+      for (int64_t k = 0; k < inner; k++) {
+        int64_t in_idx = (i * out_count + j) * inner + k;
+        int64_t j_out = idx[ref_strides_index(idx_strides, in_idx)];
+        int64_t out_idx = (i * middle + j_out) * inner + k;
+        z[out_idx] = z[out_idx] + x[in_idx];
+      }
+  store_f(dtype, out, n_out, zo);
+  free(xo);
+}
+
+/* ---- logSoftmaxGrad (BackendCPU.swift:1040-1085) ---- */
+
+void ref_log_softmax_grad(int dtype, const void* in, const void* out_grad, void* out, int64_t outer,
+                          int64_t reduce, int64_t inner) {
+  size_t total = (size_t)(outer * reduce * inner);
+  float *ao, *go, *zo;
+  const float* arr = load_f(dtype, in, total, &ao);
+  const float* grad = load_f(dtype, out_grad, total, &go);
+  float* z = out_f(dtype, out, total, &zo);
+#pragma omp parallel for num_threads(nthreads()) if (total > 65536)
+  for (int64_t i = 0; i < outer; i++) {
+    int64_t off = i * inner * reduce;
+    for (int64_t j = 0; j < inner; j++) {
+      float max = 0, grad_sum = 0;
+      for (int64_t k = 0; k < reduce; k++) {
+        int64_t idx = j + k * inner + off;
+        float item = arr[idx];
+        grad_sum += grad[idx];
+        if (k == 0 || item > max) max = item;
+      }
+      float exp_sum = 0;
+      for (int64_t k = 0; k < reduce; k++) exp_sum += expf(arr[j + k * inner + off] - max);
+      float log_sum = logf(exp_sum) + max;
+      for (int64_t k = 0; k < reduce; k++) {
+        int64_t idx = j + k * inner + off;
+        z[idx] = grad[idx] - grad_sum * expf(arr[idx] - log_sum);
+      }
+    }
+  }
+  store_f(dtype, out, total, zo);
+  free(ao);
+  free(go);
+}
+
+/* ---- clamp (BackendCPU.swift:704-782): Swift.min / Swift.max on Float or Int64 ----
+ * Swift.max(x, y) returns y unless x > y ... precisely: max(x, y) = y >= x ? y : x and
+ * min(x, y) = y < x ? y : x (stdlib Algorithm.swift), which fixes what a NaN does. */
+
+static float swift_maxf(float x, float y) { return y >= x ? y : x; }
+static float swift_minf(float x, float y) { return y < x ? y : x; }
+static int64_t swift_maxi(int64_t x, int64_t y) { return y >= x ? y : x; }
+static int64_t swift_mini(int64_t x, int64_t y) { return y < x ? y : x; }
+
+void ref_clamp(int dtype, const void* a, const ref_strides* as, const void* lo, const ref_strides* ls,
+               const void* hi, const ref_strides* hs, void* out) {
+  int64_t n = shape_product(as);
+  if (dtype == REF_I64) {
+    const int64_t *x = (const int64_t*)a, *l = (const int64_t*)lo, *h = (const int64_t*)hi;
+    int64_t* z = (int64_t*)out;
+    for (int64_t i = 0; i < n; i++) {
+      int64_t v = x[ref_strides_index(as, i)];
+      if (l) v = swift_maxi(l[ref_strides_index(ls, i)], v);
+      if (h) v = swift_mini(h[ref_strides_index(hs, i)], v);
+      z[i] = v;
+    }
+    return;
+  }
+  float *xo, *lo_o = NULL, *hi_o = NULL, *zo;
+  const float* x = load_f(dtype, a, (size_t)data_count(as), &xo);
+  const float* l = lo ? load_f(dtype, lo, (size_t)data_count(ls), &lo_o) : NULL;
+  const float* h = hi ? load_f(dtype, hi, (size_t)data_count(hs), &hi_o) : NULL;
+  float* z = out_f(dtype, out, (size_t)n, &zo);
+  for (int64_t i = 0; i < n; i++) {
+    float v = x[ref_strides_index(as, i)];
+    if (l) v = swift_maxf(l[ref_strides_index(ls, i)], v);
+    if (h) v = swift_minf(h[ref_strides_index(hs, i)], v);
+    z[i] = v;
+  }
+  store_f(dtype, out, (size_t)n, zo);
+  free(xo);
+  free(lo_o);
+  free(hi_o);
+}
+
 /* ---- when (BackendCPU.swift:1190-1220) ---- */
 
 void ref_when(int dtype, const uint8_t* mask, const ref_strides* ms, const void* a,

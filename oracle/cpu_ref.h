@@ -26,6 +26,12 @@
  *                     half patterns, and random float32 -> half)
  *   mulAdd / addMul   fused == composed (:154-191)
  *   normalize         fused == composed formula (:193-219), numpy two-pass
+ *   scatter           input gradients of testGather (:585-650) and the direct scatter
+ *                     permutation (:626-633); numpy np.add.at on random indices
+ *   logSoftmaxGrad    3x5 gradient goldens for both axes (:1552-1610); closed form
+ *                     g - sum(g) * softmax(x) in float64; rows of the result sum to ~0
+ *                     when weighted appropriately (sum_k out = sum(g) * (1 - 1) = 0)
+ *   clamp             testClamp (:1235-1323), numpy clip / minimum / maximum
  */
 #ifndef HC_ORACLE_CPU_REF_H
 #define HC_ORACLE_CPU_REF_H
@@ -96,6 +102,16 @@ void ref_log_softmax(int dtype, const void* in, void* out, int64_t outer, int64_
                      int64_t inner);
 void ref_gather(int dtype, const void* in, const int64_t* idx, const ref_strides* idx_strides,
                 void* out, int64_t outer, int64_t middle, int64_t out_count, int64_t inner);
+/* BackendCPU.swift:1149-1188. `in` holds outer*out_count*inner elements, `out` receives
+ * outer*middle*inner; contributions to one output add up in (i, j, k) order in Float/Int64. */
+void ref_scatter(int dtype, const void* in, const int64_t* idx, const ref_strides* idx_strides,
+                 void* out, int64_t outer, int64_t middle, int64_t out_count, int64_t inner);
+/* BackendCPU.swift:1040-1085. */
+void ref_log_softmax_grad(int dtype, const void* in, const void* out_grad, void* out, int64_t outer,
+                          int64_t reduce, int64_t inner);
+/* BackendCPU.swift:704-782: out = min(hi, max(lo, a)); lo or hi may be NULL (not both). */
+void ref_clamp(int dtype, const void* a, const ref_strides* as, const void* lo, const ref_strides* ls,
+               const void* hi, const ref_strides* hs, void* out);
 void ref_when(int dtype, const uint8_t* mask, const ref_strides* ms, const void* a,
               const ref_strides* as, const void* b, const ref_strides* bs, void* out);
 void ref_matmul(int dtype, int64_t batch, const void* a, int trans_a, const void* b, int trans_b,

@@ -41,6 +41,9 @@ _PROTOS = {
     "ref_reduce": (None, [c_int, c_int, _P, _P, c_int64, c_int64, c_int64]),
     "ref_log_softmax": (None, [c_int, _P, _P, c_int64, c_int64, c_int64]),
     "ref_gather": (None, [c_int, _P, _P, _S, _P, c_int64, c_int64, c_int64, c_int64]),
+    "ref_scatter": (None, [c_int, _P, _P, _S, _P, c_int64, c_int64, c_int64, c_int64]),
+    "ref_log_softmax_grad": (None, [c_int, _P, _P, _P, c_int64, c_int64, c_int64]),
+    "ref_clamp": (None, [c_int, _P, _S, _P, _S, _P, _S, _P]),
     "ref_when": (None, [c_int, _P, _S, _P, _S, _P, _S, _P]),
     "ref_matmul": (None, [c_int, c_int64, _P, c_int, _P, c_int, c_int, c_int64, c_int64, c_int64, _P]),
     "ref_matmul_rows": (None, [c_int, _P, c_int, _P, c_int, c_int64, c_int64, c_int64, c_int64, c_int64, _P]),
@@ -233,6 +236,33 @@ class OracleBackend(Backend):
         self.lib.ref_gather(int(dtype), self._host(a).ptr, self._host(s.indices.data).ptr,
                             self._s(s.indices.strides), out.ptr, s.outerCount, s.middleCount, s.outCount,
                             s.innerCount)
+        return out
+
+    def scatter(self, a, s: ScatterGatherIndices, dtype):
+        out = CPUData(s.gatherInCount * dtype.byteSize)
+        self.lib.ref_scatter(int(dtype), self._host(a).ptr, self._host(s.indices.data).ptr,
+                             self._s(s.indices.strides), out.ptr, s.outerCount, s.middleCount, s.outCount,
+                             s.innerCount)
+        return out
+
+    def logSoftmaxGrad(self, a, outGrad, dims, dtype):
+        out = CPUData(dims.inCount * dtype.byteSize)
+        self.lib.ref_log_softmax_grad(int(dtype), self._host(a).ptr, self._host(outGrad).ptr, out.ptr,
+                                      dims.outerCount, dims.reduceCount, dims.innerCount)
+        return out
+
+    def clamp(self, a, min, max, dtype):
+        assert min is not None or max is not None, "cannot use clamp() without bounds"
+        def bound(x):
+            if x is None or isinstance(x, BroadcastData):
+                return x
+            _, value, shape = x
+            return BroadcastData(BroadcastStrides(shape, [0] * len(shape)), self.constant(value, 1, dtype))
+        lo, hi = bound(min), bound(max)
+        out = CPUData(product(a.strides.shape) * dtype.byteSize)
+        self.lib.ref_clamp(int(dtype), self._host(a.data).ptr, self._s(a.strides),
+                           self._host(lo.data).ptr if lo else None, self._s(lo.strides) if lo else None,
+                           self._host(hi.data).ptr if hi else None, self._s(hi.strides) if hi else None, out.ptr)
         return out
 
     def matmul(self, a, transA, b, transB, transOut, rows, inner, cols, dtype):

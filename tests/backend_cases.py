@@ -515,6 +515,135 @@ def testSoftmax(rng):
         assertClose(out1, out2, atol=tol, rtol=tol)
 
 
+def testSoftmaxGrad(rng):
+    """BackendTests.swift:1552-1626, the gradients: logSoftmaxGrad called the way
+    Tensor.logSoftmax's backward does (Softmax.swift), golden input gradients for both axes,
+    and axis-invariance on random data."""
+    from honeycrisp_amd.backend import Backend
+    g = GOLDEN["softmax"]
+    x = Tensor(data=g["x"], shape=g["shape"])
+    og = Tensor(data=g["out_grad"], shape=g["shape"])
+    backend = Backend.current()
+    for axis, key in ((0, "axis0_grad"), (1, "axis1_grad")):
+        data = backend.logSoftmaxGrad(x.data, og.data, x.reduceDims(axis), x.dtype)
+        assertClose(Tensor(dataHandle=data, shape=x.shape, dtype=x.dtype), g[key])
+    for dtype in (F16, F32):
+        tol = 1e-2 if dtype == F16 else 1e-4
+        inp = Tensor(data=rng.random([7, 3, 292]).astype(np.float32), dtype=dtype)
+        grad = Tensor(data=rng.random([7, 3, 292]).astype(np.float32), dtype=dtype)
+        g1 = Tensor(dataHandle=backend.logSoftmaxGrad(inp.data, grad.data, inp.reduceDims(-1), dtype),
+                    shape=inp.shape, dtype=dtype)
+        moved, movedGrad = inp.move(-1, 1), grad.move(-1, 1)
+        g2 = Tensor(dataHandle=backend.logSoftmaxGrad(moved.data, movedGrad.data, moved.reduceDims(1), dtype),
+                    shape=moved.shape, dtype=dtype).move(1, -1)
+        assertClose(g1, g2, atol=tol, rtol=tol)
+
+
+def testScatter():
+    """BackendTests.swift:585-650: the input gradients of testGather are scatters of the output
+    gradient with the gather's indices (ScatterGather.swift:98-108), plus the direct scatter
+    permutation (:626-633)."""
+    for dtype in (F16, F32):
+        def grad_of_gather(axis, indices, outGrad, shape, unique=False):
+            og = Tensor(data=outGrad, shape=shape, dtype=dtype)
+            return og.scatter(axis, [1, 2, 3, 1][axis], indices, indicesAreUnique=unique)
+        for unique in (False, True):
+            got = grad_of_gather(2, Tensor(data=[2, 0, 1, 2], shape=[1, 2, 2, 1], dtype=I64),
+                                 [1.0, 2.0, 3.0, 4.0], [1, 2, 2, 1], unique)
+            assert got.shape == [1, 2, 3, 1]
+            assertDataEqual(got, [2.0, 0.0, 1.0, 0.0, 3.0, 4.0])
+            got = grad_of_gather(2, Tensor(data=[2, 0], shape=[2], dtype=I64),
+                                 [1.0, 2.0, 3.0, 4.0], [1, 2, 2, 1], unique)
+            assertDataEqual(got, [2.0, 0.0, 1.0, 4.0, 0.0, 3.0])
+        got = grad_of_gather(1, Tensor(data=[0, 1, 0, 1, 0, 0], shape=[1, 2, 3, 1], dtype=I64),
+                             [1.0, 2.0, 3.0, 4.0, 5.0, 6.0], [1, 2, 3, 1])
+        assertDataEqual(got, [1.0, 5.0, 9.0, 4.0, 2.0, 0.0])
+        got = grad_of_gather(1, Tensor(data=[1, 0], shape=[2], dtype=I64),
+                             [1.0, 2.0, 3.0, 4.0, 5.0, 6.0], [1, 2, 3, 1])
+        assertDataEqual(got, [4.0, 5.0, 6.0, 1.0, 2.0, 3.0])
+        permuteMe = Tensor(data=[1.0, 2.0, 3.0, 4.0, 5.0, 6.0], shape=[1, 2, 3, 1], dtype=dtype)
+        for unique in (False, True):
+            out = permuteMe.scatter(1, 2, Tensor(data=[1, 0], shape=[2]), indicesAreUnique=unique)
+            assertDataEqual(out, [4.0, 5.0, 6.0, 1.0, 2.0, 3.0])
+    # int64 values accumulate too
+    vals = Tensor(data=[5, 6, 7, 8], shape=[4], dtype=I64)
+    assertDataEqual(vals.scatter(0, 3, Tensor(data=[2, 0, 2, 2], shape=[4])), [6, 0, 20])
+
+
+def testScatterIsAdjointOfGather(rng):
+    """BackendTests.swift:660-681, the gradient half: scattering with broadcast indices equals
+    scattering with the explicitly expanded ones."""
+    for dtype in (F16, F32):
+        tol = 1e-2 if dtype == F16 else 1e-4
+        indices = Tensor(data=[i % 4 for i in range(20)], shape=[1, 4, 5])
+        outGrad = Tensor(data=rng.random([3, 4, 5]).astype(np.float32), dtype=dtype)
+        actual = outGrad.scatter(1, 4, indices)
+        expected = outGrad.scatter(1, 4, indices.expand([3, 4, 5]))
+        assert actual.shape == [3, 4, 5]
+        assertClose(actual, expected, atol=tol, rtol=tol)
+
+
+def testClamp():
+    """BackendTests.swift:1235-1323 (forward values)."""
+    g = GOLDEN["clamp"]
+    for dtype in (I64, F16, F32):
+        dim1 = Tensor(data=g["dim1"], shape=[5, 1, 1], dtype=dtype)
+        dim2 = Tensor(data=g["dim2"], shape=[1, 4, 1], dtype=dtype)
+        dim3 = Tensor(data=g["dim3"], shape=[1, 1, 6], dtype=dtype)
+        clamped = dim1.clamp(min=dim2, max=dim3)
+        assert clamped.shape == [5, 4, 6]
+        assertDataEqual(clamped, g["out"])
+        a = Tensor(data=[1, 2, 3, 4, 5], shape=[5, 1], dtype=dtype)
+        b = Tensor(data=[1, 2, 3], shape=[1, 3], dtype=dtype)
+        assertClose(a.clamp(min=b, max=4), g["tensor_scalar_out"])
+    x = Tensor(data=[1.0, 2.0, 3.0])
+    assertDataEqual(x.clamp(min=10, max=-3), [-3, -3, -3])
+    assertDataEqual(x.clamp(min=10, max=Tensor(data=[-3.0, -3.0, -3.0])), [-3, -3, -3])
+    assertDataEqual(x.clamp(min=2), [2, 2, 3])
+    assertDataEqual(x.clamp(max=2), [1, 2, 2])
+
+
+def testAdam():
+    """BackendTests.swift:1779-1797: three AdamW steps (lr 1, beta1 0.25, beta2 0.5, decay 0.1) on
+    a three-element parameter, moments starting at zero and the step counter at 1
+    (Optimizer.swift:129-152)."""
+    from honeycrisp_amd.backend import Backend
+    g = GOLDEN["adam"]
+    backend = Backend.current()
+    for dtype in (F16, F32):
+        tol = 0.01 if dtype == F16 else 0.0001
+        param = Tensor(data=g["param"], dtype=dtype)
+        m1 = Tensor.zeros([3], dtype=dtype)
+        m2 = Tensor.zeros([3], dtype=dtype)
+        for t, (grad, want) in enumerate(zip(g["grads"], g["expected"]), start=1):
+            gradT = Tensor(data=grad, dtype=dtype)
+            p, a, b = backend.adamW(param.data, gradT.data, m1.data, m2.data, g["beta1"], g["beta2"], g["eps"],
+                                    g["weightDecay"], g["lr"], float(t), 3, dtype)
+            param, m1, m2 = (Tensor(dataHandle=d, shape=[3], dtype=dtype) for d in (p, a, b))
+            assertClose(param, want, atol=tol, rtol=tol)
+
+
+def testNormalizeGrad(rng):
+    """Backend.normalizeGrad (Backend.swift:332-455) against central differences of normalize
+    in float64 arithmetic (numpy): the analytic gradient of (x - mean) / sqrt(var + eps)."""
+    from honeycrisp_amd.backend import Backend
+    backend = Backend.current()
+    x = rng.standard_normal((5, 7, 3)).astype(np.float32)
+    og = rng.standard_normal((5, 7, 3)).astype(np.float32)
+    eps = 1e-3
+    xt, ogt = Tensor(data=x), Tensor(data=og)
+    data = backend.normalizeGrad(xt.data, ogt.data, xt.reduceDims(1), np.float32(eps), F32)
+    got = np.asarray(Tensor(dataHandle=data, shape=[5, 7, 3], dtype=F32).floats()).reshape(5, 7, 3)
+    x64, og64 = x.astype(np.float64), og.astype(np.float64)
+    mean = x64.mean(1, keepdims=True)
+    c = x64 - mean
+    var = (c * c).mean(1, keepdims=True)
+    inv = (var + eps) ** -0.5
+    cg = og64 - og64.mean(1, keepdims=True)
+    want = cg * inv - c * (c * og64).sum(1, keepdims=True) * (var + eps) ** -1.5 / 7
+    assert_close_arrays(got, want, 1e-4, 1e-4)
+
+
 def testConcat():
     """Concatenation along an inner and an outer axis (Tensor(concat:), ConcatSplit.swift:4-75;
     CPU loop BackendCPU.swift:1768-1794); expected values follow from the definition."""
@@ -543,5 +672,6 @@ ALL_CASES = [
     testMod, testEquals, testComparison, testSum, testGather, testGatherBroadcastOtherAxis,
     testMatrixMatrixProduct, testBatchedMatmul, testMatrixVectorProduct, testTriangular, testIndexing,
     testElemwise, testRounding, testMinMax, testExpandAndRepeat, testBinaryBroadcast, testFusedBroadcast,
-    testSoftmax, testConcat, testWhen,
+    testSoftmax, testConcat, testWhen, testSoftmaxGrad, testScatter, testScatterIsAdjointOfGather, testClamp,
+    testAdam, testNormalizeGrad,
 ]

@@ -425,3 +425,104 @@ def test_bandwidth_ops_full_size(hip_backend, oracle_backend):
     with hip_backend.use():
         out = Tensor(data=table).gather(0, Tensor(data=ids)).numpy()
     assert np.array_equal(out, table[ids])
+
+
+# ---------------------------------------------------------------- backward primitives
+
+@pytest.mark.parametrize("dtype", [F32, F16, I64], ids=["f32", "f16", "i64"])
+def test_scatter_forms(hip_backend, oracle_backend, dtype):
+    rng = np.random.default_rng(31)
+    # small integers: every partial sum is exact, so the order of the atomic adds cannot matter
+    vals = rng.integers(-8, 9, size=(6, 37, 20))
+    vals = vals if dtype == I64 else vals.astype(dtype.numpy)
+    idx = rng.integers(0, 11, size=(6, 37, 20))
+    check_exact(hip_backend, oracle_backend, lambda: Tensor(data=vals).scatter(1, 11, Tensor(data=idx)))
+    # broadcast indices (one index per row), the embedding-gradient shape
+    rows = rng.integers(0, 50, size=(300,))
+    emb = rng.integers(-8, 9, size=(300, 64))
+    emb = emb if dtype == I64 else emb.astype(dtype.numpy)
+    check_exact(hip_backend, oracle_backend, lambda: Tensor(data=emb).scatter(0, 50, Tensor(data=rows)))
+    # unique indices: plain stores
+    perm = rng.permutation(300)
+    check_exact(hip_backend, oracle_backend,
+                lambda: Tensor(data=emb).scatter(0, 300, Tensor(data=perm), indicesAreUnique=True))
+    # empty input still zero-fills the output
+    empty = np.zeros((0, 4), dtype=np.int64 if dtype == I64 else dtype.numpy)
+    check_exact(hip_backend, oracle_backend,
+                lambda: Tensor(data=empty, shape=[0, 4], dtype=dtype).scatter(0, 3, Tensor(data=[], shape=[0], dtype=I64)))
+
+
+@pytest.mark.parametrize("dtype", [F32, F16], ids=["f32", "f16"])
+def test_scatter_random_floats_within_tolerance(hip_backend, oracle_backend, dtype):
+    rng = np.random.default_rng(32)
+    vals = rng.standard_normal((4096, 96)).astype(dtype.numpy)
+    rows = rng.integers(0, 257, size=(4096,))
+    check_close(hip_backend, oracle_backend, lambda: Tensor(data=vals).scatter(0, 257, Tensor(data=rows)),
+                TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", [F32, F16], ids=["f32", "f16"])
+def test_log_softmax_grad(hip_backend, oracle_backend, dtype):
+    from honeycrisp_amd.backend import Backend
+    rng = np.random.default_rng(33)
+    for shape, axis in [((64, 300), 1), ((7, 33, 40), 1), ((5, 1, 9), 2), ((3, 1000), 0), ((2048, 256), 1)]:
+        x, g = rand(rng, shape, dtype, 2.0), rand(rng, shape, dtype)
+        def run():
+            xt, gt = Tensor(data=x), Tensor(data=g)
+            data = Backend.current().logSoftmaxGrad(xt.data, gt.data, xt.reduceDims(axis), dtype)
+            return Tensor(dataHandle=data, shape=list(shape), dtype=dtype)
+        check_close(hip_backend, oracle_backend, run, TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", [F32, F16, I64], ids=["f32", "f16", "i64"])
+def test_clamp(hip_backend, oracle_backend, dtype):
+    rng = np.random.default_rng(34)
+    x, lo = rand(rng, (33, 1, 40), dtype), rand(rng, (1, 17, 40), dtype)
+    hi = rand(rng, (33, 17, 1), dtype)
+    check_exact(hip_backend, oracle_backend, lambda: Tensor(data=x).clamp(min=Tensor(data=lo), max=Tensor(data=hi)))
+    check_exact(hip_backend, oracle_backend, lambda: Tensor(data=x).clamp(min=Tensor(data=lo)))
+    check_exact(hip_backend, oracle_backend, lambda: Tensor(data=x).clamp(max=Tensor(data=hi)))
+    check_exact(hip_backend, oracle_backend, lambda: Tensor(data=x).clamp(min=-1, max=2))
+    flat = rand(rng, (100003,), dtype)
+    check_exact(hip_backend, oracle_backend, lambda: Tensor(data=flat).clamp(min=-1))
+    if dtype != I64:
+        special = np.array([np.nan, -np.inf, np.inf, -0.0, 0.0, 1.5], dtype=dtype.numpy)
+        check_exact(hip_backend, oracle_backend, lambda: Tensor(data=special).clamp(min=-1, max=1))
+
+
+@pytest.mark.parametrize("dtype", [F32, F16], ids=["f32", "f16"])
+def test_adamw_fused_equals_composition(hip_backend, oracle_backend, dtype):
+    """The fused kernel against the base class's op-by-op composition run on the same device
+    (bit for bit), and against the oracle's composition (tolerance: libm vs device powf)."""
+    from honeycrisp_amd.backend import Backend
+    rng = np.random.default_rng(35)
+    n = 100003
+    p, g = rand(rng, (n,), dtype), rand(rng, (n,), dtype)
+    m, v = rand(rng, (n,), dtype, 0.1), np.abs(rand(rng, (n,), dtype, 0.1))
+    for hyper in [(0.9, 0.999, 1e-8, 0.01, 3e-3, 7.0), (0.25, 0.5, 1e-8, 0.1, 1.0, 1.0), (0.9, 0.0, 1e-6, 0.0, 1e-2, 2.0)]:
+        def run(backend, composed):
+            with backend.use():
+                args = [Tensor(data=a).data for a in (p, g, m, v)]
+                fn = (lambda *a: Backend.adamW(backend, *a)) if composed else backend.adamW
+                outs = fn(*args, *hyper, n, dtype)
+                return [Tensor(dataHandle=d, shape=[n], dtype=dtype).numpy() for d in outs]
+        fused, composed, want = run(hip_backend, False), run(hip_backend, True), run(oracle_backend, True)
+        bits = {2: np.uint16, 4: np.uint32}[dtype.byteSize]
+        for a, b, c in zip(fused, composed, want):
+            same = (a.view(bits) == b.view(bits)) | (np.isnan(a) & np.isnan(b))
+            assert same.all(), "%d elements differ from the composition" % int((~same).sum())
+            assert_close_arrays(a, c, TOL[dtype], TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", [F32, F16], ids=["f32", "f16"])
+def test_normalize_grad(hip_backend, oracle_backend, dtype):
+    from honeycrisp_amd.backend import Backend
+    rng = np.random.default_rng(36)
+    tol = 2e-2 if dtype == F16 else 1e-4
+    for shape, axis in [((64, 512), 1), ((6, 33, 5), 1)]:
+        x, g = rand(rng, shape, dtype), rand(rng, shape, dtype)
+        def run():
+            xt, gt = Tensor(data=x), Tensor(data=g)
+            data = Backend.current().normalizeGrad(xt.data, gt.data, xt.reduceDims(axis), np.float32(1e-3), dtype)
+            return Tensor(dataHandle=data, shape=list(shape), dtype=dtype)
+        check_close(hip_backend, oracle_backend, run, tol)

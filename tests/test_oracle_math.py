@@ -280,6 +280,79 @@ def test_log_softmax_vs_scipy(oracle_backend):
         assert_close_arrays(sm.sum(axis=-1), np.ones((5, 17)), 1e-5, 1e-5)
 
 
+def test_scatter_vs_numpy_add_at(oracle_backend):
+    rng = np.random.default_rng(21)
+    with oracle_backend.use():
+        vals = rng.integers(-8, 9, size=(4, 7, 5)).astype(np.float32)      # small integers: sums are exact
+        idx = rng.integers(0, 3, size=(4, 7, 5))
+        got = Tensor(data=vals).scatter(1, 3, Tensor(data=idx)).numpy()
+        want = np.zeros((4, 3, 5), np.float32)
+        i, _, k = np.meshgrid(np.arange(4), np.arange(7), np.arange(5), indexing="ij")
+        np.add.at(want, (i, idx, k), vals)
+        assert np.array_equal(got, want)
+        rows = rng.integers(0, 6, size=(11,))
+        flat = rng.integers(-8, 9, size=(11, 4)).astype(np.int64)
+        want = np.zeros((6, 4), np.int64)
+        np.add.at(want, rows, flat)
+        assert np.array_equal(Tensor(data=flat).scatter(0, 6, Tensor(data=rows)).numpy(), want)
+        # scatter is the adjoint of gather: <gather(x), y> == <x, scatter(y)>
+        x = rng.standard_normal((4, 3, 5)).astype(np.float32)
+        y = rng.standard_normal((4, 7, 5)).astype(np.float32)
+        lhs = float((Tensor(data=x).gather(1, Tensor(data=idx)).numpy().astype(np.float64) * y).sum())
+        rhs = float((x.astype(np.float64) * Tensor(data=y).scatter(1, 3, Tensor(data=idx)).numpy()).sum())
+        assert abs(lhs - rhs) < 1e-4 * max(1.0, abs(lhs))
+
+
+def test_log_softmax_grad_closed_form(oracle_backend):
+    rng = np.random.default_rng(22)
+    x = (rng.standard_normal((5, 17, 3)) * 3).astype(np.float32)
+    g = rng.standard_normal((5, 17, 3)).astype(np.float32)
+    with oracle_backend.use():
+        for axis in (0, 1, 2):
+            t = Tensor(data=x)
+            data = oracle_backend.logSoftmaxGrad(t.data, Tensor(data=g).data, t.reduceDims(axis), F32)
+            got = arr(oracle_backend, data, F32).reshape(x.shape)
+            soft = scipy.special.softmax(x.astype(np.float64), axis=axis)
+            want = g.astype(np.float64) - g.astype(np.float64).sum(axis=axis, keepdims=True) * soft
+            assert_close_arrays(got, want, 1e-5, 1e-5)
+            # the Jacobian of log-softmax annihilates constants along the axis
+            assert np.abs(got.astype(np.float64).sum(axis=axis)).max() < 1e-4
+
+
+def test_clamp_vs_numpy(oracle_backend):
+    rng = np.random.default_rng(23)
+    x = rng.standard_normal((6, 1, 5)).astype(np.float32)
+    lo = (rng.standard_normal((1, 4, 5)) - 0.5).astype(np.float32)
+    hi = lo + np.float32(0.7)
+    with oracle_backend.use():
+        got = Tensor(data=x).clamp(min=Tensor(data=lo), max=Tensor(data=hi)).numpy()
+        assert np.array_equal(got, np.minimum(hi, np.maximum(lo, x)))
+        assert np.array_equal(Tensor(data=x).clamp(min=-0.25).numpy(), np.maximum(x, np.float32(-0.25)))
+        assert np.array_equal(Tensor(data=x).clamp(max=0.25).numpy(), np.minimum(x, np.float32(0.25)))
+        xi = rng.integers(-50, 50, size=(9,))
+        assert np.array_equal(Tensor(data=xi).clamp(min=-7, max=11).numpy(), np.clip(xi, -7, 11))
+
+
+def test_adamw_composition_vs_float64_formula(oracle_backend):
+    """The op-by-op composition against the textbook AdamW update in float64."""
+    rng = np.random.default_rng(24)
+    n = 257
+    p, g = rng.standard_normal(n).astype(np.float32), rng.standard_normal(n).astype(np.float32)
+    m, v = (rng.standard_normal(n) * 0.1).astype(np.float32), (rng.random(n) * 0.1).astype(np.float32)
+    b1, b2, eps, wd, lr, step = 0.9, 0.999, 1e-8, 0.01, 3e-3, 5.0
+    with oracle_backend.use():
+        t = lambda a: Tensor(data=a).data
+        np_, nm, nv = oracle_backend.adamW(t(p), t(g), t(m), t(v), b1, b2, eps, wd, lr, step, n, F32)
+        got_p, got_m, got_v = (arr(oracle_backend, d, F32) for d in (np_, nm, nv))
+    p64, g64, m64, v64 = (a.astype(np.float64) for a in (p, g, m, v))
+    wm = b1 * m64 + (1 - b1) * g64
+    wv = b2 * v64 + (1 - b2) * g64 * g64
+    want = p64 * (1 - lr * wd) - lr * (wm / (1 - b1 ** step)) / (np.sqrt(wv / (1 - b2 ** step)) + eps)
+    assert_close_arrays(got_m, wm, 1e-6, 1e-5)
+    assert_close_arrays(got_v, wv, 1e-6, 1e-5)
+    assert_close_arrays(got_p, want, 1e-5, 1e-5)
+
+
 def test_cast_rules(oracle_backend):
     with oracle_backend.use():
         f = Tensor(data=np.array([-2.9, -0.5, 0.0, 0.99, 7.5, 65519.0, 65520.0], dtype=np.float32))
