@@ -96,6 +96,7 @@ struct ScatterGatherIndices {
   std::vector<int64_t> valueShape;
   int axis;
   BroadcastData indices;
+  bool indicesAreUnique = false;
   int64_t outer() const { return prod(0, axis); }
   int64_t middle() const { return valueShape[axis]; }
   int64_t inner() const { return prod(axis + 1, (int)valueShape.size()); }
@@ -128,6 +129,18 @@ class HIPBackend {
   }
   void download(const Data& d, void* host, size_t bytes) { check(hc_memcpy_d2h(ctx_, host, d->ptr(), bytes)); }
   void wait() { check(hc_sync(ctx_)); }
+
+  // ---- recording and replay (no counterpart in the reference: one call replays every op
+  // issued between beginCapture and endCapture; buffers allocated in between stay reserved
+  // for the graph until it is destroyed)
+  void beginCapture() { check(hc_capture_begin(ctx_)); }
+  hc_graph* endCapture() {
+    hc_graph* g = nullptr;
+    check(hc_capture_end(ctx_, &g));
+    return g;
+  }
+  void launch(hc_graph* g) { check(hc_graph_launch(ctx_, g)); }
+  void destroy(hc_graph* g) { check(hc_graph_destroy(ctx_, g)); }
 
   // ---- ops (Backend.swift line of each declaration in the comment)
   Data broadcast(const BroadcastData& a, DType dtype) {  // :170
@@ -203,6 +216,40 @@ class HIPBackend {
     check(hc_gather(ctx_, (int)dtype, a->ptr(), s.indices.data->ptr(), &st, out->ptr(), s.outer(), s.middle(),
                     s.outCount(), s.inner()));
     return out;
+  }
+  Data scatter(const Data& a, const ScatterGatherIndices& s, DType dtype) {  // :621
+    Data out = allocate((size_t)(s.outer() * s.middle() * s.inner()) * byteSize(dtype));
+    hc_strides st = s.indices.strides.c();
+    check(hc_scatter(ctx_, (int)dtype, a->ptr(), s.indices.data->ptr(), &st, out->ptr(), s.outer(), s.middle(),
+                     s.outCount(), s.inner(), s.indicesAreUnique));
+    return out;
+  }
+  Data logSoftmaxGrad(const Data& a, const Data& outGrad, ReduceDims dims, DType dtype) {  // :578
+    Data out = allocate(dims.inCount() * byteSize(dtype));
+    check(hc_log_softmax_grad(ctx_, (int)dtype, a->ptr(), outGrad->ptr(), out->ptr(), dims.outerCount,
+                              dims.reduceCount, dims.innerCount));
+    return out;
+  }
+  // min / max: a BroadcastData with a null `data` means "no bound" (Backend.swift:512-520)
+  Data clamp(const BroadcastData& a, const BroadcastData& min, const BroadcastData& max, DType dtype) {
+    Data out = allocate(a.strides.count() * byteSize(dtype));
+    hc_strides sa = a.strides.c(), sl = min.strides.c(), sh = max.strides.c();
+    check(hc_clamp(ctx_, (int)dtype, a.data->ptr(), &sa, min.data ? min.data->ptr() : nullptr,
+                   min.data ? &sl : nullptr, max.data ? max.data->ptr() : nullptr, max.data ? &sh : nullptr,
+                   out->ptr()));
+    return out;
+  }
+  struct AdamResult {
+    Data param, moment1, moment2;
+  };
+  AdamResult adamW(const Data& param, const Data& grad, const Data& moment1, const Data& moment2, float beta1,
+                   float beta2, float eps, float weightDecay, float lr, float step, size_t count,
+                   DType dtype) {  // :818
+    AdamResult r{allocate(count * byteSize(dtype)), allocate(count * byteSize(dtype)),
+                 allocate(count * byteSize(dtype))};
+    check(hc_adamw(ctx_, (int)dtype, param->ptr(), grad->ptr(), moment1->ptr(), moment2->ptr(), beta1, beta2, eps,
+                   weightDecay, lr, step, count, r.param->ptr(), r.moment1->ptr(), r.moment2->ptr()));
+    return r;
   }
   Data when(const BroadcastData& mask, const BroadcastData& a, const BroadcastData& b, DType dtype) {  // :633
     Data out = allocate(mask.strides.count() * byteSize(dtype));

@@ -372,6 +372,121 @@ open class HIPBackend: CPUBackend, @unchecked Sendable {
         upper ? 1 : 0, Int64(offset)))
     return out
   }
+
+  // MARK: - backward pass and optimizer
+
+  override open func scatter(
+    _ a: Tensor.Data, _ s: ScatterGatherIndices, dtype: Tensor.DType
+  ) async throws -> Tensor.Data {
+    guard dtype != .bool else { return try await super.scatter(a, s, dtype: dtype) }
+    let (da, di) = (try await device(a), try await device(s.indices.data))
+    var st = hcStrides(s.indices.strides)
+    let out = try output(s.gatherInCount * dtype.byteSize)
+    let axis = s.axis
+    try check(
+      hc_scatter(
+        ctx, hcDType(dtype), da.pointer, di.pointer, &st, out.pointer,
+        Int64(s.valueShape[..<axis].product()), Int64(s.valueShape[axis]),
+        Int64(s.indices.strides.shape[axis]), Int64(s.valueShape[(axis + 1)...].product()),
+        s.indicesAreUnique ? 1 : 0))
+    return out
+  }
+
+  override open func logSoftmaxGrad(
+    _ a: Tensor.Data, _ outGrad: Tensor.Data, dims: ReduceDims, dtype: Tensor.DType
+  ) async throws -> Tensor.Data {
+    guard dtype == .float16 || dtype == .float32 else {
+      return try await super.logSoftmaxGrad(a, outGrad, dims: dims, dtype: dtype)
+    }
+    let (da, dg) = (try await device(a), try await device(outGrad))
+    let out = try output(dims.inCount * dtype.byteSize)
+    try check(
+      hc_log_softmax_grad(
+        ctx, hcDType(dtype), da.pointer, dg.pointer, out.pointer, Int64(dims.outerCount),
+        Int64(dims.reduceCount), Int64(dims.innerCount)))
+    return out
+  }
+
+  override open func clamp<T: NumericTensorElement>(
+    _ a: BroadcastData, _: T.Type, min: TensorOrScalar<T>?, max: TensorOrScalar<T>?,
+    dtype: Tensor.DType
+  ) async throws -> Tensor.Data {
+    guard dtype != .bool else { return try await super.clamp(a, T.self, min: min, max: max, dtype: dtype) }
+    // a scalar bound becomes a 1-element constant with all-zero strides
+    func bound(_ x: TensorOrScalar<T>?) async throws -> (HIPData, hc_strides)? {
+      guard let x = x else { return nil }
+      switch x {
+      case .tensor(let t): return (try await device(t.data), hcStrides(t.strides))
+      case .scalar(let v, let shape):
+        let c = try await constant(v, count: 1, dtype: dtype)
+        return (
+          try await device(c),
+          hcStrides(BroadcastStrides(shape: shape, strides: [Int](repeating: 0, count: shape.count)))
+        )
+      }
+    }
+    let da = try await device(a.data)
+    var sa = hcStrides(a.strides)
+    let lo = try await bound(min)
+    let hi = try await bound(max)
+    var (sl, sh) = (lo?.1 ?? sa, hi?.1 ?? sa)
+    let out = try output(a.strides.shape.product() * dtype.byteSize)
+    try withUnsafePointer(to: &sl) { pl in
+      try withUnsafePointer(to: &sh) { ph in
+        try check(
+          hc_clamp(
+            ctx, hcDType(dtype), da.pointer, &sa, lo?.0.pointer, lo == nil ? nil : pl, hi?.0.pointer,
+            hi == nil ? nil : ph, out.pointer))
+      }
+    }
+    return out
+  }
+
+  /// One fused kernel with the arithmetic of the base-class composition (Backend.swift:818-892).
+  override open func adamW(
+    param: Tensor.Data, grad: Tensor.Data, moment1: Tensor.Data, moment2: Tensor.Data,
+    beta1: Float, beta2: Float, eps: Float, weightDecay: Float, lr: Float, step: Float, count: Int,
+    dtype: Tensor.DType
+  ) async throws -> (param: Tensor.Data, moment1: Tensor.Data, moment2: Tensor.Data) {
+    guard dtype == .float16 || dtype == .float32 else {
+      return try await super.adamW(
+        param: param, grad: grad, moment1: moment1, moment2: moment2, beta1: beta1, beta2: beta2,
+        eps: eps, weightDecay: weightDecay, lr: lr, step: step, count: count, dtype: dtype)
+    }
+    let (dp, dg) = (try await device(param), try await device(grad))
+    let (d1, d2) = (try await device(moment1), try await device(moment2))
+    let bytes = count * dtype.byteSize
+    let (op, o1, o2) = (try output(bytes), try output(bytes), try output(bytes))
+    try check(
+      hc_adamw(
+        ctx, hcDType(dtype), dp.pointer, dg.pointer, d1.pointer, d2.pointer, beta1, beta2, eps,
+        weightDecay, lr, step, count, op.pointer, o1.pointer, o2.pointer))
+    return (param: op, moment1: o1, moment2: o2)
+  }
+
+  // MARK: - recording and replay (no counterpart in Honeycrisp)
+
+  /// A recorded sequence of backend calls; `launch()` replays all of them with one call.
+  public final class Graph {
+    let backend: HIPBackend
+    let handle: OpaquePointer
+    init(backend: HIPBackend, handle: OpaquePointer) { (self.backend, self.handle) = (backend, handle) }
+    public func launch() throws { try backend.check(hc_graph_launch(backend.ctx, handle)) }
+    deinit { _ = hc_graph_destroy(backend.ctx, handle) }
+  }
+
+  /// Runs `body` with every backend call recorded instead of executed. Inputs must already be
+  /// on the device; tensors created inside keep their buffers reserved for the graph.
+  public func capture(_ body: () async throws -> Void) async throws -> Graph {
+    try check(hc_capture_begin(ctx))
+    do { try await body() } catch {
+      _ = hc_capture_abort(ctx)
+      throw error
+    }
+    var handle: OpaquePointer?
+    try check(hc_capture_end(ctx, &handle))
+    return Graph(backend: self, handle: handle!)
+  }
 }
 
 // Enum orders match include/hchip.h by construction of that header.
