@@ -1240,6 +1240,13 @@ extern "C" int hc_gather(hc_ctx* ctx, int dtype, const void* in, const void* ind
     const void* ptrs[] = {indices};
     HC_TRY(make_bcast(1, ops, ptrs, out, 1, &k.idx, &vec, &rows));
     char name[64];
+    if (vb == 16 && k.row_vecs % 64 == 0) {
+      // long rows: one wave per 64 (or 256) vectors of a row
+      const uint32_t t = k.row_vecs % 256 == 0 ? 4 : 1;
+      snprintf(name, sizeof(name), "hc_gather_rows_wide%u", t);
+      const uint64_t units = (uint64_t)k.total_rows * (k.row_vecs / (64 * t));
+      return launch(ctx, name, ceil_div(units, HCK_BLOCK / 64), 1, &k, sizeof(k));
+    }
     snprintf(name, sizeof(name), "hc_gather_rows_b%zu", vb);
     return launch(ctx, name, ceil_div((uint64_t)k.total_rows * k.row_vecs, HCK_BLOCK), 1, &k, sizeof(k));
   }

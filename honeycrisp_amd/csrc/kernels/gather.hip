@@ -26,6 +26,33 @@ template <typename V> __device__ __forceinline__ void gather_rows_impl(const hck
 
 struct alignas(16) V16 { uint32_t x[4]; };
 
+// Long rows (a multiple of 64 * T vectors): one wave moves 64 * T consecutive vectors of one
+// row. The row index is wave-uniform, so it is fetched once per wave, and every lane has T
+// independent 16-byte loads in flight.
+template <int T> __device__ __forceinline__ void gather_rows_wide_impl(const hck_gather_rows_args& p) {
+  const uint32_t units_per_row = p.row_vecs / (64 * T);
+  const uint64_t unit = (uint64_t)blockIdx.x * (HCK_BLOCK / 64) + (threadIdx.x >> 6);
+  const uint32_t row = __builtin_amdgcn_readfirstlane((uint32_t)(unit / units_per_row));
+  if (row >= p.total_rows) return;
+  const uint32_t chunk = __builtin_amdgcn_readfirstlane((uint32_t)(unit - (uint64_t)row * units_per_row));
+  uint32_t off[1];
+  size_t unused;
+  bcast_offsets<1, 1>(p.idx, row, off, unused);
+  const int64_t idx = p.indices[off[0]];
+  const uint32_t i = row / p.out_count;
+  const int64_t src_row = (int64_t)i * p.middle + idx;
+  const uint32_t c = chunk * (64 * T) + (threadIdx.x & 63);
+  const V16* src = (const V16*)p.in + src_row * (int64_t)p.row_vecs + c;
+  V16* dst = (V16*)p.out + (uint64_t)row * p.row_vecs + c;
+  V16 v[T];
+#pragma unroll
+  for (int t = 0; t < T; t++) v[t] = src[t * 64];
+#pragma unroll
+  for (int t = 0; t < T; t++) dst[t * 64] = v[t];
+}
+HC_KERNEL void hc_gather_rows_wide4(hck_gather_rows_args p) { gather_rows_wide_impl<4>(p); }
+HC_KERNEL void hc_gather_rows_wide1(hck_gather_rows_args p) { gather_rows_wide_impl<1>(p); }
+
 HC_KERNEL void hc_gather_rows_b16(hck_gather_rows_args p) { gather_rows_impl<V16>(p); }
 HC_KERNEL void hc_gather_rows_b8(hck_gather_rows_args p) { gather_rows_impl<uint64_t>(p); }
 HC_KERNEL void hc_gather_rows_b4(hck_gather_rows_args p) { gather_rows_impl<uint32_t>(p); }

@@ -91,7 +91,19 @@ __device__ __forceinline__ void reduce_rows_impl(const hck_reduce_args& p) {
     C acc = reduce_identity<OP, C>();
     if (active) {
       if (vec_ok) {
-        for (uint32_t k = lane * VEC; k < n; k += LANES * VEC) {
+        // four independent 16-byte loads in flight per lane, combined in index order
+        constexpr uint32_t STEP = LANES * VEC;
+        uint32_t k = lane * VEC;
+        for (; k + 3 * STEP < n; k += 4 * STEP) {
+          T a[4][VEC];
+#pragma unroll
+          for (int u = 0; u < 4; u++) load_vec<T, VEC>(in, k + u * STEP, 1, a[u]);
+#pragma unroll
+          for (int u = 0; u < 4; u++)
+#pragma unroll
+            for (int i = 0; i < VEC; i++) acc = reduce_combine<OP, C>(acc, to_arith(a[u][i]));
+        }
+        for (; k < n; k += STEP) {
           T a[VEC];
           load_vec<T, VEC>(in, k, 1, a);
 #pragma unroll
@@ -113,7 +125,23 @@ __device__ __forceinline__ void reduce_rows_impl(const hck_reduce_args& p) {
     arg_init<OP>(best);
     if (active) {
       if (vec_ok) {
-        for (uint32_t k = lane * VEC; k < n; k += LANES * VEC) {
+        constexpr uint32_t STEP = LANES * VEC;
+        uint32_t k = lane * VEC;
+        for (; k + 3 * STEP < n; k += 4 * STEP) {
+          T a[4][VEC];
+#pragma unroll
+          for (int u = 0; u < 4; u++) load_vec<T, VEC>(in, k + u * STEP, 1, a[u]);
+#pragma unroll
+          for (int u = 0; u < 4; u++)
+#pragma unroll
+            for (int i = 0; i < VEC; i++) {
+              ArgPair<C> c;
+              c.v = arg_key<OP>(to_arith(a[u][i]), k + u * STEP + i);
+              c.i = k + u * STEP + i;
+              best = arg_better<OP>(best, c);
+            }
+        }
+        for (; k < n; k += STEP) {
           T a[VEC];
           load_vec<T, VEC>(in, k, 1, a);
 #pragma unroll
