@@ -58,6 +58,7 @@ struct hc_ctx {
   std::unordered_map<void*, size_t> live;
   size_t bytes_in_use = 0, bytes_cached = 0;
   hipDeviceProp_t props;
+  void* zeros = nullptr;                              // 256 zero bytes (GEMM edge kernels)
   hc_graph* capturing = nullptr;                      // the recording in progress, if any
   std::unordered_map<void*, hc_graph*> block_owner;   // blocks reserved for a graph
   std::vector<hc_graph*> graphs;
@@ -143,6 +144,11 @@ extern "C" int hc_init(int device, hc_ctx** out) {
   if (s == HC_OK) s = load_image(ctx, hc_image_gemm, hc_image_gemm_end, "gemm");
   if (s == HC_OK) s = load_image(ctx, hc_image_gemm_f16_fast, hc_image_gemm_f16_fast_end, "gemm_f16_fast");
   if (s == HC_OK) s = load_image(ctx, hc_image_gemm_dma, hc_image_gemm_dma_end, "gemm_dma");
+  if (s == HC_OK) {
+    hipError_t e = hipMalloc(&ctx->zeros, 256);
+    if (e == hipSuccess) e = hipMemset(ctx->zeros, 0, 256);
+    if (e != hipSuccess) s = hip_fail(e, "zero buffer");
+  }
   if (s != HC_OK) {
     hc_shutdown(ctx);
     return s;
@@ -171,6 +177,7 @@ extern "C" void hc_shutdown(hc_ctx* ctx) {
   for (auto& kv : ctx->free_blocks)
     for (void* p : kv.second) (void)hipFree(p);
   for (auto& kv : ctx->live) (void)hipFree(kv.first);
+  if (ctx->zeros) (void)hipFree(ctx->zeros);
   for (hipModule_t m : ctx->modules) (void)hipModuleUnload(m);
   if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
   delete ctx;
@@ -1514,32 +1521,41 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
   char ma = mode(k.a, a_rs, a_cs, k.a_bs);
   char mb = mode(k.b, b_cs, b_rs, k.b_bs);
   char name[64];
-  // Tuned kernels: whole tiles only, K in whole 64-byte slices. HCHIP_GEMM_TILE=general|<BM>x<BN>
-  // overrides the choice and HCHIP_GEMM_KERNEL=staged selects the register-staged fp16
-  // pipeline (measurements). The direct-to-LDS kernels address operands with 32-bit byte
-  // offsets.
+  // Tuned kernels. Direct-to-LDS (fp16, fp32): rows of A, B and C 16-byte aligned, operands
+  // addressed with 32-bit byte offsets; ragged M, N, K run the "_e" variants (clamped rows,
+  // zero-filled K tail, predicated stores). HCHIP_GEMM_TILE=general|<BM>x<BN> overrides the
+  // tile choice and HCHIP_GEMM_KERNEL=staged selects the register-staged fp16 pipeline
+  // (whole tiles, K % 64 == 0), both for measurements.
   uint32_t bm = 0, bn = 0;
+  bool edge = false;
   const char* which = getenv("HCHIP_GEMM_KERNEL");
   const uint64_t max_elems = 0xffffffffull / el;
   const bool dma = k.a_bs <= max_elems && k.b_bs <= max_elems && !(which && strcmp(which, "staged") == 0);
-  if ((dtype == HC_F16 || dma) && ma != 'x' && mb != 'x' && K > 0 && K % (64 / el) == 0 && aligned16(out)) {
+  const uint32_t slice = (uint32_t)(64 / el);
+  const bool eligible = ma != 'x' && mb != 'x' && K > 0 && aligned16(out) &&
+                        (dma ? (N % P == 0 && (batch <= 1 || k.c_bs % P == 0)) : (dtype == HC_F16 && K % 64 == 0));
+  if (eligible) {
     const char* force = getenv("HCHIP_GEMM_TILE");
-    auto fits = [&](uint32_t tm, uint32_t tn) { return M % tm == 0 && N % tn == 0; };
+    auto whole = [&](uint32_t tm, uint32_t tn) { return M % tm == 0 && N % tn == 0 && K % slice == 0; };
     // largest tile first; the direct-to-LDS kernels also come in narrow shapes
     static const uint32_t tiles[][2] = {{256, 256}, {256, 128}, {128, 128}, {256, 64}, {128, 64}, {64, 64}};
     const uint64_t cus = (uint64_t)ctx->props.multiProcessorCount;
     if (force && *force) {
       unsigned fm = 0, fn = 0;
-      if (sscanf(force, "%ux%u", &fm, &fn) == 2 && fits(fm, fn)) {
-        bm = fm;
-        bn = fn;
+      if (sscanf(force, "%ux%u", &fm, &fn) == 2 && (dma || whole(fm, fn))) {
+        bool known = false;
+        for (auto& t : tiles) known = known || (t[0] == fm && t[1] == fn);
+        if (known) {
+          bm = fm;
+          bn = fn;
+        }
       }
     } else {
       // the largest tile that still gives every CU a block, else the one with most blocks
       uint64_t best_blocks = 0;
       for (auto& t : tiles) {
-        if (!fits(t[0], t[1]) || (!dma && t[1] < 128)) continue;
-        const uint64_t blocks = (uint64_t)(M / t[0]) * (N / t[1]) * (uint64_t)batch;
+        if (!dma && (!whole(t[0], t[1]) || t[1] < 128)) continue;
+        const uint64_t blocks = ceil_div(M, t[0]) * ceil_div(N, t[1]) * (uint64_t)batch;
         if (blocks >= cus) {
           bm = t[0];
           bn = t[1];
@@ -1552,11 +1568,12 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
         }
       }
     }
-    if (!dma && (K % 64 != 0 || bn < 128)) bm = bn = 0;  // the staged kernels step K by 64
+    if (bm != 0) edge = !whole(bm, bn);
   }
   if (bm != 0) {
-    k.tiles_m = M / bm;
-    k.tiles_n = N / bn;
+    k.tiles_m = (uint32_t)ceil_div(M, bm);
+    k.tiles_n = (uint32_t)ceil_div(N, bn);
+    k.zeros = ctx->zeros;
     if (dma && !getenv("HCHIP_GEMM_BAND")) {
       // largest XCD rectangle whose super-block (4 x 2 XCDs) divides the tile grid
       static const uint32_t shapes[][2] = {{4, 8}, {2, 4}, {1, 2}};
@@ -1568,8 +1585,8 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
           break;
         }
     }
-    snprintf(name, sizeof(name), "hc_gemm_%s_%s_%ux%u_%c%c", dtype_name(dtype), dma ? "dma" : "fast", bm, bn,
-             ma == 'k' ? 'k' : 'm', mb == 'k' ? 'k' : 'n');
+    snprintf(name, sizeof(name), "hc_gemm_%s_%s_%ux%u_%c%c%s", dtype_name(dtype), dma ? "dma" : "fast", bm, bn,
+             ma == 'k' ? 'k' : 'm', mb == 'k' ? 'k' : 'n', edge ? "_e" : "");
   } else if (ma == 'x' || mb == 'x')
     snprintf(name, sizeof(name), "hc_gemm_%s_xx", dtype_name(dtype));
   else

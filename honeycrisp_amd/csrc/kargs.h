@@ -167,6 +167,7 @@ typedef struct {
    * (8/xcd_gn * xcd_sm) x (xcd_gn * xcd_sn) tiles, visited one after the other; inside one,
    * the 8 XCDs form an (8/xcd_gn) x xcd_gn grid and each owns xcd_sm x xcd_sn tiles. */
   uint32_t xcd_gn, xcd_sm, xcd_sn;
+  const void* zeros; /* 16 zero bytes in device memory (edge kernels: source of the K tail) */
 } hck_gemm_args;
 
 #endif

@@ -95,7 +95,10 @@ template <typename T, int ROWS, int MODE> struct DmaOperand {
   uint32_t kstride;      // bytes per unit of k
   uint32_t raddr[NADDR]; // byte offsets (inside the operand's LDS region) of the MFMA operand reads
 
-  __device__ __forceinline__ void init(uint32_t rs, uint32_t cs, uint32_t r0, uint32_t woff) {
+  // `limit` (edge kernels): extent of this operand along M / N. Rows or 16-byte pieces past it
+  // are fetched from the last valid row / piece instead: they only feed outputs that are
+  // never stored. 0 = no clamping.
+  __device__ __forceinline__ void init(uint32_t rs, uint32_t cs, uint32_t r0, uint32_t woff, uint32_t limit) {
     const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     if (MODE == DMA_K) {
       kstride = ES;
@@ -103,7 +106,9 @@ template <typename T, int ROWS, int MODE> struct DmaOperand {
       for (int i = 0; i < NI; i++) {
         const uint32_t row = (wave * NI + i) * 16 + lane / 4;
         const uint32_t c = (lane % 4) ^ swz_k(row);
-        goff[i] = (r0 + row) * rs * ES + c * 16;
+        uint32_t grow = r0 + row;
+        if (limit && grow >= limit) grow = limit - 1;
+        goff[i] = grow * rs * ES + c * 16;
       }
       const uint32_t lrow = lane & 31, lgrp = lane >> 5;
 #pragma unroll
@@ -122,7 +127,9 @@ template <typename T, int ROWS, int MODE> struct DmaOperand {
       for (int i = 0; i < NI; i++) {
         const uint32_t krow = (wave * NI + i) * KPI + lane / PIECES;
         const uint32_t piece = (lane % PIECES) ^ (((krow >> 2) & 1u) << 3);
-        goff[i] = (krow * cs + r0) * ES + piece * 16;
+        uint32_t col = r0 + piece * 4;
+        if (limit && col + 4 > limit) col = limit - 4;
+        goff[i] = (krow * cs + col) * ES;
       }
       const uint32_t lrow = lane & 31, lgrp = lane >> 5;
 #pragma unroll
@@ -138,7 +145,9 @@ template <typename T, int ROWS, int MODE> struct DmaOperand {
       for (int i = 0; i < NI; i++) {
         const uint32_t krow = (wave * NI + i) * KPI + lane / SLOTS_PER_ROW;
         const uint32_t slot = (lane % SLOTS_PER_ROW) ^ (swz_mn(krow) & (SLOTS_PER_ROW - 1));
-        goff[i] = (krow * cs + r0 + slot * 8) * 2;
+        uint32_t col = r0 + slot * 8;
+        if (limit && col + 8 > limit) col = limit - 8;
+        goff[i] = (krow * cs + col) * 2;
       }
       const uint32_t j = lane >> 4, r16 = lane & 15;
 #pragma unroll
@@ -153,10 +162,27 @@ template <typename T, int ROWS, int MODE> struct DmaOperand {
     }
   }
 
+  // k offset, inside a K-slice, of the piece this lane fetches with DMA instruction i
+  __device__ __forceinline__ uint32_t klocal(int i) const {
+    const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    if (MODE == DMA_K) {
+      const uint32_t row = (wave * NI + i) * 16 + lane / 4;
+      return ((lane % 4) ^ swz_k(row)) * (16 / ES);
+    }
+    constexpr uint32_t PER_ROW = ROWB / 16, KPI = 1024 / ROWB;
+    return (wave * NI + i) * KPI + lane / PER_ROW;
+  }
+
   // DMA instruction i of this wave for the K-slice starting at k0: 1 KiB into `region`.
-  __device__ __forceinline__ void dma(int i, const T* base, uint32_t k0, char* region) const {
+  // Edge kernels (kend != 0): pieces at k >= kend come from `zeros` (16 zero bytes) instead,
+  // so the ragged last slice contributes nothing.
+  __device__ __forceinline__ void dma(int i, const T* base, uint32_t k0, char* region, uint32_t kend = 0,
+                                      const void* zeros = nullptr) const {
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const char* src = (const char*)base + (size_t)k0 * kstride + goff[i];
+    if (kend != 0 && k0 + 64 / ES > kend) {  // wave-uniform
+      if (k0 + klocal(i) >= kend) src = (const char*)zeros;
+    }
     __builtin_amdgcn_global_load_lds((const GLOBAL_AS void*)src, (LDS_AS void*)(region + (wave * NI + i) * 1024), 16, 0, 0);
   }
 
@@ -181,7 +207,7 @@ template <typename T, int ROWS, int MODE> struct DmaOperand {
   }
 };
 
-template <typename T, int BM, int BN, int MODE_A, int MODE_B>
+template <typename T, int BM, int BN, int MODE_A, int MODE_B, bool EDGE>
 __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0, char* lds1, char* lds2, char* lds3) {
   constexpr int MT = BM / 64, NT = BN / 64;
   constexpr int SLOTS = MT * NT;
@@ -231,8 +257,9 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
 
   OpA oa;
   OpB ob;
-  oa.init(p.a_rs, p.a_cs, m0, wm);
-  ob.init(p.b_cs, p.b_rs, n0, wn);
+  oa.init(p.a_rs, p.a_cs, m0, wm, EDGE ? p.M : 0);
+  ob.init(p.b_cs, p.b_rs, n0, wn, EDGE ? p.N : 0);
+  const uint32_t kend = EDGE ? p.K : 0;
 
   struct Frags {
     Chunk a[MT];
@@ -247,8 +274,8 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
   // unit u of the DMA of the K-slice starting at k0
   auto dma_unit = [&](int u, uint32_t k0, char* stage, bool in_loop = false) {
     if ((HC_EXP & 1) && in_loop) return;
-    if (u < OpA::NI) oa.dma(u, A, k0, stage);
-    else if (u < NDMA) ob.dma(u - OpA::NI, B, k0, stage + A_BYTES);
+    if (u < OpA::NI) oa.dma(u, A, k0, stage, kend, p.zeros);
+    else if (u < NDMA) ob.dma(u - OpA::NI, B, k0, stage + A_BYTES, kend, p.zeros);
   };
   // MFMA t of a sub-step; operands swapped (B first) so that a lane holds four consecutive
   // n for one m (see the epilogue).
@@ -273,7 +300,7 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
   constexpr int DSTRIDE = SLOTS / (NDMA - HALF) > 0 ? SLOTS / (NDMA - HALF) : 1;
   static_assert(DSTRIDE * (NDMA - HALF) <= SLOTS, "more DMA instructions than MFMA slots");
 
-  const uint32_t nk = p.K / BK;
+  const uint32_t nk = (p.K + BK - 1) / BK;
   Frags f0, f1;
 
   // K-step j out of `cur`; `nxt` holds K-step j+1, `prev` held K-step j-1.
@@ -377,7 +404,8 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
     for (uint32_t it = 0; it < 32 / RPI; it++) {
       const uint32_t r = it * RPI + lane / UNITS, u = lane % UNITS;
       const Chunk v = *reinterpret_cast<const Chunk*>(slab + r * RB + ((u ^ unit_swz(r)) * 16));
-      *reinterpret_cast<Chunk*>(C + (size_t)(m0 + wm + i * 32 + r) * p.c_rs + n0 + wn + u * (16 / ES)) = v;
+      const uint32_t row = m0 + wm + i * 32 + r, col = n0 + wn + u * (16 / ES);
+      if (!EDGE || (row < p.M && col < p.N)) *reinterpret_cast<Chunk*>(C + (size_t)row * p.c_rs + col) = v;
     }
     asm volatile("" ::: "memory");
   }
@@ -391,6 +419,8 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
 #endif
 }
 
+// Two variants per kernel: whole tiles only, and "_e" (edge) for M, N that are not multiples of
+// the tile and K that is not a multiple of the K-slice.
 #define DEF_DMA(T, TN, BM, BN, AN, AM, BNAME, BMODE)                                                  \
   extern "C" __global__ __launch_bounds__(256) void hc_gemm_##TN##_dma_##BM##x##BN##_##AN##BNAME(     \
       hck_gemm_args p) {                                                                              \
@@ -398,7 +428,15 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
     __shared__ __attribute__((aligned(1024))) char lds1[(BM + BN) * 64];                              \
     __shared__ __attribute__((aligned(1024))) char lds2[(BM + BN) * 64];                              \
     __shared__ __attribute__((aligned(1024))) char lds3[(BM + BN) * 64];                              \
-    gemm_dma_impl<T, BM, BN, AM, BMODE>(p, lds0, lds1, lds2, lds3);                                   \
+    gemm_dma_impl<T, BM, BN, AM, BMODE, false>(p, lds0, lds1, lds2, lds3);                            \
+  }                                                                                                   \
+  extern "C" __global__ __launch_bounds__(256) void hc_gemm_##TN##_dma_##BM##x##BN##_##AN##BNAME##_e( \
+      hck_gemm_args p) {                                                                              \
+    __shared__ __attribute__((aligned(1024))) char lds0[(BM + BN) * 64];                              \
+    __shared__ __attribute__((aligned(1024))) char lds1[(BM + BN) * 64];                              \
+    __shared__ __attribute__((aligned(1024))) char lds2[(BM + BN) * 64];                              \
+    __shared__ __attribute__((aligned(1024))) char lds3[(BM + BN) * 64];                              \
+    gemm_dma_impl<T, BM, BN, AM, BMODE, true>(p, lds0, lds1, lds2, lds3);                             \
   }
 #define DEF_DMA_TILE(T, TN, BM, BN)                                                                   \
   DEF_DMA(T, TN, BM, BN, k, DMA_K, k, DMA_K)                                                          \
