@@ -1521,6 +1521,70 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
   char ma = mode(k.a, a_rs, a_cs, k.a_bs);
   char mb = mode(k.b, b_cs, b_rs, k.b_bs);
   char name[64];
+
+  // Operands whose rows are not 16-byte aligned (odd extents, odd base addresses) would fall
+  // to scalar loads; for anything but tiny products it pays to re-pitch them first: a copy
+  // with the leading dimension rounded up to 16 bytes, zero-filled, and likewise a padded
+  // output that is copied back at the end. The tuned kernels then run on the copies.
+  Scratch scratch(ctx);
+  void* c_padded = nullptr;
+  uint32_t c_ld = N;
+  const bool c_unaligned = !aligned16(out) || N % P != 0;
+  const double work = (double)M * (double)N * (double)K * (double)batch;
+  if ((ma == 'x' || mb == 'x' || c_unaligned) && K > 0 && work >= 16777216.0 && batch <= 65535 &&
+      !getenv("HCHIP_GEMM_NO_REPITCH")) {
+    auto round_up = [&](uint32_t v) { return (v + P - 1) / P * P; };
+    // (rows, k) element at rows*rs + k*cs with one of the strides 1 (dense storage)
+    auto repitch = [&](const void*& ptr, uint32_t& rs, uint32_t& cs, uint64_t& bs, uint32_t extent) -> int {
+      const bool k_contig = cs == 1;
+      const uint32_t nrows = k_contig ? extent : K, ncols = k_contig ? K : extent;
+      const uint32_t ld = round_up(ncols);
+      void* copy = nullptr;
+      HC_TRY(scratch.get((size_t)batch * nrows * ld * el, &copy));
+      hck_copy2d_args c;
+      memset(&c, 0, sizeof(c));
+      c.in = ptr;
+      c.out = copy;
+      c.rows = nrows;
+      c.in_cols = ncols;
+      c.out_cols = ld;
+      c.in_ld = k_contig ? rs : cs;
+      c.out_ld = ld;
+      c.in_bs = bs;
+      c.out_bs = (uint64_t)nrows * ld;
+      const uint64_t waves = (uint64_t)nrows * ceil_div(ld, 512);  // a wave moves 64 * 8 elements
+      HC_TRY(launch(ctx, el == 2 ? "hc_copy2d_b2" : "hc_copy2d_b4", ceil_div(waves, HCK_BLOCK / 64), (uint32_t)batch,
+                    &c, sizeof(c)));
+      ptr = copy;
+      (k_contig ? rs : cs) = ld;
+      bs = c.out_bs;
+      return HC_OK;
+    };
+    if (ma == 'x') {
+      HC_TRY(repitch(k.a, a_rs, a_cs, k.a_bs, M));
+      ma = mode(k.a, a_rs, a_cs, k.a_bs);
+    }
+    if (mb == 'x') {
+      HC_TRY(repitch(k.b, b_cs, b_rs, k.b_bs, N));
+      mb = mode(k.b, b_cs, b_rs, k.b_bs);
+    }
+    if (c_unaligned) {
+      c_ld = round_up(N);
+      HC_TRY(scratch.get((size_t)batch * M * c_ld * el, &c_padded));
+      k.c = c_padded;
+      k.c_rs = c_ld;
+      k.c_bs = (uint64_t)M * c_ld;
+    }
+    k.a_rs = a_rs;
+    k.a_cs = a_cs;
+    k.b_rs = b_rs;
+    k.b_cs = b_cs;
+  }
+  // what an edge kernel may fetch: all rows of a K-contiguous operand, whole 16-byte pieces of
+  // an M/N-contiguous one (its leading dimension covers them)
+  k.a_lim = ma == 'k' ? M : (M + P - 1) / P * P;
+  k.b_lim = mb == 'k' ? N : (N + P - 1) / P * P;
+
   // Tuned kernels. Direct-to-LDS (fp16, fp32): rows of A, B and C 16-byte aligned, operands
   // addressed with 32-bit byte offsets; ragged M, N, K run the "_e" variants (clamped rows,
   // zero-filled K tail, predicated stores). HCHIP_GEMM_TILE=general|<BM>x<BN> overrides the
@@ -1532,8 +1596,8 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
   const uint64_t max_elems = 0xffffffffull / el;
   const bool dma = k.a_bs <= max_elems && k.b_bs <= max_elems && !(which && strcmp(which, "staged") == 0);
   const uint32_t slice = (uint32_t)(64 / el);
-  const bool eligible = ma != 'x' && mb != 'x' && K > 0 && aligned16(out) &&
-                        (dma ? (N % P == 0 && (batch <= 1 || k.c_bs % P == 0)) : (dtype == HC_F16 && K % 64 == 0));
+  const bool eligible = ma != 'x' && mb != 'x' && K > 0 && aligned16(k.c) &&
+                        (dma ? (k.c_rs % P == 0 && (batch <= 1 || k.c_bs % P == 0)) : (dtype == HC_F16 && K % 64 == 0));
   if (eligible) {
     const char* force = getenv("HCHIP_GEMM_TILE");
     auto whole = [&](uint32_t tm, uint32_t tn) { return M % tm == 0 && N % tn == 0 && K % slice == 0; };
@@ -1551,17 +1615,30 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
         }
       }
     } else {
-      // the largest tile that still gives every CU a block, else the one with most blocks
+      // Among the tiles that give every CU a block: the best product of (rough per-CU rate of
+      // the tile) x (fraction of the last round of blocks that is busy) x (fraction of the
+      // tiles' area that is real output). If no tile fills the device: the one with most blocks.
+      static const double rate16[] = {1.0, 0.85, 0.7, 0.55, 0.45, 0.3};
+      static const double rate32[] = {1.0, 0.95, 0.85, 0.8, 0.7, 0.55};
+      const double* rate = dtype == HC_F32 ? rate32 : rate16;
       uint64_t best_blocks = 0;
-      for (auto& t : tiles) {
+      double best_score = 0.0;
+      bool filled = false;
+      for (size_t ti = 0; ti < sizeof(tiles) / sizeof(tiles[0]); ti++) {
+        const uint32_t* t = tiles[ti];
         if (!dma && (!whole(t[0], t[1]) || t[1] < 128)) continue;
         const uint64_t blocks = ceil_div(M, t[0]) * ceil_div(N, t[1]) * (uint64_t)batch;
         if (blocks >= cus) {
-          bm = t[0];
-          bn = t[1];
-          break;
-        }
-        if (blocks > best_blocks) {
+          const double rounds = (double)ceil_div(blocks, cus);
+          const double useful = ((double)M * N * (double)batch) / ((double)blocks * t[0] * t[1]);
+          const double score = rate[ti] * ((double)blocks / (rounds * (double)cus)) * useful;
+          if (!filled || score > best_score) {
+            filled = true;
+            best_score = score;
+            bm = t[0];
+            bn = t[1];
+          }
+        } else if (!filled && blocks > best_blocks) {
           best_blocks = blocks;
           bm = t[0];
           bn = t[1];
@@ -1602,6 +1679,23 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
     kk.c = (char*)k.c + (uint64_t)b0 * k.c_bs * el;
     kk.batch = nb;
     HC_TRY(launch(ctx, name, tiles, nb, &kk, sizeof(kk)));
+  }
+  if (c_padded) {
+    // padded result back into the caller's dense [M, N] matrices
+    hck_copy2d_args c;
+    memset(&c, 0, sizeof(c));
+    c.in = c_padded;
+    c.out = out;
+    c.rows = M;
+    c.in_cols = N;
+    c.out_cols = N;
+    c.in_ld = c_ld;
+    c.out_ld = N;
+    c.in_bs = (uint64_t)M * c_ld;
+    c.out_bs = (uint64_t)M * N;
+    const uint64_t waves = (uint64_t)M * ceil_div(N, 512);
+    HC_TRY(launch(ctx, el == 2 ? "hc_copy2d_b2" : "hc_copy2d_b4", ceil_div(waves, HCK_BLOCK / 64), (uint32_t)batch,
+                  &c, sizeof(c)));
   }
   return HC_OK;
 }

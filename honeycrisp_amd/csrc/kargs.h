@@ -168,6 +168,18 @@ typedef struct {
    * the 8 XCDs form an (8/xcd_gn) x xcd_gn grid and each owns xcd_sm x xcd_sn tiles. */
   uint32_t xcd_gn, xcd_sm, xcd_sn;
   const void* zeros; /* 16 zero bytes in device memory (edge kernels: source of the K tail) */
+  /* edge kernels: rows (K-contiguous operand) or elements of a k-row (M/N-contiguous operand,
+   * a multiple of 16 bytes) that may be fetched; anything beyond is clamped to the last one */
+  uint32_t a_lim, b_lim;
 } hck_gemm_args;
+
+/* Copy of a batch of [rows, in_cols] matrices with leading dimension in_ld into [rows, out_cols]
+ * with leading dimension out_ld; columns >= in_cols are written as zero. Element offsets. */
+typedef struct {
+  const void* in;
+  void* out;
+  uint32_t rows, in_cols, out_cols, pad;
+  uint64_t in_ld, out_ld, in_bs, out_bs;
+} hck_copy2d_args;
 
 #endif

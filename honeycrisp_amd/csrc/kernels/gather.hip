@@ -118,6 +118,28 @@ HC_KERNEL void hc_scatter_set_b8(hck_gather_elems_args p) { scatter_set_impl<uin
 HC_KERNEL void hc_scatter_set_b4(hck_gather_elems_args p) { scatter_set_impl<uint32_t>(p); }
 HC_KERNEL void hc_scatter_set_b2(hck_gather_elems_args p) { scatter_set_impl<uint16_t>(p); }
 
+// Re-pitching copy for GEMM operands whose rows are not 16-byte aligned: element-wise
+// accesses (either side may be unaligned), zero beyond the valid columns. A wave owns
+// 64 * G consecutive elements of one row and moves 64 consecutive elements per instruction,
+// so every access is a dense 128- or 256-byte segment. grid.y = batch.
+template <typename V, int G> __device__ __forceinline__ void copy2d_impl(const hck_copy2d_args& p) {
+  const uint32_t groups = (p.out_cols + 64 * G - 1) / (64 * G);
+  const uint64_t unit = (uint64_t)blockIdx.x * (HCK_BLOCK / 64) + (threadIdx.x >> 6);
+  const uint64_t r = unit / groups;
+  if (r >= p.rows) return;
+  const uint32_t c0 = (uint32_t)(unit - r * groups) * (64 * G) + (threadIdx.x & 63);
+  const V* src = (const V*)p.in + (uint64_t)blockIdx.y * p.in_bs + r * p.in_ld;
+  V* dst = (V*)p.out + (uint64_t)blockIdx.y * p.out_bs + r * p.out_ld;
+  V v[G];
+#pragma unroll
+  for (int e = 0; e < G; e++) v[e] = c0 + e * 64 < p.in_cols ? src[c0 + e * 64] : (V)0;
+#pragma unroll
+  for (int e = 0; e < G; e++)
+    if (c0 + e * 64 < p.out_cols) dst[c0 + e * 64] = v[e];
+}
+HC_KERNEL void hc_copy2d_b2(hck_copy2d_args p) { copy2d_impl<uint16_t, 8>(p); }
+HC_KERNEL void hc_copy2d_b4(hck_copy2d_args p) { copy2d_impl<uint32_t, 8>(p); }
+
 // axisPermutation (BackendCPU.swift:1831-1849): flat source index of every element of the
 // permuted view.
 HC_KERNEL void hc_axis_permutation(hck_axis_perm_args p) {

@@ -257,8 +257,8 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
 
   OpA oa;
   OpB ob;
-  oa.init(p.a_rs, p.a_cs, m0, wm, EDGE ? p.M : 0);
-  ob.init(p.b_cs, p.b_rs, n0, wn, EDGE ? p.N : 0);
+  oa.init(p.a_rs, p.a_cs, m0, wm, EDGE ? p.a_lim : 0);
+  ob.init(p.b_cs, p.b_rs, n0, wn, EDGE ? p.b_lim : 0);
   const uint32_t kend = EDGE ? p.K : 0;
 
   struct Frags {

@@ -58,7 +58,9 @@ def rand(rng, shape, dtype, scale=1.0):
 GEMM_SHAPES = [(128, 128, 128), (256, 64, 384), (127, 1000, 65), (1, 33, 1), (5, 4097, 3), (200, 8, 136),
                (64, 0, 16), (129, 257, 131), (512, 192, 384), (1024, 64, 2048), (256, 320, 128),
                # 16-byte aligned rows but ragged against every tile and K-slice: the edge kernels
-               (264, 72, 520), (1000, 1000, 1000), (8, 64, 8), (2040, 520, 1000)]
+               (264, 72, 520), (1000, 1000, 1000), (8, 64, 8), (2040, 520, 1000),
+               # odd extents, large enough to be re-pitched into aligned copies first
+               (1001, 515, 999), (4097, 127, 1000), (333, 4097, 129)]
 
 
 @pytest.mark.parametrize("dtype", [F32, F16], ids=["f32", "f16"])
