@@ -11,8 +11,10 @@ Also reported in the same line:
                 from HIP events recorded on the backend's own stream inside the timed region
   cpu_baseline  the reference CPUBackend algorithm (oracle/cpu_ref.c restatement, the literal
                 single-thread triple loop) timed on this box's host cores on a bounded row slab
-  extra         the other BASELINE configs: fp32 1024^3, attention-shaped batched GEMMs, the
-                bandwidth-bound ops at [8192,4096] with GB/s against the 8 TB/s HBM peak
+  extra         the other BASELINE configs: fp32 1024^3, the ragged fp16 sweep, attention-shaped
+                batched GEMMs, the bandwidth-bound ops at [8192,4096] with GB/s against the 8 TB/s
+                HBM peak (short kernels are timed as graph-replayed batches: device-side duration
+                per launch), and the transformer forward pass, eager and as one graph replay
 
 Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extra] [--no-graph]
 """
@@ -61,10 +63,34 @@ class Events:
         self.lib.hc_event_destroy(ev)
 
 
-def timed_launches(backend, events, fn, iters, warmup):
-    """Average duration (ms) of fn() launches, each bracketed by events on the stream."""
+GRAPH_TIMING = True
+
+
+def timed_launches(backend, events, fn, iters, warmup, batched=False):
+    """Average duration (ms) of fn() launches, each bracketed by events on the stream.
+    batched=True (short kernels): the host cannot enqueue a microsecond-scale kernel as fast as
+    the GPU runs it, so per-launch events would time the host. Instead `iters` launches are
+    recorded once into a graph and the replay is bracketed by two events: device-side duration
+    per launch, launch gaps included."""
     for _ in range(warmup):
         fn()
+    if batched and GRAPH_TIMING:
+        with backend.capture() as cap:
+            for _ in range(iters):
+                fn()
+        cap.graph.launch()
+        ms = []
+        for _ in range(5):
+            a, b = events.new(), events.new()
+            events.record(a)
+            cap.graph.launch()
+            events.record(b)
+            backend.sync()
+            ms.append(events.elapsed_ms(a, b) / iters)
+            events.free(a)
+            events.free(b)
+        cap.graph.destroy()
+        return float(np.mean(ms)), float(np.median(ms))
     pairs = []
     for _ in range(iters):
         a, b = events.new(), events.new()
@@ -190,19 +216,38 @@ def extra_workloads(backend, graph=True):
         x, y = sets[it[0] & 1]
         it[0] += 1
         return backend.matmul(x, False, y, False, False, 1024, 1024, 1024, F32)
-    ms, _ = timed_launches(backend, ev, gemm32, 50, 10)
+    ms, _ = timed_launches(backend, ev, gemm32, 50, 10, batched=True)
     report("cfg1_f32_gemm_1024", ms, flops=2.0 * 1024**3)
     out["cfg1_f32_gemm_1024"]["mfma_frac"] = round(out["cfg1_f32_gemm_1024"]["tflops"] / PEAK_F32_TFLOPS, 4)
+
+    # config 2, the ragged sweep: fp16 NN products with M, N, K in {127, 1000, 4097}; total FLOPs over
+    # total time of the 27 shapes, and the three cubes on their own
+    sizes = (127, 1000, 4097)
+    total_flops, total_ms = 0.0, 0.0
+    rng = np.random.default_rng(20)
+    big = rng.standard_normal(4097 * 4097).astype(np.float16)
+    for m in sizes:
+        for kk in sizes:
+            a_dev = backend.upload(big[:m * kk])
+            for n in sizes:
+                b_dev = backend.upload(big[:kk * n])
+                fn = lambda: backend.matmul(a_dev, False, b_dev, False, False, m, kk, n, F16)
+                ms, _ = timed_launches(backend, ev, fn, 5, 2, batched=True)
+                total_flops += 2.0 * m * kk * n
+                total_ms += ms
+                if m == kk == n:
+                    report("cfg2_ragged_%d_cubed" % m, ms, flops=2.0 * m * kk * n)
+    report("cfg2_ragged_sweep_27_shapes", total_ms, flops=total_flops)
 
     # config 3: attention-shaped batched GEMMs, fp16, batch 32
     q, k, v = [backend.upload(np.random.default_rng(s).standard_normal((32, 512, 64)).astype(np.float16))
                for s in (4, 5, 6)]
     scores = backend.batchedMatmul(32, q, False, k, True, False, 512, 64, 512, F16)
-    ms, _ = timed_launches(backend, ev, lambda: backend.batchedMatmul(32, q, False, k, True, False, 512, 64, 512, F16), 50, 10)
+    ms, _ = timed_launches(backend, ev, lambda: backend.batchedMatmul(32, q, False, k, True, False, 512, 64, 512, F16), 50, 10, batched=True)
     report("cfg3_qk_t", ms, flops=32 * 2.0 * 512 * 64 * 512, nbytes=32 * (2 * 512 * 64 + 512 * 512) * 2)
-    ms, _ = timed_launches(backend, ev, lambda: backend.binaryOp(scores, 0.125, NumericBinaryOp.mul, F16, count=32 * 512 * 512), 50, 10)
+    ms, _ = timed_launches(backend, ev, lambda: backend.binaryOp(scores, 0.125, NumericBinaryOp.mul, F16, count=32 * 512 * 512), 50, 10, batched=True)
     report("cfg3_scale", ms, nbytes=2 * 32 * 512 * 512 * 2)
-    ms, _ = timed_launches(backend, ev, lambda: backend.batchedMatmul(32, scores, False, v, False, False, 512, 512, 64, F16), 50, 10)
+    ms, _ = timed_launches(backend, ev, lambda: backend.batchedMatmul(32, scores, False, v, False, False, 512, 512, 64, F16), 50, 10, batched=True)
     report("cfg3_pv", ms, flops=32 * 2.0 * 512 * 512 * 64, nbytes=32 * (2 * 512 * 64 + 512 * 512) * 2)
 
     # config 4: bandwidth-bound ops at [8192, 4096] fp32
@@ -212,17 +257,17 @@ def extra_workloads(backend, graph=True):
     xs = BroadcastStrides([R, C], [C, 1])
     bs = BroadcastStrides([R, C], [0, 1])
     nb = R * C * 4
-    ms, _ = timed_launches(backend, ev, lambda: backend.binaryOp(BroadcastData(xs, x), BroadcastData(bs, bias), NumericBinaryOp.add, F32), 50, 10)
+    ms, _ = timed_launches(backend, ev, lambda: backend.binaryOp(BroadcastData(xs, x), BroadcastData(bs, bias), NumericBinaryOp.add, F32), 50, 10, batched=True)
     report("cfg4_bias_add", ms, nbytes=2 * nb + C * 4)
     # plain copy of known size (identity broadcast): the calibration kernel for HBM byte counters
-    ms, _ = timed_launches(backend, ev, lambda: backend.broadcast(BroadcastData(xs, x), F32), 50, 10)
+    ms, _ = timed_launches(backend, ev, lambda: backend.broadcast(BroadcastData(xs, x), F32), 50, 10, batched=True)
     report("copy_134MB_calibration", ms, nbytes=2 * nb)
-    ms, _ = timed_launches(backend, ev, lambda: backend.elemwise(x, ElemwiseOp.geluApprox, None, R * C, F32), 50, 10)
+    ms, _ = timed_launches(backend, ev, lambda: backend.elemwise(x, ElemwiseOp.geluApprox, None, R * C, F32), 50, 10, batched=True)
     report("cfg4_gelu", ms, nbytes=2 * nb)
     dims = ReduceDims(R, C, 1)
-    ms, _ = timed_launches(backend, ev, lambda: backend.reduce(x, ReduceOp.sum, dims, F32), 50, 10)
+    ms, _ = timed_launches(backend, ev, lambda: backend.reduce(x, ReduceOp.sum, dims, F32), 50, 10, batched=True)
     report("cfg4_sum_axis1", ms, nbytes=nb + R * 4)
-    ms, _ = timed_launches(backend, ev, lambda: backend.reduce(x, ReduceOp.argmax, dims, F32), 50, 10)
+    ms, _ = timed_launches(backend, ev, lambda: backend.reduce(x, ReduceOp.argmax, dims, F32), 50, 10, batched=True)
     report("cfg4_argmax_axis1", ms, nbytes=nb + R * 8)
     idx = backend.reduce(x, ReduceOp.argmax, dims, F32)
     max_gather = ScatterGatherIndices([R, C], 1, BroadcastData(BroadcastStrides([R, 1], [1, 0]), idx))
@@ -230,12 +275,12 @@ def extra_workloads(backend, graph=True):
     def max_axis1():  # Tensor.max(axis:) = argmax + gather (ReduceRepeat.swift:201-209)
         i = backend.reduce(x, ReduceOp.argmax, dims, F32)
         return backend.gather(x, ScatterGatherIndices([R, C], 1, BroadcastData(BroadcastStrides([R, 1], [1, 0]), i)), F32)
-    ms, _ = timed_launches(backend, ev, max_axis1, 50, 10)
+    ms, _ = timed_launches(backend, ev, max_axis1, 50, 10, batched=True)
     report("cfg4_max_axis1", ms, nbytes=nb + R * 8 + R * 8 + R * 4 + R * 4)
     table = backend.upload(np.random.default_rng(10).standard_normal((32000, 1024)).astype(np.float32))
     ids = backend.upload(np.random.default_rng(9).integers(0, 32000, size=(65536,)))
     emb = ScatterGatherIndices([32000, 1024], 0, BroadcastData(BroadcastStrides([65536, 1024], [1, 0]), ids))
-    ms, _ = timed_launches(backend, ev, lambda: backend.gather(table, emb, F32), 50, 10)
+    ms, _ = timed_launches(backend, ev, lambda: backend.gather(table, emb, F32), 50, 10, batched=True)
     report("cfg4_embedding_gather", ms, nbytes=65536 * 8 + 2 * 65536 * 1024 * 4)
     del max_gather
 
@@ -291,6 +336,8 @@ def main():
               "--gpus %d is not supported" % args.gpus, file=sys.stderr)
         sys.exit(2)
 
+    global GRAPH_TIMING
+    GRAPH_TIMING = not args.no_graph
     from honeycrisp_amd.backend import HIPBackend
     backend = HIPBackend(0)
     info = backend.deviceInfo()
