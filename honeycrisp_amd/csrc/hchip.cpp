@@ -1078,6 +1078,7 @@ extern "C" int hc_log_softmax(hc_ctx* ctx, int dtype, const void* in, void* out,
   HC_TRY(check_dims("hc_log_softmax", outer, reduce, inner));
   if (outer * reduce * inner == 0) return HC_OK;
   REQUIRE(in && out, "hc_log_softmax: null pointer");
+  REQUIRE(aligned16(in) && aligned16(out), "hc_log_softmax: buffers must be 16-byte aligned");
   hck_reduce_args k;
   memset(&k, 0, sizeof(k));
   k.in = in;
@@ -1102,6 +1103,7 @@ extern "C" int hc_log_softmax_grad(hc_ctx* ctx, int dtype, const void* in, const
   HC_TRY(check_dims("hc_log_softmax_grad", outer, reduce, inner));
   if (outer * reduce * inner == 0) return HC_OK;
   REQUIRE(in && out_grad && out, "hc_log_softmax_grad: null pointer");
+  REQUIRE(aligned16(in) && aligned16(out_grad) && aligned16(out), "hc_log_softmax_grad: buffers must be 16-byte aligned");
   hck_reduce_args k;
   memset(&k, 0, sizeof(k));
   k.in = in;
@@ -1141,6 +1143,7 @@ extern "C" int hc_normalize(hc_ctx* ctx, int dtype, const void* in, void* out, i
   HC_TRY(check_dims("hc_normalize", outer, reduce, inner));
   if (outer * reduce * inner == 0) return HC_OK;
   REQUIRE(in && out, "hc_normalize: null pointer");
+  REQUIRE(aligned16(in) && aligned16(out), "hc_normalize: buffers must be 16-byte aligned");
   if (inner == 1) {
     hck_reduce_args k;
     memset(&k, 0, sizeof(k));

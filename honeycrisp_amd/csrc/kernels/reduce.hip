@@ -233,6 +233,56 @@ DEF_REDUCE_T(f32, float)
 DEF_REDUCE_T(f16, half_t)
 DEF_REDUCE_T(i64, int64_t)
 
+// A row of up to 64 * VEC * CHUNKS elements held by one wave in registers: lane l owns the
+// 16-byte vectors l, l + 64, ... of the row (n a multiple of VEC; rows then start 16-byte
+// aligned because the buffer does).
+template <typename T> struct RowRegs {
+  static constexpr int VEC = VecWidth<T>::value;
+  static constexpr int CHUNKS = 4;
+  T v[CHUNKS][VEC];
+  static __device__ __forceinline__ bool fits(uint32_t n) { return n % VEC == 0 && n <= 64u * VEC * CHUNKS; }
+  __device__ __forceinline__ void load(const T* row, uint32_t n, uint32_t lane) {
+#pragma unroll
+    for (int c = 0; c < CHUNKS; c++) {
+      const uint32_t k = (lane + 64 * c) * VEC;
+      if (k < n) load_vec<T, VEC>(row, k, 1, v[c]);
+    }
+  }
+  template <typename F> __device__ __forceinline__ void each(uint32_t n, uint32_t lane, F f) const {
+#pragma unroll
+    for (int c = 0; c < CHUNKS; c++)
+      if ((lane + 64 * c) * VEC < n) {
+#pragma unroll
+        for (int i = 0; i < VEC; i++) f((float)v[c][i]);
+      }
+  }
+  template <typename F> __device__ __forceinline__ void store(T* row, uint32_t n, uint32_t lane, F f) const {
+#pragma unroll
+    for (int c = 0; c < CHUNKS; c++) {
+      const uint32_t k = (lane + 64 * c) * VEC;
+      if (k < n) {
+        T o[VEC];
+#pragma unroll
+        for (int i = 0; i < VEC; i++) o[i] = narrow<T>(f((float)v[c][i]));
+        store_vec<T, VEC>(row, k, o);
+      }
+    }
+  }
+  template <typename F>
+  __device__ __forceinline__ void store2(T* row, uint32_t n, uint32_t lane, const RowRegs& other, F f) const {
+#pragma unroll
+    for (int c = 0; c < CHUNKS; c++) {
+      const uint32_t k = (lane + 64 * c) * VEC;
+      if (k < n) {
+        T o[VEC];
+#pragma unroll
+        for (int i = 0; i < VEC; i++) o[i] = narrow<T>(f((float)v[c][i], (float)other.v[c][i]));
+        store_vec<T, VEC>(row, k, o);
+      }
+    }
+  }
+};
+
 // ---------------------------------------------------------------- logSoftmax
 
 // logSoftmax (BackendCPU.swift:1000-1038): max, sum of expf(x - max), x - (logf(sum) + max),
@@ -246,6 +296,20 @@ template <typename T> __device__ __forceinline__ void log_softmax_rows_impl(cons
   T* out = (T*)p.out + (size_t)row * n;
   // NaNs are skipped by the strict compare here and on the CPU alike; any NaN in the row
   // then turns the exp-sum, and with it the whole row, into NaN on both.
+  if (RowRegs<T>::fits(n)) {
+    // short rows: read once with 16-byte loads, keep the row in registers
+    RowRegs<T> r;
+    r.load(in, n, lane);
+    float m = -INFINITY;
+    r.each(n, lane, [&](float x) { if (x > m) m = x; });
+    m = wave_reduce(m, MaxOp());
+    float s = 0.0f;
+    r.each(n, lane, [&](float x) { s += expf(x - m); });
+    s = wave_reduce(s, SumOp());
+    const float log_sum = logf(s) + m;
+    r.store(out, n, lane, [&](float x) { return x - log_sum; });
+    return;
+  }
   float m = -INFINITY;
   for (uint32_t k = lane; k < n; k += 64) {
     float x = (float)in[k];
@@ -294,6 +358,22 @@ template <typename T> __device__ __forceinline__ void log_softmax_grad_rows_impl
   const T* in = (const T*)p.in + (size_t)row * n;
   const T* grad = (const T*)p.in2 + (size_t)row * n;
   T* out = (T*)p.out + (size_t)row * n;
+  if (RowRegs<T>::fits(n)) {
+    RowRegs<T> r, g;
+    r.load(in, n, lane);
+    g.load(grad, n, lane);
+    float m = -INFINITY, gs = 0.0f;
+    r.each(n, lane, [&](float x) { if (x > m) m = x; });
+    g.each(n, lane, [&](float x) { gs += x; });
+    m = wave_reduce(m, MaxOp());
+    gs = wave_reduce(gs, SumOp());
+    float s = 0.0f;
+    r.each(n, lane, [&](float x) { s += expf(x - m); });
+    s = wave_reduce(s, SumOp());
+    const float log_sum = logf(s) + m;
+    g.store2(out, n, lane, r, [&](float gv, float x) { return gv - gs * expf(x - log_sum); });
+    return;
+  }
   float m = -INFINITY, gs = 0.0f;
   for (uint32_t k = lane; k < n; k += 64) {
     float x = (float)in[k];
@@ -353,6 +433,26 @@ template <typename T> __device__ __forceinline__ void normalize_rows_impl(const 
   const T* in = (const T*)p.in + (size_t)row * n;
   T* out = (T*)p.out + (size_t)row * n;
   const float inv_n = 1.0f / (float)n;
+  if (RowRegs<T>::fits(n)) {
+    RowRegs<T> r;
+    r.load(in, n, lane);
+    float s = 0.0f;
+    r.each(n, lane, [&](float x) { s += x; });
+    s = round_through<T>(wave_reduce(s, SumOp()));
+    const float mean = round_through<T>(s * inv_n);
+    float sq = 0.0f;
+    r.each(n, lane, [&](float x) {
+      const float c = round_through<T>(x - mean);
+      const float c2 = sizeof(T) == 4 ? c * c : 1.0f * 1.0f * powf(c, 2.0f);
+      sq += round_through<T>(c2);
+    });
+    sq = round_through<T>(wave_reduce(sq, SumOp()));
+    const float var = round_through<T>(sq * inv_n);
+    const float shifted = round_through<T>(var + p.eps);
+    const float normer = round_through<T>(1.0f * 1.0f * powf(shifted, -0.5f));
+    r.store(out, n, lane, [&](float x) { return round_through<T>(x - mean) * normer; });
+    return;
+  }
   float s = 0.0f;
   for (uint32_t k = lane; k < n; k += 64) s += (float)in[k];
   s = round_through<T>(wave_reduce(s, SumOp()));
