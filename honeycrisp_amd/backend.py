@@ -283,9 +283,11 @@ class Capture:
 
     def __enter__(self):
         self.backend._check(self.backend._lib.hc_capture_begin(self.backend._ctx))
+        self.backend._capturing = True
         return self
 
     def __exit__(self, exc_type, exc, tb):
+        self.backend._capturing = False
         if exc_type is not None:
             self.backend._lib.hc_capture_abort(self.backend._ctx)
             return False
@@ -300,6 +302,8 @@ class HIPBackend(Backend):
 
     def __init__(self, device: int = 0):
         self._ctx = None
+        self._capturing = False
+        self._perm_cache, self._perm_cache_bytes = {}, 0
         self._lib = _lib.load()
         ctx = c_void_p()
         status = self._lib.hc_init(device, byref(ctx))
@@ -309,6 +313,7 @@ class HIPBackend(Backend):
 
     def close(self):
         if self._ctx:
+            self._perm_cache.clear()
             self._lib.hc_shutdown(self._ctx)
             self._ctx = None
 
@@ -615,12 +620,26 @@ class HIPBackend(Backend):
         self._check(self._lib.hc_concat(self._ctx, int(dtype), ptrs, counts, n, outerCount, c_void_p(out.ptr)))
         return out
 
+    # bytes of permutation index vectors kept for reuse
+    PERMUTATION_CACHE_BYTES = 256 << 20
+
     def axisPermutation(self, permutation: List[int], shape: List[int]) -> HIPData:
+        """The index vector depends on (permutation, shape) only and every permuted view of that
+        shape rebuilds it (Index.swift:238-266), so finished vectors are kept and shared: buffers
+        are never modified after creation. Entries are never evicted (a recorded graph may read
+        them); nothing is added while recording, because a recorded kernel has not run yet."""
+        key = (tuple(permutation), tuple(shape))
+        hit = self._perm_cache.get(key)
+        if hit is not None:
+            return hit
         n = len(shape)
         out = self.allocate(product(shape) * 8)
         perm = (c_int64 * max(n, 1))(*permutation)
         shp = (c_int64 * max(n, 1))(*shape)
         self._check(self._lib.hc_axis_permutation(self._ctx, perm, shp, n, c_void_p(out.ptr)))
+        if not self._capturing and self._perm_cache_bytes + out.byteCount <= self.PERMUTATION_CACHE_BYTES:
+            self._perm_cache[key] = out
+            self._perm_cache_bytes += out.byteCount
         return out
 
 

@@ -259,10 +259,30 @@ open class HIPBackend: CPUBackend, @unchecked Sendable {
     return out
   }
 
+  /// The index vector depends on (permutation, shape) only and every permuted view rebuilds it
+  /// (Index.swift:238-266): finished vectors are kept and shared (buffers are immutable), never
+  /// evicted (a recorded graph may read them), and not added while recording.
+  private struct PermutationKey: Hashable {
+    let permutation: [Int]
+    let shape: [Int]
+  }
+  private var permutationCache: [PermutationKey: HIPData] = [:]
+  private var permutationCacheBytes = 0
+  private let permutationCacheLock = NSLock()
+  var isCapturing = false
+
   override open func axisPermutation(permutation: [Int], shape: [Int]) async throws -> Tensor.Data {
+    let key = PermutationKey(permutation: permutation, shape: shape)
+    if let hit = permutationCacheLock.withLock({ permutationCache[key] }) { return hit }
     let out = try output(shape.product() * Tensor.DType.int64.byteSize)
     let (perm, shp) = (permutation.map { Int64($0) }, shape.map { Int64($0) })
     try check(hc_axis_permutation(ctx, perm, shp, Int32(shape.count), out.pointer))
+    permutationCacheLock.withLock {
+      if !isCapturing && permutationCacheBytes + out.byteCount <= 256 << 20 {
+        permutationCache[key] = out
+        permutationCacheBytes += out.byteCount
+      }
+    }
     return out
   }
 
@@ -479,6 +499,8 @@ open class HIPBackend: CPUBackend, @unchecked Sendable {
   /// on the device; tensors created inside keep their buffers reserved for the graph.
   public func capture(_ body: () async throws -> Void) async throws -> Graph {
     try check(hc_capture_begin(ctx))
+    isCapturing = true
+    defer { isCapturing = false }
     do { try await body() } catch {
       _ = hc_capture_abort(ctx)
       throw error
