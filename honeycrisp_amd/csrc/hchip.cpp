@@ -1079,6 +1079,7 @@ extern "C" int hc_log_softmax(hc_ctx* ctx, int dtype, const void* in, void* out,
   if (outer * reduce * inner == 0) return HC_OK;
   REQUIRE(in && out, "hc_log_softmax: null pointer");
   REQUIRE(aligned16(in) && aligned16(out), "hc_log_softmax: buffers must be 16-byte aligned");
+  const size_t el_size = dtype_size(dtype);
   hck_reduce_args k;
   memset(&k, 0, sizeof(k));
   k.in = in;
@@ -1088,8 +1089,13 @@ extern "C" int hc_log_softmax(hc_ctx* ctx, int dtype, const void* in, void* out,
   k.inner = (uint32_t)inner;
   char name[64];
   if (inner == 1) {
-    snprintf(name, sizeof(name), "hc_log_softmax_rows_%s", dtype_name(dtype));
-    return launch(ctx, name, ceil_div((uint64_t)outer, HCK_BLOCK / 64), 1, &k, sizeof(k));
+    // a wave per row while the row fits its registers (4 x 16 bytes per lane), else a block
+    if ((uint64_t)reduce * el_size <= 64 * 16 * 4) {
+      snprintf(name, sizeof(name), "hc_log_softmax_rows_%s", dtype_name(dtype));
+      return launch(ctx, name, ceil_div((uint64_t)outer, HCK_BLOCK / 64), 1, &k, sizeof(k));
+    }
+    snprintf(name, sizeof(name), "hc_log_softmax_rows256_%s", dtype_name(dtype));
+    return launch(ctx, name, (uint64_t)outer, 1, &k, sizeof(k));
   }
   snprintf(name, sizeof(name), "hc_log_softmax_cols_%s", dtype_name(dtype));
   return launch(ctx, name, ceil_div((uint64_t)inner, HCK_BLOCK) * (uint64_t)outer, 1, &k, sizeof(k));
@@ -1104,6 +1110,7 @@ extern "C" int hc_log_softmax_grad(hc_ctx* ctx, int dtype, const void* in, const
   if (outer * reduce * inner == 0) return HC_OK;
   REQUIRE(in && out_grad && out, "hc_log_softmax_grad: null pointer");
   REQUIRE(aligned16(in) && aligned16(out_grad) && aligned16(out), "hc_log_softmax_grad: buffers must be 16-byte aligned");
+  const size_t el_size = dtype_size(dtype);
   hck_reduce_args k;
   memset(&k, 0, sizeof(k));
   k.in = in;
@@ -1114,8 +1121,13 @@ extern "C" int hc_log_softmax_grad(hc_ctx* ctx, int dtype, const void* in, const
   k.inner = (uint32_t)inner;
   char name[64];
   if (inner == 1) {
-    snprintf(name, sizeof(name), "hc_log_softmax_grad_rows_%s", dtype_name(dtype));
-    return launch(ctx, name, ceil_div((uint64_t)outer, HCK_BLOCK / 64), 1, &k, sizeof(k));
+    // a wave per row while the row fits its registers (4 x 16 bytes per lane), else a block
+    if ((uint64_t)reduce * el_size <= 64 * 16 * 4) {
+      snprintf(name, sizeof(name), "hc_log_softmax_grad_rows_%s", dtype_name(dtype));
+      return launch(ctx, name, ceil_div((uint64_t)outer, HCK_BLOCK / 64), 1, &k, sizeof(k));
+    }
+    snprintf(name, sizeof(name), "hc_log_softmax_grad_rows256_%s", dtype_name(dtype));
+    return launch(ctx, name, (uint64_t)outer, 1, &k, sizeof(k));
   }
   snprintf(name, sizeof(name), "hc_log_softmax_grad_cols_%s", dtype_name(dtype));
   return launch(ctx, name, ceil_div((uint64_t)inner, HCK_BLOCK) * (uint64_t)outer, 1, &k, sizeof(k));
@@ -1144,6 +1156,7 @@ extern "C" int hc_normalize(hc_ctx* ctx, int dtype, const void* in, void* out, i
   if (outer * reduce * inner == 0) return HC_OK;
   REQUIRE(in && out, "hc_normalize: null pointer");
   REQUIRE(aligned16(in) && aligned16(out), "hc_normalize: buffers must be 16-byte aligned");
+  const size_t el_size = dtype_size(dtype);
   if (inner == 1) {
     hck_reduce_args k;
     memset(&k, 0, sizeof(k));
@@ -1154,8 +1167,13 @@ extern "C" int hc_normalize(hc_ctx* ctx, int dtype, const void* in, void* out, i
     k.inner = 1;
     k.eps = eps;
     char name[64];
-    snprintf(name, sizeof(name), "hc_normalize_rows_%s", dtype_name(dtype));
-    return launch(ctx, name, ceil_div((uint64_t)outer, HCK_BLOCK / 64), 1, &k, sizeof(k));
+    // a wave per row while the row fits its registers (4 x 16 bytes per lane), else a block
+    if ((uint64_t)reduce * el_size <= 64 * 16 * 4) {
+      snprintf(name, sizeof(name), "hc_normalize_rows_%s", dtype_name(dtype));
+      return launch(ctx, name, ceil_div((uint64_t)outer, HCK_BLOCK / 64), 1, &k, sizeof(k));
+    }
+    snprintf(name, sizeof(name), "hc_normalize_rows256_%s", dtype_name(dtype));
+    return launch(ctx, name, (uint64_t)outer, 1, &k, sizeof(k));
   }
   // inner > 1: the same composition the base class runs (Backend.swift:265-327), on device.
   const size_t el = dtype_size(dtype);
@@ -1363,9 +1381,12 @@ extern "C" int hc_adamw(hc_ctx* ctx, int dtype, const void* param, const void* g
   k.exp_root = 0.5f;
   char name[64];
   snprintf(name, sizeof(name), "hc_adamw_%s", dtype_name(dtype));
-  uint64_t blocks = ceil_div(count, HCK_BLOCK);
-  const uint64_t cap = (uint64_t)ctx->props.multiProcessorCount * 32;
-  if (blocks > cap) blocks = cap;
+  REQUIRE(aligned16(param) && aligned16(grad) && aligned16(moment1) && aligned16(moment2) && aligned16(out_param) &&
+              aligned16(out_moment1) && aligned16(out_moment2),
+          "hc_adamw: buffers must be 16-byte aligned");
+  // one 16-byte vector per lane (the kernel's loop only matters beyond 2^31 blocks)
+  uint64_t blocks = ceil_div(ceil_div(count, 16 / dtype_size(dtype)), HCK_BLOCK);
+  if (blocks > 0x7fffffffull) blocks = 0x7fffffffull;
   return launch(ctx, name, blocks, 1, &k, sizeof(k));
 }
 

@@ -91,6 +91,26 @@ __device__ __forceinline__ void bcast_offsets(const hck_bcast& d, uint32_t v, ui
   }
 }
 
+// powf for the pow / normalize / AdamW kernels. Exponents 2, 0.5 and -0.5 (squares, roots and
+// reciprocal roots: LayerNorm and Adam) take correctly rounded multiplies / square roots instead
+// of the generic exp2(y * log2(x)) evaluation, with powf's results at zero and infinity;
+// everything else is the device library's powf. All callers share this one function, so a
+// fused kernel and the op-by-op composition agree bit for bit.
+__device__ __forceinline__ float pow_like(float x, float b) {
+  if (b == 2.0f) return x * x;
+  if (b == 0.5f) {
+    if (x == 0.0f) return 0.0f;
+    if (x == -INFINITY) return INFINITY;
+    return sqrtf(x);
+  }
+  if (b == -0.5f) {
+    if (x == 0.0f) return INFINITY;
+    if (x == -INFINITY) return 0.0f;
+    return 1.0f / sqrtf(x);
+  }
+  return powf(x, b);
+}
+
 // ---- wave64 / block reductions ----
 
 template <typename V, typename Op> __device__ __forceinline__ V wave_reduce(V v, Op op) {

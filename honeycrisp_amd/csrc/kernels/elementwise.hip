@@ -452,7 +452,7 @@ template <typename T, int MODE> __device__ __forceinline__ void pow_impl(const h
     float x = (float)xv;
     float r;
     if (MODE == 0) {
-      r = scale * (scales ? (float)scales[i] : 1.0f) * powf(x, b);
+      r = scale * (scales ? (float)scales[i] : 1.0f) * pow_like(x, b);
     } else {
       if (MODE == 1) {
         r = x * x;
@@ -502,34 +502,56 @@ HC_KERNEL void hc_pow_generic_i64(hck_map_args p) {
 // a tensor, squares and roots take the same paths as the pow kernels above (fp32: x*x then
 // *scale unless scale == 1; fp16 and every root: scale * 1 * powf), and the file is built
 // without FMA contraction, so the results equal the composed ones bit for bit.
-template <typename T> __device__ __forceinline__ void adamw_impl(const hck_adamw_args& p) {
-  const uint64_t stride = (uint64_t)gridDim.x * HCK_BLOCK;
-  for (uint64_t i = (uint64_t)blockIdx.x * HCK_BLOCK + threadIdx.x; i < p.count; i += stride) {
-    const float param = (float)((const T*)p.param)[i], g = (float)((const T*)p.grad)[i];
-    const float m = (float)((const T*)p.m1)[i], v = (float)((const T*)p.m2)[i];
-    const float m_scaled = round_through<T>(p.beta1 * m);
-    const float g_scaled = round_through<T>(p.one_minus_beta1 * g);
-    const float new_m = round_through<T>(m_scaled + g_scaled);
-    float g_sq;
-    if (sizeof(T) == 4) {
-      g_sq = g * g;
-      if (p.one_minus_beta2 != 1.0f) g_sq = g_sq * p.one_minus_beta2;
-    } else {
-      g_sq = round_through<T>(p.one_minus_beta2 * 1.0f * powf(g, p.exp_square));
-    }
-    const float v_scaled = round_through<T>(p.beta2 * v);
-    const float new_v = round_through<T>(v_scaled + g_sq);
-    const float m_hat = round_through<T>(new_m * p.bias1);
-    const float v_hat = round_through<T>(new_v * p.bias2);
-    const float root = round_through<T>(1.0f * 1.0f * powf(v_hat, p.exp_root));
-    const float denom = round_through<T>(root + p.eps);
-    const float ratio = round_through<T>(m_hat / denom);
-    const float step_dir = round_through<T>(ratio * p.lr);
-    const float decayed = round_through<T>(param * p.decay);
-    ((T*)p.out_param)[i] = narrow<T>(decayed - step_dir);
-    ((T*)p.out_m1)[i] = narrow<T>(new_m);
-    ((T*)p.out_m2)[i] = narrow<T>(new_v);
+template <typename T>
+__device__ __forceinline__ void adamw_one(const hck_adamw_args& p, float param, float g, float m, float v,
+                                          T& out_param, T& out_m, T& out_v) {
+  const float m_scaled = round_through<T>(p.beta1 * m);
+  const float g_scaled = round_through<T>(p.one_minus_beta1 * g);
+  const float new_m = round_through<T>(m_scaled + g_scaled);
+  float g_sq;
+  if (sizeof(T) == 4) {
+    g_sq = g * g;
+    if (p.one_minus_beta2 != 1.0f) g_sq = g_sq * p.one_minus_beta2;
+  } else {
+    g_sq = round_through<T>(p.one_minus_beta2 * 1.0f * pow_like(g, p.exp_square));
   }
+  const float v_scaled = round_through<T>(p.beta2 * v);
+  const float new_v = round_through<T>(v_scaled + g_sq);
+  const float m_hat = round_through<T>(new_m * p.bias1);
+  const float v_hat = round_through<T>(new_v * p.bias2);
+  const float root = round_through<T>(1.0f * 1.0f * pow_like(v_hat, p.exp_root));
+  const float denom = round_through<T>(root + p.eps);
+  const float ratio = round_through<T>(m_hat / denom);
+  const float step_dir = round_through<T>(ratio * p.lr);
+  const float decayed = round_through<T>(param * p.decay);
+  out_param = narrow<T>(decayed - step_dir);
+  out_m = narrow<T>(new_m);
+  out_v = narrow<T>(new_v);
+}
+
+// 16-byte vectors, grid-stride; the ragged tail (< VEC elements) is done by the first lanes.
+template <typename T> __device__ __forceinline__ void adamw_impl(const hck_adamw_args& p) {
+  constexpr int VEC = VecWidth<T>::value;
+  const uint64_t nvec = p.count / VEC;
+  const uint64_t stride = (uint64_t)gridDim.x * HCK_BLOCK;
+  const uint64_t t = (uint64_t)blockIdx.x * HCK_BLOCK + threadIdx.x;
+  for (uint64_t i = t; i < nvec; i += stride) {
+    T pa[VEC], g[VEC], m[VEC], v[VEC], op[VEC], om[VEC], ov[VEC];
+    load_vec<T, VEC>((const T*)p.param + i * VEC, 0, 1, pa);
+    load_vec<T, VEC>((const T*)p.grad + i * VEC, 0, 1, g);
+    load_vec<T, VEC>((const T*)p.m1 + i * VEC, 0, 1, m);
+    load_vec<T, VEC>((const T*)p.m2 + i * VEC, 0, 1, v);
+#pragma unroll
+    for (int e = 0; e < VEC; e++)
+      adamw_one<T>(p, (float)pa[e], (float)g[e], (float)m[e], (float)v[e], op[e], om[e], ov[e]);
+    store_vec<T, VEC>((T*)p.out_param, i * VEC, op);
+    store_vec<T, VEC>((T*)p.out_m1, i * VEC, om);
+    store_vec<T, VEC>((T*)p.out_m2, i * VEC, ov);
+  }
+  const uint64_t i = nvec * VEC + t;
+  if (i < p.count)
+    adamw_one<T>(p, (float)((const T*)p.param)[i], (float)((const T*)p.grad)[i], (float)((const T*)p.m1)[i],
+                 (float)((const T*)p.m2)[i], ((T*)p.out_param)[i], ((T*)p.out_m1)[i], ((T*)p.out_m2)[i]);
 }
 HC_KERNEL void hc_adamw_f32(hck_adamw_args p) { adamw_impl<float>(p); }
 HC_KERNEL void hc_adamw_f16(hck_adamw_args p) { adamw_impl<half_t>(p); }

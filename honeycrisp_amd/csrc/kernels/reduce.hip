@@ -233,25 +233,42 @@ DEF_REDUCE_T(f32, float)
 DEF_REDUCE_T(f16, half_t)
 DEF_REDUCE_T(i64, int64_t)
 
-// A row of up to 64 * VEC * CHUNKS elements held by one wave in registers: lane l owns the
-// 16-byte vectors l, l + 64, ... of the row (n a multiple of VEC; rows then start 16-byte
-// aligned because the buffer does).
-template <typename T> struct RowRegs {
+// ---------------------------------------------------------------- row teams
+
+// A row is worked on by a team of LANES lanes: one wave (4 rows per block) or the whole block.
+template <int LANES> struct Team {
+  static __device__ __forceinline__ uint32_t lane() { return threadIdx.x % LANES; }
+  static __device__ __forceinline__ uint32_t row() {
+    return blockIdx.x * (HCK_BLOCK / LANES) + threadIdx.x / LANES;
+  }
+  // every lane of the team gets the result; `lds` holds >= 4 floats (block teams only)
+  template <typename Op> static __device__ __forceinline__ float reduce(float v, Op op, float* lds) {
+    if (LANES == 64) return wave_reduce(v, op);
+    return block_reduce(v, op, lds);
+  }
+};
+
+// A row of up to LANES * VEC * CHUNKS elements held by its team in registers: lane l owns the
+// 16-byte vectors l, l + LANES, ... of the row (n a multiple of VEC; rows then start 16-byte
+// aligned because the buffer does). Longer rows, or ragged ones, are streamed instead.
+template <typename T, int LANES> struct RowRegs {
   static constexpr int VEC = VecWidth<T>::value;
   static constexpr int CHUNKS = 4;
   T v[CHUNKS][VEC];
-  static __device__ __forceinline__ bool fits(uint32_t n) { return n % VEC == 0 && n <= 64u * VEC * CHUNKS; }
+  static __device__ __forceinline__ bool fits(uint32_t n) {
+    return n % VEC == 0 && n <= (uint32_t)LANES * VEC * CHUNKS;
+  }
   __device__ __forceinline__ void load(const T* row, uint32_t n, uint32_t lane) {
 #pragma unroll
     for (int c = 0; c < CHUNKS; c++) {
-      const uint32_t k = (lane + 64 * c) * VEC;
+      const uint32_t k = (lane + LANES * c) * VEC;
       if (k < n) load_vec<T, VEC>(row, k, 1, v[c]);
     }
   }
   template <typename F> __device__ __forceinline__ void each(uint32_t n, uint32_t lane, F f) const {
 #pragma unroll
     for (int c = 0; c < CHUNKS; c++)
-      if ((lane + 64 * c) * VEC < n) {
+      if ((lane + LANES * c) * VEC < n) {
 #pragma unroll
         for (int i = 0; i < VEC; i++) f((float)v[c][i]);
       }
@@ -259,7 +276,7 @@ template <typename T> struct RowRegs {
   template <typename F> __device__ __forceinline__ void store(T* row, uint32_t n, uint32_t lane, F f) const {
 #pragma unroll
     for (int c = 0; c < CHUNKS; c++) {
-      const uint32_t k = (lane + 64 * c) * VEC;
+      const uint32_t k = (lane + LANES * c) * VEC;
       if (k < n) {
         T o[VEC];
 #pragma unroll
@@ -272,7 +289,7 @@ template <typename T> struct RowRegs {
   __device__ __forceinline__ void store2(T* row, uint32_t n, uint32_t lane, const RowRegs& other, F f) const {
 #pragma unroll
     for (int c = 0; c < CHUNKS; c++) {
-      const uint32_t k = (lane + 64 * c) * VEC;
+      const uint32_t k = (lane + LANES * c) * VEC;
       if (k < n) {
         T o[VEC];
 #pragma unroll
@@ -283,44 +300,74 @@ template <typename T> struct RowRegs {
   }
 };
 
+// Streaming pass over a row that does not fit the registers: f(x, k) for every element, with
+// 16-byte loads when the row length allows them.
+template <typename T, int LANES, typename F>
+__device__ __forceinline__ void stream_row(const T* row, uint32_t n, uint32_t lane, F f) {
+  constexpr int VEC = VecWidth<T>::value;
+  if (n % VEC == 0) {
+    for (uint32_t k = lane * VEC; k < n; k += LANES * VEC) {
+      T a[VEC];
+      load_vec<T, VEC>(row, k, 1, a);
+#pragma unroll
+      for (int i = 0; i < VEC; i++) f((float)a[i], k + i);
+    }
+  } else {
+    for (uint32_t k = lane; k < n; k += LANES) f((float)row[k], k);
+  }
+}
+// ... and one that also writes: out[k] = f(x, k).
+template <typename T, int LANES, typename F>
+__device__ __forceinline__ void stream_row_out(const T* row, T* out, uint32_t n, uint32_t lane, F f) {
+  constexpr int VEC = VecWidth<T>::value;
+  if (n % VEC == 0) {
+    for (uint32_t k = lane * VEC; k < n; k += LANES * VEC) {
+      T a[VEC], o[VEC];
+      load_vec<T, VEC>(row, k, 1, a);
+#pragma unroll
+      for (int i = 0; i < VEC; i++) o[i] = narrow<T>(f((float)a[i], k + i));
+      store_vec<T, VEC>(out, k, o);
+    }
+  } else {
+    for (uint32_t k = lane; k < n; k += LANES) out[k] = narrow<T>(f((float)row[k], k));
+  }
+}
+
 // ---------------------------------------------------------------- logSoftmax
 
 // logSoftmax (BackendCPU.swift:1000-1038): max, sum of expf(x - max), x - (logf(sum) + max),
-// all in Float. Rows: one wave per row; the row is re-read from L1/L2 for passes 2 and 3.
-template <typename T> __device__ __forceinline__ void log_softmax_rows_impl(const hck_reduce_args& p) {
-  const uint32_t lane = threadIdx.x & 63;
-  const uint32_t row = blockIdx.x * (HCK_BLOCK / 64) + (threadIdx.x >> 6);
-  if (row >= p.outer) return;
+// all in Float. Rows (inner == 1): a wave or a block per row; the row stays in registers when
+// it fits, else passes 2 and 3 re-read it (L2).
+// NaNs are skipped by the strict compare here and on the CPU alike; any NaN in the row then
+// turns the exp-sum, and with it the whole row, into NaN on both.
+template <typename T, int LANES> __device__ __forceinline__ void log_softmax_rows_impl(const hck_reduce_args& p) {
+  __shared__ float lds[HCK_BLOCK / 64];
+  const uint32_t lane = Team<LANES>::lane(), row = Team<LANES>::row();
+  if (row >= p.outer) return;  // (never taken by a block team: one row per block)
   const uint32_t n = p.reduce;
   const T* in = (const T*)p.in + (size_t)row * n;
   T* out = (T*)p.out + (size_t)row * n;
-  // NaNs are skipped by the strict compare here and on the CPU alike; any NaN in the row
-  // then turns the exp-sum, and with it the whole row, into NaN on both.
-  if (RowRegs<T>::fits(n)) {
-    // short rows: read once with 16-byte loads, keep the row in registers
-    RowRegs<T> r;
+  if (RowRegs<T, LANES>::fits(n)) {
+    RowRegs<T, LANES> r;
     r.load(in, n, lane);
     float m = -INFINITY;
     r.each(n, lane, [&](float x) { if (x > m) m = x; });
-    m = wave_reduce(m, MaxOp());
+    m = Team<LANES>::reduce(m, MaxOp(), lds);
     float s = 0.0f;
     r.each(n, lane, [&](float x) { s += expf(x - m); });
-    s = wave_reduce(s, SumOp());
+    s = Team<LANES>::reduce(s, SumOp(), lds);
     const float log_sum = logf(s) + m;
     r.store(out, n, lane, [&](float x) { return x - log_sum; });
     return;
   }
   float m = -INFINITY;
-  for (uint32_t k = lane; k < n; k += 64) {
-    float x = (float)in[k];
-    if (x > m) m = x;
-  }
-  m = wave_reduce(m, MaxOp());
+  stream_row<T, LANES>(in, n, lane, [&](float x, uint32_t) { if (x > m) m = x; });
+  m = Team<LANES>::reduce(m, MaxOp(), lds);
   float s = 0.0f;
-  for (uint32_t k = lane; k < n; k += 64) s += expf((float)in[k] - m);
-  s = wave_reduce(s, SumOp());
+  stream_row<T, LANES>(in, n, lane, [&](float x, uint32_t) { s += expf(x - m); });
+  s = Team<LANES>::reduce(s, SumOp(), lds);
   const float log_sum = logf(s) + m;
-  for (uint32_t k = lane; k < n; k += 64) out[k] = narrow<T>((float)in[k] - log_sum);
+  stream_row_out<T, LANES>(in, out, n, lane, [&](float x, uint32_t) { return x - log_sum; });
 }
 
 // Columns: one lane per (outer, inner) pair, lanes along inner.
@@ -344,50 +391,50 @@ template <typename T> __device__ __forceinline__ void log_softmax_cols_impl(cons
     out[(size_t)k * p.inner] = narrow<T>((float)in[(size_t)k * p.inner] - log_sum);
 }
 
-HC_KERNEL void hc_log_softmax_rows_f32(hck_reduce_args p) { log_softmax_rows_impl<float>(p); }
-HC_KERNEL void hc_log_softmax_rows_f16(hck_reduce_args p) { log_softmax_rows_impl<half_t>(p); }
+HC_KERNEL void hc_log_softmax_rows_f32(hck_reduce_args p) { log_softmax_rows_impl<float, 64>(p); }
+HC_KERNEL void hc_log_softmax_rows_f16(hck_reduce_args p) { log_softmax_rows_impl<half_t, 64>(p); }
+HC_KERNEL void hc_log_softmax_rows256_f32(hck_reduce_args p) { log_softmax_rows_impl<float, 256>(p); }
+HC_KERNEL void hc_log_softmax_rows256_f16(hck_reduce_args p) { log_softmax_rows_impl<half_t, 256>(p); }
 HC_KERNEL void hc_log_softmax_cols_f32(hck_reduce_args p) { log_softmax_cols_impl<float>(p); }
 HC_KERNEL void hc_log_softmax_cols_f16(hck_reduce_args p) { log_softmax_cols_impl<half_t>(p); }
 
 // logSoftmaxGrad (BackendCPU.swift:1040-1085): g - sum(g) * expf(x - (logf(sum exp(x - max)) + max)).
-template <typename T> __device__ __forceinline__ void log_softmax_grad_rows_impl(const hck_reduce_args& p) {
-  const uint32_t lane = threadIdx.x & 63;
-  const uint32_t row = blockIdx.x * (HCK_BLOCK / 64) + (threadIdx.x >> 6);
+template <typename T, int LANES>
+__device__ __forceinline__ void log_softmax_grad_rows_impl(const hck_reduce_args& p) {
+  __shared__ float lds[HCK_BLOCK / 64];
+  const uint32_t lane = Team<LANES>::lane(), row = Team<LANES>::row();
   if (row >= p.outer) return;
   const uint32_t n = p.reduce;
   const T* in = (const T*)p.in + (size_t)row * n;
   const T* grad = (const T*)p.in2 + (size_t)row * n;
   T* out = (T*)p.out + (size_t)row * n;
-  if (RowRegs<T>::fits(n)) {
-    RowRegs<T> r, g;
+  if (RowRegs<T, LANES>::fits(n)) {
+    RowRegs<T, LANES> r, g;
     r.load(in, n, lane);
     g.load(grad, n, lane);
     float m = -INFINITY, gs = 0.0f;
     r.each(n, lane, [&](float x) { if (x > m) m = x; });
     g.each(n, lane, [&](float x) { gs += x; });
-    m = wave_reduce(m, MaxOp());
-    gs = wave_reduce(gs, SumOp());
+    m = Team<LANES>::reduce(m, MaxOp(), lds);
+    gs = Team<LANES>::reduce(gs, SumOp(), lds);
     float s = 0.0f;
     r.each(n, lane, [&](float x) { s += expf(x - m); });
-    s = wave_reduce(s, SumOp());
+    s = Team<LANES>::reduce(s, SumOp(), lds);
     const float log_sum = logf(s) + m;
     g.store2(out, n, lane, r, [&](float gv, float x) { return gv - gs * expf(x - log_sum); });
     return;
   }
   float m = -INFINITY, gs = 0.0f;
-  for (uint32_t k = lane; k < n; k += 64) {
-    float x = (float)in[k];
-    if (x > m) m = x;
-    gs += (float)grad[k];
-  }
-  m = wave_reduce(m, MaxOp());
-  gs = wave_reduce(gs, SumOp());
+  stream_row<T, LANES>(in, n, lane, [&](float x, uint32_t) { if (x > m) m = x; });
+  stream_row<T, LANES>(grad, n, lane, [&](float x, uint32_t) { gs += x; });
+  m = Team<LANES>::reduce(m, MaxOp(), lds);
+  gs = Team<LANES>::reduce(gs, SumOp(), lds);
   float s = 0.0f;
-  for (uint32_t k = lane; k < n; k += 64) s += expf((float)in[k] - m);
-  s = wave_reduce(s, SumOp());
+  stream_row<T, LANES>(in, n, lane, [&](float x, uint32_t) { s += expf(x - m); });
+  s = Team<LANES>::reduce(s, SumOp(), lds);
   const float log_sum = logf(s) + m;
-  for (uint32_t k = lane; k < n; k += 64)
-    out[k] = narrow<T>((float)grad[k] - gs * expf((float)in[k] - log_sum));
+  stream_row_out<T, LANES>(grad, out, n, lane,
+                           [&](float gv, uint32_t k) { return gv - gs * expf((float)in[k] - log_sum); });
 }
 
 template <typename T> __device__ __forceinline__ void log_softmax_grad_cols_impl(const hck_reduce_args& p) {
@@ -412,8 +459,10 @@ template <typename T> __device__ __forceinline__ void log_softmax_grad_cols_impl
     out[(size_t)k * p.inner] =
         narrow<T>((float)grad[(size_t)k * p.inner] - gs * expf((float)in[(size_t)k * p.inner] - log_sum));
 }
-HC_KERNEL void hc_log_softmax_grad_rows_f32(hck_reduce_args p) { log_softmax_grad_rows_impl<float>(p); }
-HC_KERNEL void hc_log_softmax_grad_rows_f16(hck_reduce_args p) { log_softmax_grad_rows_impl<half_t>(p); }
+HC_KERNEL void hc_log_softmax_grad_rows_f32(hck_reduce_args p) { log_softmax_grad_rows_impl<float, 64>(p); }
+HC_KERNEL void hc_log_softmax_grad_rows_f16(hck_reduce_args p) { log_softmax_grad_rows_impl<half_t, 64>(p); }
+HC_KERNEL void hc_log_softmax_grad_rows256_f32(hck_reduce_args p) { log_softmax_grad_rows_impl<float, 256>(p); }
+HC_KERNEL void hc_log_softmax_grad_rows256_f16(hck_reduce_args p) { log_softmax_grad_rows_impl<half_t, 256>(p); }
 HC_KERNEL void hc_log_softmax_grad_cols_f32(hck_reduce_args p) { log_softmax_grad_cols_impl<float>(p); }
 HC_KERNEL void hc_log_softmax_grad_cols_f16(hck_reduce_args p) { log_softmax_grad_cols_impl<half_t>(p); }
 
@@ -423,54 +472,46 @@ HC_KERNEL void hc_log_softmax_grad_cols_f16(hck_reduce_args p) { log_softmax_gra
 //   mean = sum(x) * (1/n); c = x - mean; var = sum(c^2) * (1/n);
 //   out = c * (var + eps)^-0.5
 // with every intermediate rounded to the tensor dtype where the composed backend calls
-// would have stored it. One wave per row; c^2 is x*x for fp32 (pow special case) and
-// powf(x, 2) for fp16 (generic path), as on the CPU.
-template <typename T> __device__ __forceinline__ void normalize_rows_impl(const hck_reduce_args& p) {
-  const uint32_t lane = threadIdx.x & 63;
-  const uint32_t row = blockIdx.x * (HCK_BLOCK / 64) + (threadIdx.x >> 6);
+// would have stored it. c^2 is x*x for fp32 (pow special case) and powf(x, 2) for fp16
+// (generic path), as on the CPU.
+template <typename T, int LANES> __device__ __forceinline__ void normalize_rows_impl(const hck_reduce_args& p) {
+  __shared__ float lds[HCK_BLOCK / 64];
+  const uint32_t lane = Team<LANES>::lane(), row = Team<LANES>::row();
   if (row >= p.outer) return;
   const uint32_t n = p.reduce;
   const T* in = (const T*)p.in + (size_t)row * n;
   T* out = (T*)p.out + (size_t)row * n;
   const float inv_n = 1.0f / (float)n;
-  if (RowRegs<T>::fits(n)) {
-    RowRegs<T> r;
+  auto square = [](float c) { return round_through<T>(sizeof(T) == 4 ? c * c : 1.0f * 1.0f * pow_like(c, 2.0f)); };
+  if (RowRegs<T, LANES>::fits(n)) {
+    RowRegs<T, LANES> r;
     r.load(in, n, lane);
     float s = 0.0f;
     r.each(n, lane, [&](float x) { s += x; });
-    s = round_through<T>(wave_reduce(s, SumOp()));
+    s = round_through<T>(Team<LANES>::reduce(s, SumOp(), lds));
     const float mean = round_through<T>(s * inv_n);
     float sq = 0.0f;
-    r.each(n, lane, [&](float x) {
-      const float c = round_through<T>(x - mean);
-      const float c2 = sizeof(T) == 4 ? c * c : 1.0f * 1.0f * powf(c, 2.0f);
-      sq += round_through<T>(c2);
-    });
-    sq = round_through<T>(wave_reduce(sq, SumOp()));
+    r.each(n, lane, [&](float x) { sq += square(round_through<T>(x - mean)); });
+    sq = round_through<T>(Team<LANES>::reduce(sq, SumOp(), lds));
     const float var = round_through<T>(sq * inv_n);
     const float shifted = round_through<T>(var + p.eps);
-    const float normer = round_through<T>(1.0f * 1.0f * powf(shifted, -0.5f));
+    const float normer = round_through<T>(1.0f * 1.0f * pow_like(shifted, -0.5f));
     r.store(out, n, lane, [&](float x) { return round_through<T>(x - mean) * normer; });
     return;
   }
   float s = 0.0f;
-  for (uint32_t k = lane; k < n; k += 64) s += (float)in[k];
-  s = round_through<T>(wave_reduce(s, SumOp()));
+  stream_row<T, LANES>(in, n, lane, [&](float x, uint32_t) { s += x; });
+  s = round_through<T>(Team<LANES>::reduce(s, SumOp(), lds));
   const float mean = round_through<T>(s * inv_n);
   float sq = 0.0f;
-  for (uint32_t k = lane; k < n; k += 64) {
-    float c = round_through<T>((float)in[k] - mean);
-    float c2 = sizeof(T) == 4 ? c * c : 1.0f * 1.0f * powf(c, 2.0f);
-    sq += round_through<T>(c2);
-  }
-  sq = round_through<T>(wave_reduce(sq, SumOp()));
+  stream_row<T, LANES>(in, n, lane, [&](float x, uint32_t) { sq += square(round_through<T>(x - mean)); });
+  sq = round_through<T>(Team<LANES>::reduce(sq, SumOp(), lds));
   const float var = round_through<T>(sq * inv_n);
   const float shifted = round_through<T>(var + p.eps);
-  const float normer = round_through<T>(1.0f * 1.0f * powf(shifted, -0.5f));
-  for (uint32_t k = lane; k < n; k += 64) {
-    float c = round_through<T>((float)in[k] - mean);
-    out[k] = narrow<T>(c * normer);
-  }
+  const float normer = round_through<T>(1.0f * 1.0f * pow_like(shifted, -0.5f));
+  stream_row_out<T, LANES>(in, out, n, lane, [&](float x, uint32_t) { return round_through<T>(x - mean) * normer; });
 }
-HC_KERNEL void hc_normalize_rows_f32(hck_reduce_args p) { normalize_rows_impl<float>(p); }
-HC_KERNEL void hc_normalize_rows_f16(hck_reduce_args p) { normalize_rows_impl<half_t>(p); }
+HC_KERNEL void hc_normalize_rows_f32(hck_reduce_args p) { normalize_rows_impl<float, 64>(p); }
+HC_KERNEL void hc_normalize_rows_f16(hck_reduce_args p) { normalize_rows_impl<half_t, 64>(p); }
+HC_KERNEL void hc_normalize_rows256_f32(hck_reduce_args p) { normalize_rows_impl<float, 256>(p); }
+HC_KERNEL void hc_normalize_rows256_f16(hck_reduce_args p) { normalize_rows_impl<half_t, 256>(p); }
