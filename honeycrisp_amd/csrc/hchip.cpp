@@ -1024,6 +1024,21 @@ extern "C" int hc_fill(hc_ctx* ctx, int dtype, float vf, int64_t vi, void* out, 
   return launch_contiguous(ctx, name, count, vec_for_size(el), &k, sizeof(k));
 }
 
+// Temporaries of one entry point: freed (stream-ordered) when it returns.
+struct Scratch {
+  hc_ctx* ctx;
+  std::vector<void*> ptrs;
+  explicit Scratch(hc_ctx* c) : ctx(c) {}
+  ~Scratch() {
+    for (void* p : ptrs) (void)hc_free(ctx, p);
+  }
+  int get(size_t bytes, void** out) {
+    int s = hc_malloc(ctx, bytes, out);
+    if (s == HC_OK) ptrs.push_back(*out);
+    return s;
+  }
+};
+
 // ------------------------------------------------------------------ reductions
 
 static const char* const kReduceNames[] = {"sum", "prod", "argmax", "argmin"};
@@ -1035,6 +1050,88 @@ static int check_dims(const char* who, int64_t outer, int64_t reduce, int64_t in
     return fail(HC_ERR_TOO_LARGE, "%s: [%lld, %lld, %lld] exceeds the 32-bit index range", who,
                 (long long)outer, (long long)reduce, (long long)inner);
   return HC_OK;
+}
+
+// Column reduction ([outer, reduce, inner], inner > 1): lanes (x 16-byte vectors when rows keep
+// the alignment) along inner, the reduce axis split over blocks until the device is full,
+// partials combined by a second launch of the same kernel over the [outer, splits, inner]
+// partials. `opname` also covers the internal float-result reductions (maxf, expsumf, sumf).
+static int reduce_cols(hc_ctx* ctx, const char* opname, int dtype, const void* in, const float* aux, void* out,
+                       int64_t outer, int64_t reduce, int64_t inner, bool arg) {
+  const size_t el = dtype_size(dtype);
+  const uint32_t vec = (aligned16(in) && ((uint64_t)inner * el) % 16 == 0) ? (uint32_t)(16 / el) : 1;
+  const uint64_t jblocks = ceil_div(ceil_div((uint64_t)inner, vec), 64);
+  const uint64_t base_blocks = jblocks * (uint64_t)outer;
+  const uint64_t want = (uint64_t)ctx->props.multiProcessorCount * 8;
+  uint64_t splits = base_blocks >= want ? 1 : ceil_div(want, base_blocks);
+  const uint64_t max_splits = reduce / 64 ? (uint64_t)reduce / 64 : 1;  // at least 64 rows per range
+  if (splits > max_splits) splits = max_splits;
+  if (splits > 256) splits = 256;
+  hck_reduce_cols_args c;
+  memset(&c, 0, sizeof(c));
+  c.in = in;
+  c.out = out;
+  c.aux = aux;
+  c.outer = (uint32_t)outer;
+  c.reduce = (uint32_t)reduce;
+  c.inner = (uint32_t)inner;
+  c.chunk = (uint32_t)(ceil_div(ceil_div((uint64_t)reduce, splits), 4) * 4);
+  if (c.chunk == 0) c.chunk = 4;
+  splits = reduce ? ceil_div((uint64_t)reduce, c.chunk) : 1;
+  c.splits = (uint32_t)splits;
+  Scratch scratch(ctx);
+  if (splits > 1) {
+    const size_t n = (size_t)outer * splits * (size_t)inner;
+    HC_TRY(scratch.get(n * (dtype == HC_I64 ? 8 : 4), &c.pvals));
+    if (arg) {
+      void* idx = nullptr;
+      HC_TRY(scratch.get(n * 4, &idx));
+      c.pidx = (uint32_t*)idx;
+    }
+  }
+  char name[64];
+  snprintf(name, sizeof(name), "hc_reduce_cols_%s_%s_%s", opname, dtype_name(dtype), vec > 1 ? "vN" : "v1");
+  HC_TRY(launch(ctx, name, base_blocks * splits, 1, &c, sizeof(c)));
+  if (splits > 1) {
+    snprintf(name, sizeof(name), "hc_reduce_cols_final_%s_%s", opname, dtype_name(dtype));
+    HC_TRY(launch(ctx, name, ceil_div((uint64_t)inner, 64) * (uint64_t)outer, 1, &c, sizeof(c)));
+  }
+  return HC_OK;
+}
+
+// logSoftmax / logSoftmaxGrad over a non-last axis: per-column maximum, exp-sum (and gradient
+// sum) as float column reductions, then one element-wise pass.
+static int softmax_cols(hc_ctx* ctx, int dtype, const void* in, const void* grad, void* out, int64_t outer,
+                        int64_t reduce, int64_t inner) {
+  Scratch scratch(ctx);
+  const size_t cols = (size_t)outer * (size_t)inner;
+  void *m = nullptr, *s = nullptr, *gs = nullptr;
+  HC_TRY(scratch.get(cols * 4, &m));
+  HC_TRY(scratch.get(cols * 4, &s));
+  HC_TRY(reduce_cols(ctx, "maxf", dtype, in, nullptr, m, outer, reduce, inner, false));
+  HC_TRY(reduce_cols(ctx, "expsumf", dtype, in, (const float*)m, s, outer, reduce, inner, false));
+  if (grad) {
+    HC_TRY(scratch.get(cols * 4, &gs));
+    HC_TRY(reduce_cols(ctx, "sumf", dtype, grad, nullptr, gs, outer, reduce, inner, false));
+  }
+  hck_softmax_cols_args k;
+  memset(&k, 0, sizeof(k));
+  k.in = in;
+  k.grad = grad;
+  k.out = out;
+  k.col_max = (const float*)m;
+  k.col_expsum = (const float*)s;
+  k.col_gradsum = (const float*)gs;
+  k.outer = (uint32_t)outer;
+  k.reduce = (uint32_t)reduce;
+  k.inner = (uint32_t)inner;
+  const size_t el = dtype_size(dtype);
+  const uint32_t vec = ((uint64_t)inner * el) % 16 == 0 ? (uint32_t)(16 / el) : 1;
+  char name[64];
+  snprintf(name, sizeof(name), "hc_log_softmax%s_cols_apply_%s_%s", grad ? "_grad" : "", dtype_name(dtype),
+           vec > 1 ? "vN" : "v1");
+  const uint64_t lanes = (uint64_t)outer * (uint64_t)reduce * ceil_div((uint64_t)inner, vec);
+  return launch(ctx, name, ceil_div(lanes, HCK_BLOCK), 1, &k, sizeof(k));
 }
 
 extern "C" int hc_reduce(hc_ctx* ctx, int op, int dtype, const void* in, void* out, int64_t outer,
@@ -1066,8 +1163,8 @@ extern "C" int hc_reduce(hc_ctx* ctx, int op, int dtype, const void* in, void* o
     snprintf(name, sizeof(name), "hc_reduce_rows256_%s_%s", kReduceNames[op], dtype_name(dtype));
     return launch(ctx, name, (uint64_t)outer, 1, &k, sizeof(k));
   }
-  snprintf(name, sizeof(name), "hc_reduce_cols_%s_%s", kReduceNames[op], dtype_name(dtype));
-  return launch(ctx, name, ceil_div((uint64_t)inner, 64) * (uint64_t)outer, 1, &k, sizeof(k));
+  return reduce_cols(ctx, kReduceNames[op], dtype, in, nullptr, out, outer, reduce, inner,
+                     op == HC_ARGMAX || op == HC_ARGMIN);
 }
 
 extern "C" int hc_log_softmax(hc_ctx* ctx, int dtype, const void* in, void* out, int64_t outer,
@@ -1097,8 +1194,7 @@ extern "C" int hc_log_softmax(hc_ctx* ctx, int dtype, const void* in, void* out,
     snprintf(name, sizeof(name), "hc_log_softmax_rows256_%s", dtype_name(dtype));
     return launch(ctx, name, (uint64_t)outer, 1, &k, sizeof(k));
   }
-  snprintf(name, sizeof(name), "hc_log_softmax_cols_%s", dtype_name(dtype));
-  return launch(ctx, name, ceil_div((uint64_t)inner, HCK_BLOCK) * (uint64_t)outer, 1, &k, sizeof(k));
+  return softmax_cols(ctx, dtype, in, nullptr, out, outer, reduce, inner);
 }
 
 extern "C" int hc_log_softmax_grad(hc_ctx* ctx, int dtype, const void* in, const void* out_grad, void* out,
@@ -1129,23 +1225,9 @@ extern "C" int hc_log_softmax_grad(hc_ctx* ctx, int dtype, const void* in, const
     snprintf(name, sizeof(name), "hc_log_softmax_grad_rows256_%s", dtype_name(dtype));
     return launch(ctx, name, (uint64_t)outer, 1, &k, sizeof(k));
   }
-  snprintf(name, sizeof(name), "hc_log_softmax_grad_cols_%s", dtype_name(dtype));
-  return launch(ctx, name, ceil_div((uint64_t)inner, HCK_BLOCK) * (uint64_t)outer, 1, &k, sizeof(k));
+  return softmax_cols(ctx, dtype, in, out_grad, out, outer, reduce, inner);
 }
 
-struct Scratch {
-  hc_ctx* ctx;
-  std::vector<void*> ptrs;
-  explicit Scratch(hc_ctx* c) : ctx(c) {}
-  ~Scratch() {
-    for (void* p : ptrs) (void)hc_free(ctx, p);
-  }
-  int get(size_t bytes, void** out) {
-    int s = hc_malloc(ctx, bytes, out);
-    if (s == HC_OK) ptrs.push_back(*out);
-    return s;
-  }
-};
 
 extern "C" int hc_normalize(hc_ctx* ctx, int dtype, const void* in, void* out, int64_t outer,
                             int64_t reduce, int64_t inner, float eps) {

@@ -78,6 +78,35 @@ typedef struct {
   const void* in2; /* logSoftmaxGrad: the output gradient */
 } hck_reduce_args;
 
+/* Column reduction ([outer, reduce, inner], inner > 1) in up to two passes: the reduce axis is
+ * cut into `splits` ranges of `chunk` rows; with splits > 1 each range leaves a partial value
+ * (and, for arg-reductions, its index) per column, combined by a second kernel. */
+typedef struct {
+  const void* in;
+  void* out;
+  void* pvals;    /* [outer, splits, inner] accumulators (float or int64) */
+  uint32_t* pidx; /* [outer, splits, inner] indices (arg-reductions) */
+  uint32_t outer;
+  uint32_t reduce;
+  uint32_t inner;
+  uint32_t splits;
+  uint32_t chunk;
+  uint32_t pad;
+  const float* aux; /* exp-sum: the per-column maximum, [outer, inner] */
+} hck_reduce_cols_args;
+
+/* Column logSoftmax / logSoftmaxGrad, last step: every element combined with per-column
+ * statistics ([outer, inner] floats). */
+typedef struct {
+  const void* in;
+  const void* grad; /* logSoftmaxGrad only */
+  void* out;
+  const float* col_max;
+  const float* col_expsum;
+  const float* col_gradsum; /* logSoftmaxGrad only */
+  uint32_t outer, reduce, inner, pad;
+} hck_softmax_cols_args;
+
 /* Fused AdamW step over `count` contiguous elements; the scalars are the ones the op-by-op
  * composition would pass to its tensor-scalar ops. */
 typedef struct {

@@ -15,7 +15,12 @@
 
 #include <math.h>
 
-enum { R_SUM = 0, R_PROD = 1, R_ARGMAX = 2, R_ARGMIN = 3 };
+#include <type_traits>
+
+enum { R_SUM = 0, R_PROD = 1, R_ARGMAX = 2, R_ARGMIN = 3,
+       // internal column reductions with float results (logSoftmax over a non-last axis):
+       // maximum, sum of expf(x - column maximum), plain sum
+       R_MAXF = 4, R_EXPSUMF = 5, R_SUMF = 6 };
 
 template <typename C> struct ArgPair {
   C v;
@@ -64,10 +69,12 @@ template <int OP> __device__ __forceinline__ void arg_init(ArgPair<int64_t>& p) 
 }
 
 template <int OP, typename C> __device__ __forceinline__ C reduce_identity() {
-  return OP == R_SUM ? (C)0 : (C)1;
+  if (OP == R_MAXF) return (C)-INFINITY;
+  return OP == R_PROD ? (C)1 : (C)0;
 }
 template <int OP, typename C> __device__ __forceinline__ C reduce_combine(C a, C b) {
-  return OP == R_SUM ? a + b : a * b;
+  if (OP == R_MAXF) return b > a ? b : a;
+  return OP == R_PROD ? a * b : a + b;
 }
 
 // ---------------------------------------------------------------- rows (inner == 1)
@@ -176,46 +183,114 @@ __device__ __forceinline__ void reduce_rows_impl(const hck_reduce_args& p) {
 
 // ---------------------------------------------------------------- columns (inner > 1)
 
-// Block = 64 lanes along inner x 4 waves along reduce.
-template <typename T, int OP> __device__ __forceinline__ void reduce_cols_impl(const hck_reduce_args& p) {
+// Block = 64 lanes along inner, VEC consecutive columns per lane (16-byte loads when the row
+// pitch allows), x 4 waves along the reduce axis, meeting in LDS. The reduce axis is also
+// cut into `splits` ranges handled by different blocks so that a tall, narrow input still
+// fills the device; with splits > 1 the ranges leave partials (accumulator type, plus the
+// index for arg-reductions) and the same kernel runs a second time with FINAL = true over
+// the [outer, splits, inner] partials.
+template <typename T, int OP, int VEC, bool FINAL>
+__device__ __forceinline__ void reduce_cols_impl(const hck_reduce_cols_args& p) {
   typedef typename Arith<T>::type C;
-  // grid.x = outer * ceil(inner / 64): no 65535 limit on outer
-  const uint32_t jblocks = (p.inner + 63) / 64;
-  const uint32_t i = blockIdx.x / jblocks;
-  const uint32_t j = (blockIdx.x - i * jblocks) * 64 + (threadIdx.x & 63);
-  const uint32_t kw = threadIdx.x >> 6;
+  typedef typename std::conditional<FINAL, C, T>::type S;  // what this pass reads
+  constexpr bool ARG = OP == R_ARGMAX || OP == R_ARGMIN;
+  const uint32_t extent = FINAL ? p.splits : p.reduce;     // length of the axis this pass reduces
+  const uint32_t splits = FINAL ? 1 : p.splits;
+  const uint32_t chunk = FINAL ? p.splits : p.chunk;
+  const uint32_t jvecs = (p.inner + VEC - 1) / VEC;
+  const uint32_t jblocks = (jvecs + 63) / 64;
+  uint32_t bid = blockIdx.x;
+  const uint32_t jb = bid % jblocks;
+  bid /= jblocks;
+  const uint32_t s = bid % splits;
+  const uint32_t i = bid / splits;
+  const uint32_t lane = threadIdx.x & 63, kw = threadIdx.x >> 6;
+  const uint32_t j = (jb * 64 + lane) * VEC;
   const bool active = j < p.inner;
-  const T* in = (const T*)p.in + (size_t)i * p.reduce * p.inner + (active ? j : 0);
-  __shared__ char lds_raw[sizeof(ArgPair<C>) * HCK_BLOCK];
+  const uint32_t k_begin = s * chunk;
+  const uint32_t k_end = k_begin + chunk < extent ? k_begin + chunk : extent;
+  const size_t col0 = (size_t)i * extent * p.inner + (active ? j : 0);
+  const S* in = (FINAL ? (const S*)p.pvals : (const S*)p.in) + col0;
+  const uint32_t* in_idx = p.pidx + col0;
+  __shared__ char lds_raw[sizeof(ArgPair<C>) * HCK_BLOCK * VEC];
 
-  if (OP == R_SUM || OP == R_PROD) {
-    C acc = reduce_identity<OP, C>();
-    if (active)
-      for (uint32_t k = kw; k < p.reduce; k += 4)
-        acc = reduce_combine<OP, C>(acc, to_arith(in[(size_t)k * p.inner]));
-    C* lds = (C*)lds_raw;
-    lds[threadIdx.x] = acc;
+  C acc[VEC];
+  ArgPair<C> best[VEC];
+  float col_aux[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; e++) {
+    acc[e] = reduce_identity<OP, C>();
+    arg_init<OP>(best[e]);
+    col_aux[e] = (OP == R_EXPSUMF && !FINAL && active) ? p.aux[(size_t)i * p.inner + j + e] : 0.0f;
+  }
+  auto take = [&](const S (&a)[VEC], uint32_t k) {
+#pragma unroll
+    for (int e = 0; e < VEC; e++) {
+      if (ARG) {
+        ArgPair<C> c;
+        if (FINAL) {  // partials already hold the ordering key and the original index
+          c.v = (C)a[e];
+          c.i = in_idx[(size_t)k * p.inner + e];
+        } else {
+          c.v = arg_key<OP>((C)to_arith(a[e]), k);
+          c.i = k;
+        }
+        best[e] = arg_better<OP>(best[e], c);
+      } else {
+        C x = (C)to_arith(a[e]);
+        if (OP == R_EXPSUMF && !FINAL) x = (C)expf((float)x - col_aux[e]);
+        acc[e] = reduce_combine<OP, C>(acc[e], x);
+      }
+    }
+  };
+  if (active) {
+    uint32_t k = k_begin + kw;
+    constexpr int U = 8;  // rows in flight per lane
+    for (; k + 4 * (U - 1) < k_end; k += 4 * U) {
+      S a[U][VEC];
+#pragma unroll
+      for (int u = 0; u < U; u++) load_vec<S, VEC>(in + (size_t)(k + 4 * u) * p.inner, 0, 1, a[u]);
+#pragma unroll
+      for (int u = 0; u < U; u++) take(a[u], k + 4 * u);
+    }
+    for (; k < k_end; k += 4) {
+      S a[VEC];
+      load_vec<S, VEC>(in + (size_t)k * p.inner, 0, 1, a);
+      take(a, k);
+    }
+  }
+  const bool last = FINAL || p.splits == 1;  // this pass writes the result itself
+  if (ARG) {
+    ArgPair<C>* lds = (ArgPair<C>*)lds_raw;
+#pragma unroll
+    for (int e = 0; e < VEC; e++) lds[threadIdx.x * VEC + e] = best[e];
     __syncthreads();
     if (kw == 0 && active) {
-      for (int w = 1; w < 4; w++) acc = reduce_combine<OP, C>(acc, lds[threadIdx.x + 64 * w]);
-      ((T*)p.out)[(size_t)i * p.inner + j] = from_arith<T>(acc);
+#pragma unroll
+      for (int e = 0; e < VEC; e++) {
+        for (int w = 1; w < 4; w++) best[e] = arg_better<OP>(best[e], lds[(threadIdx.x + 64 * w) * VEC + e]);
+        if (last) {
+          ((int64_t*)p.out)[(size_t)i * p.inner + j + e] = (int64_t)best[e].i;
+        } else {
+          const size_t o = ((size_t)i * p.splits + s) * p.inner + j + e;
+          ((C*)p.pvals)[o] = best[e].v;
+          p.pidx[o] = best[e].i;
+        }
+      }
     }
   } else {
-    ArgPair<C> best;
-    arg_init<OP>(best);
-    if (active)
-      for (uint32_t k = kw; k < p.reduce; k += 4) {
-        ArgPair<C> c;
-        c.v = arg_key<OP>(to_arith(in[(size_t)k * p.inner]), k);
-        c.i = k;
-        best = arg_better<OP>(best, c);
-      }
-    ArgPair<C>* lds = (ArgPair<C>*)lds_raw;
-    lds[threadIdx.x] = best;
+    C* lds = (C*)lds_raw;
+#pragma unroll
+    for (int e = 0; e < VEC; e++) lds[threadIdx.x * VEC + e] = acc[e];
     __syncthreads();
     if (kw == 0 && active) {
-      for (int w = 1; w < 4; w++) best = arg_better<OP>(best, lds[threadIdx.x + 64 * w]);
-      ((int64_t*)p.out)[(size_t)i * p.inner + j] = (int64_t)best.i;
+#pragma unroll
+      for (int e = 0; e < VEC; e++) {
+        for (int w = 1; w < 4; w++) acc[e] = reduce_combine<OP, C>(acc[e], lds[(threadIdx.x + 64 * w) * VEC + e]);
+        if (last && OP >= R_MAXF) ((float*)p.out)[(size_t)i * p.inner + j + e] = (float)acc[e];
+        else if (last) ((T*)p.out)[(size_t)i * p.inner + j + e] = from_arith<T>(acc[e]);
+        else ((C*)p.pvals)[((size_t)i * p.splits + s) * p.inner + j + e] = acc[e];
+      }
     }
   }
 }
@@ -223,7 +298,15 @@ template <typename T, int OP> __device__ __forceinline__ void reduce_cols_impl(c
 #define DEF_REDUCE(NAME, OP, TN, T)                                                                   \
   HC_KERNEL void hc_reduce_rows64_##NAME##_##TN(hck_reduce_args p) { reduce_rows_impl<T, OP, 64>(p); } \
   HC_KERNEL void hc_reduce_rows256_##NAME##_##TN(hck_reduce_args p) { reduce_rows_impl<T, OP, 256>(p); } \
-  HC_KERNEL void hc_reduce_cols_##NAME##_##TN(hck_reduce_args p) { reduce_cols_impl<T, OP>(p); }
+  HC_KERNEL void hc_reduce_cols_##NAME##_##TN##_v1(hck_reduce_cols_args p) {                           \
+    reduce_cols_impl<T, OP, 1, false>(p);                                                              \
+  }                                                                                                    \
+  HC_KERNEL void hc_reduce_cols_##NAME##_##TN##_vN(hck_reduce_cols_args p) {                           \
+    reduce_cols_impl<T, OP, VecWidth<T>::value, false>(p);                                             \
+  }                                                                                                    \
+  HC_KERNEL void hc_reduce_cols_final_##NAME##_##TN(hck_reduce_cols_args p) {                          \
+    reduce_cols_impl<T, OP, 1, true>(p);                                                               \
+  }
 #define DEF_REDUCE_T(TN, T)                                                                          \
   DEF_REDUCE(sum, R_SUM, TN, T)                                                                      \
   DEF_REDUCE(prod, R_PROD, TN, T)                                                                    \
@@ -370,33 +453,69 @@ template <typename T, int LANES> __device__ __forceinline__ void log_softmax_row
   stream_row_out<T, LANES>(in, out, n, lane, [&](float x, uint32_t) { return x - log_sum; });
 }
 
-// Columns: one lane per (outer, inner) pair, lanes along inner.
-template <typename T> __device__ __forceinline__ void log_softmax_cols_impl(const hck_reduce_args& p) {
-  const uint32_t jblocks = (p.inner + HCK_BLOCK - 1) / HCK_BLOCK;
-  const uint32_t i = blockIdx.x / jblocks;
-  const uint32_t j = (blockIdx.x - i * jblocks) * HCK_BLOCK + threadIdx.x;
-  if (j >= p.inner) return;
-  const size_t base = (size_t)i * p.reduce * p.inner + j;
-  const T* in = (const T*)p.in + base;
-  T* out = (T*)p.out + base;
-  float m = 0.0f;
-  for (uint32_t k = 0; k < p.reduce; k++) {
-    float x = (float)in[(size_t)k * p.inner];
-    if (k == 0 || x > m) m = x;
+// Columns (inner > 1): per-column maximum and exp-sum come from the split column reductions
+// above (R_MAXF, R_EXPSUMF), then one element-wise pass applies them.
+template <typename T, int VEC, bool GRAD> __device__ __forceinline__ void softmax_cols_apply_impl(const hck_softmax_cols_args& p) {
+  const uint32_t jvecs = (p.inner + VEC - 1) / VEC;
+  const uint64_t t = (uint64_t)blockIdx.x * HCK_BLOCK + threadIdx.x;
+  const uint64_t rows = (uint64_t)p.outer * p.reduce;
+  const uint64_t r = t / jvecs;
+  if (r >= rows) return;
+  const uint32_t j = (uint32_t)(t - r * jvecs) * VEC;
+  const uint32_t i = (uint32_t)(r / p.reduce);
+  const size_t off = (size_t)r * p.inner + j, col = (size_t)i * p.inner + j;
+  T x[VEC], g[VEC], o[VEC];
+  load_vec<T, VEC>((const T*)p.in + off, 0, 1, x);
+  if (GRAD) load_vec<T, VEC>((const T*)p.grad + off, 0, 1, g);
+#pragma unroll
+  for (int e = 0; e < VEC; e++) {
+    if (j + e < p.inner) {
+      const float log_sum = logf(p.col_expsum[col + e]) + p.col_max[col + e];
+      if (GRAD) o[e] = narrow<T>((float)g[e] - p.col_gradsum[col + e] * expf((float)x[e] - log_sum));
+      else o[e] = narrow<T>((float)x[e] - log_sum);
+    }
   }
-  float s = 0.0f;
-  for (uint32_t k = 0; k < p.reduce; k++) s += expf((float)in[(size_t)k * p.inner] - m);
-  const float log_sum = logf(s) + m;
-  for (uint32_t k = 0; k < p.reduce; k++)
-    out[(size_t)k * p.inner] = narrow<T>((float)in[(size_t)k * p.inner] - log_sum);
+  store_vec<T, VEC>((T*)p.out, off, o);
 }
+#define DEF_SOFTMAX_COLS(TN, T)                                                                        \
+  HC_KERNEL void hc_reduce_cols_maxf_##TN##_v1(hck_reduce_cols_args p) { reduce_cols_impl<T, R_MAXF, 1, false>(p); } \
+  HC_KERNEL void hc_reduce_cols_maxf_##TN##_vN(hck_reduce_cols_args p) {                               \
+    reduce_cols_impl<T, R_MAXF, VecWidth<T>::value, false>(p);                                         \
+  }                                                                                                    \
+  HC_KERNEL void hc_reduce_cols_final_maxf_##TN(hck_reduce_cols_args p) { reduce_cols_impl<T, R_MAXF, 1, true>(p); } \
+  HC_KERNEL void hc_reduce_cols_expsumf_##TN##_v1(hck_reduce_cols_args p) {                            \
+    reduce_cols_impl<T, R_EXPSUMF, 1, false>(p);                                                       \
+  }                                                                                                    \
+  HC_KERNEL void hc_reduce_cols_expsumf_##TN##_vN(hck_reduce_cols_args p) {                            \
+    reduce_cols_impl<T, R_EXPSUMF, VecWidth<T>::value, false>(p);                                      \
+  }                                                                                                    \
+  HC_KERNEL void hc_reduce_cols_final_expsumf_##TN(hck_reduce_cols_args p) {                           \
+    reduce_cols_impl<T, R_EXPSUMF, 1, true>(p);                                                        \
+  }                                                                                                    \
+  HC_KERNEL void hc_reduce_cols_sumf_##TN##_v1(hck_reduce_cols_args p) { reduce_cols_impl<T, R_SUMF, 1, false>(p); } \
+  HC_KERNEL void hc_reduce_cols_sumf_##TN##_vN(hck_reduce_cols_args p) {                               \
+    reduce_cols_impl<T, R_SUMF, VecWidth<T>::value, false>(p);                                         \
+  }                                                                                                    \
+  HC_KERNEL void hc_reduce_cols_final_sumf_##TN(hck_reduce_cols_args p) { reduce_cols_impl<T, R_SUMF, 1, true>(p); } \
+  HC_KERNEL void hc_log_softmax_cols_apply_##TN##_v1(hck_softmax_cols_args p) {                        \
+    softmax_cols_apply_impl<T, 1, false>(p);                                                           \
+  }                                                                                                    \
+  HC_KERNEL void hc_log_softmax_cols_apply_##TN##_vN(hck_softmax_cols_args p) {                        \
+    softmax_cols_apply_impl<T, VecWidth<T>::value, false>(p);                                          \
+  }                                                                                                    \
+  HC_KERNEL void hc_log_softmax_grad_cols_apply_##TN##_v1(hck_softmax_cols_args p) {                   \
+    softmax_cols_apply_impl<T, 1, true>(p);                                                            \
+  }                                                                                                    \
+  HC_KERNEL void hc_log_softmax_grad_cols_apply_##TN##_vN(hck_softmax_cols_args p) {                   \
+    softmax_cols_apply_impl<T, VecWidth<T>::value, true>(p);                                           \
+  }
+DEF_SOFTMAX_COLS(f32, float)
+DEF_SOFTMAX_COLS(f16, half_t)
 
 HC_KERNEL void hc_log_softmax_rows_f32(hck_reduce_args p) { log_softmax_rows_impl<float, 64>(p); }
 HC_KERNEL void hc_log_softmax_rows_f16(hck_reduce_args p) { log_softmax_rows_impl<half_t, 64>(p); }
 HC_KERNEL void hc_log_softmax_rows256_f32(hck_reduce_args p) { log_softmax_rows_impl<float, 256>(p); }
 HC_KERNEL void hc_log_softmax_rows256_f16(hck_reduce_args p) { log_softmax_rows_impl<half_t, 256>(p); }
-HC_KERNEL void hc_log_softmax_cols_f32(hck_reduce_args p) { log_softmax_cols_impl<float>(p); }
-HC_KERNEL void hc_log_softmax_cols_f16(hck_reduce_args p) { log_softmax_cols_impl<half_t>(p); }
 
 // logSoftmaxGrad (BackendCPU.swift:1040-1085): g - sum(g) * expf(x - (logf(sum exp(x - max)) + max)).
 template <typename T, int LANES>
@@ -437,34 +556,10 @@ __device__ __forceinline__ void log_softmax_grad_rows_impl(const hck_reduce_args
                            [&](float gv, uint32_t k) { return gv - gs * expf((float)in[k] - log_sum); });
 }
 
-template <typename T> __device__ __forceinline__ void log_softmax_grad_cols_impl(const hck_reduce_args& p) {
-  const uint32_t jblocks = (p.inner + HCK_BLOCK - 1) / HCK_BLOCK;
-  const uint32_t i = blockIdx.x / jblocks;
-  const uint32_t j = (blockIdx.x - i * jblocks) * HCK_BLOCK + threadIdx.x;
-  if (j >= p.inner) return;
-  const size_t base = (size_t)i * p.reduce * p.inner + j;
-  const T* in = (const T*)p.in + base;
-  const T* grad = (const T*)p.in2 + base;
-  T* out = (T*)p.out + base;
-  float m = 0.0f, gs = 0.0f;
-  for (uint32_t k = 0; k < p.reduce; k++) {
-    float x = (float)in[(size_t)k * p.inner];
-    gs += (float)grad[(size_t)k * p.inner];
-    if (k == 0 || x > m) m = x;
-  }
-  float s = 0.0f;
-  for (uint32_t k = 0; k < p.reduce; k++) s += expf((float)in[(size_t)k * p.inner] - m);
-  const float log_sum = logf(s) + m;
-  for (uint32_t k = 0; k < p.reduce; k++)
-    out[(size_t)k * p.inner] =
-        narrow<T>((float)grad[(size_t)k * p.inner] - gs * expf((float)in[(size_t)k * p.inner] - log_sum));
-}
 HC_KERNEL void hc_log_softmax_grad_rows_f32(hck_reduce_args p) { log_softmax_grad_rows_impl<float, 64>(p); }
 HC_KERNEL void hc_log_softmax_grad_rows_f16(hck_reduce_args p) { log_softmax_grad_rows_impl<half_t, 64>(p); }
 HC_KERNEL void hc_log_softmax_grad_rows256_f32(hck_reduce_args p) { log_softmax_grad_rows_impl<float, 256>(p); }
 HC_KERNEL void hc_log_softmax_grad_rows256_f16(hck_reduce_args p) { log_softmax_grad_rows_impl<half_t, 256>(p); }
-HC_KERNEL void hc_log_softmax_grad_cols_f32(hck_reduce_args p) { log_softmax_grad_cols_impl<float>(p); }
-HC_KERNEL void hc_log_softmax_grad_cols_f16(hck_reduce_args p) { log_softmax_grad_cols_impl<half_t>(p); }
 
 // ---------------------------------------------------------------- normalize
 

@@ -289,7 +289,9 @@ def test_when_fill_triangular_concat_broadcast(hip_backend, oracle_backend):
 # ---------------------------------------------------------------- reductions
 
 REDUCE_SHAPES = [(8, 4096, 1), (37, 513, 1), (5, 1, 1), (3, 7, 1), (1, 100000, 1), (64, 1024, 1), (4, 33, 65),
-                 (1, 300, 4096), (17, 2, 3), (9, 8192, 2)]
+                 (1, 300, 4096), (17, 2, 3), (9, 8192, 2),
+                 # tall and narrow: the reduce axis is split over blocks and combined in a second pass
+                 (2, 5000, 96), (1, 4097, 260), (1, 70000, 8)]
 
 
 @pytest.mark.parametrize("dtype", [F32, F16, I64], ids=["f32", "f16", "i64"])
@@ -353,7 +355,7 @@ def test_argmax_nan_and_tie_rules(hip_backend, oracle_backend):
 def test_log_softmax_and_normalize(hip_backend, oracle_backend, dtype):
     rng = np.random.default_rng(19)
     for shape, axis in [((64, 256), 1), ((16, 8, 32, 32), 3), ((5, 1000), 1), ((7, 33, 9), 1), ((300, 4), 0),
-                        ((2, 1), 1), ((3, 10000), 1)]:
+                        ((2, 1), 1), ((3, 10000), 1), ((4096, 96), 0), ((2, 3000, 40), 1), ((3, 129, 7), 1)]:
         x = rand(rng, shape, dtype, 3.0)
         print("logsoftmax/normalize", dtype.name, shape, axis, flush=True)
         check_close(hip_backend, oracle_backend, lambda: Tensor(data=x).logSoftmax(axis=axis), TOL[dtype])
@@ -469,7 +471,8 @@ def test_scatter_random_floats_within_tolerance(hip_backend, oracle_backend, dty
 def test_log_softmax_grad(hip_backend, oracle_backend, dtype):
     from honeycrisp_amd.backend import Backend
     rng = np.random.default_rng(33)
-    for shape, axis in [((64, 300), 1), ((7, 33, 40), 1), ((5, 1, 9), 2), ((3, 1000), 0), ((2048, 256), 1)]:
+    for shape, axis in [((64, 300), 1), ((7, 33, 40), 1), ((5, 1, 9), 2), ((3, 1000), 0), ((2048, 256), 1),
+                        ((4096, 96), 0), ((2, 3000, 40), 1), ((16, 5000), 1), ((9, 33000), 1)]:
         x, g = rand(rng, shape, dtype, 2.0), rand(rng, shape, dtype)
         def run():
             xt, gt = Tensor(data=x), Tensor(data=g)
