@@ -97,6 +97,7 @@ PROTOTYPES = {
     "hc_log_softmax": (c_int, [_P, c_int, _P, _P, c_int64, c_int64, c_int64]),
     "hc_normalize": (c_int, [_P, c_int, _P, _P, c_int64, c_int64, c_int64, c_float]),
     "hc_gather": (c_int, [_P, c_int, _P, _P, _S, _P, c_int64, c_int64, c_int64, c_int64]),
+    "hc_bitwise_op": (c_int, [_P, c_int, c_int, _P, _S, _P, _S, _P]),
     "hc_scatter": (c_int, [_P, c_int, _P, _P, _S, _P, c_int64, c_int64, c_int64, c_int64, c_int]),
     "hc_log_softmax_grad": (c_int, [_P, c_int, _P, _P, _P, c_int64, c_int64, c_int64]),
     "hc_clamp": (c_int, [_P, c_int, _P, _S, _P, _S, _P, _S, _P]),

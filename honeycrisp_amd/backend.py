@@ -18,7 +18,7 @@ from typing import List, Optional, Sequence, Union
 import numpy as np
 
 from . import _lib
-from .descriptors import (BackendError, BroadcastData, BroadcastStrides, ComparisonOp, DType,
+from .descriptors import (BackendError, BitwiseOp, BroadcastData, BroadcastStrides, ComparisonOp, DType,
                           ElemwiseOp, NumericBinaryOp, ReduceDims, ReduceOp, RepeatDims,
                           ScatterGatherIndices, product)
 
@@ -98,6 +98,17 @@ class Backend:
 
     def scatter(self, a, s, dtype):
         self._ni("scatter")
+
+    def bitwiseOp(self, a, b, op, dtype, count=None):
+        """a, b: BroadcastData, or one of them an integer bit pattern of the element's size
+        (Backend.swift:215-237)."""
+        self._ni("bitwiseOp")
+
+    @staticmethod
+    def scalarBits(value: int, dtype: DType) -> np.ndarray:
+        """The bytes of an element-sized bit pattern (TensorElementBitPattern.bitsForBitwiseOp)."""
+        size = dtype.byteSize
+        return np.frombuffer((int(value) & ((1 << (8 * size)) - 1)).to_bytes(size, "little"), dtype=np.uint8).copy()
 
     def logSoftmaxGrad(self, a, outGrad, dims, dtype):
         self._ni("logSoftmaxGrad")
@@ -541,6 +552,27 @@ class HIPBackend(Backend):
         self._check(self._lib.hc_gather(self._ctx, int(dtype), c_void_p(ad.ptr), c_void_p(idx.ptr), byref(st),
                                         c_void_p(out.ptr), s.outerCount, s.middleCount, s.outCount,
                                         s.innerCount))
+        return out
+
+    def bitwiseOp(self, a, b, op: BitwiseOp, dtype: DType, count: Optional[int] = None) -> HIPData:
+        def operand(x, other):
+            if isinstance(x, BroadcastData):
+                return x
+            shape = other.strides.shape
+            return BroadcastData(BroadcastStrides(shape, [0] * len(shape)), self.upload(self.scalarBits(x, dtype)))
+        if not isinstance(a, BroadcastData) or not isinstance(b, BroadcastData):
+            # tensor (op) scalar: the tensor side arrives as plain data of `count` elements
+            wrap = lambda x: x if isinstance(x, (BroadcastData, int, np.integer)) else BroadcastData(
+                BroadcastStrides.contiguousForShape([count]), x)
+            a, b = wrap(a), wrap(b)
+        if not isinstance(a, BroadcastData) and not isinstance(b, BroadcastData):
+            raise TypeError("bitwiseOp needs at least one tensor operand")
+        a, b = operand(a, b), operand(b, a)
+        out = self.allocate(product(a.strides.shape) * dtype.byteSize)
+        ad, bd = self._dev(a.data), self._dev(b.data)
+        sa, sb = self._s(a.strides), self._s(b.strides)
+        self._check(self._lib.hc_bitwise_op(self._ctx, int(op), int(dtype), c_void_p(ad.ptr), byref(sa),
+                                            c_void_p(bd.ptr), byref(sb), c_void_p(out.ptr)))
         return out
 
     def scatter(self, a, s: ScatterGatherIndices, dtype: DType) -> HIPData:

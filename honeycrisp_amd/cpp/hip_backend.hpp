@@ -217,6 +217,12 @@ class HIPBackend {
                     s.outCount(), s.inner()));
     return out;
   }
+  Data bitwiseOp(const BroadcastData& a, const BroadcastData& b, hc_bitwise_op_kind op, DType dtype) {  // :215
+    Data out = allocate(a.strides.count() * byteSize(dtype));
+    hc_strides sa = a.strides.c(), sb = b.strides.c();
+    check(hc_bitwise_op(ctx_, op, (int)dtype, a.data->ptr(), &sa, b.data->ptr(), &sb, out->ptr()));
+    return out;
+  }
   Data scatter(const Data& a, const ScatterGatherIndices& s, DType dtype) {  // :621
     Data out = allocate((size_t)(s.outer() * s.middle() * s.inner()) * byteSize(dtype));
     hc_strides st = s.indices.strides.c();

@@ -747,6 +747,29 @@ extern "C" int hc_binary_op(hc_ctx* ctx, int op, int dtype, const void* a, const
   return launch(ctx, name, ceil_div(k.d.total_vecs, HCK_BLOCK), 1, &k, sizeof(k));
 }
 
+extern "C" int hc_bitwise_op(hc_ctx* ctx, int op, int dtype, const void* a, const hc_strides* as,
+                             const void* b, const hc_strides* bs, void* out) {
+  REQUIRE(ctx && a && as && b && bs && out, "hc_bitwise_op: null argument");
+  REQUIRE(op >= HC_BIT_OR && op <= HC_BIT_XOR, "hc_bitwise_op: bad op %d", op);
+  REQUIRE(dtype_name(dtype), "hc_bitwise_op: bad dtype %d", dtype);
+  static const char* const names[] = {"or", "and", "xor"};
+  const size_t el = dtype_size(dtype);
+  hck_binary_args k;
+  memset(&k, 0, sizeof(k));
+  int vec;
+  uint64_t total;
+  const hc_strides* ops[] = {as, bs};
+  const void* ptrs[] = {a, b};
+  HC_TRY(make_bcast(2, ops, ptrs, out, vec_for_size(el), &k.d, &vec, &total));
+  if (total == 0) return HC_OK;
+  k.a = a;
+  k.b = b;
+  k.out = out;
+  char name[64];
+  snprintf(name, sizeof(name), "hc_bitwise_%s_b%zu_v%d", names[op], el, vec);
+  return launch(ctx, name, ceil_div(k.d.total_vecs, HCK_BLOCK), 1, &k, sizeof(k));
+}
+
 extern "C" int hc_compare(hc_ctx* ctx, int op, int dtype, const void* a, const hc_strides* as,
                           const void* b, const hc_strides* bs, void* out) {
   REQUIRE(ctx && a && as && b && bs && out, "hc_compare: null argument");

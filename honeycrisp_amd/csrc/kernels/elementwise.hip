@@ -131,6 +131,38 @@ template <typename T, int VEC> __device__ __forceinline__ void when_impl(const h
   store_vec<T, VEC>((T*)p.out, o, r);
 }
 
+// bitwiseOp (BackendCPU.swift:407-443): or / and / xor on the raw bits, any dtype, keyed by
+// element size; the scalar form repeats an element-sized bit pattern.
+enum { BIT_OR = 0, BIT_AND = 1, BIT_XOR = 2 };
+template <int OP, typename U> __device__ __forceinline__ U bitop(U a, U b) {
+  return OP == BIT_OR ? (U)(a | b) : OP == BIT_AND ? (U)(a & b) : (U)(a ^ b);
+}
+template <typename U, int OP, int VEC> __device__ __forceinline__ void bitwise_impl(const hck_binary_args& p) {
+  uint32_t v = blockIdx.x * HCK_BLOCK + threadIdx.x;
+  if (v >= p.d.total_vecs) return;
+  uint32_t off[2];
+  size_t o;
+  bcast_offsets<2, VEC>(p.d, v, off, o);
+  U a[VEC], b[VEC], r[VEC];
+  load_vec<U, VEC>((const U*)p.a, off[0], p.d.inner_stride[0], a);
+  load_vec<U, VEC>((const U*)p.b, off[1], p.d.inner_stride[1], b);
+#pragma unroll
+  for (int i = 0; i < VEC; i++) r[i] = bitop<OP>(a[i], b[i]);
+  store_vec<U, VEC>((U*)p.out, o, r);
+}
+#define DEF_BITWISE(BN, U, V)                                                                         \
+  HC_KERNEL void hc_bitwise_or_##BN##_v##V(hck_binary_args p) { bitwise_impl<U, BIT_OR, V>(p); }      \
+  HC_KERNEL void hc_bitwise_and_##BN##_v##V(hck_binary_args p) { bitwise_impl<U, BIT_AND, V>(p); }    \
+  HC_KERNEL void hc_bitwise_xor_##BN##_v##V(hck_binary_args p) { bitwise_impl<U, BIT_XOR, V>(p); }
+DEF_BITWISE(b1, uint8_t, 1)
+DEF_BITWISE(b1, uint8_t, 16)
+DEF_BITWISE(b2, uint16_t, 1)
+DEF_BITWISE(b2, uint16_t, 8)
+DEF_BITWISE(b4, uint32_t, 1)
+DEF_BITWISE(b4, uint32_t, 4)
+DEF_BITWISE(b8, uint64_t, 1)
+DEF_BITWISE(b8, uint64_t, 2)
+
 // clamp (BackendCPU.swift:704-782): Swift.min(hi, Swift.max(lo, x)) on Float / Int64, where
 // max(a, b) = b >= a ? b : a and min(a, b) = b < a ? b : a. MODE 0 both bounds, 1 lower
 // only, 2 upper only (the unused operand aliases x).

@@ -62,6 +62,13 @@ class ReduceOp(enum.IntEnum):
         return self in (ReduceOp.argmax, ReduceOp.argmin)
 
 
+class BitwiseOp(enum.IntEnum):
+    """BitwiseOps.swift:38-41 (order of include/hchip.h)."""
+    or_ = 0
+    and_ = 1
+    xor = 2
+
+
 class ComparisonOp(enum.IntEnum):
     equal = 0
     notEqual = 1

@@ -16,7 +16,7 @@ from typing import List, Optional, Sequence
 import numpy as np
 
 from .backend import Backend, convert_host_array
-from .descriptors import (BroadcastData, BroadcastStrides, ComparisonOp, DType, ElemwiseOp,
+from .descriptors import (BitwiseOp, BroadcastData, BroadcastStrides, ComparisonOp, DType, ElemwiseOp,
                           NumericBinaryOp, ReduceDims, ReduceOp, RepeatDims, ScatterGatherIndices,
                           product, stridesForShape)
 
@@ -504,6 +504,26 @@ class Tensor:
     def __gt__(self, o): return self._compare(o, ComparisonOp.greater)
     def __ge__(self, o): return self._compare(o, ComparisonOp.greaterEqual)
     __hash__ = object.__hash__
+
+    # -- bitwise operators (BitwiseOps.swift:58-110): same dtype on both sides, or an integer bit
+    # pattern of the element's size
+
+    def _bitwise(self, other, op: BitwiseOp) -> "Tensor":
+        backend = Backend.current()
+        if isinstance(other, Tensor):
+            assert self.dtype == other.dtype, "dtypes for bitwise operator do not match"
+            shape, (ls, rs) = Tensor.lazyBroadcast([self, other])
+            data = backend.bitwiseOp(BroadcastData(ls, self.data), BroadcastData(rs, other.data), op, self.dtype)
+            return Tensor(dataHandle=data, shape=shape, dtype=self.dtype)
+        data = backend.bitwiseOp(self.data, int(other), op, self.dtype, count=product(self.shape))
+        return self._new(data)
+
+    def __and__(self, o): return self._bitwise(o, BitwiseOp.and_)
+    def __rand__(self, o): return self._bitwise(o, BitwiseOp.and_)
+    def __or__(self, o): return self._bitwise(o, BitwiseOp.or_)
+    def __ror__(self, o): return self._bitwise(o, BitwiseOp.or_)
+    def __xor__(self, o): return self._bitwise(o, BitwiseOp.xor)
+    def __rxor__(self, o): return self._bitwise(o, BitwiseOp.xor)
 
     def when(self, isTrue, isFalse, dtype=None) -> "Tensor":
         """When.swift:5-109."""

@@ -236,6 +236,13 @@ int hc_gather(hc_ctx* ctx, int dtype, const void* in, const void* indices,
               const hc_strides* idx_strides, void* out, int64_t outer, int64_t middle,
               int64_t out_count, int64_t inner);
 
+/* Backend.bitwiseOp (Backend.swift:215-237; CPU BackendCPU.swift:407-443): or / and / xor of
+ * the raw element bits over the broadcast shape, any dtype. The tensor-scalar form is the same
+ * call with a 1-element buffer holding the scalar's bit pattern and all-zero strides. */
+typedef enum { HC_BIT_OR = 0, HC_BIT_AND = 1, HC_BIT_XOR = 2 } hc_bitwise_op_kind; /* BitwiseOps.swift:38-41 */
+int hc_bitwise_op(hc_ctx* ctx, int op, int dtype, const void* a, const hc_strides* as, const void* b,
+                  const hc_strides* bs, void* out);
+
 /* Backend.scatter (Backend.swift:621-626; CPU BackendCPU.swift:1149-1188), the adjoint of
  * gather: out[(i*middle + idx)*inner + k] += in[(i*out_count + j)*inner + k] over a zeroed
  * output of outer*middle*inner elements; numeric dtypes. Values sharing an index are added

@@ -709,6 +709,21 @@ void ref_gather(int dtype, const void* in, const int64_t* idx, const ref_strides
   }
 }
 
+/* ---- bitwiseOp (BackendCPU.swift:407-425): byte by byte, as the reference does ---- */
+
+void ref_bitwise_op(int op, int dtype, const void* a, const ref_strides* as, const void* b,
+                    const ref_strides* bs, void* out) {
+  int64_t count = shape_product(as);
+  int64_t el = (int64_t)dtype_size(dtype);
+  const uint8_t *x = (const uint8_t*)a, *y = (const uint8_t*)b;
+  uint8_t* z = (uint8_t*)out;
+  for (int64_t i = 0; i < count * el; i++) {
+    uint8_t p = x[ref_strides_index(as, i / el) * el + i % el];
+    uint8_t q = y[ref_strides_index(bs, i / el) * el + i % el];
+    z[i] = op == 0 ? (uint8_t)(p | q) : op == 1 ? (uint8_t)(p & q) : (uint8_t)(p ^ q);
+  }
+}
+
 /* ---- scatter (BackendCPU.swift:1149-1188): sequential accumulation in Float / Int64 ---- */
 
 void ref_scatter(int dtype, const void* in, const int64_t* idx, const ref_strides* idx_strides,

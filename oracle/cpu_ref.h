@@ -32,6 +32,7 @@
  *                     g - sum(g) * softmax(x) in float64; rows of the result sum to ~0
  *                     when weighted appropriately (sum_k out = sum(g) * (1 - 1) = 0)
  *   clamp             testClamp (:1235-1323), numpy clip / minimum / maximum
+ *   bitwiseOp         testBitwise (:312-333), numpy bitwise ops on int64 / bool / half bits
  */
 #ifndef HC_ORACLE_CPU_REF_H
 #define HC_ORACLE_CPU_REF_H
@@ -102,6 +103,9 @@ void ref_log_softmax(int dtype, const void* in, void* out, int64_t outer, int64_
                      int64_t inner);
 void ref_gather(int dtype, const void* in, const int64_t* idx, const ref_strides* idx_strides,
                 void* out, int64_t outer, int64_t middle, int64_t out_count, int64_t inner);
+/* BackendCPU.swift:407-425: byte-wise or (0) / and (1) / xor (2) over the broadcast shape. */
+void ref_bitwise_op(int op, int dtype, const void* a, const ref_strides* as, const void* b,
+                    const ref_strides* bs, void* out);
 /* BackendCPU.swift:1149-1188. `in` holds outer*out_count*inner elements, `out` receives
  * outer*middle*inner; contributions to one output add up in (i, j, k) order in Float/Int64. */
 void ref_scatter(int dtype, const void* in, const int64_t* idx, const ref_strides* idx_strides,

@@ -41,6 +41,7 @@ _PROTOS = {
     "ref_reduce": (None, [c_int, c_int, _P, _P, c_int64, c_int64, c_int64]),
     "ref_log_softmax": (None, [c_int, _P, _P, c_int64, c_int64, c_int64]),
     "ref_gather": (None, [c_int, _P, _P, _S, _P, c_int64, c_int64, c_int64, c_int64]),
+    "ref_bitwise_op": (None, [c_int, c_int, _P, _S, _P, _S, _P]),
     "ref_scatter": (None, [c_int, _P, _P, _S, _P, c_int64, c_int64, c_int64, c_int64]),
     "ref_log_softmax_grad": (None, [c_int, _P, _P, _P, c_int64, c_int64, c_int64]),
     "ref_clamp": (None, [c_int, _P, _S, _P, _S, _P, _S, _P]),
@@ -236,6 +237,22 @@ class OracleBackend(Backend):
         self.lib.ref_gather(int(dtype), self._host(a).ptr, self._host(s.indices.data).ptr,
                             self._s(s.indices.strides), out.ptr, s.outerCount, s.middleCount, s.outCount,
                             s.innerCount)
+        return out
+
+    def bitwiseOp(self, a, b, op, dtype, count=None):
+        def operand(x, other):
+            if isinstance(x, BroadcastData):
+                return x
+            shape = other.strides.shape
+            return BroadcastData(BroadcastStrides(shape, [0] * len(shape)), self._host(self.scalarBits(x, dtype)))
+        if not isinstance(a, BroadcastData) or not isinstance(b, BroadcastData):
+            wrap = lambda x: BroadcastData(BroadcastStrides.contiguousForShape([count]), x) \
+                if isinstance(x, (CPUData, np.ndarray)) or hasattr(x, "onCPU") else x
+            a, b = wrap(a), wrap(b)
+        a, b = operand(a, b), operand(b, a)
+        out = CPUData(product(a.strides.shape) * dtype.byteSize)
+        self.lib.ref_bitwise_op(int(op), int(dtype), self._host(a.data).ptr, self._s(a.strides),
+                                self._host(b.data).ptr, self._s(b.strides), out.ptr)
         return out
 
     def scatter(self, a, s: ScatterGatherIndices, dtype):

@@ -393,6 +393,17 @@ open class HIPBackend: CPUBackend, @unchecked Sendable {
     return out
   }
 
+  override open func bitwiseOp(
+    _ a: BroadcastData, _ b: BroadcastData, op: BitwiseOp, dtype: Tensor.DType
+  ) async throws -> Tensor.Data {
+    let (da, db) = (try await device(a.data), try await device(b.data))
+    var (sa, sb) = (hcStrides(a.strides), hcStrides(b.strides))
+    let out = try output(a.strides.shape.product() * dtype.byteSize)
+    let kind: Int32 = op == .or ? 0 : op == .and ? 1 : 2
+    try check(hc_bitwise_op(ctx, kind, hcDType(dtype), da.pointer, &sa, db.pointer, &sb, out.pointer))
+    return out
+  }
+
   // MARK: - backward pass and optimizer
 
   override open func scatter(

@@ -515,6 +515,30 @@ def testSoftmax(rng):
         assertClose(out1, out2, atol=tol, rtol=tol)
 
 
+def testBitwise():
+    """BackendTests.swift:312-333."""
+    x = Tensor(data=[0x123456789f, 0xff00ff00, 2, 1], shape=[4], dtype=I64)
+    y = Tensor(data=[1, 2, 0x123456789f, 0xff00ff00], shape=[4], dtype=I64)
+    ints = lambda t: [int(v) for v in t.numpy().reshape(-1)]
+    assert ints(x ^ y) == [0x123456789e, 0xff00ff02, 0x123456789d, 0xff00ff01]
+    assert ints(x & y) == [1, 0, 2, 0]
+    assert ints(x | y) == [0x123456789f, 0xff00ff02, 0x123456789f, 0xff00ff01]
+    assert ints(x ^ 2) == [0x123456789d, 0xff00ff02, 0, 3]
+    assert ints(x | 2) == [0x123456789f, 0xff00ff02, 2, 3]
+    assert ints(x & 2) == [2, 0, 2, 0]
+    assert ints(x & 0x1000000000) == [0x1000000000, 0, 0, 0]
+    assert ints(2 ^ x) == [0x123456789d, 0xff00ff02, 0, 3]
+    assert ints(2 | x) == [0x123456789f, 0xff00ff02, 2, 3]
+    assert ints(2 & x) == [2, 0, 2, 0]
+    assert ints(0x1000000000 & x) == [0x1000000000, 0, 0, 0]
+    # boolean masks, the everyday use (e.g. BackendTests.swift:1262-1264)
+    a = Tensor(data=[1, 0, 1, 0], shape=[4]).cast(BOOL)
+    b = Tensor(data=[1, 1, 0, 0], shape=[2, 1, 4][2:]).cast(BOOL)
+    assertDataEqual(a & b, [1, 0, 0, 0])
+    assertDataEqual(a | b, [1, 1, 1, 0])
+    assertDataEqual(a ^ b, [0, 1, 1, 0])
+
+
 def testSoftmaxGrad(rng):
     """BackendTests.swift:1552-1626, the gradients: logSoftmaxGrad called the way
     Tensor.logSoftmax's backward does (Softmax.swift), golden input gradients for both axes,
@@ -672,6 +696,6 @@ ALL_CASES = [
     testMod, testEquals, testComparison, testSum, testGather, testGatherBroadcastOtherAxis,
     testMatrixMatrixProduct, testBatchedMatmul, testMatrixVectorProduct, testTriangular, testIndexing,
     testElemwise, testRounding, testMinMax, testExpandAndRepeat, testBinaryBroadcast, testFusedBroadcast,
-    testSoftmax, testConcat, testWhen, testSoftmaxGrad, testScatter, testScatterIsAdjointOfGather, testClamp,
+    testSoftmax, testConcat, testWhen, testBitwise, testSoftmaxGrad, testScatter, testScatterIsAdjointOfGather, testClamp,
     testAdam, testNormalizeGrad,
 ]

@@ -533,3 +533,17 @@ def test_normalize_grad(hip_backend, oracle_backend, dtype):
             data = Backend.current().normalizeGrad(xt.data, gt.data, xt.reduceDims(axis), np.float32(1e-3), dtype)
             return Tensor(dataHandle=data, shape=list(shape), dtype=dtype)
         check_close(hip_backend, oracle_backend, run, tol)
+
+
+def test_bitwise_ops(hip_backend, oracle_backend):
+    rng = np.random.default_rng(37)
+    a64, b64 = rng.integers(-2**62, 2**62, size=(33, 1, 40)), rng.integers(-2**62, 2**62, size=(1, 17, 40))
+    ah, bh = rng.standard_normal((1000, 24)).astype(np.float16), rng.standard_normal((1, 24)).astype(np.float16)
+    af = rng.standard_normal((100003,)).astype(np.float32)
+    m1, m2 = rng.random((64, 1, 33)) < 0.5, rng.random((1, 9, 33)) < 0.5
+    for op in ("__and__", "__or__", "__xor__"):
+        check_exact(hip_backend, oracle_backend, lambda: getattr(Tensor(data=a64), op)(Tensor(data=b64)))
+        check_exact(hip_backend, oracle_backend, lambda: getattr(Tensor(data=ah), op)(Tensor(data=bh)))
+        check_exact(hip_backend, oracle_backend, lambda: getattr(Tensor(data=m1), op)(Tensor(data=m2)))
+        check_exact(hip_backend, oracle_backend, lambda: getattr(Tensor(data=a64), op)(0x00ff00ff00ff00ff))
+        check_exact(hip_backend, oracle_backend, lambda: getattr(Tensor(data=af), op)(0x7fffffff))

@@ -333,6 +333,22 @@ def test_clamp_vs_numpy(oracle_backend):
         assert np.array_equal(Tensor(data=xi).clamp(min=-7, max=11).numpy(), np.clip(xi, -7, 11))
 
 
+def test_bitwise_vs_numpy(oracle_backend):
+    rng = np.random.default_rng(25)
+    a = rng.integers(-2**62, 2**62, size=(5, 1, 7))
+    b = rng.integers(-2**62, 2**62, size=(1, 3, 7))
+    with oracle_backend.use():
+        assert np.array_equal((Tensor(data=a) & Tensor(data=b)).numpy(), a & b)
+        assert np.array_equal((Tensor(data=a) | Tensor(data=b)).numpy(), a | b)
+        assert np.array_equal((Tensor(data=a) ^ Tensor(data=b)).numpy(), a ^ b)
+        assert np.array_equal((Tensor(data=a) ^ 0x0f0f).numpy(), a ^ 0x0f0f)
+        h = rng.standard_normal((4, 9)).astype(np.float16)
+        sign = (Tensor(data=h) & 0x8000).numpy().view(np.uint16)
+        assert np.array_equal(sign, h.view(np.uint16) & 0x8000)
+        m1, m2 = rng.random((6, 5)) < 0.5, rng.random((1, 5)) < 0.5
+        assert np.array_equal((Tensor(data=m1) ^ Tensor(data=m2)).numpy(), m1 ^ m2)
+
+
 def test_adamw_composition_vs_float64_formula(oracle_backend):
     """The op-by-op composition against the textbook AdamW update in float64."""
     rng = np.random.default_rng(24)
