@@ -1,0 +1,77 @@
+"""Error behaviour of the C ABI on a live context: status codes and messages instead of
+crashes, mapped to the reference's BackendError cases (Backend.swift:6-16). Every call here
+is rejected on the host before anything is enqueued."""
+import ctypes
+from ctypes import byref, c_float, c_int64, c_size_t, c_void_p
+
+import numpy as np
+import pytest
+
+from honeycrisp_amd import _lib
+from honeycrisp_amd.descriptors import BackendError, DType
+from honeycrisp_amd.tensor import Tensor
+
+pytestmark = pytest.mark.gpu
+
+
+def status_and_message(backend, status):
+    return status, backend._lib.hc_last_error_string().decode()
+
+
+def test_status_codes_for_bad_arguments(hip_backend):
+    lib, ctx = hip_backend._lib, hip_backend._ctx
+    buf = hip_backend.allocate(4096)
+    p = c_void_p(buf.ptr)
+    # unsupported dtype for the MFMA path (int64 matmul stays on the CPU in the reference integration)
+    s, msg = status_and_message(hip_backend, lib.hc_matmul(ctx, int(DType.int64), 1, p, 0, p, 0, 0, 2, 2, 2, p))
+    assert s == _lib.HC_ERR_UNSUPPORTED and "int64" in msg
+    # negative dimension, null pointers
+    assert lib.hc_matmul(ctx, int(DType.float32), 1, p, 0, p, 0, 0, -1, 2, 2, p) == _lib.HC_ERR_INVALID
+    assert lib.hc_matmul(ctx, int(DType.float32), 1, None, 0, p, 0, 0, 2, 2, 2, p) == _lib.HC_ERR_INVALID
+    assert lib.hc_reduce(ctx, 99, int(DType.float32), p, p, 1, 4, 1) == _lib.HC_ERR_INVALID
+    # arg-reduction over an empty axis is refused, a sum over it is fine
+    assert lib.hc_reduce(ctx, 2, int(DType.float32), p, p, 4, 0, 1) == _lib.HC_ERR_INVALID
+    assert lib.hc_reduce(ctx, 0, int(DType.float32), p, p, 4, 0, 1) == _lib.HC_OK
+    # logSoftmax of a non-float dtype
+    assert lib.hc_log_softmax(ctx, int(DType.int64), p, p, 1, 4, 1) == _lib.HC_ERR_UNSUPPORTED
+    # more than 8 dimensions in a stride descriptor
+    bad = _lib.hc_strides()
+    bad.ndim = 9
+    assert lib.hc_broadcast(ctx, int(DType.float32), p, byref(bad), p) == _lib.HC_ERR_INVALID
+    # freeing something the context never handed out, or twice
+    assert lib.hc_free(ctx, c_void_p(buf.ptr + 64)) == _lib.HC_ERR_INVALID
+    q = c_void_p()
+    assert lib.hc_malloc(ctx, c_size_t(1024), byref(q)) == _lib.HC_OK
+    assert lib.hc_free(ctx, q) == _lib.HC_OK
+    assert lib.hc_free(ctx, q) == _lib.HC_ERR_INVALID
+    # an allocation nobody can satisfy
+    s, msg = status_and_message(hip_backend, lib.hc_malloc(ctx, c_size_t(1 << 50), byref(q)))
+    assert s == _lib.HC_ERR_ALLOC and "bytes" in msg
+    # zero-sized work is a no-op, not an error
+    assert lib.hc_matmul(ctx, int(DType.float16), 0, None, 0, None, 0, 0, 8, 8, 8, None) == _lib.HC_OK
+    assert lib.hc_elemwise(ctx, 0, int(DType.float32), None, None, None, c_size_t(0)) == _lib.HC_OK
+    hip_backend.sync()
+
+
+def test_errors_surface_as_backend_errors(hip_backend):
+    with hip_backend.use():
+        x = Tensor(data=np.arange(6, dtype=np.int64).reshape(2, 3))
+        with pytest.raises(BackendError) as e:
+            Tensor.matmul(x, False, x.t(), False, False)          # int64 matmul: not on this backend
+        assert e.value.kind == "notImplemented"
+        with pytest.raises(BackendError) as e:
+            hip_backend.allocate(1 << 50)
+        assert e.value.kind == "allocationFailed"
+        # the context keeps working afterwards
+        assert np.array_equal((x + 1).numpy(), np.arange(6).reshape(2, 3) + 1)
+
+
+def test_replay_api_misuse_is_reported(hip_backend):
+    lib, ctx = hip_backend._lib, hip_backend._ctx
+    g = c_void_p()
+    assert lib.hc_capture_end(ctx, byref(g)) == _lib.HC_ERR_INVALID       # nothing being recorded
+    assert lib.hc_capture_begin(ctx) == _lib.HC_OK
+    assert lib.hc_capture_begin(ctx) == _lib.HC_ERR_INVALID               # one recording at a time
+    assert lib.hc_sync(ctx) == _lib.HC_ERR_INVALID
+    assert lib.hc_capture_abort(ctx) == _lib.HC_OK
+    assert lib.hc_sync(ctx) == _lib.HC_OK
