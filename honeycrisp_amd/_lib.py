@@ -94,6 +94,8 @@ PROTOTYPES = {
     "hc_pow": (c_int, [_P, c_int, _P, c_float, c_float, c_int64, c_int64, _P, _P, c_size_t]),
     "hc_elemwise": (c_int, [_P, c_int, c_int, _P, _P, _P, c_size_t]),
     "hc_reduce": (c_int, [_P, c_int, c_int, _P, _P, c_int64, c_int64, c_int64]),
+    "hc_cumulative": (c_int, [_P, c_int, c_int, _P, _P, c_int64, c_int64, c_int64, c_int, c_int]),
+    "hc_argsort": (c_int, [_P, c_int, _P, _P, c_int64, c_int64, c_int64, c_int]),
     "hc_log_softmax": (c_int, [_P, c_int, _P, _P, c_int64, c_int64, c_int64]),
     "hc_normalize": (c_int, [_P, c_int, _P, _P, c_int64, c_int64, c_int64, c_float]),
     "hc_gather": (c_int, [_P, c_int, _P, _P, _S, _P, c_int64, c_int64, c_int64, c_int64]),

@@ -113,6 +113,15 @@ class Backend:
     def logSoftmaxGrad(self, a, outGrad, dims, dtype):
         self._ni("logSoftmaxGrad")
 
+    def cumulativeSum(self, a, dims, exclusive, reverse, dtype):
+        self._ni("cumulativeSum")
+
+    def cumulativeProd(self, a, dims, exclusive, reverse, dtype):
+        self._ni("cumulativeProd")
+
+    def argsort(self, a, dims, descending, stable, dtype):
+        self._ni("argsort")
+
     def clamp(self, a, min, max, dtype):
         self._ni("clamp")
 
@@ -590,6 +599,28 @@ class HIPBackend(Backend):
         self._check(self._lib.hc_log_softmax_grad(self._ctx, int(dtype), c_void_p(ad.ptr), c_void_p(gd.ptr),
                                                   c_void_p(out.ptr), dims.outerCount, dims.reduceCount,
                                                   dims.innerCount))
+        return out
+
+    def _cumulative(self, op: int, a, dims: ReduceDims, exclusive: bool, reverse: bool, dtype: DType) -> HIPData:
+        out = self.allocate(dims.inCount * dtype.byteSize)
+        ad = self._dev(a)
+        self._check(self._lib.hc_cumulative(self._ctx, op, int(dtype), c_void_p(ad.ptr), c_void_p(out.ptr),
+                                            dims.outerCount, dims.reduceCount, dims.innerCount, int(bool(exclusive)),
+                                            int(bool(reverse))))
+        return out
+
+    def cumulativeSum(self, a, dims: ReduceDims, exclusive: bool, reverse: bool, dtype: DType) -> HIPData:
+        return self._cumulative(0, a, dims, exclusive, reverse, dtype)
+
+    def cumulativeProd(self, a, dims: ReduceDims, exclusive: bool, reverse: bool, dtype: DType) -> HIPData:
+        return self._cumulative(1, a, dims, exclusive, reverse, dtype)
+
+    def argsort(self, a, dims: ReduceDims, descending: bool, stable: bool, dtype: DType) -> HIPData:
+        """Always stable, which `stable=False` permits (Backend.swift:535-545)."""
+        out = self.allocate(dims.inCount * 8)
+        ad = self._dev(a)
+        self._check(self._lib.hc_argsort(self._ctx, int(dtype), c_void_p(ad.ptr), c_void_p(out.ptr), dims.outerCount,
+                                         dims.reduceCount, dims.innerCount, int(bool(descending))))
         return out
 
     def clamp(self, a: BroadcastData, min, max, dtype: DType) -> HIPData:

@@ -236,6 +236,19 @@ class HIPBackend {
                               dims.reduceCount, dims.innerCount));
     return out;
   }
+  Data cumulativeSum(const Data& a, ReduceDims dims, bool exclusive, bool reverse, DType dtype) {  // :548
+    return cumulative(0, a, dims, exclusive, reverse, dtype);
+  }
+  Data cumulativeProd(const Data& a, ReduceDims dims, bool exclusive, bool reverse, DType dtype) {  // :561
+    return cumulative(1, a, dims, exclusive, reverse, dtype);
+  }
+  // Always stable, which `stable == false` allows; axes longer than 4096 are refused (:535)
+  Data argsort(const Data& a, ReduceDims dims, bool descending, bool /*stable*/, DType dtype) {
+    Data out = allocate(dims.inCount() * 8);
+    check(hc_argsort(ctx_, (int)dtype, a->ptr(), out->ptr(), dims.outerCount, dims.reduceCount, dims.innerCount,
+                     descending));
+    return out;
+  }
   // min / max: a BroadcastData with a null `data` means "no bound" (Backend.swift:512-520)
   Data clamp(const BroadcastData& a, const BroadcastData& min, const BroadcastData& max, DType dtype) {
     Data out = allocate(a.strides.count() * byteSize(dtype));
@@ -243,6 +256,12 @@ class HIPBackend {
     check(hc_clamp(ctx_, (int)dtype, a.data->ptr(), &sa, min.data ? min.data->ptr() : nullptr,
                    min.data ? &sl : nullptr, max.data ? max.data->ptr() : nullptr, max.data ? &sh : nullptr,
                    out->ptr()));
+    return out;
+  }
+  Data cumulative(int op, const Data& a, ReduceDims dims, bool exclusive, bool reverse, DType dtype) {
+    Data out = allocate(dims.inCount() * byteSize(dtype));
+    check(hc_cumulative(ctx_, op, (int)dtype, a->ptr(), out->ptr(), dims.outerCount, dims.reduceCount,
+                        dims.innerCount, exclusive, reverse));
     return out;
   }
   struct AdamResult {

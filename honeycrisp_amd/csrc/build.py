@@ -21,6 +21,7 @@ KERNELS = [
     ("elementwise", "elementwise.hip", ["-ffp-contract=off"]),
     ("reduce", "reduce.hip", ["-ffp-contract=off"]),
     ("gather", "gather.hip", []),
+    ("scan", "scan.hip", ["-ffp-contract=off"]),
     ("gemm", "gemm.hip", []),
     ("gemm_f16_fast", "gemm_f16_fast.hip", []),
     ("gemm_dma", "gemm_dma.hip", []),
@@ -48,7 +49,7 @@ def build_kernel(name, src, extra):
 
 def build_all(verbose=True):
     os.makedirs(BUILD_DIR, exist_ok=True)
-    with ThreadPoolExecutor(max_workers=6) as pool:
+    with ThreadPoolExecutor(max_workers=7) as pool:
         futures = [pool.submit(build_kernel, *k) for k in KERNELS]
         for f in futures:
             path = f.result()

@@ -25,6 +25,7 @@ extern "C" {
 extern const unsigned char hc_image_elementwise[], hc_image_elementwise_end[];
 extern const unsigned char hc_image_reduce[], hc_image_reduce_end[];
 extern const unsigned char hc_image_gather[], hc_image_gather_end[];
+extern const unsigned char hc_image_scan[], hc_image_scan_end[];
 extern const unsigned char hc_image_gemm[], hc_image_gemm_end[];
 extern const unsigned char hc_image_gemm_f16_fast[], hc_image_gemm_f16_fast_end[];
 extern const unsigned char hc_image_gemm_dma[], hc_image_gemm_dma_end[];
@@ -141,6 +142,7 @@ extern "C" int hc_init(int device, hc_ctx** out) {
   int s = load_image(ctx, hc_image_elementwise, hc_image_elementwise_end, "elementwise");
   if (s == HC_OK) s = load_image(ctx, hc_image_reduce, hc_image_reduce_end, "reduce");
   if (s == HC_OK) s = load_image(ctx, hc_image_gather, hc_image_gather_end, "gather");
+  if (s == HC_OK) s = load_image(ctx, hc_image_scan, hc_image_scan_end, "scan");
   if (s == HC_OK) s = load_image(ctx, hc_image_gemm, hc_image_gemm_end, "gemm");
   if (s == HC_OK) s = load_image(ctx, hc_image_gemm_f16_fast, hc_image_gemm_f16_fast_end, "gemm_f16_fast");
   if (s == HC_OK) s = load_image(ctx, hc_image_gemm_dma, hc_image_gemm_dma_end, "gemm_dma");
@@ -1188,6 +1190,56 @@ extern "C" int hc_reduce(hc_ctx* ctx, int op, int dtype, const void* in, void* o
   }
   return reduce_cols(ctx, kReduceNames[op], dtype, in, nullptr, out, outer, reduce, inner,
                      op == HC_ARGMAX || op == HC_ARGMIN);
+}
+
+extern "C" int hc_cumulative(hc_ctx* ctx, int op, int dtype, const void* in, void* out, int64_t outer,
+                             int64_t reduce, int64_t inner, int exclusive, int reverse) {
+  REQUIRE(ctx, "hc_cumulative: null context");
+  REQUIRE(op == 0 || op == 1, "hc_cumulative: bad op %d", op);
+  if (dtype != HC_F32 && dtype != HC_F16 && dtype != HC_I64)
+    return fail(HC_ERR_UNSUPPORTED, "hc_cumulative: dtype %d is not numeric", dtype);
+  HC_TRY(check_dims("hc_cumulative", outer, reduce, inner));
+  if (outer * reduce * inner == 0) return HC_OK;
+  REQUIRE(in && out, "hc_cumulative: null pointer");
+  hck_scan_args k;
+  memset(&k, 0, sizeof(k));
+  k.in = in;
+  k.out = out;
+  k.outer = (uint32_t)outer;
+  k.reduce = (uint32_t)reduce;
+  k.inner = (uint32_t)inner;
+  k.exclusive = exclusive != 0;
+  k.reverse = reverse != 0;
+  char name[64];
+  snprintf(name, sizeof(name), "hc_cumulative_%s_%s_%s", op == 0 ? "sum" : "prod", inner == 1 ? "rows" : "cols",
+           dtype_name(dtype));
+  const uint64_t blocks = inner == 1 ? ceil_div((uint64_t)outer, HCK_BLOCK / 64)
+                                     : ceil_div((uint64_t)outer * (uint64_t)inner, HCK_BLOCK);
+  return launch(ctx, name, blocks, 1, &k, sizeof(k));
+}
+
+extern "C" int hc_argsort(hc_ctx* ctx, int dtype, const void* in, void* out, int64_t outer, int64_t reduce,
+                          int64_t inner, int descending) {
+  REQUIRE(ctx, "hc_argsort: null context");
+  if (dtype != HC_F32 && dtype != HC_F16 && dtype != HC_I64)
+    return fail(HC_ERR_UNSUPPORTED, "hc_argsort: dtype %d is not numeric", dtype);
+  HC_TRY(check_dims("hc_argsort", outer, reduce, inner));
+  if (outer * reduce * inner == 0) return HC_OK;
+  REQUIRE(in && out, "hc_argsort: null pointer");
+  if (reduce > 4096)
+    return fail(HC_ERR_UNSUPPORTED, "hc_argsort: axis of %lld elements exceeds the 4096 the in-LDS sort holds",
+                (long long)reduce);
+  hck_scan_args k;
+  memset(&k, 0, sizeof(k));
+  k.in = in;
+  k.out = out;
+  k.outer = (uint32_t)outer;
+  k.reduce = (uint32_t)reduce;
+  k.inner = (uint32_t)inner;
+  k.reverse = descending != 0;
+  char name[64];
+  snprintf(name, sizeof(name), "hc_argsort_%s", dtype_name(dtype));
+  return launch(ctx, name, (uint64_t)outer * (uint64_t)inner, 1, &k, sizeof(k));
 }
 
 extern "C" int hc_log_softmax(hc_ctx* ctx, int dtype, const void* in, void* out, int64_t outer,

@@ -107,6 +107,15 @@ typedef struct {
   uint32_t outer, reduce, inner, pad;
 } hck_softmax_cols_args;
 
+/* cumulativeSum / cumulativeProd / argsort along the middle axis of [outer, reduce, inner].
+ * reverse: scan from the far end (cumulative ops) or sort in descending order (argsort). */
+typedef struct {
+  const void* in;
+  void* out;
+  uint32_t outer, reduce, inner;
+  uint32_t exclusive, reverse, pad;
+} hck_scan_args;
+
 /* Fused AdamW step over `count` contiguous elements; the scalars are the ones the op-by-op
  * composition would pass to its tensor-scalar ops. */
 typedef struct {

@@ -583,6 +583,20 @@ class Tensor:
     def max(self, axis=None, keepdims=False): return self.gatherFromReduce(ReduceOp.argmax, axis, keepdims)
     def min(self, axis=None, keepdims=False): return self.gatherFromReduce(ReduceOp.argmin, axis, keepdims)
 
+    def cumulativeSum(self, axis: int, exclusive=False, reverse=False) -> "Tensor":
+        """ReduceRepeat.swift: running sum along `axis`."""
+        data = Backend.current().cumulativeSum(self.data, self.reduceDims(axis), exclusive, reverse, self.dtype)
+        return self._new(data)
+
+    def cumulativeProd(self, axis: int, exclusive=False, reverse=False) -> "Tensor":
+        data = Backend.current().cumulativeProd(self.data, self.reduceDims(axis), exclusive, reverse, self.dtype)
+        return self._new(data)
+
+    def argsort(self, axis: int, descending=False, stable=False) -> "Tensor":
+        """Indices (int64) that sort the tensor along `axis`."""
+        data = Backend.current().argsort(self.data, self.reduceDims(axis), descending, stable, self.dtype)
+        return self._new(data, dtype=DType.int64)
+
     def mean(self, axis=None, keepdims=False):
         axis = self.positiveAxis(axis)
         n = self.shape[axis] if axis is not None else product(self.shape)

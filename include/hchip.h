@@ -219,6 +219,18 @@ int hc_elemwise(hc_ctx* ctx, int op, int dtype, const void* in, const void* scal
 int hc_reduce(hc_ctx* ctx, int op, int dtype, const void* in, void* out, int64_t outer,
               int64_t reduce, int64_t inner);
 
+/* Backend.cumulativeSum / cumulativeProd (Backend.swift:548-568; CPU BackendCPU.swift:922-998):
+ * op 0 = running sum, 1 = running product along the middle axis of [outer, reduce, inner];
+ * exclusive shifts the result by one position, reverse scans from the far end. */
+int hc_cumulative(hc_ctx* ctx, int op, int dtype, const void* in, void* out, int64_t outer,
+                  int64_t reduce, int64_t inner, int exclusive, int reverse);
+
+/* Backend.argsort (Backend.swift:535-545; CPU BackendCPU.swift:888-920): int64 permutation that
+ * sorts the middle axis, for every (outer, inner) pair. Always stable (equal keys keep their
+ * source order). Axes longer than 4096 return HC_ERR_UNSUPPORTED. */
+int hc_argsort(hc_ctx* ctx, int dtype, const void* in, void* out, int64_t outer, int64_t reduce,
+               int64_t inner, int descending);
+
 /* Backend.logSoftmax (Backend.swift:571-575; CPU BackendCPU.swift:1000-1038). */
 int hc_log_softmax(hc_ctx* ctx, int dtype, const void* in, void* out, int64_t outer,
                    int64_t reduce, int64_t inner);

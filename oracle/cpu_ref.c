@@ -709,6 +709,89 @@ void ref_gather(int dtype, const void* in, const int64_t* idx, const ref_strides
   }
 }
 
+/* ---- cumulativeSum / cumulativeProd (BackendCPU.swift:922-998) ---- */
+
+void ref_cumulative(int op, int dtype, const void* in, void* out, int64_t outer, int64_t reduce,
+                    int64_t inner, int exclusive, int reverse) {
+  size_t total = (size_t)(outer * reduce * inner);
+  if (dtype == REF_I64) {
+    const int64_t* x = (const int64_t*)in;
+    int64_t* z = (int64_t*)out;
+    for (int64_t i = 0; i < outer; i++)
+      for (int64_t j = 0; j < inner; j++) {
+        int64_t run = op == 0 ? 0 : 1;
+        for (int64_t t = 0; t < reduce; t++) {
+          int64_t k = reverse ? reduce - 1 - t : t;
+          int64_t idx = j + (k + i * reduce) * inner;
+          int64_t next = op == 0 ? run + x[idx] : run * x[idx];
+          z[idx] = exclusive ? run : next;
+          run = next;
+        }
+      }
+    return;
+  }
+  float *xo, *zo;
+  const float* x = load_f(dtype, in, total, &xo);
+  float* z = out_f(dtype, out, total, &zo);
+  for (int64_t i = 0; i < outer; i++)
+    for (int64_t j = 0; j < inner; j++) {
+      float run = op == 0 ? 0.0f : 1.0f;
+      for (int64_t t = 0; t < reduce; t++) {
+        int64_t k = reverse ? reduce - 1 - t : t;
+        int64_t idx = j + (k + i * reduce) * inner;
+        float next = op == 0 ? run + x[idx] : run * x[idx];
+        z[idx] = exclusive ? run : next;
+        run = next;
+      }
+    }
+  store_f(dtype, out, total, zo);
+  free(xo);
+}
+
+/* ---- argsort (BackendCPU.swift:888-920), stable: insertion into a merge sort ---- */
+
+static void argsort_merge(const double* key, int64_t* idx, int64_t* tmp, int64_t n, int descending) {
+  for (int64_t width = 1; width < n; width *= 2) {
+    for (int64_t lo = 0; lo < n; lo += 2 * width) {
+      int64_t mid = lo + width < n ? lo + width : n, hi = lo + 2 * width < n ? lo + 2 * width : n;
+      int64_t a = lo, b = mid, o = lo;
+      while (a < mid && b < hi) {
+        /* take from the right run only if it is strictly ahead: equal keys keep their order */
+        int right = descending ? key[idx[b]] > key[idx[a]] : key[idx[b]] < key[idx[a]];
+        tmp[o++] = right ? idx[b++] : idx[a++];
+      }
+      while (a < mid) tmp[o++] = idx[a++];
+      while (b < hi) tmp[o++] = idx[b++];
+    }
+    memcpy(idx, tmp, (size_t)n * sizeof(int64_t));
+  }
+}
+
+void ref_argsort(int dtype, const void* in, int64_t* out, int64_t outer, int64_t reduce, int64_t inner,
+                 int descending) {
+  size_t total = (size_t)(outer * reduce * inner);
+  float* xo = NULL;
+  const float* xf = dtype == REF_I64 ? NULL : load_f(dtype, in, total, &xo);
+  double* key = (double*)malloc((size_t)(reduce ? reduce : 1) * sizeof(double));
+  int64_t* idx = (int64_t*)malloc((size_t)(reduce ? reduce : 1) * sizeof(int64_t));
+  int64_t* tmp = (int64_t*)malloc((size_t)(reduce ? reduce : 1) * sizeof(int64_t));
+  for (int64_t i = 0; i < outer; i++)
+    for (int64_t j = 0; j < inner; j++) {
+      for (int64_t k = 0; k < reduce; k++) {
+        int64_t src = j + (k + i * reduce) * inner;
+        /* int64 keys of the tests fit a double exactly (|x| < 2^53) */
+        key[k] = dtype == REF_I64 ? (double)((const int64_t*)in)[src] : (double)xf[src];
+        idx[k] = k;
+      }
+      argsort_merge(key, idx, tmp, reduce, descending);
+      for (int64_t k = 0; k < reduce; k++) out[j + (k + i * reduce) * inner] = idx[k];
+    }
+  free(key);
+  free(idx);
+  free(tmp);
+  free(xo);
+}
+
 /* ---- bitwiseOp (BackendCPU.swift:407-425): byte by byte, as the reference does ---- */
 
 void ref_bitwise_op(int op, int dtype, const void* a, const ref_strides* as, const void* b,

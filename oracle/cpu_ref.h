@@ -32,6 +32,9 @@
  *                     g - sum(g) * softmax(x) in float64; rows of the result sum to ~0
  *                     when weighted appropriately (sum_k out = sum(g) * (1 - 1) = 0)
  *   clamp             testClamp (:1235-1323), numpy clip / minimum / maximum
+ *   cumulative ops    testCumulativeSum / testCumulativeProd vectors (:466-524), numpy cumsum /
+ *                     cumprod incl. exclusive and reversed forms
+ *   argsort           testArgsort (:526-564) incl. its stable-order vectors, numpy stable argsort
  *   bitwiseOp         testBitwise (:312-333), numpy bitwise ops on int64 / bool / half bits
  */
 #ifndef HC_ORACLE_CPU_REF_H
@@ -106,6 +109,15 @@ void ref_gather(int dtype, const void* in, const int64_t* idx, const ref_strides
 /* BackendCPU.swift:407-425: byte-wise or (0) / and (1) / xor (2) over the broadcast shape. */
 void ref_bitwise_op(int op, int dtype, const void* a, const ref_strides* as, const void* b,
                     const ref_strides* bs, void* out);
+/* BackendCPU.swift:922-998: running sum (op 0) or product (op 1) along the middle axis of
+ * [outer, reduce, inner] in Float / Int64, optionally exclusive and / or from the far end. */
+void ref_cumulative(int op, int dtype, const void* in, void* out, int64_t outer, int64_t reduce,
+                    int64_t inner, int exclusive, int reverse);
+/* BackendCPU.swift:888-920: for every (outer, inner) pair the permutation (int64) that sorts the
+ * reduce axis. The reference's comparison sort leaves the order of equal keys open; this one
+ * is stable (equal keys keep their source order), which the `stable` flag asks for. */
+void ref_argsort(int dtype, const void* in, int64_t* out, int64_t outer, int64_t reduce, int64_t inner,
+                 int descending);
 /* BackendCPU.swift:1149-1188. `in` holds outer*out_count*inner elements, `out` receives
  * outer*middle*inner; contributions to one output add up in (i, j, k) order in Float/Int64. */
 void ref_scatter(int dtype, const void* in, const int64_t* idx, const ref_strides* idx_strides,

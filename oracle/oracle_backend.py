@@ -41,6 +41,8 @@ _PROTOS = {
     "ref_reduce": (None, [c_int, c_int, _P, _P, c_int64, c_int64, c_int64]),
     "ref_log_softmax": (None, [c_int, _P, _P, c_int64, c_int64, c_int64]),
     "ref_gather": (None, [c_int, _P, _P, _S, _P, c_int64, c_int64, c_int64, c_int64]),
+    "ref_cumulative": (None, [c_int, c_int, _P, _P, c_int64, c_int64, c_int64, c_int, c_int]),
+    "ref_argsort": (None, [c_int, _P, _P, c_int64, c_int64, c_int64, c_int]),
     "ref_bitwise_op": (None, [c_int, c_int, _P, _S, _P, _S, _P]),
     "ref_scatter": (None, [c_int, _P, _P, _S, _P, c_int64, c_int64, c_int64, c_int64]),
     "ref_log_softmax_grad": (None, [c_int, _P, _P, _P, c_int64, c_int64, c_int64]),
@@ -237,6 +239,24 @@ class OracleBackend(Backend):
         self.lib.ref_gather(int(dtype), self._host(a).ptr, self._host(s.indices.data).ptr,
                             self._s(s.indices.strides), out.ptr, s.outerCount, s.middleCount, s.outCount,
                             s.innerCount)
+        return out
+
+    def cumulativeSum(self, a, dims, exclusive, reverse, dtype):
+        return self._cumulative(0, a, dims, exclusive, reverse, dtype)
+
+    def cumulativeProd(self, a, dims, exclusive, reverse, dtype):
+        return self._cumulative(1, a, dims, exclusive, reverse, dtype)
+
+    def _cumulative(self, op, a, dims, exclusive, reverse, dtype):
+        out = CPUData(dims.inCount * dtype.byteSize)
+        self.lib.ref_cumulative(op, int(dtype), self._host(a).ptr, out.ptr, dims.outerCount, dims.reduceCount,
+                                dims.innerCount, int(exclusive), int(reverse))
+        return out
+
+    def argsort(self, a, dims, descending, stable, dtype):
+        out = CPUData(dims.inCount * 8)
+        self.lib.ref_argsort(int(dtype), self._host(a).ptr, out.ptr, dims.outerCount, dims.reduceCount,
+                             dims.innerCount, int(descending))
         return out
 
     def bitwiseOp(self, a, b, op, dtype, count=None):

@@ -438,6 +438,57 @@ open class HIPBackend: CPUBackend, @unchecked Sendable {
     return out
   }
 
+  private func cumulative(
+    _ op: Int32, _ a: Tensor.Data, _ dims: ReduceDims, _ exclusive: Bool, _ reverse: Bool,
+    _ dtype: Tensor.DType
+  ) async throws -> Tensor.Data {
+    let da = try await device(a)
+    let out = try output(dims.inCount * dtype.byteSize)
+    try check(
+      hc_cumulative(
+        ctx, op, hcDType(dtype), da.pointer, out.pointer, Int64(dims.outerCount),
+        Int64(dims.reduceCount), Int64(dims.innerCount), exclusive ? 1 : 0, reverse ? 1 : 0))
+    return out
+  }
+
+  override open func cumulativeSum(
+    _ a: Tensor.Data, dims: ReduceDims, exclusive: Bool, reverse: Bool, dtype: Tensor.DType
+  ) async throws -> Tensor.Data {
+    guard dtype != .bool else {
+      return try await super.cumulativeSum(
+        a, dims: dims, exclusive: exclusive, reverse: reverse, dtype: dtype)
+    }
+    return try await cumulative(0, a, dims, exclusive, reverse, dtype)
+  }
+
+  override open func cumulativeProd(
+    _ a: Tensor.Data, dims: ReduceDims, exclusive: Bool, reverse: Bool, dtype: Tensor.DType
+  ) async throws -> Tensor.Data {
+    guard dtype != .bool else {
+      return try await super.cumulativeProd(
+        a, dims: dims, exclusive: exclusive, reverse: reverse, dtype: dtype)
+    }
+    return try await cumulative(1, a, dims, exclusive, reverse, dtype)
+  }
+
+  /// The device sort is stable whatever `stable` says; axes longer than 4096 elements go to the
+  /// inherited CPU implementation.
+  override open func argsort(
+    _ a: Tensor.Data, dims: ReduceDims, descending: Bool, stable: Bool, dtype: Tensor.DType
+  ) async throws -> Tensor.Data {
+    guard dtype != .bool && dims.reduceCount <= 4096 else {
+      return try await super.argsort(
+        a, dims: dims, descending: descending, stable: stable, dtype: dtype)
+    }
+    let da = try await device(a)
+    let out = try output(dims.inCount * 8)
+    try check(
+      hc_argsort(
+        ctx, hcDType(dtype), da.pointer, out.pointer, Int64(dims.outerCount),
+        Int64(dims.reduceCount), Int64(dims.innerCount), descending ? 1 : 0))
+    return out
+  }
+
   override open func clamp<T: NumericTensorElement>(
     _ a: BroadcastData, _: T.Type, min: TensorOrScalar<T>?, max: TensorOrScalar<T>?,
     dtype: Tensor.DType

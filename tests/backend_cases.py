@@ -515,6 +515,48 @@ def testSoftmax(rng):
         assertClose(out1, out2, atol=tol, rtol=tol)
 
 
+def testCumulativeSum():
+    """BackendTests.swift:466-500 (forward values)."""
+    for dtype in (F16, F32, I64):
+        raw = Tensor(data=[1, 2, 3, -2, 4, 7], shape=[2, 3], dtype=dtype)
+        for exclusive, reverse, want in [(False, False, [1, 3, 6, -2, 2, 9]), (True, False, [0, 1, 3, 0, -2, 2]),
+                                         (False, True, [6, 5, 3, 9, 11, 7]), (True, True, [5, 3, 0, 11, 7, 0])]:
+            assertDataEqual(raw.cumulativeSum(1, exclusive, reverse), want)
+            ax0 = raw.t().cumulativeSum(1, exclusive, reverse).t()
+            assertDataEqual(ax0, raw.cumulativeSum(0, exclusive, reverse))
+
+
+def testCumulativeProd():
+    """BackendTests.swift:502-524."""
+    for dtype in (F16, F32, I64):
+        raw = Tensor(data=[1, 2, 3, -2, 4, -2], shape=[2, 3], dtype=dtype)
+        for exclusive, reverse, want in [(False, False, [1, 2, 6, -2, -8, 16]), (True, False, [1, 1, 2, 1, -2, -8]),
+                                         (False, True, [6, 6, 3, 16, -8, -2]), (True, True, [6, 3, 1, -8, -2, 1])]:
+            assertDataEqual(raw.cumulativeProd(1, exclusive, reverse), want)
+            ax0 = raw.t().cumulativeProd(1, exclusive, reverse).t()
+            assertDataEqual(ax0, raw.cumulativeProd(0, exclusive, reverse))
+
+
+def testArgsort(rng):
+    """BackendTests.swift:526-564: gathering with the sorted indices sorts every axis, and the
+    stable order of equal keys."""
+    for dtype in (F16, F32, I64):
+        values = rng.integers(-30, 31, size=(2, 3, 4))
+        unsorted = Tensor(data=values, dtype=I64).cast(dtype)
+        for descending in (False, True):
+            for stable in (False, True):
+                for axis in (0, 1, 2):
+                    want = np.sort(values, axis=axis)
+                    if descending:
+                        want = np.flip(want, axis=axis)
+                    idx = unsorted.argsort(axis, descending=descending, stable=stable)
+                    assert idx.dtype == I64
+                    assertDataEqual(unsorted.gather(axis, idx), want.reshape(-1))
+            ties = Tensor(data=[1, 2, 3, 1, 4, 3, 5, 3], shape=[8]).cast(dtype)
+            expected = [6, 4, 2, 5, 7, 1, 0, 3] if descending else [0, 3, 1, 2, 5, 7, 4, 6]
+            assertDataEqual(ties.argsort(0, descending=descending, stable=True), expected)
+
+
 def testBitwise():
     """BackendTests.swift:312-333."""
     x = Tensor(data=[0x123456789f, 0xff00ff00, 2, 1], shape=[4], dtype=I64)
@@ -696,6 +738,6 @@ ALL_CASES = [
     testMod, testEquals, testComparison, testSum, testGather, testGatherBroadcastOtherAxis,
     testMatrixMatrixProduct, testBatchedMatmul, testMatrixVectorProduct, testTriangular, testIndexing,
     testElemwise, testRounding, testMinMax, testExpandAndRepeat, testBinaryBroadcast, testFusedBroadcast,
-    testSoftmax, testConcat, testWhen, testBitwise, testSoftmaxGrad, testScatter, testScatterIsAdjointOfGather, testClamp,
+    testSoftmax, testConcat, testWhen, testCumulativeSum, testCumulativeProd, testArgsort, testBitwise, testSoftmaxGrad, testScatter, testScatterIsAdjointOfGather, testClamp,
     testAdam, testNormalizeGrad,
 ]

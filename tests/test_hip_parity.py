@@ -547,3 +547,44 @@ def test_bitwise_ops(hip_backend, oracle_backend):
         check_exact(hip_backend, oracle_backend, lambda: getattr(Tensor(data=m1), op)(Tensor(data=m2)))
         check_exact(hip_backend, oracle_backend, lambda: getattr(Tensor(data=a64), op)(0x00ff00ff00ff00ff))
         check_exact(hip_backend, oracle_backend, lambda: getattr(Tensor(data=af), op)(0x7fffffff))
+
+
+@pytest.mark.parametrize("dtype", [F32, F16, I64], ids=["f32", "f16", "i64"])
+def test_cumulative_ops(hip_backend, oracle_backend, dtype):
+    rng = np.random.default_rng(38)
+    for shape, axis in [((7, 1000), 1), ((3, 257, 5), 1), ((5000, 3), 0), ((4, 1), 1), ((2, 64), 1), ((1, 70000), 1)]:
+        # small integers: every partial sum is exact, so the scan order cannot matter
+        x = rng.integers(-3, 4, size=shape)
+        x = x if dtype == I64 else x.astype(dtype.numpy)
+        for exclusive in (False, True):
+            for reverse in (False, True):
+                if dtype == F16 and shape[axis] > 2000:
+                    continue        # running sums leave the range in which halfs are exact integers
+                check_exact(hip_backend, oracle_backend,
+                            lambda: Tensor(data=x).cumulativeSum(axis, exclusive=exclusive, reverse=reverse))
+        signs = rng.choice([-1, 1], size=shape) * rng.choice([1, 1, 1, 2], size=shape)
+        short = tuple(slice(0, 12) if a == axis else slice(None) for a in range(len(shape)))
+        y = signs[short] if dtype == I64 else signs[short].astype(dtype.numpy)
+        check_exact(hip_backend, oracle_backend, lambda: Tensor(data=y).cumulativeProd(axis))
+        check_exact(hip_backend, oracle_backend, lambda: Tensor(data=y).cumulativeProd(axis, exclusive=True, reverse=True))
+    if dtype != I64:
+        r = rand(rng, (16, 3000), dtype)
+        got, want = both(hip_backend, oracle_backend, lambda: Tensor(data=r).cumulativeSum(1))
+        assert_close_arrays(got, want, TOL[dtype] * 60, TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", [F32, F16, I64], ids=["f32", "f16", "i64"])
+def test_argsort(hip_backend, oracle_backend, dtype):
+    rng = np.random.default_rng(39)
+    for shape, axis in [((9, 100), 1), ((3, 4096), 1), ((5, 77, 6), 1), ((300, 2), 0), ((4, 1), 1), ((2, 1025), 1)]:
+        x = rng.integers(-20, 21, size=shape)           # many ties: the stable order is pinned
+        x = x if dtype == I64 else x.astype(dtype.numpy)
+        for descending in (False, True):
+            check_exact(hip_backend, oracle_backend, lambda: Tensor(data=x).argsort(axis, descending=descending, stable=True))
+    if dtype != I64:
+        f = rand(rng, (6, 999), dtype)
+        f[0, :5] = [0.0, -0.0, np.inf, -np.inf, 0.0]
+        check_exact(hip_backend, oracle_backend, lambda: Tensor(data=f).argsort(1))
+    with hip_backend.use():
+        with pytest.raises(Exception):
+            Tensor(data=np.zeros((2, 5000), np.float32)).argsort(1)     # beyond the in-LDS sort: refused, not wrong

@@ -333,6 +333,28 @@ def test_clamp_vs_numpy(oracle_backend):
         assert np.array_equal(Tensor(data=xi).clamp(min=-7, max=11).numpy(), np.clip(xi, -7, 11))
 
 
+def test_cumulative_and_argsort_vs_numpy(oracle_backend):
+    rng = np.random.default_rng(26)
+    x = rng.integers(-4, 5, size=(3, 17, 5)).astype(np.float32)       # exact in float: order cannot matter
+    with oracle_backend.use():
+        t = Tensor(data=x)
+        for axis in (0, 1, 2):
+            assert np.array_equal(t.cumulativeSum(axis).numpy(), np.cumsum(x, axis=axis))
+            rev = np.flip(np.cumsum(np.flip(x, axis), axis=axis), axis)
+            assert np.array_equal(t.cumulativeSum(axis, reverse=True).numpy(), rev)
+            assert np.array_equal(t.cumulativeSum(axis, exclusive=True).numpy(), np.cumsum(x, axis=axis) - x)
+        small = rng.integers(1, 3, size=(4, 9)).astype(np.int64) * rng.choice([-1, 1], size=(4, 9))
+        assert np.array_equal(Tensor(data=small).cumulativeProd(1).numpy(), np.cumprod(small, axis=1))
+        keys = rng.integers(-5, 6, size=(6, 40, 3))
+        for axis in (0, 1, 2):
+            got = Tensor(data=keys).argsort(axis, stable=True).numpy()
+            assert np.array_equal(got, np.argsort(keys, axis=axis, kind="stable"))
+            got = Tensor(data=keys).argsort(axis, descending=True, stable=True).numpy()
+            assert np.array_equal(got, np.argsort(-keys, axis=axis, kind="stable"))
+        f = rng.standard_normal((5, 33)).astype(np.float32)
+        assert np.array_equal(Tensor(data=f).argsort(1).numpy(), np.argsort(f, axis=1, kind="stable"))
+
+
 def test_bitwise_vs_numpy(oracle_backend):
     rng = np.random.default_rng(25)
     a = rng.integers(-2**62, 2**62, size=(5, 1, 7))
