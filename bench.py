@@ -155,6 +155,25 @@ def headline(backend, steps, warmup):
         "per_layout_tflops": {k: round(flops / (v * 1e-3) / 1e12, 2) for k, v in layout_ms.items()},
         "per_layout_ms": {k: round(v, 4) for k, v in layout_ms.items()},
     }
+    # What the matrix cores alone sustain on these bit patterns: the same MFMA sequence as the
+    # GEMM's inner loop with no memory traffic at all. The board lowers the shader clock until
+    # power fits, and MFMA power depends on how many operand bits toggle, so this, not the
+    # 2.4 GHz figure, is the rate a GEMM on this data could approach.
+    probe_in = dev[("a", False)]
+    for _ in range(200):
+        probe_flops = backend.probeMfma(probe_in)
+    e0, e1 = events.new(), events.new()
+    events.record(e0)
+    for _ in range(200):
+        backend.probeMfma(probe_in)
+    events.record(e1)
+    backend.sync()
+    probe_tflops = 200 * probe_flops / (events.elapsed_ms(e0, e1) * 1e-3) / 1e12
+    events.free(e0)
+    events.free(e1)
+    roofline["mfma_only_same_data"] = {
+        "tflops": round(probe_tflops, 1), "gemm_frac_of_it": round(achieved / probe_tflops, 4),
+        "note": "MFMA-only kernel on the GEMM's operand bits, clock as set by power management"}
     return value, ms_per_step, roofline, (a, b)
 
 

@@ -22,6 +22,7 @@ KERNELS = [
     ("reduce", "reduce.hip", ["-ffp-contract=off"]),
     ("gather", "gather.hip", []),
     ("scan", "scan.hip", ["-ffp-contract=off"]),
+    ("probe", "probe.hip", []),
     ("gemm", "gemm.hip", []),
     ("gemm_f16_fast", "gemm_f16_fast.hip", []),
     ("gemm_dma", "gemm_dma.hip", []),
@@ -49,7 +50,7 @@ def build_kernel(name, src, extra):
 
 def build_all(verbose=True):
     os.makedirs(BUILD_DIR, exist_ok=True)
-    with ThreadPoolExecutor(max_workers=7) as pool:
+    with ThreadPoolExecutor(max_workers=8) as pool:
         futures = [pool.submit(build_kernel, *k) for k in KERNELS]
         for f in futures:
             path = f.result()

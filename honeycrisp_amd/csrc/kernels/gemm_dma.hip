@@ -41,9 +41,14 @@
 #include "common.hip.h"
 
 // Measurement switches (never set in the shipped build): bit0 no DMA in the K loop, bit1 no
-// wait/barrier, bit2 no LDS reads in the K loop. Results are wrong with any bit set.
+// wait/barrier, bit2 no LDS reads in the K loop, bit3 every K-step fetches slice 0 again, bit4
+// only every other DMA instruction, bit5 every DMA instruction fetches the same 1 KiB. Results are wrong with any bit set.
 #ifndef HC_EXP
 #define HC_EXP 0
+#endif
+// cache-policy bits of the DMA loads (0 = default policy)
+#ifndef HC_DMA_AUX
+#define HC_DMA_AUX 0
 #endif
 #ifndef HC_READS_PER_SLOT
 #define HC_READS_PER_SLOT 0
@@ -179,11 +184,15 @@ template <typename T, int ROWS, int MODE> struct DmaOperand {
   __device__ __forceinline__ void dma(int i, const T* base, uint32_t k0, char* region, uint32_t kend = 0,
                                       const void* zeros = nullptr) const {
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const char* src = (const char*)base + (size_t)k0 * kstride + goff[i];
+    // The empty asm keeps the zero-extension of the lane offset next to the load, so that the
+    // load takes the form "scalar base + 32-bit lane offset" with no vector add in front of it.
+    uint32_t off = goff[i];
+    asm volatile("" : "+v"(off));
+    const char* src = (const char*)base + (size_t)k0 * kstride + off;
     if (kend != 0 && k0 + 64 / ES > kend) {  // wave-uniform
       if (k0 + klocal(i) >= kend) src = (const char*)zeros;
     }
-    __builtin_amdgcn_global_load_lds((const GLOBAL_AS void*)src, (LDS_AS void*)(region + (wave * NI + i) * 1024), 16, 0, 0);
+    __builtin_amdgcn_global_load_lds((const GLOBAL_AS void*)src, (LDS_AS void*)(region + (wave * NI + i) * 1024), 16, 0, HC_DMA_AUX);
   }
 
   // Read number u of sub-step s into the operand registers of tile u (DMA_K), half u%2 of
@@ -274,6 +283,13 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
   // unit u of the DMA of the K-slice starting at k0
   auto dma_unit = [&](int u, uint32_t k0, char* stage, bool in_loop = false) {
     if ((HC_EXP & 1) && in_loop) return;
+    if ((HC_EXP & 16) && in_loop && (u & 1)) return;
+    if ((HC_EXP & 8) && in_loop) k0 = 0;
+    if ((HC_EXP & 32) && in_loop) {  // every instruction fetches the same 1 KiB: first-level cache hits
+      if (u < OpA::NI) oa.dma(0, A, 0, stage + u * 1024, kend, p.zeros);
+      else if (u < NDMA) ob.dma(0, B, 0, stage + A_BYTES + (u - OpA::NI) * 1024, kend, p.zeros);
+      return;
+    }
     if (u < OpA::NI) oa.dma(u, A, k0, stage, kend, p.zeros);
     else if (u < NDMA) ob.dma(u - OpA::NI, B, k0, stage + A_BYTES, kend, p.zeros);
   };
@@ -302,6 +318,9 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
 
   const uint32_t nk = (p.K + BK - 1) / BK;
   Frags f0, f1;
+#ifdef HC_PROBE_WAITS
+  uint64_t probe_wait_dma = 0, probe_wait_bar = 0;  // cycles this wave spent in the two waits
+#endif
 
   // K-step j out of `cur`; `nxt` holds K-step j+1, `prev` held K-step j-1.
   auto step = [&](char* cur, char* nxt, char* prev, uint32_t j) {
@@ -316,8 +335,18 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
       __builtin_amdgcn_sched_barrier(0);
     }
     if (!(HC_EXP & 2)) {
+#ifdef HC_PROBE_WAITS
+      const uint64_t w0 = __builtin_readcyclecounter();
+      wait_dma<2 * NDMA>();
+      const uint64_t w1 = __builtin_readcyclecounter();
+      lds_barrier();
+      const uint64_t w2 = __builtin_readcyclecounter();
+      probe_wait_dma += w1 - w0;
+      probe_wait_bar += w2 - w1;
+#else
       wait_dma<2 * NDMA>();  // K-step j+1 of this wave has landed ...
       lds_barrier();         // ... and everybody's; nobody reads cur any more
+#endif
     }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -346,7 +375,7 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
 #pragma unroll
   for (int u = 0; u < READS; u++) read_unit(f0, lds0, 0, u);
 
-#ifdef HC_PROBE_CLOCKS
+#if defined(HC_PROBE_CLOCKS) || defined(HC_PROBE_WAITS)
   const uint64_t probe_c0 = __builtin_readcyclecounter(), probe_r0 = __builtin_amdgcn_s_memrealtime();
 #endif
   uint32_t j = 0;
@@ -360,9 +389,10 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
   if (j + 1 < nk) step(lds1, lds2, lds0, j + 1);
   if (j + 2 < nk) step(lds2, lds3, lds1, j + 2);
   wait_dma<0>();  // no LDS write of this workgroup may be in flight when it ends
-#ifdef HC_PROBE_CLOCKS
+#if defined(HC_PROBE_CLOCKS) || defined(HC_PROBE_WAITS)
   // measurement build: the first 16 bytes of the block's C tile receive the K-loop duration
-  // in shader cycles and in 100 MHz ticks instead of results
+  // in shader cycles and in 100 MHz ticks instead of results (HC_PROBE_WAITS: 32 bytes per
+  // wave, with the cycles spent waiting for DMA and at the barrier)
   const uint64_t probe_c1 = __builtin_readcyclecounter(), probe_r1 = __builtin_amdgcn_s_memrealtime();
 #endif
 
@@ -409,6 +439,16 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
     }
     asm volatile("" ::: "memory");
   }
+#ifdef HC_PROBE_WAITS
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) {
+    uint64_t* dst = reinterpret_cast<uint64_t*>(C + (size_t)m0 * p.c_rs + n0) + (threadIdx.x >> 6) * 4;
+    dst[0] = probe_c1 - probe_c0;
+    dst[1] = probe_r1 - probe_r0;
+    dst[2] = probe_wait_dma;
+    dst[3] = probe_wait_bar;
+  }
+#endif
 #ifdef HC_PROBE_CLOCKS
   __syncthreads();
   if (threadIdx.x == 0) {
