@@ -242,7 +242,7 @@ class HIPBackend {
   Data cumulativeProd(const Data& a, ReduceDims dims, bool exclusive, bool reverse, DType dtype) {  // :561
     return cumulative(1, a, dims, exclusive, reverse, dtype);
   }
-  // Always stable, which `stable == false` allows; axes longer than 4096 are refused (:535)
+  // Always stable, which `stable == false` allows (:535)
   Data argsort(const Data& a, ReduceDims dims, bool descending, bool /*stable*/, DType dtype) {
     Data out = allocate(dims.inCount() * 8);
     check(hc_argsort(ctx_, (int)dtype, a->ptr(), out->ptr(), dims.outerCount, dims.reduceCount, dims.innerCount,

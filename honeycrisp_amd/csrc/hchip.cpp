@@ -1228,9 +1228,41 @@ extern "C" int hc_argsort(hc_ctx* ctx, int dtype, const void* in, void* out, int
   HC_TRY(check_dims("hc_argsort", outer, reduce, inner));
   if (outer * reduce * inner == 0) return HC_OK;
   REQUIRE(in && out, "hc_argsort: null pointer");
-  if (reduce > 4096)
-    return fail(HC_ERR_UNSUPPORTED, "hc_argsort: axis of %lld elements exceeds the 4096 the in-LDS sort holds",
-                (long long)reduce);
+  if (reduce > 4096) {
+    // runs of 4096 sorted in LDS, then merged pairwise; two sets of (key, index) arrays alternate
+    const uint64_t lines = (uint64_t)outer * (uint64_t)inner, total = lines * (uint64_t)reduce;
+    Scratch scratch(ctx);
+    void *keys[2], *idx[2];
+    for (int b = 0; b < 2; b++) {
+      HC_TRY(scratch.get(total * sizeof(uint64_t), &keys[b]));
+      HC_TRY(scratch.get(total * sizeof(uint32_t), &idx[b]));
+    }
+    hck_sort_args s;
+    memset(&s, 0, sizeof(s));
+    s.in = in;
+    s.out = out;
+    s.outer = (uint32_t)outer;
+    s.reduce = (uint32_t)reduce;
+    s.inner = (uint32_t)inner;
+    s.descending = descending != 0;
+    s.keys_out = (uint64_t*)keys[0];
+    s.idx_out = (uint32_t*)idx[0];
+    char name[64];
+    snprintf(name, sizeof(name), "hc_argsort_chunks_%s", dtype_name(dtype));
+    HC_TRY(launch(ctx, name, lines * ceil_div((uint64_t)reduce, 4096), 1, &s, sizeof(s)));
+    int cur = 0;
+    for (uint64_t run = 4096; run < (uint64_t)reduce; run *= 2, cur ^= 1) {
+      s.run = (uint32_t)run;
+      s.keys_in = (const uint64_t*)keys[cur];
+      s.idx_in = (const uint32_t*)idx[cur];
+      s.keys_out = (uint64_t*)keys[cur ^ 1];
+      s.idx_out = (uint32_t*)idx[cur ^ 1];
+      HC_TRY(launch(ctx, "hc_argsort_merge", ceil_div(lines * ceil_div((uint64_t)reduce, 8), HCK_BLOCK), 1, &s,
+                    sizeof(s)));
+    }
+    s.idx_in = (const uint32_t*)idx[cur];
+    return launch(ctx, "hc_argsort_emit", ceil_div(total, HCK_BLOCK), 1, &s, sizeof(s));
+  }
   hck_scan_args k;
   memset(&k, 0, sizeof(k));
   k.in = in;

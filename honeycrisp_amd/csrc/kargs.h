@@ -116,6 +116,19 @@ typedef struct {
   uint32_t exclusive, reverse, pad;
 } hck_scan_args;
 
+/* argsort of axes longer than one block sorts at once: sorted runs of (key, index) pairs, one
+ * array of each per line ([lines, reduce], line = outer * inner + inner index), merged pairwise. */
+typedef struct {
+  const void* in;          /* chunk pass: the tensor; emit pass: unused */
+  void* out;               /* emit pass: int64 result */
+  const uint64_t* keys_in; /* merge pass: runs of length `run` */
+  const uint32_t* idx_in;
+  uint64_t* keys_out;      /* chunk and merge passes */
+  uint32_t* idx_out;
+  uint32_t outer, reduce, inner;
+  uint32_t run, descending, pad;
+} hck_sort_args;
+
 /* MFMA rate probe: `chunks` 16-byte pieces of operand bit patterns at `data`; one float per lane
  * goes to `out` so that the arithmetic cannot be dropped. */
 typedef struct {

@@ -42,7 +42,8 @@
 
 // Measurement switches (never set in the shipped build): bit0 no DMA in the K loop, bit1 no
 // wait/barrier, bit2 no LDS reads in the K loop, bit3 every K-step fetches slice 0 again, bit4
-// only every other DMA instruction, bit5 every DMA instruction fetches the same 1 KiB. Results are wrong with any bit set.
+// only every other DMA instruction, bit5 every DMA instruction fetches the same 1 KiB,
+// bit6 / bit7 fetch A only, as pairs of adjacent 64-byte pieces / as single pieces. Results are wrong with any bit set.
 #ifndef HC_EXP
 #define HC_EXP 0
 #endif
@@ -285,6 +286,19 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
     if ((HC_EXP & 1) && in_loop) return;
     if ((HC_EXP & 16) && in_loop && (u & 1)) return;
     if ((HC_EXP & 8) && in_loop) k0 = 0;
+    if ((HC_EXP & 64) && in_loop) {  // A only, both 64-byte halves of a 128-byte line back to back
+      const int q = u >= HALF ? u - HALF : u + HALF;
+      if (q & 1) return;
+      const uint32_t kb = (k0 / (2 * BK)) * (2 * BK);
+      oa.dma((q / 2) % OpA::NI, A, kb, stage, kend, p.zeros);
+      oa.dma((q / 2) % OpA::NI, A, kb + BK, stage, kend, p.zeros);
+      return;
+    }
+    if ((HC_EXP & 128) && in_loop) {  // control for bit6: A only, one 64-byte half per instruction
+      const int q = u >= HALF ? u - HALF : u + HALF;
+      oa.dma(q % OpA::NI, A, k0, stage, kend, p.zeros);
+      return;
+    }
     if ((HC_EXP & 32) && in_loop) {  // every instruction fetches the same 1 KiB: first-level cache hits
       if (u < OpA::NI) oa.dma(0, A, 0, stage + u * 1024, kend, p.zeros);
       else if (u < NDMA) ob.dma(0, B, 0, stage + A_BYTES + (u - OpA::NI) * 1024, kend, p.zeros);

@@ -8,7 +8,8 @@
 // column, sequential along the axis, lanes coalesced along inner.
 //
 // argsort (BackendCPU.swift:888-920): one block per (outer, inner) pair sorts (key, index)
-// pairs with a bitonic network in LDS, up to 4096 elements. Keys are mapped to unsigned
+// pairs with a bitonic network in LDS, up to 4096 elements; longer axes are sorted in runs of
+// 4096 that are then merged pairwise (merge path, one lane per 8 outputs). Keys are mapped to unsigned
 // integers that order like the values (-0 counts as +0), inverted for descending order; the
 // source index breaks ties, so the sort is stable, which the reference's `stable` flag
 // asks for and its unstable variant permits.
@@ -99,28 +100,9 @@ __device__ __forceinline__ uint64_t sort_key(int64_t x) { return (uint64_t)x ^ 0
 
 constexpr int ARGSORT_MAX = 4096;
 
-template <typename T> __device__ __forceinline__ void argsort_impl(const hck_scan_args& p) {
-  typedef typename Arith<T>::type C;
-  __shared__ uint64_t keys[ARGSORT_MAX];
-  __shared__ uint32_t idxs[ARGSORT_MAX];
-  const uint32_t i = blockIdx.x / p.inner, j = blockIdx.x - i * p.inner;
-  const size_t base = (size_t)i * p.reduce * p.inner + j;
-  const T* in = (const T*)p.in + base;
-  int64_t* out = (int64_t*)p.out + base;
-  uint32_t N = 1;
-  while (N < p.reduce) N <<= 1;
-  // descending order = ascending order of the inverted key; padding sorts behind everything
-  const uint64_t flip = p.reverse ? ((sizeof(C) == 8) ? ~0ull : 0xffffffffull) : 0ull;
-  for (uint32_t t = threadIdx.x; t < N; t += HCK_BLOCK) {
-    if (t < p.reduce) {
-      keys[t] = sort_key((C)to_arith(in[(size_t)t * p.inner])) ^ flip;
-      idxs[t] = t;
-    } else {
-      keys[t] = ~0ull;
-      idxs[t] = 0xffffffffu;
-    }
-  }
-  __syncthreads();
+// Bitonic sort of up to ARGSORT_MAX (key, index) pairs in LDS; n = valid entries (already
+// stored by the caller, padding included), N = padded power of two.
+__device__ __forceinline__ void bitonic_sort_lds(uint64_t* keys, uint32_t* idxs, uint32_t N) {
   for (uint32_t k = 2; k <= N; k <<= 1) {
     for (uint32_t s = k >> 1; s > 0; s >>= 1) {
       for (uint32_t t = threadIdx.x; t < N; t += HCK_BLOCK) {
@@ -141,8 +123,137 @@ template <typename T> __device__ __forceinline__ void argsort_impl(const hck_sca
       __syncthreads();
     }
   }
+}
+
+// descending order = ascending order of the inverted key
+template <typename C> __device__ __forceinline__ uint64_t key_flip(uint32_t descending) {
+  return descending ? ((sizeof(C) == 8) ? ~0ull : 0xffffffffull) : 0ull;
+}
+
+template <typename T> __device__ __forceinline__ void argsort_impl(const hck_scan_args& p) {
+  typedef typename Arith<T>::type C;
+  __shared__ uint64_t keys[ARGSORT_MAX];
+  __shared__ uint32_t idxs[ARGSORT_MAX];
+  const uint32_t i = blockIdx.x / p.inner, j = blockIdx.x - i * p.inner;
+  const size_t base = (size_t)i * p.reduce * p.inner + j;
+  const T* in = (const T*)p.in + base;
+  int64_t* out = (int64_t*)p.out + base;
+  uint32_t N = 1;
+  while (N < p.reduce) N <<= 1;
+  const uint64_t flip = key_flip<C>(p.reverse);
+  for (uint32_t t = threadIdx.x; t < N; t += HCK_BLOCK) {
+    if (t < p.reduce) {
+      keys[t] = sort_key((C)to_arith(in[(size_t)t * p.inner])) ^ flip;
+      idxs[t] = t;
+    } else {  // padding sorts behind everything
+      keys[t] = ~0ull;
+      idxs[t] = 0xffffffffu;
+    }
+  }
+  __syncthreads();
+  bitonic_sort_lds(keys, idxs, N);
   for (uint32_t t = threadIdx.x; t < p.reduce; t += HCK_BLOCK) out[(size_t)t * p.inner] = (int64_t)idxs[t];
 }
+
+// Long axes, pass 1: block (line, chunk) sorts elements [chunk * ARGSORT_MAX, ...) of its line
+// and stores the sorted (key, index) run.
+template <typename T> __device__ __forceinline__ void argsort_chunks_impl(const hck_sort_args& p) {
+  typedef typename Arith<T>::type C;
+  __shared__ uint64_t keys[ARGSORT_MAX];
+  __shared__ uint32_t idxs[ARGSORT_MAX];
+  const uint32_t chunks = (p.reduce + ARGSORT_MAX - 1) / ARGSORT_MAX;
+  const uint32_t line = blockIdx.x / chunks, chunk = blockIdx.x - line * chunks;
+  const uint32_t i = line / p.inner, j = line - i * p.inner;
+  const T* in = (const T*)p.in + (size_t)i * p.reduce * p.inner + j;
+  const uint32_t first = chunk * ARGSORT_MAX;
+  const uint32_t count = p.reduce - first < ARGSORT_MAX ? p.reduce - first : ARGSORT_MAX;
+  const uint64_t flip = key_flip<C>(p.descending);
+  for (uint32_t t = threadIdx.x; t < ARGSORT_MAX; t += HCK_BLOCK) {
+    if (t < count) {
+      keys[t] = sort_key((C)to_arith(in[(size_t)(first + t) * p.inner])) ^ flip;
+      idxs[t] = first + t;
+    } else {
+      keys[t] = ~0ull;
+      idxs[t] = 0xffffffffu;
+    }
+  }
+  __syncthreads();
+  bitonic_sort_lds(keys, idxs, ARGSORT_MAX);
+  const size_t dst = (size_t)line * p.reduce + first;
+  for (uint32_t t = threadIdx.x; t < count; t += HCK_BLOCK) {
+    p.keys_out[dst + t] = keys[t];
+    p.idx_out[dst + t] = idxs[t];
+  }
+}
+
+// Long axes, pass 2..: runs of length `run` are merged pairwise. A lane produces MERGE_SEG
+// consecutive outputs of one pair: it finds where the merge path crosses its first output
+// position by bisection, then merges sequentially. (key, index) pairs are all distinct, so the
+// result does not depend on how ties would be broken.
+constexpr uint32_t MERGE_SEG = 8;
+
+__device__ __forceinline__ bool pair_before(uint64_t ka, uint32_t ia, uint64_t kb, uint32_t ib) {
+  return ka < kb || (ka == kb && ia < ib);
+}
+
+HC_KERNEL void hc_argsort_merge(hck_sort_args p) {
+  const uint32_t segs = (p.reduce + MERGE_SEG - 1) / MERGE_SEG;
+  const uint64_t gid = (uint64_t)blockIdx.x * HCK_BLOCK + threadIdx.x;
+  const uint64_t lines = (uint64_t)p.outer * p.inner;
+  if (gid >= lines * segs) return;
+  const uint32_t line = (uint32_t)(gid / segs), seg = (uint32_t)(gid - (uint64_t)line * segs);
+  const size_t base = (size_t)line * p.reduce;
+  const uint32_t pos = seg * MERGE_SEG;                  // first output position in the line
+  const uint32_t pair = pos / (2 * p.run) * (2 * p.run); // start of this pair of runs
+  const uint32_t a0 = pair, a1 = min(pair + p.run, p.reduce);
+  const uint32_t b0 = a1, b1 = min(pair + 2 * p.run, p.reduce);
+  const uint32_t na = a1 - a0, nb = b1 - b0, d = pos - pair;
+  const uint64_t* ka = p.keys_in + base + a0;
+  const uint64_t* kb = p.keys_in + base + b0;
+  const uint32_t* ia = p.idx_in + base + a0;
+  const uint32_t* ib = p.idx_in + base + b0;
+  // smallest x (elements taken from run A) with A[x] not before B[d - x - 1]
+  uint32_t lo = d > nb ? d - nb : 0, hi = d < na ? d : na;
+  while (lo < hi) {
+    const uint32_t x = (lo + hi) / 2, y = d - x - 1;
+    if (pair_before(ka[x], ia[x], kb[y], ib[y])) lo = x + 1;
+    else hi = x;
+  }
+  uint32_t x = lo, y = d - lo;
+  const uint32_t end = min(pos + MERGE_SEG, b1);
+  for (uint32_t o = pos; o < end; o++) {
+    bool take_a;
+    if (x >= na) take_a = false;
+    else if (y >= nb) take_a = true;
+    else take_a = pair_before(ka[x], ia[x], kb[y], ib[y]);
+    if (take_a) {
+      p.keys_out[base + o] = ka[x];
+      p.idx_out[base + o] = ia[x];
+      x++;
+    } else {
+      p.keys_out[base + o] = kb[y];
+      p.idx_out[base + o] = ib[y];
+      y++;
+    }
+  }
+}
+
+// Long axes, last pass: sorted indices to the int64 result, back in the tensor's layout.
+HC_KERNEL void hc_argsort_emit(hck_sort_args p) {
+  const uint64_t gid = (uint64_t)blockIdx.x * HCK_BLOCK + threadIdx.x;
+  const uint64_t total = (uint64_t)p.outer * p.inner * p.reduce;
+  if (gid >= total) return;
+  // gid walks the result in memory order: (i, t, j)
+  const uint32_t j = (uint32_t)(gid % p.inner);
+  const uint64_t r = gid / p.inner;
+  const uint32_t t = (uint32_t)(r % p.reduce), i = (uint32_t)(r / p.reduce);
+  const size_t line = (size_t)i * p.inner + j;
+  ((int64_t*)p.out)[gid] = (int64_t)p.idx_in[line * p.reduce + t];
+}
+
+HC_KERNEL void hc_argsort_chunks_f32(hck_sort_args p) { argsort_chunks_impl<float>(p); }
+HC_KERNEL void hc_argsort_chunks_f16(hck_sort_args p) { argsort_chunks_impl<half_t>(p); }
+HC_KERNEL void hc_argsort_chunks_i64(hck_sort_args p) { argsort_chunks_impl<int64_t>(p); }
 HC_KERNEL void hc_argsort_f32(hck_scan_args p) { argsort_impl<float>(p); }
 HC_KERNEL void hc_argsort_f16(hck_scan_args p) { argsort_impl<half_t>(p); }
 HC_KERNEL void hc_argsort_i64(hck_scan_args p) { argsort_impl<int64_t>(p); }

@@ -235,7 +235,8 @@ int hc_cumulative(hc_ctx* ctx, int op, int dtype, const void* in, void* out, int
 
 /* Backend.argsort (Backend.swift:535-545; CPU BackendCPU.swift:888-920): int64 permutation that
  * sorts the middle axis, for every (outer, inner) pair. Always stable (equal keys keep their
- * source order). Axes longer than 4096 return HC_ERR_UNSUPPORTED. */
+ * source order). Axes up to 4096 elements are sorted in one pass in LDS; longer ones as runs of
+ * 4096 merged pairwise, through scratch memory of 24 bytes per element from the context's pool. */
 int hc_argsort(hc_ctx* ctx, int dtype, const void* in, void* out, int64_t outer, int64_t reduce,
                int64_t inner, int descending);
 

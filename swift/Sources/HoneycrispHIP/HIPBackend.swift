@@ -471,12 +471,11 @@ open class HIPBackend: CPUBackend, @unchecked Sendable {
     return try await cumulative(1, a, dims, exclusive, reverse, dtype)
   }
 
-  /// The device sort is stable whatever `stable` says; axes longer than 4096 elements go to the
-  /// inherited CPU implementation.
+  /// The device sort is stable whatever `stable` says.
   override open func argsort(
     _ a: Tensor.Data, dims: ReduceDims, descending: Bool, stable: Bool, dtype: Tensor.DType
   ) async throws -> Tensor.Data {
-    guard dtype != .bool && dims.reduceCount <= 4096 else {
+    guard dtype != .bool else {
       return try await super.argsort(
         a, dims: dims, descending: descending, stable: stable, dtype: dtype)
     }

@@ -585,6 +585,21 @@ def test_argsort(hip_backend, oracle_backend, dtype):
         f = rand(rng, (6, 999), dtype)
         f[0, :5] = [0.0, -0.0, np.inf, -np.inf, 0.0]
         check_exact(hip_backend, oracle_backend, lambda: Tensor(data=f).argsort(1))
-    with hip_backend.use():
-        with pytest.raises(Exception):
-            Tensor(data=np.zeros((2, 5000), np.float32)).argsort(1)     # beyond the in-LDS sort: refused, not wrong
+
+
+@pytest.mark.parametrize("dtype", [F32, F16, I64], ids=["f32", "f16", "i64"])
+def test_argsort_long_axes(hip_backend, oracle_backend, dtype):
+    """Axes beyond one in-LDS sort: runs of 4096 merged pairwise (1, 2, 3 and 4 merge passes, ragged last
+    runs, a strided inner axis)."""
+    rng = np.random.default_rng(40)
+    for shape, axis in [((2, 4097), 1), ((3, 8192), 1), ((2, 10000), 1), ((1, 50257), 1), ((12289, 3), 0),
+                        ((2, 5000, 2), 1)]:
+        x = rng.integers(-300, 301, size=shape)         # many ties across runs
+        x = x if dtype == I64 else x.astype(dtype.numpy)
+        for descending in (False, True):
+            check_exact(hip_backend, oracle_backend, lambda: Tensor(data=x).argsort(axis, descending=descending, stable=True))
+    if dtype != I64:
+        f = rand(rng, (2, 20000), dtype)
+        check_exact(hip_backend, oracle_backend, lambda: Tensor(data=f).argsort(1))
+        got, _ = both(hip_backend, oracle_backend, lambda: Tensor(data=f).gather(1, Tensor(data=f).argsort(1)))
+        assert np.all(np.diff(got.astype(np.float32), axis=1) >= 0)
