@@ -1212,11 +1212,45 @@ extern "C" int hc_cumulative(hc_ctx* ctx, int op, int dtype, const void* in, voi
   k.inner = (uint32_t)inner;
   k.exclusive = exclusive != 0;
   k.reverse = reverse != 0;
+  const char* opn = op == 0 ? "sum" : "prod";
+  // columns: a lane takes 16 bytes of adjacent columns when the layout allows and enough lanes remain
+  const uint64_t vec = 16 / dtype_size(dtype);
+  const bool colsv = inner > 1 && (uint64_t)inner % vec == 0 && aligned16(in) && aligned16(out) &&
+                     (uint64_t)outer * (uint64_t)inner / vec >= 64;
+  const char* form = inner == 1 ? "rows" : colsv ? "colsv" : "cols";
+  const char* tn = dtype_name(dtype);
+  // Few, long lines: cut the axis so that about eight waves per compute unit have work.
+  const uint64_t cus = (uint64_t)ctx->props.multiProcessorCount;
+  uint64_t segs = 1, seg_len = (uint64_t)reduce;
+  if (inner == 1) {
+    const uint64_t want = cus * 8;  // waves
+    if ((uint64_t)outer < want && reduce >= 4096) {
+      segs = std::min<uint64_t>(ceil_div(want, (uint64_t)outer), (uint64_t)reduce / 1024);
+      seg_len = ceil_div(ceil_div((uint64_t)reduce, segs), 256) * 256;  // whole 64 x 4 tiles
+      segs = ceil_div((uint64_t)reduce, seg_len);
+    }
+  } else {
+    const uint64_t want = cus * 8 * 64, lanes = (uint64_t)outer * (uint64_t)inner / (colsv ? vec : 1);
+    if (lanes < want && reduce >= 128) {
+      segs = std::min<uint64_t>(ceil_div(want, lanes), (uint64_t)reduce / 32);
+      seg_len = ceil_div((uint64_t)reduce, segs);
+      segs = ceil_div((uint64_t)reduce, seg_len);
+    }
+  }
   char name[64];
-  snprintf(name, sizeof(name), "hc_cumulative_%s_%s_%s", op == 0 ? "sum" : "prod", inner == 1 ? "rows" : "cols",
-           dtype_name(dtype));
-  const uint64_t blocks = inner == 1 ? ceil_div((uint64_t)outer, HCK_BLOCK / 64)
-                                     : ceil_div((uint64_t)outer * (uint64_t)inner, HCK_BLOCK);
+  const uint64_t units = (uint64_t)outer * segs * (uint64_t)inner;  // waves (rows) or columns (cols)
+  const uint64_t blocks = inner == 1 ? ceil_div(units, HCK_BLOCK / 64) : ceil_div(units / (colsv ? vec : 1), HCK_BLOCK);
+  Scratch scratch(ctx);
+  if (segs > 1) {
+    k.segs = (uint32_t)segs;
+    k.seg_len = (uint32_t)seg_len;
+    HC_TRY(scratch.get(units * 8, &k.carry));
+    snprintf(name, sizeof(name), "hc_cumulative_%s_%s_totals_%s", opn, form, tn);
+    HC_TRY(launch(ctx, name, blocks, 1, &k, sizeof(k)));
+    snprintf(name, sizeof(name), "hc_cumulative_%s_carry_%s", opn, dtype == HC_I64 ? "i64" : "f32");
+    HC_TRY(launch(ctx, name, ceil_div((uint64_t)outer * (uint64_t)inner, HCK_BLOCK), 1, &k, sizeof(k)));
+  }
+  snprintf(name, sizeof(name), "hc_cumulative_%s_%s_%s", opn, form, tn);
   return launch(ctx, name, blocks, 1, &k, sizeof(k));
 }
 

@@ -112,8 +112,14 @@ typedef struct {
 typedef struct {
   const void* in;
   void* out;
+  /* cumulative ops on few, long lines: the axis is cut into `segs` segments of `seg_len`
+   * positions (in scan order) that are scanned independently; carry[(i * segs + s) * inner + j]
+   * (float for float types, int64 otherwise) first receives the segments' totals, then what
+   * precedes each segment. segs <= 1: unused. */
+  void* carry;
   uint32_t outer, reduce, inner;
-  uint32_t exclusive, reverse, pad;
+  uint32_t exclusive, reverse;
+  uint32_t segs, seg_len, pad;
 } hck_scan_args;
 
 /* argsort of axes longer than one block sorts at once: sorted runs of (key, index) pairs, one

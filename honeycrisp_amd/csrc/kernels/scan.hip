@@ -5,7 +5,9 @@
 // per row walks it in tiles of 64 x 4 elements (in-lane scan, wave scan of the lane totals
 // with shuffles, running carry); floats are combined in tree order, so they differ from the
 // sequential CPU loop by rounding only; int64 is exact. Columns (inner > 1): one lane per
-// column, sequential along the axis, lanes coalesced along inner.
+// column, sequential along the axis, lanes coalesced along inner. When there are too few lines
+// to fill the chip, the axis is cut into segments: totals per segment, a small scan of the
+// totals, then the segments are scanned starting from what precedes them.
 //
 // argsort (BackendCPU.swift:888-920): one block per (outer, inner) pair sorts (key, index)
 // pairs with a bitonic network in LDS, up to 4096 elements; longer axes are sorted in runs of
@@ -22,24 +24,34 @@ template <int OP, typename C> __device__ __forceinline__ C scan_combine(C a, C b
   return OP == SCAN_SUM ? a + b : a * b;
 }
 
-template <typename T, int OP> __device__ __forceinline__ void cumulative_rows_impl(const hck_scan_args& p) {
+// PHASE 0: the scan itself (of whole lines, or of segments that start from their carry);
+// PHASE 1: only the segments' totals, into p.carry.
+template <typename T, int OP, int PHASE> __device__ __forceinline__ void cumulative_rows_impl(const hck_scan_args& p) {
   typedef typename Arith<T>::type C;
   constexpr int E = 4;
   const uint32_t lane = threadIdx.x & 63;
-  const uint32_t row = blockIdx.x * (HCK_BLOCK / 64) + (threadIdx.x >> 6);
-  if (row >= p.outer) return;
+  const uint32_t segs = p.segs > 1 ? p.segs : 1;
+  const uint32_t unit = blockIdx.x * (HCK_BLOCK / 64) + (threadIdx.x >> 6);  // (row, segment)
+  if (unit >= p.outer * segs) return;
+  const uint32_t row = unit / segs, seg = unit - row * segs;
   const uint32_t n = p.reduce;
+  const uint32_t lo = segs > 1 ? seg * p.seg_len : 0;
+  const uint32_t hi = segs > 1 ? (lo + p.seg_len < n ? lo + p.seg_len : n) : n;
   const T* in = (const T*)p.in + (size_t)row * n;
   T* out = (T*)p.out + (size_t)row * n;
-  C carry = scan_identity<OP, C>();
-  for (uint32_t base = 0; base < n; base += 64 * E) {
+  C carry = (PHASE == 0 && segs > 1) ? ((const C*)p.carry)[unit] : scan_identity<OP, C>();
+  for (uint32_t base = lo; base < hi; base += 64 * E) {
     // logical positions t (in scan order) of this lane; the element sits at n-1-t when reversed
     C x[E], run = scan_identity<OP, C>();
 #pragma unroll
     for (int e = 0; e < E; e++) {
       const uint32_t t = base + lane * E + e;
-      x[e] = t < n ? to_arith(in[p.reverse ? n - 1 - t : t]) : scan_identity<OP, C>();
+      x[e] = t < hi ? to_arith(in[p.reverse ? n - 1 - t : t]) : scan_identity<OP, C>();
       run = scan_combine<OP, C>(run, x[e]);
+    }
+    if (PHASE == 1) {
+      carry = scan_combine<OP, C>(carry, run);  // per lane; combined across the wave at the end
+      continue;
     }
     // inclusive scan of the lane totals across the wave
     C incl = run;
@@ -55,38 +67,99 @@ template <typename T, int OP> __device__ __forceinline__ void cumulative_rows_im
     for (int e = 0; e < E; e++) {
       const uint32_t t = base + lane * E + e;
       const C next = scan_combine<OP, C>(acc, x[e]);
-      if (t < n) out[p.reverse ? n - 1 - t : t] = from_arith<T>(p.exclusive ? acc : next);
+      if (t < hi) out[p.reverse ? n - 1 - t : t] = from_arith<T>(p.exclusive ? acc : next);
       acc = next;
     }
     carry = scan_combine<OP, C>(carry, __shfl(incl, 63, 64));
   }
-}
-
-template <typename T, int OP> __device__ __forceinline__ void cumulative_cols_impl(const hck_scan_args& p) {
-  typedef typename Arith<T>::type C;
-  const uint64_t t = (uint64_t)blockIdx.x * HCK_BLOCK + threadIdx.x;
-  if (t >= (uint64_t)p.outer * p.inner) return;
-  const uint32_t i = (uint32_t)(t / p.inner), j = (uint32_t)(t - (uint64_t)i * p.inner);
-  const size_t base = (size_t)i * p.reduce * p.inner + j;
-  const T* in = (const T*)p.in + base;
-  T* out = (T*)p.out + base;
-  C run = scan_identity<OP, C>();
-  for (uint32_t s = 0; s < p.reduce; s++) {
-    const size_t k = (size_t)(p.reverse ? p.reduce - 1 - s : s) * p.inner;
-    const C next = scan_combine<OP, C>(run, to_arith(in[k]));
-    out[k] = from_arith<T>(p.exclusive ? run : next);
-    run = next;
+  if (PHASE == 1) {
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) carry = scan_combine<OP, C>(carry, __shfl_down(carry, d, 64));
+    if (lane == 0) ((C*)p.carry)[unit] = carry;
   }
 }
 
-#define DEF_CUMULATIVE(TN, T)                                                                                  \
-  HC_KERNEL void hc_cumulative_sum_rows_##TN(hck_scan_args p) { cumulative_rows_impl<T, SCAN_SUM>(p); }        \
-  HC_KERNEL void hc_cumulative_prod_rows_##TN(hck_scan_args p) { cumulative_rows_impl<T, SCAN_PROD>(p); }      \
-  HC_KERNEL void hc_cumulative_sum_cols_##TN(hck_scan_args p) { cumulative_cols_impl<T, SCAN_SUM>(p); }        \
-  HC_KERNEL void hc_cumulative_prod_cols_##TN(hck_scan_args p) { cumulative_cols_impl<T, SCAN_PROD>(p); }
+// VEC adjacent columns per lane (VEC > 1: inner is a multiple of VEC and the buffers are
+// 16-byte aligned, so every access is one 16-byte piece).
+template <typename T, int OP, int PHASE, int VEC>
+__device__ __forceinline__ void cumulative_cols_impl(const hck_scan_args& p) {
+  typedef typename Arith<T>::type C;
+  const uint32_t segs = p.segs > 1 ? p.segs : 1;
+  const uint32_t innerv = p.inner / VEC;
+  const uint64_t t = (uint64_t)blockIdx.x * HCK_BLOCK + threadIdx.x;  // (i, segment, vector column)
+  if (t >= (uint64_t)p.outer * segs * innerv) return;
+  const uint32_t j = (uint32_t)(t % innerv) * VEC;
+  const uint32_t is = (uint32_t)(t / innerv), i = is / segs, seg = is - i * segs;
+  const uint32_t lo = segs > 1 ? seg * p.seg_len : 0;
+  const uint32_t hi = segs > 1 ? (lo + p.seg_len < p.reduce ? lo + p.seg_len : p.reduce) : p.reduce;
+  const size_t base = (size_t)i * p.reduce * p.inner + j;
+  const T* in = (const T*)p.in + base;
+  T* out = (T*)p.out + base;
+  C* carry = (C*)p.carry + (size_t)is * p.inner + j;
+  C run[VEC];
+#pragma unroll
+  for (int v = 0; v < VEC; v++) run[v] = (PHASE == 0 && segs > 1) ? carry[v] : scan_identity<OP, C>();
+#pragma unroll 4
+  for (uint32_t s = lo; s < hi; s++) {
+    const size_t k = (size_t)(p.reverse ? p.reduce - 1 - s : s) * p.inner;
+    T x[VEC], o[VEC];
+    load_vec<T, VEC>(in + k, 0, 1, x);
+#pragma unroll
+    for (int v = 0; v < VEC; v++) {
+      const C next = scan_combine<OP, C>(run[v], to_arith(x[v]));
+      o[v] = from_arith<T>(p.exclusive ? run[v] : next);
+      run[v] = next;
+    }
+    if (PHASE == 0) store_vec<T, VEC>(out, k, o);
+  }
+  if (PHASE == 1) {
+#pragma unroll
+    for (int v = 0; v < VEC; v++) carry[v] = run[v];
+  }
+}
+
+// Segment totals -> what precedes each segment: one lane per (i, j) walks its `segs` totals.
+template <typename C, int OP> __device__ __forceinline__ void cumulative_carry_impl(const hck_scan_args& p) {
+  const uint64_t t = (uint64_t)blockIdx.x * HCK_BLOCK + threadIdx.x;
+  if (t >= (uint64_t)p.outer * p.inner) return;
+  const uint32_t i = (uint32_t)(t / p.inner), j = (uint32_t)(t - (uint64_t)i * p.inner);
+  C* c = (C*)p.carry + (size_t)i * p.segs * p.inner + j;
+  C run = scan_identity<OP, C>();
+  for (uint32_t s = 0; s < p.segs; s++) {
+    const C total = c[(size_t)s * p.inner];
+    c[(size_t)s * p.inner] = run;
+    run = scan_combine<OP, C>(run, total);
+  }
+}
+
+#define DEF_CUMULATIVE(TN, T)                                                                                   \
+  HC_KERNEL void hc_cumulative_sum_rows_##TN(hck_scan_args p) { cumulative_rows_impl<T, SCAN_SUM, 0>(p); }      \
+  HC_KERNEL void hc_cumulative_prod_rows_##TN(hck_scan_args p) { cumulative_rows_impl<T, SCAN_PROD, 0>(p); }    \
+  HC_KERNEL void hc_cumulative_sum_cols_##TN(hck_scan_args p) { cumulative_cols_impl<T, SCAN_SUM, 0, 1>(p); }   \
+  HC_KERNEL void hc_cumulative_prod_cols_##TN(hck_scan_args p) { cumulative_cols_impl<T, SCAN_PROD, 0, 1>(p); } \
+  HC_KERNEL void hc_cumulative_sum_colsv_##TN(hck_scan_args p) {                                                \
+    cumulative_cols_impl<T, SCAN_SUM, 0, VecWidth<T>::value>(p);                                                \
+  }                                                                                                             \
+  HC_KERNEL void hc_cumulative_prod_colsv_##TN(hck_scan_args p) {                                               \
+    cumulative_cols_impl<T, SCAN_PROD, 0, VecWidth<T>::value>(p);                                               \
+  }                                                                                                             \
+  HC_KERNEL void hc_cumulative_sum_colsv_totals_##TN(hck_scan_args p) {                                         \
+    cumulative_cols_impl<T, SCAN_SUM, 1, VecWidth<T>::value>(p);                                                \
+  }                                                                                                             \
+  HC_KERNEL void hc_cumulative_prod_colsv_totals_##TN(hck_scan_args p) {                                        \
+    cumulative_cols_impl<T, SCAN_PROD, 1, VecWidth<T>::value>(p);                                               \
+  }                                                                                                             \
+  HC_KERNEL void hc_cumulative_sum_rows_totals_##TN(hck_scan_args p) { cumulative_rows_impl<T, SCAN_SUM, 1>(p); }   \
+  HC_KERNEL void hc_cumulative_prod_rows_totals_##TN(hck_scan_args p) { cumulative_rows_impl<T, SCAN_PROD, 1>(p); } \
+  HC_KERNEL void hc_cumulative_sum_cols_totals_##TN(hck_scan_args p) { cumulative_cols_impl<T, SCAN_SUM, 1, 1>(p); }   \
+  HC_KERNEL void hc_cumulative_prod_cols_totals_##TN(hck_scan_args p) { cumulative_cols_impl<T, SCAN_PROD, 1, 1>(p); }
 DEF_CUMULATIVE(f32, float)
 DEF_CUMULATIVE(f16, half_t)
 DEF_CUMULATIVE(i64, int64_t)
+HC_KERNEL void hc_cumulative_sum_carry_f32(hck_scan_args p) { cumulative_carry_impl<float, SCAN_SUM>(p); }
+HC_KERNEL void hc_cumulative_prod_carry_f32(hck_scan_args p) { cumulative_carry_impl<float, SCAN_PROD>(p); }
+HC_KERNEL void hc_cumulative_sum_carry_i64(hck_scan_args p) { cumulative_carry_impl<int64_t, SCAN_SUM>(p); }
+HC_KERNEL void hc_cumulative_prod_carry_i64(hck_scan_args p) { cumulative_carry_impl<int64_t, SCAN_PROD>(p); }
 
 // ---------------------------------------------------------------- argsort
 

@@ -552,7 +552,8 @@ def test_bitwise_ops(hip_backend, oracle_backend):
 @pytest.mark.parametrize("dtype", [F32, F16, I64], ids=["f32", "f16", "i64"])
 def test_cumulative_ops(hip_backend, oracle_backend, dtype):
     rng = np.random.default_rng(38)
-    for shape, axis in [((7, 1000), 1), ((3, 257, 5), 1), ((5000, 3), 0), ((4, 1), 1), ((2, 64), 1), ((1, 70000), 1)]:
+    for shape, axis in [((7, 1000), 1), ((3, 257, 5), 1), ((5000, 3), 0), ((4, 1), 1), ((2, 64), 1), ((1, 70000), 1),
+                        ((300, 512), 0), ((4, 200, 256), 1)]:     # 16-byte column vectors, with / without segments
         # small integers: every partial sum is exact, so the scan order cannot matter
         x = rng.integers(-3, 4, size=shape)
         x = x if dtype == I64 else x.astype(dtype.numpy)
@@ -568,9 +569,12 @@ def test_cumulative_ops(hip_backend, oracle_backend, dtype):
         check_exact(hip_backend, oracle_backend, lambda: Tensor(data=y).cumulativeProd(axis))
         check_exact(hip_backend, oracle_backend, lambda: Tensor(data=y).cumulativeProd(axis, exclusive=True, reverse=True))
     if dtype != I64:
-        r = rand(rng, (16, 3000), dtype)
-        got, want = both(hip_backend, oracle_backend, lambda: Tensor(data=r).cumulativeSum(1))
-        assert_close_arrays(got, want, TOL[dtype] * 60, TOL[dtype])
+        # general floats: the device combines in tree / segment order, the CPU sequentially
+        for shape, axis in [((16, 3000), 1), ((2, 20000), 1), ((6000, 4), 0), ((3000, 256), 0)]:
+            r = rand(rng, shape, dtype)
+            for reverse in (False, True):
+                got, want = both(hip_backend, oracle_backend, lambda: Tensor(data=r).cumulativeSum(axis, reverse=reverse))
+                assert_close_arrays(got, want, TOL[dtype] * 60, TOL[dtype])
 
 
 @pytest.mark.parametrize("dtype", [F32, F16, I64], ids=["f32", "f16", "i64"])
