@@ -1556,6 +1556,68 @@ extern "C" int hc_scatter(hc_ctx* ctx, int dtype, const void* in, const void* in
   REQUIRE(out, "hc_scatter: null pointer");
   const size_t n_out = (size_t)outer * (size_t)middle * (size_t)inner;
   const uint64_t total = (uint64_t)outer * (uint64_t)out_count * (uint64_t)inner;
+  // Rows of at least 1 KiB in whole 16-byte vectors, index independent of the position inside
+  // the row, repeated indices allowed: group the source rows by destination and add them in
+  // source order, one workgroup per destination row. No atomics on the data, no zero fill, and
+  // float sums come out in the CPU's order.
+  if (!indices_are_unique && total != 0 && inner > 1 && idx_strides->ndim <= HC_MAX_DIMS) {
+    REQUIRE(in && indices, "hc_scatter: null pointer");
+    uint64_t tail = 1;
+    int kd = (int)idx_strides->ndim;
+    bool zero = true;
+    while (kd > 0 && tail < (uint64_t)inner) {
+      kd--;
+      tail *= (uint64_t)idx_strides->shape[kd];
+      if (idx_strides->strides[kd] != 0 && idx_strides->shape[kd] != 1) zero = false;
+    }
+    const size_t row_bytes = (size_t)inner * dtype_size(dtype);
+    // (one workgroup per destination row: their number times the workgroup size must fit 32 bits)
+    if (zero && tail == (uint64_t)inner && row_bytes % 16 == 0 && row_bytes >= 1024 && aligned16(in) &&
+        aligned16(out) && (uint64_t)outer * (uint64_t)middle < (1ull << 24)) {
+      uint64_t n = 1;
+      for (uint32_t d = 0; d < idx_strides->ndim; d++) n *= (uint64_t)idx_strides->shape[d];
+      REQUIRE(n == total, "hc_scatter: index shape has %llu elements, expected %llu", (unsigned long long)n,
+              (unsigned long long)total);
+      hc_strides row_strides;
+      memset(&row_strides, 0, sizeof(row_strides));
+      row_strides.ndim = (uint32_t)kd;
+      for (int d = 0; d < kd; d++) {
+        row_strides.shape[d] = idx_strides->shape[d];
+        row_strides.strides[d] = idx_strides->strides[d];
+      }
+      const uint64_t n_buckets = (uint64_t)outer * (uint64_t)middle, n_rows = (uint64_t)outer * (uint64_t)out_count;
+      Scratch scratch(ctx);
+      void *counters = nullptr, *starts = nullptr, *list = nullptr;
+      HC_TRY(scratch.get(2 * n_buckets * sizeof(int64_t), &counters));  // counts, then cursors
+      HC_TRY(scratch.get(n_buckets * sizeof(int64_t), &starts));
+      HC_TRY(scratch.get(n_rows * sizeof(uint32_t), &list));
+      HC_TRY(hc_fill(ctx, HC_I64, 0.0f, 0, counters, 2 * n_buckets));
+      hck_scatter_rows_args k;
+      memset(&k, 0, sizeof(k));
+      k.in = in;
+      k.indices = (const int64_t*)indices;
+      k.out = out;
+      k.counts = (int64_t*)counters;
+      k.cursor = (int64_t*)counters + n_buckets;
+      k.starts = (const int64_t*)starts;
+      k.list = (uint32_t*)list;
+      k.n_src = (uint32_t)out_count;
+      k.n_dst = (uint32_t)middle;
+      k.row_vecs = (uint32_t)(row_bytes / 16);
+      k.total_src = (uint32_t)n_rows;
+      int vec;
+      uint64_t rows;
+      const hc_strides* ops[] = {&row_strides};
+      const void* ptrs[] = {indices};
+      HC_TRY(make_bcast(1, ops, ptrs, out, 1, &k.idx, &vec, &rows));
+      HC_TRY(launch(ctx, "hc_scatter_rows_count", ceil_div(n_rows, HCK_BLOCK), 1, &k, sizeof(k)));
+      HC_TRY(hc_cumulative(ctx, 0, HC_I64, counters, starts, 1, (int64_t)n_buckets, 1, 1, 0));
+      HC_TRY(launch(ctx, "hc_scatter_rows_fill", ceil_div(n_rows, HCK_BLOCK), 1, &k, sizeof(k)));
+      char name[64];
+      snprintf(name, sizeof(name), "hc_scatter_rows_sum_%s", dtype_name(dtype));
+      return launch(ctx, name, n_buckets, 1, &k, sizeof(k));
+    }
+  }
   // half values with repeated indices add up in a float buffer that is rounded once at the end
   const bool staged = dtype == HC_F16 && !indices_are_unique;
   Scratch scratch(ctx);

@@ -175,6 +175,23 @@ typedef struct {
   hck_bcast idx; /* operand 0 = index offset for a flat row number, vec = 1 */
 } hck_gather_rows_args;
 
+/* Row scatter with repeated indices, without atomics on the data: source rows are grouped by
+ * destination row (count, scan, fill), every destination row then adds its sources in
+ * ascending source order. Row numbers are flat over the outer axis. */
+typedef struct {
+  const void* in;          /* [outer, n_src, row] */
+  const int64_t* indices;
+  void* out;               /* [outer, n_dst, row] */
+  int64_t* counts;         /* [outer * n_dst] sources per destination row */
+  const int64_t* starts;   /* exclusive running sum of counts */
+  int64_t* cursor;         /* [outer * n_dst] fill positions, zero before the fill pass */
+  uint32_t* list;          /* [outer * n_src] source rows, grouped by destination */
+  uint32_t n_src, n_dst;
+  uint32_t row_vecs;       /* 16-byte vectors per row */
+  uint32_t total_src;      /* outer * n_src */
+  hck_bcast idx;           /* operand 0 = index offset for a flat source row, vec = 1 */
+} hck_scatter_rows_args;
+
 /* Element gather: general index map over the flat output index. */
 typedef struct {
   const void* in;

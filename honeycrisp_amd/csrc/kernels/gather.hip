@@ -118,6 +118,117 @@ HC_KERNEL void hc_scatter_set_b8(hck_gather_elems_args p) { scatter_set_impl<uin
 HC_KERNEL void hc_scatter_set_b4(hck_gather_elems_args p) { scatter_set_impl<uint32_t>(p); }
 HC_KERNEL void hc_scatter_set_b2(hck_gather_elems_args p) { scatter_set_impl<uint16_t>(p); }
 
+// Row scatter with repeated indices (rows of whole 16-byte vectors): no atomics on the data.
+// Pass 1 counts the sources of every destination row, the host scans the counts, pass 2 drops
+// every source row number into its destination's slice of `list` (in whatever order the
+// atomics on the cursors resolve), pass 3 gives every destination row to one workgroup, which
+// sorts its slice and adds the sources in ascending order: the order of the CPU loop
+// (BackendCPU.swift:1149-1188), so float sums match it bit for bit and runs repeat exactly.
+HC_KERNEL void hc_scatter_rows_count(hck_scatter_rows_args p) {
+  const uint32_t r = blockIdx.x * HCK_BLOCK + threadIdx.x;
+  if (r >= p.total_src) return;
+  uint32_t off[1];
+  size_t unused;
+  bcast_offsets<1, 1>(p.idx, r, off, unused);
+  const uint64_t bucket = (uint64_t)(r / p.n_src) * p.n_dst + (uint64_t)p.indices[off[0]];
+  __hip_atomic_fetch_add((unsigned long long*)p.counts + bucket, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+HC_KERNEL void hc_scatter_rows_fill(hck_scatter_rows_args p) {
+  const uint32_t r = blockIdx.x * HCK_BLOCK + threadIdx.x;
+  if (r >= p.total_src) return;
+  uint32_t off[1];
+  size_t unused;
+  bcast_offsets<1, 1>(p.idx, r, off, unused);
+  const uint64_t bucket = (uint64_t)(r / p.n_src) * p.n_dst + (uint64_t)p.indices[off[0]];
+  const unsigned long long slot =
+      __hip_atomic_fetch_add((unsigned long long*)p.cursor + bucket, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  p.list[p.starts[bucket] + (int64_t)slot] = r;
+}
+
+// Ascending sort of n distinct values by the whole workgroup: a bitonic network whose
+// comparators all point the same way (each merge starts with a mirrored stage), so positions
+// past n behave as +infinity and n need not be a power of two. Works on LDS or global memory.
+__device__ __forceinline__ void sort_ascending(uint32_t* a, uint32_t n) {
+  uint32_t N = 1;
+  while (N < n) N <<= 1;
+  auto exchange = [&](uint32_t i, uint32_t j) {
+    if (j < n) {
+      const uint32_t x = a[i], y = a[j];
+      if (x > y) {
+        a[i] = y;
+        a[j] = x;
+      }
+    }
+  };
+  for (uint32_t k = 2; k <= N; k <<= 1) {
+    const uint32_t h = k >> 1;
+    for (uint32_t t = threadIdx.x; t < N / 2; t += HCK_BLOCK) {
+      const uint32_t blk = t / h, o = t - blk * h;
+      exchange(blk * k + o, blk * k + k - 1 - o);
+    }
+    __threadfence_block();
+    __syncthreads();
+    for (uint32_t s = h >> 1; s > 0; s >>= 1) {
+      for (uint32_t t = threadIdx.x; t < N / 2; t += HCK_BLOCK) {
+        const uint32_t i = (t / s) * 2 * s + (t % s);
+        exchange(i, i + s);
+      }
+      __threadfence_block();
+      __syncthreads();
+    }
+  }
+}
+
+constexpr uint32_t SCATTER_LDS_ROWS = 4096;
+
+template <typename T> __device__ __forceinline__ void scatter_rows_sum_impl(const hck_scatter_rows_args& p) {
+  typedef typename Arith<T>::type C;
+  constexpr int VEC = VecWidth<T>::value;
+  __shared__ uint32_t held[SCATTER_LDS_ROWS];
+  const uint32_t b = blockIdx.x;  // destination row, flat over the outer axis
+  const uint32_t n = (uint32_t)p.counts[b];
+  uint32_t* src = p.list + p.starts[b];
+  if (n > 1 && n <= SCATTER_LDS_ROWS) {
+    for (uint32_t t = threadIdx.x; t < n; t += HCK_BLOCK) held[t] = src[t];
+    __syncthreads();
+    sort_ascending(held, n);
+    src = held;
+  } else if (n > SCATTER_LDS_ROWS) {
+    sort_ascending(src, n);  // in place in global memory: rare (one row receiving > 4096 sources)
+  }
+  const T* in = (const T*)p.in;
+  T* out = (T*)p.out + (size_t)b * p.row_vecs * VEC;
+  for (uint32_t c = threadIdx.x; c < p.row_vecs; c += HCK_BLOCK) {
+    C acc[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; v++) acc[v] = (C)0;
+    uint32_t t = 0;
+    for (; t + 4 <= n; t += 4) {  // four loads in flight, added in order
+      T x[4][VEC];
+#pragma unroll
+      for (int u = 0; u < 4; u++) load_vec<T, VEC>(in + ((size_t)src[t + u] * p.row_vecs + c) * VEC, 0, 1, x[u]);
+#pragma unroll
+      for (int u = 0; u < 4; u++)
+#pragma unroll
+        for (int v = 0; v < VEC; v++) acc[v] = acc[v] + to_arith(x[u][v]);
+    }
+    for (; t < n; t++) {
+      T x[VEC];
+      load_vec<T, VEC>(in + ((size_t)src[t] * p.row_vecs + c) * VEC, 0, 1, x);
+#pragma unroll
+      for (int v = 0; v < VEC; v++) acc[v] = acc[v] + to_arith(x[v]);
+    }
+    T o[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; v++) o[v] = from_arith<T>(acc[v]);
+    store_vec<T, VEC>(out, (size_t)c * VEC, o);
+  }
+}
+HC_KERNEL void hc_scatter_rows_sum_f32(hck_scatter_rows_args p) { scatter_rows_sum_impl<float>(p); }
+HC_KERNEL void hc_scatter_rows_sum_f16(hck_scatter_rows_args p) { scatter_rows_sum_impl<half_t>(p); }
+HC_KERNEL void hc_scatter_rows_sum_i64(hck_scatter_rows_args p) { scatter_rows_sum_impl<int64_t>(p); }
+
 // Re-pitching copy for GEMM operands whose rows are not 16-byte aligned: element-wise
 // accesses (either side may be unaligned), zero beyond the valid columns. A wave owns
 // 64 * G consecutive elements of one row and moves 64 consecutive elements per instruction,

@@ -458,6 +458,33 @@ def test_scatter_forms(hip_backend, oracle_backend, dtype):
                 lambda: Tensor(data=empty, shape=[0, 4], dtype=dtype).scatter(0, 3, Tensor(data=[], shape=[0], dtype=I64)))
 
 
+@pytest.mark.parametrize("dtype", [F32, F16, I64], ids=["f32", "f16", "i64"])
+def test_scatter_long_rows_bit_exact(hip_backend, oracle_backend, dtype):
+    """Rows of 1 KiB and more whose index does not depend on the position in the row are added in
+    source order, like the CPU loop: random floats match bit for bit."""
+    rng = np.random.default_rng(33)
+    width = {F32: 256, F16: 512, I64: 128}[dtype]
+    cases = [
+        (rng.integers(0, 300, size=(2000,)), 300, 1),          # a few sources per destination, some empty rows
+        (rng.integers(0, 3, size=(700,)), 5, 1),               # hundreds per destination: sorted in LDS
+        (np.zeros(4500, dtype=np.int64), 2, 1),                # more than the LDS holds: sorted in place
+        (rng.integers(0, 40, size=(3, 90)), 40, 3),            # an outer axis in front
+    ]
+    for rows, count, outer in cases:
+        shape = (rows.shape[0], width) if outer == 1 else (outer, rows.shape[1], width)
+        vals = rand(rng, shape, dtype)
+        axis = 0 if outer == 1 else 1
+        index = rows if outer == 1 else rows[:, :, None]
+        check_exact(hip_backend, oracle_backend, lambda: Tensor(data=vals).scatter(axis, count, Tensor(data=index)))
+    # twice the same call: no run-to-run differences
+    vals = rand(rng, (3000, width), dtype)
+    rows = rng.integers(0, 17, size=(3000,))
+    with hip_backend.use():
+        first = Tensor(data=vals).scatter(0, 17, Tensor(data=rows)).numpy()
+        second = Tensor(data=vals).scatter(0, 17, Tensor(data=rows)).numpy()
+    assert first.tobytes() == second.tobytes()
+
+
 @pytest.mark.parametrize("dtype", [F32, F16], ids=["f32", "f16"])
 def test_scatter_random_floats_within_tolerance(hip_backend, oracle_backend, dtype):
     rng = np.random.default_rng(32)
