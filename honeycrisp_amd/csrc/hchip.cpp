@@ -1794,8 +1794,8 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
                          const void* b, int trans_b, int trans_out, int64_t rows, int64_t inner,
                          int64_t cols, void* out) {
   REQUIRE(ctx, "hc_matmul: null context");
-  if (dtype != HC_F32 && dtype != HC_F16)
-    return fail(HC_ERR_UNSUPPORTED, "hc_matmul: dtype %d has no MFMA path (int64 stays on the CPU)", dtype);
+  if (dtype != HC_F32 && dtype != HC_F16 && dtype != HC_I64)
+    return fail(HC_ERR_UNSUPPORTED, "hc_matmul: dtype %d is not numeric", dtype);
   REQUIRE(batch >= 0 && rows >= 0 && inner >= 0 && cols >= 0, "hc_matmul: negative dimension");
   if (batch * rows * cols == 0) return HC_OK;
   REQUIRE(out && (inner == 0 || (a && b)), "hc_matmul: null pointer");
@@ -1839,6 +1839,23 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
   k.c_cs = 1;
   k.tiles_m = (uint32_t)ceil_div(M, 128);
   k.tiles_n = (uint32_t)ceil_div(N, 128);
+
+  if (dtype == HC_I64) {
+    // no matrix instruction for 64-bit integers: one small vector-ALU kernel, any strides
+    k.tiles_m = (uint32_t)ceil_div(M, 16);
+    k.tiles_n = (uint32_t)ceil_div(N, 16);
+    const uint64_t tiles = (uint64_t)k.tiles_m * k.tiles_n;
+    for (int64_t b0 = 0; b0 < batch; b0 += 65535) {
+      const uint32_t nb = (uint32_t)(batch - b0 < 65535 ? batch - b0 : 65535);
+      hck_gemm_args kk = k;
+      kk.a = (const char*)k.a + (uint64_t)b0 * k.a_bs * el;
+      kk.b = (const char*)k.b + (uint64_t)b0 * k.b_bs * el;
+      kk.c = (char*)k.c + (uint64_t)b0 * k.c_bs * el;
+      kk.batch = nb;
+      HC_TRY(launch(ctx, "hc_gemm_i64", tiles, nb, &kk, sizeof(kk)));
+    }
+    return HC_OK;
+  }
 
   // Per-operand global->LDS path: 'k' contiguous along K, 'm'/'n' contiguous along M/N
   // (both need 16-byte aligned rows), 'x' anything else.

@@ -230,3 +230,28 @@ __device__ __forceinline__ void gemm_impl(const hck_gemm_args& p) {
   DEF_GEMM(TN, T, x, LOAD_ANY, x, LOAD_ANY)
 DEF_GEMM_T(f16, half_t)
 DEF_GEMM_T(f32, float)
+
+// int64 products (BackendCPU.swift:1307-1308 allows them; they are rare): there is no matrix
+// instruction for 64-bit integers, so this is a plain LDS-tiled loop on the vector ALU, one
+// output element per lane, 16 x 16 outputs per workgroup, sums wrapping like two's complement.
+// tiles_m / tiles_n count 16 x 16 tiles; grid.y = batch.
+HC_KERNEL void hc_gemm_i64(hck_gemm_args p) {
+  __shared__ uint64_t sa[16][17], sb[16][17];
+  const uint32_t tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+  const uint32_t tm = blockIdx.x / p.tiles_n, tn = blockIdx.x - tm * p.tiles_n;
+  const uint32_t m = tm * 16 + ty, n = tn * 16 + tx;
+  const uint64_t* A = (const uint64_t*)p.a + (uint64_t)blockIdx.y * p.a_bs;
+  const uint64_t* B = (const uint64_t*)p.b + (uint64_t)blockIdx.y * p.b_bs;
+  uint64_t* C = (uint64_t*)p.c + (uint64_t)blockIdx.y * p.c_bs;
+  uint64_t acc = 0;
+  for (uint32_t k0 = 0; k0 < p.K; k0 += 16) {
+    // sa[row][k], sb[k][col]
+    sa[ty][tx] = (m < p.M && k0 + tx < p.K) ? A[(size_t)m * p.a_rs + (size_t)(k0 + tx) * p.a_cs] : 0;
+    sb[ty][tx] = (k0 + ty < p.K && n < p.N) ? B[(size_t)(k0 + ty) * p.b_rs + (size_t)n * p.b_cs] : 0;
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < 16; kk++) acc += sa[ty][kk] * sb[kk][tx];
+    __syncthreads();
+  }
+  if (m < p.M && n < p.N) C[(size_t)m * p.c_rs + (size_t)n * p.c_cs] = acc;
+}

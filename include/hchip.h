@@ -300,7 +300,8 @@ int hc_when(hc_ctx* ctx, int dtype, const void* mask, const hc_strides* ms, cons
 /* Backend.matmul / batchedMatmul (Backend.swift:650-669; CPU BackendCPU.swift:1222-1313).
  * rows/inner/cols are M/K/N after the transposes; A is [M,K] ([K,M] if trans_a), B is
  * [K,N] ([N,K] if trans_b), C is [M,N] ([N,M] if trans_out); matrix m of the batch is at
- * element offsets m*M*K, m*K*N, m*M*N. fp16 accumulates in fp32 and rounds once. */
+ * element offsets m*M*K, m*K*N, m*M*N. fp16 accumulates in fp32 and rounds once; fp16 and fp32
+ * run on the matrix cores, int64 (wrapping sums) on the vector ALU. */
 int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, int trans_a, const void* b,
               int trans_b, int trans_out, int64_t rows, int64_t inner, int64_t cols, void* out);
 

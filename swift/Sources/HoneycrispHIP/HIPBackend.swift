@@ -149,7 +149,7 @@ open class HIPBackend: CPUBackend, @unchecked Sendable {
     matrixCount: Int, a: Tensor.Data, transA: Bool, b: Tensor.Data, transB: Bool, transOut: Bool,
     rows: Int, inner: Int, cols: Int, dtype: Tensor.DType
   ) async throws -> Tensor.Data {
-    guard dtype == .float16 || dtype == .float32 else {
+    guard dtype != .bool else {
       return try await super.batchedMatmul(
         matrixCount: matrixCount, a: a, transA: transA, b: b, transB: transB, transOut: transOut,
         rows: rows, inner: inner, cols: cols, dtype: dtype)

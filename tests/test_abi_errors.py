@@ -22,9 +22,9 @@ def test_status_codes_for_bad_arguments(hip_backend):
     lib, ctx = hip_backend._lib, hip_backend._ctx
     buf = hip_backend.allocate(4096)
     p = c_void_p(buf.ptr)
-    # unsupported dtype for the MFMA path (int64 matmul stays on the CPU in the reference integration)
-    s, msg = status_and_message(hip_backend, lib.hc_matmul(ctx, int(DType.int64), 1, p, 0, p, 0, 0, 2, 2, 2, p))
-    assert s == _lib.HC_ERR_UNSUPPORTED and "int64" in msg
+    # a dtype matmul has no arithmetic for
+    s, msg = status_and_message(hip_backend, lib.hc_matmul(ctx, int(DType.bool), 1, p, 0, p, 0, 0, 2, 2, 2, p))
+    assert s == _lib.HC_ERR_UNSUPPORTED and "not numeric" in msg
     # negative dimension, null pointers
     assert lib.hc_matmul(ctx, int(DType.float32), 1, p, 0, p, 0, 0, -1, 2, 2, p) == _lib.HC_ERR_INVALID
     assert lib.hc_matmul(ctx, int(DType.float32), 1, None, 0, p, 0, 0, 2, 2, 2, p) == _lib.HC_ERR_INVALID
@@ -57,7 +57,7 @@ def test_errors_surface_as_backend_errors(hip_backend):
     with hip_backend.use():
         x = Tensor(data=np.arange(6, dtype=np.int64).reshape(2, 3))
         with pytest.raises(BackendError) as e:
-            Tensor.matmul(x, False, x.t(), False, False)          # int64 matmul: not on this backend
+            x.logSoftmax(axis=1)                                  # no integer logSoftmax on any backend
         assert e.value.kind == "notImplemented"
         with pytest.raises(BackendError) as e:
             hip_backend.allocate(1 << 50)

@@ -139,6 +139,26 @@ def test_matmul_fp16_4096_against_oracle_slab_and_identity(hip_backend, oracle_b
         assert np.array_equal(Tensor.matmul(eye, False, tb, False, False).numpy(), b)
 
 
+def test_matmul_int64(hip_backend, oracle_backend):
+    """int64 products (BackendCPU.swift:1307): all flag combinations, ragged extents, a batch."""
+    rng = np.random.default_rng(8)
+    for (m, k, n) in [(17, 33, 9), (64, 16, 48), (1, 5, 1), (40, 0, 3)]:
+        a = rng.integers(-1000, 1000, size=(m, k))
+        b = rng.integers(-1000, 1000, size=(k, n))
+        for ta in (False, True):
+            for tb in (False, True):
+                for to in (False, True):
+                    an = np.ascontiguousarray(a.T) if ta else a
+                    bn = np.ascontiguousarray(b.T) if tb else b
+                    fn = lambda: Tensor.matmul(Tensor(data=an), ta, Tensor(data=bn), tb, to)
+                    check_exact(hip_backend, oracle_backend, fn)
+                    with hip_backend.use():
+                        assert np.array_equal(fn().numpy(), (a @ b).T if to else a @ b)
+    a = rng.integers(-(2 ** 40), 2 ** 40, size=(3, 6, 7))        # sums that wrap around 2^64
+    b = rng.integers(-(2 ** 40), 2 ** 40, size=(3, 7, 5))
+    check_exact(hip_backend, oracle_backend, lambda: Tensor.batchedMatmul(Tensor(data=a), False, Tensor(data=b), False, False))
+
+
 def test_matmul_fp32_1024(hip_backend, oracle_backend):
     """Config 1: fp32 [1024,1024] x [1024,1024], N(0,1) entries, no transposes."""
     rng = np.random.default_rng(1)
