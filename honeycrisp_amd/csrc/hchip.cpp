@@ -1291,8 +1291,7 @@ extern "C" int hc_argsort(hc_ctx* ctx, int dtype, const void* in, void* out, int
       s.idx_in = (const uint32_t*)idx[cur];
       s.keys_out = (uint64_t*)keys[cur ^ 1];
       s.idx_out = (uint32_t*)idx[cur ^ 1];
-      HC_TRY(launch(ctx, "hc_argsort_merge", ceil_div(lines * ceil_div((uint64_t)reduce, 8), HCK_BLOCK), 1, &s,
-                    sizeof(s)));
+      HC_TRY(launch(ctx, "hc_argsort_merge", lines * ceil_div((uint64_t)reduce, 8 * HCK_BLOCK), 1, &s, sizeof(s)));
     }
     s.idx_in = (const uint32_t*)idx[cur];
     return launch(ctx, "hc_argsort_emit", ceil_div(total, HCK_BLOCK), 1, &s, sizeof(s));
