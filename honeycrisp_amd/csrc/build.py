@@ -26,6 +26,7 @@ KERNELS = [
     ("gemm", "gemm.hip", []),
     ("gemm_f16_fast", "gemm_f16_fast.hip", []),
     ("gemm_dma", "gemm_dma.hip", []),
+    ("gemm_dma2", "gemm_dma2.hip", []),
 ]
 DEVICE_FLAGS = [
     "--offload-arch=gfx950", "--genco", "-O3", "-std=c++17",

@@ -21,5 +21,6 @@
     EMBED hc_image_gemm, "gemm.hsaco"
     EMBED hc_image_gemm_f16_fast, "gemm_f16_fast.hsaco"
     EMBED hc_image_gemm_dma, "gemm_dma.hsaco"
+    EMBED hc_image_gemm_dma2, "gemm_dma2.hsaco"
 
     .section .note.GNU-stack,"",@progbits

@@ -30,6 +30,7 @@ extern const unsigned char hc_image_probe[], hc_image_probe_end[];
 extern const unsigned char hc_image_gemm[], hc_image_gemm_end[];
 extern const unsigned char hc_image_gemm_f16_fast[], hc_image_gemm_f16_fast_end[];
 extern const unsigned char hc_image_gemm_dma[], hc_image_gemm_dma_end[];
+extern const unsigned char hc_image_gemm_dma2[], hc_image_gemm_dma2_end[];
 }
 
 struct hc_module {
@@ -148,6 +149,7 @@ extern "C" int hc_init(int device, hc_ctx** out) {
   if (s == HC_OK) s = load_image(ctx, hc_image_gemm, hc_image_gemm_end, "gemm");
   if (s == HC_OK) s = load_image(ctx, hc_image_gemm_f16_fast, hc_image_gemm_f16_fast_end, "gemm_f16_fast");
   if (s == HC_OK) s = load_image(ctx, hc_image_gemm_dma, hc_image_gemm_dma_end, "gemm_dma");
+  if (s == HC_OK) s = load_image(ctx, hc_image_gemm_dma2, hc_image_gemm_dma2_end, "gemm_dma2");
   if (s == HC_OK) {
     hipError_t e = hipMalloc(&ctx->zeros, 256);
     if (e == hipSuccess) e = hipMemset(ctx->zeros, 0, 256);
@@ -1941,7 +1943,12 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
   const char* which = getenv("HCHIP_GEMM_KERNEL");
   const uint64_t max_elems = 0xffffffffull / el;
   const bool dma = k.a_bs <= max_elems && k.b_bs <= max_elems && !(which && strcmp(which, "staged") == 0);
-  const uint32_t slice = (uint32_t)(64 / el);
+  // Two direct-to-LDS pipelines: four stages of 64-byte K-slices (deep prefetch: best when a CU
+  // has one short job) and two stages of 128-byte K-slices (whole cache lines for K-contiguous
+  // operands, half the barriers: best when the CUs are kept busy for long). Chosen below, after
+  // the tile; HCHIP_GEMM_KERNEL=dma|dma2 forces one.
+  bool dma2 = dma && which && strcmp(which, "dma2") == 0;
+  uint32_t slice = (uint32_t)(64 / el);
   const bool eligible = ma != 'x' && mb != 'x' && K > 0 && aligned16(k.c) &&
                         (dma ? (k.c_rs % P == 0 && (batch <= 1 || k.c_bs % P == 0)) : (dtype == HC_F16 && K % 64 == 0));
   if (eligible) {
@@ -1991,6 +1998,11 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
         }
       }
     }
+    if (bm != 0 && dma) {
+      const uint64_t blocks = ceil_div(M, bm) * ceil_div(N, bn) * (uint64_t)batch;
+      if (!which && (uint64_t)K * el >= 2048 && ((bm == 256 && bn == 256) || blocks >= 2 * cus)) dma2 = true;
+      if (dma2) slice = (uint32_t)(128 / el);
+    }
     if (bm != 0) edge = !whole(bm, bn);
   }
   if (bm != 0) {
@@ -2008,7 +2020,7 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
           break;
         }
     }
-    snprintf(name, sizeof(name), "hc_gemm_%s_%s_%ux%u_%c%c%s", dtype_name(dtype), dma ? "dma" : "fast", bm, bn,
+    snprintf(name, sizeof(name), "hc_gemm_%s_%s_%ux%u_%c%c%s", dtype_name(dtype), dma ? (dma2 ? "dma2" : "dma") : "fast", bm, bn,
              ma == 'k' ? 'k' : 'm', mb == 'k' ? 'k' : 'n', edge ? "_e" : "");
   } else if (ma == 'x' || mb == 'x')
     snprintf(name, sizeof(name), "hc_gemm_%s_xx", dtype_name(dtype));

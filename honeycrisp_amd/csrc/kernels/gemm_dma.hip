@@ -43,7 +43,8 @@
 // Measurement switches (never set in the shipped build): bit0 no DMA in the K loop, bit1 no
 // wait/barrier, bit2 no LDS reads in the K loop, bit3 every K-step fetches slice 0 again, bit4
 // only every other DMA instruction, bit5 every DMA instruction fetches the same 1 KiB,
-// bit6 / bit7 fetch A only, as pairs of adjacent 64-byte pieces / as single pieces. Results are wrong with any bit set.
+// bit6 / bit7 fetch A only, as pairs of adjacent 64-byte pieces / as single pieces, bit8
+// K-contiguous operands are fetched as whole 128-byte lines (half of the rows per K-step). Results are wrong with any bit set.
 #ifndef HC_EXP
 #define HC_EXP 0
 #endif
@@ -99,6 +100,7 @@ template <typename T, int ROWS, int MODE> struct DmaOperand {
 
   uint32_t goff[NI];     // byte offset of this lane's 16-byte piece for DMA instruction i (k = 0)
   uint32_t kstride;      // bytes per unit of k
+  uint32_t half_rows = 0; // measurement builds only
   uint32_t raddr[NADDR]; // byte offsets (inside the operand's LDS region) of the MFMA operand reads
 
   // `limit` (edge kernels): extent of this operand along M / N. Rows or 16-byte pieces past it
@@ -115,6 +117,10 @@ template <typename T, int ROWS, int MODE> struct DmaOperand {
         uint32_t grow = r0 + row;
         if (limit && grow >= limit) grow = limit - 1;
         goff[i] = grow * rs * ES + c * 16;
+        if (HC_EXP & 256) {  // whole 128-byte lines: 8 lanes per row, half of the rows per K-step
+          goff[i] = (r0 + (wave * NI + i) * 8 + lane / 8) * rs * ES + (lane % 8) * 16;
+          half_rows = (ROWS / 2) * rs * ES;
+        }
       }
       const uint32_t lrow = lane & 31, lgrp = lane >> 5;
 #pragma unroll
@@ -188,6 +194,11 @@ template <typename T, int ROWS, int MODE> struct DmaOperand {
     // The empty asm keeps the zero-extension of the lane offset next to the load, so that the
     // load takes the form "scalar base + 32-bit lane offset" with no vector add in front of it.
     uint32_t off = goff[i];
+    if ((HC_EXP & 256) && MODE == DMA_K) {
+      const uint32_t slice = k0 / (64 / ES);
+      off += (slice & 1) * half_rows;
+      k0 = (slice & ~1u) * (64 / ES);
+    }
     asm volatile("" : "+v"(off));
     const char* src = (const char*)base + (size_t)k0 * kstride + off;
     if (kend != 0 && k0 + 64 / ES > kend) {  // wave-uniform
@@ -351,7 +362,11 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
     if (!(HC_EXP & 2)) {
 #ifdef HC_PROBE_WAITS
       const uint64_t w0 = __builtin_readcyclecounter();
+#ifdef HC_PROBE_SLACK
+      wait_dma<HC_PROBE_SLACK>();  // fewer DMA instructions left in flight: less time to land
+#else
       wait_dma<2 * NDMA>();
+#endif
       const uint64_t w1 = __builtin_readcyclecounter();
       lds_barrier();
       const uint64_t w2 = __builtin_readcyclecounter();

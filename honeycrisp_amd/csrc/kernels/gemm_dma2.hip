@@ -1,0 +1,431 @@
+// fp16 and fp32 GEMM for gfx950 with direct global->LDS loads (global_load_lds_dwordx4) and,
+// for fp16 operands that are contiguous along M/N, transposing LDS reads
+// (ds_read_b64_tr_b16). Block tile BM x BN, 4 waves 2 x 2, fp32 accumulate with
+// v_mfma_f32_32x32x16_f16 / v_mfma_f32_32x32x2_f32. No operand passes through VGPRs on its
+// way to LDS.
+//
+// LDS: two stages, each one K-slice of 128 bytes (64 halfs, 32 floats):
+// [A region: BM*128 bytes][B region: BN*128 bytes]. 128 bytes because that is a cache line: a
+// K-contiguous operand is then fetched as whole lines (8 lanes per row), which costs markedly
+// less power and fewer texture-address cycles than two 64-byte halves fetched separately.
+//   K-contiguous operand (A of NN/NT, B of NT/TT): rows of 128 bytes = eight 16-byte slots,
+//     chunk c of row r in slot c ^ (r & 7); MFMA operand = one ds_read_b128, rows r .. r+7 of
+//     one read hit eight different slots. For fp32 the four floats of a chunk feed four
+//     consecutive MFMAs; lanes 0..31 take chunk 2s and lanes 32..63 chunk 2s+1 in sub-step s,
+//     a permutation of k that both operands share.
+//   M/N-contiguous fp16 operand (A of TN/TT, B of NN/TN): natural [k][m] layout, 64 k-rows of
+//     ROWS halfs, 16-byte slot x of k-row k stored at slot x ^ g(k),
+//     g(k) = ((k&7) ^ ((k>>3&1)<<2)) << 1. MFMA operand = two ds_read_b64_tr_b16: in a group
+//     of 16 lanes, lane r points at k-row k0 + r/4, columns 4*(r%4)..+3 (8 bytes); the
+//     instruction returns to lane i the four k-values of column i. Two reads (k0, k0+4) give
+//     a lane its 8 consecutive k for one m, in the same order as the K-contiguous operand.
+//   M/N-contiguous fp32 operand: [32 k][ROWS floats], MFMA operands are single ds_read_b32
+//     (32 consecutive floats of k-row k for lanes 0..31, of k-row k+4 for lanes 32..63).
+// A wave-level DMA instruction fills 1 KiB of LDS in lane order (lane l -> byte 16*l), so
+// any permutation of 16-byte pieces inside a 1 KiB block is free: the lane simply fetches
+// the global piece that belongs in its slot. Both swizzles stay inside such blocks.
+//
+// Pipeline. A K-step (one stage) is four sub-steps of one MFMA per accumulator tile, operands
+// of the next sub-step being read under the MFMAs of the current one:
+//   sub-step 0: second half of the DMA of K-step j+1 into the other stage
+//   sub-steps 1, 2: no DMA: the loads in flight get at least these 2 x SLOTS MFMAs to land
+//     (measured need: about 600 cycles)
+//   wait for this wave's DMA (vmcnt 0), one LDS barrier: the other stage is complete and
+//     nobody reads this stage any more
+//   sub-step 3: first operands of K-step j+1 are read; first half of the DMA of K-step j+2
+//     into this stage.
+// DMA instructions are spread over the MFMAs of their sub-step (a burst would stall the
+// issuing wave behind the texture-address queue). The two stages are distinct __shared__
+// arrays and the loop is unrolled by two so that every LDS access names its stage statically.
+#include "common.hip.h"
+
+// length of the DMA window in half sub-steps (see the K loop)
+#ifndef HC_DMA_WINDOW_X2
+#define HC_DMA_WINDOW_X2 4
+#endif
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef uint32_t Chunk __attribute__((ext_vector_type(4)));  // 16 bytes = 8 halfs
+
+enum { DMA_K = 0, DMA_MN = 1 };
+
+#define LDS_AS __attribute__((address_space(3)))
+#define GLOBAL_AS __attribute__((address_space(1)))
+
+__device__ __forceinline__ uint32_t swz_k(uint32_t row) { return row & 7u; }
+__device__ __forceinline__ uint32_t swz_mn(uint32_t k) { return (((k & 7u) ^ (((k >> 3) & 1u) << 2)) << 1); }
+
+// Workgroup barrier for LDS traffic only: this wave's LDS reads have returned (lgkmcnt), its
+// DMA is waited for separately (wait_dma), and nothing is said about global memory. A fence
+// builtin would do the same but also waits for every DMA instruction in flight, including
+// those that fill stages nobody is about to read. The "memory" clobber keeps the compiler
+// from moving LDS accesses across it.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+// s_waitcnt vmcnt(N) with the other counters untouched (gfx9 encoding: vmcnt in bits 3:0 and
+// 15:14, expcnt 6:4, lgkmcnt 11:8): at most N of this wave's DMA instructions still in flight.
+template <int N> __device__ __forceinline__ void wait_dma() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
+}
+
+// One operand of the block tile: where its DMA lanes fetch from and where a wave's MFMA
+// operand reads land.
+template <typename T, int ROWS, int MODE> struct DmaOperand {
+  static constexpr int ES = sizeof(T);
+  static constexpr bool F32 = ES == 4;
+  static constexpr int NI = ROWS / 32;                        // DMA instructions per wave and K-step
+  static constexpr int TILES = ROWS / 64;                     // MFMA tiles per wave along this operand
+  // LDS reads per sub-step
+  static constexpr int READS = MODE == DMA_K ? TILES : (F32 ? 4 * TILES : 2 * TILES);
+  static constexpr int NADDR = MODE == DMA_K ? TILES * 4 : TILES * 2;
+  static constexpr int ROWB = ROWS * ES;                      // bytes per k-row (DMA_MN layout)
+  static constexpr int BYTES = ROWS * 128;                    // per stage
+
+  uint32_t goff[NI];     // byte offset of this lane's 16-byte piece for DMA instruction i (k = 0)
+  uint32_t kstride;      // bytes per unit of k
+  uint32_t raddr[NADDR]; // byte offsets (inside the operand's LDS region) of the MFMA operand reads
+
+  // `limit` (edge kernels): extent of this operand along M / N. Rows or 16-byte pieces past it
+  // are fetched from the last valid row / piece instead: they only feed outputs that are
+  // never stored. 0 = no clamping.
+  __device__ __forceinline__ void init(uint32_t rs, uint32_t cs, uint32_t r0, uint32_t woff, uint32_t limit) {
+    const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    if (MODE == DMA_K) {
+      kstride = ES;
+#pragma unroll
+      for (int i = 0; i < NI; i++) {
+        const uint32_t row = (wave * NI + i) * 8 + lane / 8;
+        const uint32_t c = (lane % 8) ^ swz_k(row);
+        uint32_t grow = r0 + row;
+        if (limit && grow >= limit) grow = limit - 1;
+        goff[i] = grow * rs * ES + c * 16;
+      }
+      const uint32_t lrow = lane & 31, lgrp = lane >> 5;
+#pragma unroll
+      for (int q = 0; q < TILES; q++) {
+        const uint32_t r = woff + q * 32 + lrow;
+#pragma unroll
+        for (int s = 0; s < 4; s++) raddr[q * 4 + s] = r * 128 + (((2 * s + lgrp) ^ swz_k(r)) * 16);
+      }
+    } else if (F32) {
+      // [32 k][ROWS floats]; the 128-byte halves of every 256 bytes swap places in k-rows
+      // with bit 2 set: an MFMA operand read touches rows k and k + 4, 32 floats of each
+      constexpr uint32_t KPI = 1024 / ROWB;   // k-rows per DMA instruction
+      constexpr uint32_t PIECES = ROWB / 16;  // 16-byte pieces per k-row
+      kstride = cs * ES;
+#pragma unroll
+      for (int i = 0; i < NI; i++) {
+        const uint32_t krow = (wave * NI + i) * KPI + lane / PIECES;
+        const uint32_t piece = (lane % PIECES) ^ (((krow >> 2) & 1u) << 3);
+        uint32_t col = r0 + piece * 4;
+        if (limit && col + 4 > limit) col = limit - 4;
+        goff[i] = (krow * cs + col) * ES;
+      }
+      const uint32_t lrow = lane & 31, lgrp = lane >> 5;
+#pragma unroll
+      for (int q = 0; q < TILES; q++) {
+        const uint32_t n = woff + q * 32 + lrow;  // k = 4 * lgrp + e + 8 * s, e and s as immediates
+        raddr[q] = 4 * lgrp * ROWB + ((n ^ (lgrp << 5)) * 4);
+      }
+    } else {
+      constexpr int KPI = 512 / ROWS;       // k-rows per DMA instruction
+      constexpr uint32_t SLOTS_PER_ROW = ROWS / 8;
+      kstride = cs * 2;
+#pragma unroll
+      for (int i = 0; i < NI; i++) {
+        const uint32_t krow = (wave * NI + i) * KPI + lane / SLOTS_PER_ROW;
+        const uint32_t slot = (lane % SLOTS_PER_ROW) ^ (swz_mn(krow) & (SLOTS_PER_ROW - 1));
+        uint32_t col = r0 + slot * 8;
+        if (limit && col + 8 > limit) col = limit - 8;
+        goff[i] = (krow * cs + col) * 2;
+      }
+      const uint32_t j = lane >> 4, r16 = lane & 15;
+#pragma unroll
+      for (int q = 0; q < TILES; q++) {
+        const uint32_t m = woff + q * 32 + 16 * (j & 1) + 4 * (r16 & 3);
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+          const uint32_t k = 8 * (j >> 1) + 4 * h + (r16 >> 2);  // + 16 * s as an immediate offset
+          raddr[q * 2 + h] = k * ROWB + (((m >> 3) ^ (swz_mn(k) & (ROWS / 8 - 1))) * 16) + (m & 7) * 2;
+        }
+      }
+    }
+  }
+
+  // k offset, inside a K-slice, of the piece this lane fetches with DMA instruction i
+  __device__ __forceinline__ uint32_t klocal(int i) const {
+    const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    if (MODE == DMA_K) {
+      const uint32_t row = (wave * NI + i) * 8 + lane / 8;
+      return ((lane % 8) ^ swz_k(row)) * (16 / ES);
+    }
+    constexpr uint32_t PER_ROW = ROWB / 16, KPI = 1024 / ROWB;
+    return (wave * NI + i) * KPI + lane / PER_ROW;
+  }
+
+  // DMA instruction i of this wave for the K-slice starting at k0: 1 KiB into `region`.
+  // Edge kernels (kend != 0): pieces at k >= kend come from `zeros` (16 zero bytes) instead,
+  // so the ragged last slice contributes nothing.
+  __device__ __forceinline__ void dma(int i, const T* base, uint32_t k0, char* region, uint32_t kend = 0,
+                                      const void* zeros = nullptr) const {
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    // The empty asm keeps the zero-extension of the lane offset next to the load, so that the
+    // load takes the form "scalar base + 32-bit lane offset" with no vector add in front of it.
+    uint32_t off = goff[i];
+    asm volatile("" : "+v"(off));
+    const char* src = (const char*)base + (size_t)k0 * kstride + off;
+    if (kend != 0 && k0 + 128 / ES > kend) {  // wave-uniform
+      if (k0 + klocal(i) >= kend) src = (const char*)zeros;
+    }
+    __builtin_amdgcn_global_load_lds((const GLOBAL_AS void*)src, (LDS_AS void*)(region + (wave * NI + i) * 1024), 16, 0, 0);
+  }
+
+  // Read number u of sub-step s into the operand registers of tile u (DMA_K), half u%2 of
+  // tile u/2 (DMA_MN, fp16) or element u%4 of tile u/4 (DMA_MN, fp32).
+  __device__ __forceinline__ void read(int u, int s, const char* region, Chunk* frag) const {
+    if (MODE == DMA_K) {
+      frag[u] = *reinterpret_cast<const Chunk*>(region + raddr[u * 4 + s]);
+    } else if (F32) {
+      const int q = u / 4, e = u % 4;
+      frag[q][e] = *reinterpret_cast<const uint32_t*>(region + raddr[q] + (8 * s + e) * ROWB);
+    } else {
+      const int q = u / 2, h = u % 2;
+      typedef short short4v __attribute__((ext_vector_type(4)));
+      const short4v v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (LDS_AS short4v*)(region + raddr[q * 2 + h] + s * 16 * ROWB));
+      typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+      const u32x2 w = __builtin_bit_cast(u32x2, v);
+      frag[q][2 * h] = w[0];
+      frag[q][2 * h + 1] = w[1];
+    }
+  }
+};
+
+template <typename T, int BM, int BN, int MODE_A, int MODE_B, bool EDGE>
+__device__ __forceinline__ void gemm_dma2_impl(const hck_gemm_args& p, char* lds0, char* lds1) {
+  constexpr int MT = BM / 64, NT = BN / 64;
+  constexpr int SLOTS = MT * NT;
+  typedef DmaOperand<T, BM, MODE_A> OpA;
+  typedef DmaOperand<T, BN, MODE_B> OpB;
+  constexpr bool F32 = sizeof(T) == 4;
+  constexpr uint32_t BK = 128 / sizeof(T);  // K-slice of one stage
+  constexpr int READS = OpA::READS + OpB::READS;
+  constexpr int NDMA = OpA::NI + OpB::NI;  // per wave and K-step
+  constexpr int HALF = NDMA / 2;
+  constexpr int A_BYTES = OpA::BYTES;
+
+  // XCD-aware tile order. Block ids equal mod 8 run on one XCD and share its L2: give each
+  // XCD a compact rectangle of tiles (few distinct A and B panels), or a contiguous band.
+  const uint32_t total = p.tiles_m * p.tiles_n;
+  uint32_t tile = blockIdx.x;
+  if (p.xcd_gn != 0) {
+    const uint32_t per = 8 * p.xcd_sm * p.xcd_sn, gm = 8 / p.xcd_gn;
+    const uint32_t group = blockIdx.x / per, w = blockIdx.x - group * per;
+    const uint32_t x = w & 7u, t = w >> 3;
+    const uint32_t sbn = p.tiles_n / (p.xcd_gn * p.xcd_sn);
+    const uint32_t sb_row = group / sbn, sb_col = group - sb_row * sbn;
+    const uint32_t xm = x / p.xcd_gn, xn = x - xm * p.xcd_gn;
+    const uint32_t lm = t / p.xcd_sn, ln = t - lm * p.xcd_sn;
+    tile = (sb_row * gm * p.xcd_sm + xm * p.xcd_sm + lm) * p.tiles_n + sb_col * p.xcd_gn * p.xcd_sn + xn * p.xcd_sn + ln;
+  } else if ((total & 7u) == 0) {
+    tile = (blockIdx.x & 7u) * (total >> 3) + (blockIdx.x >> 3);
+  }
+  const uint32_t tm = tile / p.tiles_n, tn = tile - tm * p.tiles_n;
+  const uint32_t m0 = tm * BM, n0 = tn * BN;
+  const uint32_t batch = blockIdx.y;
+  const T* A = (const T*)p.a + batch * p.a_bs;
+  const T* B = (const T*)p.b + batch * p.b_bs;
+  T* C = (T*)p.c + batch * p.c_bs;
+
+  const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const uint32_t wm = (wave >> 1) * (BM / 2), wn = (wave & 1) * (BN / 2);
+  const uint32_t lrow = lane & 31, lgrp = lane >> 5;
+
+  floatx16 acc[MT][NT];
+#pragma unroll
+  for (int i = 0; i < MT; i++)
+#pragma unroll
+    for (int j = 0; j < NT; j++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+
+  OpA oa;
+  OpB ob;
+  oa.init(p.a_rs, p.a_cs, m0, wm, EDGE ? p.a_lim : 0);
+  ob.init(p.b_cs, p.b_rs, n0, wn, EDGE ? p.b_lim : 0);
+  const uint32_t kend = EDGE ? p.K : 0;
+
+  struct Frags {
+    Chunk a[MT];
+    Chunk b[NT];
+  };
+  // unit u of the operand reads of a sub-step: B's reads first, then A's
+  auto read_unit = [&](Frags& f, const char* stage, int s, int u) {
+    if (u < OpB::READS) ob.read(u, s, stage + A_BYTES, f.b);
+    else if (u < READS) oa.read(u - OpB::READS, s, stage, f.a);
+  };
+  // unit u of the DMA of the K-slice starting at k0
+  auto dma_unit = [&](int u, uint32_t k0, char* stage) {
+    if (u < OpA::NI) oa.dma(u, A, k0, stage, kend, p.zeros);
+    else if (u < NDMA) ob.dma(u - OpA::NI, B, k0, stage + A_BYTES, kend, p.zeros);
+  };
+  // MFMA t of a sub-step; operands swapped (B first) so that a lane holds four consecutive
+  // n for one m (see the epilogue).
+  auto mma_one = [&](const Frags& f, int t) {
+    const int i = t / NT, j = t % NT;
+    if constexpr (F32) {
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        // (copies first: a bit_cast applied directly to a vector element reads element 0)
+        const uint32_t wb = f.b[j][e], wa = f.a[i][e];
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(__builtin_bit_cast(float, wb),
+                                                         __builtin_bit_cast(float, wa), acc[i][j], 0, 0, 0);
+      }
+    } else {
+      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, f.b[j]),
+                                                         __builtin_bit_cast(half8, f.a[i]), acc[i][j], 0, 0, 0);
+    }
+  };
+  // reads per MFMA slot of a sub-step
+  constexpr int RPS = (READS + SLOTS - 1) / SLOTS;
+  // The DMA of a K-slice is spread evenly over a window of W MFMA slots that starts right
+  // after the barrier that frees its stage (sub-step 3 of the step before the previous one,
+  // then sub-steps 0 and 1): unit u goes out in window slot u * W / NDMA. The rest of the
+  // 3 * SLOTS .. 4 * SLOTS slots before the next barrier is the time the last loads get to land.
+  constexpr int W = SLOTS * HC_DMA_WINDOW_X2 / 2 > 0 ? SLOTS * HC_DMA_WINDOW_X2 / 2 : 1;
+  static_assert(W <= 3 * SLOTS, "the DMA window ends with sub-step 1");
+  auto window_slot = [](int u) { return u * W / NDMA; };
+  // units of the first window part (sub-step 3): [0, U0)
+  constexpr int U0 = (SLOTS * NDMA + W - 1) / W < NDMA ? (SLOTS * NDMA + W - 1) / W : NDMA;
+
+  const uint32_t nk = (p.K + BK - 1) / BK;
+  auto kclamp = [&](uint32_t j) { return (j < nk ? j : nk - 1) * BK; };  // steps past the end repeat the last one
+  Frags f0, f1;
+
+  // sub-step: MFMAs on `use`, operands of the following sub-step (number s_next of `from`)
+  // into `fill`, and the DMA units of window part `part` (0, 1, 2; -1: none) of the K-slice
+  // at k0 into `to`
+  auto substep = [&](const Frags& use, Frags& fill, const char* from, int s_next, int part, char* to, uint32_t k0) {
+#pragma unroll
+    for (int t = 0; t < SLOTS; t++) {
+      if (part >= 0) {
+#pragma unroll
+        for (int u = 0; u < NDMA; u++)
+          if (window_slot(u) == part * SLOTS + t) dma_unit(u, k0, to);
+      }
+#pragma unroll
+      for (int e = 0; e < RPS; e++) read_unit(fill, from, s_next, t * RPS + e);
+      mma_one(use, t);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  // K-step j out of `cur`; `nxt` receives the rest of K-step j+1, then `cur` the start of j+2
+  auto step = [&](char* cur, char* nxt, uint32_t j) {
+    __builtin_amdgcn_sched_barrier(0);
+    substep(f0, f1, cur, 1, 1, nxt, kclamp(j + 1));
+    substep(f1, f0, cur, 2, 2, nxt, kclamp(j + 1));
+    substep(f0, f1, cur, 3, -1, nullptr, 0);
+    wait_dma<0>();  // K-step j+1 of this wave has landed ...
+    lds_barrier();  // ... and everybody's; nobody reads cur any more
+    __builtin_amdgcn_sched_barrier(0);
+    substep(f1, f0, nxt, 0, 0, cur, kclamp(j + 2));
+  };
+
+  // prologue: K-step 0 and the first window part of K-step 1
+#pragma unroll
+  for (int u = 0; u < NDMA; u++) dma_unit(u, 0, lds0);
+#pragma unroll
+  for (int u = 0; u < U0; u++) dma_unit(u, kclamp(1), lds1);
+  wait_dma<U0>();
+  lds_barrier();
+#pragma unroll
+  for (int u = 0; u < READS; u++) read_unit(f0, lds0, 0, u);
+
+  uint32_t j = 0;
+  for (; j + 1 < nk; j += 2) {
+    step(lds0, lds1, j);
+    step(lds1, lds0, j + 1);
+  }
+  if (j < nk) step(lds0, lds1, j);
+  wait_dma<0>();  // no LDS write of this workgroup may be in flight when it ends
+
+  // Epilogue. With the operands swapped, the MFMA tile is C^T: lane l holds m = l % 32 and,
+  // in registers 4g..4g+3, the four consecutive columns n = 8g + 4*(l/32) + (0..3). Stored
+  // directly that would be short pieces of 32 different rows per instruction, so the wave's
+  // part of C goes through LDS in slabs of 32 rows (both stages are free now; wave w uses
+  // half of a stage) and leaves as 16-byte pieces, whole rows of the slab contiguous. 16-byte unit u
+  // of row r sits at unit u ^ s(r) to spread the column-wise writes over the banks. A wave's
+  // LDS instructions execute in order, so a slab may be overwritten right after its reads.
+  lds_barrier();
+  char* mine = (wave < 2 ? lds0 : lds1) + (wave & 1) * ((BM + BN) * 64);
+  constexpr uint32_t ES = sizeof(T), WN = BN / 2, RB = WN * ES, UNITS = RB / 16, RPI = 64 / UNITS;
+  constexpr uint32_t SLAB = 32 * RB, NSLAB = (BM + BN) * 64 / SLAB;
+  static_assert(NSLAB >= 1 && UNITS <= 64, "a slab must fit one stage");
+  auto unit_swz = [&](uint32_t r) { return (RB >= 256 ? r : r * RB / 256) & (UNITS - 1); };
+#pragma unroll
+  for (int i = 0; i < MT; i++) {
+    char* slab = mine + (i % NSLAB) * SLAB;
+#pragma unroll
+    for (int j = 0; j < NT; j++) {
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        if constexpr (F32) {
+          floatx4 h;
+#pragma unroll
+          for (int e = 0; e < 4; e++) h[e] = acc[i][j][4 * g + e];
+          *reinterpret_cast<floatx4*>(slab + lrow * RB + (((j * 8 + 2 * g + lgrp) ^ unit_swz(lrow)) * 16)) = h;
+        } else {
+          half4v h;
+#pragma unroll
+          for (int e = 0; e < 4; e++) h[e] = narrow<half_t>(acc[i][j][4 * g + e]);
+          *reinterpret_cast<half4v*>(slab + lrow * RB + (((j * 4 + g) ^ unit_swz(lrow)) * 16) + lgrp * 8) = h;
+        }
+      }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // wave-private region: no barrier needed
+#pragma unroll
+    for (uint32_t it = 0; it < 32 / RPI; it++) {
+      const uint32_t r = it * RPI + lane / UNITS, u = lane % UNITS;
+      const Chunk v = *reinterpret_cast<const Chunk*>(slab + r * RB + ((u ^ unit_swz(r)) * 16));
+      const uint32_t row = m0 + wm + i * 32 + r, col = n0 + wn + u * (16 / ES);
+      if (!EDGE || (row < p.M && col < p.N)) *reinterpret_cast<Chunk*>(C + (size_t)row * p.c_rs + col) = v;
+    }
+    asm volatile("" ::: "memory");
+  }
+}
+
+// Two variants per kernel: whole tiles only, and "_e" (edge) for M, N that are not multiples of
+// the tile and K that is not a multiple of the K-slice (64 halfs, 32 floats).
+#define DEF_DMA(T, TN, BM, BN, AN, AM, BNAME, BMODE)                                                  \
+  extern "C" __global__ __launch_bounds__(256) void hc_gemm_##TN##_dma2_##BM##x##BN##_##AN##BNAME(     \
+      hck_gemm_args p) {                                                                              \
+    __shared__ __attribute__((aligned(1024))) char lds0[(BM + BN) * 128];                             \
+    __shared__ __attribute__((aligned(1024))) char lds1[(BM + BN) * 128];                             \
+    gemm_dma2_impl<T, BM, BN, AM, BMODE, false>(p, lds0, lds1);                                       \
+  }                                                                                                   \
+  extern "C" __global__ __launch_bounds__(256) void hc_gemm_##TN##_dma2_##BM##x##BN##_##AN##BNAME##_e( \
+      hck_gemm_args p) {                                                                              \
+    __shared__ __attribute__((aligned(1024))) char lds0[(BM + BN) * 128];                             \
+    __shared__ __attribute__((aligned(1024))) char lds1[(BM + BN) * 128];                             \
+    gemm_dma2_impl<T, BM, BN, AM, BMODE, true>(p, lds0, lds1);                                        \
+  }
+#define DEF_DMA_TILE(T, TN, BM, BN)                                                                   \
+  DEF_DMA(T, TN, BM, BN, k, DMA_K, k, DMA_K)                                                          \
+  DEF_DMA(T, TN, BM, BN, k, DMA_K, n, DMA_MN)                                                         \
+  DEF_DMA(T, TN, BM, BN, m, DMA_MN, k, DMA_K)                                                         \
+  DEF_DMA(T, TN, BM, BN, m, DMA_MN, n, DMA_MN)
+#define DEF_DMA_TYPE(T, TN)                                                                           \
+  DEF_DMA_TILE(T, TN, 256, 256)                                                                       \
+  DEF_DMA_TILE(T, TN, 256, 128)                                                                       \
+  DEF_DMA_TILE(T, TN, 128, 128)                                                                       \
+  DEF_DMA_TILE(T, TN, 256, 64)                                                                        \
+  DEF_DMA_TILE(T, TN, 128, 64)                                                                        \
+  DEF_DMA_TILE(T, TN, 64, 64)
+DEF_DMA_TYPE(half_t, f16)
+DEF_DMA_TYPE(float, f32)
