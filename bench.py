@@ -36,7 +36,7 @@ PEAK_HBM_GBS = 8000.0     # MI355X HBM3E
 # HBM bytes per 4096^3 fp16 GEMM launch, from rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs of
 # this benchmark scaled by a plain copy kernel (not measurable live; the run that produced it is
 # summarised in profiles/bench_hbm_traffic_fetch_write_size.md): 196850 KiB read + 32768 KiB written.
-GEMM_TRAFFIC_BYTES = (196850 + 32768) * 1024
+GEMM_TRAFFIC_BYTES = (196800 + 32768) * 1024
 
 
 class Events:
