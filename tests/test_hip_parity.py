@@ -117,6 +117,30 @@ def test_batched_matmul_all_flags_small(hip_backend, oracle_backend):
                     check_close(hip_backend, oracle_backend, fn, TOL[dtype])
 
 
+@pytest.mark.parametrize("pipeline", ["dma", "dma2"])
+@pytest.mark.parametrize("dtype", [F32, F16], ids=["f32", "f16"])
+def test_matmul_both_pipelines_every_tile(hip_backend, oracle_backend, monkeypatch, pipeline, dtype):
+    """The host picks a direct-to-LDS pipeline and a tile by problem size; here every tile of both
+    pipelines is forced in turn (the library reads the two variables at every call) on whole-tile,
+    ragged (edge kernels: clamped rows, zero-filled K tail) and batched problems, all four layouts."""
+    rng = np.random.default_rng(77)
+    monkeypatch.setenv("HCHIP_GEMM_KERNEL", pipeline)
+    for tile in ("256x256", "256x128", "128x128", "256x64", "128x64", "64x64"):
+        monkeypatch.setenv("HCHIP_GEMM_TILE", tile)
+        for (batch, M, K, N) in [(1, 256, 192, 256), (2, 264, 200, 136), (3, 128, 1024, 64)]:
+            a = rand(rng, (batch, M, K), dtype, 1.0 / K ** 0.5)
+            b = rand(rng, (batch, K, N), dtype)
+            for transA in (False, True):
+                for transB in (False, True):
+                    sa = np.ascontiguousarray(a.transpose(0, 2, 1)) if transA else a
+                    sb = np.ascontiguousarray(b.transpose(0, 2, 1)) if transB else b
+                    print("matmul", pipeline, tile, dtype.name, batch, M, K, N, transA, transB, flush=True)
+                    fn = lambda: Tensor.batchedMatmul(Tensor(data=sa), transA, Tensor(data=sb), transB, False)
+                    got, want = check_close(hip_backend, oracle_backend, fn, TOL[dtype])
+                    scale = float(np.max(np.abs(want.astype(np.float64))))
+                    assert float(np.max(np.abs(got.astype(np.float64) - want.astype(np.float64)))) <= TOL[dtype] * scale
+
+
 def test_matmul_fp16_4096_against_oracle_slab_and_identity(hip_backend, oracle_backend):
     """Config 2 at full size: every layout; a 96-row slab of each product is checked against
     the oracle, and A x I == A exactly."""
