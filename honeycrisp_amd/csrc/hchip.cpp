@@ -2000,7 +2000,11 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
     }
     if (bm != 0 && dma) {
       const uint64_t blocks = ceil_div(M, bm) * ceil_div(N, bn) * (uint64_t)batch;
-      if (!which && (uint64_t)K * el >= 2048 && ((bm == 256 && bn == 256) || blocks >= 2 * cus)) dma2 = true;
+      // (whole cache lines only help an operand that is contiguous along K: TN products stay
+      // with the four-stage ring)
+      const bool k_contig = ma == 'k' || mb == 'k';
+      if (!which && k_contig && (uint64_t)K * el >= 2048 && ((bm == 256 && bn == 256) || blocks >= 2 * cus))
+        dma2 = true;
       if (dma2) slice = (uint32_t)(128 / el);
     }
     if (bm != 0) edge = !whole(bm, bn);
