@@ -27,6 +27,7 @@ KERNELS = [
     ("gemm_f16_fast", "gemm_f16_fast.hip", []),
     ("gemm_dma", "gemm_dma.hip", []),
     ("gemm_dma2", "gemm_dma2.hip", []),
+    ("gemm_mi16", "gemm_mi16.hip", []),
 ]
 DEVICE_FLAGS = [
     "--offload-arch=gfx950", "--genco", "-O3", "-std=c++17",

@@ -22,5 +22,6 @@
     EMBED hc_image_gemm_f16_fast, "gemm_f16_fast.hsaco"
     EMBED hc_image_gemm_dma, "gemm_dma.hsaco"
     EMBED hc_image_gemm_dma2, "gemm_dma2.hsaco"
+    EMBED hc_image_gemm_mi16, "gemm_mi16.hsaco"
 
     .section .note.GNU-stack,"",@progbits

@@ -31,6 +31,7 @@ extern const unsigned char hc_image_gemm[], hc_image_gemm_end[];
 extern const unsigned char hc_image_gemm_f16_fast[], hc_image_gemm_f16_fast_end[];
 extern const unsigned char hc_image_gemm_dma[], hc_image_gemm_dma_end[];
 extern const unsigned char hc_image_gemm_dma2[], hc_image_gemm_dma2_end[];
+extern const unsigned char hc_image_gemm_mi16[], hc_image_gemm_mi16_end[];
 }
 
 struct hc_module {
@@ -150,6 +151,7 @@ extern "C" int hc_init(int device, hc_ctx** out) {
   if (s == HC_OK) s = load_image(ctx, hc_image_gemm_f16_fast, hc_image_gemm_f16_fast_end, "gemm_f16_fast");
   if (s == HC_OK) s = load_image(ctx, hc_image_gemm_dma, hc_image_gemm_dma_end, "gemm_dma");
   if (s == HC_OK) s = load_image(ctx, hc_image_gemm_dma2, hc_image_gemm_dma2_end, "gemm_dma2");
+  if (s == HC_OK) s = load_image(ctx, hc_image_gemm_mi16, hc_image_gemm_mi16_end, "gemm_mi16");
   if (s == HC_OK) {
     hipError_t e = hipMalloc(&ctx->zeros, 256);
     if (e == hipSuccess) e = hipMemset(ctx->zeros, 0, 256);
@@ -1947,7 +1949,12 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
   // has one short job) and two stages of 128-byte K-slices (whole cache lines for K-contiguous
   // operands, half the barriers: best when the CUs are kept busy for long). Chosen below, after
   // the tile; HCHIP_GEMM_KERNEL=dma|dma2 forces one.
-  bool dma2 = dma && which && strcmp(which, "dma2") == 0;
+  // A third variant, fp16 only: the 128-byte-slice pipeline on the 16x16x32 MFMA shape, which
+  // needs less power per multiply-accumulate. It pays where the matrix cores run into the
+  // board's power limit: every CU busy with a 256 x 256 tile over a long K.
+  // HCHIP_GEMM_KERNEL=dma|dma2|mi16 forces one of the three.
+  bool mi16 = dma && dtype == HC_F16 && which && strcmp(which, "mi16") == 0;
+  bool dma2 = dma && which && (strcmp(which, "dma2") == 0 || mi16);
   uint32_t slice = (uint32_t)(64 / el);
   const bool eligible = ma != 'x' && mb != 'x' && K > 0 && aligned16(k.c) &&
                         (dma ? (k.c_rs % P == 0 && (batch <= 1 || k.c_bs % P == 0)) : (dtype == HC_F16 && K % 64 == 0));
@@ -2005,6 +2012,7 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
       const bool k_contig = ma == 'k' || mb == 'k';
       if (!which && k_contig && (uint64_t)K * el >= 2048 && ((bm == 256 && bn == 256) || blocks >= 2 * cus))
         dma2 = true;
+      if (!which && dtype == HC_F16 && K >= 1024 && bm == 256 && bn == 256 && blocks >= cus) dma2 = mi16 = true;
       if (dma2) slice = (uint32_t)(128 / el);
     }
     if (bm != 0) edge = !whole(bm, bn);
@@ -2024,7 +2032,7 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
           break;
         }
     }
-    snprintf(name, sizeof(name), "hc_gemm_%s_%s_%ux%u_%c%c%s", dtype_name(dtype), dma ? (dma2 ? "dma2" : "dma") : "fast", bm, bn,
+    snprintf(name, sizeof(name), "hc_gemm_%s_%s_%ux%u_%c%c%s", dtype_name(dtype), dma ? (mi16 ? "mi16" : dma2 ? "dma2" : "dma") : "fast", bm, bn,
              ma == 'k' ? 'k' : 'm', mb == 'k' ? 'k' : 'n', edge ? "_e" : "");
   } else if (ma == 'x' || mb == 'x')
     snprintf(name, sizeof(name), "hc_gemm_%s_xx", dtype_name(dtype));

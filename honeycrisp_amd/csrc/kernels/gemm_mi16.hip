@@ -1,0 +1,448 @@
+// fp16 GEMM for gfx950 on v_mfma_f32_16x16x32_f16, the power-efficient shape of the fp16 matrix
+// instruction: per multiply-accumulate it moves half as many accumulator registers as the
+// 32x32x16 shape, and on random operands a loop of nothing but these instructions sustains
+// about 1.9 PFLOP/s against 1.7 for 32x32x16 (the board lowers its clock to stay within its
+// power limit). Global->LDS traffic, LDS layouts and swizzles are those of the two-stage
+// pipeline with 128-byte K-slices (gemm_dma2.hip: whole cache lines for K-contiguous operands,
+// global_load_lds_dwordx4, ds_read_b64_tr_b16 for M/N-contiguous operands); what differs is
+// how a wave reads its operands and lays out its accumulators:
+//   wave tile (BM/2) x (BN/2) = MT x NT tiles of 16 x 16, one MFMA per tile and 32 k;
+//   operand of a tile: lane l holds row l%16, k = 8*(l/16) .. +7 (one 16-byte chunk);
+//   accumulator of a tile (operands swapped, so it is C^T): lane l holds m = l%16 and the four
+//   consecutive columns n = 4*(l/16) .. +3.
+// A K-step (one stage, 64 halfs) is two sub-steps of MT*NT MFMAs, with the barrier between them:
+//   sub-step 0: MFMAs on k 0..31; read the operands of k 32..63; the rest of the DMA of K-step j+1
+//   wait for this wave's DMA, barrier
+//   sub-step 1: MFMAs on k 32..63; read the first operands of K-step j+1; DMA of K-step j+2 into
+//     this stage, spread over the MFMAs.
+#include <type_traits>
+
+#include "common.hip.h"
+
+// length of the DMA window in quarter sub-steps (see the K loop)
+#ifndef HC_MI16_WINDOW_X4
+#define HC_MI16_WINDOW_X4 5
+#endif
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+typedef uint32_t Chunk __attribute__((ext_vector_type(4)));  // 16 bytes = 8 halfs
+
+enum { DMA_K = 0, DMA_MN = 1 };
+
+#define LDS_AS __attribute__((address_space(3)))
+#define GLOBAL_AS __attribute__((address_space(1)))
+
+__device__ __forceinline__ uint32_t swz_k(uint32_t row) { return row & 7u; }
+__device__ __forceinline__ uint32_t swz_mn(uint32_t k) { return (((k & 7u) ^ (((k >> 3) & 1u) << 2)) << 1); }
+
+// Workgroup barrier for LDS traffic only: this wave's LDS reads have returned (lgkmcnt), its
+// DMA is waited for separately (wait_dma), and nothing is said about global memory. A fence
+// builtin would do the same but also waits for every DMA instruction in flight, including
+// those that fill stages nobody is about to read. The "memory" clobber keeps the compiler
+// from moving LDS accesses across it.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+// s_waitcnt vmcnt(N) with the other counters untouched (gfx9 encoding: vmcnt in bits 3:0 and
+// 15:14, expcnt 6:4, lgkmcnt 11:8): at most N of this wave's DMA instructions still in flight.
+template <int N> __device__ __forceinline__ void wait_dma() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
+}
+
+// One operand of the block tile: where its DMA lanes fetch from and where a wave's MFMA
+// operand reads land.
+template <typename T, int ROWS, int MODE> struct DmaOperand {
+  static constexpr int ES = sizeof(T);
+  static constexpr bool F32 = ES == 4;
+  static constexpr int NI = ROWS / 32;                        // DMA instructions per wave and K-step
+  static constexpr int TILES = ROWS / 64;                     // MFMA tiles per wave along this operand
+  // LDS reads per sub-step
+  static constexpr int READS = MODE == DMA_K ? TILES : (F32 ? 4 * TILES : 2 * TILES);
+  static constexpr int NADDR = MODE == DMA_K ? TILES * 4 : TILES * 2;
+  static constexpr int ROWB = ROWS * ES;                      // bytes per k-row (DMA_MN layout)
+  static constexpr int BYTES = ROWS * 128;                    // per stage
+
+  uint32_t goff[NI];     // byte offset of this lane's 16-byte piece for DMA instruction i (k = 0)
+  uint32_t kstride;      // bytes per unit of k
+  uint32_t raddr[NADDR]; // byte offsets (inside the operand's LDS region) of the MFMA operand reads
+
+  // `limit` (edge kernels): extent of this operand along M / N. Rows or 16-byte pieces past it
+  // are fetched from the last valid row / piece instead: they only feed outputs that are
+  // never stored. 0 = no clamping.
+  __device__ __forceinline__ void init(uint32_t rs, uint32_t cs, uint32_t r0, uint32_t woff, uint32_t limit) {
+    const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    if (MODE == DMA_K) {
+      kstride = ES;
+#pragma unroll
+      for (int i = 0; i < NI; i++) {
+        const uint32_t row = (wave * NI + i) * 8 + lane / 8;
+        const uint32_t c = (lane % 8) ^ swz_k(row);
+        uint32_t grow = r0 + row;
+        if (limit && grow >= limit) grow = limit - 1;
+        goff[i] = grow * rs * ES + c * 16;
+      }
+      const uint32_t lrow = lane & 31, lgrp = lane >> 5;
+#pragma unroll
+      for (int q = 0; q < TILES; q++) {
+        const uint32_t r = woff + q * 32 + lrow;
+#pragma unroll
+        for (int s = 0; s < 4; s++) raddr[q * 4 + s] = r * 128 + (((2 * s + lgrp) ^ swz_k(r)) * 16);
+      }
+    } else if (F32) {
+      // [32 k][ROWS floats]; the 128-byte halves of every 256 bytes swap places in k-rows
+      // with bit 2 set: an MFMA operand read touches rows k and k + 4, 32 floats of each
+      constexpr uint32_t KPI = 1024 / ROWB;   // k-rows per DMA instruction
+      constexpr uint32_t PIECES = ROWB / 16;  // 16-byte pieces per k-row
+      kstride = cs * ES;
+#pragma unroll
+      for (int i = 0; i < NI; i++) {
+        const uint32_t krow = (wave * NI + i) * KPI + lane / PIECES;
+        const uint32_t piece = (lane % PIECES) ^ (((krow >> 2) & 1u) << 3);
+        uint32_t col = r0 + piece * 4;
+        if (limit && col + 4 > limit) col = limit - 4;
+        goff[i] = (krow * cs + col) * ES;
+      }
+      const uint32_t lrow = lane & 31, lgrp = lane >> 5;
+#pragma unroll
+      for (int q = 0; q < TILES; q++) {
+        const uint32_t n = woff + q * 32 + lrow;  // k = 4 * lgrp + e + 8 * s, e and s as immediates
+        raddr[q] = 4 * lgrp * ROWB + ((n ^ (lgrp << 5)) * 4);
+      }
+    } else {
+      constexpr int KPI = 512 / ROWS;       // k-rows per DMA instruction
+      constexpr uint32_t SLOTS_PER_ROW = ROWS / 8;
+      kstride = cs * 2;
+#pragma unroll
+      for (int i = 0; i < NI; i++) {
+        const uint32_t krow = (wave * NI + i) * KPI + lane / SLOTS_PER_ROW;
+        const uint32_t slot = (lane % SLOTS_PER_ROW) ^ (swz_mn(krow) & (SLOTS_PER_ROW - 1));
+        uint32_t col = r0 + slot * 8;
+        if (limit && col + 8 > limit) col = limit - 8;
+        goff[i] = (krow * cs + col) * 2;
+      }
+      const uint32_t j = lane >> 4, r16 = lane & 15;
+#pragma unroll
+      for (int q = 0; q < TILES; q++) {
+        const uint32_t m = woff + q * 32 + 16 * (j & 1) + 4 * (r16 & 3);
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+          const uint32_t k = 8 * (j >> 1) + 4 * h + (r16 >> 2);  // + 16 * s as an immediate offset
+          raddr[q * 2 + h] = k * ROWB + (((m >> 3) ^ (swz_mn(k) & (ROWS / 8 - 1))) * 16) + (m & 7) * 2;
+        }
+      }
+    }
+  }
+
+  // k offset, inside a K-slice, of the piece this lane fetches with DMA instruction i
+  __device__ __forceinline__ uint32_t klocal(int i) const {
+    const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    if (MODE == DMA_K) {
+      const uint32_t row = (wave * NI + i) * 8 + lane / 8;
+      return ((lane % 8) ^ swz_k(row)) * (16 / ES);
+    }
+    constexpr uint32_t PER_ROW = ROWB / 16, KPI = 1024 / ROWB;
+    return (wave * NI + i) * KPI + lane / PER_ROW;
+  }
+
+  // DMA instruction i of this wave for the K-slice starting at k0: 1 KiB into `region`.
+  // Edge kernels (kend != 0): pieces at k >= kend come from `zeros` (16 zero bytes) instead,
+  // so the ragged last slice contributes nothing.
+  __device__ __forceinline__ void dma(int i, const T* base, uint32_t k0, char* region, uint32_t kend = 0,
+                                      const void* zeros = nullptr) const {
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    // The empty asm keeps the zero-extension of the lane offset next to the load, so that the
+    // load takes the form "scalar base + 32-bit lane offset" with no vector add in front of it.
+    uint32_t off = goff[i];
+    asm volatile("" : "+v"(off));
+    const char* src = (const char*)base + (size_t)k0 * kstride + off;
+    if (kend != 0 && k0 + 128 / ES > kend) {  // wave-uniform
+      if (k0 + klocal(i) >= kend) src = (const char*)zeros;
+    }
+    __builtin_amdgcn_global_load_lds((const GLOBAL_AS void*)src, (LDS_AS void*)(region + (wave * NI + i) * 1024), 16, 0, 0);
+  }
+
+  // Read number u of sub-step s into the operand registers of tile u (DMA_K), half u%2 of
+  // tile u/2 (DMA_MN, fp16) or element u%4 of tile u/4 (DMA_MN, fp32).
+  __device__ __forceinline__ void read(int u, int s, const char* region, Chunk* frag) const {
+    if (MODE == DMA_K) {
+      frag[u] = *reinterpret_cast<const Chunk*>(region + raddr[u * 4 + s]);
+    } else if (F32) {
+      const int q = u / 4, e = u % 4;
+      frag[q][e] = *reinterpret_cast<const uint32_t*>(region + raddr[q] + (8 * s + e) * ROWB);
+    } else {
+      const int q = u / 2, h = u % 2;
+      typedef short short4v __attribute__((ext_vector_type(4)));
+      const short4v v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (LDS_AS short4v*)(region + raddr[q * 2 + h] + s * 16 * ROWB));
+      typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+      const u32x2 w = __builtin_bit_cast(u32x2, v);
+      frag[q][2 * h] = w[0];
+      frag[q][2 * h + 1] = w[1];
+    }
+  }
+};
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>)
+template <int N, typename F> __device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (N > 0) {
+    static_for<N - 1>(f);
+    f(std::integral_constant<int, N - 1>{});
+  }
+}
+
+// Where a wave's operand reads land, for the 16 x 16 x 32 instruction. The DMA side (which
+// global piece goes to which LDS slot) is DmaOperand's.
+template <int ROWS, int MODE> struct Mi16Reads {
+  static constexpr int TILES = ROWS / 32;  // 16-row tiles per wave along this operand
+  static constexpr int READS = MODE == DMA_K ? TILES : 2 * TILES;  // LDS reads per sub-step
+  static constexpr int ROWB = ROWS * 2;
+  uint32_t raddr[TILES * 2];
+
+  __device__ __forceinline__ void init(uint32_t woff) {
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t r16 = lane & 15, grp = lane >> 4;
+    if (MODE == DMA_K) {
+      // rows of 128 bytes, chunk c of row r in slot c ^ (r & 7); sub-step s reads chunk 4 s + grp
+#pragma unroll
+      for (int q = 0; q < TILES; q++) {
+        const uint32_t r = woff + q * 16 + r16;
+#pragma unroll
+        for (int s = 0; s < 2; s++) raddr[q * 2 + s] = r * 128 + (((4 * s + grp) ^ swz_k(r)) * 16);
+      }
+    } else {
+      // [k][m] layout; a transposing read hands lane i of a 16-lane group column i of four
+      // k-rows: the group points at k-rows 8 grp + 4 h + (0..3), lane r16 at k-row + r16 / 4,
+      // columns 4 (r16 % 4) .. +3. Sub-step s adds 32 k-rows as an immediate offset.
+#pragma unroll
+      for (int q = 0; q < TILES; q++) {
+        const uint32_t m = woff + q * 16 + 4 * (r16 & 3);
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+          const uint32_t k = 8 * grp + 4 * h + (r16 >> 2);
+          raddr[q * 2 + h] = k * ROWB + (((m >> 3) ^ (swz_mn(k) & (ROWS / 8 - 1))) * 16) + (m & 7) * 2;
+        }
+      }
+    }
+  }
+  // read number u of sub-step s
+  __device__ __forceinline__ void read(int u, int s, const char* region, Chunk* frag) const {
+    if (MODE == DMA_K) {
+      frag[u] = *reinterpret_cast<const Chunk*>(region + raddr[u * 2 + s]);
+    } else {
+      const int q = u / 2, h = u % 2;
+      typedef short short4v __attribute__((ext_vector_type(4)));
+      const short4v v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (LDS_AS short4v*)(region + raddr[q * 2 + h] + s * 32 * ROWB));
+      typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+      const u32x2 w = __builtin_bit_cast(u32x2, v);
+      frag[q][2 * h] = w[0];
+      frag[q][2 * h + 1] = w[1];
+    }
+  }
+};
+
+template <int BM, int BN, int MODE_A, int MODE_B, bool EDGE>
+__device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds0, char* lds1) {
+  typedef half_t T;
+  constexpr int MT = BM / 32, NT = BN / 32;  // 16 x 16 tiles per wave
+  constexpr int SLOTS = MT * NT;             // MFMAs per sub-step
+  typedef DmaOperand<T, BM, MODE_A> OpA;
+  typedef DmaOperand<T, BN, MODE_B> OpB;
+  typedef Mi16Reads<BM, MODE_A> RdA;
+  typedef Mi16Reads<BN, MODE_B> RdB;
+  constexpr uint32_t BK = 64;  // halfs per stage
+  constexpr int READS = RdA::READS + RdB::READS;
+  constexpr int NDMA = OpA::NI + OpB::NI;  // per wave and K-step
+  constexpr int A_BYTES = OpA::BYTES;
+
+  // XCD-aware tile order. Block ids equal mod 8 run on one XCD and share its L2: give each
+  // XCD a compact rectangle of tiles (few distinct A and B panels), or a contiguous band.
+  const uint32_t total = p.tiles_m * p.tiles_n;
+  uint32_t tile = blockIdx.x;
+  if (p.xcd_gn != 0) {
+    const uint32_t per = 8 * p.xcd_sm * p.xcd_sn, gm = 8 / p.xcd_gn;
+    const uint32_t group = blockIdx.x / per, w = blockIdx.x - group * per;
+    const uint32_t x = w & 7u, t = w >> 3;
+    const uint32_t sbn = p.tiles_n / (p.xcd_gn * p.xcd_sn);
+    const uint32_t sb_row = group / sbn, sb_col = group - sb_row * sbn;
+    const uint32_t xm = x / p.xcd_gn, xn = x - xm * p.xcd_gn;
+    const uint32_t lm = t / p.xcd_sn, ln = t - lm * p.xcd_sn;
+    tile = (sb_row * gm * p.xcd_sm + xm * p.xcd_sm + lm) * p.tiles_n + sb_col * p.xcd_gn * p.xcd_sn + xn * p.xcd_sn + ln;
+  } else if ((total & 7u) == 0) {
+    tile = (blockIdx.x & 7u) * (total >> 3) + (blockIdx.x >> 3);
+  }
+  const uint32_t tm = tile / p.tiles_n, tn = tile - tm * p.tiles_n;
+  const uint32_t m0 = tm * BM, n0 = tn * BN;
+  const uint32_t batch = blockIdx.y;
+  const T* A = (const T*)p.a + batch * p.a_bs;
+  const T* B = (const T*)p.b + batch * p.b_bs;
+  T* C = (T*)p.c + batch * p.c_bs;
+
+  const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const uint32_t wm = (wave >> 1) * (BM / 2), wn = (wave & 1) * (BN / 2);
+
+  floatx4 acc[MT][NT];
+#pragma unroll
+  for (int i = 0; i < MT; i++)
+#pragma unroll
+    for (int j = 0; j < NT; j++)
+#pragma unroll
+      for (int v = 0; v < 4; v++) acc[i][j][v] = 0.0f;
+
+  OpA oa;
+  OpB ob;
+  oa.init(p.a_rs, p.a_cs, m0, wm, EDGE ? p.a_lim : 0);
+  ob.init(p.b_cs, p.b_rs, n0, wn, EDGE ? p.b_lim : 0);
+  RdA ra;
+  RdB rb;
+  ra.init(wm);
+  rb.init(wn);
+  const uint32_t kend = EDGE ? p.K : 0;
+
+  struct Frags {
+    Chunk a[MT];
+    Chunk b[NT];
+  };
+  // unit u of the operand reads of a sub-step: B's reads first, then A's
+  auto read_unit = [&](Frags& f, const char* stage, int s, int u) {
+    if (u < RdB::READS) rb.read(u, s, stage + A_BYTES, f.b);
+    else if (u < READS) ra.read(u - RdB::READS, s, stage, f.a);
+  };
+  auto dma_unit = [&](int u, uint32_t k0, char* stage) {
+    if (u < OpA::NI) oa.dma(u, A, k0, stage, kend, p.zeros);
+    else if (u < NDMA) ob.dma(u - OpA::NI, B, k0, stage + A_BYTES, kend, p.zeros);
+  };
+  // MFMA t of a sub-step; operands swapped (B first) so that a lane holds four consecutive n
+  auto mma_one = [&](const Frags& f, int t) {
+    const int j = t / MT, i = t % MT;
+    // Written as assembly to pin the accumulators to the accumulation registers: left to itself
+    // the register allocator keeps part of them in ordinary registers and copies them back and
+    // forth around every instruction. An accumulator is touched again 63 MFMAs later at the
+    // earliest and read by the epilogue only after a barrier, so no wait states are missing.
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(f.b[j]), "v"(f.a[i]));
+  };
+  // The DMA of a K-slice is spread evenly over a window of W MFMA slots that starts right after
+  // the barrier that frees its stage (sub-step 1, then sub-step 0 of the next step): unit u
+  // goes out in window slot u * W / NDMA; the rest of sub-step 0 is the time the last loads
+  // get to land (needed: about 600 cycles = 40 MFMAs of this shape).
+  constexpr int W = SLOTS * HC_MI16_WINDOW_X4 / 4 > 0 ? SLOTS * HC_MI16_WINDOW_X4 / 4 : 1;
+  static_assert(W <= 2 * SLOTS, "the DMA window ends with sub-step 0");
+  constexpr int U0 = (SLOTS * NDMA + W - 1) / W < NDMA ? (SLOTS * NDMA + W - 1) / W : NDMA;  // units of sub-step 1
+
+  const uint32_t nk = (p.K + BK - 1) / BK;
+  auto kclamp = [&](uint32_t j) { return (j < nk ? j : nk - 1) * BK; };  // steps past the end repeat the last one
+  Frags f0, f1;
+
+  // (compile-time loop indices throughout: every register array is indexed statically)
+  auto substep = [&](const Frags& use, Frags& fill, const char* from, auto s_next_c, auto part_c, char* to,
+                     uint32_t k0) {
+    constexpr int s_next = decltype(s_next_c)::value, part = decltype(part_c)::value;
+    static_for<SLOTS>([&](auto tc) {
+      constexpr int t = decltype(tc)::value;
+      // units u with u * W / NDMA == this window slot
+      constexpr int w = part * SLOTS + t;
+      constexpr int lo = (w * NDMA + W - 1) / W < NDMA ? (w * NDMA + W - 1) / W : NDMA;
+      constexpr int hi = ((w + 1) * NDMA + W - 1) / W < NDMA ? ((w + 1) * NDMA + W - 1) / W : NDMA;
+      static_for<hi - lo>([&](auto uc) { dma_unit(lo + decltype(uc)::value, k0, to); });
+      if constexpr (t < READS) read_unit(fill, from, s_next, t);
+      mma_one(use, t);
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    static_for<(READS > SLOTS ? READS - SLOTS : 0)>(  // (tiles with more reads than MFMAs)
+        [&](auto uc) { read_unit(fill, from, s_next, SLOTS + decltype(uc)::value); });
+  };
+
+  // K-step j out of `cur`; `nxt` receives the rest of K-step j+1, then `cur` K-step j+2
+  auto step = [&](char* cur, char* nxt, uint32_t j) {
+    __builtin_amdgcn_sched_barrier(0);
+    substep(f0, f1, cur, std::integral_constant<int, 1>{}, std::integral_constant<int, 1>{}, nxt, kclamp(j + 1));
+    wait_dma<0>();  // K-step j+1 of this wave has landed ...
+    lds_barrier();  // ... and everybody's; nobody reads cur any more
+    __builtin_amdgcn_sched_barrier(0);
+    substep(f1, f0, nxt, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, cur, kclamp(j + 2));
+  };
+
+  // prologue: K-step 0 and the first window part of K-step 1
+  static_for<NDMA>([&](auto uc) { dma_unit(decltype(uc)::value, 0, lds0); });
+  static_for<U0>([&](auto uc) { dma_unit(decltype(uc)::value, kclamp(1), lds1); });
+  wait_dma<U0>();
+  lds_barrier();
+  static_for<READS>([&](auto uc) { read_unit(f0, lds0, 0, decltype(uc)::value); });
+
+  uint32_t j = 0;
+  for (; j + 1 < nk; j += 2) {
+    step(lds0, lds1, j);
+    step(lds1, lds0, j + 1);
+  }
+  if (j < nk) step(lds0, lds1, j);
+  wait_dma<0>();  // no LDS write of this workgroup may be in flight when it ends
+
+  // Epilogue. Lane l of tile (i, j) holds m = l % 16 and the four consecutive columns
+  // n = 4 * (l / 16) .. +3 (8 bytes of halfs). The wave's part of C goes through LDS in slabs
+  // of 32 rows = two rows of tiles (both stages are free now; wave w uses half of a stage) and
+  // leaves as 16-byte pieces, whole rows of the slab contiguous. 16-byte unit u of row r sits
+  // at unit u ^ s(r) to spread the writes over the banks. A wave's LDS instructions execute in
+  // order, so a slab may be overwritten right after its reads.
+  lds_barrier();
+  char* mine = (wave < 2 ? lds0 : lds1) + (wave & 1) * ((BM + BN) * 64);
+  constexpr uint32_t WN = BN / 2, RB = WN * 2, UNITS = RB / 16, RPI = 64 / UNITS;
+  constexpr uint32_t SLAB = 32 * RB, NSLAB = (BM + BN) * 64 / SLAB;
+  static_assert(NSLAB >= 1 && UNITS <= 64 && MT % 2 == 0, "a slab is two rows of tiles and must fit half a stage");
+  auto unit_swz = [&](uint32_t r) { return (RB >= 256 ? r : r * RB / 256) & (UNITS - 1); };
+  const uint32_t r16 = lane & 15, grp = lane >> 4;
+#pragma unroll
+  for (int ii = 0; ii < MT / 2; ii++) {
+    char* slab = mine + (ii % NSLAB) * SLAB;
+#pragma unroll
+    for (int half = 0; half < 2; half++) {
+      const uint32_t row = half * 16 + r16;
+#pragma unroll
+      for (int jj = 0; jj < NT; jj++) {
+        half4v h;
+#pragma unroll
+        for (int e = 0; e < 4; e++) h[e] = narrow<half_t>(acc[2 * ii + half][jj][e]);
+        // columns jj * 16 + 4 grp .. +3: unit 2 jj + grp / 2, second half of the unit if grp is odd
+        *reinterpret_cast<half4v*>(slab + row * RB + (((2 * jj + (grp >> 1)) ^ unit_swz(row)) * 16) + (grp & 1) * 8) = h;
+      }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // wave-private region: no barrier needed
+#pragma unroll
+    for (uint32_t it = 0; it < 32 / RPI; it++) {
+      const uint32_t r = it * RPI + lane / UNITS, u = lane % UNITS;
+      const Chunk v = *reinterpret_cast<const Chunk*>(slab + r * RB + ((u ^ unit_swz(r)) * 16));
+      const uint32_t row = m0 + wm + ii * 32 + r, col = n0 + wn + u * 8;
+      if (!EDGE || (row < p.M && col < p.N)) *reinterpret_cast<Chunk*>(C + (size_t)row * p.c_rs + col) = v;
+    }
+    asm volatile("" ::: "memory");
+  }
+}
+
+#define DEF_MI16(BM, BN, AN, AM, BNAME, BMODE)                                                        \
+  extern "C" __global__ __launch_bounds__(256) void hc_gemm_f16_mi16_##BM##x##BN##_##AN##BNAME(       \
+      hck_gemm_args p) {                                                                              \
+    __shared__ __attribute__((aligned(1024))) char lds0[(BM + BN) * 128];                             \
+    __shared__ __attribute__((aligned(1024))) char lds1[(BM + BN) * 128];                             \
+    gemm_mi16_impl<BM, BN, AM, BMODE, false>(p, lds0, lds1);                                          \
+  }                                                                                                   \
+  extern "C" __global__ __launch_bounds__(256) void hc_gemm_f16_mi16_##BM##x##BN##_##AN##BNAME##_e(   \
+      hck_gemm_args p) {                                                                              \
+    __shared__ __attribute__((aligned(1024))) char lds0[(BM + BN) * 128];                             \
+    __shared__ __attribute__((aligned(1024))) char lds1[(BM + BN) * 128];                             \
+    gemm_mi16_impl<BM, BN, AM, BMODE, true>(p, lds0, lds1);                                           \
+  }
+#define DEF_MI16_TILE(BM, BN)                                                                         \
+  DEF_MI16(BM, BN, k, DMA_K, k, DMA_K)                                                                \
+  DEF_MI16(BM, BN, k, DMA_K, n, DMA_MN)                                                               \
+  DEF_MI16(BM, BN, m, DMA_MN, k, DMA_K)                                                               \
+  DEF_MI16(BM, BN, m, DMA_MN, n, DMA_MN)
+DEF_MI16_TILE(256, 256)
+DEF_MI16_TILE(256, 128)
+DEF_MI16_TILE(128, 128)
+DEF_MI16_TILE(256, 64)
+DEF_MI16_TILE(128, 64)
+DEF_MI16_TILE(64, 64)

@@ -117,7 +117,7 @@ def test_batched_matmul_all_flags_small(hip_backend, oracle_backend):
                     check_close(hip_backend, oracle_backend, fn, TOL[dtype])
 
 
-@pytest.mark.parametrize("pipeline", ["dma", "dma2"])
+@pytest.mark.parametrize("pipeline", ["dma", "dma2", "mi16"])
 @pytest.mark.parametrize("dtype", [F32, F16], ids=["f32", "f16"])
 def test_matmul_both_pipelines_every_tile(hip_backend, oracle_backend, monkeypatch, pipeline, dtype):
     """The host picks a direct-to-LDS pipeline and a tile by problem size; here every tile of both
