@@ -1313,10 +1313,12 @@ extern "C" int hc_argsort(hc_ctx* ctx, int dtype, const void* in, void* out, int
   return launch(ctx, name, (uint64_t)outer * (uint64_t)inner, 1, &k, sizeof(k));
 }
 
-extern "C" int hc_probe_mfma(hc_ctx* ctx, const void* data, uint64_t bytes, uint32_t iters, double* flops) {
+extern "C" int hc_probe_mfma(hc_ctx* ctx, int shape, const void* data, uint64_t bytes, uint32_t iters,
+                             double* flops) {
   REQUIRE(ctx, "hc_probe_mfma: null context");
+  REQUIRE(shape == 0 || shape == 1, "hc_probe_mfma: shape is 0 (32x32x16) or 1 (16x16x32)");
   REQUIRE(data && bytes >= 16 && aligned16(data), "hc_probe_mfma: needs at least 16 bytes, 16-byte aligned");
-  REQUIRE(iters > 0, "hc_probe_mfma: no iterations");
+  REQUIRE(iters >= 2 && iters % 2 == 0, "hc_probe_mfma: iters must be even and positive");
   // one workgroup of four waves per compute unit, one wave per SIMD: the occupancy of the large GEMM tile
   const uint64_t blocks = (uint64_t)ctx->props.multiProcessorCount;
   Scratch scratch(ctx);
@@ -1328,8 +1330,10 @@ extern "C" int hc_probe_mfma(hc_ctx* ctx, const void* data, uint64_t bytes, uint
   k.out = out;
   k.iters = iters;
   k.chunks = (uint32_t)std::min<uint64_t>(bytes / 16, 0xffffffffull);
+  // per iteration and wave: 16 MFMAs of 32 x 32 x 16 (or 32 of 16 x 16 x 32)
   if (flops) *flops = 2.0 * 32 * 32 * 16 * 16.0 * (double)iters * (double)(blocks * HCK_BLOCK / 64);
-  return launch(ctx, "hc_probe_mfma_f16", blocks, 1, &k, sizeof(k));
+  return launch(ctx, shape == 0 ? "hc_probe_mfma_f16_32x32x16" : "hc_probe_mfma_f16_16x16x32", blocks, 1, &k,
+                sizeof(k));
 }
 
 extern "C" int hc_log_softmax(hc_ctx* ctx, int dtype, const void* in, void* out, int64_t outer,
