@@ -23,6 +23,10 @@
 #ifndef HC_MI16_WINDOW_X4
 #define HC_MI16_WINDOW_X4 5
 #endif
+// 1: the operand reads of a sub-step are spread over its MFMAs, 0: issued under the first ones
+#ifndef HC_MI16_READ_SPREAD
+#define HC_MI16_READ_SPREAD 0
+#endif
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half4v __attribute__((ext_vector_type(4)));
@@ -334,9 +338,16 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
   static_assert(W <= 2 * SLOTS, "the DMA window ends with sub-step 0");
   constexpr int U0 = (SLOTS * NDMA + W - 1) / W < NDMA ? (SLOTS * NDMA + W - 1) / W : NDMA;  // units of sub-step 1
 
+  constexpr int RSTRIDE = HC_MI16_READ_SPREAD && SLOTS / READS > 1 ? SLOTS / READS : 1;
+
   const uint32_t nk = (p.K + BK - 1) / BK;
   auto kclamp = [&](uint32_t j) { return (j < nk ? j : nk - 1) * BK; };  // steps past the end repeat the last one
   Frags f0, f1;
+#ifdef HC_PROBE_WAITS
+  // measurement build: cycles this wave spends in the two waits of a K-step; they replace the
+  // first bytes of the block's C tile (32 bytes per wave: loop cycles, 100 MHz ticks, waits)
+  uint64_t probe_wait_dma = 0, probe_wait_bar = 0;
+#endif
 
   // (compile-time loop indices throughout: every register array is indexed statically)
   auto substep = [&](const Frags& use, Frags& fill, const char* from, auto s_next_c, auto part_c, char* to,
@@ -349,20 +360,31 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
       constexpr int lo = (w * NDMA + W - 1) / W < NDMA ? (w * NDMA + W - 1) / W : NDMA;
       constexpr int hi = ((w + 1) * NDMA + W - 1) / W < NDMA ? ((w + 1) * NDMA + W - 1) / W : NDMA;
       static_for<hi - lo>([&](auto uc) { dma_unit(lo + decltype(uc)::value, k0, to); });
-      if constexpr (t < READS) read_unit(fill, from, s_next, t);
+      // operand reads of the following sub-step: one every RSTRIDE slots
+      if constexpr (t % RSTRIDE == 0 && t / RSTRIDE < READS) read_unit(fill, from, s_next, t / RSTRIDE);
       mma_one(use, t);
       __builtin_amdgcn_sched_barrier(0);
     });
-    static_for<(READS > SLOTS ? READS - SLOTS : 0)>(  // (tiles with more reads than MFMAs)
-        [&](auto uc) { read_unit(fill, from, s_next, SLOTS + decltype(uc)::value); });
+    static_for<(READS > SLOTS / RSTRIDE ? READS - SLOTS / RSTRIDE : 0)>(  // (tiles with more reads than slots)
+        [&](auto uc) { read_unit(fill, from, s_next, SLOTS / RSTRIDE + decltype(uc)::value); });
   };
 
   // K-step j out of `cur`; `nxt` receives the rest of K-step j+1, then `cur` K-step j+2
   auto step = [&](char* cur, char* nxt, uint32_t j) {
     __builtin_amdgcn_sched_barrier(0);
     substep(f0, f1, cur, std::integral_constant<int, 1>{}, std::integral_constant<int, 1>{}, nxt, kclamp(j + 1));
+#ifdef HC_PROBE_WAITS
+    const uint64_t w0 = __builtin_readcyclecounter();
+    wait_dma<0>();
+    const uint64_t w1 = __builtin_readcyclecounter();
+    lds_barrier();
+    const uint64_t w2 = __builtin_readcyclecounter();
+    probe_wait_dma += w1 - w0;
+    probe_wait_bar += w2 - w1;
+#else
     wait_dma<0>();  // K-step j+1 of this wave has landed ...
     lds_barrier();  // ... and everybody's; nobody reads cur any more
+#endif
     __builtin_amdgcn_sched_barrier(0);
     substep(f1, f0, nxt, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, cur, kclamp(j + 2));
   };
@@ -374,6 +396,9 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
   lds_barrier();
   static_for<READS>([&](auto uc) { read_unit(f0, lds0, 0, decltype(uc)::value); });
 
+#ifdef HC_PROBE_WAITS
+  const uint64_t probe_c0 = __builtin_readcyclecounter(), probe_r0 = __builtin_amdgcn_s_memrealtime();
+#endif
   uint32_t j = 0;
   for (; j + 1 < nk; j += 2) {
     step(lds0, lds1, j);
@@ -381,6 +406,9 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
   }
   if (j < nk) step(lds0, lds1, j);
   wait_dma<0>();  // no LDS write of this workgroup may be in flight when it ends
+#ifdef HC_PROBE_WAITS
+  const uint64_t probe_c1 = __builtin_readcyclecounter(), probe_r1 = __builtin_amdgcn_s_memrealtime();
+#endif
 
   // Epilogue. Lane l of tile (i, j) holds m = l % 16 and the four consecutive columns
   // n = 4 * (l / 16) .. +3 (8 bytes of halfs). The wave's part of C goes through LDS in slabs
@@ -420,6 +448,16 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
     }
     asm volatile("" ::: "memory");
   }
+#ifdef HC_PROBE_WAITS
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) {
+    uint64_t* dst = reinterpret_cast<uint64_t*>(C + (size_t)m0 * p.c_rs + n0) + (threadIdx.x >> 6) * 4;
+    dst[0] = probe_c1 - probe_c0;
+    dst[1] = probe_r1 - probe_r0;
+    dst[2] = probe_wait_dma;
+    dst[3] = probe_wait_bar | ((__builtin_amdgcn_s_memrealtime() - probe_r1) << 32);  // + epilogue ticks
+  }
+#endif
 }
 
 #define DEF_MI16(BM, BN, AN, AM, BNAME, BMODE)                                                        \
