@@ -359,9 +359,13 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
       constexpr int w = part * SLOTS + t;
       constexpr int lo = (w * NDMA + W - 1) / W < NDMA ? (w * NDMA + W - 1) / W : NDMA;
       constexpr int hi = ((w + 1) * NDMA + W - 1) / W < NDMA ? ((w + 1) * NDMA + W - 1) / W : NDMA;
+#ifndef HC_MI16_NO_LOOP_DMA  // (measurement switch: wrong results)
       static_for<hi - lo>([&](auto uc) { dma_unit(lo + decltype(uc)::value, k0, to); });
+#endif
       // operand reads of the following sub-step: one every RSTRIDE slots
+#ifndef HC_MI16_NO_LOOP_READS  // (measurement switch: wrong results)
       if constexpr (t % RSTRIDE == 0 && t / RSTRIDE < READS) read_unit(fill, from, s_next, t / RSTRIDE);
+#endif
       mma_one(use, t);
       __builtin_amdgcn_sched_barrier(0);
     });
@@ -406,6 +410,9 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
   }
   if (j < nk) step(lds0, lds1, j);
   wait_dma<0>();  // no LDS write of this workgroup may be in flight when it ends
+  // The compiler does not know that the assembly statements are MFMAs, so it would not keep the
+  // epilogue's accumulator reads the required distance from the last of them: do it by hand.
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 #ifdef HC_PROBE_WAITS
   const uint64_t probe_c1 = __builtin_readcyclecounter(), probe_r1 = __builtin_amdgcn_s_memrealtime();
 #endif

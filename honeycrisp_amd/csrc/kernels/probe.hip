@@ -47,6 +47,7 @@ HC_KERNEL void hc_probe_mfma_f16_32x32x16(hck_probe_args p) {
     asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(acc[t]) : "v"(b[t / 4]), "v"(a[t % 4]));
   };
   for (uint32_t it = 0; it < p.iters; it++) probe_static_for<16>([&](auto tc) { mma(decltype(tc)::value); });
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");  // the compiler does not know the statements above are MFMAs
   float s = 0.0f;
   probe_static_for<16>([&](auto tc) {
 #pragma unroll
@@ -70,6 +71,7 @@ HC_KERNEL void hc_probe_mfma_f16_16x16x32(hck_probe_args p) {
     asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[t]) : "v"(b[(t / 8) % 4]), "v"(a[t % 4]));
   };
   for (uint32_t it = 0; it < p.iters / 2; it++) probe_static_for<64>([&](auto tc) { mma(decltype(tc)::value); });
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
   float s = 0.0f;
   probe_static_for<64>([&](auto tc) {
 #pragma unroll
