@@ -3,6 +3,8 @@ inputs. Bit-exact for integer / index / data-movement work and for element-wise 
 arithmetic that involves no libm call; otherwise the reference's own criterion
 (|a-b| <= tol or |a/b-1| <= tol, Assertions.swift:16) with tol 1e-4 for fp32 and 1e-2 for
 fp16, plus a norm-wise bound for GEMMs."""
+import os
+
 import numpy as np
 import pytest
 
@@ -161,6 +163,34 @@ def test_matmul_fp16_4096_against_oracle_slab_and_identity(hip_backend, oracle_b
         eye = Tensor(data=np.eye(n, dtype=np.float16))
         assert np.array_equal(Tensor.matmul(ta, False, eye, False, False).numpy(), a)
         assert np.array_equal(Tensor.matmul(eye, False, tb, False, False).numpy(), b)
+
+
+def test_matmul_fp16_large_ragged_against_oracle_slab(hip_backend, oracle_backend):
+    """A product large enough for the host to pick the full-device fp16 kernel, but ragged in M, N
+    and K (edge variant: clamped rows, zero-filled K tail, predicated stores): row slabs against
+    the oracle, the whole result against the general kernel, and nothing written past the edges."""
+    rng = np.random.default_rng(12)
+    M, K, N = 4100, 1032, 4104
+    a = (rng.standard_normal((M, K)) / np.sqrt(K)).astype(np.float16)
+    b = rng.standard_normal((K, N)).astype(np.float16)
+    rows = np.r_[0:24, 2040:2064, M - 24:M]
+    with oracle_backend.use():
+        want = Tensor.matmul(Tensor(data=a[rows]), False, Tensor(data=b), False, False).numpy()
+    with hip_backend.use():
+        ta, tb = Tensor(data=a), Tensor(data=b)
+        tat, tbt = Tensor(data=np.ascontiguousarray(a.T)), Tensor(data=np.ascontiguousarray(b.T))
+        os.environ["HCHIP_GEMM_TILE"] = "general"
+        try:
+            general = Tensor.matmul(ta, False, tb, False, False).numpy()
+        finally:
+            del os.environ["HCHIP_GEMM_TILE"]
+        assert_close_arrays(general[rows], want, 1e-2, 1e-2)
+        for transA, transB in [(False, False), (False, True), (True, False), (True, True)]:
+            print("4100x1032x4104 layout", transA, transB, flush=True)
+            out = Tensor.matmul(tat if transA else ta, transA, tbt if transB else tb, transB, False).numpy()
+            assert out.shape == (M, N)
+            assert_close_arrays(out[rows], want, 1e-2, 1e-2)
+            assert_close_arrays(out, general, 1e-2, 1e-2)
 
 
 def test_matmul_int64(hip_backend, oracle_backend):
