@@ -2009,6 +2009,21 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
         }
       }
     }
+    // Long fp16 products are limited by power, not by idle CUs: CUs that sit out leave the busy
+    // ones a higher clock, so large tiles on part of the device beat small tiles on all of it
+    // well before the large tiles fill it (measured: 144 tiles of 256 x 256 on 256 CUs run
+    // at 58 % of the full-device rate, 196 at 72 %).
+    if (!(force && *force) && !which && dma && dtype == HC_F16 && K >= 1024) {
+      const uint64_t t256 = ceil_div(M, 256) * ceil_div(N, 256) * (uint64_t)batch;
+      const uint64_t t128 = ceil_div(M, 128) * ceil_div(N, 128) * (uint64_t)batch;
+      if (2 * t256 >= cus && t256 < cus) {
+        bm = bn = 256;
+        dma2 = mi16 = true;
+      } else if (t256 < cus && 2 * t128 >= 3 * cus) {
+        bm = bn = 128;
+        dma2 = mi16 = true;
+      }
+    }
     if (bm != 0 && dma) {
       const uint64_t blocks = ceil_div(M, bm) * ceil_div(N, bn) * (uint64_t)batch;
       // (whole cache lines only help an operand that is contiguous along K: TN products stay
