@@ -143,6 +143,30 @@ def test_matmul_both_pipelines_every_tile(hip_backend, oracle_backend, monkeypat
                     assert float(np.max(np.abs(got.astype(np.float64) - want.astype(np.float64)))) <= TOL[dtype] * scale
 
 
+@pytest.mark.parametrize("pipeline", ["auto", "dma", "dma2", "mi16"])
+def test_matmul_random_shapes(hip_backend, oracle_backend, monkeypatch, pipeline):
+    """Seeded random extents (aligned and odd), batches and flags through each pipeline: row and
+    K raggedness against every tile edge, re-pitched operands, transposed outputs."""
+    rng = np.random.default_rng(2024)
+    if pipeline != "auto":
+        monkeypatch.setenv("HCHIP_GEMM_KERNEL", pipeline)
+    for case in range(24):
+        dtype = F16 if (pipeline == "mi16" or case % 2 == 0) else F32
+        align = [1, 8, 8, 64][case % 4]
+        M, K, N = (int(rng.integers(1, 90 if align < 64 else 24)) * align for _ in range(3))
+        batch = int(rng.integers(1, 4))
+        transA, transB, transOut = (bool(rng.integers(0, 2)) for _ in range(3))
+        a = rand(rng, (batch, M, K), dtype, 1.0 / K ** 0.5)
+        b = rand(rng, (batch, K, N), dtype)
+        sa = np.ascontiguousarray(a.transpose(0, 2, 1)) if transA else a
+        sb = np.ascontiguousarray(b.transpose(0, 2, 1)) if transB else b
+        print("matmul", pipeline, dtype.name, batch, M, K, N, transA, transB, transOut, flush=True)
+        fn = lambda: Tensor.batchedMatmul(Tensor(data=sa), transA, Tensor(data=sb), transB, transOut)
+        got, want = check_close(hip_backend, oracle_backend, fn, TOL[dtype])
+        scale = float(np.max(np.abs(want.astype(np.float64))))
+        assert float(np.max(np.abs(got.astype(np.float64) - want.astype(np.float64)))) <= TOL[dtype] * max(scale, 1e-30)
+
+
 def test_matmul_fp16_4096_against_oracle_slab_and_identity(hip_backend, oracle_backend):
     """Config 2 at full size: every layout; a 96-row slab of each product is checked against
     the oracle, and A x I == A exactly."""
