@@ -1934,140 +1934,178 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
     k.b_rs = b_rs;
     k.b_cs = b_cs;
   }
-  // what an edge kernel may fetch: all rows of a K-contiguous operand, whole 16-byte pieces of
-  // an M/N-contiguous one (its leading dimension covers them)
-  k.a_lim = ma == 'k' ? M : (M + P - 1) / P * P;
-  k.b_lim = mb == 'k' ? N : (N + P - 1) / P * P;
+  // Kernel choice and launch for the block of C that `k` describes (pointers and strides set;
+  // M x N its extent): the whole product, or a part of it when a thin fringe is peeled off below.
+  auto run = [&](hck_gemm_args k, uint32_t M, uint32_t N) -> int {
+    // what an edge kernel may fetch: all rows of a K-contiguous operand, whole 16-byte pieces of
+    // an M/N-contiguous one (its leading dimension covers them)
+    k.M = M;
+    k.N = N;
+    k.tiles_m = (uint32_t)ceil_div(M, 128);  // (general kernel; the tuned kernels set their own below)
+    k.tiles_n = (uint32_t)ceil_div(N, 128);
+    k.a_lim = ma == 'k' ? M : (M + P - 1) / P * P;
+    k.b_lim = mb == 'k' ? N : (N + P - 1) / P * P;
 
-  // Tuned kernels. Direct-to-LDS (fp16, fp32): rows of A, B and C 16-byte aligned, operands
-  // addressed with 32-bit byte offsets; ragged M, N, K run the "_e" variants (clamped rows,
-  // zero-filled K tail, predicated stores). HCHIP_GEMM_TILE=general|<BM>x<BN> overrides the
-  // tile choice and HCHIP_GEMM_KERNEL=staged selects the register-staged fp16 pipeline
-  // (whole tiles, K % 64 == 0), both for measurements.
-  uint32_t bm = 0, bn = 0;
-  bool edge = false;
-  const char* which = getenv("HCHIP_GEMM_KERNEL");
-  const uint64_t max_elems = 0xffffffffull / el;
-  const bool dma = k.a_bs <= max_elems && k.b_bs <= max_elems && !(which && strcmp(which, "staged") == 0);
-  // Two direct-to-LDS pipelines: four stages of 64-byte K-slices (deep prefetch: best when a CU
-  // has one short job) and two stages of 128-byte K-slices (whole cache lines for K-contiguous
-  // operands, half the barriers: best when the CUs are kept busy for long). Chosen below, after
-  // the tile; HCHIP_GEMM_KERNEL=dma|dma2 forces one.
-  // A third variant, fp16 only: the 128-byte-slice pipeline on the 16x16x32 MFMA shape, which
-  // needs less power per multiply-accumulate. It pays where the matrix cores run into the
-  // board's power limit: every CU busy with a 256 x 256 tile over a long K.
-  // HCHIP_GEMM_KERNEL=dma|dma2|mi16 forces one of the three.
-  bool mi16 = dma && dtype == HC_F16 && which && strcmp(which, "mi16") == 0;
-  bool dma2 = dma && which && (strcmp(which, "dma2") == 0 || mi16);
-  uint32_t slice = (uint32_t)(64 / el);
-  const bool eligible = ma != 'x' && mb != 'x' && K > 0 && aligned16(k.c) &&
-                        (dma ? (k.c_rs % P == 0 && (batch <= 1 || k.c_bs % P == 0)) : (dtype == HC_F16 && K % 64 == 0));
-  if (eligible) {
-    const char* force = getenv("HCHIP_GEMM_TILE");
-    auto whole = [&](uint32_t tm, uint32_t tn) { return M % tm == 0 && N % tn == 0 && K % slice == 0; };
-    // largest tile first; the direct-to-LDS kernels also come in narrow shapes
-    static const uint32_t tiles[][2] = {{256, 256}, {256, 128}, {128, 128}, {256, 64}, {128, 64}, {64, 64}};
-    const uint64_t cus = (uint64_t)ctx->props.multiProcessorCount;
-    if (force && *force) {
-      unsigned fm = 0, fn = 0;
-      if (sscanf(force, "%ux%u", &fm, &fn) == 2 && (dma || whole(fm, fn))) {
-        bool known = false;
-        for (auto& t : tiles) known = known || (t[0] == fm && t[1] == fn);
-        if (known) {
-          bm = fm;
-          bn = fn;
+    // Tuned kernels. Direct-to-LDS (fp16, fp32): rows of A, B and C 16-byte aligned, operands
+    // addressed with 32-bit byte offsets; ragged M, N, K run the "_e" variants (clamped rows,
+    // zero-filled K tail, predicated stores). HCHIP_GEMM_TILE=general|<BM>x<BN> overrides the
+    // tile choice and HCHIP_GEMM_KERNEL=staged selects the register-staged fp16 pipeline
+    // (whole tiles, K % 64 == 0), both for measurements.
+    uint32_t bm = 0, bn = 0;
+    bool edge = false;
+    const char* which = getenv("HCHIP_GEMM_KERNEL");
+    const uint64_t max_elems = 0xffffffffull / el;
+    const bool dma = k.a_bs <= max_elems && k.b_bs <= max_elems && !(which && strcmp(which, "staged") == 0);
+    // Two direct-to-LDS pipelines: four stages of 64-byte K-slices (deep prefetch: best when a CU
+    // has one short job) and two stages of 128-byte K-slices (whole cache lines for K-contiguous
+    // operands, half the barriers: best when the CUs are kept busy for long). Chosen below, after
+    // the tile; HCHIP_GEMM_KERNEL=dma|dma2 forces one.
+    // A third variant, fp16 only: the 128-byte-slice pipeline on the 16x16x32 MFMA shape, which
+    // needs less power per multiply-accumulate. It pays where the matrix cores run into the
+    // board's power limit: every CU busy with a 256 x 256 tile over a long K.
+    // HCHIP_GEMM_KERNEL=dma|dma2|mi16 forces one of the three.
+    bool mi16 = dma && dtype == HC_F16 && which && strcmp(which, "mi16") == 0;
+    bool dma2 = dma && which && (strcmp(which, "dma2") == 0 || mi16);
+    uint32_t slice = (uint32_t)(64 / el);
+    const bool eligible = ma != 'x' && mb != 'x' && K > 0 && aligned16(k.c) &&
+                          (dma ? (k.c_rs % P == 0 && (batch <= 1 || k.c_bs % P == 0)) : (dtype == HC_F16 && K % 64 == 0));
+    if (eligible) {
+      const char* force = getenv("HCHIP_GEMM_TILE");
+      auto whole = [&](uint32_t tm, uint32_t tn) { return M % tm == 0 && N % tn == 0 && K % slice == 0; };
+      // largest tile first; the direct-to-LDS kernels also come in narrow shapes
+      static const uint32_t tiles[][2] = {{256, 256}, {256, 128}, {128, 128}, {256, 64}, {128, 64}, {64, 64}};
+      const uint64_t cus = (uint64_t)ctx->props.multiProcessorCount;
+      if (force && *force) {
+        unsigned fm = 0, fn = 0;
+        if (sscanf(force, "%ux%u", &fm, &fn) == 2 && (dma || whole(fm, fn))) {
+          bool known = false;
+          for (auto& t : tiles) known = known || (t[0] == fm && t[1] == fn);
+          if (known) {
+            bm = fm;
+            bn = fn;
+          }
         }
-      }
-    } else {
-      // Among the tiles that give every CU a block: the best product of (rough per-CU rate of
-      // the tile) x (fraction of the last round of blocks that is busy) x (fraction of the
-      // tiles' area that is real output). If no tile fills the device: the one with most blocks.
-      static const double rate16[] = {1.0, 0.85, 0.7, 0.55, 0.45, 0.3};
-      static const double rate32[] = {1.0, 0.95, 0.85, 0.8, 0.7, 0.55};
-      const double* rate = dtype == HC_F32 ? rate32 : rate16;
-      uint64_t best_blocks = 0;
-      double best_score = 0.0;
-      bool filled = false;
-      for (size_t ti = 0; ti < sizeof(tiles) / sizeof(tiles[0]); ti++) {
-        const uint32_t* t = tiles[ti];
-        if (!dma && (!whole(t[0], t[1]) || t[1] < 128)) continue;
-        const uint64_t blocks = ceil_div(M, t[0]) * ceil_div(N, t[1]) * (uint64_t)batch;
-        if (blocks >= cus) {
-          const double rounds = (double)ceil_div(blocks, cus);
-          const double useful = ((double)M * N * (double)batch) / ((double)blocks * t[0] * t[1]);
-          const double score = rate[ti] * ((double)blocks / (rounds * (double)cus)) * useful;
-          if (!filled || score > best_score) {
-            filled = true;
-            best_score = score;
+      } else {
+        // Among the tiles that give every CU a block: the best product of (rough per-CU rate of
+        // the tile) x (fraction of the last round of blocks that is busy) x (fraction of the
+        // tiles' area that is real output). If no tile fills the device: the one with most blocks.
+        static const double rate16[] = {1.0, 0.85, 0.7, 0.55, 0.45, 0.3};
+        static const double rate32[] = {1.0, 0.95, 0.85, 0.8, 0.7, 0.55};
+        const double* rate = dtype == HC_F32 ? rate32 : rate16;
+        uint64_t best_blocks = 0;
+        double best_score = 0.0;
+        bool filled = false;
+        for (size_t ti = 0; ti < sizeof(tiles) / sizeof(tiles[0]); ti++) {
+          const uint32_t* t = tiles[ti];
+          if (!dma && (!whole(t[0], t[1]) || t[1] < 128)) continue;
+          const uint64_t blocks = ceil_div(M, t[0]) * ceil_div(N, t[1]) * (uint64_t)batch;
+          if (blocks >= cus) {
+            const double rounds = (double)ceil_div(blocks, cus);
+            const double useful = ((double)M * N * (double)batch) / ((double)blocks * t[0] * t[1]);
+            const double score = rate[ti] * ((double)blocks / (rounds * (double)cus)) * useful;
+            if (!filled || score > best_score) {
+              filled = true;
+              best_score = score;
+              bm = t[0];
+              bn = t[1];
+            }
+          } else if (!filled && blocks > best_blocks) {
+            best_blocks = blocks;
             bm = t[0];
             bn = t[1];
           }
-        } else if (!filled && blocks > best_blocks) {
-          best_blocks = blocks;
-          bm = t[0];
-          bn = t[1];
         }
       }
-    }
-    // Long fp16 products are limited by power, not by idle CUs: CUs that sit out leave the busy
-    // ones a higher clock, so large tiles on part of the device beat small tiles on all of it
-    // well before the large tiles fill it (measured: 144 tiles of 256 x 256 on 256 CUs run
-    // at 58 % of the full-device rate, 196 at 72 %).
-    if (!(force && *force) && !which && dma && dtype == HC_F16 && K >= 1024) {
-      const uint64_t t256 = ceil_div(M, 256) * ceil_div(N, 256) * (uint64_t)batch;
-      const uint64_t t128 = ceil_div(M, 128) * ceil_div(N, 128) * (uint64_t)batch;
-      if (2 * t256 >= cus && t256 < cus) {
-        bm = bn = 256;
-        dma2 = mi16 = true;
-      } else if (t256 < cus && 2 * t128 >= 3 * cus) {
-        bm = bn = 128;
-        dma2 = mi16 = true;
-      }
-    }
-    if (bm != 0 && dma) {
-      const uint64_t blocks = ceil_div(M, bm) * ceil_div(N, bn) * (uint64_t)batch;
-      // (whole cache lines only help an operand that is contiguous along K: TN products stay
-      // with the four-stage ring)
-      const bool k_contig = ma == 'k' || mb == 'k';
-      if (!which && k_contig && (uint64_t)K * el >= 2048 && ((bm == 256 && bn == 256) || blocks >= 2 * cus))
-        dma2 = true;
-      if (!which && dtype == HC_F16 && K >= 1024 && bm == 256 && bn == 256 && blocks >= cus) dma2 = mi16 = true;
-      if (dma2) slice = (uint32_t)(128 / el);
-    }
-    if (bm != 0) edge = !whole(bm, bn);
-  }
-  if (bm != 0) {
-    k.tiles_m = (uint32_t)ceil_div(M, bm);
-    k.tiles_n = (uint32_t)ceil_div(N, bn);
-    k.zeros = ctx->zeros;
-    if (dma && !getenv("HCHIP_GEMM_BAND")) {
-      // largest XCD rectangle whose super-block (4 x 2 XCDs) divides the tile grid
-      static const uint32_t shapes[][2] = {{4, 8}, {2, 4}, {1, 2}};
-      for (auto& sh : shapes)
-        if (k.tiles_m % (4 * sh[0]) == 0 && k.tiles_n % (2 * sh[1]) == 0) {
-          k.xcd_gn = 2;
-          k.xcd_sm = sh[0];
-          k.xcd_sn = sh[1];
-          break;
+      // Long fp16 products are limited by power, not by idle CUs: CUs that sit out leave the busy
+      // ones a higher clock, so large tiles on part of the device beat small tiles on all of it
+      // well before the large tiles fill it (measured: 144 tiles of 256 x 256 on 256 CUs run
+      // at 58 % of the full-device rate, 196 at 72 %).
+      if (!(force && *force) && !which && dma && dtype == HC_F16 && K >= 1024) {
+        const uint64_t t256 = ceil_div(M, 256) * ceil_div(N, 256) * (uint64_t)batch;
+        const uint64_t t128 = ceil_div(M, 128) * ceil_div(N, 128) * (uint64_t)batch;
+        if (2 * t256 >= cus && t256 < cus) {
+          bm = bn = 256;
+          dma2 = mi16 = true;
+        } else if (t256 < cus && 2 * t128 >= 3 * cus) {
+          bm = bn = 128;
+          dma2 = mi16 = true;
         }
+      }
+      if (bm != 0 && dma) {
+        const uint64_t blocks = ceil_div(M, bm) * ceil_div(N, bn) * (uint64_t)batch;
+        // (whole cache lines only help an operand that is contiguous along K: TN products stay
+        // with the four-stage ring)
+        const bool k_contig = ma == 'k' || mb == 'k';
+        if (!which && k_contig && (uint64_t)K * el >= 2048 && ((bm == 256 && bn == 256) || blocks >= 2 * cus))
+          dma2 = true;
+        if (!which && dtype == HC_F16 && K >= 1024 && bm == 256 && bn == 256 && blocks >= cus) dma2 = mi16 = true;
+        if (dma2) slice = (uint32_t)(128 / el);
+      }
+      if (bm != 0) edge = !whole(bm, bn);
     }
-    snprintf(name, sizeof(name), "hc_gemm_%s_%s_%ux%u_%c%c%s", dtype_name(dtype), dma ? (mi16 ? "mi16" : dma2 ? "dma2" : "dma") : "fast", bm, bn,
-             ma == 'k' ? 'k' : 'm', mb == 'k' ? 'k' : 'n', edge ? "_e" : "");
-  } else if (ma == 'x' || mb == 'x')
-    snprintf(name, sizeof(name), "hc_gemm_%s_xx", dtype_name(dtype));
-  else
-    snprintf(name, sizeof(name), "hc_gemm_%s_%c%c", dtype_name(dtype), ma == 'k' ? 'k' : 'm',
-             mb == 'k' ? 'k' : 'n');
-  const uint64_t tiles = (uint64_t)k.tiles_m * k.tiles_n;
-  // grid.y carries the batch (at most 65535 per launch)
-  for (int64_t b0 = 0; b0 < batch; b0 += 65535) {
-    const uint32_t nb = (uint32_t)(batch - b0 < 65535 ? batch - b0 : 65535);
-    hck_gemm_args kk = k;
-    kk.a = (const char*)k.a + (uint64_t)b0 * k.a_bs * el;
-    kk.b = (const char*)k.b + (uint64_t)b0 * k.b_bs * el;
-    kk.c = (char*)k.c + (uint64_t)b0 * k.c_bs * el;
-    kk.batch = nb;
-    HC_TRY(launch(ctx, name, tiles, nb, &kk, sizeof(kk)));
+    if (bm != 0) {
+      k.tiles_m = (uint32_t)ceil_div(M, bm);
+      k.tiles_n = (uint32_t)ceil_div(N, bn);
+      k.zeros = ctx->zeros;
+      if (dma && !getenv("HCHIP_GEMM_BAND")) {
+        // largest XCD rectangle whose super-block (4 x 2 XCDs) divides the tile grid
+        static const uint32_t shapes[][2] = {{4, 8}, {2, 4}, {1, 2}};
+        for (auto& sh : shapes)
+          if (k.tiles_m % (4 * sh[0]) == 0 && k.tiles_n % (2 * sh[1]) == 0) {
+            k.xcd_gn = 2;
+            k.xcd_sm = sh[0];
+            k.xcd_sn = sh[1];
+            break;
+          }
+      }
+      snprintf(name, sizeof(name), "hc_gemm_%s_%s_%ux%u_%c%c%s", dtype_name(dtype), dma ? (mi16 ? "mi16" : dma2 ? "dma2" : "dma") : "fast", bm, bn,
+               ma == 'k' ? 'k' : 'm', mb == 'k' ? 'k' : 'n', edge ? "_e" : "");
+    } else if (ma == 'x' || mb == 'x')
+      snprintf(name, sizeof(name), "hc_gemm_%s_xx", dtype_name(dtype));
+    else
+      snprintf(name, sizeof(name), "hc_gemm_%s_%c%c", dtype_name(dtype), ma == 'k' ? 'k' : 'm',
+               mb == 'k' ? 'k' : 'n');
+    const uint64_t tiles = (uint64_t)k.tiles_m * k.tiles_n;
+    // grid.y carries the batch (at most 65535 per launch)
+    for (int64_t b0 = 0; b0 < batch; b0 += 65535) {
+      const uint32_t nb = (uint32_t)(batch - b0 < 65535 ? batch - b0 : 65535);
+      hck_gemm_args kk = k;
+      kk.a = (const char*)k.a + (uint64_t)b0 * k.a_bs * el;
+      kk.b = (const char*)k.b + (uint64_t)b0 * k.b_bs * el;
+      kk.c = (char*)k.c + (uint64_t)b0 * k.c_bs * el;
+      kk.batch = nb;
+      HC_TRY(launch(ctx, name, tiles, nb, &kk, sizeof(kk)));
+    }
+    return HC_OK;
+  };
+  // A last row or column of tiles that is almost empty costs as much as a full one: 4097 rows
+  // are 17 rows of 256-row tiles, i.e. two rounds on a device that 16 x 16 tiles fill exactly.
+  // Products that are a few rows or columns over a multiple of 256 are therefore split into the
+  // multiple-of-256 body and thin fringes, each run as a product of its own on sub-blocks of the
+  // same buffers (same strides, offset pointers).
+  // (only long products: the fringes are skinny products of their own that take tens of
+  // microseconds, which a short body does not win back)
+  auto fringe = [&](uint32_t d) { return d >= 2048 && d % 256 != 0 && d % 256 <= 32 ? d % 256 : 0u; };
+  const bool tuned = ma != 'x' && mb != 'x' && K >= 2048 && !getenv("HCHIP_GEMM_TILE") && !getenv("HCHIP_GEMM_NO_PEEL");
+  const bool large = (uint64_t)M * N >= (1ull << 22);
+  const uint32_t fm = tuned && large ? fringe(M) : 0, fn = tuned && large ? fringe(N) : 0;
+  if (fm != 0 || fn != 0) {
+    const uint32_t Mb = M - fm, Nb = N - fn;
+    HC_TRY(run(k, Mb, Nb));
+    if (fn != 0) {  // columns Nb .. N-1 of every row
+      hck_gemm_args f = k;
+      f.b = (const char*)k.b + (uint64_t)Nb * k.b_cs * el;
+      f.c = (char*)k.c + (uint64_t)Nb * k.c_cs * el;
+      HC_TRY(run(f, M, fn));
+    }
+    if (fm != 0) {  // rows Mb .. M-1, columns 0 .. Nb-1
+      hck_gemm_args f = k;
+      f.a = (const char*)k.a + (uint64_t)Mb * k.a_rs * el;
+      f.c = (char*)k.c + (uint64_t)Mb * k.c_rs * el;
+      HC_TRY(run(f, fm, Nb));
+    }
+  } else {
+    HC_TRY(run(k, M, N));
   }
   if (c_padded) {
     // padded result back into the caller's dense [M, N] matrices
