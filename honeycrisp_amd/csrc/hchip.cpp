@@ -1954,6 +1954,70 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
     uint32_t bm = 0, bn = 0;
     bool edge = false;
     const char* which = getenv("HCHIP_GEMM_KERNEL");
+    // Skinny products (one extent of C at most 4, the other long: matrix-vector products and
+    // the thinnest fringes peeled off below) are bound by reading the long operand once: no
+    // tiles. (Wider ones are faster on the tile kernels.)
+    if (!which && !getenv("HCHIP_GEMM_TILE") && K >= 64 && std::min(M, N) <= 4 && std::max(M, N) >= 512 &&
+        batch <= 65535) {
+      const bool thin_n = N <= M;
+      hck_skinny_args sk;
+      memset(&sk, 0, sizeof(sk));
+      sk.K = K;
+      sk.c = k.c;
+      sk.c_bs = k.c_bs;
+      if (thin_n) {  // X = A (p = m), Y = B
+        sk.x = k.a, sk.x_ps = k.a_rs, sk.x_ks = k.a_cs, sk.x_bs = k.a_bs;
+        sk.y = k.b, sk.y_ks = k.b_rs, sk.y_qs = k.b_cs, sk.y_bs = k.b_bs;
+        sk.c_ps = k.c_rs, sk.c_qs = k.c_cs, sk.L = M, sk.t = N;
+      } else {  // X = B (p = n), Y = A
+        sk.x = k.b, sk.x_ps = k.b_cs, sk.x_ks = k.b_rs, sk.x_bs = k.b_bs;
+        sk.y = k.a, sk.y_ks = k.a_cs, sk.y_qs = k.a_rs, sk.y_bs = k.a_bs;
+        sk.c_ps = k.c_cs, sk.c_qs = k.c_rs, sk.L = N, sk.t = M;
+      }
+      const char* tq = "q4";
+      char sname[64];
+      // The thin operand is read by every wave: unless it already is contiguous along k with
+      // aligned rows, pack it first as [q][k] (a few KiB that then stay in the caches).
+      Scratch packed(ctx);
+      if ((sk.x_ks == 1 || sk.x_ps == 1) &&
+          !(sk.y_ks == 1 && aligned16(sk.y) && sk.y_qs % P == 0 && (batch <= 1 || sk.y_bs % P == 0))) {
+        const uint32_t kp = (K + P - 1) / P * P;
+        void* buf = nullptr;
+        HC_TRY(packed.get((size_t)batch * sk.t * kp * el, &buf));
+        hck_skinny_args pk = sk;
+        pk.c = buf;
+        pk.c_qs = sk.y_qs;  // source stride along q
+        pk.y_qs = kp;       // packed row length
+        snprintf(sname, sizeof(sname), "hc_gemm_skinny_pack_%s", dtype_name(dtype));
+        HC_TRY(launch(ctx, sname, ceil_div((uint64_t)sk.t * kp, HCK_BLOCK), (uint32_t)batch, &pk, sizeof(pk)));
+        sk.y = buf;
+        sk.y_ks = 1;
+        sk.y_qs = kp;
+        sk.y_bs = (uint64_t)sk.t * kp;
+      }
+      if (sk.x_ks == 1 && aligned16(sk.x) && sk.x_ps % P == 0 && (batch <= 1 || sk.x_bs % P == 0)) {
+        snprintf(sname, sizeof(sname), "hc_gemm_skinny_k_%s_%s", dtype_name(dtype), tq);
+        return launch(ctx, sname, ceil_div(sk.L, HCK_BLOCK / 64), (uint32_t)batch, &sk, sizeof(sk));
+      }
+      if (sk.x_ps == 1 && aligned16(sk.x) && sk.x_ks % P == 0 && (batch <= 1 || sk.x_bs % P == 0)) {
+        // a workgroup per (64 lanes x 16 bytes of p, chunk of k): about two per CU, at least 32 k each
+        const uint64_t cus = (uint64_t)ctx->props.multiProcessorCount;
+        const uint64_t ptiles = ceil_div(sk.L, 64 * P);
+        uint64_t chunks = std::max<uint64_t>(1, std::min<uint64_t>(ceil_div(2 * cus, ptiles * (uint64_t)batch), K / 32));
+        sk.kchunk = (uint32_t)ceil_div(K, chunks);
+        chunks = ceil_div(K, sk.kchunk);
+        Scratch sums(ctx);
+        void* acc = nullptr;
+        const uint64_t n_acc = (uint64_t)batch * sk.L * sk.t;
+        HC_TRY(sums.get(n_acc * sizeof(float), &acc));
+        HC_TRY(hc_fill(ctx, HC_F32, 0.0f, 0, acc, n_acc));
+        sk.acc = (float*)acc;
+        snprintf(sname, sizeof(sname), "hc_gemm_skinny_p_%s_%s", dtype_name(dtype), tq);
+        HC_TRY(launch(ctx, sname, ptiles * chunks, (uint32_t)batch, &sk, sizeof(sk)));
+        snprintf(sname, sizeof(sname), "hc_gemm_skinny_store_%s", dtype_name(dtype));
+        return launch(ctx, sname, ceil_div((uint64_t)sk.L * sk.t, HCK_BLOCK), (uint32_t)batch, &sk, sizeof(sk));
+      }
+    }
     const uint64_t max_elems = 0xffffffffull / el;
     const bool dma = k.a_bs <= max_elems && k.b_bs <= max_elems && !(which && strcmp(which, "staged") == 0);
     // Two direct-to-LDS pipelines: four stages of 64-byte K-slices (deep prefetch: best when a CU

@@ -265,4 +265,18 @@ typedef struct {
   uint64_t in_ld, out_ld, in_bs, out_bs;
 } hck_copy2d_args;
 
+/* Skinny product C[p, q] = sum_k X[p, k] * Y[k, q]: p over a long extent L, q over a thin one
+ * t <= 32 (a matrix-vector product, or the fringe of a ragged GEMM). Element strides; which of
+ * A / B is X and whether C is stored [p, q] or [q, p] is folded into the strides by the host. */
+typedef struct {
+  const void* x;
+  const void* y;
+  void* c;
+  float* acc;  /* split-K form: fp32 partial sums [batch, L, t], zero before the launch */
+  uint32_t L, t, K;
+  uint32_t x_ps, x_ks, y_ks, y_qs, c_ps, c_qs;
+  uint32_t kchunk; /* split-K form: k-range per workgroup */
+  uint64_t x_bs, y_bs, c_bs;
+} hck_skinny_args;
+
 #endif

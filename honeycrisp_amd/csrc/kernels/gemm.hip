@@ -255,3 +255,132 @@ HC_KERNEL void hc_gemm_i64(hck_gemm_args p) {
   }
   if (m < p.M && n < p.N) C[(size_t)m * p.c_rs + (size_t)n * p.c_cs] = acc;
 }
+
+// Skinny products (one extent of C at most 4: matrix-vector products, the fringes of ragged
+// GEMMs): bound by reading the long operand once, so no matrix instructions, fp32 accumulation
+// on the vector ALU. C[p, q] = sum_k X[p, k] * Y[k, q], p long, q thin.
+//
+// Long operand contiguous along k: one wave per p. Lanes stride over k in 16-byte pieces, keep
+// one partial sum per q, and the wave adds them up at the end.
+template <typename T, int TQ> __device__ __forceinline__ void skinny_k_impl(const hck_skinny_args& a) {
+  constexpr int V = 16 / sizeof(T);
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t p = blockIdx.x * (HCK_BLOCK / 64) + (threadIdx.x >> 6);
+  if (p >= a.L) return;
+  const T* X = (const T*)a.x + (uint64_t)blockIdx.y * a.x_bs + (size_t)p * a.x_ps;
+  const T* Y = (const T*)a.y + (uint64_t)blockIdx.y * a.y_bs;
+  T* C = (T*)a.c + (uint64_t)blockIdx.y * a.c_bs + (size_t)p * a.c_ps;
+  float acc[TQ];
+#pragma unroll
+  for (int q = 0; q < TQ; q++) acc[q] = 0.0f;
+  for (uint32_t k0 = lane * V; k0 < a.K; k0 += 64 * V) {
+    T x[V];
+    if (k0 + V <= a.K) {
+      load_vec<T, V>(X, k0, 1, x);
+    } else {
+#pragma unroll
+      for (int e = 0; e < V; e++) x[e] = k0 + e < a.K ? X[k0 + e] : (T)0;
+    }
+    // Y is contiguous along k with 16-byte aligned rows that are padded to a multiple of V (the
+    // host packs it that way if need be), so the same piece of every q is one vector load
+#pragma unroll
+    for (int q = 0; q < TQ; q++) {
+      if (q < (int)a.t) {
+        T y[V];
+        load_vec<T, V>(Y + (size_t)q * a.y_qs, k0, 1, y);
+#pragma unroll
+        for (int e = 0; e < V; e++) acc[q] = acc[q] + (float)x[e] * (float)y[e];
+      }
+    }
+  }
+#pragma unroll
+  for (int q = 0; q < TQ; q++) {
+    float v = acc[q];
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) v += __shfl_down(v, d, 64);
+    if (lane == 0 && q < (int)a.t) C[(size_t)q * a.c_qs] = narrow<T>(v);
+  }
+}
+
+// Long operand contiguous along p (16-byte aligned k-rows): a lane owns V consecutive p, a
+// wave reads 64 * V consecutive elements of a k-row per step; a workgroup covers one such
+// p-tile and a chunk of the k-range (grid.x = p-tiles * k-chunks), its four waves take every
+// fourth k-row and add their partial sums up in LDS; the chunks meet in an fp32 buffer through
+// atomic adds and hc_gemm_skinny_store rounds them. Y is packed [q][k].
+template <typename T, int TQ> __device__ __forceinline__ void skinny_p_impl(const hck_skinny_args& a) {
+  constexpr int V = 16 / sizeof(T), WAVES = HCK_BLOCK / 64, TILE = 64 * V;
+  __shared__ float part[WAVES][TQ][TILE];
+  const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t ptiles = (a.L + TILE - 1) / TILE;
+  const uint32_t chunk = blockIdx.x / ptiles, pt = blockIdx.x - chunk * ptiles;
+  const uint32_t p0 = pt * TILE + lane * V;
+  const uint32_t k_lo = chunk * a.kchunk, k_hi = k_lo + a.kchunk < a.K ? k_lo + a.kchunk : a.K;
+  const T* X = (const T*)a.x + (uint64_t)blockIdx.y * a.x_bs;
+  const T* Y = (const T*)a.y + (uint64_t)blockIdx.y * a.y_bs;
+  float acc[TQ][V];
+#pragma unroll
+  for (int q = 0; q < TQ; q++)
+#pragma unroll
+    for (int e = 0; e < V; e++) acc[q][e] = 0.0f;
+  const bool whole = p0 + V <= a.L;
+#pragma unroll 2
+  for (uint32_t k = k_lo + wave; k < k_hi; k += WAVES) {
+    T x[V];
+    if (whole) {
+      load_vec<T, V>(X + (size_t)k * a.x_ks, p0, 1, x);
+    } else {
+#pragma unroll
+      for (int e = 0; e < V; e++) x[e] = p0 + e < a.L ? X[(size_t)k * a.x_ks + p0 + e] : (T)0;
+    }
+#pragma unroll
+    for (int q = 0; q < TQ; q++) {
+      if (q < (int)a.t) {
+        const float y = (float)Y[(size_t)q * a.y_qs + k];  // wave-uniform
+#pragma unroll
+        for (int e = 0; e < V; e++) acc[q][e] = acc[q][e] + (float)x[e] * y;
+      }
+    }
+  }
+#pragma unroll
+  for (int q = 0; q < TQ; q++)
+#pragma unroll
+    for (int e = 0; e < V; e++) part[wave][q][lane * V + e] = acc[q][e];
+  __syncthreads();
+  for (uint32_t i = threadIdx.x; i < a.t * TILE; i += HCK_BLOCK) {
+    const uint32_t q = i / TILE, c = i - q * TILE;
+    const uint32_t p = pt * TILE + c;
+    if (p >= a.L) continue;
+    float v = 0.0f;
+#pragma unroll
+    for (int w = 0; w < WAVES; w++) v += part[w][q][c];
+    __hip_atomic_fetch_add(a.acc + ((uint64_t)blockIdx.y * a.L + p) * a.t + q, v, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
+// Y[k, q] (any strides) -> packed[q][k], rows padded with zeros to `y_qs` elements (a multiple of
+// a 16-byte piece): a.c = packed, a.y = source, strides of the source in y_ks / c_qs.
+template <typename T> __device__ __forceinline__ void skinny_pack_impl(const hck_skinny_args& a) {
+  const uint64_t i = (uint64_t)blockIdx.x * HCK_BLOCK + threadIdx.x;
+  if (i >= (uint64_t)a.t * a.y_qs) return;
+  const uint32_t q = (uint32_t)(i / a.y_qs), k = (uint32_t)(i - (uint64_t)q * a.y_qs);
+  const T* Y = (const T*)a.y + (uint64_t)blockIdx.y * a.y_bs;
+  T* P = (T*)a.c + (uint64_t)blockIdx.y * a.t * a.y_qs;
+  P[i] = k < a.K ? Y[(size_t)k * a.y_ks + (size_t)q * a.c_qs] : (T)0;
+}
+
+template <typename T> __device__ __forceinline__ void skinny_store_impl(const hck_skinny_args& a) {
+  const uint64_t i = (uint64_t)blockIdx.x * HCK_BLOCK + threadIdx.x;
+  if (i >= (uint64_t)a.L * a.t) return;
+  const uint32_t p = (uint32_t)(i / a.t), q = (uint32_t)(i - (uint64_t)p * a.t);
+  T* C = (T*)a.c + (uint64_t)blockIdx.y * a.c_bs;
+  C[(size_t)p * a.c_ps + (size_t)q * a.c_qs] = narrow<T>(a.acc[(uint64_t)blockIdx.y * a.L * a.t + i]);
+}
+
+#define DEF_SKINNY(TN, T)                                                                          \
+  HC_KERNEL void hc_gemm_skinny_k_##TN##_q4(hck_skinny_args a) { skinny_k_impl<T, 4>(a); }         \
+  HC_KERNEL void hc_gemm_skinny_p_##TN##_q4(hck_skinny_args a) { skinny_p_impl<T, 4>(a); }         \
+  HC_KERNEL void hc_gemm_skinny_pack_##TN(hck_skinny_args a) { skinny_pack_impl<T>(a); }             \
+  HC_KERNEL void hc_gemm_skinny_store_##TN(hck_skinny_args a) { skinny_store_impl<T>(a); }
+DEF_SKINNY(f16, half_t)
+DEF_SKINNY(f32, float)

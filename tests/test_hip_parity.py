@@ -167,6 +167,27 @@ def test_matmul_random_shapes(hip_backend, oracle_backend, monkeypatch, pipeline
         assert float(np.max(np.abs(got.astype(np.float64) - want.astype(np.float64)))) <= TOL[dtype] * max(scale, 1e-30)
 
 
+@pytest.mark.parametrize("dtype", [F32, F16], ids=["f32", "f16"])
+def test_matmul_skinny_products(hip_backend, oracle_backend, dtype):
+    """One extent of C at most 32 (matrix-vector products, fringes of ragged GEMMs): the
+    wave-per-row and the lane-per-row / split-K kernels, every layout, a batch, odd strides."""
+    rng = np.random.default_rng(55)
+    for (batch, M, K, N) in [(1, 4097, 1032, 1), (1, 1, 1000, 5000), (2, 3000, 777, 7), (1, 20, 2048, 1024),
+                             (3, 1, 512, 2048), (1, 600, 64, 32), (1, 5, 4099, 515)]:
+        a = rand(rng, (batch, M, K), dtype, 1.0 / K ** 0.5)
+        b = rand(rng, (batch, K, N), dtype)
+        for transA in (False, True):
+            for transB in (False, True):
+                for transOut in (False, True):
+                    sa = np.ascontiguousarray(a.transpose(0, 2, 1)) if transA else a
+                    sb = np.ascontiguousarray(b.transpose(0, 2, 1)) if transB else b
+                    print("skinny", dtype.name, batch, M, K, N, transA, transB, transOut, flush=True)
+                    fn = lambda: Tensor.batchedMatmul(Tensor(data=sa), transA, Tensor(data=sb), transB, transOut)
+                    got, want = check_close(hip_backend, oracle_backend, fn, TOL[dtype])
+                    scale = float(np.max(np.abs(want.astype(np.float64))))
+                    assert float(np.max(np.abs(got.astype(np.float64) - want.astype(np.float64)))) <= TOL[dtype] * scale
+
+
 def test_matmul_fp16_4096_against_oracle_slab_and_identity(hip_backend, oracle_backend):
     """Config 2 at full size: every layout; a 96-row slab of each product is checked against
     the oracle, and A x I == A exactly."""
