@@ -1937,20 +1937,21 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
   // Kernel choice and launch for the block of C that `k` describes (pointers and strides set;
   // M x N its extent): the whole product, or a part of it when a thin fringe is peeled off below.
   auto run = [&](hck_gemm_args k, uint32_t M, uint32_t N) -> int {
-    // what an edge kernel may fetch: all rows of a K-contiguous operand, whole 16-byte pieces of
-    // an M/N-contiguous one (its leading dimension covers them)
     k.M = M;
     k.N = N;
     k.tiles_m = (uint32_t)ceil_div(M, 128);  // (general kernel; the tuned kernels set their own below)
     k.tiles_n = (uint32_t)ceil_div(N, 128);
+    // what an edge kernel may fetch: all rows of a K-contiguous operand, whole 16-byte pieces of
+    // an M/N-contiguous one (its leading dimension covers them)
     k.a_lim = ma == 'k' ? M : (M + P - 1) / P * P;
     k.b_lim = mb == 'k' ? N : (N + P - 1) / P * P;
 
     // Tuned kernels. Direct-to-LDS (fp16, fp32): rows of A, B and C 16-byte aligned, operands
     // addressed with 32-bit byte offsets; ragged M, N, K run the "_e" variants (clamped rows,
-    // zero-filled K tail, predicated stores). HCHIP_GEMM_TILE=general|<BM>x<BN> overrides the
-    // tile choice and HCHIP_GEMM_KERNEL=staged selects the register-staged fp16 pipeline
-    // (whole tiles, K % 64 == 0), both for measurements.
+    // zero-filled K tail, predicated stores). For measurements and tests, read at every call:
+    // HCHIP_GEMM_TILE=general|<BM>x<BN> overrides the tile choice, HCHIP_GEMM_KERNEL=
+    // dma|dma2|mi16 the pipeline, =staged selects the register-staged fp16 pipeline (whole
+    // tiles, K % 64 == 0).
     uint32_t bm = 0, bn = 0;
     bool edge = false;
     const char* which = getenv("HCHIP_GEMM_KERNEL");
