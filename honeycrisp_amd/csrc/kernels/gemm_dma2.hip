@@ -1,4 +1,4 @@
-// fp16 and fp32 GEMM for gfx950 with direct global->LDS loads (global_load_lds_dwordx4) and,
+// fp16 and fp32 GEMM for gfx950 with direct global->LDS loads (buffer_load_dwordx4 ... lds) and,
 // for fp16 operands that are contiguous along M/N, transposing LDS reads
 // (ds_read_b64_tr_b16). Block tile BM x BN, 4 waves 2 x 2, fp32 accumulate with
 // v_mfma_f32_32x32x16_f16 / v_mfma_f32_32x32x2_f32. No operand passes through VGPRs on its
@@ -53,7 +53,6 @@ typedef uint32_t Chunk __attribute__((ext_vector_type(4)));  // 16 bytes = 8 hal
 enum { DMA_K = 0, DMA_MN = 1 };
 
 #define LDS_AS __attribute__((address_space(3)))
-#define GLOBAL_AS __attribute__((address_space(1)))
 
 __device__ __forceinline__ uint32_t swz_k(uint32_t row) { return row & 7u; }
 __device__ __forceinline__ uint32_t swz_mn(uint32_t k) { return (((k & 7u) ^ (((k >> 3) & 1u) << 2)) << 1); }
@@ -169,20 +168,21 @@ template <typename T, int ROWS, int MODE> struct DmaOperand {
   }
 
   // DMA instruction i of this wave for the K-slice starting at k0: 1 KiB into `region`.
-  // Edge kernels (kend != 0): pieces at k >= kend come from `zeros` (16 zero bytes) instead,
-  // so the ragged last slice contributes nothing.
-  __device__ __forceinline__ void dma(int i, const T* base, uint32_t k0, char* region, uint32_t kend = 0,
-                                      const void* zeros = nullptr) const {
+  // A buffer load: the descriptor (base of the operand, no stride, range 2^32 - 16 bytes) lives
+  // in scalar registers, the lane offset goes in as it is and the K offset as the scalar
+  // offset, so no vector or scalar address arithmetic stands in front of the load. The host
+  // keeps operands of this kernel below 4 GiB.
+  // Edge kernels (kend != 0): lanes whose piece lies at k >= kend pass an offset beyond the
+  // descriptor's range, which reads as zero, so the ragged last slice contributes nothing.
+  __device__ __forceinline__ void dma(int i, const T* base, uint32_t k0, char* region, uint32_t kend = 0) const {
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    // The empty asm keeps the zero-extension of the lane offset next to the load, so that the
-    // load takes the form "scalar base + 32-bit lane offset" with no vector add in front of it.
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, 0xfffffff0u, 0x00020000);
     uint32_t off = goff[i];
-    asm volatile("" : "+v"(off));
-    const char* src = (const char*)base + (size_t)k0 * kstride + off;
     if (kend != 0 && k0 + 128 / ES > kend) {  // wave-uniform
-      if (k0 + klocal(i) >= kend) src = (const char*)zeros;
+      if (k0 + klocal(i) >= kend) off = 0xfffffff0u;
     }
-    __builtin_amdgcn_global_load_lds((const GLOBAL_AS void*)src, (LDS_AS void*)(region + (wave * NI + i) * 1024), 16, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (LDS_AS void*)(region + (wave * NI + i) * 1024), 16, off,
+                                             k0 * kstride, 0, 0);
   }
 
   // Read number u of sub-step s into the operand registers of tile u (DMA_K), half u%2 of
@@ -274,8 +274,8 @@ __device__ __forceinline__ void gemm_dma2_impl(const hck_gemm_args& p, char* lds
   };
   // unit u of the DMA of the K-slice starting at k0
   auto dma_unit = [&](int u, uint32_t k0, char* stage) {
-    if (u < OpA::NI) oa.dma(u, A, k0, stage, kend, p.zeros);
-    else if (u < NDMA) ob.dma(u - OpA::NI, B, k0, stage + A_BYTES, kend, p.zeros);
+    if (u < OpA::NI) oa.dma(u, A, k0, stage, kend);
+    else if (u < NDMA) ob.dma(u - OpA::NI, B, k0, stage + A_BYTES, kend);
   };
   // MFMA t of a sub-step; operands swapped (B first) so that a lane holds four consecutive
   // n for one m (see the epilogue).
