@@ -62,7 +62,6 @@ struct hc_ctx {
   std::unordered_map<void*, size_t> live;
   size_t bytes_in_use = 0, bytes_cached = 0;
   hipDeviceProp_t props;
-  void* zeros = nullptr;                              // 256 zero bytes (GEMM edge kernels)
   hc_graph* capturing = nullptr;                      // the recording in progress, if any
   std::unordered_map<void*, hc_graph*> block_owner;   // blocks reserved for a graph
   std::vector<hc_graph*> graphs;
@@ -152,11 +151,6 @@ extern "C" int hc_init(int device, hc_ctx** out) {
   if (s == HC_OK) s = load_image(ctx, hc_image_gemm_dma, hc_image_gemm_dma_end, "gemm_dma");
   if (s == HC_OK) s = load_image(ctx, hc_image_gemm_dma2, hc_image_gemm_dma2_end, "gemm_dma2");
   if (s == HC_OK) s = load_image(ctx, hc_image_gemm_mi16, hc_image_gemm_mi16_end, "gemm_mi16");
-  if (s == HC_OK) {
-    hipError_t e = hipMalloc(&ctx->zeros, 256);
-    if (e == hipSuccess) e = hipMemset(ctx->zeros, 0, 256);
-    if (e != hipSuccess) s = hip_fail(e, "zero buffer");
-  }
   if (s != HC_OK) {
     hc_shutdown(ctx);
     return s;
@@ -185,7 +179,6 @@ extern "C" void hc_shutdown(hc_ctx* ctx) {
   for (auto& kv : ctx->free_blocks)
     for (void* p : kv.second) (void)hipFree(p);
   for (auto& kv : ctx->live) (void)hipFree(kv.first);
-  if (ctx->zeros) (void)hipFree(ctx->zeros);
   for (hipModule_t m : ctx->modules) (void)hipModuleUnload(m);
   if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
   delete ctx;
@@ -2111,7 +2104,6 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
     if (bm != 0) {
       k.tiles_m = (uint32_t)ceil_div(M, bm);
       k.tiles_n = (uint32_t)ceil_div(N, bn);
-      k.zeros = ctx->zeros;
       if (dma && !getenv("HCHIP_GEMM_BAND")) {
         // largest XCD rectangle whose super-block (4 x 2 XCDs) divides the tile grid
         static const uint32_t shapes[][2] = {{4, 8}, {2, 4}, {1, 2}};

@@ -250,7 +250,6 @@ typedef struct {
    * (8/xcd_gn * xcd_sm) x (xcd_gn * xcd_sn) tiles, visited one after the other; inside one,
    * the 8 XCDs form an (8/xcd_gn) x xcd_gn grid and each owns xcd_sm x xcd_sn tiles. */
   uint32_t xcd_gn, xcd_sm, xcd_sn;
-  const void* zeros; /* 16 zero bytes in device memory (edge kernels: source of the K tail) */
   /* edge kernels: rows (K-contiguous operand) or elements of a k-row (M/N-contiguous operand,
    * a multiple of 16 bytes) that may be fetched; anything beyond is clamped to the last one */
   uint32_t a_lim, b_lim;

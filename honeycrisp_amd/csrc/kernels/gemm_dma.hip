@@ -1,4 +1,4 @@
-// fp16 and fp32 GEMM for gfx950 with direct global->LDS loads (global_load_lds_dwordx4) and,
+// fp16 and fp32 GEMM for gfx950 with direct global->LDS loads (buffer_load_dwordx4 ... lds) and,
 // for fp16 operands that are contiguous along M/N, transposing LDS reads
 // (ds_read_b64_tr_b16). Block tile BM x BN, 4 waves 2 x 2, fp32 accumulate with
 // v_mfma_f32_32x32x16_f16 / v_mfma_f32_32x32x2_f32, whole tiles only. No operand passes
@@ -40,18 +40,6 @@
 // LDS access names its stage statically.
 #include "common.hip.h"
 
-// Measurement switches (never set in the shipped build): bit0 no DMA in the K loop, bit1 no
-// wait/barrier, bit2 no LDS reads in the K loop, bit3 every K-step fetches slice 0 again, bit4
-// only every other DMA instruction, bit5 every DMA instruction fetches the same 1 KiB,
-// bit6 / bit7 fetch A only, as pairs of adjacent 64-byte pieces / as single pieces, bit8
-// K-contiguous operands are fetched as whole 128-byte lines (half of the rows per K-step). Results are wrong with any bit set.
-#ifndef HC_EXP
-#define HC_EXP 0
-#endif
-// cache-policy bits of the DMA loads (0 = default policy)
-#ifndef HC_DMA_AUX
-#define HC_DMA_AUX 0
-#endif
 #ifndef HC_READS_PER_SLOT
 #define HC_READS_PER_SLOT 0
 #endif
@@ -65,7 +53,6 @@ typedef uint32_t Chunk __attribute__((ext_vector_type(4)));  // 16 bytes = 8 hal
 enum { DMA_K = 0, DMA_MN = 1 };
 
 #define LDS_AS __attribute__((address_space(3)))
-#define GLOBAL_AS __attribute__((address_space(1)))
 
 __device__ __forceinline__ uint32_t swz_k(uint32_t row) { return ((row >> 1) & 3u) ^ ((row >> 3) & 1u); }
 __device__ __forceinline__ uint32_t swz_mn(uint32_t k) { return (((k & 7u) ^ (((k >> 3) & 1u) << 2)) << 1); }
@@ -100,7 +87,6 @@ template <typename T, int ROWS, int MODE> struct DmaOperand {
 
   uint32_t goff[NI];     // byte offset of this lane's 16-byte piece for DMA instruction i (k = 0)
   uint32_t kstride;      // bytes per unit of k
-  uint32_t half_rows = 0; // measurement builds only
   uint32_t raddr[NADDR]; // byte offsets (inside the operand's LDS region) of the MFMA operand reads
 
   // `limit` (edge kernels): extent of this operand along M / N. Rows or 16-byte pieces past it
@@ -117,10 +103,6 @@ template <typename T, int ROWS, int MODE> struct DmaOperand {
         uint32_t grow = r0 + row;
         if (limit && grow >= limit) grow = limit - 1;
         goff[i] = grow * rs * ES + c * 16;
-        if (HC_EXP & 256) {  // whole 128-byte lines: 8 lanes per row, half of the rows per K-step
-          goff[i] = (r0 + (wave * NI + i) * 8 + lane / 8) * rs * ES + (lane % 8) * 16;
-          half_rows = (ROWS / 2) * rs * ES;
-        }
       }
       const uint32_t lrow = lane & 31, lgrp = lane >> 5;
 #pragma unroll
@@ -186,25 +168,21 @@ template <typename T, int ROWS, int MODE> struct DmaOperand {
   }
 
   // DMA instruction i of this wave for the K-slice starting at k0: 1 KiB into `region`.
-  // Edge kernels (kend != 0): pieces at k >= kend come from `zeros` (16 zero bytes) instead,
-  // so the ragged last slice contributes nothing.
-  __device__ __forceinline__ void dma(int i, const T* base, uint32_t k0, char* region, uint32_t kend = 0,
-                                      const void* zeros = nullptr) const {
+  // A buffer load: the descriptor (base of the operand, no stride, range 2^32 - 16 bytes) lives
+  // in scalar registers, the lane offset goes in as it is and the K offset as the scalar
+  // offset, so no vector or scalar address arithmetic stands in front of the load. The host
+  // keeps operands of this kernel below 4 GiB.
+  // Edge kernels (kend != 0): lanes whose piece lies at k >= kend pass an offset beyond the
+  // descriptor's range, which reads as zero, so the ragged last slice contributes nothing.
+  __device__ __forceinline__ void dma(int i, const T* base, uint32_t k0, char* region, uint32_t kend = 0) const {
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    // The empty asm keeps the zero-extension of the lane offset next to the load, so that the
-    // load takes the form "scalar base + 32-bit lane offset" with no vector add in front of it.
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, 0xfffffff0u, 0x00020000);
     uint32_t off = goff[i];
-    if ((HC_EXP & 256) && MODE == DMA_K) {
-      const uint32_t slice = k0 / (64 / ES);
-      off += (slice & 1) * half_rows;
-      k0 = (slice & ~1u) * (64 / ES);
-    }
-    asm volatile("" : "+v"(off));
-    const char* src = (const char*)base + (size_t)k0 * kstride + off;
     if (kend != 0 && k0 + 64 / ES > kend) {  // wave-uniform
-      if (k0 + klocal(i) >= kend) src = (const char*)zeros;
+      if (k0 + klocal(i) >= kend) off = 0xfffffff0u;
     }
-    __builtin_amdgcn_global_load_lds((const GLOBAL_AS void*)src, (LDS_AS void*)(region + (wave * NI + i) * 1024), 16, 0, HC_DMA_AUX);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (LDS_AS void*)(region + (wave * NI + i) * 1024), 16, off,
+                                             k0 * kstride, 0, 0);
   }
 
   // Read number u of sub-step s into the operand registers of tile u (DMA_K), half u%2 of
@@ -288,35 +266,13 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
   };
   // unit u of the operand reads of a sub-step: B's reads first, then A's
   auto read_unit = [&](Frags& f, const char* stage, int s, int u) {
-    if (HC_EXP & 4) return;
     if (u < OpB::READS) ob.read(u, s, stage + A_BYTES, f.b);
     else if (u < READS) oa.read(u - OpB::READS, s, stage, f.a);
   };
   // unit u of the DMA of the K-slice starting at k0
-  auto dma_unit = [&](int u, uint32_t k0, char* stage, bool in_loop = false) {
-    if ((HC_EXP & 1) && in_loop) return;
-    if ((HC_EXP & 16) && in_loop && (u & 1)) return;
-    if ((HC_EXP & 8) && in_loop) k0 = 0;
-    if ((HC_EXP & 64) && in_loop) {  // A only, both 64-byte halves of a 128-byte line back to back
-      const int q = u >= HALF ? u - HALF : u + HALF;
-      if (q & 1) return;
-      const uint32_t kb = (k0 / (2 * BK)) * (2 * BK);
-      oa.dma((q / 2) % OpA::NI, A, kb, stage, kend, p.zeros);
-      oa.dma((q / 2) % OpA::NI, A, kb + BK, stage, kend, p.zeros);
-      return;
-    }
-    if ((HC_EXP & 128) && in_loop) {  // control for bit6: A only, one 64-byte half per instruction
-      const int q = u >= HALF ? u - HALF : u + HALF;
-      oa.dma(q % OpA::NI, A, k0, stage, kend, p.zeros);
-      return;
-    }
-    if ((HC_EXP & 32) && in_loop) {  // every instruction fetches the same 1 KiB: first-level cache hits
-      if (u < OpA::NI) oa.dma(0, A, 0, stage + u * 1024, kend, p.zeros);
-      else if (u < NDMA) ob.dma(0, B, 0, stage + A_BYTES + (u - OpA::NI) * 1024, kend, p.zeros);
-      return;
-    }
-    if (u < OpA::NI) oa.dma(u, A, k0, stage, kend, p.zeros);
-    else if (u < NDMA) ob.dma(u - OpA::NI, B, k0, stage + A_BYTES, kend, p.zeros);
+  auto dma_unit = [&](int u, uint32_t k0, char* stage) {
+    if (u < OpA::NI) oa.dma(u, A, k0, stage, kend);
+    else if (u < NDMA) ob.dma(u - OpA::NI, B, k0, stage + A_BYTES, kend);
   };
   // MFMA t of a sub-step; operands swapped (B first) so that a lane holds four consecutive
   // n for one m (see the epilogue).
@@ -353,34 +309,32 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int t = 0; t < SLOTS; t++) {  // sub-step 0
-      if (t % DSTRIDE == 0 && HALF + t / DSTRIDE < NDMA) dma_unit(HALF + t / DSTRIDE, k3, prev, true);
+      if (t % DSTRIDE == 0 && HALF + t / DSTRIDE < NDMA) dma_unit(HALF + t / DSTRIDE, k3, prev);
 #pragma unroll
       for (int e = 0; e < RPS; e++) read_unit(f1, cur, 1, t * RPS + e);
       mma_one(f0, t);
       __builtin_amdgcn_sched_barrier(0);
     }
-    if (!(HC_EXP & 2)) {
 #ifdef HC_PROBE_WAITS
-      const uint64_t w0 = __builtin_readcyclecounter();
+    const uint64_t w0 = __builtin_readcyclecounter();
 #ifdef HC_PROBE_SLACK
-      wait_dma<HC_PROBE_SLACK>();  // fewer DMA instructions left in flight: less time to land
+    wait_dma<HC_PROBE_SLACK>();  // fewer DMA instructions left in flight: less time to land
 #else
-      wait_dma<2 * NDMA>();
+    wait_dma<2 * NDMA>();
 #endif
-      const uint64_t w1 = __builtin_readcyclecounter();
-      lds_barrier();
-      const uint64_t w2 = __builtin_readcyclecounter();
-      probe_wait_dma += w1 - w0;
-      probe_wait_bar += w2 - w1;
+    const uint64_t w1 = __builtin_readcyclecounter();
+    lds_barrier();
+    const uint64_t w2 = __builtin_readcyclecounter();
+    probe_wait_dma += w1 - w0;
+    probe_wait_bar += w2 - w1;
 #else
-      wait_dma<2 * NDMA>();  // K-step j+1 of this wave has landed ...
-      lds_barrier();         // ... and everybody's; nobody reads cur any more
+    wait_dma<2 * NDMA>();  // K-step j+1 of this wave has landed ...
+    lds_barrier();         // ... and everybody's; nobody reads cur any more
 #endif
-    }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int t = 0; t < SLOTS; t++) {  // sub-step 1
-      if (t % DSTRIDE == 0 && t / DSTRIDE < HALF) dma_unit(t / DSTRIDE, k4, cur, true);
+      if (t % DSTRIDE == 0 && t / DSTRIDE < HALF) dma_unit(t / DSTRIDE, k4, cur);
 #pragma unroll
       for (int e = 0; e < RPS; e++) read_unit(f0, nxt, 0, t * RPS + e);
       mma_one(f1, t);

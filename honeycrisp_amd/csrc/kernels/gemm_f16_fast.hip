@@ -32,12 +32,6 @@ typedef uint32_t Chunk __attribute__((ext_vector_type(4)));  // 16 bytes = 8 hal
 
 enum { FAST_LOAD_K = 0, FAST_LOAD_MN = 1 };
 
-// Measurement switch (never set in a product build): bit 0 drops the global loads of the
-// main loop, bit 1 the LDS stores, bit 2 the LDS operand reads.
-#ifndef HC_EXP
-#define HC_EXP 0
-#endif
-
 __device__ __forceinline__ uint32_t swz(uint32_t row) { return (row ^ (row >> 3)) & 7u; }
 
 // One operand's share of a K-step in registers: ROWS x 128 bytes / 256 lanes = ROWS/32 chunks.
@@ -161,7 +155,6 @@ __device__ __forceinline__ void gemm_fast_impl(const hck_gemm_args& p, char* lds
   }
   // one operand read: index q < NT is B tile q, otherwise A tile q - NT
   auto read_one = [&](Frags<MT, NT>& f, const char* stage, int s, int q) {
-    if ((HC_EXP & 4) && (s != 0 || stage != lds)) return;
     const uint32_t c = 2 * s + lgrp;
     if (q < NT)
       f.b[q] = *reinterpret_cast<const Chunk*>(stage + brow[q] + ((c ^ bsw[q]) * 16));
@@ -181,12 +174,10 @@ __device__ __forceinline__ void gemm_fast_impl(const hck_gemm_args& p, char* lds
   oa.init(A, p.a_rs, p.a_cs, m0);
   ob.init(B, p.b_cs, p.b_rs, n0);
   auto load_unit = [&](int u, uint32_t k0) {
-    if ((HC_EXP & 1) && k0 > 64) return;
     if (u < OpA::N) oa.load(u, k0);
     else if (u < NLOAD) ob.load(u - OpA::N, k0);
   };
   auto store_unit = [&](int u, char* stage) {
-    if ((HC_EXP & 2) && stage != lds) return;
     if (u < OpA::STORES) oa.store(u, stage);
     else if (u < NSTORE) ob.store(u - OpA::STORES, stage + BM * 128);
   };
