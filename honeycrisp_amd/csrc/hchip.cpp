@@ -2032,12 +2032,16 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
       auto whole = [&](uint32_t tm, uint32_t tn) { return M % tm == 0 && N % tn == 0 && K % slice == 0; };
       // largest tile first; the direct-to-LDS kernels also come in narrow shapes
       static const uint32_t tiles[][2] = {{256, 256}, {256, 128}, {128, 128}, {256, 64}, {128, 64}, {64, 64}};
+      // (only the 16x16x32 pipeline has these)
+      static const uint32_t tiles192[][2] = {{256, 192}, {192, 256}, {192, 192}};
       const uint64_t cus = (uint64_t)ctx->props.multiProcessorCount;
       if (force && *force) {
         unsigned fm = 0, fn = 0;
         if (sscanf(force, "%ux%u", &fm, &fn) == 2 && (dma || whole(fm, fn))) {
           bool known = false;
           for (auto& t : tiles) known = known || (t[0] == fm && t[1] == fn);
+          if (mi16)
+            for (auto& t : tiles192) known = known || (t[0] == fm && t[1] == fn);
           if (known) {
             bm = fm;
             bn = fn;
@@ -2074,19 +2078,37 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
           }
         }
       }
-      // Long fp16 products are limited by power, not by idle CUs: CUs that sit out leave the busy
-      // ones a higher clock, so large tiles on part of the device beat small tiles on all of it
-      // well before the large tiles fill it (measured: 144 tiles of 256 x 256 on 256 CUs run
-      // at 58 % of the full-device rate, 196 at 72 %).
+      // Long fp16 products that can keep at least half of the device busy run on the 16x16x32
+      // pipeline; its tile is the one with the least estimated time = rounds of blocks x tile
+      // area / rate. Rates: full device, relative to 256 x 256, times 0.88 for the edge kernels
+      // of a ragged product. A last round that occupies a fraction f of the CUs counts as
+      // max(f^0.25, 0.5) of a round: such products are limited by power, so the busy CUs of a
+      // partly idle device get a higher clock (measured: 144 tiles of 256 x 256 on 256 CUs reach
+      // 58 % (K = 2048) to 72 % (K = 4096) of the full-device rate, 33 tiles take 0.58 of the
+      // time of 256). The constants were fitted to a sweep of 18 shapes x 3 layouts x 6 tiles;
+      // the model's pick is within 5 % of the best tile on all but two of them (14 %).
+      bool model_mi16 = false;
       if (!(force && *force) && !which && dma && dtype == HC_F16 && K >= 1024) {
         const uint64_t t256 = ceil_div(M, 256) * ceil_div(N, 256) * (uint64_t)batch;
         const uint64_t t128 = ceil_div(M, 128) * ceil_div(N, 128) * (uint64_t)batch;
-        if (2 * t256 >= cus && t256 < cus) {
-          bm = bn = 256;
-          dma2 = mi16 = true;
-        } else if (t256 < cus && 2 * t128 >= 3 * cus) {
-          bm = bn = 128;
-          dma2 = mi16 = true;
+        if (2 * t256 >= cus || 2 * t128 >= 3 * cus) {
+          static const struct { uint32_t bm, bn; double rate; } cand[] = {
+              {256, 256, 1.0}, {256, 192, 0.9}, {192, 256, 0.9}, {192, 192, 0.82}, {256, 128, 0.76}, {128, 128, 0.6}};
+          double best = 0.0;
+          for (auto& c : cand) {
+            const uint64_t blocks = ceil_div(M, c.bm) * ceil_div(N, c.bn) * (uint64_t)batch;
+            const uint64_t rem = blocks % cus;
+            double rounds = (double)(blocks / cus);
+            if (rem != 0) rounds += std::max(pow((double)rem / (double)cus, 0.25), 0.5);
+            const bool ragged = M % c.bm != 0 || N % c.bn != 0 || K % 64 != 0;
+            const double cost = rounds * c.bm * c.bn / (c.rate * (ragged ? 0.88 : 1.0));
+            if (best == 0.0 || cost < best) {
+              best = cost;
+              bm = c.bm;
+              bn = c.bn;
+            }
+          }
+          dma2 = mi16 = model_mi16 = true;
         }
       }
       if (bm != 0 && dma) {
@@ -2094,9 +2116,9 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
         // (whole cache lines only help an operand that is contiguous along K: TN products stay
         // with the four-stage ring)
         const bool k_contig = ma == 'k' || mb == 'k';
-        if (!which && k_contig && (uint64_t)K * el >= 2048 && ((bm == 256 && bn == 256) || blocks >= 2 * cus))
+        if (!which && !model_mi16 && k_contig && (uint64_t)K * el >= 2048 && ((bm == 256 && bn == 256) || blocks >= 2 * cus))
           dma2 = true;
-        if (!which && dtype == HC_F16 && K >= 1024 && bm == 256 && bn == 256 && blocks >= cus) dma2 = mi16 = true;
+
         if (dma2) slice = (uint32_t)(128 / el);
       }
       if (bm != 0) edge = !whole(bm, bn);

@@ -58,86 +58,52 @@ template <int N> __device__ __forceinline__ void wait_dma() {
   __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
 }
 
-// One operand of the block tile: where its DMA lanes fetch from and where a wave's MFMA
-// operand reads land.
-template <typename T, int ROWS, int MODE> struct DmaOperand {
-  static constexpr int ES = sizeof(T);
-  static constexpr bool F32 = ES == 4;
-  static constexpr int NI = ROWS / 32;                        // DMA instructions per wave and K-step
-  static constexpr int TILES = ROWS / 64;                     // MFMA tiles per wave along this operand
-  // LDS reads per sub-step
-  static constexpr int READS = MODE == DMA_K ? TILES : (F32 ? 4 * TILES : 2 * TILES);
-  static constexpr int NADDR = MODE == DMA_K ? TILES * 4 : TILES * 2;
-  static constexpr int ROWB = ROWS * ES;                      // bytes per k-row (DMA_MN layout)
-  static constexpr int BYTES = ROWS * 128;                    // per stage
+// DMA side of one operand of the block tile: which 16-byte piece of global memory each lane
+// fetches and where it lands. ROWS (the tile's extent along M or N) is a multiple of 64.
+//   DMA_K : LDS rows of 128 bytes (64 k of one row), chunk c of row r in slot c ^ (r & 7);
+//           one instruction covers 8 rows.
+//   DMA_MN: LDS [64 k-rows][ROWS halfs], 16-byte slot u of k-row k holds columns
+//           8 (u ^ swz(k)) .. +7; the instructions of a K-slice cover its 8 ROWS pieces in
+//           order, 64 each (a k-row need not be a whole number of instructions).
+template <int ROWS, int MODE> struct DmaOperand {
+  static constexpr int NI = ROWS / 32;           // DMA instructions per wave and K-step
+  static constexpr int ROWB = ROWS * 2;          // bytes per k-row (DMA_MN layout)
+  static constexpr int BYTES = ROWS * 128;       // per stage
+  static constexpr uint32_t SLOTS = ROWS / 8;    // 16-byte slots per k-row (DMA_MN layout)
+  // the swizzle permutes slots inside aligned groups of SWZ_MASK + 1 (a divisor of SLOTS)
+  static constexpr uint32_t SWZ_MASK = (SLOTS & (SLOTS - 1)) == 0 ? SLOTS - 1 : 7;
+  static_assert(ROWS % 64 == 0 && SLOTS % (SWZ_MASK + 1) == 0, "unsupported tile extent");
 
   uint32_t goff[NI];     // byte offset of this lane's 16-byte piece for DMA instruction i (k = 0)
   uint32_t kstride;      // bytes per unit of k
-  uint32_t raddr[NADDR]; // byte offsets (inside the operand's LDS region) of the MFMA operand reads
+
+  __device__ __forceinline__ static uint32_t mn_swz(uint32_t k) { return swz_mn(k) & SWZ_MASK; }
 
   // `limit` (edge kernels): extent of this operand along M / N. Rows or 16-byte pieces past it
   // are fetched from the last valid row / piece instead: they only feed outputs that are
   // never stored. 0 = no clamping.
-  __device__ __forceinline__ void init(uint32_t rs, uint32_t cs, uint32_t r0, uint32_t woff, uint32_t limit) {
+  __device__ __forceinline__ void init(uint32_t rs, uint32_t cs, uint32_t r0, uint32_t limit) {
     const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     if (MODE == DMA_K) {
-      kstride = ES;
+      kstride = 2;
 #pragma unroll
       for (int i = 0; i < NI; i++) {
         const uint32_t row = (wave * NI + i) * 8 + lane / 8;
         const uint32_t c = (lane % 8) ^ swz_k(row);
         uint32_t grow = r0 + row;
         if (limit && grow >= limit) grow = limit - 1;
-        goff[i] = grow * rs * ES + c * 16;
-      }
-      const uint32_t lrow = lane & 31, lgrp = lane >> 5;
-#pragma unroll
-      for (int q = 0; q < TILES; q++) {
-        const uint32_t r = woff + q * 32 + lrow;
-#pragma unroll
-        for (int s = 0; s < 4; s++) raddr[q * 4 + s] = r * 128 + (((2 * s + lgrp) ^ swz_k(r)) * 16);
-      }
-    } else if (F32) {
-      // [32 k][ROWS floats]; the 128-byte halves of every 256 bytes swap places in k-rows
-      // with bit 2 set: an MFMA operand read touches rows k and k + 4, 32 floats of each
-      constexpr uint32_t KPI = 1024 / ROWB;   // k-rows per DMA instruction
-      constexpr uint32_t PIECES = ROWB / 16;  // 16-byte pieces per k-row
-      kstride = cs * ES;
-#pragma unroll
-      for (int i = 0; i < NI; i++) {
-        const uint32_t krow = (wave * NI + i) * KPI + lane / PIECES;
-        const uint32_t piece = (lane % PIECES) ^ (((krow >> 2) & 1u) << 3);
-        uint32_t col = r0 + piece * 4;
-        if (limit && col + 4 > limit) col = limit - 4;
-        goff[i] = (krow * cs + col) * ES;
-      }
-      const uint32_t lrow = lane & 31, lgrp = lane >> 5;
-#pragma unroll
-      for (int q = 0; q < TILES; q++) {
-        const uint32_t n = woff + q * 32 + lrow;  // k = 4 * lgrp + e + 8 * s, e and s as immediates
-        raddr[q] = 4 * lgrp * ROWB + ((n ^ (lgrp << 5)) * 4);
+        goff[i] = grow * rs * 2 + c * 16;
       }
     } else {
-      constexpr int KPI = 512 / ROWS;       // k-rows per DMA instruction
-      constexpr uint32_t SLOTS_PER_ROW = ROWS / 8;
       kstride = cs * 2;
 #pragma unroll
       for (int i = 0; i < NI; i++) {
-        const uint32_t krow = (wave * NI + i) * KPI + lane / SLOTS_PER_ROW;
-        const uint32_t slot = (lane % SLOTS_PER_ROW) ^ (swz_mn(krow) & (SLOTS_PER_ROW - 1));
+        const uint32_t piece = (wave * NI + i) * 64 + lane;
+        const uint32_t krow = piece / SLOTS;
+        const uint32_t slot = (piece % SLOTS) ^ mn_swz(krow);
         uint32_t col = r0 + slot * 8;
         if (limit && col + 8 > limit) col = limit - 8;
         goff[i] = (krow * cs + col) * 2;
-      }
-      const uint32_t j = lane >> 4, r16 = lane & 15;
-#pragma unroll
-      for (int q = 0; q < TILES; q++) {
-        const uint32_t m = woff + q * 32 + 16 * (j & 1) + 4 * (r16 & 3);
-#pragma unroll
-        for (int h = 0; h < 2; h++) {
-          const uint32_t k = 8 * (j >> 1) + 4 * h + (r16 >> 2);  // + 16 * s as an immediate offset
-          raddr[q * 2 + h] = k * ROWB + (((m >> 3) ^ (swz_mn(k) & (ROWS / 8 - 1))) * 16) + (m & 7) * 2;
-        }
       }
     }
   }
@@ -147,10 +113,9 @@ template <typename T, int ROWS, int MODE> struct DmaOperand {
     const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     if (MODE == DMA_K) {
       const uint32_t row = (wave * NI + i) * 8 + lane / 8;
-      return ((lane % 8) ^ swz_k(row)) * (16 / ES);
+      return ((lane % 8) ^ swz_k(row)) * 8;
     }
-    constexpr uint32_t PER_ROW = ROWB / 16, KPI = 1024 / ROWB;
-    return (wave * NI + i) * KPI + lane / PER_ROW;
+    return ((wave * NI + i) * 64 + lane) / SLOTS;
   }
 
   // DMA instruction i of this wave for the K-slice starting at k0: 1 KiB into `region`.
@@ -160,35 +125,15 @@ template <typename T, int ROWS, int MODE> struct DmaOperand {
   // keeps operands of this kernel below 4 GiB.
   // Edge kernels (kend != 0): lanes whose piece lies at k >= kend pass an offset beyond the
   // descriptor's range, which reads as zero, so the ragged last slice contributes nothing.
-  __device__ __forceinline__ void dma(int i, const T* base, uint32_t k0, char* region, uint32_t kend = 0) const {
+  __device__ __forceinline__ void dma(int i, const half_t* base, uint32_t k0, char* region, uint32_t kend = 0) const {
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, 0xfffffff0u, 0x00020000);
     uint32_t off = goff[i];
-    if (kend != 0 && k0 + 128 / ES > kend) {  // wave-uniform
+    if (kend != 0 && k0 + 64 > kend) {  // wave-uniform
       if (k0 + klocal(i) >= kend) off = 0xfffffff0u;
     }
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (LDS_AS void*)(region + (wave * NI + i) * 1024), 16, off,
                                              k0 * kstride, 0, 0);
-  }
-
-  // Read number u of sub-step s into the operand registers of tile u (DMA_K), half u%2 of
-  // tile u/2 (DMA_MN, fp16) or element u%4 of tile u/4 (DMA_MN, fp32).
-  __device__ __forceinline__ void read(int u, int s, const char* region, Chunk* frag) const {
-    if (MODE == DMA_K) {
-      frag[u] = *reinterpret_cast<const Chunk*>(region + raddr[u * 4 + s]);
-    } else if (F32) {
-      const int q = u / 4, e = u % 4;
-      frag[q][e] = *reinterpret_cast<const uint32_t*>(region + raddr[q] + (8 * s + e) * ROWB);
-    } else {
-      const int q = u / 2, h = u % 2;
-      typedef short short4v __attribute__((ext_vector_type(4)));
-      const short4v v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-          (LDS_AS short4v*)(region + raddr[q * 2 + h] + s * 16 * ROWB));
-      typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-      const u32x2 w = __builtin_bit_cast(u32x2, v);
-      frag[q][2 * h] = w[0];
-      frag[q][2 * h + 1] = w[1];
-    }
   }
 };
 
@@ -229,7 +174,7 @@ template <int ROWS, int MODE> struct Mi16Reads {
 #pragma unroll
         for (int h = 0; h < 2; h++) {
           const uint32_t k = 8 * grp + 4 * h + (r16 >> 2);
-          raddr[q * 2 + h] = k * ROWB + (((m >> 3) ^ (swz_mn(k) & (ROWS / 8 - 1))) * 16) + (m & 7) * 2;
+          raddr[q * 2 + h] = k * ROWB + (((m >> 3) ^ DmaOperand<ROWS, MODE>::mn_swz(k)) * 16) + (m & 7) * 2;
         }
       }
     }
@@ -256,8 +201,8 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
   typedef half_t T;
   constexpr int MT = BM / 32, NT = BN / 32;  // 16 x 16 tiles per wave
   constexpr int SLOTS = MT * NT;             // MFMAs per sub-step
-  typedef DmaOperand<T, BM, MODE_A> OpA;
-  typedef DmaOperand<T, BN, MODE_B> OpB;
+  typedef DmaOperand<BM, MODE_A> OpA;
+  typedef DmaOperand<BN, MODE_B> OpB;
   typedef Mi16Reads<BM, MODE_A> RdA;
   typedef Mi16Reads<BN, MODE_B> RdB;
   constexpr uint32_t BK = 64;  // halfs per stage
@@ -301,8 +246,8 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
 
   OpA oa;
   OpB ob;
-  oa.init(p.a_rs, p.a_cs, m0, wm, EDGE ? p.a_lim : 0);
-  ob.init(p.b_cs, p.b_rs, n0, wn, EDGE ? p.b_lim : 0);
+  oa.init(p.a_rs, p.a_cs, m0, EDGE ? p.a_lim : 0);
+  ob.init(p.b_cs, p.b_rs, n0, EDGE ? p.b_lim : 0);
   RdA ra;
   RdB rb;
   ra.init(wm);
@@ -426,10 +371,13 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
   // order, so a slab may be overwritten right after its reads.
   lds_barrier();
   char* mine = (wave < 2 ? lds0 : lds1) + (wave & 1) * ((BM + BN) * 64);
-  constexpr uint32_t WN = BN / 2, RB = WN * 2, UNITS = RB / 16, RPI = 64 / UNITS;
+  constexpr uint32_t WN = BN / 2, RB = WN * 2, UNITS = RB / 16;
   constexpr uint32_t SLAB = 32 * RB, NSLAB = (BM + BN) * 64 / SLAB;
-  static_assert(NSLAB >= 1 && UNITS <= 64 && MT % 2 == 0, "a slab is two rows of tiles and must fit half a stage");
-  auto unit_swz = [&](uint32_t r) { return (RB >= 256 ? r : r * RB / 256) & (UNITS - 1); };
+  static_assert(NSLAB >= 1 && (32 * UNITS) % 64 == 0 && MT % 2 == 0, "a slab is two rows of tiles and must fit half a stage");
+  // (the swizzle stays inside aligned groups of USWZ + 1 units, a divisor of UNITS)
+  constexpr uint32_t USWZ = (UNITS & (UNITS - 1)) == 0 ? UNITS - 1 : 3;
+  static_assert(UNITS % (USWZ + 1) == 0, "unsupported tile width");
+  auto unit_swz = [&](uint32_t r) { return (RB >= 256 ? r : r * RB / 256) & USWZ; };
   const uint32_t r16 = lane & 15, grp = lane >> 4;
 #pragma unroll
   for (int ii = 0; ii < MT / 2; ii++) {
@@ -448,8 +396,8 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // wave-private region: no barrier needed
 #pragma unroll
-    for (uint32_t it = 0; it < 32 / RPI; it++) {
-      const uint32_t r = it * RPI + lane / UNITS, u = lane % UNITS;
+    for (uint32_t it = 0; it < 32 * UNITS / 64; it++) {
+      const uint32_t piece = it * 64 + lane, r = piece / UNITS, u = piece % UNITS;
       const Chunk v = *reinterpret_cast<const Chunk*>(slab + r * RB + ((u ^ unit_swz(r)) * 16));
       const uint32_t row = m0 + wm + ii * 32 + r, col = n0 + wn + u * 8;
       if (!EDGE || (row < p.M && col < p.N)) *reinterpret_cast<Chunk*>(C + (size_t)row * p.c_rs + col) = v;
@@ -487,6 +435,9 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
   DEF_MI16(BM, BN, m, DMA_MN, k, DMA_K)                                                               \
   DEF_MI16(BM, BN, m, DMA_MN, n, DMA_MN)
 DEF_MI16_TILE(256, 256)
+DEF_MI16_TILE(256, 192)
+DEF_MI16_TILE(192, 256)
+DEF_MI16_TILE(192, 192)
 DEF_MI16_TILE(256, 128)
 DEF_MI16_TILE(128, 128)
 DEF_MI16_TILE(256, 64)

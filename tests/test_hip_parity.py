@@ -127,9 +127,15 @@ def test_matmul_both_pipelines_every_tile(hip_backend, oracle_backend, monkeypat
     ragged (edge kernels: clamped rows, zero-filled K tail) and batched problems, all four layouts."""
     rng = np.random.default_rng(77)
     monkeypatch.setenv("HCHIP_GEMM_KERNEL", pipeline)
-    for tile in ("256x256", "256x128", "128x128", "256x64", "128x64", "64x64"):
+    tiles = ("256x256", "256x128", "128x128", "256x64", "128x64", "64x64")
+    if pipeline == "mi16" and dtype is F16:
+        tiles += ("256x192", "192x256", "192x192")  # (extents that are not powers of two: this pipeline only)
+    for tile in tiles:
         monkeypatch.setenv("HCHIP_GEMM_TILE", tile)
-        for (batch, M, K, N) in [(1, 256, 192, 256), (2, 264, 200, 136), (3, 128, 1024, 64)]:
+        shapes = [(1, 256, 192, 256), (2, 264, 200, 136), (3, 128, 1024, 64)]
+        if "192" in tile:
+            shapes.append((1, 768, 320, 768))  # whole tiles of every 192-extent shape
+        for (batch, M, K, N) in shapes:
             a = rand(rng, (batch, M, K), dtype, 1.0 / K ** 0.5)
             b = rand(rng, (batch, K, N), dtype)
             for transA in (False, True):
@@ -210,15 +216,17 @@ def test_matmul_fp16_4096_against_oracle_slab_and_identity(hip_backend, oracle_b
         assert np.array_equal(Tensor.matmul(eye, False, tb, False, False).numpy(), b)
 
 
-def test_matmul_fp16_large_ragged_against_oracle_slab(hip_backend, oracle_backend):
-    """A product large enough for the host to pick the full-device fp16 kernel, but ragged in M, N
-    and K (edge variant: clamped rows, zero-filled K tail, predicated stores): row slabs against
-    the oracle, the whole result against the general kernel, and nothing written past the edges."""
+@pytest.mark.parametrize("shape", [(4100, 1032, 4104), (3000, 1096, 3016)], ids=lambda s: "x".join(map(str, s)))
+def test_matmul_fp16_large_ragged_against_oracle_slab(hip_backend, oracle_backend, shape):
+    """Products large enough for the host to pick the full-device fp16 kernels (the second one
+    with 192 x 192 tiles), but ragged in M, N and K (edge variants: clamped rows, zero-filled K
+    tail, predicated stores): row slabs against the oracle, the whole result against the general
+    kernel, and nothing written past the edges."""
     rng = np.random.default_rng(12)
-    M, K, N = 4100, 1032, 4104
+    M, K, N = shape
     a = (rng.standard_normal((M, K)) / np.sqrt(K)).astype(np.float16)
     b = rng.standard_normal((K, N)).astype(np.float16)
-    rows = np.r_[0:24, 2040:2064, M - 24:M]
+    rows = np.r_[0:24, M // 2 - 10:M // 2 + 14, M - 24:M]
     with oracle_backend.use():
         want = Tensor.matmul(Tensor(data=a[rows]), False, Tensor(data=b), False, False).numpy()
     with hip_backend.use():
@@ -231,7 +239,7 @@ def test_matmul_fp16_large_ragged_against_oracle_slab(hip_backend, oracle_backen
             del os.environ["HCHIP_GEMM_TILE"]
         assert_close_arrays(general[rows], want, 1e-2, 1e-2)
         for transA, transB in [(False, False), (False, True), (True, False), (True, True)]:
-            print("4100x1032x4104 layout", transA, transB, flush=True)
+            print(shape, "layout", transA, transB, flush=True)
             out = Tensor.matmul(tat if transA else ta, transA, tbt if transB else tb, transB, False).numpy()
             assert out.shape == (M, N)
             assert_close_arrays(out[rows], want, 1e-2, 1e-2)
