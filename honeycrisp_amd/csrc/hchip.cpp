@@ -697,6 +697,8 @@ static int make_bcast(int nops, const hc_strides* const* ops, const void* const*
   *vec = v;
   d->inner_vecs = d->inner / (uint32_t)v;
   d->total_vecs = (uint32_t)(count / (uint64_t)v);
+  hck_fast_div_setup(d->inner_vecs, &d->inner_magic, &d->inner_sh);
+  for (uint32_t k = 0; k < d->n_outer; k++) hck_fast_div_setup(d->outer_shape[k], &d->outer_magic[k], &d->outer_sh[k]);
   return HC_OK;
 }
 

@@ -25,8 +25,22 @@ typedef struct {
   uint32_t outer_shape[HCK_MAX_DIMS - 1];
   uint32_t outer_stride[3][HCK_MAX_DIMS - 1];
   uint32_t inner_stride[3];
+  /* division by inner_vecs and by outer_shape[k] as multiply-high and shifts (hck_fast_div) */
+  uint32_t inner_magic, inner_sh;
+  uint32_t outer_magic[HCK_MAX_DIMS - 1];
+  uint32_t outer_sh[HCK_MAX_DIMS - 1];
   uint32_t pad;
 } hck_bcast;
+
+/* n / d for any 32-bit n with d's precomputed (magic, sh): l = ceil(log2 d),
+ * magic = floor(2^32 (2^l - d) / d) + 1, sh = min(l, 1) | max(l - 1, 0) << 8;
+ * t = high half of magic * n, quotient = (t + ((n - t) >> min(l, 1))) >> max(l - 1, 0). */
+static inline void hck_fast_div_setup(uint32_t d, uint32_t* magic, uint32_t* sh) {
+  uint32_t l = 0;
+  while ((1ull << l) < d) l++;
+  *magic = (uint32_t)(((1ull << 32) * ((1ull << l) - d)) / d + 1);
+  *sh = (l < 1 ? l : 1u) | ((l > 1 ? l - 1 : 0u) << 8);
+}
 
 /* out = a (op) b, broadcast; also compare (bool out) and broadcast copy (a only). */
 typedef struct {

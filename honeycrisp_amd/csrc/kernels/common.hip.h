@@ -3,6 +3,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <type_traits>
 #include <stdint.h>
 
 #include "../kargs.h"
@@ -63,6 +64,43 @@ __device__ __forceinline__ void load_vec(const T* base, uint32_t off, uint32_t s
   }
 }
 
+// The same with the stride known at compile time: S = 1 one 16-byte load, S = 0 one element
+// repeated, S < 0 decided at run time. Kernels branch once on the (wave-uniform) strides of
+// all their operands and run a body whose loads are unconditional, so they issue back to back;
+// with the run-time form the compiler puts a wait for the first operand's load at the join of
+// its two paths, in front of the second operand's load.
+template <typename T, int N, int S>
+__device__ __forceinline__ void load_vec_c(const T* base, uint32_t off, uint32_t stride, T (&dst)[N]) {
+  if (S == 1) {
+    Vec<T, N> t = *reinterpret_cast<const Vec<T, N>*>(base + off);
+#pragma unroll
+    for (int i = 0; i < N; i++) dst[i] = t.v[i];
+  } else if (S == 0) {
+    const T x = base[off];
+#pragma unroll
+    for (int i = 0; i < N; i++) dst[i] = x;
+  } else {
+    load_vec<T, N>(base, off, stride, dst);
+  }
+}
+template <int S> using StrideC = std::integral_constant<int, S>;
+// f(sa, sb) with the inner strides of two operands as StrideC constants: both vectors, one
+// vector and one repeated element, or "run time" for anything else (and for VEC = 1, where
+// every load is a single element anyway).
+template <int VEC, typename F> __device__ __forceinline__ void with_strides2(const uint32_t* s, F&& f) {
+  if (VEC > 1 && s[0] == 1 && s[1] == 1) f(StrideC<1>{}, StrideC<1>{});
+  else if (VEC > 1 && s[0] == 1 && s[1] == 0) f(StrideC<1>{}, StrideC<0>{});
+  else if (VEC > 1 && s[0] == 0 && s[1] == 1) f(StrideC<0>{}, StrideC<1>{});
+  else f(StrideC<-1>{}, StrideC<-1>{});
+}
+// f(s) for NOPS operands that share one constant: all vectors, or "run time".
+template <int VEC, int NOPS, typename F> __device__ __forceinline__ void with_strides_all(const uint32_t* s, F&& f) {
+  bool ones = VEC > 1;
+  for (int o = 0; o < NOPS; o++) ones = ones && s[o] == 1;
+  if (ones) f(StrideC<1>{});
+  else f(StrideC<-1>{});
+}
+
 template <typename T, int N>
 __device__ __forceinline__ void store_vec(T* base, size_t off, const T (&src)[N]) {
   Vec<T, N> t;
@@ -71,19 +109,26 @@ __device__ __forceinline__ void store_vec(T* base, size_t off, const T (&src)[N]
   *reinterpret_cast<Vec<T, N>*>(base + off) = t;
 }
 
+// n / d with the (magic, sh) pair the host derived from d (hck_fast_div_setup): exact for every
+// 32-bit n, five instructions instead of the division sequence.
+__device__ __forceinline__ uint32_t fast_div(uint32_t n, uint32_t magic, uint32_t sh) {
+  const uint32_t t = __umulhi(magic, n);
+  return (t + ((n - t) >> (sh & 0xffu))) >> (sh >> 8);
+}
+
 // Broadcast index map (Broadcast.swift:72-90) for NOPS operands at once: vector number
 // v -> element offsets of the first of VEC inner elements, and the flat output offset.
 template <int NOPS, int VEC>
 __device__ __forceinline__ void bcast_offsets(const hck_bcast& d, uint32_t v, uint32_t (&off)[NOPS],
                                               size_t& out_off) {
-  uint32_t row = v / d.inner_vecs;
+  uint32_t row = fast_div(v, d.inner_magic, d.inner_sh);
   uint32_t col = (v - row * d.inner_vecs) * VEC;
   out_off = (size_t)row * d.inner + col;
 #pragma unroll
   for (int o = 0; o < NOPS; o++) off[o] = col * d.inner_stride[o];
   for (int k = (int)d.n_outer - 1; k >= 0; k--) {
     uint32_t s = d.outer_shape[k];
-    uint32_t q = row / s;
+    uint32_t q = fast_div(row, d.outer_magic[k], d.outer_sh[k]);
     uint32_t r = row - q * s;
 #pragma unroll
     for (int o = 0; o < NOPS; o++) off[o] += r * d.outer_stride[o][k];

@@ -58,12 +58,15 @@ template <typename T, int OP, int VEC> __device__ __forceinline__ void binary_im
   uint32_t off[2];
   size_t o;
   bcast_offsets<2, VEC>(p.d, v, off, o);
-  T a[VEC], b[VEC], r[VEC];
-  load_vec<T, VEC>((const T*)p.a, off[0], p.d.inner_stride[0], a);
-  load_vec<T, VEC>((const T*)p.b, off[1], p.d.inner_stride[1], b);
+  with_strides2<VEC>(p.d.inner_stride, [&](auto sa, auto sb) {
+    T a[VEC], b[VEC], r[VEC];
+    load_vec_c<T, VEC, decltype(sa)::value>((const T*)p.a, off[0], p.d.inner_stride[0], a);
+    load_vec_c<T, VEC, decltype(sb)::value>((const T*)p.b, off[1], p.d.inner_stride[1], b);
+    __builtin_amdgcn_sched_barrier(0);  // every load is issued before the first use of one
 #pragma unroll
-  for (int i = 0; i < VEC; i++) r[i] = from_arith<T>(binop<OP, C>(to_arith(a[i]), to_arith(b[i])));
-  store_vec<T, VEC>((T*)p.out, o, r);
+    for (int i = 0; i < VEC; i++) r[i] = from_arith<T>(binop<OP, C>(to_arith(a[i]), to_arith(b[i])));
+    store_vec<T, VEC>((T*)p.out, o, r);
+  });
 }
 
 // compare(BroadcastData, BroadcastData) (BackendCPU.swift:541-571): bool output.
@@ -73,13 +76,16 @@ template <typename T, int OP, int VEC> __device__ __forceinline__ void compare_i
   uint32_t off[2];
   size_t o;
   bcast_offsets<2, VEC>(p.d, v, off, o);
-  T a[VEC], b[VEC];
-  uint8_t r[VEC];
-  load_vec<T, VEC>((const T*)p.a, off[0], p.d.inner_stride[0], a);
-  load_vec<T, VEC>((const T*)p.b, off[1], p.d.inner_stride[1], b);
+  with_strides2<VEC>(p.d.inner_stride, [&](auto sa, auto sb) {
+    T a[VEC], b[VEC];
+    uint8_t r[VEC];
+    load_vec_c<T, VEC, decltype(sa)::value>((const T*)p.a, off[0], p.d.inner_stride[0], a);
+    load_vec_c<T, VEC, decltype(sb)::value>((const T*)p.b, off[1], p.d.inner_stride[1], b);
+    __builtin_amdgcn_sched_barrier(0);  // every load is issued before the first use of one
 #pragma unroll
-  for (int i = 0; i < VEC; i++) r[i] = cmpop<OP>(to_arith(a[i]), to_arith(b[i])) ? 1 : 0;
-  store_vec<uint8_t, VEC>((uint8_t*)p.out, o, r);
+    for (int i = 0; i < VEC; i++) r[i] = cmpop<OP>(to_arith(a[i]), to_arith(b[i])) ? 1 : 0;
+    store_vec<uint8_t, VEC>((uint8_t*)p.out, o, r);
+  });
 }
 
 // broadcast (BackendCPU.swift:255-265): raw element copy, keyed by element size.
@@ -102,16 +108,20 @@ template <typename T, int MULADD, int VEC> __device__ __forceinline__ void fused
   uint32_t off[3];
   size_t o;
   bcast_offsets<3, VEC>(p.d, v, off, o);
-  T x[VEC], c[VEC], b[VEC], r[VEC];
-  load_vec<T, VEC>((const T*)p.x, off[0], p.d.inner_stride[0], x);
-  load_vec<T, VEC>((const T*)p.y, off[1], p.d.inner_stride[1], c);
-  load_vec<T, VEC>((const T*)p.z, off[2], p.d.inner_stride[2], b);
+  with_strides_all<VEC, 3>(p.d.inner_stride, [&](auto sc) {
+    constexpr int S = decltype(sc)::value;
+    T x[VEC], c[VEC], b[VEC], r[VEC];
+    load_vec_c<T, VEC, S>((const T*)p.x, off[0], p.d.inner_stride[0], x);
+    load_vec_c<T, VEC, S>((const T*)p.y, off[1], p.d.inner_stride[1], c);
+    load_vec_c<T, VEC, S>((const T*)p.z, off[2], p.d.inner_stride[2], b);
+    __builtin_amdgcn_sched_barrier(0);  // every load is issued before the first use of one
 #pragma unroll
-  for (int i = 0; i < VEC; i++) {
-    C xv = to_arith(x[i]), cv = to_arith(c[i]), bv = to_arith(b[i]);
-    r[i] = from_arith<T>(MULADD ? xv * cv + bv : (xv + bv) * cv);
-  }
-  store_vec<T, VEC>((T*)p.out, o, r);
+    for (int i = 0; i < VEC; i++) {
+      C xv = to_arith(x[i]), cv = to_arith(c[i]), bv = to_arith(b[i]);
+      r[i] = from_arith<T>(MULADD ? xv * cv + bv : (xv + bv) * cv);
+    }
+    store_vec<T, VEC>((T*)p.out, o, r);
+  });
 }
 
 // when (BackendCPU.swift:1190-1220): x = bool mask, y/z = branches; raw element copy.
@@ -121,14 +131,18 @@ template <typename T, int VEC> __device__ __forceinline__ void when_impl(const h
   uint32_t off[3];
   size_t o;
   bcast_offsets<3, VEC>(p.d, v, off, o);
-  uint8_t m[VEC];
-  T a[VEC], b[VEC], r[VEC];
-  load_vec<uint8_t, VEC>((const uint8_t*)p.x, off[0], p.d.inner_stride[0], m);
-  load_vec<T, VEC>((const T*)p.y, off[1], p.d.inner_stride[1], a);
-  load_vec<T, VEC>((const T*)p.z, off[2], p.d.inner_stride[2], b);
+  with_strides_all<VEC, 3>(p.d.inner_stride, [&](auto sc) {
+    constexpr int S = decltype(sc)::value;
+    uint8_t m[VEC];
+    T a[VEC], b[VEC], r[VEC];
+    load_vec_c<uint8_t, VEC, S>((const uint8_t*)p.x, off[0], p.d.inner_stride[0], m);
+    load_vec_c<T, VEC, S>((const T*)p.y, off[1], p.d.inner_stride[1], a);
+    load_vec_c<T, VEC, S>((const T*)p.z, off[2], p.d.inner_stride[2], b);
+    __builtin_amdgcn_sched_barrier(0);  // every load is issued before the first use of one
 #pragma unroll
-  for (int i = 0; i < VEC; i++) r[i] = m[i] != 0 ? a[i] : b[i];
-  store_vec<T, VEC>((T*)p.out, o, r);
+    for (int i = 0; i < VEC; i++) r[i] = m[i] != 0 ? a[i] : b[i];
+    store_vec<T, VEC>((T*)p.out, o, r);
+  });
 }
 
 // bitwiseOp (BackendCPU.swift:407-443): or / and / xor on the raw bits, any dtype, keyed by
@@ -143,12 +157,15 @@ template <typename U, int OP, int VEC> __device__ __forceinline__ void bitwise_i
   uint32_t off[2];
   size_t o;
   bcast_offsets<2, VEC>(p.d, v, off, o);
-  U a[VEC], b[VEC], r[VEC];
-  load_vec<U, VEC>((const U*)p.a, off[0], p.d.inner_stride[0], a);
-  load_vec<U, VEC>((const U*)p.b, off[1], p.d.inner_stride[1], b);
+  with_strides2<VEC>(p.d.inner_stride, [&](auto sa, auto sb) {
+    U a[VEC], b[VEC], r[VEC];
+    load_vec_c<U, VEC, decltype(sa)::value>((const U*)p.a, off[0], p.d.inner_stride[0], a);
+    load_vec_c<U, VEC, decltype(sb)::value>((const U*)p.b, off[1], p.d.inner_stride[1], b);
+    __builtin_amdgcn_sched_barrier(0);  // every load is issued before the first use of one
 #pragma unroll
-  for (int i = 0; i < VEC; i++) r[i] = bitop<OP>(a[i], b[i]);
-  store_vec<U, VEC>((U*)p.out, o, r);
+    for (int i = 0; i < VEC; i++) r[i] = bitop<OP>(a[i], b[i]);
+    store_vec<U, VEC>((U*)p.out, o, r);
+  });
 }
 #define DEF_BITWISE(BN, U, V)                                                                         \
   HC_KERNEL void hc_bitwise_or_##BN##_v##V(hck_binary_args p) { bitwise_impl<U, BIT_OR, V>(p); }      \
@@ -337,6 +354,18 @@ __device__ __forceinline__ float safe_sigmoid(float x) {
 }
 __device__ __forceinline__ float safe_tanh(float x) { return 2.0f * safe_sigmoid(2.0f * x) - 1.0f; }
 
+// The same for results that are rounded to fp16 (11 significant bits): the hardware's exp2 and
+// reciprocal (about 1 ulp of fp32 each) instead of the library's expf and an IEEE division.
+// With the library routines an fp16 GELU is bound by the vector ALU (8 elements per 16-byte
+// load), not by memory.
+__device__ __forceinline__ float exp_hw(float x) { return __builtin_amdgcn_exp2f(x * 1.4426950408889634f); }
+__device__ __forceinline__ float sigmoid_hw(float x) {
+  if (x < -20.0f) return 0.0f;
+  if (x > 20.0f) return 1.0f;
+  return __builtin_amdgcn_rcpf(1.0f + exp_hw(-x));
+}
+__device__ __forceinline__ float tanh_hw(float x) { return 2.0f * sigmoid_hw(2.0f * x) - 1.0f; }
+
 __device__ __forceinline__ float fast_erf(float a) {
   float r, s, t, u;
   t = fabsf(a);
@@ -381,7 +410,13 @@ enum {
   E_ERF_GRAD, E_FLOOR, E_CEIL, E_ROUND
 };
 
-template <int OP> __device__ __forceinline__ float elemwise_apply(float f) {
+// HALF: the caller rounds the result to fp16.
+template <int OP, bool HALF> __device__ __forceinline__ float elemwise_apply(float f) {
+  if (HALF) {
+    if (OP == E_EXP) return exp_hw(f);
+    if (OP == E_SIGMOID) return sigmoid_hw(f);
+    if (OP == E_GELU_APPROX) return 0.5f * f * (1.0f + tanh_hw(0.797884561f * (f + 0.044715f * (f * f * f))));
+  }
   switch (OP) {
     case E_SIN: return sinf(f);
     case E_COS: return cosf(f);
@@ -431,11 +466,11 @@ template <typename T, int OP> __device__ __forceinline__ void elemwise_impl(cons
   const T* scales = (const T*)p.scales;
   if (scales) {
     map_contiguous((const T*)p.in, (T*)p.out, p.count, [scales](T xv, uint64_t i) {
-      return narrow<T>(elemwise_apply<OP>((float)xv) * (float)scales[i]);
+      return narrow<T>(elemwise_apply<OP, sizeof(T) == 2>((float)xv) * (float)scales[i]);
     });
   } else {
     map_contiguous((const T*)p.in, (T*)p.out, p.count,
-                   [](T xv, uint64_t) { return narrow<T>(elemwise_apply<OP>((float)xv) * 1.0f); });
+                   [](T xv, uint64_t) { return narrow<T>(elemwise_apply<OP, sizeof(T) == 2>((float)xv) * 1.0f); });
   }
 }
 
