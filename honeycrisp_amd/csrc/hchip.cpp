@@ -2073,7 +2073,7 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
               bm = t[0];
               bn = t[1];
             }
-          } else if (!filled && blocks > best_blocks) {
+          } else if (!filled && blocks >= best_blocks) {  // (a tie goes to the smaller tile: less padding)
             best_blocks = blocks;
             bm = t[0];
             bn = t[1];
