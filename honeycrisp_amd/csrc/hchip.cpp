@@ -1182,9 +1182,47 @@ extern "C" int hc_reduce(hc_ctx* ctx, int op, int dtype, const void* in, void* o
   if (inner == 1) {
     const bool vec_ok = aligned16(in);
     REQUIRE(vec_ok, "hc_reduce: input must be 16-byte aligned");
+    // a team of 1, 8, 64 or 256 lanes per row, by row length
     if (reduce <= 1024) {
-      snprintf(name, sizeof(name), "hc_reduce_rows64_%s_%s", kReduceNames[op], dtype_name(dtype));
-      return launch(ctx, name, ceil_div((uint64_t)outer, HCK_BLOCK / 64), 1, &k, sizeof(k));
+      const uint32_t lanes = reduce <= 8 ? 1 : reduce <= 128 ? 8 : 64;
+      snprintf(name, sizeof(name), "hc_reduce_rows%u_%s_%s", lanes, kReduceNames[op], dtype_name(dtype));
+      return launch(ctx, name, ceil_div((uint64_t)outer, HCK_BLOCK / lanes), 1, &k, sizeof(k));
+    }
+    // Few long rows (a sum or maximum over a whole tensor): a block per row would leave most of
+    // the device idle, so the rows are cut into segments that leave partials, combined by the
+    // final pass of the column reduction (partials laid out as [outer, segs, 1]).
+    const uint64_t cus = (uint64_t)ctx->props.multiProcessorCount;
+    if ((uint64_t)outer < 2 * cus && reduce >= 32768) {
+      uint64_t segs = std::min<uint64_t>(ceil_div(4 * cus, (uint64_t)outer), (uint64_t)reduce / 8192);
+      const uint64_t seg_len = ceil_div(ceil_div((uint64_t)reduce, segs), 8192) * 8192;
+      segs = ceil_div((uint64_t)reduce, seg_len);
+      if (segs > 1) {
+        const bool arg = op == HC_ARGMAX || op == HC_ARGMIN;
+        Scratch scratch(ctx);
+        const size_t n = (size_t)outer * segs;
+        HC_TRY(scratch.get(n * 8, &k.pvals));
+        if (arg) {
+          void* idx = nullptr;
+          HC_TRY(scratch.get(n * 4, &idx));
+          k.pidx = (uint32_t*)idx;
+        }
+        k.segs = (uint32_t)segs;
+        k.seg_len = (uint32_t)seg_len;
+        snprintf(name, sizeof(name), "hc_reduce_rowsplit_%s_%s", kReduceNames[op], dtype_name(dtype));
+        HC_TRY(launch(ctx, name, n, 1, &k, sizeof(k)));
+        hck_reduce_cols_args c;
+        memset(&c, 0, sizeof(c));
+        c.out = out;
+        c.pvals = k.pvals;
+        c.pidx = k.pidx;
+        c.outer = (uint32_t)outer;
+        c.reduce = (uint32_t)reduce;
+        c.inner = 1;
+        c.splits = (uint32_t)segs;
+        c.chunk = (uint32_t)seg_len;
+        snprintf(name, sizeof(name), "hc_reduce_cols_final_%s_%s", kReduceNames[op], dtype_name(dtype));
+        return launch(ctx, name, (uint64_t)outer, 1, &c, sizeof(c));
+      }
     }
     snprintf(name, sizeof(name), "hc_reduce_rows256_%s_%s", kReduceNames[op], dtype_name(dtype));
     return launch(ctx, name, (uint64_t)outer, 1, &k, sizeof(k));
@@ -1350,7 +1388,13 @@ extern "C" int hc_log_softmax(hc_ctx* ctx, int dtype, const void* in, void* out,
   k.inner = (uint32_t)inner;
   char name[64];
   if (inner == 1) {
-    // a wave per row while the row fits its registers (4 x 16 bytes per lane), else a block
+    // a lane or 8 lanes per row for short rows, a wave per row while the row fits its registers
+    // (4 x 16 bytes per lane), else a block
+    if (reduce <= 128) {
+      const uint32_t lanes = reduce <= 8 ? 1 : 8;
+      snprintf(name, sizeof(name), "hc_log_softmax_rows%u_%s", lanes, dtype_name(dtype));
+      return launch(ctx, name, ceil_div((uint64_t)outer, HCK_BLOCK / lanes), 1, &k, sizeof(k));
+    }
     if ((uint64_t)reduce * el_size <= 64 * 16 * 4) {
       snprintf(name, sizeof(name), "hc_log_softmax_rows_%s", dtype_name(dtype));
       return launch(ctx, name, ceil_div((uint64_t)outer, HCK_BLOCK / 64), 1, &k, sizeof(k));
@@ -1381,7 +1425,13 @@ extern "C" int hc_log_softmax_grad(hc_ctx* ctx, int dtype, const void* in, const
   k.inner = (uint32_t)inner;
   char name[64];
   if (inner == 1) {
-    // a wave per row while the row fits its registers (4 x 16 bytes per lane), else a block
+    // a lane or 8 lanes per row for short rows, a wave per row while the row fits its registers
+    // (4 x 16 bytes per lane), else a block
+    if (reduce <= 128) {
+      const uint32_t lanes = reduce <= 8 ? 1 : 8;
+      snprintf(name, sizeof(name), "hc_log_softmax_grad_rows%u_%s", lanes, dtype_name(dtype));
+      return launch(ctx, name, ceil_div((uint64_t)outer, HCK_BLOCK / lanes), 1, &k, sizeof(k));
+    }
     if ((uint64_t)reduce * el_size <= 64 * 16 * 4) {
       snprintf(name, sizeof(name), "hc_log_softmax_grad_rows_%s", dtype_name(dtype));
       return launch(ctx, name, ceil_div((uint64_t)outer, HCK_BLOCK / 64), 1, &k, sizeof(k));
@@ -1413,7 +1463,13 @@ extern "C" int hc_normalize(hc_ctx* ctx, int dtype, const void* in, void* out, i
     k.inner = 1;
     k.eps = eps;
     char name[64];
-    // a wave per row while the row fits its registers (4 x 16 bytes per lane), else a block
+    // a lane or 8 lanes per row for short rows, a wave per row while the row fits its registers
+    // (4 x 16 bytes per lane), else a block
+    if (reduce <= 128) {
+      const uint32_t lanes = reduce <= 8 ? 1 : 8;
+      snprintf(name, sizeof(name), "hc_normalize_rows%u_%s", lanes, dtype_name(dtype));
+      return launch(ctx, name, ceil_div((uint64_t)outer, HCK_BLOCK / lanes), 1, &k, sizeof(k));
+    }
     if ((uint64_t)reduce * el_size <= 64 * 16 * 4) {
       snprintf(name, sizeof(name), "hc_normalize_rows_%s", dtype_name(dtype));
       return launch(ctx, name, ceil_div((uint64_t)outer, HCK_BLOCK / 64), 1, &k, sizeof(k));

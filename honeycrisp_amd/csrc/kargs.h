@@ -90,6 +90,12 @@ typedef struct {
   uint32_t inner;
   float eps;
   const void* in2; /* logSoftmaxGrad: the output gradient */
+  /* reduce, few long rows: every row is cut into `segs` segments of `seg_len` elements, one
+   * workgroup each, which leave [outer, segs] partials (accumulator type; arg-reductions: the
+   * ordering key and the index within the row) for hc_reduce_cols_final_* with inner = 1 */
+  uint32_t segs, seg_len;
+  void* pvals;
+  uint32_t* pidx;
 } hck_reduce_args;
 
 /* Column reduction ([outer, reduce, inner], inner > 1) in up to two passes: the reduce axis is

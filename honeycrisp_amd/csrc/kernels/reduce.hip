@@ -47,17 +47,6 @@ __device__ __forceinline__ ArgPair<C> arg_better(ArgPair<C> a, ArgPair<C> b) {
   return take_b ? b : a;
 }
 
-template <int OP, typename C> __device__ __forceinline__ ArgPair<C> wave_arg_reduce(ArgPair<C> p) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) {
-    ArgPair<C> q;
-    q.v = __shfl_xor(p.v, o, 64);
-    q.i = __shfl_xor(p.i, o, 64);
-    p = arg_better<OP>(p, q);
-  }
-  return p;
-}
-
 // Worst possible value, paired with the largest index, so that any real element wins.
 template <int OP> __device__ __forceinline__ void arg_init(ArgPair<float>& p) {
   p.v = OP == R_ARGMAX ? -INFINITY : INFINITY;
@@ -79,18 +68,41 @@ template <int OP, typename C> __device__ __forceinline__ C reduce_combine(C a, C
 
 // ---------------------------------------------------------------- rows (inner == 1)
 
-// LANES = 64: one wave per row, 4 rows per block. LANES = 256: one block per row.
-template <typename T, int OP, int LANES>
+// A row is reduced by a team of LANES lanes: 1 (rows of a few elements: a lane per row, adjacent
+// lanes on adjacent rows), 8, 64 (one wave) or 256 (the whole block). SPLIT (LANES = 256): few
+// long rows are cut into p.segs segments, one block each, which leave partials.
+template <int LANES, typename V, typename Op> __device__ __forceinline__ V team_reduce(V v, Op op) {
+#pragma unroll
+  for (int o = LANES / 2; o > 0; o >>= 1) v = op(v, __shfl_xor(v, o, 64));
+  return v;
+}
+template <int LANES, int OP, typename C> __device__ __forceinline__ ArgPair<C> team_arg_reduce(ArgPair<C> p) {
+#pragma unroll
+  for (int o = LANES / 2; o > 0; o >>= 1) {
+    ArgPair<C> q;
+    q.v = __shfl_xor(p.v, o, 64);
+    q.i = __shfl_xor(p.i, o, 64);
+    p = arg_better<OP>(p, q);
+  }
+  return p;
+}
+
+template <typename T, int OP, int LANES, bool SPLIT>
 __device__ __forceinline__ void reduce_rows_impl(const hck_reduce_args& p) {
   typedef typename Arith<T>::type C;
   constexpr int VEC = VecWidth<T>::value;
   constexpr int ROWS_PER_BLOCK = HCK_BLOCK / LANES;
+  static_assert(!SPLIT || LANES == HCK_BLOCK, "segments are reduced by whole blocks");
   const uint32_t lane = threadIdx.x % LANES;
-  const uint32_t row = blockIdx.x * ROWS_PER_BLOCK + threadIdx.x / LANES;
+  const uint32_t seg = SPLIT ? blockIdx.x % p.segs : 0;
+  const uint32_t row = SPLIT ? blockIdx.x / p.segs : blockIdx.x * ROWS_PER_BLOCK + threadIdx.x / LANES;
   const bool active = row < p.outer;
   const uint32_t n = p.reduce;
+  // this team's part of the row: [k0, kend)
+  const uint32_t k0 = SPLIT ? seg * p.seg_len : 0;
+  const uint32_t kend = SPLIT ? (k0 + p.seg_len < n ? k0 + p.seg_len : n) : n;
   const T* in = (const T*)p.in + (size_t)(active ? row : 0) * n;
-  // Rows start 16-byte aligned only when the row length is a multiple of VEC.
+  // Rows start 16-byte aligned only when the row length is a multiple of VEC (segments are).
   const bool vec_ok = (n % VEC) == 0;
   __shared__ char lds_raw[sizeof(ArgPair<C>) * (HCK_BLOCK / 64)];
 
@@ -100,8 +112,8 @@ __device__ __forceinline__ void reduce_rows_impl(const hck_reduce_args& p) {
       if (vec_ok) {
         // four independent 16-byte loads in flight per lane, combined in index order
         constexpr uint32_t STEP = LANES * VEC;
-        uint32_t k = lane * VEC;
-        for (; k + 3 * STEP < n; k += 4 * STEP) {
+        uint32_t k = k0 + lane * VEC;
+        for (; k + 3 * STEP < kend; k += 4 * STEP) {
           T a[4][VEC];
 #pragma unroll
           for (int u = 0; u < 4; u++) load_vec<T, VEC>(in, k + u * STEP, 1, a[u]);
@@ -110,31 +122,34 @@ __device__ __forceinline__ void reduce_rows_impl(const hck_reduce_args& p) {
 #pragma unroll
             for (int i = 0; i < VEC; i++) acc = reduce_combine<OP, C>(acc, to_arith(a[u][i]));
         }
-        for (; k < n; k += STEP) {
+        for (; k < kend; k += STEP) {
           T a[VEC];
           load_vec<T, VEC>(in, k, 1, a);
 #pragma unroll
           for (int i = 0; i < VEC; i++) acc = reduce_combine<OP, C>(acc, to_arith(a[i]));
         }
       } else {
-        for (uint32_t k = lane; k < n; k += LANES) acc = reduce_combine<OP, C>(acc, to_arith(in[k]));
+        for (uint32_t k = k0 + lane; k < kend; k += LANES) acc = reduce_combine<OP, C>(acc, to_arith(in[k]));
       }
     }
-    if (LANES == 64) {
-      acc = OP == R_SUM ? wave_reduce(acc, SumOp()) : wave_reduce(acc, ProdOp());
+    if (LANES <= 64) {
+      acc = OP == R_SUM ? team_reduce<LANES>(acc, SumOp()) : team_reduce<LANES>(acc, ProdOp());
     } else {
       acc = OP == R_SUM ? block_reduce(acc, SumOp(), (C*)lds_raw)
                         : block_reduce(acc, ProdOp(), (C*)lds_raw);
     }
-    if (active && lane == 0) ((T*)p.out)[row] = from_arith<T>(acc);
+    if (active && lane == 0) {
+      if (SPLIT) ((C*)p.pvals)[blockIdx.x] = acc;
+      else ((T*)p.out)[row] = from_arith<T>(acc);
+    }
   } else {
     ArgPair<C> best;
     arg_init<OP>(best);
     if (active) {
       if (vec_ok) {
         constexpr uint32_t STEP = LANES * VEC;
-        uint32_t k = lane * VEC;
-        for (; k + 3 * STEP < n; k += 4 * STEP) {
+        uint32_t k = k0 + lane * VEC;
+        for (; k + 3 * STEP < kend; k += 4 * STEP) {
           T a[4][VEC];
 #pragma unroll
           for (int u = 0; u < 4; u++) load_vec<T, VEC>(in, k + u * STEP, 1, a[u]);
@@ -148,7 +163,7 @@ __device__ __forceinline__ void reduce_rows_impl(const hck_reduce_args& p) {
               best = arg_better<OP>(best, c);
             }
         }
-        for (; k < n; k += STEP) {
+        for (; k < kend; k += STEP) {
           T a[VEC];
           load_vec<T, VEC>(in, k, 1, a);
 #pragma unroll
@@ -160,7 +175,7 @@ __device__ __forceinline__ void reduce_rows_impl(const hck_reduce_args& p) {
           }
         }
       } else {
-        for (uint32_t k = lane; k < n; k += LANES) {
+        for (uint32_t k = k0 + lane; k < kend; k += LANES) {
           ArgPair<C> c;
           c.v = arg_key<OP>(to_arith(in[k]), k);
           c.i = k;
@@ -168,7 +183,7 @@ __device__ __forceinline__ void reduce_rows_impl(const hck_reduce_args& p) {
         }
       }
     }
-    best = wave_arg_reduce<OP>(best);
+    best = team_arg_reduce<(LANES < 64 ? LANES : 64), OP>(best);
     if (LANES > 64) {
       ArgPair<C>* lds = (ArgPair<C>*)lds_raw;
       if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = best;
@@ -177,7 +192,14 @@ __device__ __forceinline__ void reduce_rows_impl(const hck_reduce_args& p) {
 #pragma unroll
       for (int w = 1; w < HCK_BLOCK / 64; w++) best = arg_better<OP>(best, lds[w]);
     }
-    if (active && lane == 0) ((int64_t*)p.out)[row] = (int64_t)best.i;
+    if (active && lane == 0) {
+      if (SPLIT) {
+        ((C*)p.pvals)[blockIdx.x] = best.v;
+        p.pidx[blockIdx.x] = best.i;
+      } else {
+        ((int64_t*)p.out)[row] = (int64_t)best.i;
+      }
+    }
   }
 }
 
@@ -296,8 +318,11 @@ __device__ __forceinline__ void reduce_cols_impl(const hck_reduce_cols_args& p) 
 }
 
 #define DEF_REDUCE(NAME, OP, TN, T)                                                                   \
-  HC_KERNEL void hc_reduce_rows64_##NAME##_##TN(hck_reduce_args p) { reduce_rows_impl<T, OP, 64>(p); } \
-  HC_KERNEL void hc_reduce_rows256_##NAME##_##TN(hck_reduce_args p) { reduce_rows_impl<T, OP, 256>(p); } \
+  HC_KERNEL void hc_reduce_rows1_##NAME##_##TN(hck_reduce_args p) { reduce_rows_impl<T, OP, 1, false>(p); } \
+  HC_KERNEL void hc_reduce_rows8_##NAME##_##TN(hck_reduce_args p) { reduce_rows_impl<T, OP, 8, false>(p); } \
+  HC_KERNEL void hc_reduce_rows64_##NAME##_##TN(hck_reduce_args p) { reduce_rows_impl<T, OP, 64, false>(p); } \
+  HC_KERNEL void hc_reduce_rows256_##NAME##_##TN(hck_reduce_args p) { reduce_rows_impl<T, OP, 256, false>(p); } \
+  HC_KERNEL void hc_reduce_rowsplit_##NAME##_##TN(hck_reduce_args p) { reduce_rows_impl<T, OP, 256, true>(p); } \
   HC_KERNEL void hc_reduce_cols_##NAME##_##TN##_v1(hck_reduce_cols_args p) {                           \
     reduce_cols_impl<T, OP, 1, false>(p);                                                              \
   }                                                                                                    \
@@ -318,7 +343,8 @@ DEF_REDUCE_T(i64, int64_t)
 
 // ---------------------------------------------------------------- row teams
 
-// A row is worked on by a team of LANES lanes: one wave (4 rows per block) or the whole block.
+// A row is worked on by a team of LANES lanes: 1 or 8 (short rows, many per wave), one wave
+// (4 rows per block) or the whole block.
 template <int LANES> struct Team {
   static __device__ __forceinline__ uint32_t lane() { return threadIdx.x % LANES; }
   static __device__ __forceinline__ uint32_t row() {
@@ -326,7 +352,7 @@ template <int LANES> struct Team {
   }
   // every lane of the team gets the result; `lds` holds >= 4 floats (block teams only)
   template <typename Op> static __device__ __forceinline__ float reduce(float v, Op op, float* lds) {
-    if (LANES == 64) return wave_reduce(v, op);
+    if (LANES <= 64) return team_reduce<LANES>(v, op);
     return block_reduce(v, op, lds);
   }
 };
@@ -513,7 +539,11 @@ DEF_SOFTMAX_COLS(f32, float)
 DEF_SOFTMAX_COLS(f16, half_t)
 
 HC_KERNEL void hc_log_softmax_rows_f32(hck_reduce_args p) { log_softmax_rows_impl<float, 64>(p); }
+HC_KERNEL void hc_log_softmax_rows1_f32(hck_reduce_args p) { log_softmax_rows_impl<float, 1>(p); }
+HC_KERNEL void hc_log_softmax_rows8_f32(hck_reduce_args p) { log_softmax_rows_impl<float, 8>(p); }
 HC_KERNEL void hc_log_softmax_rows_f16(hck_reduce_args p) { log_softmax_rows_impl<half_t, 64>(p); }
+HC_KERNEL void hc_log_softmax_rows1_f16(hck_reduce_args p) { log_softmax_rows_impl<half_t, 1>(p); }
+HC_KERNEL void hc_log_softmax_rows8_f16(hck_reduce_args p) { log_softmax_rows_impl<half_t, 8>(p); }
 HC_KERNEL void hc_log_softmax_rows256_f32(hck_reduce_args p) { log_softmax_rows_impl<float, 256>(p); }
 HC_KERNEL void hc_log_softmax_rows256_f16(hck_reduce_args p) { log_softmax_rows_impl<half_t, 256>(p); }
 
@@ -557,7 +587,11 @@ __device__ __forceinline__ void log_softmax_grad_rows_impl(const hck_reduce_args
 }
 
 HC_KERNEL void hc_log_softmax_grad_rows_f32(hck_reduce_args p) { log_softmax_grad_rows_impl<float, 64>(p); }
+HC_KERNEL void hc_log_softmax_grad_rows1_f32(hck_reduce_args p) { log_softmax_grad_rows_impl<float, 1>(p); }
+HC_KERNEL void hc_log_softmax_grad_rows8_f32(hck_reduce_args p) { log_softmax_grad_rows_impl<float, 8>(p); }
 HC_KERNEL void hc_log_softmax_grad_rows_f16(hck_reduce_args p) { log_softmax_grad_rows_impl<half_t, 64>(p); }
+HC_KERNEL void hc_log_softmax_grad_rows1_f16(hck_reduce_args p) { log_softmax_grad_rows_impl<half_t, 1>(p); }
+HC_KERNEL void hc_log_softmax_grad_rows8_f16(hck_reduce_args p) { log_softmax_grad_rows_impl<half_t, 8>(p); }
 HC_KERNEL void hc_log_softmax_grad_rows256_f32(hck_reduce_args p) { log_softmax_grad_rows_impl<float, 256>(p); }
 HC_KERNEL void hc_log_softmax_grad_rows256_f16(hck_reduce_args p) { log_softmax_grad_rows_impl<half_t, 256>(p); }
 
@@ -607,6 +641,10 @@ template <typename T, int LANES> __device__ __forceinline__ void normalize_rows_
   stream_row_out<T, LANES>(in, out, n, lane, [&](float x, uint32_t) { return round_through<T>(x - mean) * normer; });
 }
 HC_KERNEL void hc_normalize_rows_f32(hck_reduce_args p) { normalize_rows_impl<float, 64>(p); }
+HC_KERNEL void hc_normalize_rows1_f32(hck_reduce_args p) { normalize_rows_impl<float, 1>(p); }
+HC_KERNEL void hc_normalize_rows8_f32(hck_reduce_args p) { normalize_rows_impl<float, 8>(p); }
 HC_KERNEL void hc_normalize_rows_f16(hck_reduce_args p) { normalize_rows_impl<half_t, 64>(p); }
+HC_KERNEL void hc_normalize_rows1_f16(hck_reduce_args p) { normalize_rows_impl<half_t, 1>(p); }
+HC_KERNEL void hc_normalize_rows8_f16(hck_reduce_args p) { normalize_rows_impl<half_t, 8>(p); }
 HC_KERNEL void hc_normalize_rows256_f32(hck_reduce_args p) { normalize_rows_impl<float, 256>(p); }
 HC_KERNEL void hc_normalize_rows256_f16(hck_reduce_args p) { normalize_rows_impl<half_t, 256>(p); }

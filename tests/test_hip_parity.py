@@ -418,7 +418,10 @@ def test_when_fill_triangular_concat_broadcast(hip_backend, oracle_backend):
 REDUCE_SHAPES = [(8, 4096, 1), (37, 513, 1), (5, 1, 1), (3, 7, 1), (1, 100000, 1), (64, 1024, 1), (4, 33, 65),
                  (1, 300, 4096), (17, 2, 3), (9, 8192, 2),
                  # tall and narrow: the reduce axis is split over blocks and combined in a second pass
-                 (2, 5000, 96), (1, 4097, 260), (1, 70000, 8)]
+                 (2, 5000, 96), (1, 4097, 260), (1, 70000, 8),
+                 # rows of a few elements (a lane or 8 lanes per row) and few long rows (cut into
+                 # segments that leave partials; 300001 is odd, so its segments are read element-wise)
+                 (70000, 3, 1), (5000, 8, 1), (4097, 100, 1), (1, 400000, 1), (3, 300001, 1), (2, 65536, 1)]
 
 
 @pytest.mark.parametrize("dtype", [F32, F16, I64], ids=["f32", "f16", "i64"])
@@ -476,13 +479,28 @@ def test_argmax_nan_and_tie_rules(hip_backend, oracle_backend):
     check_exact(hip_backend, oracle_backend, lambda: Tensor(data=y).max(axis=1))
     check_exact(hip_backend, oracle_backend, lambda: Tensor(data=y).min(axis=0))
     check_exact(hip_backend, oracle_backend, lambda: Tensor(data=y).max())
+    # one long row in segments: ties and NaNs across segment boundaries, NaN at element 0
+    z = rng.integers(-3, 4, size=(2, 200000)).astype(np.float32)
+    z[rng.random(z.shape) < 0.001] = nan
+    z[1, 0] = nan
+    for op in (ReduceOp.argmax, ReduceOp.argmin):
+        check_exact(hip_backend, oracle_backend, lambda: Tensor(data=z).reduce(op, axis=1))
+        check_exact(hip_backend, oracle_backend, lambda: Tensor(data=z[0]).reduce(op, axis=0))
+    # rows of 3 and of 100 elements with ties and NaNs
+    for width in (3, 100):
+        w = rng.integers(-1, 2, size=(3000, width)).astype(np.float32)
+        w[rng.random(w.shape) < 0.05] = nan
+        for op in (ReduceOp.argmax, ReduceOp.argmin):
+            check_exact(hip_backend, oracle_backend, lambda: Tensor(data=w).reduce(op, axis=1))
 
 
 @pytest.mark.parametrize("dtype", [F32, F16], ids=["f32", "f16"])
 def test_log_softmax_and_normalize(hip_backend, oracle_backend, dtype):
     rng = np.random.default_rng(19)
     for shape, axis in [((64, 256), 1), ((16, 8, 32, 32), 3), ((5, 1000), 1), ((7, 33, 9), 1), ((300, 4), 0),
-                        ((2, 1), 1), ((3, 10000), 1), ((4096, 96), 0), ((2, 3000, 40), 1), ((3, 129, 7), 1)]:
+                        ((2, 1), 1), ((3, 10000), 1), ((4096, 96), 0), ((2, 3000, 40), 1), ((3, 129, 7), 1),
+                        # short rows: a lane or 8 lanes per row
+                        ((7000, 3), 1), ((3001, 8), 1), ((1000, 100), 1), ((999, 128), 1), ((500, 16), 1)]:
         x = rand(rng, shape, dtype, 3.0)
         print("logsoftmax/normalize", dtype.name, shape, axis, flush=True)
         check_close(hip_backend, oracle_backend, lambda: Tensor(data=x).logSoftmax(axis=axis), TOL[dtype])
@@ -626,7 +644,8 @@ def test_log_softmax_grad(hip_backend, oracle_backend, dtype):
     from honeycrisp_amd.backend import Backend
     rng = np.random.default_rng(33)
     for shape, axis in [((64, 300), 1), ((7, 33, 40), 1), ((5, 1, 9), 2), ((3, 1000), 0), ((2048, 256), 1),
-                        ((4096, 96), 0), ((2, 3000, 40), 1), ((16, 5000), 1), ((9, 33000), 1)]:
+                        ((4096, 96), 0), ((2, 3000, 40), 1), ((16, 5000), 1), ((9, 33000), 1),
+                        ((7000, 3), 1), ((3001, 8), 1), ((1000, 100), 1), ((999, 128), 1)]:
         x, g = rand(rng, shape, dtype, 2.0), rand(rng, shape, dtype)
         def run():
             xt, gt = Tensor(data=x), Tensor(data=g)
