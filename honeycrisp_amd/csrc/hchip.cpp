@@ -1254,12 +1254,17 @@ extern "C" int hc_cumulative(hc_ctx* ctx, int op, int dtype, const void* in, voi
   const uint64_t vec = 16 / dtype_size(dtype);
   const bool colsv = inner > 1 && (uint64_t)inner % vec == 0 && aligned16(in) && aligned16(out) &&
                      (uint64_t)outer * (uint64_t)inner / vec >= 64;
-  const char* form = inner == 1 ? "rows" : colsv ? "colsv" : "cols";
+  // (rows of a few elements: the column form with inner = 1 is a lane per row, adjacent lanes on
+  // adjacent rows, instead of a wave per row)
+  const bool lane_rows = inner == 1 && reduce <= 16;
+  const char* form = lane_rows ? "cols" : inner == 1 ? "rows" : colsv ? "colsv" : "cols";
   const char* tn = dtype_name(dtype);
   // Few, long lines: cut the axis so that about eight waves per compute unit have work.
   const uint64_t cus = (uint64_t)ctx->props.multiProcessorCount;
   uint64_t segs = 1, seg_len = (uint64_t)reduce;
-  if (inner == 1) {
+  if (lane_rows) {
+    // one pass, no segments
+  } else if (inner == 1) {
     const uint64_t want = cus * 8;  // waves
     if ((uint64_t)outer < want && reduce >= 4096) {
       segs = std::min<uint64_t>(ceil_div(want, (uint64_t)outer), (uint64_t)reduce / 1024);
@@ -1276,7 +1281,7 @@ extern "C" int hc_cumulative(hc_ctx* ctx, int op, int dtype, const void* in, voi
   }
   char name[64];
   const uint64_t units = (uint64_t)outer * segs * (uint64_t)inner;  // waves (rows) or columns (cols)
-  const uint64_t blocks = inner == 1 ? ceil_div(units, HCK_BLOCK / 64) : ceil_div(units / (colsv ? vec : 1), HCK_BLOCK);
+  const uint64_t blocks = inner == 1 && !lane_rows ? ceil_div(units, HCK_BLOCK / 64) : ceil_div(units / (colsv ? vec : 1), HCK_BLOCK);
   Scratch scratch(ctx);
   if (segs > 1) {
     k.segs = (uint32_t)segs;
@@ -1285,7 +1290,7 @@ extern "C" int hc_cumulative(hc_ctx* ctx, int op, int dtype, const void* in, voi
     snprintf(name, sizeof(name), "hc_cumulative_%s_%s_totals_%s", opn, form, tn);
     HC_TRY(launch(ctx, name, blocks, 1, &k, sizeof(k)));
     snprintf(name, sizeof(name), "hc_cumulative_%s_carry_%s", opn, dtype == HC_I64 ? "i64" : "f32");
-    HC_TRY(launch(ctx, name, ceil_div((uint64_t)outer * (uint64_t)inner, HCK_BLOCK), 1, &k, sizeof(k)));
+    HC_TRY(launch(ctx, name, ceil_div((uint64_t)outer * (uint64_t)inner, HCK_BLOCK / 64), 1, &k, sizeof(k)));  // a wave per line
   }
   snprintf(name, sizeof(name), "hc_cumulative_%s_%s_%s", opn, form, tn);
   return launch(ctx, name, blocks, 1, &k, sizeof(k));

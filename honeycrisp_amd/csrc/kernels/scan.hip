@@ -118,17 +118,29 @@ __device__ __forceinline__ void cumulative_cols_impl(const hck_scan_args& p) {
   }
 }
 
-// Segment totals -> what precedes each segment: one lane per (i, j) walks its `segs` totals.
+// Segment totals -> what precedes each segment: one wave per line (i, j) scans its `segs` totals
+// 64 at a time with shuffles (a lane walking them one by one would take longer than the scan
+// of the data itself once a line has thousands of segments).
 template <typename C, int OP> __device__ __forceinline__ void cumulative_carry_impl(const hck_scan_args& p) {
-  const uint64_t t = (uint64_t)blockIdx.x * HCK_BLOCK + threadIdx.x;
-  if (t >= (uint64_t)p.outer * p.inner) return;
-  const uint32_t i = (uint32_t)(t / p.inner), j = (uint32_t)(t - (uint64_t)i * p.inner);
+  const uint64_t line = (uint64_t)blockIdx.x * (HCK_BLOCK / 64) + (threadIdx.x >> 6);
+  if (line >= (uint64_t)p.outer * p.inner) return;  // (whole waves)
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t i = (uint32_t)(line / p.inner), j = (uint32_t)(line - (uint64_t)i * p.inner);
   C* c = (C*)p.carry + (size_t)i * p.segs * p.inner + j;
   C run = scan_identity<OP, C>();
-  for (uint32_t s = 0; s < p.segs; s++) {
-    const C total = c[(size_t)s * p.inner];
-    c[(size_t)s * p.inner] = run;
-    run = scan_combine<OP, C>(run, total);
+  for (uint32_t s0 = 0; s0 < p.segs; s0 += 64) {
+    const uint32_t s = s0 + lane;
+    const bool ok = s < p.segs;
+    C incl = ok ? c[(size_t)s * p.inner] : scan_identity<OP, C>();
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const C up = __shfl_up(incl, d, 64);
+      if ((int)lane >= d) incl = scan_combine<OP, C>(up, incl);
+    }
+    C before = __shfl_up(incl, 1, 64);
+    if (lane == 0) before = scan_identity<OP, C>();
+    if (ok) c[(size_t)s * p.inner] = scan_combine<OP, C>(run, before);
+    run = scan_combine<OP, C>(run, __shfl(incl, 63, 64));
   }
 }
 

@@ -726,7 +726,9 @@ def test_bitwise_ops(hip_backend, oracle_backend):
 def test_cumulative_ops(hip_backend, oracle_backend, dtype):
     rng = np.random.default_rng(38)
     for shape, axis in [((7, 1000), 1), ((3, 257, 5), 1), ((5000, 3), 0), ((4, 1), 1), ((2, 64), 1), ((1, 70000), 1),
-                        ((300, 512), 0), ((4, 200, 256), 1)]:     # 16-byte column vectors, with / without segments
+                        ((300, 512), 0), ((4, 200, 256), 1),      # 16-byte column vectors, with / without segments
+                        # a lane per row; thousands of segments per line (the carry scan works in waves)
+                        ((5000, 3), 1), ((777, 16), 1), ((40000, 3), 0), ((30000, 64), 0)]:
         # small integers: every partial sum is exact, so the scan order cannot matter
         x = rng.integers(-3, 4, size=shape)
         x = x if dtype == I64 else x.astype(dtype.numpy)
