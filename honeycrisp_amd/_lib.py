@@ -111,6 +111,7 @@ PROTOTYPES = {
     "hc_triangular": (c_int, [_P, c_int, _P, _P, c_int64, c_int64, c_int64, c_int, c_int64]),
     "hc_fill": (c_int, [_P, c_int, c_float, c_int64, _P, c_size_t]),
     "hc_axis_permutation": (c_int, [_P, POINTER(c_int64), POINTER(c_int64), c_int, _P]),
+    "hc_permute": (c_int, [_P, c_int, _P, POINTER(c_int64), POINTER(c_int64), c_int, c_int64, _P]),
     "hc_concat": (c_int, [_P, c_int, POINTER(c_void_p), POINTER(c_int64), c_int, c_int64, _P]),
 }
 

@@ -273,6 +273,43 @@ class HIPData:
             backend._lib.hc_free(backend._ctx, c_void_p(ptr))
 
 
+class PermutationData(HIPData):
+    """The int64 index vector of axisPermutation(permutation, shape), produced on first use of its
+    pointer: the usual consumer is the gather of t / swap / move, which HIPBackend.gather runs as a
+    direct copy from (permutation, shape) alone, so most vectors are never written."""
+
+    def __init__(self, backend: "HIPBackend", permutation, shape):
+        self.backend = backend
+        self.permutation = (tuple(permutation), tuple(shape))
+        self.byteCount = product(shape) * 8
+        self._ptr = None
+
+    @property
+    def ptr(self):
+        if self._ptr is None and self.backend is not None:
+            backend = self.backend
+            perm, shape = self.permutation
+            n = len(shape)
+            block = backend.allocate(self.byteCount)
+            self._ptr, block.ptr = block.ptr, None      # this object owns the block now
+            backend._check(backend._lib.hc_axis_permutation(
+                backend._ctx, (c_int64 * max(n, 1))(*perm), (c_int64 * max(n, 1))(*shape), n, c_void_p(self._ptr)))
+            if backend._capturing:
+                # written by a recorded kernel, i.e. not before the graph runs: stop sharing it
+                backend._perm_cache.pop(self.permutation, None)
+        return self._ptr
+
+    @ptr.setter
+    def ptr(self, value):
+        self._ptr = value
+
+    def __del__(self):
+        backend, ptr = self.backend, self._ptr
+        self._ptr = None
+        if ptr and backend is not None and backend._ctx:
+            backend._lib.hc_free(backend._ctx, c_void_p(ptr))
+
+
 Scalar = Union[int, float, np.floating, np.integer]
 
 
@@ -566,6 +603,22 @@ class HIPBackend(Backend):
 
     def gather(self, a, s: ScatterGatherIndices, dtype: DType) -> HIPData:
         out = self.allocate(s.gatherOutCount * dtype.byteSize)
+        # The gather of t / swap / move / PermuteAxes: its index vector came from axisPermutation
+        # and runs along the gathered axis only. One direct copy moves the same bytes without
+        # reading 8 bytes of index per element.
+        meta = getattr(s.indices.data, "permutation", None)
+        st_ = s.indices.strides
+        if (meta is not None and st_.shape[s.axis] == s.middleCount == product(meta[1])
+                and all(stride == (1 if ax == s.axis else 0) or size == 1
+                        for ax, (stride, size) in enumerate(zip(st_.strides, st_.shape)))):
+            perm, shape = list(meta[0]), list(meta[1])
+            if s.outerCount > 1:
+                perm, shape = [0] + [p + 1 for p in perm], [s.outerCount] + shape
+            n = len(shape)
+            self._check(self._lib.hc_permute(self._ctx, int(dtype), c_void_p(self._dev(a).ptr),
+                                             (c_int64 * max(n, 1))(*perm), (c_int64 * max(n, 1))(*shape), n,
+                                             s.innerCount, c_void_p(out.ptr)))
+            return out
         ad, idx = self._dev(a), self._dev(s.indices.data)
         st = self._s(s.indices.strides)
         self._check(self._lib.hc_gather(self._ctx, int(dtype), c_void_p(ad.ptr), c_void_p(idx.ptr), byref(st),
@@ -698,19 +751,16 @@ class HIPBackend(Backend):
 
     def axisPermutation(self, permutation: List[int], shape: List[int]) -> HIPData:
         """The index vector depends on (permutation, shape) only and every permuted view of that
-        shape rebuilds it (Index.swift:238-266), so finished vectors are kept and shared: buffers
-        are never modified after creation. Entries are never evicted (a recorded graph may read
-        them); nothing is added while recording, because a recorded kernel has not run yet."""
+        shape asks for it again (Index.swift:238-266). It is handed out as a PermutationData, which
+        writes the vector only if somebody reads its pointer, and shared: buffers are never
+        modified after creation. Entries are never evicted (a recorded graph may read them),
+        except that a vector first written while recording stops being shared."""
         key = (tuple(permutation), tuple(shape))
         hit = self._perm_cache.get(key)
         if hit is not None:
             return hit
-        n = len(shape)
-        out = self.allocate(product(shape) * 8)
-        perm = (c_int64 * max(n, 1))(*permutation)
-        shp = (c_int64 * max(n, 1))(*shape)
-        self._check(self._lib.hc_axis_permutation(self._ctx, perm, shp, n, c_void_p(out.ptr)))
-        if not self._capturing and self._perm_cache_bytes + out.byteCount <= self.PERMUTATION_CACHE_BYTES:
+        out = PermutationData(self, permutation, shape)
+        if self._perm_cache_bytes + out.byteCount <= self.PERMUTATION_CACHE_BYTES:
             self._perm_cache[key] = out
             self._perm_cache_bytes += out.byteCount
         return out

@@ -1794,6 +1794,115 @@ extern "C" int hc_axis_permutation(hc_ctx* ctx, const int64_t* perm, const int64
   return launch(ctx, "hc_axis_permutation", ceil_div(total, HCK_BLOCK), 1, &k, sizeof(k));
 }
 
+extern "C" int hc_permute(hc_ctx* ctx, int dtype, const void* in, const int64_t* perm, const int64_t* shape,
+                          int ndim, int64_t inner, void* out) {
+  REQUIRE(ctx, "hc_permute: null context");
+  REQUIRE(dtype_name(dtype), "hc_permute: bad dtype %d", dtype);
+  REQUIRE(ndim >= 0 && ndim <= HC_MAX_DIMS - 1, "hc_permute: ndim %d out of range", ndim);
+  REQUIRE(ndim == 0 || (perm && shape), "hc_permute: null argument");
+  REQUIRE(inner >= 0, "hc_permute: negative inner count");
+  const size_t el = dtype_size(dtype);
+  bool seen[HC_MAX_DIMS] = {false};
+  uint64_t total = (uint64_t)inner;
+  for (int d = 0; d < ndim; d++) {
+    REQUIRE(shape[d] >= 0, "hc_permute: negative extent");
+    REQUIRE(perm[d] >= 0 && perm[d] < ndim && !seen[perm[d]], "hc_permute: invalid permutation");
+    seen[perm[d]] = true;
+    total *= (uint64_t)shape[d];
+    if (total > 0xffffffffull) return fail(HC_ERR_TOO_LARGE, "hc_permute: more than 2^32-1 elements");
+  }
+  if (total == 0) return HC_OK;
+  REQUIRE(in && out, "hc_permute: null pointer");
+  // Axes in output order with their source strides (elements); the untouched trailing block is
+  // one more innermost axis. Unit axes go, axes adjacent in both orders merge.
+  struct Axis { uint64_t extent, stride; };
+  Axis ax[HC_MAX_DIMS + 1];
+  int n = 0;
+  for (int d = 0; d < ndim; d++) {
+    uint64_t stride = (uint64_t)inner;
+    for (int e = (int)perm[d] + 1; e < ndim; e++) stride *= (uint64_t)shape[e];
+    if (shape[perm[d]] == 1) continue;
+    if (n > 0 && ax[n - 1].stride == stride * (uint64_t)shape[perm[d]]) {
+      ax[n - 1].extent *= (uint64_t)shape[perm[d]];
+      ax[n - 1].stride = stride;
+    } else {
+      ax[n].extent = (uint64_t)shape[perm[d]];
+      ax[n].stride = stride;
+      n++;
+    }
+  }
+  if (inner > 1) {
+    if (n > 0 && ax[n - 1].stride == (uint64_t)inner) {
+      ax[n - 1].extent *= (uint64_t)inner;
+      ax[n - 1].stride = 1;
+    } else {
+      ax[n].extent = (uint64_t)inner;
+      ax[n].stride = 1;
+      n++;
+    }
+  }
+  hck_permute_args k;
+  memset(&k, 0, sizeof(k));
+  k.in = in;
+  k.out = out;
+  char name[64];
+  if (n == 0 || ax[n - 1].stride == 1) {
+    // row form: the innermost axis is the same in source and output
+    const uint64_t row_len = n == 0 ? 1 : ax[n - 1].extent;
+    const int rows_n = n == 0 ? 0 : n - 1;
+    uint32_t vec = (uint32_t)(16 / el);
+    if (row_len % vec != 0 || !aligned16(in) || !aligned16(out)) vec = 1;
+    for (int d = 0; d < rows_n && vec > 1; d++)
+      if (ax[d].stride % vec != 0) vec = 1;
+    k.ndim = (uint32_t)rows_n;
+    k.inner = (uint32_t)row_len;
+    k.inner_vecs = (uint32_t)(row_len / vec);
+    k.total = (uint32_t)(total / vec);
+    hck_fast_div_setup(k.inner_vecs, &k.inner_magic, &k.inner_sh);
+    for (int d = 0; d < rows_n; d++) {
+      k.shape[d] = (uint32_t)ax[d].extent;
+      k.in_stride[d] = (uint32_t)ax[d].stride;
+      hck_fast_div_setup(k.shape[d], &k.magic[d], &k.sh[d]);
+    }
+    snprintf(name, sizeof(name), "hc_permute_rows_b%zu_%s", el, vec > 1 ? "vN" : "v1");
+    return launch(ctx, name, ceil_div((uint64_t)k.total, HCK_BLOCK), 1, &k, sizeof(k));
+  }
+  // tile form: the output's innermost axis a is not the source's innermost axis c
+  int c = -1;
+  for (int d = 0; d < n; d++)
+    if (ax[d].stride == 1) c = d;
+  REQUIRE(c >= 0 && c != n - 1, "hc_permute: internal error (no contiguous source axis)");
+  uint64_t out_stride[HC_MAX_DIMS + 1];
+  uint64_t acc = 1;
+  for (int d = n - 1; d >= 0; d--) {
+    out_stride[d] = acc;
+    acc *= ax[d].extent;
+  }
+  k.tile_a = (uint32_t)ax[n - 1].extent;
+  k.a_stride = (uint32_t)ax[n - 1].stride;
+  k.tile_c = (uint32_t)ax[c].extent;
+  k.c_out_stride = (uint32_t)out_stride[c];
+  k.tiles_a = (uint32_t)ceil_div(ax[n - 1].extent, 64);
+  k.tiles_c = (uint32_t)ceil_div(ax[c].extent, 64);
+  hck_fast_div_setup(k.tiles_a, &k.tiles_a_magic, &k.tiles_a_sh);
+  hck_fast_div_setup(k.tiles_c, &k.tiles_c_magic, &k.tiles_c_sh);
+  uint64_t batch = 1;
+  for (int d = 0; d < n - 1; d++) {
+    if (d == c) continue;
+    k.shape[k.ndim] = (uint32_t)ax[d].extent;
+    k.in_stride[k.ndim] = (uint32_t)ax[d].stride;
+    k.out_stride[k.ndim] = (uint32_t)out_stride[d];
+    hck_fast_div_setup(k.shape[k.ndim], &k.magic[k.ndim], &k.sh[k.ndim]);
+    batch *= ax[d].extent;
+    k.ndim++;
+  }
+  const uint64_t tiles = batch * k.tiles_a * k.tiles_c;
+  if (tiles > 0x7fffffffull) return fail(HC_ERR_TOO_LARGE, "hc_permute: too many tiles");
+  k.total = (uint32_t)tiles;
+  snprintf(name, sizeof(name), "hc_permute_tile_b%zu", el);
+  return launch(ctx, name, tiles, 1, &k, sizeof(k));
+}
+
 extern "C" int hc_triangular(hc_ctx* ctx, int dtype, const void* in, void* out, int64_t batch,
                              int64_t rows, int64_t cols, int upper, int64_t offset) {
   REQUIRE(ctx, "hc_triangular: null context");

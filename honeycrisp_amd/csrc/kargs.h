@@ -233,6 +233,33 @@ typedef struct {
   uint32_t permuted_strides[HCK_MAX_DIMS];
 } hck_axis_perm_args;
 
+/* Direct axis permutation (the gather that follows an axisPermutation, without its index vector).
+ * Axes are the output's, outermost first, after the host dropped unit axes and merged axes that are
+ * adjacent in both orders; strides in elements.
+ * Row form: the innermost axis is contiguous in both; a lane moves `vec` of its `inner` elements, the
+ * row number is unravelled over shape[0..ndim) (divisions by multiply-high, hck_fast_div_setup).
+ * Tile form: the output's innermost axis (extent tile_a, source stride a_stride) differs from the
+ * source's (extent tile_c, output stride c_out_stride): 64 x 64 tiles go through LDS, read along
+ * the source's innermost axis and written along the output's; shape[]/in_stride[]/out_stride[] then
+ * describe the remaining axes. */
+typedef struct {
+  const void* in;
+  void* out;
+  uint32_t ndim;
+  uint32_t inner;
+  uint32_t inner_vecs;
+  uint32_t total; /* row form: vectors; tile form: tiles */
+  uint32_t shape[HCK_MAX_DIMS];
+  uint32_t in_stride[HCK_MAX_DIMS];
+  uint32_t out_stride[HCK_MAX_DIMS];
+  uint32_t magic[HCK_MAX_DIMS];
+  uint32_t sh[HCK_MAX_DIMS];
+  uint32_t inner_magic, inner_sh;
+  uint32_t tile_a, tile_c, a_stride, c_out_stride;
+  uint32_t tiles_a, tiles_c;
+  uint32_t tiles_a_magic, tiles_a_sh, tiles_c_magic, tiles_c_sh;
+} hck_permute_args;
+
 typedef struct {
   const void* in;
   void* out;

@@ -262,6 +262,68 @@ HC_KERNEL void hc_axis_permutation(hck_axis_perm_args p) {
   p.out[i] = (int64_t)flat;
 }
 
+// The gather that follows an axisPermutation, done directly: the same data movement as
+// gather(in, axisPermutation(perm, shape)) (Index.swift:238-266, BackendCPU.swift:1108-1147),
+// without writing and re-reading 8 bytes of index per element.
+// Row form: a lane per VEC consecutive elements of the shared innermost axis.
+template <typename V, int VEC> __device__ __forceinline__ void permute_rows_impl(const hck_permute_args& p) {
+  const uint32_t v = blockIdx.x * HCK_BLOCK + threadIdx.x;
+  if (v >= p.total) return;
+  uint32_t row = fast_div(v, p.inner_magic, p.inner_sh);
+  const uint32_t col = (v - row * p.inner_vecs) * VEC;
+  const size_t out_off = (size_t)row * p.inner + col;
+  size_t in_off = col;
+  for (int d = (int)p.ndim - 1; d >= 0; d--) {
+    const uint32_t q = fast_div(row, p.magic[d], p.sh[d]);
+    in_off += (size_t)(row - q * p.shape[d]) * p.in_stride[d];
+    row = q;
+  }
+  typedef Vec<V, VEC> Pack;
+  *reinterpret_cast<Pack*>((V*)p.out + out_off) = *reinterpret_cast<const Pack*>((const V*)p.in + in_off);
+}
+// Tile form: 64 x 64 elements through LDS. Reads run along the source's innermost axis c, writes
+// along the output's innermost axis a; one padding element per LDS row keeps both off the same banks.
+template <typename V> __device__ __forceinline__ void permute_tile_impl(const hck_permute_args& p) {
+  __shared__ V tile[64][65];
+  uint32_t t = blockIdx.x;
+  uint32_t q = fast_div(t, p.tiles_c_magic, p.tiles_c_sh);
+  const uint32_t c0 = (t - q * p.tiles_c) * 64;
+  t = q;
+  q = fast_div(t, p.tiles_a_magic, p.tiles_a_sh);
+  const uint32_t a0 = (t - q * p.tiles_a) * 64;
+  uint32_t rest = q;
+  size_t in_base = 0, out_base = 0;
+  for (int d = (int)p.ndim - 1; d >= 0; d--) {
+    const uint32_t qq = fast_div(rest, p.magic[d], p.sh[d]);
+    const uint32_t r = rest - qq * p.shape[d];
+    in_base += (size_t)r * p.in_stride[d];
+    out_base += (size_t)r * p.out_stride[d];
+    rest = qq;
+  }
+  const uint32_t x = threadIdx.x & 63, y0 = threadIdx.x >> 6;
+  const V* in = (const V*)p.in + in_base;
+  V* out = (V*)p.out + out_base;
+#pragma unroll 4
+  for (uint32_t i = 0; i < 16; i++) {
+    const uint32_t a = y0 + 4 * i;
+    if (a0 + a < p.tile_a && c0 + x < p.tile_c) tile[a][x] = in[(size_t)(a0 + a) * p.a_stride + c0 + x];
+  }
+  __syncthreads();
+#pragma unroll 4
+  for (uint32_t i = 0; i < 16; i++) {
+    const uint32_t c = y0 + 4 * i;
+    if (c0 + c < p.tile_c && a0 + x < p.tile_a) out[(size_t)(c0 + c) * p.c_out_stride + a0 + x] = tile[x][c];
+  }
+}
+#define DEF_PERMUTE(B, V)                                                                              \
+  HC_KERNEL void hc_permute_rows_b##B##_v1(hck_permute_args p) { permute_rows_impl<V, 1>(p); }         \
+  HC_KERNEL void hc_permute_rows_b##B##_vN(hck_permute_args p) { permute_rows_impl<V, 16 / B>(p); }    \
+  HC_KERNEL void hc_permute_tile_b##B(hck_permute_args p) { permute_tile_impl<V>(p); }
+DEF_PERMUTE(8, uint64_t)
+DEF_PERMUTE(4, uint32_t)
+DEF_PERMUTE(2, uint16_t)
+DEF_PERMUTE(1, uint8_t)
+
 // triangular (BackendCPU.swift:1315-1348): keep the lower (upper) triangle shifted by
 // `offset`, zero elsewhere. Row j keeps columns [0, j+1+offset) or [j+offset, cols).
 template <typename V> __device__ __forceinline__ void triangular_impl(const hck_triangular_args& p) {

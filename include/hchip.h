@@ -318,6 +318,16 @@ int hc_fill(hc_ctx* ctx, int dtype, float vf, int64_t vi, void* out, size_t coun
 int hc_axis_permutation(hc_ctx* ctx, const int64_t* perm, const int64_t* shape, int ndim,
                         void* out);
 
+/* The gather that Tensor.t / swap / move / PermuteAxes issue right after axisPermutation
+ * (Index.swift:238-266: gather(axis 0 of [count, inner], indices = the permutation vector)), as one
+ * direct copy: out[new axes..., k] = in[old axes..., k] with new axis d = old axis perm[d], `shape`
+ * the extents of the permuted (leading) old axes and `inner` the number of untouched trailing
+ * elements per position. Same bytes as hc_axis_permutation + hc_gather, without the 8-byte index
+ * per element: rows move as 16-byte vectors, a moved innermost axis goes through 64 x 64 LDS tiles.
+ * A backend may hand out the index vector lazily and call this when the consumer is that gather. */
+int hc_permute(hc_ctx* ctx, int dtype, const void* in, const int64_t* perm, const int64_t* shape,
+               int ndim, int64_t inner, void* out);
+
 /* Backend.concat (Backend.swift:777-784; CPU BackendCPU.swift:1768-1794): `inputs` and
  * `inner_counts` are host arrays of n_inputs entries (device pointers / element counts). */
 int hc_concat(hc_ctx* ctx, int dtype, const void* const* inputs, const int64_t* inner_counts,

@@ -42,6 +42,8 @@ open class HIPBackend: CPUBackend, @unchecked Sendable {
     public let backend: HIPBackend
     public let pointer: UnsafeMutableRawPointer
     public let byteCount: Int
+    /// Set by axisPermutation: what this index vector permutes (lets gather copy directly).
+    public var permutation: (permutation: [Int], shape: [Int])? = nil
 
     init(backend: HIPBackend, byteCount: Int) throws {
       self.backend = backend
@@ -251,6 +253,28 @@ open class HIPBackend: CPUBackend, @unchecked Sendable {
     var st = hcStrides(s.indices.strides)
     let out = try output(s.gatherOutCount * dtype.byteSize)
     let axis = s.axis
+    // The gather of t / swap / move / PermuteAxes (Index.swift:238-266): indices from
+    // axisPermutation that run along the gathered axis only. hc_permute moves the same bytes
+    // without reading 8 bytes of index per element.
+    if let meta = di.permutation, s.indices.strides.shape[axis] == meta.shape.product(),
+      s.valueShape[axis] == meta.shape.product(),
+      zip(s.indices.strides.shape, s.indices.strides.strides).enumerated().allSatisfy({ ax, e in
+        e.0 == 1 || e.1 == (ax == axis ? 1 : 0)
+      })
+    {
+      var perm = meta.permutation.map { Int64($0) }
+      var shape = meta.shape.map { Int64($0) }
+      let outer = s.valueShape[..<axis].product()
+      if outer > 1 {
+        perm = [0] + perm.map { $0 + 1 }
+        shape = [Int64(outer)] + shape
+      }
+      try check(
+        hc_permute(
+          ctx, hcDType(dtype), da.pointer, perm, shape, Int32(shape.count),
+          Int64(s.valueShape[(axis + 1)...].product()), out.pointer))
+      return out
+    }
     try check(
       hc_gather(
         ctx, hcDType(dtype), da.pointer, di.pointer, &st, out.pointer,
@@ -277,6 +301,7 @@ open class HIPBackend: CPUBackend, @unchecked Sendable {
     let out = try output(shape.product() * Tensor.DType.int64.byteSize)
     let (perm, shp) = (permutation.map { Int64($0) }, shape.map { Int64($0) })
     try check(hc_axis_permutation(ctx, perm, shp, Int32(shape.count), out.pointer))
+    out.permutation = (permutation, shape)
     permutationCacheLock.withLock {
       if !isCapturing && permutationCacheBytes + out.byteCount <= 256 << 20 {
         permutationCache[key] = out

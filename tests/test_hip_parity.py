@@ -547,6 +547,45 @@ def test_axis_permutation(hip_backend, oracle_backend):
         check_exact(hip_backend, oracle_backend, fn)
 
 
+@pytest.mark.parametrize("dtype", [F32, F16, I64, BOOL], ids=["f32", "f16", "i64", "bool"])
+def test_permuted_views_take_the_direct_copy(hip_backend, oracle_backend, dtype):
+    """t / swap / move / PermuteAxes: the gather whose indices come from axisPermutation runs as
+    one direct copy (rows as vectors, a moved innermost axis through LDS tiles). Same result as the
+    oracle's gather and as numpy's transpose, bit for bit, for every element size, ragged tiles,
+    batch prefixes, odd row lengths, and the index vector itself stays readable."""
+    rng = np.random.default_rng(61)
+    cases = [((100, 70), (1, 0)), ((64, 64), (1, 0)), ((1, 300), (1, 0)), ((129, 1), (1, 0)),
+             ((6, 33, 65), (0, 2, 1)), ((5, 8, 16, 32), (0, 2, 1, 3)), ((5, 8, 16, 6), (2, 0, 1, 3)),
+             ((3, 4, 5, 6), (3, 2, 1, 0)), ((7, 9, 11), (2, 0, 1)), ((4, 40, 24), (1, 0, 2)),
+             ((2, 3, 130, 67), (0, 1, 3, 2)), ((2050, 3), (1, 0)), ((8, 256, 8, 64), (0, 2, 1, 3))]
+    for shape, perm in cases:
+        x = rng.integers(0, 2, size=shape) if dtype == BOOL else rand(rng, shape, dtype)
+        print("permute", dtype.name, shape, perm, flush=True)
+        n = len(perm)
+        lead = 0
+        while lead < n and perm[lead] == lead:
+            lead += 1
+        from honeycrisp_amd.tensor import FullRange, PermuteAxes
+        def fn():
+            t = Tensor(data=x, dtype=dtype)
+            return t[PermuteAxes(*perm)]
+        check_exact(hip_backend, oracle_backend, fn)
+        with hip_backend.use():
+            got = fn().numpy()
+        assert np.array_equal(got, np.ascontiguousarray(np.transpose(np.asarray(x).astype(got.dtype), perm)))
+    # the 2-D helpers, with a batch prefix
+    y = rand(rng, (3, 50, 70), F32)
+    check_exact(hip_backend, oracle_backend, lambda: Tensor(data=y).t())
+    check_exact(hip_backend, oracle_backend, lambda: Tensor(data=y).swap(0, 2))
+    check_exact(hip_backend, oracle_backend, lambda: Tensor(data=y).move(2, 0))
+    # the index vector is still a tensor like any other
+    from honeycrisp_amd.backend import Backend
+    def indices():
+        data = Backend.current().axisPermutation([1, 0], [50, 70])
+        return Tensor(dataHandle=data, shape=[3500], dtype=I64) + 1
+    check_exact(hip_backend, oracle_backend, indices)
+
+
 # ---------------------------------------------------------------- config 4 at full size
 
 def test_bandwidth_ops_full_size(hip_backend, oracle_backend):
