@@ -38,6 +38,11 @@ def test_status_codes_for_bad_arguments(hip_backend):
     bad = _lib.hc_strides()
     bad.ndim = 9
     assert lib.hc_broadcast(ctx, int(DType.float32), p, byref(bad), p) == _lib.HC_ERR_INVALID
+    # a permutation that repeats an axis, too many axes, an empty tensor
+    two = (c_int64 * 2)
+    assert lib.hc_permute(ctx, int(DType.float32), p, two(0, 0), two(4, 4), 2, 1, p) == _lib.HC_ERR_INVALID
+    assert lib.hc_permute(ctx, int(DType.float32), p, two(1, 0), two(4, 4), 9, 1, p) == _lib.HC_ERR_INVALID
+    assert lib.hc_permute(ctx, int(DType.float32), None, two(1, 0), two(4, 0), 2, 1, None) == _lib.HC_OK
     # freeing something the context never handed out, or twice
     assert lib.hc_free(ctx, c_void_p(buf.ptr + 64)) == _lib.HC_ERR_INVALID
     q = c_void_p()
