@@ -1086,7 +1086,14 @@ static int reduce_cols(hc_ctx* ctx, const char* opname, int dtype, const void* i
                        int64_t outer, int64_t reduce, int64_t inner, bool arg) {
   const size_t el = dtype_size(dtype);
   const uint32_t vec = (aligned16(in) && ((uint64_t)inner * el) % 16 == 0) ? (uint32_t)(16 / el) : 1;
-  const uint64_t jblocks = ceil_div(ceil_div((uint64_t)inner, vec), 64);
+  // lanes of a wave along inner: a power of two that covers it, at most 64
+  auto lanes_for = [](uint64_t jvecs) {
+    uint32_t jl = 1;
+    while (jl < 64 && jl < jvecs) jl <<= 1;
+    return jl;
+  };
+  const uint32_t jl = lanes_for(ceil_div((uint64_t)inner, vec)), jl_final = lanes_for((uint64_t)inner);
+  const uint64_t jblocks = ceil_div(ceil_div((uint64_t)inner, vec), jl);
   const uint64_t base_blocks = jblocks * (uint64_t)outer;
   const uint64_t want = (uint64_t)ctx->props.multiProcessorCount * 8;
   uint64_t splits = base_blocks >= want ? 1 : ceil_div(want, base_blocks);
@@ -1101,6 +1108,8 @@ static int reduce_cols(hc_ctx* ctx, const char* opname, int dtype, const void* i
   c.outer = (uint32_t)outer;
   c.reduce = (uint32_t)reduce;
   c.inner = (uint32_t)inner;
+  c.jl = jl;
+  c.jl_final = jl_final;
   c.chunk = (uint32_t)(ceil_div(ceil_div((uint64_t)reduce, splits), 4) * 4);
   if (c.chunk == 0) c.chunk = 4;
   splits = reduce ? ceil_div((uint64_t)reduce, c.chunk) : 1;
@@ -1120,7 +1129,7 @@ static int reduce_cols(hc_ctx* ctx, const char* opname, int dtype, const void* i
   HC_TRY(launch(ctx, name, base_blocks * splits, 1, &c, sizeof(c)));
   if (splits > 1) {
     snprintf(name, sizeof(name), "hc_reduce_cols_final_%s_%s", opname, dtype_name(dtype));
-    HC_TRY(launch(ctx, name, ceil_div((uint64_t)inner, 64) * (uint64_t)outer, 1, &c, sizeof(c)));
+    HC_TRY(launch(ctx, name, ceil_div((uint64_t)inner, jl_final) * (uint64_t)outer, 1, &c, sizeof(c)));
   }
   return HC_OK;
 }
@@ -1220,6 +1229,7 @@ extern "C" int hc_reduce(hc_ctx* ctx, int op, int dtype, const void* in, void* o
         c.inner = 1;
         c.splits = (uint32_t)segs;
         c.chunk = (uint32_t)seg_len;
+        c.jl_final = 1;  // one column: all 64 lanes of a wave along the partials
         snprintf(name, sizeof(name), "hc_reduce_cols_final_%s_%s", kReduceNames[op], dtype_name(dtype));
         return launch(ctx, name, (uint64_t)outer, 1, &c, sizeof(c));
       }

@@ -111,8 +111,12 @@ typedef struct {
   uint32_t inner;
   uint32_t splits;
   uint32_t chunk;
-  uint32_t pad;
+  /* lanes of a wave along inner (a power of two <= 64); the other 64 / jl lanes of the wave
+   * take further rows. 0 = 64. The final pass over the partials uses jl_final. */
+  uint32_t jl;
   const float* aux; /* exp-sum: the per-column maximum, [outer, inner] */
+  uint32_t jl_final;
+  uint32_t pad;
 } hck_reduce_cols_args;
 
 /* Column logSoftmax / logSoftmaxGrad, last step: every element combined with per-column

@@ -205,8 +205,9 @@ __device__ __forceinline__ void reduce_rows_impl(const hck_reduce_args& p) {
 
 // ---------------------------------------------------------------- columns (inner > 1)
 
-// Block = 64 lanes along inner, VEC consecutive columns per lane (16-byte loads when the row
-// pitch allows), x 4 waves along the reduce axis, meeting in LDS. The reduce axis is also
+// Block = up to 64 lanes along inner, VEC consecutive columns per lane (16-byte loads when the row
+// pitch allows), x 4 waves along the reduce axis, meeting in LDS. When inner is narrower than a
+// wave (jl < 64 lanes cover it), the wave's other lanes take further rows and meet by shuffles. The reduce axis is also
 // cut into `splits` ranges handled by different blocks so that a tall, narrow input still
 // fills the device; with splits > 1 the ranges leave partials (accumulator type, plus the
 // index for arg-reductions) and the same kernel runs a second time with FINAL = true over
@@ -220,14 +221,18 @@ __device__ __forceinline__ void reduce_cols_impl(const hck_reduce_cols_args& p) 
   const uint32_t splits = FINAL ? 1 : p.splits;
   const uint32_t chunk = FINAL ? p.splits : p.chunk;
   const uint32_t jvecs = (p.inner + VEC - 1) / VEC;
-  const uint32_t jblocks = (jvecs + 63) / 64;
+  const uint32_t jl_arg = FINAL ? p.jl_final : p.jl;
+  const uint32_t jl = jl_arg ? jl_arg : 64;   // lanes along inner
+  const uint32_t rl = 64 / jl;                // rows per wave and step
+  const uint32_t jblocks = (jvecs + jl - 1) / jl;
   uint32_t bid = blockIdx.x;
   const uint32_t jb = bid % jblocks;
   bid /= jblocks;
   const uint32_t s = bid % splits;
   const uint32_t i = bid / splits;
   const uint32_t lane = threadIdx.x & 63, kw = threadIdx.x >> 6;
-  const uint32_t j = (jb * 64 + lane) * VEC;
+  const uint32_t jlane = lane & (jl - 1), rsub = lane / jl;
+  const uint32_t j = (jb * jl + jlane) * VEC;
   const bool active = j < p.inner;
   const uint32_t k_begin = s * chunk;
   const uint32_t k_end = k_begin + chunk < extent ? k_begin + chunk : extent;
@@ -266,28 +271,45 @@ __device__ __forceinline__ void reduce_cols_impl(const hck_reduce_cols_args& p) 
     }
   };
   if (active) {
-    uint32_t k = k_begin + kw;
+    const uint32_t step = 4 * rl;  // rows the block covers per step
+    uint32_t k = k_begin + kw * rl + rsub;
     constexpr int U = 8;  // rows in flight per lane
-    for (; k + 4 * (U - 1) < k_end; k += 4 * U) {
+    for (; k + step * (U - 1) < k_end; k += step * U) {
       S a[U][VEC];
 #pragma unroll
-      for (int u = 0; u < U; u++) load_vec<S, VEC>(in + (size_t)(k + 4 * u) * p.inner, 0, 1, a[u]);
+      for (int u = 0; u < U; u++) load_vec<S, VEC>(in + (size_t)(k + step * u) * p.inner, 0, 1, a[u]);
 #pragma unroll
-      for (int u = 0; u < U; u++) take(a[u], k + 4 * u);
+      for (int u = 0; u < U; u++) take(a[u], k + step * u);
     }
-    for (; k < k_end; k += 4) {
+    for (; k < k_end; k += step) {
       S a[VEC];
       load_vec<S, VEC>(in + (size_t)k * p.inner, 0, 1, a);
       take(a, k);
     }
   }
+  // the wave's row groups meet in the lanes of group 0 (every lane takes part; idle ones hold
+  // the identity / the worst pair)
+  for (uint32_t o = jl; o < 64; o <<= 1) {
+#pragma unroll
+    for (int e = 0; e < VEC; e++) {
+      if (ARG) {
+        ArgPair<C> q;
+        q.v = __shfl_xor(best[e].v, o, 64);
+        q.i = __shfl_xor(best[e].i, o, 64);
+        best[e] = arg_better<OP>(best[e], q);
+      } else {
+        acc[e] = reduce_combine<OP, C>(acc[e], __shfl_xor(acc[e], o, 64));
+      }
+    }
+  }
+  const bool writer = kw == 0 && rsub == 0 && active;
   const bool last = FINAL || p.splits == 1;  // this pass writes the result itself
   if (ARG) {
     ArgPair<C>* lds = (ArgPair<C>*)lds_raw;
 #pragma unroll
     for (int e = 0; e < VEC; e++) lds[threadIdx.x * VEC + e] = best[e];
     __syncthreads();
-    if (kw == 0 && active) {
+    if (writer) {
 #pragma unroll
       for (int e = 0; e < VEC; e++) {
         for (int w = 1; w < 4; w++) best[e] = arg_better<OP>(best[e], lds[(threadIdx.x + 64 * w) * VEC + e]);
@@ -305,7 +327,7 @@ __device__ __forceinline__ void reduce_cols_impl(const hck_reduce_cols_args& p) 
 #pragma unroll
     for (int e = 0; e < VEC; e++) lds[threadIdx.x * VEC + e] = acc[e];
     __syncthreads();
-    if (kw == 0 && active) {
+    if (writer) {
 #pragma unroll
       for (int e = 0; e < VEC; e++) {
         for (int w = 1; w < 4; w++) acc[e] = reduce_combine<OP, C>(acc[e], lds[(threadIdx.x + 64 * w) * VEC + e]);

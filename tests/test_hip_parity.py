@@ -421,7 +421,9 @@ REDUCE_SHAPES = [(8, 4096, 1), (37, 513, 1), (5, 1, 1), (3, 7, 1), (1, 100000, 1
                  (2, 5000, 96), (1, 4097, 260), (1, 70000, 8),
                  # rows of a few elements (a lane or 8 lanes per row) and few long rows (cut into
                  # segments that leave partials; 300001 is odd, so its segments are read element-wise)
-                 (70000, 3, 1), (5000, 8, 1), (4097, 100, 1), (1, 400000, 1), (3, 300001, 1), (2, 65536, 1)]
+                 (70000, 3, 1), (5000, 8, 1), (4097, 100, 1), (1, 400000, 1), (3, 300001, 1), (2, 65536, 1),
+                 # inner narrower than a wave: the wave's other lanes take further rows
+                 (1, 100000, 3), (2, 30000, 64), (3, 1000, 20), (5, 77, 1), (1, 9000, 5)]
 
 
 @pytest.mark.parametrize("dtype", [F32, F16, I64], ids=["f32", "f16", "i64"])
@@ -500,7 +502,8 @@ def test_log_softmax_and_normalize(hip_backend, oracle_backend, dtype):
     for shape, axis in [((64, 256), 1), ((16, 8, 32, 32), 3), ((5, 1000), 1), ((7, 33, 9), 1), ((300, 4), 0),
                         ((2, 1), 1), ((3, 10000), 1), ((4096, 96), 0), ((2, 3000, 40), 1), ((3, 129, 7), 1),
                         # short rows: a lane or 8 lanes per row
-                        ((7000, 3), 1), ((3001, 8), 1), ((1000, 100), 1), ((999, 128), 1), ((500, 16), 1)]:
+                        ((7000, 3), 1), ((3001, 8), 1), ((1000, 100), 1), ((999, 128), 1), ((500, 16), 1),
+                        ((30000, 3), 0), ((5000, 64), 0), ((2, 900, 20), 1)]:
         x = rand(rng, shape, dtype, 3.0)
         print("logsoftmax/normalize", dtype.name, shape, axis, flush=True)
         check_close(hip_backend, oracle_backend, lambda: Tensor(data=x).logSoftmax(axis=axis), TOL[dtype])
