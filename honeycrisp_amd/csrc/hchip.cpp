@@ -1892,8 +1892,19 @@ extern "C" int hc_permute(hc_ctx* ctx, int dtype, const void* in, const int64_t*
   k.a_stride = (uint32_t)ax[n - 1].stride;
   k.tile_c = (uint32_t)ax[c].extent;
   k.c_out_stride = (uint32_t)out_stride[c];
-  k.tiles_a = (uint32_t)ceil_div(ax[n - 1].extent, 64);
-  k.tiles_c = (uint32_t)ceil_div(ax[c].extent, 64);
+  // 64 x 64 tiles; when one of the two axes is shorter, the tile grows along the other (4096 elements)
+  auto log2_ceil = [](uint64_t v) {
+    uint32_t l = 0;
+    while ((1ull << l) < v) l++;
+    return l;
+  };
+  const uint32_t la = log2_ceil(ax[n - 1].extent), lc = log2_ceil(ax[c].extent);
+  k.ta_log2 = std::min<uint32_t>(la, 6);
+  k.tc_log2 = std::min<uint32_t>(lc, 6);
+  if (k.tc_log2 < 6) k.ta_log2 = std::min<uint32_t>(la, std::min<uint32_t>(12 - k.tc_log2, 10));  // (LDS rows are padded)
+  if (k.ta_log2 < 6) k.tc_log2 = std::min<uint32_t>(lc, 12 - k.ta_log2);
+  k.tiles_a = (uint32_t)ceil_div(ax[n - 1].extent, 1ull << k.ta_log2);
+  k.tiles_c = (uint32_t)ceil_div(ax[c].extent, 1ull << k.tc_log2);
   hck_fast_div_setup(k.tiles_a, &k.tiles_a_magic, &k.tiles_a_sh);
   hck_fast_div_setup(k.tiles_c, &k.tiles_c_magic, &k.tiles_c_sh);
   uint64_t batch = 1;

@@ -243,8 +243,8 @@ typedef struct {
  * Row form: the innermost axis is contiguous in both; a lane moves `vec` of its `inner` elements, the
  * row number is unravelled over shape[0..ndim) (divisions by multiply-high, hck_fast_div_setup).
  * Tile form: the output's innermost axis (extent tile_a, source stride a_stride) differs from the
- * source's (extent tile_c, output stride c_out_stride): 64 x 64 tiles go through LDS, read along
- * the source's innermost axis and written along the output's; shape[]/in_stride[]/out_stride[] then
+ * source's (extent tile_c, output stride c_out_stride): tiles of 2^ta_log2 x 2^tc_log2 elements go
+ * through LDS, read along the source's innermost axis and written along the output's; shape[]/in_stride[]/out_stride[] then
  * describe the remaining axes. */
 typedef struct {
   const void* in;
@@ -262,6 +262,7 @@ typedef struct {
   uint32_t tile_a, tile_c, a_stride, c_out_stride;
   uint32_t tiles_a, tiles_c;
   uint32_t tiles_a_magic, tiles_a_sh, tiles_c_magic, tiles_c_sh;
+  uint32_t ta_log2, tc_log2; /* tile extents along a and c: powers of two, product <= 4096 */
 } hck_permute_args;
 
 typedef struct {

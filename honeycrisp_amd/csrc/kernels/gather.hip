@@ -281,16 +281,18 @@ template <typename V, int VEC> __device__ __forceinline__ void permute_rows_impl
   typedef Vec<V, VEC> Pack;
   *reinterpret_cast<Pack*>((V*)p.out + out_off) = *reinterpret_cast<const Pack*>((const V*)p.in + in_off);
 }
-// Tile form: 64 x 64 elements through LDS. Reads run along the source's innermost axis c, writes
-// along the output's innermost axis a; one padding element per LDS row keeps both off the same banks.
+// Tile form: tiles of ta x tc elements (powers of two, ta * tc <= 4096: 64 x 64, or longer and
+// narrower when one of the two axes is short) through LDS. Reads run along the source's innermost
+// axis c, writes along the output's innermost axis a, both with all lanes on consecutive
+// elements; one padding element per LDS row keeps the transposed accesses off the same banks.
 template <typename V> __device__ __forceinline__ void permute_tile_impl(const hck_permute_args& p) {
-  __shared__ V tile[64][65];
+  __shared__ V tile[4096 + 1024];
   uint32_t t = blockIdx.x;
   uint32_t q = fast_div(t, p.tiles_c_magic, p.tiles_c_sh);
-  const uint32_t c0 = (t - q * p.tiles_c) * 64;
+  const uint32_t c0 = (t - q * p.tiles_c) << p.tc_log2;
   t = q;
   q = fast_div(t, p.tiles_a_magic, p.tiles_a_sh);
-  const uint32_t a0 = (t - q * p.tiles_a) * 64;
+  const uint32_t a0 = (t - q * p.tiles_a) << p.ta_log2;
   uint32_t rest = q;
   size_t in_base = 0, out_base = 0;
   for (int d = (int)p.ndim - 1; d >= 0; d--) {
@@ -300,19 +302,33 @@ template <typename V> __device__ __forceinline__ void permute_tile_impl(const hc
     out_base += (size_t)r * p.out_stride[d];
     rest = qq;
   }
-  const uint32_t x = threadIdx.x & 63, y0 = threadIdx.x >> 6;
   const V* in = (const V*)p.in + in_base;
   V* out = (V*)p.out + out_base;
+  if (p.ta_log2 == 6 && p.tc_log2 == 6) {
+    // the common shape, with compile-time extents
+    const uint32_t x = threadIdx.x & 63, y0 = threadIdx.x >> 6;
 #pragma unroll 4
-  for (uint32_t i = 0; i < 16; i++) {
-    const uint32_t a = y0 + 4 * i;
-    if (a0 + a < p.tile_a && c0 + x < p.tile_c) tile[a][x] = in[(size_t)(a0 + a) * p.a_stride + c0 + x];
+    for (uint32_t i = 0; i < 16; i++) {
+      const uint32_t a = y0 + 4 * i;
+      if (a0 + a < p.tile_a && c0 + x < p.tile_c) tile[a * 65 + x] = in[(size_t)(a0 + a) * p.a_stride + c0 + x];
+    }
+    __syncthreads();
+#pragma unroll 4
+    for (uint32_t i = 0; i < 16; i++) {
+      const uint32_t c = y0 + 4 * i;
+      if (c0 + c < p.tile_c && a0 + x < p.tile_a) out[(size_t)(c0 + c) * p.c_out_stride + a0 + x] = tile[x * 65 + c];
+    }
+    return;
+  }
+  const uint32_t n = 1u << (p.ta_log2 + p.tc_log2), pitch = (1u << p.tc_log2) + 1;
+  for (uint32_t idx = threadIdx.x; idx < n; idx += HCK_BLOCK) {
+    const uint32_t a = idx >> p.tc_log2, c = idx & ((1u << p.tc_log2) - 1);
+    if (a0 + a < p.tile_a && c0 + c < p.tile_c) tile[a * pitch + c] = in[(size_t)(a0 + a) * p.a_stride + c0 + c];
   }
   __syncthreads();
-#pragma unroll 4
-  for (uint32_t i = 0; i < 16; i++) {
-    const uint32_t c = y0 + 4 * i;
-    if (c0 + c < p.tile_c && a0 + x < p.tile_a) out[(size_t)(c0 + c) * p.c_out_stride + a0 + x] = tile[x][c];
+  for (uint32_t idx = threadIdx.x; idx < n; idx += HCK_BLOCK) {
+    const uint32_t c = idx >> p.ta_log2, a = idx & ((1u << p.ta_log2) - 1);
+    if (a0 + a < p.tile_a && c0 + c < p.tile_c) out[(size_t)(c0 + c) * p.c_out_stride + a0 + a] = tile[a * pitch + c];
   }
 }
 #define DEF_PERMUTE(B, V)                                                                              \

@@ -560,7 +560,9 @@ def test_permuted_views_take_the_direct_copy(hip_backend, oracle_backend, dtype)
     cases = [((100, 70), (1, 0)), ((64, 64), (1, 0)), ((1, 300), (1, 0)), ((129, 1), (1, 0)),
              ((6, 33, 65), (0, 2, 1)), ((5, 8, 16, 32), (0, 2, 1, 3)), ((5, 8, 16, 6), (2, 0, 1, 3)),
              ((3, 4, 5, 6), (3, 2, 1, 0)), ((7, 9, 11), (2, 0, 1)), ((4, 40, 24), (1, 0, 2)),
-             ((2, 3, 130, 67), (0, 1, 3, 2)), ((2050, 3), (1, 0)), ((8, 256, 8, 64), (0, 2, 1, 3))]
+             ((2, 3, 130, 67), (0, 1, 3, 2)), ((2050, 3), (1, 0)), ((8, 256, 8, 64), (0, 2, 1, 3)),
+             # one of the two transposed axes short: long narrow tiles
+             ((5000, 2), (1, 0)), ((2, 5000), (1, 0)), ((3, 1500, 5), (0, 2, 1)), ((7, 3000), (1, 0)), ((1100, 20), (1, 0))]
     for shape, perm in cases:
         x = rng.integers(0, 2, size=shape) if dtype == BOOL else rand(rng, shape, dtype)
         print("permute", dtype.name, shape, perm, flush=True)
