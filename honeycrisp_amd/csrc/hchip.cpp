@@ -1402,7 +1402,10 @@ extern "C" int hc_log_softmax(hc_ctx* ctx, int dtype, const void* in, void* out,
   k.reduce = (uint32_t)reduce;
   k.inner = (uint32_t)inner;
   char name[64];
-  if (inner == 1) {
+  // (few long rows: a block per row would leave most of the device idle; the column path cuts the
+  // axis over many blocks)
+  const bool few_long_rows = inner == 1 && (uint64_t)outer < 2 * (uint64_t)ctx->props.multiProcessorCount && reduce >= 32768;
+  if (inner == 1 && !few_long_rows) {
     // a lane or 8 lanes per row for short rows, a wave per row while the row fits its registers
     // (4 x 16 bytes per lane), else a block
     if (reduce <= 128) {
@@ -1439,7 +1442,10 @@ extern "C" int hc_log_softmax_grad(hc_ctx* ctx, int dtype, const void* in, const
   k.reduce = (uint32_t)reduce;
   k.inner = (uint32_t)inner;
   char name[64];
-  if (inner == 1) {
+  // (few long rows: a block per row would leave most of the device idle; the column path cuts the
+  // axis over many blocks)
+  const bool few_long_rows = inner == 1 && (uint64_t)outer < 2 * (uint64_t)ctx->props.multiProcessorCount && reduce >= 32768;
+  if (inner == 1 && !few_long_rows) {
     // a lane or 8 lanes per row for short rows, a wave per row while the row fits its registers
     // (4 x 16 bytes per lane), else a block
     if (reduce <= 128) {
@@ -1468,7 +1474,10 @@ extern "C" int hc_normalize(hc_ctx* ctx, int dtype, const void* in, void* out, i
   REQUIRE(in && out, "hc_normalize: null pointer");
   REQUIRE(aligned16(in) && aligned16(out), "hc_normalize: buffers must be 16-byte aligned");
   const size_t el_size = dtype_size(dtype);
-  if (inner == 1) {
+  // (few long rows: a block per row would leave most of the device idle; the op-by-op composition
+  // below runs every step over the whole device, at the price of nine launches)
+  const bool few_long_rows = inner == 1 && (uint64_t)outer * 8 < (uint64_t)ctx->props.multiProcessorCount && reduce >= 32768;
+  if (inner == 1 && !few_long_rows) {
     hck_reduce_args k;
     memset(&k, 0, sizeof(k));
     k.in = in;

@@ -503,7 +503,9 @@ def test_log_softmax_and_normalize(hip_backend, oracle_backend, dtype):
                         ((2, 1), 1), ((3, 10000), 1), ((4096, 96), 0), ((2, 3000, 40), 1), ((3, 129, 7), 1),
                         # short rows: a lane or 8 lanes per row
                         ((7000, 3), 1), ((3001, 8), 1), ((1000, 100), 1), ((999, 128), 1), ((500, 16), 1),
-                        ((30000, 3), 0), ((5000, 64), 0), ((2, 900, 20), 1)]:
+                        ((30000, 3), 0), ((5000, 64), 0), ((2, 900, 20), 1),
+                        # few long rows: cut over many blocks (column path / op-by-op composition)
+                        ((2, 70000), 1), ((1, 40001), 1)]:
         x = rand(rng, shape, dtype, 3.0)
         print("logsoftmax/normalize", dtype.name, shape, axis, flush=True)
         check_close(hip_backend, oracle_backend, lambda: Tensor(data=x).logSoftmax(axis=axis), TOL[dtype])
@@ -689,7 +691,7 @@ def test_log_softmax_grad(hip_backend, oracle_backend, dtype):
     rng = np.random.default_rng(33)
     for shape, axis in [((64, 300), 1), ((7, 33, 40), 1), ((5, 1, 9), 2), ((3, 1000), 0), ((2048, 256), 1),
                         ((4096, 96), 0), ((2, 3000, 40), 1), ((16, 5000), 1), ((9, 33000), 1),
-                        ((7000, 3), 1), ((3001, 8), 1), ((1000, 100), 1), ((999, 128), 1)]:
+                        ((7000, 3), 1), ((3001, 8), 1), ((1000, 100), 1), ((999, 128), 1), ((2, 70000), 1)]:
         x, g = rand(rng, shape, dtype, 2.0), rand(rng, shape, dtype)
         def run():
             xt, gt = Tensor(data=x), Tensor(data=g)
