@@ -1160,6 +1160,7 @@ static int softmax_cols(hc_ctx* ctx, int dtype, const void* in, const void* grad
   k.outer = (uint32_t)outer;
   k.reduce = (uint32_t)reduce;
   k.inner = (uint32_t)inner;
+  HC_TRY(launch(ctx, "hc_log_softmax_cols_logsum", ceil_div((uint64_t)cols, HCK_BLOCK), 1, &k, sizeof(k)));
   const size_t el = dtype_size(dtype);
   const uint32_t vec = ((uint64_t)inner * el) % 16 == 0 ? (uint32_t)(16 / el) : 1;
   char name[64];

@@ -126,7 +126,7 @@ typedef struct {
   const void* grad; /* logSoftmaxGrad only */
   void* out;
   const float* col_max;
-  const float* col_expsum;
+  const float* col_expsum;  /* hc_log_softmax_cols_logsum turns it into logf(exp-sum) + maximum in place */
   const float* col_gradsum; /* logSoftmaxGrad only */
   uint32_t outer, reduce, inner, pad;
 } hck_softmax_cols_args;

@@ -518,12 +518,20 @@ template <typename T, int VEC, bool GRAD> __device__ __forceinline__ void softma
 #pragma unroll
   for (int e = 0; e < VEC; e++) {
     if (j + e < p.inner) {
-      const float log_sum = logf(p.col_expsum[col + e]) + p.col_max[col + e];
+      const float log_sum = p.col_expsum[col + e];  // (already logf(exp-sum) + maximum, see below)
       if (GRAD) o[e] = narrow<T>((float)g[e] - p.col_gradsum[col + e] * expf((float)x[e] - log_sum));
       else o[e] = narrow<T>((float)x[e] - log_sum);
     }
   }
   store_vec<T, VEC>((T*)p.out, off, o);
+}
+// exp-sum -> logf(exp-sum) + maximum, once per column and in place (the apply pass would
+// otherwise evaluate logf once per element).
+HC_KERNEL void hc_log_softmax_cols_logsum(hck_softmax_cols_args p) {
+  const uint64_t t = (uint64_t)blockIdx.x * HCK_BLOCK + threadIdx.x;
+  if (t >= (uint64_t)p.outer * p.inner) return;
+  float* s = const_cast<float*>(p.col_expsum);
+  s[t] = logf(s[t]) + p.col_max[t];
 }
 #define DEF_SOFTMAX_COLS(TN, T)                                                                        \
   HC_KERNEL void hc_reduce_cols_maxf_##TN##_v1(hck_reduce_cols_args p) { reduce_cols_impl<T, R_MAXF, 1, false>(p); } \
