@@ -1409,7 +1409,7 @@ extern "C" int hc_log_softmax(hc_ctx* ctx, int dtype, const void* in, void* out,
   if (inner == 1 && !few_long_rows) {
     // a lane or 8 lanes per row for short rows, a wave per row while the row fits its registers
     // (4 x 16 bytes per lane), else a block
-    if (reduce <= 128) {
+    if ((uint64_t)reduce * el_size <= 512) {  // (8 lanes x 4 x 16 bytes: the row still fits the team's registers)
       const uint32_t lanes = reduce <= 8 ? 1 : 8;
       snprintf(name, sizeof(name), "hc_log_softmax_rows%u_%s", lanes, dtype_name(dtype));
       return launch(ctx, name, ceil_div((uint64_t)outer, HCK_BLOCK / lanes), 1, &k, sizeof(k));
@@ -1449,7 +1449,7 @@ extern "C" int hc_log_softmax_grad(hc_ctx* ctx, int dtype, const void* in, const
   if (inner == 1 && !few_long_rows) {
     // a lane or 8 lanes per row for short rows, a wave per row while the row fits its registers
     // (4 x 16 bytes per lane), else a block
-    if (reduce <= 128) {
+    if ((uint64_t)reduce * el_size <= 512) {  // (8 lanes x 4 x 16 bytes: the row still fits the team's registers)
       const uint32_t lanes = reduce <= 8 ? 1 : 8;
       snprintf(name, sizeof(name), "hc_log_softmax_grad_rows%u_%s", lanes, dtype_name(dtype));
       return launch(ctx, name, ceil_div((uint64_t)outer, HCK_BLOCK / lanes), 1, &k, sizeof(k));
@@ -1490,7 +1490,7 @@ extern "C" int hc_normalize(hc_ctx* ctx, int dtype, const void* in, void* out, i
     char name[64];
     // a lane or 8 lanes per row for short rows, a wave per row while the row fits its registers
     // (4 x 16 bytes per lane), else a block
-    if (reduce <= 128) {
+    if ((uint64_t)reduce * el_size <= 512) {  // (8 lanes x 4 x 16 bytes: the row still fits the team's registers)
       const uint32_t lanes = reduce <= 8 ? 1 : 8;
       snprintf(name, sizeof(name), "hc_normalize_rows%u_%s", lanes, dtype_name(dtype));
       return launch(ctx, name, ceil_div((uint64_t)outer, HCK_BLOCK / lanes), 1, &k, sizeof(k));
