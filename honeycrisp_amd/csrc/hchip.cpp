@@ -1978,13 +1978,19 @@ extern "C" int hc_concat(hc_ctx* ctx, int dtype, const void* const* inputs, cons
       REQUIRE(inputs[t] && out, "hc_concat: null pointer");
       hck_concat_args k;
       memset(&k, 0, sizeof(k));
+      // the widest unit that every row piece and both addresses are multiples of
+      uint64_t unit = 16;
+      while (unit > 1 && ((bytes | total_inner | off | (uint64_t)(uintptr_t)inputs[t] | (uint64_t)(uintptr_t)out) & (unit - 1)) != 0)
+        unit >>= 1;
       k.in = inputs[t];
       k.out = out;
       k.outer = (uint32_t)outer;
-      k.inner = (uint32_t)bytes;
-      k.total_inner = (uint32_t)total_inner;
-      k.out_off = (uint32_t)off;
-      HC_TRY(launch(ctx, "hc_concat_bytes", ceil_div((uint64_t)outer * bytes, HCK_BLOCK), 1, &k, sizeof(k)));
+      k.inner = (uint32_t)(bytes / unit);
+      k.total_inner = (uint32_t)(total_inner / unit);
+      k.out_off = (uint32_t)(off / unit);
+      char name[32];
+      snprintf(name, sizeof(name), "hc_concat_b%u", (unsigned)unit);
+      HC_TRY(launch(ctx, name, ceil_div((uint64_t)outer * (bytes / unit), HCK_BLOCK), 1, &k, sizeof(k)));
     }
     off += bytes;
   }

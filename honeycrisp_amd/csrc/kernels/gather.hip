@@ -360,13 +360,20 @@ HC_KERNEL void hc_triangular_b4(hck_triangular_args p) { triangular_impl<uint32_
 HC_KERNEL void hc_triangular_b2(hck_triangular_args p) { triangular_impl<uint16_t>(p); }
 HC_KERNEL void hc_triangular_b1(hck_triangular_args p) { triangular_impl<uint8_t>(p); }
 
-// concat (BackendCPU.swift:1768-1794), one launch per input: byte copy of an
-// [outer, inner] block into a column range of the [outer, total_inner] output.
-HC_KERNEL void hc_concat_bytes(hck_concat_args p) {
+// concat (BackendCPU.swift:1768-1794), one launch per input: copy of an [outer, inner] block
+// into a column range of the [outer, total_inner] output, in units of U bytes: the host picks the
+// largest U <= 16 that divides the block's row length, the output's row length, the column offset
+// and both addresses. inner, total_inner and out_off count units.
+template <typename U> __device__ __forceinline__ void concat_impl(const hck_concat_args& p) {
   const uint64_t t = (uint64_t)blockIdx.x * HCK_BLOCK + threadIdx.x;
   const uint64_t total = (uint64_t)p.outer * p.inner;
   if (t >= total) return;
   const uint32_t o = (uint32_t)(t / p.inner);
   const uint32_t c = (uint32_t)(t - (uint64_t)o * p.inner);
-  ((uint8_t*)p.out)[(uint64_t)o * p.total_inner + p.out_off + c] = ((const uint8_t*)p.in)[t];
+  ((U*)p.out)[(uint64_t)o * p.total_inner + p.out_off + c] = ((const U*)p.in)[t];
 }
+HC_KERNEL void hc_concat_b1(hck_concat_args p) { concat_impl<uint8_t>(p); }
+HC_KERNEL void hc_concat_b2(hck_concat_args p) { concat_impl<uint16_t>(p); }
+HC_KERNEL void hc_concat_b4(hck_concat_args p) { concat_impl<uint32_t>(p); }
+HC_KERNEL void hc_concat_b8(hck_concat_args p) { concat_impl<uint64_t>(p); }
+HC_KERNEL void hc_concat_b16(hck_concat_args p) { concat_impl<V16>(p); }

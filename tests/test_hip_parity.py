@@ -407,6 +407,13 @@ def test_when_fill_triangular_concat_broadcast(hip_backend, oracle_backend):
                     lambda: Tensor.concat([Tensor(data=m, dtype=dtype), Tensor(data=m[:, :5], dtype=dtype)], axis=1))
         check_exact(hip_backend, oracle_backend,
                     lambda: Tensor.concat([Tensor(data=m, dtype=dtype), Tensor(data=m[:, :, :9], dtype=dtype)], axis=2))
+        # pieces whose widths allow 16-, 8-, 4- and 2-byte copy units, three inputs, axis 0
+        w = rand(rng, (9, 64), dtype) if dtype != BOOL else rng.integers(0, 2, size=(9, 64)).astype(np.bool_)
+        for widths in [(64, 32), (8, 64, 24), (4, 60), (2, 6, 64), (1, 63), (64, 64, 64)]:
+            check_exact(hip_backend, oracle_backend,
+                        lambda: Tensor.concat([Tensor(data=w[:, :c], dtype=dtype) for c in widths], axis=1))
+        check_exact(hip_backend, oracle_backend,
+                    lambda: Tensor.concat([Tensor(data=w, dtype=dtype), Tensor(data=w[:4], dtype=dtype), Tensor(data=w[:1], dtype=dtype)], axis=0))
         check_exact(hip_backend, oracle_backend, lambda: Tensor(data=b, dtype=dtype).expand([7, 3, 40]))
         check_exact(hip_backend, oracle_backend, lambda: Tensor(data=a, dtype=dtype).reshape([5, 1, 40]).expand([5, 6, 40]))
         check_exact(hip_backend, oracle_backend, lambda: Tensor(data=a, dtype=dtype).repeating(1, 3))
