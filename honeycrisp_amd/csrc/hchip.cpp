@@ -1953,7 +1953,13 @@ extern "C" int hc_triangular(hc_ctx* ctx, int dtype, const void* in, void* out, 
   k.upper = upper ? 1 : 0;
   k.offset = offset;
   char name[64];
-  snprintf(name, sizeof(name), "hc_triangular_b%zu", dtype_size(dtype));
+  const size_t el = dtype_size(dtype);
+  if (((uint64_t)cols * el) % 16 == 0 && aligned16(in) && aligned16(out)) {  // 16 bytes of a row per lane
+    k.total = (uint32_t)((uint64_t)k.total * el / 16);
+    snprintf(name, sizeof(name), "hc_triangular_b%zu_vN", el);
+    return launch(ctx, name, ceil_div(k.total, HCK_BLOCK), 1, &k, sizeof(k));
+  }
+  snprintf(name, sizeof(name), "hc_triangular_b%zu", el);
   return launch(ctx, name, ceil_div(k.total, HCK_BLOCK), 1, &k, sizeof(k));
 }
 

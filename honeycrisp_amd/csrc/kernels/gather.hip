@@ -355,6 +355,28 @@ template <typename V> __device__ __forceinline__ void triangular_impl(const hck_
   }
   ((V*)p.out)[o] = keep ? ((const V*)p.in)[o] : (V)0;
 }
+// The same with N = 16 / sizeof(V) consecutive columns per lane (cols a multiple of N, buffers
+// 16-byte aligned): p.total counts vectors.
+template <typename V> __device__ __forceinline__ void triangular_vec_impl(const hck_triangular_args& p) {
+  constexpr int N = 16 / sizeof(V);
+  const uint32_t v = blockIdx.x * HCK_BLOCK + threadIdx.x;
+  if (v >= p.total) return;
+  const uint32_t cvecs = p.cols / N;
+  const uint32_t col0 = (v % cvecs) * N;
+  const uint32_t row = (v / cvecs) % p.rows;
+  Vec<V, N> x = reinterpret_cast<const Vec<V, N>*>(p.in)[v];
+#pragma unroll
+  for (int e = 0; e < N; e++) {
+    const int64_t col = (int64_t)col0 + e;
+    const bool keep = p.upper ? col >= (int64_t)row + p.offset : col < (int64_t)row + 1 + p.offset;
+    if (!keep) x.v[e] = (V)0;
+  }
+  reinterpret_cast<Vec<V, N>*>(p.out)[v] = x;
+}
+HC_KERNEL void hc_triangular_b8_vN(hck_triangular_args p) { triangular_vec_impl<uint64_t>(p); }
+HC_KERNEL void hc_triangular_b4_vN(hck_triangular_args p) { triangular_vec_impl<uint32_t>(p); }
+HC_KERNEL void hc_triangular_b2_vN(hck_triangular_args p) { triangular_vec_impl<uint16_t>(p); }
+HC_KERNEL void hc_triangular_b1_vN(hck_triangular_args p) { triangular_vec_impl<uint8_t>(p); }
 HC_KERNEL void hc_triangular_b8(hck_triangular_args p) { triangular_impl<uint64_t>(p); }
 HC_KERNEL void hc_triangular_b4(hck_triangular_args p) { triangular_impl<uint32_t>(p); }
 HC_KERNEL void hc_triangular_b2(hck_triangular_args p) { triangular_impl<uint16_t>(p); }

@@ -407,6 +407,10 @@ def test_when_fill_triangular_concat_broadcast(hip_backend, oracle_backend):
                     lambda: Tensor.concat([Tensor(data=m, dtype=dtype), Tensor(data=m[:, :5], dtype=dtype)], axis=1))
         check_exact(hip_backend, oracle_backend,
                     lambda: Tensor.concat([Tensor(data=m, dtype=dtype), Tensor(data=m[:, :, :9], dtype=dtype)], axis=2))
+        wide = rand(rng, (2, 70, 64), dtype) if dtype != BOOL else rng.integers(0, 2, size=(2, 70, 64)).astype(np.bool_)
+        for off in (-65, -7, 0, 1, 33, 80):       # rows that are whole 16-byte vectors
+            check_exact(hip_backend, oracle_backend, lambda: Tensor(data=wide, dtype=dtype).tril(off))
+            check_exact(hip_backend, oracle_backend, lambda: Tensor(data=wide, dtype=dtype).triu(off))
         # pieces whose widths allow 16-, 8-, 4- and 2-byte copy units, three inputs, axis 0
         w = rand(rng, (9, 64), dtype) if dtype != BOOL else rng.integers(0, 2, size=(9, 64)).astype(np.bool_)
         for widths in [(64, 32), (8, 64, 24), (4, 60), (2, 6, 64), (1, 63), (64, 64, 64)]:
