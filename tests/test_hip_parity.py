@@ -604,6 +604,64 @@ def test_permuted_views_take_the_direct_copy(hip_backend, oracle_backend, dtype)
     check_exact(hip_backend, oracle_backend, indices)
 
 
+@pytest.mark.parametrize("seed", list(range(12)))
+def test_random_shapes_against_oracle(hip_backend, oracle_backend, seed):
+    """Seeded random shapes with awkward extents (around vector, wave and tile sizes, extent 1, a
+    few long axes) through the ops whose kernels choose a form by shape: reductions, arg-reductions,
+    logSoftmax, normalize, cumulative sums, permuted views, concat, triangular."""
+    from honeycrisp_amd.tensor import PermuteAxes
+    rng = np.random.default_rng(1000 + seed)
+    extents = [1, 2, 3, 5, 7, 8, 9, 15, 16, 17, 31, 33, 63, 64, 65, 100, 127, 128, 129, 255, 257, 1000, 1023, 4099]
+    long_extents = [20000, 40001, 70000]
+    for case in range(40):
+        nd = int(rng.integers(1, 5))
+        shape = [int(rng.choice(extents)) for _ in range(nd)]
+        if rng.random() < 0.3:
+            shape[int(rng.integers(0, nd))] = int(rng.choice(long_extents))
+        while int(np.prod(shape)) > 1 << 20:
+            shape[int(np.argmax(shape))] = max(1, max(shape) // 8)
+        dtype = [F32, F16, I64][int(rng.integers(0, 3))]
+        axis = int(rng.integers(0, nd))
+        x = rand(rng, shape, dtype)
+        if dtype != I64:
+            x = (np.round(x * 4) / 4).astype(dtype.numpy)      # ties for the arg-reductions, exact partial sums
+        op = ["sum", "argmax", "argmin", "logSoftmax", "normalize", "cumsum", "permute", "concat", "tril"][int(rng.integers(0, 9))]
+        print("random case", seed, case, op, dtype.name, shape, "axis", axis, flush=True)
+        t = lambda: Tensor(data=x, dtype=dtype)
+        if op == "sum":
+            fn = lambda: t().sum(axis=axis)
+            if dtype == I64:
+                check_exact(hip_backend, oracle_backend, fn)
+            else:
+                got, want = both(hip_backend, oracle_backend, fn)
+                assert_close_arrays(got, want, TOL[dtype] * max(1.0, float(np.sqrt(shape[axis]))), TOL[dtype])
+        elif op in ("argmax", "argmin"):
+            check_exact(hip_backend, oracle_backend, lambda: getattr(t(), op)(axis=axis))
+        elif op in ("logSoftmax", "normalize"):
+            if dtype == I64:
+                continue
+            tol = TOL[dtype] if op == "logSoftmax" or dtype == F32 else 2e-2
+            if op == "logSoftmax":
+                check_close(hip_backend, oracle_backend, lambda: t().logSoftmax(axis=axis), tol)
+            elif shape[axis] > 1:
+                check_close(hip_backend, oracle_backend, lambda: t().normalize(axis=axis, eps=1e-3), tol)
+        elif op == "cumsum":
+            if dtype == F16 and shape[axis] > 500:
+                continue    # running sums leave the range in which halfs are exact
+            excl, rev = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+            small = t if dtype == I64 else (lambda: Tensor(data=np.sign(x).astype(dtype.numpy), dtype=dtype))
+            check_exact(hip_backend, oracle_backend, lambda: small().cumulativeSum(axis, exclusive=excl, reverse=rev))
+        elif op == "permute":
+            perm = [int(p) for p in rng.permutation(nd)]
+            check_exact(hip_backend, oracle_backend, lambda: t()[PermuteAxes(*perm)])
+        elif op == "concat":
+            other = rand(rng, [s if a != axis else int(rng.choice([1, 2, 8, 17])) for a, s in enumerate(shape)], dtype)
+            check_exact(hip_backend, oracle_backend, lambda: Tensor.concat([t(), Tensor(data=other, dtype=dtype), t()], axis=axis))
+        elif op == "tril" and nd >= 2:
+            off = int(rng.integers(-3, 4))
+            check_exact(hip_backend, oracle_backend, lambda: t().tril(off))
+
+
 # ---------------------------------------------------------------- config 4 at full size
 
 def test_bandwidth_ops_full_size(hip_backend, oracle_backend):
