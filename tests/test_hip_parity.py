@@ -604,6 +604,52 @@ def test_permuted_views_take_the_direct_copy(hip_backend, oracle_backend, dtype)
     check_exact(hip_backend, oracle_backend, indices)
 
 
+@pytest.mark.parametrize("seed", list(range(6)))
+def test_random_broadcasts_against_oracle(hip_backend, oracle_backend, seed):
+    """Seeded random broadcast patterns (each operand drops a random subset of the axes) through the
+    broadcasting kernels, which pick a load form per operand from its innermost stride: binary
+    arithmetic, comparison, when, mulAdd / addMul. All bit-exact (fp32 arithmetic without library
+    calls, halfs computed in fp32 and rounded once on both sides)."""
+    rng = np.random.default_rng(2000 + seed)
+    extents = [1, 2, 3, 7, 8, 9, 16, 17, 33, 64, 65, 128, 257, 1000]
+    for case in range(40):
+        nd = int(rng.integers(1, 5))
+        shape = [int(rng.choice(extents)) for _ in range(nd)]
+        while int(np.prod(shape)) > 1 << 19:
+            shape[int(np.argmax(shape))] = max(1, max(shape) // 4)
+        dtype = [F32, F16, I64][int(rng.integers(0, 3))]
+        def operand():
+            keep = [bool(rng.integers(0, 2)) for _ in range(nd)]
+            lead = int(rng.integers(0, nd + 1))        # also drop leading axes altogether
+            shp = [s if k else 1 for s, k in zip(shape, keep)][lead:]
+            v = rand(rng, shp if shp else [1], dtype)
+            if dtype != I64:
+                v = (np.round(v * 8) / 8).astype(dtype.numpy)
+            return v
+        a, b, c = operand(), operand(), operand()
+        full = rand(rng, shape, dtype)                 # one operand of the full shape fixes the output shape
+        op = ["add", "mul", "sub", "lt", "eq", "when", "mulAdd", "addMul"][int(rng.integers(0, 8))]
+        print("broadcast case", seed, case, op, dtype.name, shape, a.shape, b.shape, c.shape, flush=True)
+        T_ = lambda v: Tensor(data=v, dtype=dtype)
+        if op == "add":
+            fn = lambda: T_(full) + T_(a) + T_(b)
+        elif op == "mul":
+            fn = lambda: T_(a) * T_(full) * T_(b)
+        elif op == "sub":
+            fn = lambda: T_(a) - T_(full)
+        elif op == "lt":
+            fn = lambda: (T_(a) + T_(full) * 0) < T_(b)
+        elif op == "eq":
+            fn = lambda: T_(full) == T_(a)
+        elif op == "when":
+            fn = lambda: (T_(full) < T_(a)).when(T_(b), T_(c))
+        elif op == "mulAdd":
+            fn = lambda: T_(full).mul(T_(a), thenAdd=T_(b))
+        else:
+            fn = lambda: T_(full).add(T_(a), thenMul=T_(b))
+        check_exact(hip_backend, oracle_backend, fn)
+
+
 @pytest.mark.parametrize("seed", list(range(12)))
 def test_random_shapes_against_oracle(hip_backend, oracle_backend, seed):
     """Seeded random shapes with awkward extents (around vector, wave and tile sizes, extent 1, a
