@@ -575,7 +575,9 @@ def test_permuted_views_take_the_direct_copy(hip_backend, oracle_backend, dtype)
              ((3, 4, 5, 6), (3, 2, 1, 0)), ((7, 9, 11), (2, 0, 1)), ((4, 40, 24), (1, 0, 2)),
              ((2, 3, 130, 67), (0, 1, 3, 2)), ((2050, 3), (1, 0)), ((8, 256, 8, 64), (0, 2, 1, 3)),
              # one of the two transposed axes short: long narrow tiles
-             ((5000, 2), (1, 0)), ((2, 5000), (1, 0)), ((3, 1500, 5), (0, 2, 1)), ((7, 3000), (1, 0)), ((1100, 20), (1, 0))]
+             ((5000, 2), (1, 0)), ((2, 5000), (1, 0)), ((3, 1500, 5), (0, 2, 1)), ((7, 3000), (1, 0)), ((1100, 20), (1, 0)),
+             # both axes long, ragged against the tiles
+             ((256, 384), (1, 0)), ((3, 130, 258), (0, 2, 1)), ((200, 128), (1, 0)), ((2, 128, 3, 128), (3, 1, 2, 0))]
     for shape, perm in cases:
         x = rng.integers(0, 2, size=shape) if dtype == BOOL else rand(rng, shape, dtype)
         print("permute", dtype.name, shape, perm, flush=True)
