@@ -615,10 +615,11 @@ class HIPBackend(Backend):
             if s.outerCount > 1:
                 perm, shape = [0] + [p + 1 for p in perm], [s.outerCount] + shape
             n = len(shape)
-            self._check(self._lib.hc_permute(self._ctx, int(dtype), c_void_p(self._dev(a).ptr),
-                                             (c_int64 * max(n, 1))(*perm), (c_int64 * max(n, 1))(*shape), n,
-                                             s.innerCount, c_void_p(out.ptr)))
-            return out
+            if n <= 8:      # (hc_permute takes up to 8 axes; more fall through to the index gather)
+                self._check(self._lib.hc_permute(self._ctx, int(dtype), c_void_p(self._dev(a).ptr),
+                                                 (c_int64 * max(n, 1))(*perm), (c_int64 * max(n, 1))(*shape), n,
+                                                 s.innerCount, c_void_p(out.ptr)))
+                return out
         ad, idx = self._dev(a), self._dev(s.indices.data)
         st = self._s(s.indices.strides)
         self._check(self._lib.hc_gather(self._ctx, int(dtype), c_void_p(ad.ptr), c_void_p(idx.ptr), byref(st),

@@ -230,8 +230,10 @@ class HIPBackend {
           perm.insert(perm.begin(), 0);
           shape.insert(shape.begin(), s.outer());
         }
-        check(hc_permute(ctx_, (int)dtype, a->ptr(), perm.data(), shape.data(), (int)shape.size(), s.inner(), out->ptr()));
-        return out;
+        if (shape.size() <= HC_MAX_DIMS) {  // (more axes fall through to the index gather)
+          check(hc_permute(ctx_, (int)dtype, a->ptr(), perm.data(), shape.data(), (int)shape.size(), s.inner(), out->ptr()));
+          return out;
+        }
       }
     }
     hc_strides st = s.indices.strides.c();

@@ -1818,7 +1818,7 @@ extern "C" int hc_permute(hc_ctx* ctx, int dtype, const void* in, const int64_t*
                           int ndim, int64_t inner, void* out) {
   REQUIRE(ctx, "hc_permute: null context");
   REQUIRE(dtype_name(dtype), "hc_permute: bad dtype %d", dtype);
-  REQUIRE(ndim >= 0 && ndim <= HC_MAX_DIMS - 1, "hc_permute: ndim %d out of range", ndim);
+  REQUIRE(ndim >= 0 && ndim <= HC_MAX_DIMS, "hc_permute: ndim %d out of range", ndim);
   REQUIRE(ndim == 0 || (perm && shape), "hc_permute: null argument");
   REQUIRE(inner >= 0, "hc_permute: negative inner count");
   const size_t el = dtype_size(dtype);

@@ -269,11 +269,13 @@ open class HIPBackend: CPUBackend, @unchecked Sendable {
         perm = [0] + perm.map { $0 + 1 }
         shape = [Int64(outer)] + shape
       }
-      try check(
-        hc_permute(
-          ctx, hcDType(dtype), da.pointer, perm, shape, Int32(shape.count),
-          Int64(s.valueShape[(axis + 1)...].product()), out.pointer))
-      return out
+      if shape.count <= 8 {  // (more axes fall through to the index gather)
+        try check(
+          hc_permute(
+            ctx, hcDType(dtype), da.pointer, perm, shape, Int32(shape.count),
+            Int64(s.valueShape[(axis + 1)...].product()), out.pointer))
+        return out
+      }
     }
     try check(
       hc_gather(

@@ -593,6 +593,10 @@ def test_permuted_views_take_the_direct_copy(hip_backend, oracle_backend, dtype)
         with hip_backend.use():
             got = fn().numpy()
         assert np.array_equal(got, np.ascontiguousarray(np.transpose(np.asarray(x).astype(got.dtype), perm)))
+    # eight permuted axes, and eight behind a leading axis (one more than the direct copy takes)
+    z8 = rand(rng, (2, 3, 2, 2, 3, 2, 2, 3), F32)
+    check_exact(hip_backend, oracle_backend, lambda: Tensor(data=z8)[PermuteAxes(7, 6, 5, 4, 3, 2, 1, 0)])
+    check_exact(hip_backend, oracle_backend, lambda: Tensor(data=z8)[PermuteAxes(0, 7, 1, 6, 2, 5, 3, 4)])
     # the 2-D helpers, with a batch prefix
     y = rand(rng, (3, 50, 70), F32)
     check_exact(hip_backend, oracle_backend, lambda: Tensor(data=y).t())
