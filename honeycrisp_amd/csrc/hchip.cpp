@@ -2247,7 +2247,7 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
       auto whole = [&](uint32_t tm, uint32_t tn) { return M % tm == 0 && N % tn == 0 && K % slice == 0; };
       // largest tile first; the direct-to-LDS kernels also come in narrow shapes
       static const uint32_t tiles[][2] = {{256, 256}, {256, 128}, {128, 128}, {256, 64}, {128, 64}, {64, 64}};
-      // (only the 16x16x32 pipeline has these)
+      // (only the 16x16x32 pipeline and, for fp32, the two-stage pipeline have these)
       static const uint32_t tiles192[][2] = {{256, 192}, {192, 256}, {192, 192}};
       const uint64_t cus = (uint64_t)ctx->props.multiProcessorCount;
       if (force && *force) {
@@ -2255,7 +2255,7 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
         if (sscanf(force, "%ux%u", &fm, &fn) == 2 && (dma || whole(fm, fn))) {
           bool known = false;
           for (auto& t : tiles) known = known || (t[0] == fm && t[1] == fn);
-          if (mi16)
+          if (mi16 || (dma2 && dtype == HC_F32))
             for (auto& t : tiles192) known = known || (t[0] == fm && t[1] == fn);
           if (known) {
             bm = fm;
@@ -2290,6 +2290,27 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
             best_blocks = blocks;
             bm = t[0];
             bn = t[1];
+          }
+        }
+        // fp32 products with K >= 512 also have the 192-extent tiles of the two-stage pipeline: fp32
+        // runs every large tile at the same rate (it is not limited by power), so what counts is
+        // how evenly the tiles fill the device (3072^2 outputs: 16 x 16 tiles of 192 x 192 are one
+        // full round, 144 tiles of 256 x 256 leave 44 % of the CUs idle).
+        if (dtype == HC_F32 && dma && !which && K >= 512 && filled) {
+          static const double rate192[] = {0.97, 0.97, 0.95};
+          for (size_t ti = 0; ti < sizeof(tiles192) / sizeof(tiles192[0]); ti++) {
+            const uint32_t* t = tiles192[ti];
+            const uint64_t blocks = ceil_div(M, t[0]) * ceil_div(N, t[1]) * (uint64_t)batch;
+            if (blocks < cus) continue;
+            const double rounds = (double)ceil_div(blocks, cus);
+            const double useful = ((double)M * N * (double)batch) / ((double)blocks * t[0] * t[1]);
+            const double score = rate192[ti] * ((double)blocks / (rounds * (double)cus)) * useful;
+            if (score > best_score) {
+              best_score = score;
+              bm = t[0];
+              bn = t[1];
+              dma2 = true;
+            }
           }
         }
       }

@@ -84,6 +84,10 @@ template <typename T, int ROWS, int MODE> struct DmaOperand {
   static constexpr int NADDR = MODE == DMA_K ? TILES * 4 : TILES * 2;
   static constexpr int ROWB = ROWS * ES;                      // bytes per k-row (DMA_MN layout)
   static constexpr int BYTES = ROWS * 128;                    // per stage
+  // fp16 DMA_MN: the swizzle permutes the ROWS / 8 slots of a k-row inside aligned groups of
+  // MN_SWZ_MASK + 1 (a divisor of ROWS / 8 also when that is not a power of two)
+  static constexpr uint32_t MN_SWZ_MASK = ((ROWS / 8) & (ROWS / 8 - 1)) == 0 ? ROWS / 8 - 1 : 7;
+  static_assert(ROWS % 64 == 0 && (ROWS / 8) % (MN_SWZ_MASK + 1) == 0, "unsupported tile extent");
 
   uint32_t goff[NI];     // byte offset of this lane's 16-byte piece for DMA instruction i (k = 0)
   uint32_t kstride;      // bytes per unit of k
@@ -114,13 +118,16 @@ template <typename T, int ROWS, int MODE> struct DmaOperand {
     } else if (F32) {
       // [32 k][ROWS floats]; the 128-byte halves of every 256 bytes swap places in k-rows
       // with bit 2 set: an MFMA operand read touches rows k and k + 4, 32 floats of each
-      constexpr uint32_t KPI = 1024 / ROWB;   // k-rows per DMA instruction
+      // (the instructions of a K-slice cover its pieces in order, 64 each: a k-row need not be a
+      // whole number of instructions)
       constexpr uint32_t PIECES = ROWB / 16;  // 16-byte pieces per k-row
+      static_assert(!F32 || PIECES % 16 == 0, "the swap permutes pieces inside aligned groups of 16");
       kstride = cs * ES;
 #pragma unroll
       for (int i = 0; i < NI; i++) {
-        const uint32_t krow = (wave * NI + i) * KPI + lane / PIECES;
-        const uint32_t piece = (lane % PIECES) ^ (((krow >> 2) & 1u) << 3);
+        const uint32_t flat = (wave * NI + i) * 64 + lane;
+        const uint32_t krow = flat / PIECES;
+        const uint32_t piece = (flat % PIECES) ^ (((krow >> 2) & 1u) << 3);
         uint32_t col = r0 + piece * 4;
         if (limit && col + 4 > limit) col = limit - 4;
         goff[i] = (krow * cs + col) * ES;
@@ -132,13 +139,13 @@ template <typename T, int ROWS, int MODE> struct DmaOperand {
         raddr[q] = 4 * lgrp * ROWB + ((n ^ (lgrp << 5)) * 4);
       }
     } else {
-      constexpr int KPI = 512 / ROWS;       // k-rows per DMA instruction
       constexpr uint32_t SLOTS_PER_ROW = ROWS / 8;
       kstride = cs * 2;
 #pragma unroll
       for (int i = 0; i < NI; i++) {
-        const uint32_t krow = (wave * NI + i) * KPI + lane / SLOTS_PER_ROW;
-        const uint32_t slot = (lane % SLOTS_PER_ROW) ^ (swz_mn(krow) & (SLOTS_PER_ROW - 1));
+        const uint32_t flat = (wave * NI + i) * 64 + lane;
+        const uint32_t krow = flat / SLOTS_PER_ROW;
+        const uint32_t slot = (flat % SLOTS_PER_ROW) ^ (swz_mn(krow) & MN_SWZ_MASK);
         uint32_t col = r0 + slot * 8;
         if (limit && col + 8 > limit) col = limit - 8;
         goff[i] = (krow * cs + col) * 2;
@@ -150,7 +157,7 @@ template <typename T, int ROWS, int MODE> struct DmaOperand {
 #pragma unroll
         for (int h = 0; h < 2; h++) {
           const uint32_t k = 8 * (j >> 1) + 4 * h + (r16 >> 2);  // + 16 * s as an immediate offset
-          raddr[q * 2 + h] = k * ROWB + (((m >> 3) ^ (swz_mn(k) & (ROWS / 8 - 1))) * 16) + (m & 7) * 2;
+          raddr[q * 2 + h] = k * ROWB + (((m >> 3) ^ (swz_mn(k) & MN_SWZ_MASK)) * 16) + (m & 7) * 2;
         }
       }
     }
@@ -163,8 +170,8 @@ template <typename T, int ROWS, int MODE> struct DmaOperand {
       const uint32_t row = (wave * NI + i) * 8 + lane / 8;
       return ((lane % 8) ^ swz_k(row)) * (16 / ES);
     }
-    constexpr uint32_t PER_ROW = ROWB / 16, KPI = 1024 / ROWB;
-    return (wave * NI + i) * KPI + lane / PER_ROW;
+    constexpr uint32_t PER_ROW = ROWB / 16;
+    return ((wave * NI + i) * 64 + lane) / PER_ROW;
   }
 
   // DMA instruction i of this wave for the K-slice starting at k0: 1 KiB into `region`.
@@ -388,10 +395,13 @@ __device__ __forceinline__ void gemm_dma2_impl(const hck_gemm_args& p, char* lds
   // LDS instructions execute in order, so a slab may be overwritten right after its reads.
   lds_barrier();
   char* mine = (wave < 2 ? lds0 : lds1) + (wave & 1) * ((BM + BN) * 64);
-  constexpr uint32_t ES = sizeof(T), WN = BN / 2, RB = WN * ES, UNITS = RB / 16, RPI = 64 / UNITS;
+  constexpr uint32_t ES = sizeof(T), WN = BN / 2, RB = WN * ES, UNITS = RB / 16;
   constexpr uint32_t SLAB = 32 * RB, NSLAB = (BM + BN) * 64 / SLAB;
-  static_assert(NSLAB >= 1 && UNITS <= 64, "a slab must fit one stage");
-  auto unit_swz = [&](uint32_t r) { return (RB >= 256 ? r : r * RB / 256) & (UNITS - 1); };
+  static_assert(NSLAB >= 1 && (32 * UNITS) % 64 == 0, "a slab must fit half a stage");
+  // (the swizzle stays inside aligned groups of USWZ + 1 units, a divisor of UNITS)
+  constexpr uint32_t USWZ = (UNITS & (UNITS - 1)) == 0 ? UNITS - 1 : (UNITS % 8 == 0 ? 7 : 3);
+  static_assert(UNITS % (USWZ + 1) == 0, "unsupported tile width");
+  auto unit_swz = [&](uint32_t r) { return (RB >= 256 ? r : r * RB / 256) & USWZ; };
 #pragma unroll
   for (int i = 0; i < MT; i++) {
     char* slab = mine + (i % NSLAB) * SLAB;
@@ -414,8 +424,8 @@ __device__ __forceinline__ void gemm_dma2_impl(const hck_gemm_args& p, char* lds
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // wave-private region: no barrier needed
 #pragma unroll
-    for (uint32_t it = 0; it < 32 / RPI; it++) {
-      const uint32_t r = it * RPI + lane / UNITS, u = lane % UNITS;
+    for (uint32_t it = 0; it < 32 * UNITS / 64; it++) {
+      const uint32_t piece = it * 64 + lane, r = piece / UNITS, u = piece % UNITS;
       const Chunk v = *reinterpret_cast<const Chunk*>(slab + r * RB + ((u ^ unit_swz(r)) * 16));
       const uint32_t row = m0 + wm + i * 32 + r, col = n0 + wn + u * (16 / ES);
       if (!EDGE || (row < p.M && col < p.N)) *reinterpret_cast<Chunk*>(C + (size_t)row * p.c_rs + col) = v;
@@ -463,3 +473,7 @@ __device__ __forceinline__ void gemm_dma2_impl(const hck_gemm_args& p, char* lds
   DEF_DMA_TILE(T, TN, 64, 64)
 DEF_DMA_TYPE(half_t, f16)
 DEF_DMA_TYPE(float, f32)
+// (extents that are not powers of two: fp32 only, fp16 has them on the 16x16x32 pipeline)
+DEF_DMA_TILE(float, f32, 256, 192)
+DEF_DMA_TILE(float, f32, 192, 256)
+DEF_DMA_TILE(float, f32, 192, 192)

@@ -128,8 +128,8 @@ def test_matmul_both_pipelines_every_tile(hip_backend, oracle_backend, monkeypat
     rng = np.random.default_rng(77)
     monkeypatch.setenv("HCHIP_GEMM_KERNEL", pipeline)
     tiles = ("256x256", "256x128", "128x128", "256x64", "128x64", "64x64")
-    if pipeline == "mi16" and dtype is F16:
-        tiles += ("256x192", "192x256", "192x192")  # (extents that are not powers of two: this pipeline only)
+    if (pipeline == "mi16" and dtype is F16) or (pipeline == "dma2" and dtype is F32):
+        tiles += ("256x192", "192x256", "192x192")  # (extents that are not powers of two: these pipelines only)
     for tile in tiles:
         monkeypatch.setenv("HCHIP_GEMM_TILE", tile)
         shapes = [(1, 256, 192, 256), (2, 264, 200, 136), (3, 128, 1024, 64)]
@@ -244,6 +244,33 @@ def test_matmul_fp16_large_ragged_against_oracle_slab(hip_backend, oracle_backen
             assert out.shape == (M, N)
             assert_close_arrays(out[rows], want, 1e-2, 1e-2)
             assert_close_arrays(out, general, 1e-2, 1e-2)
+
+
+def test_matmul_fp32_192_tiles_against_oracle_slab(hip_backend, oracle_backend):
+    """An fp32 product whose output the host covers with 192 x 192 tiles (ragged in M, N and K:
+    edge variant): row slabs against the oracle, the whole result against the general kernel."""
+    rng = np.random.default_rng(13)
+    M, K, N = 3000, 520, 3016
+    a = (rng.standard_normal((M, K)) / np.sqrt(K)).astype(np.float32)
+    b = rng.standard_normal((K, N)).astype(np.float32)
+    rows = np.r_[0:16, M // 2 - 8:M // 2 + 8, M - 16:M]
+    with oracle_backend.use():
+        want = Tensor.matmul(Tensor(data=a[rows]), False, Tensor(data=b), False, False).numpy()
+    with hip_backend.use():
+        ta, tb = Tensor(data=a), Tensor(data=b)
+        tat, tbt = Tensor(data=np.ascontiguousarray(a.T)), Tensor(data=np.ascontiguousarray(b.T))
+        os.environ["HCHIP_GEMM_TILE"] = "general"
+        try:
+            general = Tensor.matmul(ta, False, tb, False, False).numpy()
+        finally:
+            del os.environ["HCHIP_GEMM_TILE"]
+        assert_close_arrays(general[rows], want, 1e-4, 1e-4)
+        for transA, transB in [(False, False), (False, True), (True, False), (True, True)]:
+            print("3000x520x3016 fp32 layout", transA, transB, flush=True)
+            out = Tensor.matmul(tat if transA else ta, transA, tbt if transB else tb, transB, False).numpy()
+            assert out.shape == (M, N)
+            assert_close_arrays(out[rows], want, 1e-4, 1e-4)
+            assert_close_arrays(out, general, 1e-4, 1e-4)
 
 
 def test_matmul_int64(hip_backend, oracle_backend):
