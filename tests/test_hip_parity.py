@@ -683,6 +683,60 @@ def test_random_broadcasts_against_oracle(hip_backend, oracle_backend, seed):
         check_exact(hip_backend, oracle_backend, fn)
 
 
+@pytest.mark.parametrize("seed", list(range(6)))
+def test_random_gathers_and_scatters_against_oracle(hip_backend, oracle_backend, seed):
+    """Seeded random gathers and scatters: value shapes with awkward extents, any axis, index tensors
+    that are 1-D (one index per position of the axis), full-shaped, or broadcast along some of the other
+    axes; scatters with unique and with repeated indices. Gathers and int64 / unique scatters are
+    bit-exact; float scatters with repeated indices add in hardware-atomic order (tolerance), except
+    the long-row form, which follows the CPU's order."""
+    rng = np.random.default_rng(3000 + seed)
+    extents = [1, 2, 3, 5, 8, 16, 17, 33, 64, 65, 127, 128, 256, 300, 1024]
+    for case in range(30):
+        nd = int(rng.integers(1, 5))
+        shape = [int(rng.choice(extents)) for _ in range(nd)]
+        while int(np.prod(shape)) > 1 << 19:
+            shape[int(np.argmax(shape))] = max(1, max(shape) // 4)
+        axis = int(rng.integers(0, nd))
+        dtype = [F32, F16, I64, BOOL][int(rng.integers(0, 4))]
+        count = int(rng.choice([1, 2, 7, 64, 300]))           # gathered positions along the axis
+        form = int(rng.integers(0, 3))
+        if form == 0:
+            idx_shape = [count]
+        else:
+            idx_shape = list(shape)
+            idx_shape[axis] = count
+            if form == 2:                                      # broadcast along a random subset of the other axes
+                for a in range(nd):
+                    if a != axis and rng.random() < 0.5:
+                        idx_shape[a] = 1
+        x = rng.integers(0, 2, size=shape).astype(np.bool_) if dtype == BOOL else rand(rng, shape, dtype)
+        idx = rng.integers(0, shape[axis], size=idx_shape)
+        print("gather case", seed, case, dtype.name, shape, "axis", axis, "indices", idx_shape, flush=True)
+        gather = lambda: Tensor(data=x, dtype=dtype).gather(axis, Tensor(data=idx))
+        check_exact(hip_backend, oracle_backend, gather)
+        if dtype == BOOL:
+            continue
+        # scatter the gathered values back into an axis of `target` positions
+        with oracle_backend.use():
+            g = gather().numpy()
+        target = int(rng.choice([shape[axis], shape[axis] + 3, 2 * count + 1]))
+        sidx = rng.integers(0, target, size=idx_shape)
+        unique = False
+        if rng.random() < 0.4 and count <= target:              # distinct indices along the axis
+            perm = np.stack([rng.permutation(target)[:count] for _ in range(int(np.prod(idx_shape)) // count)])
+            sidx = np.moveaxis(perm.reshape([s for a, s in enumerate(idx_shape) if a != (axis if form else 0)] + [count]),
+                               -1, axis if form else 0)
+            unique = True
+        scatter = lambda: Tensor(data=g, dtype=dtype).scatter(axis, target, Tensor(data=np.ascontiguousarray(sidx)),
+                                                              indicesAreUnique=unique)
+        if dtype == I64 or unique:
+            check_exact(hip_backend, oracle_backend, scatter)
+        else:
+            got, want = both(hip_backend, oracle_backend, scatter)
+            assert_close_arrays(got, want, TOL[dtype] * 8, TOL[dtype])
+
+
 @pytest.mark.parametrize("seed", list(range(12)))
 def test_random_shapes_against_oracle(hip_backend, oracle_backend, seed):
     """Seeded random shapes with awkward extents (around vector, wave and tile sizes, extent 1, a
