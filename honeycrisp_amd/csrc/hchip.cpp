@@ -65,7 +65,16 @@ struct hc_ctx {
   hc_graph* capturing = nullptr;                      // the recording in progress, if any
   std::unordered_map<void*, hc_graph*> block_owner;   // blocks reserved for a graph
   std::vector<hc_graph*> graphs;
+  // Small host-to-device uploads go through pinned memory so that they need no host-side wait:
+  // two halves used in turn, each guarded by an event recorded when the upload path leaves it.
+  char* stage = nullptr;
+  size_t stage_off = 0;
+  int stage_cur = 0;
+  hipEvent_t stage_ev[2] = {nullptr, nullptr};
+  bool stage_busy[2] = {false, false};
 };
+static const size_t kStageHalf = 2u << 20;    // bytes per half of the staging buffer
+static const size_t kStageMax = 256u << 10;   // largest upload that is staged
 
 static thread_local std::string g_last_error;
 
@@ -141,6 +150,18 @@ extern "C" int hc_init(int device, hc_ctx** out) {
     delete ctx;
     return hip_fail(e, "hipStreamCreateWithFlags");
   }
+  // (without the staging buffer uploads simply stay synchronous; HCHIP_NO_STAGING=1 asks for that)
+  if (getenv("HCHIP_NO_STAGING")) {
+    ctx->stage = nullptr;
+  } else if (hipHostMalloc((void**)&ctx->stage, 2 * kStageHalf, hipHostMallocDefault) != hipSuccess) {
+    ctx->stage = nullptr;
+    (void)hipGetLastError();
+  } else if (hipEventCreateWithFlags(&ctx->stage_ev[0], hipEventDisableTiming) != hipSuccess ||
+             hipEventCreateWithFlags(&ctx->stage_ev[1], hipEventDisableTiming) != hipSuccess) {
+    (void)hipHostFree(ctx->stage);
+    ctx->stage = nullptr;
+    (void)hipGetLastError();
+  }
   int s = load_image(ctx, hc_image_elementwise, hc_image_elementwise_end, "elementwise");
   if (s == HC_OK) s = load_image(ctx, hc_image_reduce, hc_image_reduce_end, "reduce");
   if (s == HC_OK) s = load_image(ctx, hc_image_gather, hc_image_gather_end, "gather");
@@ -181,6 +202,9 @@ extern "C" void hc_shutdown(hc_ctx* ctx) {
   for (auto& kv : ctx->live) (void)hipFree(kv.first);
   for (hipModule_t m : ctx->modules) (void)hipModuleUnload(m);
   if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
+  for (hipEvent_t ev : ctx->stage_ev)
+    if (ev) (void)hipEventDestroy(ev);
+  if (ctx->stage) (void)hipHostFree(ctx->stage);
   delete ctx;
 }
 
@@ -331,6 +355,24 @@ static int copy(hc_ctx* ctx, void* dst, const void* src, size_t bytes, hipMemcpy
   std::lock_guard<std::mutex> lock(ctx->mu);
   REQUIRE(!ctx->capturing || kind == hipMemcpyDeviceToDevice,
           "memcpy: host transfers are not allowed while capturing (upload inputs before hc_capture_begin)");
+  if (kind == hipMemcpyHostToDevice && wait && bytes <= kStageMax && ctx->stage) {
+    // The caller may reuse `src` as soon as this returns: copy it into pinned memory and let the
+    // stream pick it up from there. No wait, so the device keeps running what is already queued
+    // (index vectors of slices, small constants in the middle of a forward pass).
+    if (ctx->stage_off + bytes > kStageHalf) {
+      HIP_TRY(hipEventRecord(ctx->stage_ev[ctx->stage_cur], ctx->stream));
+      ctx->stage_busy[ctx->stage_cur] = true;
+      ctx->stage_cur ^= 1;
+      ctx->stage_off = 0;
+      if (ctx->stage_busy[ctx->stage_cur]) HIP_TRY(hipEventSynchronize(ctx->stage_ev[ctx->stage_cur]));
+      ctx->stage_busy[ctx->stage_cur] = false;
+    }
+    char* slot = ctx->stage + (size_t)ctx->stage_cur * kStageHalf + ctx->stage_off;
+    memcpy(slot, src, bytes);
+    ctx->stage_off += (bytes + 63) & ~(size_t)63;
+    HIP_TRY(hipMemcpyAsync(dst, slot, bytes, kind, ctx->stream));
+    return HC_OK;
+  }
   HIP_TRY(hipMemcpyAsync(dst, src, bytes, kind, ctx->stream));
   if (wait) HIP_TRY(hipStreamSynchronize(ctx->stream));
   return HC_OK;

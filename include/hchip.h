@@ -111,8 +111,12 @@ int hc_mem_stats(hc_ctx* ctx, size_t* in_use, size_t* cached);
 /* Pinned host staging memory (hipHostMalloc). */
 int hc_host_alloc(hc_ctx* ctx, size_t bytes, void** out);
 int hc_host_free(hc_ctx* ctx, void* ptr);
-/* Blocking copies ordered after everything already enqueued: what Tensor.Data.onCPU /
- * mutateOnCPU need (Tensor.swift:74-84). */
+/* Copies ordered after everything already enqueued: what Tensor.Data.onCPU / mutateOnCPU need
+ * (Tensor.swift:74-84). When a call returns the host buffer is the caller's again: d2h has
+ * completed; h2d has completed, or (uploads up to 256 KiB) the bytes were taken into pinned
+ * staging memory from which the stream copies them in order, so that small uploads in the middle
+ * of a forward pass (index vectors of slices, constants) do not make the host wait for the
+ * device. */
 int hc_memcpy_h2d(hc_ctx* ctx, void* dst, const void* src, size_t bytes);
 int hc_memcpy_d2h(hc_ctx* ctx, void* dst, const void* src, size_t bytes);
 int hc_memcpy_d2d(hc_ctx* ctx, void* dst, const void* src, size_t bytes);
