@@ -139,7 +139,8 @@ class _RangeIndex:
         assert end >= start and 0 <= start <= n and 0 <= end <= n
         if start == 0 and end == n:
             return FullRange().tensorIndex(inShape)
-        return TensorIndexResult(inShape, Tensor(data=range(start, end), dtype=DType.int64), True, 0, None)
+        return TensorIndexResult(inShape, Tensor(data=np.arange(start, end, dtype=np.int64), dtype=DType.int64),
+                                 True, 0, None)
 
 
 def _index_list(items, inShape) -> TensorIndexResult:
