@@ -10,7 +10,9 @@ Also reported in the same line:
   roofline      the slowest layout's GEMM kernel: algorithmic FLOPs / average launch duration
                 from HIP events recorded on the backend's own stream inside the timed region
   cpu_baseline  the reference CPUBackend algorithm (oracle/cpu_ref.c restatement, the literal
-                single-thread triple loop) timed on this box's host cores on a bounded row slab
+                single-thread triple loop) timed on this box's host cores on a bounded row slab;
+                extra.cpu_reference_path holds the same for configs 1 and 4 (sgemm through OpenBLAS
+                with its thread count, the bandwidth-bound ops on one thread)
   extra         the other BASELINE configs: fp32 1024^3, the ragged fp16 sweep, attention-shaped
                 batched GEMMs, the bandwidth-bound ops at [8192,4096] with GB/s against the 8 TB/s
                 HBM peak (short kernels are timed as graph-replayed batches: device-side duration
@@ -239,6 +241,71 @@ def cpu_baseline(a, b, budget_s=20.0):
     }
 
 
+def cpu_reference_ops(budget_s=15.0):
+    """Configs 1 and 4 on the host cores the way the reference CPUBackend would run them on Linux:
+    the fp32 NN product through cblas_sgemm (the stand-in for vDSP_mmul, BackendCPU.swift:1256;
+    here numpy's bundled OpenBLAS, all the threads it takes) and through the literal loop, and the
+    bandwidth-bound ops through the CPUBackend restatement on ONE thread (the reference serialises
+    its CPU work on one worker thread, BackendCPU.swift:226,235-248). Full-size inputs; an op is
+    skipped once the budget is spent."""
+    from oracle.oracle_backend import OracleBackend
+    from honeycrisp_amd.descriptors import (BroadcastData, BroadcastStrides, DType, ElemwiseOp, NumericBinaryOp,
+                                            ReduceDims, ReduceOp, ScatterGatherIndices)
+    F32 = DType.float32
+    out = {}
+    spent = [0.0]
+
+    def timed(name, fn, flops=None, nbytes=None, cores=1, reps=1):
+        if spent[0] > budget_s:
+            return
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        dt = (time.perf_counter() - t0) / reps
+        spent[0] += dt * reps
+        r = {"ms": round(dt * 1e3, 2), "cores": cores}
+        if flops is not None:
+            r["tflops"] = round(flops / dt / 1e12, 5)
+        if nbytes is not None:
+            r["gbs"] = round(nbytes / dt / 1e9, 3)
+        out[name] = r
+
+    rng = np.random.default_rng(1)
+    a = rng.standard_normal((1024, 1024)).astype(np.float32)
+    b = rng.standard_normal((1024, 1024)).astype(np.float32)
+    try:
+        import threadpoolctl
+        blas_threads = max([i.get("num_threads", 1) for i in threadpoolctl.threadpool_info()
+                            if i.get("user_api") == "blas"] or [1])
+    except Exception:
+        blas_threads = os.cpu_count() or 1
+    a @ b
+    timed("cfg1_f32_gemm_1024_openblas_sgemm", lambda: a @ b, flops=2.0 * 1024**3, cores=blas_threads, reps=10)
+    ob = OracleBackend(threads=1)
+    da, db = ob.upload(a), ob.upload(b)
+    timed("cfg1_f32_gemm_1024_literal_loop", lambda: ob.matmul(da, False, db, False, False, 1024, 1024, 1024, F32),
+          flops=2.0 * 1024**3)
+
+    R, C = 8192, 4096
+    x = ob.upload(np.random.default_rng(7).standard_normal((R, C)).astype(np.float32))
+    bias = ob.upload(np.random.default_rng(8).standard_normal((1, C)).astype(np.float32))
+    xs, bs = BroadcastStrides([R, C], [C, 1]), BroadcastStrides([R, C], [0, 1])
+    nb = R * C * 4
+    dims = ReduceDims(R, C, 1)
+    timed("cfg4_bias_add", lambda: ob.binaryOp(BroadcastData(xs, x), BroadcastData(bs, bias), NumericBinaryOp.add, F32),
+          nbytes=2 * nb + C * 4)
+    timed("cfg4_gelu", lambda: ob.elemwise(x, ElemwiseOp.geluApprox, None, R * C, F32), nbytes=2 * nb)
+    timed("cfg4_sum_axis1", lambda: ob.reduce(x, ReduceOp.sum, dims, F32), nbytes=nb + R * 4)
+    timed("cfg4_argmax_axis1", lambda: ob.reduce(x, ReduceOp.argmax, dims, F32), nbytes=nb + R * 8)
+    table = ob.upload(np.random.default_rng(10).standard_normal((32000, 1024)).astype(np.float32))
+    ids = ob.upload(np.random.default_rng(9).integers(0, 32000, size=(65536,)))
+    emb = ScatterGatherIndices([32000, 1024], 0, BroadcastData(BroadcastStrides([65536, 1024], [1, 0]), ids))
+    timed("cfg4_embedding_gather", lambda: ob.gather(table, emb, F32), nbytes=65536 * 8 + 2 * 65536 * 1024 * 4)
+    out["note"] = ("host cores of this box; sgemm = numpy's bundled OpenBLAS standing in for the cblas shim of "
+                   "vDSP_mmul, everything else the CPUBackend restatement on one thread, full-size inputs")
+    return out
+
+
 def extra_workloads(backend, graph=True):
     """Configs 1, 3 and 4 of BASELINE.json: per-op launch durations from HIP events."""
     from honeycrisp_amd.descriptors import (BroadcastData, BroadcastStrides, DType, ElemwiseOp, NumericBinaryOp,
@@ -408,6 +475,8 @@ def main():
         result["extra"] = extra_workloads(backend, graph=not args.no_graph)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(a, b)
+        if not args.no_extra:
+            result["extra"]["cpu_reference_path"] = cpu_reference_ops()
     else:
         result["cpu_baseline"] = None
     backend.sync()
