@@ -2157,8 +2157,8 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
       c.in_bs = bs;
       c.out_bs = (uint64_t)nrows * ld;
       const uint64_t waves = (uint64_t)nrows * ceil_div(ld, 512);  // a wave moves 64 * 8 elements
-      HC_TRY(launch(ctx, el == 2 ? "hc_copy2d_b2" : "hc_copy2d_b4", ceil_div(waves, HCK_BLOCK / 64), (uint32_t)batch,
-                    &c, sizeof(c)));
+      HC_TRY(launch(ctx, el == 2 ? "hc_copy2d_pad_b2" : "hc_copy2d_pad_b4", ceil_div(waves, HCK_BLOCK / 64),
+                    (uint32_t)batch, &c, sizeof(c)));
       ptr = copy;
       (k_contig ? rs : cs) = ld;
       bs = c.out_bs;
@@ -2444,7 +2444,9 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
   // microseconds, which a short body does not win back)
   auto fringe = [&](uint32_t d) { return d >= 2048 && d % 256 != 0 && d % 256 <= 32 ? d % 256 : 0u; };
   const bool tuned = ma != 'x' && mb != 'x' && K >= 2048 && !getenv("HCHIP_GEMM_TILE") && !getenv("HCHIP_GEMM_NO_PEEL");
-  const bool large = (uint64_t)M * N >= (1ull << 22);
+  // (an output of 4 M elements, or half of that over a K long enough for 2^33 multiply-adds)
+  const bool large = (uint64_t)M * N >= (1ull << 22) ||
+                     ((uint64_t)M * N >= (1ull << 21) && (uint64_t)M * N * K >= (1ull << 33));
   const uint32_t fm = tuned && large ? fringe(M) : 0, fn = tuned && large ? fringe(N) : 0;
   if (fm != 0 || fn != 0) {
     const uint32_t Mb = M - fm, Nb = N - fn;
@@ -2478,8 +2480,8 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
     c.in_bs = (uint64_t)M * c_ld;
     c.out_bs = (uint64_t)M * N;
     const uint64_t waves = (uint64_t)M * ceil_div(N, 512);
-    HC_TRY(launch(ctx, el == 2 ? "hc_copy2d_b2" : "hc_copy2d_b4", ceil_div(waves, HCK_BLOCK / 64), (uint32_t)batch,
-                  &c, sizeof(c)));
+    HC_TRY(launch(ctx, el == 2 ? "hc_copy2d_unpad_b2" : "hc_copy2d_unpad_b4", ceil_div(waves, HCK_BLOCK / 64),
+                  (uint32_t)batch, &c, sizeof(c)));
   }
   return HC_OK;
 }

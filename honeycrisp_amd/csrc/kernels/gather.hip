@@ -229,27 +229,123 @@ HC_KERNEL void hc_scatter_rows_sum_f32(hck_scatter_rows_args p) { scatter_rows_s
 HC_KERNEL void hc_scatter_rows_sum_f16(hck_scatter_rows_args p) { scatter_rows_sum_impl<half_t>(p); }
 HC_KERNEL void hc_scatter_rows_sum_i64(hck_scatter_rows_args p) { scatter_rows_sum_impl<int64_t>(p); }
 
-// Re-pitching copy for GEMM operands whose rows are not 16-byte aligned: element-wise
-// accesses (either side may be unaligned), zero beyond the valid columns. A wave owns
-// 64 * G consecutive elements of one row and moves 64 consecutive elements per instruction,
-// so every access is a dense 128- or 256-byte segment. grid.y = batch.
-template <typename V, int G> __device__ __forceinline__ void copy2d_impl(const hck_copy2d_args& p) {
-  const uint32_t groups = (p.out_cols + 64 * G - 1) / (64 * G);
+// Re-pitching copies for GEMM operands and outputs whose rows are not 16-byte aligned. One side
+// is always the library's own padded copy (base, leading dimension and batch stride multiples
+// of 16 bytes), the other side is the caller's matrix, aligned to its element size only.
+// A lane owns a 16-byte piece of the padded side, a wave 512 consecutive elements of one row;
+// grid.y = batch. Multi-dword accesses of the caller's side need dword alignment only:
+//   pad   (caller -> padded copy, zero beyond in_cols): 4-byte elements load the piece directly;
+//         2-byte elements on an odd element address load the five dwords around the piece and
+//         shift them by two bytes. Lanes whose window would reach past the last element of the
+//         last matrix take element-wise loads instead.
+//   unpad (padded result -> caller): a piece on an odd element address leaves as
+//         half + three dwords + half.
+typedef uint32_t CopyPiece __attribute__((ext_vector_type(4)));
+typedef CopyPiece CopyPieceA4 __attribute__((aligned(4)));
+template <typename V> __device__ __forceinline__ void copy2d_pad_impl(const hck_copy2d_args& p) {
+  constexpr uint32_t PE = 16 / sizeof(V);            // elements per piece
+  constexpr uint32_t NP = 512 / (64 * PE);           // pieces per lane
+  const uint32_t groups = (p.out_cols + 511) / 512;
   const uint64_t unit = (uint64_t)blockIdx.x * (HCK_BLOCK / 64) + (threadIdx.x >> 6);
   const uint64_t r = unit / groups;
   if (r >= p.rows) return;
-  const uint32_t c0 = (uint32_t)(unit - r * groups) * (64 * G) + (threadIdx.x & 63);
-  const V* src = (const V*)p.in + (uint64_t)blockIdx.y * p.in_bs + r * p.in_ld;
+  const uint32_t g0 = (uint32_t)(unit - r * groups) * 512;
+  // one past the last element that may be read, relative to p.in
+  const uint64_t lim = (uint64_t)(gridDim.y - 1) * p.in_bs + (uint64_t)(p.rows - 1) * p.in_ld + p.in_cols;
+  const uint64_t row0 = (uint64_t)blockIdx.y * p.in_bs + r * p.in_ld;
   V* dst = (V*)p.out + (uint64_t)blockIdx.y * p.out_bs + r * p.out_ld;
-  V v[G];
 #pragma unroll
-  for (int e = 0; e < G; e++) v[e] = c0 + e * 64 < p.in_cols ? src[c0 + e * 64] : (V)0;
+  for (uint32_t i = 0; i < NP; i++) {
+    const uint32_t c = g0 + ((threadIdx.x & 63) + 64 * i) * PE;
+    if (c >= p.out_cols) continue;
+    const uint64_t e0 = row0 + c;
+    const V* src = (const V*)p.in + e0;
+    CopyPiece o = {0u, 0u, 0u, 0u};
+    if (c < p.in_cols) {
+      if (e0 + PE + 2 <= lim) {
+        const uint32_t sh = sizeof(V) == 2 ? (uint32_t)((uintptr_t)src & 2) : 0u;
+        const char* sa = (const char*)src - sh;
+        const CopyPiece w = *reinterpret_cast<const CopyPieceA4*>(sa);
+        if (sh != 0) {
+          const uint32_t w4 = *reinterpret_cast<const uint32_t*>(sa + 16);
+          o[0] = (w[0] >> 16) | (w[1] << 16);
+          o[1] = (w[1] >> 16) | (w[2] << 16);
+          o[2] = (w[2] >> 16) | (w[3] << 16);
+          o[3] = (w[3] >> 16) | (w4 << 16);
+        } else {
+          o = w;
+        }
+      } else {
+        V e[PE];
 #pragma unroll
-  for (int e = 0; e < G; e++)
-    if (c0 + e * 64 < p.out_cols) dst[c0 + e * 64] = v[e];
+        for (uint32_t j = 0; j < PE; j++) e[j] = e0 + j < lim ? src[j] : (V)0;
+        if constexpr (sizeof(V) == 2) {
+#pragma unroll
+          for (uint32_t j = 0; j < 4; j++) o[j] = (uint32_t)e[2 * j] | ((uint32_t)e[2 * j + 1] << 16);
+        } else {
+#pragma unroll
+          for (uint32_t j = 0; j < 4; j++) o[j] = (uint32_t)e[j];
+        }
+      }
+      if (c + PE > p.in_cols) {  // zero beyond the valid columns
+        const uint32_t n = p.in_cols - c;  // 1 .. PE-1 valid elements
+#pragma unroll
+        for (uint32_t j = 0; j < 4; j++) {
+          if constexpr (sizeof(V) == 2) {
+            if (2 * j >= n) o[j] = 0u;
+            else if (2 * j + 1 >= n) o[j] &= 0xffffu;
+          } else {
+            if (j >= n) o[j] = 0u;
+          }
+        }
+      }
+    }
+    *reinterpret_cast<CopyPiece*>(dst + c) = o;
+  }
 }
-HC_KERNEL void hc_copy2d_b2(hck_copy2d_args p) { copy2d_impl<uint16_t, 8>(p); }
-HC_KERNEL void hc_copy2d_b4(hck_copy2d_args p) { copy2d_impl<uint32_t, 8>(p); }
+HC_KERNEL void hc_copy2d_pad_b2(hck_copy2d_args p) { copy2d_pad_impl<uint16_t>(p); }
+HC_KERNEL void hc_copy2d_pad_b4(hck_copy2d_args p) { copy2d_pad_impl<uint32_t>(p); }
+
+template <typename V> __device__ __forceinline__ void copy2d_unpad_impl(const hck_copy2d_args& p) {
+  constexpr uint32_t PE = 16 / sizeof(V);
+  constexpr uint32_t NP = 512 / (64 * PE);
+  const uint32_t groups = (p.out_cols + 511) / 512;
+  const uint64_t unit = (uint64_t)blockIdx.x * (HCK_BLOCK / 64) + (threadIdx.x >> 6);
+  const uint64_t r = unit / groups;
+  if (r >= p.rows) return;
+  const uint32_t g0 = (uint32_t)(unit - r * groups) * 512;
+  const V* src = (const V*)p.in + (uint64_t)blockIdx.y * p.in_bs + r * p.in_ld;
+  V* drow = (V*)p.out + (uint64_t)blockIdx.y * p.out_bs + r * p.out_ld;
+#pragma unroll
+  for (uint32_t i = 0; i < NP; i++) {
+    const uint32_t c = g0 + ((threadIdx.x & 63) + 64 * i) * PE;
+    if (c >= p.out_cols) continue;
+    const CopyPiece v = *reinterpret_cast<const CopyPiece*>(src + c);
+    V* dst = drow + c;
+    const uint32_t n = p.out_cols - c < PE ? p.out_cols - c : PE;
+    if (n == PE && ((uintptr_t)dst & 3) == 0) {
+      *reinterpret_cast<CopyPieceA4*>(dst) = v;
+    } else if (sizeof(V) == 2 && n == PE) {
+      uint16_t* d16 = reinterpret_cast<uint16_t*>(dst);
+      d16[0] = (uint16_t)v[0];
+      uint32_t* d32 = reinterpret_cast<uint32_t*>(d16 + 1);
+      d32[0] = (v[0] >> 16) | (v[1] << 16);
+      d32[1] = (v[1] >> 16) | (v[2] << 16);
+      d32[2] = (v[2] >> 16) | (v[3] << 16);
+      d16[7] = (uint16_t)(v[3] >> 16);
+    } else {
+#pragma unroll
+      for (uint32_t j = 0; j < PE; j++) {
+        if (j < n) {
+          if constexpr (sizeof(V) == 2) dst[j] = (V)(v[j / 2] >> (16 * (j & 1)));
+          else dst[j] = (V)v[j];
+        }
+      }
+    }
+  }
+}
+HC_KERNEL void hc_copy2d_unpad_b2(hck_copy2d_args p) { copy2d_unpad_impl<uint16_t>(p); }
+HC_KERNEL void hc_copy2d_unpad_b4(hck_copy2d_args p) { copy2d_unpad_impl<uint32_t>(p); }
 
 // axisPermutation (BackendCPU.swift:1831-1849): flat source index of every element of the
 // permuted view.

@@ -174,6 +174,34 @@ def test_matmul_random_shapes(hip_backend, oracle_backend, monkeypatch, pipeline
 
 
 @pytest.mark.parametrize("dtype", [F32, F16], ids=["f32", "f16"])
+def test_matmul_repitched_operands_every_residue(hip_backend, oracle_backend, dtype):
+    """Operands and outputs whose rows are not 16-byte aligned are copied into padded buffers and
+    back. Every residue of the row length modulo a 16-byte piece, batches of odd-sized matrices
+    (so matrices start on odd element addresses) and buffers that end exactly with the last
+    element; `A x I` must come back bit for bit, which checks the copies on their own."""
+    rng = np.random.default_rng(808)
+    for r in range(9):
+        batch, M, K, N = 3, 129 + (r % 3), 263 + r, 257 + r  # >= 2^24 multiply-adds: the copies are used
+        a = rand(rng, (batch, M, K), dtype, 1.0 / K ** 0.5)
+        b = rand(rng, (batch, K, N), dtype)
+        for transA, transB, transOut in ((False, False, False), (True, True, False), (False, True, True), (True, False, True)):
+            sa = np.ascontiguousarray(a.transpose(0, 2, 1)) if transA else a
+            sb = np.ascontiguousarray(b.transpose(0, 2, 1)) if transB else b
+            print("repitch", dtype.name, batch, M, K, N, transA, transB, transOut, flush=True)
+            fn = lambda: Tensor.batchedMatmul(Tensor(data=sa), transA, Tensor(data=sb), transB, transOut)
+            got, want = check_close(hip_backend, oracle_backend, fn, TOL[dtype])
+            scale = float(np.max(np.abs(want.astype(np.float64))))
+            assert float(np.max(np.abs(got.astype(np.float64) - want.astype(np.float64)))) <= TOL[dtype] * scale
+        # identity on the right: the product is A itself, exactly (but for -0, which x*1 + 0*0 turns into +0)
+        a[a == 0] = 0
+        eye = np.broadcast_to(np.eye(K, dtype=a.dtype), (batch, K, K)).copy()
+        with hip_backend.use():
+            out = Tensor.batchedMatmul(Tensor(data=a), False, Tensor(data=eye), False, False).numpy()
+        np.testing.assert_array_equal(out.view(np.uint16 if dtype is F16 else np.uint32),
+                                      a.view(np.uint16 if dtype is F16 else np.uint32))
+
+
+@pytest.mark.parametrize("dtype", [F32, F16], ids=["f32", "f16"])
 def test_matmul_skinny_products(hip_backend, oracle_backend, dtype):
     """One extent of C at most 32 (matrix-vector products, fringes of ragged GEMMs): the
     wave-per-row and the lane-per-row / split-K kernels, every layout, a batch, odd strides."""
