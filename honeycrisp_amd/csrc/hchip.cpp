@@ -2135,7 +2135,10 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
   uint32_t c_ld = N;
   const bool c_unaligned = !aligned16(out) || N % P != 0;
   const double work = (double)M * (double)N * (double)K * (double)batch;
-  if ((ma == 'x' || mb == 'x' || c_unaligned) && K > 0 && work >= 16777216.0 && batch <= 65535 &&
+  // (the scalar loads of the general kernel cost about 4 us per 64 of K and tile: a long K pays
+  // for the copies much earlier than a large output does)
+  if ((ma == 'x' || mb == 'x' || c_unaligned) && K > 0 && (work >= 16777216.0 || (work >= 2097152.0 && K >= 256)) &&
+      batch <= 65535 &&
       !getenv("HCHIP_GEMM_NO_REPITCH")) {
     auto round_up = [&](uint32_t v) { return (v + P - 1) / P * P; };
     // (rows, k) element at rows*rs + k*cs with one of the strides 1 (dense storage)
