@@ -99,3 +99,40 @@ def test_row_argmax_and_gather_beyond_2_31_elements(hip_backend, big):
     s = ScatterGatherIndices([ROWS, COLS], 0, BroadcastData(BroadcastStrides([len(ids), COLS], [1, 0]), hip_backend.upload(ids)))
     out = hip_backend.gather(dev, s, F16).onCPU().view(np.float16).reshape(len(ids), COLS)
     assert_same_bits(out, x[ids], "gather")
+
+
+def _pattern(shape, seed):
+    block = np.random.default_rng(seed).standard_normal(33554467).astype(np.float16)
+    block[block == 0] = 0  # no -0: x * 1 + 0 * 0 would turn it into +0
+    return np.resize(block, int(np.prod(shape))).reshape(shape)
+
+
+def test_batched_matmul_operands_beyond_4_gib_in_total(hip_backend):
+    """36 products of 8192^2 fp16 matrices (4.8 GB per operand) with the identity on the right:
+    every matrix must come back bit for bit, so batch offsets beyond 2^32 bytes are right."""
+    batch, n = 36, 8192
+    a = _pattern((batch, n, n), 41)
+    eye = np.ascontiguousarray(np.broadcast_to(np.eye(n, dtype=np.float16), (batch, n, n)))
+    print("batched matmul %d x %d^3" % (batch, n), flush=True)
+    da, de = hip_backend.upload(a), hip_backend.upload(eye)
+    del eye
+    out = hip_backend.batchedMatmul(batch, da, False, de, False, False, n, n, n, F16).onCPU().view(np.float16).reshape(batch, n, n)
+    for b in range(batch):
+        assert_same_bits(out[b], a[b], "A x I, matrix %d" % b)
+
+
+@pytest.mark.parametrize("transA", [False, True], ids=["k_contiguous", "m_contiguous"])
+def test_matmul_single_operand_beyond_4_gib(hip_backend, transA):
+    """One fp16 operand of 4.4 GB (its element offsets no longer fit 32 bits of bytes) times a
+    0/1 selection matrix: column j of the product is column sel[j] of A, exactly."""
+    M, K, N = 36000, 61440, 64
+    a = _pattern((K, M) if transA else (M, K), 42)
+    sel = np.random.default_rng(43).integers(0, K, size=N)
+    sel[:4] = (0, K - 1, K - 64, 32768)
+    b = np.zeros((K, N), dtype=np.float16)
+    b[sel, np.arange(N)] = 1
+    print("matmul %d x %d x %d, transA=%s" % (M, K, N, transA), flush=True)
+    out = hip_backend.matmul(hip_backend.upload(a), transA, hip_backend.upload(b), False, False, M, K, N, F16)
+    out = out.onCPU().view(np.float16).reshape(M, N)
+    want = np.ascontiguousarray((a[sel, :].T if transA else a[:, sel]))
+    assert_same_bits(out, want, "A x selection")
