@@ -1058,3 +1058,36 @@ def test_argsort_long_axes(hip_backend, oracle_backend, dtype):
         check_exact(hip_backend, oracle_backend, lambda: Tensor(data=f).argsort(1))
         got, _ = both(hip_backend, oracle_backend, lambda: Tensor(data=f).gather(1, Tensor(data=f).argsort(1)))
         assert np.all(np.diff(got.astype(np.float32), axis=1) >= 0)
+
+
+@pytest.mark.parametrize("dtype", [F32, F16], ids=["f32", "f16"])
+def test_matmul_pointers_at_odd_element_offsets(hip_backend, oracle_backend, dtype):
+    """Straight through the C ABI: operands and output that start 1, 3 and 5 elements into their
+    allocations (a view into a larger buffer), so that no pointer is 16-byte aligned and, for
+    fp16, some are not even 4-byte aligned. Aligned and odd extents, large enough for the padded
+    copies; the elements around the output must stay untouched."""
+    from ctypes import c_void_p
+    lib, ctx = hip_backend._lib, hip_backend._ctx
+    es = np.dtype(dtype.numpy).itemsize
+    rng = np.random.default_rng(909)
+    for (M, K, N) in [(256, 512, 256), (255, 513, 259), (130, 1000, 131)]:
+        a = rand(rng, (M, K), dtype, 1.0 / K ** 0.5)
+        b = rand(rng, (K, N), dtype)
+        with oracle_backend.use():
+            want = Tensor.matmul(Tensor(data=a), False, Tensor(data=b), False, False).numpy()
+        offs = (1, 3, 5)
+        host_a = np.zeros(M * K + 16, dtype=a.dtype)
+        host_a[offs[0]:offs[0] + M * K] = a.reshape(-1)
+        host_b = np.zeros(K * N + 16, dtype=a.dtype)
+        host_b[offs[1]:offs[1] + K * N] = b.reshape(-1)
+        guard = rand(rng, (M * N + 16,), dtype)
+        da, db, dc = hip_backend.upload(host_a), hip_backend.upload(host_b), hip_backend.upload(guard)
+        print("matmul at odd offsets", dtype.name, M, K, N, flush=True)
+        hip_backend._check(lib.hc_matmul(ctx, int(dtype), 1, c_void_p(da.ptr + offs[0] * es), 0,
+                                         c_void_p(db.ptr + offs[1] * es), 0, 0, M, K, N, c_void_p(dc.ptr + offs[2] * es)))
+        out = dc.onCPU().view(a.dtype)
+        got = out[offs[2]:offs[2] + M * N].reshape(M, N)
+        assert_close_arrays(got, want, TOL[dtype], TOL[dtype])
+        bits = np.uint16 if dtype is F16 else np.uint32
+        assert np.array_equal(out[:offs[2]].view(bits), guard[:offs[2]].view(bits))
+        assert np.array_equal(out[offs[2] + M * N:].view(bits), guard[offs[2] + M * N:].view(bits))
