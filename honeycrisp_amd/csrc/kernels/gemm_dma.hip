@@ -39,6 +39,7 @@
 // The stages are distinct __shared__ arrays and the loop is unrolled by four so that every
 // LDS access names its stage statically.
 #include "common.hip.h"
+#include <type_traits>
 
 #ifndef HC_READS_PER_SLOT
 #define HC_READS_PER_SLOT 0
@@ -270,10 +271,16 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
     else if (u < READS) oa.read(u - OpB::READS, s, stage, f.a);
   };
   // unit u of the DMA of the K-slice starting at k0
-  auto dma_unit = [&](int u, uint32_t k0, char* stage) {
-    if (u < OpA::NI) oa.dma(u, A, k0, stage, kend);
-    else if (u < NDMA) ob.dma(u - OpA::NI, B, k0, stage + A_BYTES, kend);
+  // `tail`: a compile-time flag. Only the last K-slice can be ragged, so only the DMA that may
+  // fetch it carries the range check of the edge kernels (a scalar compare and a branch in
+  // front of every DMA instruction otherwise, in the middle of the MFMA stream).
+  auto dma_unit = [&](auto tail, int u, uint32_t k0, char* stage) {
+    const uint32_t ke = decltype(tail)::value ? kend : 0;
+    if (u < OpA::NI) oa.dma(u, A, k0, stage, ke);
+    else if (u < NDMA) ob.dma(u - OpA::NI, B, k0, stage + A_BYTES, ke);
   };
+  typedef std::integral_constant<bool, EDGE> Tail;     // checks where the kernel has them at all
+  typedef std::integral_constant<bool, false> NoTail;
   // MFMA t of a sub-step; operands swapped (B first) so that a lane holds four consecutive
   // n for one m (see the epilogue).
   auto mma_one = [&](const Frags& f, int t) {
@@ -304,12 +311,12 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
 #endif
 
   // K-step j out of `cur`; `nxt` holds K-step j+1, `prev` held K-step j-1.
-  auto step = [&](char* cur, char* nxt, char* prev, uint32_t j) {
+  auto step = [&](auto tail, char* cur, char* nxt, char* prev, uint32_t j) {
     const uint32_t k3 = (j + 3 < nk ? j + 3 : nk - 1) * BK, k4 = (j + 4 < nk ? j + 4 : nk - 1) * BK;
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int t = 0; t < SLOTS; t++) {  // sub-step 0
-      if (t % DSTRIDE == 0 && HALF + t / DSTRIDE < NDMA) dma_unit(HALF + t / DSTRIDE, k3, prev);
+      if (t % DSTRIDE == 0 && HALF + t / DSTRIDE < NDMA) dma_unit(tail, HALF + t / DSTRIDE, k3, prev);
 #pragma unroll
       for (int e = 0; e < RPS; e++) read_unit(f1, cur, 1, t * RPS + e);
       mma_one(f0, t);
@@ -334,7 +341,7 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int t = 0; t < SLOTS; t++) {  // sub-step 1
-      if (t % DSTRIDE == 0 && t / DSTRIDE < HALF) dma_unit(t / DSTRIDE, k4, cur);
+      if (t % DSTRIDE == 0 && t / DSTRIDE < HALF) dma_unit(tail, t / DSTRIDE, k4, cur);
 #pragma unroll
       for (int e = 0; e < RPS; e++) read_unit(f0, nxt, 0, t * RPS + e);
       mma_one(f1, t);
@@ -346,13 +353,13 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
   // last one; nobody reads them)
   auto kclamp = [&](uint32_t j) { return (j < nk ? j : nk - 1) * BK; };
 #pragma unroll
-  for (int u = 0; u < NDMA; u++) dma_unit(u, 0, lds0);
+  for (int u = 0; u < NDMA; u++) dma_unit(Tail{}, u, 0, lds0);
 #pragma unroll
-  for (int u = 0; u < NDMA; u++) dma_unit(u, kclamp(1), lds1);
+  for (int u = 0; u < NDMA; u++) dma_unit(Tail{}, u, kclamp(1), lds1);
 #pragma unroll
-  for (int u = 0; u < NDMA; u++) dma_unit(u, kclamp(2), lds2);
+  for (int u = 0; u < NDMA; u++) dma_unit(Tail{}, u, kclamp(2), lds2);
 #pragma unroll
-  for (int u = 0; u < HALF; u++) dma_unit(u, kclamp(3), lds3);
+  for (int u = 0; u < HALF; u++) dma_unit(Tail{}, u, kclamp(3), lds3);
   wait_dma<2 * NDMA + HALF>();
   lds_barrier();
 #pragma unroll
@@ -362,15 +369,23 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
   const uint64_t probe_c0 = __builtin_readcyclecounter(), probe_r0 = __builtin_amdgcn_s_memrealtime();
 #endif
   uint32_t j = 0;
-  for (; j + 3 < nk; j += 4) {
-    step(lds0, lds1, lds3, j);
-    step(lds1, lds2, lds0, j + 1);
-    step(lds2, lds3, lds1, j + 2);
-    step(lds3, lds0, lds2, j + 3);
+  if constexpr (EDGE) {  // K-step j fetches slices j+3 and j+4: up to j = nk-6 the last slice is not among them
+    for (; j + 9 <= nk; j += 4) {
+      step(NoTail{}, lds0, lds1, lds3, j);
+      step(NoTail{}, lds1, lds2, lds0, j + 1);
+      step(NoTail{}, lds2, lds3, lds1, j + 2);
+      step(NoTail{}, lds3, lds0, lds2, j + 3);
+    }
   }
-  if (j < nk) step(lds0, lds1, lds3, j);
-  if (j + 1 < nk) step(lds1, lds2, lds0, j + 1);
-  if (j + 2 < nk) step(lds2, lds3, lds1, j + 2);
+  for (; j + 3 < nk; j += 4) {
+    step(Tail{}, lds0, lds1, lds3, j);
+    step(Tail{}, lds1, lds2, lds0, j + 1);
+    step(Tail{}, lds2, lds3, lds1, j + 2);
+    step(Tail{}, lds3, lds0, lds2, j + 3);
+  }
+  if (j < nk) step(Tail{}, lds0, lds1, lds3, j);
+  if (j + 1 < nk) step(Tail{}, lds1, lds2, lds0, j + 1);
+  if (j + 2 < nk) step(Tail{}, lds2, lds3, lds1, j + 2);
   wait_dma<0>();  // no LDS write of this workgroup may be in flight when it ends
 #if defined(HC_PROBE_CLOCKS) || defined(HC_PROBE_WAITS)
   // measurement build: the first 16 bytes of the block's C tile receive the K-loop duration

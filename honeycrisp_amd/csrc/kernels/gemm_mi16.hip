@@ -263,10 +263,16 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
     if (u < RdB::READS) rb.read(u, s, stage + A_BYTES, f.b);
     else if (u < READS) ra.read(u - RdB::READS, s, stage, f.a);
   };
-  auto dma_unit = [&](int u, uint32_t k0, char* stage) {
-    if (u < OpA::NI) oa.dma(u, A, k0, stage, kend);
-    else if (u < NDMA) ob.dma(u - OpA::NI, B, k0, stage + A_BYTES, kend);
+  // `tail`: a compile-time flag. Only the last K-slice can be ragged, so only the DMA that may
+  // fetch it carries the range check of the edge kernels (a scalar compare and a branch in
+  // front of every DMA instruction otherwise, in the middle of the MFMA stream).
+  auto dma_unit = [&](auto tail, int u, uint32_t k0, char* stage) {
+    const uint32_t ke = decltype(tail)::value ? kend : 0;
+    if (u < OpA::NI) oa.dma(u, A, k0, stage, ke);
+    else if (u < NDMA) ob.dma(u - OpA::NI, B, k0, stage + A_BYTES, ke);
   };
+  typedef std::integral_constant<bool, EDGE> Tail;     // checks where the kernel has them at all
+  typedef std::integral_constant<bool, false> NoTail;
   // MFMA t of a sub-step; operands swapped (B first) so that a lane holds four consecutive n
   auto mma_one = [&](const Frags& f, int t) {
     const int j = t / MT, i = t % MT;
@@ -296,8 +302,8 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
 #endif
 
   // (compile-time loop indices throughout: every register array is indexed statically)
-  auto substep = [&](const Frags& use, Frags& fill, const char* from, auto s_next_c, auto part_c, char* to,
-                     uint32_t k0) {
+  auto substep = [&](auto tail, const Frags& use, Frags& fill, const char* from, auto s_next_c, auto part_c,
+                     char* to, uint32_t k0) {
     constexpr int s_next = decltype(s_next_c)::value, part = decltype(part_c)::value;
     static_for<SLOTS>([&](auto tc) {
       constexpr int t = decltype(tc)::value;
@@ -306,7 +312,7 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
       constexpr int lo = (w * NDMA + W - 1) / W < NDMA ? (w * NDMA + W - 1) / W : NDMA;
       constexpr int hi = ((w + 1) * NDMA + W - 1) / W < NDMA ? ((w + 1) * NDMA + W - 1) / W : NDMA;
 #ifndef HC_MI16_NO_LOOP_DMA  // (measurement switch: wrong results)
-      static_for<hi - lo>([&](auto uc) { dma_unit(lo + decltype(uc)::value, k0, to); });
+      static_for<hi - lo>([&](auto uc) { dma_unit(tail, lo + decltype(uc)::value, k0, to); });
 #endif
       // operand reads of the following sub-step: one every RSTRIDE slots
 #ifndef HC_MI16_NO_LOOP_READS  // (measurement switch: wrong results)
@@ -320,9 +326,9 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
   };
 
   // K-step j out of `cur`; `nxt` receives the rest of K-step j+1, then `cur` K-step j+2
-  auto step = [&](char* cur, char* nxt, uint32_t j) {
+  auto step = [&](auto tail, char* cur, char* nxt, uint32_t j) {
     __builtin_amdgcn_sched_barrier(0);
-    substep(f0, f1, cur, std::integral_constant<int, 1>{}, std::integral_constant<int, 1>{}, nxt, kclamp(j + 1));
+    substep(tail, f0, f1, cur, std::integral_constant<int, 1>{}, std::integral_constant<int, 1>{}, nxt, kclamp(j + 1));
 #ifdef HC_PROBE_WAITS
     const uint64_t w0 = __builtin_readcyclecounter();
     wait_dma<0>();
@@ -336,12 +342,12 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
     lds_barrier();  // ... and everybody's; nobody reads cur any more
 #endif
     __builtin_amdgcn_sched_barrier(0);
-    substep(f1, f0, nxt, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, cur, kclamp(j + 2));
+    substep(tail, f1, f0, nxt, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, cur, kclamp(j + 2));
   };
 
   // prologue: K-step 0 and the first window part of K-step 1
-  static_for<NDMA>([&](auto uc) { dma_unit(decltype(uc)::value, 0, lds0); });
-  static_for<U0>([&](auto uc) { dma_unit(decltype(uc)::value, kclamp(1), lds1); });
+  static_for<NDMA>([&](auto uc) { dma_unit(Tail{}, decltype(uc)::value, 0, lds0); });
+  static_for<U0>([&](auto uc) { dma_unit(Tail{}, decltype(uc)::value, kclamp(1), lds1); });
   wait_dma<U0>();
   lds_barrier();
   static_for<READS>([&](auto uc) { read_unit(f0, lds0, 0, decltype(uc)::value); });
@@ -350,11 +356,17 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
   const uint64_t probe_c0 = __builtin_readcyclecounter(), probe_r0 = __builtin_amdgcn_s_memrealtime();
 #endif
   uint32_t j = 0;
-  for (; j + 1 < nk; j += 2) {
-    step(lds0, lds1, j);
-    step(lds1, lds0, j + 1);
+  if constexpr (EDGE) {  // K-step j fetches slices j+1 and j+2: up to j = nk-4 the last slice is not among them
+    for (; j + 5 <= nk; j += 2) {
+      step(NoTail{}, lds0, lds1, j);
+      step(NoTail{}, lds1, lds0, j + 1);
+    }
   }
-  if (j < nk) step(lds0, lds1, j);
+  for (; j + 1 < nk; j += 2) {
+    step(Tail{}, lds0, lds1, j);
+    step(Tail{}, lds1, lds0, j + 1);
+  }
+  if (j < nk) step(Tail{}, lds0, lds1, j);
   wait_dma<0>();  // no LDS write of this workgroup may be in flight when it ends
   // The compiler does not know that the assembly statements are MFMAs, so it would not keep the
   // epilogue's accumulator reads the required distance from the last of them: do it by hand.
