@@ -38,6 +38,7 @@
 // issuing wave behind the texture-address queue). The two stages are distinct __shared__
 // arrays and the loop is unrolled by two so that every LDS access names its stage statically.
 #include "common.hip.h"
+#include <type_traits>
 
 // length of the DMA window in half sub-steps (see the K loop)
 #ifndef HC_DMA_WINDOW_X2
@@ -280,10 +281,16 @@ __device__ __forceinline__ void gemm_dma2_impl(const hck_gemm_args& p, char* lds
     else if (u < READS) oa.read(u - OpB::READS, s, stage, f.a);
   };
   // unit u of the DMA of the K-slice starting at k0
-  auto dma_unit = [&](int u, uint32_t k0, char* stage) {
-    if (u < OpA::NI) oa.dma(u, A, k0, stage, kend);
-    else if (u < NDMA) ob.dma(u - OpA::NI, B, k0, stage + A_BYTES, kend);
+  // `tail`: a compile-time flag. Only the last K-slice can be ragged, so only the DMA that may
+  // fetch it carries the range check of the edge kernels (a scalar compare and a branch in
+  // front of every DMA instruction otherwise, in the middle of the MFMA stream).
+  auto dma_unit = [&](auto tail, int u, uint32_t k0, char* stage) {
+    const uint32_t ke = decltype(tail)::value ? kend : 0;
+    if (u < OpA::NI) oa.dma(u, A, k0, stage, ke);
+    else if (u < NDMA) ob.dma(u - OpA::NI, B, k0, stage + A_BYTES, ke);
   };
+  typedef std::integral_constant<bool, EDGE> Tail;     // checks where the kernel has them at all
+  typedef std::integral_constant<bool, false> NoTail;
   // MFMA t of a sub-step; operands swapped (B first) so that a lane holds four consecutive
   // n for one m (see the epilogue).
   auto mma_one = [&](const Frags& f, int t) {
@@ -325,13 +332,14 @@ __device__ __forceinline__ void gemm_dma2_impl(const hck_gemm_args& p, char* lds
   // sub-step: MFMAs on `use`, operands of the following sub-step (number s_next of `from`)
   // into `fill`, and the DMA units of window part `part` (0, 1, 2; -1: none) of the K-slice
   // at k0 into `to`
-  auto substep = [&](const Frags& use, Frags& fill, const char* from, int s_next, int part, char* to, uint32_t k0) {
+  auto substep = [&](auto tail, const Frags& use, Frags& fill, const char* from, int s_next, int part, char* to,
+                     uint32_t k0) {
 #pragma unroll
     for (int t = 0; t < SLOTS; t++) {
       if (part >= 0) {
 #pragma unroll
         for (int u = 0; u < NDMA; u++)
-          if (window_slot(u) == part * SLOTS + t) dma_unit(u, k0, to);
+          if (window_slot(u) == part * SLOTS + t) dma_unit(tail, u, k0, to);
       }
 #pragma unroll
       for (int e = 0; e < RPS; e++) read_unit(fill, from, s_next, t * RPS + e);
@@ -341,11 +349,11 @@ __device__ __forceinline__ void gemm_dma2_impl(const hck_gemm_args& p, char* lds
   };
 
   // K-step j out of `cur`; `nxt` receives the rest of K-step j+1, then `cur` the start of j+2
-  auto step = [&](char* cur, char* nxt, uint32_t j) {
+  auto step = [&](auto tail, char* cur, char* nxt, uint32_t j) {
     __builtin_amdgcn_sched_barrier(0);
-    substep(f0, f1, cur, 1, 1, nxt, kclamp(j + 1));
-    substep(f1, f0, cur, 2, 2, nxt, kclamp(j + 1));
-    substep(f0, f1, cur, 3, -1, nullptr, 0);
+    substep(tail, f0, f1, cur, 1, 1, nxt, kclamp(j + 1));
+    substep(tail, f1, f0, cur, 2, 2, nxt, kclamp(j + 1));
+    substep(tail, f0, f1, cur, 3, -1, nullptr, 0);
 #ifdef HC_PROBE_WAITS
     const uint64_t w0 = __builtin_readcyclecounter();
     wait_dma<0>();
@@ -359,14 +367,14 @@ __device__ __forceinline__ void gemm_dma2_impl(const hck_gemm_args& p, char* lds
     lds_barrier();  // ... and everybody's; nobody reads cur any more
 #endif
     __builtin_amdgcn_sched_barrier(0);
-    substep(f1, f0, nxt, 0, 0, cur, kclamp(j + 2));
+    substep(tail, f1, f0, nxt, 0, 0, cur, kclamp(j + 2));
   };
 
   // prologue: K-step 0 and the first window part of K-step 1
 #pragma unroll
-  for (int u = 0; u < NDMA; u++) dma_unit(u, 0, lds0);
+  for (int u = 0; u < NDMA; u++) dma_unit(Tail{}, u, 0, lds0);
 #pragma unroll
-  for (int u = 0; u < U0; u++) dma_unit(u, kclamp(1), lds1);
+  for (int u = 0; u < U0; u++) dma_unit(Tail{}, u, kclamp(1), lds1);
   wait_dma<U0>();
   lds_barrier();
 #pragma unroll
@@ -376,11 +384,17 @@ __device__ __forceinline__ void gemm_dma2_impl(const hck_gemm_args& p, char* lds
   const uint64_t probe_c0 = __builtin_readcyclecounter(), probe_r0 = __builtin_amdgcn_s_memrealtime();
 #endif
   uint32_t j = 0;
-  for (; j + 1 < nk; j += 2) {
-    step(lds0, lds1, j);
-    step(lds1, lds0, j + 1);
+  if constexpr (EDGE) {  // K-step j fetches slices j+1 and j+2: up to j = nk-4 the last slice is not among them
+    for (; j + 5 <= nk; j += 2) {
+      step(NoTail{}, lds0, lds1, j);
+      step(NoTail{}, lds1, lds0, j + 1);
+    }
   }
-  if (j < nk) step(lds0, lds1, j);
+  for (; j + 1 < nk; j += 2) {
+    step(Tail{}, lds0, lds1, j);
+    step(Tail{}, lds1, lds0, j + 1);
+  }
+  if (j < nk) step(Tail{}, lds0, lds1, j);
   wait_dma<0>();  // no LDS write of this workgroup may be in flight when it ends
 #ifdef HC_PROBE_WAITS
   const uint64_t probe_c1 = __builtin_readcyclecounter(), probe_r1 = __builtin_amdgcn_s_memrealtime();
