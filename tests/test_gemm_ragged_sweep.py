@@ -1,0 +1,141 @@
+"""The ragged-shape sweep M, K, N in {127, 1000, 4097} of the fp16 GEMM workload, all 27 shapes, and
+the products that the host splits into a multiple-of-256 body plus thin fringes (extents 1..32 over
+a multiple of 256, K >= 2048): straight through hc_matmul (the C ABI), every storage layout.
+
+What is compared, per product:
+  * row slabs (first / middle / last rows, the last ones being the fringe rows) x all columns and
+    all rows x column slabs (first / last columns: the fringe columns) against the CPU oracle
+    (BackendCPU.swift:1260-1304 restated), tolerance 1e-2 (fp16) / 1e-4 (fp32);
+  * the whole result against the general kernel (HCHIP_GEMM_TILE=general: no tuned tile, no split)
+    and against the same call with HCHIP_GEMM_NO_PEEL=1 (tuned tiles, no split);
+  * guard elements in front of and behind the output: nothing may be written outside C.
+"""
+import os
+from contextlib import contextmanager
+from ctypes import c_void_p
+
+import numpy as np
+import pytest
+
+from honeycrisp_amd.descriptors import DType
+from honeycrisp_amd.tensor import Tensor
+from backend_cases import assert_close_arrays
+
+pytestmark = pytest.mark.gpu
+
+F32, F16 = DType.float32, DType.float16
+TOL = {F32: 1e-4, F16: 1e-2}
+GUARD = 64  # elements on either side of C (a multiple of 16 bytes: C keeps its natural alignment)
+
+
+@contextmanager
+def env(**kv):
+    old = {k: os.environ.get(k) for k in kv}
+    os.environ.update(kv)
+    try:
+        yield
+    finally:
+        for k, v in old.items():
+            if v is None:
+                os.environ.pop(k, None)
+            else:
+                os.environ[k] = v
+
+
+def slabs(n, width=8):
+    """First, middle and last `width` indices of range(n), without repeats."""
+    idx = np.r_[0:min(width, n), max(n // 2 - width // 2, 0):min(n // 2 + width // 2, n), max(n - width, 0):n]
+    return np.unique(idx)
+
+
+class Product:
+    """One product A[batch, M, K] x B[batch, K, N] with its operands on the device in both storage
+    orders and oracle values for row and column slabs of C."""
+
+    def __init__(self, hip, oracle, dtype, batch, M, K, N, seed):
+        rng = np.random.default_rng(seed)
+        self.hip, self.dtype, self.batch, self.M, self.K, self.N = hip, dtype, batch, M, K, N
+        np_t = dtype.numpy
+        a = (rng.standard_normal((batch, M, K)) / np.sqrt(K)).astype(np_t)
+        b = rng.standard_normal((batch, K, N)).astype(np_t)
+        self.rows, self.cols = slabs(M), slabs(N)
+        with oracle.use():
+            self.want_rows = Tensor.batchedMatmul(Tensor(data=np.ascontiguousarray(a[:, self.rows])), False,
+                                                  Tensor(data=b), False, False).numpy()
+            self.want_cols = Tensor.batchedMatmul(Tensor(data=a), False,
+                                                  Tensor(data=np.ascontiguousarray(b[:, :, self.cols])), False,
+                                                  False).numpy()
+        self.dev = {("a", False): hip.upload(a), ("a", True): hip.upload(np.ascontiguousarray(a.transpose(0, 2, 1))),
+                    ("b", False): hip.upload(b), ("b", True): hip.upload(np.ascontiguousarray(b.transpose(0, 2, 1)))}
+        self.guard = rng.standard_normal(batch * M * N + 2 * GUARD).astype(np_t)
+        self.guard_dev = hip.upload(self.guard)
+
+    def run(self, transA, transB, transOut):
+        """C as [batch, M, N] (a transposed output is transposed back on the host)."""
+        hip, es = self.hip, np.dtype(self.dtype.numpy).itemsize
+        n_out = self.batch * self.M * self.N
+        out = hip.allocate(self.guard.nbytes)
+        hip._check(hip._lib.hc_memcpy_d2d(hip._ctx, c_void_p(out.ptr), c_void_p(self.guard_dev.ptr), self.guard.nbytes))
+        hip._check(hip._lib.hc_matmul(hip._ctx, int(self.dtype), self.batch, c_void_p(self.dev[("a", transA)].ptr),
+                                      int(transA), c_void_p(self.dev[("b", transB)].ptr), int(transB), int(transOut),
+                                      self.M, self.K, self.N, c_void_p(out.ptr + GUARD * es)))
+        host = out.onCPU().view(self.dtype.numpy)
+        bits = np.uint16 if self.dtype is F16 else np.uint32
+        assert np.array_equal(host[:GUARD].view(bits), self.guard[:GUARD].view(bits)), "wrote in front of C"
+        assert np.array_equal(host[GUARD + n_out:].view(bits), self.guard[GUARD + n_out:].view(bits)), "wrote behind C"
+        c = host[GUARD:GUARD + n_out]
+        if transOut:
+            return c.reshape(self.batch, self.N, self.M).transpose(0, 2, 1)
+        return c.reshape(self.batch, self.M, self.N)
+
+    def check_against_oracle(self, c):
+        tol = TOL[self.dtype]
+        assert_close_arrays(np.ascontiguousarray(c[:, self.rows]), self.want_rows, tol, tol)
+        assert_close_arrays(np.ascontiguousarray(c[:, :, self.cols]), self.want_cols, tol, tol)
+        scale = float(np.max(np.abs(self.want_rows.astype(np.float64))))
+        err = float(np.max(np.abs(c[:, self.rows].astype(np.float64) - self.want_rows.astype(np.float64))))
+        assert err <= tol * scale
+
+    def check_all(self, layouts, label):
+        tol = TOL[self.dtype]
+        with env(HCHIP_GEMM_TILE="general"):
+            general = self.run(False, False, False)
+        self.check_against_oracle(general)
+        for (transA, transB, transOut) in layouts:
+            print(label, self.dtype.name, self.batch, self.M, self.K, self.N, transA, transB, transOut, flush=True)
+            c = self.run(transA, transB, transOut)
+            self.check_against_oracle(c)
+            assert_close_arrays(np.ascontiguousarray(c), general, tol, tol)
+            with env(HCHIP_GEMM_NO_PEEL="1"):
+                whole = self.run(transA, transB, transOut)
+            assert_close_arrays(np.ascontiguousarray(c), np.ascontiguousarray(whole), tol, tol)
+
+
+ALL_LAYOUTS = [(ta, tb, to) for to in (False, True) for ta in (False, True) for tb in (False, True)]
+FOUR_LAYOUTS = [(ta, tb, False) for ta in (False, True) for tb in (False, True)]
+SWEEP = [(m, k, n) for m in (127, 1000, 4097) for k in (127, 1000, 4097) for n in (127, 1000, 4097)]
+
+
+@pytest.mark.parametrize("shape", SWEEP, ids=lambda s: "x".join(map(str, s)))
+def test_ragged_sweep_fp16(hip_backend, oracle_backend, shape):
+    """All 27 shapes of the sweep in the four storage layouts; the cubes and the three shapes that
+    are split into body and fringes (4097^3, 4097 x 4097 x 1000, 1000 x 4097 x 4097 as M x K x N)
+    also with a transposed output."""
+    M, K, N = shape
+    peeled = K == 4097 and ((M == 4097 and N >= 1000) or (N == 4097 and M >= 1000))
+    layouts = ALL_LAYOUTS if (M == K == N or peeled) else FOUR_LAYOUTS
+    Product(hip_backend, oracle_backend, F16, 1, M, K, N, seed=M * 7 + K * 3 + N).check_all(layouts, "sweep")
+
+
+# (batch, M, K, N): extents 1..32 over a multiple of 256 with K >= 2048. Fringes of 1..4 rows or
+# columns run on the skinny kernels, 5..32 on 64 x 64 edge tiles. 16-byte aligned rows need no
+# padded copies (sub-blocks of the caller's own buffers); odd extents go through them.
+PEEL_SHAPES = [(1, 4104, 4096, 4112), (1, 4128, 2048, 2056), (1, 4097, 2048, 4100), (2, 2050, 2304, 4128),
+               (1, 2056, 4100, 2049), (3, 2052, 2048, 2080)]
+
+
+@pytest.mark.parametrize("dtype", [F16, F32], ids=["f16", "f32"])
+@pytest.mark.parametrize("shape", PEEL_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_body_plus_fringes(hip_backend, oracle_backend, dtype, shape):
+    batch, M, K, N = shape
+    Product(hip_backend, oracle_backend, dtype, batch, M, K, N, seed=batch + M + K + N).check_all(ALL_LAYOUTS, "peel")
