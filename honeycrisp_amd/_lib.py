@@ -94,6 +94,7 @@ PROTOTYPES = {
     "hc_pow": (c_int, [_P, c_int, _P, c_float, c_float, c_int64, c_int64, _P, _P, c_size_t]),
     "hc_elemwise": (c_int, [_P, c_int, c_int, _P, _P, _P, c_size_t]),
     "hc_reduce": (c_int, [_P, c_int, c_int, _P, _P, c_int64, c_int64, c_int64]),
+    "hc_reduce_noalloc": (c_int, [_P, c_int, c_int, _P, _P, c_int64, c_int64, c_int64]),
     "hc_cumulative": (c_int, [_P, c_int, c_int, _P, _P, c_int64, c_int64, c_int64, c_int, c_int]),
     "hc_argsort": (c_int, [_P, c_int, _P, _P, c_int64, c_int64, c_int64, c_int]),
     "hc_probe_mfma": (c_int, [_P, c_int, _P, ctypes.c_uint64, ctypes.c_uint32, POINTER(ctypes.c_double)]),

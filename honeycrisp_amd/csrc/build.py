@@ -58,10 +58,16 @@ def build_all(verbose=True):
             path = f.result()
             if verbose:
                 print("built", os.path.relpath(path, HERE), os.path.getsize(path), "bytes")
+    # The one source with device code linked into the library itself (a file-scope device array whose
+    # address the host takes with hipGetSymbolAddress): compiled by hipcc to an object.
+    noalloc_obj = os.path.join(BUILD_DIR, "noalloc.o")
+    _run([HIPCC, "--offload-arch=gfx950", "-O2", "-std=c++17", "-fPIC", "-c",
+          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+          os.path.join(HERE, "noalloc.hip"), "-o", noalloc_obj])
     host_flags = ["-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-I" + os.path.join(ROCM, "include")]
     _run(["g++"] + host_flags + [
         "-Wa,-I," + BUILD_DIR,
-        os.path.join(HERE, "hchip.cpp"), os.path.join(HERE, "embed.S"),
+        os.path.join(HERE, "hchip.cpp"), os.path.join(HERE, "embed.S"), noalloc_obj,
         "-o", LIB_PATH,
         "-L" + os.path.join(ROCM, "lib"), "-lamdhip64", "-Wl,-rpath," + os.path.join(ROCM, "lib"),
         "-lpthread",

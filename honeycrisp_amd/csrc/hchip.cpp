@@ -34,6 +34,9 @@ extern const unsigned char hc_image_gemm_dma2[], hc_image_gemm_dma2_end[];
 extern const unsigned char hc_image_gemm_mi16[], hc_image_gemm_mi16_end[];
 }
 
+// noalloc.hip: looks up this device's copy of the library's fixed scratch array (device current)
+int hc_noalloc_setup(int device);
+
 struct hc_module {
   hipModule_t mod;
 };
@@ -132,6 +135,7 @@ extern "C" int hc_init(int device, hc_ctx** out) {
     return fail(HC_ERR_NO_DEVICE, "no HIP device available (%s)", hipGetErrorString(e));
   REQUIRE(device >= 0 && device < count, "hc_init: device %d out of range (have %d)", device, count);
   HIP_TRY(hipSetDevice(device));
+  HC_TRY(hc_noalloc_setup(device));
   hc_ctx* ctx = new hc_ctx();
   ctx->device = device;
   e = hipGetDeviceProperties(&ctx->props, device);
@@ -1092,15 +1096,31 @@ extern "C" int hc_fill(hc_ctx* ctx, int dtype, float vf, int64_t vi, void* out, 
   return launch_contiguous(ctx, name, count, vec_for_size(el), &k, sizeof(k));
 }
 
-// Temporaries of one entry point: freed (stream-ordered) when it returns.
+// Temporaries of one entry point. Normally blocks of the context's pool, freed (stream-ordered)
+// when the entry point returns. With an arena (a caller-provided device range) the pieces are cut
+// from that range instead, 256-byte aligned, and nothing is allocated or freed.
 struct Scratch {
   hc_ctx* ctx;
   std::vector<void*> ptrs;
+  char* arena = nullptr;
+  size_t arena_bytes = 0, arena_used = 0;
   explicit Scratch(hc_ctx* c) : ctx(c) {}
+  Scratch(hc_ctx* c, void* base, size_t bytes) : ctx(c), arena((char*)base), arena_bytes(bytes) {}
   ~Scratch() {
     for (void* p : ptrs) (void)hc_free(ctx, p);
   }
+  bool fixed() const { return arena != nullptr; }
   int get(size_t bytes, void** out) {
+    if (arena) {
+      const size_t need = (bytes + 255) / 256 * 256;
+      if (need > arena_bytes - arena_used)
+        return fail(HC_ERR_TOO_LARGE,
+                    "this call needs %zu bytes of scratch memory, the fixed scratch buffer holds %zu (%zu in use)",
+                    bytes, arena_bytes, arena_used);
+      *out = arena + arena_used;
+      arena_used += need;
+      return HC_OK;
+    }
     int s = hc_malloc(ctx, bytes, out);
     if (s == HC_OK) ptrs.push_back(*out);
     return s;
@@ -1124,8 +1144,8 @@ static int check_dims(const char* who, int64_t outer, int64_t reduce, int64_t in
 // the alignment) along inner, the reduce axis split over blocks until the device is full,
 // partials combined by a second launch of the same kernel over the [outer, splits, inner]
 // partials. `opname` also covers the internal float-result reductions (maxf, expsumf, sumf).
-static int reduce_cols(hc_ctx* ctx, const char* opname, int dtype, const void* in, const float* aux, void* out,
-                       int64_t outer, int64_t reduce, int64_t inner, bool arg) {
+static int reduce_cols(hc_ctx* ctx, Scratch& scratch, const char* opname, int dtype, const void* in, const float* aux,
+                       void* out, int64_t outer, int64_t reduce, int64_t inner, bool arg) {
   const size_t el = dtype_size(dtype);
   const uint32_t vec = (aligned16(in) && ((uint64_t)inner * el) % 16 == 0) ? (uint32_t)(16 / el) : 1;
   // lanes of a wave along inner: a power of two that covers it, at most 64
@@ -1156,7 +1176,6 @@ static int reduce_cols(hc_ctx* ctx, const char* opname, int dtype, const void* i
   if (c.chunk == 0) c.chunk = 4;
   splits = reduce ? ceil_div((uint64_t)reduce, c.chunk) : 1;
   c.splits = (uint32_t)splits;
-  Scratch scratch(ctx);
   if (splits > 1) {
     const size_t n = (size_t)outer * splits * (size_t)inner;
     HC_TRY(scratch.get(n * (dtype == HC_I64 ? 8 : 4), &c.pvals));
@@ -1185,11 +1204,11 @@ static int softmax_cols(hc_ctx* ctx, int dtype, const void* in, const void* grad
   void *m = nullptr, *s = nullptr, *gs = nullptr;
   HC_TRY(scratch.get(cols * 4, &m));
   HC_TRY(scratch.get(cols * 4, &s));
-  HC_TRY(reduce_cols(ctx, "maxf", dtype, in, nullptr, m, outer, reduce, inner, false));
-  HC_TRY(reduce_cols(ctx, "expsumf", dtype, in, (const float*)m, s, outer, reduce, inner, false));
+  HC_TRY(reduce_cols(ctx, scratch, "maxf", dtype, in, nullptr, m, outer, reduce, inner, false));
+  HC_TRY(reduce_cols(ctx, scratch, "expsumf", dtype, in, (const float*)m, s, outer, reduce, inner, false));
   if (grad) {
     HC_TRY(scratch.get(cols * 4, &gs));
-    HC_TRY(reduce_cols(ctx, "sumf", dtype, grad, nullptr, gs, outer, reduce, inner, false));
+    HC_TRY(reduce_cols(ctx, scratch, "sumf", dtype, grad, nullptr, gs, outer, reduce, inner, false));
   }
   hck_softmax_cols_args k;
   memset(&k, 0, sizeof(k));
@@ -1212,8 +1231,9 @@ static int softmax_cols(hc_ctx* ctx, int dtype, const void* in, const void* grad
   return launch(ctx, name, ceil_div(lanes, HCK_BLOCK), 1, &k, sizeof(k));
 }
 
-extern "C" int hc_reduce(hc_ctx* ctx, int op, int dtype, const void* in, void* out, int64_t outer,
-                         int64_t reduce, int64_t inner) {
+// hc_reduce proper; `scratch` says where partial results live (the pool, or a fixed range).
+static int reduce_impl(hc_ctx* ctx, Scratch& scratch, int op, int dtype, const void* in, void* out, int64_t outer,
+                       int64_t reduce, int64_t inner) {
   REQUIRE(ctx, "hc_reduce: null context");
   REQUIRE(op >= HC_SUM && op <= HC_ARGMIN, "hc_reduce: bad op %d", op);
   if (dtype != HC_F32 && dtype != HC_F16 && dtype != HC_I64)
@@ -1250,7 +1270,6 @@ extern "C" int hc_reduce(hc_ctx* ctx, int op, int dtype, const void* in, void* o
       segs = ceil_div((uint64_t)reduce, seg_len);
       if (segs > 1) {
         const bool arg = op == HC_ARGMAX || op == HC_ARGMIN;
-        Scratch scratch(ctx);
         const size_t n = (size_t)outer * segs;
         HC_TRY(scratch.get(n * 8, &k.pvals));
         if (arg) {
@@ -1280,8 +1299,33 @@ extern "C" int hc_reduce(hc_ctx* ctx, int op, int dtype, const void* in, void* o
     snprintf(name, sizeof(name), "hc_reduce_rows256_%s_%s", kReduceNames[op], dtype_name(dtype));
     return launch(ctx, name, (uint64_t)outer, 1, &k, sizeof(k));
   }
-  return reduce_cols(ctx, kReduceNames[op], dtype, in, nullptr, out, outer, reduce, inner,
+  return reduce_cols(ctx, scratch, kReduceNames[op], dtype, in, nullptr, out, outer, reduce, inner,
                      op == HC_ARGMAX || op == HC_ARGMIN);
+}
+
+extern "C" int hc_reduce(hc_ctx* ctx, int op, int dtype, const void* in, void* out, int64_t outer,
+                         int64_t reduce, int64_t inner) {
+  REQUIRE(ctx, "hc_reduce: null context");
+  Scratch scratch(ctx);
+  return reduce_impl(ctx, scratch, op, dtype, in, out, outer, reduce, inner);
+}
+
+// hc_reduce with its partial results in the caller's device range [scratch, scratch + scratch_bytes)
+// instead of pool blocks: the body of hc_reduce_noalloc (noalloc.hip), which owns that range.
+__attribute__((visibility("hidden"))) int hc_reduce_in_scratch(hc_ctx* ctx, int op, int dtype, const void* in,
+                                                               void* out, int64_t outer, int64_t reduce,
+                                                               int64_t inner, void* scratch_base,
+                                                               size_t scratch_bytes) {
+  REQUIRE(ctx, "hc_reduce_noalloc: null context");
+  REQUIRE(scratch_base, "hc_reduce_noalloc: the scratch buffer of device %d was not set up", ctx->device);
+  Scratch scratch(ctx, scratch_base, scratch_bytes);
+  return reduce_impl(ctx, scratch, op, dtype, in, out, outer, reduce, inner);
+}
+
+__attribute__((visibility("hidden"))) int hc_ctx_device(const hc_ctx* ctx) { return ctx ? ctx->device : -1; }
+
+__attribute__((visibility("hidden"))) int hc_set_error(int code, const char* message) {
+  return fail(code, "%s", message);
 }
 
 extern "C" int hc_cumulative(hc_ctx* ctx, int op, int dtype, const void* in, void* out, int64_t outer,

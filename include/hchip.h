@@ -223,6 +223,19 @@ int hc_elemwise(hc_ctx* ctx, int op, int dtype, const void* in, const void* scal
 int hc_reduce(hc_ctx* ctx, int op, int dtype, const void* in, void* out, int64_t outer,
               int64_t reduce, int64_t inner);
 
+/* hc_reduce for callers that cannot allocate device memory: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc. No counterpart in the reference. Same arguments,
+ * kernels and results as hc_reduce, but the partial results of split reductions (a column
+ * reduction cut into ranges, long rows cut into segments) live in a fixed array of
+ * HC_NOALLOC_SCRATCH_BYTES of device memory that the library holds on every device it runs on
+ * until the process ends, so the call allocates and frees nothing, not even from the context's
+ * pool. A reduction whose partials need more returns HC_ERR_TOO_LARGE (the message says how
+ * much). All calls on one GPU share that array: calls that overlap there (two contexts, i.e.
+ * two streams, on the same device) race; calls through one context are ordered by its stream. */
+#define HC_NOALLOC_SCRATCH_BYTES (8u << 20)
+int hc_reduce_noalloc(hc_ctx* ctx, int op, int dtype, const void* in, void* out, int64_t outer,
+                      int64_t reduce, int64_t inner);
+
 /* Measurement aid with no counterpart in the reference: one launch of a kernel that only issues
  * fp16 MFMAs on a 128 x 128 wave tile of accumulators (one workgroup per compute unit, no memory
  * traffic in the loop) with operand bit patterns taken from `data` (`bytes` long, 16-byte
