@@ -1236,8 +1236,8 @@ static int reduce_impl(hc_ctx* ctx, Scratch& scratch, int op, int dtype, const v
                        int64_t reduce, int64_t inner) {
   REQUIRE(ctx, "hc_reduce: null context");
   REQUIRE(op >= HC_SUM && op <= HC_ARGMIN, "hc_reduce: bad op %d", op);
-  if (dtype != HC_F32 && dtype != HC_F16 && dtype != HC_I64)
-    return fail(HC_ERR_UNSUPPORTED, "hc_reduce: dtype %d is not numeric", dtype);
+  if (dtype != HC_F32 && dtype != HC_F16 && dtype != HC_I64 && dtype != HC_BOOL)
+    return fail(HC_ERR_UNSUPPORTED, "hc_reduce: bad dtype %d", dtype);
   HC_TRY(check_dims("hc_reduce", outer, reduce, inner));
   if (outer * inner == 0) return HC_OK;
   REQUIRE(out, "hc_reduce: null output");

@@ -38,6 +38,8 @@ template <typename T> __device__ __forceinline__ T from_arith(typename Arith<T>:
   return (T)v;
 }
 template <> __device__ __forceinline__ half_t from_arith<half_t>(float v) { return narrow<half_t>(v); }
+// Bool(Float) is `value != 0` (TensorElement.swift:179-181), not an integer conversion.
+template <> __device__ __forceinline__ uint8_t from_arith<uint8_t>(float v) { return v == 0.0f ? 0 : 1; }
 
 // Round an fp32 intermediate to what the tensor dtype can hold (identity for float).
 template <typename T> __device__ __forceinline__ float round_through(float v) {

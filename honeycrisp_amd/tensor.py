@@ -221,12 +221,13 @@ class Tensor:
             arr = arr.reshape(-1)
         else:
             values = list(data)
+            is_bool = len(values) > 0 and all(isinstance(v, (bool, np.bool_)) for v in values)
             is_int = all(isinstance(v, (int, np.integer)) and not isinstance(v, bool) for v in values)
             if dtype is None:
-                # T.dtype of the element type: Int collections make int64 tensors, Float /
-                # Double collections float32
-                dtype = DType.int64 if is_int else DType.float32
-            arr = np.asarray(values, dtype=np.int64 if is_int else np.float64)
+                # T.dtype of the element type: Bool collections make bool tensors, Int collections
+                # int64 tensors, Float / Double collections float32
+                dtype = DType.bool if is_bool else DType.int64 if is_int else DType.float32
+            arr = np.asarray(values, dtype=np.bool_ if is_bool else np.int64 if is_int else np.float64)
             if shape is None:
                 shape = [len(values)]
         self.dtype = DType(dtype)
@@ -583,6 +584,22 @@ class Tensor:
 
     def max(self, axis=None, keepdims=False): return self.gatherFromReduce(ReduceOp.argmax, axis, keepdims)
     def min(self, axis=None, keepdims=False): return self.gatherFromReduce(ReduceOp.argmin, axis, keepdims)
+
+    def _allSome(self, axis, keepdims, isAll: bool) -> "Tensor":
+        """ReduceRepeat.swift:103-162: min (all) / max (some) of a bool tensor; an empty axis yields
+        the constant true (all) / false (some)."""
+        assert self.dtype == DType.bool, "can only apply all() / some() to boolean tensors"
+        axis = self.positiveAxis(axis)
+        if axis is not None:
+            if self.shape[axis] == 0:
+                outShape = self.shape[:axis] + ([1] if keepdims else []) + self.shape[axis + 1:]
+                return Tensor.constant(isAll, outShape, DType.bool)
+        elif product(self.shape) == 0:
+            return Tensor.constant(isAll, [1] * len(self.shape) if keepdims else [], DType.bool)
+        return self.min(axis, keepdims) if isAll else self.max(axis, keepdims)
+
+    def all(self, axis=None, keepdims=False): return self._allSome(axis, keepdims, True)
+    def some(self, axis=None, keepdims=False): return self._allSome(axis, keepdims, False)
 
     def cumulativeSum(self, axis: int, exclusive=False, reverse=False) -> "Tensor":
         """ReduceRepeat.swift: running sum along `axis`."""

@@ -9,7 +9,6 @@ import PackageDescription
 
 let package = Package(
   name: "HoneycrispHIP",
-  platforms: [.macOS(.v13)],
   products: [
     .library(name: "HoneycrispHIP", targets: ["HoneycrispHIP"]),
     .executable(name: "HCMatrixBench", targets: ["HCMatrixBench"]),

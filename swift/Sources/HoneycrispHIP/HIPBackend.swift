@@ -6,8 +6,9 @@
 // generator, keep working on the host; the overrides below enqueue one hchip call each on the
 // context's in-order stream and return a device buffer (`HIPData`) immediately.
 //
-// Not compiled in the authoring environment (no Swift toolchain); written against
-// Sources/Honeycrisp/Backend.swift:170-815 and the C ABI in include/hchip.h.
+// Not compiled in the authoring environment, nor on the GPU machines it was tested on (neither
+// has a Swift toolchain): written against Sources/Honeycrisp/Backend.swift:170-815 and the C ABI
+// in include/hchip.h, unverified by a compiler.
 import CHCHIP
 import Foundation
 import Honeycrisp
@@ -235,8 +236,7 @@ open class HIPBackend: CPUBackend, @unchecked Sendable {
   override open func reduce(
     _ a: Tensor.Data, op: ReduceOp, dims: ReduceDims, dtype: Tensor.DType
   ) async throws -> Tensor.Data {
-    guard dtype != .bool else { return try await super.reduce(a, op: op, dims: dims, dtype: dtype) }
-    let da = try await device(a)
+    let da = try await device(a)  // (bool reduces as Float 0 / 1, like the CPU: Tensor.all / some)
     let outType: Tensor.DType = op.isIntOut ? .int64 : dtype
     let out = try output(dims.outCount * outType.byteSize)
     try check(
@@ -399,6 +399,121 @@ open class HIPBackend: CPUBackend, @unchecked Sendable {
     return out
   }
 
+  /// compare(Tensor.Data, T) / compare(T, Tensor.Data) (Backend.swift:468-486): the scalar is
+  /// compared as Float, or as Int64 for int64 tensors (BackendCPU.swift:574-624).
+  private func compareScalar<T: TensorElement>(
+    _ a: Tensor.Data, _ b: T, scalarFirst: Bool, op: ComparisonOp, count: Int, dtype: Tensor.DType
+  ) async throws -> Tensor.Data {
+    let da = try await device(a)
+    let out = try output(count)
+    try check(
+      hc_compare_scalar(
+        ctx, hcOp(op), hcDType(dtype), da.pointer, b.toFloat(), dtype == .int64 ? b.toInt64() : 0,
+        scalarFirst ? 1 : 0, out.pointer, count))
+    return out
+  }
+
+  override open func compare<T: TensorElement>(
+    _ a: Tensor.Data, _ b: T, op: ComparisonOp, count: Int, dtype: Tensor.DType
+  ) async throws -> Tensor.Data {
+    try await compareScalar(a, b, scalarFirst: false, op: op, count: count, dtype: dtype)
+  }
+
+  override open func compare<T: TensorElement>(
+    _ a: T, _ b: Tensor.Data, op: ComparisonOp, count: Int, dtype: Tensor.DType
+  ) async throws -> Tensor.Data {
+    try await compareScalar(b, a, scalarFirst: true, op: op, count: count, dtype: dtype)
+  }
+
+  /// A TensorOrScalar operand as (device buffer, strides): a scalar becomes a 1-element constant
+  /// with all-zero strides, which is what CPUBackend.tensorOrScalarData makes of it too.
+  private func operand<T: TensorElement>(_ x: TensorOrScalar<T>, dtype: Tensor.DType) async throws
+    -> (HIPData, hc_strides)
+  {
+    switch x {
+    case .tensor(let t): return (try await device(t.data), hcStrides(t.strides))
+    case .scalar(let v, let shape):
+      let c = try await constant(v, count: 1, dtype: dtype)
+      return (
+        try await device(c),
+        hcStrides(BroadcastStrides(shape: shape, strides: [Int](repeating: 0, count: shape.count)))
+      )
+    }
+  }
+
+  /// Backend.when (Backend.swift:633-641): mask ? a : b over the mask's broadcast shape.
+  override open func when<T>(
+    _ mask: BroadcastData, _ a: TensorOrScalar<T>, _ b: TensorOrScalar<T>, _: T.Type,
+    dtype: Tensor.DType
+  ) async throws -> Tensor.Data {
+    let dm = try await device(mask.data)
+    var sm = hcStrides(mask.strides)
+    var (da, sa) = try await operand(a, dtype: dtype)
+    var (db, sb) = try await operand(b, dtype: dtype)
+    let out = try output(mask.strides.shape.product() * dtype.byteSize)
+    try check(hc_when(ctx, hcDType(dtype), dm.pointer, &sm, da.pointer, &sa, db.pointer, &sb, out.pointer))
+    _ = (da, db)  // (the operands stay alive until the call has been enqueued)
+    return out
+  }
+
+  /// Backend.concat (Backend.swift:777-784): input t contributes innerCounts[t] elements to each
+  /// of the outerCount output rows.
+  override open func concat(
+    _ inputs: [Tensor.Data], outerCount: Int, innerCounts: [Int], dtype: Tensor.DType
+  ) async throws -> Tensor.Data {
+    var buffers: [HIPData] = []
+    for x in inputs { buffers.append(try await device(x)) }
+    let pointers: [UnsafeRawPointer?] = buffers.map { UnsafeRawPointer($0.pointer) }
+    let counts = innerCounts.map { Int64($0) }
+    let out = try output(outerCount * innerCounts.reduce(0, +) * dtype.byteSize)
+    try check(
+      hc_concat(ctx, hcDType(dtype), pointers, counts, Int32(inputs.count), Int64(outerCount), out.pointer))
+    return out
+  }
+
+  /// Backend.collection (Backend.swift:794-800): the element conversion stays the host's
+  /// (CPUBackend.collection, BackendCPU.swift:1817-1829); the result is uploaded once, here,
+  /// instead of at every op that reads it.
+  override open func collection<T: TensorElement>(
+    _ collection: some Collection<T>, reverse: Bool, dtype: Tensor.DType
+  ) async throws -> Tensor.Data {
+    try await device(try await super.collection(collection, reverse: reverse, dtype: dtype))
+  }
+
+  /// Backend.repeated (Backend.swift:590-606) as the broadcast it is defined as; CPUBackend
+  /// overrides it with a host loop (BackendCPU.swift:1087-1106).
+  override open func repeated(_ a: Tensor.Data, dims: RepeatDims, dtype: Tensor.DType) async throws
+    -> Tensor.Data
+  {
+    try await broadcast(
+      BroadcastData(
+        strides: BroadcastStrides(
+          shape: [dims.outerCount, dims.repeatCount, dims.innerCount],
+          strides: [dims.innerCount, 0, 1]),
+        data: a),
+      dtype: dtype)
+  }
+
+  /// bitwiseOp(Tensor.Data, T) (Backend.swift:227-235): the scalar's bit pattern as a 1-element
+  /// buffer with a zero stride.
+  override open func bitwiseOp<T: TensorElementBitPattern>(
+    _ a: Tensor.Data, _ b: T, op: BitwiseOp, count: Int, dtype: Tensor.DType
+  ) async throws -> Tensor.Data {
+    let bits = b.bitsForBitwiseOp
+    guard bits.count == dtype.byteSize else {
+      return try await super.bitwiseOp(a, b, op: op, count: count, dtype: dtype)
+    }
+    let da = try await device(a)
+    let db = try output(bits.count)
+    try bits.withUnsafeBytes { try check(hc_memcpy_h2d(ctx, db.pointer, $0.baseAddress, bits.count)) }
+    var sa = hcStrides(BroadcastStrides(shape: [count], strides: [1]))
+    var sb = hcStrides(BroadcastStrides(shape: [count], strides: [0]))
+    let out = try output(count * dtype.byteSize)
+    let kind: Int32 = op == .or ? 0 : op == .and ? 1 : 2
+    try check(hc_bitwise_op(ctx, kind, hcDType(dtype), da.pointer, &sa, db.pointer, &sb, out.pointer))
+    return out
+  }
+
   override open func constant<T: TensorElement>(_ value: T, count: Int, dtype: Tensor.DType) async throws
     -> Tensor.Data
   {
@@ -520,23 +635,10 @@ open class HIPBackend: CPUBackend, @unchecked Sendable {
     dtype: Tensor.DType
   ) async throws -> Tensor.Data {
     guard dtype != .bool else { return try await super.clamp(a, T.self, min: min, max: max, dtype: dtype) }
-    // a scalar bound becomes a 1-element constant with all-zero strides
-    func bound(_ x: TensorOrScalar<T>?) async throws -> (HIPData, hc_strides)? {
-      guard let x = x else { return nil }
-      switch x {
-      case .tensor(let t): return (try await device(t.data), hcStrides(t.strides))
-      case .scalar(let v, let shape):
-        let c = try await constant(v, count: 1, dtype: dtype)
-        return (
-          try await device(c),
-          hcStrides(BroadcastStrides(shape: shape, strides: [Int](repeating: 0, count: shape.count)))
-        )
-      }
-    }
     let da = try await device(a.data)
     var sa = hcStrides(a.strides)
-    let lo = try await bound(min)
-    let hi = try await bound(max)
+    let lo = min == nil ? nil : try await operand(min!, dtype: dtype)
+    let hi = max == nil ? nil : try await operand(max!, dtype: dtype)
     var (sl, sh) = (lo?.1 ?? sa, hi?.1 ?? sa)
     let out = try output(a.strides.shape.product() * dtype.byteSize)
     try withUnsafePointer(to: &sl) { pl in

@@ -710,6 +710,81 @@ def testNormalizeGrad(rng):
     assert_close_arrays(got, want, 1e-4, 1e-4)
 
 
+def testProd(rng):
+    """BackendTests.swift:436-465 (forward values): a product over positive inputs equals
+    exp(sum(log x)); signs."""
+    raw = Tensor(data=(rng.random((3, 4, 5)) + 0.5).astype(np.float32))
+    for axis in range(3):
+        expected = raw.log().sum(axis=axis).exp()
+        for dtype in (F16, F32):
+            tol = 1e-4 if dtype == F32 else 1e-2
+            assertClose(expected, raw.cast(dtype).prod(axis=axis).cast(F32), atol=tol, rtol=tol)
+    x = Tensor(data=[2.0, -3.0, 4.0, 2.0, -3.0, -4.0], shape=[2, 3])
+    for dtype in (F16, F32, I64):
+        assertDataEqual(x.cast(dtype).prod(axis=0), [4.0, 9.0, -16.0])
+        assertDataEqual(x.cast(dtype).prod(axis=1), [-24.0, 24.0])
+
+
+def testRepeat():
+    """BackendTests.swift:566-583: repeating along an axis; its gradient is the sum over the
+    copies (flatApplySums of the inverse RepeatDims, ReduceRepeat.swift:283-305)."""
+    x = Tensor(data=[1.0, 2.0, 3.0, -2.0, 3.0, 7.0], shape=[1, 2, 3, 1])
+    repeated = x.repeating(axis=2, count=2)
+    assert repeated.shape == [1, 2, 6, 1]
+    assertDataEqual(repeated, [1.0, 2.0, 3.0, 1.0, 2.0, 3.0, -2.0, 3.0, 7.0, -2.0, 3.0, 7.0])
+    grad = Tensor(data=[float(i) for i in range(1, 13)], shape=[1, 2, 6, 1])
+    assertDataEqual(grad.reshape([2, 2, 3]).sum(axis=1), [5.0, 7.0, 9.0, 17.0, 19.0, 21.0])
+
+
+def testAllSome():
+    """BackendTests.swift:1364-1425."""
+    def checkEqual(t1, t2):
+        assert t1.shape == t2.shape and t1.dtype == t2.dtype
+        assertDataEqual(t1, t2)
+
+    bits = [False, True, False, False, True, True, True, False]
+    checkEqual(Tensor(data=bits, shape=[4, 2]).all(axis=1), Tensor(data=[False, False, True, False], shape=[4]))
+    checkEqual(Tensor(data=bits, shape=[4, 2]).all(axis=1, keepdims=True),
+               Tensor(data=[False, False, True, False], shape=[4, 1]))
+    checkEqual(Tensor(data=bits, shape=[4, 2]).some(axis=1), Tensor(data=[True, False, True, True], shape=[4]))
+    checkEqual(Tensor(data=bits, shape=[4, 2]).some(axis=1, keepdims=True),
+               Tensor(data=[True, False, True, True], shape=[4, 1]))
+    empty = lambda: Tensor(data=[], shape=[4, 0], dtype=BOOL)
+    none = lambda shape: Tensor(data=[], shape=shape, dtype=BOOL)
+    for fn, unit in ((Tensor.all, True), (Tensor.some, False)):
+        checkEqual(fn(empty()), Tensor(data=[unit], shape=[]))
+        checkEqual(fn(empty(), keepdims=True), Tensor(data=[unit], shape=[1, 1]))
+        checkEqual(fn(empty(), axis=1), Tensor(data=[unit] * 4, shape=[4]))
+        checkEqual(fn(empty(), axis=1, keepdims=True), Tensor(data=[unit] * 4, shape=[4, 1]))
+        checkEqual(fn(empty(), axis=0), none([0]))
+        checkEqual(fn(empty(), axis=0, keepdims=True), none([1, 0]))
+
+
+def testConcatInner():
+    """BackendTests.swift:1629-1642; the gradients of a concatenation are the matching slices of
+    the output gradient (ConcatSplit.swift)."""
+    x = Tensor(data=[1, 2, 3, 4, 5, 6], shape=[2, 3]).cast(F32)
+    y = Tensor(data=[7, 8, 9, 10], shape=[2, 2]).cast(F32)
+    combined = Tensor.concat([x, y], axis=1)
+    assert combined.shape == [2, 5]
+    assertDataEqual(combined, [1, 2, 3, 7, 8, 4, 5, 6, 9, 10])
+    grad = Tensor(data=[1, 2, 3, 4, 5, 6, 7, 8, 9, 10], shape=[2, 5]).cast(F32)
+    assertDataEqual(grad[:, 0:3], [1, 2, 3, 6, 7, 8])
+    assertDataEqual(grad[:, 3:5], [4, 5, 9, 10])
+
+
+def testConcatOuter():
+    """BackendTests.swift:1644-1657."""
+    x = Tensor(data=[1, 2, 3, 4, 5, 6], shape=[2, 3]).cast(F32)
+    y = Tensor(data=[7, 8, 9], shape=[1, 3]).cast(F32)
+    combined = Tensor.concat([x, y], axis=0)
+    assert combined.shape == [3, 3]
+    assertDataEqual(combined, [1, 2, 3, 4, 5, 6, 7, 8, 9])
+    grad = Tensor(data=[1, 2, 3, 4, 5, 6, 7, 8, 9], shape=[3, 3]).cast(F32)
+    assertDataEqual(grad[0:2], [1, 2, 3, 4, 5, 6])
+    assertDataEqual(grad[2:3], [7, 8, 9])
+
+
 def testConcat():
     """Concatenation along an inner and an outer axis (Tensor(concat:), ConcatSplit.swift:4-75;
     CPU loop BackendCPU.swift:1768-1794); expected values follow from the definition."""
@@ -739,5 +814,5 @@ ALL_CASES = [
     testMatrixMatrixProduct, testBatchedMatmul, testMatrixVectorProduct, testTriangular, testIndexing,
     testElemwise, testRounding, testMinMax, testExpandAndRepeat, testBinaryBroadcast, testFusedBroadcast,
     testSoftmax, testConcat, testWhen, testCumulativeSum, testCumulativeProd, testArgsort, testBitwise, testSoftmaxGrad, testScatter, testScatterIsAdjointOfGather, testClamp,
-    testAdam, testNormalizeGrad,
+    testAdam, testNormalizeGrad, testProd, testRepeat, testAllSome, testConcatInner, testConcatOuter,
 ]
