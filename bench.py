@@ -19,6 +19,10 @@ Also reported in the same line:
                 per launch), and the transformer forward pass, eager and as one graph replay
 
 Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extra] [--no-graph]
+                       [--only headline,cfg1,cfg2,cfg3,cfg4,cfg5]
+`--only` restricts the run to the named parts (the headline always runs, shortened when it is not
+named): what the per-config rocprofv3 summaries under profiles/ are made with, so that a kernel's
+launches of one config are not pooled with another's.
 """
 import argparse
 import ctypes
@@ -39,6 +43,49 @@ PEAK_HBM_GBS = 8000.0     # MI355X HBM3E
 # this benchmark scaled by a plain copy kernel (not measurable live; the run that produced it is
 # summarised in profiles/bench_hbm_traffic_fetch_write_size.md): 196850 KiB read + 32768 KiB written.
 GEMM_TRAFFIC_BYTES = (196800 + 32768) * 1024
+GEMM_TRAFFIC_SOURCE = "constant from profiles/bench_hbm_traffic_fetch_write_size.md (rocprofv3 --pmc runs), not measured in this run"
+
+
+class MfmaProbe:
+    """The MFMA-only measurement kernels of bench_probe.hip: bench.py's own code object, loaded
+    through the library's raw module entry points (hc_module_load / hc_launch)."""
+
+    class Args(ctypes.Structure):
+        _fields_ = [("data", ctypes.c_void_p), ("out", ctypes.c_void_p), ("iters", ctypes.c_uint32),
+                    ("chunks", ctypes.c_uint32)]
+
+    def __init__(self, backend):
+        self.b, self.lib = backend, backend._lib
+        path = os.path.join(ROOT, "bench_probe.hsaco")
+        if not os.path.exists(path):
+            import subprocess
+            subprocess.run(["/opt/rocm/bin/hipcc", "--offload-arch=gfx950", "--genco", "-O3", "-std=c++17",
+                            "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+                            "-o", path, os.path.join(ROOT, "bench_probe.hip")], check=True)
+        image = open(path, "rb").read()
+        self.image = ctypes.create_string_buffer(image, len(image))
+        self.module = ctypes.c_void_p()
+        backend._check(self.lib.hc_module_load(backend._ctx, self.image, len(image), ctypes.byref(self.module)))
+        self.fn = {}
+        for shape, name in ((0, b"hc_probe_mfma_f16_32x32x16"), (1, b"hc_probe_mfma_f16_16x16x32")):
+            fn = ctypes.c_void_p()
+            backend._check(self.lib.hc_module_get_function(self.module, name, ctypes.byref(fn)))
+            self.fn[shape] = fn
+        self.cus = backend.deviceInfo()["compute_units"]
+        self.out = backend.allocate(self.cus * 256 * 4)
+
+    def launch(self, data, shape, iters=1024):
+        """One launch (a workgroup of four waves per compute unit: the occupancy of the large GEMM
+        tile); returns its floating-point operations."""
+        args = MfmaProbe.Args(data.ptr, self.out.ptr, iters, min(data.byteCount // 16, 0xffffffff))
+        grid, block = (ctypes.c_uint32 * 3)(self.cus, 1, 1), (ctypes.c_uint32 * 3)(256, 1, 1)
+        self.b._check(self.lib.hc_launch(self.b._ctx, self.fn[shape], grid, block, 0, ctypes.byref(args),
+                                         ctypes.sizeof(args)))
+        # per iteration and wave: 16 MFMAs of 32 x 32 x 16 (or 32 of 16 x 16 x 32)
+        return 2.0 * 32 * 32 * 16 * 16.0 * iters * (self.cus * 256 / 64)
+
+    def close(self):
+        self.lib.hc_module_unload(self.b._ctx, self.module)
 
 
 class Events:
@@ -151,7 +198,8 @@ def headline(backend, steps, warmup):
     backend.sync()
     t1 = time.perf_counter()
     flops = 2.0 * n * n * n
-    launch_ms = float(np.mean([events.elapsed_ms(marks[i], marks[i + 1]) for i in range(steps)])) / 4
+    step_ms = [events.elapsed_ms(marks[i], marks[i + 1]) for i in range(steps)]
+    launch_ms = float(np.mean(step_ms)) / 4
     for m in marks:
         events.free(m)
     ms_per_step = (t1 - t0) * 1e3 / steps
@@ -179,7 +227,12 @@ def headline(backend, steps, warmup):
         "bound": "mfma", "kernel": "fp16 GEMM 4096^3 (hc_gemm_f16_mi16_256x256_*), mean over the timed region's launches",
         "achieved": round(achieved, 2),
         "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s", "frac": round(achieved / PEAK_F16_TFLOPS, 4),
-        "traffic": GEMM_TRAFFIC_BYTES, "launch_ms": round(launch_ms, 5),
+        "traffic": GEMM_TRAFFIC_BYTES, "traffic_source": GEMM_TRAFFIC_SOURCE, "launch_ms": round(launch_ms, 5),
+        "step_ms_min_median_max": [round(float(np.min(step_ms)), 4), round(float(np.median(step_ms)), 4),
+                                   round(float(np.max(step_ms)), 4)],
+        "step_tflops_min_median_max": [round(4 * flops / (float(np.max(step_ms)) * 1e-3) / 1e12, 1),
+                                       round(4 * flops / (float(np.median(step_ms)) * 1e-3) / 1e12, 1),
+                                       round(4 * flops / (float(np.min(step_ms)) * 1e-3) / 1e12, 1)],
         "per_layout_tflops": {k: round(flops / (v * 1e-3) / 1e12, 2) for k, v in layout_ms.items()},
         "per_layout_ms": {k: round(v, 4) for k, v in layout_ms.items()},
         "per_layout_note": "separate untimed pass, one event per launch",
@@ -189,19 +242,21 @@ def headline(backend, steps, warmup):
     # power fits, and MFMA power depends on how many operand bits toggle, so this, not the
     # 2.4 GHz figure, is the rate a GEMM on this data could approach.
     probe_in = dev[("a", False)]
+    probe = MfmaProbe(backend)
     probe_tflops = {}
     for shape, name in ((1, "16x16x32"), (0, "32x32x16")):
         for _ in range(200):
-            probe_flops = backend.probeMfma(probe_in, shape)
+            probe_flops = probe.launch(probe_in, shape)
         e0, e1 = events.new(), events.new()
         events.record(e0)
         for _ in range(200):
-            backend.probeMfma(probe_in, shape)
+            probe.launch(probe_in, shape)
         events.record(e1)
         backend.sync()
         probe_tflops[name] = 200 * probe_flops / (events.elapsed_ms(e0, e1) * 1e-3) / 1e12
         events.free(e0)
         events.free(e1)
+    probe.close()
     roofline["mfma_only_same_data"] = {
         "tflops": round(probe_tflops["16x16x32"], 1), "gemm_frac_of_it": round(achieved / probe_tflops["16x16x32"], 4),
         "tflops_32x32x16": round(probe_tflops["32x32x16"], 1),
@@ -306,134 +361,152 @@ def cpu_reference_ops(budget_s=15.0):
     return out
 
 
-def extra_workloads(backend, graph=True):
-    """Configs 1, 3 and 4 of BASELINE.json: per-op launch durations from HIP events."""
+def extra_workloads(backend, graph=True, only=("cfg1", "cfg2", "cfg3", "cfg4", "cfg5")):
+    """The other configs of BASELINE.json: per-op launch durations from HIP events."""
     from honeycrisp_amd.descriptors import (BroadcastData, BroadcastStrides, DType, ElemwiseOp, NumericBinaryOp,
                                             ReduceDims, ReduceOp, ScatterGatherIndices)
     ev = Events(backend)
     out = {}
     F32, F16, I64 = DType.float32, DType.float16, DType.int64
 
-    def report(name, ms, flops=None, nbytes=None):
+    def report(name, ms, flops=None, nbytes=None, peak_tflops=None):
         r = {"ms": round(ms, 4)}
         if flops is not None:
             r["tflops"] = round(flops / (ms * 1e-3) / 1e12, 3)
+            if peak_tflops:
+                r["mfma_frac"] = round(r["tflops"] / peak_tflops, 4)
         if nbytes is not None:
             r["gbs"] = round(nbytes / (ms * 1e-3) / 1e9, 1)
             r["hbm_frac"] = round(r["gbs"] / PEAK_HBM_GBS, 4)
         out[name] = r
 
-    # config 1: fp32 1024^3 (two input sets alternate so the operands are not L2-resident twice in a row)
-    rng = np.random.default_rng(1)
-    sets = [(backend.upload(rng.standard_normal((1024, 1024)).astype(np.float32)),
-             backend.upload(rng.standard_normal((1024, 1024)).astype(np.float32))) for _ in range(2)]
-    it = [0]
+    def cfg1():
+        # config 1: fp32 1024^3 (two input sets alternate so the operands are not L2-resident twice in a row)
+        rng = np.random.default_rng(1)
+        sets = [(backend.upload(rng.standard_normal((1024, 1024)).astype(np.float32)),
+                 backend.upload(rng.standard_normal((1024, 1024)).astype(np.float32))) for _ in range(2)]
+        it = [0]
 
-    def gemm32():
-        x, y = sets[it[0] & 1]
-        it[0] += 1
-        return backend.matmul(x, False, y, False, False, 1024, 1024, 1024, F32)
-    ms, _ = timed_launches(backend, ev, gemm32, 50, 10, batched=True)
-    report("cfg1_f32_gemm_1024", ms, flops=2.0 * 1024**3)
-    out["cfg1_f32_gemm_1024"]["mfma_frac"] = round(out["cfg1_f32_gemm_1024"]["tflops"] / PEAK_F32_TFLOPS, 4)
+        def gemm32():
+            x, y = sets[it[0] & 1]
+            it[0] += 1
+            return backend.matmul(x, False, y, False, False, 1024, 1024, 1024, F32)
+        ms, _ = timed_launches(backend, ev, gemm32, 50, 10, batched=True)
+        report("cfg1_f32_gemm_1024", ms, flops=2.0 * 1024**3, peak_tflops=PEAK_F32_TFLOPS)
 
-    # config 2, the ragged sweep: fp16 NN products with M, N, K in {127, 1000, 4097}; total FLOPs over
-    # total time of the 27 shapes, and the three cubes on their own
-    sizes = (127, 1000, 4097)
-    total_flops, total_ms = 0.0, 0.0
-    rng = np.random.default_rng(20)
-    big = rng.standard_normal(4097 * 4097).astype(np.float16)
-    for m in sizes:
-        for kk in sizes:
-            a_dev = backend.upload(big[:m * kk])
-            for n in sizes:
-                b_dev = backend.upload(big[:kk * n])
-                fn = lambda: backend.matmul(a_dev, False, b_dev, False, False, m, kk, n, F16)
-                ms, _ = timed_launches(backend, ev, fn, 5, 2, batched=True)
-                total_flops += 2.0 * m * kk * n
-                total_ms += ms
-                if m == kk == n:
-                    report("cfg2_ragged_%d_cubed" % m, ms, flops=2.0 * m * kk * n)
-    report("cfg2_ragged_sweep_27_shapes", total_ms, flops=total_flops)
+    def cfg2():
+        # the metric's fp32 leg: fp32 4096^3, N(0,1)/sqrt(K) entries, NN and NT (B stored transposed)
+        n = 4096
+        a32 = backend.upload((np.random.default_rng(2).standard_normal((n, n)) / np.sqrt(n)).astype(np.float32))
+        b32 = backend.upload((np.random.default_rng(3).standard_normal((n, n)) / np.sqrt(n)).astype(np.float32))
+        for name, tb in (("NN", False), ("NT", True)):
+            fn = lambda: backend.matmul(a32, False, b32, tb, False, n, n, n, F32)
+            for _ in range(30):     # (the clocks settle under load, see headline())
+                fn()
+            ms, _ = timed_launches(backend, ev, fn, 30, 10)
+            report("cfg2_f32_gemm_4096_" + name, ms, flops=2.0 * n**3, peak_tflops=PEAK_F32_TFLOPS)
+        del a32, b32
+        # the ragged sweep: fp16 NN products with M, N, K in {127, 1000, 4097}; total FLOPs over
+        # total time of the 27 shapes, and the three cubes on their own
+        sizes = (127, 1000, 4097)
+        total_flops, total_ms = 0.0, 0.0
+        rng = np.random.default_rng(20)
+        big = rng.standard_normal(4097 * 4097).astype(np.float16)
+        for m in sizes:
+            for kk in sizes:
+                a_dev = backend.upload(big[:m * kk])
+                for n in sizes:
+                    b_dev = backend.upload(big[:kk * n])
+                    fn = lambda: backend.matmul(a_dev, False, b_dev, False, False, m, kk, n, F16)
+                    ms, _ = timed_launches(backend, ev, fn, 5, 2, batched=True)
+                    total_flops += 2.0 * m * kk * n
+                    total_ms += ms
+                    if m == kk == n:
+                        report("cfg2_ragged_%d_cubed" % m, ms, flops=2.0 * m * kk * n)
+        report("cfg2_ragged_sweep_27_shapes", total_ms, flops=total_flops)
 
-    # config 3: attention-shaped batched GEMMs, fp16, batch 32
-    q, k, v = [backend.upload(np.random.default_rng(s).standard_normal((32, 512, 64)).astype(np.float16))
-               for s in (4, 5, 6)]
-    scores = backend.batchedMatmul(32, q, False, k, True, False, 512, 64, 512, F16)
-    ms, _ = timed_launches(backend, ev, lambda: backend.batchedMatmul(32, q, False, k, True, False, 512, 64, 512, F16), 50, 10, batched=True)
-    report("cfg3_qk_t", ms, flops=32 * 2.0 * 512 * 64 * 512, nbytes=32 * (2 * 512 * 64 + 512 * 512) * 2)
-    ms, _ = timed_launches(backend, ev, lambda: backend.binaryOp(scores, 0.125, NumericBinaryOp.mul, F16, count=32 * 512 * 512), 50, 10, batched=True)
-    report("cfg3_scale", ms, nbytes=2 * 32 * 512 * 512 * 2)
-    ms, _ = timed_launches(backend, ev, lambda: backend.batchedMatmul(32, scores, False, v, False, False, 512, 512, 64, F16), 50, 10, batched=True)
-    report("cfg3_pv", ms, flops=32 * 2.0 * 512 * 512 * 64, nbytes=32 * (2 * 512 * 64 + 512 * 512) * 2)
+    def cfg3():
+        # config 3: attention-shaped batched GEMMs, fp16, batch 32
+        q, k, v = [backend.upload(np.random.default_rng(s).standard_normal((32, 512, 64)).astype(np.float16))
+                   for s in (4, 5, 6)]
+        scores = backend.batchedMatmul(32, q, False, k, True, False, 512, 64, 512, F16)
+        ms, _ = timed_launches(backend, ev, lambda: backend.batchedMatmul(32, q, False, k, True, False, 512, 64, 512, F16), 50, 10, batched=True)
+        report("cfg3_qk_t", ms, flops=32 * 2.0 * 512 * 64 * 512, nbytes=32 * (2 * 512 * 64 + 512 * 512) * 2)
+        ms, _ = timed_launches(backend, ev, lambda: backend.binaryOp(scores, 0.125, NumericBinaryOp.mul, F16, count=32 * 512 * 512), 50, 10, batched=True)
+        report("cfg3_scale", ms, nbytes=2 * 32 * 512 * 512 * 2)
+        ms, _ = timed_launches(backend, ev, lambda: backend.batchedMatmul(32, scores, False, v, False, False, 512, 512, 64, F16), 50, 10, batched=True)
+        report("cfg3_pv", ms, flops=32 * 2.0 * 512 * 512 * 64, nbytes=32 * (2 * 512 * 64 + 512 * 512) * 2)
 
-    # config 4: bandwidth-bound ops at [8192, 4096] fp32
-    R, C = 8192, 4096
-    x = backend.upload(np.random.default_rng(7).standard_normal((R, C)).astype(np.float32))
-    bias = backend.upload(np.random.default_rng(8).standard_normal((1, C)).astype(np.float32))
-    xs = BroadcastStrides([R, C], [C, 1])
-    bs = BroadcastStrides([R, C], [0, 1])
-    nb = R * C * 4
-    ms, _ = timed_launches(backend, ev, lambda: backend.binaryOp(BroadcastData(xs, x), BroadcastData(bs, bias), NumericBinaryOp.add, F32), 50, 10, batched=True)
-    report("cfg4_bias_add", ms, nbytes=2 * nb + C * 4)
-    # plain copy of known size (identity broadcast): the calibration kernel for HBM byte counters
-    ms, _ = timed_launches(backend, ev, lambda: backend.broadcast(BroadcastData(xs, x), F32), 50, 10, batched=True)
-    report("copy_134MB_calibration", ms, nbytes=2 * nb)
-    ms, _ = timed_launches(backend, ev, lambda: backend.elemwise(x, ElemwiseOp.geluApprox, None, R * C, F32), 50, 10, batched=True)
-    report("cfg4_gelu", ms, nbytes=2 * nb)
-    dims = ReduceDims(R, C, 1)
-    ms, _ = timed_launches(backend, ev, lambda: backend.reduce(x, ReduceOp.sum, dims, F32), 50, 10, batched=True)
-    report("cfg4_sum_axis1", ms, nbytes=nb + R * 4)
-    ms, _ = timed_launches(backend, ev, lambda: backend.reduce(x, ReduceOp.argmax, dims, F32), 50, 10, batched=True)
-    report("cfg4_argmax_axis1", ms, nbytes=nb + R * 8)
-    idx = backend.reduce(x, ReduceOp.argmax, dims, F32)
-    max_gather = ScatterGatherIndices([R, C], 1, BroadcastData(BroadcastStrides([R, 1], [1, 0]), idx))
+    def cfg4():
+        # config 4: bandwidth-bound ops at [8192, 4096] fp32
+        R, C = 8192, 4096
+        x = backend.upload(np.random.default_rng(7).standard_normal((R, C)).astype(np.float32))
+        bias = backend.upload(np.random.default_rng(8).standard_normal((1, C)).astype(np.float32))
+        xs = BroadcastStrides([R, C], [C, 1])
+        bs = BroadcastStrides([R, C], [0, 1])
+        nb = R * C * 4
+        ms, _ = timed_launches(backend, ev, lambda: backend.binaryOp(BroadcastData(xs, x), BroadcastData(bs, bias), NumericBinaryOp.add, F32), 50, 10, batched=True)
+        report("cfg4_bias_add", ms, nbytes=2 * nb + C * 4)
+        # plain copy of known size (identity broadcast): the calibration kernel for HBM byte counters
+        ms, _ = timed_launches(backend, ev, lambda: backend.broadcast(BroadcastData(xs, x), F32), 50, 10, batched=True)
+        report("copy_134MB_calibration", ms, nbytes=2 * nb)
+        ms, _ = timed_launches(backend, ev, lambda: backend.elemwise(x, ElemwiseOp.geluApprox, None, R * C, F32), 50, 10, batched=True)
+        report("cfg4_gelu", ms, nbytes=2 * nb)
+        dims = ReduceDims(R, C, 1)
+        ms, _ = timed_launches(backend, ev, lambda: backend.reduce(x, ReduceOp.sum, dims, F32), 50, 10, batched=True)
+        report("cfg4_sum_axis1", ms, nbytes=nb + R * 4)
+        ms, _ = timed_launches(backend, ev, lambda: backend.reduce(x, ReduceOp.argmax, dims, F32), 50, 10, batched=True)
+        report("cfg4_argmax_axis1", ms, nbytes=nb + R * 8)
 
-    def max_axis1():  # Tensor.max(axis:) = argmax + gather (ReduceRepeat.swift:201-209)
-        i = backend.reduce(x, ReduceOp.argmax, dims, F32)
-        return backend.gather(x, ScatterGatherIndices([R, C], 1, BroadcastData(BroadcastStrides([R, 1], [1, 0]), i)), F32)
-    ms, _ = timed_launches(backend, ev, max_axis1, 50, 10, batched=True)
-    report("cfg4_max_axis1", ms, nbytes=nb + R * 8 + R * 8 + R * 4 + R * 4)
-    table = backend.upload(np.random.default_rng(10).standard_normal((32000, 1024)).astype(np.float32))
-    ids = backend.upload(np.random.default_rng(9).integers(0, 32000, size=(65536,)))
-    emb = ScatterGatherIndices([32000, 1024], 0, BroadcastData(BroadcastStrides([65536, 1024], [1, 0]), ids))
-    ms, _ = timed_launches(backend, ev, lambda: backend.gather(table, emb, F32), 50, 10, batched=True)
-    report("cfg4_embedding_gather", ms, nbytes=65536 * 8 + 2 * 65536 * 1024 * 4)
-    del max_gather
+        def max_axis1():  # Tensor.max(axis:) = argmax + gather (ReduceRepeat.swift:201-209)
+            i = backend.reduce(x, ReduceOp.argmax, dims, F32)
+            return backend.gather(x, ScatterGatherIndices([R, C], 1, BroadcastData(BroadcastStrides([R, 1], [1, 0]), i)), F32)
+        ms, _ = timed_launches(backend, ev, max_axis1, 50, 10, batched=True)
+        report("cfg4_max_axis1", ms, nbytes=nb + R * 8 + R * 8 + R * 4 + R * 4)
+        table = backend.upload(np.random.default_rng(10).standard_normal((32000, 1024)).astype(np.float32))
+        ids = backend.upload(np.random.default_rng(9).integers(0, 32000, size=(65536,)))
+        emb = ScatterGatherIndices([32000, 1024], 0, BroadcastData(BroadcastStrides([65536, 1024], [1, 0]), ids))
+        ms, _ = timed_launches(backend, ev, lambda: backend.gather(table, emb, F32), 50, 10, batched=True)
+        report("cfg4_embedding_gather", ms, nbytes=65536 * 8 + 2 * 65536 * 1024 * 4)
 
-    # config 5: decoder-only transformer forward, 8 x 256 tokens; tokens/s = 2048 / wall time of
-    # a forward pass ending in wait() on the logits (host-side op dispatch included)
-    from honeycrisp_amd.nn import Transformer
-    from honeycrisp_amd.tensor import Tensor
-    ids = np.random.default_rng(11).integers(0, 8192, size=(8, 256))
-    with backend.use():
-        for name, dtype in (("cfg5_transformer_fwd_f32", F32), ("cfg5_transformer_fwd_f16", F16)):
-            model = Transformer(dtype=dtype)
-            tokens = Tensor(data=ids)
-            for _ in range(2):
-                model(tokens).wait()
-            t0 = time.perf_counter()
-            for _ in range(5):
-                model(tokens).wait()
-            dt = (time.perf_counter() - t0) / 5
-            out[name] = {"ms": round(dt * 1e3, 3), "tokens_per_s": round(2048 / dt, 1),
-                         "tflops": round(100.9e9 / dt / 1e12, 2)}
-            if not graph:
-                continue
-            # the same forward pass recorded once and replayed as one graph launch
-            with backend.capture() as cap:
-                logits = model(tokens)
-            for _ in range(3):
-                cap.graph.launch()
-            logits.wait()
-            t0 = time.perf_counter()
-            for _ in range(20):
-                cap.graph.launch()
+    def cfg5():
+        # config 5: decoder-only transformer forward, 8 x 256 tokens; tokens/s = 2048 / wall time of
+        # a forward pass ending in wait() on the logits (host-side op dispatch included)
+        from honeycrisp_amd.nn import Transformer
+        from honeycrisp_amd.tensor import Tensor
+        ids = np.random.default_rng(11).integers(0, 8192, size=(8, 256))
+        with backend.use():
+            for name, dtype in (("cfg5_transformer_fwd_f32", F32), ("cfg5_transformer_fwd_f16", F16)):
+                model = Transformer(dtype=dtype)
+                tokens = Tensor(data=ids)
+                for _ in range(2):
+                    model(tokens).wait()
+                t0 = time.perf_counter()
+                for _ in range(5):
+                    model(tokens).wait()
+                dt = (time.perf_counter() - t0) / 5
+                out[name] = {"ms": round(dt * 1e3, 3), "tokens_per_s": round(2048 / dt, 1),
+                             "tflops": round(100.9e9 / dt / 1e12, 2)}
+                if not graph:
+                    continue
+                # the same forward pass recorded once and replayed as one graph launch
+                with backend.capture() as cap:
+                    logits = model(tokens)
+                for _ in range(3):
+                    cap.graph.launch()
                 logits.wait()
-            dt = (time.perf_counter() - t0) / 20
-            out[name + "_graph"] = {"ms": round(dt * 1e3, 3), "tokens_per_s": round(2048 / dt, 1),
-                                    "tflops": round(100.9e9 / dt / 1e12, 2)}
-            cap.graph.destroy()
+                t0 = time.perf_counter()
+                for _ in range(20):
+                    cap.graph.launch()
+                    logits.wait()
+                dt = (time.perf_counter() - t0) / 20
+                out[name + "_graph"] = {"ms": round(dt * 1e3, 3), "tokens_per_s": round(2048 / dt, 1),
+                                        "tflops": round(100.9e9 / dt / 1e12, 2)}
+                cap.graph.destroy()
+
+    for name, fn in (("cfg1", cfg1), ("cfg2", cfg2), ("cfg3", cfg3), ("cfg4", cfg4), ("cfg5", cfg5)):
+        if name in only:
+            fn()
     return out
 
 
@@ -444,6 +517,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the other BASELINE configs")
+    ap.add_argument("--only", default="", help="comma-separated parts to run: headline,cfg1,...,cfg5 (default: all)")
     ap.add_argument("--no-graph", action="store_true",
                     help="skip the graph-replay variant of the transformer (rocprofv3's tracer crashes "
                          "inside hipGraphLaunch on this ROCm)")
@@ -458,6 +532,15 @@ def main():
     from honeycrisp_amd.backend import HIPBackend
     backend = HIPBackend(0)
     info = backend.deviceInfo()
+    parts = [x for x in args.only.split(",") if x] or ["headline", "cfg1", "cfg2", "cfg3", "cfg4", "cfg5"]
+    unknown = [x for x in parts if x not in ("headline", "cfg1", "cfg2", "cfg3", "cfg4", "cfg5")]
+    if unknown:
+        ap.error("--only: unknown part(s) %s" % ",".join(unknown))
+    if "headline" not in parts:      # a profiling run of another config: keep the headline to a token length
+        args.steps, args.warmup = min(args.steps, 2), min(args.warmup, 1)
+        global SPINUP_MS
+        SPINUP_MS = 1.0
+        args.no_cpu = True
     value, ms_per_step, roofline, (a, b) = headline(backend, args.steps, args.warmup)
     result = {
         "metric": "matmul TFLOP/s (fp16 in, fp32 accumulate, 4096^3, mean over NN/NT/TN/TT)",
@@ -471,11 +554,14 @@ def main():
         "frac_of_peak": round(value / PEAK_F16_TFLOPS, 4),
         "roofline": roofline,
     }
+    if args.only:
+        result["only"] = parts
     if not args.no_extra:
-        result["extra"] = extra_workloads(backend, graph=not args.no_graph)
+        result["extra"] = extra_workloads(backend, graph=not args.no_graph,
+                                          only=[x for x in parts if x != "headline"])
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(a, b)
-        if not args.no_extra:
+        if not args.no_extra and "cfg1" in parts and "cfg4" in parts:
             result["extra"]["cpu_reference_path"] = cpu_reference_ops()
     else:
         result["cpu_baseline"] = None

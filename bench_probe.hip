@@ -8,10 +8,26 @@
 // tiles of 4 registers; per multiply-accumulate it moves half as many accumulator registers and
 // runs at a higher clock under the same power limit). The MFMAs are written as assembly so
 // that the accumulators stay in the accumulation registers.
+//
+// Belongs to bench.py, not to the library: bench.py loads the code object built from this file
+// (`hipcc --genco`, see __graft_entry__.build) through hc_module_load and launches it with
+// hc_launch, one 256-lane workgroup per compute unit.
+#include <hip/hip_runtime.h>
+
+#include <stdint.h>
 #include <type_traits>
 
-#include "common.hip.h"
-#include "../kargs.h"
+#define HCK_BLOCK 256
+#define HC_KERNEL extern "C" __global__ __launch_bounds__(HCK_BLOCK)
+
+// `chunks` 16-byte pieces of operand bit patterns at `data`; one float per lane goes to `out`
+// so that the arithmetic cannot be dropped. The kernel's only parameter (24 bytes of kernarg).
+typedef struct {
+  const void* data;
+  void* out;
+  uint32_t iters;
+  uint32_t chunks;
+} hck_probe_args;
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));

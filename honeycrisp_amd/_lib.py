@@ -97,7 +97,6 @@ PROTOTYPES = {
     "hc_reduce_noalloc": (c_int, [_P, c_int, c_int, _P, _P, c_int64, c_int64, c_int64]),
     "hc_cumulative": (c_int, [_P, c_int, c_int, _P, _P, c_int64, c_int64, c_int64, c_int, c_int]),
     "hc_argsort": (c_int, [_P, c_int, _P, _P, c_int64, c_int64, c_int64, c_int]),
-    "hc_probe_mfma": (c_int, [_P, c_int, _P, ctypes.c_uint64, ctypes.c_uint32, POINTER(ctypes.c_double)]),
     "hc_log_softmax": (c_int, [_P, c_int, _P, _P, c_int64, c_int64, c_int64]),
     "hc_normalize": (c_int, [_P, c_int, _P, _P, c_int64, c_int64, c_int64, c_float]),
     "hc_gather": (c_int, [_P, c_int, _P, _P, _S, _P, c_int64, c_int64, c_int64, c_int64]),

@@ -410,16 +410,6 @@ class HIPBackend(Backend):
     def sync(self):
         self._check(self._lib.hc_sync(self._ctx))
 
-    def probeMfma(self, data, shape: int = 1, iters: int = 1024) -> float:
-        """Launches the MFMA-only measurement kernel once on the bit patterns of `data` (shape 0:
-        32x32x16, 1: 16x16x32); returns the floating-point operations of that launch (time it with
-        events). No Backend counterpart."""
-        d = self._dev(data)
-        flops = ctypes.c_double(0.0)
-        self._check(self._lib.hc_probe_mfma(self._ctx, shape, c_void_p(d.ptr), d.byteCount, iters,
-                                            ctypes.byref(flops)))
-        return flops.value
-
     def capture(self) -> "Capture":
         """`with backend.capture() as cap: out = model(x)` records every op issued inside the
         block instead of running it; `cap.graph.launch()` then replays the whole recording with

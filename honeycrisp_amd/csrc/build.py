@@ -22,7 +22,6 @@ KERNELS = [
     ("reduce", "reduce.hip", ["-ffp-contract=off"]),
     ("gather", "gather.hip", []),
     ("scan", "scan.hip", ["-ffp-contract=off"]),
-    ("probe", "probe.hip", []),
     ("gemm", "gemm.hip", []),
     ("gemm_f16_fast", "gemm_f16_fast.hip", []),
     ("gemm_dma", "gemm_dma.hip", []),

@@ -26,7 +26,6 @@ extern const unsigned char hc_image_elementwise[], hc_image_elementwise_end[];
 extern const unsigned char hc_image_reduce[], hc_image_reduce_end[];
 extern const unsigned char hc_image_gather[], hc_image_gather_end[];
 extern const unsigned char hc_image_scan[], hc_image_scan_end[];
-extern const unsigned char hc_image_probe[], hc_image_probe_end[];
 extern const unsigned char hc_image_gemm[], hc_image_gemm_end[];
 extern const unsigned char hc_image_gemm_f16_fast[], hc_image_gemm_f16_fast_end[];
 extern const unsigned char hc_image_gemm_dma[], hc_image_gemm_dma_end[];
@@ -170,7 +169,6 @@ extern "C" int hc_init(int device, hc_ctx** out) {
   if (s == HC_OK) s = load_image(ctx, hc_image_reduce, hc_image_reduce_end, "reduce");
   if (s == HC_OK) s = load_image(ctx, hc_image_gather, hc_image_gather_end, "gather");
   if (s == HC_OK) s = load_image(ctx, hc_image_scan, hc_image_scan_end, "scan");
-  if (s == HC_OK) s = load_image(ctx, hc_image_probe, hc_image_probe_end, "probe");
   if (s == HC_OK) s = load_image(ctx, hc_image_gemm, hc_image_gemm_end, "gemm");
   if (s == HC_OK) s = load_image(ctx, hc_image_gemm_f16_fast, hc_image_gemm_f16_fast_end, "gemm_f16_fast");
   if (s == HC_OK) s = load_image(ctx, hc_image_gemm_dma, hc_image_gemm_dma_end, "gemm_dma");
@@ -1446,29 +1444,6 @@ extern "C" int hc_argsort(hc_ctx* ctx, int dtype, const void* in, void* out, int
   char name[64];
   snprintf(name, sizeof(name), "hc_argsort_%s", dtype_name(dtype));
   return launch(ctx, name, (uint64_t)outer * (uint64_t)inner, 1, &k, sizeof(k));
-}
-
-extern "C" int hc_probe_mfma(hc_ctx* ctx, int shape, const void* data, uint64_t bytes, uint32_t iters,
-                             double* flops) {
-  REQUIRE(ctx, "hc_probe_mfma: null context");
-  REQUIRE(shape == 0 || shape == 1, "hc_probe_mfma: shape is 0 (32x32x16) or 1 (16x16x32)");
-  REQUIRE(data && bytes >= 16 && aligned16(data), "hc_probe_mfma: needs at least 16 bytes, 16-byte aligned");
-  REQUIRE(iters >= 2 && iters % 2 == 0, "hc_probe_mfma: iters must be even and positive");
-  // one workgroup of four waves per compute unit, one wave per SIMD: the occupancy of the large GEMM tile
-  const uint64_t blocks = (uint64_t)ctx->props.multiProcessorCount;
-  Scratch scratch(ctx);
-  void* out = nullptr;
-  HC_TRY(scratch.get(blocks * HCK_BLOCK * sizeof(float), &out));
-  hck_probe_args k;
-  memset(&k, 0, sizeof(k));
-  k.data = data;
-  k.out = out;
-  k.iters = iters;
-  k.chunks = (uint32_t)std::min<uint64_t>(bytes / 16, 0xffffffffull);
-  // per iteration and wave: 16 MFMAs of 32 x 32 x 16 (or 32 of 16 x 16 x 32)
-  if (flops) *flops = 2.0 * 32 * 32 * 16 * 16.0 * (double)iters * (double)(blocks * HCK_BLOCK / 64);
-  return launch(ctx, shape == 0 ? "hc_probe_mfma_f16_32x32x16" : "hc_probe_mfma_f16_16x16x32", blocks, 1, &k,
-                sizeof(k));
 }
 
 extern "C" int hc_log_softmax(hc_ctx* ctx, int dtype, const void* in, void* out, int64_t outer,

@@ -159,15 +159,6 @@ typedef struct {
   uint32_t run, descending, pad;
 } hck_sort_args;
 
-/* MFMA rate probe: `chunks` 16-byte pieces of operand bit patterns at `data`; one float per lane
- * goes to `out` so that the arithmetic cannot be dropped. */
-typedef struct {
-  const void* data;
-  void* out;
-  uint32_t iters;
-  uint32_t chunks;
-} hck_probe_args;
-
 /* Fused AdamW step over `count` contiguous elements; the scalars are the ones the op-by-op
  * composition would pass to its tensor-scalar ops. */
 typedef struct {

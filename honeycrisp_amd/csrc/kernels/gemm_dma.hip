@@ -306,9 +306,6 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
 
   const uint32_t nk = (p.K + BK - 1) / BK;
   Frags f0, f1;
-#ifdef HC_PROBE_WAITS
-  uint64_t probe_wait_dma = 0, probe_wait_bar = 0;  // cycles this wave spent in the two waits
-#endif
 
   // K-step j out of `cur`; `nxt` holds K-step j+1, `prev` held K-step j-1.
   auto step = [&](auto tail, char* cur, char* nxt, char* prev, uint32_t j) {
@@ -322,22 +319,8 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
       mma_one(f0, t);
       __builtin_amdgcn_sched_barrier(0);
     }
-#ifdef HC_PROBE_WAITS
-    const uint64_t w0 = __builtin_readcyclecounter();
-#ifdef HC_PROBE_SLACK
-    wait_dma<HC_PROBE_SLACK>();  // fewer DMA instructions left in flight: less time to land
-#else
-    wait_dma<2 * NDMA>();
-#endif
-    const uint64_t w1 = __builtin_readcyclecounter();
-    lds_barrier();
-    const uint64_t w2 = __builtin_readcyclecounter();
-    probe_wait_dma += w1 - w0;
-    probe_wait_bar += w2 - w1;
-#else
     wait_dma<2 * NDMA>();  // K-step j+1 of this wave has landed ...
     lds_barrier();         // ... and everybody's; nobody reads cur any more
-#endif
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int t = 0; t < SLOTS; t++) {  // sub-step 1
@@ -365,9 +348,6 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
 #pragma unroll
   for (int u = 0; u < READS; u++) read_unit(f0, lds0, 0, u);
 
-#if defined(HC_PROBE_CLOCKS) || defined(HC_PROBE_WAITS)
-  const uint64_t probe_c0 = __builtin_readcyclecounter(), probe_r0 = __builtin_amdgcn_s_memrealtime();
-#endif
   uint32_t j = 0;
   if constexpr (EDGE) {  // K-step j fetches slices j+3 and j+4: up to j = nk-6 the last slice is not among them
     for (; j + 9 <= nk; j += 4) {
@@ -387,12 +367,6 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
   if (j + 1 < nk) step(Tail{}, lds1, lds2, lds0, j + 1);
   if (j + 2 < nk) step(Tail{}, lds2, lds3, lds1, j + 2);
   wait_dma<0>();  // no LDS write of this workgroup may be in flight when it ends
-#if defined(HC_PROBE_CLOCKS) || defined(HC_PROBE_WAITS)
-  // measurement build: the first 16 bytes of the block's C tile receive the K-loop duration
-  // in shader cycles and in 100 MHz ticks instead of results (HC_PROBE_WAITS: 32 bytes per
-  // wave, with the cycles spent waiting for DMA and at the barrier)
-  const uint64_t probe_c1 = __builtin_readcyclecounter(), probe_r1 = __builtin_amdgcn_s_memrealtime();
-#endif
 
   // Epilogue. With the operands swapped, the MFMA tile is C^T: lane l holds m = l % 32 and,
   // in registers 4g..4g+3, the four consecutive columns n = 8g + 4*(l/32) + (0..3). Stored
@@ -437,24 +411,6 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
     }
     asm volatile("" ::: "memory");
   }
-#ifdef HC_PROBE_WAITS
-  __syncthreads();
-  if ((threadIdx.x & 63) == 0) {
-    uint64_t* dst = reinterpret_cast<uint64_t*>(C + (size_t)m0 * p.c_rs + n0) + (threadIdx.x >> 6) * 4;
-    dst[0] = probe_c1 - probe_c0;
-    dst[1] = probe_r1 - probe_r0;
-    dst[2] = probe_wait_dma;
-    dst[3] = probe_wait_bar;
-  }
-#endif
-#ifdef HC_PROBE_CLOCKS
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    uint64_t* dst = reinterpret_cast<uint64_t*>(C + (size_t)m0 * p.c_rs + n0);
-    dst[0] = probe_c1 - probe_c0;
-    dst[1] = probe_r1 - probe_r0;
-  }
-#endif
 }
 
 // Two variants per kernel: whole tiles only, and "_e" (edge) for M, N that are not multiples of

@@ -229,9 +229,6 @@ __device__ __forceinline__ void gemm_dma2_impl(const hck_gemm_args& p, char* lds
 
   // XCD-aware tile order. Block ids equal mod 8 run on one XCD and share its L2: give each
   // XCD a compact rectangle of tiles (few distinct A and B panels), or a contiguous band.
-#ifdef HC_PROBE_WAITS
-  const uint64_t probe_rs = __builtin_amdgcn_s_memrealtime();
-#endif
   const uint32_t total = p.tiles_m * p.tiles_n;
   uint32_t tile = blockIdx.x;
   if (p.xcd_gn != 0) {
@@ -323,11 +320,6 @@ __device__ __forceinline__ void gemm_dma2_impl(const hck_gemm_args& p, char* lds
   const uint32_t nk = (p.K + BK - 1) / BK;
   auto kclamp = [&](uint32_t j) { return (j < nk ? j : nk - 1) * BK; };  // steps past the end repeat the last one
   Frags f0, f1;
-#ifdef HC_PROBE_WAITS
-  // measurement build: cycles this wave spends in the two waits of a K-step; they replace the
-  // first bytes of the block's C tile (32 bytes per wave: loop cycles, 100 MHz ticks, waits)
-  uint64_t probe_wait_dma = 0, probe_wait_bar = 0;
-#endif
 
   // sub-step: MFMAs on `use`, operands of the following sub-step (number s_next of `from`)
   // into `fill`, and the DMA units of window part `part` (0, 1, 2; -1: none) of the K-slice
@@ -354,18 +346,8 @@ __device__ __forceinline__ void gemm_dma2_impl(const hck_gemm_args& p, char* lds
     substep(tail, f0, f1, cur, 1, 1, nxt, kclamp(j + 1));
     substep(tail, f1, f0, cur, 2, 2, nxt, kclamp(j + 1));
     substep(tail, f0, f1, cur, 3, -1, nullptr, 0);
-#ifdef HC_PROBE_WAITS
-    const uint64_t w0 = __builtin_readcyclecounter();
-    wait_dma<0>();
-    const uint64_t w1 = __builtin_readcyclecounter();
-    lds_barrier();
-    const uint64_t w2 = __builtin_readcyclecounter();
-    probe_wait_dma += w1 - w0;
-    probe_wait_bar += w2 - w1;
-#else
     wait_dma<0>();  // K-step j+1 of this wave has landed ...
     lds_barrier();  // ... and everybody's; nobody reads cur any more
-#endif
     __builtin_amdgcn_sched_barrier(0);
     substep(tail, f1, f0, nxt, 0, 0, cur, kclamp(j + 2));
   };
@@ -380,9 +362,6 @@ __device__ __forceinline__ void gemm_dma2_impl(const hck_gemm_args& p, char* lds
 #pragma unroll
   for (int u = 0; u < READS; u++) read_unit(f0, lds0, 0, u);
 
-#ifdef HC_PROBE_WAITS
-  const uint64_t probe_c0 = __builtin_readcyclecounter(), probe_r0 = __builtin_amdgcn_s_memrealtime();
-#endif
   uint32_t j = 0;
   if constexpr (EDGE) {  // K-step j fetches slices j+1 and j+2: up to j = nk-4 the last slice is not among them
     for (; j + 5 <= nk; j += 2) {
@@ -396,9 +375,6 @@ __device__ __forceinline__ void gemm_dma2_impl(const hck_gemm_args& p, char* lds
   }
   if (j < nk) step(Tail{}, lds0, lds1, j);
   wait_dma<0>();  // no LDS write of this workgroup may be in flight when it ends
-#ifdef HC_PROBE_WAITS
-  const uint64_t probe_c1 = __builtin_readcyclecounter(), probe_r1 = __builtin_amdgcn_s_memrealtime();
-#endif
 
   // Epilogue. With the operands swapped, the MFMA tile is C^T: lane l holds m = l % 32 and,
   // in registers 4g..4g+3, the four consecutive columns n = 8g + 4*(l/32) + (0..3). Stored
@@ -446,16 +422,6 @@ __device__ __forceinline__ void gemm_dma2_impl(const hck_gemm_args& p, char* lds
     }
     asm volatile("" ::: "memory");
   }
-#ifdef HC_PROBE_WAITS
-  __syncthreads();
-  if ((threadIdx.x & 63) == 0) {
-    uint64_t* dst = reinterpret_cast<uint64_t*>(C + (size_t)m0 * p.c_rs + n0) + (threadIdx.x >> 6) * 4;
-    dst[0] = probe_c1 - probe_c0;
-    dst[1] = probe_r1 - probe_r0;
-    dst[2] = probe_wait_dma | ((probe_r0 - probe_rs) << 32);                           // + prologue ticks
-    dst[3] = probe_wait_bar | ((__builtin_amdgcn_s_memrealtime() - probe_r1) << 32);  // + epilogue ticks
-  }
-#endif
 }
 
 // Two variants per kernel: whole tiles only, and "_e" (edge) for M, N that are not multiples of

@@ -295,11 +295,6 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
   const uint32_t nk = (p.K + BK - 1) / BK;
   auto kclamp = [&](uint32_t j) { return (j < nk ? j : nk - 1) * BK; };  // steps past the end repeat the last one
   Frags f0, f1;
-#ifdef HC_PROBE_WAITS
-  // measurement build: cycles this wave spends in the two waits of a K-step; they replace the
-  // first bytes of the block's C tile (32 bytes per wave: loop cycles, 100 MHz ticks, waits)
-  uint64_t probe_wait_dma = 0, probe_wait_bar = 0;
-#endif
 
   // (compile-time loop indices throughout: every register array is indexed statically)
   auto substep = [&](auto tail, const Frags& use, Frags& fill, const char* from, auto s_next_c, auto part_c,
@@ -311,13 +306,9 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
       constexpr int w = part * SLOTS + t;
       constexpr int lo = (w * NDMA + W - 1) / W < NDMA ? (w * NDMA + W - 1) / W : NDMA;
       constexpr int hi = ((w + 1) * NDMA + W - 1) / W < NDMA ? ((w + 1) * NDMA + W - 1) / W : NDMA;
-#ifndef HC_MI16_NO_LOOP_DMA  // (measurement switch: wrong results)
       static_for<hi - lo>([&](auto uc) { dma_unit(tail, lo + decltype(uc)::value, k0, to); });
-#endif
       // operand reads of the following sub-step: one every RSTRIDE slots
-#ifndef HC_MI16_NO_LOOP_READS  // (measurement switch: wrong results)
       if constexpr (t % RSTRIDE == 0 && t / RSTRIDE < READS) read_unit(fill, from, s_next, t / RSTRIDE);
-#endif
       mma_one(use, t);
       __builtin_amdgcn_sched_barrier(0);
     });
@@ -329,18 +320,8 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
   auto step = [&](auto tail, char* cur, char* nxt, uint32_t j) {
     __builtin_amdgcn_sched_barrier(0);
     substep(tail, f0, f1, cur, std::integral_constant<int, 1>{}, std::integral_constant<int, 1>{}, nxt, kclamp(j + 1));
-#ifdef HC_PROBE_WAITS
-    const uint64_t w0 = __builtin_readcyclecounter();
-    wait_dma<0>();
-    const uint64_t w1 = __builtin_readcyclecounter();
-    lds_barrier();
-    const uint64_t w2 = __builtin_readcyclecounter();
-    probe_wait_dma += w1 - w0;
-    probe_wait_bar += w2 - w1;
-#else
     wait_dma<0>();  // K-step j+1 of this wave has landed ...
     lds_barrier();  // ... and everybody's; nobody reads cur any more
-#endif
     __builtin_amdgcn_sched_barrier(0);
     substep(tail, f1, f0, nxt, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, cur, kclamp(j + 2));
   };
@@ -352,9 +333,6 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
   lds_barrier();
   static_for<READS>([&](auto uc) { read_unit(f0, lds0, 0, decltype(uc)::value); });
 
-#ifdef HC_PROBE_WAITS
-  const uint64_t probe_c0 = __builtin_readcyclecounter(), probe_r0 = __builtin_amdgcn_s_memrealtime();
-#endif
   uint32_t j = 0;
   if constexpr (EDGE) {  // K-step j fetches slices j+1 and j+2: up to j = nk-4 the last slice is not among them
     for (; j + 5 <= nk; j += 2) {
@@ -371,9 +349,6 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
   // The compiler does not know that the assembly statements are MFMAs, so it would not keep the
   // epilogue's accumulator reads the required distance from the last of them: do it by hand.
   asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
-#ifdef HC_PROBE_WAITS
-  const uint64_t probe_c1 = __builtin_readcyclecounter(), probe_r1 = __builtin_amdgcn_s_memrealtime();
-#endif
 
   // Epilogue. Lane l of tile (i, j) holds m = l % 16 and the four consecutive columns
   // n = 4 * (l / 16) .. +3 (8 bytes of halfs). The wave's part of C goes through LDS in slabs
@@ -416,16 +391,6 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
     }
     asm volatile("" ::: "memory");
   }
-#ifdef HC_PROBE_WAITS
-  __syncthreads();
-  if ((threadIdx.x & 63) == 0) {
-    uint64_t* dst = reinterpret_cast<uint64_t*>(C + (size_t)m0 * p.c_rs + n0) + (threadIdx.x >> 6) * 4;
-    dst[0] = probe_c1 - probe_c0;
-    dst[1] = probe_r1 - probe_r0;
-    dst[2] = probe_wait_dma;
-    dst[3] = probe_wait_bar | ((__builtin_amdgcn_s_memrealtime() - probe_r1) << 32);  // + epilogue ticks
-  }
-#endif
 }
 
 #define DEF_MI16(BM, BN, AN, AM, BNAME, BMODE)                                                        \

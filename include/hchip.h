@@ -236,15 +236,6 @@ int hc_reduce(hc_ctx* ctx, int op, int dtype, const void* in, void* out, int64_t
 int hc_reduce_noalloc(hc_ctx* ctx, int op, int dtype, const void* in, void* out, int64_t outer,
                       int64_t reduce, int64_t inner);
 
-/* Measurement aid with no counterpart in the reference: one launch of a kernel that only issues
- * fp16 MFMAs on a 128 x 128 wave tile of accumulators (one workgroup per compute unit, no memory
- * traffic in the loop) with operand bit patterns taken from `data` (`bytes` long, 16-byte
- * aligned). shape 0 = v_mfma_f32_32x32x16_f16, 1 = v_mfma_f32_16x16x32_f16 (the one the large
- * fp16 GEMM uses); `iters` (even) steps of 16 k; `*flops` receives the floating-point operations
- * of the launch. Timed over many launches it gives the rate the matrix cores sustain on that
- * data under the board's power management, which is what bench.py reports next to the GEMM rate. */
-int hc_probe_mfma(hc_ctx* ctx, int shape, const void* data, uint64_t bytes, uint32_t iters, double* flops);
-
 /* Backend.cumulativeSum / cumulativeProd (Backend.swift:548-568; CPU BackendCPU.swift:922-998):
  * op 0 = running sum, 1 = running product along the middle axis of [outer, reduce, inner];
  * exclusive shifts the result by one position, reverse scans from the far end. */
