@@ -189,3 +189,30 @@ __device__ __forceinline__ V block_reduce(V v, Op op, V* lds /* >= 4 entries */)
   for (int w = 1; w < HCK_BLOCK / 64; w++) r = op(r, lds[w]);
   return r;
 }
+
+// Tile (tm, tn) of a GEMM block for the direct-to-LDS kernels. Block ids equal mod 8 run on one
+// XCD and share its L2: each XCD gets a compact rectangle of tiles (few distinct A and B panels)
+// inside a super-block, or, without the rectangle parameters, a contiguous band. The host only
+// passes powers of two for xcd_gn, xcd_sm and xcd_sn, so their divisions are shifts; one real
+// division (by the number of super-blocks per row, or by tiles_n) remains.
+__device__ __forceinline__ void gemm_tile_of_block(const hck_gemm_args& p, uint32_t block, uint32_t& tm, uint32_t& tn) {
+  if (p.xcd_gn != 0) {
+    const uint32_t lg = (uint32_t)__builtin_ctz(p.xcd_gn), lsm = (uint32_t)__builtin_ctz(p.xcd_sm),
+                   lsn = (uint32_t)__builtin_ctz(p.xcd_sn);
+    const uint32_t lper = 3 + lsm + lsn;             // blocks per super-block: 8 XCDs x sm x sn
+    const uint32_t group = block >> lper, w = block & ((1u << lper) - 1u);
+    const uint32_t x = w & 7u, t = w >> 3;
+    const uint32_t sbn = p.tiles_n >> (lg + lsn);    // super-blocks per row of super-blocks
+    const uint32_t sb_row = group / sbn, sb_col = group - sb_row * sbn;
+    const uint32_t xm = x >> lg, xn = x & (p.xcd_gn - 1u);
+    const uint32_t lm = t >> lsn, ln = t & (p.xcd_sn - 1u);
+    tm = (((sb_row << (3 - lg)) + xm) << lsm) + lm;
+    tn = (((sb_col << lg) + xn) << lsn) + ln;
+    return;
+  }
+  const uint32_t total = p.tiles_m * p.tiles_n;
+  uint32_t tile = block;
+  if ((total & 7u) == 0) tile = (block & 7u) * (total >> 3) + (block >> 3);
+  tm = tile / p.tiles_n;
+  tn = tile - tm * p.tiles_n;
+}

@@ -220,23 +220,8 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
   constexpr int HALF = NDMA / 2;
   constexpr int A_BYTES = OpA::BYTES;
 
-  // XCD-aware tile order. Block ids equal mod 8 run on one XCD and share its L2: give each
-  // XCD a compact rectangle of tiles (few distinct A and B panels), or a contiguous band.
-  const uint32_t total = p.tiles_m * p.tiles_n;
-  uint32_t tile = blockIdx.x;
-  if (p.xcd_gn != 0) {
-    const uint32_t per = 8 * p.xcd_sm * p.xcd_sn, gm = 8 / p.xcd_gn;
-    const uint32_t group = blockIdx.x / per, w = blockIdx.x - group * per;
-    const uint32_t x = w & 7u, t = w >> 3;
-    const uint32_t sbn = p.tiles_n / (p.xcd_gn * p.xcd_sn);
-    const uint32_t sb_row = group / sbn, sb_col = group - sb_row * sbn;
-    const uint32_t xm = x / p.xcd_gn, xn = x - xm * p.xcd_gn;
-    const uint32_t lm = t / p.xcd_sn, ln = t - lm * p.xcd_sn;
-    tile = (sb_row * gm * p.xcd_sm + xm * p.xcd_sm + lm) * p.tiles_n + sb_col * p.xcd_gn * p.xcd_sn + xn * p.xcd_sn + ln;
-  } else if ((total & 7u) == 0) {
-    tile = (blockIdx.x & 7u) * (total >> 3) + (blockIdx.x >> 3);
-  }
-  const uint32_t tm = tile / p.tiles_n, tn = tile - tm * p.tiles_n;
+  uint32_t tm, tn;
+  gemm_tile_of_block(p, blockIdx.x, tm, tn);
   const uint32_t m0 = tm * BM, n0 = tn * BN;
   const uint32_t batch = blockIdx.y;
   const T* A = (const T*)p.a + batch * p.a_bs;

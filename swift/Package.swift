@@ -14,25 +14,26 @@ let package = Package(
     .executable(name: "HCMatrixBench", targets: ["HCMatrixBench"]),
   ],
   dependencies: [
-    // A Linux-buildable checkout of Honeycrisp (Accelerate / Metal shim modules in place).
-    .package(path: "../../honeycrisp")
+    // The offline Linux package of Honeycrisp: honeycrisp-linux/prepare.py derives its sources from an
+    // upstream checkout (macros expanded ahead of time; Accelerate, Metal and Gzip stand-ins in place).
+    .package(path: "honeycrisp-linux")
   ],
   targets: [
     .systemLibrary(name: "CHCHIP", path: "Sources/CHCHIP"),
     .target(
       name: "HoneycrispHIP",
-      dependencies: ["CHCHIP", .product(name: "Honeycrisp", package: "honeycrisp")],
+      dependencies: ["CHCHIP", .product(name: "Honeycrisp", package: "honeycrisp-linux")],
       linkerSettings: [
         .unsafeFlags(["-L../honeycrisp_amd/csrc", "-Xlinker", "-rpath", "-Xlinker", "../honeycrisp_amd/csrc"])
       ]),
     .executableTarget(
       name: "HCMatrixBench",
-      dependencies: ["HoneycrispHIP", .product(name: "Honeycrisp", package: "honeycrisp")]),
+      dependencies: ["HoneycrispHIP", .product(name: "Honeycrisp", package: "honeycrisp-linux")]),
     .testTarget(
       name: "HoneycrispHIPTests",
       dependencies: [
-        "HoneycrispHIP", .product(name: "Honeycrisp", package: "honeycrisp"),
-        .product(name: "HCTestUtils", package: "honeycrisp"),
+        "HoneycrispHIP", .product(name: "Honeycrisp", package: "honeycrisp-linux"),
+        .product(name: "HCTestUtils", package: "honeycrisp-linux"),
       ]),
   ]
 )
