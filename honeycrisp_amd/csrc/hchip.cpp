@@ -74,6 +74,7 @@ struct hc_ctx {
   int stage_cur = 0;
   hipEvent_t stage_ev[2] = {nullptr, nullptr};
   bool stage_busy[2] = {false, false};
+  std::vector<hipEvent_t> wait_events;  // spare events of blocking transfers (waited for outside the mutex)
 };
 static const size_t kStageHalf = 2u << 20;    // bytes per half of the staging buffer
 static const size_t kStageMax = 256u << 10;   // largest upload that is staged
@@ -206,6 +207,7 @@ extern "C" void hc_shutdown(hc_ctx* ctx) {
   if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
   for (hipEvent_t ev : ctx->stage_ev)
     if (ev) (void)hipEventDestroy(ev);
+  for (hipEvent_t ev : ctx->wait_events) (void)hipEventDestroy(ev);
   if (ctx->stage) (void)hipHostFree(ctx->stage);
   delete ctx;
 }
@@ -350,34 +352,82 @@ extern "C" int hc_host_free(hc_ctx* ctx, void* ptr) {
   return HC_OK;
 }
 
+// An event recorded on the stream now (mutex held by the caller), from the context's spare list.
+static int record_wait_event_locked(hc_ctx* ctx, hipEvent_t* out) {
+  hipEvent_t ev = nullptr;
+  if (!ctx->wait_events.empty()) {
+    ev = ctx->wait_events.back();
+    ctx->wait_events.pop_back();
+  } else {
+    HIP_TRY(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+  }
+  hipError_t e = hipEventRecord(ev, ctx->stream);
+  if (e != hipSuccess) {
+    ctx->wait_events.push_back(ev);
+    return hip_fail(e, "hipEventRecord");
+  }
+  *out = ev;
+  return HC_OK;
+}
+
+// Waits for `ev` WITHOUT the mutex, so that other threads keep allocating and enqueueing while
+// this one sleeps, then puts the event back.
+static int wait_event_unlocked(hc_ctx* ctx, hipEvent_t ev) {
+  hipError_t e = hipEventSynchronize(ev);
+  {
+    std::lock_guard<std::mutex> lock(ctx->mu);
+    ctx->wait_events.push_back(ev);
+  }
+  if (e != hipSuccess) return hip_fail(e, "hipEventSynchronize");
+  return HC_OK;
+}
+
 static int copy(hc_ctx* ctx, void* dst, const void* src, size_t bytes, hipMemcpyKind kind, bool wait) {
   REQUIRE(ctx, "memcpy: null context");
   if (bytes == 0) return HC_OK;
   REQUIRE(dst && src, "memcpy: null pointer");
-  std::lock_guard<std::mutex> lock(ctx->mu);
-  REQUIRE(!ctx->capturing || kind == hipMemcpyDeviceToDevice,
-          "memcpy: host transfers are not allowed while capturing (upload inputs before hc_capture_begin)");
-  if (kind == hipMemcpyHostToDevice && wait && bytes <= kStageMax && ctx->stage) {
-    // The caller may reuse `src` as soon as this returns: copy it into pinned memory and let the
-    // stream pick it up from there. No wait, so the device keeps running what is already queued
-    // (index vectors of slices, small constants in the middle of a forward pass).
-    if (ctx->stage_off + bytes > kStageHalf) {
-      HIP_TRY(hipEventRecord(ctx->stage_ev[ctx->stage_cur], ctx->stream));
-      ctx->stage_busy[ctx->stage_cur] = true;
-      ctx->stage_cur ^= 1;
-      ctx->stage_off = 0;
-      if (ctx->stage_busy[ctx->stage_cur]) HIP_TRY(hipEventSynchronize(ctx->stage_ev[ctx->stage_cur]));
-      ctx->stage_busy[ctx->stage_cur] = false;
+  hipEvent_t ev = nullptr;
+  {
+    std::lock_guard<std::mutex> lock(ctx->mu);
+    REQUIRE(!ctx->capturing || kind == hipMemcpyDeviceToDevice,
+            "memcpy: host transfers are not allowed while capturing (upload inputs before hc_capture_begin)");
+    if (kind == hipMemcpyHostToDevice && wait && bytes <= kStageMax && ctx->stage) {
+      // The caller may reuse `src` as soon as this returns: copy it into pinned memory and let the
+      // stream pick it up from there. No wait, so the device keeps running what is already queued
+      // (index vectors of slices, small constants in the middle of a forward pass).
+      if (ctx->stage_off + bytes > kStageHalf) {
+        HIP_TRY(hipEventRecord(ctx->stage_ev[ctx->stage_cur], ctx->stream));
+        ctx->stage_busy[ctx->stage_cur] = true;
+        ctx->stage_cur ^= 1;
+        ctx->stage_off = 0;
+        if (ctx->stage_busy[ctx->stage_cur]) HIP_TRY(hipEventSynchronize(ctx->stage_ev[ctx->stage_cur]));
+        ctx->stage_busy[ctx->stage_cur] = false;
+      }
+      char* slot = ctx->stage + (size_t)ctx->stage_cur * kStageHalf + ctx->stage_off;
+      memcpy(slot, src, bytes);
+      ctx->stage_off += (bytes + 63) & ~(size_t)63;
+      HIP_TRY(hipMemcpyAsync(dst, slot, bytes, kind, ctx->stream));
+      return HC_OK;
     }
-    char* slot = ctx->stage + (size_t)ctx->stage_cur * kStageHalf + ctx->stage_off;
-    memcpy(slot, src, bytes);
-    ctx->stage_off += (bytes + 63) & ~(size_t)63;
-    HIP_TRY(hipMemcpyAsync(dst, slot, bytes, kind, ctx->stream));
-    return HC_OK;
+    if (!wait) {
+      HIP_TRY(hipMemcpyAsync(dst, src, bytes, kind, ctx->stream));
+      return HC_OK;
+    }
+    // A blocking transfer first lets everything that is already enqueued finish, with the mutex
+    // released (a readback at the end of a long queue would otherwise stall every other thread's
+    // allocations and launches for the whole drain) ...
+    HC_TRY(record_wait_event_locked(ctx, &ev));
   }
-  HIP_TRY(hipMemcpyAsync(dst, src, bytes, kind, ctx->stream));
-  if (wait) HIP_TRY(hipStreamSynchronize(ctx->stream));
-  return HC_OK;
+  HC_TRY(wait_event_unlocked(ctx, ev));
+  {
+    // ... and then holds it only for the copy itself. Work that other threads enqueued in the
+    // meantime runs before the copy, which is what stream order promises anyway.
+    std::lock_guard<std::mutex> lock(ctx->mu);
+    REQUIRE(!ctx->capturing, "memcpy: host transfers are not allowed while capturing");
+    HIP_TRY(hipMemcpyAsync(dst, src, bytes, kind, ctx->stream));
+    HC_TRY(record_wait_event_locked(ctx, &ev));
+  }
+  return wait_event_unlocked(ctx, ev);
 }
 
 extern "C" int hc_memcpy_h2d(hc_ctx* ctx, void* dst, const void* src, size_t bytes) {
@@ -2281,9 +2331,11 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
         chunks = ceil_div(K, sk.kchunk);
         Scratch sums(ctx);
         void* acc = nullptr;
-        const uint64_t n_acc = (uint64_t)batch * sk.L * sk.t;
+        // one slice of partial sums per chunk, added in chunk order by the store kernel: the
+        // result is the same on every run (no atomics, nothing to clear)
+        sk.chunks = (uint32_t)chunks;
+        const uint64_t n_acc = (uint64_t)batch * chunks * sk.L * sk.t;
         HC_TRY(sums.get(n_acc * sizeof(float), &acc));
-        HC_TRY(hc_fill(ctx, HC_F32, 0.0f, 0, acc, n_acc));
         sk.acc = (float*)acc;
         snprintf(sname, sizeof(sname), "hc_gemm_skinny_p_%s_%s", dtype_name(dtype), tq);
         HC_TRY(launch(ctx, sname, ptiles * chunks, (uint32_t)batch, &sk, sizeof(sk)));

@@ -314,10 +314,11 @@ typedef struct {
   const void* x;
   const void* y;
   void* c;
-  float* acc;  /* split-K form: fp32 partial sums [batch, L, t], zero before the launch */
+  float* acc;  /* split-K form: fp32 partial sums [batch, chunks, L, t], one slice per k-chunk */
   uint32_t L, t, K;
   uint32_t x_ps, x_ks, y_ks, y_qs, c_ps, c_qs;
   uint32_t kchunk; /* split-K form: k-range per workgroup */
+  uint32_t chunks; /* split-K form: number of k-chunks */
   uint64_t x_bs, y_bs, c_bs;
 } hck_skinny_args;
 

@@ -305,8 +305,9 @@ template <typename T, int TQ> __device__ __forceinline__ void skinny_k_impl(cons
 // Long operand contiguous along p (16-byte aligned k-rows): a lane owns V consecutive p, a
 // wave reads 64 * V consecutive elements of a k-row per step; a workgroup covers one such
 // p-tile and a chunk of the k-range (grid.x = p-tiles * k-chunks), its four waves take every
-// fourth k-row and add their partial sums up in LDS; the chunks meet in an fp32 buffer through
-// atomic adds and hc_gemm_skinny_store rounds them. Y is packed [q][k].
+// fourth k-row and add their partial sums up in LDS; every chunk leaves its sums in a slice of its
+// own of an fp32 buffer and hc_gemm_skinny_store adds the slices in chunk order and rounds, so
+// the result does not depend on which workgroup finishes first. Y is packed [q][k].
 template <typename T, int TQ> __device__ __forceinline__ void skinny_p_impl(const hck_skinny_args& a) {
   constexpr int V = 16 / sizeof(T), WAVES = HCK_BLOCK / 64, TILE = 64 * V;
   __shared__ float part[WAVES][TQ][TILE];
@@ -353,8 +354,7 @@ template <typename T, int TQ> __device__ __forceinline__ void skinny_p_impl(cons
     float v = 0.0f;
 #pragma unroll
     for (int w = 0; w < WAVES; w++) v += part[w][q][c];
-    __hip_atomic_fetch_add(a.acc + ((uint64_t)blockIdx.y * a.L + p) * a.t + q, v, __ATOMIC_RELAXED,
-                           __HIP_MEMORY_SCOPE_AGENT);
+    a.acc[(((uint64_t)blockIdx.y * a.chunks + chunk) * a.L + p) * a.t + q] = v;
   }
 }
 
@@ -374,7 +374,11 @@ template <typename T> __device__ __forceinline__ void skinny_store_impl(const hc
   if (i >= (uint64_t)a.L * a.t) return;
   const uint32_t p = (uint32_t)(i / a.t), q = (uint32_t)(i - (uint64_t)p * a.t);
   T* C = (T*)a.c + (uint64_t)blockIdx.y * a.c_bs;
-  C[(size_t)p * a.c_ps + (size_t)q * a.c_qs] = narrow<T>(a.acc[(uint64_t)blockIdx.y * a.L * a.t + i]);
+  const uint64_t slice = (uint64_t)a.L * a.t;
+  const float* part = a.acc + (uint64_t)blockIdx.y * a.chunks * slice + i;
+  float v = 0.0f;
+  for (uint32_t c = 0; c < a.chunks; c++) v += part[c * slice];
+  C[(size_t)p * a.c_ps + (size_t)q * a.c_qs] = narrow<T>(v);
 }
 
 #define DEF_SKINNY(TN, T)                                                                          \

@@ -361,6 +361,7 @@ __device__ __forceinline__ void reduce_cols_impl(const hck_reduce_cols_args& p) 
   DEF_REDUCE(argmin, R_ARGMIN, TN, T)
 DEF_REDUCE_T(f32, float)
 DEF_REDUCE_T(f16, half_t)
+DEF_REDUCE_T(i64, int64_t)
 // bool tensors reduce as Float 0 / 1 (readBuffer(Float.self), BackendCPU.swift:2018-2030): what
 // Tensor.all / some issue (argmin / argmax + gather, ReduceRepeat.swift:103-162); a sum or product
 // written back as bool is "any" / "all".

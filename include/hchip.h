@@ -170,7 +170,19 @@ int hc_launch(hc_ctx* ctx, hc_function* fn, const uint32_t grid[3], const uint32
 
 /* ---- operations ----
  * Every pointer below is a device pointer from hc_malloc unless stated otherwise;
- * outputs are caller-allocated, dense, and never alias inputs. */
+ * outputs are caller-allocated, dense, and never alias inputs.
+ *
+ * Alignment. hc_malloc returns 256-byte aligned blocks, which satisfies every entry point. A
+ * pointer into the middle of a block (a view) must at least be aligned to its element size, and
+ *  - the contiguous maps and row kernels require 16-byte aligned buffers and return
+ *    HC_ERR_INVALID otherwise: hc_binary_op_scalar, hc_compare_scalar, hc_cast, hc_pow,
+ *    hc_elemwise, hc_fill, hc_adamw, hc_log_softmax, hc_log_softmax_grad, hc_normalize, hc_reduce
+ *    with inner == 1, and hc_scatter (whose output is cleared with hc_fill);
+ *  - everything else takes any element-aligned pointer and only loses its 16-byte vector
+ *    accesses: the broadcasting ops (hc_broadcast, hc_binary_op, hc_bitwise_op, hc_compare,
+ *    hc_mul_add, hc_add_mul, hc_when, hc_clamp), hc_reduce with inner > 1, hc_cumulative,
+ *    hc_argsort, hc_gather, hc_permute, hc_concat, hc_triangular and hc_matmul (which re-pitches
+ *    unaligned operands of large products into aligned scratch copies). */
 
 /* Backend.broadcast (Backend.swift:170-172; CPU BackendCPU.swift:255-265). */
 int hc_broadcast(hc_ctx* ctx, int dtype, const void* a, const hc_strides* as, void* out);

@@ -58,6 +58,40 @@ def test_status_codes_for_bad_arguments(hip_backend):
     hip_backend.sync()
 
 
+def test_alignment_contract(hip_backend):
+    """Views that start in the middle of an allocation: the contiguous maps and row kernels ask
+    for 16-byte aligned buffers (HC_ERR_INVALID with a message that says so), the broadcasting
+    and data-movement entry points take any element-aligned pointer and compute the same values."""
+    lib, ctx = hip_backend._lib, hip_backend._ctx
+    F32 = int(DType.float32)
+    x = np.arange(64, dtype=np.float32)
+    buf, out = hip_backend.upload(np.concatenate([[0.0], x]).astype(np.float32)), hip_backend.allocate(4 * 80)
+    view, dst = c_void_p(buf.ptr + 4), c_void_p(out.ptr + 4)        # 4-byte aligned only
+    whole = c_void_p(out.ptr)
+    for status in (lib.hc_elemwise(ctx, 11, F32, view, None, whole, c_size_t(64)),
+                   lib.hc_elemwise(ctx, 11, F32, c_void_p(buf.ptr), None, dst, c_size_t(64)),
+                   lib.hc_cast(ctx, view, F32, whole, int(DType.float16), c_size_t(64)),
+                   lib.hc_pow(ctx, F32, view, c_float(2.0), c_float(1.0), 0, 0, None, whole, c_size_t(64)),
+                   lib.hc_binary_op_scalar(ctx, 0, F32, view, c_float(1.0), 0, 0, whole, c_size_t(64)),
+                   lib.hc_fill(ctx, F32, c_float(1.0), 0, dst, c_size_t(64)),
+                   lib.hc_log_softmax(ctx, F32, view, whole, 4, 16, 1),
+                   lib.hc_normalize(ctx, F32, view, whole, 4, 16, 1, c_float(1e-5)),
+                   lib.hc_reduce(ctx, 0, F32, view, whole, 4, 16, 1)):
+        assert status == _lib.HC_ERR_INVALID
+        assert "16-byte aligned" in lib.hc_last_error_string().decode()
+    # element-aligned views are fine here
+    s = _lib.make_strides([64], [1])
+    hip_backend._check(lib.hc_binary_op(ctx, 0, F32, view, byref(s), view, byref(s), dst))
+    got = out.onCPU().view(np.float32)[1:65]
+    assert np.array_equal(got, x + x)
+    hip_backend._check(lib.hc_reduce(ctx, 0, F32, view, dst, 1, 8, 8))       # column sums, inner > 1
+    assert np.array_equal(out.onCPU().view(np.float32)[1:9], x.reshape(8, 8).sum(0))
+    idx = hip_backend.upload(np.array([3, 0, 5], dtype=np.int64))
+    si = _lib.make_strides([3, 8], [1, 0])
+    hip_backend._check(lib.hc_gather(ctx, F32, view, c_void_p(idx.ptr), byref(si), dst, 1, 8, 3, 8))
+    assert np.array_equal(out.onCPU().view(np.float32)[1:25].reshape(3, 8), x.reshape(8, 8)[[3, 0, 5]])
+
+
 def test_errors_surface_as_backend_errors(hip_backend):
     with hip_backend.use():
         x = Tensor(data=np.arange(6, dtype=np.int64).reshape(2, 3))

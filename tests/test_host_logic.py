@@ -65,3 +65,36 @@ def test_fast_division_constants_are_exact(tmp_path):
     out = subprocess.run([str(exe)], stdout=subprocess.PIPE, text=True)
     assert out.returncode == 0, out.stdout
     assert " 0 wrong" in out.stdout
+
+
+def test_code_objects_hold_every_reduce_and_gemm_kernel_the_host_names():
+    """The host builds kernel names from (form, op, dtype) at run time and looks them up in the
+    embedded code objects; a family that was dropped from a source file would only show on a GPU.
+    The names are plain strings in the built code objects."""
+    import itertools
+    build = os.path.join(ROOT, "honeycrisp_amd", "csrc", "build")
+    blob = {}
+    for name in ("reduce", "gemm", "gemm_dma", "gemm_dma2", "gemm_mi16", "elementwise", "gather"):
+        path = os.path.join(build, name + ".hsaco")
+        if not os.path.exists(path):
+            pytest.skip("code objects not built")
+        blob[name] = open(path, "rb").read()
+    forms = ["rows1", "rows8", "rows64", "rows256", "rowsplit", "cols"]
+    for form, op, dt in itertools.product(forms, ["sum", "prod", "argmax", "argmin"], ["f32", "f16", "i64", "b8"]):
+        names = ["hc_reduce_%s_%s_%s" % (form, op, dt)] if form != "cols" else \
+            ["hc_reduce_cols_%s_%s_v1" % (op, dt), "hc_reduce_cols_%s_%s_vN" % (op, dt), "hc_reduce_cols_final_%s_%s" % (op, dt)]
+        for n in names:
+            assert n.encode() + b"\0" in blob["reduce"], n
+    layouts = ["kk", "kn", "mk", "mn"]
+    for tile, lay, edge in itertools.product(["256x256", "256x192", "192x256", "192x192", "256x128", "128x128", "256x64",
+                                              "128x64", "64x64"], layouts, ["", "_e"]):
+        assert ("hc_gemm_f16_mi16_%s_%s%s" % (tile, lay, edge)).encode() + b"\0" in blob["gemm_mi16"]
+    for pipe, dt, tile, lay, edge in itertools.product(["dma", "dma2"], ["f16", "f32"],
+                                                       ["256x256", "256x128", "128x128", "256x64", "128x64", "64x64"],
+                                                       layouts, ["", "_e"]):
+        assert ("hc_gemm_%s_%s_%s_%s%s" % (dt, pipe, tile, lay, edge)).encode() + b"\0" in blob["gemm_" + pipe]
+    for dt in ("f16", "f32"):
+        for n in ("hc_gemm_%s_xx", "hc_gemm_%s_kk", "hc_gemm_skinny_k_%s_q4", "hc_gemm_skinny_p_%s_q4",
+                  "hc_gemm_skinny_pack_%s", "hc_gemm_skinny_store_%s", "hc_copy2d_pad_b%d", "hc_copy2d_unpad_b%d"):
+            name = n % (dt if "%s" in n else (2 if dt == "f16" else 4))
+            assert any(name.encode() + b"\0" in b for b in blob.values()), name
