@@ -2408,6 +2408,22 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
             bn = t[1];
           }
         }
+        // A K of one 128-byte slice is load -> one step of MFMAs -> store with nothing to overlap
+        // inside a workgroup, so what hides the latencies is several workgroups per CU: the largest
+        // tile that still gives every CU two blocks (QK^T of 32 x [512,64] x [64,512]: 256 x 128
+        // tiles 6.8 us, 128 x 128 tiles 6.2 us).
+        if (dma && (uint64_t)K * el <= 128) {
+          for (size_t ti = 0; ti < sizeof(tiles) / sizeof(tiles[0]); ti++) {
+            const uint32_t* t = tiles[ti];
+            const uint64_t blocks = ceil_div(M, t[0]) * ceil_div(N, t[1]) * (uint64_t)batch;
+            const double useful = ((double)M * N * (double)batch) / ((double)blocks * t[0] * t[1]);
+            if (blocks >= 2 * cus && useful >= 0.75) {
+              bm = t[0];
+              bn = t[1];
+              break;
+            }
+          }
+        }
         // fp32 products with K >= 512 also have the 192-extent tiles of the two-stage pipeline: fp32
         // runs every large tile at the same rate (it is not limited by power), so what counts is
         // how evenly the tiles fill the device (3072^2 outputs: 16 x 16 tiles of 192 x 192 are one

@@ -376,8 +376,18 @@ template <typename T> __device__ __forceinline__ void skinny_store_impl(const hc
   T* C = (T*)a.c + (uint64_t)blockIdx.y * a.c_bs;
   const uint64_t slice = (uint64_t)a.L * a.t;
   const float* part = a.acc + (uint64_t)blockIdx.y * a.chunks * slice + i;
+  // chunk order, 16 loads in flight at a time (one dependent load after the other would cost a
+  // memory latency per chunk)
   float v = 0.0f;
-  for (uint32_t c = 0; c < a.chunks; c++) v += part[c * slice];
+  uint32_t c = 0;
+  for (; c + 16 <= a.chunks; c += 16) {
+    float t[16];
+#pragma unroll
+    for (int u = 0; u < 16; u++) t[u] = part[(uint64_t)(c + u) * slice];
+#pragma unroll
+    for (int u = 0; u < 16; u++) v += t[u];
+  }
+  for (; c < a.chunks; c++) v += part[(uint64_t)c * slice];
   C[(size_t)p * a.c_ps + (size_t)q * a.c_qs] = narrow<T>(v);
 }
 
