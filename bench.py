@@ -20,9 +20,9 @@ Also reported in the same line:
 
 Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extra] [--no-graph]
                        [--only headline,cfg1,cfg2,cfg3,cfg4,cfg5]
-`--only` restricts the run to the named parts (the headline always runs, shortened when it is not
-named): what the per-config rocprofv3 summaries under profiles/ are made with, so that a kernel's
-launches of one config are not pooled with another's.
+`--only` restricts the run to the named parts (without `headline` the line's `value` is null): what
+the per-config rocprofv3 summaries under profiles/ are made with, so that a kernel's launches of
+one config are not pooled with another's.
 """
 import argparse
 import ctypes
@@ -164,7 +164,7 @@ def timed_launches(backend, events, fn, iters, warmup, batched=False):
     return float(np.mean(ms)), float(np.median(ms))
 
 
-def headline(backend, steps, warmup, full=True):
+def headline(backend, steps, warmup):
     from honeycrisp_amd.descriptors import DType
     n = 4096
     a = (np.random.default_rng(2).standard_normal((n, n)) / np.sqrt(n)).astype(np.float16)
@@ -212,11 +212,6 @@ def headline(backend, steps, warmup, full=True):
         events.free(m)
     ms_per_step = (t1 - t0) * 1e3 / steps
     value = 4 * flops / (ms_per_step * 1e-3) / 1e12
-    if not full:    # (a run restricted to other configs: no per-layout pass, no MFMA-only kernels)
-        achieved = flops / (launch_ms * 1e-3) / 1e12
-        return value, ms_per_step, {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_F16_TFLOPS,
-                                    "unit": "TFLOP/s", "frac": round(achieved / PEAK_F16_TFLOPS, 4),
-                                    "traffic": None, "note": "token headline of a run restricted with --only"}, (a, b)
     # Per-layout breakdown: a second, untimed pass with one event between consecutive launches.
     per_layout = {name: [] for name, _, _ in layouts}
     reps = min(steps, 50)
@@ -580,22 +575,21 @@ def main():
     unknown = [x for x in parts if x not in ("headline", "cfg1", "cfg2", "cfg3", "cfg4", "cfg5")]
     if unknown:
         ap.error("--only: unknown part(s) %s" % ",".join(unknown))
-    if "headline" not in parts:      # a profiling run of another config: keep the headline to a token length
-        args.steps, args.warmup = min(args.steps, 2), min(args.warmup, 1)
-        global SPINUP_MS
-        SPINUP_MS = 1.0
+    if "headline" in parts:
+        value, ms_per_step, roofline, (a, b) = headline(backend, args.steps, args.warmup)
+    else:      # a profiling run restricted to other configs: no headline launches in its trace
+        value, ms_per_step, roofline, a, b = None, None, None, None, None
         args.no_cpu = True
-    value, ms_per_step, roofline, (a, b) = headline(backend, args.steps, args.warmup, full="headline" in parts)
     result = {
         "metric": "matmul TFLOP/s (fp16 in, fp32 accumulate, 4096^3, mean over NN/NT/TN/TT)",
-        "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "value": None if value is None else round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": None if value is None else round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
         "config": {"workload": "configs[1]: fp16 GEMM M=N=K=4096, four transA/transB layouts per step, "
                                "entries N(0,1)/sqrt(K), seeds 2/3",
                    "device": info["name"], "arch": info["arch"], "compute_units": info["compute_units"],
                    "clock_mhz": info["clock_mhz"], "untimed_spinup_ms": SPINUP_MS},
-        "frac_of_peak": round(value / PEAK_F16_TFLOPS, 4),
+        "frac_of_peak": None if value is None else round(value / PEAK_F16_TFLOPS, 4),
         "roofline": roofline,
     }
     if args.only:
