@@ -2302,7 +2302,10 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
       // The thin operand is read by every wave: unless it already is contiguous along k with
       // aligned rows, pack it first as [q][k] (a few KiB that then stay in the caches).
       Scratch packed(ctx);
-      if ((sk.x_ks == 1 || sk.x_ps == 1) &&
+      const bool x_along_k = sk.x_ks == 1 && aligned16(sk.x) && sk.x_ps % P == 0 && (batch <= 1 || sk.x_bs % P == 0);
+      // (only the wave-per-row kernel reads the thin operand with vector loads; the other one takes
+      // it element by element with any strides)
+      if (x_along_k &&
           !(sk.y_ks == 1 && aligned16(sk.y) && sk.y_qs % P == 0 && (batch <= 1 || sk.y_bs % P == 0))) {
         const uint32_t kp = (K + P - 1) / P * P;
         void* buf = nullptr;
@@ -2318,7 +2321,7 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
         sk.y_qs = kp;
         sk.y_bs = (uint64_t)sk.t * kp;
       }
-      if (sk.x_ks == 1 && aligned16(sk.x) && sk.x_ps % P == 0 && (batch <= 1 || sk.x_bs % P == 0)) {
+      if (x_along_k) {
         snprintf(sname, sizeof(sname), "hc_gemm_skinny_k_%s_%s", dtype_name(dtype), tq);
         return launch(ctx, sname, ceil_div(sk.L, HCK_BLOCK / 64), (uint32_t)batch, &sk, sizeof(sk));
       }

@@ -307,7 +307,8 @@ template <typename T, int TQ> __device__ __forceinline__ void skinny_k_impl(cons
 // p-tile and a chunk of the k-range (grid.x = p-tiles * k-chunks), its four waves take every
 // fourth k-row and add their partial sums up in LDS; every chunk leaves its sums in a slice of its
 // own of an fp32 buffer and hc_gemm_skinny_store adds the slices in chunk order and rounds, so
-// the result does not depend on which workgroup finishes first. Y is packed [q][k].
+// the result does not depend on which workgroup finishes first. Y is read one element per wave
+// and step (wave-uniform), so it is taken as it lies, whatever its strides.
 template <typename T, int TQ> __device__ __forceinline__ void skinny_p_impl(const hck_skinny_args& a) {
   constexpr int V = 16 / sizeof(T), WAVES = HCK_BLOCK / 64, TILE = 64 * V;
   __shared__ float part[WAVES][TQ][TILE];
@@ -336,7 +337,7 @@ template <typename T, int TQ> __device__ __forceinline__ void skinny_p_impl(cons
 #pragma unroll
     for (int q = 0; q < TQ; q++) {
       if (q < (int)a.t) {
-        const float y = (float)Y[(size_t)q * a.y_qs + k];  // wave-uniform
+        const float y = (float)Y[(size_t)q * a.y_qs + (size_t)k * a.y_ks];  // wave-uniform, any strides
 #pragma unroll
         for (int e = 0; e < V; e++) acc[q][e] = acc[q][e] + (float)x[e] * y;
       }

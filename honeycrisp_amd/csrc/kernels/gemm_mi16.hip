@@ -379,10 +379,7 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
       const uint32_t piece = it * 64 + lane, r = piece / UNITS, u = piece % UNITS;
       const Chunk v = *reinterpret_cast<const Chunk*>(slab + r * RB + ((u ^ unit_swz(r)) * 16));
       const uint32_t row = m0 + wm + ii * 32 + r, col = n0 + wn + u * 8;
-      // (a streaming store: this pipeline only runs products whose output is far larger than the L2
-      // caches, and lines that do not linger there leave less to write back when the kernel ends:
-      // 0.7-1 us per launch at 4096 x 4096 outputs)
-      if (!EDGE || (row < p.M && col < p.N)) __builtin_nontemporal_store(v, reinterpret_cast<Chunk*>(C + (size_t)row * p.c_rs + col));
+      if (!EDGE || (row < p.M && col < p.N)) *reinterpret_cast<Chunk*>(C + (size_t)row * p.c_rs + col) = v;
     }
     asm volatile("" ::: "memory");
   }

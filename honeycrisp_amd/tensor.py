@@ -763,6 +763,35 @@ class Tensor:
     def tril(self, offset=0): return self._triangular(False, offset)
     def triu(self, offset=0): return self._triangular(True, offset)
 
+    # -- split / chunk (ConcatSplit.swift:87-115), one-hot rows (OneHot.swift)
+
+    def split(self, axis: int, counts: Sequence[int]) -> List["Tensor"]:
+        axis = self.positiveAxis(axis)
+        assert 0 <= axis < len(self.shape), "axis %d out of bounds for shape %s" % (axis, self.shape)
+        assert self.shape[axis] == sum(counts), "split counts %s do not sum to axis %d of shape %s" % (counts, axis, self.shape)
+        results, start = [], 0
+        for count in counts:
+            results.append(self[(FullRange(axis), slice(start, start + count))] if axis else self[start:start + count])
+            start += count
+        return results
+
+    def chunk(self, axis: int, count: int) -> List["Tensor"]:
+        axis = self.positiveAxis(axis)
+        assert self.shape[axis] >= count and self.shape[axis] % count == 0, \
+            "shape %s incompatible with chunk of count %d on axis %d" % (self.shape, count, axis)
+        return self.split(axis, [self.shape[axis] // count] * count)
+
+    @staticmethod
+    def oneHot(indices, count: int, dtype=DType.float32) -> "Tensor":
+        """Tensor(oneHot:count:): a host-built vector (one index) or matrix of rows (a list)."""
+        single = isinstance(indices, (int, np.integer))
+        rows = [indices] if single else list(indices)
+        data = np.zeros((len(rows), count), dtype=np.float32)
+        for i, idx in enumerate(rows):
+            assert 0 <= idx < count, "oneHot index %d out of range [0, %d)" % (idx, count)
+            data[i, idx] = 1
+        return Tensor(data=data.reshape(-1), shape=[count] if single else [len(rows), count], dtype=dtype)
+
     # -- concat (ConcatSplit.swift:4-75)
 
     @staticmethod

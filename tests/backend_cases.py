@@ -795,7 +795,52 @@ def testConcat():
     assertDataEqual(Tensor.concat([x, z], axis=0), [1, 2, 3, 4, 5, 6, 7, 8, 9])
 
 
-def testWhen():
+def testWhen(rng):
+    """BackendTests.swift:1659-1755: values, the gradients (mask.when(grad, 0) / mask.when(0, grad),
+    When.swift), pure scalar branches, and implicit == explicit broadcasting over every pairing of
+    the three shapes with tensor and scalar branches."""
+    x = Tensor(data=[1.0, 2.0, 3.0, 4.0], shape=[4])
+    y = Tensor(data=[-1.0, -2.0, -3.0, -4.0], shape=[4])
+    mask = Tensor(data=[False, True, True, False], shape=[4])
+    assertDataEqual(mask.when(x, y), [-1.0, 2.0, 3.0, -4.0])
+    grad = Tensor(data=[5.0, 6.0, 7.0, 8.0], shape=[4])
+    assertDataEqual(mask.when(grad, 0.0), [0, 6.0, 7.0, 0.0])
+    assertDataEqual(mask.when(0.0, grad), [5.0, 0.0, 0.0, 8.0])
+    assertDataEqual(mask.when(1.0, -1.0, dtype=F32), [-1, 1, 1, -1])
+    shapes = [[1, 6, 1], [3, 6, 2], [3, 1, 2]]
+    for maskShape in shapes:
+        m = Tensor(data=rng.random(maskShape).astype(np.float32)) < 0.5
+        for trueShape in shapes:
+            t = Tensor(data=rng.random(trueShape).astype(np.float32))
+            for falseShape in shapes:
+                f = Tensor(data=rng.random(falseShape).astype(np.float32))
+                b = Tensor.broadcast([m, t, f])
+                assertDataEqual(m.when(t, f), b[0].when(b[1], b[2]))
+                b = Tensor.broadcast([m, t])
+                assertDataEqual(m.when(t, 3.1415), b[0].when(b[1], 3.1415))
+                b = Tensor.broadcast([m, f])
+                assertDataEqual(m.when(3.1415, f), b[0].when(3.1415, b[1]))
+
+
+def testChunk():
+    """BackendTests.swift:1031-1048."""
+    for i in range(1, 10):
+        for count in range(1, i + 1):
+            if i % count != 0:
+                continue
+            parts = Tensor(data=range(i)).chunk(axis=0, count=count)
+            assert len(parts) == count
+            assert all(p.shape[0] == parts[0].shape[0] for p in parts)
+            assertDataEqual(Tensor.concat(parts, axis=0), [float(v) for v in range(i)])
+
+
+def testOneHot():
+    """BackendTests.swift:1757-1760."""
+    assertDataEqual(Tensor.oneHot(3, count=5), [0, 0, 0, 1, 0])
+    assertDataEqual(Tensor.oneHot([3, 1], count=5), [0, 0, 0, 1, 0, 0, 1, 0, 0, 0])
+
+
+def testWhenForms():
     """When.swift semantics: mask ? a : b with tensor / scalar branches, broadcasting."""
     mask = Tensor(data=[1, 0, 1, 0, 0, 1], shape=[2, 3]).cast(BOOL)
     a = Tensor(data=[1.0, 2.0, 3.0], shape=[3])
@@ -815,4 +860,5 @@ ALL_CASES = [
     testElemwise, testRounding, testMinMax, testExpandAndRepeat, testBinaryBroadcast, testFusedBroadcast,
     testSoftmax, testConcat, testWhen, testCumulativeSum, testCumulativeProd, testArgsort, testBitwise, testSoftmaxGrad, testScatter, testScatterIsAdjointOfGather, testClamp,
     testAdam, testNormalizeGrad, testProd, testRepeat, testAllSome, testConcatInner, testConcatOuter,
+    testWhenForms, testChunk, testOneHot,
 ]

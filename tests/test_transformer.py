@@ -19,6 +19,50 @@ def logits(backend, dtype, ids, **cfg):
 SMALL = dict(layers=2, d_model=64, heads=4, mlp=128, vocab=97, seq=16, seed=3)
 
 
+def numpy_forward(model, ids):
+    """The same decoder written directly in numpy float64 from the model's weights: no Tensor
+    front-end, no backend calls, no descriptors. A lowering mistake in the front-end mirror (a
+    wrong stride map, permutation or reduce axis) would hit both backends alike and cancel in a
+    backend-against-backend comparison; it cannot cancel here."""
+    f = lambda t: t.numpy().astype(np.float64)
+
+    def layer_norm(x, ln):
+        mean = x.mean(-1, keepdims=True)
+        var = ((x - mean) ** 2).mean(-1, keepdims=True)
+        return (x - mean) / np.sqrt(var + float(ln.eps)) * (f(ln.gain) + 1.0) + f(ln.bias)
+
+    def linear(x, lin):
+        return x @ f(lin.weight) + f(lin.bias)
+
+    B, T = ids.shape
+    x = f(model.table)[ids] + f(model.pos)[:T]
+    mask = np.where(np.arange(T)[:, None] >= np.arange(T)[None, :], 0.0, -1e4)
+    for blk in model.blocks:
+        H = blk.heads
+        hd = x.shape[-1] // H
+        h = layer_norm(x, blk.ln1)
+        q, k, v = (linear(h, w).reshape(B, T, H, hd).transpose(0, 2, 1, 3) for w in (blk.q, blk.k, blk.v))
+        scores = q @ k.transpose(0, 1, 3, 2) / np.sqrt(hd) + mask
+        scores = scores - scores.max(-1, keepdims=True)
+        probs = np.exp(scores)
+        probs /= probs.sum(-1, keepdims=True)
+        ctx = (probs @ v).transpose(0, 2, 1, 3).reshape(B, T, H * hd)
+        x = x + linear(ctx, blk.o)
+        u = linear(layer_norm(x, blk.ln2), blk.fc1)
+        u = 0.5 * u * (1.0 + np.tanh(0.797884561 * (u + 0.044715 * u ** 3)))      # GELU, tanh form (Elemwise.swift:109-111)
+        x = x + linear(u, blk.fc2)
+    return linear(layer_norm(x, model.ln_f), model.unembed)
+
+
+def test_small_transformer_matches_an_independent_numpy_model(oracle_backend):
+    ids = np.random.default_rng(0).integers(0, 97, size=(3, 16))
+    with oracle_backend.use():
+        model = Transformer(dtype=DType.float32, **SMALL)
+        got = model(Tensor(data=ids)).numpy()
+        want = numpy_forward(model, ids)
+    assert_close_arrays(got, want, 1e-4, 1e-4)
+
+
 def test_small_transformer_is_causal_under_the_oracle(oracle_backend):
     rng = np.random.default_rng(0)
     ids = rng.integers(0, 97, size=(3, 16))
@@ -54,6 +98,19 @@ def test_small_transformer_parity(hip_backend, oracle_backend, dtype, tol):
     got = logits(hip_backend, dtype, ids, **SMALL)
     want = logits(oracle_backend, dtype, ids, **SMALL)
     assert_close_arrays(got, want, tol, tol)
+
+
+@pytest.mark.gpu
+def test_config5_transformer_matches_an_independent_numpy_model(hip_backend):
+    """Config 5 in fp32 on the device against the float64 numpy model (same weights): independent of
+    the front-end mirror and of the oracle."""
+    ids = np.random.default_rng(11).integers(0, 8192, size=(8, 256))
+    with hip_backend.use():
+        model = Transformer(dtype=DType.float32)
+        got = model(Tensor(data=ids)).numpy()
+        want = numpy_forward(model, ids)
+    assert_close_arrays(got, want, 1e-4, 1e-4)
+    assert float(np.max(np.abs(got - want))) / float(np.max(np.abs(want))) <= 1e-4
 
 
 @pytest.mark.gpu
