@@ -34,4 +34,24 @@ final class HIPBackendTests: XCTestCase {
   func testBinaryBroadcast() async throws { try await runInHIP(BackendTests.testBinaryBroadcast) }
   func testFusedBroadcast() async throws { try await runInHIP(BackendTests.testFusedBroadcast) }
   func testSoftmax() async throws { try await runInHIP(BackendTests.testSoftmax) }
+  func testCreateFromData() async throws { try await runInHIP(BackendTests.testCreateFromData) }
+  func testEquals() async throws { try await runInHIP(BackendTests.testEquals) }
+  func testComparison() async throws { try await runInHIP(BackendTests.testComparison) }
+  func testBitwise() async throws { try await runInHIP(BackendTests.testBitwise) }
+  func testProd() async throws { try await runInHIP(BackendTests.testProd) }
+  func testCumulativeSum() async throws { try await runInHIP(BackendTests.testCumulativeSum) }
+  func testCumulativeProd() async throws { try await runInHIP(BackendTests.testCumulativeProd) }
+  func testArgsort() async throws { try await runInHIP(BackendTests.testArgsort) }
+  func testRepeat() async throws { try await runInHIP(BackendTests.testRepeat) }
+  func testTriangular() async throws { try await runInHIP(BackendTests.testTriangular) }
+  func testChunk() async throws { try await runInHIP(BackendTests.testChunk) }
+  func testClamp() async throws { try await runInHIP(BackendTests.testClamp) }
+  func testAllSome() async throws { try await runInHIP(BackendTests.testAllSome) }
+  func testConcatInner() async throws { try await runInHIP(BackendTests.testConcatInner) }
+  func testConcatOuter() async throws { try await runInHIP(BackendTests.testConcatOuter) }
+  func testWhen() async throws { try await runInHIP(BackendTests.testWhen) }
+  func testOneHot() async throws { try await runInHIP(BackendTests.testOneHot) }
+  func testAdam() async throws { try await runInHIP(BackendTests.testAdam) }
+  func testMulGrad() async throws { try await runInHIP(BackendTests.testMulGrad) }
+  func testMSEGrad() async throws { try await runInHIP(BackendTests.testMSEGrad) }
 }
