@@ -78,6 +78,7 @@ PROTOTYPES = {
     "hc_capture_end": (c_int, [_P, POINTER(c_void_p)]),
     "hc_capture_abort": (c_int, [_P]),
     "hc_graph_launch": (c_int, [_P, _P]),
+    "hc_graph_node_count": (c_int, [_P, POINTER(c_size_t)]),
     "hc_graph_destroy": (c_int, [_P, _P]),
     "hc_module_load": (c_int, [_P, _P, c_size_t, POINTER(c_void_p)]),
     "hc_module_unload": (c_int, [_P, _P]),

@@ -322,6 +322,12 @@ class Graph:
     def launch(self):
         self.backend._check(self.backend._lib.hc_graph_launch(self.backend._ctx, c_void_p(self._handle)))
 
+    def node_count(self) -> int:
+        """Kernel launches and copies one replay issues (after the recording's rewrite)."""
+        n = c_size_t(0)
+        self.backend._check(self.backend._lib.hc_graph_node_count(c_void_p(self._handle), byref(n)))
+        return int(n.value)
+
     def destroy(self):
         if self._handle and self.backend._ctx:
             self.backend._check(self.backend._lib.hc_graph_destroy(self.backend._ctx, c_void_p(self._handle)))

@@ -24,9 +24,10 @@ KERNELS = [
     ("scan", "scan.hip", ["-ffp-contract=off"]),
     ("gemm", "gemm.hip", []),
     ("gemm_f16_fast", "gemm_f16_fast.hip", []),
-    ("gemm_dma", "gemm_dma.hip", []),
-    ("gemm_dma2", "gemm_dma2.hip", []),
-    ("gemm_mi16", "gemm_mi16.hip", []),
+    # (their epilogues can apply a bias / residual / GELU with the element-wise kernels' arithmetic)
+    ("gemm_dma", "gemm_dma.hip", ["-ffp-contract=off"]),
+    ("gemm_dma2", "gemm_dma2.hip", ["-ffp-contract=off"]),
+    ("gemm_mi16", "gemm_mi16.hip", ["-ffp-contract=off"]),
 ]
 DEVICE_FLAGS = [
     "--offload-arch=gfx950", "--genco", "-O3", "-std=c++17",
@@ -41,11 +42,39 @@ def _run(cmd):
     return proc.stdout
 
 
+# Code objects whose kernels keep their accumulators in registers by construction: a kernel of these
+# that needs private (scratch) memory has lost that property (a loop over the accumulators that the
+# compiler no longer unrolls puts the whole array there and the kernel runs several times slower,
+# with correct results), so the build refuses it. Up to SCRATCH_ALLOWED bytes per lane pass: a few
+# registers spilled once between the main loop and the epilogue of the largest edge kernels.
+NO_SCRATCH = {"gemm_dma", "gemm_dma2", "gemm_mi16", "gemm_f16_fast"}
+SCRATCH_ALLOWED = 128
+
+
+def kernels_with_scratch(remarks):
+    """Names of kernels whose ScratchSize in -Rpass-analysis=kernel-resource-usage output exceeds
+    SCRATCH_ALLOWED."""
+    bad, current = [], None
+    for line in remarks.splitlines():
+        if "Function Name:" in line:
+            current = line.split("Function Name:")[1].split()[0]
+        elif "ScratchSize [bytes/lane]:" in line:
+            size = int(line.split("ScratchSize [bytes/lane]:")[1].split()[0])
+            if size > SCRATCH_ALLOWED:
+                bad.append("%s (%d bytes/lane)" % (current, size))
+    return bad
+
+
 def build_kernel(name, src, extra):
     out = os.path.join(BUILD_DIR, name + ".hsaco")
     # HCHIP_EXTRA_FLAGS: additional device-compile flags (kernel experiments, e.g. -DNAME=1)
     more = os.environ.get("HCHIP_EXTRA_FLAGS", "").split()
-    _run([HIPCC] + DEVICE_FLAGS + extra + more + ["-o", out, os.path.join(KERNEL_DIR, src)])
+    check = ["-Rpass-analysis=kernel-resource-usage"] if name in NO_SCRATCH else []
+    remarks = _run([HIPCC] + DEVICE_FLAGS + extra + more + check + ["-o", out, os.path.join(KERNEL_DIR, src)])
+    bad = kernels_with_scratch(remarks) if check else []
+    if bad:
+        os.remove(out)
+        raise RuntimeError("%s: kernels that must not use scratch memory do: %s" % (src, ", ".join(bad)))
     return out
 
 

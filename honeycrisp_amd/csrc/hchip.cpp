@@ -48,10 +48,53 @@ struct hc_event {
 
 // A captured recording plus the buffers it owns: `parked` holds, by bucket size, blocks that
 // were freed but must stay out of the general pool while the graph exists.
+// One entry of a recording in progress. While a capture runs, kernels are not handed to the
+// stream one by one: they are listed here, in call order, with the caller-visible buffers they
+// read and write, and hc_capture_end rewrites the list (producer / consumer chains whose
+// intermediate results nobody else reads become one kernel, see fuse_recording) before it
+// enqueues what is left on the capturing stream.
+struct hc_pending {
+  enum Kind { KERNEL, RAW_KERNEL, COPY_D2D, FREE } kind = KERNEL;
+  hipFunction_t fn = nullptr;
+  uint32_t grid[3] = {1, 1, 1}, block[3] = {HCK_BLOCK, 1, 1}, shared = 0;
+  std::vector<char> args;              // the kernel's by-value argument struct
+  void* dst = nullptr;                 // COPY_D2D / FREE
+  const void* src = nullptr;
+  size_t bytes = 0;
+  // Buffers of the operation this launch belongs to (OpNote). known == false: the entry point
+  // declared nothing, so the launch may touch anything and nothing is moved across it.
+  bool known = false;
+  std::vector<const void*> reads;
+  std::vector<const void*> writes;
+  // what the rewrite needs to know about the operations it can merge
+  enum Tag { NONE, GEMM, ADD, GELU, CAST, NORMALIZE, LOG_SOFTMAX, SCALAR, MUL_ADD, EXP } tag = NONE;
+  int dtype = 0;                       // element type of the output
+  int src_dtype = 0;                   // CAST: element type of the input
+  uint64_t rows = 0, cols = 0;         // GEMM: M, N; ADD: leading x trailing extent; GELU, CAST: 1 x count
+  const void* in0 = nullptr;           // ADD: a; GELU, CAST: input
+  const void* in1 = nullptr;           // ADD: b
+  int add_form = 0;                    // ADD: 1 = b is a row of `cols` elements repeated over the rows,
+                                       //      2 = a is such a row, 3 = both dense
+  // NORMALIZE (fp32, a wave per row) / LOG_SOFTMAX: rows x cols, in0; sf = eps; lanes of a row's team
+  // SCALAR: out = in0 (op) sf over `cols` elements, op = HC_ADD or HC_MUL as the kernel computes it
+  // MUL_ADD: out = in0 * in1 + in2 with in0 dense [rows, cols] and in1, in2 rows of `cols` elements
+  // EXP: ElemwiseOp.exp over `cols` elements of in0
+  const void* in2 = nullptr;
+  float sf = 0.0f;
+  int op = 0;
+  int lanes = 0;
+  void* out = nullptr;
+  bool dropped = false;                // merged into another entry
+};
+
 struct hc_graph {
   hipGraph_t graph = nullptr;
   hipGraphExec_t exec = nullptr;
   std::unordered_map<size_t, std::vector<void*>> parked;
+  // HCHIP_GRAPH_AS_LAUNCHES=1 at hc_capture_end: the rewritten list, replayed launch by launch
+  // instead of through hipGraphLaunch (for kernel traces: the tracer of this ROCm release aborts
+  // inside hipGraphLaunch)
+  std::vector<hc_pending> launches;
 };
 
 struct hc_ctx {
@@ -75,6 +118,8 @@ struct hc_ctx {
   hipEvent_t stage_ev[2] = {nullptr, nullptr};
   bool stage_busy[2] = {false, false};
   std::vector<hipEvent_t> wait_events;  // spare events of blocking transfers (waited for outside the mutex)
+  bool lazy = false;                    // a capture that lists its launches (see hc_pending)
+  std::vector<hc_pending> pending;
 };
 static const size_t kStageHalf = 2u << 20;    // bytes per half of the staging buffer
 static const size_t kStageMax = 256u << 10;   // largest upload that is staged
@@ -256,8 +301,11 @@ extern "C" int hc_malloc(hc_ctx* ctx, size_t bytes, void** out) {
   std::lock_guard<std::mutex> lock(ctx->mu);
   auto it = ctx->free_blocks.find(b);
   void* p = nullptr;
-  if (ctx->capturing) {
-    // blocks this recording already owns come first; anything else it takes becomes its own
+  if (ctx->capturing && !ctx->lazy) {
+    // blocks this recording already owns come first; anything else it takes becomes its own.
+    // (Not while the recording lists its launches for rewriting: there every buffer stays a
+    // buffer of its own until the recording ends, so that an operation can be moved next to its
+    // consumer without running into a block that was handed out again in between.)
     auto& parked = ctx->capturing->parked[b];
     if (!parked.empty()) {
       p = parked.back();
@@ -303,6 +351,13 @@ extern "C" int hc_free(hc_ctx* ctx, void* ptr) {
   const size_t b = it->second;
   ctx->live.erase(it);
   ctx->bytes_in_use -= b;
+  if (ctx->lazy) {   // from here on nobody reads this buffer: what the rewrite of the recording looks for
+    hc_pending e;
+    e.kind = hc_pending::FREE;
+    e.dst = ptr;
+    e.bytes = b;
+    ctx->pending.push_back(std::move(e));
+  }
   auto owner = ctx->block_owner.find(ptr);
   if (owner != ctx->block_owner.end()) {
     // recorded kernels keep using this block on every replay
@@ -410,6 +465,18 @@ static int copy(hc_ctx* ctx, void* dst, const void* src, size_t bytes, hipMemcpy
       return HC_OK;
     }
     if (!wait) {
+      if (ctx->lazy) {   // (only device-to-device copies get here while capturing)
+        hc_pending e;
+        e.kind = hc_pending::COPY_D2D;
+        e.dst = dst;
+        e.src = src;
+        e.bytes = bytes;
+        e.known = true;
+        e.reads = {src};
+        e.writes = {dst};
+        ctx->pending.push_back(std::move(e));
+        return HC_OK;
+      }
       HIP_TRY(hipMemcpyAsync(dst, src, bytes, kind, ctx->stream));
       return HC_OK;
     }
@@ -524,6 +591,32 @@ extern "C" int hc_capture_begin(hc_ctx* ctx) {
   HIP_TRY(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed));
   ctx->capturing = new hc_graph();
   ctx->graphs.push_back(ctx->capturing);
+  // HCHIP_NO_FUSION=1: launches go to the capturing stream one by one, as issued
+  ctx->lazy = getenv("HCHIP_NO_FUSION") == nullptr;
+  ctx->pending.clear();
+  return HC_OK;
+}
+
+static void fuse_recording(hc_ctx* ctx);
+static int launch_fn(hc_ctx* ctx, hipFunction_t fn, uint32_t gx, uint32_t gy, uint32_t gz, uint32_t bx,
+                     uint32_t shared, const void* kernarg, size_t kernarg_bytes);
+
+// Enqueues the (rewritten) list of a recording on the capturing stream. Caller holds the lock.
+static int emit_recording_locked(hc_ctx* ctx, std::vector<hc_pending>& list) {
+  for (hc_pending& e : list) {
+    if (e.dropped) continue;
+    if (e.kind == hc_pending::KERNEL) {
+      HC_TRY(launch_fn(ctx, e.fn, e.grid[0], e.grid[1], 1, HCK_BLOCK, 0, e.args.data(), e.args.size()));
+    } else if (e.kind == hc_pending::RAW_KERNEL) {
+      size_t n = e.args.size();
+      void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, e.args.data(), HIP_LAUNCH_PARAM_BUFFER_SIZE, &n,
+                        HIP_LAUNCH_PARAM_END};
+      HIP_TRY(hipModuleLaunchKernel(e.fn, e.grid[0], e.grid[1], e.grid[2], e.block[0], e.block[1], e.block[2],
+                                    e.shared, ctx->stream, nullptr, config));
+    } else if (e.kind == hc_pending::COPY_D2D) {
+      HIP_TRY(hipMemcpyAsync(e.dst, e.src, e.bytes, hipMemcpyDeviceToDevice, ctx->stream));
+    }
+  }
   return HC_OK;
 }
 
@@ -549,8 +642,27 @@ static int end_capture(hc_ctx* ctx, hc_graph** out) {
   std::lock_guard<std::mutex> lock(ctx->mu);
   REQUIRE(ctx->capturing, "hc_capture_end: no capture in progress");
   hc_graph* g = ctx->capturing;
+  int emitted = HC_OK;
+  if (ctx->lazy) {
+    ctx->lazy = false;
+    if (out) {
+      fuse_recording(ctx);
+      emitted = emit_recording_locked(ctx, ctx->pending);
+      if (getenv("HCHIP_GRAPH_AS_LAUNCHES"))
+        for (hc_pending& e : ctx->pending)
+          if (!e.dropped && e.kind != hc_pending::FREE) g->launches.push_back(e);
+    }
+    ctx->pending.clear();
+  }
   ctx->capturing = nullptr;
   hipError_t e = hipStreamEndCapture(ctx->stream, &g->graph);
+  if (emitted != HC_OK) {
+    (void)hipGetLastError();
+    if (g->graph) (void)hipGraphDestroy(g->graph);
+    release_graph_blocks_locked(ctx, g);
+    delete g;
+    return emitted;
+  }
   if (e == hipSuccess && out) e = hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0);
   if (e != hipSuccess || !out) {
     (void)hipGetLastError();
@@ -580,7 +692,14 @@ extern "C" int hc_graph_launch(hc_ctx* ctx, hc_graph* graph) {
   REQUIRE(ctx && graph && graph->exec, "hc_graph_launch: null argument");
   std::lock_guard<std::mutex> lock(ctx->mu);
   REQUIRE(!ctx->capturing, "hc_graph_launch: not allowed while capturing");
+  if (!graph->launches.empty()) return emit_recording_locked(ctx, graph->launches);
   HIP_TRY(hipGraphLaunch(graph->exec, ctx->stream));
+  return HC_OK;
+}
+
+extern "C" int hc_graph_node_count(hc_graph* graph, size_t* out) {
+  REQUIRE(graph && graph->graph && out, "hc_graph_node_count: null argument");
+  HIP_TRY(hipGraphGetNodes(graph->graph, nullptr, out));
   return HC_OK;
 }
 
@@ -596,6 +715,149 @@ extern "C" int hc_graph_destroy(hc_ctx* ctx, hc_graph* graph) {
   release_graph_blocks_locked(ctx, graph);
   delete graph;
   return HC_OK;
+}
+
+// ------------------------------------------------------------------ rewriting a recording
+
+// ---- rewrite of a recording before it is enqueued ----
+//
+// Inside a recording every buffer has an address of its own (released blocks are not handed out
+// again until the recording ends), entry points declare what they read and write, and a release
+// says that nobody reads a buffer afterwards. That is enough to see, without any knowledge of the
+// caller's program, that the result of a product has exactly one reader, and to let the product's
+// kernel do that reader's work on the tile it is about to store:
+//     matmul -> + bias row -> GELU          (Linear followed by an activation)
+//     matmul -> + bias row -> + residual    (Linear inside a residual connection)
+// (up to three operations, one of them with a matrix operand) with the bias row possibly cast
+// from fp32 on the way. The merged operations are applied with
+// the arithmetic of the kernels they replace (each one on the value rounded to the output type),
+// so a replay produces the bits the unmerged sequence produces. HCHIP_NO_FUSION=1 at
+// hc_capture_begin turns the rewrite off.
+
+static bool aligned16(const void* p);
+static bool in_block(const void* p, const void* base, size_t bytes) {
+  return (const char*)p >= (const char*)base && (const char*)p < (const char*)base + bytes;
+}
+static bool touches(const std::vector<const void*>& v, const void* base, size_t bytes) {
+  for (const void* p : v)
+    if (p && in_block(p, base, bytes)) return true;
+  return false;
+}
+
+// The only entry after `from` that reads or writes the block at `base`, which is released at
+// entry `free_at`: its index, or -1 if there are several, none, or a launch in between whose
+// buffers are not declared.
+static long sole_user(const std::vector<hc_pending>& list, size_t from, const void* base, size_t bytes, size_t free_at) {
+  long user = -1;
+  for (size_t k = from + 1; k < free_at; k++) {
+    const hc_pending& e = list[k];
+    if (e.dropped || e.kind == hc_pending::FREE) continue;
+    if (!e.known) return -1;
+    if (touches(e.reads, base, bytes) || touches(e.writes, base, bytes)) {
+      if (user >= 0) return -1;
+      user = (long)k;
+    }
+  }
+  return user;
+}
+
+static void fuse_recording(hc_ctx* ctx) {
+  std::vector<hc_pending>& list = ctx->pending;
+  struct Freed { size_t at, bytes; };
+  std::unordered_map<const void*, Freed> freed;
+  for (size_t i = 0; i < list.size(); i++)
+    if (list[i].kind == hc_pending::FREE) freed[list[i].dst] = Freed{i, list[i].bytes};
+
+  for (size_t i = 0; i < list.size(); i++) {
+    if (list[i].kind != hc_pending::KERNEL || list[i].dropped || list[i].tag != hc_pending::GEMM) continue;
+    if (list[i].args.size() != sizeof(hck_gemm_args)) continue;
+    hck_gemm_args g;
+    memcpy(&g, list[i].args.data(), sizeof(g));
+    const int dtype = list[i].dtype;
+    const uint64_t M = list[i].rows, N = list[i].cols;
+    std::vector<const void*> inputs = {g.a, g.b};   // what the merged kernel reads
+    std::vector<size_t> merged;                      // entries whose work it takes over
+    const void* cur = list[i].out;
+    size_t pos = i;
+    int nops = 0;
+    while (nops < 3) {
+      auto fr = freed.find(cur);
+      if (fr == freed.end() || fr->second.at <= pos) break;
+      const long j = sole_user(list, pos, cur, fr->second.bytes, fr->second.at);
+      if (j < 0) break;
+      const hc_pending& c = list[(size_t)j];
+      if (c.kind != hc_pending::KERNEL || c.dtype != dtype || !c.out || !aligned16(c.out)) break;
+      uint32_t kind = HCK_EP_NONE;
+      const void* other = nullptr;
+      if (c.tag == hc_pending::GELU && c.in0 == cur && c.cols == M * N) {
+        kind = HCK_EP_GELU;
+      } else if (c.tag == hc_pending::ADD && (c.in0 == cur) != (c.in1 == cur)) {
+        const bool first = c.in0 == cur;
+        other = first ? c.in1 : c.in0;
+        if (c.add_form == 3 && c.rows * c.cols == M * N) kind = HCK_EP_ADD_MATRIX;
+        if (c.add_form == (first ? 1 : 2) && c.rows == M && c.cols == N) kind = HCK_EP_ADD_ROW;
+        if (!aligned16(other)) kind = HCK_EP_NONE;
+        // (the kernels fetch one matrix operand per output piece)
+        if (kind == HCK_EP_ADD_MATRIX)
+          for (int s = 0; s < nops; s++)
+            if (g.ep_kind[s] == HCK_EP_ADD_MATRIX) kind = HCK_EP_NONE;
+      }
+      if (kind == HCK_EP_NONE) break;
+      // the product moves to its reader's place: nothing in between may write what it reads
+      bool clean = true;
+      for (size_t k2 = pos + 1; k2 < (size_t)j && clean; k2++) {
+        const hc_pending& e = list[k2];
+        if (e.dropped || e.kind == hc_pending::FREE) continue;
+        for (const void* in : inputs)
+          for (const void* w : e.writes)
+            if (w == in) clean = false;
+      }
+      if (!clean) break;
+      g.ep_kind[nops] = kind;
+      g.ep_ptr[nops] = other;
+      g.ep_ld[nops] = (uint32_t)N;
+      if (other) inputs.push_back(other);
+      merged.push_back((size_t)j);
+      cur = c.out;
+      pos = (size_t)j;
+      nops++;
+    }
+    if (nops == 0) continue;
+    // a bias row that is an fp32 parameter cast to fp16 just for this addition: read the fp32 row
+    if (dtype == HC_F16)
+      for (int s = 0; s < nops; s++) {
+        if (g.ep_kind[s] != HCK_EP_ADD_ROW) continue;
+        auto fr = freed.find(g.ep_ptr[s]);
+        if (fr == freed.end()) continue;
+        for (size_t c2 = 0; c2 < merged[(size_t)s]; c2++) {
+          hc_pending& e = list[c2];
+          if (e.dropped || e.kind != hc_pending::KERNEL || e.tag != hc_pending::CAST || e.out != g.ep_ptr[s]) continue;
+          if (e.src_dtype != HC_F32 || e.dtype != HC_F16 || e.cols != N || !aligned16(e.in0)) break;
+          if (sole_user(list, c2, e.out, fr->second.bytes, fr->second.at) != (long)merged[(size_t)s]) break;
+          bool clean = true;   // the fp32 row must still hold the same values where the product now runs
+          for (size_t k2 = c2 + 1; k2 < pos && clean; k2++)
+            for (const void* w : list[k2].writes)
+              if (!list[k2].dropped && w == e.in0) clean = false;
+          if (!clean) break;
+          for (const void*& in : inputs)
+            if (in == g.ep_ptr[s]) in = e.in0;
+          g.ep_kind[s] = HCK_EP_ADD_ROW_F32;
+          g.ep_ptr[s] = e.in0;
+          e.dropped = true;
+          break;
+        }
+      }
+    g.c = const_cast<void*>(cur);
+    hc_pending fused = list[i];
+    memcpy(fused.args.data(), &g, sizeof(g));
+    fused.tag = hc_pending::NONE;
+    fused.reads = inputs;
+    fused.writes = {cur};
+    fused.out = const_cast<void*>(cur);
+    for (size_t m : merged) list[m].dropped = true;
+    list[i].dropped = true;
+    list[pos] = std::move(fused);   // (not dropped: copied from the product's entry before that was marked)
+  }
 }
 
 // ------------------------------------------------------------------ raw module API
@@ -629,6 +891,58 @@ extern "C" int hc_module_get_function(hc_module* mod, const char* name, hc_funct
   return HC_OK;
 }
 
+// Declared by an entry point for the duration of its launches: the caller-visible buffers the
+// operation reads and writes (scratch memory the entry point takes from the pool is its own
+// business). Nests: an entry point that calls another one is covered by the inner declaration
+// while that one runs.
+struct OpNote {
+  std::vector<const void*> reads, writes;
+  hc_pending::Tag tag = hc_pending::NONE;
+  hc_pending meta;    // tag fields for the next launch only (consumed by it)
+  OpNote* outer;
+  static thread_local OpNote* current;
+  OpNote(std::initializer_list<const void*> r, std::initializer_list<const void*> w) : reads(r), writes(w), outer(current) {
+    current = this;
+  }
+  ~OpNote() { current = outer; }
+  OpNote(const OpNote&) = delete;
+  OpNote& operator=(const OpNote&) = delete;
+};
+thread_local OpNote* OpNote::current = nullptr;
+
+// Adds a launch to the recording in progress (caller holds the mutex).
+static void record_launch_locked(hc_ctx* ctx, hipFunction_t fn, uint32_t gx, uint32_t gy, const void* args,
+                                 size_t bytes) {
+  hc_pending e;
+  e.kind = hc_pending::KERNEL;
+  e.fn = fn;
+  e.grid[0] = gx;
+  e.grid[1] = gy;
+  e.args.assign((const char*)args, (const char*)args + bytes);
+  if (OpNote* n = OpNote::current) {
+    e.known = true;
+    e.reads = n->reads;
+    e.writes = n->writes;
+    if (n->tag != hc_pending::NONE) {   // the tag describes exactly one launch: the next one
+      e.tag = n->tag;
+      e.dtype = n->meta.dtype;
+      e.src_dtype = n->meta.src_dtype;
+      e.rows = n->meta.rows;
+      e.cols = n->meta.cols;
+      e.in0 = n->meta.in0;
+      e.in1 = n->meta.in1;
+      e.add_form = n->meta.add_form;
+      e.in2 = n->meta.in2;
+      e.sf = n->meta.sf;
+      e.op = n->meta.op;
+      e.lanes = n->meta.lanes;
+      e.out = n->meta.out;
+      n->tag = hc_pending::NONE;
+    }
+  }
+  ctx->pending.push_back(std::move(e));
+}
+
 static int launch_fn(hc_ctx* ctx, hipFunction_t fn, uint32_t gx, uint32_t gy, uint32_t gz, uint32_t bx,
                      uint32_t shared, const void* kernarg, size_t kernarg_bytes) {
   // every built-in kernel takes one struct by value: pass it as the single kernel parameter,
@@ -645,6 +959,16 @@ extern "C" int hc_launch(hc_ctx* ctx, hc_function* fn, const uint32_t grid[3], c
   void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, const_cast<void*>(kernarg),
                     HIP_LAUNCH_PARAM_BUFFER_SIZE, &kernarg_bytes, HIP_LAUNCH_PARAM_END};
   std::lock_guard<std::mutex> lock(ctx->mu);
+  if (ctx->lazy) {   // a caller's own kernel: listed as it is, and nothing is moved across it
+    hc_pending e;
+    e.kind = hc_pending::RAW_KERNEL;
+    e.fn = fn->fn;
+    for (int i = 0; i < 3; i++) e.grid[i] = grid[i], e.block[i] = block[i];
+    e.shared = shared_bytes;
+    e.args.assign((const char*)kernarg, (const char*)kernarg + kernarg_bytes);
+    ctx->pending.push_back(std::move(e));
+    return HC_OK;
+  }
   HIP_TRY(hipModuleLaunchKernel(fn->fn, grid[0], grid[1], grid[2], block[0], block[1], block[2],
                                 shared_bytes, ctx->stream, nullptr, config));
   return HC_OK;
@@ -671,6 +995,10 @@ static int launch(hc_ctx* ctx, const std::string& name, uint64_t blocks_x, uint3
     }
     if (!fn) return fail(HC_ERR_LOAD, "kernel '%s' is not in the embedded code objects", name.c_str());
     ctx->functions[name] = fn;
+  }
+  if (ctx->lazy) {
+    record_launch_locked(ctx, fn, (uint32_t)blocks_x, blocks_y, args, bytes);
+    return HC_OK;
   }
   return launch_fn(ctx, fn, (uint32_t)blocks_x, blocks_y, 1, HCK_BLOCK, 0, args, bytes);
 }
@@ -839,6 +1167,28 @@ extern "C" int hc_binary_op(hc_ctx* ctx, int op, int dtype, const void* a, const
   k.a = a;
   k.b = b;
   k.out = out;
+  OpNote note({a, b}, {out});
+  if (op == HC_ADD && dtype != HC_I64) {
+    // the two forms a recording can merge into the product that made one operand: dense + dense,
+    // and a dense [rows, cols] operand plus a row of `cols` elements repeated over the rows
+    const hck_bcast& d = k.d;
+    int form = 0;
+    if (d.n_outer == 0 && d.inner_stride[0] == 1 && d.inner_stride[1] == 1) form = 3;
+    if (d.n_outer == 1 && d.inner_stride[0] == 1 && d.inner_stride[1] == 1) {
+      if (d.outer_stride[0][0] == d.inner && d.outer_stride[1][0] == 0) form = 1;
+      if (d.outer_stride[0][0] == 0 && d.outer_stride[1][0] == d.inner) form = 2;
+    }
+    if (form != 0) {
+      note.tag = hc_pending::ADD;
+      note.meta.dtype = dtype;
+      note.meta.rows = form == 3 ? 1 : d.outer_shape[0];
+      note.meta.cols = d.inner;
+      note.meta.in0 = a;
+      note.meta.in1 = b;
+      note.meta.add_form = form;
+      note.meta.out = out;
+    }
+  }
   char name[64];
   snprintf(name, sizeof(name), "hc_binary_%s_%s_v%d", kBinaryNames[op], dtype_name(dtype), vec);
   return launch(ctx, name, ceil_div(k.d.total_vecs, HCK_BLOCK), 1, &k, sizeof(k));
@@ -904,6 +1254,19 @@ static int fused3(hc_ctx* ctx, const char* kernel, int dtype, const void* x, con
   k.y = y;
   k.z = z;
   k.out = out;
+  OpNote note({x, y, z}, {out});
+  if (strcmp(kernel, "hc_mul_add") == 0 && dtype != HC_I64 && k.d.n_outer == 1 && k.d.inner_stride[0] == 1 &&
+      k.d.inner_stride[1] == 1 && k.d.inner_stride[2] == 1 && k.d.outer_stride[0][0] == k.d.inner &&
+      k.d.outer_stride[1][0] == 0 && k.d.outer_stride[2][0] == 0) {
+    note.tag = hc_pending::MUL_ADD;
+    note.meta.dtype = dtype;
+    note.meta.rows = k.d.outer_shape[0];
+    note.meta.cols = k.d.inner;
+    note.meta.in0 = x;
+    note.meta.in1 = y;
+    note.meta.in2 = z;
+    note.meta.out = out;
+  }
   char name[64];
   snprintf(name, sizeof(name), "%s_%s_v%d", kernel, tname, vec);
   return launch(ctx, name, ceil_div(k.d.total_vecs, HCK_BLOCK), 1, &k, sizeof(k));
@@ -996,6 +1359,17 @@ extern "C" int hc_binary_op_scalar(hc_ctx* ctx, int op, int dtype, const void* a
     else if (op == HC_SUB) kop = "rsub";
     else if (op == HC_MOD) kop = "rmod";
   }
+  OpNote note({a}, {out});
+  if (dtype != HC_I64 && (strcmp(kop, "add") == 0 || strcmp(kop, "mul") == 0)) {
+    note.tag = hc_pending::SCALAR;
+    note.meta.dtype = dtype;
+    note.meta.op = kop[0] == 'a' ? HC_ADD : HC_MUL;
+    note.meta.sf = k.sf;
+    note.meta.rows = 1;
+    note.meta.cols = count;
+    note.meta.in0 = a;
+    note.meta.out = out;
+  }
   char name[64];
   snprintf(name, sizeof(name), "hc_scalar_%s_%s", kop, dtype_name(dtype));
   return launch_contiguous(ctx, name, count, vec_for_size(dtype_size(dtype)), &k, sizeof(k));
@@ -1035,6 +1409,14 @@ extern "C" int hc_cast(hc_ctx* ctx, const void* in, int in_type, void* out, int 
   k.in = in;
   k.out = out;
   k.count = count;
+  OpNote note({in}, {out});
+  note.tag = hc_pending::CAST;
+  note.meta.dtype = out_type;
+  note.meta.src_dtype = in_type;
+  note.meta.rows = 1;
+  note.meta.cols = count;
+  note.meta.in0 = in;
+  note.meta.out = out;
   char name[64];
   snprintf(name, sizeof(name), "hc_cast_%s_%s", dtype_name(in_type), dtype_name(out_type));
   const int vi = vec_for_size(dtype_size(in_type)), vo = vec_for_size(dtype_size(out_type));
@@ -1091,6 +1473,23 @@ extern "C" int hc_elemwise(hc_ctx* ctx, int op, int dtype, const void* in, const
   k.scales = scales;
   k.out = out;
   k.count = count;
+  OpNote note({in, scales}, {out});
+  if (op == HC_EXP && !scales) {
+    note.tag = hc_pending::EXP;
+    note.meta.dtype = dtype;
+    note.meta.rows = 1;
+    note.meta.cols = count;
+    note.meta.in0 = in;
+    note.meta.out = out;
+  }
+  if (op == HC_GELU_APPROX && !scales) {
+    note.tag = hc_pending::GELU;
+    note.meta.dtype = dtype;
+    note.meta.rows = 1;
+    note.meta.cols = count;
+    note.meta.in0 = in;
+    note.meta.out = out;
+  }
   char name[64];
   snprintf(name, sizeof(name), "hc_elemwise_%s_%s", kElemwiseNames[op], dtype_name(dtype));
   return launch_contiguous(ctx, name, count, vec_for_size(dtype_size(dtype)), &k, sizeof(k));
@@ -1517,15 +1916,28 @@ extern "C" int hc_log_softmax(hc_ctx* ctx, int dtype, const void* in, void* out,
   // (few long rows: a block per row would leave most of the device idle; the column path cuts the
   // axis over many blocks)
   const bool few_long_rows = inner == 1 && (uint64_t)outer < 2 * (uint64_t)ctx->props.multiProcessorCount && reduce >= 32768;
+  OpNote note({in}, {out});
+  auto tag_rows = [&](int lanes) {   // rows held in the registers of a team of `lanes` lanes
+    if (reduce % (int64_t)(16 / el_size) != 0) return;
+    note.tag = hc_pending::LOG_SOFTMAX;
+    note.meta.dtype = dtype;
+    note.meta.rows = (uint64_t)outer;
+    note.meta.cols = (uint64_t)reduce;
+    note.meta.lanes = lanes;
+    note.meta.in0 = in;
+    note.meta.out = out;
+  };
   if (inner == 1 && !few_long_rows) {
     // a lane or 8 lanes per row for short rows, a wave per row while the row fits its registers
     // (4 x 16 bytes per lane), else a block
     if ((uint64_t)reduce * el_size <= 512) {  // (8 lanes x 4 x 16 bytes: the row still fits the team's registers)
       const uint32_t lanes = reduce <= 8 ? 1 : 8;
+      if (lanes == 8) tag_rows(8);
       snprintf(name, sizeof(name), "hc_log_softmax_rows%u_%s", lanes, dtype_name(dtype));
       return launch(ctx, name, ceil_div((uint64_t)outer, HCK_BLOCK / lanes), 1, &k, sizeof(k));
     }
     if ((uint64_t)reduce * el_size <= 64 * 16 * 4) {
+      tag_rows(64);
       snprintf(name, sizeof(name), "hc_log_softmax_rows_%s", dtype_name(dtype));
       return launch(ctx, name, ceil_div((uint64_t)outer, HCK_BLOCK / 64), 1, &k, sizeof(k));
     }
@@ -1589,6 +2001,7 @@ extern "C" int hc_normalize(hc_ctx* ctx, int dtype, const void* in, void* out, i
   // (few long rows: a block per row would leave most of the device idle; the op-by-op composition
   // below runs every step over the whole device, at the price of nine launches)
   const bool few_long_rows = inner == 1 && (uint64_t)outer * 8 < (uint64_t)ctx->props.multiProcessorCount && reduce >= 32768;
+  OpNote note({in}, {out});
   if (inner == 1 && !few_long_rows) {
     hck_reduce_args k;
     memset(&k, 0, sizeof(k));
@@ -1607,6 +2020,15 @@ extern "C" int hc_normalize(hc_ctx* ctx, int dtype, const void* in, void* out, i
       return launch(ctx, name, ceil_div((uint64_t)outer, HCK_BLOCK / lanes), 1, &k, sizeof(k));
     }
     if ((uint64_t)reduce * el_size <= 64 * 16 * 4) {
+      if (dtype == HC_F32 && reduce % 4 == 0) {   // the form a recording can merge a LayerNorm's other steps into
+        note.tag = hc_pending::NORMALIZE;
+        note.meta.dtype = dtype;
+        note.meta.rows = (uint64_t)outer;
+        note.meta.cols = (uint64_t)reduce;
+        note.meta.sf = eps;
+        note.meta.in0 = in;
+        note.meta.out = out;
+      }
       snprintf(name, sizeof(name), "hc_normalize_rows_%s", dtype_name(dtype));
       return launch(ctx, name, ceil_div((uint64_t)outer, HCK_BLOCK / 64), 1, &k, sizeof(k));
     }
@@ -2131,6 +2553,8 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
     return fail(HC_ERR_TOO_LARGE, "hc_matmul: a matrix has more than 2^32-1 elements");
   const size_t el = dtype_size(dtype);
   const uint32_t P = (uint32_t)(16 / el);
+  OpNote note({a, b}, {out});
+  bool whole_call = false;  // the launch in progress computes the whole product (nothing peeled off)
   hck_gemm_args k;
   memset(&k, 0, sizeof(k));
   uint32_t M = (uint32_t)rows, N = (uint32_t)cols, K = (uint32_t)inner;
@@ -2519,6 +2943,16 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
       snprintf(name, sizeof(name), "hc_gemm_%s_%c%c", dtype_name(dtype), ma == 'k' ? 'k' : 'm',
                mb == 'k' ? 'k' : 'n');
     const uint64_t tiles = (uint64_t)k.tiles_m * k.tiles_n;
+    // One launch of a direct-to-LDS kernel that writes the caller's dense [M, N] matrix from the
+    // caller's own operands: a recording may merge what follows into its epilogue.
+    if (whole_call && bm != 0 && dma && batch == 1 && !trans_out && !c_padded && k.a == a && k.b == b && k.c == out &&
+        k.c_rs == N) {
+      note.tag = hc_pending::GEMM;
+      note.meta.dtype = dtype;
+      note.meta.rows = M;
+      note.meta.cols = N;
+      note.meta.out = out;
+    }
     // grid.y carries the batch (at most 65535 per launch)
     for (int64_t b0 = 0; b0 < batch; b0 += 65535) {
       const uint32_t nb = (uint32_t)(batch - b0 < 65535 ? batch - b0 : 65535);
@@ -2560,6 +2994,7 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
       HC_TRY(run(f, fm, Nb));
     }
   } else {
+    whole_call = true;
     HC_TRY(run(k, M, N));
   }
   if (c_padded) {

@@ -98,6 +98,40 @@ typedef struct {
   uint32_t* pidx;
 } hck_reduce_args;
 
+/* Row kernels that a recording's rewrite substitutes for chains of launches (same arithmetic,
+ * intermediate by intermediate). */
+typedef struct {
+  /* [cast to fp32 ->] normalize rows in fp32 [-> x * (gain [+ gain_add]) + bias] [-> cast] */
+  const void* in;
+  void* out;
+  const void* gain; /* `reduce` fp32 elements */
+  const void* bias;
+  uint32_t outer;
+  uint32_t reduce;
+  float eps;
+  float gain_add;
+  uint32_t flags; /* HCK_LN_* */
+  uint32_t pad;
+} hck_layernorm_args;
+#define HCK_LN_AFFINE 1u   /* x * gain + bias follows */
+#define HCK_LN_GAIN_ADD 2u /* ... with gain + gain_add formed first */
+
+typedef struct {
+  /* [x * scale ->] [+ mask ->] logSoftmax over rows [-> exp] */
+  const void* in;
+  void* out;
+  const void* mask; /* [mask_rows, reduce]; row r of the input takes mask row r % mask_rows */
+  uint32_t outer;
+  uint32_t reduce;
+  uint32_t mask_rows;
+  float scale;
+  uint32_t flags; /* HCK_SM_* */
+  uint32_t pad;
+} hck_softmax_chain_args;
+#define HCK_SM_SCALE 1u
+#define HCK_SM_MASK 2u
+#define HCK_SM_EXP 4u
+
 /* Column reduction ([outer, reduce, inner], inner > 1) in up to two passes: the reduce axis is
  * cut into `splits` ranges of `chunk` rows; with splits > 1 each range leaves a partial value
  * (and, for arg-reductions, its index) per column, combined by a second kernel. */
@@ -296,7 +330,19 @@ typedef struct {
   /* edge kernels: rows (K-contiguous operand) or elements of a k-row (M/N-contiguous operand,
    * a multiple of 16 bytes) that may be fetched; anything beyond is clamped to the last one */
   uint32_t a_lim, b_lim;
+  /* Operations applied to the finished tile before it is stored (direct-to-LDS kernels only), in
+   * order, each on the value rounded to the output type, i.e. with the arithmetic of the
+   * separate kernels they replace: what a recording's rewrite merges into the product. */
+  uint32_t ep_kind[3];    /* HCK_EP_* ; 0 ends the list */
+  uint32_t ep_ld[3];      /* HCK_EP_ADD_MATRIX: leading dimension of the matrix, elements */
+  const void* ep_ptr[3];  /* HCK_EP_ADD_ROW: N elements; HCK_EP_ADD_MATRIX: [M, ld] */
 } hck_gemm_args;
+
+#define HCK_EP_NONE 0
+#define HCK_EP_ADD_ROW 1     /* x + row[n]   (a bias broadcast over the rows) */
+#define HCK_EP_ADD_MATRIX 2  /* x + other[m, n] (a residual connection) */
+#define HCK_EP_GELU 3        /* ElemwiseOp.geluApprox */
+#define HCK_EP_ADD_ROW_F32 4 /* x + T(row[n]) with the row held in fp32 (a parameter cast at call time) */
 
 /* Copy of a batch of [rows, in_cols] matrices with leading dimension in_ld into [rows, out_cols]
  * with leading dimension out_ld; columns >= in_cols are written as zero. Element offsets. */

@@ -216,3 +216,133 @@ __device__ __forceinline__ void gemm_tile_of_block(const hck_gemm_args& p, uint3
   tm = tile / p.tiles_n;
   tn = tile - tm * p.tiles_n;
 }
+
+// ---- operations merged into a GEMM's epilogue (hck_gemm_args::ep_*) ----
+#include "elemwise_formulas.hip.h"
+
+// The operations are applied to 16-byte pieces of finished outputs of type T (already rounded to
+// T), in order, each in float with one rounding to T: bit for bit what the separate broadcast-add /
+// element-wise kernels would have produced. A lane's pieces all lie in the same columns, so the row
+// operands (a bias) are fetched once per kernel; the matrix operand (at most one of the three
+// operations) is fetched for a few pieces at a time, all loads in flight before the first use.
+template <typename T, typename Chunk16>
+__device__ __forceinline__ Chunk16 gemm_epilogue_row_piece(uint32_t kind, const void* ptr, uint32_t col, bool col_ok) {
+  constexpr int V = 16 / sizeof(T);
+  static_assert(sizeof(Chunk16) == 16, "a 16-byte piece");
+  Chunk16 out = Chunk16{};
+  if (!col_ok) return out;
+  if (kind == HCK_EP_ADD_ROW) {
+    out = *reinterpret_cast<const Chunk16*>((const T*)ptr + col);
+  } else if (kind == HCK_EP_ADD_ROW_F32) {
+    const float* src = (const float*)ptr + col;
+    T y[V];
+#pragma unroll
+    for (int e = 0; e < V; e += 4) {
+      const float4 w = *reinterpret_cast<const float4*>(src + e);
+      y[e] = narrow<T>(w.x), y[e + 1] = narrow<T>(w.y), y[e + 2] = narrow<T>(w.z), y[e + 3] = narrow<T>(w.w);
+    }
+    __builtin_memcpy(&out, y, 16);
+  }
+  return out;
+}
+
+// the matrix operand's piece for the output piece at (row, col); zeros if there is none
+template <typename T, typename Chunk16>
+__device__ __forceinline__ Chunk16 gemm_epilogue_matrix_piece(const hck_gemm_args& p, uint32_t row, uint32_t col) {
+  Chunk16 m = Chunk16{};
+#pragma unroll
+  for (int s = 0; s < 3; s++)
+    if (p.ep_kind[s] == HCK_EP_ADD_MATRIX)
+      m = *reinterpret_cast<const Chunk16*>((const T*)p.ep_ptr[s] + (size_t)row * p.ep_ld[s] + col);
+  return m;
+}
+
+// r0, r1, r2: the row operands of the three stages (gemm_epilogue_row_piece; passed as three values
+// so that nothing can index them and they stay in registers)
+template <typename T, typename Chunk16>
+__device__ __forceinline__ Chunk16 gemm_epilogue_apply(const hck_gemm_args& p, Chunk16 v, Chunk16 r0, Chunk16 r1, Chunk16 r2,
+                                                       Chunk16 matrix_piece) {
+  constexpr int V = 16 / sizeof(T);
+  T x[V];
+  __builtin_memcpy(x, &v, 16);
+  // One copy of the code for the three stages (the stage's kind and operand are picked with
+  // selects): this function is instantiated for every slab of the tile.
+  const uint32_t k0 = p.ep_kind[0], k1 = p.ep_kind[1], k2 = p.ep_kind[2];
+#pragma nounroll
+  for (int s = 0; s < 3; s++) {
+    const uint32_t kind = s == 0 ? k0 : s == 1 ? k1 : k2;
+    if (kind == HCK_EP_NONE) break;
+    if (kind == HCK_EP_GELU) {
+#pragma unroll
+      for (int e = 0; e < V; e++) x[e] = narrow<T>(gelu_approx<sizeof(T) == 2>((float)x[e]) * 1.0f);
+    } else {
+      Chunk16 w = s == 0 ? r0 : s == 1 ? r1 : r2;
+      if (kind == HCK_EP_ADD_MATRIX) {
+        // The loaded piece is used inside this branch only (the empty asm keeps the compiler from
+        // turning the branch into a select): loads and stores share one in-order counter, and a
+        // wait for this load on the common path would also wait, in every product without a
+        // matrix operand, for all the stores issued so far.
+        w = matrix_piece;
+        asm volatile("" : "+v"(w));
+      }
+      T y[V];
+      __builtin_memcpy(y, &w, 16);
+#pragma unroll
+      for (int e = 0; e < V; e++) x[e] = narrow<T>((float)x[e] + (float)y[e]);
+    }
+  }
+  Chunk16 out;
+  __builtin_memcpy(&out, x, 16);
+  return out;
+}
+
+// Stores GROUP pieces a lane holds of one 32-row slab, with the merged operations: all loads
+// first, then the arithmetic. lds_piece(it) reads piece `it` from the slab; row_of(it), col_of(it)
+// say where it goes in C. COL_FIXED: all of a lane's pieces lie in the same columns and r0, r1, r2
+// are the row operands for them (fetched once per kernel); otherwise they are fetched per piece.
+// `matrix` (wave-uniform): one of the operations has a matrix operand.
+template <typename T, typename Chunk16, bool EDGE, uint32_t GROUP, bool COL_FIXED, typename LdsPiece, typename RowOf, typename ColOf>
+__device__ __forceinline__ void gemm_store_group_merged(const hck_gemm_args& p, bool matrix, Chunk16 r0, Chunk16 r1, Chunk16 r2,
+                                                        T* C, uint32_t it0, LdsPiece lds_piece, RowOf row_of, ColOf col_of) {
+  Chunk16 v[GROUP], m[GROUP], q0[GROUP], q1[GROUP], q2[GROUP];
+#pragma unroll
+  for (uint32_t b = 0; b < GROUP; b++) {
+    const uint32_t row = row_of(it0 + b), col = col_of(it0 + b);
+    const bool inside = !EDGE || (row < p.M && col < p.N);
+    v[b] = lds_piece(it0 + b);
+    m[b] = Chunk16{};
+    q0[b] = COL_FIXED ? r0 : gemm_epilogue_row_piece<T, Chunk16>(p.ep_kind[0], p.ep_ptr[0], col, inside);
+    q1[b] = COL_FIXED ? r1 : gemm_epilogue_row_piece<T, Chunk16>(p.ep_kind[1], p.ep_ptr[1], col, inside);
+    q2[b] = COL_FIXED ? r2 : gemm_epilogue_row_piece<T, Chunk16>(p.ep_kind[2], p.ep_ptr[2], col, inside);
+  }
+  if (matrix) {
+#pragma unroll
+    for (uint32_t b = 0; b < GROUP; b++) {
+      const uint32_t row = row_of(it0 + b), col = col_of(it0 + b);
+      if (!EDGE || (row < p.M && col < p.N)) m[b] = gemm_epilogue_matrix_piece<T, Chunk16>(p, row, col);
+    }
+  }
+#pragma unroll
+  for (uint32_t b = 0; b < GROUP; b++) {
+    const uint32_t row = row_of(it0 + b), col = col_of(it0 + b);
+    if (!EDGE || (row < p.M && col < p.N))
+      *reinterpret_cast<Chunk16*>(C + (size_t)row * p.c_rs + col) = gemm_epilogue_apply<T, Chunk16>(p, v[b], q0[b], q1[b], q2[b], m[b]);
+  }
+}
+
+// The NIT pieces of a slab in groups of at most MAX_GROUP: a loop that is not unrolled (it reads
+// LDS, not the accumulators, and copies of it for every slab would multiply the kernel's code).
+template <typename T, typename Chunk16, bool EDGE, uint32_t NIT, bool COL_FIXED, uint32_t MAX_GROUP, typename LdsPiece,
+          typename RowOf, typename ColOf>
+__device__ __forceinline__ void gemm_store_slab_merged(const hck_gemm_args& p, Chunk16 r0, Chunk16 r1, Chunk16 r2, T* C,
+                                                       LdsPiece lds_piece, RowOf row_of, ColOf col_of) {
+  constexpr uint32_t GROUP = (MAX_GROUP >= 4 && NIT % 4 == 0) ? 4 : (MAX_GROUP >= 3 && NIT % 3 == 0) ? 3 : NIT % 2 == 0 ? 2 : 1;
+  const bool matrix = p.ep_kind[0] == HCK_EP_ADD_MATRIX || p.ep_kind[1] == HCK_EP_ADD_MATRIX || p.ep_kind[2] == HCK_EP_ADD_MATRIX;
+  if constexpr (NIT == GROUP) {
+    gemm_store_group_merged<T, Chunk16, EDGE, GROUP, COL_FIXED>(p, matrix, r0, r1, r2, C, 0u, lds_piece, row_of, col_of);
+  } else {
+#pragma nounroll
+    for (uint32_t it0 = 0; it0 < NIT; it0 += GROUP)
+      gemm_store_group_merged<T, Chunk16, EDGE, GROUP, COL_FIXED>(p, matrix, r0, r1, r2, C, it0, lds_piece, row_of, col_of);
+  }
+}

@@ -346,25 +346,7 @@ DEF_CMP_SCALAR(b8, uint8_t)
 
 // ---------------------------------------------------------------- unary (elemwise)
 
-// Formulas of ElemwiseOp.apply (Elemwise.swift:44-183), same expression trees.
-__device__ __forceinline__ float safe_sigmoid(float x) {
-  if (x < -20.0f) return 0.0f;
-  if (x > 20.0f) return 1.0f;
-  return 1.0f / (1.0f + expf(-x));
-}
-__device__ __forceinline__ float safe_tanh(float x) { return 2.0f * safe_sigmoid(2.0f * x) - 1.0f; }
-
-// The same for results that are rounded to fp16 (11 significant bits): the hardware's exp2 and
-// reciprocal (about 1 ulp of fp32 each) instead of the library's expf and an IEEE division.
-// With the library routines an fp16 GELU is bound by the vector ALU (8 elements per 16-byte
-// load), not by memory.
-__device__ __forceinline__ float exp_hw(float x) { return __builtin_amdgcn_exp2f(x * 1.4426950408889634f); }
-__device__ __forceinline__ float sigmoid_hw(float x) {
-  if (x < -20.0f) return 0.0f;
-  if (x > 20.0f) return 1.0f;
-  return __builtin_amdgcn_rcpf(1.0f + exp_hw(-x));
-}
-__device__ __forceinline__ float tanh_hw(float x) { return 2.0f * sigmoid_hw(2.0f * x) - 1.0f; }
+#include "elemwise_formulas.hip.h"
 
 __device__ __forceinline__ float fast_erf(float a) {
   float r, s, t, u;
@@ -395,14 +377,6 @@ __device__ __forceinline__ float simple_erf_grad(float f) {
   return fabsf(f) > 20.0f ? 0.0f : 1.1283791670955126f * expf(-f * f);
 }
 
-// powf(f, 3.0f) of the reference formula: the cube formed in double and rounded once is the
-// correctly rounded result, which is what a libm powf returns for this exponent, at a
-// fraction of the cost of a general powf.
-__device__ __forceinline__ float cube(float f) {
-  const double d = (double)f;
-  return (float)(d * d * d);
-}
-
 enum {
   E_SIN = 0, E_COS, E_MINUS_SIN, E_TAN, E_TAN_GRAD, E_ATAN, E_ATAN_GRAD, E_ACOS, E_ACOS_GRAD,
   E_ASIN, E_ASIN_GRAD, E_EXP, E_LOG, E_RECIP, E_SIGMOID, E_SIGMOID_GRAD, E_RELU, E_RELU_GRAD,
@@ -415,7 +389,7 @@ template <int OP, bool HALF> __device__ __forceinline__ float elemwise_apply(flo
   if (HALF) {
     if (OP == E_EXP) return exp_hw(f);
     if (OP == E_SIGMOID) return sigmoid_hw(f);
-    if (OP == E_GELU_APPROX) return 0.5f * f * (1.0f + tanh_hw(0.797884561f * (f + 0.044715f * (f * f * f))));
+    if (OP == E_GELU_APPROX) return gelu_approx<true>(f);
   }
   switch (OP) {
     case E_SIN: return sinf(f);
@@ -438,8 +412,7 @@ template <int OP, bool HALF> __device__ __forceinline__ float elemwise_apply(flo
     case E_RELU_GRAD: return f < 0.0f ? 0.0f : 1.0f;
     case E_ABS: return f < 0.0f ? -f : f;
     case E_ABS_GRAD: return f < 0.0f ? -1.0f : 1.0f;
-    case E_GELU_APPROX:
-      return 0.5f * f * (1.0f + safe_tanh(0.797884561f * (f + 0.044715f * cube(f))));
+    case E_GELU_APPROX: return gelu_approx<false>(f);
     case E_GELU_APPROX_GRAD: {
       float tanh_term = tanhf(0.035677408145115f * powf(f, 3.0f) + 0.797884561f * f);
       return 0.5f * f * (1.0f - powf(tanh_term, 2.0f)) *

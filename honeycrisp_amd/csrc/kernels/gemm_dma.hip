@@ -366,6 +366,15 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
   constexpr uint32_t SLAB = 32 * RB, NSLAB = (BM + BN) * 64 / SLAB;
   static_assert(NSLAB >= 1 && UNITS <= 64, "a slab must fit one stage");
   auto unit_swz = [&](uint32_t r) { return (RB >= 256 ? r : r * RB / 256) & (UNITS - 1); };
+  // (operations merged into this product: the lane's columns are the same for all its pieces)
+  const uint32_t ep_col = n0 + wn + (lane % UNITS) * (16 / ES);
+  Chunk ep_r0 = Chunk{}, ep_r1 = Chunk{}, ep_r2 = Chunk{};
+  if (p.ep_kind[0] != HCK_EP_NONE) {
+    const bool ok = !EDGE || ep_col < p.N;
+    ep_r0 = gemm_epilogue_row_piece<T, Chunk>(p.ep_kind[0], p.ep_ptr[0], ep_col, ok);
+    ep_r1 = gemm_epilogue_row_piece<T, Chunk>(p.ep_kind[1], p.ep_ptr[1], ep_col, ok);
+    ep_r2 = gemm_epilogue_row_piece<T, Chunk>(p.ep_kind[2], p.ep_ptr[2], ep_col, ok);
+  }
 #pragma unroll
   for (int i = 0; i < MT; i++) {
     char* slab = mine + (i % NSLAB) * SLAB;
@@ -387,12 +396,24 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
       }
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // wave-private region: no barrier needed
+    // (a merged epilogue is a loop of its own that is not unrolled: it reads LDS, not the
+    // accumulators, and unrolled copies of it would multiply the kernel's code)
+    if (p.ep_kind[0] == HCK_EP_NONE) {
 #pragma unroll
-    for (uint32_t it = 0; it < 32 / RPI; it++) {
-      const uint32_t r = it * RPI + lane / UNITS, u = lane % UNITS;
-      const Chunk v = *reinterpret_cast<const Chunk*>(slab + r * RB + ((u ^ unit_swz(r)) * 16));
-      const uint32_t row = m0 + wm + i * 32 + r, col = n0 + wn + u * (16 / ES);
-      if (!EDGE || (row < p.M && col < p.N)) *reinterpret_cast<Chunk*>(C + (size_t)row * p.c_rs + col) = v;
+      for (uint32_t it = 0; it < 32 / RPI; it++) {
+        const uint32_t r = it * RPI + lane / UNITS, u = lane % UNITS;
+        const Chunk v = *reinterpret_cast<const Chunk*>(slab + r * RB + ((u ^ unit_swz(r)) * 16));
+        const uint32_t row = m0 + wm + i * 32 + r, col = n0 + wn + u * (16 / ES);
+        if (!EDGE || (row < p.M && col < p.N)) *reinterpret_cast<Chunk*>(C + (size_t)row * p.c_rs + col) = v;
+      }
+    } else {
+      gemm_store_slab_merged<T, Chunk, EDGE, 32 / RPI, true, 4>(
+          p, ep_r0, ep_r1, ep_r2, C,
+          [=](uint32_t it) {
+            const uint32_t r = it * RPI + lane / UNITS, u = lane % UNITS;
+            return *reinterpret_cast<const Chunk*>(slab + r * RB + ((u ^ unit_swz(r)) * 16));
+          },
+          [=](uint32_t it) { return m0 + wm + i * 32 + it * RPI + lane / UNITS; }, [=](uint32_t) { return ep_col; });
     }
     asm volatile("" ::: "memory");
   }

@@ -377,6 +377,17 @@ __device__ __forceinline__ void gemm_dma2_impl(const hck_gemm_args& p, char* lds
   constexpr uint32_t USWZ = (UNITS & (UNITS - 1)) == 0 ? UNITS - 1 : (UNITS % 8 == 0 ? 7 : 3);
   static_assert(UNITS % (USWZ + 1) == 0, "unsupported tile width");
   auto unit_swz = [&](uint32_t r) { return (RB >= 256 ? r : r * RB / 256) & USWZ; };
+  // (operations merged into this product: if 64 lanes are whole rows of units, a lane's columns
+  // are the same for all its pieces and the row operands are fetched once)
+  constexpr bool EP_COL_FIXED = 64 % UNITS == 0;
+  const uint32_t ep_col = n0 + wn + (lane % UNITS) * (16 / ES);
+  Chunk ep_r0 = Chunk{}, ep_r1 = Chunk{}, ep_r2 = Chunk{};
+  if (EP_COL_FIXED && p.ep_kind[0] != HCK_EP_NONE) {
+    const bool ok = !EDGE || ep_col < p.N;
+    ep_r0 = gemm_epilogue_row_piece<T, Chunk>(p.ep_kind[0], p.ep_ptr[0], ep_col, ok);
+    ep_r1 = gemm_epilogue_row_piece<T, Chunk>(p.ep_kind[1], p.ep_ptr[1], ep_col, ok);
+    ep_r2 = gemm_epilogue_row_piece<T, Chunk>(p.ep_kind[2], p.ep_ptr[2], ep_col, ok);
+  }
 #pragma unroll
   for (int i = 0; i < MT; i++) {
     char* slab = mine + (i % NSLAB) * SLAB;
@@ -398,12 +409,25 @@ __device__ __forceinline__ void gemm_dma2_impl(const hck_gemm_args& p, char* lds
       }
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // wave-private region: no barrier needed
+    // (a merged epilogue is a loop of its own that is not unrolled: it reads LDS, not the
+    // accumulators, and unrolled copies of it would multiply the kernel's code)
+    if (p.ep_kind[0] == HCK_EP_NONE) {
 #pragma unroll
-    for (uint32_t it = 0; it < 32 * UNITS / 64; it++) {
-      const uint32_t piece = it * 64 + lane, r = piece / UNITS, u = piece % UNITS;
-      const Chunk v = *reinterpret_cast<const Chunk*>(slab + r * RB + ((u ^ unit_swz(r)) * 16));
-      const uint32_t row = m0 + wm + i * 32 + r, col = n0 + wn + u * (16 / ES);
-      if (!EDGE || (row < p.M && col < p.N)) *reinterpret_cast<Chunk*>(C + (size_t)row * p.c_rs + col) = v;
+      for (uint32_t it = 0; it < 32 * UNITS / 64; it++) {
+        const uint32_t piece = it * 64 + lane, r = piece / UNITS, u = piece % UNITS;
+        const Chunk v = *reinterpret_cast<const Chunk*>(slab + r * RB + ((u ^ unit_swz(r)) * 16));
+        const uint32_t row = m0 + wm + i * 32 + r, col = n0 + wn + u * (16 / ES);
+        if (!EDGE || (row < p.M && col < p.N)) *reinterpret_cast<Chunk*>(C + (size_t)row * p.c_rs + col) = v;
+      }
+    } else {
+      gemm_store_slab_merged<T, Chunk, EDGE, 32 * UNITS / 64, EP_COL_FIXED, 4>(
+          p, ep_r0, ep_r1, ep_r2, C,
+          [=](uint32_t it) {
+            const uint32_t piece = it * 64 + lane, r = piece / UNITS, u = piece % UNITS;
+            return *reinterpret_cast<const Chunk*>(slab + r * RB + ((u ^ unit_swz(r)) * 16));
+          },
+          [=](uint32_t it) { return m0 + wm + i * 32 + (it * 64 + lane) / UNITS; },
+          [=](uint32_t it) { return n0 + wn + ((it * 64 + lane) % UNITS) * (16 / ES); });
     }
     asm volatile("" ::: "memory");
   }

@@ -581,6 +581,55 @@ HC_KERNEL void hc_log_softmax_rows8_f16(hck_reduce_args p) { log_softmax_rows_im
 HC_KERNEL void hc_log_softmax_rows256_f32(hck_reduce_args p) { log_softmax_rows_impl<float, 256>(p); }
 HC_KERNEL void hc_log_softmax_rows256_f16(hck_reduce_args p) { log_softmax_rows_impl<half_t, 256>(p); }
 
+// The chain [x * scale] [+ mask] -> logSoftmax [-> exp] (an attention softmax as a Honeycrisp
+// model writes it) in one pass over rows that fit the team's registers: the arithmetic of the
+// separate kernels, with every intermediate rounded to T where they would have stored it.
+template <typename T, int LANES> __device__ __forceinline__ void softmax_chain_rows_impl(const hck_softmax_chain_args& p) {
+  __shared__ float lds[HCK_BLOCK / 64];
+  const uint32_t lane = Team<LANES>::lane(), row = Team<LANES>::row();
+  if (row >= p.outer) return;
+  const uint32_t n = p.reduce;
+  constexpr int VEC = RowRegs<T, LANES>::VEC, CHUNKS = RowRegs<T, LANES>::CHUNKS;
+  RowRegs<T, LANES> r;
+  r.load((const T*)p.in + (size_t)row * n, n, lane);
+  if (p.flags & HCK_SM_SCALE) {
+    const float s = p.scale;
+#pragma unroll
+    for (int c = 0; c < CHUNKS; c++)
+#pragma unroll
+      for (int i = 0; i < VEC; i++) r.v[c][i] = narrow<T>((float)r.v[c][i] * s);
+  }
+  if (p.flags & HCK_SM_MASK) {
+    RowRegs<T, LANES> m;
+    m.load((const T*)p.mask + (size_t)(row % p.mask_rows) * n, n, lane);
+#pragma unroll
+    for (int c = 0; c < CHUNKS; c++)
+      if ((lane + LANES * c) * VEC < n) {
+#pragma unroll
+        for (int i = 0; i < VEC; i++) r.v[c][i] = narrow<T>((float)r.v[c][i] + (float)m.v[c][i]);
+      }
+  }
+  float mx = -INFINITY;
+  r.each(n, lane, [&](float x) { if (x > mx) mx = x; });
+  mx = Team<LANES>::reduce(mx, MaxOp(), lds);
+  float s = 0.0f;
+  r.each(n, lane, [&](float x) { s += expf(x - mx); });
+  s = Team<LANES>::reduce(s, SumOp(), lds);
+  const float log_sum = logf(s) + mx;
+  const bool then_exp = (p.flags & HCK_SM_EXP) != 0;
+  r.store((T*)p.out + (size_t)row * n, n, lane, [&](float x) {
+    const float ls = x - log_sum;
+    if (!then_exp) return ls;
+    // ElemwiseOp.exp on the stored log-probability (fp16: the hardware exponential, as the element-wise kernel)
+    const float stored = (float)narrow<T>(ls);
+    return (sizeof(T) == 2 ? exp_hw(stored) : expf(stored)) * 1.0f;
+  });
+}
+HC_KERNEL void hc_softmax_chain_rows_f32(hck_softmax_chain_args p) { softmax_chain_rows_impl<float, 64>(p); }
+HC_KERNEL void hc_softmax_chain_rows8_f32(hck_softmax_chain_args p) { softmax_chain_rows_impl<float, 8>(p); }
+HC_KERNEL void hc_softmax_chain_rows_f16(hck_softmax_chain_args p) { softmax_chain_rows_impl<half_t, 64>(p); }
+HC_KERNEL void hc_softmax_chain_rows8_f16(hck_softmax_chain_args p) { softmax_chain_rows_impl<half_t, 8>(p); }
+
 // logSoftmaxGrad (BackendCPU.swift:1040-1085): g - sum(g) * expf(x - (logf(sum exp(x - max)) + max)).
 template <typename T, int LANES>
 __device__ __forceinline__ void log_softmax_grad_rows_impl(const hck_reduce_args& p) {
@@ -682,3 +731,77 @@ HC_KERNEL void hc_normalize_rows1_f16(hck_reduce_args p) { normalize_rows_impl<h
 HC_KERNEL void hc_normalize_rows8_f16(hck_reduce_args p) { normalize_rows_impl<half_t, 8>(p); }
 HC_KERNEL void hc_normalize_rows256_f32(hck_reduce_args p) { normalize_rows_impl<float, 256>(p); }
 HC_KERNEL void hc_normalize_rows256_f16(hck_reduce_args p) { normalize_rows_impl<half_t, 256>(p); }
+
+// The chain [cast to fp32] -> normalize (fp32, a wave per row) [-> x * (gain [+ c]) + bias] [-> cast]
+// (a LayerNorm as Trainable.swift:787-829 issues it) in one pass. Elements are spread over the
+// lanes as the fp32 normalize kernel spreads them (lane l: the 4-element groups l, l + 64, ...) and
+// summed in its order, so the row statistics have the same bits; the affine part is mulAdd's
+// x * c + b and the scalar kernel's gain + c.
+template <typename TI, typename TO> __device__ __forceinline__ void layernorm_rows_impl(const hck_layernorm_args& p) {
+  constexpr int VEC = 4, CHUNKS = 4, LANES = 64;
+  const uint32_t lane = Team<LANES>::lane(), row = Team<LANES>::row();
+  if (row >= p.outer) return;
+  const uint32_t n = p.reduce;
+  const TI* in = (const TI*)p.in + (size_t)row * n;
+  TO* out = (TO*)p.out + (size_t)row * n;
+  float v[CHUNKS][VEC];
+#pragma unroll
+  for (int c = 0; c < CHUNKS; c++) {
+    const uint32_t k = (lane + LANES * c) * VEC;
+    if (k < n) {
+      TI a[VEC];
+      load_vec<TI, VEC>(in, k, 1, a);
+#pragma unroll
+      for (int i = 0; i < VEC; i++) v[c][i] = (float)a[i];
+    }
+  }
+  auto each = [&](auto f) {
+#pragma unroll
+    for (int c = 0; c < CHUNKS; c++)
+      if ((lane + LANES * c) * VEC < n) {
+#pragma unroll
+        for (int i = 0; i < VEC; i++) f(v[c][i]);
+      }
+  };
+  const float inv_n = 1.0f / (float)n;
+  float s = 0.0f;
+  each([&](float x) { s += x; });
+  s = Team<LANES>::reduce(s, SumOp(), nullptr);
+  const float mean = s * inv_n;
+  float sq = 0.0f;
+  each([&](float x) {
+    const float d = x - mean;
+    sq += d * d;
+  });
+  sq = Team<LANES>::reduce(sq, SumOp(), nullptr);
+  const float var = sq * inv_n;
+  const float shifted = var + p.eps;
+  const float normer = 1.0f * 1.0f * pow_like(shifted, -0.5f);
+  const bool affine = (p.flags & HCK_LN_AFFINE) != 0, gain_add = (p.flags & HCK_LN_GAIN_ADD) != 0;
+#pragma unroll
+  for (int c = 0; c < CHUNKS; c++) {
+    const uint32_t k = (lane + LANES * c) * VEC;
+    if (k < n) {
+      float g[VEC] = {1.0f, 1.0f, 1.0f, 1.0f}, b[VEC] = {0.0f, 0.0f, 0.0f, 0.0f};
+      if (affine) {
+        load_vec<float, VEC>((const float*)p.gain, k, 1, g);
+        load_vec<float, VEC>((const float*)p.bias, k, 1, b);
+      }
+      TO o[VEC];
+#pragma unroll
+      for (int i = 0; i < VEC; i++) {
+        float y = (v[c][i] - mean) * normer;
+        if (affine) {
+          const float coeff = gain_add ? g[i] + p.gain_add : g[i];
+          y = y * coeff + b[i];
+        }
+        o[i] = narrow<TO>(y);
+      }
+      store_vec<TO, VEC>(out, k, o);
+    }
+  }
+}
+HC_KERNEL void hc_layernorm_rows_f32_f32(hck_layernorm_args p) { layernorm_rows_impl<float, float>(p); }
+HC_KERNEL void hc_layernorm_rows_f16_f32(hck_layernorm_args p) { layernorm_rows_impl<half_t, float>(p); }
+HC_KERNEL void hc_layernorm_rows_f32_f16(hck_layernorm_args p) { layernorm_rows_impl<float, half_t>(p); }
+HC_KERNEL void hc_layernorm_rows_f16_f16(hck_layernorm_args p) { layernorm_rows_impl<half_t, half_t>(p); }

@@ -150,13 +150,22 @@ int hc_launch_host_func(hc_ctx* ctx, void (*fn)(void*), void* user);
  *    kept alive by the caller for as long as the graph is replayed; results are read from
  *    the buffers the captured ops returned.
  *  - Host transfers, hc_sync, event and host-function calls are refused while capturing
- *    (HC_ERR_INVALID). One capture at a time per context. */
+ *    (HC_ERR_INVALID). One capture at a time per context.
+ *  - The launches of a capture are listed first and enqueued at hc_capture_end, after a
+ *    rewrite that merges the single reader of a product's result into the product's kernel
+ *    (matmul -> + bias row -> geluApprox, matmul -> + bias row -> + other matrix; the row may
+ *    be an fp32 buffer cast to fp16 for the addition). The merged kernel applies each
+ *    operation to the value rounded to the output type, so a replay returns the bits of the
+ *    unmerged sequence. Intermediate buffers that were merged away are never written.
+ *    HCHIP_NO_FUSION=1 in the environment at hc_capture_begin turns the rewrite off. */
 typedef struct hc_graph hc_graph;
 int hc_capture_begin(hc_ctx* ctx);
 int hc_capture_end(hc_ctx* ctx, hc_graph** out);
 /* Ends a capture and throws the recording away (error paths). */
 int hc_capture_abort(hc_ctx* ctx);
 int hc_graph_launch(hc_ctx* ctx, hc_graph* graph);
+/* Number of nodes (kernel launches and copies) one replay of the graph issues. */
+int hc_graph_node_count(hc_graph* graph, size_t* out);
 int hc_graph_destroy(hc_ctx* ctx, hc_graph* graph);
 
 /* ---- raw module API (thin wrappers over hipModuleLoadData / hipModuleGetFunction /

@@ -1,0 +1,164 @@
+"""The rewrite of a recording (hc_capture_end): a product whose result has exactly one reader takes
+that reader's work into its own kernel. A replay must return the bits the same ops return when
+issued one by one, the rewrite must actually remove launches where it applies, and it must leave
+the recording alone where a merged intermediate would be missed (a second reader, a result the
+caller still holds)."""
+import numpy as np
+import pytest
+
+from honeycrisp_amd.descriptors import DType
+from honeycrisp_amd.nn import Linear, Transformer
+from honeycrisp_amd.tensor import Tensor
+
+pytestmark = pytest.mark.gpu
+
+NP = {DType.float32: np.float32, DType.float16: np.float16}
+
+
+def record(backend, fn, fusion=True, monkeypatch=None):
+    """Records fn() and returns (graph, output tensor, node count)."""
+    if not fusion:
+        monkeypatch.setenv("HCHIP_NO_FUSION", "1")
+    try:
+        with backend.capture() as cap:
+            out = fn()
+    finally:
+        if not fusion:
+            monkeypatch.delenv("HCHIP_NO_FUSION")
+    return cap.graph, out, cap.graph.node_count()
+
+
+def check(backend, monkeypatch, fn, removed):
+    """fn() recorded with and without the rewrite and issued eagerly: same bits from all three;
+    the rewrite removes exactly `removed` launches."""
+    want = fn().numpy().copy()
+    plain, plain_out, plain_nodes = record(backend, fn, fusion=False, monkeypatch=monkeypatch)
+    fused, fused_out, fused_nodes = record(backend, fn)
+    for replay in range(2):
+        plain.launch()
+        fused.launch()
+        assert np.array_equal(plain_out.numpy(), want)
+        got = fused_out.numpy()
+        assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), \
+            "replay %d: %d of %d elements differ" % (replay, int((got != want).sum()), want.size)
+    assert plain_nodes - fused_nodes == removed, (plain_nodes, fused_nodes)
+    plain.destroy()
+    fused.destroy()
+
+
+def operands(rng, dtype, m, k, n):
+    x = Tensor(data=rng.standard_normal((m, k)).astype(np.float32), dtype=dtype)
+    w = Tensor(data=(rng.standard_normal((k, n)) / np.sqrt(k)).astype(np.float32), dtype=dtype)
+    bias = Tensor(data=rng.standard_normal((n,)).astype(np.float32), dtype=dtype)
+    res = Tensor(data=rng.standard_normal((m, n)).astype(np.float32), dtype=dtype)
+    return x, w, bias, res
+
+
+SHAPES = [(2048, 512, 2048), (2048, 2048, 512), (2048, 512, 8192), (96, 64, 128), (200, 72, 136)]
+
+
+@pytest.mark.parametrize("dtype", [DType.float32, DType.float16], ids=["f32", "f16"])
+@pytest.mark.parametrize("m,k,n", SHAPES)
+def test_bias_and_gelu_join_the_product(hip_backend, monkeypatch, dtype, m, k, n):
+    rng = np.random.default_rng(m + n)
+    with hip_backend.use():
+        x, w, bias, _ = operands(rng, dtype, m, k, n)
+        check(hip_backend, monkeypatch, lambda: (Tensor.matmul(x, False, w, False, False) + bias).gelu(), removed=2)
+
+
+@pytest.mark.parametrize("dtype", [DType.float32, DType.float16], ids=["f32", "f16"])
+@pytest.mark.parametrize("m,k,n", SHAPES)
+def test_bias_and_residual_join_the_product(hip_backend, monkeypatch, dtype, m, k, n):
+    rng = np.random.default_rng(m + n + 1)
+    with hip_backend.use():
+        x, w, bias, res = operands(rng, dtype, m, k, n)
+        check(hip_backend, monkeypatch, lambda: res + (Tensor.matmul(x, False, w, False, False) + bias), removed=2)
+        check(hip_backend, monkeypatch, lambda: (bias + Tensor.matmul(x, False, w, False, False)) + res, removed=2)
+        # one matrix operand per merged kernel: the second dense addition stays a kernel of its own
+        check(hip_backend, monkeypatch, lambda: (Tensor.matmul(x, False, w, False, False) + res) + res, removed=1)
+        # three merged operations is the limit: the fourth stays a kernel of its own
+        check(hip_backend, monkeypatch,
+              lambda: ((Tensor.matmul(x, False, w, False, False) + bias).gelu() + res).gelu(), removed=3)
+
+
+def test_transposed_operands_and_a_three_axis_input(hip_backend, monkeypatch):
+    rng = np.random.default_rng(5)
+    with hip_backend.use():
+        x, w, bias, res = operands(rng, DType.float16, 512, 256, 384)
+        wt = Tensor(data=w.numpy().T.copy(), dtype=DType.float16)
+        check(hip_backend, monkeypatch, lambda: (Tensor.matmul(x, False, wt, True, False) + bias).gelu(), removed=2)
+        # `Linear` on [B, T, D]: reshapes around the product do not get in the way
+        lin = Linear(256, 384, rng, dtype=DType.float16, castParams=DType.float16)
+        x3 = Tensor(data=rng.standard_normal((4, 128, 256)).astype(np.float32), dtype=DType.float16)
+        res3 = Tensor(data=rng.standard_normal((4, 128, 384)).astype(np.float32), dtype=DType.float16)
+        # (the fp32 bias is cast to fp16 at call time: that cast is merged as well)
+        check(hip_backend, monkeypatch, lambda: res3 + lin(x3), removed=3)
+
+
+def test_a_result_with_two_readers_stays(hip_backend, monkeypatch):
+    rng = np.random.default_rng(6)
+    with hip_backend.use():
+        x, w, bias, res = operands(rng, DType.float32, 256, 128, 256)
+
+        def two_readers():
+            h = Tensor.matmul(x, False, w, False, False)
+            return (h + bias) + h.gelu()
+
+        check(hip_backend, monkeypatch, two_readers, removed=0)
+
+        def same_operand_twice():
+            h = Tensor.matmul(x, False, w, False, False)
+            return h + h
+
+        check(hip_backend, monkeypatch, same_operand_twice, removed=0)
+
+
+def test_a_result_the_caller_keeps_is_written(hip_backend):
+    rng = np.random.default_rng(7)
+    with hip_backend.use():
+        x, w, bias, _ = operands(rng, DType.float32, 256, 128, 256)
+        want_h = Tensor.matmul(x, False, w, False, False).numpy()
+        want = (Tensor.matmul(x, False, w, False, False) + bias).numpy()
+        with hip_backend.capture() as cap:
+            h = Tensor.matmul(x, False, w, False, False)        # still referenced after the capture
+            out = h + bias
+        cap.graph.launch()
+        assert np.array_equal(h.numpy(), want_h)
+        assert np.array_equal(out.numpy(), want)
+        cap.graph.destroy()
+
+
+def test_other_forms_of_add_are_left_alone(hip_backend, monkeypatch):
+    rng = np.random.default_rng(8)
+    with hip_backend.use():
+        x, w, _, _ = operands(rng, DType.float32, 256, 128, 256)
+        col = Tensor(data=rng.standard_normal((256, 1)).astype(np.float32))
+        ints = Tensor(data=rng.integers(-5, 5, size=(256, 128)))
+        iw = Tensor(data=rng.integers(-5, 5, size=(128, 256)))
+        irow = Tensor(data=rng.integers(-5, 5, size=(256,)))
+        check(hip_backend, monkeypatch, lambda: Tensor.matmul(x, False, w, False, False) + col, removed=0)
+        check(hip_backend, monkeypatch, lambda: Tensor.matmul(x, False, w, False, False) * w.sum(axis=0), removed=0)
+        check(hip_backend, monkeypatch, lambda: Tensor.matmul(ints, False, iw, False, False) + irow, removed=0)
+
+
+@pytest.mark.parametrize("dtype", [DType.float32, DType.float16], ids=["f32", "f16"])
+def test_config5_forward_recorded_with_the_rewrite(hip_backend, monkeypatch, dtype):
+    rng = np.random.default_rng(9)
+    with hip_backend.use():
+        model = Transformer(dtype=dtype)
+        ids = Tensor(data=rng.integers(0, 8192, size=(8, 256)))
+        want = model(ids).numpy().copy()
+        plain, plain_out, plain_nodes = record(hip_backend, lambda: model(ids), fusion=False, monkeypatch=monkeypatch)
+        fused, fused_out, fused_nodes = record(hip_backend, lambda: model(ids))
+        print("config 5", dtype.name, "launches per forward pass:", plain_nodes, "->", fused_nodes, flush=True)
+        for replay in range(3):
+            fused.launch()
+            assert np.array_equal(fused_out.numpy().view(np.uint8), want.view(np.uint8)), "replay %d" % replay
+        plain.launch()
+        assert np.array_equal(plain_out.numpy(), want)
+        # per block: q, k, v (+bias), o and fc2 (+bias, +residual), fc1 (+bias, GELU) = 9, and the
+        # unembedding's bias; in fp16 also the 6 + 1 casts of the fp32 biases
+        per_block = 9 + (6 if dtype == DType.float16 else 0)
+        assert plain_nodes - fused_nodes == 6 * per_block + (2 if dtype == DType.float16 else 1)
+        plain.destroy()
+        fused.destroy()

@@ -98,3 +98,22 @@ def test_code_objects_hold_every_reduce_and_gemm_kernel_the_host_names():
                   "hc_gemm_skinny_pack_%s", "hc_gemm_skinny_store_%s", "hc_copy2d_pad_b%d", "hc_copy2d_unpad_b%d"):
             name = n % (dt if "%s" in n else (2 if dt == "f16" else 4))
             assert any(name.encode() + b"\0" in b for b in blob.values()), name
+
+
+def test_build_refuses_register_tiled_kernels_that_use_scratch_memory():
+    """The build reads the compiler's resource remarks for the tiled GEMM code objects: a kernel
+    whose accumulators ended up in private memory still gives correct results, only several
+    times slower, so no parity test would notice it."""
+    from honeycrisp_amd.csrc import build
+    remarks = textwrap.dedent("""\
+        k.hip:9:1: remark: Function Name: hc_gemm_a [-Rpass-analysis=kernel-resource-usage]
+        k.hip:9:1: remark:     VGPRs: 110 [-Rpass-analysis=kernel-resource-usage]
+        k.hip:9:1: remark:     ScratchSize [bytes/lane]: 0 [-Rpass-analysis=kernel-resource-usage]
+        k.hip:9:1: remark: Function Name: hc_gemm_b [-Rpass-analysis=kernel-resource-usage]
+        k.hip:9:1: remark:     ScratchSize [bytes/lane]: 1088 [-Rpass-analysis=kernel-resource-usage]
+        k.hip:9:1: remark: Function Name: hc_gemm_c [-Rpass-analysis=kernel-resource-usage]
+        k.hip:9:1: remark:     ScratchSize [bytes/lane]: 68 [-Rpass-analysis=kernel-resource-usage]
+        """)
+    assert build.kernels_with_scratch(remarks) == ["hc_gemm_b (1088 bytes/lane)"]
+    assert {"gemm_dma", "gemm_dma2", "gemm_mi16"} <= build.NO_SCRATCH
+    assert build.NO_SCRATCH <= {name for name, _src, _flags in build.KERNELS}
