@@ -647,6 +647,16 @@ static int end_capture(hc_ctx* ctx, hc_graph** out) {
     ctx->lazy = false;
     if (out) {
       fuse_recording(ctx);
+      if (getenv("HCHIP_RECORDING_LOG")) {   // the launches of the recording as they will be enqueued, to stderr
+        size_t n = 0;
+        for (const hc_pending& e : ctx->pending) {
+          if (e.dropped || e.kind == hc_pending::FREE) continue;
+          const char* name = e.kind == hc_pending::COPY_D2D ? "(copy)" : "(caller's kernel)";
+          for (const auto& kv : ctx->functions)
+            if (e.kind == hc_pending::KERNEL && kv.second == e.fn) name = kv.first.c_str();
+          fprintf(stderr, "hchip recording %3zu: %s grid %u x %u\n", n++, name, e.grid[0], e.grid[1]);
+        }
+      }
       emitted = emit_recording_locked(ctx, ctx->pending);
       if (getenv("HCHIP_GRAPH_AS_LAUNCHES"))
         for (hc_pending& e : ctx->pending)
@@ -735,6 +745,9 @@ extern "C" int hc_graph_destroy(hc_ctx* ctx, hc_graph* graph) {
 // hc_capture_begin turns the rewrite off.
 
 static bool aligned16(const void* p);
+static const char* dtype_name(int dtype);
+static inline uint64_t ceil_div_u64(uint64_t a, uint64_t b) { return (a + b - 1) / b; }
+static int find_kernel_locked(hc_ctx* ctx, const std::string& name, hipFunction_t* out);
 static bool in_block(const void* p, const void* base, size_t bytes) {
   return (const char*)p >= (const char*)base && (const char*)p < (const char*)base + bytes;
 }
@@ -761,12 +774,210 @@ static long sole_user(const std::vector<hc_pending>& list, size_t from, const vo
   return user;
 }
 
+struct Freed { size_t at, bytes; };
+typedef std::unordered_map<const void*, Freed> FreedMap;
+
+// The tagged launch before entry `before` that produced the buffer `ptr`, or -1 (also when a
+// launch with undeclared buffers lies in between: it may have written `ptr`).
+static long producer_of(const std::vector<hc_pending>& list, size_t before, const void* ptr) {
+  for (size_t k = before; k-- > 0;) {
+    const hc_pending& e = list[k];
+    if (e.dropped || e.kind == hc_pending::FREE) continue;
+    if (!e.known) return -1;
+    if (e.kind == hc_pending::KERNEL && e.out == ptr) return (long)k;
+    for (const void* w : e.writes)
+      if (w == ptr) return -1;
+  }
+  return -1;
+}
+
+// The one entry that uses the buffer `ptr` written by entry `from`, provided the buffer is released
+// inside the recording; -1 otherwise.
+static long only_user(const std::vector<hc_pending>& list, const FreedMap& freed, size_t from, const void* ptr) {
+  auto fr = freed.find(ptr);
+  if (fr == freed.end() || fr->second.at <= from) return -1;
+  return sole_user(list, from, ptr, fr->second.bytes, fr->second.at);
+}
+
+// A chain's work moves to the place of its last entry: between its first and last entries, nothing
+// outside the chain may write what the merged kernel reads (and every launch there must have
+// declared its buffers).
+static bool inputs_stable(const std::vector<hc_pending>& list, const std::vector<size_t>& chain,
+                          std::initializer_list<const void*> inputs) {
+  size_t first = chain[0], last = chain[0];
+  for (size_t c : chain) {
+    first = std::min(first, c);
+    last = std::max(last, c);
+  }
+  for (size_t k = first + 1; k < last; k++) {
+    const hc_pending& e = list[k];
+    if (e.dropped || e.kind == hc_pending::FREE) continue;
+    bool member = false;
+    for (size_t c : chain) member = member || c == k;
+    if (member) continue;
+    if (!e.known) return false;
+    for (const void* w : e.writes)
+      for (const void* in : inputs)
+        if (in && w == in) return false;
+  }
+  return true;
+}
+
+// Replaces the entries of `chain` by one launch at the place of the last of them.
+static void replace_chain(std::vector<hc_pending>& list, const std::vector<size_t>& chain, hipFunction_t fn, uint64_t blocks,
+                          const void* args, size_t bytes, std::initializer_list<const void*> reads, const void* out) {
+  size_t last = chain[0];
+  for (size_t c : chain) {
+    last = std::max(last, c);
+    list[c].dropped = true;
+  }
+  hc_pending e;
+  e.kind = hc_pending::KERNEL;
+  e.fn = fn;
+  e.grid[0] = (uint32_t)blocks;
+  e.args.assign((const char*)args, (const char*)args + bytes);
+  e.known = true;
+  for (const void* r : reads)
+    if (r) e.reads.push_back(r);
+  e.writes = {out};
+  e.out = const_cast<void*>(out);
+  list[last] = std::move(e);
+}
+
+// [cast fp16 -> fp32] -> normalize (fp32 rows) [-> mulAdd with row operands, the coefficient
+// possibly gain + c] [-> cast fp32 -> fp16]: a LayerNorm (Trainable.swift:787-829) as one kernel.
+static void fuse_layernorms(hc_ctx* ctx, std::vector<hc_pending>& list, const FreedMap& freed) {
+  for (size_t i = 0; i < list.size(); i++) {
+    if (list[i].dropped || list[i].kind != hc_pending::KERNEL || list[i].tag != hc_pending::NORMALIZE) continue;
+    const hc_pending norm = list[i];
+    const uint64_t total = norm.rows * norm.cols;
+    std::vector<size_t> chain = {i};
+    hck_layernorm_args k;
+    memset(&k, 0, sizeof(k));
+    k.in = norm.in0;
+    k.outer = (uint32_t)norm.rows;
+    k.reduce = (uint32_t)norm.cols;
+    k.eps = norm.sf;
+    int in_type = HC_F32, out_type = HC_F32;
+    const void* out = norm.out;
+    size_t last = i;
+    const long up = producer_of(list, i, norm.in0);
+    if (up >= 0 && list[up].tag == hc_pending::CAST && list[up].src_dtype == HC_F16 && list[up].dtype == HC_F32 &&
+        list[up].cols == total && only_user(list, freed, (size_t)up, norm.in0) == (long)i) {
+      k.in = list[up].in0;
+      in_type = HC_F16;
+      chain.push_back((size_t)up);
+    }
+    long next = only_user(list, freed, last, out);
+    if (next >= 0 && list[next].tag == hc_pending::MUL_ADD && list[next].dtype == HC_F32 && list[next].in0 == out &&
+        list[next].rows == norm.rows && list[next].cols == norm.cols && aligned16(list[next].in1) && aligned16(list[next].in2)) {
+      const hc_pending& m = list[next];
+      k.flags |= HCK_LN_AFFINE;
+      k.gain = m.in1;
+      k.bias = m.in2;
+      const long sc = producer_of(list, (size_t)next, m.in1);
+      if (sc >= 0 && list[sc].tag == hc_pending::SCALAR && list[sc].op == HC_ADD && list[sc].dtype == HC_F32 &&
+          list[sc].cols == norm.cols && aligned16(list[sc].in0) && only_user(list, freed, (size_t)sc, m.in1) == next) {
+        k.flags |= HCK_LN_GAIN_ADD;
+        k.gain = list[sc].in0;
+        k.gain_add = list[sc].sf;
+        chain.push_back((size_t)sc);
+      }
+      chain.push_back((size_t)next);
+      last = (size_t)next;
+      out = m.out;
+      next = only_user(list, freed, last, out);
+    }
+    if (next >= 0 && list[next].tag == hc_pending::CAST && list[next].src_dtype == HC_F32 && list[next].dtype == HC_F16 &&
+        list[next].in0 == out && list[next].cols == total) {
+      out_type = HC_F16;
+      chain.push_back((size_t)next);
+      last = (size_t)next;
+      out = list[next].out;
+    }
+    if (chain.size() == 1 || !aligned16(k.in) || !aligned16(out)) continue;
+    if (!inputs_stable(list, chain, {k.in, k.gain, k.bias})) continue;
+    k.out = const_cast<void*>(out);
+    char name[64];
+    snprintf(name, sizeof(name), "hc_layernorm_rows_%s_%s", dtype_name(in_type), dtype_name(out_type));
+    hipFunction_t fn = nullptr;
+    if (find_kernel_locked(ctx, name, &fn) != HC_OK) continue;
+    replace_chain(list, chain, fn, ceil_div_u64(norm.rows, HCK_BLOCK / 64), &k, sizeof(k), {k.in, k.gain, k.bias}, out);
+  }
+}
+
+// [x * s] [+ mask] -> logSoftmax over rows [-> exp]: an attention softmax as one kernel.
+static void fuse_softmaxes(hc_ctx* ctx, std::vector<hc_pending>& list, const FreedMap& freed) {
+  for (size_t i = 0; i < list.size(); i++) {
+    if (list[i].dropped || list[i].kind != hc_pending::KERNEL || list[i].tag != hc_pending::LOG_SOFTMAX) continue;
+    const hc_pending sm = list[i];
+    const uint64_t total = sm.rows * sm.cols;
+    std::vector<size_t> chain = {i};
+    hck_softmax_chain_args k;
+    memset(&k, 0, sizeof(k));
+    k.in = sm.in0;
+    k.outer = (uint32_t)sm.rows;
+    k.reduce = (uint32_t)sm.cols;
+    k.mask_rows = 1;
+    size_t consumer = i;
+    long up = producer_of(list, consumer, k.in);
+    if (up >= 0 && list[up].tag == hc_pending::ADD && list[up].dtype == sm.dtype && list[up].rows * list[up].cols == total &&
+        only_user(list, freed, (size_t)up, k.in) == (long)consumer) {
+      const hc_pending& a = list[up];
+      // which operand is the one of `total` elements the rows come from, and how often the other repeats
+      const void* stream = a.add_form == 2 ? a.in1 : a.in0;
+      const void* mask = a.add_form == 2 ? a.in0 : a.in1;
+      const uint64_t mask_elems = a.add_form == 3 ? total : a.cols;
+      if (mask_elems % sm.cols == 0 && aligned16(mask) && aligned16(stream) && stream != mask) {
+        k.flags |= HCK_SM_MASK;
+        k.mask = mask;
+        k.mask_rows = (uint32_t)(mask_elems / sm.cols);
+        k.in = stream;
+        chain.push_back((size_t)up);
+        consumer = (size_t)up;
+      }
+    }
+    up = producer_of(list, consumer, k.in);
+    if (up >= 0 && list[up].tag == hc_pending::SCALAR && list[up].op == HC_MUL && list[up].dtype == sm.dtype &&
+        list[up].cols == total && aligned16(list[up].in0) && only_user(list, freed, (size_t)up, k.in) == (long)consumer) {
+      k.flags |= HCK_SM_SCALE;
+      k.scale = list[up].sf;
+      k.in = list[up].in0;
+      chain.push_back((size_t)up);
+    }
+    const void* out = sm.out;
+    const long next = only_user(list, freed, i, out);
+    if (next >= 0 && list[next].tag == hc_pending::EXP && list[next].dtype == sm.dtype && list[next].in0 == out &&
+        list[next].cols == total && aligned16(list[next].out)) {
+      k.flags |= HCK_SM_EXP;
+      chain.push_back((size_t)next);
+      out = list[next].out;
+    }
+    if (chain.size() == 1) continue;
+    if (!inputs_stable(list, chain, {k.in, k.mask})) continue;
+    k.out = const_cast<void*>(out);
+    char name[64];
+    snprintf(name, sizeof(name), "hc_softmax_chain_rows%s_%s", sm.lanes == 8 ? "8" : "", dtype_name(sm.dtype));
+    hipFunction_t fn = nullptr;
+    if (find_kernel_locked(ctx, name, &fn) != HC_OK) continue;
+    replace_chain(list, chain, fn, ceil_div_u64(sm.rows, HCK_BLOCK / (uint64_t)sm.lanes), &k, sizeof(k), {k.in, k.mask}, out);
+  }
+}
+
+static void fuse_products(hc_ctx* ctx, std::vector<hc_pending>& list, const FreedMap& freed);
+
 static void fuse_recording(hc_ctx* ctx) {
   std::vector<hc_pending>& list = ctx->pending;
-  struct Freed { size_t at, bytes; };
-  std::unordered_map<const void*, Freed> freed;
+  FreedMap freed;
   for (size_t i = 0; i < list.size(); i++)
     if (list[i].kind == hc_pending::FREE) freed[list[i].dst] = Freed{i, list[i].bytes};
+  fuse_products(ctx, list, freed);
+  fuse_layernorms(ctx, list, freed);
+  fuse_softmaxes(ctx, list, freed);
+}
+
+static void fuse_products(hc_ctx* ctx, std::vector<hc_pending>& list, const FreedMap& freed) {
+  (void)ctx;
 
   for (size_t i = 0; i < list.size(); i++) {
     if (list[i].kind != hc_pending::KERNEL || list[i].dropped || list[i].tag != hc_pending::GEMM) continue;
@@ -976,6 +1187,25 @@ extern "C" int hc_launch(hc_ctx* ctx, hc_function* fn, const uint32_t grid[3], c
 
 // Look a kernel up by name in the embedded code objects (cached) and launch it with a
 // 256-lane block.
+// A built-in kernel by name (caller holds the mutex).
+static int find_kernel_locked(hc_ctx* ctx, const std::string& name, hipFunction_t* out) {
+  auto it = ctx->functions.find(name);
+  if (it != ctx->functions.end()) {
+    *out = it->second;
+    return HC_OK;
+  }
+  hipFunction_t fn = nullptr;
+  for (hipModule_t m : ctx->modules) {
+    if (hipModuleGetFunction(&fn, m, name.c_str()) == hipSuccess) break;
+    (void)hipGetLastError();
+    fn = nullptr;
+  }
+  if (!fn) return fail(HC_ERR_LOAD, "kernel '%s' is not in the embedded code objects", name.c_str());
+  ctx->functions[name] = fn;
+  *out = fn;
+  return HC_OK;
+}
+
 static int launch(hc_ctx* ctx, const std::string& name, uint64_t blocks_x, uint32_t blocks_y,
                   const void* args, size_t bytes) {
   if (blocks_x == 0 || blocks_y == 0) return HC_OK;
@@ -984,18 +1214,7 @@ static int launch(hc_ctx* ctx, const std::string& name, uint64_t blocks_x, uint3
                 (unsigned long long)blocks_x);
   std::lock_guard<std::mutex> lock(ctx->mu);
   hipFunction_t fn = nullptr;
-  auto it = ctx->functions.find(name);
-  if (it != ctx->functions.end()) {
-    fn = it->second;
-  } else {
-    for (hipModule_t m : ctx->modules) {
-      if (hipModuleGetFunction(&fn, m, name.c_str()) == hipSuccess) break;
-      (void)hipGetLastError();
-      fn = nullptr;
-    }
-    if (!fn) return fail(HC_ERR_LOAD, "kernel '%s' is not in the embedded code objects", name.c_str());
-    ctx->functions[name] = fn;
-  }
+  HC_TRY(find_kernel_locked(ctx, name, &fn));
   if (ctx->lazy) {
     record_launch_locked(ctx, fn, (uint32_t)blocks_x, blocks_y, args, bytes);
     return HC_OK;
@@ -1132,6 +1351,7 @@ static const char* const kBinaryNames[] = {"add", "mul", "sub", "div", "mod"};
 static const char* const kCompareNames[] = {"eq", "ne", "lt", "le", "gt", "ge"};
 
 extern "C" int hc_broadcast(hc_ctx* ctx, int dtype, const void* a, const hc_strides* as, void* out) {
+  OpNote note({a}, {out});
   REQUIRE(ctx && a && as && out, "hc_broadcast: null argument");
   REQUIRE(dtype_name(dtype), "hc_broadcast: bad dtype %d", dtype);
   const size_t el = dtype_size(dtype);
@@ -1196,6 +1416,7 @@ extern "C" int hc_binary_op(hc_ctx* ctx, int op, int dtype, const void* a, const
 
 extern "C" int hc_bitwise_op(hc_ctx* ctx, int op, int dtype, const void* a, const hc_strides* as,
                              const void* b, const hc_strides* bs, void* out) {
+  OpNote note({a, b}, {out});
   REQUIRE(ctx && a && as && b && bs && out, "hc_bitwise_op: null argument");
   REQUIRE(op >= HC_BIT_OR && op <= HC_BIT_XOR, "hc_bitwise_op: bad op %d", op);
   REQUIRE(dtype_name(dtype), "hc_bitwise_op: bad dtype %d", dtype);
@@ -1219,6 +1440,7 @@ extern "C" int hc_bitwise_op(hc_ctx* ctx, int op, int dtype, const void* a, cons
 
 extern "C" int hc_compare(hc_ctx* ctx, int op, int dtype, const void* a, const hc_strides* as,
                           const void* b, const hc_strides* bs, void* out) {
+  OpNote note({a, b}, {out});
   REQUIRE(ctx && a && as && b && bs && out, "hc_compare: null argument");
   REQUIRE(op >= HC_EQ && op <= HC_GE, "hc_compare: bad op %d", op);
   REQUIRE(dtype_name(dtype), "hc_compare: bad dtype %d", dtype);
@@ -1294,6 +1516,7 @@ extern "C" int hc_add_mul(hc_ctx* ctx, int dtype, const void* input, const hc_st
 
 extern "C" int hc_when(hc_ctx* ctx, int dtype, const void* mask, const hc_strides* ms, const void* a,
                        const hc_strides* as, const void* b, const hc_strides* bs, void* out) {
+  OpNote note({mask, a, b}, {out});
   REQUIRE(ctx && mask && ms && a && as && b && bs && out, "hc_when: null argument");
   REQUIRE(dtype_name(dtype), "hc_when: bad dtype %d", dtype);
   const size_t el = dtype_size(dtype);
@@ -1304,6 +1527,7 @@ extern "C" int hc_when(hc_ctx* ctx, int dtype, const void* mask, const hc_stride
 
 extern "C" int hc_clamp(hc_ctx* ctx, int dtype, const void* a, const hc_strides* as, const void* lo,
                         const hc_strides* ls, const void* hi, const hc_strides* hs, void* out) {
+  OpNote note({a, lo, hi}, {out});
   REQUIRE(ctx && a && as && out, "hc_clamp: null argument");
   REQUIRE((lo && ls) || (hi && hs), "hc_clamp: cannot clamp without bounds");
   if (dtype != HC_F32 && dtype != HC_F16 && dtype != HC_I64)
@@ -1377,6 +1601,7 @@ extern "C" int hc_binary_op_scalar(hc_ctx* ctx, int op, int dtype, const void* a
 
 extern "C" int hc_compare_scalar(hc_ctx* ctx, int op, int dtype, const void* a, float sf, int64_t si,
                                  int scalar_first, void* out, size_t count) {
+  OpNote note({a}, {out});
   REQUIRE(ctx, "hc_compare_scalar: null context");
   REQUIRE(op >= HC_EQ && op <= HC_GE, "hc_compare_scalar: bad op %d", op);
   REQUIRE(dtype_name(dtype), "hc_compare_scalar: bad dtype %d", dtype);
@@ -1425,6 +1650,7 @@ extern "C" int hc_cast(hc_ctx* ctx, const void* in, int in_type, void* out, int 
 
 extern "C" int hc_pow(hc_ctx* ctx, int dtype, const void* in, float bf, float scalef, int64_t bi,
                       int64_t scalei, const void* scales, void* out, size_t count) {
+  OpNote note({in, scales}, {out});
   REQUIRE(ctx, "hc_pow: null context");
   if (dtype != HC_F32 && dtype != HC_F16 && dtype != HC_I64)
     return fail(HC_ERR_UNSUPPORTED, "hc_pow: dtype %d is not numeric", dtype);
@@ -1518,6 +1744,7 @@ static uint16_t f32_to_f16_bits(float f) {
 }
 
 extern "C" int hc_fill(hc_ctx* ctx, int dtype, float vf, int64_t vi, void* out, size_t count) {
+  OpNote note({}, {out});
   REQUIRE(ctx, "hc_fill: null context");
   REQUIRE(dtype_name(dtype), "hc_fill: bad dtype %d", dtype);
   if (count == 0) return HC_OK;
@@ -1752,6 +1979,7 @@ static int reduce_impl(hc_ctx* ctx, Scratch& scratch, int op, int dtype, const v
 
 extern "C" int hc_reduce(hc_ctx* ctx, int op, int dtype, const void* in, void* out, int64_t outer,
                          int64_t reduce, int64_t inner) {
+  OpNote note({in}, {out});
   REQUIRE(ctx, "hc_reduce: null context");
   Scratch scratch(ctx);
   return reduce_impl(ctx, scratch, op, dtype, in, out, outer, reduce, inner);
@@ -1777,6 +2005,7 @@ __attribute__((visibility("hidden"))) int hc_set_error(int code, const char* mes
 
 extern "C" int hc_cumulative(hc_ctx* ctx, int op, int dtype, const void* in, void* out, int64_t outer,
                              int64_t reduce, int64_t inner, int exclusive, int reverse) {
+  OpNote note({in}, {out});
   REQUIRE(ctx, "hc_cumulative: null context");
   REQUIRE(op == 0 || op == 1, "hc_cumulative: bad op %d", op);
   if (dtype != HC_F32 && dtype != HC_F16 && dtype != HC_I64)
@@ -1842,6 +2071,7 @@ extern "C" int hc_cumulative(hc_ctx* ctx, int op, int dtype, const void* in, voi
 
 extern "C" int hc_argsort(hc_ctx* ctx, int dtype, const void* in, void* out, int64_t outer, int64_t reduce,
                           int64_t inner, int descending) {
+  OpNote note({in}, {out});
   REQUIRE(ctx, "hc_argsort: null context");
   if (dtype != HC_F32 && dtype != HC_F16 && dtype != HC_I64)
     return fail(HC_ERR_UNSUPPORTED, "hc_argsort: dtype %d is not numeric", dtype);
@@ -1949,6 +2179,7 @@ extern "C" int hc_log_softmax(hc_ctx* ctx, int dtype, const void* in, void* out,
 
 extern "C" int hc_log_softmax_grad(hc_ctx* ctx, int dtype, const void* in, const void* out_grad, void* out,
                                    int64_t outer, int64_t reduce, int64_t inner) {
+  OpNote note({in, out_grad}, {out});
   REQUIRE(ctx, "hc_log_softmax_grad: null context");
   if (dtype != HC_F32 && dtype != HC_F16)
     return fail(HC_ERR_UNSUPPORTED, "hc_log_softmax_grad: dtype %d is not a float type", dtype);
@@ -2066,6 +2297,7 @@ extern "C" int hc_normalize(hc_ctx* ctx, int dtype, const void* in, void* out, i
 extern "C" int hc_gather(hc_ctx* ctx, int dtype, const void* in, const void* indices,
                          const hc_strides* idx_strides, void* out, int64_t outer, int64_t middle,
                          int64_t out_count, int64_t inner) {
+  OpNote note({in, indices}, {out});
   REQUIRE(ctx && idx_strides, "hc_gather: null argument");
   REQUIRE(dtype_name(dtype), "hc_gather: bad dtype %d", dtype);
   REQUIRE(outer >= 0 && middle >= 0 && out_count >= 0 && inner >= 0, "hc_gather: negative dimension");
@@ -2160,6 +2392,7 @@ extern "C" int hc_gather(hc_ctx* ctx, int dtype, const void* in, const void* ind
 extern "C" int hc_scatter(hc_ctx* ctx, int dtype, const void* in, const void* indices,
                           const hc_strides* idx_strides, void* out, int64_t outer, int64_t middle,
                           int64_t out_count, int64_t inner, int indices_are_unique) {
+  OpNote note({in, indices}, {out});
   REQUIRE(ctx && idx_strides, "hc_scatter: null argument");
   if (dtype != HC_F32 && dtype != HC_F16 && dtype != HC_I64)
     return fail(HC_ERR_UNSUPPORTED, "hc_scatter: dtype %d is not numeric", dtype);
@@ -2273,6 +2506,7 @@ extern "C" int hc_adamw(hc_ctx* ctx, int dtype, const void* param, const void* g
                         const void* moment2, float beta1, float beta2, float eps, float weight_decay,
                         float lr, float step, size_t count, void* out_param, void* out_moment1,
                         void* out_moment2) {
+  OpNote note({param, grad, moment1, moment2}, {out_param, out_moment1, out_moment2});
   REQUIRE(ctx, "hc_adamw: null context");
   if (dtype != HC_F32 && dtype != HC_F16)
     return fail(HC_ERR_UNSUPPORTED, "hc_adamw: dtype %d is not a float type", dtype);
@@ -2314,6 +2548,7 @@ extern "C" int hc_adamw(hc_ctx* ctx, int dtype, const void* param, const void* g
 
 extern "C" int hc_axis_permutation(hc_ctx* ctx, const int64_t* perm, const int64_t* shape, int ndim,
                                    void* out) {
+  OpNote note({}, {out});
   REQUIRE(ctx, "hc_axis_permutation: null context");
   REQUIRE(ndim >= 0 && ndim <= HC_MAX_DIMS, "hc_axis_permutation: ndim %d out of range", ndim);
   REQUIRE(ndim == 0 || (perm && shape), "hc_axis_permutation: null argument");
@@ -2349,6 +2584,7 @@ extern "C" int hc_axis_permutation(hc_ctx* ctx, const int64_t* perm, const int64
 
 extern "C" int hc_permute(hc_ctx* ctx, int dtype, const void* in, const int64_t* perm, const int64_t* shape,
                           int ndim, int64_t inner, void* out) {
+  OpNote note({in}, {out});
   REQUIRE(ctx, "hc_permute: null context");
   REQUIRE(dtype_name(dtype), "hc_permute: bad dtype %d", dtype);
   REQUIRE(ndim >= 0 && ndim <= HC_MAX_DIMS, "hc_permute: ndim %d out of range", ndim);
@@ -2469,6 +2705,7 @@ extern "C" int hc_permute(hc_ctx* ctx, int dtype, const void* in, const int64_t*
 
 extern "C" int hc_triangular(hc_ctx* ctx, int dtype, const void* in, void* out, int64_t batch,
                              int64_t rows, int64_t cols, int upper, int64_t offset) {
+  OpNote note({in}, {out});
   REQUIRE(ctx, "hc_triangular: null context");
   REQUIRE(dtype_name(dtype), "hc_triangular: bad dtype %d", dtype);
   REQUIRE(batch >= 0 && rows >= 0 && cols >= 0, "hc_triangular: negative dimension");
@@ -2498,6 +2735,9 @@ extern "C" int hc_triangular(hc_ctx* ctx, int dtype, const void* in, void* out, 
 
 extern "C" int hc_concat(hc_ctx* ctx, int dtype, const void* const* inputs, const int64_t* inner_counts,
                          int n_inputs, int64_t outer, void* out) {
+  OpNote note({}, {out});
+  if (inputs)
+    for (int i = 0; i < n_inputs; i++) note.reads.push_back(inputs[i]);
   REQUIRE(ctx, "hc_concat: null context");
   REQUIRE(dtype_name(dtype), "hc_concat: bad dtype %d", dtype);
   REQUIRE(n_inputs >= 0 && outer >= 0, "hc_concat: negative count");

@@ -1,13 +1,14 @@
 """The rewrite of a recording (hc_capture_end): a product whose result has exactly one reader takes
-that reader's work into its own kernel. A replay must return the bits the same ops return when
-issued one by one, the rewrite must actually remove launches where it applies, and it must leave
-the recording alone where a merged intermediate would be missed (a second reader, a result the
-caller still holds)."""
+that reader's work into its own kernel, and the launches of a LayerNorm and of an attention
+softmax become one kernel each. A replay must return the bits the same ops return when issued one
+by one, the rewrite must actually remove launches where it applies, and it must leave the
+recording alone where a merged intermediate would be missed (a second reader, a result the caller
+still holds)."""
 import numpy as np
 import pytest
 
 from honeycrisp_amd.descriptors import DType
-from honeycrisp_amd.nn import Linear, Transformer
+from honeycrisp_amd.nn import LayerNorm, Linear, Transformer
 from honeycrisp_amd.tensor import Tensor
 
 pytestmark = pytest.mark.gpu
@@ -141,6 +142,79 @@ def test_other_forms_of_add_are_left_alone(hip_backend, monkeypatch):
         check(hip_backend, monkeypatch, lambda: Tensor.matmul(ints, False, iw, False, False) + irow, removed=0)
 
 
+@pytest.mark.parametrize("dtype,removed", [(DType.float32, 2), (DType.float16, 4)], ids=["f32", "f16"])
+@pytest.mark.parametrize("rows,width", [(2048, 512), (77, 1024), (300, 132), (5, 256)])
+def test_layernorm_becomes_one_kernel(hip_backend, monkeypatch, dtype, removed, rows, width):
+    """cast -> normalize -> gain + 1 -> mulAdd -> cast (the casts only around fp16 activations)."""
+    rng = np.random.default_rng(rows + width)
+    with hip_backend.use():
+        ln = LayerNorm([width], rng=rng)
+        x = Tensor(data=(rng.standard_normal((rows, width)) * 3 + 1).astype(np.float32), dtype=dtype)
+        check(hip_backend, monkeypatch, lambda: ln(x), removed=removed)
+        x3 = Tensor(data=rng.standard_normal((3, 7, width)).astype(np.float32), dtype=dtype)
+        check(hip_backend, monkeypatch, lambda: ln(x3), removed=removed)
+
+
+def test_layernorm_variants(hip_backend, monkeypatch):
+    rng = np.random.default_rng(21)
+    with hip_backend.use():
+        x = Tensor(data=rng.standard_normal((64, 256)).astype(np.float32))
+        plain = LayerNorm([256], affine=False)
+        check(hip_backend, monkeypatch, lambda: plain(x), removed=0)                 # normalize alone: nothing to merge
+        xh = x.cast(DType.float16)
+        check(hip_backend, monkeypatch, lambda: plain(xh), removed=2)                # cast, normalize, cast
+        ln = LayerNorm([256], rng=rng)
+        # the coefficient used as it is (no gain + 1), and a normalized tensor that is read twice
+        check(hip_backend, monkeypatch,
+              lambda: x.normalize(axis=1, eps=1e-5).mul(ln.gain, thenAdd=ln.bias), removed=1)
+
+        def read_twice():
+            n = x.normalize(axis=1, eps=1e-5)
+            return n.mul(ln.gain + 1, thenAdd=ln.bias) + n
+
+        check(hip_backend, monkeypatch, read_twice, removed=0)
+        # rows of 1028 floats do not fit a wave's registers, rows of 16 take a smaller team: left alone
+        for width in (1028, 16):
+            wide = LayerNorm([width], rng=rng)
+            xw = Tensor(data=rng.standard_normal((32, width)).astype(np.float32))
+            check(hip_backend, monkeypatch, lambda: wide(xw), removed=0)
+
+
+@pytest.mark.parametrize("dtype", [DType.float32, DType.float16], ids=["f32", "f16"])
+@pytest.mark.parametrize("heads,t", [(32, 256), (6, 40), (3, 512), (2, 1024)])
+def test_attention_softmax_becomes_one_kernel(hip_backend, monkeypatch, dtype, heads, t):
+    """scores * s -> + mask -> logSoftmax -> exp."""
+    rng = np.random.default_rng(heads + t)
+    with hip_backend.use():
+        scores = Tensor(data=(rng.standard_normal((2, heads, t, t)) * 4).astype(np.float32), dtype=dtype)
+        mask = Tensor(data=np.where(np.tril(np.ones((t, t))) > 0, 0.0, -1e4).astype(np.float32), dtype=dtype)
+        full = Tensor(data=rng.standard_normal((2, heads, t, t)).astype(np.float32), dtype=dtype)
+        check(hip_backend, monkeypatch, lambda: (scores * 0.125 + mask).softmax(), removed=3)
+        check(hip_backend, monkeypatch, lambda: (mask + scores * 0.125).softmax(), removed=3)
+        check(hip_backend, monkeypatch, lambda: (scores * 0.125 + full).softmax(), removed=3)
+        check(hip_backend, monkeypatch, lambda: (scores * 0.125).softmax(), removed=2)
+        check(hip_backend, monkeypatch, lambda: (scores + mask).logSoftmax(), removed=1)
+        check(hip_backend, monkeypatch, lambda: scores.softmax(), removed=1)
+
+
+def test_softmax_forms_that_are_left_alone(hip_backend, monkeypatch):
+    rng = np.random.default_rng(33)
+    with hip_backend.use():
+        x = Tensor(data=rng.standard_normal((64, 100)).astype(np.float32), dtype=DType.float16)   # 100 halfs: no 16-byte rows
+        check(hip_backend, monkeypatch, lambda: (x * 0.5).softmax(), removed=0)
+        y = Tensor(data=rng.standard_normal((64, 4096)).astype(np.float32))                        # a block per row
+        check(hip_backend, monkeypatch, lambda: (y * 0.5).softmax(), removed=0)
+        z = Tensor(data=rng.standard_normal((64, 256)).astype(np.float32))
+
+        def scaled_read_twice():
+            s = z * 0.5
+            return s.softmax() + s
+
+        check(hip_backend, monkeypatch, scaled_read_twice, removed=1)       # only the exp joins
+        col = Tensor(data=rng.standard_normal((64, 1)).astype(np.float32))
+        check(hip_backend, monkeypatch, lambda: (z + col).softmax(), removed=1)  # a column operand is no mask
+
+
 @pytest.mark.parametrize("dtype", [DType.float32, DType.float16], ids=["f32", "f16"])
 def test_config5_forward_recorded_with_the_rewrite(hip_backend, monkeypatch, dtype):
     rng = np.random.default_rng(9)
@@ -156,9 +230,12 @@ def test_config5_forward_recorded_with_the_rewrite(hip_backend, monkeypatch, dty
             assert np.array_equal(fused_out.numpy().view(np.uint8), want.view(np.uint8)), "replay %d" % replay
         plain.launch()
         assert np.array_equal(plain_out.numpy(), want)
-        # per block: q, k, v (+bias), o and fc2 (+bias, +residual), fc1 (+bias, GELU) = 9, and the
-        # unembedding's bias; in fp16 also the 6 + 1 casts of the fp32 biases
-        per_block = 9 + (6 if dtype == DType.float16 else 0)
-        assert plain_nodes - fused_nodes == 6 * per_block + (2 if dtype == DType.float16 else 1)
+        # per block: q, k, v (+bias), o and fc2 (+bias, +residual), fc1 (+bias, GELU) = 9 launches
+        # merged into products, 2 LayerNorms of 3 launches (fp16: 5) and a softmax of 4; then the
+        # last LayerNorm and the unembedding's bias; in fp16 also the 6 + 1 casts of the fp32 biases
+        half = dtype == DType.float16
+        per_block = 9 + 2 * (4 if half else 2) + 3 + (6 if half else 0)
+        assert plain_nodes - fused_nodes == 6 * per_block + (4 if half else 2) + (2 if half else 1)
+        assert fused_nodes == 94
         plain.destroy()
         fused.destroy()
