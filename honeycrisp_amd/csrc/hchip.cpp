@@ -67,7 +67,7 @@ struct hc_pending {
   std::vector<const void*> reads;
   std::vector<const void*> writes;
   // what the rewrite needs to know about the operations it can merge
-  enum Tag { NONE, GEMM, ADD, GELU, CAST, NORMALIZE, LOG_SOFTMAX, SCALAR, MUL_ADD, EXP } tag = NONE;
+  enum Tag { NONE, GEMM, BMM, PERMUTE, ADD, GELU, CAST, NORMALIZE, LOG_SOFTMAX, SCALAR, MUL_ADD, EXP } tag = NONE;
   int dtype = 0;                       // element type of the output
   int src_dtype = 0;                   // CAST: element type of the input
   uint64_t rows = 0, cols = 0;         // GEMM: M, N; ADD: leading x trailing extent; GELU, CAST: 1 x count
@@ -79,6 +79,11 @@ struct hc_pending {
   // SCALAR: out = in0 (op) sf over `cols` elements, op = HC_ADD or HC_MUL as the kernel computes it
   // MUL_ADD: out = in0 * in1 + in2 with in0 dense [rows, cols] and in1, in2 rows of `cols` elements
   // EXP: ElemwiseOp.exp over `cols` elements of in0
+  // BMM: a batched product in one launch of a direct-to-LDS kernel (operands in the argument struct)
+  // PERMUTE (row form): in0 -> out; axis d of the dense output has extent pext[d] and lies at
+  // stride pstr[d] (elements) in the source, the last axis contiguous in both
+  int pn = 0;
+  uint64_t pext[HC_MAX_DIMS + 1] = {0}, pstr[HC_MAX_DIMS + 1] = {0};
   const void* in2 = nullptr;
   float sf = 0.0f;
   int op = 0;
@@ -746,6 +751,7 @@ extern "C" int hc_graph_destroy(hc_ctx* ctx, hc_graph* graph) {
 
 static bool aligned16(const void* p);
 static const char* dtype_name(int dtype);
+static size_t dtype_size(int dtype);
 static inline uint64_t ceil_div_u64(uint64_t a, uint64_t b) { return (a + b - 1) / b; }
 static int find_kernel_locked(hc_ctx* ctx, const std::string& name, hipFunction_t* out);
 static bool in_block(const void* p, const void* base, size_t bytes) {
@@ -799,37 +805,38 @@ static long only_user(const std::vector<hc_pending>& list, const FreedMap& freed
   return sole_user(list, from, ptr, fr->second.bytes, fr->second.at);
 }
 
-// A chain's work moves to the place of its last entry: between its first and last entries, nothing
-// outside the chain may write what the merged kernel reads (and every launch there must have
-// declared its buffers).
-static bool inputs_stable(const std::vector<hc_pending>& list, const std::vector<size_t>& chain,
-                          std::initializer_list<const void*> inputs) {
-  size_t first = chain[0], last = chain[0];
-  for (size_t c : chain) {
-    first = std::min(first, c);
-    last = std::max(last, c);
-  }
-  for (size_t k = first + 1; k < last; k++) {
-    const hc_pending& e = list[k];
-    if (e.dropped || e.kind == hc_pending::FREE) continue;
-    bool member = false;
-    for (size_t c : chain) member = member || c == k;
-    if (member) continue;
-    if (!e.known) return false;
-    for (const void* w : e.writes)
-      for (const void* in : inputs)
-        if (in && w == in) return false;
-  }
+// A chain's work moves to the place of its last entry. What an entry of the chain reads must
+// still hold the same values there: between that entry and the last one, nothing outside the
+// chain may write it (and every launch in between must have declared its buffers).
+struct Deferred {
+  size_t at;                       // index of the chain's entry
+  std::vector<const void*> reads;  // the caller-visible buffers the merged kernel reads on its behalf
+};
+static bool inputs_stable(const std::vector<hc_pending>& list, const std::vector<Deferred>& chain) {
+  size_t last = 0;
+  for (const Deferred& d : chain) last = std::max(last, d.at);
+  for (const Deferred& d : chain)
+    for (size_t k = d.at + 1; k < last; k++) {
+      const hc_pending& e = list[k];
+      if (e.dropped || e.kind == hc_pending::FREE) continue;
+      bool member = false;
+      for (const Deferred& c : chain) member = member || c.at == k;
+      if (member) continue;
+      if (!e.known) return false;
+      for (const void* w : e.writes)
+        for (const void* in : d.reads)
+          if (in && w == in) return false;
+    }
   return true;
 }
 
 // Replaces the entries of `chain` by one launch at the place of the last of them.
-static void replace_chain(std::vector<hc_pending>& list, const std::vector<size_t>& chain, hipFunction_t fn, uint64_t blocks,
+static void replace_chain(std::vector<hc_pending>& list, const std::vector<Deferred>& chain, hipFunction_t fn, uint64_t blocks,
                           const void* args, size_t bytes, std::initializer_list<const void*> reads, const void* out) {
-  size_t last = chain[0];
-  for (size_t c : chain) {
-    last = std::max(last, c);
-    list[c].dropped = true;
+  size_t last = chain[0].at;
+  for (const Deferred& c : chain) {
+    last = std::max(last, c.at);
+    list[c.at].dropped = true;
   }
   hc_pending e;
   e.kind = hc_pending::KERNEL;
@@ -851,7 +858,7 @@ static void fuse_layernorms(hc_ctx* ctx, std::vector<hc_pending>& list, const Fr
     if (list[i].dropped || list[i].kind != hc_pending::KERNEL || list[i].tag != hc_pending::NORMALIZE) continue;
     const hc_pending norm = list[i];
     const uint64_t total = norm.rows * norm.cols;
-    std::vector<size_t> chain = {i};
+    std::vector<Deferred> chain = {{i, {norm.in0}}};
     hck_layernorm_args k;
     memset(&k, 0, sizeof(k));
     k.in = norm.in0;
@@ -866,7 +873,8 @@ static void fuse_layernorms(hc_ctx* ctx, std::vector<hc_pending>& list, const Fr
         list[up].cols == total && only_user(list, freed, (size_t)up, norm.in0) == (long)i) {
       k.in = list[up].in0;
       in_type = HC_F16;
-      chain.push_back((size_t)up);
+      chain[0].reads.clear();
+      chain.push_back({(size_t)up, {k.in}});
     }
     long next = only_user(list, freed, last, out);
     if (next >= 0 && list[next].tag == hc_pending::MUL_ADD && list[next].dtype == HC_F32 && list[next].in0 == out &&
@@ -881,9 +889,9 @@ static void fuse_layernorms(hc_ctx* ctx, std::vector<hc_pending>& list, const Fr
         k.flags |= HCK_LN_GAIN_ADD;
         k.gain = list[sc].in0;
         k.gain_add = list[sc].sf;
-        chain.push_back((size_t)sc);
+        chain.push_back({(size_t)sc, {k.gain}});
       }
-      chain.push_back((size_t)next);
+      chain.push_back({(size_t)next, {k.flags & HCK_LN_GAIN_ADD ? nullptr : k.gain, k.bias}});
       last = (size_t)next;
       out = m.out;
       next = only_user(list, freed, last, out);
@@ -891,12 +899,12 @@ static void fuse_layernorms(hc_ctx* ctx, std::vector<hc_pending>& list, const Fr
     if (next >= 0 && list[next].tag == hc_pending::CAST && list[next].src_dtype == HC_F32 && list[next].dtype == HC_F16 &&
         list[next].in0 == out && list[next].cols == total) {
       out_type = HC_F16;
-      chain.push_back((size_t)next);
+      chain.push_back({(size_t)next, {}});
       last = (size_t)next;
       out = list[next].out;
     }
     if (chain.size() == 1 || !aligned16(k.in) || !aligned16(out)) continue;
-    if (!inputs_stable(list, chain, {k.in, k.gain, k.bias})) continue;
+    if (!inputs_stable(list, chain)) continue;
     k.out = const_cast<void*>(out);
     char name[64];
     snprintf(name, sizeof(name), "hc_layernorm_rows_%s_%s", dtype_name(in_type), dtype_name(out_type));
@@ -912,7 +920,7 @@ static void fuse_softmaxes(hc_ctx* ctx, std::vector<hc_pending>& list, const Fre
     if (list[i].dropped || list[i].kind != hc_pending::KERNEL || list[i].tag != hc_pending::LOG_SOFTMAX) continue;
     const hc_pending sm = list[i];
     const uint64_t total = sm.rows * sm.cols;
-    std::vector<size_t> chain = {i};
+    std::vector<Deferred> chain = {{i, {sm.in0}}};
     hck_softmax_chain_args k;
     memset(&k, 0, sizeof(k));
     k.in = sm.in0;
@@ -933,7 +941,8 @@ static void fuse_softmaxes(hc_ctx* ctx, std::vector<hc_pending>& list, const Fre
         k.mask = mask;
         k.mask_rows = (uint32_t)(mask_elems / sm.cols);
         k.in = stream;
-        chain.push_back((size_t)up);
+        chain[0].reads.clear();
+        chain.push_back({(size_t)up, {stream, mask}});
         consumer = (size_t)up;
       }
     }
@@ -942,25 +951,157 @@ static void fuse_softmaxes(hc_ctx* ctx, std::vector<hc_pending>& list, const Fre
         list[up].cols == total && aligned16(list[up].in0) && only_user(list, freed, (size_t)up, k.in) == (long)consumer) {
       k.flags |= HCK_SM_SCALE;
       k.scale = list[up].sf;
+      for (Deferred& d : chain)   // whoever read the scaled tensor reads nothing of it any more
+        for (const void*& r : d.reads)
+          if (r == k.in) r = nullptr;
       k.in = list[up].in0;
-      chain.push_back((size_t)up);
+      chain.push_back({(size_t)up, {k.in}});
     }
     const void* out = sm.out;
     const long next = only_user(list, freed, i, out);
     if (next >= 0 && list[next].tag == hc_pending::EXP && list[next].dtype == sm.dtype && list[next].in0 == out &&
         list[next].cols == total && aligned16(list[next].out)) {
       k.flags |= HCK_SM_EXP;
-      chain.push_back((size_t)next);
+      chain.push_back({(size_t)next, {}});
       out = list[next].out;
     }
     if (chain.size() == 1) continue;
-    if (!inputs_stable(list, chain, {k.in, k.mask})) continue;
+    if (!inputs_stable(list, chain)) continue;
     k.out = const_cast<void*>(out);
     char name[64];
     snprintf(name, sizeof(name), "hc_softmax_chain_rows%s_%s", sm.lanes == 8 ? "8" : "", dtype_name(sm.dtype));
     hipFunction_t fn = nullptr;
     if (find_kernel_locked(ctx, name, &fn) != HC_OK) continue;
     replace_chain(list, chain, fn, ceil_div_u64(sm.rows, HCK_BLOCK / (uint64_t)sm.lanes), &k, sizeof(k), {k.in, k.mask}, out);
+  }
+}
+
+// A batched product whose operand is a tensor with two axes swapped ([B, T, H, d] read as
+// [B, H, T, d]: the heads of an attention layer), or whose result is swapped back, reads and
+// writes through the strides instead: the copies disappear.
+static void fuse_swapped_batches(std::vector<hc_pending>& list, const FreedMap& freed) {
+  for (size_t i = 0; i < list.size(); i++) {
+    if (list[i].dropped || list[i].kind != hc_pending::KERNEL || list[i].tag != hc_pending::BMM) continue;
+    if (list[i].args.size() != sizeof(hck_gemm_args)) continue;
+    hck_gemm_args g;
+    memcpy(&g, list[i].args.data(), sizeof(g));
+    if (g.bdiv != 0) continue;
+    const uint64_t P = 16 / dtype_size(list[i].dtype), el = dtype_size(list[i].dtype);
+    std::vector<Deferred> chain = {{i, {g.a, g.b}}};
+    uint32_t bdiv = 0;            // 0: not decided yet
+    bool two_level = false;
+    // slice strides as they will be: {hi, lo}; an operand that stays as it is keeps hi = bdiv * bs, lo = bs
+    uint64_t a_hi = 0, a_lo = g.a_bs, b_hi = 0, b_lo = g.b_bs, c_hi = 0, c_lo = g.c_bs;
+    bool a_set = false, b_set = false, c_set = false;
+    auto read_through = [&](const void*& ptr, uint32_t& rs, uint32_t& cs, uint32_t rows, uint32_t cols, uint64_t bs,
+                            uint64_t& hi, uint64_t& lo, bool& set) {
+      // the operand's slices: [R, I] row-major with row stride I; (rs, cs) = strides of (rows, cols)
+      const bool row_major = cs == 1;
+      const uint64_t R = row_major ? rows : cols, I = row_major ? cols : rows;
+      if ((row_major ? rs : cs) != I || (row_major ? cs : rs) != 1 || bs != R * I) return;
+      const long up = producer_of(list, i, ptr);
+      if (up < 0 || list[up].tag != hc_pending::PERMUTE || list[up].dtype != list[i].dtype) return;
+      const hc_pending& pm = list[up];
+      if (only_user(list, freed, (size_t)up, ptr) != (long)i) return;
+      const int n = pm.pn;
+      if (n != 3 && n != 4) return;
+      if (pm.pext[n - 1] != I || pm.pstr[n - 1] != 1 || pm.pext[n - 2] != R) return;
+      uint64_t z_hi, s_hi, z_lo = 1, s_lo = 0;
+      if (n == 4) {
+        z_hi = pm.pext[0], s_hi = pm.pstr[0], z_lo = pm.pext[1], s_lo = pm.pstr[1];
+        if ((bdiv != 0 && bdiv != z_lo) || ((a_set || b_set) && !two_level)) return;
+      } else {
+        z_hi = pm.pext[0], s_hi = pm.pstr[0];
+        if (two_level) return;   // (a single-level operand next to a two-level one: expressible, not needed)
+      }
+      if (z_hi * z_lo != g.batch) return;
+      const uint64_t row_stride = pm.pstr[n - 2];
+      if (row_stride % P || s_hi % P || s_lo % P || !aligned16(pm.in0) || row_stride > 0xffffffffull ||
+          R * row_stride * el > 0xffffffffull)
+        return;
+      if (n == 4) {
+        bdiv = (uint32_t)z_lo;
+        two_level = true;
+        hi = s_hi, lo = s_lo;
+      } else {
+        hi = 0, lo = s_hi;   // single level: z * lo
+      }
+      set = true;
+      for (const void*& r : chain[0].reads)   // the product no longer reads the copy
+        if (r == ptr) r = nullptr;
+      ptr = pm.in0;
+      (row_major ? rs : cs) = (uint32_t)row_stride;
+      chain.push_back({(size_t)up, {pm.in0}});
+    };
+    read_through(g.a, g.a_rs, g.a_cs, g.M, g.K, g.a_bs, a_hi, a_lo, a_set);
+    read_through(g.b, g.b_rs, g.b_cs, g.K, g.N, g.b_bs, b_hi, b_lo, b_set);
+    // the result, swapped by its only reader
+    const void* out = list[i].out;
+    {
+      const long next = only_user(list, freed, i, out);
+      if (next >= 0 && list[next].tag == hc_pending::PERMUTE && list[next].dtype == list[i].dtype && list[next].in0 == out &&
+          g.c_rs == g.N && g.c_cs == 1 && g.c_bs == (uint64_t)g.M * g.N && aligned16(list[next].out)) {
+        const hc_pending& pm = list[next];
+        const int n = pm.pn;
+        // strides of the permute's dense output, and the role of each axis by its source stride
+        uint64_t ostr[HC_MAX_DIMS + 1];
+        uint64_t acc = 1;
+        for (int d = n - 1; d >= 0; d--) {
+          ostr[d] = acc;
+          acc *= pm.pext[d];
+        }
+        long m_ax = -1, lo_ax = -1, hi_ax = -1;
+        for (int d = 0; d < n - 1; d++) {
+          if (pm.pstr[d] == g.N && pm.pext[d] == g.M) m_ax = d;
+          else if (pm.pstr[d] == (uint64_t)g.M * g.N) lo_ax = d;
+          else hi_ax = d;
+        }
+        bool ok = (n == 3 || n == 4) && pm.pext[n - 1] == g.N && pm.pstr[n - 1] == 1 && m_ax >= 0 && lo_ax >= 0;
+        if (ok && n == 4)
+          ok = !((a_set || b_set) && !two_level) && hi_ax >= 0 && pm.pstr[hi_ax] == pm.pext[lo_ax] * (uint64_t)g.M * g.N &&
+               pm.pext[hi_ax] * pm.pext[lo_ax] == g.batch && (bdiv == 0 || bdiv == pm.pext[lo_ax]);
+        if (ok && n == 3) ok = pm.pext[lo_ax] == g.batch && !two_level;
+        if (ok) ok = ostr[m_ax] % P == 0 && ostr[lo_ax] % P == 0 && (n == 3 || ostr[hi_ax] % P == 0) && ostr[m_ax] <= 0xffffffffull;
+        if (ok) {
+          if (n == 4) {
+            bdiv = (uint32_t)pm.pext[lo_ax];
+            two_level = true;
+            c_hi = ostr[hi_ax], c_lo = ostr[lo_ax];
+          } else {
+            c_hi = 0, c_lo = ostr[lo_ax];
+          }
+          c_set = true;
+          g.c_rs = (uint32_t)ostr[m_ax];
+          g.c = pm.out;
+          out = pm.out;
+          chain.push_back({(size_t)next, {}});
+        }
+      }
+    }
+    if (chain.size() == 1) continue;
+    if (two_level) {
+      // operands that stay as they are: slice z = hi * bdiv + lo of a dense batch
+      if (!a_set) a_hi = (uint64_t)bdiv * g.a_bs, a_lo = g.a_bs;
+      if (!b_set) b_hi = (uint64_t)bdiv * g.b_bs, b_lo = g.b_bs;
+      if (!c_set) c_hi = (uint64_t)bdiv * g.c_bs, c_lo = g.c_bs;
+      g.bdiv = bdiv;
+      g.a_bs = a_hi, g.a_bs2 = a_lo;
+      g.b_bs = b_hi, g.b_bs2 = b_lo;
+      g.c_bs = c_hi, g.c_bs2 = c_lo;
+    } else {
+      g.a_bs = a_lo, g.b_bs = b_lo, g.c_bs = c_lo;
+    }
+    if (!inputs_stable(list, chain)) continue;
+    size_t last = i;
+    for (const Deferred& c : chain) last = std::max(last, c.at);
+    hc_pending fused = list[i];
+    memcpy(fused.args.data(), &g, sizeof(g));
+    fused.tag = hc_pending::NONE;
+    fused.reads = {g.a, g.b};
+    fused.writes = {out};
+    fused.out = const_cast<void*>(out);
+    for (const Deferred& c : chain) list[c.at].dropped = true;
+    list[last] = std::move(fused);
   }
 }
 
@@ -972,6 +1113,7 @@ static void fuse_recording(hc_ctx* ctx) {
   for (size_t i = 0; i < list.size(); i++)
     if (list[i].kind == hc_pending::FREE) freed[list[i].dst] = Freed{i, list[i].bytes};
   fuse_products(ctx, list, freed);
+  fuse_swapped_batches(list, freed);
   fuse_layernorms(ctx, list, freed);
   fuse_softmaxes(ctx, list, freed);
 }
@@ -1143,6 +1285,9 @@ static void record_launch_locked(hc_ctx* ctx, hipFunction_t fn, uint32_t gx, uin
       e.in0 = n->meta.in0;
       e.in1 = n->meta.in1;
       e.add_form = n->meta.add_form;
+      e.pn = n->meta.pn;
+      memcpy(e.pext, n->meta.pext, sizeof(e.pext));
+      memcpy(e.pstr, n->meta.pstr, sizeof(e.pstr));
       e.in2 = n->meta.in2;
       e.sf = n->meta.sf;
       e.op = n->meta.op;
@@ -2653,6 +2798,17 @@ extern "C" int hc_permute(hc_ctx* ctx, int dtype, const void* in, const int64_t*
       k.in_stride[d] = (uint32_t)ax[d].stride;
       hck_fast_div_setup(k.shape[d], &k.magic[d], &k.sh[d]);
     }
+    if (n >= 2) {
+      note.tag = hc_pending::PERMUTE;
+      note.meta.dtype = dtype;
+      note.meta.in0 = in;
+      note.meta.out = out;
+      note.meta.pn = n;
+      for (int d = 0; d < n; d++) {
+        note.meta.pext[d] = ax[d].extent;
+        note.meta.pstr[d] = ax[d].stride;
+      }
+    }
     snprintf(name, sizeof(name), "hc_permute_rows_b%zu_%s", el, vec > 1 ? "vN" : "v1");
     return launch(ctx, name, ceil_div((uint64_t)k.total, HCK_BLOCK), 1, &k, sizeof(k));
   }
@@ -3191,6 +3347,17 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
       note.meta.dtype = dtype;
       note.meta.rows = M;
       note.meta.cols = N;
+      note.meta.out = out;
+    }
+    // ... and a batched one may read or write through a swap of the batch axes
+    if (whole_call && bm != 0 && dma && batch > 1 && batch <= 65535 && !trans_out && !c_padded && k.a == a && k.b == b &&
+        k.c == out && k.c_rs == N) {
+      note.tag = hc_pending::BMM;
+      note.meta.dtype = dtype;
+      note.meta.rows = M;
+      note.meta.cols = N;
+      note.meta.in0 = a;
+      note.meta.in1 = b;
       note.meta.out = out;
     }
     // grid.y carries the batch (at most 65535 per launch)

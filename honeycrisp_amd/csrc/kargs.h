@@ -336,6 +336,11 @@ typedef struct {
   uint32_t ep_kind[3];    /* HCK_EP_* ; 0 ends the list */
   uint32_t ep_ld[3];      /* HCK_EP_ADD_MATRIX: leading dimension of the matrix, elements */
   const void* ep_ptr[3];  /* HCK_EP_ADD_ROW: N elements; HCK_EP_ADD_MATRIX: [M, ld] */
+  /* Two-level batch (direct-to-LDS kernels only; 0 = off): slice z lies at
+   * (z / bdiv) * x_bs + (z % bdiv) * x_bs2. What a batched product reads or writes when a
+   * recording folds a swap of the batch axes ([B, T, H, d] <-> [B, H, T, d]) into it. */
+  uint32_t bdiv, pad2;
+  uint64_t a_bs2, b_bs2, c_bs2;
 } hck_gemm_args;
 
 #define HCK_EP_NONE 0

@@ -231,9 +231,14 @@ __device__ __forceinline__ void gemm_dma2_impl(const hck_gemm_args& p, char* lds
   gemm_tile_of_block(p, blockIdx.x, tm, tn);
   const uint32_t m0 = tm * BM, n0 = tn * BN;
   const uint32_t batch = blockIdx.y;
-  const T* A = (const T*)p.a + batch * p.a_bs;
-  const T* B = (const T*)p.b + batch * p.b_bs;
-  T* C = (T*)p.c + batch * p.c_bs;
+  uint32_t batch_hi = batch, batch_lo = 0;
+  if (p.bdiv != 0) {
+    batch_hi = batch / p.bdiv;
+    batch_lo = batch - batch_hi * p.bdiv;
+  }
+  const T* A = (const T*)p.a + batch_hi * p.a_bs + batch_lo * p.a_bs2;
+  const T* B = (const T*)p.b + batch_hi * p.b_bs + batch_lo * p.b_bs2;
+  T* C = (T*)p.c + batch_hi * p.c_bs + batch_lo * p.c_bs2;
 
   const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const uint32_t wm = (wave >> 1) * (BM / 2), wn = (wave & 1) * (BN / 2);

@@ -216,6 +216,38 @@ def test_softmax_forms_that_are_left_alone(hip_backend, monkeypatch):
 
 
 @pytest.mark.parametrize("dtype", [DType.float32, DType.float16], ids=["f32", "f16"])
+@pytest.mark.parametrize("B,T,H,hd", [(8, 256, 8, 64), (2, 96, 3, 40), (1, 128, 4, 64)])
+def test_head_swaps_fold_into_the_batched_products(hip_backend, monkeypatch, dtype, B, T, H, hd):
+    """[B, T, H*hd] -> [B, T, H, hd] -> swap(1, 2) around batchedMatmul: the products read q, k, v
+    through the strides and write the context back in [B, T, H, hd] order; no copy is left."""
+    rng = np.random.default_rng(B + T + H)
+    D = H * hd
+    with hip_backend.use():
+        q, k, v = (Tensor(data=rng.standard_normal((B, T, D)).astype(np.float32), dtype=dtype) for _ in range(3))
+
+        def heads(x):
+            return x.reshape([B, T, H, hd]).swap(1, 2)
+
+        def attention():
+            scores = Tensor.batchedMatmul(heads(q), False, heads(k), True, False)
+            probs = (scores * 0.125).softmax()
+            return Tensor.batchedMatmul(probs, False, heads(v), False, False).swap(1, 2).reshape([B, T, D])
+
+        # 4 swaps, and scale + logSoftmax + exp -> 1
+        check(hip_backend, monkeypatch, attention, removed=4 + 2)
+        # one operand swapped, the other dense; result kept in [B, H, T, T] order
+        kt = Tensor(data=rng.standard_normal((B, H, T, hd)).astype(np.float32), dtype=dtype)
+        check(hip_backend, monkeypatch, lambda: Tensor.batchedMatmul(heads(q), False, kt, True, False), removed=1)
+        check(hip_backend, monkeypatch, lambda: Tensor.batchedMatmul(kt, False, heads(q), True, False), removed=1)
+        # a swapped tensor with a second reader stays a copy
+        def two_readers():
+            hq = heads(q)
+            return Tensor.batchedMatmul(hq, False, kt, True, False) + hq.sum(axis=3, keepdims=True)
+
+        check(hip_backend, monkeypatch, two_readers, removed=0)
+
+
+@pytest.mark.parametrize("dtype", [DType.float32, DType.float16], ids=["f32", "f16"])
 def test_config5_forward_recorded_with_the_rewrite(hip_backend, monkeypatch, dtype):
     rng = np.random.default_rng(9)
     with hip_backend.use():
@@ -231,11 +263,12 @@ def test_config5_forward_recorded_with_the_rewrite(hip_backend, monkeypatch, dty
         plain.launch()
         assert np.array_equal(plain_out.numpy(), want)
         # per block: q, k, v (+bias), o and fc2 (+bias, +residual), fc1 (+bias, GELU) = 9 launches
-        # merged into products, 2 LayerNorms of 3 launches (fp16: 5) and a softmax of 4; then the
-        # last LayerNorm and the unembedding's bias; in fp16 also the 6 + 1 casts of the fp32 biases
+        # merged into products, 2 LayerNorms of 3 launches (fp16: 5), a softmax of 4 and the 4 swaps
+        # of the heads; then the last LayerNorm and the unembedding's bias; in fp16 also the 6 + 1
+        # casts of the fp32 biases
         half = dtype == DType.float16
-        per_block = 9 + 2 * (4 if half else 2) + 3 + (6 if half else 0)
+        per_block = 9 + 2 * (4 if half else 2) + 3 + 4 + (6 if half else 0)
         assert plain_nodes - fused_nodes == 6 * per_block + (4 if half else 2) + (2 if half else 1)
-        assert fused_nodes == 94
+        assert fused_nodes == 70
         plain.destroy()
         fused.destroy()
