@@ -67,7 +67,7 @@ struct hc_pending {
   std::vector<const void*> reads;
   std::vector<const void*> writes;
   // what the rewrite needs to know about the operations it can merge
-  enum Tag { NONE, GEMM, BMM, PERMUTE, ADD, GELU, CAST, NORMALIZE, LOG_SOFTMAX, SCALAR, MUL_ADD, EXP } tag = NONE;
+  enum Tag { NONE, GEMM, PRODUCT, BMM, PERMUTE, ADD, GELU, CAST, NORMALIZE, LOG_SOFTMAX, SCALAR, MUL_ADD, EXP } tag = NONE;
   int dtype = 0;                       // element type of the output
   int src_dtype = 0;                   // CAST: element type of the input
   uint64_t rows = 0, cols = 0;         // GEMM: M, N; ADD: leading x trailing extent; GELU, CAST: 1 x count
@@ -1105,6 +1105,77 @@ static void fuse_swapped_batches(std::vector<hc_pending>& list, const FreedMap& 
   }
 }
 
+// Products over the same A with the same shape, strides and merged operations (the q, k, v
+// projections of an attention layer) become one launch: a workgroup's blockIdx.y picks the
+// member's B, C and epilogue operands.
+static void fuse_product_groups(std::vector<hc_pending>& list, const FreedMap& freed) {
+  auto is_product = [](const hc_pending& e) {
+    return !e.dropped && e.kind == hc_pending::KERNEL && (e.tag == hc_pending::GEMM || e.tag == hc_pending::PRODUCT) &&
+           e.args.size() == sizeof(hck_gemm_args);
+  };
+  auto uses = [&](const hc_pending& e, const void* buf) {   // e reads or writes the buffer at `buf`
+    auto fr = freed.find(buf);
+    const size_t bytes = fr == freed.end() ? 1 : fr->second.bytes;
+    return touches(e.reads, buf, bytes) || touches(e.writes, buf, bytes);
+  };
+  for (size_t i = 0; i < list.size(); i++) {
+    if (!is_product(list[i])) continue;
+    hck_gemm_args g;
+    memcpy(&g, list[i].args.data(), sizeof(g));
+    if (g.batch != 1 || g.bdiv != 0 || g.group != 0 || list[i].grid[1] != 1) continue;
+    std::vector<size_t> members = {i};
+    std::vector<hck_gemm_args> margs = {g};
+    for (size_t j = i + 1; j < list.size() && members.size() < HCK_GEMM_GROUP; j++) {
+      const hc_pending& e = list[j];
+      if (e.dropped || e.kind == hc_pending::FREE) continue;
+      if (!e.known) break;
+      bool joins = false;
+      hck_gemm_args h;
+      if (is_product(e) && e.fn == list[i].fn && e.dtype == list[i].dtype && e.grid[0] == list[i].grid[0] && e.grid[1] == 1) {
+        memcpy(&h, e.args.data(), sizeof(h));
+        joins = h.a == g.a && h.M == g.M && h.N == g.N && h.K == g.K && h.batch == 1 && h.bdiv == 0 && h.group == 0 &&
+                h.a_rs == g.a_rs && h.a_cs == g.a_cs && h.b_rs == g.b_rs && h.b_cs == g.b_cs && h.c_rs == g.c_rs &&
+                h.c_cs == g.c_cs && h.tiles_m == g.tiles_m && h.tiles_n == g.tiles_n && h.xcd_gn == g.xcd_gn &&
+                h.xcd_sm == g.xcd_sm && h.xcd_sn == g.xcd_sn && h.a_lim == g.a_lim && h.b_lim == g.b_lim &&
+                memcmp(h.ep_kind, g.ep_kind, sizeof(g.ep_kind)) == 0 && memcmp(h.ep_ld, g.ep_ld, sizeof(g.ep_ld)) == 0;
+      }
+      // The earlier members run where the last one stands: nothing in between (a later member
+      // included) may use their results or write what they read.
+      bool conflict = false;
+      for (size_t m = 0; m < members.size() && !conflict; m++) {
+        const hck_gemm_args& a = margs[m];
+        conflict = uses(e, a.c);
+        for (const void* w : e.writes)
+          conflict = conflict || w == a.a || w == a.b || w == a.ep_ptr[0] || w == a.ep_ptr[1] || w == a.ep_ptr[2];
+      }
+      if (conflict) break;
+      if (joins) {
+        members.push_back(j);
+        margs.push_back(h);
+      }
+    }
+    if (members.size() < 2) continue;
+    const uint32_t n = (uint32_t)members.size();
+    hc_pending grouped = list[i];
+    grouped.tag = hc_pending::NONE;
+    grouped.out = nullptr;
+    grouped.grid[1] = n;
+    grouped.reads.clear();
+    grouped.writes.clear();
+    g.group = n;
+    for (uint32_t m = 0; m < n; m++) {
+      g.g_b[m] = margs[m].b;
+      g.g_c[m] = margs[m].c;
+      for (int s = 0; s < 3; s++) g.g_ep[s][m] = margs[m].ep_ptr[s];
+      for (const void* r : list[members[m]].reads) grouped.reads.push_back(r);
+      grouped.writes.push_back(margs[m].c);
+      list[members[m]].dropped = true;
+    }
+    memcpy(grouped.args.data(), &g, sizeof(g));
+    list[members.back()] = std::move(grouped);
+  }
+}
+
 static void fuse_products(hc_ctx* ctx, std::vector<hc_pending>& list, const FreedMap& freed);
 
 static void fuse_recording(hc_ctx* ctx) {
@@ -1116,6 +1187,7 @@ static void fuse_recording(hc_ctx* ctx) {
   fuse_swapped_batches(list, freed);
   fuse_layernorms(ctx, list, freed);
   fuse_softmaxes(ctx, list, freed);
+  fuse_product_groups(list, freed);
 }
 
 static void fuse_products(hc_ctx* ctx, std::vector<hc_pending>& list, const FreedMap& freed) {
@@ -1203,7 +1275,7 @@ static void fuse_products(hc_ctx* ctx, std::vector<hc_pending>& list, const Free
     g.c = const_cast<void*>(cur);
     hc_pending fused = list[i];
     memcpy(fused.args.data(), &g, sizeof(g));
-    fused.tag = hc_pending::NONE;
+    fused.tag = hc_pending::PRODUCT;   // (no further operations are merged; it may still join a group)
     fused.reads = inputs;
     fused.writes = {cur};
     fused.out = const_cast<void*>(cur);

@@ -339,9 +339,18 @@ typedef struct {
   /* Two-level batch (direct-to-LDS kernels only; 0 = off): slice z lies at
    * (z / bdiv) * x_bs + (z % bdiv) * x_bs2. What a batched product reads or writes when a
    * recording folds a swap of the batch axes ([B, T, H, d] <-> [B, H, T, d]) into it. */
-  uint32_t bdiv, pad2;
+  uint32_t bdiv;
+  /* A group of up to HCK_GEMM_GROUP products over the same A with the same shape, operations and
+   * strides in one launch (direct-to-LDS kernels only; 0 = off): blockIdx.y picks the member's B,
+   * C and epilogue operands from the tables. What a recording makes of the q, k, v projections of
+   * an attention layer. */
+  uint32_t group;
   uint64_t a_bs2, b_bs2, c_bs2;
+  const void* g_b[4];
+  void* g_c[4];
+  const void* g_ep[3][4];
 } hck_gemm_args;
+#define HCK_GEMM_GROUP 4
 
 #define HCK_EP_NONE 0
 #define HCK_EP_ADD_ROW 1     /* x + row[n]   (a bias broadcast over the rows) */

@@ -225,6 +225,15 @@ __device__ __forceinline__ void gemm_tile_of_block(const hck_gemm_args& p, uint3
 // element-wise kernels would have produced. A lane's pieces all lie in the same columns, so the row
 // operands (a bias) are fetched once per kernel; the matrix operand (at most one of the three
 // operations) is fetched for a few pieces at a time, all loads in flight before the first use.
+// The operands of the three stages for this workgroup's product (a member of a group has its own).
+struct GemmEpilogueOperands {
+  const void *p0, *p1, *p2;
+};
+__device__ __forceinline__ GemmEpilogueOperands gemm_epilogue_operands(const hck_gemm_args& p, uint32_t member) {
+  if (p.group != 0) return GemmEpilogueOperands{p.g_ep[0][member], p.g_ep[1][member], p.g_ep[2][member]};
+  return GemmEpilogueOperands{p.ep_ptr[0], p.ep_ptr[1], p.ep_ptr[2]};
+}
+
 template <typename T, typename Chunk16>
 __device__ __forceinline__ Chunk16 gemm_epilogue_row_piece(uint32_t kind, const void* ptr, uint32_t col, bool col_ok) {
   constexpr int V = 16 / sizeof(T);
@@ -248,12 +257,12 @@ __device__ __forceinline__ Chunk16 gemm_epilogue_row_piece(uint32_t kind, const 
 
 // the matrix operand's piece for the output piece at (row, col); zeros if there is none
 template <typename T, typename Chunk16>
-__device__ __forceinline__ Chunk16 gemm_epilogue_matrix_piece(const hck_gemm_args& p, uint32_t row, uint32_t col) {
+__device__ __forceinline__ Chunk16 gemm_epilogue_matrix_piece(const hck_gemm_args& p, const GemmEpilogueOperands& ops,
+                                                              uint32_t row, uint32_t col) {
   Chunk16 m = Chunk16{};
-#pragma unroll
-  for (int s = 0; s < 3; s++)
-    if (p.ep_kind[s] == HCK_EP_ADD_MATRIX)
-      m = *reinterpret_cast<const Chunk16*>((const T*)p.ep_ptr[s] + (size_t)row * p.ep_ld[s] + col);
+  if (p.ep_kind[0] == HCK_EP_ADD_MATRIX) m = *reinterpret_cast<const Chunk16*>((const T*)ops.p0 + (size_t)row * p.ep_ld[0] + col);
+  if (p.ep_kind[1] == HCK_EP_ADD_MATRIX) m = *reinterpret_cast<const Chunk16*>((const T*)ops.p1 + (size_t)row * p.ep_ld[1] + col);
+  if (p.ep_kind[2] == HCK_EP_ADD_MATRIX) m = *reinterpret_cast<const Chunk16*>((const T*)ops.p2 + (size_t)row * p.ep_ld[2] + col);
   return m;
 }
 
@@ -302,8 +311,9 @@ __device__ __forceinline__ Chunk16 gemm_epilogue_apply(const hck_gemm_args& p, C
 // are the row operands for them (fetched once per kernel); otherwise they are fetched per piece.
 // `matrix` (wave-uniform): one of the operations has a matrix operand.
 template <typename T, typename Chunk16, bool EDGE, uint32_t GROUP, bool COL_FIXED, typename LdsPiece, typename RowOf, typename ColOf>
-__device__ __forceinline__ void gemm_store_group_merged(const hck_gemm_args& p, bool matrix, Chunk16 r0, Chunk16 r1, Chunk16 r2,
-                                                        T* C, uint32_t it0, LdsPiece lds_piece, RowOf row_of, ColOf col_of) {
+__device__ __forceinline__ void gemm_store_group_merged(const hck_gemm_args& p, const GemmEpilogueOperands& ops, bool matrix,
+                                                        Chunk16 r0, Chunk16 r1, Chunk16 r2, T* C, uint32_t it0, LdsPiece lds_piece,
+                                                        RowOf row_of, ColOf col_of) {
   Chunk16 v[GROUP], m[GROUP], q0[GROUP], q1[GROUP], q2[GROUP];
 #pragma unroll
   for (uint32_t b = 0; b < GROUP; b++) {
@@ -311,15 +321,15 @@ __device__ __forceinline__ void gemm_store_group_merged(const hck_gemm_args& p, 
     const bool inside = !EDGE || (row < p.M && col < p.N);
     v[b] = lds_piece(it0 + b);
     m[b] = Chunk16{};
-    q0[b] = COL_FIXED ? r0 : gemm_epilogue_row_piece<T, Chunk16>(p.ep_kind[0], p.ep_ptr[0], col, inside);
-    q1[b] = COL_FIXED ? r1 : gemm_epilogue_row_piece<T, Chunk16>(p.ep_kind[1], p.ep_ptr[1], col, inside);
-    q2[b] = COL_FIXED ? r2 : gemm_epilogue_row_piece<T, Chunk16>(p.ep_kind[2], p.ep_ptr[2], col, inside);
+    q0[b] = COL_FIXED ? r0 : gemm_epilogue_row_piece<T, Chunk16>(p.ep_kind[0], ops.p0, col, inside);
+    q1[b] = COL_FIXED ? r1 : gemm_epilogue_row_piece<T, Chunk16>(p.ep_kind[1], ops.p1, col, inside);
+    q2[b] = COL_FIXED ? r2 : gemm_epilogue_row_piece<T, Chunk16>(p.ep_kind[2], ops.p2, col, inside);
   }
   if (matrix) {
 #pragma unroll
     for (uint32_t b = 0; b < GROUP; b++) {
       const uint32_t row = row_of(it0 + b), col = col_of(it0 + b);
-      if (!EDGE || (row < p.M && col < p.N)) m[b] = gemm_epilogue_matrix_piece<T, Chunk16>(p, row, col);
+      if (!EDGE || (row < p.M && col < p.N)) m[b] = gemm_epilogue_matrix_piece<T, Chunk16>(p, ops, row, col);
     }
   }
 #pragma unroll
@@ -334,15 +344,15 @@ __device__ __forceinline__ void gemm_store_group_merged(const hck_gemm_args& p, 
 // LDS, not the accumulators, and copies of it for every slab would multiply the kernel's code).
 template <typename T, typename Chunk16, bool EDGE, uint32_t NIT, bool COL_FIXED, uint32_t MAX_GROUP, typename LdsPiece,
           typename RowOf, typename ColOf>
-__device__ __forceinline__ void gemm_store_slab_merged(const hck_gemm_args& p, Chunk16 r0, Chunk16 r1, Chunk16 r2, T* C,
-                                                       LdsPiece lds_piece, RowOf row_of, ColOf col_of) {
+__device__ __forceinline__ void gemm_store_slab_merged(const hck_gemm_args& p, const GemmEpilogueOperands& ops, Chunk16 r0,
+                                                       Chunk16 r1, Chunk16 r2, T* C, LdsPiece lds_piece, RowOf row_of, ColOf col_of) {
   constexpr uint32_t GROUP = (MAX_GROUP >= 4 && NIT % 4 == 0) ? 4 : (MAX_GROUP >= 3 && NIT % 3 == 0) ? 3 : NIT % 2 == 0 ? 2 : 1;
   const bool matrix = p.ep_kind[0] == HCK_EP_ADD_MATRIX || p.ep_kind[1] == HCK_EP_ADD_MATRIX || p.ep_kind[2] == HCK_EP_ADD_MATRIX;
   if constexpr (NIT == GROUP) {
-    gemm_store_group_merged<T, Chunk16, EDGE, GROUP, COL_FIXED>(p, matrix, r0, r1, r2, C, 0u, lds_piece, row_of, col_of);
+    gemm_store_group_merged<T, Chunk16, EDGE, GROUP, COL_FIXED>(p, ops, matrix, r0, r1, r2, C, 0u, lds_piece, row_of, col_of);
   } else {
 #pragma nounroll
     for (uint32_t it0 = 0; it0 < NIT; it0 += GROUP)
-      gemm_store_group_merged<T, Chunk16, EDGE, GROUP, COL_FIXED>(p, matrix, r0, r1, r2, C, it0, lds_piece, row_of, col_of);
+      gemm_store_group_merged<T, Chunk16, EDGE, GROUP, COL_FIXED>(p, ops, matrix, r0, r1, r2, C, it0, lds_piece, row_of, col_of);
   }
 }

@@ -222,6 +222,12 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
   const T* A = (const T*)p.a + batch_hi * p.a_bs + batch_lo * p.a_bs2;
   const T* B = (const T*)p.b + batch_hi * p.b_bs + batch_lo * p.b_bs2;
   T* C = (T*)p.c + batch_hi * p.c_bs + batch_lo * p.c_bs2;
+  if (p.group != 0) {  // a member of a group of products over the same A
+    A = (const T*)p.a;
+    B = (const T*)p.g_b[batch];
+    C = (T*)p.g_c[batch];
+  }
+  const GemmEpilogueOperands ep_ops = gemm_epilogue_operands(p, batch);
 
   const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const uint32_t wm = (wave >> 1) * (BM / 2), wn = (wave & 1) * (BN / 2);
@@ -369,9 +375,9 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
   Chunk ep_r0 = Chunk{}, ep_r1 = Chunk{}, ep_r2 = Chunk{};
   if (EP_COL_FIXED && p.ep_kind[0] != HCK_EP_NONE) {
     const bool ok = !EDGE || ep_col < p.N;
-    ep_r0 = gemm_epilogue_row_piece<T, Chunk>(p.ep_kind[0], p.ep_ptr[0], ep_col, ok);
-    ep_r1 = gemm_epilogue_row_piece<T, Chunk>(p.ep_kind[1], p.ep_ptr[1], ep_col, ok);
-    ep_r2 = gemm_epilogue_row_piece<T, Chunk>(p.ep_kind[2], p.ep_ptr[2], ep_col, ok);
+    ep_r0 = gemm_epilogue_row_piece<T, Chunk>(p.ep_kind[0], ep_ops.p0, ep_col, ok);
+    ep_r1 = gemm_epilogue_row_piece<T, Chunk>(p.ep_kind[1], ep_ops.p1, ep_col, ok);
+    ep_r2 = gemm_epilogue_row_piece<T, Chunk>(p.ep_kind[2], ep_ops.p2, ep_col, ok);
   }
   const uint32_t r16 = lane & 15, grp = lane >> 4;
 #pragma unroll
@@ -402,7 +408,7 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
       }
     } else {
       gemm_store_slab_merged<T, Chunk, EDGE, 32 * UNITS / 64, EP_COL_FIXED, 2>(
-          p, ep_r0, ep_r1, ep_r2, C,
+          p, ep_ops, ep_r0, ep_r1, ep_r2, C,
           [=](uint32_t it) {
             const uint32_t piece = it * 64 + lane, r = piece / UNITS, u = piece % UNITS;
             return *reinterpret_cast<const Chunk*>(slab + r * RB + ((u ^ unit_swz(r)) * 16));

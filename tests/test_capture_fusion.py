@@ -216,6 +216,44 @@ def test_softmax_forms_that_are_left_alone(hip_backend, monkeypatch):
 
 
 @pytest.mark.parametrize("dtype", [DType.float32, DType.float16], ids=["f32", "f16"])
+@pytest.mark.parametrize("m,k,n", [(2048, 512, 512), (192, 72, 136)])
+def test_products_over_the_same_input_share_a_launch(hip_backend, monkeypatch, dtype, m, k, n):
+    """q, k, v = three Linear layers of one shape applied to the same activations."""
+    rng = np.random.default_rng(m + k)
+    cast = DType.float16 if dtype == DType.float16 else None
+    with hip_backend.use():
+        x = Tensor(data=rng.standard_normal((m, k)).astype(np.float32), dtype=dtype)
+        lins = [Linear(k, n, rng, dtype=dtype, castParams=cast) for _ in range(5)]
+        for lin in lins:
+            lin.bias = Tensor(data=rng.standard_normal((n,)).astype(np.float32))
+        other = Linear(k, n + 8, rng, dtype=dtype, castParams=cast)
+        per_linear = 2 if dtype == DType.float16 else 1      # bias add (and the bias's cast) merged into each product
+
+        def three():
+            q, kk, v = (lin(x) for lin in lins[:3])
+            return q * kk * v           # (products of results: nothing else to merge into the matmuls)
+
+        check(hip_backend, monkeypatch, three, removed=3 * per_linear + 2)
+
+        def five():          # at most four products per launch: the fifth stays alone
+            outs = [lin(x) for lin in lins]
+            return ((outs[0] * outs[1]) * (outs[2] * outs[3])) * outs[4]
+
+        check(hip_backend, monkeypatch, five, removed=5 * per_linear + 3)
+
+        def chained():       # the second product reads the first one's result: no group
+            h = lins[0](x)
+            return lins[1](h) if k == n else lins[1](x) * h.gelu()
+
+        check(hip_backend, monkeypatch, chained, removed=2 * per_linear + (0 if k == n else 1))
+
+        def different_shapes():
+            return lins[0](x).sum(axis=1) * other(x).sum(axis=1)
+
+        check(hip_backend, monkeypatch, different_shapes, removed=2 * per_linear)
+
+
+@pytest.mark.parametrize("dtype", [DType.float32, DType.float16], ids=["f32", "f16"])
 @pytest.mark.parametrize("B,T,H,hd", [(8, 256, 8, 64), (2, 96, 3, 40), (1, 128, 4, 64)])
 def test_head_swaps_fold_into_the_batched_products(hip_backend, monkeypatch, dtype, B, T, H, hd):
     """[B, T, H*hd] -> [B, T, H, hd] -> swap(1, 2) around batchedMatmul: the products read q, k, v
@@ -263,12 +301,12 @@ def test_config5_forward_recorded_with_the_rewrite(hip_backend, monkeypatch, dty
         plain.launch()
         assert np.array_equal(plain_out.numpy(), want)
         # per block: q, k, v (+bias), o and fc2 (+bias, +residual), fc1 (+bias, GELU) = 9 launches
-        # merged into products, 2 LayerNorms of 3 launches (fp16: 5), a softmax of 4 and the 4 swaps
-        # of the heads; then the last LayerNorm and the unembedding's bias; in fp16 also the 6 + 1
-        # casts of the fp32 biases
+        # merged into products, 2 LayerNorms of 3 launches (fp16: 5), a softmax of 4, the 4 swaps of
+        # the heads, and q, k, v in one launch; then the last LayerNorm and the unembedding's bias;
+        # in fp16 also the 6 + 1 casts of the fp32 biases
         half = dtype == DType.float16
-        per_block = 9 + 2 * (4 if half else 2) + 3 + 4 + (6 if half else 0)
+        per_block = 9 + 2 * (4 if half else 2) + 3 + 4 + 2 + (6 if half else 0)
         assert plain_nodes - fused_nodes == 6 * per_block + (4 if half else 2) + (2 if half else 1)
-        assert fused_nodes == 70
+        assert fused_nodes == 58
         plain.destroy()
         fused.destroy()
