@@ -528,20 +528,29 @@ def extra_workloads(backend, graph=True, only=("cfg1", "cfg2", "cfg3", "cfg4", "
                              "tflops": round(100.9e9 / dt / 1e12, 2)}
                 if not graph:
                     continue
-                # the same forward pass recorded once and replayed as one graph launch
-                with backend.capture() as cap:
-                    logits = model(tokens)
-                for _ in range(3):
-                    cap.graph.launch()
-                logits.wait()
-                t0 = time.perf_counter()
-                for _ in range(20):
-                    cap.graph.launch()
+                # the same forward pass recorded once and replayed as one graph launch: as recorded
+                # (one launch per backend call), and with the recording's rewrite, which merges
+                # bias / GELU / residual into the products, LayerNorm and softmax chains into one
+                # kernel each, the head swaps into the batched products and q, k, v into one launch
+                for suffix, env in (("_graph_unmerged", "1"), ("_graph", None)):
+                    if env:
+                        os.environ["HCHIP_NO_FUSION"] = env
+                    try:
+                        with backend.capture() as cap:
+                            logits = model(tokens)
+                    finally:
+                        os.environ.pop("HCHIP_NO_FUSION", None)
+                    for _ in range(5):
+                        cap.graph.launch()
                     logits.wait()
-                dt = (time.perf_counter() - t0) / 20
-                out[name + "_graph"] = {"ms": round(dt * 1e3, 3), "tokens_per_s": round(2048 / dt, 1),
-                                        "tflops": round(100.9e9 / dt / 1e12, 2)}
-                cap.graph.destroy()
+                    t0 = time.perf_counter()
+                    for _ in range(20):
+                        cap.graph.launch()
+                        logits.wait()
+                    dt = (time.perf_counter() - t0) / 20
+                    out[name + suffix] = {"ms": round(dt * 1e3, 3), "tokens_per_s": round(2048 / dt, 1),
+                                          "tflops": round(100.9e9 / dt / 1e12, 2), "launches": cap.graph.node_count()}
+                    cap.graph.destroy()
 
     for name, fn in (("cfg1", cfg1), ("cfg2", cfg2), ("cfg3", cfg3), ("cfg4", cfg4), ("cfg5", cfg5)):
         if name in only:

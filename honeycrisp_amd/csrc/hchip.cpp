@@ -743,8 +743,8 @@ extern "C" int hc_graph_destroy(hc_ctx* ctx, hc_graph* graph) {
 // kernel do that reader's work on the tile it is about to store:
 //     matmul -> + bias row -> GELU          (Linear followed by an activation)
 //     matmul -> + bias row -> + residual    (Linear inside a residual connection)
-// (up to three operations, one of them with a matrix operand) with the bias row possibly cast
-// from fp32 on the way. The merged operations are applied with
+// (up to three operations, one of them with a matrix operand; GELU only as the last, and not
+// after a matrix operand) with the bias row possibly cast from fp32 on the way. The merged operations are applied with
 // the arithmetic of the kernels they replace (each one on the value rounded to the output type),
 // so a replay produces the bits the unmerged sequence produces. HCHIP_NO_FUSION=1 at
 // hc_capture_begin turns the rewrite off.
@@ -1214,7 +1214,9 @@ static void fuse_products(hc_ctx* ctx, std::vector<hc_pending>& list, const Free
       if (c.kind != hc_pending::KERNEL || c.dtype != dtype || !c.out || !aligned16(c.out)) break;
       uint32_t kind = HCK_EP_NONE;
       const void* other = nullptr;
-      if (c.tag == hc_pending::GELU && c.in0 == cur && c.cols == M * N) {
+      bool has_matrix = false;
+      for (int s = 0; s < nops; s++) has_matrix = has_matrix || g.ep_kind[s] == HCK_EP_ADD_MATRIX;
+      if (c.tag == hc_pending::GELU && c.in0 == cur && c.cols == M * N && !has_matrix) {
         kind = HCK_EP_GELU;
       } else if (c.tag == hc_pending::ADD && (c.in0 == cur) != (c.in1 == cur)) {
         const bool first = c.in0 == cur;
@@ -1240,12 +1242,14 @@ static void fuse_products(hc_ctx* ctx, std::vector<hc_pending>& list, const Free
       if (!clean) break;
       g.ep_kind[nops] = kind;
       g.ep_ptr[nops] = other;
+      const bool ends_list = kind == HCK_EP_GELU;   // (the kernels apply GELU after the additions)
       g.ep_ld[nops] = (uint32_t)N;
       if (other) inputs.push_back(other);
       merged.push_back((size_t)j);
       cur = c.out;
       pos = (size_t)j;
       nops++;
+      if (ends_list) break;
     }
     if (nops == 0) continue;
     // a bias row that is an fp32 parameter cast to fp16 just for this addition: read the fp32 row

@@ -355,7 +355,7 @@ typedef struct {
 #define HCK_EP_NONE 0
 #define HCK_EP_ADD_ROW 1     /* x + row[n]   (a bias broadcast over the rows) */
 #define HCK_EP_ADD_MATRIX 2  /* x + other[m, n] (a residual connection) */
-#define HCK_EP_GELU 3        /* ElemwiseOp.geluApprox */
+#define HCK_EP_GELU 3        /* ElemwiseOp.geluApprox; only as the last operation of the list */
 #define HCK_EP_ADD_ROW_F32 4 /* x + T(row[n]) with the row held in fp32 (a parameter cast at call time) */
 
 /* Copy of a batch of [rows, in_cols] matrices with leading dimension in_ld into [rows, out_cols]

@@ -255,50 +255,44 @@ __device__ __forceinline__ Chunk16 gemm_epilogue_row_piece(uint32_t kind, const 
   return out;
 }
 
-// the matrix operand's piece for the output piece at (row, col); zeros if there is none
+// the matrix operand's piece for the output piece at (row, col); one of the stages has one
 template <typename T, typename Chunk16>
 __device__ __forceinline__ Chunk16 gemm_epilogue_matrix_piece(const hck_gemm_args& p, const GemmEpilogueOperands& ops,
                                                               uint32_t row, uint32_t col) {
-  Chunk16 m = Chunk16{};
-  if (p.ep_kind[0] == HCK_EP_ADD_MATRIX) m = *reinterpret_cast<const Chunk16*>((const T*)ops.p0 + (size_t)row * p.ep_ld[0] + col);
-  if (p.ep_kind[1] == HCK_EP_ADD_MATRIX) m = *reinterpret_cast<const Chunk16*>((const T*)ops.p1 + (size_t)row * p.ep_ld[1] + col);
-  if (p.ep_kind[2] == HCK_EP_ADD_MATRIX) m = *reinterpret_cast<const Chunk16*>((const T*)ops.p2 + (size_t)row * p.ep_ld[2] + col);
-  return m;
+  // (stage picked with scalar selects, then a single load: no register is written twice)
+  const bool s0 = p.ep_kind[0] == HCK_EP_ADD_MATRIX, s1 = p.ep_kind[1] == HCK_EP_ADD_MATRIX;
+  const void* base = s0 ? ops.p0 : s1 ? ops.p1 : ops.p2;
+  const uint32_t ld = s0 ? p.ep_ld[0] : s1 ? p.ep_ld[1] : p.ep_ld[2];
+  return *reinterpret_cast<const Chunk16*>((const T*)base + (size_t)row * ld + col);
 }
 
 // r0, r1, r2: the row operands of the three stages (gemm_epilogue_row_piece; passed as three values
-// so that nothing can index them and they stay in registers)
-template <typename T, typename Chunk16>
+// so that nothing can index them and they stay in registers). Straight-line code: up to three
+// additions (wave-uniform branches skip the absent ones), then, in the GELU instantiation, the
+// activation: the host puts GELU only at the end of a list, and never together with a matrix
+// operand. (A loop over the stages with the operation picked inside cost 7 us on a 256 x 256 tile
+// for a single bias addition; this form costs 1 us.)
+template <typename T, typename Chunk16, bool MATRIX, bool GELU>
 __device__ __forceinline__ Chunk16 gemm_epilogue_apply(const hck_gemm_args& p, Chunk16 v, Chunk16 r0, Chunk16 r1, Chunk16 r2,
                                                        Chunk16 matrix_piece) {
   constexpr int V = 16 / sizeof(T);
   T x[V];
   __builtin_memcpy(x, &v, 16);
-  // One copy of the code for the three stages (the stage's kind and operand are picked with
-  // selects): this function is instantiated for every slab of the tile.
   const uint32_t k0 = p.ep_kind[0], k1 = p.ep_kind[1], k2 = p.ep_kind[2];
-#pragma nounroll
-  for (int s = 0; s < 3; s++) {
-    const uint32_t kind = s == 0 ? k0 : s == 1 ? k1 : k2;
-    if (kind == HCK_EP_NONE) break;
-    if (kind == HCK_EP_GELU) {
+  auto add = [&](uint32_t kind, Chunk16 row) {
+    const Chunk16 w = MATRIX && kind == HCK_EP_ADD_MATRIX ? matrix_piece : row;
+    T y[V];
+    __builtin_memcpy(y, &w, 16);
 #pragma unroll
-      for (int e = 0; e < V; e++) x[e] = narrow<T>(gelu_approx<sizeof(T) == 2>((float)x[e]) * 1.0f);
-    } else {
-      Chunk16 w = s == 0 ? r0 : s == 1 ? r1 : r2;
-      if (kind == HCK_EP_ADD_MATRIX) {
-        // The loaded piece is used inside this branch only (the empty asm keeps the compiler from
-        // turning the branch into a select): loads and stores share one in-order counter, and a
-        // wait for this load on the common path would also wait, in every product without a
-        // matrix operand, for all the stores issued so far.
-        w = matrix_piece;
-        asm volatile("" : "+v"(w));
-      }
-      T y[V];
-      __builtin_memcpy(y, &w, 16);
+    for (int e = 0; e < V; e++) x[e] = narrow<T>((float)x[e] + (float)y[e]);
+  };
+  auto is_add = [](uint32_t kind) { return kind == HCK_EP_ADD_ROW || kind == HCK_EP_ADD_ROW_F32 || kind == HCK_EP_ADD_MATRIX; };
+  if (is_add(k0)) add(k0, r0);
+  if (is_add(k1)) add(k1, r1);
+  if (is_add(k2)) add(k2, r2);
+  if (GELU) {
 #pragma unroll
-      for (int e = 0; e < V; e++) x[e] = narrow<T>((float)x[e] + (float)y[e]);
-    }
+    for (int e = 0; e < V; e++) x[e] = narrow<T>(gelu_approx<sizeof(T) == 2>((float)x[e]) * 1.0f);
   }
   Chunk16 out;
   __builtin_memcpy(&out, x, 16);
@@ -309,50 +303,64 @@ __device__ __forceinline__ Chunk16 gemm_epilogue_apply(const hck_gemm_args& p, C
 // first, then the arithmetic. lds_piece(it) reads piece `it` from the slab; row_of(it), col_of(it)
 // say where it goes in C. COL_FIXED: all of a lane's pieces lie in the same columns and r0, r1, r2
 // are the row operands for them (fetched once per kernel); otherwise they are fetched per piece.
-// `matrix` (wave-uniform): one of the operations has a matrix operand.
-template <typename T, typename Chunk16, bool EDGE, uint32_t GROUP, bool COL_FIXED, typename LdsPiece, typename RowOf, typename ColOf>
-__device__ __forceinline__ void gemm_store_group_merged(const hck_gemm_args& p, const GemmEpilogueOperands& ops, bool matrix,
-                                                        Chunk16 r0, Chunk16 r1, Chunk16 r2, T* C, uint32_t it0, LdsPiece lds_piece,
-                                                        RowOf row_of, ColOf col_of) {
-  Chunk16 v[GROUP], m[GROUP], q0[GROUP], q1[GROUP], q2[GROUP];
+// MATRIX: one of the operations has a matrix operand. Loads and stores share one in-order counter:
+// code that loads in a loop waits, before it touches the loaded registers again, for everything
+// older, stores included. The variants without a matrix operand therefore are instantiations of
+// their own in which no such register exists, and their stores are never waited for.
+template <typename T, typename Chunk16, bool EDGE, uint32_t GROUP, bool COL_FIXED, bool MATRIX, bool GELU, typename LdsPiece,
+          typename RowOf, typename ColOf>
+__device__ __forceinline__ void gemm_store_group_merged(const hck_gemm_args& p, const GemmEpilogueOperands& ops, Chunk16 r0,
+                                                        Chunk16 r1, Chunk16 r2, T* C, uint32_t it0, LdsPiece lds_piece, RowOf row_of,
+                                                        ColOf col_of) {
+  Chunk16 v[GROUP], m[MATRIX ? GROUP : 1], q0[GROUP], q1[GROUP], q2[GROUP];
 #pragma unroll
   for (uint32_t b = 0; b < GROUP; b++) {
     const uint32_t row = row_of(it0 + b), col = col_of(it0 + b);
     const bool inside = !EDGE || (row < p.M && col < p.N);
     v[b] = lds_piece(it0 + b);
-    m[b] = Chunk16{};
+    if (MATRIX) m[b] = inside ? gemm_epilogue_matrix_piece<T, Chunk16>(p, ops, row, col) : Chunk16{};
     q0[b] = COL_FIXED ? r0 : gemm_epilogue_row_piece<T, Chunk16>(p.ep_kind[0], ops.p0, col, inside);
     q1[b] = COL_FIXED ? r1 : gemm_epilogue_row_piece<T, Chunk16>(p.ep_kind[1], ops.p1, col, inside);
     q2[b] = COL_FIXED ? r2 : gemm_epilogue_row_piece<T, Chunk16>(p.ep_kind[2], ops.p2, col, inside);
-  }
-  if (matrix) {
-#pragma unroll
-    for (uint32_t b = 0; b < GROUP; b++) {
-      const uint32_t row = row_of(it0 + b), col = col_of(it0 + b);
-      if (!EDGE || (row < p.M && col < p.N)) m[b] = gemm_epilogue_matrix_piece<T, Chunk16>(p, ops, row, col);
-    }
   }
 #pragma unroll
   for (uint32_t b = 0; b < GROUP; b++) {
     const uint32_t row = row_of(it0 + b), col = col_of(it0 + b);
     if (!EDGE || (row < p.M && col < p.N))
-      *reinterpret_cast<Chunk16*>(C + (size_t)row * p.c_rs + col) = gemm_epilogue_apply<T, Chunk16>(p, v[b], q0[b], q1[b], q2[b], m[b]);
+      *reinterpret_cast<Chunk16*>(C + (size_t)row * p.c_rs + col) =
+          gemm_epilogue_apply<T, Chunk16, MATRIX, GELU>(p, v[b], q0[b], q1[b], q2[b], MATRIX ? m[MATRIX ? b : 0] : Chunk16{});
   }
 }
 
 // The NIT pieces of a slab in groups of at most MAX_GROUP: a loop that is not unrolled (it reads
 // LDS, not the accumulators, and copies of it for every slab would multiply the kernel's code).
+template <typename T, typename Chunk16, bool EDGE, uint32_t NIT, bool COL_FIXED, uint32_t MAX_GROUP, bool MATRIX, bool GELU,
+          typename LdsPiece, typename RowOf, typename ColOf>
+__device__ __forceinline__ void gemm_store_slab_merged_as(const hck_gemm_args& p, const GemmEpilogueOperands& ops, Chunk16 r0,
+                                                          Chunk16 r1, Chunk16 r2, T* C, LdsPiece lds_piece, RowOf row_of,
+                                                          ColOf col_of) {
+  constexpr uint32_t GROUP = (MAX_GROUP >= 4 && NIT % 4 == 0) ? 4 : (MAX_GROUP >= 3 && NIT % 3 == 0) ? 3 : (MAX_GROUP >= 2 && NIT % 2 == 0) ? 2 : 1;
+  if constexpr (NIT == GROUP) {
+    gemm_store_group_merged<T, Chunk16, EDGE, GROUP, COL_FIXED, MATRIX, GELU>(p, ops, r0, r1, r2, C, 0u, lds_piece, row_of, col_of);
+  } else {
+#pragma nounroll
+    for (uint32_t it0 = 0; it0 < NIT; it0 += GROUP)
+      gemm_store_group_merged<T, Chunk16, EDGE, GROUP, COL_FIXED, MATRIX, GELU>(p, ops, r0, r1, r2, C, it0, lds_piece, row_of, col_of);
+  }
+}
+
 template <typename T, typename Chunk16, bool EDGE, uint32_t NIT, bool COL_FIXED, uint32_t MAX_GROUP, typename LdsPiece,
           typename RowOf, typename ColOf>
 __device__ __forceinline__ void gemm_store_slab_merged(const hck_gemm_args& p, const GemmEpilogueOperands& ops, Chunk16 r0,
                                                        Chunk16 r1, Chunk16 r2, T* C, LdsPiece lds_piece, RowOf row_of, ColOf col_of) {
-  constexpr uint32_t GROUP = (MAX_GROUP >= 4 && NIT % 4 == 0) ? 4 : (MAX_GROUP >= 3 && NIT % 3 == 0) ? 3 : NIT % 2 == 0 ? 2 : 1;
   const bool matrix = p.ep_kind[0] == HCK_EP_ADD_MATRIX || p.ep_kind[1] == HCK_EP_ADD_MATRIX || p.ep_kind[2] == HCK_EP_ADD_MATRIX;
-  if constexpr (NIT == GROUP) {
-    gemm_store_group_merged<T, Chunk16, EDGE, GROUP, COL_FIXED>(p, ops, matrix, r0, r1, r2, C, 0u, lds_piece, row_of, col_of);
-  } else {
-#pragma nounroll
-    for (uint32_t it0 = 0; it0 < NIT; it0 += GROUP)
-      gemm_store_group_merged<T, Chunk16, EDGE, GROUP, COL_FIXED>(p, ops, matrix, r0, r1, r2, C, it0, lds_piece, row_of, col_of);
-  }
+  const bool gelu = p.ep_kind[0] == HCK_EP_GELU || p.ep_kind[1] == HCK_EP_GELU || p.ep_kind[2] == HCK_EP_GELU;
+  // (the activation is long enough to hide the latencies of one piece: its loop takes the pieces
+  // one by one, which keeps that code to one copy per slab)
+  if (gelu)
+    gemm_store_slab_merged_as<T, Chunk16, EDGE, NIT, COL_FIXED, 1, false, true>(p, ops, r0, r1, r2, C, lds_piece, row_of, col_of);
+  else if (matrix)
+    gemm_store_slab_merged_as<T, Chunk16, EDGE, NIT, COL_FIXED, MAX_GROUP, true, false>(p, ops, r0, r1, r2, C, lds_piece, row_of, col_of);
+  else
+    gemm_store_slab_merged_as<T, Chunk16, EDGE, NIT, COL_FIXED, MAX_GROUP, false, false>(p, ops, r0, r1, r2, C, lds_piece, row_of, col_of);
 }

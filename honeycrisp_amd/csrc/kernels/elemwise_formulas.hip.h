@@ -18,9 +18,9 @@ __device__ __forceinline__ float safe_tanh(float x) { return 2.0f * safe_sigmoid
 // load), not by memory.
 __device__ __forceinline__ float exp_hw(float x) { return __builtin_amdgcn_exp2f(x * 1.4426950408889634f); }
 __device__ __forceinline__ float sigmoid_hw(float x) {
-  if (x < -20.0f) return 0.0f;
-  if (x > 20.0f) return 1.0f;
-  return __builtin_amdgcn_rcpf(1.0f + exp_hw(-x));
+  // (computed first, then selected: no branch per element, so the elements of a vector overlap)
+  const float inside = __builtin_amdgcn_rcpf(1.0f + exp_hw(-x));
+  return x < -20.0f ? 0.0f : (x > 20.0f ? 1.0f : inside);
 }
 __device__ __forceinline__ float tanh_hw(float x) { return 2.0f * sigmoid_hw(2.0f * x) - 1.0f; }
 

@@ -79,7 +79,12 @@ def test_bias_and_residual_join_the_product(hip_backend, monkeypatch, dtype, m, 
         check(hip_backend, monkeypatch, lambda: (Tensor.matmul(x, False, w, False, False) + res) + res, removed=1)
         # three merged operations is the limit: the fourth stays a kernel of its own
         check(hip_backend, monkeypatch,
-              lambda: ((Tensor.matmul(x, False, w, False, False) + bias).gelu() + res).gelu(), removed=3)
+              lambda: (((Tensor.matmul(x, False, w, False, False) + bias) + bias) + res) + bias, removed=3)
+        # GELU ends a list, and does not follow a matrix operand
+        check(hip_backend, monkeypatch,
+              lambda: ((Tensor.matmul(x, False, w, False, False) + bias).gelu() + res).gelu(), removed=2)
+        check(hip_backend, monkeypatch,
+              lambda: (res + (Tensor.matmul(x, False, w, False, False) + bias)).gelu(), removed=2)
 
 
 def test_transposed_operands_and_a_three_axis_input(hip_backend, monkeypatch):
