@@ -783,6 +783,26 @@ static long sole_user(const std::vector<hc_pending>& list, size_t from, const vo
 struct Freed { size_t at, bytes; };
 typedef std::unordered_map<const void*, Freed> FreedMap;
 
+// Whether a write declared at `w` may change what a read declared at `r` sees: the two pointers
+// are the same, or one lies inside the other's block (the sizes of blocks that are live or were
+// released inside the recording are known; an unknown pointer counts as one byte).
+struct Overlap {
+  const hc_ctx* ctx;
+  const FreedMap* freed;
+  size_t size_of(const void* p) const {
+    auto live = ctx->live.find(const_cast<void*>(p));
+    if (live != ctx->live.end()) return live->second;
+    auto fr = freed->find(p);
+    return fr == freed->end() ? 1 : fr->second.bytes;
+  }
+  bool operator()(const void* w, const void* r) const {
+    if (!w || !r) return false;
+    return w == r || in_block(w, r, size_of(r)) || in_block(r, w, size_of(w));
+  }
+};
+static thread_local const Overlap* g_overlap = nullptr;   // set for the duration of fuse_recording
+static bool may_alias(const void* w, const void* r) { return g_overlap ? (*g_overlap)(w, r) : w == r; }
+
 // The tagged launch before entry `before` that produced the buffer `ptr`, or -1 (also when a
 // launch with undeclared buffers lies in between: it may have written `ptr`).
 static long producer_of(const std::vector<hc_pending>& list, size_t before, const void* ptr) {
@@ -792,7 +812,7 @@ static long producer_of(const std::vector<hc_pending>& list, size_t before, cons
     if (!e.known) return -1;
     if (e.kind == hc_pending::KERNEL && e.out == ptr) return (long)k;
     for (const void* w : e.writes)
-      if (w == ptr) return -1;
+      if (may_alias(w, ptr)) return -1;
   }
   return -1;
 }
@@ -825,7 +845,7 @@ static bool inputs_stable(const std::vector<hc_pending>& list, const std::vector
       if (!e.known) return false;
       for (const void* w : e.writes)
         for (const void* in : d.reads)
-          if (in && w == in) return false;
+          if (in && may_alias(w, in)) return false;
     }
   return true;
 }
@@ -1146,7 +1166,8 @@ static void fuse_product_groups(std::vector<hc_pending>& list, const FreedMap& f
         const hck_gemm_args& a = margs[m];
         conflict = uses(e, a.c);
         for (const void* w : e.writes)
-          conflict = conflict || w == a.a || w == a.b || w == a.ep_ptr[0] || w == a.ep_ptr[1] || w == a.ep_ptr[2];
+          conflict = conflict || may_alias(w, a.a) || may_alias(w, a.b) || may_alias(w, a.ep_ptr[0]) ||
+                     may_alias(w, a.ep_ptr[1]) || may_alias(w, a.ep_ptr[2]);
       }
       if (conflict) break;
       if (joins) {
@@ -1183,11 +1204,14 @@ static void fuse_recording(hc_ctx* ctx) {
   FreedMap freed;
   for (size_t i = 0; i < list.size(); i++)
     if (list[i].kind == hc_pending::FREE) freed[list[i].dst] = Freed{i, list[i].bytes};
+  const Overlap overlap{ctx, &freed};
+  g_overlap = &overlap;
   fuse_products(ctx, list, freed);
   fuse_swapped_batches(list, freed);
   fuse_layernorms(ctx, list, freed);
   fuse_softmaxes(ctx, list, freed);
   fuse_product_groups(list, freed);
+  g_overlap = nullptr;
 }
 
 static void fuse_products(hc_ctx* ctx, std::vector<hc_pending>& list, const FreedMap& freed) {
@@ -1237,7 +1261,7 @@ static void fuse_products(hc_ctx* ctx, std::vector<hc_pending>& list, const Free
         if (e.dropped || e.kind == hc_pending::FREE) continue;
         for (const void* in : inputs)
           for (const void* w : e.writes)
-            if (w == in) clean = false;
+            if (may_alias(w, in)) clean = false;
       }
       if (!clean) break;
       g.ep_kind[nops] = kind;
@@ -1266,7 +1290,7 @@ static void fuse_products(hc_ctx* ctx, std::vector<hc_pending>& list, const Free
           bool clean = true;   // the fp32 row must still hold the same values where the product now runs
           for (size_t k2 = c2 + 1; k2 < pos && clean; k2++)
             for (const void* w : list[k2].writes)
-              if (!list[k2].dropped && w == e.in0) clean = false;
+              if (!list[k2].dropped && may_alias(w, e.in0)) clean = false;
           if (!clean) break;
           for (const void*& in : inputs)
             if (in == g.ep_ptr[s]) in = e.in0;

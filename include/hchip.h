@@ -152,11 +152,21 @@ int hc_launch_host_func(hc_ctx* ctx, void (*fn)(void*), void* user);
  *  - Host transfers, hc_sync, event and host-function calls are refused while capturing
  *    (HC_ERR_INVALID). One capture at a time per context.
  *  - The launches of a capture are listed first and enqueued at hc_capture_end, after a
- *    rewrite that merges the single reader of a product's result into the product's kernel
- *    (matmul -> + bias row -> geluApprox, matmul -> + bias row -> + other matrix; the row may
- *    be an fp32 buffer cast to fp16 for the addition). The merged kernel applies each
- *    operation to the value rounded to the output type, so a replay returns the bits of the
- *    unmerged sequence. Intermediate buffers that were merged away are never written.
+ *    rewrite. Every entry point declares the buffers it reads and writes, every buffer has
+ *    an address of its own while the capture lasts, and hc_free says that a buffer has no
+ *    further reader: from that alone the rewrite sees results with a single reader and
+ *    replaces chains of launches by one launch that does the same arithmetic, intermediate
+ *    by intermediate, so a replay returns the bits of the unmerged sequence:
+ *      matmul -> + row -> [+ matrix | geluApprox]   one product with an epilogue (the row may
+ *                                                    be an fp32 buffer cast to fp16 on the way)
+ *      [cast ->] normalize -> [(gain + c) *, + bias] -> [cast]      one LayerNorm kernel
+ *      [* s ->] [+ mask ->] logSoftmax -> [exp]                     one softmax kernel
+ *      swap of two batch axes -> batchedMatmul -> swap back         read / written through strides
+ *      products of one shape over the same input (q, k, v)          one launch
+ *    Buffers that only held merged intermediates are never written by a replay.
+ *    HCHIP_RECORDING_LOG=1 at hc_capture_end lists the launches of the rewritten recording on
+ *    stderr; HCHIP_GRAPH_AS_LAUNCHES=1 makes hc_graph_launch issue them one by one instead of
+ *    through hipGraphLaunch (for kernel traces).
  *    HCHIP_NO_FUSION=1 in the environment at hc_capture_begin turns the rewrite off. */
 typedef struct hc_graph hc_graph;
 int hc_capture_begin(hc_ctx* ctx);

@@ -134,6 +134,34 @@ def test_a_result_the_caller_keeps_is_written(hip_backend):
         cap.graph.destroy()
 
 
+def test_a_write_into_a_deferred_input_keeps_the_original_order(hip_backend):
+    """The fp32 bias is cast, then overwritten in part (a copy into the middle of its buffer), then
+    the cast copy is added to a product. Merging the cast into the product would read the bias
+    after the overwrite; the rewrite must see the partial write and leave the cast where it was."""
+    from ctypes import c_void_p
+    rng = np.random.default_rng(12)
+    with hip_backend.use():
+        x, w, _, _ = operands(rng, DType.float16, 256, 128, 256)
+        bias32 = Tensor(data=rng.standard_normal((256,)).astype(np.float32))
+        patch = Tensor(data=np.full((16,), 100.0, np.float32))
+        old = bias32.numpy().copy()
+
+        def run():
+            b16 = bias32.cast(DType.float16)
+            hip_backend._check(hip_backend._lib.hc_memcpy_d2d(hip_backend._ctx, c_void_p(bias32.data.ptr + 64),
+                                                               c_void_p(patch.data.ptr), 64))
+            return Tensor.matmul(x, False, w, False, False) + b16
+
+        want = (Tensor.matmul(x, False, w, False, False) + Tensor(data=old, dtype=DType.float16)).numpy()
+        with hip_backend.capture() as cap:
+            out = run()
+        for _ in range(2):
+            bias32.data.mutateOnCPU(lambda host: host.view(np.float32).__setitem__(slice(None), old))
+            cap.graph.launch()
+            assert np.array_equal(out.numpy(), want)
+        cap.graph.destroy()
+
+
 def test_other_forms_of_add_are_left_alone(hip_backend, monkeypatch):
     rng = np.random.default_rng(8)
     with hip_backend.use():
