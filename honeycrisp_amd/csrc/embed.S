@@ -22,5 +22,8 @@
     EMBED hc_image_gemm_dma, "gemm_dma.hsaco"
     EMBED hc_image_gemm_dma2, "gemm_dma2.hsaco"
     EMBED hc_image_gemm_mi16, "gemm_mi16.hsaco"
+    EMBED hc_image_gemm_dma_m, "gemm_dma_m.hsaco"
+    EMBED hc_image_gemm_dma2_m, "gemm_dma2_m.hsaco"
+    EMBED hc_image_gemm_mi16_m, "gemm_mi16_m.hsaco"
 
     .section .note.GNU-stack,"",@progbits

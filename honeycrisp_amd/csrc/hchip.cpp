@@ -31,6 +31,9 @@ extern const unsigned char hc_image_gemm_f16_fast[], hc_image_gemm_f16_fast_end[
 extern const unsigned char hc_image_gemm_dma[], hc_image_gemm_dma_end[];
 extern const unsigned char hc_image_gemm_dma2[], hc_image_gemm_dma2_end[];
 extern const unsigned char hc_image_gemm_mi16[], hc_image_gemm_mi16_end[];
+extern const unsigned char hc_image_gemm_dma_m[], hc_image_gemm_dma_m_end[];
+extern const unsigned char hc_image_gemm_dma2_m[], hc_image_gemm_dma2_m_end[];
+extern const unsigned char hc_image_gemm_mi16_m[], hc_image_gemm_mi16_m_end[];
 }
 
 // noalloc.hip: looks up this device's copy of the library's fixed scratch array (device current)
@@ -56,6 +59,7 @@ struct hc_event {
 struct hc_pending {
   enum Kind { KERNEL, RAW_KERNEL, COPY_D2D, FREE } kind = KERNEL;
   hipFunction_t fn = nullptr;
+  std::string name;                    // KERNEL: the built-in kernel's name
   uint32_t grid[3] = {1, 1, 1}, block[3] = {HCK_BLOCK, 1, 1}, shared = 0;
   std::vector<char> args;              // the kernel's by-value argument struct
   void* dst = nullptr;                 // COPY_D2D / FREE
@@ -225,6 +229,9 @@ extern "C" int hc_init(int device, hc_ctx** out) {
   if (s == HC_OK) s = load_image(ctx, hc_image_gemm_dma, hc_image_gemm_dma_end, "gemm_dma");
   if (s == HC_OK) s = load_image(ctx, hc_image_gemm_dma2, hc_image_gemm_dma2_end, "gemm_dma2");
   if (s == HC_OK) s = load_image(ctx, hc_image_gemm_mi16, hc_image_gemm_mi16_end, "gemm_mi16");
+  if (s == HC_OK) s = load_image(ctx, hc_image_gemm_dma_m, hc_image_gemm_dma_m_end, "gemm_dma_m");
+  if (s == HC_OK) s = load_image(ctx, hc_image_gemm_dma2_m, hc_image_gemm_dma2_m_end, "gemm_dma2_m");
+  if (s == HC_OK) s = load_image(ctx, hc_image_gemm_mi16_m, hc_image_gemm_mi16_m_end, "gemm_mi16_m");
   if (s != HC_OK) {
     hc_shutdown(ctx);
     return s;
@@ -596,8 +603,7 @@ extern "C" int hc_capture_begin(hc_ctx* ctx) {
   HIP_TRY(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed));
   ctx->capturing = new hc_graph();
   ctx->graphs.push_back(ctx->capturing);
-  // HCHIP_NO_FUSION=1: launches go to the capturing stream one by one, as issued
-  ctx->lazy = getenv("HCHIP_NO_FUSION") == nullptr;
+  ctx->lazy = true;   // launches are listed, and enqueued on the capturing stream at hc_capture_end
   ctx->pending.clear();
   return HC_OK;
 }
@@ -651,7 +657,8 @@ static int end_capture(hc_ctx* ctx, hc_graph** out) {
   if (ctx->lazy) {
     ctx->lazy = false;
     if (out) {
-      fuse_recording(ctx);
+      // HCHIP_NO_FUSION=1: the launches are enqueued as they were issued
+      if (!getenv("HCHIP_NO_FUSION")) fuse_recording(ctx);
       if (getenv("HCHIP_RECORDING_LOG")) {   // the launches of the recording as they will be enqueued, to stderr
         size_t n = 0;
         for (const hc_pending& e : ctx->pending) {
@@ -996,10 +1003,21 @@ static void fuse_softmaxes(hc_ctx* ctx, std::vector<hc_pending>& list, const Fre
   }
 }
 
+// The kernel of the same name from the second build of the tiled GEMM sources (*_m): the one that
+// knows merged operations, two-level batches and groups. False if there is none.
+static bool use_merged_kernel(hc_ctx* ctx, hc_pending& e) {
+  if (e.name.size() >= 2 && e.name.compare(e.name.size() - 2, 2, "_m") == 0) return true;
+  hipFunction_t fn = nullptr;
+  if (find_kernel_locked(ctx, e.name + "_m", &fn) != HC_OK) return false;
+  e.fn = fn;
+  e.name += "_m";
+  return true;
+}
+
 // A batched product whose operand is a tensor with two axes swapped ([B, T, H, d] read as
 // [B, H, T, d]: the heads of an attention layer), or whose result is swapped back, reads and
 // writes through the strides instead: the copies disappear.
-static void fuse_swapped_batches(std::vector<hc_pending>& list, const FreedMap& freed) {
+static void fuse_swapped_batches(hc_ctx* ctx, std::vector<hc_pending>& list, const FreedMap& freed) {
   for (size_t i = 0; i < list.size(); i++) {
     if (list[i].dropped || list[i].kind != hc_pending::KERNEL || list[i].tag != hc_pending::BMM) continue;
     if (list[i].args.size() != sizeof(hck_gemm_args)) continue;
@@ -1115,6 +1133,7 @@ static void fuse_swapped_batches(std::vector<hc_pending>& list, const FreedMap& 
     size_t last = i;
     for (const Deferred& c : chain) last = std::max(last, c.at);
     hc_pending fused = list[i];
+    if (!use_merged_kernel(ctx, fused)) continue;
     memcpy(fused.args.data(), &g, sizeof(g));
     fused.tag = hc_pending::NONE;
     fused.reads = {g.a, g.b};
@@ -1128,7 +1147,7 @@ static void fuse_swapped_batches(std::vector<hc_pending>& list, const FreedMap& 
 // Products over the same A with the same shape, strides and merged operations (the q, k, v
 // projections of an attention layer) become one launch: a workgroup's blockIdx.y picks the
 // member's B, C and epilogue operands.
-static void fuse_product_groups(std::vector<hc_pending>& list, const FreedMap& freed) {
+static void fuse_product_groups(hc_ctx* ctx, std::vector<hc_pending>& list, const FreedMap& freed) {
   auto is_product = [](const hc_pending& e) {
     return !e.dropped && e.kind == hc_pending::KERNEL && (e.tag == hc_pending::GEMM || e.tag == hc_pending::PRODUCT) &&
            e.args.size() == sizeof(hck_gemm_args);
@@ -1178,6 +1197,7 @@ static void fuse_product_groups(std::vector<hc_pending>& list, const FreedMap& f
     if (members.size() < 2) continue;
     const uint32_t n = (uint32_t)members.size();
     hc_pending grouped = list[i];
+    if (!use_merged_kernel(ctx, grouped)) continue;
     grouped.tag = hc_pending::NONE;
     grouped.out = nullptr;
     grouped.grid[1] = n;
@@ -1207,15 +1227,14 @@ static void fuse_recording(hc_ctx* ctx) {
   const Overlap overlap{ctx, &freed};
   g_overlap = &overlap;
   fuse_products(ctx, list, freed);
-  fuse_swapped_batches(list, freed);
+  fuse_swapped_batches(ctx, list, freed);
   fuse_layernorms(ctx, list, freed);
   fuse_softmaxes(ctx, list, freed);
-  fuse_product_groups(list, freed);
+  fuse_product_groups(ctx, list, freed);
   g_overlap = nullptr;
 }
 
 static void fuse_products(hc_ctx* ctx, std::vector<hc_pending>& list, const FreedMap& freed) {
-  (void)ctx;
 
   for (size_t i = 0; i < list.size(); i++) {
     if (list[i].kind != hc_pending::KERNEL || list[i].dropped || list[i].tag != hc_pending::GEMM) continue;
@@ -1276,6 +1295,9 @@ static void fuse_products(hc_ctx* ctx, std::vector<hc_pending>& list, const Free
       if (ends_list) break;
     }
     if (nops == 0) continue;
+    // the kernel of the same name that knows how to apply the operations
+    hc_pending fused = list[i];
+    if (!use_merged_kernel(ctx, fused)) continue;
     // a bias row that is an fp32 parameter cast to fp16 just for this addition: read the fp32 row
     if (dtype == HC_F16)
       for (int s = 0; s < nops; s++) {
@@ -1301,7 +1323,6 @@ static void fuse_products(hc_ctx* ctx, std::vector<hc_pending>& list, const Free
         }
       }
     g.c = const_cast<void*>(cur);
-    hc_pending fused = list[i];
     memcpy(fused.args.data(), &g, sizeof(g));
     fused.tag = hc_pending::PRODUCT;   // (no further operations are merged; it may still join a group)
     fused.reads = inputs;
@@ -1364,11 +1385,12 @@ struct OpNote {
 thread_local OpNote* OpNote::current = nullptr;
 
 // Adds a launch to the recording in progress (caller holds the mutex).
-static void record_launch_locked(hc_ctx* ctx, hipFunction_t fn, uint32_t gx, uint32_t gy, const void* args,
-                                 size_t bytes) {
+static void record_launch_locked(hc_ctx* ctx, const std::string& name, hipFunction_t fn, uint32_t gx, uint32_t gy,
+                                 const void* args, size_t bytes) {
   hc_pending e;
   e.kind = hc_pending::KERNEL;
   e.fn = fn;
+  e.name = name;
   e.grid[0] = gx;
   e.grid[1] = gy;
   e.args.assign((const char*)args, (const char*)args + bytes);
@@ -1461,7 +1483,7 @@ static int launch(hc_ctx* ctx, const std::string& name, uint64_t blocks_x, uint3
   hipFunction_t fn = nullptr;
   HC_TRY(find_kernel_locked(ctx, name, &fn));
   if (ctx->lazy) {
-    record_launch_locked(ctx, fn, (uint32_t)blocks_x, blocks_y, args, bytes);
+    record_launch_locked(ctx, name, fn, (uint32_t)blocks_x, blocks_y, args, bytes);
     return HC_OK;
   }
   return launch_fn(ctx, fn, (uint32_t)blocks_x, blocks_y, 1, HCK_BLOCK, 0, args, bytes);

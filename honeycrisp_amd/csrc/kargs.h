@@ -330,18 +330,20 @@ typedef struct {
   /* edge kernels: rows (K-contiguous operand) or elements of a k-row (M/N-contiguous operand,
    * a multiple of 16 bytes) that may be fetched; anything beyond is clamped to the last one */
   uint32_t a_lim, b_lim;
-  /* Operations applied to the finished tile before it is stored (direct-to-LDS kernels only), in
+  /* The fields from here on are read only by the second build of the direct-to-LDS kernels (names
+   * ending in _m), which a recording's rewrite substitutes for the plain ones.
+   * Operations applied to the finished tile before it is stored, in
    * order, each on the value rounded to the output type, i.e. with the arithmetic of the
    * separate kernels they replace: what a recording's rewrite merges into the product. */
   uint32_t ep_kind[3];    /* HCK_EP_* ; 0 ends the list */
   uint32_t ep_ld[3];      /* HCK_EP_ADD_MATRIX: leading dimension of the matrix, elements */
   const void* ep_ptr[3];  /* HCK_EP_ADD_ROW: N elements; HCK_EP_ADD_MATRIX: [M, ld] */
-  /* Two-level batch (direct-to-LDS kernels only; 0 = off): slice z lies at
+  /* Two-level batch (0 = off): slice z lies at
    * (z / bdiv) * x_bs + (z % bdiv) * x_bs2. What a batched product reads or writes when a
    * recording folds a swap of the batch axes ([B, T, H, d] <-> [B, H, T, d]) into it. */
   uint32_t bdiv;
   /* A group of up to HCK_GEMM_GROUP products over the same A with the same shape, operations and
-   * strides in one launch (direct-to-LDS kernels only; 0 = off): blockIdx.y picks the member's B,
+   * strides in one launch (0 = off): blockIdx.y picks the member's B,
    * C and epilogue operands from the tables. What a recording makes of the q, k, v projections of
    * an attention layer. */
   uint32_t group;

@@ -348,19 +348,3 @@ __device__ __forceinline__ void gemm_store_slab_merged_as(const hck_gemm_args& p
       gemm_store_group_merged<T, Chunk16, EDGE, GROUP, COL_FIXED, MATRIX, GELU>(p, ops, r0, r1, r2, C, it0, lds_piece, row_of, col_of);
   }
 }
-
-template <typename T, typename Chunk16, bool EDGE, uint32_t NIT, bool COL_FIXED, uint32_t MAX_GROUP, typename LdsPiece,
-          typename RowOf, typename ColOf>
-__device__ __forceinline__ void gemm_store_slab_merged(const hck_gemm_args& p, const GemmEpilogueOperands& ops, Chunk16 r0,
-                                                       Chunk16 r1, Chunk16 r2, T* C, LdsPiece lds_piece, RowOf row_of, ColOf col_of) {
-  const bool matrix = p.ep_kind[0] == HCK_EP_ADD_MATRIX || p.ep_kind[1] == HCK_EP_ADD_MATRIX || p.ep_kind[2] == HCK_EP_ADD_MATRIX;
-  const bool gelu = p.ep_kind[0] == HCK_EP_GELU || p.ep_kind[1] == HCK_EP_GELU || p.ep_kind[2] == HCK_EP_GELU;
-  // (the activation is long enough to hide the latencies of one piece: its loop takes the pieces
-  // one by one, which keeps that code to one copy per slab)
-  if (gelu)
-    gemm_store_slab_merged_as<T, Chunk16, EDGE, NIT, COL_FIXED, 1, false, true>(p, ops, r0, r1, r2, C, lds_piece, row_of, col_of);
-  else if (matrix)
-    gemm_store_slab_merged_as<T, Chunk16, EDGE, NIT, COL_FIXED, MAX_GROUP, true, false>(p, ops, r0, r1, r2, C, lds_piece, row_of, col_of);
-  else
-    gemm_store_slab_merged_as<T, Chunk16, EDGE, NIT, COL_FIXED, MAX_GROUP, false, false>(p, ops, r0, r1, r2, C, lds_piece, row_of, col_of);
-}

@@ -231,6 +231,8 @@ __device__ __forceinline__ void gemm_dma2_impl(const hck_gemm_args& p, char* lds
   gemm_tile_of_block(p, blockIdx.x, tm, tn);
   const uint32_t m0 = tm * BM, n0 = tn * BN;
   const uint32_t batch = blockIdx.y;
+#ifdef HC_GEMM_MERGED
+  // (the second build of this file, kernels *_m: what a recording's rewrite needs)
   uint32_t batch_hi = batch, batch_lo = 0;
   if (p.bdiv != 0) {
     batch_hi = batch / p.bdiv;
@@ -245,6 +247,11 @@ __device__ __forceinline__ void gemm_dma2_impl(const hck_gemm_args& p, char* lds
     C = (T*)p.g_c[batch];
   }
   const GemmEpilogueOperands ep_ops = gemm_epilogue_operands(p, batch);
+#else
+  const T* A = (const T*)p.a + batch * p.a_bs;
+  const T* B = (const T*)p.b + batch * p.b_bs;
+  T* C = (T*)p.c + batch * p.c_bs;
+#endif
 
   const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const uint32_t wm = (wave >> 1) * (BM / 2), wn = (wave & 1) * (BN / 2);
@@ -388,6 +395,7 @@ __device__ __forceinline__ void gemm_dma2_impl(const hck_gemm_args& p, char* lds
   constexpr uint32_t USWZ = (UNITS & (UNITS - 1)) == 0 ? UNITS - 1 : (UNITS % 8 == 0 ? 7 : 3);
   static_assert(UNITS % (USWZ + 1) == 0, "unsupported tile width");
   auto unit_swz = [&](uint32_t r) { return (RB >= 256 ? r : r * RB / 256) & USWZ; };
+#ifdef HC_GEMM_MERGED
   // (operations merged into this product: if 64 lanes are whole rows of units, a lane's columns
   // are the same for all its pieces and the row operands are fetched once)
   constexpr bool EP_COL_FIXED = 64 % UNITS == 0;
@@ -399,61 +407,95 @@ __device__ __forceinline__ void gemm_dma2_impl(const hck_gemm_args& p, char* lds
     ep_r1 = gemm_epilogue_row_piece<T, Chunk>(p.ep_kind[1], ep_ops.p1, ep_col, ok);
     ep_r2 = gemm_epilogue_row_piece<T, Chunk>(p.ep_kind[2], ep_ops.p2, ep_col, ok);
   }
+#endif
+  // One copy of the write-out per kind of epilogue (MODE 0: plain stores; 1: merged additions; 2:
+  // with a matrix operand; 3: additions and GELU). The plain one is all that the kernels of the
+  // ordinary build contain; the kernels a recording's rewrite uses are a second build of this file
+  // (HC_GEMM_MERGED, names ending in _m) that picks the mode per launch and also knows two-level
+  // batches and groups of products. Kept apart on purpose: with the merged code in the same kernel
+  // the plain fp16 4096^3 product ran 7 % slower (1216 against 1313 TFLOP/s on the same device, same
+  // main loop instruction for instruction), and where the plain path shared blocks with code that
+  // loads, the compiler guarded those loads' registers with waits that, at run time, wait for the
+  // plain path's own stores (one in-order counter for loads and stores).
+#ifdef HC_GEMM_MERGED
+  auto write_out = [&](auto mode_c) {
+    constexpr int MODE = decltype(mode_c)::value;
+#else
+  {
+    constexpr int MODE = 0;
+#endif
 #pragma unroll
-  for (int i = 0; i < MT; i++) {
-    char* slab = mine + (i % NSLAB) * SLAB;
+    for (int i = 0; i < MT; i++) {
+      char* slab = mine + (i % NSLAB) * SLAB;
 #pragma unroll
-    for (int j = 0; j < NT; j++) {
+      for (int j = 0; j < NT; j++) {
 #pragma unroll
-      for (int g = 0; g < 4; g++) {
-        if constexpr (F32) {
-          floatx4 h;
+        for (int g = 0; g < 4; g++) {
+          if constexpr (F32) {
+            floatx4 h;
 #pragma unroll
-          for (int e = 0; e < 4; e++) h[e] = acc[i][j][4 * g + e];
-          *reinterpret_cast<floatx4*>(slab + lrow * RB + (((j * 8 + 2 * g + lgrp) ^ unit_swz(lrow)) * 16)) = h;
-        } else {
-          half4v h;
+            for (int e = 0; e < 4; e++) h[e] = acc[i][j][4 * g + e];
+            *reinterpret_cast<floatx4*>(slab + lrow * RB + (((j * 8 + 2 * g + lgrp) ^ unit_swz(lrow)) * 16)) = h;
+          } else {
+            half4v h;
 #pragma unroll
-          for (int e = 0; e < 4; e++) h[e] = narrow<half_t>(acc[i][j][4 * g + e]);
-          *reinterpret_cast<half4v*>(slab + lrow * RB + (((j * 4 + g) ^ unit_swz(lrow)) * 16) + lgrp * 8) = h;
+            for (int e = 0; e < 4; e++) h[e] = narrow<half_t>(acc[i][j][4 * g + e]);
+            *reinterpret_cast<half4v*>(slab + lrow * RB + (((j * 4 + g) ^ unit_swz(lrow)) * 16) + lgrp * 8) = h;
+          }
         }
       }
-    }
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // wave-private region: no barrier needed
-    // (a merged epilogue is a loop of its own that is not unrolled: it reads LDS, not the
-    // accumulators, and unrolled copies of it would multiply the kernel's code)
-    if (p.ep_kind[0] == HCK_EP_NONE) {
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // wave-private region: no barrier needed
+      if constexpr (MODE == 0) {
 #pragma unroll
-      for (uint32_t it = 0; it < 32 * UNITS / 64; it++) {
-        const uint32_t piece = it * 64 + lane, r = piece / UNITS, u = piece % UNITS;
-        const Chunk v = *reinterpret_cast<const Chunk*>(slab + r * RB + ((u ^ unit_swz(r)) * 16));
-        const uint32_t row = m0 + wm + i * 32 + r, col = n0 + wn + u * (16 / ES);
-        if (!EDGE || (row < p.M && col < p.N)) *reinterpret_cast<Chunk*>(C + (size_t)row * p.c_rs + col) = v;
+        for (uint32_t it = 0; it < 32 * UNITS / 64; it++) {
+          const uint32_t piece = it * 64 + lane, r = piece / UNITS, u = piece % UNITS;
+          const Chunk v = *reinterpret_cast<const Chunk*>(slab + r * RB + ((u ^ unit_swz(r)) * 16));
+          const uint32_t row = m0 + wm + i * 32 + r, col = n0 + wn + u * (16 / ES);
+          if (!EDGE || (row < p.M && col < p.N)) *reinterpret_cast<Chunk*>(C + (size_t)row * p.c_rs + col) = v;
+        }
       }
-    } else {
-      gemm_store_slab_merged<T, Chunk, EDGE, 32 * UNITS / 64, EP_COL_FIXED, 4>(
-          p, ep_ops, ep_r0, ep_r1, ep_r2, C,
-          [=](uint32_t it) {
-            const uint32_t piece = it * 64 + lane, r = piece / UNITS, u = piece % UNITS;
-            return *reinterpret_cast<const Chunk*>(slab + r * RB + ((u ^ unit_swz(r)) * 16));
-          },
-          [=](uint32_t it) { return m0 + wm + i * 32 + (it * 64 + lane) / UNITS; },
-          [=](uint32_t it) { return n0 + wn + ((it * 64 + lane) % UNITS) * (16 / ES); });
+#ifdef HC_GEMM_MERGED
+      if constexpr (MODE != 0) {
+        gemm_store_slab_merged_as<T, Chunk, EDGE, 32 * UNITS / 64, EP_COL_FIXED, (MODE == 3 ? 1 : 4), MODE == 2, MODE == 3>(
+            p, ep_ops, ep_r0, ep_r1, ep_r2, C,
+            [=](uint32_t it) {
+              const uint32_t piece = it * 64 + lane, r = piece / UNITS, u = piece % UNITS;
+              return *reinterpret_cast<const Chunk*>(slab + r * RB + ((u ^ unit_swz(r)) * 16));
+            },
+            [=](uint32_t it) { return m0 + wm + i * 32 + (it * 64 + lane) / UNITS; },
+            [=](uint32_t it) { return n0 + wn + ((it * 64 + lane) % UNITS) * (16 / ES); });
+      }
+#endif
+      asm volatile("" ::: "memory");
     }
-    asm volatile("" ::: "memory");
+#ifdef HC_GEMM_MERGED
+  };
+  const bool ep_matrix = p.ep_kind[0] == HCK_EP_ADD_MATRIX || p.ep_kind[1] == HCK_EP_ADD_MATRIX || p.ep_kind[2] == HCK_EP_ADD_MATRIX;
+  const bool ep_gelu = p.ep_kind[0] == HCK_EP_GELU || p.ep_kind[1] == HCK_EP_GELU || p.ep_kind[2] == HCK_EP_GELU;
+  if (p.ep_kind[0] == HCK_EP_NONE) write_out(std::integral_constant<int, 0>{});
+  else if (ep_gelu) write_out(std::integral_constant<int, 3>{});
+  else if (ep_matrix) write_out(std::integral_constant<int, 2>{});
+  else write_out(std::integral_constant<int, 1>{});
+#else
   }
+#endif
 }
 
 // Two variants per kernel: whole tiles only, and "_e" (edge) for M, N that are not multiples of
 // the tile and K that is not a multiple of the K-slice (64 halfs, 32 floats).
+#ifdef HC_GEMM_MERGED
+#define HC_GEMM_NAME(base) base##_m
+#else
+#define HC_GEMM_NAME(base) base
+#endif
 #define DEF_DMA(T, TN, BM, BN, AN, AM, BNAME, BMODE)                                                  \
-  extern "C" __global__ __launch_bounds__(256) void hc_gemm_##TN##_dma2_##BM##x##BN##_##AN##BNAME(     \
+  extern "C" __global__ __launch_bounds__(256) void HC_GEMM_NAME(hc_gemm_##TN##_dma2_##BM##x##BN##_##AN##BNAME)( \
       hck_gemm_args p) {                                                                              \
     __shared__ __attribute__((aligned(1024))) char lds0[(BM + BN) * 128];                             \
     __shared__ __attribute__((aligned(1024))) char lds1[(BM + BN) * 128];                             \
     gemm_dma2_impl<T, BM, BN, AM, BMODE, false>(p, lds0, lds1);                                       \
   }                                                                                                   \
-  extern "C" __global__ __launch_bounds__(256) void hc_gemm_##TN##_dma2_##BM##x##BN##_##AN##BNAME##_e( \
+  extern "C" __global__ __launch_bounds__(256) void HC_GEMM_NAME(hc_gemm_##TN##_dma2_##BM##x##BN##_##AN##BNAME##_e)( \
       hck_gemm_args p) {                                                                              \
     __shared__ __attribute__((aligned(1024))) char lds0[(BM + BN) * 128];                             \
     __shared__ __attribute__((aligned(1024))) char lds1[(BM + BN) * 128];                             \

@@ -167,7 +167,7 @@ int hc_launch_host_func(hc_ctx* ctx, void (*fn)(void*), void* user);
  *    HCHIP_RECORDING_LOG=1 at hc_capture_end lists the launches of the rewritten recording on
  *    stderr; HCHIP_GRAPH_AS_LAUNCHES=1 makes hc_graph_launch issue them one by one instead of
  *    through hipGraphLaunch (for kernel traces).
- *    HCHIP_NO_FUSION=1 in the environment at hc_capture_begin turns the rewrite off. */
+ *    HCHIP_NO_FUSION=1 in the environment at hc_capture_end turns the rewrite off. */
 typedef struct hc_graph hc_graph;
 int hc_capture_begin(hc_ctx* ctx);
 int hc_capture_end(hc_ctx* ctx, hc_graph** out);

@@ -114,6 +114,7 @@ def test_build_refuses_register_tiled_kernels_that_use_scratch_memory():
         k.hip:9:1: remark: Function Name: hc_gemm_c [-Rpass-analysis=kernel-resource-usage]
         k.hip:9:1: remark:     ScratchSize [bytes/lane]: 68 [-Rpass-analysis=kernel-resource-usage]
         """)
-    assert build.kernels_with_scratch(remarks) == ["hc_gemm_b (1088 bytes/lane)"]
-    assert {"gemm_dma", "gemm_dma2", "gemm_mi16"} <= build.NO_SCRATCH
-    assert build.NO_SCRATCH <= {name for name, _src, _flags in build.KERNELS}
+    assert build.kernels_with_scratch(remarks, 128) == ["hc_gemm_b (1088 bytes/lane)"]
+    assert build.kernels_with_scratch(remarks, 16) == ["hc_gemm_b (1088 bytes/lane)", "hc_gemm_c (68 bytes/lane)"]
+    assert {"gemm_dma", "gemm_dma2", "gemm_mi16", "gemm_mi16_m"} <= set(build.NO_SCRATCH)
+    assert set(build.NO_SCRATCH) <= {name for name, _src, _flags in build.KERNELS}
