@@ -43,7 +43,7 @@ PEAK_HBM_GBS = 8000.0     # MI355X HBM3E
 # this benchmark scaled by a plain copy kernel (not measurable live; the run that produced it is
 # summarised in profiles/bench_hbm_traffic_fetch_write_size.md): 196850 KiB read + 32768 KiB written.
 GEMM_TRAFFIC_BYTES = (196800 + 32768) * 1024
-GEMM_TRAFFIC_SOURCE = "constant from profiles/bench_hbm_traffic_fetch_write_size.md (rocprofv3 --pmc runs), not measured in this run"
+GEMM_TRAFFIC_SOURCE = "constant from profiles/gemm_f16_4096_and_cfg4_hbm_traffic_fetch_write_size.md (rocprofv3 --pmc runs), not measured in this run"
 
 
 class MfmaProbe:
