@@ -8,6 +8,7 @@
 #endif
 #include <hip/hip_runtime_api.h>
 
+#include <algorithm>
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
@@ -129,6 +130,9 @@ struct hc_ctx {
   std::vector<hipEvent_t> wait_events;  // spare events of blocking transfers (waited for outside the mutex)
   bool lazy = false;                    // a capture that lists its launches (see hc_pending)
   std::vector<hc_pending> pending;
+  // buffers whose only writer and only reader were merged away by the rewrite of the recording in
+  // progress: no launch of the graph touches them, so they need not stay reserved for it
+  std::vector<std::pair<void*, size_t>> dead;
 };
 static const size_t kStageHalf = 2u << 20;    // bytes per half of the staging buffer
 static const size_t kStageMax = 256u << 10;   // largest upload that is staged
@@ -695,6 +699,20 @@ static int end_capture(hc_ctx* ctx, hc_graph** out) {
     if (e != hipSuccess) return hip_fail(e, "hipStreamEndCapture / hipGraphInstantiate");
     return HC_OK;
   }
+  // Blocks that only held merged-away intermediates go back to the general pool now instead of
+  // staying reserved until hc_graph_destroy.
+  for (const auto& d : ctx->dead) {
+    auto parked = g->parked.find(d.second);
+    if (parked == g->parked.end()) continue;
+    auto& v = parked->second;
+    auto it = std::find(v.begin(), v.end(), d.first);
+    if (it == v.end()) continue;
+    v.erase(it);
+    ctx->block_owner.erase(d.first);
+    ctx->free_blocks[d.second].push_back(d.first);
+    ctx->bytes_cached += d.second;
+  }
+  ctx->dead.clear();
   *out = g;
   return HC_OK;
 }
@@ -808,6 +826,20 @@ struct Overlap {
   }
 };
 static thread_local const Overlap* g_overlap = nullptr;   // set for the duration of fuse_recording
+static thread_local std::vector<std::pair<void*, size_t>>* g_dead = nullptr;   // likewise
+
+// The results of a chain's entries, other than the chain's final result, are written by no launch
+// any more (every one of them was released inside the recording: that is what made it mergeable).
+static void note_dead_results(const std::vector<hc_pending>& list, const std::vector<size_t>& members, const void* final_out,
+                              const FreedMap& freed) {
+  if (!g_dead) return;
+  for (size_t m : members) {
+    const void* out = list[m].out;
+    if (!out || out == final_out) continue;
+    auto fr = freed.find(out);
+    if (fr != freed.end()) g_dead->push_back({const_cast<void*>(out), fr->second.bytes});
+  }
+}
 static bool may_alias(const void* w, const void* r) { return g_overlap ? (*g_overlap)(w, r) : w == r; }
 
 // The tagged launch before entry `before` that produced the buffer `ptr`, or -1 (also when a
@@ -858,13 +890,17 @@ static bool inputs_stable(const std::vector<hc_pending>& list, const std::vector
 }
 
 // Replaces the entries of `chain` by one launch at the place of the last of them.
-static void replace_chain(std::vector<hc_pending>& list, const std::vector<Deferred>& chain, hipFunction_t fn, uint64_t blocks,
-                          const void* args, size_t bytes, std::initializer_list<const void*> reads, const void* out) {
+static void replace_chain(std::vector<hc_pending>& list, const FreedMap& freed, const std::vector<Deferred>& chain,
+                          hipFunction_t fn, uint64_t blocks, const void* args, size_t bytes,
+                          std::initializer_list<const void*> reads, const void* out) {
   size_t last = chain[0].at;
+  std::vector<size_t> members;
   for (const Deferred& c : chain) {
     last = std::max(last, c.at);
-    list[c.at].dropped = true;
+    members.push_back(c.at);
   }
+  note_dead_results(list, members, out, freed);
+  for (size_t m : members) list[m].dropped = true;
   hc_pending e;
   e.kind = hc_pending::KERNEL;
   e.fn = fn;
@@ -937,7 +973,7 @@ static void fuse_layernorms(hc_ctx* ctx, std::vector<hc_pending>& list, const Fr
     snprintf(name, sizeof(name), "hc_layernorm_rows_%s_%s", dtype_name(in_type), dtype_name(out_type));
     hipFunction_t fn = nullptr;
     if (find_kernel_locked(ctx, name, &fn) != HC_OK) continue;
-    replace_chain(list, chain, fn, ceil_div_u64(norm.rows, HCK_BLOCK / 64), &k, sizeof(k), {k.in, k.gain, k.bias}, out);
+    replace_chain(list, freed, chain, fn, ceil_div_u64(norm.rows, HCK_BLOCK / 64), &k, sizeof(k), {k.in, k.gain, k.bias}, out);
   }
 }
 
@@ -999,7 +1035,7 @@ static void fuse_softmaxes(hc_ctx* ctx, std::vector<hc_pending>& list, const Fre
     snprintf(name, sizeof(name), "hc_softmax_chain_rows%s_%s", sm.lanes == 8 ? "8" : "", dtype_name(sm.dtype));
     hipFunction_t fn = nullptr;
     if (find_kernel_locked(ctx, name, &fn) != HC_OK) continue;
-    replace_chain(list, chain, fn, ceil_div_u64(sm.rows, HCK_BLOCK / (uint64_t)sm.lanes), &k, sizeof(k), {k.in, k.mask}, out);
+    replace_chain(list, freed, chain, fn, ceil_div_u64(sm.rows, HCK_BLOCK / (uint64_t)sm.lanes), &k, sizeof(k), {k.in, k.mask}, out);
   }
 }
 
@@ -1139,6 +1175,11 @@ static void fuse_swapped_batches(hc_ctx* ctx, std::vector<hc_pending>& list, con
     fused.reads = {g.a, g.b};
     fused.writes = {out};
     fused.out = const_cast<void*>(out);
+    {
+      std::vector<size_t> members;
+      for (const Deferred& c : chain) members.push_back(c.at);
+      note_dead_results(list, members, out, freed);
+    }
     for (const Deferred& c : chain) list[c.at].dropped = true;
     list[last] = std::move(fused);
   }
@@ -1226,12 +1267,15 @@ static void fuse_recording(hc_ctx* ctx) {
     if (list[i].kind == hc_pending::FREE) freed[list[i].dst] = Freed{i, list[i].bytes};
   const Overlap overlap{ctx, &freed};
   g_overlap = &overlap;
+  ctx->dead.clear();
+  g_dead = &ctx->dead;
   fuse_products(ctx, list, freed);
   fuse_swapped_batches(ctx, list, freed);
   fuse_layernorms(ctx, list, freed);
   fuse_softmaxes(ctx, list, freed);
   fuse_product_groups(ctx, list, freed);
   g_overlap = nullptr;
+  g_dead = nullptr;
 }
 
 static void fuse_products(hc_ctx* ctx, std::vector<hc_pending>& list, const FreedMap& freed) {
@@ -1318,6 +1362,7 @@ static void fuse_products(hc_ctx* ctx, std::vector<hc_pending>& list, const Free
             if (in == g.ep_ptr[s]) in = e.in0;
           g.ep_kind[s] = HCK_EP_ADD_ROW_F32;
           g.ep_ptr[s] = e.in0;
+          note_dead_results(list, {c2}, nullptr, freed);
           e.dropped = true;
           break;
         }
@@ -1328,6 +1373,11 @@ static void fuse_products(hc_ctx* ctx, std::vector<hc_pending>& list, const Free
     fused.reads = inputs;
     fused.writes = {cur};
     fused.out = const_cast<void*>(cur);
+    {
+      std::vector<size_t> members = merged;
+      members.push_back(i);
+      note_dead_results(list, members, cur, freed);
+    }
     for (size_t m : merged) list[m].dropped = true;
     list[i].dropped = true;
     list[pos] = std::move(fused);   // (not dropped: copied from the product's entry before that was marked)
