@@ -142,6 +142,12 @@ class HIPBackend {
     return g;
   }
   void launch(hc_graph* g) { check(hc_graph_launch(ctx_, g)); }
+  // launches and copies one replay issues (after the library's rewrite of the recording)
+  size_t nodeCount(hc_graph* g) {
+    size_t n = 0;
+    check(hc_graph_node_count(g, &n));
+    return n;
+  }
   void destroy(hc_graph* g) { check(hc_graph_destroy(ctx_, g)); }
 
   // ---- ops (Backend.swift line of each declaration in the comment)

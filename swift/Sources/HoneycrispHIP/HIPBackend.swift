@@ -682,6 +682,12 @@ open class HIPBackend: CPUBackend, @unchecked Sendable {
     let handle: OpaquePointer
     init(backend: HIPBackend, handle: OpaquePointer) { (self.backend, self.handle) = (backend, handle) }
     public func launch() throws { try backend.check(hc_graph_launch(backend.ctx, handle)) }
+    /// Kernel launches and copies one replay issues (after the library's rewrite of the recording).
+    public func nodeCount() throws -> Int {
+      var n: Int = 0
+      try backend.check(hc_graph_node_count(handle, &n))
+      return n
+    }
     deinit { _ = hc_graph_destroy(backend.ctx, handle) }
   }
 
