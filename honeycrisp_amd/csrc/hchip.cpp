@@ -764,15 +764,19 @@ extern "C" int hc_graph_destroy(hc_ctx* ctx, hc_graph* graph) {
 // Inside a recording every buffer has an address of its own (released blocks are not handed out
 // again until the recording ends), entry points declare what they read and write, and a release
 // says that nobody reads a buffer afterwards. That is enough to see, without any knowledge of the
-// caller's program, that the result of a product has exactly one reader, and to let the product's
-// kernel do that reader's work on the tile it is about to store:
-//     matmul -> + bias row -> GELU          (Linear followed by an activation)
-//     matmul -> + bias row -> + residual    (Linear inside a residual connection)
-// (up to three operations, one of them with a matrix operand; GELU only as the last, and not
-// after a matrix operand) with the bias row possibly cast from fp32 on the way. The merged operations are applied with
-// the arithmetic of the kernels they replace (each one on the value rounded to the output type),
-// so a replay produces the bits the unmerged sequence produces. HCHIP_NO_FUSION=1 at
-// hc_capture_begin turns the rewrite off.
+// caller's program, that a result has exactly one reader, and to replace a chain of launches by
+// one launch that does the same arithmetic, intermediate by intermediate (each value rounded to
+// the tensor type where the separate kernel would have stored it), so that a replay produces the
+// bits the unmerged sequence produces. The passes, in the order fuse_recording runs them:
+//   fuse_products         matmul -> + row -> + row | + matrix | GELU   (a Linear layer's bias,
+//                         activation, residual; <= 3 operations, <= 1 matrix operand, GELU last
+//                         and not after a matrix operand; the row may be fp32 -> cast -> fp16)
+//   fuse_swapped_batches  swap of two batch axes -> batchedMatmul -> swap back: through strides
+//   fuse_layernorms       [cast] -> normalize -> [gain + c] -> mulAdd -> [cast]: one row kernel
+//   fuse_softmaxes        [* s] -> [+ mask] -> logSoftmax -> [exp]: one row kernel
+//   fuse_product_groups   products of one shape over the same input (q, k, v): one launch
+// A merged launch stands where the last entry of its chain stood. HCHIP_NO_FUSION=1 at
+// hc_capture_end turns the rewrite off.
 
 static bool aligned16(const void* p);
 static const char* dtype_name(int dtype);
