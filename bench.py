@@ -13,7 +13,7 @@ Also reported in the same line:
                 single-thread triple loop) timed on this box's host cores on a bounded row slab;
                 extra.cpu_reference_path holds the same for configs 1 and 4 (sgemm through OpenBLAS
                 with its thread count, the bandwidth-bound ops on one thread)
-  extra         the other BASELINE configs: fp32 1024^3, the ragged fp16 sweep, attention-shaped
+  extra         the other benchmark configurations: fp32 1024^3, the ragged fp16 sweep, attention-shaped
                 batched GEMMs, the bandwidth-bound ops at [8192,4096] with GB/s against the 8 TB/s
                 HBM peak (short kernels are timed as graph-replayed batches: device-side duration
                 per launch), and the transformer forward pass, eager and as one graph replay
@@ -564,7 +564,7 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--no-extra", action="store_true", help="skip the other BASELINE configs")
+    ap.add_argument("--no-extra", action="store_true", help="skip the other benchmark configurations")
     ap.add_argument("--only", default="", help="comma-separated parts to run: headline,cfg1,...,cfg5 (default: all)")
     ap.add_argument("--no-graph", action="store_true",
                     help="skip the graph-replay variant of the transformer (rocprofv3's tracer crashes "
