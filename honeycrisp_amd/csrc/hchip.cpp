@@ -609,6 +609,7 @@ extern "C" int hc_capture_begin(hc_ctx* ctx) {
   ctx->graphs.push_back(ctx->capturing);
   ctx->lazy = true;   // launches are listed, and enqueued on the capturing stream at hc_capture_end
   ctx->pending.clear();
+  ctx->dead.clear();
   return HC_OK;
 }
 
