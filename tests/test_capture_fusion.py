@@ -204,6 +204,58 @@ def test_blocks_of_merged_intermediates_return_to_the_pool(hip_backend, monkeypa
         fused.graph.destroy()
 
 
+def test_a_callers_own_kernel_is_a_barrier(hip_backend, monkeypatch):
+    """A launch through hc_launch declares no buffers: it may read or write anything, so nothing
+    is merged across it (here it sits between a product and the addition of its bias)."""
+    import ctypes
+    import os
+    path = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "bench_probe.hsaco")
+    if not os.path.exists(path):
+        pytest.skip("bench_probe.hsaco is not built")
+    lib, ctx = hip_backend._lib, hip_backend._ctx
+    image = open(path, "rb").read()
+    buf = ctypes.create_string_buffer(image, len(image))
+    module, fn = ctypes.c_void_p(), ctypes.c_void_p()
+    hip_backend._check(lib.hc_module_load(ctx, buf, len(image), ctypes.byref(module)))
+    hip_backend._check(lib.hc_module_get_function(module, b"hc_probe_mfma_f16_16x16x32", ctypes.byref(fn)))
+
+    class Args(ctypes.Structure):
+        _fields_ = [("data", ctypes.c_void_p), ("out", ctypes.c_void_p), ("iters", ctypes.c_uint32), ("chunks", ctypes.c_uint32)]
+
+    rng = np.random.default_rng(15)
+    with hip_backend.use():
+        x, w, bias, _ = operands(rng, DType.float16, 256, 128, 256)
+        data = Tensor(data=rng.standard_normal((4096,)).astype(np.float32), dtype=DType.float16)
+        sink = Tensor(data=np.zeros((4 * 256,), np.float32))
+
+        def own_kernel():
+            args = Args(data.data.ptr, sink.data.ptr, 1, 4096 * 2 // 16)
+            grid, block = (ctypes.c_uint32 * 3)(4, 1, 1), (ctypes.c_uint32 * 3)(256, 1, 1)
+            hip_backend._check(lib.hc_launch(ctx, fn, grid, block, 0, ctypes.byref(args), ctypes.sizeof(args)))
+
+        def with_barrier():
+            h = Tensor.matmul(x, False, w, False, False)
+            own_kernel()
+            return (h + bias).gelu()
+
+        def without():      # (the product's result is released before the caller's kernel is issued)
+            out = (Tensor.matmul(x, False, w, False, False) + bias).gelu()
+            own_kernel()
+            return out
+
+        def still_held():   # ... and here it is not: the caller's kernel might read it
+            h = Tensor.matmul(x, False, w, False, False)
+            out = (h + bias).gelu()
+            own_kernel()
+            return out
+
+        check(hip_backend, monkeypatch, with_barrier, removed=0)
+        check(hip_backend, monkeypatch, without, removed=2)
+        check(hip_backend, monkeypatch, still_held, removed=0)
+    hip_backend.sync()
+    hip_backend._check(lib.hc_module_unload(ctx, module))
+
+
 def test_other_forms_of_add_are_left_alone(hip_backend, monkeypatch):
     rng = np.random.default_rng(8)
     with hip_backend.use():
