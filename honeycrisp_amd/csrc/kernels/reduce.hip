@@ -470,6 +470,11 @@ __device__ __forceinline__ void stream_row_out(const T* row, T* out, uint32_t n,
 
 // ---------------------------------------------------------------- logSoftmax
 
+// exp of an fp32 value inside a kernel whose results are rounded to T: the library's expf for fp32
+// tensors; for fp16 tensors (11 significant bits) the hardware's exp2, about 1 ulp of fp32, at a
+// fifth of the instructions: an fp16 softmax row is bound by these, not by memory.
+template <typename T> __device__ __forceinline__ float exp_in(float x) { return sizeof(T) == 2 ? exp_hw(x) : expf(x); }
+
 // logSoftmax (BackendCPU.swift:1000-1038): max, sum of expf(x - max), x - (logf(sum) + max),
 // all in Float. Rows (inner == 1): a wave or a block per row; the row stays in registers when
 // it fits, else passes 2 and 3 re-read it (L2).
@@ -489,7 +494,7 @@ template <typename T, int LANES> __device__ __forceinline__ void log_softmax_row
     r.each(n, lane, [&](float x) { if (x > m) m = x; });
     m = Team<LANES>::reduce(m, MaxOp(), lds);
     float s = 0.0f;
-    r.each(n, lane, [&](float x) { s += expf(x - m); });
+    r.each(n, lane, [&](float x) { s += exp_in<T>(x - m); });
     s = Team<LANES>::reduce(s, SumOp(), lds);
     const float log_sum = logf(s) + m;
     r.store(out, n, lane, [&](float x) { return x - log_sum; });
@@ -499,7 +504,7 @@ template <typename T, int LANES> __device__ __forceinline__ void log_softmax_row
   stream_row<T, LANES>(in, n, lane, [&](float x, uint32_t) { if (x > m) m = x; });
   m = Team<LANES>::reduce(m, MaxOp(), lds);
   float s = 0.0f;
-  stream_row<T, LANES>(in, n, lane, [&](float x, uint32_t) { s += expf(x - m); });
+  stream_row<T, LANES>(in, n, lane, [&](float x, uint32_t) { s += exp_in<T>(x - m); });
   s = Team<LANES>::reduce(s, SumOp(), lds);
   const float log_sum = logf(s) + m;
   stream_row_out<T, LANES>(in, out, n, lane, [&](float x, uint32_t) { return x - log_sum; });
@@ -613,7 +618,7 @@ template <typename T, int LANES> __device__ __forceinline__ void softmax_chain_r
   r.each(n, lane, [&](float x) { if (x > mx) mx = x; });
   mx = Team<LANES>::reduce(mx, MaxOp(), lds);
   float s = 0.0f;
-  r.each(n, lane, [&](float x) { s += expf(x - mx); });
+  r.each(n, lane, [&](float x) { s += exp_in<T>(x - mx); });
   s = Team<LANES>::reduce(s, SumOp(), lds);
   const float log_sum = logf(s) + mx;
   const bool then_exp = (p.flags & HCK_SM_EXP) != 0;
@@ -763,6 +768,19 @@ template <typename TI, typename TO> __device__ __forceinline__ void layernorm_ro
         for (int i = 0; i < VEC; i++) f(v[c][i]);
       }
   };
+  // the row operands of the affine part: fetched now, used after the two reductions
+  const bool affine = (p.flags & HCK_LN_AFFINE) != 0, gain_add = (p.flags & HCK_LN_GAIN_ADD) != 0;
+  float g[CHUNKS][VEC], b[CHUNKS][VEC];
+  if (affine) {
+#pragma unroll
+    for (int c = 0; c < CHUNKS; c++) {
+      const uint32_t k = (lane + LANES * c) * VEC;
+      if (k < n) {
+        load_vec<float, VEC>((const float*)p.gain, k, 1, g[c]);
+        load_vec<float, VEC>((const float*)p.bias, k, 1, b[c]);
+      }
+    }
+  }
   const float inv_n = 1.0f / (float)n;
   float s = 0.0f;
   each([&](float x) { s += x; });
@@ -777,23 +795,17 @@ template <typename TI, typename TO> __device__ __forceinline__ void layernorm_ro
   const float var = sq * inv_n;
   const float shifted = var + p.eps;
   const float normer = 1.0f * 1.0f * pow_like(shifted, -0.5f);
-  const bool affine = (p.flags & HCK_LN_AFFINE) != 0, gain_add = (p.flags & HCK_LN_GAIN_ADD) != 0;
 #pragma unroll
   for (int c = 0; c < CHUNKS; c++) {
     const uint32_t k = (lane + LANES * c) * VEC;
     if (k < n) {
-      float g[VEC] = {1.0f, 1.0f, 1.0f, 1.0f}, b[VEC] = {0.0f, 0.0f, 0.0f, 0.0f};
-      if (affine) {
-        load_vec<float, VEC>((const float*)p.gain, k, 1, g);
-        load_vec<float, VEC>((const float*)p.bias, k, 1, b);
-      }
       TO o[VEC];
 #pragma unroll
       for (int i = 0; i < VEC; i++) {
         float y = (v[c][i] - mean) * normer;
         if (affine) {
-          const float coeff = gain_add ? g[i] + p.gain_add : g[i];
-          y = y * coeff + b[i];
+          const float coeff = gain_add ? g[c][i] + p.gain_add : g[c][i];
+          y = y * coeff + b[c][i];
         }
         o[i] = narrow<TO>(y);
       }
