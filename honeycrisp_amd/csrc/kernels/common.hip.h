@@ -225,13 +225,21 @@ __device__ __forceinline__ void gemm_tile_of_block(const hck_gemm_args& p, uint3
 // element-wise kernels would have produced. A lane's pieces all lie in the same columns, so the row
 // operands (a bias) are fetched once per kernel; the matrix operand (at most one of the three
 // operations) is fetched for a few pieces at a time, all loads in flight before the first use.
-// The operands of the three stages for this workgroup's product (a member of a group has its own).
-struct GemmEpilogueOperands {
-  const void *p0, *p1, *p2;
-};
-__device__ __forceinline__ GemmEpilogueOperands gemm_epilogue_operands(const hck_gemm_args& p, uint32_t member) {
-  if (p.group != 0) return GemmEpilogueOperands{p.g_ep[0][member], p.g_ep[1][member], p.g_ep[2][member]};
-  return GemmEpilogueOperands{p.ep_ptr[0], p.ep_ptr[1], p.ep_ptr[2]};
+// Entry `member` (wave-uniform, < 4) of a table in the kernel's argument struct, picked with scalar
+// selects. An index computed at run time would make the compiler fetch the entry with a vector
+// load; its result then sits in the same in-order counter as the direct-to-LDS loads of the main
+// loop, and the first use waits for every one of those: the whole prefetch pipeline drains before
+// the first MFMA (a 2048 x 512 x 2048 product took 24 us instead of 9).
+template <typename P> __device__ __forceinline__ P gemm_table_entry(const P (&table)[4], uint32_t member) {
+  return member == 0 ? table[0] : member == 1 ? table[1] : member == 2 ? table[2] : table[3];
+}
+// The operand of stage s for this workgroup's product (a member of a group has its own). The three
+// are kept as three values, never as a struct or an array: an aggregate whose member is picked by
+// a run-time condition ends up in memory (the compiler promoted it to LDS, and the LDS write that
+// this takes waits for every direct-to-LDS load in flight).
+__device__ __forceinline__ const void* gemm_epilogue_operand(const hck_gemm_args& p, int s, uint32_t member) {
+  if (p.group != 0) return s == 0 ? gemm_table_entry(p.g_ep[0], member) : s == 1 ? gemm_table_entry(p.g_ep[1], member) : gemm_table_entry(p.g_ep[2], member);
+  return s == 0 ? p.ep_ptr[0] : s == 1 ? p.ep_ptr[1] : p.ep_ptr[2];
 }
 
 template <typename T, typename Chunk16>
@@ -257,11 +265,11 @@ __device__ __forceinline__ Chunk16 gemm_epilogue_row_piece(uint32_t kind, const 
 
 // the matrix operand's piece for the output piece at (row, col); one of the stages has one
 template <typename T, typename Chunk16>
-__device__ __forceinline__ Chunk16 gemm_epilogue_matrix_piece(const hck_gemm_args& p, const GemmEpilogueOperands& ops,
-                                                              uint32_t row, uint32_t col) {
+__device__ __forceinline__ Chunk16 gemm_epilogue_matrix_piece(const hck_gemm_args& p, const void* p0, const void* p1,
+                                                              const void* p2, uint32_t row, uint32_t col) {
   // (stage picked with scalar selects, then a single load: no register is written twice)
   const bool s0 = p.ep_kind[0] == HCK_EP_ADD_MATRIX, s1 = p.ep_kind[1] == HCK_EP_ADD_MATRIX;
-  const void* base = s0 ? ops.p0 : s1 ? ops.p1 : ops.p2;
+  const void* base = s0 ? p0 : s1 ? p1 : p2;
   const uint32_t ld = s0 ? p.ep_ld[0] : s1 ? p.ep_ld[1] : p.ep_ld[2];
   return *reinterpret_cast<const Chunk16*>((const T*)base + (size_t)row * ld + col);
 }
@@ -309,7 +317,7 @@ __device__ __forceinline__ Chunk16 gemm_epilogue_apply(const hck_gemm_args& p, C
 // their own in which no such register exists, and their stores are never waited for.
 template <typename T, typename Chunk16, bool EDGE, uint32_t GROUP, bool COL_FIXED, bool MATRIX, bool GELU, typename LdsPiece,
           typename RowOf, typename ColOf>
-__device__ __forceinline__ void gemm_store_group_merged(const hck_gemm_args& p, const GemmEpilogueOperands& ops, Chunk16 r0,
+__device__ __forceinline__ void gemm_store_group_merged(const hck_gemm_args& p, const void* p0, const void* p1, const void* p2, Chunk16 r0,
                                                         Chunk16 r1, Chunk16 r2, T* C, uint32_t it0, LdsPiece lds_piece, RowOf row_of,
                                                         ColOf col_of) {
   Chunk16 v[GROUP], m[MATRIX ? GROUP : 1], q0[GROUP], q1[GROUP], q2[GROUP];
@@ -318,10 +326,10 @@ __device__ __forceinline__ void gemm_store_group_merged(const hck_gemm_args& p, 
     const uint32_t row = row_of(it0 + b), col = col_of(it0 + b);
     const bool inside = !EDGE || (row < p.M && col < p.N);
     v[b] = lds_piece(it0 + b);
-    if (MATRIX) m[b] = inside ? gemm_epilogue_matrix_piece<T, Chunk16>(p, ops, row, col) : Chunk16{};
-    q0[b] = COL_FIXED ? r0 : gemm_epilogue_row_piece<T, Chunk16>(p.ep_kind[0], ops.p0, col, inside);
-    q1[b] = COL_FIXED ? r1 : gemm_epilogue_row_piece<T, Chunk16>(p.ep_kind[1], ops.p1, col, inside);
-    q2[b] = COL_FIXED ? r2 : gemm_epilogue_row_piece<T, Chunk16>(p.ep_kind[2], ops.p2, col, inside);
+    if (MATRIX) m[b] = inside ? gemm_epilogue_matrix_piece<T, Chunk16>(p, p0, p1, p2, row, col) : Chunk16{};
+    q0[b] = COL_FIXED ? r0 : gemm_epilogue_row_piece<T, Chunk16>(p.ep_kind[0], p0, col, inside);
+    q1[b] = COL_FIXED ? r1 : gemm_epilogue_row_piece<T, Chunk16>(p.ep_kind[1], p1, col, inside);
+    q2[b] = COL_FIXED ? r2 : gemm_epilogue_row_piece<T, Chunk16>(p.ep_kind[2], p2, col, inside);
   }
 #pragma unroll
   for (uint32_t b = 0; b < GROUP; b++) {
@@ -336,15 +344,15 @@ __device__ __forceinline__ void gemm_store_group_merged(const hck_gemm_args& p, 
 // LDS, not the accumulators, and copies of it for every slab would multiply the kernel's code).
 template <typename T, typename Chunk16, bool EDGE, uint32_t NIT, bool COL_FIXED, uint32_t MAX_GROUP, bool MATRIX, bool GELU,
           typename LdsPiece, typename RowOf, typename ColOf>
-__device__ __forceinline__ void gemm_store_slab_merged_as(const hck_gemm_args& p, const GemmEpilogueOperands& ops, Chunk16 r0,
+__device__ __forceinline__ void gemm_store_slab_merged_as(const hck_gemm_args& p, const void* p0, const void* p1, const void* p2, Chunk16 r0,
                                                           Chunk16 r1, Chunk16 r2, T* C, LdsPiece lds_piece, RowOf row_of,
                                                           ColOf col_of) {
   constexpr uint32_t GROUP = (MAX_GROUP >= 4 && NIT % 4 == 0) ? 4 : (MAX_GROUP >= 3 && NIT % 3 == 0) ? 3 : (MAX_GROUP >= 2 && NIT % 2 == 0) ? 2 : 1;
   if constexpr (NIT == GROUP) {
-    gemm_store_group_merged<T, Chunk16, EDGE, GROUP, COL_FIXED, MATRIX, GELU>(p, ops, r0, r1, r2, C, 0u, lds_piece, row_of, col_of);
+    gemm_store_group_merged<T, Chunk16, EDGE, GROUP, COL_FIXED, MATRIX, GELU>(p, p0, p1, p2, r0, r1, r2, C, 0u, lds_piece, row_of, col_of);
   } else {
 #pragma nounroll
     for (uint32_t it0 = 0; it0 < NIT; it0 += GROUP)
-      gemm_store_group_merged<T, Chunk16, EDGE, GROUP, COL_FIXED, MATRIX, GELU>(p, ops, r0, r1, r2, C, it0, lds_piece, row_of, col_of);
+      gemm_store_group_merged<T, Chunk16, EDGE, GROUP, COL_FIXED, MATRIX, GELU>(p, p0, p1, p2, r0, r1, r2, C, it0, lds_piece, row_of, col_of);
   }
 }

@@ -226,10 +226,12 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
   T* C = (T*)p.c + batch_hi * p.c_bs + batch_lo * p.c_bs2;
   if (p.group != 0) {  // a member of a group of products over the same A
     A = (const T*)p.a;
-    B = (const T*)p.g_b[batch];
-    C = (T*)p.g_c[batch];
+    B = (const T*)gemm_table_entry(p.g_b, batch);
+    C = (T*)gemm_table_entry(p.g_c, batch);
   }
-  const GemmEpilogueOperands ep_ops = gemm_epilogue_operands(p, batch);
+  const void* const ep_p0 = gemm_epilogue_operand(p, 0, batch);
+  const void* const ep_p1 = gemm_epilogue_operand(p, 1, batch);
+  const void* const ep_p2 = gemm_epilogue_operand(p, 2, batch);
 #else
   const T* A = (const T*)p.a + batch * p.a_bs;
   const T* B = (const T*)p.b + batch * p.b_bs;
@@ -383,9 +385,9 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
   Chunk ep_r0 = Chunk{}, ep_r1 = Chunk{}, ep_r2 = Chunk{};
   if (EP_COL_FIXED && p.ep_kind[0] != HCK_EP_NONE) {
     const bool ok = !EDGE || ep_col < p.N;
-    ep_r0 = gemm_epilogue_row_piece<T, Chunk>(p.ep_kind[0], ep_ops.p0, ep_col, ok);
-    ep_r1 = gemm_epilogue_row_piece<T, Chunk>(p.ep_kind[1], ep_ops.p1, ep_col, ok);
-    ep_r2 = gemm_epilogue_row_piece<T, Chunk>(p.ep_kind[2], ep_ops.p2, ep_col, ok);
+    ep_r0 = gemm_epilogue_row_piece<T, Chunk>(p.ep_kind[0], ep_p0, ep_col, ok);
+    ep_r1 = gemm_epilogue_row_piece<T, Chunk>(p.ep_kind[1], ep_p1, ep_col, ok);
+    ep_r2 = gemm_epilogue_row_piece<T, Chunk>(p.ep_kind[2], ep_p2, ep_col, ok);
   }
 #endif
   const uint32_t r16 = lane & 15, grp = lane >> 4;
@@ -433,7 +435,7 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
 #ifdef HC_GEMM_MERGED
       if constexpr (MODE != 0) {
         gemm_store_slab_merged_as<T, Chunk, EDGE, 32 * UNITS / 64, EP_COL_FIXED, (MODE == 3 ? 1 : 2), MODE == 2, MODE == 3>(
-            p, ep_ops, ep_r0, ep_r1, ep_r2, C,
+            p, ep_p0, ep_p1, ep_p2, ep_r0, ep_r1, ep_r2, C,
             [=](uint32_t it) {
               const uint32_t piece = it * 64 + lane, r = piece / UNITS, u = piece % UNITS;
               return *reinterpret_cast<const Chunk*>(slab + r * RB + ((u ^ unit_swz(r)) * 16));

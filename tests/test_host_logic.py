@@ -116,5 +116,12 @@ def test_build_refuses_register_tiled_kernels_that_use_scratch_memory():
         """)
     assert build.kernels_with_scratch(remarks, 128) == ["hc_gemm_b (1088 bytes/lane)"]
     assert build.kernels_with_scratch(remarks, 16) == ["hc_gemm_b (1088 bytes/lane)", "hc_gemm_c (68 bytes/lane)"]
+    lds = textwrap.dedent("""\
+        k.hip:9:1: remark: Function Name: hc_gemm_a [-Rpass-analysis=kernel-resource-usage]
+        k.hip:9:1: remark:     LDS Size [bytes/block]: 65536 [-Rpass-analysis=kernel-resource-usage]
+        k.hip:9:1: remark: Function Name: hc_gemm_b [-Rpass-analysis=kernel-resource-usage]
+        k.hip:9:1: remark:     LDS Size [bytes/block]: 71680 [-Rpass-analysis=kernel-resource-usage]
+        """)
+    assert build.kernels_with_promoted_private_data(lds) == ["hc_gemm_b (71680 bytes of LDS)"]
     assert {"gemm_dma", "gemm_dma2", "gemm_mi16", "gemm_mi16_m"} <= set(build.NO_SCRATCH)
     assert set(build.NO_SCRATCH) <= {name for name, _src, _flags in build.KERNELS}
