@@ -3111,6 +3111,22 @@ extern "C" int hc_concat(hc_ctx* ctx, int dtype, const void* const* inputs, cons
 
 // ------------------------------------------------------------------ matmul
 
+// True if `slack` bytes after the `bytes` at `ptr` can be read: both lie inside one block that this
+// context handed out. (The tiled GEMM kernels fetch whole 16-byte pieces; with rows that are not a
+// whole number of pieces, the last piece of the last row ends up to 14 bytes after the operand.)
+static bool readable_past(hc_ctx* ctx, const void* ptr, uint64_t bytes, uint64_t slack) {
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  const uintptr_t lo = (uintptr_t)ptr, hi = lo + bytes + slack;
+  auto it = ctx->live.find(const_cast<void*>(ptr));
+  if (it != ctx->live.end()) return bytes + slack <= it->second;
+  for (auto& blk : ctx->live) {  // a view into a block
+    const uintptr_t start = (uintptr_t)blk.first;
+    if (lo >= start && lo < start + blk.second) return hi <= start + blk.second;
+  }
+  return false;
+}
+
+
 extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, int trans_a,
                          const void* b, int trans_b, int trans_out, int64_t rows, int64_t inner,
                          int64_t cols, void* out) {
@@ -3191,6 +3207,44 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
   char ma = mode(k.a, a_rs, a_cs, k.a_bs);
   char mb = mode(k.b, b_cs, b_rs, k.b_bs);
   char name[64];
+  const bool c_unaligned = !aligned16(out) || N % P != 0;
+
+  // A last row or column of tiles that is almost empty costs as much as a full one: 4097 rows
+  // are 17 rows of 256-row tiles, i.e. two rounds on a device that 16 x 16 tiles fill exactly.
+  // Products that are a few rows or columns over a multiple of 256 are therefore split into the
+  // multiple-of-256 body and thin fringes, each run as a product of its own on sub-blocks of the
+  // same buffers (same strides, offset pointers).
+  // (only long products: the fringes are skinny products of their own that take tens of
+  // microseconds, which a short body does not win back)
+  auto fringe = [&](uint32_t d) { return d >= 2048 && d % 256 != 0 && d % 256 <= 32 ? d % 256 : 0u; };
+  // (an output of 4 M elements, or half of that over a K long enough for 2^33 multiply-adds)
+  const bool large = (uint64_t)M * N >= (1ull << 22) ||
+                     ((uint64_t)M * N >= (1ull << 21) && (uint64_t)M * N * K >= (1ull << 33));
+  const bool peelable = K >= 2048 && large && (fringe(M) != 0 || fringe(N) != 0) && !getenv("HCHIP_GEMM_TILE") &&
+                        !getenv("HCHIP_GEMM_NO_PEEL");
+
+  // Operands and outputs whose rows are not 16-byte aligned (odd extents, odd base addresses): the
+  // edge variants of the direct-to-LDS kernels take them as they are. Their loads and stores need
+  // no alignment; what a 16-byte piece holds beyond K is cleared in LDS, beyond N it feeds columns
+  // that are never stored, and the piece of C that straddles N leaves element by element. Needed
+  // for that: the up to 14 bytes after an operand that the last piece of its last row covers are
+  // readable (the operand lies inside a block of this context with that much room).
+  // HCHIP_GEMM_NO_DIRECT=1 switches this off (measurements, tests).
+  bool loose = false;
+  if ((ma == 'x' || mb == 'x' || c_unaligned) && K > 0 && batch <= 65535 && !getenv("HCHIP_GEMM_NO_DIRECT")) {
+    auto loose_mode = [&](char m, uint32_t row_stride, uint32_t k_stride) -> char {
+      return m != 'x' ? m : k_stride == 1 ? 'k' : row_stride == 1 ? 'r' : 'x';
+    };
+    const char la = loose_mode(ma, a_rs, a_cs), lb = loose_mode(mb, b_cs, b_rs);
+    const uint64_t a_bytes = ((uint64_t)(batch - 1) * k.a_bs + (uint64_t)M * K) * el;
+    const uint64_t b_bytes = ((uint64_t)(batch - 1) * k.b_bs + (uint64_t)K * N) * el;
+    if (la != 'x' && lb != 'x' && (ma != 'x' || readable_past(ctx, k.a, a_bytes, 16)) &&
+        (mb != 'x' || readable_past(ctx, k.b, b_bytes, 16))) {
+      ma = la;
+      mb = lb;
+      loose = true;
+    }
+  }
 
   // Operands whose rows are not 16-byte aligned (odd extents, odd base addresses) would fall
   // to scalar loads; for anything but tiny products it pays to re-pitch them first: a copy
@@ -3199,11 +3253,10 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
   Scratch scratch(ctx);
   void* c_padded = nullptr;
   uint32_t c_ld = N;
-  const bool c_unaligned = !aligned16(out) || N % P != 0;
   const double work = (double)M * (double)N * (double)K * (double)batch;
   // (the scalar loads of the general kernel cost about 4 us per 64 of K and tile: a long K pays
   // for the copies much earlier than a large output does)
-  if ((ma == 'x' || mb == 'x' || c_unaligned) && K > 0 && (work >= 16777216.0 || (work >= 2097152.0 && K >= 256)) &&
+  if (!loose && (ma == 'x' || mb == 'x' || c_unaligned) && K > 0 && (work >= 16777216.0 || (work >= 2097152.0 && K >= 256)) &&
       batch <= 65535 &&
       !getenv("HCHIP_GEMM_NO_REPITCH")) {
     auto round_up = [&](uint32_t v) { return (v + P - 1) / P * P; };
@@ -3299,7 +3352,8 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
       // The thin operand is read by every wave: unless it already is contiguous along k with
       // aligned rows, pack it first as [q][k] (a few KiB that then stay in the caches).
       Scratch packed(ctx);
-      const bool x_along_k = sk.x_ks == 1 && aligned16(sk.x) && sk.x_ps % P == 0 && (batch <= 1 || sk.x_bs % P == 0);
+      // (the long operand is taken at any alignment)
+      const bool x_along_k = sk.x_ks == 1;
       // (only the wave-per-row kernel reads the thin operand with vector loads; the other one takes
       // it element by element with any strides)
       if (x_along_k &&
@@ -3322,7 +3376,7 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
         snprintf(sname, sizeof(sname), "hc_gemm_skinny_k_%s_%s", dtype_name(dtype), tq);
         return launch(ctx, sname, ceil_div(sk.L, HCK_BLOCK / 64), (uint32_t)batch, &sk, sizeof(sk));
       }
-      if (sk.x_ps == 1 && aligned16(sk.x) && sk.x_ks % P == 0 && (batch <= 1 || sk.x_bs % P == 0)) {
+      if (sk.x_ps == 1) {
         // a workgroup per (64 lanes x 16 bytes of p, chunk of k): about two per CU, at least 32 k each
         const uint64_t cus = (uint64_t)ctx->props.multiProcessorCount;
         const uint64_t ptiles = ceil_div(sk.L, 64 * P);
@@ -3356,8 +3410,10 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
     bool mi16 = dma && dtype == HC_F16 && which && strcmp(which, "mi16") == 0;
     bool dma2 = dma && which && (strcmp(which, "dma2") == 0 || mi16);
     uint32_t slice = (uint32_t)(64 / el);
-    const bool eligible = ma != 'x' && mb != 'x' && K > 0 && aligned16(k.c) &&
-                          (dma ? (k.c_rs % P == 0 && (batch <= 1 || k.c_bs % P == 0)) : (dtype == HC_F16 && K % 64 == 0));
+    const bool eligible = ma != 'x' && mb != 'x' && K > 0 &&
+                          (loose ? dma
+                                 : aligned16(k.c) && (dma ? (k.c_rs % P == 0 && (batch <= 1 || k.c_bs % P == 0))
+                                                          : (dtype == HC_F16 && K % 64 == 0)));
     if (eligible) {
       const char* force = getenv("HCHIP_GEMM_TILE");
       auto whole = [&](uint32_t tm, uint32_t tn) { return M % tm == 0 && N % tn == 0 && K % slice == 0; };
@@ -3492,7 +3548,7 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
 
         if (dma2) slice = (uint32_t)(128 / el);
       }
-      if (bm != 0) edge = !whole(bm, bn);
+      if (bm != 0) edge = !whole(bm, bn) || loose;   // (only the edge kernels take rows at any alignment)
     }
     if (bm != 0) {
       k.tiles_m = (uint32_t)ceil_div(M, bm);
@@ -3510,7 +3566,7 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
       }
       snprintf(name, sizeof(name), "hc_gemm_%s_%s_%ux%u_%c%c%s", dtype_name(dtype), dma ? (mi16 ? "mi16" : dma2 ? "dma2" : "dma") : "fast", bm, bn,
                ma == 'k' ? 'k' : 'm', mb == 'k' ? 'k' : 'n', edge ? "_e" : "");
-    } else if (ma == 'x' || mb == 'x')
+    } else if (ma == 'x' || mb == 'x' || loose)
       snprintf(name, sizeof(name), "hc_gemm_%s_xx", dtype_name(dtype));
     else
       snprintf(name, sizeof(name), "hc_gemm_%s_%c%c", dtype_name(dtype), ma == 'k' ? 'k' : 'm',
@@ -3518,8 +3574,8 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
     const uint64_t tiles = (uint64_t)k.tiles_m * k.tiles_n;
     // One launch of a direct-to-LDS kernel that writes the caller's dense [M, N] matrix from the
     // caller's own operands: a recording may merge what follows into its epilogue.
-    if (whole_call && bm != 0 && dma && batch == 1 && !trans_out && !c_padded && k.a == a && k.b == b && k.c == out &&
-        k.c_rs == N) {
+    if (whole_call && bm != 0 && dma && !loose && batch == 1 && !trans_out && !c_padded && k.a == a && k.b == b &&
+        k.c == out && k.c_rs == N) {
       note.tag = hc_pending::GEMM;
       note.meta.dtype = dtype;
       note.meta.rows = M;
@@ -3527,8 +3583,8 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
       note.meta.out = out;
     }
     // ... and a batched one may read or write through a swap of the batch axes
-    if (whole_call && bm != 0 && dma && batch > 1 && batch <= 65535 && !trans_out && !c_padded && k.a == a && k.b == b &&
-        k.c == out && k.c_rs == N) {
+    if (whole_call && bm != 0 && dma && !loose && batch > 1 && batch <= 65535 && !trans_out && !c_padded && k.a == a &&
+        k.b == b && k.c == out && k.c_rs == N) {
       note.tag = hc_pending::BMM;
       note.meta.dtype = dtype;
       note.meta.rows = M;
@@ -3549,19 +3605,9 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
     }
     return HC_OK;
   };
-  // A last row or column of tiles that is almost empty costs as much as a full one: 4097 rows
-  // are 17 rows of 256-row tiles, i.e. two rounds on a device that 16 x 16 tiles fill exactly.
-  // Products that are a few rows or columns over a multiple of 256 are therefore split into the
-  // multiple-of-256 body and thin fringes, each run as a product of its own on sub-blocks of the
-  // same buffers (same strides, offset pointers).
-  // (only long products: the fringes are skinny products of their own that take tens of
-  // microseconds, which a short body does not win back)
-  auto fringe = [&](uint32_t d) { return d >= 2048 && d % 256 != 0 && d % 256 <= 32 ? d % 256 : 0u; };
-  const bool tuned = ma != 'x' && mb != 'x' && K >= 2048 && !getenv("HCHIP_GEMM_TILE") && !getenv("HCHIP_GEMM_NO_PEEL");
-  // (an output of 4 M elements, or half of that over a K long enough for 2^33 multiply-adds)
-  const bool large = (uint64_t)M * N >= (1ull << 22) ||
-                     ((uint64_t)M * N >= (1ull << 21) && (uint64_t)M * N * K >= (1ull << 33));
-  const uint32_t fm = tuned && large ? fringe(M) : 0, fn = tuned && large ? fringe(N) : 0;
+  // The body-plus-fringes split (see `peelable` above), for operands the tuned kernels can take
+  const bool tuned = ma != 'x' && mb != 'x' && peelable;
+  const uint32_t fm = tuned ? fringe(M) : 0, fn = tuned ? fringe(N) : 0;
   if (fm != 0 || fn != 0) {
     const uint32_t Mb = M - fm, Nb = N - fn;
     HC_TRY(run(k, Mb, Nb));

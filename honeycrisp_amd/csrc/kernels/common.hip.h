@@ -66,6 +66,17 @@ __device__ __forceinline__ void load_vec(const T* base, uint32_t off, uint32_t s
   }
 }
 
+// N consecutive elements from an address that is aligned to the element only (in the access mode
+// the runtime sets, a multi-dword load needs no alignment).
+template <typename T, int N> __device__ __forceinline__ void load_vec_loose(const T* src, T (&dst)[N]) {
+  struct __attribute__((packed, aligned(sizeof(T)))) Loose {
+    Vec<T, N> v;
+  };
+  const Vec<T, N> t = reinterpret_cast<const Loose*>(src)->v;
+#pragma unroll
+  for (int i = 0; i < N; i++) dst[i] = t.v[i];
+}
+
 // The same with the stride known at compile time: S = 1 one 16-byte load, S = 0 one element
 // repeated, S < 0 decided at run time. Kernels branch once on the (wave-uniform) strides of
 // all their operands and run a body whose loads are unconditional, so they issue back to back;
@@ -220,6 +231,14 @@ __device__ __forceinline__ void gemm_tile_of_block(const hck_gemm_args& p, uint3
 // ---- operations merged into a GEMM's epilogue (hck_gemm_args::ep_*) ----
 #include "elemwise_formulas.hip.h"
 
+// 1 in the second build of the tiled GEMM sources (kernels *_m, whose write-out applies the operations
+// a recording merged into the product), 0 in the ordinary build
+#ifdef HC_GEMM_MERGED
+#define HC_GEMM_IS_MERGED 1
+#else
+#define HC_GEMM_IS_MERGED 0
+#endif
+
 // The operations are applied to 16-byte pieces of finished outputs of type T (already rounded to
 // T), in order, each in float with one rounding to T: bit for bit what the separate broadcast-add /
 // element-wise kernels would have produced. A lane's pieces all lie in the same columns, so the row
@@ -240,6 +259,48 @@ template <typename P> __device__ __forceinline__ P gemm_table_entry(const P (&ta
 __device__ __forceinline__ const void* gemm_epilogue_operand(const hck_gemm_args& p, int s, uint32_t member) {
   if (p.group != 0) return s == 0 ? gemm_table_entry(p.g_ep[0], member) : s == 1 ? gemm_table_entry(p.g_ep[1], member) : gemm_table_entry(p.g_ep[2], member);
   return s == 0 ? p.ep_ptr[0] : s == 1 ? p.ep_ptr[1] : p.ep_ptr[2];
+}
+
+// One 16-byte piece of C (row `row`, columns col .. col + 16 / sizeof(T) - 1) leaves a tiled GEMM
+// kernel; `staged` is where the piece sits in LDS. Edge kernels skip pieces outside C. LOOSE (the
+// edge kernels of the ordinary build): a row of C may start at any element (in the access mode the
+// runtime sets, multi-dword stores need no alignment), and the piece that straddles N leaves
+// element by element, in a loop that stays rolled (it runs for one piece per row at most and must
+// not cost the write-out registers). Without LOOSE, N is a whole number of pieces.
+template <typename T, typename Chunk16, bool EDGE, bool LOOSE>
+__device__ __forceinline__ void gemm_store_piece(T* dst, uint32_t row, uint32_t col, uint32_t M, uint32_t N, Chunk16 v,
+                                                 const char* staged) {
+  static_assert(sizeof(Chunk16) == 16, "a 16-byte piece");
+  if constexpr (!LOOSE) {
+    if (!EDGE || (row < M && col < N)) *reinterpret_cast<Chunk16*>(dst) = v;
+  } else if (row < M) {
+    constexpr uint32_t PER = 16 / sizeof(T);
+    if (col + PER <= N) {
+      struct __attribute__((packed, aligned(sizeof(T)))) Loose {
+        Chunk16 v;
+      };
+      reinterpret_cast<Loose*>(dst)->v = v;
+    } else if (col < N) {
+      const T* e = reinterpret_cast<const T*>(staged);
+#pragma nounroll
+      for (uint32_t x = 0; x < N - col; x++) dst[x] = e[x];
+    }
+  }
+}
+
+// Edge kernels, K-contiguous operand (a lane's DMA piece i of a K-slice covers k = kl .. kl +
+// 16 / sizeof(T) - 1 of one row and sits at `piece`): when K is not a whole number of pieces, the
+// piece that straddles K also holds what follows the row in memory (the next row's first elements
+// where rows abut). The lane that fetched it clears those elements once its DMA has landed and
+// before the barrier that lets anybody read the slice.
+template <typename T> __device__ __forceinline__ void gemm_zero_piece_tail(char* piece, uint32_t kl, uint32_t kend) {
+  constexpr uint32_t PER = 16 / sizeof(T);
+  if (kl < kend && kl + PER > kend) {
+    T* e = reinterpret_cast<T*>(piece);
+#pragma unroll
+    for (uint32_t x = 1; x < PER; x++)
+      if (kl + x >= kend) e[x] = T(0);
+  }
 }
 
 template <typename T, typename Chunk16>

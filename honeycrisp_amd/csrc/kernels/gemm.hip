@@ -276,7 +276,7 @@ template <typename T, int TQ> __device__ __forceinline__ void skinny_k_impl(cons
   for (uint32_t k0 = lane * V; k0 < a.K; k0 += 64 * V) {
     T x[V];
     if (k0 + V <= a.K) {
-      load_vec<T, V>(X, k0, 1, x);
+      load_vec_loose<T, V>(X + k0, x);   // (rows of X start at any element)
     } else {
 #pragma unroll
       for (int e = 0; e < V; e++) x[e] = k0 + e < a.K ? X[k0 + e] : (T)0;
@@ -302,7 +302,7 @@ template <typename T, int TQ> __device__ __forceinline__ void skinny_k_impl(cons
   }
 }
 
-// Long operand contiguous along p (16-byte aligned k-rows): a lane owns V consecutive p, a
+// Long operand contiguous along p: a lane owns V consecutive p, a
 // wave reads 64 * V consecutive elements of a k-row per step; a workgroup covers one such
 // p-tile and a chunk of the k-range (grid.x = p-tiles * k-chunks), its four waves take every
 // fourth k-row and add their partial sums up in LDS; every chunk leaves its sums in a slice of its
@@ -329,7 +329,7 @@ template <typename T, int TQ> __device__ __forceinline__ void skinny_p_impl(cons
   for (uint32_t k = k_lo + wave; k < k_hi; k += WAVES) {
     T x[V];
     if (whole) {
-      load_vec<T, V>(X + (size_t)k * a.x_ks, p0, 1, x);
+      load_vec_loose<T, V>(X + (size_t)k * a.x_ks + p0, x);   // (k-rows of X start at any element)
     } else {
 #pragma unroll
       for (int e = 0; e < V; e++) x[e] = p0 + e < a.L ? X[(size_t)k * a.x_ks + p0 + e] : (T)0;

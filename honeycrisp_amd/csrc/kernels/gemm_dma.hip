@@ -186,6 +186,16 @@ template <typename T, int ROWS, int MODE> struct DmaOperand {
                                              k0 * kstride, 0, 0);
   }
 
+  // Edge kernels: clears what the piece straddling `kend` holds beyond it (gemm_zero_piece_tail),
+  // after this wave's DMA of the K-slice starting at k0 has landed in `region`.
+  __device__ __forceinline__ void zero_k_tail(char* region, uint32_t k0, uint32_t kend) const {
+    if (MODE != DMA_K) return;
+    const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+#pragma unroll
+    for (int i = 0; i < NI; i++)
+      gemm_zero_piece_tail<T>(region + (wave * NI + i) * 1024 + lane * 16, k0 + klocal(i), kend);
+  }
+
   // Read number u of sub-step s into the operand registers of tile u (DMA_K), half u%2 of
   // tile u/2 (DMA_MN, fp16) or element u%4 of tile u/4 (DMA_MN, fp32).
   __device__ __forceinline__ void read(int u, int s, const char* region, Chunk* frag) const {
@@ -310,6 +320,13 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
   static_assert(DSTRIDE * (NDMA - HALF) <= SLOTS, "more DMA instructions than MFMA slots");
 
   const uint32_t nk = (p.K + BK - 1) / BK;
+  // (edge kernels) K is not a whole number of 16-byte pieces: the last slice of a K-contiguous
+  // operand is cleaned up after it has landed
+  const bool ktail = EDGE && p.K % (16 / sizeof(T)) != 0;
+  auto zero_tail = [&](char* stage, uint32_t k0) {
+    oa.zero_k_tail(stage, k0, kend);
+    ob.zero_k_tail(stage + A_BYTES, k0, kend);
+  };
   Frags f0, f1;
 
   // K-step j out of `cur`; `nxt` holds K-step j+1, `prev` held K-step j-1.
@@ -325,6 +342,9 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
       __builtin_amdgcn_sched_barrier(0);
     }
     wait_dma<2 * NDMA>();  // K-step j+1 of this wave has landed ...
+    if constexpr (decltype(tail)::value) {
+      if (ktail && j + 2 == nk) zero_tail(nxt, (j + 1) * BK);
+    }
     lds_barrier();         // ... and everybody's; nobody reads cur any more
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -349,6 +369,9 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
 #pragma unroll
   for (int u = 0; u < HALF; u++) dma_unit(Tail{}, u, kclamp(3), lds3);
   wait_dma<2 * NDMA + HALF>();
+  if constexpr (EDGE) {
+    if (ktail && nk == 1) zero_tail(lds0, 0);
+  }
   lds_barrier();
 #pragma unroll
   for (int u = 0; u < READS; u++) read_unit(f0, lds0, 0, u);
@@ -440,7 +463,7 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
           const uint32_t r = it * RPI + lane / UNITS, u = lane % UNITS;
           const Chunk v = *reinterpret_cast<const Chunk*>(slab + r * RB + ((u ^ unit_swz(r)) * 16));
           const uint32_t row = m0 + wm + i * 32 + r, col = n0 + wn + u * (16 / ES);
-          if (!EDGE || (row < p.M && col < p.N)) *reinterpret_cast<Chunk*>(C + (size_t)row * p.c_rs + col) = v;
+          gemm_store_piece<T, Chunk, EDGE, EDGE && !HC_GEMM_IS_MERGED>(C + (size_t)row * p.c_rs + col, row, col, p.M, p.N, v, slab + r * RB + ((u ^ unit_swz(r)) * 16));
         }
       }
 #ifdef HC_GEMM_MERGED

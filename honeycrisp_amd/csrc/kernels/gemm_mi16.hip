@@ -135,6 +135,16 @@ template <int ROWS, int MODE> struct DmaOperand {
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (LDS_AS void*)(region + (wave * NI + i) * 1024), 16, off,
                                              k0 * kstride, 0, 0);
   }
+
+  // Edge kernels: clears what the piece straddling `kend` holds beyond it (gemm_zero_piece_tail),
+  // after this wave's DMA of the K-slice starting at k0 has landed in `region`.
+  __device__ __forceinline__ void zero_k_tail(char* region, uint32_t k0, uint32_t kend) const {
+    if (MODE != DMA_K) return;
+    const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+#pragma unroll
+    for (int i = 0; i < NI; i++)
+      gemm_zero_piece_tail<half_t>(region + (wave * NI + i) * 1024 + lane * 16, k0 + klocal(i), kend);
+  }
 };
 
 // f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>)
@@ -299,6 +309,13 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
 
   const uint32_t nk = (p.K + BK - 1) / BK;
   auto kclamp = [&](uint32_t j) { return (j < nk ? j : nk - 1) * BK; };  // steps past the end repeat the last one
+  // (edge kernels) K is not a whole number of 16-byte pieces: the last slice of a K-contiguous
+  // operand is cleaned up after it has landed
+  const bool ktail = EDGE && p.K % (16 / sizeof(half_t)) != 0;
+  auto zero_tail = [&](char* stage, uint32_t k0) {
+    oa.zero_k_tail(stage, k0, kend);
+    ob.zero_k_tail(stage + A_BYTES, k0, kend);
+  };
   Frags f0, f1;
 
   // (compile-time loop indices throughout: every register array is indexed statically)
@@ -326,6 +343,9 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
     __builtin_amdgcn_sched_barrier(0);
     substep(tail, f0, f1, cur, std::integral_constant<int, 1>{}, std::integral_constant<int, 1>{}, nxt, kclamp(j + 1));
     wait_dma<0>();  // K-step j+1 of this wave has landed ...
+    if constexpr (decltype(tail)::value) {
+      if (ktail && j + 2 == nk) zero_tail(nxt, (j + 1) * BK);
+    }
     lds_barrier();  // ... and everybody's; nobody reads cur any more
     __builtin_amdgcn_sched_barrier(0);
     substep(tail, f1, f0, nxt, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, cur, kclamp(j + 2));
@@ -342,6 +362,9 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
   static_for<SLOTS>([&](auto tc) { pin_acc(decltype(tc)::value); });
   __builtin_amdgcn_sched_barrier(0);
   wait_dma<U0>();
+  if constexpr (EDGE) {
+    if (ktail && nk == 1) zero_tail(lds0, 0);
+  }
   lds_barrier();
   static_for<READS>([&](auto uc) { read_unit(f0, lds0, 0, decltype(uc)::value); });
 
@@ -429,7 +452,7 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
           const uint32_t piece = it * 64 + lane, r = piece / UNITS, u = piece % UNITS;
           const Chunk v = *reinterpret_cast<const Chunk*>(slab + r * RB + ((u ^ unit_swz(r)) * 16));
           const uint32_t row = m0 + wm + ii * 32 + r, col = n0 + wn + u * 8;
-          if (!EDGE || (row < p.M && col < p.N)) *reinterpret_cast<Chunk*>(C + (size_t)row * p.c_rs + col) = v;
+          gemm_store_piece<half_t, Chunk, EDGE, EDGE && !HC_GEMM_IS_MERGED>(C + (size_t)row * p.c_rs + col, row, col, p.M, p.N, v, slab + r * RB + ((u ^ unit_swz(r)) * 16));
         }
       }
 #ifdef HC_GEMM_MERGED
