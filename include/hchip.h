@@ -200,8 +200,10 @@ int hc_launch(hc_ctx* ctx, hc_function* fn, const uint32_t grid[3], const uint32
  *  - everything else takes any element-aligned pointer and only loses its 16-byte vector
  *    accesses: the broadcasting ops (hc_broadcast, hc_binary_op, hc_bitwise_op, hc_compare,
  *    hc_mul_add, hc_add_mul, hc_when, hc_clamp), hc_reduce with inner > 1, hc_cumulative,
- *    hc_argsort, hc_gather, hc_permute, hc_concat, hc_triangular and hc_matmul (which re-pitches
- *    unaligned operands of large products into aligned scratch copies). */
+ *    hc_argsort, hc_gather, hc_permute, hc_concat, hc_triangular and hc_matmul (whose tiled
+ *    kernels fetch and store rows at any element alignment; an operand that does not leave 16
+ *    readable bytes behind its last row inside its hc_malloc block, or that was not allocated by
+ *    this context, goes through a zero-padded scratch copy instead). */
 
 /* Backend.broadcast (Backend.swift:170-172; CPU BackendCPU.swift:255-265). */
 int hc_broadcast(hc_ctx* ctx, int dtype, const void* a, const hc_strides* as, void* out);

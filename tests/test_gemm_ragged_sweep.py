@@ -6,8 +6,10 @@ What is compared, per product:
   * row slabs (first / middle / last rows, the last ones being the fringe rows) x all columns and
     all rows x column slabs (first / last columns: the fringe columns) against the CPU oracle
     (BackendCPU.swift:1260-1304 restated), tolerance 1e-2 (fp16) / 1e-4 (fp32);
-  * the whole result against the general kernel (HCHIP_GEMM_TILE=general: no tuned tile, no split)
-    and against the same call with HCHIP_GEMM_NO_PEEL=1 (tuned tiles, no split);
+  * the whole result against the general kernel (HCHIP_GEMM_TILE=general: no tuned tile, no split),
+    against the same call with HCHIP_GEMM_NO_PEEL=1 (tuned tiles, no split) and against the same call
+    with HCHIP_GEMM_NO_DIRECT=1 (rows that are not 16-byte aligned go through zero-padded copies
+    instead of being fetched and stored where they lie);
   * guard elements in front of and behind the output: nothing may be written outside C.
 """
 import os
@@ -109,6 +111,9 @@ class Product:
             with env(HCHIP_GEMM_NO_PEEL="1"):
                 whole = self.run(transA, transB, transOut)
             assert_close_arrays(np.ascontiguousarray(c), np.ascontiguousarray(whole), tol, tol)
+            with env(HCHIP_GEMM_NO_DIRECT="1"):
+                padded = self.run(transA, transB, transOut)
+            assert_close_arrays(np.ascontiguousarray(c), np.ascontiguousarray(padded), tol, tol)
 
 
 ALL_LAYOUTS = [(ta, tb, to) for to in (False, True) for ta in (False, True) for tb in (False, True)]
@@ -139,3 +144,73 @@ PEEL_SHAPES = [(1, 4104, 4096, 4112), (1, 4128, 2048, 2056), (1, 4097, 2048, 410
 def test_body_plus_fringes(hip_backend, oracle_backend, dtype, shape):
     batch, M, K, N = shape
     Product(hip_backend, oracle_backend, dtype, batch, M, K, N, seed=batch + M + K + N).check_all(ALL_LAYOUTS, "peel")
+
+
+# Rows that are not a whole number of 16-byte pieces, fetched where they lie: the piece that
+# straddles the end of a row also holds the first elements of the next row. (M, K, N); K or N odd.
+LOOSE_SHAPES = [(130, 127, 72), (66, 1001, 257), (300, 71, 129), (64, 8, 127), (257, 3, 1000), (1000, 4097, 135)]
+
+
+@pytest.mark.parametrize("dtype", [F16, F32], ids=["f16", "f32"])
+@pytest.mark.parametrize("shape", LOOSE_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_neighbouring_rows_do_not_leak(hip_backend, dtype, shape):
+    """Every other row of A (and of B^T) is infinite. A finite row's last piece reaches into its
+    infinite neighbour, so anything that leaks across the end of a row turns finite outputs into
+    NaN; they must match a float64 product of the finite rows, and the others must not be finite."""
+    M, K, N = shape
+    rng = np.random.default_rng(M + K + N)
+    np_t = dtype.numpy
+    a = (rng.standard_normal((M, K)) / np.sqrt(K)).astype(np_t)
+    b = rng.standard_normal((K, N)).astype(np_t)
+    want = a.astype(np.float64) @ b.astype(np.float64)
+    tol = TOL[dtype]
+    hip = hip_backend
+
+    def product(a_host, trans_a, b_host, trans_b):
+        da = hip.upload(np.ascontiguousarray(a_host.T if trans_a else a_host))
+        db = hip.upload(np.ascontiguousarray(b_host.T if trans_b else b_host))
+        out = hip.allocate(M * N * np.dtype(np_t).itemsize)
+        hip._check(hip._lib.hc_matmul(hip._ctx, int(dtype), 1, c_void_p(da.ptr), int(trans_a), c_void_p(db.ptr),
+                                      int(trans_b), 0, M, K, N, c_void_p(out.ptr)))
+        return out.onCPU().view(np_t)[:M * N].reshape(M, N).astype(np.float64)
+
+    # infinite rows of A (stored [M, K], K-contiguous): the odd m
+    a_inf = a.copy()
+    a_inf[1::2] = np.inf
+    for trans_b in (False, True):
+        print("rows of A", dtype.name, shape, trans_b, flush=True)
+        c = product(a_inf, False, b, trans_b)
+        assert np.all(np.isfinite(c[0::2])), "an infinite neighbouring row of A leaked into a finite one"
+        assert not np.any(np.isfinite(c[1::2]))
+        assert_close_arrays(c[0::2], want[0::2], tol, tol)
+    # infinite rows of B^T (stored [N, K], K-contiguous): the odd n
+    b_inf = b.copy()
+    b_inf[:, 1::2] = np.inf
+    for trans_a in (False, True):
+        print("rows of B^T", dtype.name, shape, trans_a, flush=True)
+        c = product(a, trans_a, b_inf, True)
+        assert np.all(np.isfinite(c[:, 0::2])), "an infinite neighbouring row of B^T leaked into a finite one"
+        assert not np.any(np.isfinite(c[:, 1::2]))
+        assert_close_arrays(c[:, 0::2], want[:, 0::2], tol, tol)
+
+
+@pytest.mark.parametrize("dtype", [F16, F32], ids=["f16", "f32"])
+def test_operand_that_fills_its_block(hip_backend, oracle_backend, dtype):
+    """Operands whose bytes are exactly a block of the allocator (a power of two) leave no room
+    behind the last row for the last piece's 16 bytes: such products go through padded copies."""
+    es = np.dtype(dtype.numpy).itemsize
+    K = 8 // es          # rows of 8 bytes: half a piece
+    M = 4096 // (K * es)  # A = 4096 bytes
+    N = 4096 // (K * es)  # B^T = 4096 bytes
+    rng = np.random.default_rng(5)
+    a = rng.standard_normal((M, K)).astype(dtype.numpy)
+    bt = rng.standard_normal((N, K)).astype(dtype.numpy)
+    with oracle_backend.use():
+        want = Tensor.batchedMatmul(Tensor(data=a[None]), False, Tensor(data=bt[None]), True, False).numpy()[0]
+    hip = hip_backend
+    da, db = hip.upload(a), hip.upload(bt)
+    out = hip.allocate(M * N * es)
+    hip._check(hip._lib.hc_matmul(hip._ctx, int(dtype), 1, c_void_p(da.ptr), 0, c_void_p(db.ptr), 1, 0, M, K, N,
+                                  c_void_p(out.ptr)))
+    got = out.onCPU().view(dtype.numpy)[:M * N].reshape(M, N)
+    assert_close_arrays(got, want, TOL[dtype], TOL[dtype])
