@@ -499,6 +499,9 @@ __device__ __forceinline__ void gemm_dma_impl(const hck_gemm_args& p, char* lds0
 #else
 #define HC_GEMM_NAME(base) base
 #endif
+// (Every stage is a __shared__ array of its own on purpose: the compiler then knows that a DMA into
+// one stage does not touch the stage a read comes from. As parts of one array it guards every LDS
+// read with a wait for all DMA in flight, and the kernels run three times slower.)
 #define DEF_DMA(T, TN, BM, BN, AN, AM, BNAME, BMODE)                                                  \
   extern "C" __global__ __launch_bounds__(256) void HC_GEMM_NAME(hc_gemm_##TN##_dma_##BM##x##BN##_##AN##BNAME)( \
       hck_gemm_args p) {                                                                              \
