@@ -72,9 +72,10 @@ def kernels_with_scratch(remarks, allowed=0):
     return bad
 
 
-def kernels_with_promoted_private_data(remarks, granule=16384):
+def kernels_with_promoted_private_data(remarks, granule=8192):
     """Names of kernels whose LDS size is not a whole number of `granule` bytes. The tiled GEMM
-    kernels declare (BM + BN) * 256 bytes of LDS, always a multiple of 16 KiB; anything on top is
+    kernels declare (BM + BN) * 256 bytes of LDS (the single-slice variants half of that), always a
+    multiple of 8 KiB; anything on top is
     a private aggregate that the compiler moved into LDS (it does that with a struct or array whose
     member is picked at run time). Writing it there waits for every direct-to-LDS load in flight:
     one such 24-byte struct made a 2048 x 512 x 2048 product take 24 us instead of 9."""

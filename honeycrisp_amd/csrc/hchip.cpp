@@ -1568,6 +1568,10 @@ static size_t dtype_size(int dtype) {
 }
 
 static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+static bool getenv_is(const char* name, const char* value) {
+  const char* v = getenv(name);
+  return v && strcmp(v, value) == 0;
+}
 
 // Build the joint broadcast descriptor for `nops` operands over one virtual shape:
 // drop size-1 axes, merge axes that are jointly mergeable (stride[d] == stride[d+1] *
@@ -3325,7 +3329,7 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
     // dma|dma2|mi16 the pipeline, =staged selects the register-staged fp16 pipeline (whole
     // tiles, K % 64 == 0).
     uint32_t bm = 0, bn = 0;
-    bool edge = false;
+    bool edge = false, one = false;
     const char* which = getenv("HCHIP_GEMM_KERNEL");
     // Skinny products (one extent of C at most 4, the other long: matrix-vector products and
     // the thinnest fringes peeled off below) are bound by reading the long operand once: no
@@ -3468,16 +3472,24 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
         // inside a workgroup, so what hides the latencies is several workgroups per CU: the largest
         // tile that still gives every CU two blocks (QK^T of 32 x [512,64] x [64,512]: 256 x 128
         // tiles 6.8 us, 128 x 128 tiles 6.2 us).
+        // With an operand that is contiguous along K such a product runs the single-slice variant
+        // (one stage of LDS, see below), which fits twice as many workgroups: four blocks per CU
+        // where a tile offers them (same scores: 128 x 64 tiles 6.7 us against 7.2 with 128 x 128).
         if (dma && (uint64_t)K * el <= 128) {
-          for (size_t ti = 0; ti < sizeof(tiles) / sizeof(tiles[0]); ti++) {
-            const uint32_t* t = tiles[ti];
-            const uint64_t blocks = ceil_div(M, t[0]) * ceil_div(N, t[1]) * (uint64_t)batch;
-            const double useful = ((double)M * N * (double)batch) / ((double)blocks * t[0] * t[1]);
-            if (blocks >= 2 * cus && useful >= 0.75) {
-              bm = t[0];
-              bn = t[1];
-              break;
+          bool found = false;
+          for (uint64_t want : {(uint64_t)4, (uint64_t)2}) {
+            if (want == 4 && !(ma == 'k' || mb == 'k')) continue;
+            for (size_t ti = 0; ti < sizeof(tiles) / sizeof(tiles[0]) && !found; ti++) {
+              const uint32_t* t = tiles[ti];
+              const uint64_t blocks = ceil_div(M, t[0]) * ceil_div(N, t[1]) * (uint64_t)batch;
+              const double useful = ((double)M * N * (double)batch) / ((double)blocks * t[0] * t[1]);
+              if (blocks >= want * cus && useful >= 0.75) {
+                bm = t[0];
+                bn = t[1];
+                found = true;
+              }
             }
+            if (found) break;
           }
         }
         // fp32 products with K >= 512 also have the 192-extent tiles of the two-stage pipeline: fp32
@@ -3547,6 +3559,9 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
         if (!which && !model_mi16 && k_contig && (uint64_t)K * el <= 128) dma2 = true;
 
         if (dma2) slice = (uint32_t)(128 / el);
+        // (the single-slice variants: one stage of LDS, no second fetch; HCHIP_GEMM_ONE=0 keeps the general loop)
+        const bool one_tile = (bm == 256 && bn == 128) || (bm == 128 && bn == 128) || (bm == 128 && bn == 64) || (bm == 64 && bn == 64);
+        one = dma2 && !mi16 && k_contig && (uint64_t)K * el <= 128 && one_tile && !getenv_is("HCHIP_GEMM_ONE", "0");
       }
       if (bm != 0) edge = !whole(bm, bn) || loose;   // (only the edge kernels take rows at any alignment)
     }
@@ -3564,8 +3579,8 @@ extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, i
             break;
           }
       }
-      snprintf(name, sizeof(name), "hc_gemm_%s_%s_%ux%u_%c%c%s", dtype_name(dtype), dma ? (mi16 ? "mi16" : dma2 ? "dma2" : "dma") : "fast", bm, bn,
-               ma == 'k' ? 'k' : 'm', mb == 'k' ? 'k' : 'n', edge ? "_e" : "");
+      snprintf(name, sizeof(name), "hc_gemm_%s_%s_%ux%u_%c%c%s%s", dtype_name(dtype), dma ? (mi16 ? "mi16" : dma2 ? "dma2" : "dma") : "fast", bm, bn,
+               ma == 'k' ? 'k' : 'm', mb == 'k' ? 'k' : 'n', one ? "_1" : "", edge ? "_e" : "");
     } else if (ma == 'x' || mb == 'x' || loose)
       snprintf(name, sizeof(name), "hc_gemm_%s_xx", dtype_name(dtype));
     else

@@ -224,7 +224,12 @@ template <typename T, int ROWS, int MODE> struct DmaOperand {
   }
 };
 
-template <typename T, int BM, int BN, int MODE_A, int MODE_B, bool EDGE>
+// ONE: the whole K is a single 128-byte slice (attention scores over 64-wide heads). Nothing to
+// prefetch and nothing to overlap inside the workgroup, so the variant fetches its one slice,
+// multiplies and stores, with one stage of LDS (`lds1` unused): twice as many workgroups fit a CU,
+// which is what hides the latencies of such a launch. (The general loop would fetch the clamped
+// "next" slices into the second stage and wait for them twice before the write-out.)
+template <typename T, int BM, int BN, int MODE_A, int MODE_B, bool EDGE, bool ONE = false>
 __device__ __forceinline__ void gemm_dma2_impl(const hck_gemm_args& p, char* lds0, char* lds1) {
   constexpr int MT = BM / 64, NT = BN / 64;
   constexpr int SLOTS = MT * NT;
@@ -377,31 +382,47 @@ __device__ __forceinline__ void gemm_dma2_impl(const hck_gemm_args& p, char* lds
     substep(tail, f1, f0, nxt, 0, 0, cur, kclamp(j + 2));
   };
 
-  // prologue: K-step 0 and the first window part of K-step 1
+  if constexpr (ONE) {
 #pragma unroll
-  for (int u = 0; u < NDMA; u++) dma_unit(Tail{}, u, 0, lds0);
-#pragma unroll
-  for (int u = 0; u < U0; u++) dma_unit(Tail{}, u, kclamp(1), lds1);
-  wait_dma<U0>();
-  if constexpr (EDGE) {
-    if (ktail && nk == 1) zero_tail(lds0, 0);
-  }
-  lds_barrier();
-#pragma unroll
-  for (int u = 0; u < READS; u++) read_unit(f0, lds0, 0, u);
-
-  uint32_t j = 0;
-  if constexpr (EDGE) {  // K-step j fetches slices j+1 and j+2: up to j = nk-4 the last slice is not among them
-    for (; j + 5 <= nk; j += 2) {
-      step(NoTail{}, lds0, lds1, j);
-      step(NoTail{}, lds1, lds0, j + 1);
+    for (int u = 0; u < NDMA; u++) dma_unit(Tail{}, u, 0, lds0);
+    wait_dma<0>();
+    if constexpr (EDGE) {
+      if (ktail) zero_tail(lds0, 0);
     }
+    lds_barrier();
+#pragma unroll
+    for (int u = 0; u < READS; u++) read_unit(f0, lds0, 0, u);
+    substep(NoTail{}, f0, f1, lds0, 1, -1, nullptr, 0);
+    substep(NoTail{}, f1, f0, lds0, 2, -1, nullptr, 0);
+    substep(NoTail{}, f0, f1, lds0, 3, -1, nullptr, 0);
+    substep(NoTail{}, f1, f0, lds0, 0, -1, nullptr, 0);  // (its reads repeat sub-step 0's: nobody uses them)
+  } else {
+    // prologue: K-step 0 and the first window part of K-step 1
+#pragma unroll
+    for (int u = 0; u < NDMA; u++) dma_unit(Tail{}, u, 0, lds0);
+#pragma unroll
+    for (int u = 0; u < U0; u++) dma_unit(Tail{}, u, kclamp(1), lds1);
+    wait_dma<U0>();
+    if constexpr (EDGE) {
+      if (ktail && nk == 1) zero_tail(lds0, 0);
+    }
+    lds_barrier();
+#pragma unroll
+    for (int u = 0; u < READS; u++) read_unit(f0, lds0, 0, u);
+
+    uint32_t j = 0;
+    if constexpr (EDGE) {  // K-step j fetches slices j+1 and j+2: up to j = nk-4 the last slice is not among them
+      for (; j + 5 <= nk; j += 2) {
+        step(NoTail{}, lds0, lds1, j);
+        step(NoTail{}, lds1, lds0, j + 1);
+      }
+    }
+    for (; j + 1 < nk; j += 2) {
+      step(Tail{}, lds0, lds1, j);
+      step(Tail{}, lds1, lds0, j + 1);
+    }
+    if (j < nk) step(Tail{}, lds0, lds1, j);
   }
-  for (; j + 1 < nk; j += 2) {
-    step(Tail{}, lds0, lds1, j);
-    step(Tail{}, lds1, lds0, j + 1);
-  }
-  if (j < nk) step(Tail{}, lds0, lds1, j);
   wait_dma<0>();  // no LDS write of this workgroup may be in flight when it ends
 
   // Epilogue. With the operands swapped, the MFMA tile is C^T: lane l holds m = l % 32 and,
@@ -412,9 +433,10 @@ __device__ __forceinline__ void gemm_dma2_impl(const hck_gemm_args& p, char* lds
   // of row r sits at unit u ^ s(r) to spread the column-wise writes over the banks. A wave's
   // LDS instructions execute in order, so a slab may be overwritten right after its reads.
   lds_barrier();
-  char* mine = (wave < 2 ? lds0 : lds1) + (wave & 1) * ((BM + BN) * 64);
+  constexpr uint32_t MINE = ONE ? (BM + BN) * 32 : (BM + BN) * 64;  // bytes of LDS per wave for the write-out
+  char* mine = ONE ? lds0 + wave * MINE : (wave < 2 ? lds0 : lds1) + (wave & 1) * MINE;
   constexpr uint32_t ES = sizeof(T), WN = BN / 2, RB = WN * ES, UNITS = RB / 16;
-  constexpr uint32_t SLAB = 32 * RB, NSLAB = (BM + BN) * 64 / SLAB;
+  constexpr uint32_t SLAB = 32 * RB, NSLAB = MINE / SLAB;
   static_assert(NSLAB >= 1 && (32 * UNITS) % 64 == 0, "a slab must fit half a stage");
   // (the swizzle stays inside aligned groups of USWZ + 1 units, a divisor of UNITS)
   constexpr uint32_t USWZ = (UNITS & (UNITS - 1)) == 0 ? UNITS - 1 : (UNITS % 8 == 0 ? 7 : 3);
@@ -526,6 +548,23 @@ __device__ __forceinline__ void gemm_dma2_impl(const hck_gemm_args& p, char* lds
     __shared__ __attribute__((aligned(1024))) char lds1[(BM + BN) * 128];                             \
     gemm_dma2_impl<T, BM, BN, AM, BMODE, true>(p, lds0, lds1);                                        \
   }
+#define DEF_DMA_ONE(T, TN, BM, BN, AN, AM, BNAME, BMODE)                                              \
+  extern "C" __global__ __launch_bounds__(256) void HC_GEMM_NAME(hc_gemm_##TN##_dma2_##BM##x##BN##_##AN##BNAME##_1)( \
+      hck_gemm_args p) {                                                                              \
+    __shared__ __attribute__((aligned(1024))) char lds0[(BM + BN) * 128];                             \
+    gemm_dma2_impl<T, BM, BN, AM, BMODE, false, true>(p, lds0, nullptr);                              \
+  }                                                                                                   \
+  extern "C" __global__ __launch_bounds__(256) void HC_GEMM_NAME(hc_gemm_##TN##_dma2_##BM##x##BN##_##AN##BNAME##_1_e)( \
+      hck_gemm_args p) {                                                                              \
+    __shared__ __attribute__((aligned(1024))) char lds0[(BM + BN) * 128];                             \
+    gemm_dma2_impl<T, BM, BN, AM, BMODE, true, true>(p, lds0, nullptr);                               \
+  }
+// (single-slice variants: layouts with an operand that is contiguous along K, the only ones the host
+// sends here)
+#define DEF_DMA_ONE_TILE(T, TN, BM, BN)                                                               \
+  DEF_DMA_ONE(T, TN, BM, BN, k, DMA_K, k, DMA_K)                                                      \
+  DEF_DMA_ONE(T, TN, BM, BN, k, DMA_K, n, DMA_MN)                                                     \
+  DEF_DMA_ONE(T, TN, BM, BN, m, DMA_MN, k, DMA_K)
 #define DEF_DMA_TILE(T, TN, BM, BN)                                                                   \
   DEF_DMA(T, TN, BM, BN, k, DMA_K, k, DMA_K)                                                          \
   DEF_DMA(T, TN, BM, BN, k, DMA_K, n, DMA_MN)                                                         \
@@ -540,6 +579,14 @@ __device__ __forceinline__ void gemm_dma2_impl(const hck_gemm_args& p, char* lds
   DEF_DMA_TILE(T, TN, 64, 64)
 DEF_DMA_TYPE(half_t, f16)
 DEF_DMA_TYPE(float, f32)
+DEF_DMA_ONE_TILE(half_t, f16, 256, 128)
+DEF_DMA_ONE_TILE(half_t, f16, 128, 128)
+DEF_DMA_ONE_TILE(half_t, f16, 128, 64)
+DEF_DMA_ONE_TILE(half_t, f16, 64, 64)
+DEF_DMA_ONE_TILE(float, f32, 256, 128)
+DEF_DMA_ONE_TILE(float, f32, 128, 128)
+DEF_DMA_ONE_TILE(float, f32, 128, 64)
+DEF_DMA_ONE_TILE(float, f32, 64, 64)
 // (extents that are not powers of two: fp32 only, fp16 has them on the 16x16x32 pipeline)
 DEF_DMA_TILE(float, f32, 256, 192)
 DEF_DMA_TILE(float, f32, 192, 256)

@@ -149,6 +149,34 @@ def test_matmul_both_pipelines_every_tile(hip_backend, oracle_backend, monkeypat
                     assert float(np.max(np.abs(got.astype(np.float64) - want.astype(np.float64)))) <= TOL[dtype] * scale
 
 
+@pytest.mark.parametrize("dtype", [F32, F16], ids=["f32", "f16"])
+def test_matmul_single_slice_variant(hip_backend, oracle_backend, monkeypatch, dtype):
+    """Products whose whole K is one 128-byte slice (attention scores over 64-wide heads) run a
+    variant of the two-stage kernels that fetches once and uses one stage of LDS. Every tile that
+    has it, the layouts with a K-contiguous operand, whole and ragged extents, short and odd K,
+    batches: against the oracle, and bit for bit against the general loop (HCHIP_GEMM_ONE=0)."""
+    rng = np.random.default_rng(123)
+    slice_k = 64 if dtype is F16 else 32
+    bits = np.uint16 if dtype is F16 else np.uint32
+    for tile in ("256x128", "128x128", "128x64", "64x64"):
+        monkeypatch.setenv("HCHIP_GEMM_TILE", tile)
+        for K in (slice_k, slice_k - 24, slice_k // 2 + 1, 8, 1):
+            for (batch, M, N) in ((1, 256, 128), (3, 512, 512), (2, 200, 72), (1, 67, 129)):
+                a = rand(rng, (batch, M, K), dtype, 1.0 / K ** 0.5)
+                b = rand(rng, (batch, K, N), dtype)
+                for transA, transB in ((False, False), (False, True), (True, True)):
+                    sa = np.ascontiguousarray(a.transpose(0, 2, 1)) if transA else a
+                    sb = np.ascontiguousarray(b.transpose(0, 2, 1)) if transB else b
+                    print("single slice", tile, dtype.name, batch, M, K, N, transA, transB, flush=True)
+                    fn = lambda: Tensor.batchedMatmul(Tensor(data=sa), transA, Tensor(data=sb), transB, False)
+                    got, want = check_close(hip_backend, oracle_backend, fn, TOL[dtype])
+                    monkeypatch.setenv("HCHIP_GEMM_ONE", "0")
+                    with hip_backend.use():
+                        loop = fn().numpy()
+                    monkeypatch.delenv("HCHIP_GEMM_ONE")
+                    assert np.array_equal(np.ascontiguousarray(got).view(bits), np.ascontiguousarray(loop).view(bits))
+
+
 @pytest.mark.parametrize("pipeline", ["auto", "dma", "dma2", "mi16"])
 def test_matmul_random_shapes(hip_backend, oracle_backend, monkeypatch, pipeline):
     """Seeded random extents (aligned and odd), batches and flags through each pipeline: row and
