@@ -759,635 +759,7 @@ extern "C" int hc_graph_destroy(hc_ctx* ctx, hc_graph* graph) {
 }
 
 // ------------------------------------------------------------------ rewriting a recording
-
-// ---- rewrite of a recording before it is enqueued ----
-//
-// Inside a recording every buffer has an address of its own (released blocks are not handed out
-// again until the recording ends), entry points declare what they read and write, and a release
-// says that nobody reads a buffer afterwards. That is enough to see, without any knowledge of the
-// caller's program, that a result has exactly one reader, and to replace a chain of launches by
-// one launch that does the same arithmetic, intermediate by intermediate (each value rounded to
-// the tensor type where the separate kernel would have stored it), so that a replay produces the
-// bits the unmerged sequence produces. The passes, in the order fuse_recording runs them:
-//   fuse_products         matmul -> + row -> + row | + matrix | GELU   (a Linear layer's bias,
-//                         activation, residual; <= 3 operations, <= 1 matrix operand, GELU last
-//                         and not after a matrix operand; the row may be fp32 -> cast -> fp16)
-//   fuse_swapped_batches  swap of two batch axes -> batchedMatmul -> swap back: through strides
-//   fuse_layernorms       [cast] -> normalize -> [gain + c] -> mulAdd -> [cast]: one row kernel
-//   fuse_softmaxes        [* s] -> [+ mask] -> logSoftmax -> [exp]: one row kernel
-//   fuse_product_groups   products of one shape over the same input (q, k, v): one launch
-// A merged launch stands where the last entry of its chain stood. HCHIP_NO_FUSION=1 at
-// hc_capture_end turns the rewrite off.
-
-static bool aligned16(const void* p);
-static const char* dtype_name(int dtype);
-static size_t dtype_size(int dtype);
-static inline uint64_t ceil_div_u64(uint64_t a, uint64_t b) { return (a + b - 1) / b; }
-static int find_kernel_locked(hc_ctx* ctx, const std::string& name, hipFunction_t* out);
-static bool in_block(const void* p, const void* base, size_t bytes) {
-  return (const char*)p >= (const char*)base && (const char*)p < (const char*)base + bytes;
-}
-static bool touches(const std::vector<const void*>& v, const void* base, size_t bytes) {
-  for (const void* p : v)
-    if (p && in_block(p, base, bytes)) return true;
-  return false;
-}
-
-// The only entry after `from` that reads or writes the block at `base`, which is released at
-// entry `free_at`: its index, or -1 if there are several, none, or a launch in between whose
-// buffers are not declared.
-static long sole_user(const std::vector<hc_pending>& list, size_t from, const void* base, size_t bytes, size_t free_at) {
-  long user = -1;
-  for (size_t k = from + 1; k < free_at; k++) {
-    const hc_pending& e = list[k];
-    if (e.dropped || e.kind == hc_pending::FREE) continue;
-    if (!e.known) return -1;
-    if (touches(e.reads, base, bytes) || touches(e.writes, base, bytes)) {
-      if (user >= 0) return -1;
-      user = (long)k;
-    }
-  }
-  return user;
-}
-
-struct Freed { size_t at, bytes; };
-typedef std::unordered_map<const void*, Freed> FreedMap;
-
-// Whether a write declared at `w` may change what a read declared at `r` sees: the two pointers
-// are the same, or one lies inside the other's block (the sizes of blocks that are live or were
-// released inside the recording are known; an unknown pointer counts as one byte).
-struct Overlap {
-  const hc_ctx* ctx;
-  const FreedMap* freed;
-  size_t size_of(const void* p) const {
-    auto live = ctx->live.find(const_cast<void*>(p));
-    if (live != ctx->live.end()) return live->second;
-    auto fr = freed->find(p);
-    return fr == freed->end() ? 1 : fr->second.bytes;
-  }
-  bool operator()(const void* w, const void* r) const {
-    if (!w || !r) return false;
-    return w == r || in_block(w, r, size_of(r)) || in_block(r, w, size_of(w));
-  }
-};
-static thread_local const Overlap* g_overlap = nullptr;   // set for the duration of fuse_recording
-static thread_local std::vector<std::pair<void*, size_t>>* g_dead = nullptr;   // likewise
-
-// The results of a chain's entries, other than the chain's final result, are written by no launch
-// any more (every one of them was released inside the recording: that is what made it mergeable).
-static void note_dead_results(const std::vector<hc_pending>& list, const std::vector<size_t>& members, const void* final_out,
-                              const FreedMap& freed) {
-  if (!g_dead) return;
-  for (size_t m : members) {
-    const void* out = list[m].out;
-    if (!out || out == final_out) continue;
-    auto fr = freed.find(out);
-    if (fr != freed.end()) g_dead->push_back({const_cast<void*>(out), fr->second.bytes});
-  }
-}
-static bool may_alias(const void* w, const void* r) { return g_overlap ? (*g_overlap)(w, r) : w == r; }
-
-// The tagged launch before entry `before` that produced the buffer `ptr`, or -1 (also when a
-// launch with undeclared buffers lies in between: it may have written `ptr`).
-static long producer_of(const std::vector<hc_pending>& list, size_t before, const void* ptr) {
-  for (size_t k = before; k-- > 0;) {
-    const hc_pending& e = list[k];
-    if (e.dropped || e.kind == hc_pending::FREE) continue;
-    if (!e.known) return -1;
-    if (e.kind == hc_pending::KERNEL && e.out == ptr) return (long)k;
-    for (const void* w : e.writes)
-      if (may_alias(w, ptr)) return -1;
-  }
-  return -1;
-}
-
-// The one entry that uses the buffer `ptr` written by entry `from`, provided the buffer is released
-// inside the recording; -1 otherwise.
-static long only_user(const std::vector<hc_pending>& list, const FreedMap& freed, size_t from, const void* ptr) {
-  auto fr = freed.find(ptr);
-  if (fr == freed.end() || fr->second.at <= from) return -1;
-  return sole_user(list, from, ptr, fr->second.bytes, fr->second.at);
-}
-
-// A chain's work moves to the place of its last entry. What an entry of the chain reads must
-// still hold the same values there: between that entry and the last one, nothing outside the
-// chain may write it (and every launch in between must have declared its buffers).
-struct Deferred {
-  size_t at;                       // index of the chain's entry
-  std::vector<const void*> reads;  // the caller-visible buffers the merged kernel reads on its behalf
-};
-static bool inputs_stable(const std::vector<hc_pending>& list, const std::vector<Deferred>& chain) {
-  size_t last = 0;
-  for (const Deferred& d : chain) last = std::max(last, d.at);
-  for (const Deferred& d : chain)
-    for (size_t k = d.at + 1; k < last; k++) {
-      const hc_pending& e = list[k];
-      if (e.dropped || e.kind == hc_pending::FREE) continue;
-      bool member = false;
-      for (const Deferred& c : chain) member = member || c.at == k;
-      if (member) continue;
-      if (!e.known) return false;
-      for (const void* w : e.writes)
-        for (const void* in : d.reads)
-          if (in && may_alias(w, in)) return false;
-    }
-  return true;
-}
-
-// Replaces the entries of `chain` by one launch at the place of the last of them.
-static void replace_chain(std::vector<hc_pending>& list, const FreedMap& freed, const std::vector<Deferred>& chain,
-                          hipFunction_t fn, uint64_t blocks, const void* args, size_t bytes,
-                          std::initializer_list<const void*> reads, const void* out) {
-  size_t last = chain[0].at;
-  std::vector<size_t> members;
-  for (const Deferred& c : chain) {
-    last = std::max(last, c.at);
-    members.push_back(c.at);
-  }
-  note_dead_results(list, members, out, freed);
-  for (size_t m : members) list[m].dropped = true;
-  hc_pending e;
-  e.kind = hc_pending::KERNEL;
-  e.fn = fn;
-  e.grid[0] = (uint32_t)blocks;
-  e.args.assign((const char*)args, (const char*)args + bytes);
-  e.known = true;
-  for (const void* r : reads)
-    if (r) e.reads.push_back(r);
-  e.writes = {out};
-  e.out = const_cast<void*>(out);
-  list[last] = std::move(e);
-}
-
-// [cast fp16 -> fp32] -> normalize (fp32 rows) [-> mulAdd with row operands, the coefficient
-// possibly gain + c] [-> cast fp32 -> fp16]: a LayerNorm (Trainable.swift:787-829) as one kernel.
-static void fuse_layernorms(hc_ctx* ctx, std::vector<hc_pending>& list, const FreedMap& freed) {
-  for (size_t i = 0; i < list.size(); i++) {
-    if (list[i].dropped || list[i].kind != hc_pending::KERNEL || list[i].tag != hc_pending::NORMALIZE) continue;
-    const hc_pending norm = list[i];
-    const uint64_t total = norm.rows * norm.cols;
-    std::vector<Deferred> chain = {{i, {norm.in0}}};
-    hck_layernorm_args k;
-    memset(&k, 0, sizeof(k));
-    k.in = norm.in0;
-    k.outer = (uint32_t)norm.rows;
-    k.reduce = (uint32_t)norm.cols;
-    k.eps = norm.sf;
-    int in_type = HC_F32, out_type = HC_F32;
-    const void* out = norm.out;
-    size_t last = i;
-    const long up = producer_of(list, i, norm.in0);
-    if (up >= 0 && list[up].tag == hc_pending::CAST && list[up].src_dtype == HC_F16 && list[up].dtype == HC_F32 &&
-        list[up].cols == total && only_user(list, freed, (size_t)up, norm.in0) == (long)i) {
-      k.in = list[up].in0;
-      in_type = HC_F16;
-      chain[0].reads.clear();
-      chain.push_back({(size_t)up, {k.in}});
-    }
-    long next = only_user(list, freed, last, out);
-    if (next >= 0 && list[next].tag == hc_pending::MUL_ADD && list[next].dtype == HC_F32 && list[next].in0 == out &&
-        list[next].rows == norm.rows && list[next].cols == norm.cols && aligned16(list[next].in1) && aligned16(list[next].in2)) {
-      const hc_pending& m = list[next];
-      k.flags |= HCK_LN_AFFINE;
-      k.gain = m.in1;
-      k.bias = m.in2;
-      const long sc = producer_of(list, (size_t)next, m.in1);
-      if (sc >= 0 && list[sc].tag == hc_pending::SCALAR && list[sc].op == HC_ADD && list[sc].dtype == HC_F32 &&
-          list[sc].cols == norm.cols && aligned16(list[sc].in0) && only_user(list, freed, (size_t)sc, m.in1) == next) {
-        k.flags |= HCK_LN_GAIN_ADD;
-        k.gain = list[sc].in0;
-        k.gain_add = list[sc].sf;
-        chain.push_back({(size_t)sc, {k.gain}});
-      }
-      chain.push_back({(size_t)next, {k.flags & HCK_LN_GAIN_ADD ? nullptr : k.gain, k.bias}});
-      last = (size_t)next;
-      out = m.out;
-      next = only_user(list, freed, last, out);
-    }
-    if (next >= 0 && list[next].tag == hc_pending::CAST && list[next].src_dtype == HC_F32 && list[next].dtype == HC_F16 &&
-        list[next].in0 == out && list[next].cols == total) {
-      out_type = HC_F16;
-      chain.push_back({(size_t)next, {}});
-      last = (size_t)next;
-      out = list[next].out;
-    }
-    if (chain.size() == 1 || !aligned16(k.in) || !aligned16(out)) continue;
-    if (!inputs_stable(list, chain)) continue;
-    k.out = const_cast<void*>(out);
-    char name[64];
-    snprintf(name, sizeof(name), "hc_layernorm_rows_%s_%s", dtype_name(in_type), dtype_name(out_type));
-    hipFunction_t fn = nullptr;
-    if (find_kernel_locked(ctx, name, &fn) != HC_OK) continue;
-    replace_chain(list, freed, chain, fn, ceil_div_u64(norm.rows, HCK_BLOCK / 64), &k, sizeof(k), {k.in, k.gain, k.bias}, out);
-  }
-}
-
-// [x * s] [+ mask] -> logSoftmax over rows [-> exp]: an attention softmax as one kernel.
-static void fuse_softmaxes(hc_ctx* ctx, std::vector<hc_pending>& list, const FreedMap& freed) {
-  for (size_t i = 0; i < list.size(); i++) {
-    if (list[i].dropped || list[i].kind != hc_pending::KERNEL || list[i].tag != hc_pending::LOG_SOFTMAX) continue;
-    const hc_pending sm = list[i];
-    const uint64_t total = sm.rows * sm.cols;
-    std::vector<Deferred> chain = {{i, {sm.in0}}};
-    hck_softmax_chain_args k;
-    memset(&k, 0, sizeof(k));
-    k.in = sm.in0;
-    k.outer = (uint32_t)sm.rows;
-    k.reduce = (uint32_t)sm.cols;
-    k.mask_rows = 1;
-    size_t consumer = i;
-    long up = producer_of(list, consumer, k.in);
-    if (up >= 0 && list[up].tag == hc_pending::ADD && list[up].dtype == sm.dtype && list[up].rows * list[up].cols == total &&
-        only_user(list, freed, (size_t)up, k.in) == (long)consumer) {
-      const hc_pending& a = list[up];
-      // which operand is the one of `total` elements the rows come from, and how often the other repeats
-      const void* stream = a.add_form == 2 ? a.in1 : a.in0;
-      const void* mask = a.add_form == 2 ? a.in0 : a.in1;
-      const uint64_t mask_elems = a.add_form == 3 ? total : a.cols;
-      if (mask_elems % sm.cols == 0 && aligned16(mask) && aligned16(stream) && stream != mask) {
-        k.flags |= HCK_SM_MASK;
-        k.mask = mask;
-        k.mask_rows = (uint32_t)(mask_elems / sm.cols);
-        k.in = stream;
-        chain[0].reads.clear();
-        chain.push_back({(size_t)up, {stream, mask}});
-        consumer = (size_t)up;
-      }
-    }
-    up = producer_of(list, consumer, k.in);
-    if (up >= 0 && list[up].tag == hc_pending::SCALAR && list[up].op == HC_MUL && list[up].dtype == sm.dtype &&
-        list[up].cols == total && aligned16(list[up].in0) && only_user(list, freed, (size_t)up, k.in) == (long)consumer) {
-      k.flags |= HCK_SM_SCALE;
-      k.scale = list[up].sf;
-      for (Deferred& d : chain)   // whoever read the scaled tensor reads nothing of it any more
-        for (const void*& r : d.reads)
-          if (r == k.in) r = nullptr;
-      k.in = list[up].in0;
-      chain.push_back({(size_t)up, {k.in}});
-    }
-    const void* out = sm.out;
-    const long next = only_user(list, freed, i, out);
-    if (next >= 0 && list[next].tag == hc_pending::EXP && list[next].dtype == sm.dtype && list[next].in0 == out &&
-        list[next].cols == total && aligned16(list[next].out)) {
-      k.flags |= HCK_SM_EXP;
-      chain.push_back({(size_t)next, {}});
-      out = list[next].out;
-    }
-    if (chain.size() == 1) continue;
-    if (!inputs_stable(list, chain)) continue;
-    k.out = const_cast<void*>(out);
-    char name[64];
-    snprintf(name, sizeof(name), "hc_softmax_chain_rows%s_%s", sm.lanes == 8 ? "8" : "", dtype_name(sm.dtype));
-    hipFunction_t fn = nullptr;
-    if (find_kernel_locked(ctx, name, &fn) != HC_OK) continue;
-    replace_chain(list, freed, chain, fn, ceil_div_u64(sm.rows, HCK_BLOCK / (uint64_t)sm.lanes), &k, sizeof(k), {k.in, k.mask}, out);
-  }
-}
-
-// The kernel of the same name from the second build of the tiled GEMM sources (*_m): the one that
-// knows merged operations, two-level batches and groups. False if there is none.
-static bool use_merged_kernel(hc_ctx* ctx, hc_pending& e) {
-  if (e.name.size() >= 2 && e.name.compare(e.name.size() - 2, 2, "_m") == 0) return true;
-  hipFunction_t fn = nullptr;
-  if (find_kernel_locked(ctx, e.name + "_m", &fn) != HC_OK) return false;
-  e.fn = fn;
-  e.name += "_m";
-  return true;
-}
-
-// A batched product whose operand is a tensor with two axes swapped ([B, T, H, d] read as
-// [B, H, T, d]: the heads of an attention layer), or whose result is swapped back, reads and
-// writes through the strides instead: the copies disappear.
-static void fuse_swapped_batches(hc_ctx* ctx, std::vector<hc_pending>& list, const FreedMap& freed) {
-  for (size_t i = 0; i < list.size(); i++) {
-    if (list[i].dropped || list[i].kind != hc_pending::KERNEL || list[i].tag != hc_pending::BMM) continue;
-    if (list[i].args.size() != sizeof(hck_gemm_args)) continue;
-    hck_gemm_args g;
-    memcpy(&g, list[i].args.data(), sizeof(g));
-    if (g.bdiv != 0) continue;
-    const uint64_t P = 16 / dtype_size(list[i].dtype), el = dtype_size(list[i].dtype);
-    std::vector<Deferred> chain = {{i, {g.a, g.b}}};
-    uint32_t bdiv = 0;            // 0: not decided yet
-    bool two_level = false;
-    // slice strides as they will be: {hi, lo}; an operand that stays as it is keeps hi = bdiv * bs, lo = bs
-    uint64_t a_hi = 0, a_lo = g.a_bs, b_hi = 0, b_lo = g.b_bs, c_hi = 0, c_lo = g.c_bs;
-    bool a_set = false, b_set = false, c_set = false;
-    auto read_through = [&](const void*& ptr, uint32_t& rs, uint32_t& cs, uint32_t rows, uint32_t cols, uint64_t bs,
-                            uint64_t& hi, uint64_t& lo, bool& set) {
-      // the operand's slices: [R, I] row-major with row stride I; (rs, cs) = strides of (rows, cols)
-      const bool row_major = cs == 1;
-      const uint64_t R = row_major ? rows : cols, I = row_major ? cols : rows;
-      if ((row_major ? rs : cs) != I || (row_major ? cs : rs) != 1 || bs != R * I) return;
-      const long up = producer_of(list, i, ptr);
-      if (up < 0 || list[up].tag != hc_pending::PERMUTE || list[up].dtype != list[i].dtype) return;
-      const hc_pending& pm = list[up];
-      if (only_user(list, freed, (size_t)up, ptr) != (long)i) return;
-      const int n = pm.pn;
-      if (n != 3 && n != 4) return;
-      if (pm.pext[n - 1] != I || pm.pstr[n - 1] != 1 || pm.pext[n - 2] != R) return;
-      uint64_t z_hi, s_hi, z_lo = 1, s_lo = 0;
-      if (n == 4) {
-        z_hi = pm.pext[0], s_hi = pm.pstr[0], z_lo = pm.pext[1], s_lo = pm.pstr[1];
-        if ((bdiv != 0 && bdiv != z_lo) || ((a_set || b_set) && !two_level)) return;
-      } else {
-        z_hi = pm.pext[0], s_hi = pm.pstr[0];
-        if (two_level) return;   // (a single-level operand next to a two-level one: expressible, not needed)
-      }
-      if (z_hi * z_lo != g.batch) return;
-      const uint64_t row_stride = pm.pstr[n - 2];
-      if (row_stride % P || s_hi % P || s_lo % P || !aligned16(pm.in0) || row_stride > 0xffffffffull ||
-          R * row_stride * el > 0xffffffffull)
-        return;
-      if (n == 4) {
-        bdiv = (uint32_t)z_lo;
-        two_level = true;
-        hi = s_hi, lo = s_lo;
-      } else {
-        hi = 0, lo = s_hi;   // single level: z * lo
-      }
-      set = true;
-      for (const void*& r : chain[0].reads)   // the product no longer reads the copy
-        if (r == ptr) r = nullptr;
-      ptr = pm.in0;
-      (row_major ? rs : cs) = (uint32_t)row_stride;
-      chain.push_back({(size_t)up, {pm.in0}});
-    };
-    read_through(g.a, g.a_rs, g.a_cs, g.M, g.K, g.a_bs, a_hi, a_lo, a_set);
-    read_through(g.b, g.b_rs, g.b_cs, g.K, g.N, g.b_bs, b_hi, b_lo, b_set);
-    // the result, swapped by its only reader
-    const void* out = list[i].out;
-    {
-      const long next = only_user(list, freed, i, out);
-      if (next >= 0 && list[next].tag == hc_pending::PERMUTE && list[next].dtype == list[i].dtype && list[next].in0 == out &&
-          g.c_rs == g.N && g.c_cs == 1 && g.c_bs == (uint64_t)g.M * g.N && aligned16(list[next].out)) {
-        const hc_pending& pm = list[next];
-        const int n = pm.pn;
-        // strides of the permute's dense output, and the role of each axis by its source stride
-        uint64_t ostr[HC_MAX_DIMS + 1];
-        uint64_t acc = 1;
-        for (int d = n - 1; d >= 0; d--) {
-          ostr[d] = acc;
-          acc *= pm.pext[d];
-        }
-        long m_ax = -1, lo_ax = -1, hi_ax = -1;
-        for (int d = 0; d < n - 1; d++) {
-          if (pm.pstr[d] == g.N && pm.pext[d] == g.M) m_ax = d;
-          else if (pm.pstr[d] == (uint64_t)g.M * g.N) lo_ax = d;
-          else hi_ax = d;
-        }
-        bool ok = (n == 3 || n == 4) && pm.pext[n - 1] == g.N && pm.pstr[n - 1] == 1 && m_ax >= 0 && lo_ax >= 0;
-        if (ok && n == 4)
-          ok = !((a_set || b_set) && !two_level) && hi_ax >= 0 && pm.pstr[hi_ax] == pm.pext[lo_ax] * (uint64_t)g.M * g.N &&
-               pm.pext[hi_ax] * pm.pext[lo_ax] == g.batch && (bdiv == 0 || bdiv == pm.pext[lo_ax]);
-        if (ok && n == 3) ok = pm.pext[lo_ax] == g.batch && !two_level;
-        if (ok) ok = ostr[m_ax] % P == 0 && ostr[lo_ax] % P == 0 && (n == 3 || ostr[hi_ax] % P == 0) && ostr[m_ax] <= 0xffffffffull;
-        if (ok) {
-          if (n == 4) {
-            bdiv = (uint32_t)pm.pext[lo_ax];
-            two_level = true;
-            c_hi = ostr[hi_ax], c_lo = ostr[lo_ax];
-          } else {
-            c_hi = 0, c_lo = ostr[lo_ax];
-          }
-          c_set = true;
-          g.c_rs = (uint32_t)ostr[m_ax];
-          g.c = pm.out;
-          out = pm.out;
-          chain.push_back({(size_t)next, {}});
-        }
-      }
-    }
-    if (chain.size() == 1) continue;
-    if (two_level) {
-      // operands that stay as they are: slice z = hi * bdiv + lo of a dense batch
-      if (!a_set) a_hi = (uint64_t)bdiv * g.a_bs, a_lo = g.a_bs;
-      if (!b_set) b_hi = (uint64_t)bdiv * g.b_bs, b_lo = g.b_bs;
-      if (!c_set) c_hi = (uint64_t)bdiv * g.c_bs, c_lo = g.c_bs;
-      g.bdiv = bdiv;
-      g.a_bs = a_hi, g.a_bs2 = a_lo;
-      g.b_bs = b_hi, g.b_bs2 = b_lo;
-      g.c_bs = c_hi, g.c_bs2 = c_lo;
-    } else {
-      g.a_bs = a_lo, g.b_bs = b_lo, g.c_bs = c_lo;
-    }
-    if (!inputs_stable(list, chain)) continue;
-    size_t last = i;
-    for (const Deferred& c : chain) last = std::max(last, c.at);
-    hc_pending fused = list[i];
-    if (!use_merged_kernel(ctx, fused)) continue;
-    memcpy(fused.args.data(), &g, sizeof(g));
-    fused.tag = hc_pending::NONE;
-    fused.reads = {g.a, g.b};
-    fused.writes = {out};
-    fused.out = const_cast<void*>(out);
-    {
-      std::vector<size_t> members;
-      for (const Deferred& c : chain) members.push_back(c.at);
-      note_dead_results(list, members, out, freed);
-    }
-    for (const Deferred& c : chain) list[c.at].dropped = true;
-    list[last] = std::move(fused);
-  }
-}
-
-// Products over the same A with the same shape, strides and merged operations (the q, k, v
-// projections of an attention layer) become one launch: a workgroup's blockIdx.y picks the
-// member's B, C and epilogue operands.
-static void fuse_product_groups(hc_ctx* ctx, std::vector<hc_pending>& list, const FreedMap& freed) {
-  auto is_product = [](const hc_pending& e) {
-    return !e.dropped && e.kind == hc_pending::KERNEL && (e.tag == hc_pending::GEMM || e.tag == hc_pending::PRODUCT) &&
-           e.args.size() == sizeof(hck_gemm_args);
-  };
-  auto uses = [&](const hc_pending& e, const void* buf) {   // e reads or writes the buffer at `buf`
-    auto fr = freed.find(buf);
-    const size_t bytes = fr == freed.end() ? 1 : fr->second.bytes;
-    return touches(e.reads, buf, bytes) || touches(e.writes, buf, bytes);
-  };
-  for (size_t i = 0; i < list.size(); i++) {
-    if (!is_product(list[i])) continue;
-    hck_gemm_args g;
-    memcpy(&g, list[i].args.data(), sizeof(g));
-    if (g.batch != 1 || g.bdiv != 0 || g.group != 0 || list[i].grid[1] != 1) continue;
-    std::vector<size_t> members = {i};
-    std::vector<hck_gemm_args> margs = {g};
-    for (size_t j = i + 1; j < list.size() && members.size() < HCK_GEMM_GROUP; j++) {
-      const hc_pending& e = list[j];
-      if (e.dropped || e.kind == hc_pending::FREE) continue;
-      if (!e.known) break;
-      bool joins = false;
-      hck_gemm_args h;
-      if (is_product(e) && e.fn == list[i].fn && e.dtype == list[i].dtype && e.grid[0] == list[i].grid[0] && e.grid[1] == 1) {
-        memcpy(&h, e.args.data(), sizeof(h));
-        joins = h.a == g.a && h.M == g.M && h.N == g.N && h.K == g.K && h.batch == 1 && h.bdiv == 0 && h.group == 0 &&
-                h.a_rs == g.a_rs && h.a_cs == g.a_cs && h.b_rs == g.b_rs && h.b_cs == g.b_cs && h.c_rs == g.c_rs &&
-                h.c_cs == g.c_cs && h.tiles_m == g.tiles_m && h.tiles_n == g.tiles_n && h.xcd_gn == g.xcd_gn &&
-                h.xcd_sm == g.xcd_sm && h.xcd_sn == g.xcd_sn && h.a_lim == g.a_lim && h.b_lim == g.b_lim &&
-                memcmp(h.ep_kind, g.ep_kind, sizeof(g.ep_kind)) == 0 && memcmp(h.ep_ld, g.ep_ld, sizeof(g.ep_ld)) == 0;
-      }
-      // The earlier members run where the last one stands: nothing in between (a later member
-      // included) may use their results or write what they read.
-      bool conflict = false;
-      for (size_t m = 0; m < members.size() && !conflict; m++) {
-        const hck_gemm_args& a = margs[m];
-        conflict = uses(e, a.c);
-        for (const void* w : e.writes)
-          conflict = conflict || may_alias(w, a.a) || may_alias(w, a.b) || may_alias(w, a.ep_ptr[0]) ||
-                     may_alias(w, a.ep_ptr[1]) || may_alias(w, a.ep_ptr[2]);
-      }
-      if (conflict) break;
-      if (joins) {
-        members.push_back(j);
-        margs.push_back(h);
-      }
-    }
-    if (members.size() < 2) continue;
-    const uint32_t n = (uint32_t)members.size();
-    hc_pending grouped = list[i];
-    if (!use_merged_kernel(ctx, grouped)) continue;
-    grouped.tag = hc_pending::NONE;
-    grouped.out = nullptr;
-    grouped.grid[1] = n;
-    grouped.reads.clear();
-    grouped.writes.clear();
-    g.group = n;
-    for (uint32_t m = 0; m < n; m++) {
-      g.g_b[m] = margs[m].b;
-      g.g_c[m] = margs[m].c;
-      for (int s = 0; s < 3; s++) g.g_ep[s][m] = margs[m].ep_ptr[s];
-      for (const void* r : list[members[m]].reads) grouped.reads.push_back(r);
-      grouped.writes.push_back(margs[m].c);
-      list[members[m]].dropped = true;
-    }
-    memcpy(grouped.args.data(), &g, sizeof(g));
-    list[members.back()] = std::move(grouped);
-  }
-}
-
-static void fuse_products(hc_ctx* ctx, std::vector<hc_pending>& list, const FreedMap& freed);
-
-static void fuse_recording(hc_ctx* ctx) {
-  std::vector<hc_pending>& list = ctx->pending;
-  FreedMap freed;
-  for (size_t i = 0; i < list.size(); i++)
-    if (list[i].kind == hc_pending::FREE) freed[list[i].dst] = Freed{i, list[i].bytes};
-  const Overlap overlap{ctx, &freed};
-  g_overlap = &overlap;
-  ctx->dead.clear();
-  g_dead = &ctx->dead;
-  fuse_products(ctx, list, freed);
-  fuse_swapped_batches(ctx, list, freed);
-  fuse_layernorms(ctx, list, freed);
-  fuse_softmaxes(ctx, list, freed);
-  fuse_product_groups(ctx, list, freed);
-  g_overlap = nullptr;
-  g_dead = nullptr;
-}
-
-static void fuse_products(hc_ctx* ctx, std::vector<hc_pending>& list, const FreedMap& freed) {
-
-  for (size_t i = 0; i < list.size(); i++) {
-    if (list[i].kind != hc_pending::KERNEL || list[i].dropped || list[i].tag != hc_pending::GEMM) continue;
-    if (list[i].args.size() != sizeof(hck_gemm_args)) continue;
-    hck_gemm_args g;
-    memcpy(&g, list[i].args.data(), sizeof(g));
-    const int dtype = list[i].dtype;
-    const uint64_t M = list[i].rows, N = list[i].cols;
-    std::vector<const void*> inputs = {g.a, g.b};   // what the merged kernel reads
-    std::vector<size_t> merged;                      // entries whose work it takes over
-    const void* cur = list[i].out;
-    size_t pos = i;
-    int nops = 0;
-    while (nops < 3) {
-      auto fr = freed.find(cur);
-      if (fr == freed.end() || fr->second.at <= pos) break;
-      const long j = sole_user(list, pos, cur, fr->second.bytes, fr->second.at);
-      if (j < 0) break;
-      const hc_pending& c = list[(size_t)j];
-      if (c.kind != hc_pending::KERNEL || c.dtype != dtype || !c.out || !aligned16(c.out)) break;
-      uint32_t kind = HCK_EP_NONE;
-      const void* other = nullptr;
-      bool has_matrix = false;
-      for (int s = 0; s < nops; s++) has_matrix = has_matrix || g.ep_kind[s] == HCK_EP_ADD_MATRIX;
-      if (c.tag == hc_pending::GELU && c.in0 == cur && c.cols == M * N && !has_matrix) {
-        kind = HCK_EP_GELU;
-      } else if (c.tag == hc_pending::ADD && (c.in0 == cur) != (c.in1 == cur)) {
-        const bool first = c.in0 == cur;
-        other = first ? c.in1 : c.in0;
-        if (c.add_form == 3 && c.rows * c.cols == M * N) kind = HCK_EP_ADD_MATRIX;
-        if (c.add_form == (first ? 1 : 2) && c.rows == M && c.cols == N) kind = HCK_EP_ADD_ROW;
-        if (!aligned16(other)) kind = HCK_EP_NONE;
-        // (the kernels fetch one matrix operand per output piece)
-        if (kind == HCK_EP_ADD_MATRIX)
-          for (int s = 0; s < nops; s++)
-            if (g.ep_kind[s] == HCK_EP_ADD_MATRIX) kind = HCK_EP_NONE;
-      }
-      if (kind == HCK_EP_NONE) break;
-      // the product moves to its reader's place: nothing in between may write what it reads
-      bool clean = true;
-      for (size_t k2 = pos + 1; k2 < (size_t)j && clean; k2++) {
-        const hc_pending& e = list[k2];
-        if (e.dropped || e.kind == hc_pending::FREE) continue;
-        for (const void* in : inputs)
-          for (const void* w : e.writes)
-            if (may_alias(w, in)) clean = false;
-      }
-      if (!clean) break;
-      g.ep_kind[nops] = kind;
-      g.ep_ptr[nops] = other;
-      const bool ends_list = kind == HCK_EP_GELU;   // (the kernels apply GELU after the additions)
-      g.ep_ld[nops] = (uint32_t)N;
-      if (other) inputs.push_back(other);
-      merged.push_back((size_t)j);
-      cur = c.out;
-      pos = (size_t)j;
-      nops++;
-      if (ends_list) break;
-    }
-    if (nops == 0) continue;
-    // the kernel of the same name that knows how to apply the operations
-    hc_pending fused = list[i];
-    if (!use_merged_kernel(ctx, fused)) continue;
-    // a bias row that is an fp32 parameter cast to fp16 just for this addition: read the fp32 row
-    if (dtype == HC_F16)
-      for (int s = 0; s < nops; s++) {
-        if (g.ep_kind[s] != HCK_EP_ADD_ROW) continue;
-        auto fr = freed.find(g.ep_ptr[s]);
-        if (fr == freed.end()) continue;
-        for (size_t c2 = 0; c2 < merged[(size_t)s]; c2++) {
-          hc_pending& e = list[c2];
-          if (e.dropped || e.kind != hc_pending::KERNEL || e.tag != hc_pending::CAST || e.out != g.ep_ptr[s]) continue;
-          if (e.src_dtype != HC_F32 || e.dtype != HC_F16 || e.cols != N || !aligned16(e.in0)) break;
-          if (sole_user(list, c2, e.out, fr->second.bytes, fr->second.at) != (long)merged[(size_t)s]) break;
-          bool clean = true;   // the fp32 row must still hold the same values where the product now runs
-          for (size_t k2 = c2 + 1; k2 < pos && clean; k2++)
-            for (const void* w : list[k2].writes)
-              if (!list[k2].dropped && may_alias(w, e.in0)) clean = false;
-          if (!clean) break;
-          for (const void*& in : inputs)
-            if (in == g.ep_ptr[s]) in = e.in0;
-          g.ep_kind[s] = HCK_EP_ADD_ROW_F32;
-          g.ep_ptr[s] = e.in0;
-          note_dead_results(list, {c2}, nullptr, freed);
-          e.dropped = true;
-          break;
-        }
-      }
-    g.c = const_cast<void*>(cur);
-    memcpy(fused.args.data(), &g, sizeof(g));
-    fused.tag = hc_pending::PRODUCT;   // (no further operations are merged; it may still join a group)
-    fused.reads = inputs;
-    fused.writes = {cur};
-    fused.out = const_cast<void*>(cur);
-    {
-      std::vector<size_t> members = merged;
-      members.push_back(i);
-      note_dead_results(list, members, cur, freed);
-    }
-    for (size_t m : merged) list[m].dropped = true;
-    list[i].dropped = true;
-    list[pos] = std::move(fused);   // (not dropped: copied from the product's entry before that was marked)
-  }
-}
+#include "hchip_rewrite.inc"
 
 // ------------------------------------------------------------------ raw module API
 
@@ -3114,550 +2486,4 @@ extern "C" int hc_concat(hc_ctx* ctx, int dtype, const void* const* inputs, cons
 }
 
 // ------------------------------------------------------------------ matmul
-
-// True if `slack` bytes after the `bytes` at `ptr` can be read: both lie inside one block that this
-// context handed out. (The tiled GEMM kernels fetch whole 16-byte pieces; with rows that are not a
-// whole number of pieces, the last piece of the last row ends up to 14 bytes after the operand.)
-static bool readable_past(hc_ctx* ctx, const void* ptr, uint64_t bytes, uint64_t slack) {
-  std::lock_guard<std::mutex> lock(ctx->mu);
-  const uintptr_t lo = (uintptr_t)ptr, hi = lo + bytes + slack;
-  auto it = ctx->live.find(const_cast<void*>(ptr));
-  if (it != ctx->live.end()) return bytes + slack <= it->second;
-  for (auto& blk : ctx->live) {  // a view into a block
-    const uintptr_t start = (uintptr_t)blk.first;
-    if (lo >= start && lo < start + blk.second) return hi <= start + blk.second;
-  }
-  return false;
-}
-
-
-extern "C" int hc_matmul(hc_ctx* ctx, int dtype, int64_t batch, const void* a, int trans_a,
-                         const void* b, int trans_b, int trans_out, int64_t rows, int64_t inner,
-                         int64_t cols, void* out) {
-  REQUIRE(ctx, "hc_matmul: null context");
-  if (dtype != HC_F32 && dtype != HC_F16 && dtype != HC_I64)
-    return fail(HC_ERR_UNSUPPORTED, "hc_matmul: dtype %d is not numeric", dtype);
-  REQUIRE(batch >= 0 && rows >= 0 && inner >= 0 && cols >= 0, "hc_matmul: negative dimension");
-  if (batch * rows * cols == 0) return HC_OK;
-  REQUIRE(out && (inner == 0 || (a && b)), "hc_matmul: null pointer");
-  if (rows > 0x7fffffffll || cols > 0x7fffffffll || inner > 0x7fffffffll ||
-      (double)rows * (double)inner > 4294967295.0 || (double)inner * (double)cols > 4294967295.0 ||
-      (double)rows * (double)cols > 4294967295.0)
-    return fail(HC_ERR_TOO_LARGE, "hc_matmul: a matrix has more than 2^32-1 elements");
-  const size_t el = dtype_size(dtype);
-  const uint32_t P = (uint32_t)(16 / el);
-  OpNote note({a, b}, {out});
-  bool whole_call = false;  // the launch in progress computes the whole product (nothing peeled off)
-  hck_gemm_args k;
-  memset(&k, 0, sizeof(k));
-  uint32_t M = (uint32_t)rows, N = (uint32_t)cols, K = (uint32_t)inner;
-  uint32_t a_rs = trans_a ? 1 : K, a_cs = trans_a ? M : 1;
-  uint32_t b_rs = trans_b ? 1 : N, b_cs = trans_b ? K : 1;
-  k.a = a;
-  k.b = b;
-  k.a_bs = (uint64_t)M * K;
-  k.b_bs = (uint64_t)K * N;
-  k.c_bs = (uint64_t)M * N;
-  if (trans_out) {
-    // C^T = B^T * A^T: swap the operands so that the stored output is row-major again.
-    k.a = b;
-    k.b = a;
-    const uint32_t na_rs = b_cs, na_cs = b_rs, nb_rs = a_cs, nb_cs = a_rs;
-    a_rs = na_rs;
-    a_cs = na_cs;
-    b_rs = nb_rs;
-    b_cs = nb_cs;
-    std::swap(k.a_bs, k.b_bs);
-    std::swap(M, N);
-  }
-  k.c = out;
-  k.M = M;
-  k.N = N;
-  k.K = K;
-  k.a_rs = a_rs;
-  k.a_cs = a_cs;
-  k.b_rs = b_rs;
-  k.b_cs = b_cs;
-  k.c_rs = N;
-  k.c_cs = 1;
-  k.tiles_m = (uint32_t)ceil_div(M, 128);
-  k.tiles_n = (uint32_t)ceil_div(N, 128);
-
-  if (dtype == HC_I64) {
-    // no matrix instruction for 64-bit integers: one small vector-ALU kernel, any strides
-    k.tiles_m = (uint32_t)ceil_div(M, 16);
-    k.tiles_n = (uint32_t)ceil_div(N, 16);
-    const uint64_t tiles = (uint64_t)k.tiles_m * k.tiles_n;
-    for (int64_t b0 = 0; b0 < batch; b0 += 65535) {
-      const uint32_t nb = (uint32_t)(batch - b0 < 65535 ? batch - b0 : 65535);
-      hck_gemm_args kk = k;
-      kk.a = (const char*)k.a + (uint64_t)b0 * k.a_bs * el;
-      kk.b = (const char*)k.b + (uint64_t)b0 * k.b_bs * el;
-      kk.c = (char*)k.c + (uint64_t)b0 * k.c_bs * el;
-      kk.batch = nb;
-      HC_TRY(launch(ctx, "hc_gemm_i64", tiles, nb, &kk, sizeof(kk)));
-    }
-    return HC_OK;
-  }
-
-  // Per-operand global->LDS path: 'k' contiguous along K, 'm'/'n' contiguous along M/N
-  // (both need 16-byte aligned rows), 'x' anything else.
-  auto mode = [&](const void* ptr, uint32_t row_stride, uint32_t k_stride, uint64_t batch_stride) -> char {
-    const bool base_ok = aligned16(ptr) && (batch <= 1 || batch_stride % P == 0);
-    if (base_ok && k_stride == 1 && row_stride % P == 0) return 'k';
-    if (base_ok && row_stride == 1 && k_stride % P == 0) return 'r';
-    return 'x';
-  };
-  char ma = mode(k.a, a_rs, a_cs, k.a_bs);
-  char mb = mode(k.b, b_cs, b_rs, k.b_bs);
-  char name[64];
-  const bool c_unaligned = !aligned16(out) || N % P != 0;
-
-  // A last row or column of tiles that is almost empty costs as much as a full one: 4097 rows
-  // are 17 rows of 256-row tiles, i.e. two rounds on a device that 16 x 16 tiles fill exactly.
-  // Products that are a few rows or columns over a multiple of 256 are therefore split into the
-  // multiple-of-256 body and thin fringes, each run as a product of its own on sub-blocks of the
-  // same buffers (same strides, offset pointers).
-  // (only long products: the fringes are skinny products of their own that take tens of
-  // microseconds, which a short body does not win back)
-  auto fringe = [&](uint32_t d) { return d >= 2048 && d % 256 != 0 && d % 256 <= 32 ? d % 256 : 0u; };
-  // (an output of 4 M elements, or half of that over a K long enough for 2^33 multiply-adds)
-  const bool large = (uint64_t)M * N >= (1ull << 22) ||
-                     ((uint64_t)M * N >= (1ull << 21) && (uint64_t)M * N * K >= (1ull << 33));
-  const bool peelable = K >= 2048 && large && (fringe(M) != 0 || fringe(N) != 0) && !getenv("HCHIP_GEMM_TILE") &&
-                        !getenv("HCHIP_GEMM_NO_PEEL");
-
-  // Operands and outputs whose rows are not 16-byte aligned (odd extents, odd base addresses): the
-  // edge variants of the direct-to-LDS kernels take them as they are. Their loads and stores need
-  // no alignment; what a 16-byte piece holds beyond K is cleared in LDS, beyond N it feeds columns
-  // that are never stored, and the piece of C that straddles N leaves element by element. Needed
-  // for that: the up to 14 bytes after an operand that the last piece of its last row covers are
-  // readable (the operand lies inside a block of this context with that much room).
-  // HCHIP_GEMM_NO_DIRECT=1 switches this off (measurements, tests).
-  bool loose = false;
-  if ((ma == 'x' || mb == 'x' || c_unaligned) && K > 0 && batch <= 65535 && !getenv("HCHIP_GEMM_NO_DIRECT")) {
-    auto loose_mode = [&](char m, uint32_t row_stride, uint32_t k_stride) -> char {
-      return m != 'x' ? m : k_stride == 1 ? 'k' : row_stride == 1 ? 'r' : 'x';
-    };
-    const char la = loose_mode(ma, a_rs, a_cs), lb = loose_mode(mb, b_cs, b_rs);
-    const uint64_t a_bytes = ((uint64_t)(batch - 1) * k.a_bs + (uint64_t)M * K) * el;
-    const uint64_t b_bytes = ((uint64_t)(batch - 1) * k.b_bs + (uint64_t)K * N) * el;
-    if (la != 'x' && lb != 'x' && (ma != 'x' || readable_past(ctx, k.a, a_bytes, 16)) &&
-        (mb != 'x' || readable_past(ctx, k.b, b_bytes, 16))) {
-      ma = la;
-      mb = lb;
-      loose = true;
-    }
-  }
-
-  // Operands whose rows are not 16-byte aligned (odd extents, odd base addresses) would fall
-  // to scalar loads; for anything but tiny products it pays to re-pitch them first: a copy
-  // with the leading dimension rounded up to 16 bytes, zero-filled, and likewise a padded
-  // output that is copied back at the end. The tuned kernels then run on the copies.
-  Scratch scratch(ctx);
-  void* c_padded = nullptr;
-  uint32_t c_ld = N;
-  const double work = (double)M * (double)N * (double)K * (double)batch;
-  // (the scalar loads of the general kernel cost about 4 us per 64 of K and tile: a long K pays
-  // for the copies much earlier than a large output does)
-  if (!loose && (ma == 'x' || mb == 'x' || c_unaligned) && K > 0 && (work >= 16777216.0 || (work >= 2097152.0 && K >= 256)) &&
-      batch <= 65535 &&
-      !getenv("HCHIP_GEMM_NO_REPITCH")) {
-    auto round_up = [&](uint32_t v) { return (v + P - 1) / P * P; };
-    // (rows, k) element at rows*rs + k*cs with one of the strides 1 (dense storage)
-    auto repitch = [&](const void*& ptr, uint32_t& rs, uint32_t& cs, uint64_t& bs, uint32_t extent) -> int {
-      const bool k_contig = cs == 1;
-      const uint32_t nrows = k_contig ? extent : K, ncols = k_contig ? K : extent;
-      const uint32_t ld = round_up(ncols);
-      void* copy = nullptr;
-      HC_TRY(scratch.get((size_t)batch * nrows * ld * el, &copy));
-      hck_copy2d_args c;
-      memset(&c, 0, sizeof(c));
-      c.in = ptr;
-      c.out = copy;
-      c.rows = nrows;
-      c.in_cols = ncols;
-      c.out_cols = ld;
-      c.in_ld = k_contig ? rs : cs;
-      c.out_ld = ld;
-      c.in_bs = bs;
-      c.out_bs = (uint64_t)nrows * ld;
-      const uint64_t waves = (uint64_t)nrows * ceil_div(ld, 512);  // a wave moves 64 * 8 elements
-      HC_TRY(launch(ctx, el == 2 ? "hc_copy2d_pad_b2" : "hc_copy2d_pad_b4", ceil_div(waves, HCK_BLOCK / 64),
-                    (uint32_t)batch, &c, sizeof(c)));
-      ptr = copy;
-      (k_contig ? rs : cs) = ld;
-      bs = c.out_bs;
-      return HC_OK;
-    };
-    if (ma == 'x') {
-      HC_TRY(repitch(k.a, a_rs, a_cs, k.a_bs, M));
-      ma = mode(k.a, a_rs, a_cs, k.a_bs);
-    }
-    if (mb == 'x') {
-      HC_TRY(repitch(k.b, b_cs, b_rs, k.b_bs, N));
-      mb = mode(k.b, b_cs, b_rs, k.b_bs);
-    }
-    if (c_unaligned) {
-      c_ld = round_up(N);
-      HC_TRY(scratch.get((size_t)batch * M * c_ld * el, &c_padded));
-      k.c = c_padded;
-      k.c_rs = c_ld;
-      k.c_bs = (uint64_t)M * c_ld;
-    }
-    k.a_rs = a_rs;
-    k.a_cs = a_cs;
-    k.b_rs = b_rs;
-    k.b_cs = b_cs;
-  }
-  // Kernel choice and launch for the block of C that `k` describes (pointers and strides set;
-  // M x N its extent): the whole product, or a part of it when a thin fringe is peeled off below.
-  auto run = [&](hck_gemm_args k, uint32_t M, uint32_t N) -> int {
-    k.M = M;
-    k.N = N;
-    k.tiles_m = (uint32_t)ceil_div(M, 128);  // (general kernel; the tuned kernels set their own below)
-    k.tiles_n = (uint32_t)ceil_div(N, 128);
-    // what an edge kernel may fetch: all rows of a K-contiguous operand, whole 16-byte pieces of
-    // an M/N-contiguous one (its leading dimension covers them)
-    k.a_lim = ma == 'k' ? M : (M + P - 1) / P * P;
-    k.b_lim = mb == 'k' ? N : (N + P - 1) / P * P;
-
-    // Tuned kernels. Direct-to-LDS (fp16, fp32): rows of A, B and C 16-byte aligned, operands
-    // addressed with 32-bit byte offsets; ragged M, N, K run the "_e" variants (clamped rows,
-    // zero-filled K tail, predicated stores). For measurements and tests, read at every call:
-    // HCHIP_GEMM_TILE=general|<BM>x<BN> overrides the tile choice, HCHIP_GEMM_KERNEL=
-    // dma|dma2|mi16 the pipeline, =staged selects the register-staged fp16 pipeline (whole
-    // tiles, K % 64 == 0).
-    uint32_t bm = 0, bn = 0;
-    bool edge = false, one = false;
-    const char* which = getenv("HCHIP_GEMM_KERNEL");
-    // Skinny products (one extent of C at most 4, the other long: matrix-vector products and
-    // the thinnest fringes peeled off below) are bound by reading the long operand once: no
-    // tiles. (Wider ones are faster on the tile kernels.)
-    if (!which && !getenv("HCHIP_GEMM_TILE") && K >= 64 && std::min(M, N) <= 4 && std::max(M, N) >= 512 &&
-        batch <= 65535) {
-      const bool thin_n = N <= M;
-      hck_skinny_args sk;
-      memset(&sk, 0, sizeof(sk));
-      sk.K = K;
-      sk.c = k.c;
-      sk.c_bs = k.c_bs;
-      if (thin_n) {  // X = A (p = m), Y = B
-        sk.x = k.a, sk.x_ps = k.a_rs, sk.x_ks = k.a_cs, sk.x_bs = k.a_bs;
-        sk.y = k.b, sk.y_ks = k.b_rs, sk.y_qs = k.b_cs, sk.y_bs = k.b_bs;
-        sk.c_ps = k.c_rs, sk.c_qs = k.c_cs, sk.L = M, sk.t = N;
-      } else {  // X = B (p = n), Y = A
-        sk.x = k.b, sk.x_ps = k.b_cs, sk.x_ks = k.b_rs, sk.x_bs = k.b_bs;
-        sk.y = k.a, sk.y_ks = k.a_cs, sk.y_qs = k.a_rs, sk.y_bs = k.a_bs;
-        sk.c_ps = k.c_cs, sk.c_qs = k.c_rs, sk.L = N, sk.t = M;
-      }
-      const char* tq = "q4";
-      char sname[64];
-      // The thin operand is read by every wave: unless it already is contiguous along k with
-      // aligned rows, pack it first as [q][k] (a few KiB that then stay in the caches).
-      Scratch packed(ctx);
-      // (the long operand is taken at any alignment)
-      const bool x_along_k = sk.x_ks == 1;
-      // (only the wave-per-row kernel reads the thin operand with vector loads; the other one takes
-      // it element by element with any strides)
-      if (x_along_k &&
-          !(sk.y_ks == 1 && aligned16(sk.y) && sk.y_qs % P == 0 && (batch <= 1 || sk.y_bs % P == 0))) {
-        const uint32_t kp = (K + P - 1) / P * P;
-        void* buf = nullptr;
-        HC_TRY(packed.get((size_t)batch * sk.t * kp * el, &buf));
-        hck_skinny_args pk = sk;
-        pk.c = buf;
-        pk.c_qs = sk.y_qs;  // source stride along q
-        pk.y_qs = kp;       // packed row length
-        snprintf(sname, sizeof(sname), "hc_gemm_skinny_pack_%s", dtype_name(dtype));
-        HC_TRY(launch(ctx, sname, ceil_div((uint64_t)sk.t * kp, HCK_BLOCK), (uint32_t)batch, &pk, sizeof(pk)));
-        sk.y = buf;
-        sk.y_ks = 1;
-        sk.y_qs = kp;
-        sk.y_bs = (uint64_t)sk.t * kp;
-      }
-      if (x_along_k) {
-        snprintf(sname, sizeof(sname), "hc_gemm_skinny_k_%s_%s", dtype_name(dtype), tq);
-        return launch(ctx, sname, ceil_div(sk.L, HCK_BLOCK / 64), (uint32_t)batch, &sk, sizeof(sk));
-      }
-      if (sk.x_ps == 1) {
-        // a workgroup per (64 lanes x 16 bytes of p, chunk of k): about two per CU, at least 32 k each
-        const uint64_t cus = (uint64_t)ctx->props.multiProcessorCount;
-        const uint64_t ptiles = ceil_div(sk.L, 64 * P);
-        uint64_t chunks = std::max<uint64_t>(1, std::min<uint64_t>(ceil_div(2 * cus, ptiles * (uint64_t)batch), K / 32));
-        sk.kchunk = (uint32_t)ceil_div(K, chunks);
-        chunks = ceil_div(K, sk.kchunk);
-        Scratch sums(ctx);
-        void* acc = nullptr;
-        // one slice of partial sums per chunk, added in chunk order by the store kernel: the
-        // result is the same on every run (no atomics, nothing to clear)
-        sk.chunks = (uint32_t)chunks;
-        const uint64_t n_acc = (uint64_t)batch * chunks * sk.L * sk.t;
-        HC_TRY(sums.get(n_acc * sizeof(float), &acc));
-        sk.acc = (float*)acc;
-        snprintf(sname, sizeof(sname), "hc_gemm_skinny_p_%s_%s", dtype_name(dtype), tq);
-        HC_TRY(launch(ctx, sname, ptiles * chunks, (uint32_t)batch, &sk, sizeof(sk)));
-        snprintf(sname, sizeof(sname), "hc_gemm_skinny_store_%s", dtype_name(dtype));
-        return launch(ctx, sname, ceil_div((uint64_t)sk.L * sk.t, HCK_BLOCK), (uint32_t)batch, &sk, sizeof(sk));
-      }
-    }
-    const uint64_t max_elems = 0xffffffffull / el;
-    const bool dma = k.a_bs <= max_elems && k.b_bs <= max_elems && !(which && strcmp(which, "staged") == 0);
-    // Two direct-to-LDS pipelines: four stages of 64-byte K-slices (deep prefetch: best when a CU
-    // has one short job) and two stages of 128-byte K-slices (whole cache lines for K-contiguous
-    // operands, half the barriers: best when the CUs are kept busy for long). Chosen below, after
-    // the tile; HCHIP_GEMM_KERNEL=dma|dma2 forces one.
-    // A third variant, fp16 only: the 128-byte-slice pipeline on the 16x16x32 MFMA shape, which
-    // needs less power per multiply-accumulate. It pays where the matrix cores run into the
-    // board's power limit: every CU busy with a 256 x 256 tile over a long K.
-    // HCHIP_GEMM_KERNEL=dma|dma2|mi16 forces one of the three.
-    bool mi16 = dma && dtype == HC_F16 && which && strcmp(which, "mi16") == 0;
-    bool dma2 = dma && which && (strcmp(which, "dma2") == 0 || mi16);
-    uint32_t slice = (uint32_t)(64 / el);
-    const bool eligible = ma != 'x' && mb != 'x' && K > 0 &&
-                          (loose ? dma
-                                 : aligned16(k.c) && (dma ? (k.c_rs % P == 0 && (batch <= 1 || k.c_bs % P == 0))
-                                                          : (dtype == HC_F16 && K % 64 == 0)));
-    if (eligible) {
-      const char* force = getenv("HCHIP_GEMM_TILE");
-      auto whole = [&](uint32_t tm, uint32_t tn) { return M % tm == 0 && N % tn == 0 && K % slice == 0; };
-      // largest tile first; the direct-to-LDS kernels also come in narrow shapes
-      static const uint32_t tiles[][2] = {{256, 256}, {256, 128}, {128, 128}, {256, 64}, {128, 64}, {64, 64}};
-      // (only the 16x16x32 pipeline and, for fp32, the two-stage pipeline have these)
-      static const uint32_t tiles192[][2] = {{256, 192}, {192, 256}, {192, 192}};
-      const uint64_t cus = (uint64_t)ctx->props.multiProcessorCount;
-      if (force && *force) {
-        unsigned fm = 0, fn = 0;
-        if (sscanf(force, "%ux%u", &fm, &fn) == 2 && (dma || whole(fm, fn))) {
-          bool known = false;
-          for (auto& t : tiles) known = known || (t[0] == fm && t[1] == fn);
-          if (mi16 || (dma2 && dtype == HC_F32))
-            for (auto& t : tiles192) known = known || (t[0] == fm && t[1] == fn);
-          if (known) {
-            bm = fm;
-            bn = fn;
-          }
-        }
-      } else {
-        // Among the tiles that give every CU a block: the best product of (rough per-CU rate of
-        // the tile) x (fraction of the last round of blocks that is busy) x (fraction of the
-        // tiles' area that is real output). If no tile fills the device: the one with most blocks.
-        static const double rate16[] = {1.0, 0.85, 0.7, 0.55, 0.45, 0.3};
-        static const double rate32[] = {1.0, 0.95, 0.85, 0.8, 0.7, 0.55};
-        const double* rate = dtype == HC_F32 ? rate32 : rate16;
-        uint64_t best_blocks = 0;
-        double best_score = 0.0;
-        bool filled = false;
-        for (size_t ti = 0; ti < sizeof(tiles) / sizeof(tiles[0]); ti++) {
-          const uint32_t* t = tiles[ti];
-          if (!dma && (!whole(t[0], t[1]) || t[1] < 128)) continue;
-          const uint64_t blocks = ceil_div(M, t[0]) * ceil_div(N, t[1]) * (uint64_t)batch;
-          if (blocks >= cus) {
-            const double rounds = (double)ceil_div(blocks, cus);
-            const double useful = ((double)M * N * (double)batch) / ((double)blocks * t[0] * t[1]);
-            const double score = rate[ti] * ((double)blocks / (rounds * (double)cus)) * useful;
-            if (!filled || score > best_score) {
-              filled = true;
-              best_score = score;
-              bm = t[0];
-              bn = t[1];
-            }
-          } else if (!filled && blocks >= best_blocks) {  // (a tie goes to the smaller tile: less padding)
-            best_blocks = blocks;
-            bm = t[0];
-            bn = t[1];
-          }
-        }
-        // A K of one 128-byte slice is load -> one step of MFMAs -> store with nothing to overlap
-        // inside a workgroup, so what hides the latencies is several workgroups per CU: the largest
-        // tile that still gives every CU two blocks (QK^T of 32 x [512,64] x [64,512]: 256 x 128
-        // tiles 6.8 us, 128 x 128 tiles 6.2 us).
-        // With an operand that is contiguous along K such a product runs the single-slice variant
-        // (one stage of LDS, see below), which fits twice as many workgroups: four blocks per CU
-        // where a tile offers them (same scores: 128 x 64 tiles 6.7 us against 7.2 with 128 x 128).
-        if (dma && (uint64_t)K * el <= 128) {
-          bool found = false;
-          for (uint64_t want : {(uint64_t)4, (uint64_t)2}) {
-            if (want == 4 && !(ma == 'k' || mb == 'k')) continue;
-            for (size_t ti = 0; ti < sizeof(tiles) / sizeof(tiles[0]) && !found; ti++) {
-              const uint32_t* t = tiles[ti];
-              const uint64_t blocks = ceil_div(M, t[0]) * ceil_div(N, t[1]) * (uint64_t)batch;
-              const double useful = ((double)M * N * (double)batch) / ((double)blocks * t[0] * t[1]);
-              if (blocks >= want * cus && useful >= 0.75) {
-                bm = t[0];
-                bn = t[1];
-                found = true;
-              }
-            }
-            if (found) break;
-          }
-        }
-        // fp32 products with K >= 512 also have the 192-extent tiles of the two-stage pipeline: fp32
-        // runs every large tile at the same rate (it is not limited by power), so what counts is
-        // how evenly the tiles fill the device (3072^2 outputs: 16 x 16 tiles of 192 x 192 are one
-        // full round, 144 tiles of 256 x 256 leave 44 % of the CUs idle).
-        if (dtype == HC_F32 && dma && !which && K >= 512 && filled) {
-          static const double rate192[] = {0.97, 0.97, 0.95};
-          for (size_t ti = 0; ti < sizeof(tiles192) / sizeof(tiles192[0]); ti++) {
-            const uint32_t* t = tiles192[ti];
-            const uint64_t blocks = ceil_div(M, t[0]) * ceil_div(N, t[1]) * (uint64_t)batch;
-            if (blocks < cus) continue;
-            const double rounds = (double)ceil_div(blocks, cus);
-            const double useful = ((double)M * N * (double)batch) / ((double)blocks * t[0] * t[1]);
-            const double score = rate192[ti] * ((double)blocks / (rounds * (double)cus)) * useful;
-            if (score > best_score) {
-              best_score = score;
-              bm = t[0];
-              bn = t[1];
-              dma2 = true;
-            }
-          }
-        }
-      }
-      // Long fp16 products that can keep at least half of the device busy run on the 16x16x32
-      // pipeline; its tile is the one with the least estimated time = rounds of blocks x tile
-      // area / rate. Rates: full device, relative to 256 x 256, times 0.88 for the edge kernels
-      // of a ragged product. A last round that occupies a fraction f of the CUs counts as
-      // max(f^0.25, 0.5) of a round: such products are limited by power, so the busy CUs of a
-      // partly idle device get a higher clock (measured: 144 tiles of 256 x 256 on 256 CUs reach
-      // 58 % (K = 2048) to 72 % (K = 4096) of the full-device rate, 33 tiles take 0.58 of the
-      // time of 256). The constants were fitted to a sweep of 18 shapes x 3 layouts x 6 tiles;
-      // the model's pick is within 5 % of the best tile on all but two of them (14 %).
-      bool model_mi16 = false;
-      if (!(force && *force) && !which && dma && dtype == HC_F16 && K >= 1024) {
-        const uint64_t t256 = ceil_div(M, 256) * ceil_div(N, 256) * (uint64_t)batch;
-        const uint64_t t128 = ceil_div(M, 128) * ceil_div(N, 128) * (uint64_t)batch;
-        if (2 * t256 >= cus || 2 * t128 >= 3 * cus) {
-          static const struct { uint32_t bm, bn; double rate; } cand[] = {
-              {256, 256, 1.0}, {256, 192, 0.9}, {192, 256, 0.9}, {192, 192, 0.82}, {256, 128, 0.76}, {128, 128, 0.6}};
-          double best = 0.0;
-          for (auto& c : cand) {
-            const uint64_t blocks = ceil_div(M, c.bm) * ceil_div(N, c.bn) * (uint64_t)batch;
-            const uint64_t rem = blocks % cus;
-            double rounds = (double)(blocks / cus);
-            if (rem != 0) rounds += std::max(pow((double)rem / (double)cus, 0.25), 0.5);
-            const bool ragged = M % c.bm != 0 || N % c.bn != 0 || K % 64 != 0;
-            const double cost = rounds * c.bm * c.bn / (c.rate * (ragged ? 0.88 : 1.0));
-            if (best == 0.0 || cost < best) {
-              best = cost;
-              bm = c.bm;
-              bn = c.bn;
-            }
-          }
-          dma2 = mi16 = model_mi16 = true;
-        }
-      }
-      if (bm != 0 && dma) {
-        const uint64_t blocks = ceil_div(M, bm) * ceil_div(N, bn) * (uint64_t)batch;
-        // (whole cache lines only help an operand that is contiguous along K: TN products stay
-        // with the four-stage ring)
-        const bool k_contig = ma == 'k' || mb == 'k';
-        if (!which && !model_mi16 && k_contig && (uint64_t)K * el >= 2048 && ((bm == 256 && bn == 256) || blocks >= 2 * cus))
-          dma2 = true;
-        // (a K of one 128-byte slice is a single step of that pipeline: nothing to prefetch, and the
-        // four-stage ring would fill stages that nobody reads; QK^T with 64-wide heads 7.6 -> 6.5 us)
-        if (!which && !model_mi16 && k_contig && (uint64_t)K * el <= 128) dma2 = true;
-
-        if (dma2) slice = (uint32_t)(128 / el);
-        // (the single-slice variants: one stage of LDS, no second fetch; HCHIP_GEMM_ONE=0 keeps the general loop)
-        const bool one_tile = (bm == 256 && bn == 128) || (bm == 128 && bn == 128) || (bm == 128 && bn == 64) || (bm == 64 && bn == 64);
-        one = dma2 && !mi16 && k_contig && (uint64_t)K * el <= 128 && one_tile && !getenv_is("HCHIP_GEMM_ONE", "0");
-      }
-      if (bm != 0) edge = !whole(bm, bn) || loose;   // (only the edge kernels take rows at any alignment)
-    }
-    if (bm != 0) {
-      k.tiles_m = (uint32_t)ceil_div(M, bm);
-      k.tiles_n = (uint32_t)ceil_div(N, bn);
-      if (dma && !getenv("HCHIP_GEMM_BAND")) {
-        // largest XCD rectangle whose super-block (4 x 2 XCDs) divides the tile grid
-        static const uint32_t shapes[][2] = {{4, 8}, {2, 4}, {1, 2}};
-        for (auto& sh : shapes)
-          if (k.tiles_m % (4 * sh[0]) == 0 && k.tiles_n % (2 * sh[1]) == 0) {
-            k.xcd_gn = 2;
-            k.xcd_sm = sh[0];
-            k.xcd_sn = sh[1];
-            break;
-          }
-      }
-      snprintf(name, sizeof(name), "hc_gemm_%s_%s_%ux%u_%c%c%s%s", dtype_name(dtype), dma ? (mi16 ? "mi16" : dma2 ? "dma2" : "dma") : "fast", bm, bn,
-               ma == 'k' ? 'k' : 'm', mb == 'k' ? 'k' : 'n', one ? "_1" : "", edge ? "_e" : "");
-    } else if (ma == 'x' || mb == 'x' || loose)
-      snprintf(name, sizeof(name), "hc_gemm_%s_xx", dtype_name(dtype));
-    else
-      snprintf(name, sizeof(name), "hc_gemm_%s_%c%c", dtype_name(dtype), ma == 'k' ? 'k' : 'm',
-               mb == 'k' ? 'k' : 'n');
-    const uint64_t tiles = (uint64_t)k.tiles_m * k.tiles_n;
-    // One launch of a direct-to-LDS kernel that writes the caller's dense [M, N] matrix from the
-    // caller's own operands: a recording may merge what follows into its epilogue.
-    if (whole_call && bm != 0 && dma && !loose && batch == 1 && !trans_out && !c_padded && k.a == a && k.b == b &&
-        k.c == out && k.c_rs == N) {
-      note.tag = hc_pending::GEMM;
-      note.meta.dtype = dtype;
-      note.meta.rows = M;
-      note.meta.cols = N;
-      note.meta.out = out;
-    }
-    // ... and a batched one may read or write through a swap of the batch axes
-    if (whole_call && bm != 0 && dma && !loose && batch > 1 && batch <= 65535 && !trans_out && !c_padded && k.a == a &&
-        k.b == b && k.c == out && k.c_rs == N) {
-      note.tag = hc_pending::BMM;
-      note.meta.dtype = dtype;
-      note.meta.rows = M;
-      note.meta.cols = N;
-      note.meta.in0 = a;
-      note.meta.in1 = b;
-      note.meta.out = out;
-    }
-    // grid.y carries the batch (at most 65535 per launch)
-    for (int64_t b0 = 0; b0 < batch; b0 += 65535) {
-      const uint32_t nb = (uint32_t)(batch - b0 < 65535 ? batch - b0 : 65535);
-      hck_gemm_args kk = k;
-      kk.a = (const char*)k.a + (uint64_t)b0 * k.a_bs * el;
-      kk.b = (const char*)k.b + (uint64_t)b0 * k.b_bs * el;
-      kk.c = (char*)k.c + (uint64_t)b0 * k.c_bs * el;
-      kk.batch = nb;
-      HC_TRY(launch(ctx, name, tiles, nb, &kk, sizeof(kk)));
-    }
-    return HC_OK;
-  };
-  // The body-plus-fringes split (see `peelable` above), for operands the tuned kernels can take
-  const bool tuned = ma != 'x' && mb != 'x' && peelable;
-  const uint32_t fm = tuned ? fringe(M) : 0, fn = tuned ? fringe(N) : 0;
-  if (fm != 0 || fn != 0) {
-    const uint32_t Mb = M - fm, Nb = N - fn;
-    HC_TRY(run(k, Mb, Nb));
-    if (fn != 0) {  // columns Nb .. N-1 of every row
-      hck_gemm_args f = k;
-      f.b = (const char*)k.b + (uint64_t)Nb * k.b_cs * el;
-      f.c = (char*)k.c + (uint64_t)Nb * k.c_cs * el;
-      HC_TRY(run(f, M, fn));
-    }
-    if (fm != 0) {  // rows Mb .. M-1, columns 0 .. Nb-1
-      hck_gemm_args f = k;
-      f.a = (const char*)k.a + (uint64_t)Mb * k.a_rs * el;
-      f.c = (char*)k.c + (uint64_t)Mb * k.c_rs * el;
-      HC_TRY(run(f, fm, Nb));
-    }
-  } else {
-    whole_call = true;
-    HC_TRY(run(k, M, N));
-  }
-  if (c_padded) {
-    // padded result back into the caller's dense [M, N] matrices
-    hck_copy2d_args c;
-    memset(&c, 0, sizeof(c));
-    c.in = c_padded;
-    c.out = out;
-    c.rows = M;
-    c.in_cols = N;
-    c.out_cols = N;
-    c.in_ld = c_ld;
-    c.out_ld = N;
-    c.in_bs = (uint64_t)M * c_ld;
-    c.out_bs = (uint64_t)M * N;
-    const uint64_t waves = (uint64_t)M * ceil_div(N, 512);
-    HC_TRY(launch(ctx, el == 2 ? "hc_copy2d_unpad_b2" : "hc_copy2d_unpad_b4", ceil_div(waves, HCK_BLOCK / 64),
-                  (uint32_t)batch, &c, sizeof(c)));
-  }
-  return HC_OK;
-}
+#include "hchip_matmul.inc"
