@@ -229,8 +229,15 @@ template <typename T, int ROWS, int MODE> struct DmaOperand {
 // multiplies and stores, with one stage of LDS (`lds1` unused): twice as many workgroups fit a CU,
 // which is what hides the latencies of such a launch. (The general loop would fetch the clamped
 // "next" slices into the second stage and wait for them twice before the write-out.)
-template <typename T, int BM, int BN, int MODE_A, int MODE_B, bool EDGE, bool ONE = false>
-__device__ __forceinline__ void gemm_dma2_impl(const hck_gemm_args& p, char* lds0, char* lds1) {
+// RING4: four stages instead of two (`lds2`, `lds3`), three K-slices ahead. For the small tiles
+// whose workgroup has a compute unit to itself: what a K-step of such a tile costs is mostly fixed
+// (waits, barrier, scalar bookkeeping: the four-stage pipeline of 64-byte slices spends about 275
+// cycles per slice on a 64 x 64 tile, of which the MFMAs are 128), so the slices should be long,
+// and with one workgroup per compute unit only a deep ring keeps enough loads in flight.
+template <typename T, int BM, int BN, int MODE_A, int MODE_B, bool EDGE, bool ONE = false, bool RING4 = false>
+__device__ __forceinline__ void gemm_dma2_impl(const hck_gemm_args& p, char* lds0, char* lds1, char* lds2 = nullptr,
+                                               char* lds3 = nullptr) {
+  static_assert(!(ONE && RING4), "one slice needs no ring");
   constexpr int MT = BM / 64, NT = BN / 64;
   constexpr int SLOTS = MT * NT;
   typedef DmaOperand<T, BM, MODE_A> OpA;
@@ -382,7 +389,60 @@ __device__ __forceinline__ void gemm_dma2_impl(const hck_gemm_args& p, char* lds
     substep(tail, f1, f0, nxt, 0, 0, cur, kclamp(j + 2));
   };
 
-  if constexpr (ONE) {
+  // Ring of four: K-step j out of `cur`; `nxt` holds K-step j+1 once the wait passes; the stage
+  // of K-step j-1 (`prev`, free since the barrier of the step before) receives K-step j+3.
+  auto step4 = [&](auto tail, char* cur, char* nxt, char* prev, uint32_t j) {
+    const uint32_t k3 = kclamp(j + 3);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int u = 0; u < NDMA; u++) dma_unit(tail, u, k3, prev);
+    substep(tail, f0, f1, cur, 1, -1, nullptr, 0);
+    substep(tail, f1, f0, cur, 2, -1, nullptr, 0);
+    substep(tail, f0, f1, cur, 3, -1, nullptr, 0);
+    static_assert(2 * NDMA < 64, "more loads in flight than the counter holds");
+    wait_dma<2 * NDMA>();  // K-step j+1 of this wave has landed (in flight: j+2 and j+3) ...
+    if constexpr (decltype(tail)::value) {
+      if (ktail && j + 2 == nk) zero_tail(nxt, (j + 1) * BK);
+    }
+    lds_barrier();  // ... and everybody's; nobody reads cur any more
+    __builtin_amdgcn_sched_barrier(0);
+    substep(tail, f1, f0, nxt, 0, -1, nullptr, 0);
+  };
+
+  if constexpr (RING4) {
+    // prologue: K-steps 0, 1 and 2
+#pragma unroll
+    for (int u = 0; u < NDMA; u++) dma_unit(Tail{}, u, 0, lds0);
+#pragma unroll
+    for (int u = 0; u < NDMA; u++) dma_unit(Tail{}, u, kclamp(1), lds1);
+#pragma unroll
+    for (int u = 0; u < NDMA; u++) dma_unit(Tail{}, u, kclamp(2), lds2);
+    wait_dma<2 * NDMA>();
+    if constexpr (EDGE) {
+      if (ktail && nk == 1) zero_tail(lds0, 0);
+    }
+    lds_barrier();
+#pragma unroll
+    for (int u = 0; u < READS; u++) read_unit(f0, lds0, 0, u);
+    uint32_t j = 0;
+    if constexpr (EDGE) {  // K-step j fetches slice j+3: a group of four steps from j <= nk - 8 never fetches the last slice
+      for (; j + 8 <= nk; j += 4) {
+        step4(NoTail{}, lds0, lds1, lds3, j);
+        step4(NoTail{}, lds1, lds2, lds0, j + 1);
+        step4(NoTail{}, lds2, lds3, lds1, j + 2);
+        step4(NoTail{}, lds3, lds0, lds2, j + 3);
+      }
+    }
+    for (; j + 3 < nk; j += 4) {
+      step4(Tail{}, lds0, lds1, lds3, j);
+      step4(Tail{}, lds1, lds2, lds0, j + 1);
+      step4(Tail{}, lds2, lds3, lds1, j + 2);
+      step4(Tail{}, lds3, lds0, lds2, j + 3);
+    }
+    if (j < nk) step4(Tail{}, lds0, lds1, lds3, j);
+    if (j + 1 < nk) step4(Tail{}, lds1, lds2, lds0, j + 1);
+    if (j + 2 < nk) step4(Tail{}, lds2, lds3, lds1, j + 2);
+  } else if constexpr (ONE) {
 #pragma unroll
     for (int u = 0; u < NDMA; u++) dma_unit(Tail{}, u, 0, lds0);
     wait_dma<0>();
@@ -559,6 +619,30 @@ __device__ __forceinline__ void gemm_dma2_impl(const hck_gemm_args& p, char* lds
     __shared__ __attribute__((aligned(1024))) char lds0[(BM + BN) * 128];                             \
     gemm_dma2_impl<T, BM, BN, AM, BMODE, true, true>(p, lds0, nullptr);                               \
   }
+// (every stage a __shared__ array of its own: the compiler then knows that a DMA into one stage does
+// not touch the stage a read comes from)
+#define DEF_DMA_RING4(T, TN, BM, BN, AN, AM, BNAME, BMODE)                                            \
+  extern "C" __global__ __launch_bounds__(256) void HC_GEMM_NAME(hc_gemm_##TN##_dma2_##BM##x##BN##_##AN##BNAME##_r4)( \
+      hck_gemm_args p) {                                                                              \
+    __shared__ __attribute__((aligned(1024))) char lds0[(BM + BN) * 128];                             \
+    __shared__ __attribute__((aligned(1024))) char lds1[(BM + BN) * 128];                             \
+    __shared__ __attribute__((aligned(1024))) char lds2[(BM + BN) * 128];                             \
+    __shared__ __attribute__((aligned(1024))) char lds3[(BM + BN) * 128];                             \
+    gemm_dma2_impl<T, BM, BN, AM, BMODE, false, false, true>(p, lds0, lds1, lds2, lds3);              \
+  }                                                                                                   \
+  extern "C" __global__ __launch_bounds__(256) void HC_GEMM_NAME(hc_gemm_##TN##_dma2_##BM##x##BN##_##AN##BNAME##_r4_e)( \
+      hck_gemm_args p) {                                                                              \
+    __shared__ __attribute__((aligned(1024))) char lds0[(BM + BN) * 128];                             \
+    __shared__ __attribute__((aligned(1024))) char lds1[(BM + BN) * 128];                             \
+    __shared__ __attribute__((aligned(1024))) char lds2[(BM + BN) * 128];                             \
+    __shared__ __attribute__((aligned(1024))) char lds3[(BM + BN) * 128];                             \
+    gemm_dma2_impl<T, BM, BN, AM, BMODE, true, false, true>(p, lds0, lds1, lds2, lds3);               \
+  }
+#define DEF_DMA_RING4_TILE(T, TN, BM, BN)                                                             \
+  DEF_DMA_RING4(T, TN, BM, BN, k, DMA_K, k, DMA_K)                                                    \
+  DEF_DMA_RING4(T, TN, BM, BN, k, DMA_K, n, DMA_MN)                                                   \
+  DEF_DMA_RING4(T, TN, BM, BN, m, DMA_MN, k, DMA_K)                                                   \
+  DEF_DMA_RING4(T, TN, BM, BN, m, DMA_MN, n, DMA_MN)
 // (single-slice variants: layouts with an operand that is contiguous along K, the only ones the host
 // sends here)
 #define DEF_DMA_ONE_TILE(T, TN, BM, BN)                                                               \
@@ -579,6 +663,10 @@ __device__ __forceinline__ void gemm_dma2_impl(const hck_gemm_args& p, char* lds
   DEF_DMA_TILE(T, TN, 64, 64)
 DEF_DMA_TYPE(half_t, f16)
 DEF_DMA_TYPE(float, f32)
+// (fp16, the two smallest tiles: 2048 x 2048 x 512 on 64 x 64 tiles 11.9 -> 9.7 us, 512 x 4096 x 512
+// 19.1 -> 15.0; 128 x 128 tiles and fp32 gain nothing from it)
+DEF_DMA_RING4_TILE(half_t, f16, 128, 64)
+DEF_DMA_RING4_TILE(half_t, f16, 64, 64)
 DEF_DMA_ONE_TILE(half_t, f16, 256, 128)
 DEF_DMA_ONE_TILE(half_t, f16, 128, 128)
 DEF_DMA_ONE_TILE(half_t, f16, 128, 64)

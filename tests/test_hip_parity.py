@@ -177,6 +177,36 @@ def test_matmul_single_slice_variant(hip_backend, oracle_backend, monkeypatch, d
                     assert np.array_equal(np.ascontiguousarray(got).view(bits), np.ascontiguousarray(loop).view(bits))
 
 
+def test_matmul_ring_of_four(hip_backend, oracle_backend, monkeypatch):
+    """The 128-byte-slice pipeline's two smallest fp16 tiles also exist with a ring of four stages
+    (picked when a workgroup has a compute unit, or half of one, to itself). Forced here on products
+    whose K is shorter than the ring, as long as it, a multiple of it and ragged, whole tiles and
+    edges, odd leading dimensions, batches: against the oracle, and bit for bit against the
+    two-stage kernels (same instructions on the same accumulators in the same order)."""
+    rng = np.random.default_rng(98)
+    dtype, bits = F16, np.uint16
+    for tile in ("64x64", "128x64"):
+        monkeypatch.setenv("HCHIP_GEMM_TILE", tile)
+        for K in (192, 200, 256, 320, 512 + 5, 1024, 1001, 64 * 11 - 7):
+            for (batch, M, N) in ((1, 128, 128), (2, 200, 72), (1, 67, 129)):
+                a = rand(rng, (batch, M, K), dtype, 1.0 / K ** 0.5)
+                b = rand(rng, (batch, K, N), dtype)
+                for transA, transB in ((False, False), (True, True), (False, True), (True, False)):
+                    sa = np.ascontiguousarray(a.transpose(0, 2, 1)) if transA else a
+                    sb = np.ascontiguousarray(b.transpose(0, 2, 1)) if transB else b
+                    print("ring of four", tile, batch, M, K, N, transA, transB, flush=True)
+                    fn = lambda: Tensor.batchedMatmul(Tensor(data=sa), transA, Tensor(data=sb), transB, False)
+                    monkeypatch.setenv("HCHIP_GEMM_RING", "4")
+                    got, want = check_close(hip_backend, oracle_backend, fn, TOL[dtype])
+                    monkeypatch.setenv("HCHIP_GEMM_RING", "2")
+                    monkeypatch.setenv("HCHIP_GEMM_KERNEL", "dma2")
+                    with hip_backend.use():
+                        two = fn().numpy()
+                    monkeypatch.delenv("HCHIP_GEMM_RING")
+                    monkeypatch.delenv("HCHIP_GEMM_KERNEL")
+                    assert np.array_equal(np.ascontiguousarray(got).view(bits), np.ascontiguousarray(two).view(bits))
+
+
 @pytest.mark.parametrize("pipeline", ["auto", "dma", "dma2", "mi16"])
 def test_matmul_random_shapes(hip_backend, oracle_backend, monkeypatch, pipeline):
     """Seeded random extents (aligned and odd), batches and flags through each pipeline: row and
