@@ -31,7 +31,8 @@ KERNELS = [
     # the same three sources once more: kernels named *_m whose write-out applies the operations a
     # recording merged into the product (the plain kernels above contain none of that code)
     ("gemm_dma_m", "gemm_dma.hip", ["-ffp-contract=off", "-DHC_GEMM_MERGED=1"]),
-    ("gemm_dma2_m", "gemm_dma2.hip", ["-ffp-contract=off", "-DHC_GEMM_MERGED=1"]),
+    ("gemm_dma2_m_f16", "gemm_dma2.hip", ["-ffp-contract=off", "-DHC_GEMM_MERGED=1", "-DHC_GEMM_ONLY=16"]),
+    ("gemm_dma2_m_f32", "gemm_dma2.hip", ["-ffp-contract=off", "-DHC_GEMM_MERGED=1", "-DHC_GEMM_ONLY=32"]),
     ("gemm_mi16_m", "gemm_mi16.hip", ["-ffp-contract=off", "-DHC_GEMM_MERGED=1"]),
 ]
 DEVICE_FLAGS = [
@@ -55,7 +56,7 @@ def _run(cmd):
 # sit at the 256-VGPR limit; the edge kernels' write-out needs a few registers more): up to 96 bytes
 # per lane in the plain kernels, up to 128 in the kernels with merged epilogues.
 NO_SCRATCH = {"gemm_dma": 96, "gemm_dma2": 96, "gemm_mi16": 96, "gemm_f16_fast": 16,
-              "gemm_dma_m": 128, "gemm_dma2_m": 128, "gemm_mi16_m": 128}
+              "gemm_dma_m": 128, "gemm_dma2_m_f16": 128, "gemm_dma2_m_f32": 128, "gemm_mi16_m": 128}
 
 
 def kernels_with_scratch(remarks, allowed=0):

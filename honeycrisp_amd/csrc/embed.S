@@ -23,7 +23,8 @@
     EMBED hc_image_gemm_dma2, "gemm_dma2.hsaco"
     EMBED hc_image_gemm_mi16, "gemm_mi16.hsaco"
     EMBED hc_image_gemm_dma_m, "gemm_dma_m.hsaco"
-    EMBED hc_image_gemm_dma2_m, "gemm_dma2_m.hsaco"
+    EMBED hc_image_gemm_dma2_m_f16, "gemm_dma2_m_f16.hsaco"
+    EMBED hc_image_gemm_dma2_m_f32, "gemm_dma2_m_f32.hsaco"
     EMBED hc_image_gemm_mi16_m, "gemm_mi16_m.hsaco"
 
     .section .note.GNU-stack,"",@progbits

@@ -33,7 +33,8 @@ extern const unsigned char hc_image_gemm_dma[], hc_image_gemm_dma_end[];
 extern const unsigned char hc_image_gemm_dma2[], hc_image_gemm_dma2_end[];
 extern const unsigned char hc_image_gemm_mi16[], hc_image_gemm_mi16_end[];
 extern const unsigned char hc_image_gemm_dma_m[], hc_image_gemm_dma_m_end[];
-extern const unsigned char hc_image_gemm_dma2_m[], hc_image_gemm_dma2_m_end[];
+extern const unsigned char hc_image_gemm_dma2_m_f16[], hc_image_gemm_dma2_m_f16_end[];
+extern const unsigned char hc_image_gemm_dma2_m_f32[], hc_image_gemm_dma2_m_f32_end[];
 extern const unsigned char hc_image_gemm_mi16_m[], hc_image_gemm_mi16_m_end[];
 }
 
@@ -234,7 +235,8 @@ extern "C" int hc_init(int device, hc_ctx** out) {
   if (s == HC_OK) s = load_image(ctx, hc_image_gemm_dma2, hc_image_gemm_dma2_end, "gemm_dma2");
   if (s == HC_OK) s = load_image(ctx, hc_image_gemm_mi16, hc_image_gemm_mi16_end, "gemm_mi16");
   if (s == HC_OK) s = load_image(ctx, hc_image_gemm_dma_m, hc_image_gemm_dma_m_end, "gemm_dma_m");
-  if (s == HC_OK) s = load_image(ctx, hc_image_gemm_dma2_m, hc_image_gemm_dma2_m_end, "gemm_dma2_m");
+  if (s == HC_OK) s = load_image(ctx, hc_image_gemm_dma2_m_f16, hc_image_gemm_dma2_m_f16_end, "gemm_dma2_m_f16");
+  if (s == HC_OK) s = load_image(ctx, hc_image_gemm_dma2_m_f32, hc_image_gemm_dma2_m_f32_end, "gemm_dma2_m_f32");
   if (s == HC_OK) s = load_image(ctx, hc_image_gemm_mi16_m, hc_image_gemm_mi16_m_end, "gemm_mi16_m");
   if (s != HC_OK) {
     hc_shutdown(ctx);

@@ -661,8 +661,10 @@ __device__ __forceinline__ void gemm_dma2_impl(const hck_gemm_args& p, char* lds
   DEF_DMA_TILE(T, TN, 256, 64)                                                                        \
   DEF_DMA_TILE(T, TN, 128, 64)                                                                        \
   DEF_DMA_TILE(T, TN, 64, 64)
+// HC_GEMM_ONLY=16 / 32: the fp16 / fp32 kernels only (the second build of this file is compiled as two
+// code objects side by side; as one it was the longest step of the whole build)
+#if !defined(HC_GEMM_ONLY) || HC_GEMM_ONLY == 16
 DEF_DMA_TYPE(half_t, f16)
-DEF_DMA_TYPE(float, f32)
 // (fp16, the two smallest tiles: 2048 x 2048 x 512 on 64 x 64 tiles 11.9 -> 9.7 us, 512 x 4096 x 512
 // 19.1 -> 15.0; 128 x 128 tiles and fp32 gain nothing from it)
 DEF_DMA_RING4_TILE(half_t, f16, 128, 64)
@@ -671,6 +673,9 @@ DEF_DMA_ONE_TILE(half_t, f16, 256, 128)
 DEF_DMA_ONE_TILE(half_t, f16, 128, 128)
 DEF_DMA_ONE_TILE(half_t, f16, 128, 64)
 DEF_DMA_ONE_TILE(half_t, f16, 64, 64)
+#endif
+#if !defined(HC_GEMM_ONLY) || HC_GEMM_ONLY == 32
+DEF_DMA_TYPE(float, f32)
 DEF_DMA_ONE_TILE(float, f32, 256, 128)
 DEF_DMA_ONE_TILE(float, f32, 128, 128)
 DEF_DMA_ONE_TILE(float, f32, 128, 64)
@@ -679,3 +684,4 @@ DEF_DMA_ONE_TILE(float, f32, 64, 64)
 DEF_DMA_TILE(float, f32, 256, 192)
 DEF_DMA_TILE(float, f32, 192, 256)
 DEF_DMA_TILE(float, f32, 192, 192)
+#endif
