@@ -214,3 +214,51 @@ def test_operand_that_fills_its_block(hip_backend, oracle_backend, dtype):
                                   c_void_p(out.ptr)))
     got = out.onCPU().view(dtype.numpy)[:M * N].reshape(M, N)
     assert_close_arrays(got, want, TOL[dtype], TOL[dtype])
+
+
+def test_random_products_with_infinite_surroundings(hip_backend):
+    """Seeded random extents (around the piece, wave and tile sizes, a few long K), dtypes, batches
+    and flags; operands and output start at random element offsets inside their buffers, the
+    elements in front of and behind each operand are infinite, the output's surroundings are
+    checked bit for bit. Whatever a kernel fetches beyond an operand's rows (the last 16-byte piece
+    of the last row reaches into the infinities) must not reach the result."""
+    hip = hip_backend
+    rng = np.random.default_rng(31)
+    dims = [1, 2, 3, 5, 7, 8, 9, 15, 16, 17, 31, 33, 63, 64, 65, 100, 127, 129, 191, 200, 255, 257, 264, 320, 383, 500, 513,
+            640, 1000, 1023, 1025]
+    for case in range(160):
+        dtype = F16 if rng.integers(0, 3) else F32
+        np_t = dtype.numpy
+        es = np.dtype(np_t).itemsize
+        bits = np.uint16 if es == 2 else np.uint32
+        M, K, N = (int(rng.choice(dims)) for _ in range(3))
+        if case % 11 == 0:
+            K = int(rng.choice([1500, 2050, 2304, 4097]))
+        if case % 13 == 0:
+            M, N = int(rng.choice([2049, 2052, 2080])), int(rng.choice([1024, 2049, 1000]))
+        batch = int(rng.choice([1, 1, 1, 2, 3]))
+        ta, tb, to = (bool(rng.integers(0, 2)) for _ in range(3))
+        offa, offb, offc = (int(rng.integers(0, 9)) for _ in range(3))
+        a = (rng.standard_normal((batch, M, K)) / np.sqrt(K)).astype(np_t)
+        b = rng.standard_normal((batch, K, N)).astype(np_t)
+        sa = np.ascontiguousarray(a.transpose(0, 2, 1)) if ta else a
+        sb = np.ascontiguousarray(b.transpose(0, 2, 1)) if tb else b
+        abuf = np.full(offa + sa.size + 16, np.inf, np_t)
+        abuf[offa:offa + sa.size] = sa.reshape(-1)
+        bbuf = np.full(offb + sb.size + 16, np.inf, np_t)
+        bbuf[offb:offb + sb.size] = sb.reshape(-1)
+        cbuf = rng.standard_normal(offc + batch * M * N + 16).astype(np_t)
+        da, db, dc = hip.upload(abuf), hip.upload(bbuf), hip.upload(cbuf)
+        print("case", case, dtype.name, batch, M, K, N, ta, tb, to, offa, offb, offc, flush=True)
+        hip._check(hip._lib.hc_matmul(hip._ctx, int(dtype), batch, c_void_p(da.ptr + offa * es), int(ta),
+                                      c_void_p(db.ptr + offb * es), int(tb), int(to), M, K, N, c_void_p(dc.ptr + offc * es)))
+        host = dc.onCPU().view(np_t)[:cbuf.size]
+        n_out = batch * M * N
+        assert np.array_equal(host[:offc].view(bits), cbuf[:offc].view(bits)), "wrote in front of C"
+        assert np.array_equal(host[offc + n_out:].view(bits), cbuf[offc + n_out:].view(bits)), "wrote behind C"
+        c = host[offc:offc + n_out].astype(np.float64)
+        c = c.reshape(batch, N, M).transpose(0, 2, 1) if to else c.reshape(batch, M, N)
+        want = a.astype(np.float64) @ b.astype(np.float64)
+        assert np.all(np.isfinite(c)), "something outside the operands reached the result"
+        tol = TOL[dtype]
+        assert float(np.max(np.abs(c - want))) <= 1.5 * tol * max(float(np.max(np.abs(want))), 1e-30)
