@@ -40,8 +40,9 @@ PEAK_F16_TFLOPS = 2516.6  # MI355X dense fp16 MFMA
 PEAK_F32_TFLOPS = 157.3   # MI355X fp32 MFMA
 PEAK_HBM_GBS = 8000.0     # MI355X HBM3E
 # HBM bytes per 4096^3 fp16 GEMM launch, from rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs of
-# this benchmark scaled by a plain copy kernel (not measurable live; the run that produced it is
-# summarised in profiles/bench_hbm_traffic_fetch_write_size.md): 196850 KiB read + 32768 KiB written.
+# this benchmark scaled by a plain copy kernel (not measurable live; the runs that produced it are
+# summarised in profiles/gemm_f16_4096_and_cfg4_hbm_traffic_fetch_write_size.md): 196800 KiB read +
+# 32768 KiB written.
 GEMM_TRAFFIC_BYTES = (196800 + 32768) * 1024
 GEMM_TRAFFIC_SOURCE = "constant from profiles/gemm_f16_4096_and_cfg4_hbm_traffic_fetch_write_size.md (rocprofv3 --pmc runs), not measured in this run"
 
@@ -533,13 +534,9 @@ def extra_workloads(backend, graph=True, only=("cfg1", "cfg2", "cfg3", "cfg4", "
                 # bias / GELU / residual into the products, LayerNorm and softmax chains into one
                 # kernel each, the head swaps into the batched products and q, k, v into one launch
                 for suffix, env in (("_graph_unmerged", "1"), ("_graph", None)):
-                    if env:
-                        os.environ["HCHIP_NO_FUSION"] = env
-                    try:
+                    with backend.switches(**({"HCHIP_NO_FUSION": env} if env else {})):
                         with backend.capture() as cap:
                             logits = model(tokens)
-                    finally:
-                        os.environ.pop("HCHIP_NO_FUSION", None)
                     for _ in range(5):
                         cap.graph.launch()
                     logits.wait()

@@ -55,6 +55,7 @@ PROTOTYPES = {
     "hc_shutdown": (None, [_P]),
     "hc_last_error_string": (c_char_p, []),
     "hc_get_device_info": (c_int, [_P, POINTER(hc_device_info)]),
+    "hc_debug_set": (c_int, [_P, c_char_p, c_char_p]),
     "hc_malloc": (c_int, [_P, c_size_t, POINTER(c_void_p)]),
     "hc_free": (c_int, [_P, _P]),
     "hc_trim": (c_int, [_P]),

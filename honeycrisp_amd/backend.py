@@ -10,6 +10,7 @@ the C ABI (include/hchip.h) on the context's in-order stream and returns a devic
 There is no CPU fallback here: an op or dtype the kernels do not cover raises
 `BackendError.notImplemented`, and a missing libhchip.so is an ImportError.
 """
+import contextlib
 import ctypes
 import threading
 from ctypes import byref, c_float, c_int64, c_size_t, c_void_p
@@ -412,6 +413,23 @@ class HIPBackend(Backend):
             "clock_mhz": info.clock_mhz, "wavefront_size": info.wavefront_size,
             "lds_bytes_per_block": info.lds_bytes_per_block, "total_mem": info.total_mem,
         }
+
+    def debugSet(self, name: str, value=None):
+        """Sets one of the library's measurement / test switches on this context (hc_debug_set);
+        `value` None restores the default."""
+        self._check(self._lib.hc_debug_set(self._ctx, name.encode(), None if value is None else str(value).encode()))
+
+    @contextlib.contextmanager
+    def switches(self, **kv):
+        """`with backend.switches(HCHIP_GEMM_TILE="256x256"):` sets the named switches for the
+        block and restores their defaults afterwards."""
+        for k, v in kv.items():
+            self.debugSet(k, v)
+        try:
+            yield self
+        finally:
+            for k in kv:
+                self.debugSet(k, None)
 
     def sync(self):
         self._check(self._lib.hc_sync(self._ctx))

@@ -14,6 +14,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <cmath>
+#include <map>
 #include <mutex>
 #include <string>
 #include <unordered_map>
@@ -108,14 +109,64 @@ struct hc_graph {
   std::vector<hc_pending> launches;
 };
 
+// Switches for measurements and tests (the names are those of the environment variables that
+// give them their first value when a context is created; hc_debug_set changes one later). Plain
+// data: an entry point copies the struct under the context's mutex and works on its copy, so a
+// thread that flips a switch never races a thread that launches.
+struct hc_switches {
+  char gemm_tile[16] = "";      // HCHIP_GEMM_TILE=general|<BM>x<BN>: overrides the tile choice
+  char gemm_kernel[16] = "";    // HCHIP_GEMM_KERNEL=dma|dma2|mi16|staged: the pipeline
+  char gemm_ring[8] = "";       // HCHIP_GEMM_RING=4|2: ring-of-four variant of the smallest tiles forced / off
+  char gemm_one[8] = "";        // HCHIP_GEMM_ONE=0: no single-slice variants
+  bool gemm_no_peel = false;    // HCHIP_GEMM_NO_PEEL: no body-plus-fringes split
+  bool gemm_no_direct = false;  // HCHIP_GEMM_NO_DIRECT: unaligned operands through padded copies
+  bool gemm_no_repitch = false; // HCHIP_GEMM_NO_REPITCH: ... or not even those (general kernel)
+  bool gemm_band = false;       // HCHIP_GEMM_BAND: plain band order of tiles instead of XCD rectangles
+  bool no_fusion = false;       // HCHIP_NO_FUSION: recordings are enqueued as they were issued
+  bool recording_log = false;   // HCHIP_RECORDING_LOG: the launches of a recording, to stderr
+  bool graph_as_launches = false;  // HCHIP_GRAPH_AS_LAUNCHES: replays issue their launches one by one
+};
+
+static bool switch_is_on(const char* v) { return v && *v && strcmp(v, "0") != 0; }
+
+// Sets the switch called `name` from `value` (NULL or "" = default). False for an unknown name.
+static bool set_switch(hc_switches& sw, const char* name, const char* value) {
+  struct Text { const char* name; char* dst; size_t cap; };
+  const Text texts[] = {{"HCHIP_GEMM_TILE", sw.gemm_tile, sizeof(sw.gemm_tile)},
+                        {"HCHIP_GEMM_KERNEL", sw.gemm_kernel, sizeof(sw.gemm_kernel)},
+                        {"HCHIP_GEMM_RING", sw.gemm_ring, sizeof(sw.gemm_ring)},
+                        {"HCHIP_GEMM_ONE", sw.gemm_one, sizeof(sw.gemm_one)}};
+  for (const Text& t : texts)
+    if (strcmp(name, t.name) == 0) {
+      snprintf(t.dst, t.cap, "%s", value ? value : "");
+      return true;
+    }
+  struct Flag { const char* name; bool* dst; };
+  const Flag flags[] = {{"HCHIP_GEMM_NO_PEEL", &sw.gemm_no_peel},     {"HCHIP_GEMM_NO_DIRECT", &sw.gemm_no_direct},
+                        {"HCHIP_GEMM_NO_REPITCH", &sw.gemm_no_repitch}, {"HCHIP_GEMM_BAND", &sw.gemm_band},
+                        {"HCHIP_NO_FUSION", &sw.no_fusion},           {"HCHIP_RECORDING_LOG", &sw.recording_log},
+                        {"HCHIP_GRAPH_AS_LAUNCHES", &sw.graph_as_launches}};
+  for (const Flag& f : flags)
+    if (strcmp(name, f.name) == 0) {
+      *f.dst = switch_is_on(value);
+      return true;
+    }
+  return false;
+}
+static const char* const kSwitchNames[] = {"HCHIP_GEMM_TILE",      "HCHIP_GEMM_KERNEL",     "HCHIP_GEMM_RING",
+                                           "HCHIP_GEMM_ONE",       "HCHIP_GEMM_NO_PEEL",    "HCHIP_GEMM_NO_DIRECT",
+                                           "HCHIP_GEMM_NO_REPITCH", "HCHIP_GEMM_BAND",       "HCHIP_NO_FUSION",
+                                           "HCHIP_RECORDING_LOG",  "HCHIP_GRAPH_AS_LAUNCHES"};
+
 struct hc_ctx {
   int device = 0;
   hipStream_t stream = nullptr;
   std::mutex mu;
+  hc_switches sw;                        // guarded by mu
   std::vector<hipModule_t> modules;
   std::unordered_map<std::string, hipFunction_t> functions;
   std::unordered_map<size_t, std::vector<void*>> free_blocks;
-  std::unordered_map<void*, size_t> live;
+  std::map<void*, size_t> live;          // blocks handed out: base -> bucket size, ordered by address
   size_t bytes_in_use = 0, bytes_cached = 0;
   hipDeviceProp_t props;
   hc_graph* capturing = nullptr;                      // the recording in progress, if any
@@ -130,6 +181,7 @@ struct hc_ctx {
   bool stage_busy[2] = {false, false};
   std::vector<hipEvent_t> wait_events;  // spare events of blocking transfers (waited for outside the mutex)
   bool lazy = false;                    // a capture that lists its launches (see hc_pending)
+  bool rewrite = false;                 // ... and will rewrite the list (decided when the capture begins)
   std::vector<hc_pending> pending;
   // buffers whose only writer and only reader were merged away by the rewrite of the recording in
   // progress: no launch of the graph touches them, so they need not stay reserved for it
@@ -194,9 +246,9 @@ extern "C" int hc_init(int device, hc_ctx** out) {
     return fail(HC_ERR_NO_DEVICE, "no HIP device available (%s)", hipGetErrorString(e));
   REQUIRE(device >= 0 && device < count, "hc_init: device %d out of range (have %d)", device, count);
   HIP_TRY(hipSetDevice(device));
-  HC_TRY(hc_noalloc_setup(device));
   hc_ctx* ctx = new hc_ctx();
   ctx->device = device;
+  for (const char* name : kSwitchNames) set_switch(ctx->sw, name, getenv(name));
   e = hipGetDeviceProperties(&ctx->props, device);
   if (e != hipSuccess) {
     delete ctx;
@@ -207,6 +259,13 @@ extern "C" int hc_init(int device, hc_ctx** out) {
                  ctx->props.gcnArchName);
     delete ctx;
     return s;
+  }
+  {  // (after the architecture check: on another device the lookup fails with a less telling message)
+    const int s = hc_noalloc_setup(device);
+    if (s != HC_OK) {
+      delete ctx;
+      return s;
+    }
   }
   e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
   if (e != hipSuccess) {
@@ -275,6 +334,29 @@ extern "C" void hc_shutdown(hc_ctx* ctx) {
   delete ctx;
 }
 
+extern "C" int hc_debug_set(hc_ctx* ctx, const char* name, const char* value) {
+  REQUIRE(ctx && name, "hc_debug_set: null argument");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  REQUIRE(set_switch(ctx->sw, name, value), "hc_debug_set: no switch called '%s'", name);
+  return HC_OK;
+}
+
+// The context's switches as they are now (a copy: see hc_switches).
+static hc_switches switches_of(hc_ctx* ctx) {
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  return ctx->sw;
+}
+
+// The block of this context that holds the address `p`: its base and size, or {nullptr, 0}.
+// Caller holds the mutex.
+static std::pair<void*, size_t> block_of_locked(const hc_ctx* ctx, const void* p) {
+  auto it = ctx->live.upper_bound(const_cast<void*>(p));
+  if (it == ctx->live.begin()) return {nullptr, 0};
+  --it;
+  if ((const char*)p < (const char*)it->first + it->second) return {it->first, it->second};
+  return {nullptr, 0};
+}
+
 extern "C" int hc_get_device_info(hc_ctx* ctx, hc_device_info* out) {
   REQUIRE(ctx && out, "hc_get_device_info: null argument");
   memset(out, 0, sizeof(*out));
@@ -319,11 +401,12 @@ extern "C" int hc_malloc(hc_ctx* ctx, size_t bytes, void** out) {
   std::lock_guard<std::mutex> lock(ctx->mu);
   auto it = ctx->free_blocks.find(b);
   void* p = nullptr;
-  if (ctx->capturing && !ctx->lazy) {
+  if (ctx->capturing && !ctx->rewrite) {
     // blocks this recording already owns come first; anything else it takes becomes its own.
-    // (Not while the recording lists its launches for rewriting: there every buffer stays a
+    // (Not while the recording's list is going to be rewritten: there every buffer stays a
     // buffer of its own until the recording ends, so that an operation can be moved next to its
-    // consumer without running into a block that was handed out again in between.)
+    // consumer without running into a block that was handed out again in between. The price is a
+    // footprint of the sum of all intermediates instead of their peak.)
     auto& parked = ctx->capturing->parked[b];
     if (!parked.empty()) {
       p = parked.back();
@@ -610,6 +693,7 @@ extern "C" int hc_capture_begin(hc_ctx* ctx) {
   ctx->capturing = new hc_graph();
   ctx->graphs.push_back(ctx->capturing);
   ctx->lazy = true;   // launches are listed, and enqueued on the capturing stream at hc_capture_end
+  ctx->rewrite = !ctx->sw.no_fusion;
   ctx->pending.clear();
   ctx->dead.clear();
   return HC_OK;
@@ -664,9 +748,9 @@ static int end_capture(hc_ctx* ctx, hc_graph** out) {
   if (ctx->lazy) {
     ctx->lazy = false;
     if (out) {
-      // HCHIP_NO_FUSION=1: the launches are enqueued as they were issued
-      if (!getenv("HCHIP_NO_FUSION")) fuse_recording(ctx);
-      if (getenv("HCHIP_RECORDING_LOG")) {   // the launches of the recording as they will be enqueued, to stderr
+      // HCHIP_NO_FUSION=1 when the capture began: the launches are enqueued as they were issued
+      if (ctx->rewrite) fuse_recording(ctx);
+      if (ctx->sw.recording_log) {   // the launches of the recording as they will be enqueued, to stderr
         size_t n = 0;
         for (const hc_pending& e : ctx->pending) {
           if (e.dropped || e.kind == hc_pending::FREE) continue;
@@ -677,12 +761,13 @@ static int end_capture(hc_ctx* ctx, hc_graph** out) {
         }
       }
       emitted = emit_recording_locked(ctx, ctx->pending);
-      if (getenv("HCHIP_GRAPH_AS_LAUNCHES"))
+      if (ctx->sw.graph_as_launches)
         for (hc_pending& e : ctx->pending)
           if (!e.dropped && e.kind != hc_pending::FREE) g->launches.push_back(e);
     }
     ctx->pending.clear();
   }
+  ctx->rewrite = false;
   ctx->capturing = nullptr;
   hipError_t e = hipStreamEndCapture(ctx->stream, &g->graph);
   if (emitted != HC_OK) {
@@ -942,10 +1027,6 @@ static size_t dtype_size(int dtype) {
 }
 
 static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
-static bool getenv_is(const char* name, const char* value) {
-  const char* v = getenv(name);
-  return v && strcmp(v, value) == 0;
-}
 
 // Build the joint broadcast descriptor for `nops` operands over one virtual shape:
 // drop size-1 axes, merge axes that are jointly mergeable (stride[d] == stride[d+1] *
@@ -1693,6 +1774,7 @@ __attribute__((visibility("hidden"))) int hc_reduce_in_scratch(hc_ctx* ctx, int 
                                                                size_t scratch_bytes) {
   REQUIRE(ctx, "hc_reduce_noalloc: null context");
   REQUIRE(scratch_base, "hc_reduce_noalloc: the scratch buffer of device %d was not set up", ctx->device);
+  OpNote note({in}, {out});   // (in a recording: the launches stay where they are, nothing is merged into them)
   Scratch scratch(ctx, scratch_base, scratch_bytes);
   return reduce_impl(ctx, scratch, op, dtype, in, out, outer, reduce, inner);
 }

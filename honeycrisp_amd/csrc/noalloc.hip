@@ -19,6 +19,10 @@ static __device__ __align__(256) unsigned char scratch[HC_NOALLOC_SCRATCH_BYTES]
 static const int kMaxDevices = 64;
 static void* g_scratch_ptr[kMaxDevices];
 static std::mutex g_setup_mu;
+// One per device, held for the whole of a call: a split reduction is two launches that meet in the
+// array, and with the lock both are enqueued back to back, so that calls from several threads
+// through one context run one after the other in its stream's order.
+static std::mutex g_call_mu[kMaxDevices];
 
 // hchip.cpp
 int hc_reduce_in_scratch(hc_ctx* ctx, int op, int dtype, const void* in, void* out, int64_t outer, int64_t reduce,
@@ -49,6 +53,7 @@ extern "C" int hc_reduce_noalloc(hc_ctx* ctx, int op, int dtype, const void* in,
   if (device < 0 || device >= kMaxDevices) return hc_set_error(HC_ERR_INVALID, "hc_reduce_noalloc: null context");
   // Every partial result is written by the first pass before the second pass reads it, so nothing
   // in the array has to start at zero.
+  std::lock_guard<std::mutex> lock(g_call_mu[device]);
   return hc_reduce_in_scratch(ctx, op, dtype, in, out, outer, reduce, inner, g_scratch_ptr[device],
                               (size_t)HC_NOALLOC_SCRATCH_BYTES);
 }

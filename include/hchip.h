@@ -96,6 +96,18 @@ void hc_shutdown(hc_ctx* ctx);
 const char* hc_last_error_string(void);
 int hc_get_device_info(hc_ctx* ctx, hc_device_info* out);
 
+/* Switches for measurements and tests. No counterpart in the reference (its backends are
+ * configured in code). A context takes the first value of each switch from the environment
+ * variable of the same name when it is created; this call changes one afterwards, safely while
+ * other threads launch through the context (an entry point works on a copy it takes when it
+ * starts). `value` NULL or "" restores the default; for the on/off switches anything but "0"
+ * means on. Names: HCHIP_GEMM_TILE (general | <BM>x<BN>), HCHIP_GEMM_KERNEL (dma | dma2 | mi16 |
+ * staged), HCHIP_GEMM_RING (4 | 2), HCHIP_GEMM_ONE (0), and the on/off switches
+ * HCHIP_GEMM_NO_PEEL, HCHIP_GEMM_NO_DIRECT, HCHIP_GEMM_NO_REPITCH, HCHIP_GEMM_BAND,
+ * HCHIP_NO_FUSION (looked at when a capture begins), HCHIP_RECORDING_LOG,
+ * HCHIP_GRAPH_AS_LAUNCHES (both looked at when a capture ends). HC_ERR_INVALID for any other name. */
+int hc_debug_set(hc_ctx* ctx, const char* name, const char* value);
+
 /* ---- memory: backs Tensor.Data (Tensor.swift:69-85) and DataAllocator
  * (Backend.swift:894-896; precedent BackendMPS.swift:468-556) ---- */
 
@@ -263,8 +275,10 @@ int hc_reduce(hc_ctx* ctx, int op, int dtype, const void* in, void* out, int64_t
  * HC_NOALLOC_SCRATCH_BYTES of device memory that the library holds on every device it runs on
  * until the process ends, so the call allocates and frees nothing, not even from the context's
  * pool. A reduction whose partials need more returns HC_ERR_TOO_LARGE (the message says how
- * much). All calls on one GPU share that array: calls that overlap there (two contexts, i.e.
- * two streams, on the same device) race; calls through one context are ordered by its stream. */
+ * much). All calls on one GPU share that array, which keeps the last call's contents. Calls
+ * through one context, from any number of threads, run one after the other: a per-device lock is
+ * held while a call enqueues its (up to two) launches, and the context's stream keeps that order.
+ * Calls that overlap on one GPU through two contexts (two streams) race on the array. */
 #define HC_NOALLOC_SCRATCH_BYTES (8u << 20)
 int hc_reduce_noalloc(hc_ctx* ctx, int op, int dtype, const void* in, void* out, int64_t outer,
                       int64_t reduce, int64_t inner);

@@ -30,3 +30,29 @@ def hip_backend():
     backend = HIPBackend()
     yield backend
     backend.sync()
+
+
+class _Switches:
+    """The library's measurement / test switches on the session's context (hc_debug_set), with
+    monkeypatch's method names; whatever a test sets is back at its default when the test ends."""
+
+    def __init__(self, backend):
+        self.backend, self.touched = backend, set()
+
+    def setenv(self, name, value):
+        self.backend.debugSet(name, value)
+        self.touched.add(name)
+
+    def delenv(self, name):
+        self.backend.debugSet(name, None)
+
+    def restore(self):
+        for name in self.touched:
+            self.backend.debugSet(name, None)
+
+
+@pytest.fixture
+def switch(hip_backend):
+    s = _Switches(hip_backend)
+    yield s
+    s.restore()

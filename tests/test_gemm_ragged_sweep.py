@@ -12,8 +12,6 @@ What is compared, per product:
     instead of being fetched and stored where they lie);
   * guard elements in front of and behind the output: nothing may be written outside C.
 """
-import os
-from contextlib import contextmanager
 from ctypes import c_void_p
 
 import numpy as np
@@ -28,20 +26,6 @@ pytestmark = pytest.mark.gpu
 F32, F16 = DType.float32, DType.float16
 TOL = {F32: 1e-4, F16: 1e-2}
 GUARD = 64  # elements on either side of C (a multiple of 16 bytes: C keeps its natural alignment)
-
-
-@contextmanager
-def env(**kv):
-    old = {k: os.environ.get(k) for k in kv}
-    os.environ.update(kv)
-    try:
-        yield
-    finally:
-        for k, v in old.items():
-            if v is None:
-                os.environ.pop(k, None)
-            else:
-                os.environ[k] = v
 
 
 def slabs(n, width=8):
@@ -100,7 +84,7 @@ class Product:
 
     def check_all(self, layouts, label):
         tol = TOL[self.dtype]
-        with env(HCHIP_GEMM_TILE="general"):
+        with self.hip.switches(HCHIP_GEMM_TILE="general"):
             general = self.run(False, False, False)
         self.check_against_oracle(general)
         for (transA, transB, transOut) in layouts:
@@ -108,10 +92,10 @@ class Product:
             c = self.run(transA, transB, transOut)
             self.check_against_oracle(c)
             assert_close_arrays(np.ascontiguousarray(c), general, tol, tol)
-            with env(HCHIP_GEMM_NO_PEEL="1"):
+            with self.hip.switches(HCHIP_GEMM_NO_PEEL="1"):
                 whole = self.run(transA, transB, transOut)
             assert_close_arrays(np.ascontiguousarray(c), np.ascontiguousarray(whole), tol, tol)
-            with env(HCHIP_GEMM_NO_DIRECT="1"):
+            with self.hip.switches(HCHIP_GEMM_NO_DIRECT="1"):
                 padded = self.run(transA, transB, transOut)
             assert_close_arrays(np.ascontiguousarray(c), np.ascontiguousarray(padded), tol, tol)
 

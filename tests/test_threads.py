@@ -61,3 +61,85 @@ def test_concurrent_op_chains_match_serial_runs(hip_backend):
     for th in pool:
         th.join()
     assert not failures, failures[:5]
+
+
+def test_a_switch_flipped_by_one_thread_while_others_launch(hip_backend):
+    """hc_debug_set from one thread while others run products through the same context: a call
+    works on the copy of the switches it took when it started, so every product is computed by one
+    consistent choice of kernel (forced tile or the host's own pick, all of which agree within the
+    fp16 tolerance and with the result the thread gets alone), and nothing crashes or deadlocks."""
+    rng = np.random.default_rng(5)
+    M, K, N = 512, 320, 384
+    a = hip_backend.upload((rng.standard_normal((M, K)) / K ** 0.5).astype(np.float16))
+    b = hip_backend.upload(rng.standard_normal((K, N)).astype(np.float16))
+    want = hip_backend.matmul(a, False, b, False, False, M, K, N, F16).onCPU().view(np.float16).astype(np.float32)
+    stop, failures = threading.Event(), []
+
+    def flipper():
+        values = ["64x64", "128x128", None, "general", "256x128", None]
+        i = 0
+        while not stop.is_set():
+            hip_backend.debugSet("HCHIP_GEMM_TILE", values[i % len(values)])
+            hip_backend.debugSet("HCHIP_GEMM_KERNEL", ["dma", None, "dma2"][i % 3])
+            i += 1
+        hip_backend.debugSet("HCHIP_GEMM_TILE", None)
+        hip_backend.debugSet("HCHIP_GEMM_KERNEL", None)
+
+    def worker(t):
+        try:
+            for _ in range(60):
+                got = hip_backend.matmul(a, False, b, False, False, M, K, N, F16).onCPU().view(np.float16).astype(np.float32)
+                if not np.allclose(got, want, rtol=1e-2, atol=1e-2):
+                    failures.append("thread %d: a product differs beyond the fp16 tolerance" % t)
+                    return
+        except Exception as e:
+            failures.append("thread %d: %r" % (t, e))
+
+    flip = threading.Thread(target=flipper)
+    pool = [threading.Thread(target=worker, args=(t,)) for t in range(4)]
+    flip.start()
+    for th in pool:
+        th.start()
+    for th in pool:
+        th.join()
+    stop.set()
+    flip.join()
+    assert not failures, failures[:5]
+    with pytest.raises(Exception):
+        hip_backend.debugSet("HCHIP_NO_SUCH_SWITCH", "1")
+
+
+def test_concurrent_reductions_through_the_fixed_scratch_array(hip_backend):
+    """hc_reduce_noalloc from several threads through one context: a split reduction is two launches
+    that meet in the library's one scratch array, and a per-device lock keeps the two together, so
+    each thread sees, bit for bit, what hc_reduce gives for its input."""
+    from ctypes import c_void_p
+    lib, ctx = hip_backend._lib, hip_backend._ctx
+    shapes = [(1, 3000, 512), (1, 2048, 1024), (2, 70000, 1), (1, 1500, 256)]
+    jobs = []
+    for t, (outer, reduce, inner) in enumerate(shapes):
+        rng = np.random.default_rng(100 + t)
+        x = hip_backend.upload(rng.standard_normal((outer, reduce, inner)).astype(np.float32))
+        want = hip_backend.allocate(outer * inner * 4)
+        hip_backend._check(lib.hc_reduce(ctx, 0, int(F32), c_void_p(x.ptr), c_void_p(want.ptr), outer, reduce, inner))
+        jobs.append((x, want.onCPU().copy(), outer, reduce, inner))
+    failures = []
+
+    def worker(t):
+        x, want, outer, reduce, inner = jobs[t]
+        try:
+            for _ in range(40):
+                out = hip_backend.allocate(outer * inner * 4)
+                hip_backend._check(lib.hc_reduce_noalloc(ctx, 0, int(F32), c_void_p(x.ptr), c_void_p(out.ptr), outer, reduce, inner))
+                if not np.array_equal(out.onCPU(), want):
+                    failures.append("thread %d: result differs from hc_reduce" % t)
+                    return
+        except Exception as e:
+            failures.append("thread %d: %r" % (t, e))
+
+    pool = [threading.Thread(target=worker, args=(t,)) for t in range(len(jobs))]
+    for th in pool:
+        th.start()
+    for th in pool:
+        th.join()
+    assert not failures, failures[:5]
