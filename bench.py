@@ -72,6 +72,9 @@ class MfmaProbe:
             fn = ctypes.c_void_p()
             backend._check(self.lib.hc_module_get_function(self.module, name, ctypes.byref(fn)))
             self.fn[shape] = fn
+        marker = ctypes.c_void_p()
+        backend._check(self.lib.hc_module_get_function(self.module, b"hc_bench_marker", ctypes.byref(marker)))
+        self.marker = marker
         self.cus = backend.deviceInfo()["compute_units"]
         self.out = backend.allocate(self.cus * 256 * 4)
 
@@ -85,8 +88,29 @@ class MfmaProbe:
         # per iteration and wave: 16 MFMAs of 32 x 32 x 16 (or 32 of 16 x 16 x 32)
         return 2.0 * 32 * 32 * 16 * 16.0 * iters * (self.cus * 256 / 64)
 
+    def mark(self, region):
+        """An empty kernel with a grid of `region` workgroups of 64 lanes: in a kernel trace of this
+        run, the launches between two markers of the same size are that region's."""
+        args = MfmaProbe.Args(None, None, 0, 0)
+        grid, block = (ctypes.c_uint32 * 3)(region, 1, 1), (ctypes.c_uint32 * 3)(64, 1, 1)
+        self.b._check(self.lib.hc_launch(self.b._ctx, self.marker, grid, block, 0, ctypes.byref(args),
+                                         ctypes.sizeof(args)))
+
     def close(self):
         self.lib.hc_module_unload(self.b._ctx, self.module)
+
+
+# Regions of a run, by marker size (see MfmaProbe.mark); written into the result as `trace_regions`.
+REGIONS = {}
+_PROBE = [None]
+
+
+def mark(backend, name):
+    """Launches the marker of the region called `name` (a number is assigned at first use)."""
+    if _PROBE[0] is None:
+        _PROBE[0] = MfmaProbe(backend)
+    region = REGIONS.setdefault(name, len(REGIONS) + 1)
+    _PROBE[0].mark(region)
 
 
 class Events:
@@ -118,7 +142,7 @@ SPINUP_MS = 200.0  # untimed load before the warmup steps, see headline()
 BATCH_SPINUP_MS = 60.0  # the same for the graph-replayed batches of short kernels
 
 
-def timed_launches(backend, events, fn, iters, warmup, batched=False):
+def timed_launches(backend, events, fn, iters, warmup, batched=False, region=None):
     """Average duration (ms) of fn() launches, each bracketed by events on the stream.
     batched=True (short kernels): the host cannot enqueue a microsecond-scale kernel as fast as
     the GPU runs it, so per-launch events would time the host. Instead `iters` launches are
@@ -127,9 +151,14 @@ def timed_launches(backend, events, fn, iters, warmup, batched=False):
     for _ in range(warmup):
         fn()
     if batched and GRAPH_TIMING:
-        with backend.capture() as cap:
-            for _ in range(iters):
-                fn()
+        # (recorded as issued: the rewrite of a recording would merge the batch's independent launches,
+        # e.g. products over the same input into one launch, and the figure would no longer be that of
+        # the kernel a single call runs)
+        # (every launch of the batch keeps its own output buffer, so that no launch writes into lines
+        # the launch before it left in the caches)
+        with backend.switches(HCHIP_NO_FUSION="1"):
+            with backend.capture() as cap:
+                keep = [fn() for _ in range(iters)]
         # the board's clocks settle only after some tens of milliseconds under load (see headline()):
         # replay untimed for a while first, so that a batch of microsecond kernels is measured at
         # the sustained clocks as well
@@ -139,6 +168,8 @@ def timed_launches(backend, events, fn, iters, warmup, batched=False):
                 cap.graph.launch()
             backend.sync()
         ms = []
+        if region:
+            mark(backend, region)
         for _ in range(5):
             a, b = events.new(), events.new()
             events.record(a)
@@ -148,15 +179,22 @@ def timed_launches(backend, events, fn, iters, warmup, batched=False):
             ms.append(events.elapsed_ms(a, b) / iters)
             events.free(a)
             events.free(b)
+        if region:
+            mark(backend, region)
         cap.graph.destroy()
+        del keep
         return float(np.mean(ms)), float(np.median(ms))
     pairs = []
+    if region:
+        mark(backend, region)
     for _ in range(iters):
         a, b = events.new(), events.new()
         events.record(a)
         fn()
         events.record(b)
         pairs.append((a, b))
+    if region:
+        mark(backend, region)
     backend.sync()
     ms = [events.elapsed_ms(a, b) for a, b in pairs]
     for a, b in pairs:
@@ -198,6 +236,8 @@ def headline(backend, steps, warmup):
     # stream (an event after every launch would cost the job 3 %). The average launch duration
     # over the timed region is a step's event-to-event time / 4, gaps between launches included.
     marks = [events.new() for _ in range(steps + 1)]
+    mark(backend, "headline_timed_steps")
+    backend.sync()
     t0 = time.perf_counter()
     events.record(marks[0])
     for i in range(steps):
@@ -206,6 +246,7 @@ def headline(backend, steps, warmup):
         events.record(marks[i + 1])
     backend.sync()
     t1 = time.perf_counter()
+    mark(backend, "headline_timed_steps")
     flops = 2.0 * n * n * n
     step_ms = [events.elapsed_ms(marks[i], marks[i + 1]) for i in range(steps)]
     launch_ms = float(np.mean(step_ms)) / 4
@@ -251,7 +292,8 @@ def headline(backend, steps, warmup):
     # power fits, and MFMA power depends on how many operand bits toggle, so this, not the
     # 2.4 GHz figure, is the rate a GEMM on this data could approach.
     probe_in = dev[("a", False)]
-    probe = MfmaProbe(backend)
+    mark(backend, "headline_mfma_only")
+    probe = _PROBE[0]
     probe_tflops = {}
     for shape, name in ((1, "16x16x32"), (0, "32x32x16")):
         for _ in range(200):
@@ -265,7 +307,7 @@ def headline(backend, steps, warmup):
         probe_tflops[name] = 200 * probe_flops / (events.elapsed_ms(e0, e1) * 1e-3) / 1e12
         events.free(e0)
         events.free(e1)
-    probe.close()
+    mark(backend, "headline_mfma_only")
     roofline["mfma_only_same_data"] = {
         "tflops": round(probe_tflops["16x16x32"], 1), "gemm_frac_of_it": round(achieved / probe_tflops["16x16x32"], 4),
         "tflops_32x32x16": round(probe_tflops["32x32x16"], 1),
@@ -401,6 +443,26 @@ def cpu_reference_ops(budget_s=15.0):
     return out
 
 
+def native_eager_transformer(dtype_name):
+    """Runs `HCMatrixBench --transformer` and returns its figures, or None if the program is not built."""
+    import subprocess
+    binary = os.path.join(ROOT, "honeycrisp_amd", "cpp", "HCMatrixBench")
+    if not os.path.exists(binary):
+        return None
+    proc = subprocess.run([binary, "--transformer", "--dtype", dtype_name, "--iters", "20"], stdout=subprocess.PIPE,
+                          stderr=subprocess.PIPE, text=True, timeout=120)
+    if proc.returncode != 0:
+        return {"error": (proc.stdout + proc.stderr)[-300:]}
+    r = dict(kv.split("=", 1) for kv in proc.stdout.strip().splitlines()[-1].split())
+    return {"ms": round(float(r["us"]) / 1e3, 3), "tokens_per_s": round(float(r["tokens_per_s"]), 1),
+            "tflops": round(100.9e9 / (float(r["us"]) * 1e-6) / 1e12, 2),
+            "ms_back_to_back": round(float(r["us_back_to_back"]) / 1e3, 3),
+            "tokens_per_s_back_to_back": round(float(r["tokens_per_s_back_to_back"]), 1),
+            "host_enqueue_ms": round(float(r["host_enqueue_us"]) / 1e3, 3),
+            "note": "eager, one backend call per op from a C++ host (HCMatrixBench --transformer, child process); "
+                    "back_to_back: passes enqueued without a wait in between"}
+
+
 def extra_workloads(backend, graph=True, only=("cfg1", "cfg2", "cfg3", "cfg4", "cfg5")):
     """The other configs of BASELINE.json: per-op launch durations from HIP events."""
     from honeycrisp_amd.descriptors import (BroadcastData, BroadcastStrides, DType, ElemwiseOp, NumericBinaryOp,
@@ -431,7 +493,7 @@ def extra_workloads(backend, graph=True, only=("cfg1", "cfg2", "cfg3", "cfg4", "
             x, y = sets[it[0] & 1]
             it[0] += 1
             return backend.matmul(x, False, y, False, False, 1024, 1024, 1024, F32)
-        ms, _ = timed_launches(backend, ev, gemm32, 50, 10, batched=True)
+        ms, _ = timed_launches(backend, ev, gemm32, 50, 10, batched=True, region="cfg1_f32_gemm_1024")
         report("cfg1_f32_gemm_1024", ms, flops=2.0 * 1024**3, peak_tflops=PEAK_F32_TFLOPS)
 
     def cfg2():
@@ -443,7 +505,7 @@ def extra_workloads(backend, graph=True, only=("cfg1", "cfg2", "cfg3", "cfg4", "
             fn = lambda: backend.matmul(a32, False, b32, tb, False, n, n, n, F32)
             for _ in range(30):     # (the clocks settle under load, see headline())
                 fn()
-            ms, _ = timed_launches(backend, ev, fn, 30, 10)
+            ms, _ = timed_launches(backend, ev, fn, 30, 10, region="cfg2_f32_gemm_4096_" + name)
             report("cfg2_f32_gemm_4096_" + name, ms, flops=2.0 * n**3, peak_tflops=PEAK_F32_TFLOPS)
         del a32, b32
         # the ragged sweep: fp16 NN products with M, N, K in {127, 1000, 4097}; total FLOPs over
@@ -458,7 +520,7 @@ def extra_workloads(backend, graph=True, only=("cfg1", "cfg2", "cfg3", "cfg4", "
                 for n in sizes:
                     b_dev = backend.upload(big[:kk * n])
                     fn = lambda: backend.matmul(a_dev, False, b_dev, False, False, m, kk, n, F16)
-                    ms, _ = timed_launches(backend, ev, fn, 5, 2, batched=True)
+                    ms, _ = timed_launches(backend, ev, fn, 5, 2, batched=True, region="cfg2_ragged_sweep_27_shapes")
                     total_flops += 2.0 * m * kk * n
                     total_ms += ms
                     if m == kk == n:
@@ -466,15 +528,34 @@ def extra_workloads(backend, graph=True, only=("cfg1", "cfg2", "cfg3", "cfg4", "
         report("cfg2_ragged_sweep_27_shapes", total_ms, flops=total_flops)
 
     def cfg3():
-        # config 3: attention-shaped batched GEMMs, fp16, batch 32
-        q, k, v = [backend.upload(np.random.default_rng(s).standard_normal((32, 512, 64)).astype(np.float16))
-                   for s in (4, 5, 6)]
-        scores = backend.batchedMatmul(32, q, False, k, True, False, 512, 64, 512, F16)
-        ms, _ = timed_launches(backend, ev, lambda: backend.batchedMatmul(32, q, False, k, True, False, 512, 64, 512, F16), 50, 10, batched=True)
+        # config 3: attention-shaped batched GEMMs, fp16, batch 32 (two sets of inputs alternate, so that no
+        # launch finds its operands in the caches because the launch before it used the same ones)
+        sets = []
+        for s0 in (4, 40):
+            q, k, v = [backend.upload(np.random.default_rng(s0 + i).standard_normal((32, 512, 64)).astype(np.float16))
+                       for i in range(3)]
+            sets.append((q, k, v, backend.batchedMatmul(32, q, False, k, True, False, 512, 64, 512, F16)))
+        it = [0]
+
+        def pick():
+            it[0] += 1
+            return sets[it[0] & 1]
+
+        def qk_t():
+            q, k, _, _ = pick()
+            return backend.batchedMatmul(32, q, False, k, True, False, 512, 64, 512, F16)
+
+        def scale():
+            return backend.binaryOp(pick()[3], 0.125, NumericBinaryOp.mul, F16, count=32 * 512 * 512)
+
+        def pv():
+            _, _, v, scores = pick()
+            return backend.batchedMatmul(32, scores, False, v, False, False, 512, 512, 64, F16)
+        ms, _ = timed_launches(backend, ev, qk_t, 50, 10, batched=True, region="cfg3_qk_t")
         report("cfg3_qk_t", ms, flops=32 * 2.0 * 512 * 64 * 512, nbytes=32 * (2 * 512 * 64 + 512 * 512) * 2)
-        ms, _ = timed_launches(backend, ev, lambda: backend.binaryOp(scores, 0.125, NumericBinaryOp.mul, F16, count=32 * 512 * 512), 50, 10, batched=True)
+        ms, _ = timed_launches(backend, ev, scale, 50, 10, batched=True, region="cfg3_scale")
         report("cfg3_scale", ms, nbytes=2 * 32 * 512 * 512 * 2)
-        ms, _ = timed_launches(backend, ev, lambda: backend.batchedMatmul(32, scores, False, v, False, False, 512, 512, 64, F16), 50, 10, batched=True)
+        ms, _ = timed_launches(backend, ev, pv, 50, 10, batched=True, region="cfg3_pv")
         report("cfg3_pv", ms, flops=32 * 2.0 * 512 * 512 * 64, nbytes=32 * (2 * 512 * 64 + 512 * 512) * 2)
 
     def cfg4():
@@ -485,28 +566,28 @@ def extra_workloads(backend, graph=True, only=("cfg1", "cfg2", "cfg3", "cfg4", "
         xs = BroadcastStrides([R, C], [C, 1])
         bs = BroadcastStrides([R, C], [0, 1])
         nb = R * C * 4
-        ms, _ = timed_launches(backend, ev, lambda: backend.binaryOp(BroadcastData(xs, x), BroadcastData(bs, bias), NumericBinaryOp.add, F32), 50, 10, batched=True)
+        ms, _ = timed_launches(backend, ev, lambda: backend.binaryOp(BroadcastData(xs, x), BroadcastData(bs, bias), NumericBinaryOp.add, F32), 50, 10, batched=True, region="cfg4_bias_add")
         report("cfg4_bias_add", ms, nbytes=2 * nb + C * 4)
         # plain copy of known size (identity broadcast): the calibration kernel for HBM byte counters
-        ms, _ = timed_launches(backend, ev, lambda: backend.broadcast(BroadcastData(xs, x), F32), 50, 10, batched=True)
+        ms, _ = timed_launches(backend, ev, lambda: backend.broadcast(BroadcastData(xs, x), F32), 50, 10, batched=True, region="copy_134MB_calibration")
         report("copy_134MB_calibration", ms, nbytes=2 * nb)
-        ms, _ = timed_launches(backend, ev, lambda: backend.elemwise(x, ElemwiseOp.geluApprox, None, R * C, F32), 50, 10, batched=True)
+        ms, _ = timed_launches(backend, ev, lambda: backend.elemwise(x, ElemwiseOp.geluApprox, None, R * C, F32), 50, 10, batched=True, region="cfg4_gelu")
         report("cfg4_gelu", ms, nbytes=2 * nb)
         dims = ReduceDims(R, C, 1)
-        ms, _ = timed_launches(backend, ev, lambda: backend.reduce(x, ReduceOp.sum, dims, F32), 50, 10, batched=True)
+        ms, _ = timed_launches(backend, ev, lambda: backend.reduce(x, ReduceOp.sum, dims, F32), 50, 10, batched=True, region="cfg4_sum_axis1")
         report("cfg4_sum_axis1", ms, nbytes=nb + R * 4)
-        ms, _ = timed_launches(backend, ev, lambda: backend.reduce(x, ReduceOp.argmax, dims, F32), 50, 10, batched=True)
+        ms, _ = timed_launches(backend, ev, lambda: backend.reduce(x, ReduceOp.argmax, dims, F32), 50, 10, batched=True, region="cfg4_argmax_axis1")
         report("cfg4_argmax_axis1", ms, nbytes=nb + R * 8)
 
         def max_axis1():  # Tensor.max(axis:) = argmax + gather (ReduceRepeat.swift:201-209)
             i = backend.reduce(x, ReduceOp.argmax, dims, F32)
             return backend.gather(x, ScatterGatherIndices([R, C], 1, BroadcastData(BroadcastStrides([R, 1], [1, 0]), i)), F32)
-        ms, _ = timed_launches(backend, ev, max_axis1, 50, 10, batched=True)
+        ms, _ = timed_launches(backend, ev, max_axis1, 50, 10, batched=True, region="cfg4_max_axis1")
         report("cfg4_max_axis1", ms, nbytes=nb + R * 8 + R * 8 + R * 4 + R * 4)
         table = backend.upload(np.random.default_rng(10).standard_normal((32000, 1024)).astype(np.float32))
         ids = backend.upload(np.random.default_rng(9).integers(0, 32000, size=(65536,)))
         emb = ScatterGatherIndices([32000, 1024], 0, BroadcastData(BroadcastStrides([65536, 1024], [1, 0]), ids))
-        ms, _ = timed_launches(backend, ev, lambda: backend.gather(table, emb, F32), 50, 10, batched=True)
+        ms, _ = timed_launches(backend, ev, lambda: backend.gather(table, emb, F32), 50, 10, batched=True, region="cfg4_embedding_gather")
         report("cfg4_embedding_gather", ms, nbytes=65536 * 8 + 2 * 65536 * 1024 * 4)
 
     def cfg5():
@@ -527,6 +608,12 @@ def extra_workloads(backend, graph=True, only=("cfg1", "cfg2", "cfg3", "cfg4", "
                 dt = (time.perf_counter() - t0) / 5
                 out[name] = {"ms": round(dt * 1e3, 3), "tokens_per_s": round(2048 / dt, 1),
                              "tflops": round(100.9e9 / dt / 1e12, 2)}
+                # The same pass issued eagerly from native host code (the C++ HCMatrixBench as a child process:
+                # same backend calls in the same order through the C++ mirror of the Backend interface), i.e.
+                # what a compiled host program pays per call instead of the Python mirror's interpreter time.
+                native = native_eager_transformer("f32" if dtype is F32 else "f16")
+                if native:
+                    out[name + "_native_host"] = native
                 if not graph:
                     continue
                 # the same forward pass recorded once and replayed as one graph launch: as recorded
@@ -577,6 +664,7 @@ def main():
     from honeycrisp_amd.backend import HIPBackend
     backend = HIPBackend(0)
     info = backend.deviceInfo()
+    _PROBE[0] = MfmaProbe(backend)
     parts = [x for x in args.only.split(",") if x] or ["headline", "cfg1", "cfg2", "cfg3", "cfg4", "cfg5"]
     unknown = [x for x in parts if x not in ("headline", "cfg1", "cfg2", "cfg3", "cfg4", "cfg5")]
     if unknown:
@@ -609,6 +697,9 @@ def main():
             result["extra"]["cpu_reference_path"] = cpu_reference_ops()
     else:
         result["cpu_baseline"] = None
+    result["trace_regions"] = {"kernel": "hc_bench_marker", "workgroups_of_marker": dict(REGIONS),
+                               "note": "in a kernel trace of this run, a region's launches lie between two launches "
+                                       "of the marker kernel with that many workgroups"}
     backend.sync()
     print(json.dumps(result))
 

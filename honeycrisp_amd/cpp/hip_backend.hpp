@@ -7,6 +7,7 @@
 
 #include <cstdint>
 #include <cstring>
+#include <functional>
 #include <memory>
 #include <stdexcept>
 #include <string>
@@ -73,10 +74,18 @@ class HIPBackend;
 class Buffer {
  public:
   Buffer(hc_ctx* ctx, void* ptr, size_t bytes) : ctx_(ctx), ptr_(ptr), bytes_(bytes) {}
+  // A buffer whose contents are produced on first use of its pointer (`fill` allocates and writes)
+  Buffer(hc_ctx* ctx, size_t bytes, std::function<void*()> fill) : ctx_(ctx), ptr_(nullptr), bytes_(bytes), fill_(std::move(fill)) {}
   ~Buffer() { hc_free(ctx_, ptr_); }
   Buffer(const Buffer&) = delete;
   Buffer& operator=(const Buffer&) = delete;
-  void* ptr() const { return ptr_; }
+  void* ptr() {
+    if (!ptr_ && fill_) {
+      ptr_ = fill_();
+      fill_ = nullptr;
+    }
+    return ptr_;
+  }
   size_t byteCount() const { return bytes_; }
   // set by axisPermutation: what this index vector permutes (lets gather copy directly)
   std::vector<int64_t> permutation, permutedShape;
@@ -85,6 +94,7 @@ class Buffer {
   hc_ctx* ctx_;
   void* ptr_;
   size_t bytes_;
+  std::function<void*()> fill_;
 };
 typedef std::shared_ptr<Buffer> Data;
 
@@ -222,7 +232,7 @@ class HIPBackend {
     Data out = allocate(s.indices.strides.count() * byteSize(dtype));
     // The gather of t / swap / move: indices from axisPermutation that run along the gathered axis
     // only. hc_permute moves the same bytes without reading 8 bytes of index per element.
-    const Buffer& idx = *s.indices.data;
+    Buffer& idx = *s.indices.data;
     if (!idx.permutedShape.empty() || idx.byteCount() == 8) {
       int64_t n = 1;
       for (int64_t d : idx.permutedShape) n *= d;
@@ -337,11 +347,19 @@ class HIPBackend {
     check(hc_fill(ctx_, (int)dtype, (float)value, (int64_t)value, out->ptr(), count));
     return out;
   }
+  // The int64 index vector is written on first use of its pointer: the usual consumer is the gather
+  // of t / swap / move, which runs as a direct copy from (permutation, shape) alone.
   Data axisPermutation(const std::vector<int64_t>& permutation, const std::vector<int64_t>& shape) {  // :803
     int64_t n = 1;
     for (int64_t d : shape) n *= d;
-    Data out = allocate((size_t)n * 8);
-    check(hc_axis_permutation(ctx_, permutation.data(), shape.data(), (int)shape.size(), out->ptr()));
+    hc_ctx* ctx = ctx_;
+    Data out = std::make_shared<Buffer>(ctx_, (size_t)n * 8, [=]() -> void* {
+      void* p = nullptr;
+      if (hc_malloc(ctx, (size_t)n * 8, &p) != HC_OK) throw BackendError(BackendError::allocationFailed, hc_last_error_string());
+      if (hc_axis_permutation(ctx, permutation.data(), shape.data(), (int)shape.size(), p) != HC_OK)
+        throw BackendError(BackendError::kernelFailed, hc_last_error_string());
+      return p;
+    });
     out->permutation = permutation;
     out->permutedShape = shape;
     return out;

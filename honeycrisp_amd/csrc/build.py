@@ -133,12 +133,17 @@ def build_all(verbose=True):
     if verbose:
         print("built", os.path.relpath(LIB_PATH, HERE), os.path.getsize(LIB_PATH), "bytes")
     if LIB_PATH == os.path.join(HERE, "libhchip.so"):
-        # C++ host mirror + HCMatrixBench (links the library just built)
+        # C++ host mirror + HCMatrixBench (links the library just built, and the Linux stand-in for
+        # Accelerate that its CPU leg calls the way the reference's CPUBackend calls Accelerate)
         cpp = os.path.join(os.path.dirname(HERE), "cpp")
         bench = os.path.join(cpp, "HCMatrixBench")
-        _run(["g++", "-O2", "-std=c++17", os.path.join(cpp, "HCMatrixBench.cpp"), "-o", bench,
+        shim = os.path.join(os.path.dirname(os.path.dirname(HERE)), "swift", "honeycrisp-linux", "Sources", "Accelerate",
+                            "accelerate_shim.c")
+        shim_obj = os.path.join(BUILD_DIR, "accelerate_shim.o")
+        _run(["gcc", "-O2", "-std=gnu11", "-fPIC", "-ffp-contract=off", "-fno-fast-math", "-c", shim, "-o", shim_obj])
+        _run(["g++", "-O2", "-std=c++17", "-ffp-contract=off", os.path.join(cpp, "HCMatrixBench.cpp"), shim_obj, "-o", bench,
               "-L" + HERE, "-lhchip", "-Wl,-rpath,$ORIGIN/../csrc",
-              "-L" + os.path.join(ROCM, "lib"), "-Wl,-rpath-link," + os.path.join(ROCM, "lib")])
+              "-L" + os.path.join(ROCM, "lib"), "-Wl,-rpath-link," + os.path.join(ROCM, "lib"), "-ldl", "-lm", "-lpthread"])
         if verbose:
             print("built", os.path.relpath(bench, HERE))
     return LIB_PATH

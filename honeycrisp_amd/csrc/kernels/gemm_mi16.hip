@@ -224,6 +224,11 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
   gemm_tile_of_block(p, blockIdx.x, tm, tn);
   const uint32_t m0 = tm * BM, n0 = tn * BN;
   const uint32_t batch = blockIdx.y;
+#ifdef HC_MI16_TIMESTAMPS
+  // (measurement build: when a workgroup starts, leaves its K loop and ends, on the 100 MHz clock)
+  const uint64_t ts_start = __builtin_amdgcn_s_memrealtime();
+  const uint64_t tc_start = __builtin_amdgcn_s_memtime();
+#endif
 #ifdef HC_GEMM_MERGED
   // (the second build of this file, kernels *_m: what a recording's rewrite needs)
   uint32_t batch_hi = batch, batch_lo = 0;
@@ -381,6 +386,9 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
   }
   if (j < nk) step(Tail{}, lds0, lds1, j);
   wait_dma<0>();  // no LDS write of this workgroup may be in flight when it ends
+#ifdef HC_MI16_TIMESTAMPS
+  const uint64_t ts_loop = __builtin_amdgcn_s_memrealtime();
+#endif
   // The compiler does not know that the assembly statements are MFMAs, so it would not keep the
   // epilogue's accumulator reads the required distance from the last of them: do it by hand.
   asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
@@ -469,6 +477,19 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
 #endif
       asm volatile("" ::: "memory");
     }
+#ifdef HC_MI16_TIMESTAMPS
+  if (threadIdx.x == 0) {  // over the first 32 bytes of the tile's first row (the result is not used)
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    uint64_t* t = (uint64_t*)(C + (size_t)m0 * p.c_rs + n0);
+    uint32_t hw_id, xcc_id;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hw_id));
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc_id));
+    t[0] = ts_start;
+    t[1] = ts_loop;
+    t[2] = __builtin_amdgcn_s_memrealtime();
+    t[3] = ((__builtin_amdgcn_s_memtime() - tc_start) << 16) | ((uint64_t)(xcc_id & 0xf) << 12) | (hw_id & 0xfff);
+  }
+#endif
 #ifdef HC_GEMM_MERGED
   };
   const bool ep_matrix = p.ep_kind[0] == HCK_EP_ADD_MATRIX || p.ep_kind[1] == HCK_EP_ADD_MATRIX || p.ep_kind[2] == HCK_EP_ADD_MATRIX;
@@ -506,6 +527,7 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
   DEF_MI16(BM, BN, m, DMA_MN, k, DMA_K)                                                               \
   DEF_MI16(BM, BN, m, DMA_MN, n, DMA_MN)
 DEF_MI16_TILE(256, 256)
+#ifndef HC_MI16_ONLY_256  // (a quick build with the largest tile only, for kernel experiments)
 DEF_MI16_TILE(256, 192)
 DEF_MI16_TILE(192, 256)
 DEF_MI16_TILE(192, 192)
@@ -514,3 +536,4 @@ DEF_MI16_TILE(128, 128)
 DEF_MI16_TILE(256, 64)
 DEF_MI16_TILE(128, 64)
 DEF_MI16_TILE(64, 64)
+#endif
