@@ -142,7 +142,7 @@ SPINUP_MS = 200.0  # untimed load before the warmup steps, see headline()
 BATCH_SPINUP_MS = 60.0  # the same for the graph-replayed batches of short kernels
 
 
-def timed_launches(backend, events, fn, iters, warmup, batched=False, region=None):
+def timed_launches(backend, events, fn, iters, warmup, batched=False, region=None, fusion=False):
     """Average duration (ms) of fn() launches, each bracketed by events on the stream.
     batched=True (short kernels): the host cannot enqueue a microsecond-scale kernel as fast as
     the GPU runs it, so per-launch events would time the host. Instead `iters` launches are
@@ -156,7 +156,8 @@ def timed_launches(backend, events, fn, iters, warmup, batched=False, region=Non
         # the kernel a single call runs)
         # (every launch of the batch keeps its own output buffer, so that no launch writes into lines
         # the launch before it left in the caches)
-        with backend.switches(HCHIP_NO_FUSION="1"):
+        # (fusion=True: a chain of calls that a recording is meant to merge, measured as recorded)
+        with backend.switches(**({} if fusion else {"HCHIP_NO_FUSION": "1"})):
             with backend.capture() as cap:
                 keep = [fn() for _ in range(iters)]
         # the board's clocks settle only after some tens of milliseconds under load (see headline()):
@@ -557,6 +558,23 @@ def extra_workloads(backend, graph=True, only=("cfg1", "cfg2", "cfg3", "cfg4", "
         report("cfg3_scale", ms, nbytes=2 * 32 * 512 * 512 * 2)
         ms, _ = timed_launches(backend, ev, pv, 50, 10, batched=True, region="cfg3_pv")
         report("cfg3_pv", ms, flops=32 * 2.0 * 512 * 512 * 64, nbytes=32 * (2 * 512 * 64 + 512 * 512) * 2)
+
+        # The whole chain q k^T -> * 1/8 -> softmax -> x v as a Honeycrisp program writes it (Softmax.swift:64-66:
+        # logSoftmax, then exp): call by call (five launches), and as a recording merges it (one attention
+        # kernel with the same bits). Algorithmic bytes of the chain: q, k, v in, the context out.
+        from honeycrisp_amd.tensor import Tensor
+
+        def chain():
+            q, k, v, _ = pick()
+            with backend.use():
+                tq, tk, tv = (Tensor(dataHandle=d, shape=[32, 512, 64], dtype=F16) for d in (q, k, v))
+                p = (Tensor.batchedMatmul(tq, False, tk, True, False) * 0.125).softmax()
+                return Tensor.batchedMatmul(p, False, tv, False, False)
+        chain_flops, chain_bytes = 2 * 32 * 2.0 * 512 * 64 * 512, 4 * 32 * 512 * 64 * 2
+        ms, _ = timed_launches(backend, ev, chain, 20, 5, batched=True, region="cfg3_chain_five_launches")
+        report("cfg3_chain_five_launches", ms, flops=chain_flops, nbytes=chain_bytes)
+        ms, _ = timed_launches(backend, ev, chain, 20, 5, batched=True, region="cfg3_chain_recorded_one_kernel", fusion=True)
+        report("cfg3_chain_recorded_one_kernel", ms, flops=chain_flops, nbytes=chain_bytes)
 
     def cfg4():
         # config 4: bandwidth-bound ops at [8192, 4096] fp32

@@ -22,6 +22,7 @@ KERNELS = [
     ("reduce", "reduce.hip", ["-ffp-contract=off"]),
     ("gather", "gather.hip", []),
     ("scan", "scan.hip", ["-ffp-contract=off"]),
+    ("attention", "attention.hip", ["-ffp-contract=off"]),
     ("gemm", "gemm.hip", []),
     ("gemm_f16_fast", "gemm_f16_fast.hip", []),
     # (their epilogues can apply a bias / residual / GELU with the element-wise kernels' arithmetic)

@@ -17,6 +17,7 @@
     EMBED hc_image_reduce, "reduce.hsaco"
     EMBED hc_image_gather, "gather.hsaco"
     EMBED hc_image_scan, "scan.hsaco"
+    EMBED hc_image_attention, "attention.hsaco"
     EMBED hc_image_gemm, "gemm.hsaco"
     EMBED hc_image_gemm_f16_fast, "gemm_f16_fast.hsaco"
     EMBED hc_image_gemm_dma, "gemm_dma.hsaco"

@@ -28,6 +28,7 @@ extern const unsigned char hc_image_elementwise[], hc_image_elementwise_end[];
 extern const unsigned char hc_image_reduce[], hc_image_reduce_end[];
 extern const unsigned char hc_image_gather[], hc_image_gather_end[];
 extern const unsigned char hc_image_scan[], hc_image_scan_end[];
+extern const unsigned char hc_image_attention[], hc_image_attention_end[];
 extern const unsigned char hc_image_gemm[], hc_image_gemm_end[];
 extern const unsigned char hc_image_gemm_f16_fast[], hc_image_gemm_f16_fast_end[];
 extern const unsigned char hc_image_gemm_dma[], hc_image_gemm_dma_end[];
@@ -74,7 +75,7 @@ struct hc_pending {
   std::vector<const void*> reads;
   std::vector<const void*> writes;
   // what the rewrite needs to know about the operations it can merge
-  enum Tag { NONE, GEMM, PRODUCT, BMM, PERMUTE, ADD, GELU, CAST, NORMALIZE, LOG_SOFTMAX, SCALAR, MUL_ADD, EXP } tag = NONE;
+  enum Tag { NONE, GEMM, PRODUCT, BMM, PERMUTE, ADD, GELU, CAST, NORMALIZE, LOG_SOFTMAX, SCALAR, MUL_ADD, EXP, SOFTMAX_CHAIN } tag = NONE;
   int dtype = 0;                       // element type of the output
   int src_dtype = 0;                   // CAST: element type of the input
   uint64_t rows = 0, cols = 0;         // GEMM: M, N; ADD: leading x trailing extent; GELU, CAST: 1 x count
@@ -86,7 +87,9 @@ struct hc_pending {
   // SCALAR: out = in0 (op) sf over `cols` elements, op = HC_ADD or HC_MUL as the kernel computes it
   // MUL_ADD: out = in0 * in1 + in2 with in0 dense [rows, cols] and in1, in2 rows of `cols` elements
   // EXP: ElemwiseOp.exp over `cols` elements of in0
-  // BMM: a batched product in one launch of a direct-to-LDS kernel (operands in the argument struct)
+  // BMM: a batched product in one launch of a direct-to-LDS kernel (operands in the argument struct);
+  //   stays a BMM when the rewrite has made it read or write through a swap of the batch axes
+  // SOFTMAX_CHAIN: the merged [scale] [mask] logSoftmax [exp] row kernel (rows x cols, lanes; args hck_softmax_chain_args)
   // PERMUTE (row form): in0 -> out; axis d of the dense output has extent pext[d] and lies at
   // stride pstr[d] (elements) in the source, the last axis contiguous in both
   int pn = 0;
@@ -172,6 +175,7 @@ struct hc_ctx {
   hc_graph* capturing = nullptr;                      // the recording in progress, if any
   std::unordered_map<void*, hc_graph*> block_owner;   // blocks reserved for a graph
   std::vector<hc_graph*> graphs;
+  std::vector<hc_graph*> doomed;   // hc_graph_destroy during a capture: destroyed when the capture ends
   // Small host-to-device uploads go through pinned memory so that they need no host-side wait:
   // two halves used in turn, each guarded by an event recorded when the upload path leaves it.
   char* stage = nullptr;
@@ -288,6 +292,7 @@ extern "C" int hc_init(int device, hc_ctx** out) {
   if (s == HC_OK) s = load_image(ctx, hc_image_reduce, hc_image_reduce_end, "reduce");
   if (s == HC_OK) s = load_image(ctx, hc_image_gather, hc_image_gather_end, "gather");
   if (s == HC_OK) s = load_image(ctx, hc_image_scan, hc_image_scan_end, "scan");
+  if (s == HC_OK) s = load_image(ctx, hc_image_attention, hc_image_attention_end, "attention");
   if (s == HC_OK) s = load_image(ctx, hc_image_gemm, hc_image_gemm_end, "gemm");
   if (s == HC_OK) s = load_image(ctx, hc_image_gemm_f16_fast, hc_image_gemm_f16_fast_end, "gemm_f16_fast");
   if (s == HC_OK) s = load_image(ctx, hc_image_gemm_dma, hc_image_gemm_dma_end, "gemm_dma");
@@ -740,9 +745,20 @@ static void release_graph_blocks_locked(hc_ctx* ctx, hc_graph* g) {
     }
 }
 
+static int destroy_graph_locked(hc_ctx* ctx, hc_graph* graph);
+static int end_capture_locked(hc_ctx* ctx, hc_graph** out);
+
 static int end_capture(hc_ctx* ctx, hc_graph** out) {
   std::lock_guard<std::mutex> lock(ctx->mu);
   REQUIRE(ctx->capturing, "hc_capture_end: no capture in progress");
+  const int status = end_capture_locked(ctx, out);
+  std::vector<hc_graph*> doomed;
+  doomed.swap(ctx->doomed);
+  for (hc_graph* g : doomed) (void)destroy_graph_locked(ctx, g);
+  return status;
+}
+
+static int end_capture_locked(hc_ctx* ctx, hc_graph** out) {
   hc_graph* g = ctx->capturing;
   int emitted = HC_OK;
   if (ctx->lazy) {
@@ -831,11 +847,8 @@ extern "C" int hc_graph_node_count(hc_graph* graph, size_t* out) {
   return HC_OK;
 }
 
-extern "C" int hc_graph_destroy(hc_ctx* ctx, hc_graph* graph) {
-  REQUIRE(ctx, "hc_graph_destroy: null context");
-  if (!graph) return HC_OK;
-  std::lock_guard<std::mutex> lock(ctx->mu);
-  REQUIRE(graph != ctx->capturing, "hc_graph_destroy: this recording is still in progress");
+// Caller holds the lock; no capture in progress.
+static int destroy_graph_locked(hc_ctx* ctx, hc_graph* graph) {
   // replays already enqueued still use the parked blocks: let them finish first
   HIP_TRY(hipStreamSynchronize(ctx->stream));
   if (graph->exec) (void)hipGraphExecDestroy(graph->exec);
@@ -843,6 +856,20 @@ extern "C" int hc_graph_destroy(hc_ctx* ctx, hc_graph* graph) {
   release_graph_blocks_locked(ctx, graph);
   delete graph;
   return HC_OK;
+}
+
+extern "C" int hc_graph_destroy(hc_ctx* ctx, hc_graph* graph) {
+  REQUIRE(ctx, "hc_graph_destroy: null context");
+  if (!graph) return HC_OK;
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  REQUIRE(graph != ctx->capturing, "hc_graph_destroy: this recording is still in progress");
+  if (ctx->capturing) {
+    // (waiting for the stream would invalidate the capture in progress: an owner that lets go of an
+    // older graph in the middle of a recording gets its destruction when the recording ends)
+    ctx->doomed.push_back(graph);
+    return HC_OK;
+  }
+  return destroy_graph_locked(ctx, graph);
 }
 
 // ------------------------------------------------------------------ rewriting a recording

@@ -132,6 +132,28 @@ typedef struct {
 #define HCK_SM_MASK 2u
 #define HCK_SM_EXP 4u
 
+/* One attention head per workgroup column: out = softmax-chain(q k^T) v with 64-wide heads, fp16.
+ * q, out: [T, 64] rows at row strides q_rs / o_rs; k: [T, 64] at k_rs; v: [T, 64] at v_rs (all
+ * contiguous along the 64). Slice z of an operand starts at z * bs, or with bdiv != 0 at
+ * (z / bdiv) * bs + (z % bdiv) * bs2 (heads that are an inner axis of [B, T, H, 64]). The chain
+ * between the two products is that of hck_softmax_chain_args (flags, scale, mask, mask_rows: row
+ * r of all batch * T score rows takes mask row r % mask_rows). */
+typedef struct {
+  const void* q;
+  const void* k;
+  const void* v;
+  const void* mask;
+  void* out;
+  uint32_t T;      /* queries = keys per head, a multiple of 64 */
+  uint32_t bdiv;
+  uint32_t q_rs, k_rs, v_rs, o_rs;
+  uint64_t q_bs, q_bs2, k_bs, k_bs2, v_bs, v_bs2, o_bs, o_bs2;
+  uint32_t mask_rows;
+  uint32_t flags; /* HCK_SM_* */
+  float scale;
+  uint32_t pad;
+} hck_attention_args;
+
 /* Column reduction ([outer, reduce, inner], inner > 1) in up to two passes: the reduce axis is
  * cut into `splits` ranges of `chunk` rows; with splits > 1 each range leaves a partial value
  * (and, for arg-reductions, its index) per column, combined by a second kernel. */

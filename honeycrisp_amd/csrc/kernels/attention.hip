@@ -1,0 +1,246 @@
+// One kernel for the attention of a head: scores = q k^T, the softmax chain over every row of
+// scores ([* scale] [+ mask] logSoftmax [exp]), out = probabilities x v; fp16, 64-wide heads. It
+// exists for recordings: the rewrite of a recording replaces the three launches (batched product,
+// row kernel, batched product) by this one when the scores and the probabilities have no other
+// reader, and a replay must return the bits of the three launches. So this kernel does their
+// arithmetic, not a rearranged one:
+//   * both products accumulate in fp32 with v_mfma_f32_32x32x16_f16, the second operand of the
+//     product first, k ascending in steps of 16, as every tiled 32x32x16 kernel of the library does
+//     (gemm_dma.hip, gemm_dma2.hip), and round once to fp16;
+//   * the scores are rounded to fp16 and laid out in LDS as a [64, T] tile; a team of LANES lanes
+//     then takes a row exactly as the row kernel takes it from memory (RowRegs: lane l owns the
+//     16-byte vectors l, l + LANES, ...; the same order of partial sums, the same shuffles, the same
+//     exponential), writes the probabilities back in fp16, and the second product reads them.
+// The softmax is over the whole row (true maximum and sum, as the reference computes it,
+// BackendCPU.swift:1000-1038), not a running one, so the score tile must hold whole rows: T <= TMAX.
+//
+// A workgroup (4 waves) owns 64 query rows of one head. grid.x = T / 64, grid.y = heads.
+//   phase 0: q tile and all keys into LDS (rows of 128 bytes, 16-byte chunk c of row r in slot
+//            c ^ (r & 7), so that the MFMA operand reads of 32 rows hit different banks); the
+//            values are fetched into registers meanwhile
+//   phase 1: wave w multiplies the q tile with keys 128 p + 32 w .. + 31 (p = 0, 1, ...): two
+//            32 x 32 accumulators, four MFMAs each; scores to LDS
+//   phase 2: row teams run the chain in place; the values go to LDS over the keys
+//   phase 3: wave w owns a 32 x 32 tile of the [64, 64] output, k over the T keys; the values are
+//            stored [key][64] and read with the transposing LDS read, like an operand that is
+//            contiguous along n in the tiled GEMM kernels
+#include "row_teams.hip.h"
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef uint32_t Chunk __attribute__((ext_vector_type(4)));
+#define LDS_AS __attribute__((address_space(3)))
+
+template <int TMAX, int LANES> __device__ __forceinline__ void attention_impl(const hck_attention_args& p) {
+  constexpr uint32_t BQ = 64;
+  constexpr uint32_t SP = TMAX * 2 + 16;  // bytes per row of the score tile (rows stay 16-byte aligned)
+  constexpr uint32_t VP = 144;            // bytes per key row of the values (128 + a shift of the banks)
+  constexpr int KV_CHUNKS = TMAX * 8 / HCK_BLOCK;  // 16-byte chunks of k (or v) per lane
+  __shared__ __attribute__((aligned(16))) char q_lds[BQ * 128];
+  __shared__ __attribute__((aligned(16))) char kv_lds[TMAX * VP];
+  __shared__ __attribute__((aligned(16))) char s_lds[BQ * SP];
+
+  const uint32_t T = p.T, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const uint32_t z = blockIdx.y, m0 = blockIdx.x * BQ;
+  uint32_t zh = z, zl = 0;
+  if (p.bdiv != 0) {
+    zh = z / p.bdiv;
+    zl = z - zh * p.bdiv;
+  }
+  const half_t* Q = (const half_t*)p.q + zh * p.q_bs + zl * p.q_bs2 + (size_t)m0 * p.q_rs;
+  const half_t* K = (const half_t*)p.k + zh * p.k_bs + zl * p.k_bs2;
+  const half_t* V = (const half_t*)p.v + zh * p.v_bs + zl * p.v_bs2;
+  half_t* O = (half_t*)p.out + zh * p.o_bs + zl * p.o_bs2 + (size_t)m0 * p.o_rs;
+
+#ifdef HC_ATTENTION_TIMESTAMPS
+  uint64_t ts[6];
+  ts[0] = __builtin_amdgcn_s_memrealtime();
+#define HC_TS(i) ts[i] = __builtin_amdgcn_s_memrealtime()
+#else
+#define HC_TS(i)
+#endif
+  // ---- phase 0
+  Chunk vreg[KV_CHUNKS];
+#pragma unroll
+  for (int i = 0; i < KV_CHUNKS; i++) {
+    const uint32_t piece = i * HCK_BLOCK + tid, r = piece >> 3, c = piece & 7;
+    if (r < T) vreg[i] = *reinterpret_cast<const Chunk*>(V + (size_t)r * p.v_rs + c * 8);
+  }
+#pragma unroll
+  for (int i = 0; i < (int)(BQ * 8 / HCK_BLOCK); i++) {
+    const uint32_t piece = i * HCK_BLOCK + tid, r = piece >> 3, c = piece & 7;
+    *reinterpret_cast<Chunk*>(q_lds + r * 128 + ((c ^ (r & 7)) * 16)) = *reinterpret_cast<const Chunk*>(Q + (size_t)r * p.q_rs + c * 8);
+  }
+#pragma unroll
+  for (int i = 0; i < KV_CHUNKS; i++) {
+    const uint32_t piece = i * HCK_BLOCK + tid, r = piece >> 3, c = piece & 7;
+    if (r < T)
+      *reinterpret_cast<Chunk*>(kv_lds + r * 128 + ((c ^ (r & 7)) * 16)) = *reinterpret_cast<const Chunk*>(K + (size_t)r * p.k_rs + c * 8);
+  }
+  __syncthreads();
+  HC_TS(1);
+
+  // ---- phase 1: scores
+  const uint32_t l32 = lane & 31, lgrp = lane >> 5;
+  Chunk qf[2][4];  // the q tile's operands: rows 32 mt + l32, k = 16 s + 8 lgrp .. + 7
+#pragma unroll
+  for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+      const uint32_t r = mt * 32 + l32;
+      qf[mt][s] = *reinterpret_cast<const Chunk*>(q_lds + r * 128 + (((2 * s + lgrp) ^ (r & 7)) * 16));
+    }
+  for (uint32_t nb = wave * 32; nb < T; nb += 128) {
+    floatx16 acc[2];
+#pragma unroll
+    for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+      for (int e = 0; e < 16; e++) acc[mt][e] = 0.0f;
+    const uint32_t r = nb + l32;
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+      const Chunk kf = *reinterpret_cast<const Chunk*>(kv_lds + r * 128 + (((2 * s + lgrp) ^ (r & 7)) * 16));
+#pragma unroll
+      for (int mt = 0; mt < 2; mt++)
+        acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, kf), __builtin_bit_cast(half8, qf[mt][s]), acc[mt], 0, 0, 0);
+    }
+    // lane: query row 32 mt + l32, keys nb + 8 g + 4 lgrp .. + 3 in registers 4 g .. 4 g + 3
+#pragma unroll
+    for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        half4v h;
+#pragma unroll
+        for (int e = 0; e < 4; e++) h[e] = narrow<half_t>(acc[mt][4 * g + e]);
+        *reinterpret_cast<half4v*>(s_lds + (mt * 32 + l32) * SP + (nb + 8 * g + 4 * lgrp) * 2) = h;
+      }
+  }
+  __syncthreads();  // scores complete; nobody reads the keys any more
+  HC_TS(2);
+
+  // the values over the keys: [key][64 halfs], rows of VP bytes
+#pragma unroll
+  for (int i = 0; i < KV_CHUNKS; i++) {
+    const uint32_t piece = i * HCK_BLOCK + tid, r = piece >> 3, c = piece & 7;
+    if (r < T) *reinterpret_cast<Chunk*>(kv_lds + r * VP + c * 16) = vreg[i];
+  }
+
+  // ---- phase 2: the chain over the rows of the score tile, in place (softmax_chain_rows_impl of
+  // the row kernels, with the row in LDS instead of memory). A team works on R rows at a time (8, or all it has), stage
+  // by stage, so that the latencies of one row's shuffles and exponentials hide behind the others'
+  // (there is one wave per SIMD here, not the many of the row kernel); per row the arithmetic and its
+  // order are the row kernel's.
+  {
+    // (vectors per lane: what rows of TMAX elements need, at most the row kernel's four)
+    constexpr int NCH = (TMAX + LANES * 8 - 1) / (LANES * 8);
+    static_assert(NCH <= 4, "rows of TMAX elements fit the team's registers");
+    typedef RowRegs<half_t, LANES, NCH> Row;
+    constexpr int VEC = Row::VEC, CHUNKS = Row::CHUNKS;
+    constexpr uint32_t TEAMS = HCK_BLOCK / LANES;       // rows the workgroup's teams take in one go
+    constexpr int R = TEAMS * 8 <= BQ ? 8 : BQ / TEAMS;  // 8 rows per team at a time (2 with 32 teams)
+    static_assert(BQ % (TEAMS * R) == 0, "the teams' passes cover the tile exactly");
+    const uint32_t tl = tid % LANES, team = tid / LANES;
+    const bool then_exp = (p.flags & HCK_SM_EXP) != 0;
+    for (uint32_t first = team * R; first < BQ; first += TEAMS * R) {
+      Row r[R];
+#pragma unroll
+      for (int j = 0; j < R; j++) r[j].load((const half_t*)(s_lds + (first + j) * SP), T, tl);
+      if (p.flags & HCK_SM_SCALE) {
+        const float s = p.scale;
+#pragma unroll
+        for (int j = 0; j < R; j++)
+#pragma unroll
+          for (int c = 0; c < CHUNKS; c++)
+#pragma unroll
+            for (int i = 0; i < VEC; i++) r[j].v[c][i] = narrow<half_t>((float)r[j].v[c][i] * s);
+      }
+      if (p.flags & HCK_SM_MASK) {
+        Row m[R];
+#pragma unroll
+        for (int j = 0; j < R; j++) {
+          const uint64_t grow = (uint64_t)z * T + m0 + first + j;  // this row among all score rows
+          m[j].load((const half_t*)p.mask + (size_t)(grow % p.mask_rows) * T, T, tl);
+        }
+#pragma unroll
+        for (int j = 0; j < R; j++)
+#pragma unroll
+          for (int c = 0; c < CHUNKS; c++)
+            if ((tl + LANES * c) * VEC < T) {
+#pragma unroll
+              for (int i = 0; i < VEC; i++) r[j].v[c][i] = narrow<half_t>((float)r[j].v[c][i] + (float)m[j].v[c][i]);
+            }
+      }
+      float mx[R], sum[R];
+#pragma unroll
+      for (int j = 0; j < R; j++) {
+        mx[j] = -INFINITY;
+        r[j].each(T, tl, [&](float x) { if (x > mx[j]) mx[j] = x; });
+      }
+#pragma unroll
+      for (int j = 0; j < R; j++) mx[j] = team_reduce<LANES>(mx[j], MaxOp());
+#pragma unroll
+      for (int j = 0; j < R; j++) {
+        sum[j] = 0.0f;
+        r[j].each(T, tl, [&](float x) { sum[j] += exp_in<half_t>(x - mx[j]); });
+      }
+#pragma unroll
+      for (int j = 0; j < R; j++) sum[j] = team_reduce<LANES>(sum[j], SumOp());
+#pragma unroll
+      for (int j = 0; j < R; j++) {
+        const float log_sum = logf(sum[j]) + mx[j];
+        r[j].store((half_t*)(s_lds + (first + j) * SP), T, tl, [&](float x) {
+          const float ls = x - log_sum;
+          if (!then_exp) return ls;
+          const float stored = (float)narrow<half_t>(ls);
+          return exp_hw(stored) * 1.0f;
+        });
+      }
+    }
+  }
+  __syncthreads();
+  HC_TS(3);
+
+  // ---- phase 3: out tile (mt, nt) of wave w; operands: probabilities rows 32 mt + l32 (k-contiguous),
+  // values columns 32 nt + l32 through the transposing read (a group of 16 lanes: k-rows
+  // 8 (grp / 2) + 4 h + r / 4, columns 16 (grp % 2) + 4 (r % 4) .. + 3; lane i receives column i)
+  {
+    const uint32_t mt = wave >> 1, nt = wave & 1;
+    const uint32_t r16 = lane & 15, grp = lane >> 4;
+    floatx16 acc;
+#pragma unroll
+    for (int e = 0; e < 16; e++) acc[e] = 0.0f;
+    const char* prow = s_lds + (mt * 32 + l32) * SP + lgrp * 16;
+    const char* vcol = kv_lds + (8 * (grp >> 1) + (r16 >> 2)) * VP + (nt * 32 + 16 * (grp & 1) + 4 * (r16 & 3)) * 2;
+    for (uint32_t k0 = 0; k0 < T; k0 += 16) {
+      const Chunk pf = *reinterpret_cast<const Chunk*>(prow + k0 * 2);
+      typedef short short4v __attribute__((ext_vector_type(4)));
+      typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+      const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS short4v*)(vcol + k0 * VP)));
+      const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS short4v*)(vcol + (k0 + 4) * VP)));
+      const Chunk vf = {lo[0], lo[1], hi[0], hi[1]};
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, vf), __builtin_bit_cast(half8, pf), acc, 0, 0, 0);
+    }
+    // lane: query row 32 mt + l32, columns 32 nt + 8 g + 4 lgrp .. + 3
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+      half4v h;
+#pragma unroll
+      for (int e = 0; e < 4; e++) h[e] = narrow<half_t>(acc[4 * g + e]);
+      *reinterpret_cast<half4v*>(O + (size_t)(mt * 32 + l32) * p.o_rs + nt * 32 + 8 * g + 4 * lgrp) = h;
+    }
+  }
+#ifdef HC_ATTENTION_TIMESTAMPS
+  HC_TS(4);
+  if (tid == 0) {   // (measurement build: over the first bytes of the tile's first row)
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    ts[5] = __builtin_amdgcn_s_memrealtime();
+    for (int i = 0; i < 6; i++) ((uint64_t*)O)[i] = ts[i];
+  }
+#endif
+}
+
+// (rows of up to 256 halfs are taken by teams of 8 lanes, longer ones by a wave: what hc_log_softmax
+// picks for rows of these lengths)
+HC_KERNEL void hc_attention_f16_t256(hck_attention_args p) { attention_impl<256, 8>(p); }
+HC_KERNEL void hc_attention_f16_t512(hck_attention_args p) { attention_impl<512, 64>(p); }

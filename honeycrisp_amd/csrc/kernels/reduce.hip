@@ -12,6 +12,7 @@
 // k = 0 does (BackendCPU.swift:848-877): ties go to the smaller index, a NaN at k > 0
 // never replaces the running extremum, and a NaN at k = 0 is never replaced.
 #include "common.hip.h"
+#include "row_teams.hip.h"
 
 #include <math.h>
 
@@ -71,11 +72,6 @@ template <int OP, typename C> __device__ __forceinline__ C reduce_combine(C a, C
 // A row is reduced by a team of LANES lanes: 1 (rows of a few elements: a lane per row, adjacent
 // lanes on adjacent rows), 8, 64 (one wave) or 256 (the whole block). SPLIT (LANES = 256): few
 // long rows are cut into p.segs segments, one block each, which leave partials.
-template <int LANES, typename V, typename Op> __device__ __forceinline__ V team_reduce(V v, Op op) {
-#pragma unroll
-  for (int o = LANES / 2; o > 0; o >>= 1) v = op(v, __shfl_xor(v, o, 64));
-  return v;
-}
 template <int LANES, int OP, typename C> __device__ __forceinline__ ArgPair<C> team_arg_reduce(ArgPair<C> p) {
 #pragma unroll
   for (int o = LANES / 2; o > 0; o >>= 1) {
@@ -383,58 +379,6 @@ template <int LANES> struct Team {
   }
 };
 
-// A row of up to LANES * VEC * CHUNKS elements held by its team in registers: lane l owns the
-// 16-byte vectors l, l + LANES, ... of the row (n a multiple of VEC; rows then start 16-byte
-// aligned because the buffer does). Longer rows, or ragged ones, are streamed instead.
-template <typename T, int LANES> struct RowRegs {
-  static constexpr int VEC = VecWidth<T>::value;
-  static constexpr int CHUNKS = 4;
-  T v[CHUNKS][VEC];
-  static __device__ __forceinline__ bool fits(uint32_t n) {
-    return n % VEC == 0 && n <= (uint32_t)LANES * VEC * CHUNKS;
-  }
-  __device__ __forceinline__ void load(const T* row, uint32_t n, uint32_t lane) {
-#pragma unroll
-    for (int c = 0; c < CHUNKS; c++) {
-      const uint32_t k = (lane + LANES * c) * VEC;
-      if (k < n) load_vec<T, VEC>(row, k, 1, v[c]);
-    }
-  }
-  template <typename F> __device__ __forceinline__ void each(uint32_t n, uint32_t lane, F f) const {
-#pragma unroll
-    for (int c = 0; c < CHUNKS; c++)
-      if ((lane + LANES * c) * VEC < n) {
-#pragma unroll
-        for (int i = 0; i < VEC; i++) f((float)v[c][i]);
-      }
-  }
-  template <typename F> __device__ __forceinline__ void store(T* row, uint32_t n, uint32_t lane, F f) const {
-#pragma unroll
-    for (int c = 0; c < CHUNKS; c++) {
-      const uint32_t k = (lane + LANES * c) * VEC;
-      if (k < n) {
-        T o[VEC];
-#pragma unroll
-        for (int i = 0; i < VEC; i++) o[i] = narrow<T>(f((float)v[c][i]));
-        store_vec<T, VEC>(row, k, o);
-      }
-    }
-  }
-  template <typename F>
-  __device__ __forceinline__ void store2(T* row, uint32_t n, uint32_t lane, const RowRegs& other, F f) const {
-#pragma unroll
-    for (int c = 0; c < CHUNKS; c++) {
-      const uint32_t k = (lane + LANES * c) * VEC;
-      if (k < n) {
-        T o[VEC];
-#pragma unroll
-        for (int i = 0; i < VEC; i++) o[i] = narrow<T>(f((float)v[c][i], (float)other.v[c][i]));
-        store_vec<T, VEC>(row, k, o);
-      }
-    }
-  }
-};
-
 // Streaming pass over a row that does not fit the registers: f(x, k) for every element, with
 // 16-byte loads when the row length allows them.
 template <typename T, int LANES, typename F>
@@ -469,11 +413,6 @@ __device__ __forceinline__ void stream_row_out(const T* row, T* out, uint32_t n,
 }
 
 // ---------------------------------------------------------------- logSoftmax
-
-// exp of an fp32 value inside a kernel whose results are rounded to T: the library's expf for fp32
-// tensors; for fp16 tensors (11 significant bits) the hardware's exp2, about 1 ulp of fp32, at a
-// fifth of the instructions: an fp16 softmax row is bound by these, not by memory.
-template <typename T> __device__ __forceinline__ float exp_in(float x) { return sizeof(T) == 2 ? exp_hw(x) : expf(x); }
 
 // logSoftmax (BackendCPU.swift:1000-1038): max, sum of expf(x - max), x - (logf(sum) + max),
 // all in Float. Rows (inner == 1): a wave or a block per row; the row stays in registers when

@@ -395,8 +395,9 @@ def test_head_swaps_fold_into_the_batched_products(hip_backend, dtype, B, T, H, 
             probs = (scores * 0.125).softmax()
             return Tensor.batchedMatmul(probs, False, heads(v), False, False).swap(1, 2).reshape([B, T, D])
 
-        # 4 swaps, and scale + logSoftmax + exp -> 1
-        check(hip_backend, attention, removed=4 + 2)
+        # 4 swaps, and scale + logSoftmax + exp -> 1; with 64-wide fp16 heads the two products and that
+        # row kernel then become the attention kernel
+        check(hip_backend, attention, removed=4 + 2 + (2 if dtype == DType.float16 and hd == 64 else 0))
         # one operand swapped, the other dense; result kept in [B, H, T, T] order
         kt = Tensor(data=rng.standard_normal((B, H, T, hd)).astype(np.float32), dtype=dtype)
         check(hip_backend, lambda: Tensor.batchedMatmul(heads(q), False, kt, True, False), removed=1)
@@ -407,6 +408,72 @@ def test_head_swaps_fold_into_the_batched_products(hip_backend, dtype, B, T, H, 
             return Tensor.batchedMatmul(hq, False, kt, True, False) + hq.sum(axis=3, keepdims=True)
 
         check(hip_backend, two_readers, removed=0)
+
+
+@pytest.mark.parametrize("heads,t", [(64, 256), (32, 512), (5, 64), (3, 128), (2, 192), (3, 320), (2, 448)])
+def test_attention_becomes_one_kernel(hip_backend, heads, t):
+    """q k^T -> [* s] [+ mask] softmax -> x v over fp16 heads of 64: one launch per recording, and a replay
+    returns the bits of the five separate launches (same accumulation order in both products, fp16
+    scores and probabilities, the row kernel's own reduction)."""
+    rng = np.random.default_rng(heads * 1000 + t)
+    f16 = DType.float16
+    with hip_backend.use():
+        q, k, v = (Tensor(data=rng.standard_normal((heads, t, 64)).astype(np.float32), dtype=f16) for _ in range(3))
+        mask = Tensor(data=np.where(np.tril(np.ones((t, t))) > 0, 0.0, -1e4).astype(np.float32), dtype=f16)
+
+        def attention(scale=True, masked=True, log=False):
+            s = Tensor.batchedMatmul(q, False, k, True, False)
+            if scale:
+                s = s * 0.125
+            if masked:
+                s = s + mask
+            p = s.logSoftmax() if log else s.softmax()
+            return Tensor.batchedMatmul(p, False, v, False, False)
+
+        check(hip_backend, attention, removed=3 + 2)                                   # scale, mask, logSoftmax, exp -> 1; -> attention
+        check(hip_backend, lambda: attention(masked=False), removed=2 + 2)
+        check(hip_backend, lambda: attention(scale=False), removed=2 + 2)
+        check(hip_backend, lambda: attention(log=True), removed=2 + 2)                # (log-probabilities times v: same machinery)
+        # a bare softmax is a row kernel of its own plus exp: the chain of two still merges, and then the three
+        check(hip_backend, lambda: attention(scale=False, masked=False), removed=1 + 2)
+
+
+def test_attention_forms_that_are_left_alone(hip_backend):
+    rng = np.random.default_rng(77)
+    f16 = DType.float16
+
+    def qkv(heads, t, hd, dtype=f16):
+        return (Tensor(data=rng.standard_normal((heads, t, hd)).astype(np.float32), dtype=dtype) for _ in range(3))
+
+    with hip_backend.use():
+        def attention(q, k, v):
+            s = Tensor.batchedMatmul(q, False, k, True, False) * 0.125
+            return Tensor.batchedMatmul(s.softmax(), False, v, False, False)
+
+        q, k, v = qkv(8, 128, 32)                # heads of 32
+        check(hip_backend, lambda: attention(q, k, v), removed=2)
+        q, k, v = qkv(8, 128, 64, DType.float32)  # fp32
+        check(hip_backend, lambda: attention(q, k, v), removed=2)
+        q, k, v = qkv(2, 576, 64)                # rows longer than the score tile holds
+        check(hip_backend, lambda: attention(q, k, v), removed=2)
+        q, k, v = qkv(4, 128, 64)
+
+        def probabilities_read_twice():
+            p = (Tensor.batchedMatmul(q, False, k, True, False) * 0.125).softmax()
+            return Tensor.batchedMatmul(p, False, v, False, False).sum(axis=2) + p.sum(axis=2)
+
+        check(hip_backend, probabilities_read_twice, removed=2)
+
+        def scores_kept():                        # the caller keeps the scores: they must be written
+            s = Tensor.batchedMatmul(q, False, k, True, False)
+            return s, Tensor.batchedMatmul((s * 0.125).softmax(), False, v, False, False)
+
+        want_s, want_o = (x.numpy().copy() for x in scores_kept())
+        with hip_backend.capture() as cap:
+            s, o = scores_kept()
+        cap.graph.launch()
+        assert np.array_equal(s.numpy(), want_s) and np.array_equal(o.numpy(), want_o)
+        cap.graph.destroy()
 
 
 @pytest.mark.parametrize("dtype", [DType.float32, DType.float16], ids=["f32", "f16"])
@@ -430,8 +497,10 @@ def test_config5_forward_recorded_with_the_rewrite(hip_backend, dtype):
         # in fp16 also the 6 + 1 casts of the fp32 biases
         half = dtype == DType.float16
         per_block = 9 + 2 * (4 if half else 2) + 3 + 4 + 2 + (6 if half else 0)
+        # ... and in fp16 (64-wide heads) scores, softmax and context of a block are one attention kernel
+        per_block += 2 if half else 0
         assert plain_nodes - fused_nodes == 6 * per_block + (4 if half else 2) + (2 if half else 1)
-        assert fused_nodes == 58
+        assert fused_nodes == (46 if half else 58)
         plain.destroy()
         fused.destroy()
 

@@ -84,3 +84,22 @@ def test_transformer_forward_replay(hip_backend, dtype):
             want = model(ids).numpy()
             assert np.array_equal(got, want), "replay %d" % replay
         cap.graph.destroy()
+
+
+def test_a_graph_destroyed_during_another_recording(hip_backend):
+    """hc_graph_destroy waits for the stream, which a capture in progress does not survive: a graph
+    that its owner lets go of in the middle of a recording is destroyed when the recording ends."""
+    rng = np.random.default_rng(21)
+    with hip_backend.use():
+        x = Tensor(data=rng.standard_normal((64, 64)).astype(np.float32))
+        with hip_backend.capture() as first:
+            y = x * 2.0
+        first.graph.launch()
+        assert np.array_equal(y.numpy(), x.numpy() * 2.0)
+        with hip_backend.capture() as second:
+            z = x + 1.0
+            first.graph.destroy()          # in the middle of the second recording
+            w = z * 3.0
+        second.graph.launch()
+        assert np.array_equal(w.numpy(), (x.numpy() + 1.0) * 3.0)
+        second.graph.destroy()
