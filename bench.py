@@ -620,10 +620,12 @@ def extra_workloads(backend, graph=True, only=("cfg1", "cfg2", "cfg3", "cfg4", "
                 tokens = Tensor(data=ids)
                 for _ in range(2):
                     model(tokens).wait()
+                mark(backend, name + "_5_passes")
                 t0 = time.perf_counter()
                 for _ in range(5):
                     model(tokens).wait()
                 dt = (time.perf_counter() - t0) / 5
+                mark(backend, name + "_5_passes")
                 out[name] = {"ms": round(dt * 1e3, 3), "tokens_per_s": round(2048 / dt, 1),
                              "tflops": round(100.9e9 / dt / 1e12, 2)}
                 # The same pass issued eagerly from native host code (the C++ HCMatrixBench as a child process:
@@ -645,11 +647,13 @@ def extra_workloads(backend, graph=True, only=("cfg1", "cfg2", "cfg3", "cfg4", "
                     for _ in range(5):
                         cap.graph.launch()
                     logits.wait()
+                    mark(backend, name + suffix + "_20_passes")
                     t0 = time.perf_counter()
                     for _ in range(20):
                         cap.graph.launch()
                         logits.wait()
                     dt = (time.perf_counter() - t0) / 20
+                    mark(backend, name + suffix + "_20_passes")
                     out[name + suffix] = {"ms": round(dt * 1e3, 3), "tokens_per_s": round(2048 / dt, 1),
                                           "tflops": round(100.9e9 / dt / 1e12, 2), "launches": cap.graph.node_count()}
                     cap.graph.destroy()
