@@ -48,8 +48,15 @@ __device__ __forceinline__ uint32_t swz_mn(uint32_t k) { return (((k & 7u) ^ (((
 // builtin would do the same but also waits for every DMA instruction in flight, including
 // those that fill stages nobody is about to read. The "memory" clobber keeps the compiler
 // from moving LDS accesses across it.
+// (builtins, not an assembly statement: the compiler's wait-count pass then knows that no LDS read is
+// outstanding behind the barrier and does not guard the first MFMAs of the next sub-step with waits
+// of its own, each of which would take one of the three issue slots between two MFMAs. The empty
+// assembly statements keep the compiler from moving memory accesses across the pair.)
 __device__ __forceinline__ void lds_barrier() {
-  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0); vmcnt and expcnt untouched
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
 }
 // s_waitcnt vmcnt(N) with the other counters untouched (gfx9 encoding: vmcnt in bits 3:0 and
 // 15:14, expcnt 6:4, lgkmcnt 11:8): at most N of this wave's DMA instructions still in flight.
@@ -74,7 +81,17 @@ template <int ROWS, int MODE> struct DmaOperand {
   static constexpr uint32_t SWZ_MASK = (SLOTS & (SLOTS - 1)) == 0 ? SLOTS - 1 : 7;
   static_assert(ROWS % 64 == 0 && SLOTS % (SWZ_MASK + 1) == 0, "unsupported tile extent");
 
-  uint32_t goff[NI];     // byte offset of this lane's 16-byte piece for DMA instruction i (k = 0)
+  // Four consecutive DMA instructions of a wave share one LDS base (the M0 register) and differ in the
+  // instruction's immediate offset, which the hardware adds to the LDS address and to the memory
+  // address alike: instruction i targets base + (i % 4) KiB. The lane offsets take the immediate out
+  // again, and the buffer descriptor starts IMM_SPAN bytes in front of the operand so that they stay
+  // non-negative. (One M0 write and its wait state per four loads instead of per load: between two
+  // MFMAs a wave has three issue slots.)
+  static constexpr uint32_t IMM_SPAN = 3 * 1024;
+  // The descriptor's range, and the lane offset that reads as zero: lane offset + immediate is a 32-bit
+  // sum, so the offset of a lane that must not fetch stays out of range with any immediate added.
+  static constexpr uint32_t RANGE = 0xffffe000u;
+  uint32_t goff[NI];     // byte offset of this lane's 16-byte piece for DMA instruction i (k = 0), see above
   uint32_t kstride;      // bytes per unit of k
 
   __device__ __forceinline__ static uint32_t mn_swz(uint32_t k) { return swz_mn(k) & SWZ_MASK; }
@@ -92,7 +109,7 @@ template <int ROWS, int MODE> struct DmaOperand {
         const uint32_t c = (lane % 8) ^ swz_k(row);
         uint32_t grow = r0 + row;
         if (limit && grow >= limit) grow = limit - 1;
-        goff[i] = grow * rs * 2 + c * 16;
+        goff[i] = grow * rs * 2 + c * 16 + IMM_SPAN - (i & 3) * 1024;
       }
     } else {
       kstride = cs * 2;
@@ -103,7 +120,7 @@ template <int ROWS, int MODE> struct DmaOperand {
         const uint32_t slot = (piece % SLOTS) ^ mn_swz(krow);
         uint32_t col = r0 + slot * 8;
         if (limit && col + 8 > limit) col = limit - 8;
-        goff[i] = (krow * cs + col) * 2;
+        goff[i] = (krow * cs + col) * 2 + IMM_SPAN - (i & 3) * 1024;
       }
     }
   }
@@ -118,22 +135,23 @@ template <int ROWS, int MODE> struct DmaOperand {
     return ((wave * NI + i) * 64 + lane) / SLOTS;
   }
 
-  // DMA instruction i of this wave for the K-slice starting at k0: 1 KiB into `region`.
-  // A buffer load: the descriptor (base of the operand, no stride, range 2^32 - 16 bytes) lives
-  // in scalar registers, the lane offset goes in as it is and the K offset as the scalar
+  // DMA instruction I of this wave for the K-slice starting at k0: 1 KiB into `region`.
+  // A buffer load: the descriptor (base of the operand less IMM_SPAN, no stride, range RANGE
+  // bytes) lives in scalar registers, the lane offset goes in as it is and the K offset as the scalar
   // offset, so no vector or scalar address arithmetic stands in front of the load. The host
-  // keeps operands of this kernel below 4 GiB.
+  // keeps operands of this kernel 16 KiB below 4 GiB.
   // Edge kernels (kend != 0): lanes whose piece lies at k >= kend pass an offset beyond the
   // descriptor's range, which reads as zero, so the ragged last slice contributes nothing.
-  __device__ __forceinline__ void dma(int i, const half_t* base, uint32_t k0, char* region, uint32_t kend = 0) const {
+  template <int I> __device__ __forceinline__ void dma(const half_t* base, uint32_t k0, char* region, uint32_t kend = 0) const {
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, 0xfffffff0u, 0x00020000);
-    uint32_t off = goff[i];
+    const __amdgpu_buffer_rsrc_t rsrc =
+        __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)base - IMM_SPAN), 0, RANGE, 0x00020000);
+    uint32_t off = goff[I];
     if (kend != 0 && k0 + 64 > kend) {  // wave-uniform
-      if (k0 + klocal(i) >= kend) off = 0xfffffff0u;
+      if (k0 + klocal(I) >= kend) off = RANGE;
     }
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (LDS_AS void*)(region + (wave * NI + i) * 1024), 16, off,
-                                             k0 * kstride, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (LDS_AS void*)(region + (wave * NI + (I & ~3)) * 1024), 16, off,
+                                             k0 * kstride, (I & 3) * 1024, 0);
   }
 
   // Edge kernels: clears what the piece straddling `kend` holds beyond it (gemm_zero_piece_tail),
@@ -286,10 +304,11 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
   // `tail`: a compile-time flag. Only the last K-slice can be ragged, so only the DMA that may
   // fetch it carries the range check of the edge kernels (a scalar compare and a branch in
   // front of every DMA instruction otherwise, in the middle of the MFMA stream).
-  auto dma_unit = [&](auto tail, int u, uint32_t k0, char* stage) {
+  auto dma_unit = [&](auto tail, auto uc, uint32_t k0, char* stage) {
+    constexpr int u = decltype(uc)::value;
     const uint32_t ke = decltype(tail)::value ? kend : 0;
-    if (u < OpA::NI) oa.dma(u, A, k0, stage, ke);
-    else if (u < NDMA) ob.dma(u - OpA::NI, B, k0, stage + A_BYTES, ke);
+    if constexpr (u < OpA::NI) oa.template dma<u>(A, k0, stage, ke);
+    else if constexpr (u < NDMA) ob.template dma<u - OpA::NI>(B, k0, stage + A_BYTES, ke);
   };
   typedef std::integral_constant<bool, EDGE> Tail;     // checks where the kernel has them at all
   typedef std::integral_constant<bool, false> NoTail;
@@ -333,7 +352,7 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
       constexpr int w = part * SLOTS + t;
       constexpr int lo = (w * NDMA + W - 1) / W < NDMA ? (w * NDMA + W - 1) / W : NDMA;
       constexpr int hi = ((w + 1) * NDMA + W - 1) / W < NDMA ? ((w + 1) * NDMA + W - 1) / W : NDMA;
-      static_for<hi - lo>([&](auto uc) { dma_unit(tail, lo + decltype(uc)::value, k0, to); });
+      static_for<hi - lo>([&](auto uc) { dma_unit(tail, std::integral_constant<int, lo + decltype(uc)::value>{}, k0, to); });
       // operand reads of the following sub-step: one every RSTRIDE slots
       if constexpr (t % RSTRIDE == 0 && t / RSTRIDE < READS) read_unit(fill, from, s_next, t / RSTRIDE);
       mma_one(use, t);
@@ -357,8 +376,8 @@ __device__ __forceinline__ void gemm_mi16_impl(const hck_gemm_args& p, char* lds
   };
 
   // prologue: K-step 0 and the first window part of K-step 1
-  static_for<NDMA>([&](auto uc) { dma_unit(Tail{}, decltype(uc)::value, 0, lds0); });
-  static_for<U0>([&](auto uc) { dma_unit(Tail{}, decltype(uc)::value, kclamp(1), lds1); });
+  static_for<NDMA>([&](auto uc) { dma_unit(Tail{}, uc, 0, lds0); });
+  static_for<U0>([&](auto uc) { dma_unit(Tail{}, uc, kclamp(1), lds1); });
   // The accumulators are cleared here, while the first loads are on their way: left to the
   // compiler the 256 register writes sit after the barrier, in front of the first MFMA.
   __builtin_amdgcn_sched_barrier(0);
