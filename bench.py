@@ -444,14 +444,14 @@ def cpu_reference_ops(budget_s=15.0):
     return out
 
 
-def native_eager_transformer(dtype_name):
+def native_eager_transformer(dtype_name, batching=0):
     """Runs `HCMatrixBench --transformer` and returns its figures, or None if the program is not built."""
     import subprocess
     binary = os.path.join(ROOT, "honeycrisp_amd", "cpp", "HCMatrixBench")
     if not os.path.exists(binary):
         return None
-    proc = subprocess.run([binary, "--transformer", "--dtype", dtype_name, "--iters", "20"], stdout=subprocess.PIPE,
-                          stderr=subprocess.PIPE, text=True, timeout=120)
+    proc = subprocess.run([binary, "--transformer", "--dtype", dtype_name, "--iters", "20", "--batching", str(batching)],
+                          stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=120)
     if proc.returncode != 0:
         return {"error": (proc.stdout + proc.stderr)[-300:]}
     r = dict(kv.split("=", 1) for kv in proc.stdout.strip().splitlines()[-1].split())
@@ -460,8 +460,11 @@ def native_eager_transformer(dtype_name):
             "ms_back_to_back": round(float(r["us_back_to_back"]) / 1e3, 3),
             "tokens_per_s_back_to_back": round(float(r["tokens_per_s_back_to_back"]), 1),
             "host_enqueue_ms": round(float(r["host_enqueue_us"]) / 1e3, 3),
-            "note": "eager, one backend call per op from a C++ host (HCMatrixBench --transformer, child process); "
-                    "back_to_back: passes enqueued without a wait in between"}
+            **({"launches_listed": int(r["launches_listed"]), "launches_enqueued": int(r["launches_enqueued"])} if batching else {}),
+            "note": ("the same calls with hc_set_batching(%d): listed, rewritten and enqueued batch by batch; " % batching
+                     if batching else "eager, ") +
+                    "one backend call per op from a C++ host (HCMatrixBench --transformer, child process); "
+                    "back_to_back: passes issued without a wait in between"}
 
 
 def extra_workloads(backend, graph=True, only=("cfg1", "cfg2", "cfg3", "cfg4", "cfg5")):
@@ -634,6 +637,9 @@ def extra_workloads(backend, graph=True, only=("cfg1", "cfg2", "cfg3", "cfg4", "
                 native = native_eager_transformer("f32" if dtype is F32 else "f16")
                 if native:
                     out[name + "_native_host"] = native
+                    # ... and with the library's batching on: still one call per op and no recording in
+                    # the program, the launches listed and rewritten in batches of 128
+                    out[name + "_native_host_batched"] = native_eager_transformer("f32" if dtype is F32 else "f16", 128)
                 if not graph:
                     continue
                 # the same forward pass recorded once and replayed as one graph launch: as recorded

@@ -5,7 +5,7 @@ There is no fallback: if the library has not been built, importing this module r
 import ctypes
 import os
 from ctypes import (POINTER, Structure, c_char, c_char_p, c_float, c_int, c_int64, c_size_t,
-                    c_uint32, c_void_p)
+                    c_uint32, c_uint64, c_void_p)
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 # HCHIP_LIB points at an alternative build of the library (kernel experiments).
@@ -56,6 +56,9 @@ PROTOTYPES = {
     "hc_last_error_string": (c_char_p, []),
     "hc_get_device_info": (c_int, [_P, POINTER(hc_device_info)]),
     "hc_debug_set": (c_int, [_P, c_char_p, c_char_p]),
+    "hc_set_batching": (c_int, [_P, c_size_t]),
+    "hc_flush": (c_int, [_P]),
+    "hc_batching_stats": (c_int, [_P, POINTER(c_uint64), POINTER(c_uint64)]),
     "hc_malloc": (c_int, [_P, c_size_t, POINTER(c_void_p)]),
     "hc_free": (c_int, [_P, _P]),
     "hc_trim": (c_int, [_P]),

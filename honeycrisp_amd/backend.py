@@ -12,6 +12,7 @@ There is no CPU fallback here: an op or dtype the kernels do not cover raises
 """
 import contextlib
 import ctypes
+import os
 import threading
 from ctypes import byref, c_float, c_int64, c_size_t, c_void_p
 from typing import List, Optional, Sequence, Union
@@ -374,6 +375,8 @@ class HIPBackend(Backend):
         if status != _lib.HC_OK:
             self._raise(status)
         self._ctx = ctx
+        # hc_set_batching's current value (HCHIP_BATCHING in the environment gives a context its first)
+        self._batch_limit = int(os.environ.get("HCHIP_BATCHING") or 0)
 
     def close(self):
         if self._ctx:
@@ -433,6 +436,40 @@ class HIPBackend(Backend):
 
     def sync(self):
         self._check(self._lib.hc_sync(self._ctx))
+
+    def memStats(self):
+        """(bytes in blocks handed out, bytes in the pool's free blocks) of this context (hc_mem_stats)."""
+        used, cached = c_size_t(0), c_size_t(0)
+        self._check(self._lib.hc_mem_stats(self._ctx, byref(used), byref(cached)))
+        return used.value, cached.value
+
+    def setBatching(self, max_launches: int):
+        """hc_set_batching: with max_launches > 0 the ops of ordinary, call-by-call code are listed
+        and enqueued batch by batch, each batch rewritten like a recording (same bits, fewer
+        launches); 0 goes back to one launch per call."""
+        self._check(self._lib.hc_set_batching(self._ctx, int(max_launches)))
+        self._batch_limit = int(max_launches)
+
+    @contextlib.contextmanager
+    def batching(self, max_launches: int = 512):
+        """`with backend.batching():` batches the ops of the block (see setBatching) and restores
+        the setting of before afterwards."""
+        before = self._batch_limit
+        self.setBatching(max_launches)
+        try:
+            yield self
+        finally:
+            self.setBatching(before)
+
+    def flush(self):
+        """Enqueues what batching has listed so far (hc_flush)."""
+        self._check(self._lib.hc_flush(self._ctx))
+
+    def batchingStats(self):
+        """(launches listed by batches, launches enqueued in their place) since the context was created."""
+        listed, enqueued = ctypes.c_uint64(0), ctypes.c_uint64(0)
+        self._check(self._lib.hc_batching_stats(self._ctx, ctypes.byref(listed), ctypes.byref(enqueued)))
+        return listed.value, enqueued.value
 
     def capture(self) -> "Capture":
         """`with backend.capture() as cap: out = model(x)` records every op issued inside the

@@ -9,14 +9,14 @@
 // bandwidth-bound ops of a forward pass at [8192, 4096] fp32 (broadcast bias add, GELU, sum, argmax and
 // max = argmax + gather over axis 1) and an int64 row gather of 65536 ids from a [32000, 1024] table
 // (config 4); with --transformer, the eager forward pass of the 6-layer transformer (config 5) issued
-// from native host code, tokens/s.
+// from native host code, tokens/s (--batching N: the same calls with the library's batching on).
 // One `key=value` line per op with both rates, the ratio, a self-check of the HIP result (known sums /
 // identities) and, when both backends ran, the parity of the two results on the rows the CPU computed.
 // The scalar CPU loop takes minutes at 4096^3, so the CPU leg computes a slab of output rows sized to
 // --cpu-seconds per product (cpu_rows=<computed>/<all>); its rate per row does not depend on the row.
 //
 // Usage: HCMatrixBench [--backend cpu|hip|both] [--iters N] [--max-size S] [--cpu-seconds T]
-//                      [--transformer [--dtype f16|f32] [--weights FILE --ids FILE --logits-out FILE]]
+//                      [--transformer [--dtype f16|f32] [--batching N] [--weights FILE --ids FILE --logits-out FILE]]
 // Build: see honeycrisp_amd/csrc/build.py (g++ -O2, links libhchip.so and the Accelerate stand-in).
 #include <algorithm>
 #include <chrono>
@@ -40,7 +40,7 @@ static double seconds_since(Clock::time_point t0) { return std::chrono::duration
 
 struct Options {
   bool hip = true, cpu = true, transformer = false;
-  int iters = 10, max_size = 8192;
+  int iters = 10, max_size = 8192, batching = 0;
   double cpu_seconds = 2.0;
   std::string dtype = "f16", weights, ids, logits_out;
 };
@@ -358,8 +358,11 @@ static int bench_transformer(hc::HIPBackend& backend, const Options& opt) {
   }
   hc::Transformer model(backend, dtype, cfg, weights);
   hc::Data tokens = backend.upload(ids.data(), ids.size() * 8);
+  backend.setBatching((size_t)opt.batching);
+  const auto stats0 = backend.batchingStats();
   hc::Data logits = model.forward(tokens, B);
   backend.wait();
+  const auto stats1 = backend.batchingStats();
   if (!opt.logits_out.empty()) {
     std::vector<char> host((size_t)(B * T * cfg.vocab) * hc::byteSize(dtype));
     backend.download(logits, host.data(), host.size());
@@ -379,10 +382,12 @@ static int bench_transformer(hc::HIPBackend& backend, const Options& opt) {
   const double enqueue_s = seconds_since(t1) / opt.iters;
   backend.wait();
   const double back_to_back_s = seconds_since(t1) / opt.iters;
-  std::printf("op=transformer_forward mode=eager_native_host dtype=%s tokens=%lld us=%.1f tokens_per_s=%.1f "
-              "us_back_to_back=%.1f tokens_per_s_back_to_back=%.1f host_enqueue_us=%.1f\n",
+  std::printf("op=transformer_forward mode=%s dtype=%s tokens=%lld us=%.1f tokens_per_s=%.1f "
+              "us_back_to_back=%.1f tokens_per_s_back_to_back=%.1f host_enqueue_us=%.1f launches_listed=%llu launches_enqueued=%llu\n",
+              opt.batching > 0 ? "batched_native_host" : "eager_native_host",
               dtype == hc::DType::float32 ? "float32" : "float16", (long long)(B * T), s * 1e6, (double)(B * T) / s,
-              back_to_back_s * 1e6, (double)(B * T) / back_to_back_s, enqueue_s * 1e6);
+              back_to_back_s * 1e6, (double)(B * T) / back_to_back_s, enqueue_s * 1e6,
+              (unsigned long long)(stats1.first - stats0.first), (unsigned long long)(stats1.second - stats0.second));
   return 0;
 }
 
@@ -412,6 +417,7 @@ int main(int argc, char** argv) {
     else if (a == "--weights") opt.weights = value();
     else if (a == "--ids") opt.ids = value();
     else if (a == "--logits-out") opt.logits_out = value();
+    else if (a == "--batching") opt.batching = std::atoi(value().c_str());
     else {
       std::fprintf(stderr, "unknown argument %s\n", a.c_str());
       return 2;

@@ -160,6 +160,16 @@ class HIPBackend {
   }
   void destroy(hc_graph* g) { check(hc_graph_destroy(ctx_, g)); }
 
+  // ---- batching (no counterpart in the reference either): the calls of ordinary code are listed
+  // and enqueued batch by batch, each batch rewritten like a recording; 0 = one launch per call
+  void setBatching(size_t maxLaunches) { check(hc_set_batching(ctx_, maxLaunches)); }
+  void flush() { check(hc_flush(ctx_)); }
+  std::pair<uint64_t, uint64_t> batchingStats() {   // launches listed, launches enqueued in their place
+    uint64_t listed = 0, enqueued = 0;
+    check(hc_batching_stats(ctx_, &listed, &enqueued));
+    return {listed, enqueued};
+  }
+
   // ---- ops (Backend.swift line of each declaration in the comment)
   Data broadcast(const BroadcastData& a, DType dtype) {  // :170
     Data out = allocate(a.strides.count() * byteSize(dtype));

@@ -100,6 +100,7 @@ struct hc_pending {
   int lanes = 0;
   void* out = nullptr;
   bool dropped = false;                // merged into another entry
+  bool merged = false;                 // the rewrite's own launch: stands where the last entry of its chain stood
 };
 
 struct hc_graph {
@@ -184,15 +185,24 @@ struct hc_ctx {
   hipEvent_t stage_ev[2] = {nullptr, nullptr};
   bool stage_busy[2] = {false, false};
   std::vector<hipEvent_t> wait_events;  // spare events of blocking transfers (waited for outside the mutex)
-  bool lazy = false;                    // a capture that lists its launches (see hc_pending)
-  bool rewrite = false;                 // ... and will rewrite the list (decided when the capture begins)
+  bool lazy = false;                    // launches are listed, not enqueued (see hc_pending): a capture, or batching
+  bool rewrite = false;                 // the capture in progress will rewrite its list (decided when it begins)
   std::vector<hc_pending> pending;
+  // hc_set_batching: outside a capture, launches are listed too and enqueued batch by batch, each
+  // batch rewritten like a recording. Blocks released while their batch is listed wait here, by
+  // bucket size, and go back to the pool when the batch has been enqueued.
+  size_t batch_limit = 0;               // launches per batch at most; 0 = every launch is enqueued at once
+  size_t batch_launches = 0;            // launches in the list now
+  std::unordered_map<size_t, std::vector<void*>> batch_parked;
+  size_t batch_parked_bytes = 0;
+  uint64_t batch_listed = 0, batch_enqueued = 0;   // launches and copies, since the context was created
   // buffers whose only writer and only reader were merged away by the rewrite of the recording in
   // progress: no launch of the graph touches them, so they need not stay reserved for it
   std::vector<std::pair<void*, size_t>> dead;
 };
 static const size_t kStageHalf = 2u << 20;    // bytes per half of the staging buffer
 static const size_t kStageMax = 256u << 10;   // largest upload that is staged
+static const size_t kBatchParkedMax = (size_t)8 << 30;   // batching: released bytes a listed batch may hold back
 
 static thread_local std::string g_last_error;
 
@@ -253,6 +263,10 @@ extern "C" int hc_init(int device, hc_ctx** out) {
   hc_ctx* ctx = new hc_ctx();
   ctx->device = device;
   for (const char* name : kSwitchNames) set_switch(ctx->sw, name, getenv(name));
+  if (const char* v = getenv("HCHIP_BATCHING")) {   // hc_set_batching from the environment (whole programs, test runs)
+    ctx->batch_limit = (size_t)strtoull(v, nullptr, 10);
+    ctx->lazy = ctx->batch_limit > 0;
+  }
   e = hipGetDeviceProperties(&ctx->props, device);
   if (e != hipSuccess) {
     delete ctx;
@@ -329,6 +343,8 @@ extern "C" void hc_shutdown(hc_ctx* ctx) {
   }
   for (auto& kv : ctx->free_blocks)
     for (void* p : kv.second) (void)hipFree(p);
+  for (auto& kv : ctx->batch_parked)   // (a batch still listed is dropped: nobody can read its results any more)
+    for (void* p : kv.second) (void)hipFree(p);
   for (auto& kv : ctx->live) (void)hipFree(kv.first);
   for (hipModule_t m : ctx->modules) (void)hipModuleUnload(m);
   if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
@@ -392,6 +408,9 @@ static size_t bucket_size(size_t bytes) {
   return (bytes + g - 1) / g * g;
 }
 
+static int flush_batch_locked(hc_ctx* ctx);
+static int batch_grew_locked(hc_ctx* ctx);
+
 static void release_cache_locked(hc_ctx* ctx) {
   for (auto& kv : ctx->free_blocks)
     for (void* p : kv.second) (void)hipFree(p);
@@ -430,8 +449,10 @@ extern "C" int hc_malloc(hc_ctx* ctx, size_t bytes, void** out) {
     (void)hipSetDevice(ctx->device);
     hipError_t e = hipMalloc(&p, b);
     if (e != hipSuccess && !ctx->capturing) {
-      // Give cached blocks back to the driver and retry once.
+      // Enqueue what is listed (its released blocks come back with it), give cached blocks back
+      // to the driver and retry once.
       (void)hipGetLastError();
+      (void)flush_batch_locked(ctx);
       (void)hipStreamSynchronize(ctx->stream);
       release_cache_locked(ctx);
       e = hipMalloc(&p, b);
@@ -472,6 +493,11 @@ extern "C" int hc_free(hc_ctx* ctx, void* ptr) {
     // allocated before the capture, released inside it: the recording read (or wrote) it
     ctx->block_owner[ptr] = ctx->capturing;
     ctx->capturing->parked[b].push_back(ptr);
+  } else if (ctx->lazy) {
+    // batching: listed launches may still use it, so it stays out of the pool until they are enqueued
+    ctx->batch_parked[b].push_back(ptr);
+    ctx->batch_parked_bytes += b;
+    if (ctx->batch_parked_bytes > kBatchParkedMax) return flush_batch_locked(ctx);
   } else {
     ctx->free_blocks[b].push_back(ptr);
     ctx->bytes_cached += b;
@@ -483,6 +509,7 @@ extern "C" int hc_trim(hc_ctx* ctx) {
   REQUIRE(ctx, "hc_trim: null context");
   std::lock_guard<std::mutex> lock(ctx->mu);
   REQUIRE(!ctx->capturing, "hc_trim: not allowed while capturing");
+  HC_TRY(flush_batch_locked(ctx));
   HIP_TRY(hipStreamSynchronize(ctx->stream));
   release_cache_locked(ctx);
   return HC_OK;
@@ -543,6 +570,22 @@ static int wait_event_unlocked(hc_ctx* ctx, hipEvent_t ev) {
   return HC_OK;
 }
 
+// Batching: whether a launch that is listed, not yet enqueued, may read or write the block that
+// holds `p` (or `p` itself, for memory this context did not allocate). Caller holds the mutex.
+static bool batch_touches_locked(const hc_ctx* ctx, const void* p) {
+  std::pair<void*, size_t> blk = block_of_locked(ctx, p);
+  if (!blk.first) blk = {const_cast<void*>(p), 1};
+  for (const hc_pending& e : ctx->pending) {
+    if (e.kind == hc_pending::FREE) continue;
+    if (!e.known) return true;
+    for (const void* q : e.reads)
+      if ((const char*)q >= (const char*)blk.first && (const char*)q < (const char*)blk.first + blk.second) return true;
+    for (const void* q : e.writes)
+      if ((const char*)q >= (const char*)blk.first && (const char*)q < (const char*)blk.first + blk.second) return true;
+  }
+  return false;
+}
+
 static int copy(hc_ctx* ctx, void* dst, const void* src, size_t bytes, hipMemcpyKind kind, bool wait) {
   REQUIRE(ctx, "memcpy: null context");
   if (bytes == 0) return HC_OK;
@@ -552,6 +595,12 @@ static int copy(hc_ctx* ctx, void* dst, const void* src, size_t bytes, hipMemcpy
     std::lock_guard<std::mutex> lock(ctx->mu);
     REQUIRE(!ctx->capturing || kind == hipMemcpyDeviceToDevice,
             "memcpy: host transfers are not allowed while capturing (upload inputs before hc_capture_begin)");
+    // Batching: a transfer is enqueued at once, ahead of the launches still listed. An upload
+    // may overtake them when none of them uses the block it fills (a fresh buffer: constants and
+    // index vectors in the middle of a forward pass); everything else enqueues the list first.
+    if (!ctx->capturing && !ctx->pending.empty() && kind != hipMemcpyDeviceToDevice &&
+        (kind != hipMemcpyHostToDevice || batch_touches_locked(ctx, dst)))
+      HC_TRY(flush_batch_locked(ctx));
     if (kind == hipMemcpyHostToDevice && wait && bytes <= kStageMax && ctx->stage) {
       // The caller may reuse `src` as soon as this returns: copy it into pinned memory and let the
       // stream pick it up from there. No wait, so the device keeps running what is already queued
@@ -581,7 +630,7 @@ static int copy(hc_ctx* ctx, void* dst, const void* src, size_t bytes, hipMemcpy
         e.reads = {src};
         e.writes = {dst};
         ctx->pending.push_back(std::move(e));
-        return HC_OK;
+        return batch_grew_locked(ctx);
       }
       HIP_TRY(hipMemcpyAsync(dst, src, bytes, kind, ctx->stream));
       return HC_OK;
@@ -623,7 +672,11 @@ extern "C" int hc_memcpy_d2h_async(hc_ctx* ctx, void* dst, const void* src, size
 
 extern "C" int hc_sync(hc_ctx* ctx) {
   REQUIRE(ctx, "hc_sync: null context");
-  REQUIRE(!ctx->capturing, "hc_sync: not allowed while capturing");
+  {
+    std::lock_guard<std::mutex> lock(ctx->mu);
+    REQUIRE(!ctx->capturing, "hc_sync: not allowed while capturing");
+    HC_TRY(flush_batch_locked(ctx));
+  }
   HIP_TRY(hipStreamSynchronize(ctx->stream));
   return HC_OK;
 }
@@ -644,6 +697,7 @@ extern "C" int hc_event_record(hc_ctx* ctx, hc_event* ev) {
   REQUIRE(ctx && ev, "hc_event_record: null argument");
   std::lock_guard<std::mutex> lock(ctx->mu);
   REQUIRE(!ctx->capturing, "hc_event_record: not allowed while capturing");
+  HC_TRY(flush_batch_locked(ctx));
   HIP_TRY(hipEventRecord(ev->ev, ctx->stream));
   return HC_OK;
 }
@@ -683,6 +737,7 @@ extern "C" int hc_launch_host_func(hc_ctx* ctx, void (*fn)(void*), void* user) {
   REQUIRE(ctx && fn, "hc_launch_host_func: null argument");
   std::lock_guard<std::mutex> lock(ctx->mu);
   REQUIRE(!ctx->capturing, "hc_launch_host_func: not allowed while capturing");
+  HC_TRY(flush_batch_locked(ctx));
   HIP_TRY(hipLaunchHostFunc(ctx->stream, fn, user));
   return HC_OK;
 }
@@ -693,6 +748,7 @@ extern "C" int hc_capture_begin(hc_ctx* ctx) {
   REQUIRE(ctx, "hc_capture_begin: null context");
   std::lock_guard<std::mutex> lock(ctx->mu);
   REQUIRE(!ctx->capturing, "hc_capture_begin: a capture is already in progress");
+  HC_TRY(flush_batch_locked(ctx));
   // relaxed mode: the allocator may still call hipMalloc for sizes its pool does not hold
   HIP_TRY(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed));
   ctx->capturing = new hc_graph();
@@ -725,6 +781,72 @@ static int emit_recording_locked(hc_ctx* ctx, std::vector<hc_pending>& list) {
     }
   }
   return HC_OK;
+}
+
+// HCHIP_RECORDING_LOG: the launches of a list as they will be enqueued, to stderr
+static void log_launches_locked(const hc_ctx* ctx, const char* what) {
+  size_t n = 0;
+  for (const hc_pending& e : ctx->pending) {
+    if (e.dropped || e.kind == hc_pending::FREE) continue;
+    const char* name = e.kind == hc_pending::COPY_D2D ? "(copy)" : "(caller's kernel)";
+    for (const auto& kv : ctx->functions)
+      if (e.kind == hc_pending::KERNEL && kv.second == e.fn) name = kv.first.c_str();
+    fprintf(stderr, "hchip %s %3zu: %s grid %u x %u\n", what, n++, name, e.grid[0], e.grid[1]);
+  }
+}
+
+// Batching: rewrites the listed launches like a recording and enqueues them; the blocks released
+// since the last batch go back to the pool (in stream order behind the launches that used them,
+// which is what the pool assumes of every block it holds). Nothing to do outside batching, or
+// during a capture (whose list is the capture's). Caller holds the lock.
+static int flush_batch_locked(hc_ctx* ctx) {
+  if (ctx->capturing || ctx->batch_limit == 0) return HC_OK;
+  int status = HC_OK;
+  if (!ctx->pending.empty()) {
+    ctx->lazy = false;
+    for (const hc_pending& e : ctx->pending) ctx->batch_listed += e.kind != hc_pending::FREE;
+    if (!ctx->sw.no_fusion) fuse_recording(ctx);
+    for (const hc_pending& e : ctx->pending) ctx->batch_enqueued += e.kind != hc_pending::FREE && !e.dropped;
+    if (ctx->sw.recording_log) log_launches_locked(ctx, "batch");
+    status = emit_recording_locked(ctx, ctx->pending);
+    ctx->pending.clear();
+    ctx->dead.clear();
+    ctx->lazy = true;
+  }
+  ctx->batch_launches = 0;
+  for (auto& kv : ctx->batch_parked) {
+    auto& pool = ctx->free_blocks[kv.first];
+    pool.insert(pool.end(), kv.second.begin(), kv.second.end());
+    ctx->bytes_cached += kv.first * kv.second.size();
+  }
+  ctx->batch_parked.clear();
+  ctx->batch_parked_bytes = 0;
+  return status;
+}
+
+extern "C" int hc_set_batching(hc_ctx* ctx, size_t max_launches) {
+  REQUIRE(ctx, "hc_set_batching: null context");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  REQUIRE(!ctx->capturing, "hc_set_batching: not allowed while capturing");
+  HC_TRY(flush_batch_locked(ctx));
+  ctx->batch_limit = max_launches;
+  ctx->lazy = max_launches > 0;
+  return HC_OK;
+}
+
+extern "C" int hc_batching_stats(hc_ctx* ctx, uint64_t* listed, uint64_t* enqueued) {
+  REQUIRE(ctx, "hc_batching_stats: null context");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  if (listed) *listed = ctx->batch_listed;
+  if (enqueued) *enqueued = ctx->batch_enqueued;
+  return HC_OK;
+}
+
+extern "C" int hc_flush(hc_ctx* ctx) {
+  REQUIRE(ctx, "hc_flush: null context");
+  std::lock_guard<std::mutex> lock(ctx->mu);
+  REQUIRE(!ctx->capturing, "hc_flush: not allowed while capturing");
+  return flush_batch_locked(ctx);
 }
 
 // Gives a graph's parked blocks back to the general pool and forgets its ownership of
@@ -766,16 +888,7 @@ static int end_capture_locked(hc_ctx* ctx, hc_graph** out) {
     if (out) {
       // HCHIP_NO_FUSION=1 when the capture began: the launches are enqueued as they were issued
       if (ctx->rewrite) fuse_recording(ctx);
-      if (ctx->sw.recording_log) {   // the launches of the recording as they will be enqueued, to stderr
-        size_t n = 0;
-        for (const hc_pending& e : ctx->pending) {
-          if (e.dropped || e.kind == hc_pending::FREE) continue;
-          const char* name = e.kind == hc_pending::COPY_D2D ? "(copy)" : "(caller's kernel)";
-          for (const auto& kv : ctx->functions)
-            if (e.kind == hc_pending::KERNEL && kv.second == e.fn) name = kv.first.c_str();
-          fprintf(stderr, "hchip recording %3zu: %s grid %u x %u\n", n++, name, e.grid[0], e.grid[1]);
-        }
-      }
+      if (ctx->sw.recording_log) log_launches_locked(ctx, "recording");
       emitted = emit_recording_locked(ctx, ctx->pending);
       if (ctx->sw.graph_as_launches)
         for (hc_pending& e : ctx->pending)
@@ -785,6 +898,8 @@ static int end_capture_locked(hc_ctx* ctx, hc_graph** out) {
   }
   ctx->rewrite = false;
   ctx->capturing = nullptr;
+  ctx->lazy = ctx->batch_limit > 0;   // batching goes on where the capture interrupted it
+  ctx->batch_launches = 0;
   hipError_t e = hipStreamEndCapture(ctx->stream, &g->graph);
   if (emitted != HC_OK) {
     (void)hipGetLastError();
@@ -836,6 +951,7 @@ extern "C" int hc_graph_launch(hc_ctx* ctx, hc_graph* graph) {
   REQUIRE(ctx && graph && graph->exec, "hc_graph_launch: null argument");
   std::lock_guard<std::mutex> lock(ctx->mu);
   REQUIRE(!ctx->capturing, "hc_graph_launch: not allowed while capturing");
+  HC_TRY(flush_batch_locked(ctx));
   if (!graph->launches.empty()) return emit_recording_locked(ctx, graph->launches);
   HIP_TRY(hipGraphLaunch(graph->exec, ctx->stream));
   return HC_OK;
@@ -849,7 +965,9 @@ extern "C" int hc_graph_node_count(hc_graph* graph, size_t* out) {
 
 // Caller holds the lock; no capture in progress.
 static int destroy_graph_locked(hc_ctx* ctx, hc_graph* graph) {
-  // replays already enqueued still use the parked blocks: let them finish first
+  // listed launches may use blocks that are parked with this graph, and replays already enqueued
+  // still use them: enqueue the former, let all of it finish
+  HC_TRY(flush_batch_locked(ctx));
   HIP_TRY(hipStreamSynchronize(ctx->stream));
   if (graph->exec) (void)hipGraphExecDestroy(graph->exec);
   if (graph->graph) (void)hipGraphDestroy(graph->graph);
@@ -925,7 +1043,14 @@ struct OpNote {
 };
 thread_local OpNote* OpNote::current = nullptr;
 
-// Adds a launch to the recording in progress (caller holds the mutex).
+// Batching: one more launch is listed; a full batch is enqueued. Caller holds the mutex.
+static int batch_grew_locked(hc_ctx* ctx) {
+  if (ctx->capturing || ctx->batch_limit == 0) return HC_OK;
+  if (++ctx->batch_launches >= ctx->batch_limit) return flush_batch_locked(ctx);
+  return HC_OK;
+}
+
+// Adds a launch to the list in progress (caller holds the mutex).
 static void record_launch_locked(hc_ctx* ctx, const std::string& name, hipFunction_t fn, uint32_t gx, uint32_t gy,
                                  const void* args, size_t bytes) {
   hc_pending e;
@@ -986,7 +1111,7 @@ extern "C" int hc_launch(hc_ctx* ctx, hc_function* fn, const uint32_t grid[3], c
     e.shared = shared_bytes;
     e.args.assign((const char*)kernarg, (const char*)kernarg + kernarg_bytes);
     ctx->pending.push_back(std::move(e));
-    return HC_OK;
+    return batch_grew_locked(ctx);
   }
   HIP_TRY(hipModuleLaunchKernel(fn->fn, grid[0], grid[1], grid[2], block[0], block[1], block[2],
                                 shared_bytes, ctx->stream, nullptr, config));
@@ -1025,7 +1150,7 @@ static int launch(hc_ctx* ctx, const std::string& name, uint64_t blocks_x, uint3
   HC_TRY(find_kernel_locked(ctx, name, &fn));
   if (ctx->lazy) {
     record_launch_locked(ctx, name, fn, (uint32_t)blocks_x, blocks_y, args, bytes);
-    return HC_OK;
+    return batch_grew_locked(ctx);
   }
   return launch_fn(ctx, fn, (uint32_t)blocks_x, blocks_y, 1, HCK_BLOCK, 0, args, bytes);
 }

@@ -190,6 +190,32 @@ int hc_graph_launch(hc_ctx* ctx, hc_graph* graph);
 int hc_graph_node_count(hc_graph* graph, size_t* out);
 int hc_graph_destroy(hc_ctx* ctx, hc_graph* graph);
 
+/* ---- batching: the rewrite of a recording for ordinary, call-by-call use ----
+ * No counterpart in the reference, whose API has no notion of a recording either: a program
+ * written against it issues one backend call per op and never says where a forward pass begins
+ * or ends (Tensor.swift:634-657). With max_launches > 0 the op entry points list their launches
+ * instead of enqueueing them, exactly as inside a capture, and the list is rewritten (the same
+ * passes, the same guarantee: the bits of the call-by-call result) and enqueued
+ *  - when it holds max_launches launches,
+ *  - before anything that must see or order against the results: hc_memcpy_d2h (Tensor.Data.onCPU),
+ *    hc_sync, hc_event_record, hc_launch_host_func (Tensor.Data.wait), hc_graph_launch,
+ *    hc_capture_begin, hc_trim, hc_flush; an upload is enqueued at once and overtakes the list
+ *    when no listed launch uses the block it fills, else the list goes first,
+ *  - when the blocks released since the last batch exceed 8 GiB, or an allocation fails.
+ * A block released while its batch is listed is not handed out again before the batch has been
+ * enqueued (the rewrite needs every buffer of a batch at an address of its own), so the
+ * footprint of a batch is the sum of its intermediates. Errors of a listed launch surface in
+ * the call that enqueues the batch. max_launches = 0 (the default) enqueues what is listed and
+ * goes back to one launch per call. Refused during a capture; a capture inside batching works
+ * (the list is enqueued first). HCHIP_BATCHING=<n> in the environment at hc_init starts a
+ * context with hc_set_batching(n). */
+int hc_set_batching(hc_ctx* ctx, size_t max_launches);
+/* Enqueues what batching has listed so far. Nothing to do outside batching. */
+int hc_flush(hc_ctx* ctx);
+/* Launches and device-to-device copies that batches listed, and that were enqueued in their
+ * place after the rewrite, since the context was created (either pointer may be NULL). */
+int hc_batching_stats(hc_ctx* ctx, uint64_t* listed, uint64_t* enqueued);
+
 /* ---- raw module API (thin wrappers over hipModuleLoadData / hipModuleGetFunction /
  * hipModuleLaunchKernel) for callers that bring their own gfx950 code objects ---- */
 

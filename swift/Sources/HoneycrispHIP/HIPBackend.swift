@@ -79,7 +79,12 @@ open class HIPBackend: CPUBackend, @unchecked Sendable {
 
   let ctx: OpaquePointer
 
-  public init(device: Int = 0) throws {
+  /// `batching` > 0: the library lists the launches of the backend calls and enqueues them in
+  /// batches of at most that many, each batch rewritten (a Linear layer's bias, activation and
+  /// residual go into the product's kernel, LayerNorm / softmax / attention become one kernel
+  /// each) with the bits of the call-by-call result; anything that reads or waits for a result
+  /// (`Tensor.Data.onCPU`, `wait()`) enqueues what is listed first. 0 = one launch per call.
+  public init(device: Int = 0, batching: Int = 0) throws {
     var c: OpaquePointer? = nil
     let status = hc_init(Int32(device), &c)
     guard status == HC_OK.rawValue, let c = c else {
@@ -87,6 +92,7 @@ open class HIPBackend: CPUBackend, @unchecked Sendable {
     }
     ctx = c
     super.init()
+    try check(hc_set_batching(ctx, batching))
   }
 
   deinit { hc_shutdown(ctx) }

@@ -43,6 +43,15 @@ def check(backend, fn, removed):
     assert plain_nodes - fused_nodes == removed, (plain_nodes, fused_nodes)
     plain.destroy()
     fused.destroy()
+    # ... and the same ops issued call by call under batching: listed, rewritten the same way and
+    # enqueued when the result is read
+    listed, enqueued = backend.batchingStats()
+    with backend.batching():
+        got = fn().numpy().copy()
+    listed, enqueued = (after - before for after, before in zip(backend.batchingStats(), (listed, enqueued)))
+    assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), \
+        "batching: %d of %d elements differ" % (int((got != want).sum()), want.size)
+    assert listed - enqueued == removed, (listed, enqueued)
 
 
 def operands(rng, dtype, m, k, n):
@@ -503,6 +512,13 @@ def test_config5_forward_recorded_with_the_rewrite(hip_backend, dtype):
         assert fused_nodes == (46 if half else 58)
         plain.destroy()
         fused.destroy()
+        # the same forward pass call by call under batching: one batch, the same launches
+        listed, enqueued = hip_backend.batchingStats()
+        with hip_backend.batching(1024):
+            for _ in range(2):
+                assert np.array_equal(model(ids).numpy().view(np.uint8), want.view(np.uint8))
+        listed, enqueued = (after - before for after, before in zip(hip_backend.batchingStats(), (listed, enqueued)))
+        assert (listed, enqueued) == (2 * plain_nodes, 2 * fused_nodes)
 
 
 class _Raw:

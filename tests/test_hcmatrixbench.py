@@ -83,8 +83,9 @@ def export_weights(model, path):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("batching", [0, 128], ids=["eager", "batched"])
 @pytest.mark.parametrize("dtype_name", ["f16", "f32"])
-def test_native_eager_transformer_reproduces_the_python_path(hip_backend, tmp_path, dtype_name):
+def test_native_eager_transformer_reproduces_the_python_path(hip_backend, tmp_path, dtype_name, batching):
     from honeycrisp_amd.descriptors import DType
     from honeycrisp_amd.nn import Transformer
     from honeycrisp_amd.tensor import Tensor
@@ -96,9 +97,14 @@ def test_native_eager_transformer_reproduces_the_python_path(hip_backend, tmp_pa
         export_weights(model, str(tmp_path / "weights.bin"))
     ids.astype(np.int64).tofile(str(tmp_path / "ids.bin"))
     lines, out = run(["--transformer", "--dtype", dtype_name, "--iters", "5", "--weights", str(tmp_path / "weights.bin"),
-                      "--ids", str(tmp_path / "ids.bin"), "--logits-out", str(tmp_path / "logits.bin")])
+                      "--ids", str(tmp_path / "ids.bin"), "--logits-out", str(tmp_path / "logits.bin"),
+                      "--batching", str(batching)])
     (r,) = lines
-    assert r["op"] == "transformer_forward" and r["mode"] == "eager_native_host" and int(r["tokens"]) == 2048
+    assert r["op"] == "transformer_forward" and int(r["tokens"]) == 2048
+    assert r["mode"] == ("batched_native_host" if batching else "eager_native_host")
+    if batching:    # the same calls, listed and rewritten batch by batch: fewer launches, the same bits
+        assert int(r["launches_listed"]) == (256 if dtype_name == "f16" else 193)
+        assert int(r["launches_enqueued"]) < int(r["launches_listed"]) // 3
     assert float(r["tokens_per_s"]) > 2.0e5, out
     got = np.fromfile(str(tmp_path / "logits.bin"), dtype=want.dtype).reshape(want.shape)
     assert np.array_equal(got.view(np.uint16 if dtype_name == "f16" else np.uint32),
