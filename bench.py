@@ -444,13 +444,14 @@ def cpu_reference_ops(budget_s=15.0):
     return out
 
 
-def native_eager_transformer(dtype_name, batching=0):
+def native_eager_transformer(dtype_name, batching=0, idle_after=0):
     """Runs `HCMatrixBench --transformer` and returns its figures, or None if the program is not built."""
     import subprocess
     binary = os.path.join(ROOT, "honeycrisp_amd", "cpp", "HCMatrixBench")
     if not os.path.exists(binary):
         return None
-    proc = subprocess.run([binary, "--transformer", "--dtype", dtype_name, "--iters", "20", "--batching", str(batching)],
+    proc = subprocess.run([binary, "--transformer", "--dtype", dtype_name, "--iters", "20", "--batching", str(batching),
+                           "--idle-after", str(idle_after)],
                           stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=120)
     if proc.returncode != 0:
         return {"error": (proc.stdout + proc.stderr)[-300:]}
@@ -461,7 +462,7 @@ def native_eager_transformer(dtype_name, batching=0):
             "tokens_per_s_back_to_back": round(float(r["tokens_per_s_back_to_back"]), 1),
             "host_enqueue_ms": round(float(r["host_enqueue_us"]) / 1e3, 3),
             **({"launches_listed": int(r["launches_listed"]), "launches_enqueued": int(r["launches_enqueued"])} if batching else {}),
-            "note": ("the same calls with hc_set_batching(%d): listed, rewritten and enqueued batch by batch; " % batching
+            "note": ("the same calls with hc_set_batching(%d, %d): listed, rewritten and enqueued batch by batch; " % (batching, idle_after)
                      if batching else "eager, ") +
                     "one backend call per op from a C++ host (HCMatrixBench --transformer, child process); "
                     "back_to_back: passes issued without a wait in between"}
@@ -638,8 +639,9 @@ def extra_workloads(backend, graph=True, only=("cfg1", "cfg2", "cfg3", "cfg4", "
                 if native:
                     out[name + "_native_host"] = native
                     # ... and with the library's batching on: still one call per op and no recording in
-                    # the program, the launches listed and rewritten in batches of 128
-                    out[name + "_native_host_batched"] = native_eager_transformer("f32" if dtype is F32 else "f16", 128)
+                    # the program, the launches listed and rewritten in batches of up to 256 (earlier when
+                    # the device has run dry and 16 are listed)
+                    out[name + "_native_host_batched"] = native_eager_transformer("f32" if dtype is F32 else "f16", 256, 16)
                 if not graph:
                     continue
                 # the same forward pass recorded once and replayed as one graph launch: as recorded

@@ -56,7 +56,7 @@ PROTOTYPES = {
     "hc_last_error_string": (c_char_p, []),
     "hc_get_device_info": (c_int, [_P, POINTER(hc_device_info)]),
     "hc_debug_set": (c_int, [_P, c_char_p, c_char_p]),
-    "hc_set_batching": (c_int, [_P, c_size_t]),
+    "hc_set_batching": (c_int, [_P, c_size_t, c_size_t]),
     "hc_flush": (c_int, [_P]),
     "hc_batching_stats": (c_int, [_P, POINTER(c_uint64), POINTER(c_uint64)]),
     "hc_malloc": (c_int, [_P, c_size_t, POINTER(c_void_p)]),

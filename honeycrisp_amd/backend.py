@@ -375,8 +375,9 @@ class HIPBackend(Backend):
         if status != _lib.HC_OK:
             self._raise(status)
         self._ctx = ctx
-        # hc_set_batching's current value (HCHIP_BATCHING in the environment gives a context its first)
-        self._batch_limit = int(os.environ.get("HCHIP_BATCHING") or 0)
+        # hc_set_batching's current values (HCHIP_BATCHING in the environment gives a context its first)
+        env = (os.environ.get("HCHIP_BATCHING") or "0").split(",")
+        self._batching = (int(env[0]), int(env[1]) if len(env) > 1 else 0)
 
     def close(self):
         if self._ctx:
@@ -443,23 +444,24 @@ class HIPBackend(Backend):
         self._check(self._lib.hc_mem_stats(self._ctx, byref(used), byref(cached)))
         return used.value, cached.value
 
-    def setBatching(self, max_launches: int):
+    def setBatching(self, max_launches: int, idle_after: int = 0):
         """hc_set_batching: with max_launches > 0 the ops of ordinary, call-by-call code are listed
         and enqueued batch by batch, each batch rewritten like a recording (same bits, fewer
-        launches); 0 goes back to one launch per call."""
-        self._check(self._lib.hc_set_batching(self._ctx, int(max_launches)))
-        self._batch_limit = int(max_launches)
+        launches); 0 goes back to one launch per call. idle_after > 0: a list of at least that
+        many launches is also enqueued as soon as the device has run out of work."""
+        self._check(self._lib.hc_set_batching(self._ctx, int(max_launches), int(idle_after)))
+        self._batching = (int(max_launches), int(idle_after))
 
     @contextlib.contextmanager
-    def batching(self, max_launches: int = 512):
+    def batching(self, max_launches: int = 512, idle_after: int = 0):
         """`with backend.batching():` batches the ops of the block (see setBatching) and restores
         the setting of before afterwards."""
-        before = self._batch_limit
-        self.setBatching(max_launches)
+        before = self._batching
+        self.setBatching(max_launches, idle_after)
         try:
             yield self
         finally:
-            self.setBatching(before)
+            self.setBatching(*before)
 
     def flush(self):
         """Enqueues what batching has listed so far (hc_flush)."""

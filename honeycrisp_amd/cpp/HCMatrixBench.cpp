@@ -16,7 +16,7 @@
 // --cpu-seconds per product (cpu_rows=<computed>/<all>); its rate per row does not depend on the row.
 //
 // Usage: HCMatrixBench [--backend cpu|hip|both] [--iters N] [--max-size S] [--cpu-seconds T]
-//                      [--transformer [--dtype f16|f32] [--batching N] [--weights FILE --ids FILE --logits-out FILE]]
+//                      [--transformer [--dtype f16|f32] [--batching N [--idle-after M]] [--weights FILE --ids FILE --logits-out FILE]]
 // Build: see honeycrisp_amd/csrc/build.py (g++ -O2, links libhchip.so and the Accelerate stand-in).
 #include <algorithm>
 #include <chrono>
@@ -40,7 +40,7 @@ static double seconds_since(Clock::time_point t0) { return std::chrono::duration
 
 struct Options {
   bool hip = true, cpu = true, transformer = false;
-  int iters = 10, max_size = 8192, batching = 0;
+  int iters = 10, max_size = 8192, batching = 0, idle_after = 0;
   double cpu_seconds = 2.0;
   std::string dtype = "f16", weights, ids, logits_out;
 };
@@ -358,7 +358,7 @@ static int bench_transformer(hc::HIPBackend& backend, const Options& opt) {
   }
   hc::Transformer model(backend, dtype, cfg, weights);
   hc::Data tokens = backend.upload(ids.data(), ids.size() * 8);
-  backend.setBatching((size_t)opt.batching);
+  backend.setBatching((size_t)opt.batching, (size_t)opt.idle_after);
   const auto stats0 = backend.batchingStats();
   hc::Data logits = model.forward(tokens, B);
   backend.wait();
@@ -418,6 +418,7 @@ int main(int argc, char** argv) {
     else if (a == "--ids") opt.ids = value();
     else if (a == "--logits-out") opt.logits_out = value();
     else if (a == "--batching") opt.batching = std::atoi(value().c_str());
+    else if (a == "--idle-after") opt.idle_after = std::atoi(value().c_str());
     else {
       std::fprintf(stderr, "unknown argument %s\n", a.c_str());
       return 2;

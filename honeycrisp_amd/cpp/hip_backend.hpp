@@ -162,7 +162,8 @@ class HIPBackend {
 
   // ---- batching (no counterpart in the reference either): the calls of ordinary code are listed
   // and enqueued batch by batch, each batch rewritten like a recording; 0 = one launch per call
-  void setBatching(size_t maxLaunches) { check(hc_set_batching(ctx_, maxLaunches)); }
+  // (idleAfter > 0: a list of at least that many launches is also enqueued once the device has run dry)
+  void setBatching(size_t maxLaunches, size_t idleAfter = 0) { check(hc_set_batching(ctx_, maxLaunches, idleAfter)); }
   void flush() { check(hc_flush(ctx_)); }
   std::pair<uint64_t, uint64_t> batchingStats() {   // launches listed, launches enqueued in their place
     uint64_t listed = 0, enqueued = 0;

@@ -15,6 +15,7 @@
 #include <cstring>
 #include <cmath>
 #include <map>
+#include <unordered_set>
 #include <mutex>
 #include <string>
 #include <unordered_map>
@@ -192,6 +193,13 @@ struct hc_ctx {
   // batch rewritten like a recording. Blocks released while their batch is listed wait here, by
   // bucket size, and go back to the pool when the batch has been enqueued.
   size_t batch_limit = 0;               // launches per batch at most; 0 = every launch is enqueued at once
+  size_t batch_idle_after = 0;          // > 0: a list this long is also enqueued when the stream has run dry (see hc_free)
+  std::unordered_set<void*> batch_born; // blocks handed out since the last batch was enqueued and still in use
+  // "has the stream run dry" without a call into the runtime: behind every batch a one-lane
+  // kernel stores the batch's number into pinned host memory, which hc_free compares with the
+  // number of the last batch it enqueued
+  uint64_t* batch_done = nullptr;
+  uint64_t batch_seq = 0;
   size_t batch_launches = 0;            // launches in the list now
   std::unordered_map<size_t, std::vector<void*>> batch_parked;
   size_t batch_parked_bytes = 0;
@@ -205,6 +213,7 @@ static const size_t kStageMax = 256u << 10;   // largest upload that is staged
 static const size_t kBatchParkedMax = (size_t)8 << 30;   // batching: released bytes a listed batch may hold back
 
 static thread_local std::string g_last_error;
+static int alloc_batch_flag_locked(hc_ctx* ctx);
 
 static int fail(int code, const char* fmt, ...) {
   char buf[512];
@@ -263,8 +272,10 @@ extern "C" int hc_init(int device, hc_ctx** out) {
   hc_ctx* ctx = new hc_ctx();
   ctx->device = device;
   for (const char* name : kSwitchNames) set_switch(ctx->sw, name, getenv(name));
-  if (const char* v = getenv("HCHIP_BATCHING")) {   // hc_set_batching from the environment (whole programs, test runs)
-    ctx->batch_limit = (size_t)strtoull(v, nullptr, 10);
+  if (const char* v = getenv("HCHIP_BATCHING")) {   // hc_set_batching from the environment: <max>[,<idle_after>]
+    char* end = nullptr;
+    ctx->batch_limit = (size_t)strtoull(v, &end, 10);
+    ctx->batch_idle_after = end && *end == ',' ? (size_t)strtoull(end + 1, nullptr, 10) : 0;
     ctx->lazy = ctx->batch_limit > 0;
   }
   e = hipGetDeviceProperties(&ctx->props, device);
@@ -316,6 +327,7 @@ extern "C" int hc_init(int device, hc_ctx** out) {
   if (s == HC_OK) s = load_image(ctx, hc_image_gemm_dma2_m_f16, hc_image_gemm_dma2_m_f16_end, "gemm_dma2_m_f16");
   if (s == HC_OK) s = load_image(ctx, hc_image_gemm_dma2_m_f32, hc_image_gemm_dma2_m_f32_end, "gemm_dma2_m_f32");
   if (s == HC_OK) s = load_image(ctx, hc_image_gemm_mi16_m, hc_image_gemm_mi16_m_end, "gemm_mi16_m");
+  if (s == HC_OK && ctx->batch_idle_after > 0) s = alloc_batch_flag_locked(ctx);
   if (s != HC_OK) {
     hc_shutdown(ctx);
     return s;
@@ -352,6 +364,7 @@ extern "C" void hc_shutdown(hc_ctx* ctx) {
     if (ev) (void)hipEventDestroy(ev);
   for (hipEvent_t ev : ctx->wait_events) (void)hipEventDestroy(ev);
   if (ctx->stage) (void)hipHostFree(ctx->stage);
+  if (ctx->batch_done) (void)hipHostFree(ctx->batch_done);
   delete ctx;
 }
 
@@ -465,6 +478,7 @@ extern "C" int hc_malloc(hc_ctx* ctx, size_t bytes, void** out) {
   ctx->live[p] = b;
   ctx->bytes_in_use += b;
   if (ctx->capturing) ctx->block_owner[p] = ctx->capturing;
+  else if (ctx->lazy && ctx->batch_idle_after > 0) ctx->batch_born.insert(p);
   *out = p;
   return HC_OK;
 }
@@ -497,7 +511,16 @@ extern "C" int hc_free(hc_ctx* ctx, void* ptr) {
     // batching: listed launches may still use it, so it stays out of the pool until they are enqueued
     ctx->batch_parked[b].push_back(ptr);
     ctx->batch_parked_bytes += b;
+    ctx->batch_born.erase(ptr);
     if (ctx->batch_parked_bytes > kBatchParkedMax) return flush_batch_locked(ctx);
+    // A device that has nothing left to do gains nothing from a longer list. The place to cut
+    // the list is where the program holds at most one result of the listed launches (between
+    // two layers of a model, say): every other intermediate has been released, so no chain that
+    // the rewrite could merge is open. There, once the list is long enough to be worth a
+    // rewrite, look whether the stream has run dry.
+    if (ctx->batch_idle_after > 0 && ctx->batch_launches >= ctx->batch_idle_after && ctx->batch_born.size() <= 1 &&
+        ctx->batch_done && __atomic_load_n(ctx->batch_done, __ATOMIC_ACQUIRE) == ctx->batch_seq)
+      return flush_batch_locked(ctx);
   } else {
     ctx->free_blocks[b].push_back(ptr);
     ctx->bytes_cached += b;
@@ -761,6 +784,7 @@ extern "C" int hc_capture_begin(hc_ctx* ctx) {
 }
 
 static void fuse_recording(hc_ctx* ctx);
+static int find_kernel_locked(hc_ctx* ctx, const std::string& name, hipFunction_t* out);
 static int launch_fn(hc_ctx* ctx, hipFunction_t fn, uint32_t gx, uint32_t gy, uint32_t gz, uint32_t bx,
                      uint32_t shared, const void* kernarg, size_t kernarg_bytes);
 
@@ -811,9 +835,20 @@ static int flush_batch_locked(hc_ctx* ctx) {
     status = emit_recording_locked(ctx, ctx->pending);
     ctx->pending.clear();
     ctx->dead.clear();
+    if (status == HC_OK && ctx->batch_idle_after > 0 && ctx->batch_done) {
+      hck_map_args k;
+      memset(&k, 0, sizeof(k));
+      k.out = ctx->batch_done;
+      k.count = 1;
+      k.i0 = (int64_t)++ctx->batch_seq;
+      hipFunction_t fn = nullptr;
+      status = find_kernel_locked(ctx, "hc_fill_b8", &fn);
+      if (status == HC_OK) status = launch_fn(ctx, fn, 1, 1, 1, HCK_BLOCK, 0, &k, sizeof(k));
+    }
     ctx->lazy = true;
   }
   ctx->batch_launches = 0;
+  ctx->batch_born.clear();
   for (auto& kv : ctx->batch_parked) {
     auto& pool = ctx->free_blocks[kv.first];
     pool.insert(pool.end(), kv.second.begin(), kv.second.end());
@@ -824,12 +859,25 @@ static int flush_batch_locked(hc_ctx* ctx) {
   return status;
 }
 
-extern "C" int hc_set_batching(hc_ctx* ctx, size_t max_launches) {
+static int alloc_batch_flag_locked(hc_ctx* ctx) {
+  (void)hipSetDevice(ctx->device);
+  hipError_t e = hipHostMalloc((void**)&ctx->batch_done, 64, hipHostMallocDefault);
+  if (e != hipSuccess) {
+    ctx->batch_done = nullptr;
+    return hip_fail(e, "hipHostMalloc (batching's completion flag)");
+  }
+  *ctx->batch_done = ctx->batch_seq;
+  return HC_OK;
+}
+
+extern "C" int hc_set_batching(hc_ctx* ctx, size_t max_launches, size_t idle_after) {
   REQUIRE(ctx, "hc_set_batching: null context");
   std::lock_guard<std::mutex> lock(ctx->mu);
   REQUIRE(!ctx->capturing, "hc_set_batching: not allowed while capturing");
   HC_TRY(flush_batch_locked(ctx));
+  if (idle_after > 0 && !ctx->batch_done) HC_TRY(alloc_batch_flag_locked(ctx));
   ctx->batch_limit = max_launches;
+  ctx->batch_idle_after = idle_after;
   ctx->lazy = max_launches > 0;
   return HC_OK;
 }

@@ -196,7 +196,11 @@ int hc_graph_destroy(hc_ctx* ctx, hc_graph* graph);
  * or ends (Tensor.swift:634-657). With max_launches > 0 the op entry points list their launches
  * instead of enqueueing them, exactly as inside a capture, and the list is rewritten (the same
  * passes, the same guarantee: the bits of the call-by-call result) and enqueued
- *  - when it holds max_launches launches,
+ *  - when it holds max_launches launches, or (idle_after > 0) at least idle_after launches
+ *    while the device has finished everything enqueued so far: looked up in hc_free when the
+ *    caller holds at most one buffer allocated since the last batch (between two layers of a
+ *    model: every other intermediate is released, so no chain the rewrite could merge is cut).
+ *    While the device is busy a batch grows; once it has run dry it gets what there is,
  *  - before anything that must see or order against the results: hc_memcpy_d2h (Tensor.Data.onCPU),
  *    hc_sync, hc_event_record, hc_launch_host_func (Tensor.Data.wait), hc_graph_launch,
  *    hc_capture_begin, hc_trim, hc_flush; an upload is enqueued at once and overtakes the list
@@ -207,9 +211,9 @@ int hc_graph_destroy(hc_ctx* ctx, hc_graph* graph);
  * footprint of a batch is the sum of its intermediates. Errors of a listed launch surface in
  * the call that enqueues the batch. max_launches = 0 (the default) enqueues what is listed and
  * goes back to one launch per call. Refused during a capture; a capture inside batching works
- * (the list is enqueued first). HCHIP_BATCHING=<n> in the environment at hc_init starts a
- * context with hc_set_batching(n). */
-int hc_set_batching(hc_ctx* ctx, size_t max_launches);
+ * (the list is enqueued first). HCHIP_BATCHING=<max>[,<idle_after>] in the environment at
+ * hc_init starts a context with hc_set_batching(max, idle_after). */
+int hc_set_batching(hc_ctx* ctx, size_t max_launches, size_t idle_after);
 /* Enqueues what batching has listed so far. Nothing to do outside batching. */
 int hc_flush(hc_ctx* ctx);
 /* Launches and device-to-device copies that batches listed, and that were enqueued in their

@@ -83,8 +83,9 @@ open class HIPBackend: CPUBackend, @unchecked Sendable {
   /// batches of at most that many, each batch rewritten (a Linear layer's bias, activation and
   /// residual go into the product's kernel, LayerNorm / softmax / attention become one kernel
   /// each) with the bits of the call-by-call result; anything that reads or waits for a result
-  /// (`Tensor.Data.onCPU`, `wait()`) enqueues what is listed first. 0 = one launch per call.
-  public init(device: Int = 0, batching: Int = 0) throws {
+  /// (`Tensor.Data.onCPU`, `wait()`) enqueues what is listed first, and so does a device that has
+  /// run out of work once `idleAfter` launches are listed. 0 = one launch per call.
+  public init(device: Int = 0, batching: Int = 0, idleAfter: Int = 16) throws {
     var c: OpaquePointer? = nil
     let status = hc_init(Int32(device), &c)
     guard status == HC_OK.rawValue, let c = c else {
@@ -92,7 +93,7 @@ open class HIPBackend: CPUBackend, @unchecked Sendable {
     }
     ctx = c
     super.init()
-    try check(hc_set_batching(ctx, batching))
+    try check(hc_set_batching(ctx, batching, idleAfter))
   }
 
   deinit { hc_shutdown(ctx) }

@@ -30,6 +30,9 @@ def hip_backend():
     backend = HIPBackend()
     yield backend
     backend.sync()
+    if os.environ.get("HCHIP_BATCHING"):   # a run of the whole suite with batching on: say how much of it was batched
+        print("\nHCHIP_BATCHING=%s: launches listed / enqueued: %d / %d"
+              % ((os.environ["HCHIP_BATCHING"],) + backend.batchingStats()))
 
 
 class _Switches:

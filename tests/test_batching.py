@@ -162,10 +162,32 @@ def test_config5_forward_pass_batch_limits(hip_backend):
         model = Transformer(dtype=F16)
         ids = Tensor(data=rng.integers(0, 8192, size=(8, 256)))
         want = model(ids).numpy().copy()
-        for limit in (50, 4096):
-            with hip_backend.batching(limit):
-                got = model(ids).numpy()
-            assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), "limit %d" % limit
+        for limit, idle_after in ((50, 0), (4096, 0), (256, 16), (64, 1)):
+            with hip_backend.batching(limit, idle_after):
+                for _ in range(2):
+                    got = model(ids).numpy()
+                    assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), "limit %d, %d" % (limit, idle_after)
+
+
+def test_a_device_that_has_run_dry_gets_the_list_early(hip_backend):
+    """idle_after: with nothing left on the stream, a list of at least that many launches is
+    enqueued when the caller lets go of its intermediates (hc_free with at most one buffer of the
+    batch still held), long before the limit."""
+    n = 1 << 16
+    x = hip_backend.upload(np.full(n, 0.25, np.float32))
+    want = x
+    for _ in range(6):
+        want = hip_backend.elemwise(want, ElemwiseOp.exp if _ % 2 == 0 else ElemwiseOp.log, None, n, F32)
+    want = want.onCPU().copy()
+    hip_backend.sync()
+    with hip_backend.batching(1000, 2):
+        before = hip_backend.batchingStats()
+        y = x
+        for i in range(6):
+            y = hip_backend.elemwise(y, ElemwiseOp.exp if i % 2 == 0 else ElemwiseOp.log, None, n, F32)   # releases the previous y
+        early = hip_backend.batchingStats()[1] - before[1]
+        assert np.array_equal(y.onCPU(), want)
+    assert early >= 2, early
 
 
 def test_concurrent_op_chains_under_batching(hip_backend):
@@ -184,7 +206,7 @@ def test_concurrent_op_chains_under_batching(hip_backend):
         except Exception as e:
             failures.append("thread %d: %r" % (t, e))
 
-    with hip_backend.batching(32):
+    with hip_backend.batching(32, 4):
         pool = [threading.Thread(target=worker, args=(t,)) for t in range(threads)]
         for th in pool:
             th.start()
