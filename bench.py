@@ -11,7 +11,7 @@ Also reported in the same line:
                 from HIP events recorded on the backend's own stream inside the timed region
   cpu_baseline  the reference CPUBackend algorithm (oracle/cpu_ref.c restatement, the literal
                 single-thread triple loop) timed on this box's host cores on a bounded row slab;
-                extra.cpu_reference_path holds the same for configs 1 and 4 (sgemm through OpenBLAS
+                extra.cpu_reference_path holds the same for configs 1, 3, 4 and 5 (sgemm through OpenBLAS
                 with its thread count, the bandwidth-bound ops on one thread)
   extra         the other benchmark configurations: fp32 1024^3, the ragged fp16 sweep, attention-shaped
                 batched GEMMs, the bandwidth-bound ops at [8192,4096] with GB/s against the 8 TB/s
@@ -348,7 +348,7 @@ def cpu_baseline(a, b, budget_s=20.0):
     }
 
 
-def cpu_reference_ops(budget_s=15.0):
+def cpu_reference_ops(budget_s=25.0):
     """Configs 1 and 4 on the host cores the way the reference CPUBackend would run them on Linux:
     the fp32 NN product through cblas_sgemm (the stand-in for vDSP_mmul, BackendCPU.swift:1256;
     here numpy's bundled OpenBLAS, all the threads it takes) and through the literal loop, and the
@@ -438,9 +438,36 @@ def cpu_reference_ops(budget_s=15.0):
     ids = ob.upload(np.random.default_rng(9).integers(0, 32000, size=(65536,)))
     emb = ScatterGatherIndices([32000, 1024], 0, BroadcastData(BroadcastStrides([65536, 1024], [1, 0]), ids))
     timed("cfg4_embedding_gather", lambda: ob.gather(table, emb, F32), nbytes=65536 * 8 + 2 * 65536 * 1024 * 4)
+    # config 3 on 4 of its 32 heads (the per-head cost does not depend on the head), fp16 through the
+    # CPUBackend's whole-buffer conversions: q k^T, the scale, x v
+    F16 = DType.float16
+    heads = 4
+    rng3 = np.random.default_rng(3)
+    q, k_, v = (ob.upload(rng3.standard_normal((heads, 512, 64)).astype(np.float16)) for _ in range(3))
+    scores = ob.batchedMatmul(heads, q, False, k_, True, False, 512, 64, 512, F16)
+    timed("cfg3_qk_t_4_of_32_heads", lambda: ob.batchedMatmul(heads, q, False, k_, True, False, 512, 64, 512, F16),
+          flops=2.0 * heads * 512 * 512 * 64)
+    timed("cfg3_scale_4_of_32_heads", lambda: ob.binaryOp(scores, 0.125, NumericBinaryOp.mul, F16, count=heads * 512 * 512),
+          nbytes=2 * heads * 512 * 512 * 2)
+    timed("cfg3_pv_4_of_32_heads", lambda: ob.batchedMatmul(heads, scores, False, v, False, False, 512, 512, 64, F16),
+          flops=2.0 * heads * 512 * 512 * 64)
+    # config 5 on one of its 8 sequences (256 tokens, 12.6 GFLOP), fp32: the whole forward pass of the
+    # front-end mirror over the CPUBackend restatement
+    if spent[0] <= budget_s:
+        from honeycrisp_amd.nn import Transformer
+        from honeycrisp_amd.tensor import Tensor
+        with ob.use():
+            model = Transformer(dtype=F32)
+            ids5 = Tensor(data=np.random.default_rng(5).integers(0, 8192, size=(1, 256)))
+            timed("cfg5_transformer_fwd_f32_1_of_8_sequences", lambda: model(ids5).numpy())
+        r = out.get("cfg5_transformer_fwd_f32_1_of_8_sequences")
+        if r:
+            r["tokens_per_s"] = round(256 / (r["ms"] * 1e-3), 1)
+            r["tflops"] = round(100.9e9 / 8 / (r["ms"] * 1e-3) / 1e12, 5)
     out["note"] = ("host cores of this box; the fp32 product through numpy's bundled OpenBLAS and through vDSP_mmul of "
                    "the Linux Accelerate stand-in (which forwards to the cblas_sgemm named in `blas`), everything else "
-                   "the CPUBackend restatement on one thread, full-size inputs")
+                   "the CPUBackend restatement on one thread; full-size inputs for configs 1 and 4, 4 of 32 heads for "
+                   "config 3, one of 8 sequences for config 5")
     return out
 
 

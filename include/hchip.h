@@ -174,12 +174,14 @@ int hc_launch_host_func(hc_ctx* ctx, void (*fn)(void*), void* user);
  *      [cast ->] normalize -> [(gain + c) *, + bias] -> [cast]      one LayerNorm kernel
  *      [* s ->] [+ mask ->] logSoftmax -> [exp]                     one softmax kernel
  *      swap of two batch axes -> batchedMatmul -> swap back         read / written through strides
+ *      q k^T -> that softmax kernel -> x v, 64-wide fp16 heads,
+ *      T a multiple of 64 up to 512                                 one attention kernel
  *      products of one shape over the same input (q, k, v)          one launch
  *    Buffers that only held merged intermediates are never written by a replay.
- *    HCHIP_RECORDING_LOG=1 at hc_capture_end lists the launches of the rewritten recording on
- *    stderr; HCHIP_GRAPH_AS_LAUNCHES=1 makes hc_graph_launch issue them one by one instead of
- *    through hipGraphLaunch (for kernel traces).
- *    HCHIP_NO_FUSION=1 in the environment at hc_capture_end turns the rewrite off. */
+ *    Switches (environment at hc_init, or hc_debug_set): HCHIP_RECORDING_LOG=1 lists the
+ *    launches of the rewritten recording on stderr at hc_capture_end; HCHIP_GRAPH_AS_LAUNCHES=1
+ *    makes hc_graph_launch issue them one by one instead of through hipGraphLaunch (for kernel
+ *    traces); HCHIP_NO_FUSION=1 when a capture begins turns its rewrite off. */
 typedef struct hc_graph hc_graph;
 int hc_capture_begin(hc_ctx* ctx);
 int hc_capture_end(hc_ctx* ctx, hc_graph** out);
