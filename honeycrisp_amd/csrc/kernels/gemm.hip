@@ -273,7 +273,29 @@ template <typename T, int TQ> __device__ __forceinline__ void skinny_k_impl(cons
   float acc[TQ];
 #pragma unroll
   for (int q = 0; q < TQ; q++) acc[q] = 0.0f;
-  for (uint32_t k0 = lane * V; k0 < a.K; k0 += 64 * V) {
+  // U steps at a time with all their loads issued first (a row is a handful of steps: one load in
+  // flight per lane would make it as many memory latencies in a row); the sums are formed in the
+  // order of the plain loop below, which takes what is left
+  constexpr int U = 8;
+  uint32_t k0 = lane * V;
+  for (; k0 + (U - 1) * 64 * V + V <= a.K; k0 += U * 64 * V) {
+    T x[U][V];
+#pragma unroll
+    for (int u = 0; u < U; u++) load_vec_loose<T, V>(X + k0 + u * 64 * V, x[u]);
+#pragma unroll
+    for (int q = 0; q < TQ; q++) {
+      if (q < (int)a.t) {
+        T y[U][V];
+#pragma unroll
+        for (int u = 0; u < U; u++) load_vec<T, V>(Y + (size_t)q * a.y_qs, k0 + u * 64 * V, 1, y[u]);
+#pragma unroll
+        for (int u = 0; u < U; u++)
+#pragma unroll
+          for (int e = 0; e < V; e++) acc[q] = acc[q] + (float)x[u][e] * (float)y[u][e];
+      }
+    }
+  }
+  for (; k0 < a.K; k0 += 64 * V) {
     T x[V];
     if (k0 + V <= a.K) {
       load_vec_loose<T, V>(X + k0, x);   // (rows of X start at any element)
@@ -325,8 +347,29 @@ template <typename T, int TQ> __device__ __forceinline__ void skinny_p_impl(cons
 #pragma unroll
     for (int e = 0; e < V; e++) acc[q][e] = 0.0f;
   const bool whole = p0 + V <= a.L;
-#pragma unroll 2
-  for (uint32_t k = k_lo + wave; k < k_hi; k += WAVES) {
+  uint32_t k = k_lo + wave;
+  if (whole) {
+    // U of this wave's k-rows at a time, loads first (see skinny_k_impl), sums in the plain loop's order
+    constexpr int U = 6;
+    for (; k + (U - 1) * WAVES < k_hi; k += U * WAVES) {
+      T x[U][V];
+#pragma unroll
+      for (int u = 0; u < U; u++) load_vec_loose<T, V>(X + (size_t)(k + u * WAVES) * a.x_ks + p0, x[u]);
+#pragma unroll
+      for (int q = 0; q < TQ; q++) {
+        if (q < (int)a.t) {
+          float y[U];
+#pragma unroll
+          for (int u = 0; u < U; u++) y[u] = (float)Y[(size_t)q * a.y_qs + (size_t)(k + u * WAVES) * a.y_ks];
+#pragma unroll
+          for (int u = 0; u < U; u++)
+#pragma unroll
+            for (int e = 0; e < V; e++) acc[q][e] = acc[q][e] + (float)x[u][e] * y[u];
+        }
+      }
+    }
+  }
+  for (; k < k_hi; k += WAVES) {
     T x[V];
     if (whole) {
       load_vec_loose<T, V>(X + (size_t)k * a.x_ks + p0, x);   // (k-rows of X start at any element)
