@@ -84,8 +84,9 @@ open class HIPBackend: CPUBackend, @unchecked Sendable {
   /// residual go into the product's kernel, LayerNorm / softmax / attention become one kernel
   /// each) with the bits of the call-by-call result; anything that reads or waits for a result
   /// (`Tensor.Data.onCPU`, `wait()`) enqueues what is listed first, and so does a device that has
-  /// run out of work once `idleAfter` launches are listed. 0 = one launch per call.
-  public init(device: Int = 0, batching: Int = 0, idleAfter: Int = 16) throws {
+  /// run out of work once `idleAfter` launches are listed. `batching: 0` = one launch per call
+  /// (what the C ABI does unless told otherwise).
+  public init(device: Int = 0, batching: Int = 256, idleAfter: Int = 16) throws {
     var c: OpaquePointer? = nil
     let status = hc_init(Int32(device), &c)
     guard status == HC_OK.rawValue, let c = c else {
