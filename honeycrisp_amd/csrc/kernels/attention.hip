@@ -28,9 +28,117 @@
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef uint32_t Chunk __attribute__((ext_vector_type(4)));
 #define LDS_AS __attribute__((address_space(3)))
+
+// Workgroup barrier for LDS traffic only: this wave's LDS accesses are done (lgkmcnt), nothing is said
+// about loads from memory that are still on their way into registers.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_waitcnt(0xC07F);
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
+// Phase 2 of the kernel below: the softmax chain over the BQ rows of the score tile in LDS, in place.
+// NCH = vectors of eight scores a lane holds per row. `n` is the row length the lanes test their
+// vectors against: the caller passes a constant (the full NCH * LANES * 8) when T fills the vectors
+// exactly, and the tests fold away: straight-line code, where the tested form has an exec-mask
+// branch around every vector of every step.
+template <int LANES, int NCH, uint32_t BQ, uint32_t SP>
+__device__ __forceinline__ void attention_softmax_rows(const hck_attention_args& p, char* s_lds, const uint32_t n, const uint32_t T,
+                                                       const uint32_t z, const uint32_t m0) {
+  const uint32_t tid = threadIdx.x;
+  typedef RowRegs<half_t, LANES, NCH> Row;
+  constexpr int VEC = Row::VEC, CHUNKS = Row::CHUNKS;
+  constexpr uint32_t TEAMS = HCK_BLOCK / LANES;       // rows the workgroup's teams take in one go
+  constexpr int R = TEAMS * 8 <= BQ ? 8 : BQ / TEAMS;  // 8 rows per team at a time (2 with 32 teams)
+  static_assert(BQ % (TEAMS * R) == 0, "the teams' passes cover the tile exactly");
+  const uint32_t tl = tid % LANES, team = tid / LANES;
+  const bool then_exp = (p.flags & HCK_SM_EXP) != 0;
+  for (uint32_t first = team * R; first < BQ; first += TEAMS * R) {
+    Row r[R];
+#pragma unroll
+    for (int j = 0; j < R; j++) r[j].load((const half_t*)(s_lds + (first + j) * SP), n, tl);
+    // Two of the chain's steps are fp16 in, fp16 out with one operation in between, formed in fp32 by
+    // the separate kernels: x * s and x + mask. With both operands fp16 values the fp32 result is exact
+    // (product: 22 significant bits) or rounds innocuously twice (sum: fp32 has 2 * 11 + 2 bits), so the
+    // packed fp16 instruction returns the same bits at an eighth of the instructions (no conversions,
+    // two elements each). The scale qualifies when it is an fp16 value itself (1 / 8 is), which is
+    // wave-uniform; otherwise the fp32 form stays.
+    if (p.flags & HCK_SM_SCALE) {
+      const float s = p.scale;
+      const half_t s16 = (half_t)s;
+      if ((float)s16 == s) {
+        const half2_t s2 = {s16, s16};
+#pragma unroll
+        for (int j = 0; j < R; j++)
+#pragma unroll
+          for (int c = 0; c < CHUNKS; c++)
+#pragma unroll
+            for (int i = 0; i < VEC; i += 2) {
+              const half2_t x = {r[j].v[c][i], r[j].v[c][i + 1]};
+              const half2_t y = x * s2;
+              r[j].v[c][i] = y[0], r[j].v[c][i + 1] = y[1];
+            }
+      } else {
+#pragma unroll
+        for (int j = 0; j < R; j++)
+#pragma unroll
+          for (int c = 0; c < CHUNKS; c++)
+#pragma unroll
+            for (int i = 0; i < VEC; i++) r[j].v[c][i] = narrow<half_t>((float)r[j].v[c][i] * s);
+      }
+    }
+    if (p.flags & HCK_SM_MASK) {
+      Row m[R];
+#pragma unroll
+      for (int j = 0; j < R; j++) {
+        const uint64_t grow = (uint64_t)z * T + m0 + first + j;  // this row among all score rows
+        m[j].load((const half_t*)p.mask + (size_t)(grow % p.mask_rows) * T, n, tl);
+      }
+#pragma unroll
+      for (int j = 0; j < R; j++)
+#pragma unroll
+        for (int c = 0; c < CHUNKS; c++)
+          if ((tl + LANES * c) * VEC < n) {
+#pragma unroll
+            for (int i = 0; i < VEC; i += 2) {
+              const half2_t x = {r[j].v[c][i], r[j].v[c][i + 1]}, y = {m[j].v[c][i], m[j].v[c][i + 1]};
+              const half2_t z = x + y;
+              r[j].v[c][i] = z[0], r[j].v[c][i + 1] = z[1];
+            }
+          }
+    }
+    float mx[R], sum[R];
+#pragma unroll
+    for (int j = 0; j < R; j++) {
+      mx[j] = -INFINITY;
+      r[j].each(n, tl, [&](float x) { if (x > mx[j]) mx[j] = x; });
+    }
+#pragma unroll
+    for (int j = 0; j < R; j++) mx[j] = team_reduce<LANES>(mx[j], MaxOp());
+#pragma unroll
+    for (int j = 0; j < R; j++) {
+      sum[j] = 0.0f;
+      r[j].each(n, tl, [&](float x) { sum[j] += exp_in<half_t>(x - mx[j]); });
+    }
+#pragma unroll
+    for (int j = 0; j < R; j++) sum[j] = team_reduce<LANES>(sum[j], SumOp());
+#pragma unroll
+    for (int j = 0; j < R; j++) {
+      const float log_sum = logf(sum[j]) + mx[j];
+      r[j].store((half_t*)(s_lds + (first + j) * SP), n, tl, [&](float x) {
+        const float ls = x - log_sum;
+        if (!then_exp) return ls;
+        const float stored = (float)narrow<half_t>(ls);
+        return exp_hw(stored) * 1.0f;
+      });
+    }
+  }
+}
 
 template <int TMAX, int LANES> __device__ __forceinline__ void attention_impl(const hck_attention_args& p) {
   constexpr uint32_t BQ = 64;
@@ -60,25 +168,30 @@ template <int TMAX, int LANES> __device__ __forceinline__ void attention_impl(co
 #else
 #define HC_TS(i)
 #endif
-  // ---- phase 0
-  Chunk vreg[KV_CHUNKS];
+  // ---- phase 0: q and k first, v behind them: v is not needed before phase 3, so its loads stay in flight
+  // through the scores (the barrier below waits for LDS only, not for them)
+#pragma unroll
+  for (int i = 0; i < (int)(BQ * 8 / HCK_BLOCK); i++) {
+    const uint32_t piece = i * HCK_BLOCK + tid, r = piece >> 3, c = piece & 7;
+    *reinterpret_cast<Chunk*>(q_lds + r * 128 + ((c ^ (r & 7)) * 16)) = *reinterpret_cast<const Chunk*>(Q + (size_t)r * p.q_rs + c * 8);
+  }
+  Chunk kreg[KV_CHUNKS], vreg[KV_CHUNKS];
+#pragma unroll
+  for (int i = 0; i < KV_CHUNKS; i++) {
+    const uint32_t piece = i * HCK_BLOCK + tid, r = piece >> 3, c = piece & 7;
+    if (r < T) kreg[i] = *reinterpret_cast<const Chunk*>(K + (size_t)r * p.k_rs + c * 8);
+  }
 #pragma unroll
   for (int i = 0; i < KV_CHUNKS; i++) {
     const uint32_t piece = i * HCK_BLOCK + tid, r = piece >> 3, c = piece & 7;
     if (r < T) vreg[i] = *reinterpret_cast<const Chunk*>(V + (size_t)r * p.v_rs + c * 8);
   }
 #pragma unroll
-  for (int i = 0; i < (int)(BQ * 8 / HCK_BLOCK); i++) {
-    const uint32_t piece = i * HCK_BLOCK + tid, r = piece >> 3, c = piece & 7;
-    *reinterpret_cast<Chunk*>(q_lds + r * 128 + ((c ^ (r & 7)) * 16)) = *reinterpret_cast<const Chunk*>(Q + (size_t)r * p.q_rs + c * 8);
-  }
-#pragma unroll
   for (int i = 0; i < KV_CHUNKS; i++) {
     const uint32_t piece = i * HCK_BLOCK + tid, r = piece >> 3, c = piece & 7;
-    if (r < T)
-      *reinterpret_cast<Chunk*>(kv_lds + r * 128 + ((c ^ (r & 7)) * 16)) = *reinterpret_cast<const Chunk*>(K + (size_t)r * p.k_rs + c * 8);
+    if (r < T) *reinterpret_cast<Chunk*>(kv_lds + r * 128 + ((c ^ (r & 7)) * 16)) = kreg[i];
   }
-  __syncthreads();
+  lds_barrier();
   HC_TS(1);
 
   // ---- phase 1: scores
@@ -135,68 +248,13 @@ template <int TMAX, int LANES> __device__ __forceinline__ void attention_impl(co
     // (vectors per lane: what rows of TMAX elements need, at most the row kernel's four)
     constexpr int NCH = (TMAX + LANES * 8 - 1) / (LANES * 8);
     static_assert(NCH <= 4, "rows of TMAX elements fit the team's registers");
-    typedef RowRegs<half_t, LANES, NCH> Row;
-    constexpr int VEC = Row::VEC, CHUNKS = Row::CHUNKS;
-    constexpr uint32_t TEAMS = HCK_BLOCK / LANES;       // rows the workgroup's teams take in one go
-    constexpr int R = TEAMS * 8 <= BQ ? 8 : BQ / TEAMS;  // 8 rows per team at a time (2 with 32 teams)
-    static_assert(BQ % (TEAMS * R) == 0, "the teams' passes cover the tile exactly");
-    const uint32_t tl = tid % LANES, team = tid / LANES;
-    const bool then_exp = (p.flags & HCK_SM_EXP) != 0;
-    for (uint32_t first = team * R; first < BQ; first += TEAMS * R) {
-      Row r[R];
-#pragma unroll
-      for (int j = 0; j < R; j++) r[j].load((const half_t*)(s_lds + (first + j) * SP), T, tl);
-      if (p.flags & HCK_SM_SCALE) {
-        const float s = p.scale;
-#pragma unroll
-        for (int j = 0; j < R; j++)
-#pragma unroll
-          for (int c = 0; c < CHUNKS; c++)
-#pragma unroll
-            for (int i = 0; i < VEC; i++) r[j].v[c][i] = narrow<half_t>((float)r[j].v[c][i] * s);
-      }
-      if (p.flags & HCK_SM_MASK) {
-        Row m[R];
-#pragma unroll
-        for (int j = 0; j < R; j++) {
-          const uint64_t grow = (uint64_t)z * T + m0 + first + j;  // this row among all score rows
-          m[j].load((const half_t*)p.mask + (size_t)(grow % p.mask_rows) * T, T, tl);
-        }
-#pragma unroll
-        for (int j = 0; j < R; j++)
-#pragma unroll
-          for (int c = 0; c < CHUNKS; c++)
-            if ((tl + LANES * c) * VEC < T) {
-#pragma unroll
-              for (int i = 0; i < VEC; i++) r[j].v[c][i] = narrow<half_t>((float)r[j].v[c][i] + (float)m[j].v[c][i]);
-            }
-      }
-      float mx[R], sum[R];
-#pragma unroll
-      for (int j = 0; j < R; j++) {
-        mx[j] = -INFINITY;
-        r[j].each(T, tl, [&](float x) { if (x > mx[j]) mx[j] = x; });
-      }
-#pragma unroll
-      for (int j = 0; j < R; j++) mx[j] = team_reduce<LANES>(mx[j], MaxOp());
-#pragma unroll
-      for (int j = 0; j < R; j++) {
-        sum[j] = 0.0f;
-        r[j].each(T, tl, [&](float x) { sum[j] += exp_in<half_t>(x - mx[j]); });
-      }
-#pragma unroll
-      for (int j = 0; j < R; j++) sum[j] = team_reduce<LANES>(sum[j], SumOp());
-#pragma unroll
-      for (int j = 0; j < R; j++) {
-        const float log_sum = logf(sum[j]) + mx[j];
-        r[j].store((half_t*)(s_lds + (first + j) * SP), T, tl, [&](float x) {
-          const float ls = x - log_sum;
-          if (!then_exp) return ls;
-          const float stored = (float)narrow<half_t>(ls);
-          return exp_hw(stored) * 1.0f;
-        });
-      }
-    }
+    constexpr uint32_t FULL = LANES * 8;   // scores per vector round of a team
+    // T is a multiple of 64 (the host's condition): with teams of 8 lanes it fills T / 64 rounds exactly
+    if (T == NCH * FULL) attention_softmax_rows<LANES, NCH, BQ, SP>(p, s_lds, NCH * FULL, T, z, m0);
+    else if (NCH > 1 && T == (NCH - 1) * FULL) attention_softmax_rows<LANES, (NCH > 1 ? NCH - 1 : 1), BQ, SP>(p, s_lds, (NCH - 1) * FULL, T, z, m0);
+    else if (NCH > 2 && T == (NCH - 2) * FULL) attention_softmax_rows<LANES, (NCH > 2 ? NCH - 2 : 1), BQ, SP>(p, s_lds, (NCH - 2) * FULL, T, z, m0);
+    else if (NCH > 3 && T == (NCH - 3) * FULL) attention_softmax_rows<LANES, (NCH > 3 ? NCH - 3 : 1), BQ, SP>(p, s_lds, (NCH - 3) * FULL, T, z, m0);
+    else attention_softmax_rows<LANES, NCH, BQ, SP>(p, s_lds, T, T, z, m0);
   }
   __syncthreads();
   HC_TS(3);
