@@ -194,6 +194,7 @@ struct hc_ctx {
   // bucket size, and go back to the pool when the batch has been enqueued.
   size_t batch_limit = 0;               // launches per batch at most; 0 = every launch is enqueued at once
   size_t batch_idle_after = 0;          // > 0: a list this long is also enqueued when the stream has run dry (see hc_free)
+  size_t batch_idle_now = 0;            // ... the length that applies at the moment (see flush_batch_locked)
   std::unordered_set<void*> batch_born; // blocks handed out since the last batch was enqueued and still in use
   // "has the stream run dry" without a call into the runtime: behind every batch a one-lane
   // kernel stores the batch's number into pinned host memory, which hc_free compares with the
@@ -276,6 +277,7 @@ extern "C" int hc_init(int device, hc_ctx** out) {
     char* end = nullptr;
     ctx->batch_limit = (size_t)strtoull(v, &end, 10);
     ctx->batch_idle_after = end && *end == ',' ? (size_t)strtoull(end + 1, nullptr, 10) : 0;
+    ctx->batch_idle_now = ctx->batch_idle_after;
     ctx->lazy = ctx->batch_limit > 0;
   }
   e = hipGetDeviceProperties(&ctx->props, device);
@@ -421,7 +423,8 @@ static size_t bucket_size(size_t bytes) {
   return (bytes + g - 1) / g * g;
 }
 
-static int flush_batch_locked(hc_ctx* ctx);
+enum BatchEnd { BATCH_END_OTHER, BATCH_END_WAIT, BATCH_END_IDLE };
+static int flush_batch_locked(hc_ctx* ctx, BatchEnd why = BATCH_END_OTHER);
 static int batch_grew_locked(hc_ctx* ctx);
 
 static void release_cache_locked(hc_ctx* ctx) {
@@ -518,9 +521,9 @@ extern "C" int hc_free(hc_ctx* ctx, void* ptr) {
     // two layers of a model, say): every other intermediate has been released, so no chain that
     // the rewrite could merge is open. There, once the list is long enough to be worth a
     // rewrite, look whether the stream has run dry.
-    if (ctx->batch_idle_after > 0 && ctx->batch_launches >= ctx->batch_idle_after && ctx->batch_born.size() <= 1 &&
+    if (ctx->batch_idle_after > 0 && ctx->batch_launches >= ctx->batch_idle_now && ctx->batch_born.size() <= 1 &&
         ctx->batch_done && __atomic_load_n(ctx->batch_done, __ATOMIC_ACQUIRE) == ctx->batch_seq)
-      return flush_batch_locked(ctx);
+      return flush_batch_locked(ctx, BATCH_END_IDLE);
   } else {
     ctx->free_blocks[b].push_back(ptr);
     ctx->bytes_cached += b;
@@ -623,7 +626,7 @@ static int copy(hc_ctx* ctx, void* dst, const void* src, size_t bytes, hipMemcpy
     // index vectors in the middle of a forward pass); everything else enqueues the list first.
     if (!ctx->capturing && !ctx->pending.empty() && kind != hipMemcpyDeviceToDevice &&
         (kind != hipMemcpyHostToDevice || batch_touches_locked(ctx, dst)))
-      HC_TRY(flush_batch_locked(ctx));
+      HC_TRY(flush_batch_locked(ctx, BATCH_END_WAIT));
     if (kind == hipMemcpyHostToDevice && wait && bytes <= kStageMax && ctx->stage) {
       // The caller may reuse `src` as soon as this returns: copy it into pinned memory and let the
       // stream pick it up from there. No wait, so the device keeps running what is already queued
@@ -698,7 +701,7 @@ extern "C" int hc_sync(hc_ctx* ctx) {
   {
     std::lock_guard<std::mutex> lock(ctx->mu);
     REQUIRE(!ctx->capturing, "hc_sync: not allowed while capturing");
-    HC_TRY(flush_batch_locked(ctx));
+    HC_TRY(flush_batch_locked(ctx, BATCH_END_WAIT));
   }
   HIP_TRY(hipStreamSynchronize(ctx->stream));
   return HC_OK;
@@ -720,7 +723,7 @@ extern "C" int hc_event_record(hc_ctx* ctx, hc_event* ev) {
   REQUIRE(ctx && ev, "hc_event_record: null argument");
   std::lock_guard<std::mutex> lock(ctx->mu);
   REQUIRE(!ctx->capturing, "hc_event_record: not allowed while capturing");
-  HC_TRY(flush_batch_locked(ctx));
+  HC_TRY(flush_batch_locked(ctx, BATCH_END_WAIT));
   HIP_TRY(hipEventRecord(ev->ev, ctx->stream));
   return HC_OK;
 }
@@ -760,7 +763,7 @@ extern "C" int hc_launch_host_func(hc_ctx* ctx, void (*fn)(void*), void* user) {
   REQUIRE(ctx && fn, "hc_launch_host_func: null argument");
   std::lock_guard<std::mutex> lock(ctx->mu);
   REQUIRE(!ctx->capturing, "hc_launch_host_func: not allowed while capturing");
-  HC_TRY(flush_batch_locked(ctx));
+  HC_TRY(flush_batch_locked(ctx, BATCH_END_WAIT));
   HIP_TRY(hipLaunchHostFunc(ctx->stream, fn, user));
   return HC_OK;
 }
@@ -823,7 +826,7 @@ static void log_launches_locked(const hc_ctx* ctx, const char* what) {
 // since the last batch go back to the pool (in stream order behind the launches that used them,
 // which is what the pool assumes of every block it holds). Nothing to do outside batching, or
 // during a capture (whose list is the capture's). Caller holds the lock.
-static int flush_batch_locked(hc_ctx* ctx) {
+static int flush_batch_locked(hc_ctx* ctx, BatchEnd why) {
   if (ctx->capturing || ctx->batch_limit == 0) return HC_OK;
   int status = HC_OK;
   if (!ctx->pending.empty()) {
@@ -849,6 +852,13 @@ static int flush_batch_locked(hc_ctx* ctx) {
   }
   ctx->batch_launches = 0;
   ctx->batch_born.clear();
+  // An early batch pays for itself when the device would otherwise sit idle until a wait (a program
+  // that reads a result after every pass): the first one goes out after idle_after launches. Every
+  // early batch doubles the length the next one needs, so that a program that never waits, and
+  // whose device runs dry because the host is the slower side, ends up with full batches (fewer
+  // rewrites and launches on the host, which is what it is short of); a wait starts over.
+  if (why == BATCH_END_IDLE) ctx->batch_idle_now = std::min(ctx->batch_idle_now * 2, ctx->batch_limit);
+  else if (why == BATCH_END_WAIT) ctx->batch_idle_now = ctx->batch_idle_after;
   for (auto& kv : ctx->batch_parked) {
     auto& pool = ctx->free_blocks[kv.first];
     pool.insert(pool.end(), kv.second.begin(), kv.second.end());
@@ -878,6 +888,7 @@ extern "C" int hc_set_batching(hc_ctx* ctx, size_t max_launches, size_t idle_aft
   if (idle_after > 0 && !ctx->batch_done) HC_TRY(alloc_batch_flag_locked(ctx));
   ctx->batch_limit = max_launches;
   ctx->batch_idle_after = idle_after;
+  ctx->batch_idle_now = idle_after;
   ctx->lazy = max_launches > 0;
   return HC_OK;
 }

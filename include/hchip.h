@@ -202,7 +202,11 @@ int hc_graph_destroy(hc_ctx* ctx, hc_graph* graph);
  *    while the device has finished everything enqueued so far: looked up in hc_free when the
  *    caller holds at most one buffer allocated since the last batch (between two layers of a
  *    model: every other intermediate is released, so no chain the rewrite could merge is cut).
- *    While the device is busy a batch grows; once it has run dry it gets what there is,
+ *    While the device is busy a batch grows; once it has run dry it gets what there is. Every
+ *    batch that goes out early this way doubles the number of launches the next early one needs
+ *    (up to max_launches); a call that waits or transfers starts over at idle_after: a program
+ *    that reads a result after every pass gets its device started after idle_after launches,
+ *    one that never waits and keeps the device short of work ends up with full batches,
  *  - before anything that must see or order against the results: hc_memcpy_d2h (Tensor.Data.onCPU),
  *    hc_sync, hc_event_record, hc_launch_host_func (Tensor.Data.wait), hc_graph_launch,
  *    hc_capture_begin, hc_trim, hc_flush; an upload is enqueued at once and overtakes the list
