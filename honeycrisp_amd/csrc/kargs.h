@@ -406,4 +406,15 @@ typedef struct {
   uint64_t x_bs, y_bs, c_bs;
 } hck_skinny_args;
 
+/* hc_gemm_skinny_pair_*: two independent skinny launches as one. Workgroups [0, split) run `a`,
+ * [split, split + blocks_b) run `b`, each with the kernel its kind names. */
+#define HCK_SKINNY_K 0u     /* hc_gemm_skinny_k_*    */
+#define HCK_SKINNY_P 1u     /* hc_gemm_skinny_p_*    */
+#define HCK_SKINNY_PACK 2u  /* hc_gemm_skinny_pack_* */
+#define HCK_SKINNY_STORE 3u /* hc_gemm_skinny_store_* */
+typedef struct {
+  hck_skinny_args a, b;
+  uint32_t split, blocks_b, kind_a, kind_b;
+} hck_skinny_pair_args;
+
 #endif

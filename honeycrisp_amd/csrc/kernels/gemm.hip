@@ -262,10 +262,10 @@ HC_KERNEL void hc_gemm_i64(hck_gemm_args p) {
 //
 // Long operand contiguous along k: one wave per p. Lanes stride over k in 16-byte pieces, keep
 // one partial sum per q, and the wave adds them up at the end.
-template <typename T, int TQ> __device__ __forceinline__ void skinny_k_impl(const hck_skinny_args& a) {
+template <typename T, int TQ> __device__ __forceinline__ void skinny_k_impl(const hck_skinny_args& a, const uint32_t block) {
   constexpr int V = 16 / sizeof(T);
   const uint32_t lane = threadIdx.x & 63;
-  const uint32_t p = blockIdx.x * (HCK_BLOCK / 64) + (threadIdx.x >> 6);
+  const uint32_t p = block * (HCK_BLOCK / 64) + (threadIdx.x >> 6);
   if (p >= a.L) return;
   const T* X = (const T*)a.x + (uint64_t)blockIdx.y * a.x_bs + (size_t)p * a.x_ps;
   const T* Y = (const T*)a.y + (uint64_t)blockIdx.y * a.y_bs;
@@ -331,12 +331,12 @@ template <typename T, int TQ> __device__ __forceinline__ void skinny_k_impl(cons
 // own of an fp32 buffer and hc_gemm_skinny_store adds the slices in chunk order and rounds, so
 // the result does not depend on which workgroup finishes first. Y is read one element per wave
 // and step (wave-uniform), so it is taken as it lies, whatever its strides.
-template <typename T, int TQ> __device__ __forceinline__ void skinny_p_impl(const hck_skinny_args& a) {
+template <typename T, int TQ> __device__ __forceinline__ void skinny_p_impl(const hck_skinny_args& a, const uint32_t block) {
   constexpr int V = 16 / sizeof(T), WAVES = HCK_BLOCK / 64, TILE = 64 * V;
   __shared__ float part[WAVES][TQ][TILE];
   const uint32_t lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const uint32_t ptiles = (a.L + TILE - 1) / TILE;
-  const uint32_t chunk = blockIdx.x / ptiles, pt = blockIdx.x - chunk * ptiles;
+  const uint32_t chunk = block / ptiles, pt = block - chunk * ptiles;
   const uint32_t p0 = pt * TILE + lane * V;
   const uint32_t k_lo = chunk * a.kchunk, k_hi = k_lo + a.kchunk < a.K ? k_lo + a.kchunk : a.K;
   const T* X = (const T*)a.x + (uint64_t)blockIdx.y * a.x_bs;
@@ -404,8 +404,8 @@ template <typename T, int TQ> __device__ __forceinline__ void skinny_p_impl(cons
 
 // Y[k, q] (any strides) -> packed[q][k], rows padded with zeros to `y_qs` elements (a multiple of
 // a 16-byte piece): a.c = packed, a.y = source, strides of the source in y_ks / c_qs.
-template <typename T> __device__ __forceinline__ void skinny_pack_impl(const hck_skinny_args& a) {
-  const uint64_t i = (uint64_t)blockIdx.x * HCK_BLOCK + threadIdx.x;
+template <typename T> __device__ __forceinline__ void skinny_pack_impl(const hck_skinny_args& a, const uint32_t block) {
+  const uint64_t i = (uint64_t)block * HCK_BLOCK + threadIdx.x;
   if (i >= (uint64_t)a.t * a.y_qs) return;
   const uint32_t q = (uint32_t)(i / a.y_qs), k = (uint32_t)(i - (uint64_t)q * a.y_qs);
   const T* Y = (const T*)a.y + (uint64_t)blockIdx.y * a.y_bs;
@@ -413,8 +413,8 @@ template <typename T> __device__ __forceinline__ void skinny_pack_impl(const hck
   P[i] = k < a.K ? Y[(size_t)k * a.y_ks + (size_t)q * a.c_qs] : (T)0;
 }
 
-template <typename T> __device__ __forceinline__ void skinny_store_impl(const hck_skinny_args& a) {
-  const uint64_t i = (uint64_t)blockIdx.x * HCK_BLOCK + threadIdx.x;
+template <typename T> __device__ __forceinline__ void skinny_store_impl(const hck_skinny_args& a, const uint32_t block) {
+  const uint64_t i = (uint64_t)block * HCK_BLOCK + threadIdx.x;
   if (i >= (uint64_t)a.L * a.t) return;
   const uint32_t p = (uint32_t)(i / a.t), q = (uint32_t)(i - (uint64_t)p * a.t);
   T* C = (T*)a.c + (uint64_t)blockIdx.y * a.c_bs;
@@ -435,10 +435,28 @@ template <typename T> __device__ __forceinline__ void skinny_store_impl(const hc
   C[(size_t)p * a.c_ps + (size_t)q * a.c_qs] = narrow<T>(v);
 }
 
+// Two skinny launches that do not depend on each other (the thin fringes of a ragged product: a
+// column strip and a row strip of C) as one: workgroups below `split` work on `a`, the others on
+// `b`, each with the kernel its `kind` names and the block index it would have had on its own.
+template <typename T> __device__ __forceinline__ void skinny_pair_impl(const hck_skinny_pair_args& p) {
+  const bool first = blockIdx.x < p.split;
+  const uint32_t block = first ? blockIdx.x : blockIdx.x - p.split;
+  const uint32_t kind = first ? p.kind_a : p.kind_b;
+  const hck_skinny_args& a = first ? p.a : p.b;
+  if (block >= (first ? p.split : p.blocks_b)) return;
+  switch (kind) {
+    case HCK_SKINNY_K: skinny_k_impl<T, 4>(a, block); break;
+    case HCK_SKINNY_P: skinny_p_impl<T, 4>(a, block); break;
+    case HCK_SKINNY_PACK: skinny_pack_impl<T>(a, block); break;
+    default: skinny_store_impl<T>(a, block); break;
+  }
+}
+
 #define DEF_SKINNY(TN, T)                                                                          \
-  HC_KERNEL void hc_gemm_skinny_k_##TN##_q4(hck_skinny_args a) { skinny_k_impl<T, 4>(a); }         \
-  HC_KERNEL void hc_gemm_skinny_p_##TN##_q4(hck_skinny_args a) { skinny_p_impl<T, 4>(a); }         \
-  HC_KERNEL void hc_gemm_skinny_pack_##TN(hck_skinny_args a) { skinny_pack_impl<T>(a); }             \
-  HC_KERNEL void hc_gemm_skinny_store_##TN(hck_skinny_args a) { skinny_store_impl<T>(a); }
+  HC_KERNEL void hc_gemm_skinny_k_##TN##_q4(hck_skinny_args a) { skinny_k_impl<T, 4>(a, blockIdx.x); } \
+  HC_KERNEL void hc_gemm_skinny_p_##TN##_q4(hck_skinny_args a) { skinny_p_impl<T, 4>(a, blockIdx.x); } \
+  HC_KERNEL void hc_gemm_skinny_pack_##TN(hck_skinny_args a) { skinny_pack_impl<T>(a, blockIdx.x); }   \
+  HC_KERNEL void hc_gemm_skinny_store_##TN(hck_skinny_args a) { skinny_store_impl<T>(a, blockIdx.x); } \
+  HC_KERNEL void hc_gemm_skinny_pair_##TN(hck_skinny_pair_args p) { skinny_pair_impl<T>(p); }
 DEF_SKINNY(f16, half_t)
 DEF_SKINNY(f32, float)
