@@ -205,6 +205,8 @@ struct hc_ctx {
   std::unordered_map<size_t, std::vector<void*>> batch_parked;
   size_t batch_parked_bytes = 0;
   uint64_t batch_listed = 0, batch_enqueued = 0;   // launches and copies, since the context was created
+  int batch_failed = 0;                 // status of a batch that could not be enqueued, until a call has reported it
+  std::string batch_failed_why;
   // buffers whose only writer and only reader were merged away by the rewrite of the recording in
   // progress: no launch of the graph touches them, so they need not stay reserved for it
   std::vector<std::pair<void*, size_t>> dead;
@@ -829,24 +831,33 @@ static void log_launches_locked(const hc_ctx* ctx, const char* what) {
 static int flush_batch_locked(hc_ctx* ctx, BatchEnd why) {
   if (ctx->capturing || ctx->batch_limit == 0) return HC_OK;
   int status = HC_OK;
+  // A batch that failed to go out inside a call whose status nobody looks at (hc_free from a
+  // destructor) is reported again by the next call that would have enqueued it.
+  if (ctx->batch_failed != HC_OK) {
+    status = ctx->batch_failed;
+    g_last_error = ctx->batch_failed_why;
+    ctx->batch_failed = HC_OK;
+  }
   if (!ctx->pending.empty()) {
     ctx->lazy = false;
     for (const hc_pending& e : ctx->pending) ctx->batch_listed += e.kind != hc_pending::FREE;
     if (!ctx->sw.no_fusion) fuse_recording(ctx);
     for (const hc_pending& e : ctx->pending) ctx->batch_enqueued += e.kind != hc_pending::FREE && !e.dropped;
     if (ctx->sw.recording_log) log_launches_locked(ctx, "batch");
-    status = emit_recording_locked(ctx, ctx->pending);
+    const int emitted = emit_recording_locked(ctx, ctx->pending);
+    if (status == HC_OK) status = emitted;
     ctx->pending.clear();
     ctx->dead.clear();
-    if (status == HC_OK && ctx->batch_idle_after > 0 && ctx->batch_done) {
+    if (emitted == HC_OK && ctx->batch_idle_after > 0 && ctx->batch_done) {
       hck_map_args k;
       memset(&k, 0, sizeof(k));
       k.out = ctx->batch_done;
       k.count = 1;
       k.i0 = (int64_t)++ctx->batch_seq;
       hipFunction_t fn = nullptr;
-      status = find_kernel_locked(ctx, "hc_fill_b8", &fn);
-      if (status == HC_OK) status = launch_fn(ctx, fn, 1, 1, 1, HCK_BLOCK, 0, &k, sizeof(k));
+      int marked = find_kernel_locked(ctx, "hc_fill_b8", &fn);
+      if (marked == HC_OK) marked = launch_fn(ctx, fn, 1, 1, 1, HCK_BLOCK, 0, &k, sizeof(k));
+      if (status == HC_OK) status = marked;
     }
     ctx->lazy = true;
   }
@@ -857,6 +868,10 @@ static int flush_batch_locked(hc_ctx* ctx, BatchEnd why) {
   // early batch doubles the length the next one needs, so that a program that never waits, and
   // whose device runs dry because the host is the slower side, ends up with full batches (fewer
   // rewrites and launches on the host, which is what it is short of); a wait starts over.
+  if (status != HC_OK && why != BATCH_END_WAIT) {
+    ctx->batch_failed = status;
+    ctx->batch_failed_why = g_last_error;
+  }
   if (why == BATCH_END_IDLE) ctx->batch_idle_now = std::min(ctx->batch_idle_now * 2, ctx->batch_limit);
   else if (why == BATCH_END_WAIT) ctx->batch_idle_now = ctx->batch_idle_after;
   for (auto& kv : ctx->batch_parked) {

@@ -213,3 +213,34 @@ def test_concurrent_op_chains_under_batching(hip_backend):
         for th in pool:
             th.join()
     assert not failures, failures[:5]
+
+
+def test_a_batch_that_cannot_be_enqueued_is_reported(hip_backend):
+    """A listed launch that the runtime refuses (here a caller's kernel with an empty grid, rejected on
+    the host before anything runs) surfaces in the call that enqueues the batch; when that call is
+    one whose status the caller may not see (the batch went out because it was full, or from a
+    release), the next wait reports it again, once."""
+    import ctypes
+    import os
+    path = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "bench_probe.hsaco")
+    if not os.path.exists(path):
+        pytest.skip("bench_probe.hsaco is not built")
+    lib, ctx = hip_backend._lib, hip_backend._ctx
+    image = open(path, "rb").read()
+    buf = ctypes.create_string_buffer(image, len(image))
+    module, fn = ctypes.c_void_p(), ctypes.c_void_p()
+    hip_backend._check(lib.hc_module_load(ctx, buf, len(image), ctypes.byref(module)))
+    hip_backend._check(lib.hc_module_get_function(module, b"hc_bench_marker", ctypes.byref(fn)))
+    n = 4096
+    x = hip_backend.upload(np.full(n, 0.5, np.float32))
+    want = hip_backend.elemwise(x, ElemwiseOp.exp, None, n, F32).onCPU().copy()
+    grid, block = (ctypes.c_uint32 * 3)(0, 1, 1), (ctypes.c_uint32 * 3)(64, 1, 1)
+    with hip_backend.batching(2):
+        hip_backend._check(lib.hc_launch(ctx, fn, grid, block, 0, None, 0))     # listed: nothing is checked yet
+        with pytest.raises(Exception):
+            hip_backend.elemwise(x, ElemwiseOp.exp, None, n, F32)                # second launch: the batch is full and goes out
+        with pytest.raises(Exception):
+            hip_backend.sync()                                                   # ... reported once more
+        hip_backend.sync()                                                       # and then no more
+        y = hip_backend.elemwise(x, ElemwiseOp.exp, None, n, F32)                # the context works on
+        assert np.array_equal(y.onCPU(), want)
