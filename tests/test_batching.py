@@ -154,15 +154,17 @@ def test_waits_and_events_enqueue_the_list(hip_backend):
         assert np.array_equal(z.onCPU(), want)
 
 
-def test_config5_forward_pass_batch_limits(hip_backend):
-    """The transformer's forward pass under batches of 50 launches (batches end in the middle of
-    layers) and of one whole pass: the logits of the call-by-call run, bit for bit."""
+@pytest.mark.parametrize("dtype", [F16, F32], ids=["f16", "f32"])
+def test_config5_forward_pass_batch_limits(hip_backend, dtype):
+    """The transformer's forward pass under batches of a few to a few thousand launches (batches end
+    anywhere inside layers, chains and attention blocks) and with early batches: the logits of the
+    call-by-call run, bit for bit, in both precisions."""
     rng = np.random.default_rng(9)
     with hip_backend.use():
-        model = Transformer(dtype=F16)
+        model = Transformer(dtype=dtype)
         ids = Tensor(data=rng.integers(0, 8192, size=(8, 256)))
         want = model(ids).numpy().copy()
-        for limit, idle_after in ((50, 0), (4096, 0), (256, 16), (64, 1)):
+        for limit, idle_after in ((50, 0), (4096, 0), (256, 16), (64, 1), (7, 0), (13, 0), (29, 3), (97, 0), (3, 0)):
             with hip_backend.batching(limit, idle_after):
                 for _ in range(2):
                     got = model(ids).numpy()
