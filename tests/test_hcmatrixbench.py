@@ -20,7 +20,9 @@ BINARY = os.path.join(ROOT, "honeycrisp_amd", "cpp", "HCMatrixBench")
 def run(args, timeout=170):
     assert os.path.exists(BINARY), "build it with `python -m honeycrisp_amd.csrc.build`"
     print("running", BINARY, *args, flush=True)
-    proc = subprocess.run([BINARY] + args, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=timeout)
+    # (the program sets its own batching: a setting meant for this process's context stays here)
+    env = {k: v for k, v in os.environ.items() if k != "HCHIP_BATCHING"}
+    proc = subprocess.run([BINARY] + args, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=timeout, env=env)
     assert proc.returncode == 0, proc.stdout + proc.stderr
     return [dict(kv.split("=", 1) for kv in line.split()) for line in proc.stdout.strip().splitlines()], proc.stdout
 
