@@ -95,7 +95,7 @@ def test_code_objects_hold_every_reduce_and_gemm_kernel_the_host_names():
         assert ("hc_gemm_%s_%s_%s_%s%s" % (dt, pipe, tile, lay, edge)).encode() + b"\0" in blob["gemm_" + pipe]
     for dt in ("f16", "f32"):
         for n in ("hc_gemm_%s_xx", "hc_gemm_%s_kk", "hc_gemm_skinny_k_%s_q4", "hc_gemm_skinny_p_%s_q4",
-                  "hc_gemm_skinny_pack_%s", "hc_gemm_skinny_store_%s", "hc_copy2d_pad_b%d", "hc_copy2d_unpad_b%d"):
+                  "hc_gemm_skinny_pack_%s", "hc_gemm_skinny_store_%s", "hc_gemm_skinny_pair_%s", "hc_copy2d_pad_b%d", "hc_copy2d_unpad_b%d"):
             name = n % (dt if "%s" in n else (2 if dt == "f16" else 4))
             assert any(name.encode() + b"\0" in b for b in blob.values()), name
 
