@@ -217,9 +217,9 @@ int hc_graph_destroy(hc_ctx* ctx, hc_graph* graph);
  * footprint of a batch is the sum of its intermediates. Errors of a listed launch surface in
  * the call that enqueues the batch; if that was not a call that waits or transfers (the batch
  * was full, or went out from hc_free), the next such call reports the failure once more, so a
- * caller that ignores the status of a release still learns of it. max_launches = 0 (the default) enqueues what is listed and
- * goes back to one launch per call. Refused during a capture; a capture inside batching works
- * (the list is enqueued first). HCHIP_BATCHING=<max>[,<idle_after>] in the environment at
+ * caller that ignores the status of a release still learns of it. max_launches = 0 (the
+ * default) enqueues what is listed and goes back to one launch per call. Refused during a
+ * capture; a capture inside batching works (the list is enqueued first). HCHIP_BATCHING=<max>[,<idle_after>] in the environment at
  * hc_init starts a context with hc_set_batching(max, idle_after). */
 int hc_set_batching(hc_ctx* ctx, size_t max_launches, size_t idle_after);
 /* Enqueues what batching has listed so far. Nothing to do outside batching. */
