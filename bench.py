@@ -633,6 +633,9 @@ def extra_workloads(backend, graph=True, only=("cfg1", "cfg2", "cfg3", "cfg4", "
             return backend.gather(x, ScatterGatherIndices([R, C], 1, BroadcastData(BroadcastStrides([R, 1], [1, 0]), i)), F32)
         ms, _ = timed_launches(backend, ev, max_axis1, 50, 10, batched=True, region="cfg4_max_axis1")
         report("cfg4_max_axis1", ms, nbytes=nb + R * 8 + R * 8 + R * 4 + R * 4)
+        # ... and as a recording (or a batch) merges the pair: the row kernel that finds the index stores the element
+        ms, _ = timed_launches(backend, ev, max_axis1, 50, 10, batched=True, region="cfg4_max_axis1_recorded_one_kernel", fusion=True)
+        report("cfg4_max_axis1_recorded_one_kernel", ms, nbytes=nb + R * 4)
         table = backend.upload(np.random.default_rng(10).standard_normal((32000, 1024)).astype(np.float32))
         ids = backend.upload(np.random.default_rng(9).integers(0, 32000, size=(65536,)))
         emb = ScatterGatherIndices([32000, 1024], 0, BroadcastData(BroadcastStrides([65536, 1024], [1, 0]), ids))

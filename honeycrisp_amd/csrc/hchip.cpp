@@ -76,7 +76,7 @@ struct hc_pending {
   std::vector<const void*> reads;
   std::vector<const void*> writes;
   // what the rewrite needs to know about the operations it can merge
-  enum Tag { NONE, GEMM, PRODUCT, BMM, PERMUTE, ADD, GELU, CAST, NORMALIZE, LOG_SOFTMAX, SCALAR, MUL_ADD, EXP, SOFTMAX_CHAIN } tag = NONE;
+  enum Tag { NONE, GEMM, PRODUCT, BMM, PERMUTE, ADD, GELU, CAST, NORMALIZE, LOG_SOFTMAX, SCALAR, MUL_ADD, EXP, SOFTMAX_CHAIN, ARG_REDUCE, GATHER_ONE } tag = NONE;
   int dtype = 0;                       // element type of the output
   int src_dtype = 0;                   // CAST: element type of the input
   uint64_t rows = 0, cols = 0;         // GEMM: M, N; ADD: leading x trailing extent; GELU, CAST: 1 x count
@@ -90,6 +90,9 @@ struct hc_pending {
   // EXP: ElemwiseOp.exp over `cols` elements of in0
   // BMM: a batched product in one launch of a direct-to-LDS kernel (operands in the argument struct);
   //   stays a BMM when the rewrite has made it read or write through a swap of the batch axes
+  // ARG_REDUCE: argmax / argmin (op) over the rows of a dense rows x cols input (in0, of type dtype) by one
+  //   launch of a row kernel with teams of `lanes` lanes; out holds rows int64 indices
+  // GATHER_ONE: out[r] = in0[r * cols + in1[r]] for rows rows, in1 dense int64 indices
   // SOFTMAX_CHAIN: the merged [scale] [mask] logSoftmax [exp] row kernel (rows x cols, lanes; args hck_softmax_chain_args)
   // PERMUTE (row form): in0 -> out; axis d of the dense output has extent pext[d] and lies at
   // stride pstr[d] (elements) in the source, the last axis contiguous in both
@@ -1914,7 +1917,7 @@ static int softmax_cols(hc_ctx* ctx, int dtype, const void* in, const void* grad
 
 // hc_reduce proper; `scratch` says where partial results live (the pool, or a fixed range).
 static int reduce_impl(hc_ctx* ctx, Scratch& scratch, int op, int dtype, const void* in, void* out, int64_t outer,
-                       int64_t reduce, int64_t inner) {
+                       int64_t reduce, int64_t inner, OpNote* note) {
   REQUIRE(ctx, "hc_reduce: null context");
   REQUIRE(op >= HC_SUM && op <= HC_ARGMIN, "hc_reduce: bad op %d", op);
   if (dtype != HC_F32 && dtype != HC_F16 && dtype != HC_I64 && dtype != HC_BOOL)
@@ -1935,9 +1938,21 @@ static int reduce_impl(hc_ctx* ctx, Scratch& scratch, int op, int dtype, const v
   if (inner == 1) {
     const bool vec_ok = aligned16(in);
     REQUIRE(vec_ok, "hc_reduce: input must be 16-byte aligned");
+    auto tag_arg = [&](int lanes) {   // an arg-reduction in one launch: a gather of its indices can join it
+      if (!note || (op != HC_ARGMAX && op != HC_ARGMIN)) return;
+      note->tag = hc_pending::ARG_REDUCE;
+      note->meta.dtype = dtype;
+      note->meta.op = op;
+      note->meta.rows = (uint64_t)outer;
+      note->meta.cols = (uint64_t)reduce;
+      note->meta.lanes = lanes;
+      note->meta.in0 = in;
+      note->meta.out = out;
+    };
     // a team of 1, 8, 64 or 256 lanes per row, by row length
     if (reduce <= 1024) {
       const uint32_t lanes = reduce <= 8 ? 1 : reduce <= 128 ? 8 : 64;
+      tag_arg((int)lanes);
       snprintf(name, sizeof(name), "hc_reduce_rows%u_%s_%s", lanes, kReduceNames[op], dtype_name(dtype));
       return launch(ctx, name, ceil_div((uint64_t)outer, HCK_BLOCK / lanes), 1, &k, sizeof(k));
     }
@@ -1977,6 +1992,7 @@ static int reduce_impl(hc_ctx* ctx, Scratch& scratch, int op, int dtype, const v
         return launch(ctx, name, (uint64_t)outer, 1, &c, sizeof(c));
       }
     }
+    tag_arg(256);
     snprintf(name, sizeof(name), "hc_reduce_rows256_%s_%s", kReduceNames[op], dtype_name(dtype));
     return launch(ctx, name, (uint64_t)outer, 1, &k, sizeof(k));
   }
@@ -1989,7 +2005,7 @@ extern "C" int hc_reduce(hc_ctx* ctx, int op, int dtype, const void* in, void* o
   OpNote note({in}, {out});
   REQUIRE(ctx, "hc_reduce: null context");
   Scratch scratch(ctx);
-  return reduce_impl(ctx, scratch, op, dtype, in, out, outer, reduce, inner);
+  return reduce_impl(ctx, scratch, op, dtype, in, out, outer, reduce, inner, &note);
 }
 
 // hc_reduce with its partial results in the caller's device range [scratch, scratch + scratch_bytes)
@@ -2002,7 +2018,7 @@ __attribute__((visibility("hidden"))) int hc_reduce_in_scratch(hc_ctx* ctx, int 
   REQUIRE(scratch_base, "hc_reduce_noalloc: the scratch buffer of device %d was not set up", ctx->device);
   OpNote note({in}, {out});   // (in a recording: the launches stay where they are, nothing is merged into them)
   Scratch scratch(ctx, scratch_base, scratch_bytes);
-  return reduce_impl(ctx, scratch, op, dtype, in, out, outer, reduce, inner);
+  return reduce_impl(ctx, scratch, op, dtype, in, out, outer, reduce, inner, nullptr);
 }
 
 __attribute__((visibility("hidden"))) int hc_ctx_device(const hc_ctx* ctx) { return ctx ? ctx->device : -1; }
@@ -2392,6 +2408,26 @@ extern "C" int hc_gather(hc_ctx* ctx, int dtype, const void* in, const void* ind
   const hc_strides* ops[] = {idx_strides};
   const void* ptrs[] = {indices};
   HC_TRY(make_bcast(1, ops, ptrs, out, 1, &k.idx, &vec, &n));
+  if (out_count == 1 && inner == 1) {
+    // one element per row, the rows' indices dense in memory: what follows an arg-reduction in
+    // Tensor.max / min (ReduceRepeat.swift:201-209)
+    bool dense = true;
+    int64_t expect = 1;
+    for (uint32_t d = idx_strides->ndim; d-- > 0;) {
+      if (idx_strides->shape[d] == 1) continue;
+      dense = dense && idx_strides->strides[d] == expect;
+      expect *= idx_strides->shape[d];
+    }
+    if (dense) {
+      note.tag = hc_pending::GATHER_ONE;
+      note.meta.dtype = dtype;
+      note.meta.rows = (uint64_t)outer;
+      note.meta.cols = (uint64_t)middle;
+      note.meta.in0 = in;
+      note.meta.in1 = indices;
+      note.meta.out = out;
+    }
+  }
   char name[64];
   snprintf(name, sizeof(name), "hc_gather_elems_b%zu", el);
   return launch(ctx, name, ceil_div(total, HCK_BLOCK), 1, &k, sizeof(k));

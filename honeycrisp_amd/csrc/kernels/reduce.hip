@@ -83,7 +83,10 @@ template <int LANES, int OP, typename C> __device__ __forceinline__ ArgPair<C> t
   return p;
 }
 
-template <typename T, int OP, int LANES, bool SPLIT>
+// VALUE (arg-reductions, not SPLIT): the output holds the extremum itself, in the input's element
+// type, instead of its index: what an arg-reduction followed by a gather of its indices from the
+// same input leaves (Tensor.max / min, ReduceRepeat.swift:201-209), in one pass.
+template <typename T, int OP, int LANES, bool SPLIT, bool VALUE = false>
 __device__ __forceinline__ void reduce_rows_impl(const hck_reduce_args& p) {
   typedef typename Arith<T>::type C;
   constexpr int VEC = VecWidth<T>::value;
@@ -192,6 +195,8 @@ __device__ __forceinline__ void reduce_rows_impl(const hck_reduce_args& p) {
       if (SPLIT) {
         ((C*)p.pvals)[blockIdx.x] = best.v;
         p.pidx[blockIdx.x] = best.i;
+      } else if (VALUE) {
+        ((T*)p.out)[row] = in[best.i];
       } else {
         ((int64_t*)p.out)[row] = (int64_t)best.i;
       }
@@ -350,11 +355,18 @@ __device__ __forceinline__ void reduce_cols_impl(const hck_reduce_cols_args& p) 
   HC_KERNEL void hc_reduce_cols_final_##NAME##_##TN(hck_reduce_cols_args p) {                          \
     reduce_cols_impl<T, OP, 1, true>(p);                                                               \
   }
+#define DEF_REDUCE_VALUE(NAME, OP, TN, T)                                                             \
+  HC_KERNEL void hc_reduce_rows1_##NAME##_value_##TN(hck_reduce_args p) { reduce_rows_impl<T, OP, 1, false, true>(p); } \
+  HC_KERNEL void hc_reduce_rows8_##NAME##_value_##TN(hck_reduce_args p) { reduce_rows_impl<T, OP, 8, false, true>(p); } \
+  HC_KERNEL void hc_reduce_rows64_##NAME##_value_##TN(hck_reduce_args p) { reduce_rows_impl<T, OP, 64, false, true>(p); } \
+  HC_KERNEL void hc_reduce_rows256_##NAME##_value_##TN(hck_reduce_args p) { reduce_rows_impl<T, OP, 256, false, true>(p); }
 #define DEF_REDUCE_T(TN, T)                                                                          \
   DEF_REDUCE(sum, R_SUM, TN, T)                                                                      \
   DEF_REDUCE(prod, R_PROD, TN, T)                                                                    \
   DEF_REDUCE(argmax, R_ARGMAX, TN, T)                                                                \
-  DEF_REDUCE(argmin, R_ARGMIN, TN, T)
+  DEF_REDUCE(argmin, R_ARGMIN, TN, T)                                                                \
+  DEF_REDUCE_VALUE(argmax, R_ARGMAX, TN, T)                                                          \
+  DEF_REDUCE_VALUE(argmin, R_ARGMIN, TN, T)
 DEF_REDUCE_T(f32, float)
 DEF_REDUCE_T(f16, half_t)
 DEF_REDUCE_T(i64, int64_t)

@@ -177,6 +177,8 @@ int hc_launch_host_func(hc_ctx* ctx, void (*fn)(void*), void* user);
  *      q k^T -> that softmax kernel -> x v, 64-wide fp16 heads,
  *      T a multiple of 64 up to 512                                 one attention kernel
  *      products of one shape over the same input (q, k, v)          one launch
+ *      argmax | argmin over rows -> gather of those indices from
+ *      the same tensor (Tensor.max / min / all / some)              one row kernel
  *    Buffers that only held merged intermediates are never written by a replay.
  *    Switches (environment at hc_init, or hc_debug_set): HCHIP_RECORDING_LOG=1 lists the
  *    launches of the rewritten recording on stderr at hc_capture_end; HCHIP_GRAPH_AS_LAUNCHES=1

@@ -30,15 +30,16 @@ def record(backend, fn, fusion=True):
 def check(backend, fn, removed):
     """fn() recorded with and without the rewrite and issued eagerly: same bits from all three;
     the rewrite removes exactly `removed` launches."""
+    bits = lambda a: np.atleast_1d(a).view(np.uint8)
     want = fn().numpy().copy()
     plain, plain_out, plain_nodes = record(backend, fn, fusion=False)
     fused, fused_out, fused_nodes = record(backend, fn)
     for replay in range(2):
         plain.launch()
         fused.launch()
-        assert np.array_equal(plain_out.numpy(), want)
+        assert np.array_equal(bits(plain_out.numpy()), bits(want))
         got = fused_out.numpy()
-        assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), \
+        assert np.array_equal(bits(got), bits(want)), \
             "replay %d: %d of %d elements differ" % (replay, int((got != want).sum()), want.size)
     assert plain_nodes - fused_nodes == removed, (plain_nodes, fused_nodes)
     plain.destroy()
@@ -49,7 +50,7 @@ def check(backend, fn, removed):
     with backend.batching():
         got = fn().numpy().copy()
     listed, enqueued = (after - before for after, before in zip(backend.batchingStats(), (listed, enqueued)))
-    assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), \
+    assert np.array_equal(bits(got), bits(want)), \
         "batching: %d of %d elements differ" % (int((got != want).sum()), want.size)
     assert listed - enqueued == removed, (listed, enqueued)
 
@@ -657,3 +658,70 @@ def test_a_buffer_written_before_the_merged_product_stays_with_the_graph(hip_bac
         for o in others:
             assert np.all(o.onCPU().view(np.float32) == 9.0)
     cap.graph.destroy()
+
+
+def extremum_input(rng, dtype, rows, cols):
+    """Rows with repeated extrema (the first one's index decides) and, for floats, a few NaNs."""
+    if dtype == DType.bool:
+        return Tensor(data=(rng.random((rows, cols)) < 0.5).astype(np.float32)).cast(DType.bool)
+    if dtype == DType.int64:
+        return Tensor(data=rng.integers(-50, 50, (rows, cols)), dtype=DType.int64)
+    data = np.round(rng.standard_normal((rows, cols)) * 8).astype(np.float32) / 4
+    data[rng.random((rows, cols)) < 0.002] = np.nan
+    return Tensor(data=data, dtype=dtype)
+
+
+@pytest.mark.parametrize("dtype", [DType.float32, DType.float16, DType.int64, DType.bool], ids=["f32", "f16", "i64", "bool"])
+@pytest.mark.parametrize("rows,cols", [(1000, 5), (333, 100), (257, 1000), (9, 3001), (2, 30000)])
+def test_max_and_min_over_rows_become_one_kernel(hip_backend, dtype, rows, cols):
+    """Tensor.max / min are an arg-reduction and a gather of its indices (ReduceRepeat.swift:201-209);
+    over the last axis, the row kernel that finds the index leaves the element itself."""
+    rng = np.random.default_rng(rows * 7 + cols)
+    with hip_backend.use():
+        x = extremum_input(rng, dtype, rows, cols)
+        check(hip_backend, lambda: x.max(axis=1), removed=1)
+        check(hip_backend, lambda: x.min(axis=-1, keepdims=True), removed=1)
+        if dtype == DType.bool:
+            check(hip_backend, lambda: x.some(axis=1), removed=1)
+            check(hip_backend, lambda: x.all(axis=1, keepdims=True), removed=1)
+        # three axes, the last one reduced: still rows
+        if rows % 3 == 0:
+            y = x.reshape([3, rows // 3, cols])
+            check(hip_backend, lambda: y.max(axis=2), removed=1)
+
+
+def test_extrema_that_are_left_alone(hip_backend):
+    rng = np.random.default_rng(5)
+    with hip_backend.use():
+        x = extremum_input(rng, DType.float32, 300, 64)
+        other = extremum_input(rng, DType.float32, 300, 64)
+        # an axis that is not the last one: a column reduction
+        check(hip_backend, lambda: x.max(axis=0), removed=0)
+        # the indices pick from another tensor
+        check(hip_backend, lambda: other.gather(1, x.argmax(axis=1, keepdims=True)), removed=0)
+        # the caller keeps the indices
+        held = []
+
+        def both():
+            idx = x.argmax(axis=1, keepdims=True)
+            held.append(idx)
+            return x.gather(1, idx)
+
+        check(hip_backend, both, removed=0)
+        # a long row cut into segments: two launches find the index
+        long_row = extremum_input(rng, DType.float32, 1, 300000)
+        check(hip_backend, lambda: long_row.max(), removed=0)
+        # the input changes between the two launches: the gather must see the new values
+        first = Tensor(data=rng.standard_normal((64, 32)).astype(np.float32))
+        second = Tensor(data=rng.standard_normal((64, 32)).astype(np.float32))
+
+        def rewritten():
+            t = first + 0.0
+            idx = t.argmax(axis=1, keepdims=True)
+            hip_backend._check(hip_backend._lib.hc_memcpy_d2d(hip_backend._ctx, c_void_p(t.data.ptr),
+                                                               c_void_p(second.data.ptr), 64 * 32 * 4))
+            return t.gather(1, idx)
+
+        check(hip_backend, rewritten, removed=0)
+        want = np.take_along_axis(second.numpy(), first.numpy().argmax(axis=1)[:, None], axis=1)
+        assert np.array_equal(rewritten().numpy(), want)

@@ -83,6 +83,8 @@ def test_code_objects_hold_every_reduce_and_gemm_kernel_the_host_names():
     for form, op, dt in itertools.product(forms, ["sum", "prod", "argmax", "argmin"], ["f32", "f16", "i64", "b8"]):
         names = ["hc_reduce_%s_%s_%s" % (form, op, dt)] if form != "cols" else \
             ["hc_reduce_cols_%s_%s_v1" % (op, dt), "hc_reduce_cols_%s_%s_vN" % (op, dt), "hc_reduce_cols_final_%s_%s" % (op, dt)]
+        if op.startswith("arg") and form.startswith("rows") and form != "rowsplit":   # the form that also leaves the extremum itself
+            names.append("hc_reduce_%s_%s_value_%s" % (form, op, dt))
         for n in names:
             assert n.encode() + b"\0" in blob["reduce"], n
     layouts = ["kk", "kn", "mk", "mn"]

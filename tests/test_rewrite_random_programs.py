@@ -1,5 +1,5 @@
 """Random programs over the operations the rewrite of a recording knows (products, row and
-matrix additions, GELU, LayerNorm, the scaled and masked softmax), with random lifetimes of
+matrix additions, GELU, LayerNorm, the scaled and masked softmax, row maxima), with random lifetimes of
 the intermediates: results with several readers, results the program keeps, results released
 at once. Whatever the rewrite merges or leaves alone, and wherever a batch happens to end, a
 program's results must have the bits of the same calls issued one by one; here the same seeded
@@ -35,7 +35,7 @@ class Program:
         pool, kept = [self.x0], []
         for _ in range(self.steps):
             a = pool[rng.integers(len(pool))]
-            op = rng.choice(["linear", "row", "matrix", "gelu", "norm", "softmax", "linear", "row"])
+            op = rng.choice(["linear", "row", "matrix", "gelu", "norm", "softmax", "linear", "row", "center"])
             if op == "linear":
                 t = Tensor.matmul(a, False, self.weights[rng.integers(3)], False, False)
             elif op == "row":
@@ -46,6 +46,8 @@ class Program:
                 t = a.gelu()
             elif op == "norm":
                 t = self.norms[rng.integers(2)](a)
+            elif op == "center":
+                t = a - (a.max(axis=1, keepdims=True) if rng.random() < 0.5 else a.min(axis=1, keepdims=True))
             else:
                 s = a * 0.125 if rng.random() < 0.7 else a
                 if rng.random() < 0.5:
