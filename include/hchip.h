@@ -174,8 +174,8 @@ int hc_launch_host_func(hc_ctx* ctx, void (*fn)(void*), void* user);
  *      [cast ->] normalize -> [(gain + c) *, + bias] -> [cast]      one LayerNorm kernel
  *      [* s ->] [+ mask ->] logSoftmax -> [exp]                     one softmax kernel
  *      swap of two batch axes -> batchedMatmul -> swap back         read / written through strides
- *      q k^T -> that softmax kernel -> x v, 64-wide fp16 heads,
- *      T a multiple of 64 up to 512                                 one attention kernel
+ *      q k^T -> that softmax kernel -> x v, 64-wide heads, T a
+ *      multiple of 64 up to 512 (fp16) / 256 (fp32)                 one attention kernel
  *      products of one shape over the same input (q, k, v)          one launch
  *      argmax | argmin over rows -> gather of those indices from
  *      the same tensor (Tensor.max / min / all / some)              one row kernel

@@ -405,9 +405,9 @@ def test_head_swaps_fold_into_the_batched_products(hip_backend, dtype, B, T, H, 
             probs = (scores * 0.125).softmax()
             return Tensor.batchedMatmul(probs, False, heads(v), False, False).swap(1, 2).reshape([B, T, D])
 
-        # 4 swaps, and scale + logSoftmax + exp -> 1; with 64-wide fp16 heads the two products and that
+        # 4 swaps, and scale + logSoftmax + exp -> 1; with 64-wide heads the two products and that
         # row kernel then become the attention kernel
-        check(hip_backend, attention, removed=4 + 2 + (2 if dtype == DType.float16 and hd == 64 else 0))
+        check(hip_backend, attention, removed=4 + 2 + (2 if hd == 64 else 0))
         # one operand swapped, the other dense; result kept in [B, H, T, T] order
         kt = Tensor(data=rng.standard_normal((B, H, T, hd)).astype(np.float32), dtype=dtype)
         check(hip_backend, lambda: Tensor.batchedMatmul(heads(q), False, kt, True, False), removed=1)
@@ -420,13 +420,16 @@ def test_head_swaps_fold_into_the_batched_products(hip_backend, dtype, B, T, H, 
         check(hip_backend, two_readers, removed=0)
 
 
-@pytest.mark.parametrize("heads,t", [(64, 256), (32, 512), (5, 64), (3, 128), (2, 192), (3, 320), (2, 448)])
-def test_attention_becomes_one_kernel(hip_backend, heads, t):
-    """q k^T -> [* s] [+ mask] softmax -> x v over fp16 heads of 64: one launch per recording, and a replay
-    returns the bits of the five separate launches (same accumulation order in both products, fp16
-    scores and probabilities, the row kernel's own reduction)."""
+@pytest.mark.parametrize("dtype,heads,t", [(DType.float16, h, t) for h, t in
+                                           [(64, 256), (32, 512), (5, 64), (3, 128), (2, 192), (3, 320), (2, 448)]] +
+                         [(DType.float32, h, t) for h, t in [(64, 256), (5, 64), (3, 128), (2, 192)]],
+                         ids=lambda v: v.name if isinstance(v, DType) else str(v))
+def test_attention_becomes_one_kernel(hip_backend, dtype, heads, t):
+    """q k^T -> [* s] [+ mask] softmax -> x v over heads of 64 (fp16 up to 512 keys, fp32 up to 256): one launch
+    per recording, and a replay returns the bits of the five separate launches (same accumulation order in
+    both products, scores and probabilities rounded to the tensor type, the row kernel's own reduction)."""
     rng = np.random.default_rng(heads * 1000 + t)
-    f16 = DType.float16
+    f16 = dtype
     with hip_backend.use():
         q, k, v = (Tensor(data=rng.standard_normal((heads, t, 64)).astype(np.float32), dtype=f16) for _ in range(3))
         mask = Tensor(data=np.where(np.tril(np.ones((t, t))) > 0, 0.0, -1e4).astype(np.float32), dtype=f16)
@@ -462,7 +465,7 @@ def test_attention_forms_that_are_left_alone(hip_backend):
 
         q, k, v = qkv(8, 128, 32)                # heads of 32
         check(hip_backend, lambda: attention(q, k, v), removed=2)
-        q, k, v = qkv(8, 128, 64, DType.float32)  # fp32
+        q, k, v = qkv(2, 320, 64, DType.float32)  # fp32 rows longer than the score tile holds
         check(hip_backend, lambda: attention(q, k, v), removed=2)
         q, k, v = qkv(2, 576, 64)                # rows longer than the score tile holds
         check(hip_backend, lambda: attention(q, k, v), removed=2)
@@ -507,10 +510,10 @@ def test_config5_forward_recorded_with_the_rewrite(hip_backend, dtype):
         # in fp16 also the 6 + 1 casts of the fp32 biases
         half = dtype == DType.float16
         per_block = 9 + 2 * (4 if half else 2) + 3 + 4 + 2 + (6 if half else 0)
-        # ... and in fp16 (64-wide heads) scores, softmax and context of a block are one attention kernel
-        per_block += 2 if half else 0
+        # ... and (64-wide heads) scores, softmax and context of a block are one attention kernel
+        per_block += 2
         assert plain_nodes - fused_nodes == 6 * per_block + (4 if half else 2) + (2 if half else 1)
-        assert fused_nodes == (46 if half else 58)
+        assert fused_nodes == 46
         plain.destroy()
         fused.destroy()
         # the same forward pass call by call under batching: one batch, the same launches
