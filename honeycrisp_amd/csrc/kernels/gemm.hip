@@ -328,7 +328,7 @@ template <typename T, int TQ> __device__ __forceinline__ void skinny_k_impl(cons
 // wave reads 64 * V consecutive elements of a k-row per step; a workgroup covers one such
 // p-tile and a chunk of the k-range (grid.x = p-tiles * k-chunks), its four waves take every
 // fourth k-row and add their partial sums up in LDS; every chunk leaves its sums in a slice of its
-// own of an fp32 buffer and hc_gemm_skinny_store adds the slices in chunk order and rounds, so
+// own of an fp32 buffer and hc_gemm_skinny_store adds the slices in a fixed order and rounds, so
 // the result does not depend on which workgroup finishes first. Y is read one element per wave
 // and step (wave-uniform), so it is taken as it lies, whatever its strides.
 template <typename T, int TQ> __device__ __forceinline__ void skinny_p_impl(const hck_skinny_args& a, const uint32_t block) {
@@ -413,26 +413,35 @@ template <typename T> __device__ __forceinline__ void skinny_pack_impl(const hck
   P[i] = k < a.K ? Y[(size_t)k * a.y_ks + (size_t)q * a.c_qs] : (T)0;
 }
 
+// The chunks' partial sums of one output -> the output: a team of 16 adjacent lanes per output. Lane j of the
+// team adds the chunks j, j + 16, ... in this order (all its loads issued first: one load after the other would
+// cost a memory latency per chunk), then the 16 lanes add up over lane distances 8, 4, 2, 1: a fixed order, the
+// same on every run. A workgroup finishes 16 outputs (grid.x = ceil(L * t / 16)).
+constexpr int SKINNY_STORE_TEAM = 16, SKINNY_STORE_ROUNDS = 8;   // chunks <= 16 * 8 (the host's limit)
 template <typename T> __device__ __forceinline__ void skinny_store_impl(const hck_skinny_args& a, const uint32_t block) {
-  const uint64_t i = (uint64_t)block * HCK_BLOCK + threadIdx.x;
-  if (i >= (uint64_t)a.L * a.t) return;
+  const uint32_t j = threadIdx.x % SKINNY_STORE_TEAM;
+  const uint64_t total = (uint64_t)a.L * a.t;
+  uint64_t i = (uint64_t)block * (HCK_BLOCK / SKINNY_STORE_TEAM) + threadIdx.x / SKINNY_STORE_TEAM;
+  const bool live = i < total;
+  if (!live) i = total - 1;   // (whole teams: every lane takes part in the exchanges below)
   const uint32_t p = (uint32_t)(i / a.t), q = (uint32_t)(i - (uint64_t)p * a.t);
-  T* C = (T*)a.c + (uint64_t)blockIdx.y * a.c_bs;
-  const uint64_t slice = (uint64_t)a.L * a.t;
-  const float* part = a.acc + (uint64_t)blockIdx.y * a.chunks * slice + i;
-  // chunk order, 16 loads in flight at a time (one dependent load after the other would cost a
-  // memory latency per chunk)
-  float v = 0.0f;
-  uint32_t c = 0;
-  for (; c + 16 <= a.chunks; c += 16) {
-    float t[16];
+  const float* part = a.acc + (uint64_t)blockIdx.y * a.chunks * total + i;
+  float t[SKINNY_STORE_ROUNDS];
 #pragma unroll
-    for (int u = 0; u < 16; u++) t[u] = part[(uint64_t)(c + u) * slice];
-#pragma unroll
-    for (int u = 0; u < 16; u++) v += t[u];
+  for (int r = 0; r < SKINNY_STORE_ROUNDS; r++) {
+    const uint32_t c = j + r * SKINNY_STORE_TEAM;
+    t[r] = c < a.chunks ? part[(uint64_t)c * total] : 0.0f;
   }
-  for (; c < a.chunks; c++) v += part[(uint64_t)c * slice];
-  C[(size_t)p * a.c_ps + (size_t)q * a.c_qs] = narrow<T>(v);
+  float v = 0.0f;
+#pragma unroll
+  for (int r = 0; r < SKINNY_STORE_ROUNDS; r++)
+    if (j + r * SKINNY_STORE_TEAM < a.chunks) v += t[r];
+#pragma unroll
+  for (int d = SKINNY_STORE_TEAM / 2; d > 0; d >>= 1) v += __shfl_xor(v, d, 64);
+  if (live && j == 0) {
+    T* C = (T*)a.c + (uint64_t)blockIdx.y * a.c_bs;
+    C[(size_t)p * a.c_ps + (size_t)q * a.c_qs] = narrow<T>(v);
+  }
 }
 
 // Two skinny launches that do not depend on each other (the thin fringes of a ragged product: a

@@ -131,7 +131,7 @@ __device__ __forceinline__ void reduce_rows_impl(const hck_reduce_args& p) {
         for (uint32_t k = k0 + lane; k < kend; k += LANES) acc = reduce_combine<OP, C>(acc, to_arith(in[k]));
       }
     }
-    if (LANES <= 64) {
+    if constexpr (LANES <= 64) {
       acc = OP == R_SUM ? team_reduce<LANES>(acc, SumOp()) : team_reduce<LANES>(acc, ProdOp());
     } else {
       acc = OP == R_SUM ? block_reduce(acc, SumOp(), (C*)lds_raw)
@@ -386,8 +386,8 @@ template <int LANES> struct Team {
   }
   // every lane of the team gets the result; `lds` holds >= 4 floats (block teams only)
   template <typename Op> static __device__ __forceinline__ float reduce(float v, Op op, float* lds) {
-    if (LANES <= 64) return team_reduce<LANES>(v, op);
-    return block_reduce(v, op, lds);
+    if constexpr (LANES <= 64) return team_reduce<LANES>(v, op);
+    else return block_reduce(v, op, lds);
   }
 };
 
