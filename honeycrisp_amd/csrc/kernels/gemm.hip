@@ -346,15 +346,18 @@ template <typename T, int TQ> __device__ __forceinline__ void skinny_p_impl(cons
   for (int q = 0; q < TQ; q++)
 #pragma unroll
     for (int e = 0; e < V; e++) acc[q][e] = 0.0f;
-  const bool whole = p0 + V <= a.L;
-  uint32_t k = k_lo + wave;
-  if (whole) {
-    // U of this wave's k-rows at a time, loads first (see skinny_k_impl), sums in the plain loop's order
-    constexpr int U = 6;
+  // (k-rows of X start at any element; the one lane that straddles the end of a row takes its elements one by
+  // one, lanes past the end have nothing to add. Two bodies, chosen once per lane: a test around every load
+  // would put a wait at each join and the U loads of a step would no longer be in flight together.)
+  const bool whole = p0 + V <= a.L, some = p0 < a.L;
+  // U of this wave's k-rows at a time, loads first (see skinny_k_impl), sums in the plain loop's order
+  constexpr int U = 6;
+  auto run = [&](auto load_x) {
+    uint32_t k = k_lo + wave;
     for (; k + (U - 1) * WAVES < k_hi; k += U * WAVES) {
       T x[U][V];
 #pragma unroll
-      for (int u = 0; u < U; u++) load_vec_loose<T, V>(X + (size_t)(k + u * WAVES) * a.x_ks + p0, x[u]);
+      for (int u = 0; u < U; u++) load_x(k + u * WAVES, x[u]);
 #pragma unroll
       for (int q = 0; q < TQ; q++) {
         if (q < (int)a.t) {
@@ -368,23 +371,31 @@ template <typename T, int TQ> __device__ __forceinline__ void skinny_p_impl(cons
         }
       }
     }
-  }
-  for (; k < k_hi; k += WAVES) {
-    T x[V];
-    if (whole) {
-      load_vec_loose<T, V>(X + (size_t)k * a.x_ks + p0, x);   // (k-rows of X start at any element)
-    } else {
+    for (; k < k_hi; k += WAVES) {
+      T x[V];
+      load_x(k, x);
 #pragma unroll
-      for (int e = 0; e < V; e++) x[e] = p0 + e < a.L ? X[(size_t)k * a.x_ks + p0 + e] : (T)0;
-    }
+      for (int q = 0; q < TQ; q++) {
+        if (q < (int)a.t) {
+          const float y = (float)Y[(size_t)q * a.y_qs + (size_t)k * a.y_ks];  // wave-uniform, any strides
 #pragma unroll
-    for (int q = 0; q < TQ; q++) {
-      if (q < (int)a.t) {
-        const float y = (float)Y[(size_t)q * a.y_qs + (size_t)k * a.y_ks];  // wave-uniform, any strides
-#pragma unroll
-        for (int e = 0; e < V; e++) acc[q][e] = acc[q][e] + (float)x[e] * y;
+          for (int e = 0; e < V; e++) acc[q][e] = acc[q][e] + (float)x[e] * y;
+        }
       }
     }
+  };
+  if (whole) {
+    run([&](uint32_t kk, T (&x)[V]) { load_vec_loose<T, V>(X + (size_t)kk * a.x_ks + p0, x); });
+  } else if (some) {
+    const uint32_t valid = a.L - p0;   // 1 .. V - 1 elements of this lane's piece lie inside the row
+    run([&](uint32_t kk, T (&x)[V]) {
+#pragma unroll
+      for (int e = 0; e < V; e++) x[e] = (T)0;
+      const T* src = X + (size_t)kk * a.x_ks + p0;
+#pragma unroll
+      for (int e = 0; e < V - 1; e++)
+        if (e < (int)valid) x[e] = src[e];
+    });
   }
 #pragma unroll
   for (int q = 0; q < TQ; q++)
