@@ -250,9 +250,11 @@ __device__ __forceinline__ void gemm_dma2_impl(const hck_gemm_args& p, char* lds
   constexpr int A_BYTES = OpA::BYTES;
 
   uint32_t tm, tn;
-  gemm_tile_of_block(p, blockIdx.x, tm, tn);
+  uint32_t block_in_product, batch_of_block;
+  gemm_block_and_batch(block_in_product, batch_of_block);
+  gemm_tile_of_block(p, block_in_product, tm, tn);
   const uint32_t m0 = tm * BM, n0 = tn * BN;
-  const uint32_t batch = blockIdx.y;
+  const uint32_t batch = batch_of_block;
 #ifdef HC_GEMM_MERGED
   // (the second build of this file, kernels *_m: what a recording's rewrite needs)
   uint32_t batch_hi = batch, batch_lo = 0;
