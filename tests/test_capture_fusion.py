@@ -421,8 +421,8 @@ def test_head_swaps_fold_into_the_batched_products(hip_backend, dtype, B, T, H, 
 
 
 @pytest.mark.parametrize("dtype,heads,t", [(DType.float16, h, t) for h, t in
-                                           [(64, 256), (32, 512), (5, 64), (3, 128), (2, 192), (3, 320), (2, 448)]] +
-                         [(DType.float32, h, t) for h, t in [(64, 256), (5, 64), (3, 128), (2, 192)]],
+                                           [(64, 256), (32, 512), (5, 64), (3, 128), (2, 192), (3, 320), (2, 448), (12, 128), (19, 192)]] +
+                         [(DType.float32, h, t) for h, t in [(64, 256), (5, 64), (3, 128), (2, 192), (12, 128), (19, 256)]],
                          ids=lambda v: v.name if isinstance(v, DType) else str(v))
 def test_attention_becomes_one_kernel(hip_backend, dtype, heads, t):
     """q k^T -> [* s] [+ mask] softmax -> x v over heads of 64 (fp16 up to 512 keys, fp32 up to 256): one launch

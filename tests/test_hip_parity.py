@@ -105,6 +105,25 @@ def test_batched_matmul_attention_shapes(hip_backend, oracle_backend, dtype):
     check_close(hip_backend, oracle_backend, fn, TOL[dtype])
 
 
+@pytest.mark.parametrize("dtype", [F32, F16], ids=["f32", "f16"])
+@pytest.mark.parametrize("batch", [8, 12, 20, 33])
+def test_batched_matmul_slices_in_groups_of_eight(hip_backend, oracle_backend, dtype, batch):
+    """Small batched products (at most 8 blocks per slice, 8 slices or more) hand the blocks of a slice to
+    workgroups 8 apart so that a slice runs on one XCD; slices beyond the last whole group of 8 keep the
+    launch order. Every slice must still get its own operands, whatever the batch count leaves over."""
+    rng = np.random.default_rng(batch)
+    # every slice scaled differently: a block that took another slice's operands cannot pass
+    scale = (1.0 + np.arange(batch, dtype=np.float32))[:, None, None]
+    for m, k, n in ((128, 64, 64), (256, 192, 64), (64, 64, 128), (130, 72, 60)):
+        a = (rand(rng, (batch, m, k), F32) * scale / np.sqrt(k)).astype(dtype.numpy)
+        b = rand(rng, (batch, k, n), dtype)
+        fn = lambda: Tensor.batchedMatmul(Tensor(data=a), False, Tensor(data=b), False, False)
+        check_close(hip_backend, oracle_backend, fn, TOL[dtype])
+        bt = np.ascontiguousarray(np.swapaxes(b, 1, 2))
+        fn = lambda: Tensor.batchedMatmul(Tensor(data=a), False, Tensor(data=bt), True, False)
+        check_close(hip_backend, oracle_backend, fn, TOL[dtype])
+
+
 def test_batched_matmul_all_flags_small(hip_backend, oracle_backend):
     rng = np.random.default_rng(5)
     for dtype in (F32, F16):
