@@ -173,6 +173,7 @@ struct hc_ctx {
   hc_switches sw;                        // guarded by mu
   std::vector<hipModule_t> modules;
   std::unordered_map<std::string, hipFunction_t> functions;
+  std::unordered_set<std::string> functions_missing;   // names no embedded code object has
   std::unordered_map<size_t, std::vector<void*>> free_blocks;
   std::map<void*, size_t> live;          // blocks handed out: base -> bucket size, ordered by address
   size_t bytes_in_use = 0, bytes_cached = 0;
@@ -521,13 +522,15 @@ extern "C" int hc_free(hc_ctx* ctx, void* ptr) {
     ctx->batch_parked_bytes += b;
     ctx->batch_born.erase(ptr);
     if (ctx->batch_parked_bytes > kBatchParkedMax) return flush_batch_locked(ctx);
+    if (ctx->batch_launches >= ctx->batch_limit && ctx->batch_born.size() <= 1) return flush_batch_locked(ctx);   // (a full list, see batch_grew_locked)
     // A device that has nothing left to do gains nothing from a longer list. The place to cut
     // the list is where the program holds at most one result of the listed launches (between
     // two layers of a model, say): every other intermediate has been released, so no chain that
     // the rewrite could merge is open. There, once the list is long enough to be worth a
-    // rewrite, look whether the stream has run dry.
+    // rewrite, look whether the device is past the middle of the last batch (or has never had one): the
+    // list then goes out while the rest of that batch runs.
     if (ctx->batch_idle_after > 0 && ctx->batch_launches >= ctx->batch_idle_now && ctx->batch_born.size() <= 1 &&
-        ctx->batch_done && __atomic_load_n(ctx->batch_done, __ATOMIC_ACQUIRE) == ctx->batch_seq)
+        ctx->batch_done && __atomic_load_n(ctx->batch_done + 1, __ATOMIC_ACQUIRE) == ctx->batch_seq)
       return flush_batch_locked(ctx, BATCH_END_IDLE);
   } else {
     ctx->free_blocks[b].push_back(ptr);
@@ -797,9 +800,14 @@ static int launch_fn(hc_ctx* ctx, hipFunction_t fn, uint32_t gx, uint32_t gy, ui
                      uint32_t shared, const void* kernarg, size_t kernarg_bytes);
 
 // Enqueues the (rewritten) list of a recording on the capturing stream. Caller holds the lock.
-static int emit_recording_locked(hc_ctx* ctx, std::vector<hc_pending>& list) {
+// `mark_at` / `mark_fn` / `mark_args` (batching): a one-lane marker kernel goes out behind the first `mark_at`
+// entries that are enqueued.
+static int emit_recording_locked(hc_ctx* ctx, std::vector<hc_pending>& list, size_t mark_at = (size_t)-1,
+                                 hipFunction_t mark_fn = nullptr, const hck_map_args* mark_args = nullptr) {
+  size_t sent = 0;
   for (hc_pending& e : list) {
-    if (e.dropped) continue;
+    if (e.dropped || e.kind == hc_pending::FREE) continue;
+    if (sent++ == mark_at && mark_fn) HC_TRY(launch_fn(ctx, mark_fn, 1, 1, 1, HCK_BLOCK, 0, mark_args, sizeof(*mark_args)));
     if (e.kind == hc_pending::KERNEL) {
       HC_TRY(launch_fn(ctx, e.fn, e.grid[0], e.grid[1], 1, HCK_BLOCK, 0, e.args.data(), e.args.size()));
     } else if (e.kind == hc_pending::RAW_KERNEL) {
@@ -847,19 +855,32 @@ static int flush_batch_locked(hc_ctx* ctx, BatchEnd why) {
     if (!ctx->sw.no_fusion) fuse_recording(ctx);
     for (const hc_pending& e : ctx->pending) ctx->batch_enqueued += e.kind != hc_pending::FREE && !e.dropped;
     if (ctx->sw.recording_log) log_launches_locked(ctx, "batch");
-    const int emitted = emit_recording_locked(ctx, ctx->pending);
+    // Two markers tell the host how far the device has got with this batch (one-lane kernels that write the
+    // batch's number into pinned host memory): one behind the last launch, and one behind the first half of
+    // the launches, which is what the idle rule of hc_free looks at: the next batch is rewritten and enqueued
+    // while the second half still runs, instead of after the device has run dry.
+    hipFunction_t mark_fn = nullptr;
+    const bool marking = ctx->batch_idle_after > 0 && ctx->batch_done && find_kernel_locked(ctx, "hc_fill_b8", &mark_fn) == HC_OK;
+    hck_map_args near_end, at_end;
+    memset(&near_end, 0, sizeof(near_end));
+    near_end.count = 1;
+    at_end = near_end;
+    size_t to_send = 0;
+    for (const hc_pending& e : ctx->pending) to_send += e.kind != hc_pending::FREE && !e.dropped;
+    if (marking) {
+      ++ctx->batch_seq;
+      near_end.out = ctx->batch_done + 1, near_end.i0 = (int64_t)ctx->batch_seq;
+      at_end.out = ctx->batch_done, at_end.i0 = (int64_t)ctx->batch_seq;
+    }
+    const int emitted = emit_recording_locked(ctx, ctx->pending, marking ? to_send / 2 : (size_t)-1, mark_fn, &near_end);
     if (status == HC_OK) status = emitted;
     ctx->pending.clear();
     ctx->dead.clear();
-    if (emitted == HC_OK && ctx->batch_idle_after > 0 && ctx->batch_done) {
-      hck_map_args k;
-      memset(&k, 0, sizeof(k));
-      k.out = ctx->batch_done;
-      k.count = 1;
-      k.i0 = (int64_t)++ctx->batch_seq;
-      hipFunction_t fn = nullptr;
-      int marked = find_kernel_locked(ctx, "hc_fill_b8", &fn);
-      if (marked == HC_OK) marked = launch_fn(ctx, fn, 1, 1, 1, HCK_BLOCK, 0, &k, sizeof(k));
+    if (marking) {
+      // (the end marker goes out even after a failed launch, and writes both words: the host must not wait
+      // for a number that no kernel will ever write)
+      int marked = launch_fn(ctx, mark_fn, 1, 1, 1, HCK_BLOCK, 0, &at_end, sizeof(at_end));
+      if (marked == HC_OK && (emitted != HC_OK || to_send < 2)) marked = launch_fn(ctx, mark_fn, 1, 1, 1, HCK_BLOCK, 0, &near_end, sizeof(near_end));
       if (status == HC_OK) status = marked;
     }
     ctx->lazy = true;
@@ -894,7 +915,8 @@ static int alloc_batch_flag_locked(hc_ctx* ctx) {
     ctx->batch_done = nullptr;
     return hip_fail(e, "hipHostMalloc (batching's completion flag)");
   }
-  *ctx->batch_done = ctx->batch_seq;
+  ctx->batch_done[0] = ctx->batch_seq;   // [0]: the last batch has run, [1]: ... or is past its middle
+  ctx->batch_done[1] = ctx->batch_seq;
   return HC_OK;
 }
 
@@ -1123,7 +1145,12 @@ thread_local OpNote* OpNote::current = nullptr;
 // Batching: one more launch is listed; a full batch is enqueued. Caller holds the mutex.
 static int batch_grew_locked(hc_ctx* ctx) {
   if (ctx->capturing || ctx->batch_limit == 0) return HC_OK;
-  if (++ctx->batch_launches >= ctx->batch_limit) return flush_batch_locked(ctx);
+  // A full list goes out at the next place where no chain that the rewrite could merge is open (the caller
+  // holds at most one result of the listed launches: hc_free looks), or a quarter of the limit later at the
+  // latest: cut in the middle of a layer, the launches around the cut stay unmerged.
+  if (++ctx->batch_launches < ctx->batch_limit) return HC_OK;
+  if (ctx->batch_born.size() <= 1 || ctx->batch_launches >= ctx->batch_limit + ctx->batch_limit / 4)
+    return flush_batch_locked(ctx);
   return HC_OK;
 }
 
@@ -1205,10 +1232,15 @@ static int find_kernel_locked(hc_ctx* ctx, const std::string& name, hipFunction_
     return HC_OK;
   }
   hipFunction_t fn = nullptr;
-  for (hipModule_t m : ctx->modules) {
-    if (hipModuleGetFunction(&fn, m, name.c_str()) == hipSuccess) break;
-    (void)hipGetLastError();
-    fn = nullptr;
+  // (a name that was looked for in vain is remembered too: the rewrite of a recording asks for variants of a
+  // kernel that need not exist, once per launch it considers)
+  if (!ctx->functions_missing.count(name)) {
+    for (hipModule_t m : ctx->modules) {
+      if (hipModuleGetFunction(&fn, m, name.c_str()) == hipSuccess) break;
+      (void)hipGetLastError();
+      fn = nullptr;
+    }
+    if (!fn) ctx->functions_missing.insert(name);
   }
   if (!fn) return fail(HC_ERR_LOAD, "kernel '%s' is not in the embedded code objects", name.c_str());
   ctx->functions[name] = fn;

@@ -200,11 +200,15 @@ int hc_graph_destroy(hc_ctx* ctx, hc_graph* graph);
  * or ends (Tensor.swift:634-657). With max_launches > 0 the op entry points list their launches
  * instead of enqueueing them, exactly as inside a capture, and the list is rewritten (the same
  * passes, the same guarantee: the bits of the call-by-call result) and enqueued
- *  - when it holds max_launches launches, or (idle_after > 0) at least idle_after launches
- *    while the device has finished everything enqueued so far: looked up in hc_free when the
- *    caller holds at most one buffer allocated since the last batch (between two layers of a
- *    model: every other intermediate is released, so no chain the rewrite could merge is cut).
- *    While the device is busy a batch grows; once it has run dry it gets what there is. Every
+ *  - when it holds max_launches launches (at the next hc_free that leaves the caller with at most one
+ *    buffer allocated since the last batch, or a quarter of max_launches later at the latest: a
+ *    list cut in the middle of a layer leaves the launches around the cut unmerged), or
+ *    (idle_after > 0) at least idle_after launches
+ *    while the device is past the middle of the last batch (or has had none): looked up in
+ *    hc_free when the caller holds at most one buffer allocated since the last batch (between
+ *    two layers of a model: every other intermediate is released, so no chain the rewrite could
+ *    merge is cut). While the device has more than half a batch in front of it the list grows;
+ *    after that it gets what there is, rewritten and enqueued while the rest still runs. Every
  *    batch that goes out early this way doubles the number of launches the next early one needs
  *    (up to max_launches); a call that waits or transfers starts over at idle_after: a program
  *    that reads a result after every pass gets its device started after idle_after launches,
