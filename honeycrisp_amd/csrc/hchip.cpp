@@ -530,7 +530,7 @@ extern "C" int hc_free(hc_ctx* ctx, void* ptr) {
     // rewrite, look whether the device is past the middle of the last batch (or has never had one): the
     // list then goes out while the rest of that batch runs.
     if (ctx->batch_idle_after > 0 && ctx->batch_launches >= ctx->batch_idle_now && ctx->batch_born.size() <= 1 &&
-        ctx->batch_done && __atomic_load_n(ctx->batch_done + 1, __ATOMIC_ACQUIRE) == ctx->batch_seq)
+        ctx->batch_done && __atomic_load_n(ctx->batch_done, __ATOMIC_ACQUIRE) == ctx->batch_seq)
       return flush_batch_locked(ctx, BATCH_END_IDLE);
   } else {
     ctx->free_blocks[b].push_back(ptr);
@@ -855,36 +855,37 @@ static int flush_batch_locked(hc_ctx* ctx, BatchEnd why) {
     if (!ctx->sw.no_fusion) fuse_recording(ctx);
     for (const hc_pending& e : ctx->pending) ctx->batch_enqueued += e.kind != hc_pending::FREE && !e.dropped;
     if (ctx->sw.recording_log) log_launches_locked(ctx, "batch");
-    // Two markers tell the host how far the device has got with this batch (one-lane kernels that write the
-    // batch's number into pinned host memory): one behind the last launch, and one behind the first half of
-    // the launches, which is what the idle rule of hc_free looks at: the next batch is rewritten and enqueued
-    // while the second half still runs, instead of after the device has run dry.
+    // A marker tells the host how far the device has got with this batch: a one-lane kernel behind the first half
+    // of the launches that writes the batch's number into pinned host memory, which is what the idle rule of hc_free
+    // looks at: the next batch is rewritten and enqueued while the second half still runs, instead of after the
+    // device has run dry. (One marker, not a second one behind the batch: its store to host memory makes the
+    // device write its caches back, about 17 us on the device per marker in a pass of config 5. And none once the
+    // early batches have grown to the limit: a full list goes out whatever the device is doing. After a wait,
+    // which starts the early batches over, the number in host memory is at most batch_seq and the device idle.)
     hipFunction_t mark_fn = nullptr;
-    const bool marking = ctx->batch_idle_after > 0 && ctx->batch_done && find_kernel_locked(ctx, "hc_fill_b8", &mark_fn) == HC_OK;
-    hck_map_args near_end, at_end;
-    memset(&near_end, 0, sizeof(near_end));
-    near_end.count = 1;
-    at_end = near_end;
+    const bool marking = ctx->batch_idle_after > 0 && ctx->batch_idle_now < ctx->batch_limit && ctx->batch_done &&
+                         find_kernel_locked(ctx, "hc_fill_b8", &mark_fn) == HC_OK;
+    hck_map_args mark;
+    memset(&mark, 0, sizeof(mark));
+    mark.count = 1;
     size_t to_send = 0;
     for (const hc_pending& e : ctx->pending) to_send += e.kind != hc_pending::FREE && !e.dropped;
     if (marking) {
-      ++ctx->batch_seq;
-      near_end.out = ctx->batch_done + 1, near_end.i0 = (int64_t)ctx->batch_seq;
-      at_end.out = ctx->batch_done, at_end.i0 = (int64_t)ctx->batch_seq;
+      mark.out = ctx->batch_done;
+      mark.i0 = (int64_t)++ctx->batch_seq;
     }
-    const int emitted = emit_recording_locked(ctx, ctx->pending, marking ? to_send / 2 : (size_t)-1, mark_fn, &near_end);
+    const int emitted = emit_recording_locked(ctx, ctx->pending, marking ? to_send / 2 : (size_t)-1, mark_fn, &mark);
     if (status == HC_OK) status = emitted;
     ctx->pending.clear();
     ctx->dead.clear();
-    if (marking) {
-      // (the end marker goes out even after a failed launch, and writes both words: the host must not wait
-      // for a number that no kernel will ever write)
-      int marked = launch_fn(ctx, mark_fn, 1, 1, 1, HCK_BLOCK, 0, &at_end, sizeof(at_end));
-      if (marked == HC_OK && (emitted != HC_OK || to_send < 2)) marked = launch_fn(ctx, mark_fn, 1, 1, 1, HCK_BLOCK, 0, &near_end, sizeof(near_end));
+    if (marking && (emitted != HC_OK || to_send == 0)) {
+      // (the marker did not go out inside the list: the host must not wait for a number that no kernel will write)
+      const int marked = launch_fn(ctx, mark_fn, 1, 1, 1, HCK_BLOCK, 0, &mark, sizeof(mark));
       if (status == HC_OK) status = marked;
     }
     ctx->lazy = true;
   }
+  const bool full = ctx->batch_launches >= ctx->batch_limit;
   ctx->batch_launches = 0;
   ctx->batch_born.clear();
   // An early batch pays for itself when the device would otherwise sit idle until a wait (a program
@@ -896,8 +897,11 @@ static int flush_batch_locked(hc_ctx* ctx, BatchEnd why) {
     ctx->batch_failed = status;
     ctx->batch_failed_why = g_last_error;
   }
+  // (a list that filled up while the device still had half a batch in front of it: the device is the slower side,
+  // early batches have nothing to give until the next wait, and the markers they need can stay away)
   if (why == BATCH_END_IDLE) ctx->batch_idle_now = std::min(ctx->batch_idle_now * 2, ctx->batch_limit);
   else if (why == BATCH_END_WAIT) ctx->batch_idle_now = ctx->batch_idle_after;
+  else if (full && ctx->batch_idle_after > 0) ctx->batch_idle_now = ctx->batch_limit;
   for (auto& kv : ctx->batch_parked) {
     auto& pool = ctx->free_blocks[kv.first];
     pool.insert(pool.end(), kv.second.begin(), kv.second.end());
@@ -915,8 +919,7 @@ static int alloc_batch_flag_locked(hc_ctx* ctx) {
     ctx->batch_done = nullptr;
     return hip_fail(e, "hipHostMalloc (batching's completion flag)");
   }
-  ctx->batch_done[0] = ctx->batch_seq;   // [0]: the last batch has run, [1]: ... or is past its middle
-  ctx->batch_done[1] = ctx->batch_seq;
+  *ctx->batch_done = ctx->batch_seq;   // the number of the last batch whose first half the device has run
   return HC_OK;
 }
 
